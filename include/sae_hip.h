@@ -1,0 +1,185 @@
+/*
+ * sae_hip.h -- C ABI of libsae_hip.so: the sparse-autoencoder train step on MI355X (gfx950).
+ *
+ * Conventions (all entry points):
+ *   - plain device pointers, 64-bit sizes, a dtype enum and a hipStream_t passed as void*;
+ *   - return 0 on success, a negative SAE_ERR_* code otherwise; sae_last_error() then
+ *     returns a thread-local, human-readable message;
+ *   - nothing here allocates or frees device memory, and nothing synchronises the stream:
+ *     outputs and workspaces are caller-owned (sizes from the *_workspace_bytes queries);
+ *   - inputs are never modified unless the parameter is documented "in/out".
+ *
+ * Layout vocabulary:
+ *   B tokens, d = d_model, F = d_sae, k = top_k.
+ *   "feature-major" = [F, d] row-major: one feature's d_model-vector is contiguous.
+ *   The decoder W_D [F, d] is feature-major in the reference already
+ *   (src/llamascopium/models/sae.py:69).  The encoder is W_E [d, F] in the reference
+ *   (models/sae.py:67); this library consumes its transpose W_E^T [F, d] (feature-major),
+ *   i.e. the same memory a [d, F] tensor with strides (1, d) views.
+ *
+ * Sparse code ("feature activations" in sparse form), produced by the select entry points:
+ *   idx     int32  flat array of feature indices,
+ *   val     fp32   flat array of feature activations (already divided by the decoder-norm
+ *                  scale when one was applied),
+ *   row_off int64  [B]  first slot of token b in idx/val,
+ *   row_nnz int32  [B]  number of valid slots of token b; indices ascend within a token.
+ *   For per-token TopK row_off[b] = b*k and unused slots hold idx 0 / val 0.
+ *
+ * Each declaration cites the reference code it replaces (paths relative to the reference
+ * checkout, src/llamascopium/...).
+ */
+#ifndef SAE_HIP_H
+#define SAE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { SAE_F32 = 0, SAE_BF16 = 1 } sae_dtype;
+
+enum {
+  SAE_OK = 0,
+  SAE_ERR_INVALID_ARG = -1,   /* null pointer, non-positive size, bad enum            */
+  SAE_ERR_UNSUPPORTED = -2,   /* shape outside what the kernels are built for         */
+  SAE_ERR_LAUNCH = -3,        /* hipGetLastError() after a launch                     */
+  SAE_ERR_WORKSPACE = -4      /* workspace pointer null or too small                  */
+};
+
+/* Library identification and error text. */
+int sae_abi_version(void);
+const char *sae_last_error(void);
+
+/* ---- element-wise helpers --------------------------------------------------------- */
+
+/* dst[i] = bf16(src[i]) (round-to-nearest-even).  What torch.autocast does to the GEMM
+ * operands (trainer.py:613). */
+int sae_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream);
+
+/* out[f] = ||W[f, :]||_2 for feature-major W [F, d] fp32.
+ * Replaces decoder_norm()/encoder_norm() (models/sae.py:136-160). */
+int sae_row_norm(const float *w, float *out, int64_t F, int64_t d, void *stream);
+
+/* dst[c, r] = src[r, c] for fp32 src [rows, cols] -> dst [cols, rows].  Used to import
+ * a reference-layout W_E [d, F] into feature-major form and back. */
+int sae_transpose_f32(const float *src, float *dst, int64_t rows, int64_t cols, void *stream);
+
+/* out[j] (+)= sum_b src[b, j] for src [B, n] fp32.  accumulate != 0 adds to out.
+ * workspace: sae_col_sum_workspace_bytes(B, n) bytes.  The summation order is fixed, so the
+ * result is reproducible.  Replaces the bias gradients autograd produces (sum over the
+ * token dim). */
+int64_t sae_col_sum_workspace_bytes(int64_t B, int64_t n);
+int sae_col_sum(const float *src, float *out, int64_t B, int64_t n, int accumulate, void *workspace,
+                int64_t workspace_bytes, void *stream);
+
+/* ---- encoder ---------------------------------------------------------------------- */
+
+/* pre[b, f] = sum_j x[b, j] * w_enc_t[f, j]          (no bias: the select kernels add it)
+ * x [B, d] and w_enc_t [F, d] share in_dtype (SAE_BF16: bf16 operands, fp32 accumulate;
+ * SAE_F32: fp32 MFMA).  pre [B, F] is written as out_dtype; SAE_BF16 rounds the fp32
+ * accumulator to bf16, which is what the autocast matmul returns.
+ * Requires d % 64 == 0 (bf16) / d % 32 == 0 (fp32); B and F arbitrary (edge tiles masked).
+ * Replaces `x @ self.W_E` (models/sae.py:324). */
+int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, int64_t B, int64_t d, int64_t F,
+                     int in_dtype, int out_dtype, void *stream);
+
+/* ---- activation select ------------------------------------------------------------ */
+
+/* Per-token TopK with fused bias and decoder-norm scale.
+ *   h0 = pre[b, f] + b_enc[f]            (b_enc may be null = 0)
+ *   h1 = h0 * scale[f]                   (scale may be null = 1; it is ||W_D[f]||)
+ *   keep the k largest h1 > 0 of each token; ties -> lowest feature index;
+ *   val = h1 / scale (= feature_acts), idx ascending within the token.
+ * Outputs idx/val [B, k], row_off [B] (= b*k), row_nnz [B] (<= k; fewer when a token has
+ * fewer than k positive pre-activations).
+ * Replaces the topk closure (models/sparse_dictionary.py:733-759) + utils/math.py:81-171 and
+ * the scale/unscale around it (models/sae.py:334-341). */
+int sae_select_topk_row(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                        int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
+                        int32_t *row_nnz, void *stream);
+
+/* Same, with the capacity of the in-LDS candidate list exposed (0..4096).  A token whose
+ * candidates do not fit takes the general path (radix histograms over the whole row), which
+ * returns the identical result; cand_cap = 0 forces it for every token.  For testing and
+ * tuning; no counterpart in the reference. */
+int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                           int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
+                           int32_t *row_nnz, int cand_cap, void *stream);
+
+/* ---- sparse decoder --------------------------------------------------------------- */
+
+/* recon[b, :] = sum_s val[s] * W_D[idx[s], :] + b_dec,  s over token b's slots.
+ * w_dec [F, d] in w_dtype (bf16 shadow or fp32 master); recon [B, d] fp32; b_dec fp32 [d]
+ * or null.  Requires d % 8 == 0.
+ * Replaces `feature_acts @ self.W_D + self.b_D` (models/sae.py:367-371) and the Triton SpMM
+ * (kernels/kernels.py:382-436). */
+int sae_sparse_decode_fwd(const int32_t *idx, const float *val, const int64_t *row_off,
+                          const int32_t *row_nnz, const void *w_dec, int w_dtype, const float *b_dec,
+                          float *recon, int64_t B, int64_t d, int64_t F, void *stream);
+
+/* dval[s] = grad_recon[b, :] . W_D[idx[s], :] for every valid slot s of token b
+ * (0 for unused slots).  Replaces the "dense x dense -> sparse out" backward
+ * (kernels/kernels.py:326-379, 562-563). */
+int sae_sparse_decode_bwd_dval(const int32_t *idx, const int64_t *row_off, const int32_t *row_nnz,
+                               const float *grad_recon, const void *w_dec, int w_dtype, float *dval,
+                               int64_t B, int64_t d, int64_t F, int64_t n_slots, void *stream);
+
+/* Fused forward+backward of decode and the reconstruction loss for one batch:
+ *   recon = decode(idx, val) + b_dec
+ *   loss_tok[b]     = tok_w[b] * sum_j (recon[b,j] - label[b,j])^2
+ *   grad_recon[b,:] = 2 * tok_w[b] * (recon[b,:] - label[b,:])
+ *   dval[s]         = grad_recon[b,:] . W_D[idx[s],:]
+ * tok_w[b] is the per-token weight of the masked mean (mask[b] / mask.sum(); 1/B without a
+ * mask), or null for 1.  recon may be null when the caller does not need it.
+ * Replaces models/sae.py:367-371 + models/sparse_dictionary.py:881-886
+ * (+ utils/tensor_specs.py:64-84) and their autograd twins. */
+int sae_sparse_decode_mse_fused(const int32_t *idx, const float *val, const int64_t *row_off,
+                                const int32_t *row_nnz, const void *w_dec, int w_dtype,
+                                const float *b_dec, const float *label, const float *tok_w,
+                                float *recon, float *loss_tok, float *grad_recon, float *dval,
+                                int64_t B, int64_t d, int64_t F, int64_t n_slots, void *stream);
+
+/* ---- sparse backward -------------------------------------------------------------- */
+
+/* Feature-major index of a sparse code (a CSR transpose): for every feature f the list of
+ * slots s with idx[s] == f, in ascending slot (= token) order.
+ *   feat_ptr  int32 [F + 1]   segment bounds,
+ *   feat_slot int32 [n_valid] slot ids grouped by feature (n_valid = sum row_nnz),
+ *   slot_tok  int32 [n_slots] token of every slot (filled for valid slots).
+ * workspace: sae_feature_index_workspace_bytes(B, F, n_slots) bytes.
+ * Replaces the global sort into COO (kernels/kernels.py:61-134). */
+int64_t sae_feature_index_workspace_bytes(int64_t B, int64_t F, int64_t n_slots);
+int sae_build_feature_index(const int32_t *idx, const int64_t *row_off, const int32_t *row_nnz,
+                            int64_t B, int64_t F, int64_t n_slots, int32_t *feat_ptr,
+                            int32_t *feat_slot, int32_t *slot_tok, void *workspace,
+                            int64_t workspace_bytes, void *stream);
+
+/* out[f, :] = sum_{s in segment f} coef[s] * dense[slot_tok[s], :]   for every f in [0, F)
+ * (rows with an empty segment are written as zeros, so `out` needs no prior clearing);
+ * optionally bias_out[f] = sum coef[s].  dense [B, d] in dense_dtype, out [F, d] fp32.
+ * With coef = val and dense = grad_recon this is dW_D; with coef = d(pre) and dense = x it
+ * is dW_E^T and bias_out = db_E.
+ * Replaces the sorted atomic-add SpMM (kernels/kernels.py:137-225) and the dense
+ * `f^T @ grad` / `x^T @ dh` GEMMs autograd runs. */
+int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                         const float *coef, const void *dense, int dense_dtype, float *out,
+                         float *bias_out, int64_t F, int64_t d, void *stream);
+
+/* ---- optimiser -------------------------------------------------------------------- */
+
+/* One bias-corrected Adam update over n contiguous fp32 elements (p, m, v in/out):
+ *   m = b1*m + (1-b1)*g;  v = b2*v + (1-b2)*g*g;
+ *   p -= lr / (1 - b1^t) * m / (sqrt(v) / sqrt(1 - b2^t) + eps)
+ * (torch.optim.Adam, no weight decay, no amsgrad: trainer.py:375-390).  step = t >= 1.
+ * shadow_bf16 (nullable) receives bf16(p) for the next step's GEMM / gather operands.
+ * row_norm_out (nullable, requires row_len > 0 and n % row_len == 0) receives the L2 norm
+ * of every updated row of length row_len, i.e. the next step's decoder_norm(). */
+int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
+                  float beta2, float eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                  int64_t row_len, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAE_HIP_H */

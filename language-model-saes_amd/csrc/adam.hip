@@ -1,0 +1,119 @@
+// Fused Adam for gfx950: one streaming pass that reads g, p, m, v and writes p, m, v
+// (28 bytes per parameter), optionally the bf16 shadow of p that the next step's GEMM and
+// row gathers read (+2 bytes) and the L2 norm of every updated row (the next step's
+// decoder_norm(), free because the row is in registers anyway).
+#include "common.h"
+
+namespace sae {
+
+struct AdamScalars {
+  float beta1, beta2, one_minus_beta1, one_minus_beta2, step_size, inv_bc2_sqrt, eps;
+};
+
+__device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v, const AdamScalars &a) {
+  m = m + a.one_minus_beta1 * (g - m);               // lerp, as torch does
+  v = a.beta2 * v + a.one_minus_beta2 * g * g;
+  const float denom = sqrtf(v) * a.inv_bc2_sqrt + a.eps;
+  p = p - a.step_size * (m / denom);
+  return p;
+}
+
+// flat: grid-stride over float4 groups
+__global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, const float *__restrict__ g,
+                                                        float *__restrict__ m, float *__restrict__ v, int64_t n,
+                                                        AdamScalars a, uint16_t *__restrict__ shadow) {
+  const int64_t n4 = n >> 2;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    float4 pp = reinterpret_cast<float4 *>(p)[i];
+    const float4 gg = reinterpret_cast<const float4 *>(g)[i];
+    float4 mm = reinterpret_cast<float4 *>(m)[i];
+    float4 vv = reinterpret_cast<float4 *>(v)[i];
+    adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
+    adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
+    reinterpret_cast<float4 *>(p)[i] = pp;
+    reinterpret_cast<float4 *>(m)[i] = mm;
+    reinterpret_cast<float4 *>(v)[i] = vv;
+    if (shadow) {
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
+      o.y = (uint32_t)f32_to_bf16_bits(pp.z) | ((uint32_t)f32_to_bf16_bits(pp.w) << 16);
+      reinterpret_cast<uint2 *>(shadow)[i] = o;
+    }
+  }
+  const int64_t t = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) {
+    float pp = p[t], mm = m[t], vv = v[t];
+    adam_one(pp, g[t], mm, vv, a);
+    p[t] = pp; m[t] = mm; v[t] = vv;
+    if (shadow) shadow[t] = f32_to_bf16_bits(pp);
+  }
+}
+
+// row-wise: one workgroup per row of row_len (a multiple of 4) elements; also emits the row norm
+__global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, const float *__restrict__ g,
+                                                        float *__restrict__ m, float *__restrict__ v, int row_len,
+                                                        AdamScalars a, uint16_t *__restrict__ shadow,
+                                                        float *__restrict__ row_norm) {
+  __shared__ float red[4];
+  const int64_t base4 = (int64_t)blockIdx.x * (row_len >> 2);
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < (row_len >> 2); i += 256) {
+    const int64_t q = base4 + i;
+    float4 pp = reinterpret_cast<float4 *>(p)[q];
+    const float4 gg = reinterpret_cast<const float4 *>(g)[q];
+    float4 mm = reinterpret_cast<float4 *>(m)[q];
+    float4 vv = reinterpret_cast<float4 *>(v)[q];
+    adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
+    adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
+    reinterpret_cast<float4 *>(p)[q] = pp;
+    reinterpret_cast<float4 *>(m)[q] = mm;
+    reinterpret_cast<float4 *>(v)[q] = vv;
+    sq = fmaf(pp.x, pp.x, sq); sq = fmaf(pp.y, pp.y, sq); sq = fmaf(pp.z, pp.z, sq); sq = fmaf(pp.w, pp.w, sq);
+    if (shadow) {
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
+      o.y = (uint32_t)f32_to_bf16_bits(pp.z) | ((uint32_t)f32_to_bf16_bits(pp.w) << 16);
+      reinterpret_cast<uint2 *>(shadow)[q] = o;
+    }
+  }
+  const float tot = block_sum<4>(sq, red);
+  if (threadIdx.x == 0) row_norm[blockIdx.x] = sqrtf(tot);
+}
+
+}  // namespace sae
+
+extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
+                             float beta2, float eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                             int64_t row_len, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(p && g && m && v, SAE_ERR_INVALID_ARG, "adam_step: null pointer");
+  SAE_REQUIRE(n > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step: n must be positive and step >= 1");
+  SAE_REQUIRE((((uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "adam_step: 16-byte alignment required");
+  AdamScalars a;
+  a.beta1 = beta1; a.beta2 = beta2;
+  a.one_minus_beta1 = 1.f - beta1;
+  a.one_minus_beta2 = 1.f - beta2;
+  const double bc1 = 1.0 - pow((double)beta1, (double)step);
+  const double bc2 = 1.0 - pow((double)beta2, (double)step);
+  a.step_size = (float)((double)lr / bc1);
+  a.inv_bc2_sqrt = (float)(1.0 / sqrt(bc2));
+  a.eps = eps;
+  hipStream_t st = (hipStream_t)stream;
+  if (row_norm_out) {
+    SAE_REQUIRE(row_len > 0 && row_len % 4 == 0 && n % row_len == 0 && row_len < (1LL << 31), SAE_ERR_INVALID_ARG,
+                "adam_step: row_norm_out needs row_len %% 4 == 0 dividing n");
+    const int64_t rows = n / row_len;
+    SAE_REQUIRE(rows < (1LL << 31), SAE_ERR_UNSUPPORTED, "adam_step: too many rows");
+    hipLaunchKernelGGL(adam_rows_kernel, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
+                       reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out);
+  } else {
+    int64_t blocks = ((n >> 2) + 255) / 256;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(adam_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
+                       reinterpret_cast<uint16_t *>(shadow_bf16));
+  }
+  return check_launch("adam_step");
+}

@@ -1,0 +1,75 @@
+// Shared helpers for the gfx950 kernels of libsae_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/sae_hip.h"
+
+namespace sae {
+
+// ---- error reporting ----------------------------------------------------------------
+char *error_buffer();            // thread-local, 512 bytes (defined in capi.hip)
+int fail(int code, const char *fmt, ...);
+
+#define SAE_REQUIRE(cond, code, ...)                 \
+  do {                                               \
+    if (!(cond)) return ::sae::fail((code), __VA_ARGS__); \
+  } while (0)
+
+inline int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return SAE_OK;
+}
+
+// Clears `bytes` bytes (a multiple of 4) with a fill kernel; safe under HIP graph capture,
+// where a memset node is not.  Defined in elementwise.hip.
+int zero_fill(void *p, size_t bytes, hipStream_t st);
+
+// ---- bf16 <-> fp32 (bit level, round-to-nearest-even like torch) ---------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+// ---- wave (64 lanes) and block reductions ---------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Sum over a block of NW waves; every thread gets the result.  `red` holds >= NW floats.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float *red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) t += red[i];
+  return t;
+}
+
+// 16-byte vector of raw bits
+struct __attribute__((aligned(16))) u32x4 {
+  uint32_t x, y, z, w;
+};
+
+}  // namespace sae

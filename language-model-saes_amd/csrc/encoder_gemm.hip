@@ -1,0 +1,240 @@
+// Encoder pre-activation GEMM for gfx950:  pre[B, F] = x[B, d] * W_E^T[F, d]^T.
+//
+// Both operands are K-contiguous ("NT" GEMM), so a 16-byte global load fetches exactly the
+// 8 bf16 (or 4 fp32) one lane feeds to a matrix-core instruction.
+//
+// Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile
+// and walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32).  Waves are arranged 2 x 4:
+// each owns 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32 accumulators per
+// lane).  Slabs are double-buffered in LDS (2 x (32 + 32) KiB = 128 of the CU's 160 KiB); the
+// next slab's global loads are in flight while the current one feeds the matrix cores.
+//
+// LDS layout: row r of a slab is 128 bytes = 8 chunks of 16 bytes; chunk c is stored at
+// physical chunk c ^ ((r >> 1) & 7).  A group of 16 lanes then covers 256 distinct bytes both
+// when the slab is written (8 lanes per row, 2 rows) and when MFMA fragments are read
+// (16 rows, one logical chunk), so neither side bank-conflicts.
+//
+// The matrix cores compute D = Wtile * xtile^T (features along the 32 "rows" of the
+// instruction), which leaves every lane holding 4 consecutive features of one token: the
+// epilogue packs them into one 8-byte (bf16) or 16-byte (fp32) store.
+//
+// Workgroups are numbered so that consecutive ids land on the 8 XCDs round-robin, and the
+// workgroups of one XCD walk all token tiles of one feature tile before moving on: a W_E
+// slab is pulled from HBM once per XCD-L2 and shared by the 16 token tiles.
+#include "common.h"
+
+namespace sae {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+constexpr int GEMM_BM = 256;       // tokens per workgroup tile
+constexpr int GEMM_BN = 256;       // features per workgroup tile
+constexpr int GEMM_SLAB = 128;     // bytes of K per row per slab
+constexpr int GEMM_THREADS = 512;
+constexpr int GEMM_LDS_BYTES = 2 * (GEMM_BM + GEMM_BN) * GEMM_SLAB;
+
+__device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+template <bool BF16_IN>
+__device__ __forceinline__ void mma_chunk(const u32x4 &wf, const u32x4 &xf, f32x16_t &acc) {
+  if constexpr (BF16_IN) {
+    bf16x8_t a = __builtin_bit_cast(bf16x8_t, wf);
+    bf16x8_t b = __builtin_bit_cast(bf16x8_t, xf);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+  } else {
+    f32x4_t a = __builtin_bit_cast(f32x4_t, wf);
+    f32x4_t b = __builtin_bit_cast(f32x4_t, xf);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
+  }
+}
+
+template <bool BF16_IN, bool BF16_OUT>
+__global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
+    const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
+    int row_bytes /* d * sizeof(elem) */, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  // [x slab 0][x slab 1][w slab 0][w slab 1]
+  constexpr int X_BYTES = GEMM_BM * GEMM_SLAB, W_BYTES = GEMM_BN * GEMM_SLAB;
+
+  // ---- XCD-aware tile assignment ----
+  const int bid = blockIdx.x;
+  const int total = tiles_m * tiles_n;
+  int tile_m, tile_n;
+  {
+    const int xcd = bid & 7, slot = bid >> 3;
+    const int full = (tiles_n >> 3) << 3;  // feature tiles that split evenly over 8 XCDs
+    const int lin_limit = full * tiles_m;
+    if (bid < lin_limit) {
+      tile_n = (slot / tiles_m) * 8 + xcd;
+      tile_m = slot % tiles_m;
+    } else {  // remainder: plain row-major walk
+      const int r = bid - lin_limit;
+      tile_n = full + r / tiles_m;
+      tile_m = r % tiles_m;
+    }
+    (void)total;
+  }
+  const int m0 = tile_m * GEMM_BM, n0 = tile_n * GEMM_BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+
+  // ---- global -> LDS staging assignment: 8 lanes cover one 128-byte row slab ----
+  const int ld_chunk = tid & 7, ld_row = tid >> 3;  // rows ld_row + 64*i, i = 0..3
+  const char *xg[4];
+  const char *wg[4];
+  bool xok[4], wok[4];
+  int lds_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ld_row + 64 * i;
+    xok[i] = (m0 + r) < M;
+    wok[i] = (n0 + r) < N;
+    xg[i] = x + (size_t)(xok[i] ? (m0 + r) : 0) * row_bytes + ld_chunk * 16;
+    wg[i] = w + (size_t)(wok[i] ? (n0 + r) : 0) * row_bytes + ld_chunk * 16;
+    lds_off[i] = swz(r, ld_chunk);
+  }
+
+  f32x16_t acc[2][4];  // [feature sub-tile][token sub-tile]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int n_slabs = row_bytes / GEMM_SLAB;
+  u32x4 xr[4], wr[4];
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+  auto load_global = [&](int slab) {
+    const size_t off = (size_t)slab * GEMM_SLAB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xg[i] + off) : zero4;
+      wr[i] = wok[i] ? *reinterpret_cast<const u32x4 *>(wg[i] + off) : zero4;
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4 *>(lds + buf * X_BYTES + lds_off[i]) = xr[i];
+      *reinterpret_cast<u32x4 *>(lds + 2 * X_BYTES + buf * W_BYTES + lds_off[i]) = wr[i];
+    }
+  };
+
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  for (int slab = 0; slab < n_slabs; ++slab) {
+    const int buf = slab & 1;
+    if (slab + 1 < n_slabs) load_global(slab + 1);
+    const char *lx = lds + buf * X_BYTES;
+    const char *lw = lds + 2 * X_BYTES + buf * W_BYTES;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {  // 4 MFMA k-steps per slab (32 bytes of K each)
+      const int chunk = 2 * s + frag_half;
+      u32x4 wf[2], xf[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 32 + frag_row, chunk));
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mma_chunk<BF16_IN>(wf[i], xf[j], acc[i][j]);
+    }
+    if (slab + 1 < n_slabs) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds, per (i, j, g): 4 consecutive features of one token ----
+  // D[row = feature, col = token]: token = lane % 32, feature = 8*g + 4*(lane/32) + r
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int tok = m0 + wm * 128 + j * 32 + frag_row;
+    if (tok >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int f = n0 + wn * 64 + i * 32 + 8 * g + 4 * frag_half;
+        const float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
+        const float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+        if constexpr (BF16_OUT) {
+          uint16_t *o = reinterpret_cast<uint16_t *>(out) + (size_t)tok * N + f;
+          if (f + 3 < N && (N & 3) == 0) {
+            uint2 pk;
+            pk.x = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+            pk.y = (uint32_t)f32_to_bf16_bits(v2) | ((uint32_t)f32_to_bf16_bits(v3) << 16);
+            *reinterpret_cast<uint2 *>(o) = pk;
+          } else {
+            if (f + 0 < N) o[0] = f32_to_bf16_bits(v0);
+            if (f + 1 < N) o[1] = f32_to_bf16_bits(v1);
+            if (f + 2 < N) o[2] = f32_to_bf16_bits(v2);
+            if (f + 3 < N) o[3] = f32_to_bf16_bits(v3);
+          }
+        } else {
+          float *o = reinterpret_cast<float *>(out) + (size_t)tok * N + f;
+          if (f + 3 < N && (N & 3) == 0) {
+            *reinterpret_cast<float4 *>(o) = make_float4(v0, v1, v2, v3);
+          } else {
+            if (f + 0 < N) o[0] = v0;
+            if (f + 1 < N) o[1] = v1;
+            if (f + 2 < N) o[2] = v2;
+            if (f + 3 < N) o[3] = v3;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <bool BF16_IN, bool BF16_OUT>
+static int launch_gemm(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, hipStream_t st) {
+  const int esz = BF16_IN ? 2 : 4;
+  const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
+  auto kern = encoder_gemm_kernel<BF16_IN, BF16_OUT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       GEMM_LDS_BYTES);
+    if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "encoder_gemm: cannot reserve %d bytes of LDS: %s", GEMM_LDS_BYTES,
+                                     hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
+                     (const char *)w, out, (int)B, (int)F, (int)(d * esz), tiles_m, tiles_n);
+  return check_launch("encoder_gemm");
+}
+
+}  // namespace sae
+
+extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, int64_t B, int64_t d, int64_t F,
+                                int in_dtype, int out_dtype, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x && w_enc_t && pre, SAE_ERR_INVALID_ARG, "encoder_gemm: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0, SAE_ERR_INVALID_ARG, "encoder_gemm: B, d, F must be positive");
+  SAE_REQUIRE(in_dtype == SAE_F32 || in_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad in_dtype %d", in_dtype);
+  SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad out_dtype %d", out_dtype);
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm: size too large");
+  const int64_t per_slab = in_dtype == SAE_BF16 ? 64 : 32;
+  SAE_REQUIRE(d % per_slab == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm: d_model=%lld must be a multiple of %lld",
+              (long long)d, (long long)per_slab);
+  SAE_REQUIRE((((uintptr_t)x | (uintptr_t)w_enc_t | (uintptr_t)pre) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "encoder_gemm: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (in_dtype == SAE_BF16) {
+    return out_dtype == SAE_BF16 ? launch_gemm<true, true>(x, w_enc_t, pre, B, d, F, st)
+                                 : launch_gemm<true, false>(x, w_enc_t, pre, B, d, F, st);
+  }
+  return out_dtype == SAE_BF16 ? launch_gemm<false, true>(x, w_enc_t, pre, B, d, F, st)
+                               : launch_gemm<false, false>(x, w_enc_t, pre, B, d, F, st);
+}

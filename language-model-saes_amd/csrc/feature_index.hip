@@ -1,0 +1,270 @@
+// Feature-major index of a sparse code, and the weight-gradient rows built from it (gfx950).
+//
+// The select kernels emit the code token-major (slots of token 0, then token 1, ...).  The
+// weight gradients need the transpose: for every feature, the slots that name it.
+//
+//   count   one global atomic per valid slot into counts[F]; also records slot -> token
+//   scan    exclusive prefix sum over counts -> feat_ptr[F + 1]
+//   fill    slot ids dropped into their feature's segment through a per-feature cursor
+//   order   every segment is put into ascending slot order, so the result (and every sum
+//           taken over a segment afterwards) is independent of the order in which the
+//           atomics of `fill` landed: short segments by a rank count inside one wave, long
+//           ones by a bitmap counting sort over the token range.
+//
+// The gradient kernel then owns one feature per workgroup and writes the whole [d] row:
+// sum over the segment of coef[slot] * dense[token(slot), :].  Features with an empty
+// segment get zeros, so no clearing pass over the [F, d] gradient is needed, and no atomics
+// touch it.
+#include "common.h"
+
+namespace sae {
+
+constexpr int FI_THREADS = 256;
+
+__global__ void fi_zero_kernel(int32_t *p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// one wave per token; lanes stride over its slots
+__global__ __launch_bounds__(FI_THREADS) void fi_count_kernel(const int32_t *__restrict__ idx,
+                                                              const int64_t *__restrict__ row_off,
+                                                              const int32_t *__restrict__ row_nnz, int B, int F,
+                                                              int32_t *__restrict__ counts,
+                                                              int32_t *__restrict__ slot_tok) {
+  const int b = blockIdx.x * (FI_THREADS / 64) + (threadIdx.x >> 6);
+  if (b >= B) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t off = row_off[b];
+  const int nnz = row_nnz[b];
+  for (int j = lane; j < nnz; j += 64) {
+    const int f = idx[off + j];
+    if ((unsigned)f < (unsigned)F) atomicAdd(&counts[f], 1);
+    slot_tok[off + j] = b;
+  }
+}
+
+// Single-workgroup exclusive scan: thread t owns a contiguous run of ceil(F/1024) counters.
+__global__ __launch_bounds__(1024) void fi_scan_kernel(const int32_t *__restrict__ counts, int F,
+                                                       int32_t *__restrict__ feat_ptr,
+                                                       int32_t *__restrict__ cursor) {
+  __shared__ int32_t part[1024];
+  const int tid = threadIdx.x;
+  const int per = (F + 1023) / 1024;
+  const int lo = tid * per, hi = min(F, lo + per);
+  int s = 0;
+  for (int i = lo; i < hi; ++i) s += counts[i];
+  part[tid] = s;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over 1024 partials
+  for (int o = 1; o < 1024; o <<= 1) {
+    const int v = tid >= o ? part[tid - o] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;  // exclusive prefix of my run
+  for (int i = lo; i < hi; ++i) {
+    const int c = counts[i];
+    feat_ptr[i] = run;
+    cursor[i] = run;
+    run += c;
+  }
+  if (tid == 1023) feat_ptr[F] = part[1023];
+}
+
+__global__ __launch_bounds__(FI_THREADS) void fi_fill_kernel(const int32_t *__restrict__ idx,
+                                                             const int64_t *__restrict__ row_off,
+                                                             const int32_t *__restrict__ row_nnz, int B, int F,
+                                                             int32_t *__restrict__ cursor,
+                                                             int32_t *__restrict__ feat_slot) {
+  const int b = blockIdx.x * (FI_THREADS / 64) + (threadIdx.x >> 6);
+  if (b >= B) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t off = row_off[b];
+  const int nnz = row_nnz[b];
+  for (int j = lane; j < nnz; j += 64) {
+    const int f = idx[off + j];
+    if ((unsigned)f < (unsigned)F) {
+      const int pos = atomicAdd(&cursor[f], 1);
+      feat_slot[pos] = (int32_t)(off + j);
+    }
+  }
+}
+
+// Put every segment into ascending slot order (out of place: `unordered` -> feat_slot).
+// One wave per feature handles segments of up to 64 slots with a rank count across lanes.
+__global__ __launch_bounds__(FI_THREADS) void fi_order_kernel(const int32_t *__restrict__ feat_ptr, int F,
+                                                              const int32_t *__restrict__ unordered,
+                                                              int32_t *__restrict__ feat_slot) {
+  const int f = blockIdx.x * (FI_THREADS / 64) + (threadIdx.x >> 6);
+  if (f >= F) return;
+  const int lane = threadIdx.x & 63;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  const int len = hi - lo;
+  if (len == 0 || len > 64) return;
+  const int mine = lane < len ? unordered[lo + lane] : 0x7fffffff;
+  int rank = 0;
+  for (int j = 0; j < len; ++j) rank += __shfl(mine, j, 64) < mine;
+  if (lane < len) feat_slot[lo + rank] = mine;
+}
+
+// Segments longer than 64 slots: one workgroup per feature runs a counting sort keyed by
+// token.  A feature occurs at most once per token, so a bitmap over the B tokens plus a
+// prefix popcount gives every slot its rank.  LDS: bitmap[ceil(B/32)] + prefix[ceil(B/32)].
+__global__ __launch_bounds__(FI_THREADS) void fi_order_long_kernel(const int32_t *__restrict__ feat_ptr,
+                                                                   const int32_t *__restrict__ unordered,
+                                                                   const int32_t *__restrict__ slot_tok, int B,
+                                                                   int32_t *__restrict__ feat_slot) {
+  extern __shared__ uint32_t fi_lds[];
+  __shared__ int32_t part[FI_THREADS];
+  const int f = blockIdx.x, tid = threadIdx.x;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  if (hi - lo <= 64) return;
+  const int W = (B + 31) >> 5;
+  uint32_t *bitmap = fi_lds;
+  uint32_t *prefix = fi_lds + W;
+  for (int w = tid; w < W; w += FI_THREADS) bitmap[w] = 0u;
+  __syncthreads();
+  for (int i = lo + tid; i < hi; i += FI_THREADS) {
+    const int t = slot_tok[unordered[i]];
+    atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+  }
+  __syncthreads();
+  const int per = (W + FI_THREADS - 1) / FI_THREADS;
+  const int wlo = tid * per, whi = min(W, wlo + per);
+  int s = 0;
+  for (int w = wlo; w < whi; ++w) s += __popc(bitmap[w]);
+  part[tid] = s;
+  __syncthreads();
+  for (int o = 1; o < FI_THREADS; o <<= 1) {
+    const int v = tid >= o ? part[tid - o] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;
+  for (int w = wlo; w < whi; ++w) {
+    prefix[w] = (uint32_t)run;
+    run += __popc(bitmap[w]);
+  }
+  __syncthreads();
+  for (int i = lo + tid; i < hi; i += FI_THREADS) {
+    const int slot = unordered[i];
+    const int t = slot_tok[slot];
+    const int rank = (int)prefix[t >> 5] + __popc(bitmap[t >> 5] & ((1u << (t & 31)) - 1u));
+    feat_slot[lo + rank] = slot;
+  }
+}
+
+// out[f, :] = sum_{s in segment f} coef[s] * dense[slot_tok[s], :]
+template <bool DENSE_BF16>
+__global__ __launch_bounds__(FI_THREADS) void sparse_grad_rows_kernel(
+    const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
+    const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
+    float *__restrict__ out, float *__restrict__ bias_out, int d) {
+  const int f = blockIdx.x, tid = threadIdx.x;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  const int n_seg = d >> 2;  // float4 segments of the output row
+  const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
+  const char *dbase = reinterpret_cast<const char *>(dense);
+  float *orow = out + (size_t)f * d;
+
+  if (bias_out && tid < 64) {
+    float s = 0.f;
+    for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
+    s = wave_sum(s);
+    if (tid == 0) bias_out[f] = s;
+  }
+  for (int seg0 = tid; seg0 < n_seg; seg0 += FI_THREADS * 4) {
+    float4 acc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = lo; i < hi; ++i) {
+      const int s = feat_slot[i];
+      const float c = coef[s];
+      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int seg = seg0 + u * FI_THREADS;
+        if (seg < n_seg) {
+          float4 x;
+          if constexpr (DENSE_BF16) {
+            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
+            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
+            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
+          } else {
+            x = reinterpret_cast<const float4 *>(row)[seg];
+          }
+          acc[u].x = fmaf(c, x.x, acc[u].x); acc[u].y = fmaf(c, x.y, acc[u].y);
+          acc[u].z = fmaf(c, x.z, acc[u].z); acc[u].w = fmaf(c, x.w, acc[u].w);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int seg = seg0 + u * FI_THREADS;
+      if (seg < n_seg) reinterpret_cast<float4 *>(orow)[seg] = acc[u];
+    }
+  }
+}
+
+}  // namespace sae
+
+extern "C" int64_t sae_feature_index_workspace_bytes(int64_t B, int64_t F, int64_t n_slots) {
+  (void)B;
+  if (F <= 0 || n_slots <= 0) return 0;
+  // counts[F] + cursor[F] + ordering scratch[n_slots]
+  return (int64_t)sizeof(int32_t) * (2 * F + n_slots) + 256;
+}
+
+extern "C" int sae_build_feature_index(const int32_t *idx, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
+                                       int64_t F, int64_t n_slots, int32_t *feat_ptr, int32_t *feat_slot,
+                                       int32_t *slot_tok, void *workspace, int64_t workspace_bytes, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(idx && row_off && row_nnz && feat_ptr && feat_slot && slot_tok, SAE_ERR_INVALID_ARG,
+              "build_feature_index: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && n_slots > 0, SAE_ERR_INVALID_ARG, "build_feature_index: sizes must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) - 1 && n_slots < (1LL << 31), SAE_ERR_UNSUPPORTED,
+              "build_feature_index: size too large for 32-bit slots");
+  SAE_REQUIRE(B <= 131072, SAE_ERR_UNSUPPORTED, "build_feature_index: B=%lld above 131072 tokens per call", (long long)B);
+  SAE_REQUIRE(workspace && workspace_bytes >= sae_feature_index_workspace_bytes(B, F, n_slots), SAE_ERR_WORKSPACE,
+              "build_feature_index: workspace of %lld bytes needed", (long long)sae_feature_index_workspace_bytes(B, F, n_slots));
+  hipStream_t st = (hipStream_t)stream;
+  int32_t *counts = reinterpret_cast<int32_t *>(workspace);
+  int32_t *cursor = counts + F;
+  int32_t *unordered = cursor + F;
+  hipLaunchKernelGGL(fi_zero_kernel, dim3((unsigned)((F + 255) / 256)), dim3(256), 0, st, counts, F);
+  const unsigned tok_blocks = (unsigned)((B + (FI_THREADS / 64) - 1) / (FI_THREADS / 64));
+  hipLaunchKernelGGL(fi_count_kernel, dim3(tok_blocks), dim3(FI_THREADS), 0, st, idx, row_off, row_nnz, (int)B, (int)F,
+                     counts, slot_tok);
+  hipLaunchKernelGGL(fi_scan_kernel, dim3(1), dim3(1024), 0, st, counts, (int)F, feat_ptr, cursor);
+  hipLaunchKernelGGL(fi_fill_kernel, dim3(tok_blocks), dim3(FI_THREADS), 0, st, idx, row_off, row_nnz, (int)B, (int)F,
+                     cursor, unordered);
+  const unsigned feat_blocks = (unsigned)((F + (FI_THREADS / 64) - 1) / (FI_THREADS / 64));
+  hipLaunchKernelGGL(fi_order_kernel, dim3(feat_blocks), dim3(FI_THREADS), 0, st, feat_ptr, (int)F, unordered, feat_slot);
+  const size_t bitmap_lds = (size_t)2 * ((B + 31) / 32) * sizeof(uint32_t);
+  hipLaunchKernelGGL(fi_order_long_kernel, dim3((unsigned)F), dim3(FI_THREADS), bitmap_lds, st, feat_ptr, unordered,
+                     slot_tok, (int)B, feat_slot);
+  return check_launch("build_feature_index");
+}
+
+extern "C" int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                    const float *coef, const void *dense, int dense_dtype, float *out, float *bias_out,
+                                    int64_t F, int64_t d, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && out, SAE_ERR_INVALID_ARG,
+              "sparse_grad_rows: null pointer");
+  SAE_REQUIRE(F > 0 && d > 0, SAE_ERR_INVALID_ARG, "sparse_grad_rows: F and d must be positive");
+  SAE_REQUIRE(dense_dtype == SAE_F32 || dense_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "sparse_grad_rows: bad dtype %d", dense_dtype);
+  SAE_REQUIRE(d % 4 == 0, SAE_ERR_UNSUPPORTED, "sparse_grad_rows: d_model=%lld must be a multiple of 4", (long long)d);
+  SAE_REQUIRE(F < (1LL << 31), SAE_ERR_UNSUPPORTED, "sparse_grad_rows: F too large");
+  hipStream_t st = (hipStream_t)stream;
+  if (dense_dtype == SAE_BF16)
+    hipLaunchKernelGGL(sparse_grad_rows_kernel<true>, dim3((unsigned)F), dim3(FI_THREADS), 0, st, feat_ptr, feat_slot,
+                       slot_tok, coef, dense, out, bias_out, (int)d);
+  else
+    hipLaunchKernelGGL(sparse_grad_rows_kernel<false>, dim3((unsigned)F), dim3(FI_THREADS), 0, st, feat_ptr, feat_slot,
+                       slot_tok, coef, dense, out, bias_out, (int)d);
+  return check_launch("sparse_grad_rows");
+}

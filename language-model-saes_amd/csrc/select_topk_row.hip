@@ -1,0 +1,365 @@
+// Per-token TopK select with fused encoder bias and decoder-norm scale (gfx950).
+//
+// One workgroup of 1024 threads owns one token's row of F pre-activations.  The key of an
+// element is the bit pattern of h1 = (pre + b_enc) * scale when h1 > 0 and 0 otherwise: for
+// positive floats unsigned-integer order equals float order, and non-positive entries can
+// never be kept (the reference applies a relu mask before the top-k).
+//
+// Fast path (two streaming reads of the row, no histogram over the row):
+//   1. every thread takes the maximum key of the elements it owns; the k-th largest of those
+//      1024 maxima is a lower bound L of the k-th largest key of the row, because k distinct
+//      elements are >= L;
+//   2. the row is read again (it sits in L2 now) and every element with key >= L is appended
+//      to a candidate list in LDS -- for i.i.d. data about k + a few elements;
+//   3. an exact radix select over the candidates in LDS yields the threshold key T; among
+//      the candidates with key == T the lowest indices win (a second radix select over the
+//      indices); the kept elements are ranked by index and written in ascending order.
+// General path (any row, any k <= 4096): the same exact select, but with the 8-bit-digit
+// histograms taken over the whole row in global memory.  It is used when the candidate list
+// would overflow (massive ties, k above the thread count) and by the tests, which check both
+// paths against each other.
+#include "common.h"
+
+namespace sae {
+
+constexpr int SEL_THREADS = 1024;
+constexpr int SEL_WAVES = SEL_THREADS / 64;
+constexpr int SEL_CAP = 4096;      // candidate capacity == largest supported k
+constexpr int SEL_MAX_K = 4096;
+
+struct SelShared {
+  uint32_t cand_key[SEL_CAP];
+  int32_t cand_idx[SEL_CAP];
+  uint32_t tmax[SEL_THREADS];
+  uint32_t hist[256];
+  int32_t count;        // candidates appended
+  uint32_t prefix;      // radix-select state
+  int32_t remaining;
+  int32_t digit_found;
+};
+
+__device__ __forceinline__ uint32_t key_of(float pre, float b, float s) {
+  const float h1 = (pre + b) * s;
+  return h1 > 0.f ? __float_as_uint(h1) : 0u;
+}
+
+// Scan hist[255..0] from the top and find the bin where the running count reaches
+// `remaining`.  Executed by wave 0; results go to sh->prefix / sh->remaining.
+__device__ __forceinline__ void pick_digit(SelShared *sh, int shift) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    // lane 0 owns the top four bins (255..252), lane 63 the bottom four
+    const int top = 255 - 4 * lane;
+    const uint32_t h0 = sh->hist[top], h1 = sh->hist[top - 1], h2 = sh->hist[top - 2], h3 = sh->hist[top - 3];
+    const int local = (int)(h0 + h1 + h2 + h3);
+    int incl = local;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    const int excl = incl - local;
+    const int remaining = sh->remaining;
+    if (excl < remaining && incl >= remaining) {
+      int need = remaining - excl;  // still to take inside my four bins
+      int bin;
+      if ((int)h0 >= need) bin = top;
+      else if ((int)(h0 + h1) >= need) { bin = top - 1; need -= (int)h0; }
+      else if ((int)(h0 + h1 + h2) >= need) { bin = top - 2; need -= (int)(h0 + h1); }
+      else { bin = top - 3; need -= (int)(h0 + h1 + h2); }
+      sh->prefix |= ((uint32_t)bin) << shift;
+      sh->remaining = need;
+      sh->digit_found = 1;
+    }
+  }
+}
+
+// Exact k-th largest of `n` keys held in LDS (n >= k >= 1).  On return (after the final
+// barrier) sh->prefix is that key and sh->remaining the number of elements equal to it that
+// belong to the top k.  `xform` maps a stored key to the ordering key.
+template <typename KeyAt>
+__device__ __forceinline__ void lds_kth_largest(SelShared *sh, int n, int k, KeyAt key_at) {
+  if (threadIdx.x == 0) { sh->prefix = 0u; sh->remaining = k; }
+  uint32_t mask = 0u;
+#pragma unroll 1
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (threadIdx.x < 256) sh->hist[threadIdx.x] = 0u;
+    __syncthreads();
+    const uint32_t prefix = sh->prefix;
+    for (int i = threadIdx.x; i < n; i += SEL_THREADS) {
+      const uint32_t key = key_at(i);
+      if ((key & mask) == prefix) atomicAdd(&sh->hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    pick_digit(sh, shift);
+    mask |= 255u << shift;
+    __syncthreads();
+  }
+}
+
+template <bool BF16>
+struct RowReader {
+  const void *row;
+  const float *b_enc;
+  const float *scale;
+  int F;
+  // calls fn(index, key) for every element of the row, vectorised when the row allows it
+  template <typename Fn>
+  __device__ __forceinline__ void for_each(Fn fn) const {
+    constexpr int V = BF16 ? 8 : 4;  // elements per 16-byte load
+    const bool vec_ok = (F % V == 0) && ((((uintptr_t)row) & 15) == 0);
+    if (vec_ok) {
+      const int n_chunks = F / V;
+      for (int c = threadIdx.x; c < n_chunks; c += SEL_THREADS) {
+        const u32x4 raw = reinterpret_cast<const u32x4 *>(row)[c];
+        float pre[V];
+        if constexpr (BF16) {
+          const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            pre[2 * q] = __uint_as_float(w[q] << 16);
+            pre[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u);
+          }
+        } else {
+          pre[0] = __uint_as_float(raw.x); pre[1] = __uint_as_float(raw.y);
+          pre[2] = __uint_as_float(raw.z); pre[3] = __uint_as_float(raw.w);
+        }
+        const int base = c * V;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const float b = b_enc ? b_enc[base + e] : 0.f;
+          const float s = scale ? scale[base + e] : 1.f;
+          fn(base + e, key_of(pre[e], b, s));
+        }
+      }
+    } else {
+      for (int i = threadIdx.x; i < F; i += SEL_THREADS) {
+        float pre;
+        if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
+        else pre = reinterpret_cast<const float *>(row)[i];
+        fn(i, key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f));
+      }
+    }
+  }
+};
+
+// Exact k-th largest over the whole row in global memory (general path).
+template <bool BF16>
+__device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<BF16> &rr, int k) {
+  if (threadIdx.x == 0) { sh->prefix = 0u; sh->remaining = k; }
+  uint32_t mask = 0u;
+#pragma unroll 1
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (threadIdx.x < 256) sh->hist[threadIdx.x] = 0u;
+    __syncthreads();
+    const uint32_t prefix = sh->prefix;
+    rr.for_each([&](int, uint32_t key) {
+      if (key != 0u && (key & mask) == prefix) atomicAdd(&sh->hist[(key >> shift) & 255u], 1u);
+    });
+    __syncthreads();
+    pick_digit(sh, shift);
+    mask |= 255u << shift;
+    __syncthreads();
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale, int F, int k,
+    int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
+    int32_t *__restrict__ row_nnz, int cand_cap) {
+  __shared__ SelShared sh;
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  RowReader<BF16> rr;
+  rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
+  rr.b_enc = b_enc;
+  rr.scale = scale;
+  rr.F = F;
+
+  // ---- pass 1: per-thread maximum key and number of positive elements ----
+  uint32_t my_max = 0u;
+  int my_pos = 0;
+  rr.for_each([&](int, uint32_t key) {
+    my_max = key > my_max ? key : my_max;
+    my_pos += key != 0u;
+  });
+  sh.tmax[tid] = my_max;
+  if (tid == 0) sh.count = 0;
+  // total positives in the row
+  int pos = wave_sum_i(my_pos);
+  __syncthreads();
+  if ((tid & 63) == 0) sh.hist[tid >> 6] = (uint32_t)pos;
+  __syncthreads();
+  int n_pos = 0;
+#pragma unroll
+  for (int w = 0; w < SEL_WAVES; ++w) n_pos += (int)sh.hist[w];
+  __syncthreads();
+
+  const int k_eff = n_pos < k ? n_pos : k;  // how many elements will be kept
+  bool general = false;
+  uint32_t T = 0u;       // threshold key: keep key > T and `need` lowest-index elements with key == T
+  int need = 0;
+  int n_cand = 0;
+
+  if (k_eff == 0) {
+    if (tid == 0) { row_off[b] = (int64_t)b * k; row_nnz[b] = 0; }
+    for (int i = tid; i < k; i += SEL_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
+    return;
+  }
+
+  if (n_pos <= k) {
+    // fewer positives than k: everything positive is kept
+    if (n_pos > cand_cap) general = true;  // cannot happen for k <= cand_cap; kept for safety
+    T = 0u; need = 0;
+  } else if (k <= SEL_THREADS) {
+    // ---- lower bound L from the per-thread maxima ----
+    lds_kth_largest(&sh, SEL_THREADS, k, [&](int i) { return sh.tmax[i]; });
+    T = sh.prefix;  // = L for now (may be 0 when fewer than k threads saw a positive)
+    __syncthreads();
+  } else {
+    general = true;
+  }
+
+  if (!general) {
+    // ---- pass 2: gather candidates with key >= L (and key > 0) into LDS ----
+    const uint32_t L = (n_pos <= k) ? 1u : (T == 0u ? 1u : T);
+    rr.for_each([&](int i, uint32_t key) {
+      if (key >= L) {
+        const int slot = atomicAdd(&sh.count, 1);
+        if (slot < cand_cap) { sh.cand_key[slot] = key; sh.cand_idx[slot] = i; }
+      }
+    });
+    __syncthreads();
+    n_cand = sh.count;
+    if (n_cand > cand_cap) general = true;
+  }
+
+  if (general) {
+    // ---- general path: exact threshold over the whole row ----
+    __syncthreads();
+    row_kth_largest<BF16>(&sh, rr, k_eff);
+    T = sh.prefix;
+    need = sh.remaining;  // elements equal to T that are kept
+    __syncthreads();
+    // lowest `need` indices among the ties: radix select over ~idx restricted to key == T.
+    // Count ties first; if all ties are kept no index threshold is needed.
+    if (tid == 0) sh.count = 0;
+    __syncthreads();
+    int my_ties = 0;
+    rr.for_each([&](int, uint32_t key) { my_ties += key == T; });
+    my_ties = wave_sum_i(my_ties);
+    if ((tid & 63) == 0 && my_ties) atomicAdd(&sh.count, my_ties);
+    __syncthreads();
+    const int n_ties = sh.count;
+    uint32_t idx_limit = 0xffffffffu;  // keep ties with idx <= idx_limit
+    __syncthreads();
+    if (n_ties > need) {
+      if (tid == 0) { sh.prefix = 0u; sh.remaining = need; }
+      uint32_t mask = 0u;
+#pragma unroll 1
+      for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) sh.hist[tid] = 0u;
+        __syncthreads();
+        const uint32_t prefix = sh.prefix;
+        rr.for_each([&](int i, uint32_t key) {
+          const uint32_t ik = ~(uint32_t)i;
+          if (key == T && (ik & mask) == prefix) atomicAdd(&sh.hist[(ik >> shift) & 255u], 1u);
+        });
+        __syncthreads();
+        pick_digit(&sh, shift);
+        mask |= 255u << shift;
+        __syncthreads();
+      }
+      idx_limit = ~sh.prefix;
+      __syncthreads();
+    }
+    // emit the kept elements into the candidate arrays (exactly k_eff of them)
+    if (tid == 0) sh.count = 0;
+    __syncthreads();
+    rr.for_each([&](int i, uint32_t key) {
+      if (key > T || (key == T && key != 0u && (uint32_t)i <= idx_limit)) {
+        const int slot = atomicAdd(&sh.count, 1);
+        if (slot < SEL_CAP) { sh.cand_key[slot] = key; sh.cand_idx[slot] = i; }
+      }
+    });
+    __syncthreads();
+    n_cand = sh.count < SEL_CAP ? sh.count : SEL_CAP;  // == k_eff
+  } else if (n_cand > k_eff) {
+    // ---- exact threshold among the candidates ----
+    lds_kth_largest(&sh, n_cand, k_eff, [&](int i) { return sh.cand_key[i]; });
+    T = sh.prefix;
+    need = sh.remaining;
+    __syncthreads();
+    // ties: keep the `need` lowest indices among candidates with key == T
+    int my_ties = 0;
+    for (int i = tid; i < n_cand; i += SEL_THREADS) my_ties += sh.cand_key[i] == T;
+    if (tid == 0) sh.count = 0;
+    __syncthreads();
+    my_ties = wave_sum_i(my_ties);
+    if ((tid & 63) == 0 && my_ties) atomicAdd(&sh.count, my_ties);
+    __syncthreads();
+    const int n_ties = sh.count;
+    __syncthreads();
+    uint32_t idx_limit = 0xffffffffu;
+    if (n_ties > need) {
+      lds_kth_largest(&sh, n_cand, need, [&](int i) { return sh.cand_key[i] == T ? ~(uint32_t)sh.cand_idx[i] : 0u; });
+      idx_limit = ~sh.prefix;
+      __syncthreads();
+    }
+    // mark dropped candidates by clearing their key
+    for (int i = tid; i < n_cand; i += SEL_THREADS) {
+      const uint32_t key = sh.cand_key[i];
+      const bool keep = key > T || (key == T && (uint32_t)sh.cand_idx[i] <= idx_limit);
+      if (!keep) sh.cand_key[i] = 0u;
+    }
+    __syncthreads();
+  }
+
+  // ---- rank the kept candidates by index and write them out in ascending order ----
+  for (int i = tid; i < n_cand; i += SEL_THREADS) {
+    const uint32_t key = sh.cand_key[i];
+    if (key == 0u) continue;
+    const int my_idx = sh.cand_idx[i];
+    int rank = 0;
+    for (int j = 0; j < n_cand; ++j) rank += (sh.cand_key[j] != 0u) && (sh.cand_idx[j] < my_idx);
+    const float h1 = __uint_as_float(key);
+    const float s = scale ? scale[my_idx] : 1.f;
+    if (rank < k) {
+      idx_out[(size_t)b * k + rank] = my_idx;
+      val_out[(size_t)b * k + rank] = scale ? h1 / s : h1;
+    }
+  }
+  for (int i = k_eff + tid; i < k; i += SEL_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
+  if (tid == 0) { row_off[b] = (int64_t)b * k; row_nnz[b] = k_eff; }
+}
+
+}  // namespace sae
+
+extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale, int64_t B,
+                                      int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
+                                      int cand_cap, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0, SAE_ERR_INVALID_ARG, "select_topk_row: B and F must be positive");
+  SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_row: bad dtype %d", pre_dtype);
+  SAE_REQUIRE(k >= 1 && k <= SEL_MAX_K, SAE_ERR_UNSUPPORTED, "select_topk_row: k=%d outside [1, %d]", k, SEL_MAX_K);
+  SAE_REQUIRE(F < (1LL << 31) && B < (1LL << 31), SAE_ERR_UNSUPPORTED, "select_topk_row: size too large");
+  SAE_REQUIRE(cand_cap >= 0 && cand_cap <= SEL_CAP, SAE_ERR_INVALID_ARG, "select_topk_row: cand_cap outside [0, %d]", SEL_CAP);
+  const int kk = k > F ? (int)F : k;
+  (void)kk;
+  hipStream_t st = (hipStream_t)stream;
+  if (pre_dtype == SAE_BF16)
+    hipLaunchKernelGGL(select_topk_row_kernel<true>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,
+                       (int)F, k, idx, val, row_off, row_nnz, cand_cap);
+  else
+    hipLaunchKernelGGL(select_topk_row_kernel<false>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,
+                       (int)F, k, idx, val, row_off, row_nnz, cand_cap);
+  return check_launch("select_topk_row");
+}
+
+extern "C" int sae_select_topk_row(const void *pre, int pre_dtype, const float *b_enc, const float *scale, int64_t B,
+                                   int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
+                                   void *stream) {
+  return sae_select_topk_row_ex(pre, pre_dtype, b_enc, scale, B, F, k, idx, val, row_off, row_nnz, sae::SEL_CAP, stream);
+}

@@ -1,0 +1,295 @@
+"""Tensor-level wrappers over the C ABI: validate, allocate outputs, pass raw pointers.
+
+Every function launches on torch's current stream of the tensors' device and returns without
+synchronising.  torch is used for device memory and streams only.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import SAE_BF16, SAE_F32, check
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return SAE_F32
+    if t.dtype == torch.bfloat16:
+        return SAE_BF16
+    raise TypeError(f"unsupported dtype {t.dtype} (float32 or bfloat16 expected)")
+
+
+def _req(t: torch.Tensor, name: str, dtype=None, ndim=None):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); the HIP path has no CPU fallback")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if ndim is not None and t.ndim != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+
+
+@dataclass
+class SparseCode:
+    """Feature activations in sparse form (see include/sae_hip.h, "Sparse code")."""
+
+    idx: torch.Tensor       # int32 [n_slots]
+    val: torch.Tensor       # fp32  [n_slots]
+    row_off: torch.Tensor   # int64 [B]
+    row_nnz: torch.Tensor   # int32 [B]
+    n_tokens: int
+    d_sae: int
+
+    @property
+    def n_slots(self) -> int:
+        return self.idx.numel()
+
+    def to_dense(self) -> torch.Tensor:
+        """[B, F] fp32 tensor with the code scattered in (unused slots carry 0 at index 0)."""
+        B, F = self.n_tokens, self.d_sae
+        out = torch.zeros(B, F, dtype=torch.float32, device=self.val.device)
+        slots = torch.arange(self.n_slots, device=self.val.device)
+        tok = torch.searchsorted(self.row_off, slots, right=True) - 1
+        valid = (slots - self.row_off[tok]) < self.row_nnz[tok]
+        out.index_put_((tok[valid], self.idx[valid].long()), self.val[valid], accumulate=True)
+        return out
+
+
+@dataclass
+class FeatureIndex:
+    feat_ptr: torch.Tensor   # int32 [F + 1]
+    feat_slot: torch.Tensor  # int32 [n_slots]
+    slot_tok: torch.Tensor   # int32 [n_slots]
+
+
+# ---- element-wise ---------------------------------------------------------------------------
+
+def cast_bf16(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _req(src, "src", torch.float32)
+    if out is None:
+        out = torch.empty(src.shape, dtype=torch.bfloat16, device=src.device)
+    check(_lib.load().sae_cast_f32_to_bf16(src.data_ptr(), out.data_ptr(), src.numel(), _stream(src)), "cast_f32_to_bf16")
+    return out
+
+
+def row_norm(w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _req(w, "w", torch.float32, 2)
+    F, d = w.shape
+    if out is None:
+        out = torch.empty(F, dtype=torch.float32, device=w.device)
+    check(_lib.load().sae_row_norm(w.data_ptr(), out.data_ptr(), F, d, _stream(w)), "row_norm")
+    return out
+
+
+def transpose(src: torch.Tensor) -> torch.Tensor:
+    _req(src, "src", torch.float32, 2)
+    r, c = src.shape
+    out = torch.empty(c, r, dtype=torch.float32, device=src.device)
+    check(_lib.load().sae_transpose_f32(src.data_ptr(), out.data_ptr(), r, c, _stream(src)), "transpose_f32")
+    return out
+
+
+def col_sum(src: torch.Tensor, out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    _req(src, "src", torch.float32, 2)
+    B, n = src.shape
+    lib = _lib.load()
+    if out is None:
+        out = torch.empty(n, dtype=torch.float32, device=src.device)
+        accumulate = False
+    ws_bytes = lib.sae_col_sum_workspace_bytes(B, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=src.device)
+    check(lib.sae_col_sum(src.data_ptr(), out.data_ptr(), B, n, int(accumulate), ws.data_ptr(), ws_bytes, _stream(src)), "col_sum")
+    return out
+
+
+# ---- encoder --------------------------------------------------------------------------------
+
+def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """pre[B, F] = x[B, d] @ w_enc_t[F, d]^T."""
+    _req(x, "x", ndim=2)
+    _req(w_enc_t, "w_enc_t", ndim=2)
+    if x.dtype != w_enc_t.dtype:
+        raise TypeError(f"x ({x.dtype}) and w_enc_t ({w_enc_t.dtype}) must share a dtype")
+    B, d = x.shape
+    F, d2 = w_enc_t.shape
+    if d != d2:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
+    pre = torch.empty(B, F, dtype=out_dtype, device=x.device)
+    check(
+        _lib.load().sae_encoder_gemm(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _dt(x), _dt(pre), _stream(x)),
+        "encoder_gemm",
+    )
+    return pre
+
+
+# ---- select ---------------------------------------------------------------------------------
+
+def select_topk_row(
+    pre: torch.Tensor,
+    b_enc: Optional[torch.Tensor],
+    scale: Optional[torch.Tensor],
+    k: int,
+    cand_cap: Optional[int] = None,
+) -> SparseCode:
+    _req(pre, "pre", ndim=2)
+    B, F = pre.shape
+    for name, t in (("b_enc", b_enc), ("scale", scale)):
+        if t is not None:
+            _req(t, name, torch.float32, 1)
+            if t.numel() != F:
+                raise ValueError(f"{name} must have {F} elements")
+    k = int(k)
+    dev = pre.device
+    idx = torch.empty(B * k, dtype=torch.int32, device=dev)
+    val = torch.empty(B * k, dtype=torch.float32, device=dev)
+    row_off = torch.empty(B, dtype=torch.int64, device=dev)
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    if cand_cap is None:
+        rc = lib.sae_select_topk_row(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
+                                     val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+    else:
+        rc = lib.sae_select_topk_row_ex(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
+                                        val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), int(cand_cap), _stream(pre))
+    check(rc, "select_topk_row")
+    return SparseCode(idx, val, row_off, row_nnz, B, F)
+
+
+# ---- sparse decoder -------------------------------------------------------------------------
+
+def _check_code(code: SparseCode, w_dec: torch.Tensor):
+    _req(code.idx, "idx", torch.int32, 1)
+    _req(code.val, "val", torch.float32, 1)
+    _req(code.row_off, "row_off", torch.int64, 1)
+    _req(code.row_nnz, "row_nnz", torch.int32, 1)
+    _req(w_dec, "w_dec", ndim=2)
+    if w_dec.shape[0] != code.d_sae:
+        raise ValueError(f"w_dec has {w_dec.shape[0]} rows, the code addresses {code.d_sae} features")
+
+
+def sparse_decode_fwd(code: SparseCode, w_dec: torch.Tensor, b_dec: Optional[torch.Tensor]) -> torch.Tensor:
+    _check_code(code, w_dec)
+    F, d = w_dec.shape
+    B = code.n_tokens
+    if b_dec is not None:
+        _req(b_dec, "b_dec", torch.float32, 1)
+    recon = torch.empty(B, d, dtype=torch.float32, device=w_dec.device)
+    check(
+        _lib.load().sae_sparse_decode_fwd(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                          code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
+                                          recon.data_ptr(), B, d, F, _stream(w_dec)),
+        "sparse_decode_fwd",
+    )
+    return recon
+
+
+def sparse_decode_bwd_dval(code: SparseCode, grad_recon: torch.Tensor, w_dec: torch.Tensor) -> torch.Tensor:
+    _check_code(code, w_dec)
+    _req(grad_recon, "grad_recon", torch.float32, 2)
+    F, d = w_dec.shape
+    B = code.n_tokens
+    dval = torch.empty(code.n_slots, dtype=torch.float32, device=w_dec.device)
+    check(
+        _lib.load().sae_sparse_decode_bwd_dval(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(),
+                                               grad_recon.data_ptr(), w_dec.data_ptr(), _dt(w_dec), dval.data_ptr(),
+                                               B, d, F, code.n_slots, _stream(w_dec)),
+        "sparse_decode_bwd_dval",
+    )
+    return dval
+
+
+def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Optional[torch.Tensor], label: torch.Tensor,
+                            tok_w: Optional[torch.Tensor], want_recon: bool = True):
+    """Returns (recon or None, loss_tok [B], grad_recon [B, d], dval [n_slots])."""
+    _check_code(code, w_dec)
+    _req(label, "label", torch.float32, 2)
+    F, d = w_dec.shape
+    B = code.n_tokens
+    if tuple(label.shape) != (B, d):
+        raise ValueError(f"label must be {(B, d)}, got {tuple(label.shape)}")
+    if tok_w is not None:
+        _req(tok_w, "tok_w", torch.float32, 1)
+    dev = w_dec.device
+    recon = torch.empty(B, d, dtype=torch.float32, device=dev) if want_recon else None
+    loss_tok = torch.empty(B, dtype=torch.float32, device=dev)
+    grad_recon = torch.empty(B, d, dtype=torch.float32, device=dev)
+    dval = torch.empty(code.n_slots, dtype=torch.float32, device=dev)
+    check(
+        _lib.load().sae_sparse_decode_mse_fused(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                                code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
+                                                label.data_ptr(), _ptr(tok_w), _ptr(recon), loss_tok.data_ptr(),
+                                                grad_recon.data_ptr(), dval.data_ptr(), B, d, F, code.n_slots,
+                                                _stream(w_dec)),
+        "sparse_decode_mse_fused",
+    )
+    return recon, loss_tok, grad_recon, dval
+
+
+# ---- sparse backward ------------------------------------------------------------------------
+
+def build_feature_index(code: SparseCode) -> FeatureIndex:
+    dev = code.idx.device
+    B, F, n = code.n_tokens, code.d_sae, code.n_slots
+    lib = _lib.load()
+    ws_bytes = lib.sae_feature_index_workspace_bytes(B, F, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    feat_ptr = torch.empty(F + 1, dtype=torch.int32, device=dev)
+    feat_slot = torch.empty(n, dtype=torch.int32, device=dev)
+    slot_tok = torch.zeros(n, dtype=torch.int32, device=dev)
+    check(
+        lib.sae_build_feature_index(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(), B, F, n,
+                                    feat_ptr.data_ptr(), feat_slot.data_ptr(), slot_tok.data_ptr(), ws.data_ptr(),
+                                    ws_bytes, _stream(code.idx)),
+        "build_feature_index",
+    )
+    return FeatureIndex(feat_ptr, feat_slot, slot_tok)
+
+
+def sparse_grad_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, F: int, want_bias: bool = False,
+                     out: Optional[torch.Tensor] = None):
+    """out[f, :] = sum over feature f's slots of coef[slot] * dense[token(slot), :]; optional bias_out[f] = sum coef."""
+    _req(coef, "coef", torch.float32, 1)
+    _req(dense, "dense", ndim=2)
+    d = dense.shape[1]
+    dev = dense.device
+    if out is None:
+        out = torch.empty(F, d, dtype=torch.float32, device=dev)
+    bias = torch.empty(F, dtype=torch.float32, device=dev) if want_bias else None
+    check(
+        _lib.load().sae_sparse_grad_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
+                                         coef.data_ptr(), dense.data_ptr(), _dt(dense), out.data_ptr(), _ptr(bias), F, d,
+                                         _stream(dense)),
+        "sparse_grad_rows",
+    )
+    return out, bias
+
+
+# ---- optimiser ------------------------------------------------------------------------------
+
+def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, *, lr: float, beta1: float,
+              beta2: float, eps: float, step: int, shadow_bf16: Optional[torch.Tensor] = None,
+              row_norm_out: Optional[torch.Tensor] = None, row_len: int = 0) -> None:
+    for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
+        _req(t, name, torch.float32)
+        if t.numel() != p.numel():
+            raise ValueError(f"{name} must have {p.numel()} elements")
+    if shadow_bf16 is not None:
+        _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
+    check(
+        _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
+                                  eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _stream(p)),
+        "adam_step",
+    )

@@ -1,0 +1,344 @@
+"""Kernel-level parity of the HIP path (through the C ABI) against the CPU oracle.
+
+Tolerances (relative to the largest magnitude of the expected tensor):
+  fp32 path 1e-5, bf16 path 2e-2; indices bit-exact.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def code_to_rows(code):
+    """list of (idx list, val list) per token from a SparseCode on any device"""
+    idx, val = code.idx.cpu().numpy(), code.val.cpu().numpy()
+    off, nnz = code.row_off.cpu().numpy(), code.row_nnz.cpu().numpy()
+    return [(idx[o:o + n], val[o:o + n]) for o, n in zip(off, nnz)]
+
+
+# ---------------------------------------------------------------------------------------------
+# encoder GEMM
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (64, 768, 6144), (1, 64, 8), (513, 256, 260)])
+def test_encoder_gemm_fp32(pkg, dev, B, d, F):
+    print(f"gemm fp32 B={B} d={d} F={F}", flush=True)
+    g = torch.Generator().manual_seed(B * 7 + F)
+    x = torch.randn(B, d, generator=g)
+    w = torch.randn(F, d, generator=g) / d ** 0.5
+    pre = pkg.ops.encoder_gemm(x.to(dev), w.to(dev), torch.float32)
+    want = x.double() @ w.double().t()
+    assert rel_err(pre, want) < FP32_TOL
+
+
+@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (512, 2048, 4096), (33, 64, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_encoder_gemm_bf16(pkg, dev, B, d, F, out_dtype):
+    print(f"gemm bf16 B={B} d={d} F={F} out={out_dtype}", flush=True)
+    g = torch.Generator().manual_seed(B * 11 + F)
+    x = torch.randn(B, d, generator=g).bfloat16()
+    w = (torch.randn(F, d, generator=g) / d ** 0.5).bfloat16()
+    pre = pkg.ops.encoder_gemm(x.to(dev), w.to(dev), out_dtype)
+    want = x.double() @ w.double().t()  # exact products of the bf16 operands
+    if out_dtype == torch.float32:
+        assert rel_err(pre, want) < FP32_TOL
+    else:
+        # one bf16 rounding of the fp32 accumulator: bit-exact against rounding the fp64 result,
+        # except where fp32 accumulation noise straddles a rounding boundary (<= 1 bf16 ulp)
+        want_bf = want.float().bfloat16()
+        diff = (pre.cpu().float() - want_bf.float()).abs()
+        ulp = want_bf.float().abs() * 2 ** -7
+        assert (diff <= ulp + 1e-30).all()
+        assert (diff == 0).float().mean() > 0.99
+
+
+def test_encoder_gemm_rejects_bad_shapes(pkg, dev):
+    x = torch.randn(8, 48, device=dev)
+    w = torch.randn(16, 48, device=dev)
+    with pytest.raises(RuntimeError, match="multiple of"):
+        pkg.ops.encoder_gemm(x, w, torch.float32)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        pkg.ops.encoder_gemm(x.cpu(), w.cpu(), torch.float32)
+
+
+# ---------------------------------------------------------------------------------------------
+# TopK select
+# ---------------------------------------------------------------------------------------------
+
+def oracle_topk_code(oracle, pre, b_enc, scale, k):
+    """(idx, val) per row by the oracle's rule: relu mask, k largest, ties -> lowest index."""
+    h0 = pre.float() + (b_enc if b_enc is not None else 0.0)
+    h1 = h0 * scale if scale is not None else h0
+    r = h1 * h1.gt(0).to(h1.dtype)
+    a = oracle.topk(r, k=k, dim=-1)
+    f = a / scale if scale is not None else a
+    rows = []
+    for b in range(pre.shape[0]):
+        nz = torch.nonzero(a[b] > 0).flatten()
+        rows.append((nz.numpy().astype(np.int32), f[b, nz].numpy()))
+    return rows
+
+
+def check_select(pkg, oracle, dev, pre, b_enc, scale, k, cand_cap=None):
+    code = pkg.ops.select_topk_row(
+        pre.to(dev), None if b_enc is None else b_enc.to(dev), None if scale is None else scale.to(dev), k, cand_cap
+    )
+    got = code_to_rows(code)
+    want = oracle_topk_code(oracle, pre, b_enc, scale, k)
+    assert code.row_off.cpu().tolist() == [b * k for b in range(pre.shape[0])]
+    for b, ((gi, gv), (wi, wv)) in enumerate(zip(got, want)):
+        assert np.array_equal(gi, wi), f"row {b}: indices differ\n got {gi}\nwant {wi}"
+        assert np.array_equal(gv, wv), f"row {b}: values differ"
+    # unused slots are zero-filled
+    idx = code.idx.view(-1, k).cpu()
+    val = code.val.view(-1, k).cpu()
+    pad = torch.arange(k)[None, :] >= code.row_nnz.cpu()[:, None]
+    assert (val[pad] == 0).all() and (idx[pad] == 0).all()
+    return code
+
+
+@pytest.mark.parametrize("B,F,k", [(7, 1000, 5), (16, 4096, 32), (4, 131072, 64), (3, 37, 37), (5, 2048, 512)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_select_topk_row_random(pkg, oracle, dev, B, F, k, dtype):
+    print(f"select B={B} F={F} k={k} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(F + k)
+    pre = torch.randn(B, F, generator=g).to(dtype)
+    b_enc = 0.1 * torch.randn(F, generator=g)
+    scale = 0.5 + torch.rand(F, generator=g)
+    check_select(pkg, oracle, dev, pre, b_enc, scale, k)
+    check_select(pkg, oracle, dev, pre, None, None, k)
+
+
+@pytest.mark.parametrize("cand_cap", [0, 8, 4096])
+def test_select_topk_row_paths_agree(pkg, oracle, dev, cand_cap):
+    """fast path (candidate list) and general path (row histograms) give the same code"""
+    g = torch.Generator().manual_seed(5)
+    pre = torch.randn(9, 5000, generator=g)
+    check_select(pkg, oracle, dev, pre, None, None, 40, cand_cap)
+
+
+def test_select_topk_row_reference_kat(pkg, oracle, dev):
+    """tests/unit/test_sae.py:92-113 of the reference: TopK(k=2)"""
+    pre = torch.tensor([[1.0, 1.5, 3.0, 4.0], [4.0, 3.0, 1.5, 1.0]])
+    code = check_select(pkg, oracle, dev, pre, None, None, 2)
+    dense = code.to_dense().cpu()
+    assert torch.equal(dense, torch.tensor([[0.0, 0.0, 3.0, 4.0], [4.0, 3.0, 0.0, 0.0]]))
+
+
+@pytest.mark.parametrize("cand_cap", [None, 0])
+def test_select_topk_row_ties_and_degenerate_rows(pkg, oracle, dev, cand_cap):
+    F, k = 3000, 16
+    rows = []
+    rows.append(torch.full((F,), 2.0))                      # all equal: lowest k indices win
+    rows.append(torch.zeros(F))                             # nothing positive
+    rows.append(-torch.ones(F))                             # all negative
+    r = torch.zeros(F); r[[5, 77, 2999]] = torch.tensor([1.0, 3.0, 2.0]); rows.append(r)  # fewer than k positives
+    r = torch.ones(F); r[100:110] = 5.0; rows.append(r)     # 10 clear winners + 6 of a 2990-way tie
+    g = torch.Generator().manual_seed(3)
+    r = torch.randint(0, 4, (F,), generator=g).float(); rows.append(r)  # heavy ties on a few levels
+    r = torch.randn(F, generator=g).bfloat16().float(); rows.append(r)  # bf16-quantised values
+    pre = torch.stack(rows)
+    code = check_select(pkg, oracle, dev, pre, None, None, k, cand_cap)
+    assert code.row_nnz.cpu().tolist()[:4] == [k, 0, 0, 3]
+    assert code.idx.view(-1, k)[0].cpu().tolist() == list(range(k))
+
+
+def test_select_topk_row_matches_torch_topk_when_tie_free(pkg, dev):
+    g = torch.Generator().manual_seed(11)
+    pre = torch.randn(32, 8192, generator=g)
+    k = 50
+    code = pkg.ops.select_topk_row(pre.to(dev), None, None, k)
+    want = torch.topk(pre * (pre > 0), k, dim=-1).indices.sort(dim=-1).values
+    assert torch.equal(code.idx.view(-1, k).cpu().long(), want)
+
+
+# ---------------------------------------------------------------------------------------------
+# sparse decode, fused loss, d val
+# ---------------------------------------------------------------------------------------------
+
+def random_code(pkg, dev, B, F, k, seed, ragged=True):
+    g = torch.Generator().manual_seed(seed)
+    pre = torch.randn(B, F, generator=g)
+    if ragged:
+        pre[0] = -1.0                 # an empty token
+        pre[1, 3:] = -1.0             # a token with at most 3 active features
+    return pkg.ops.select_topk_row(pre.to(dev), None, None, k)
+
+
+@pytest.mark.parametrize("B,d,F,k", [(10, 64, 512, 8), (33, 768, 2048, 32), (6, 4096, 1024, 64), (4, 8, 16, 3), (5, 16384, 64, 4)])
+@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
+def test_sparse_decode_fwd(pkg, dev, B, d, F, k, w_dtype):
+    print(f"decode B={B} d={d} F={F} k={k} {w_dtype}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=d + k)
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(F, d, generator=g) / d ** 0.5).to(w_dtype)
+    b_dec = torch.randn(d, generator=g)
+    recon = pkg.ops.sparse_decode_fwd(code, w.to(dev), b_dec.to(dev))
+    want = code.to_dense().cpu().double() @ w.double() + b_dec.double()
+    assert rel_err(recon, want) < FP32_TOL
+    recon_nb = pkg.ops.sparse_decode_fwd(code, w.to(dev), None)
+    assert rel_err(recon_nb, want - b_dec.double()) < FP32_TOL
+
+
+@pytest.mark.parametrize("B,d,F,k", [(10, 64, 512, 8), (33, 768, 2048, 32), (6, 4096, 1024, 64)])
+@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("masked", [False, True])
+def test_sparse_decode_mse_fused(pkg, dev, B, d, F, k, w_dtype, masked):
+    print(f"fused B={B} d={d} F={F} k={k} {w_dtype} masked={masked}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=d + 3 * k)
+    g = torch.Generator().manual_seed(2)
+    w = (torch.randn(F, d, generator=g) / d ** 0.5).to(w_dtype)
+    b_dec = torch.randn(d, generator=g)
+    label = torch.randn(B, d, generator=g)
+    if masked:
+        mask = (torch.rand(B, generator=g) > 0.3).float()
+        tok_w = mask / mask.sum()
+    else:
+        tok_w = torch.full((B,), 1.0 / B)
+    recon, loss_tok, grad_recon, dval = pkg.ops.sparse_decode_mse_fused(
+        code, w.to(dev), b_dec.to(dev), label.to(dev), tok_w.to(dev)
+    )
+    # autograd of the dense restatement in fp64
+    fa = code.to_dense().cpu().double().requires_grad_(True)
+    wd = w.double()
+    rec = fa @ wd + b_dec.double()
+    rec.retain_grad()
+    loss = (((rec - label.double()) ** 2).sum(-1) * tok_w.double()).sum()
+    loss.backward()
+    assert rel_err(recon, rec) < FP32_TOL
+    assert abs(loss_tok.sum().item() - loss.item()) / loss.item() < FP32_TOL
+    assert rel_err(grad_recon, rec.grad) < FP32_TOL
+    # d val against the dense gradient gathered at the code's slots
+    rows = code_to_rows(code)
+    dv = dval.cpu().numpy()
+    off = code.row_off.cpu().numpy()
+    scale = fa.grad.abs().max().item()
+    for b, (ri, _) in enumerate(rows):
+        want = fa.grad[b, torch.as_tensor(ri, dtype=torch.long)].numpy()
+        got = dv[off[b]: off[b] + len(ri)]
+        assert np.abs(got - want).max() <= FP32_TOL * scale + 1e-30
+        assert (dv[off[b] + len(ri): off[b] + k] == 0).all()
+    # the stand-alone backward kernel agrees with the fused one
+    dval2 = pkg.ops.sparse_decode_bwd_dval(code, grad_recon, w.to(dev))
+    assert rel_err(dval2, dval) < 1e-6
+
+
+# ---------------------------------------------------------------------------------------------
+# feature index and gradient rows
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("B,F,k", [(50, 64, 8), (300, 1000, 16), (1024, 512, 32), (7, 10000, 3)])
+def test_build_feature_index(pkg, dev, B, F, k):
+    print(f"feature index B={B} F={F} k={k}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=B + F)
+    fi = pkg.ops.build_feature_index(code)
+    idx = code.idx.cpu().numpy()
+    off, nnz = code.row_off.cpu().numpy(), code.row_nnz.cpu().numpy()
+    slots = np.concatenate([np.arange(o, o + n) for o, n in zip(off, nnz)]).astype(np.int64)
+    feats = idx[slots]
+    order = np.argsort(feats, kind="stable")          # ascending feature, then ascending slot
+    want_slots = slots[order].astype(np.int32)
+    want_ptr = np.concatenate([[0], np.cumsum(np.bincount(feats, minlength=F))]).astype(np.int32)
+    assert np.array_equal(fi.feat_ptr.cpu().numpy(), want_ptr)
+    n_valid = int(nnz.sum())
+    assert np.array_equal(fi.feat_slot.cpu().numpy()[:n_valid], want_slots)
+    tok = np.repeat(np.arange(B), nnz).astype(np.int32)
+    assert np.array_equal(fi.slot_tok.cpu().numpy()[slots], tok)
+
+
+def test_build_feature_index_long_segments(pkg, dev):
+    """a feature active on every token exercises the bitmap ordering of long segments"""
+    B, F, k = 700, 256, 4
+    g = torch.Generator().manual_seed(0)
+    pre = torch.randn(B, F, generator=g)
+    pre[:, 17] = 10.0
+    pre[::2, 200] = 9.0
+    code = pkg.ops.select_topk_row(pre.to(dev), None, None, k)
+    fi = pkg.ops.build_feature_index(code)
+    ptr = fi.feat_ptr.cpu().numpy()
+    seg = fi.feat_slot.cpu().numpy()[ptr[17]:ptr[18]]
+    assert len(seg) == B and np.all(np.diff(seg) > 0)
+    seg = fi.feat_slot.cpu().numpy()[ptr[200]:ptr[201]]
+    assert len(seg) == B // 2 and np.all(np.diff(seg) > 0)
+
+
+@pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (128, 4096, 512, 4)])
+@pytest.mark.parametrize("dense_dtype", [torch.float32, torch.bfloat16])
+def test_sparse_grad_rows(pkg, dev, B, d, F, k, dense_dtype):
+    print(f"grad rows B={B} d={d} F={F} k={k} {dense_dtype}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=d + B)
+    fi = pkg.ops.build_feature_index(code)
+    g = torch.Generator().manual_seed(4)
+    dense = torch.randn(B, d, generator=g).to(dense_dtype)
+    coef = torch.randn(code.n_slots, generator=g)
+    out, bias = pkg.ops.sparse_grad_rows(fi, coef.to(dev), dense.to(dev), F, want_bias=True)
+    # dense restatement: C[b, f] = coef at the valid slots; out = C^T @ dense
+    import dataclasses
+    c_code = dataclasses.replace(code, val=coef.to(dev))
+    C = c_code.to_dense().cpu().double()
+    want = C.t() @ dense.double()
+    assert rel_err(out, want) < FP32_TOL
+    assert rel_err(bias, C.sum(0)) < FP32_TOL
+    # reproducible: the atomics only decide an order that is then canonicalised
+    fi2 = pkg.ops.build_feature_index(code)
+    out2, _ = pkg.ops.sparse_grad_rows(fi2, coef.to(dev), dense.to(dev), F)
+    assert torch.equal(out, out2)
+
+
+# ---------------------------------------------------------------------------------------------
+# element-wise helpers and Adam
+# ---------------------------------------------------------------------------------------------
+
+def test_cast_rownorm_transpose_colsum(pkg, dev):
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(301, 520, generator=g)
+    assert torch.equal(pkg.ops.cast_bf16(a.to(dev)).cpu(), a.bfloat16())
+    assert rel_err(pkg.ops.row_norm(a.to(dev)), a.double().norm(dim=1)) < 1e-6
+    assert torch.equal(pkg.ops.transpose(a.to(dev)).cpu(), a.t().contiguous())
+    assert rel_err(pkg.ops.col_sum(a.to(dev)), a.double().sum(0)) < 1e-6
+    b = torch.randn(77, 13, generator=g)  # odd sizes: scalar tails
+    assert torch.equal(pkg.ops.cast_bf16(b.to(dev)).cpu(), b.bfloat16())
+    assert rel_err(pkg.ops.row_norm(b.to(dev)), b.double().norm(dim=1)) < 1e-6
+
+
+def test_row_norm_reference_fixture(pkg, dev):
+    """decoder norms of the reference's test fixture (tests/unit/test_sae.py:31-55): closed forms"""
+    W_D = torch.tensor([[1.0, 5.0], [2.0, 6.0], [3.0, 7.0], [4.0, 8.0]])
+    want = torch.tensor([26.0, 40.0, 58.0, 80.0]).sqrt()
+    assert torch.allclose(pkg.ops.row_norm(W_D.to(dev)).cpu(), want, rtol=1e-6)
+
+
+@pytest.mark.parametrize("n,row_len", [(1000, 0), (4096 * 3, 4096), (77, 0), (64 * 128, 128)])
+def test_adam_step_matches_torch(pkg, dev, n, row_len):
+    g = torch.Generator().manual_seed(n)
+    p0 = torch.randn(n, generator=g)
+    ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.Adam([ref], lr=4e-4, betas=(0.9, 0.999))
+    p = p0.clone().to(dev)
+    m = torch.zeros(n, device=dev)
+    v = torch.zeros(n, device=dev)
+    shadow = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    norms = torch.empty(n // row_len, device=dev) if row_len else None
+    for step in range(1, 4):
+        grad = torch.randn(n, generator=g) * (torch.rand(n, generator=g) > 0.5)  # exact zeros included
+        ref.grad = grad.clone()
+        opt.step()
+        pkg.ops.adam_step(p, grad.to(dev), m, v, lr=4e-4, beta1=0.9, beta2=0.999, eps=1e-8, step=step,
+                          shadow_bf16=shadow, row_norm_out=norms, row_len=row_len)
+        # both sides round p to fp32 after an lr-sized move: allow a few ulps of |p|
+        assert (p.cpu() - ref.detach()).abs().max() <= 4 * 1.2e-7 * p0.abs().max()
+        assert torch.equal(shadow.cpu(), p.cpu().bfloat16())
+        if row_len:
+            assert rel_err(norms, p.cpu().view(-1, row_len).double().norm(dim=1)) < 1e-6
+    st = opt.state[ref]
+    assert rel_err(m, st["exp_avg"]) < 1e-6 and rel_err(v, st["exp_avg_sq"]) < 1e-6
