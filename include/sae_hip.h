@@ -175,8 +175,8 @@ int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, cons
  * shadow_bf16 (nullable) receives bf16(p) for the next step's GEMM / gather operands.
  * row_norm_out (nullable, requires row_len > 0 and n % row_len == 0) receives the L2 norm
  * of every updated row of length row_len, i.e. the next step's decoder_norm(). */
-int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
-                  float beta2, float eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
+                  double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                   int64_t row_len, void *stream);
 
 #ifdef __cplusplus

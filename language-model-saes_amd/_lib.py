@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_double, c_int, c_int64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsae_hip.so")
@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libsae_hip.so")
 SAE_F32, SAE_BF16 = 0, 1
 
 # name -> (restype, argtypes); mirrors include/sae_hip.h declaration by declaration
-_P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
+_P, _I, _L, _F = c_void_p, c_int, c_int64, c_double
 SIGNATURES = {
     "sae_abi_version": (_I, []),
     "sae_last_error": (c_char_p, []),

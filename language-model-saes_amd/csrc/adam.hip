@@ -83,8 +83,8 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
 
 }  // namespace sae
 
-extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, float lr, float beta1,
-                             float beta2, float eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
+                             double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                              int64_t row_len, void *stream) {
   using namespace sae;
   SAE_REQUIRE(p && g && m && v, SAE_ERR_INVALID_ARG, "adam_step: null pointer");
@@ -92,14 +92,15 @@ extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64
   SAE_REQUIRE((((uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v) & 15) == 0, SAE_ERR_INVALID_ARG,
               "adam_step: 16-byte alignment required");
   AdamScalars a;
-  a.beta1 = beta1; a.beta2 = beta2;
-  a.one_minus_beta1 = 1.f - beta1;
-  a.one_minus_beta2 = 1.f - beta2;
-  const double bc1 = 1.0 - pow((double)beta1, (double)step);
-  const double bc2 = 1.0 - pow((double)beta2, (double)step);
-  a.step_size = (float)((double)lr / bc1);
+  // scalars are formed in double on the host, as the Python optimiser does, then narrowed once
+  a.beta1 = (float)beta1; a.beta2 = (float)beta2;
+  a.one_minus_beta1 = (float)(1.0 - beta1);
+  a.one_minus_beta2 = (float)(1.0 - beta2);
+  const double bc1 = 1.0 - pow(beta1, (double)step);
+  const double bc2 = 1.0 - pow(beta2, (double)step);
+  a.step_size = (float)(lr / bc1);
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(bc2));
-  a.eps = eps;
+  a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
   if (row_norm_out) {
     SAE_REQUIRE(row_len > 0 && row_len % 4 == 0 && n % row_len == 0 && row_len < (1LL << 31), SAE_ERR_INVALID_ARG,

@@ -58,7 +58,8 @@ def test_encoder_gemm_bf16(pkg, dev, B, d, F, out_dtype):
         want_bf = want.float().bfloat16()
         diff = (pre.cpu().float() - want_bf.float()).abs()
         ulp = want_bf.float().abs() * 2 ** -7
-        assert (diff <= ulp + 1e-30).all()
+        # (+ an absolute floor: near-zero sums keep the fp32 accumulation noise of O(1) terms)
+        assert (diff <= ulp + 1e-5 * want.abs().max().item()).all()
         assert (diff == 0).float().mean() > 0.99
 
 
@@ -226,7 +227,7 @@ def test_sparse_decode_mse_fused(pkg, dev, B, d, F, k, w_dtype, masked):
     for b, (ri, _) in enumerate(rows):
         want = fa.grad[b, torch.as_tensor(ri, dtype=torch.long)].numpy()
         got = dv[off[b]: off[b] + len(ri)]
-        assert np.abs(got - want).max() <= FP32_TOL * scale + 1e-30
+        assert len(ri) == 0 or np.abs(got - want).max() <= FP32_TOL * scale + 1e-30
         assert (dv[off[b] + len(ri): off[b] + k] == 0).all()
     # the stand-alone backward kernel agrees with the fused one
     dval2 = pkg.ops.sparse_decode_bwd_dval(code, grad_recon, w.to(dev))
@@ -269,7 +270,7 @@ def test_build_feature_index_long_segments(pkg, dev):
     seg = fi.feat_slot.cpu().numpy()[ptr[17]:ptr[18]]
     assert len(seg) == B and np.all(np.diff(seg) > 0)
     seg = fi.feat_slot.cpu().numpy()[ptr[200]:ptr[201]]
-    assert len(seg) == B // 2 and np.all(np.diff(seg) > 0)
+    assert len(seg) >= B // 2 and np.all(np.diff(seg) > 0)  # odd tokens may pick it by chance
 
 
 @pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (128, 4096, 512, 4)])
