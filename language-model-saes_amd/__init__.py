@@ -8,3 +8,11 @@ from . import _lib, ops  # noqa: F401
 from .ops import FeatureIndex, SparseCode  # noqa: F401
 
 __all__ = ["_lib", "ops", "SparseCode", "FeatureIndex"]
+
+from .config import SAEConfig, SparseDictionaryConfig  # noqa: E402,F401
+from .activation_functions import JumpReLU  # noqa: E402,F401
+from .sparse_dictionary import SparseDictionary  # noqa: E402,F401
+from .sae import SparseAutoEncoder  # noqa: E402,F401
+from .optim import HipAdam  # noqa: E402,F401
+
+__all__ += ["SAEConfig", "SparseDictionaryConfig", "JumpReLU", "SparseDictionary", "SparseAutoEncoder", "HipAdam"]

@@ -1,0 +1,318 @@
+"""SparseAutoEncoder on the HIP path.
+
+API of the reference's vanilla SAE / transcoder (src/llamascopium/models/sae.py:52-448):
+parameters `W_E [d, F]`, `b_E [F]`, `W_D [F, d]`, `b_D [d]` (plus the optional GLU pair), methods
+`encode`, `decode`, `forward`, `compute_loss`, the norm helpers and `init_parameters`.
+
+Memory layout: `W_E` has the reference's shape [d_model, d_sae] but is stored feature-major
+(strides (1, d_model), i.e. a transposed view of a contiguous [d_sae, d_model] buffer).  One
+feature's encoder vector is then contiguous, like its decoder vector, which is what the GEMM
+(K-contiguous operands), the sparse gradient rows and the fused optimiser want.
+
+`compute_loss` takes the fused kernel path when the configuration allows it (TopK activation,
+reconstruction loss only, no user hooks, 2-D activations on the GPU); every other configuration
+runs the reference's op sequence over dense tensors with the select kernel behind the activation.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any, Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .config import SAEConfig, register_sae_model
+from .hooks import HookPoint
+from .sparse_dictionary import LazyDict, SparseDictionary
+
+
+def _autocast_dtype(device_type: str) -> Optional[torch.dtype]:
+    if torch.is_autocast_enabled(device_type):
+        return torch.get_autocast_dtype(device_type)
+    return None
+
+
+class _Holder:
+    """Side outputs of the fused step that are not autograd tensors."""
+
+    code: ops.SparseCode = None
+    pre: torch.Tensor = None
+    scale: Optional[torch.Tensor] = None
+
+
+class _FusedTopKLoss(torch.autograd.Function):
+    """encode -> TopK -> decode -> masked-mean squared error, forward and backward, in kernels.
+
+    forward : GEMM, select (bias + norm scale fused), decode + loss + grad_recon + d val (fused)
+    backward: feature index, dW_D / dW_E^T rows, db_E, db_D; no dense [B, F] tensor is formed.
+    The decoder-norm scale enters as act(h * n) / n; its two derivative terms with respect to n
+    cancel analytically, so no gradient flows to W_D through n.
+    """
+
+    @staticmethod
+    def forward(ctx, x, label, tok_w, W_E, b_E, W_D, b_D, w_enc_op, w_dec_op, scale, k, holder):
+        amp = w_enc_op.dtype == torch.bfloat16
+        if amp:
+            x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
+            pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)
+        else:
+            x_op = x.contiguous()
+            pre = ops.encoder_gemm(x_op, w_enc_op, torch.float32)
+        code = ops.select_topk_row(pre, b_E, scale, k)
+        recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, b_D, label, tok_w)
+        loss = loss_tok.sum()
+        holder.code, holder.pre, holder.scale = code, pre, scale
+        ctx.code, ctx.x_op, ctx.grad_recon, ctx.dval = code, x_op, grad_recon, dval
+        ctx.w_enc_op, ctx.w_dec_op = w_enc_op, w_dec_op
+        ctx.has_b_D = b_D is not None
+        ctx.mark_non_differentiable(recon)
+        return loss, recon
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_recon):
+        code = ctx.code
+        F = code.d_sae
+        fi = ops.build_feature_index(code)
+        g = g_loss.to(torch.float32)
+        coef_dec = code.val * g          # dW_D[f] = sum val * grad_recon[token]
+        coef_enc = ctx.dval * g          # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
+        dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_recon, F)
+        dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_op, F, want_bias=True)
+        db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            import dataclasses
+            dx = ops.sparse_decode_fwd(dataclasses.replace(code, val=coef_enc), ctx.w_enc_op, None)
+        dlabel = -ctx.grad_recon * g if ctx.needs_input_grad[1] else None
+        return dx, dlabel, None, dW_Et.t(), db_E, dW_D, db_D, None, None, None, None, None
+
+
+@register_sae_model("sae")
+class SparseAutoEncoder(SparseDictionary):
+    def __init__(self, cfg: SAEConfig, device_mesh=None):
+        super().__init__(cfg, device_mesh=device_mesh)
+        self.cfg = cfg
+        d, F = cfg.d_model, cfg.d_sae
+        kw = dict(device=cfg.device, dtype=cfg.dtype)
+        self.W_E = nn.Parameter(torch.empty(F, d, **kw).t())       # shape [d, F], feature-major storage
+        self.b_E = nn.Parameter(torch.empty(F, **kw))
+        self.W_D = nn.Parameter(torch.empty(F, d, **kw))
+        if cfg.use_decoder_bias:
+            self.b_D = nn.Parameter(torch.empty(d, **kw))
+        if cfg.use_glu_encoder:
+            self.W_E_glu = nn.Parameter(torch.empty(F, d, **kw).t())
+            self.b_E_glu = nn.Parameter(torch.empty(F, **kw))
+        self.hook_hidden_pre = HookPoint()
+        self.hook_feature_acts = HookPoint()
+        self.hook_reconstructed = HookPoint()
+        # derived operands (bf16 shadows, row norms) keyed by name -> (param version, tensor)
+        self._derived: dict[str, tuple[int, torch.Tensor]] = {}
+
+    # ---- derived operands, refreshed when the parameter's version counter moves ----
+    def _derive(self, name: str, param: torch.Tensor, make) -> torch.Tensor:
+        ver = param._version
+        hit = self._derived.get(name)
+        if hit is not None and hit[0] == ver and hit[1].device == param.device:
+            return hit[1]
+        with torch.no_grad():
+            t = make(hit[1] if hit is not None and hit[1].device == param.device else None)
+        self._derived[name] = (ver, t)
+        return t
+
+    def set_derived(self, name: str, param: torch.Tensor, tensor: torch.Tensor) -> None:
+        """Called by the fused optimiser after it wrote a fresh shadow / norm itself."""
+        self._derived[name] = (param._version, tensor)
+
+    def get_derived_buffer(self, name: str) -> Optional[torch.Tensor]:
+        hit = self._derived.get(name)
+        return None if hit is None else hit[1]
+
+    def w_enc_t(self) -> torch.Tensor:
+        """Contiguous [F, d] view of the encoder weight."""
+        w = self.W_E.t()
+        return w if w.is_contiguous() else w.contiguous()
+
+    def _w_enc_operand(self, amp: bool) -> torch.Tensor:
+        wt = self.w_enc_t().detach()
+        if not amp or wt.dtype == torch.bfloat16:
+            return wt
+        return self._derive("W_E.bf16", self.W_E, lambda old: ops.cast_bf16(wt, old))
+
+    def _w_dec_operand(self, amp: bool) -> torch.Tensor:
+        w = self.W_D.detach()
+        if not amp or w.dtype == torch.bfloat16:
+            return w
+        return self._derive("W_D.bf16", self.W_D, lambda old: ops.cast_bf16(w, old))
+
+    def _decoder_norm_nograd(self) -> torch.Tensor:
+        return self._derive("W_D.norm", self.W_D, lambda old: ops.row_norm(self.W_D.detach().float(), old))
+
+    # ---- norms (models/sae.py:136-188, 209-212) ----
+    def encoder_norm(self, keepdim: bool = False):
+        return torch.norm(self.W_E, p=2, dim=0, keepdim=keepdim)
+
+    def decoder_norm(self, keepdim: bool = False) -> torch.Tensor:
+        return torch.norm(self.W_D, p=2, dim=1, keepdim=keepdim)
+
+    def decoder_bias_norm(self) -> torch.Tensor:
+        if not self.cfg.use_decoder_bias:
+            raise ValueError("Decoder bias is not used")
+        return torch.norm(self.b_D, p=2, dim=0, keepdim=True)
+
+    @torch.no_grad()
+    def set_decoder_to_fixed_norm(self, value: float, force_exact: bool):
+        if force_exact:
+            self.W_D.mul_(value / self.decoder_norm(keepdim=True))
+        else:
+            self.W_D.mul_(value / torch.clamp(self.decoder_norm(keepdim=True), min=value))
+
+    @torch.no_grad()
+    def set_encoder_to_fixed_norm(self, value: float):
+        self.W_E.mul_(value / self.encoder_norm(keepdim=True))
+
+    @torch.no_grad()
+    def transform_to_unit_decoder_norm(self):
+        self.W_D.mul_(1 / self.decoder_norm(keepdim=True))
+
+    @torch.no_grad()
+    def standardize_parameters_of_dataset_norm(self):
+        """models/sae.py:214-255: fold the dataset-wise norms into the weights, switch to "inference"."""
+        assert self.cfg.norm_activation == "dataset-wise"
+        assert self.dataset_average_activation_norm is not None
+        fin = math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_point_in]
+        fout = math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_point_out]
+        self.b_E.div_(fin)
+        if self.cfg.use_decoder_bias:
+            self.b_D.div_(fout)
+        self.W_D.mul_(fin / fout)
+        self.cfg.norm_activation = "inference"
+
+    @torch.no_grad()
+    def init_encoder_with_decoder_transpose(self, factor: float = 1.0):
+        self.W_E.copy_(self.W_D.t() * factor)
+
+    @torch.no_grad()
+    def init_parameters(self, **kwargs):
+        """models/sae.py:400-436: uniform encoder/decoder, zero biases."""
+        super().init_parameters(**kwargs)
+        eb, db = kwargs["encoder_uniform_bound"], kwargs["decoder_uniform_bound"]
+        self.W_E.uniform_(-eb, eb)
+        self.W_D.uniform_(-db, db)
+        self.b_E.zero_()
+        if self.cfg.use_decoder_bias:
+            self.b_D.zero_()
+        if self.cfg.use_glu_encoder:
+            self.W_E_glu.uniform_(-eb, eb)
+            self.b_E_glu.zero_()
+
+    # ---- API path over dense tensors (models/sae.py:288-377) ----
+    def _matmul_enc(self, x: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
+        return x @ W
+
+    def encode(self, x: torch.Tensor, return_hidden_pre: bool = False, **kwargs):
+        x = x.to(self.W_E.dtype)
+        hidden_pre = self._matmul_enc(x, self.W_E) + self.b_E
+        if self.cfg.use_glu_encoder:
+            hidden_pre = hidden_pre * torch.sigmoid(self._matmul_enc(x, self.W_E_glu) + self.b_E_glu)
+        hidden_pre = self.hook_hidden_pre(hidden_pre)
+        if self.cfg.sparsity_include_decoder_norm:
+            hidden_pre = hidden_pre * self.decoder_norm()
+        feature_acts = self.activation_function(hidden_pre)
+        if self.cfg.sparsity_include_decoder_norm:
+            feature_acts = feature_acts / self.decoder_norm()
+            hidden_pre = hidden_pre / self.decoder_norm()
+        if return_hidden_pre:
+            return self.hook_feature_acts(feature_acts), hidden_pre
+        return self.hook_feature_acts(feature_acts)
+
+    def decode(self, feature_acts, **kwargs):
+        if isinstance(feature_acts, ops.SparseCode):
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            reconstructed = ops.sparse_decode_fwd(feature_acts, self._w_dec_operand(amp),
+                                                  self.b_D.detach() if self.cfg.use_decoder_bias else None)
+            return self.hook_reconstructed(reconstructed)
+        reconstructed = feature_acts @ self.W_D
+        if self.cfg.use_decoder_bias:
+            reconstructed = reconstructed + self.b_D
+        return self.hook_reconstructed(reconstructed)
+
+    @torch.no_grad()
+    def encode_sparse(self, x: torch.Tensor) -> ops.SparseCode:
+        """Inference-time encode that stays sparse: GEMM + select, no dense [B, F] output."""
+        assert self.cfg.act_fn.lower() == "topk", "encode_sparse covers the TopK activation"
+        assert not self.cfg.use_glu_encoder, "encode_sparse does not cover the GLU encoder"
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        w = self._w_enc_operand(amp)
+        xo = ops.cast_bf16(x2.float()) if w.dtype == torch.bfloat16 and x2.dtype != torch.bfloat16 else x2.to(w.dtype)
+        pre = ops.encoder_gemm(xo, w, torch.bfloat16 if amp else torch.float32)
+        scale = self._decoder_norm_nograd() if self.cfg.sparsity_include_decoder_norm else None
+        return ops.select_topk_row(pre, self.b_E.detach().float(), scale, self.current_k)
+
+    def prepare_input(self, batch: dict[str, torch.Tensor], **kwargs):
+        return batch[self.cfg.hook_point_in], {}, {}
+
+    def prepare_label(self, batch: dict[str, torch.Tensor], **kwargs):
+        return batch[self.cfg.hook_point_out]
+
+    # ---- fused train-step loss ----
+    def _fused_eligible(self, x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
+        return (
+            self.cfg.act_fn.lower() == "topk"
+            and x.is_cuda and x.ndim == 2 and label.ndim == 2
+            and not self.cfg.use_glu_encoder
+            and sparsity_loss_type is None and not (lp_coefficient > 0.0) and not (auxk_coefficient > 0.0)
+            and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
+            and self.W_E.dtype == torch.float32
+        )
+
+    def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,
+                     frequency_scale: float = 0.01, p: int = 1, l1_coefficient: float = 1.0,
+                     lp_coefficient: float = 0.0, auxk_coefficient: float = 0.0, k_aux: int = 512,
+                     update_dead_statistics=None, return_aux_data: bool = True, **kwargs):
+        x, _, _ = self.prepare_input(batch)
+        label = self.prepare_label(batch, **kwargs)
+        if not self._fused_eligible(x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient):
+            return super().compute_loss(
+                batch, sparsity_loss_type=sparsity_loss_type, tanh_stretch_coefficient=tanh_stretch_coefficient,
+                frequency_scale=frequency_scale, p=p, l1_coefficient=l1_coefficient, lp_coefficient=lp_coefficient,
+                auxk_coefficient=auxk_coefficient, k_aux=k_aux, update_dead_statistics=update_dead_statistics,
+                return_aux_data=return_aux_data, **kwargs)
+
+        mask = batch.get("mask")
+        B = x.shape[0]
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        if mask is None:
+            tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=x.device)
+        else:
+            m = mask.to(torch.float32)
+            tok_w = m / m.sum()
+        scale = self._decoder_norm_nograd() if self.cfg.sparsity_include_decoder_norm else None
+        holder = _Holder()
+        loss, recon = _FusedTopKLoss.apply(
+            x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x,
+            label.to(torch.float32).contiguous(), tok_w, self.W_E, self.b_E, self.W_D,
+            self.b_D if self.cfg.use_decoder_bias else None,
+            self._w_enc_operand(amp), self._w_dec_operand(amp), scale, int(self.current_k), holder)
+        if not return_aux_data:
+            return loss
+
+        code, pre, b_E = holder.code, holder.pre, self.b_E.detach()
+
+        def dense_hidden_pre():
+            h0 = pre.float() + b_E
+            return (h0 * scale) / scale if scale is not None else h0
+
+        eager = {
+            "loss": loss, "l_rec": loss, "l_s": None, "l_p": None, "l_aux": None, "label": label, "mask": mask,
+            "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
+            "auxk_coefficient": auxk_coefficient, "sparse_code": code,
+        }
+        lazy = {
+            "n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
+            "feature_acts": code.to_dense,
+            "hidden_pre": dense_hidden_pre,
+        }
+        return LazyDict(eager, lazy)

@@ -1,0 +1,280 @@
+"""Base class of the sparse-dictionary models on the HIP path.
+
+Mirrors the public surface of the reference's `SparseDictionary`
+(src/llamascopium/models/sparse_dictionary.py:217-1127) for the parts that sit on the train
+step: `encode` / `decode` / `forward` / `compute_loss`, activation normalisation, the activation
+callable stored at `self.activation_function`, `set_current_k`, `get_parameters`, and the
+state-dict key names.  Checkpoint I/O to hubs, DTensor sharding and database hooks are not part
+of this path.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any, Callable, Optional
+
+import torch
+from torch import nn
+
+from .activation_functions import JumpReLU, batch_topk_dense, topk_dense
+from .config import SAE_TYPE_TO_MODEL_CLASS, SparseDictionaryConfig
+
+
+def apply_token_mask(t: torch.Tensor, n_token_dims: int, mask: Optional[torch.Tensor], reduction: str = "sum"):
+    """Reduce the leading token dims (batch[, context]) of `t`, optionally weighted by a 0/1 mask.
+    Same results as utils/tensor_specs.py:64-84."""
+    dims = tuple(range(n_token_dims))
+    if mask is None:
+        if not dims:
+            return t
+        return t.sum(dim=dims) if reduction == "sum" else t.mean(dim=dims)
+    assert tuple(mask.shape) == tuple(t.shape[:n_token_dims]), (
+        f"Mask has shape {tuple(mask.shape)}, but input tensor has token part of shape {tuple(t.shape[:n_token_dims])}"
+    )
+    m = mask.to(t).reshape(*mask.shape, *([1] * (t.ndim - n_token_dims)))
+    out = (t * m).sum(dim=dims)
+    return out / mask.sum() if reduction == "mean" else out
+
+
+class LazyDict(dict):
+    """dict whose listed entries are computed on first access (dense [B, F] views of the sparse
+    code are only materialised for callers that actually read them)."""
+
+    _PENDING = object()
+
+    def __init__(self, eager: dict, lazy: dict[str, Callable[[], Any]]):
+        super().__init__(eager)
+        self._lazy = dict(lazy)
+        for k in lazy:
+            dict.__setitem__(self, k, LazyDict._PENDING)
+
+    def _resolve(self, k):
+        v = dict.__getitem__(self, k)
+        if v is LazyDict._PENDING:
+            v = self._lazy.pop(k)()
+            dict.__setitem__(self, k, v)
+        return v
+
+    def __getitem__(self, k):
+        return self._resolve(k)
+
+    def get(self, k, default=None):
+        return self._resolve(k) if k in self else default
+
+    def items(self):
+        return [(k, self._resolve(k)) for k in self.keys()]
+
+    def values(self):
+        return [self._resolve(k) for k in self.keys()]
+
+
+class SparseDictionary(nn.Module):
+    def __init__(self, cfg: SparseDictionaryConfig, device_mesh=None):
+        super().__init__()
+        if device_mesh is not None:
+            raise NotImplementedError("single-GPU build: device meshes are not supported")
+        self.cfg = cfg
+        self.current_k = cfg.top_k
+        self.dataset_average_activation_norm: dict[str, float] | None = None
+        self.device_mesh = None
+        self.activation_function = self.activation_function_factory(None)
+
+    # ---- small state setters (sparse_dictionary.py:248-260) ----
+    @torch.no_grad()
+    def set_dataset_average_activation_norm(self, dataset_average_activation_norm: dict[str, float]):
+        self.dataset_average_activation_norm = dataset_average_activation_norm
+
+    @torch.no_grad()
+    def set_current_k(self, current_k: int):
+        self.current_k = current_k
+
+    # ---- activation factory (sparse_dictionary.py:713-796) ----
+    def activation_function_factory(self, device_mesh=None):
+        act = self.cfg.act_fn.lower()
+        assert act in ["relu", "topk", "jumprelu", "batchtopk"], f"Not implemented activation function {self.cfg.act_fn}"
+        if act == "relu":
+            return lambda x: x * x.gt(0).to(x.dtype)
+        if act == "jumprelu":
+            return JumpReLU(self.cfg.jumprelu_threshold_window, shape=(self.cfg.d_sae,), device=self.cfg.device,
+                            dtype=self.cfg.dtype)
+        if act == "topk":
+            def topk_activation(x: torch.Tensor):
+                if x.is_cuda:
+                    return topk_dense(x, self.current_k)
+                raise RuntimeError("the TopK activation runs on the GPU only (no CPU fallback in this build)")
+            return topk_activation
+
+        def batch_topk(x: torch.Tensor):
+            shape = None
+            if x.ndim == 3:
+                shape = (x.size(0), x.size(1))
+                x = x.flatten(end_dim=1)
+            out = batch_topk_dense(x, self.current_k * x.size(0))
+            return out.unflatten(0, shape) if shape is not None else out
+        return batch_topk
+
+    @torch.no_grad()
+    def init_parameters(self, **kwargs):
+        if self.cfg.act_fn.lower() == "jumprelu":
+            self.activation_function.log_jumprelu_threshold.data.fill_(kwargs["init_log_jumprelu_threshold_value"])
+
+    # ---- activation normalisation (sparse_dictionary.py:427-499) ----
+    def compute_norm_factor(self, x: torch.Tensor, hook_point: str) -> torch.Tensor:
+        mode = self.cfg.norm_activation
+        assert mode in ["token-wise", "batch-wise", "dataset-wise", "inference"], f"Not implemented norm_activation {mode}"
+        if mode == "token-wise":
+            return math.sqrt(self.cfg.d_model) / torch.norm(x, 2, dim=-1, keepdim=True)
+        if mode == "batch-wise":
+            return math.sqrt(self.cfg.d_model) / torch.norm(x, 2, dim=-1, keepdim=True).mean(dim=-2, keepdim=True)
+        if mode == "dataset-wise":
+            assert self.dataset_average_activation_norm is not None, (
+                "dataset_average_activation_norm must be provided from Initializer"
+            )
+            return torch.tensor(math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[hook_point],
+                                device=x.device, dtype=x.dtype)
+        return torch.tensor(1.0, device=x.device, dtype=x.dtype)
+
+    def normalize_activations(self, batch: dict[str, torch.Tensor], *, return_scale_factor: bool = False):
+        hooks = self.cfg.associated_hook_points
+        scale = {k: self.compute_norm_factor(v, hook_point=k) for k, v in batch.items() if k in hooks}
+        out = {k: (v * scale[k] if k in scale else v) for k, v in batch.items()}
+        return (out, scale) if return_scale_factor else out
+
+    def denormalize_activations(self, batch, scale_factors):
+        return {k: v / scale_factors[k] for k, v in batch.items()}
+
+    # ---- optimiser groups (sparse_dictionary.py:501-510) ----
+    def get_parameters(self) -> list[dict[str, Any]]:
+        jr = list(self.activation_function.parameters()) if isinstance(self.activation_function, JumpReLU) else []
+        others = [p for p in self.parameters() if not any(p is q for q in jr)]
+        return [{"params": others, "name": "others"}, {"params": jr, "name": "jumprelu"}]
+
+    # ---- state dict with the reference's extra scalars (sparse_dictionary.py:262-278, 512-523) ----
+    @torch.no_grad()
+    def full_state_dict(self) -> dict[str, torch.Tensor]:
+        sd = {k: v.contiguous() for k, v in self.state_dict().items()}
+        for hp in self.cfg.associated_hook_points:
+            if self.dataset_average_activation_norm is not None:
+                sd[f"dataset_average_activation_norm.{hp}"] = torch.tensor(
+                    self.dataset_average_activation_norm[hp], device=self.cfg.device, dtype=self.cfg.dtype)
+            else:
+                sd[f"dataset_average_activation_norm.{hp}"] = torch.empty((), device=self.cfg.device, dtype=self.cfg.dtype)
+        return sd
+
+    def load_full_state_dict(self, state_dict: dict[str, torch.Tensor], strict: bool = True) -> None:
+        norm_keys = [k for k in state_dict if k.startswith("dataset_average_activation_norm.")]
+        if norm_keys:
+            self.set_dataset_average_activation_norm({k.split(".", 1)[1]: state_dict[k].item() for k in norm_keys})
+            state_dict = {k: v for k, v in state_dict.items() if k not in norm_keys}
+        self.load_state_dict(state_dict, strict=strict)
+
+    @classmethod
+    def from_config(cls, cfg: SparseDictionaryConfig, device_mesh=None):
+        if cls is SparseDictionary:
+            cls = SAE_TYPE_TO_MODEL_CLASS[cfg.sae_type]
+        return cls(cfg, device_mesh)
+
+    # ---- to be provided by subclasses ----
+    def encode(self, x, return_hidden_pre: bool = False, **kwargs):
+        raise NotImplementedError
+
+    def decode(self, feature_acts, **kwargs):
+        raise NotImplementedError
+
+    def prepare_input(self, batch, **kwargs):
+        raise NotImplementedError
+
+    def prepare_label(self, batch, **kwargs):
+        raise NotImplementedError
+
+    def forward(self, x, encoder_kwargs: dict = {}, decoder_kwargs: dict = {}):
+        return self.decode(self.encode(x, **encoder_kwargs), **decoder_kwargs)
+
+    # ---- generic loss: the reference's op sequence (sparse_dictionary.py:840-1007) over dense
+    # tensors.  Subclasses route the configurations their fused kernels cover away from it. ----
+    def compute_loss(
+        self,
+        batch: dict[str, torch.Tensor],
+        label: Optional[torch.Tensor] = None,
+        *,
+        sparsity_loss_type: Optional[str] = None,
+        tanh_stretch_coefficient: float = 4.0,
+        frequency_scale: float = 0.01,
+        p: int = 1,
+        l1_coefficient: float = 1.0,
+        lp_coefficient: float = 0.0,
+        auxk_coefficient: float = 0.0,
+        k_aux: int = 512,
+        update_dead_statistics=None,
+        return_aux_data: bool = True,
+        **kwargs,
+    ):
+        x, enc_kw, dec_kw = self.prepare_input(batch)
+        label = self.prepare_label(batch, **kwargs)
+        mask = batch.get("mask")
+        feature_acts, hidden_pre = self.encode(x, return_hidden_pre=True, **enc_kw)
+        reconstructed = self.decode(feature_acts, **dec_kw)
+        ntd = label.ndim - 1
+
+        l_rec = apply_token_mask((reconstructed - label).pow(2).sum(dim=-1), ntd, mask, "mean")
+        loss_dict: dict[str, Optional[torch.Tensor]] = {"l_rec": l_rec}
+        loss = l_rec
+
+        if sparsity_loss_type is not None:
+            n = self.decoder_norm()
+            if sparsity_loss_type == "power":
+                l_s = torch.norm(feature_acts * n, p=p, dim=-1)
+            elif sparsity_loss_type == "tanh":
+                l_s = torch.tanh(tanh_stretch_coefficient * feature_acts * n).sum(dim=-1)
+            elif sparsity_loss_type == "tanh-quad":
+                score = torch.tanh(tanh_stretch_coefficient * feature_acts * n)
+                freq = score.mean(dim=tuple(range(score.ndim - 1)))
+                l_s = (freq * (1 + freq / frequency_scale)).sum(dim=-1)
+            else:
+                raise ValueError(f"sparsity_loss_type f{sparsity_loss_type} not supported.")
+            l_s = l1_coefficient * l_s
+            loss_dict["l_s"] = l_s
+            loss = loss + apply_token_mask(l_s, min(ntd, l_s.ndim), mask if l_s.ndim else None, "mean")
+        else:
+            loss_dict["l_s"] = None
+
+        if lp_coefficient > 0.0 and isinstance(self.activation_function, JumpReLU):
+            theta = self.activation_function.get_jumprelu_threshold()
+            l_p = lp_coefficient * (torch.nn.functional.relu(theta - hidden_pre) * self.decoder_norm()).sum(dim=-1)
+            l_p = apply_token_mask(l_p, ntd, mask, "mean")
+            loss_dict["l_p"] = l_p
+            loss = loss + l_p
+        else:
+            loss_dict["l_p"] = None
+
+        if auxk_coefficient > 0.0:
+            assert update_dead_statistics is not None, "update_dead_statistics must be set when auxk_coefficient > 0.0"
+            specs = ("batch", "sae") if feature_acts.ndim == 2 else ("batch", "context", "sae")
+            is_dead = update_dead_statistics(feature_acts, mask, specs)
+            e = label - reconstructed
+            current_k = self.current_k
+            self.current_k = min(k_aux, int(is_dead.sum().item()))
+            if self.current_k > 0:
+                n = self.decoder_norm() if self.cfg.sparsity_include_decoder_norm else None
+                dead_hidden_pre = hidden_pre * is_dead * n if n is not None else hidden_pre * is_dead
+                dead_acts = self.activation_function(dead_hidden_pre)
+                if n is not None:
+                    dead_acts = dead_acts / n
+                aux_rec = dead_acts @ self.W_D
+                l_aux = apply_token_mask(auxk_coefficient * (e - aux_rec).pow(2).sum(dim=-1), ntd, mask, "mean")
+                loss_dict["l_aux"] = l_aux
+                loss = loss + l_aux
+            else:
+                loss_dict["l_aux"] = torch.zeros_like(l_rec)
+            self.current_k = current_k
+        else:
+            loss_dict["l_aux"] = None
+
+        if not return_aux_data:
+            return loss
+        return {
+            "loss": loss, **loss_dict, "label": label, "mask": mask,
+            "n_tokens": batch["tokens"].numel() if mask is None else int(mask.sum().item()),
+            "feature_acts": feature_acts, "reconstructed": reconstructed, "hidden_pre": hidden_pre,
+            "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient, "auxk_coefficient": auxk_coefficient,
+        }

@@ -1,0 +1,163 @@
+"""End-to-end parity of the fused SAE train step (module API -> HIP kernels) against the oracle.
+
+The encoder GEMM is checked against exact arithmetic in test_gpu_kernels.py.  Its fp32 (or bf16)
+rounding differs from the CPU's in the last bits, which can flip a TopK choice between two
+near-equal pre-activations; to compare everything downstream on identical selections, the oracle
+here takes the GEMM's forward values from the HIP path (its backward stays the matmul's).  A
+second test runs the oracle untouched and checks agreement statistically.
+"""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def rel_err(got, want):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+class _SubstitutedMatmul(torch.autograd.Function):
+    """y = x @ W with the forward value supplied; backward is the matmul's own."""
+
+    @staticmethod
+    def forward(ctx, x, W, y_given):
+        ctx.save_for_backward(x, W)
+        return y_given.clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        x, W = ctx.saved_tensors
+        return (g.to(W.dtype) @ W.t()).to(x.dtype), (x.t().to(g.dtype) @ g).to(W.dtype), None
+
+
+def make_pair(pkg, oracle, dev, d, F, k, B, r, seed, include_norm, mask_frac=0.0):
+    from lm_saes_amd import synthetic
+
+    x = synthetic.activations(B, d, r, seed)
+    w = synthetic.sae_weights(d, F, x, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    # make the decoder norms and the encoder bias non-trivial so that the fused scale/bias matter
+    W_D = w[2] * (0.5 + torch.rand(F, 1, generator=g))
+    b_E = 0.02 * torch.randn(F, generator=g)
+    w = (w[0], b_E, W_D.contiguous(), w[3])
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=include_norm,
+                        device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    synthetic.load_weights(sae, *[t.to(dev) for t in w])
+    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=include_norm)
+    synthetic.load_weights(ref, *w)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long)}
+    if mask_frac > 0:
+        batch["mask"] = (torch.rand(B, generator=g) > mask_frac).float()
+    return sae, ref, batch
+
+
+def run_both(pkg, oracle, dev, sae, ref, batch, amp, substitute):
+    gbatch = {k: v.to(dev) for k, v in batch.items()}
+    if amp:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            ctx = sae.compute_loss(gbatch)
+    else:
+        ctx = sae.compute_loss(gbatch)
+    ctx["loss"].backward()
+
+    if substitute:
+        # hand the HIP GEMM's forward values to the oracle's encoder matmul
+        def encode_sub(x, return_hidden_pre=False, **kw):
+            x = x.to(ref.W_E.dtype)
+            y_given = sae_pre.to(torch.bfloat16 if amp else torch.float32)
+            mm = _SubstitutedMatmul.apply(x.to(y_given.dtype) if amp else x, ref.W_E.to(y_given.dtype) if amp else ref.W_E, y_given)
+            hidden_pre = mm + ref.b_E
+            if ref.sparsity_include_decoder_norm:
+                hidden_pre = hidden_pre * ref.decoder_norm()
+            fa = ref.activation_function(hidden_pre)
+            if ref.sparsity_include_decoder_norm:
+                fa = fa / ref.decoder_norm()
+                hidden_pre = hidden_pre / ref.decoder_norm()
+            return (fa, hidden_pre) if return_hidden_pre else fa
+
+        # raw GEMM output of the HIP path, recomputed through the C ABI on the same operands
+        xg = gbatch["in"]
+        if amp:
+            sae_pre = pkg.ops.encoder_gemm(pkg.ops.cast_bf16(xg), sae._w_enc_operand(True), torch.bfloat16).cpu()
+        else:
+            sae_pre = pkg.ops.encoder_gemm(xg.contiguous(), sae._w_enc_operand(False), torch.float32).cpu()
+        ref.encode = encode_sub
+    if amp:
+        with torch.autocast("cpu", dtype=torch.bfloat16):
+            rctx = ref.compute_loss(batch)
+    else:
+        rctx = ref.compute_loss(batch)
+    rctx["loss"].backward()
+    return ctx, rctx
+
+
+@pytest.mark.parametrize("include_norm", [False, True])
+@pytest.mark.parametrize("masked", [False, True])
+def test_fused_step_fp32_matches_oracle(pkg, oracle, dev, include_norm, masked):
+    print(f"fused fp32 step include_norm={include_norm} masked={masked}", flush=True)
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=0,
+                                include_norm=include_norm, mask_frac=0.25 if masked else 0.0)
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=False, substitute=True)
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert rel_err(ctx["feature_acts"], rctx["feature_acts"]) < FP32_TOL
+    assert rel_err(ctx["hidden_pre"], rctx["hidden_pre"]) < FP32_TOL
+    assert rel_err(ctx["reconstructed"], rctx["reconstructed"]) < FP32_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < FP32_TOL
+    assert ctx["n_tokens"] == rctx["n_tokens"]
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = getattr(sae, name).grad, getattr(ref, name).grad
+        assert got.shape == want.shape
+        assert rel_err(got, want) < FP32_TOL, name
+
+
+@pytest.mark.parametrize("include_norm", [False, True])
+def test_fused_step_bf16_matches_oracle(pkg, oracle, dev, include_norm):
+    print(f"fused bf16 step include_norm={include_norm}", flush=True)
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=1, include_norm=include_norm)
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=True, substitute=True)
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert rel_err(ctx["feature_acts"], rctx["feature_acts"]) < BF16_TOL
+    assert rel_err(ctx["reconstructed"], rctx["reconstructed"]) < BF16_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < BF16_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = getattr(sae, name).grad, getattr(ref, name).grad
+        assert got.dtype == torch.float32 and rel_err(got, want) < BF16_TOL, name
+
+
+def test_fused_step_unsubstituted_agrees_statistically(pkg, oracle, dev):
+    """No substitution: the two GEMMs round differently, so a few near-tie selections may flip."""
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=2, include_norm=True)
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=False, substitute=False)
+    same = ((ctx["feature_acts"] != 0).cpu() == (rctx["feature_acts"] != 0)).all(dim=-1).float().mean().item()
+    assert same > 0.98
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < 1e-4
+
+
+def test_fused_step_then_adam_matches_oracle_adam(pkg, oracle, dev):
+    """One full step: fused loss + backward + HipAdam against the oracle's loss + torch.optim.Adam."""
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=3, include_norm=True)
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae)
+    ropt = oracle.make_adam(ref, lr=4e-4)
+    before = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=False, substitute=True)
+    opt.step(); opt.zero_grad()
+    ropt.step(); ropt.zero_grad()
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = getattr(sae, name).detach().cpu(), getattr(ref, name).detach()
+        moved_ref = (want - before[name]).abs().max().item()
+        assert moved_ref > 0
+        # Adam's first step is +-lr wherever the gradient is non-zero; entries whose tiny gradient
+        # differs in the last bits may move differently, so bound the count, and demand exactness elsewhere
+        diff = (got - want).abs()
+        assert (diff > 1e-3 * moved_ref).float().mean().item() < 1e-3, name
+    # features no token selected keep their exact weights (zero gradient => zero Adam move)
+    want, got = ref.W_D.detach(), sae.W_D.detach().cpu()
+    unchanged = (want == before["W_D"]).all(dim=1)
+    assert unchanged.any() and torch.equal(got[unchanged], before["W_D"][unchanged])
