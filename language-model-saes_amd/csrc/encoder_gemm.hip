@@ -1,29 +1,40 @@
 // Encoder pre-activation GEMM for gfx950:  pre[B, F] = x[B, d] * W_E^T[F, d]^T.
 //
-// Both operands are K-contiguous ("NT" GEMM), so a 16-byte global load fetches exactly the
-// 8 bf16 (or 4 fp32) one lane feeds to a matrix-core instruction.
+// Both operands are K-contiguous ("NT" GEMM), so a 16-byte piece of a row is exactly the 8 bf16
+// (or 4 fp32) one lane feeds to a matrix-core instruction.
 //
-// Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile
-// and walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32).  Waves are arranged 2 x 4:
-// each owns 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32 accumulators per
-// lane).  Slabs are double-buffered in LDS (2 x (32 + 32) KiB = 128 of the CU's 160 KiB); the
-// next slab's global loads are in flight while the current one feeds the matrix cores.
+// Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile and
+// walks K in stages of 64 bytes per row (32 bf16 / 16 fp32).  Waves are arranged 2 x 4: each owns
+// 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32 accumulators per lane).
 //
-// LDS layout: row r of a slab is 128 bytes = 8 chunks of 16 bytes; chunk c is stored at
-// physical chunk c ^ ((r >> 1) & 7).  A group of 16 lanes then covers 256 distinct bytes both
-// when the slab is written (8 lanes per row, 2 rows) and when MFMA fragments are read
-// (16 rows, one logical chunk), so neither side bank-conflicts.
+// Pipeline: four stages of (256 + 256) rows x 64 bytes = 32 KiB live in LDS (128 of the CU's
+// 160 KiB).  Stages are filled by LDS-direct loads (global_load_lds_dwordx4: the data never
+// passes through VGPRs), three stages ahead of the one being consumed; one s_waitcnt vmcnt(8) +
+// s_barrier per stage both publishes the stage that just landed and frees the one just consumed.
+// The loads are issued through inline assembly so that the compiler's wait-count insertion does
+// not serialise them against the LDS reads of the other stages.
 //
-// The matrix cores compute D = Wtile * xtile^T (features along the 32 "rows" of the
-// instruction), which leaves every lane holding 4 consecutive features of one token: the
-// epilogue packs them into one 8-byte (bf16) or 16-byte (fp32) store.
+// LDS layout: row r of a stage is 64 bytes = 4 chunks of 16 bytes; chunk c is stored at physical
+// chunk c ^ ((r >> 2) & 3).  A group of 16 lanes then covers 256 distinct bytes when MFMA
+// fragments are read (16 rows, one logical chunk): zero bank conflicts (SQ_LDS_BANK_CONFLICT = 0).
+// An LDS-direct load writes 1 KiB linearly (lane l -> base + 16 l), so the swizzle is applied on
+// the global side: lane l fetches the logical chunk that belongs at its physical slot.
+//
+// The matrix cores compute D = Wtile * xtile^T (features along the 32 "rows" of the instruction),
+// which leaves every lane holding 4 consecutive features of one token: the epilogue packs them
+// into one 8-byte (bf16) or 16-byte (fp32) store.
 //
 // Workgroups are numbered so that consecutive ids land on the 8 XCDs round-robin, and the
-// workgroups of one XCD walk all token tiles of one feature tile before moving on: a W_E
-// slab is pulled from HBM once per XCD-L2 and shared by the 16 token tiles.
+// workgroups of one XCD walk all token tiles of one feature tile before moving on: a W_E stage
+// is pulled from HBM once per XCD-L2 and shared by the token tiles.
+//
+// Rows beyond B or F are clamped to the last valid row when loading (their products land in
+// accumulators that the epilogue never stores), so the main loop has no bounds checks.
 #include "common.h"
 
 namespace sae {
+
+#define WAITCNT_VM8 ((8 & 0xf) | (0x7 << 4) | (0xf << 8) | ((8 >> 4) << 14))
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -31,11 +42,12 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 constexpr int GEMM_BM = 256;       // tokens per workgroup tile
 constexpr int GEMM_BN = 256;       // features per workgroup tile
-constexpr int GEMM_SLAB = 128;     // bytes of K per row per slab
+constexpr int GEMM_SLAB = 64;      // bytes of K per row per stage
+constexpr int GEMM_STAGES = 4;
 constexpr int GEMM_THREADS = 512;
-constexpr int GEMM_LDS_BYTES = 2 * (GEMM_BM + GEMM_BN) * GEMM_SLAB;
+constexpr int GEMM_LDS_BYTES = GEMM_STAGES * (GEMM_BM + GEMM_BN) * GEMM_SLAB;
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 1) & 7)) << 4); }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 2) & 3)) << 4); }
 
 template <bool BF16_IN>
 __device__ __forceinline__ void mma_chunk(const u32x4 &wf, const u32x4 &xf, f32x16_t &acc) {
@@ -85,19 +97,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
   const int wm = wave >> 2, wn = wave & 3;
 
   // ---- global -> LDS staging assignment: 8 lanes cover one 128-byte row slab ----
-  const int ld_chunk = tid & 7, ld_row = tid >> 3;  // rows ld_row + 64*i, i = 0..3
-  const char *xg[4];
-  const char *wg[4];
-  bool xok[4], wok[4];
-  int lds_off[4];
+  const int ld_phys = lane & 3;  // physical 16-byte chunk this lane fills
+  const char *xg[2];
+  const char *wg[2];
+  bool xok[2], wok[2];
+  int lds_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = ld_row + 64 * i;
+  for (int i = 0; i < 2; ++i) {
+    const int r = wave * 32 + i * 16 + (lane >> 2);
+    const int ld_chunk = ld_phys ^ ((r >> 2) & 3);  // logical chunk that lives at this physical slot
     xok[i] = (m0 + r) < M;
     wok[i] = (n0 + r) < N;
-    xg[i] = x + (size_t)(xok[i] ? (m0 + r) : 0) * row_bytes + ld_chunk * 16;
-    wg[i] = w + (size_t)(wok[i] ? (n0 + r) : 0) * row_bytes + ld_chunk * 16;
-    lds_off[i] = swz(r, ld_chunk);
+    xg[i] = x + (size_t)(xok[i] ? (m0 + r) : (M - 1)) * row_bytes + ld_chunk * 16;
+    wg[i] = w + (size_t)(wok[i] ? (n0 + r) : (N - 1)) * row_bytes + ld_chunk * 16;
+    lds_off[i] = (wave * 32 + i * 16) * GEMM_SLAB;  // wave-uniform base of the 1 KiB this load fills
   }
 
   f32x16_t acc[2][4];  // [feature sub-tile][token sub-tile]
@@ -109,37 +122,38 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int n_slabs = row_bytes / GEMM_SLAB;
-  u32x4 xr[4], wr[4];
-  const u32x4 zero4 = {0u, 0u, 0u, 0u};
-
-  auto load_global = [&](int slab) {
-    const size_t off = (size_t)slab * GEMM_SLAB;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xg[i] + off) : zero4;
-      wr[i] = wok[i] ? *reinterpret_cast<const u32x4 *>(wg[i] + off) : zero4;
-    }
-  };
-  auto store_lds = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4 *>(lds + buf * X_BYTES + lds_off[i]) = xr[i];
-      *reinterpret_cast<u32x4 *>(lds + 2 * X_BYTES + buf * W_BYTES + lds_off[i]) = wr[i];
-    }
-  };
-
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+#if defined(__HIP_DEVICE_COMPILE__)
+#define LDS_DMA16(GPTR, LDSADDR)                                                          \
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(LDSADDR)), "v"(GPTR) : "memory")
+#else
+#define LDS_DMA16(GPTR, LDSADDR) ((void)0)
+#endif
+#define LOAD_SLAB_TO_LDS(SLAB, BUF)                                                                      \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                       \
+    LDS_DMA16(xg[i] + (size_t)(SLAB) * GEMM_SLAB, lds_base + (BUF) * X_BYTES + lds_off[i]);             \
+    LDS_DMA16(wg[i] + (size_t)(SLAB) * GEMM_SLAB, lds_base + GEMM_STAGES * X_BYTES + (BUF) * W_BYTES + lds_off[i]); \
+  }
+  // prologue: stages 0..2 in flight
+  LOAD_SLAB_TO_LDS(0, 0)
+  LOAD_SLAB_TO_LDS(n_slabs > 1 ? 1 : 0, 1)
+  LOAD_SLAB_TO_LDS(n_slabs > 2 ? 2 : 0, 2)
 
   const int frag_row = lane & 31, frag_half = lane >> 5;
   for (int slab = 0; slab < n_slabs; ++slab) {
-    const int buf = slab & 1;
-    if (slab + 1 < n_slabs) load_global(slab + 1);
+    const int buf = slab & (GEMM_STAGES - 1);
+    // my loads of this slab have landed when at most the two younger stages (8 loads) are outstanding
+    __builtin_amdgcn_s_waitcnt(WAITCNT_VM8);
+    __builtin_amdgcn_s_barrier();  // everyone's part of this slab landed; everyone is done reading the previous slab
+    const int nxt = slab + 3 < n_slabs ? slab + 3 : n_slabs - 1;  // tail re-reads the last slab (never used)
+    LOAD_SLAB_TO_LDS(nxt, (slab + 3) & (GEMM_STAGES - 1))
+    __builtin_amdgcn_sched_barrier(0);
     const char *lx = lds + buf * X_BYTES;
-    const char *lw = lds + 2 * X_BYTES + buf * W_BYTES;
+    const char *lw = lds + GEMM_STAGES * X_BYTES + buf * W_BYTES;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {  // 4 MFMA k-steps per slab (32 bytes of K each)
+    for (int s = 0; s < 2; ++s) {  // 2 MFMA k-steps per stage (32 bytes of K each)
       const int chunk = 2 * s + frag_half;
       u32x4 wf[2], xf[4];
 #pragma unroll
@@ -151,9 +165,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) mma_chunk<BF16_IN>(wf[i], xf[j], acc[i][j]);
     }
-    if (slab + 1 < n_slabs) store_lds(buf ^ 1);
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
   }
+  __builtin_amdgcn_s_waitcnt(0);
 
   // ---- epilogue: lane holds, per (i, j, g): 4 consecutive features of one token ----
   // D[row = feature, col = token]: token = lane % 32, feature = 8*g + 4*(lane/32) + r
@@ -225,7 +239,7 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
   SAE_REQUIRE(in_dtype == SAE_F32 || in_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad in_dtype %d", in_dtype);
   SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad out_dtype %d", out_dtype);
   SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm: size too large");
-  const int64_t per_slab = in_dtype == SAE_BF16 ? 64 : 32;
+  const int64_t per_slab = in_dtype == SAE_BF16 ? 32 : 16;  // elements in one 64-byte stage row
   SAE_REQUIRE(d % per_slab == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm: d_model=%lld must be a multiple of %lld",
               (long long)d, (long long)per_slab);
   SAE_REQUIRE((((uintptr_t)x | (uintptr_t)w_enc_t | (uintptr_t)pre) & 15) == 0, SAE_ERR_INVALID_ARG,

@@ -107,7 +107,7 @@ struct RowReader {
   template <typename Fn>
   __device__ __forceinline__ void for_each(Fn fn) const {
     constexpr int V = BF16 ? 8 : 4;  // elements per 16-byte load
-    const bool vec_ok = (F % V == 0) && ((((uintptr_t)row) & 15) == 0);
+    const bool vec_ok = (F % V == 0) && (((((uintptr_t)row) | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0);
     if (vec_ok) {
       const int n_chunks = F / V;
       for (int c = threadIdx.x; c < n_chunks; c += SEL_THREADS) {
@@ -125,12 +125,29 @@ struct RowReader {
           pre[2] = __uint_as_float(raw.z); pre[3] = __uint_as_float(raw.w);
         }
         const int base = c * V;
+        float bb[V], ss[V];
+        if (b_enc) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) {
-          const float b = b_enc ? b_enc[base + e] : 0.f;
-          const float s = scale ? scale[base + e] : 1.f;
-          fn(base + e, key_of(pre[e], b, s));
+          for (int q = 0; q < V / 4; ++q) {
+            const float4 t = reinterpret_cast<const float4 *>(b_enc + base)[q];
+            bb[4 * q] = t.x; bb[4 * q + 1] = t.y; bb[4 * q + 2] = t.z; bb[4 * q + 3] = t.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) bb[e] = 0.f;
         }
+        if (scale) {
+#pragma unroll
+          for (int q = 0; q < V / 4; ++q) {
+            const float4 t = reinterpret_cast<const float4 *>(scale + base)[q];
+            ss[4 * q] = t.x; ss[4 * q + 1] = t.y; ss[4 * q + 2] = t.z; ss[4 * q + 3] = t.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) ss[e] = 1.f;
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e) fn(base + e, key_of(pre[e], bb[e], ss[e]));
       }
     } else {
       for (int i = threadIdx.x; i < F; i += SEL_THREADS) {

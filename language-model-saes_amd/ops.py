@@ -19,6 +19,50 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class KernelTimer:
+    """Collects HIP-event pairs around every library call made while it is installed.
+
+    Events are recorded on the stream the kernels are launched on (torch's current stream), so
+    `elapsed_time` is the device-side duration of that call's kernels.  Read after a synchronize.
+    """
+
+    def __init__(self):
+        self.records: dict[str, list[tuple[torch.cuda.Event, torch.cuda.Event]]] = {}
+
+    def summary(self) -> dict[str, dict[str, float]]:
+        out = {}
+        for name, evs in self.records.items():
+            ms = [a.elapsed_time(b) for a, b in evs]
+            out[name] = {"calls": len(ms), "avg_ms": sum(ms) / len(ms), "total_ms": sum(ms)}
+        return out
+
+
+_timer: Optional[KernelTimer] = None
+
+
+def set_kernel_timer(timer: Optional[KernelTimer]) -> None:
+    global _timer
+    _timer = timer
+
+
+class _timed:
+    def __init__(self, name: str):
+        self.name = name
+
+    def __enter__(self):
+        if _timer is not None:
+            self.a = torch.cuda.Event(enable_timing=True)
+            self.a.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _timer is not None:
+            b = torch.cuda.Event(enable_timing=True)
+            b.record()
+            _timer.records.setdefault(self.name, []).append((self.a, b))
+        return False
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -81,7 +125,8 @@ def cast_bf16(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     _req(src, "src", torch.float32)
     if out is None:
         out = torch.empty(src.shape, dtype=torch.bfloat16, device=src.device)
-    check(_lib.load().sae_cast_f32_to_bf16(src.data_ptr(), out.data_ptr(), src.numel(), _stream(src)), "cast_f32_to_bf16")
+    with _timed("cast_f32_to_bf16"):
+        check(_lib.load().sae_cast_f32_to_bf16(src.data_ptr(), out.data_ptr(), src.numel(), _stream(src)), "cast_f32_to_bf16")
     return out
 
 
@@ -90,7 +135,8 @@ def row_norm(w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tenso
     F, d = w.shape
     if out is None:
         out = torch.empty(F, dtype=torch.float32, device=w.device)
-    check(_lib.load().sae_row_norm(w.data_ptr(), out.data_ptr(), F, d, _stream(w)), "row_norm")
+    with _timed("row_norm"):
+        check(_lib.load().sae_row_norm(w.data_ptr(), out.data_ptr(), F, d, _stream(w)), "row_norm")
     return out
 
 
@@ -98,7 +144,8 @@ def transpose(src: torch.Tensor) -> torch.Tensor:
     _req(src, "src", torch.float32, 2)
     r, c = src.shape
     out = torch.empty(c, r, dtype=torch.float32, device=src.device)
-    check(_lib.load().sae_transpose_f32(src.data_ptr(), out.data_ptr(), r, c, _stream(src)), "transpose_f32")
+    with _timed("transpose_f32"):
+        check(_lib.load().sae_transpose_f32(src.data_ptr(), out.data_ptr(), r, c, _stream(src)), "transpose_f32")
     return out
 
 
@@ -111,7 +158,8 @@ def col_sum(src: torch.Tensor, out: Optional[torch.Tensor] = None, accumulate: b
         accumulate = False
     ws_bytes = lib.sae_col_sum_workspace_bytes(B, n)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=src.device)
-    check(lib.sae_col_sum(src.data_ptr(), out.data_ptr(), B, n, int(accumulate), ws.data_ptr(), ws_bytes, _stream(src)), "col_sum")
+    with _timed("col_sum"):
+        check(lib.sae_col_sum(src.data_ptr(), out.data_ptr(), B, n, int(accumulate), ws.data_ptr(), ws_bytes, _stream(src)), "col_sum")
     return out
 
 
@@ -128,10 +176,11 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     if d != d2:
         raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
     pre = torch.empty(B, F, dtype=out_dtype, device=x.device)
-    check(
-        _lib.load().sae_encoder_gemm(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _dt(x), _dt(pre), _stream(x)),
-        "encoder_gemm",
-    )
+    with _timed("encoder_gemm"):
+        check(
+            _lib.load().sae_encoder_gemm(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _dt(x), _dt(pre), _stream(x)),
+            "encoder_gemm",
+        )
     return pre
 
 
@@ -158,12 +207,15 @@ def select_topk_row(
     row_off = torch.empty(B, dtype=torch.int64, device=dev)
     row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
     lib = _lib.load()
+    _t = _timed("select_topk_row")
+    _t.__enter__()
     if cand_cap is None:
         rc = lib.sae_select_topk_row(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
                                      val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     else:
         rc = lib.sae_select_topk_row_ex(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
                                         val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), int(cand_cap), _stream(pre))
+    _t.__exit__()
     check(rc, "select_topk_row")
     return SparseCode(idx, val, row_off, row_nnz, B, F)
 
@@ -187,12 +239,13 @@ def sparse_decode_fwd(code: SparseCode, w_dec: torch.Tensor, b_dec: Optional[tor
     if b_dec is not None:
         _req(b_dec, "b_dec", torch.float32, 1)
     recon = torch.empty(B, d, dtype=torch.float32, device=w_dec.device)
-    check(
-        _lib.load().sae_sparse_decode_fwd(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
-                                          code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
-                                          recon.data_ptr(), B, d, F, _stream(w_dec)),
-        "sparse_decode_fwd",
-    )
+    with _timed("sparse_decode_fwd"):
+        check(
+            _lib.load().sae_sparse_decode_fwd(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                              code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
+                                              recon.data_ptr(), B, d, F, _stream(w_dec)),
+            "sparse_decode_fwd",
+        )
     return recon
 
 
@@ -202,12 +255,13 @@ def sparse_decode_bwd_dval(code: SparseCode, grad_recon: torch.Tensor, w_dec: to
     F, d = w_dec.shape
     B = code.n_tokens
     dval = torch.empty(code.n_slots, dtype=torch.float32, device=w_dec.device)
-    check(
-        _lib.load().sae_sparse_decode_bwd_dval(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(),
-                                               grad_recon.data_ptr(), w_dec.data_ptr(), _dt(w_dec), dval.data_ptr(),
-                                               B, d, F, code.n_slots, _stream(w_dec)),
-        "sparse_decode_bwd_dval",
-    )
+    with _timed("sparse_decode_bwd_dval"):
+        check(
+            _lib.load().sae_sparse_decode_bwd_dval(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(),
+                                                   grad_recon.data_ptr(), w_dec.data_ptr(), _dt(w_dec), dval.data_ptr(),
+                                                   B, d, F, code.n_slots, _stream(w_dec)),
+            "sparse_decode_bwd_dval",
+        )
     return dval
 
 
@@ -227,14 +281,15 @@ def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Option
     loss_tok = torch.empty(B, dtype=torch.float32, device=dev)
     grad_recon = torch.empty(B, d, dtype=torch.float32, device=dev)
     dval = torch.empty(code.n_slots, dtype=torch.float32, device=dev)
-    check(
-        _lib.load().sae_sparse_decode_mse_fused(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
-                                                code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
-                                                label.data_ptr(), _ptr(tok_w), _ptr(recon), loss_tok.data_ptr(),
-                                                grad_recon.data_ptr(), dval.data_ptr(), B, d, F, code.n_slots,
-                                                _stream(w_dec)),
-        "sparse_decode_mse_fused",
-    )
+    with _timed("sparse_decode_mse_fused"):
+        check(
+            _lib.load().sae_sparse_decode_mse_fused(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                                    code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
+                                                    label.data_ptr(), _ptr(tok_w), _ptr(recon), loss_tok.data_ptr(),
+                                                    grad_recon.data_ptr(), dval.data_ptr(), B, d, F, code.n_slots,
+                                                    _stream(w_dec)),
+            "sparse_decode_mse_fused",
+        )
     return recon, loss_tok, grad_recon, dval
 
 
@@ -249,12 +304,13 @@ def build_feature_index(code: SparseCode) -> FeatureIndex:
     feat_ptr = torch.empty(F + 1, dtype=torch.int32, device=dev)
     feat_slot = torch.empty(n, dtype=torch.int32, device=dev)
     slot_tok = torch.zeros(n, dtype=torch.int32, device=dev)
-    check(
-        lib.sae_build_feature_index(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(), B, F, n,
-                                    feat_ptr.data_ptr(), feat_slot.data_ptr(), slot_tok.data_ptr(), ws.data_ptr(),
-                                    ws_bytes, _stream(code.idx)),
-        "build_feature_index",
-    )
+    with _timed("build_feature_index"):
+        check(
+            lib.sae_build_feature_index(code.idx.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(), B, F, n,
+                                        feat_ptr.data_ptr(), feat_slot.data_ptr(), slot_tok.data_ptr(), ws.data_ptr(),
+                                        ws_bytes, _stream(code.idx)),
+            "build_feature_index",
+        )
     return FeatureIndex(feat_ptr, feat_slot, slot_tok)
 
 
@@ -268,12 +324,13 @@ def sparse_grad_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, 
     if out is None:
         out = torch.empty(F, d, dtype=torch.float32, device=dev)
     bias = torch.empty(F, dtype=torch.float32, device=dev) if want_bias else None
-    check(
-        _lib.load().sae_sparse_grad_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
-                                         coef.data_ptr(), dense.data_ptr(), _dt(dense), out.data_ptr(), _ptr(bias), F, d,
-                                         _stream(dense)),
-        "sparse_grad_rows",
-    )
+    with _timed("sparse_grad_rows[bf16 dense]" if dense.dtype == torch.bfloat16 else "sparse_grad_rows[f32 dense]"):
+        check(
+            _lib.load().sae_sparse_grad_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
+                                             coef.data_ptr(), dense.data_ptr(), _dt(dense), out.data_ptr(), _ptr(bias), F, d,
+                                             _stream(dense)),
+            "sparse_grad_rows",
+        )
     return out, bias
 
 
@@ -288,8 +345,9 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
             raise ValueError(f"{name} must have {p.numel()} elements")
     if shadow_bf16 is not None:
         _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
-    check(
-        _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
-                                  eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _stream(p)),
-        "adam_step",
-    )
+    with _timed("adam_step[matrix]" if p.ndim == 2 else "adam_step[vector]"):
+        check(
+            _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
+                                      eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _stream(p)),
+            "adam_step",
+        )
