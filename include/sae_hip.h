@@ -179,6 +179,21 @@ int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, doubl
                   double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                   int64_t row_len, void *stream);
 
+/* Adam on a feature-major weight matrix [F, d] whose gradient is given in factored form:
+ *   g[f, :] = sum_{s in segment f of the feature index} coef[s] * dense[slot_tok[s], :]
+ * (the quantity sae_sparse_grad_rows would write).  The row gradient is formed in registers and
+ * consumed at once; no dense gradient is stored.  Same update rule, scalars and by-products
+ * (shadow_bf16, row_norm_out) as sae_adam_step; bias_grad_out (nullable) receives
+ * sum_{s in segment f} coef[s], the gradient of the per-feature bias.  Bit-identical to
+ * sae_sparse_grad_rows followed by sae_adam_step.
+ * Replaces loss.backward()'s dense `f^T @ grad` / `x^T @ dh` GEMMs together with
+ * torch.optim.Adam.step for W_D / W_E (trainer.py:627-647). */
+int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                              const float *coef, const void *dense, int dense_dtype, float *p, float *m,
+                              float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
+                              double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                              float *bias_grad_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

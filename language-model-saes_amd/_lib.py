@@ -36,6 +36,7 @@ SIGNATURES = {
     "sae_build_feature_index": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P]),
     "sae_sparse_grad_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _P]),
     "sae_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _L, _P, _P, _L, _P]),
+    "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P]),
 }
 
 _lib = None

@@ -118,3 +118,133 @@ extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64
   }
   return check_launch("adam_step");
 }
+
+// ---------------------------------------------------------------------------------------------
+// Adam with the gradient row rebuilt on the fly from the sparse code.
+//
+// For the two weight matrices the gradient of feature f is a short sum,
+//   g[f, :] = sum_{slot in segment f} coef[slot] * dense[token(slot), :],
+// (dW_D: coef = feature activation, dense = grad_recon; dW_E^T: coef = d pre-activation, dense = x).
+// One workgroup owns a feature: it forms g[f, :] in registers from the feature index (the dense
+// operand rows come from L2 / Infinity Cache: 64 MB and 32 MB at the headline shape), and applies
+// the Adam update to that row at once.  The dense [F, d] gradient never exists in HBM: per
+// parameter the pass moves 12 B in + 12 B out (+ 2 B bf16 shadow) instead of 4 B gradient write +
+// 16 B in + 12 B out (+ 2 B).  The summation order inside a segment is the feature index's
+// (ascending token), the same as sae_sparse_grad_rows, so both routes give identical bits.
+// ---------------------------------------------------------------------------------------------
+namespace sae {
+
+template <bool DENSE_BF16>
+__global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
+    const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
+    const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
+    float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
+    uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad) {
+  __shared__ float red[4];
+  const int f = blockIdx.x, tid = threadIdx.x;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  const int n_seg = d >> 2;
+  const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
+  const char *dbase = reinterpret_cast<const char *>(dense);
+  const int64_t base4 = (int64_t)f * n_seg;
+
+  if (bias_grad && tid < 64) {
+    float s = 0.f;
+    for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
+    s = wave_sum(s);
+    if (tid == 0) bias_grad[f] = s;
+  }
+
+  float sq = 0.f;
+  for (int seg0 = tid; seg0 < n_seg; seg0 += 256 * 4) {
+    // issue the streaming reads of p, m, v first: they are the HBM traffic; the gradient operands hit cache
+    float4 pp[4], mm[4], vv[4], g[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int seg = seg0 + u * 256;
+      if (seg < n_seg) {
+        pp[u] = reinterpret_cast<const float4 *>(p)[base4 + seg];
+        mm[u] = reinterpret_cast<const float4 *>(m)[base4 + seg];
+        vv[u] = reinterpret_cast<const float4 *>(v)[base4 + seg];
+      }
+      g[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int i = lo; i < hi; ++i) {
+      const int s = feat_slot[i];
+      const float c = coef[s];
+      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int seg = seg0 + u * 256;
+        if (seg < n_seg) {
+          float4 x;
+          if constexpr (DENSE_BF16) {
+            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
+            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
+            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
+          } else {
+            x = reinterpret_cast<const float4 *>(row)[seg];
+          }
+          g[u].x = fmaf(c, x.x, g[u].x); g[u].y = fmaf(c, x.y, g[u].y);
+          g[u].z = fmaf(c, x.z, g[u].z); g[u].w = fmaf(c, x.w, g[u].w);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int seg = seg0 + u * 256;
+      if (seg < n_seg) {
+        adam_one(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_one(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
+        adam_one(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_one(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
+        reinterpret_cast<float4 *>(p)[base4 + seg] = pp[u];
+        reinterpret_cast<float4 *>(m)[base4 + seg] = mm[u];
+        reinterpret_cast<float4 *>(v)[base4 + seg] = vv[u];
+        sq = fmaf(pp[u].x, pp[u].x, sq); sq = fmaf(pp[u].y, pp[u].y, sq);
+        sq = fmaf(pp[u].z, pp[u].z, sq); sq = fmaf(pp[u].w, pp[u].w, sq);
+        if (shadow) {
+          uint2 o;
+          o.x = (uint32_t)f32_to_bf16_bits(pp[u].x) | ((uint32_t)f32_to_bf16_bits(pp[u].y) << 16);
+          o.y = (uint32_t)f32_to_bf16_bits(pp[u].z) | ((uint32_t)f32_to_bf16_bits(pp[u].w) << 16);
+          reinterpret_cast<uint2 *>(shadow)[base4 + seg] = o;
+        }
+      }
+    }
+  }
+  if (row_norm) {
+    const float tot = block_sum<4>(sq, red);
+    if (tid == 0) row_norm[f] = sqrtf(tot);
+  }
+}
+
+}  // namespace sae
+
+extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                         const float *coef, const void *dense, int dense_dtype, float *p, float *m,
+                                         float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
+                                         double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                                         float *bias_grad_out, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
+              "adam_step_sparse_rows: null pointer");
+  SAE_REQUIRE(F > 0 && d > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step_sparse_rows: bad sizes / step");
+  SAE_REQUIRE(dense_dtype == SAE_F32 || dense_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "adam_step_sparse_rows: bad dtype %d", dense_dtype);
+  SAE_REQUIRE(d % 4 == 0 && F < (1LL << 31) && d < (1LL << 31), SAE_ERR_UNSUPPORTED,
+              "adam_step_sparse_rows: d_model=%lld must be a multiple of 4", (long long)d);
+  SAE_REQUIRE((((uintptr_t)p | (uintptr_t)m | (uintptr_t)v | (uintptr_t)dense) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "adam_step_sparse_rows: 16-byte alignment required");
+  AdamScalars a;
+  a.beta1 = (float)beta1; a.beta2 = (float)beta2;
+  a.one_minus_beta1 = (float)(1.0 - beta1);
+  a.one_minus_beta2 = (float)(1.0 - beta2);
+  a.step_size = (float)(lr / (1.0 - pow(beta1, (double)step)));
+  a.inv_bc2_sqrt = (float)(1.0 / sqrt(1.0 - pow(beta2, (double)step)));
+  a.eps = (float)eps;
+  hipStream_t st = (hipStream_t)stream;
+  if (dense_dtype == SAE_BF16)
+    hipLaunchKernelGGL(adam_sparse_rows_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out);
+  else
+    hipLaunchKernelGGL(adam_sparse_rows_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out);
+  return check_launch("adam_step_sparse_rows");
+}

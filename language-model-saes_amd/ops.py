@@ -351,3 +351,29 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
                                       eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _stream(p)),
             "adam_step",
         )
+
+
+def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, p: torch.Tensor, m: torch.Tensor,
+                          v: torch.Tensor, *, lr: float, beta1: float, beta2: float, eps: float, step: int,
+                          shadow_bf16: Optional[torch.Tensor] = None, row_norm_out: Optional[torch.Tensor] = None,
+                          bias_grad_out: Optional[torch.Tensor] = None) -> None:
+    """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense)."""
+    for name, t in (("p", p), ("m", m), ("v", v)):
+        _req(t, name, torch.float32, 2)
+    _req(coef, "coef", torch.float32, 1)
+    _req(dense, "dense", ndim=2)
+    F, d = p.shape
+    if dense.shape[1] != d or m.shape != p.shape or v.shape != p.shape:
+        raise ValueError("shape mismatch between p, m, v and the dense operand")
+    if fi.feat_ptr.numel() != F + 1:
+        raise ValueError("feature index was built for a different number of features")
+    if shadow_bf16 is not None:
+        _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
+    with _timed("adam_step_sparse_rows[bf16 dense]" if dense.dtype == torch.bfloat16 else "adam_step_sparse_rows[f32 dense]"):
+        check(
+            _lib.load().sae_adam_step_sparse_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
+                                                  coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),
+                                                  v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step), _ptr(shadow_bf16),
+                                                  _ptr(row_norm_out), _ptr(bias_grad_out), _stream(p)),
+            "adam_step_sparse_rows",
+        )

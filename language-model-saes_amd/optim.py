@@ -30,7 +30,8 @@ def _flat_view(p: torch.Tensor) -> torch.Tensor:
 
 
 class HipAdam(Optimizer):
-    def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, model=None):
+    def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, model=None,
+                 defer_weight_grads: bool = True):
         if lr < 0.0 or eps < 0.0 or not (0.0 <= betas[0] < 1.0) or not (0.0 <= betas[1] < 1.0):
             raise ValueError("invalid Adam hyper-parameters")
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps))
@@ -41,6 +42,59 @@ class HipAdam(Optimizer):
                 p = getattr(model, name, None)
                 if p is not None:
                     self._roles[id(p)] = name
+            if defer_weight_grads and hasattr(model, "defer_weight_grads"):
+                model.defer_weight_grads = True
+
+    def zero_grad(self, set_to_none: bool = True):
+        super().zero_grad(set_to_none=set_to_none)
+        for group in self.param_groups:
+            for p in group["params"]:
+                if getattr(p, "_sparse_grad", None) is not None:
+                    p._sparse_grad = None
+
+    @torch.no_grad()
+    def materialize_grads(self) -> None:
+        """Turn factored weight gradients into ordinary dense `.grad` tensors (for gradient clipping,
+        the grad-norm diagnostic, or a different optimiser)."""
+        for group in self.param_groups:
+            for p in group["params"]:
+                sg = getattr(p, "_sparse_grad", None)
+                if sg is None:
+                    continue
+                rows, bias = sg.dense()
+                p.grad = rows if p.is_contiguous() else rows.t()
+                if bias is not None:
+                    sg.bias_param.grad = bias
+                p._sparse_grad = None
+
+    def _state(self, p):
+        st = self.state[p]
+        if len(st) == 0:
+            st["step"] = torch.zeros((), dtype=torch.float32)
+            st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+        return st
+
+    def _by_products(self, p, pv):
+        """(role, bf16 shadow buffer or None, row-norm buffer or None) for the two weight matrices."""
+        role = self._roles.get(id(p))
+        shadow = norm_out = None
+        if role is not None and pv.ndim == 2:
+            shadow = self._model.get_derived_buffer(f"{role}.bf16")
+            if role == "W_D" and pv.shape[1] % 4 == 0:
+                norm_out = self._model.get_derived_buffer("W_D.norm")
+                if norm_out is None:
+                    norm_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
+        return role, shadow, norm_out
+
+    def _publish(self, p, role, shadow, norm_out):
+        # the kernel wrote through raw pointers: move the version counter like an in-place op would
+        torch.autograd.graph.increment_version(p)
+        if role is not None:
+            if shadow is not None:
+                self._model.set_derived(f"{role}.bf16", p, shadow)
+            if norm_out is not None:
+                self._model.set_derived("W_D.norm", p, norm_out)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -48,6 +102,31 @@ class HipAdam(Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        # pass 1: weights whose gradient arrives in factored form (also yields the encoder-bias gradient)
+        for group in self.param_groups:
+            b1, b2 = group["betas"]
+            for p in group["params"]:
+                sg = getattr(p, "_sparse_grad", None)
+                if sg is None:
+                    continue
+                if p.grad is not None:
+                    raise RuntimeError("parameter has both a dense and a factored gradient")
+                st = self._state(p)
+                st["step"] += 1
+                pv = _flat_view(p)
+                mv, vv = _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"])
+                role, shadow, norm_out = self._by_products(p, pv)
+                bias_out = None
+                if sg.bias_param is not None:
+                    bias_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
+                ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
+                                          eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
+                                          row_norm_out=norm_out, bias_grad_out=bias_out)
+                if bias_out is not None:
+                    sg.bias_param.grad = bias_out if sg.bias_param.grad is None else sg.bias_param.grad + bias_out
+                p._sparse_grad = None
+                self._publish(p, role, shadow, norm_out)
+        # pass 2: everything with a dense gradient
         for group in self.param_groups:
             b1, b2 = group["betas"]
             for p in group["params"]:
@@ -55,11 +134,7 @@ class HipAdam(Optimizer):
                     continue
                 if p.dtype != torch.float32:
                     raise TypeError("HipAdam updates fp32 master parameters")
-                st = self.state[p]
-                if len(st) == 0:
-                    st["step"] = torch.zeros((), dtype=torch.float32)
-                    st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                    st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                st = self._state(p)
                 st["step"] += 1
                 pv = _flat_view(p)
                 same_layout = lambda t: _flat_view(t) if t.stride() == p.stride() else None  # noqa: E731
@@ -67,26 +142,9 @@ class HipAdam(Optimizer):
                 if gv is None:
                     gv = _flat_view(p.grad.contiguous()) if p.is_contiguous() else p.grad.t().contiguous()
                 assert mv is not None and vv is not None, "optimizer state must share the parameter's layout"
-                role = self._roles.get(id(p))
-                shadow = norm_out = None
-                row_len = 0
-                if role is not None and pv.ndim == 2:
-                    model = self._model
-                    shadow = model.get_derived_buffer(f"{role}.bf16")
-                    if role == "W_D":
-                        norm_out = model.get_derived_buffer("W_D.norm")
-                        if norm_out is None:
-                            norm_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
-                        row_len = pv.shape[1] if pv.shape[1] % 4 == 0 else 0
-                        if row_len == 0:
-                            norm_out = None
+                role, shadow, norm_out = self._by_products(p, pv)
                 ops.adam_step(pv, gv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"],
-                              step=int(st["step"].item()), shadow_bf16=shadow, row_norm_out=norm_out, row_len=row_len)
-                # the kernel wrote through raw pointers: move the version counter like an in-place op would
-                torch.autograd.graph.increment_version(p)
-                if role is not None:
-                    if shadow is not None:
-                        self._model.set_derived(f"{role}.bf16", p, shadow)
-                    if norm_out is not None:
-                        self._model.set_derived("W_D.norm", p, norm_out)
+                              step=int(st["step"].item()), shadow_bf16=shadow, row_norm_out=norm_out,
+                              row_len=pv.shape[1] if norm_out is not None else 0)
+                self._publish(p, role, shadow, norm_out)
         return loss

@@ -40,6 +40,23 @@ class _Holder:
     code: ops.SparseCode = None
     pre: torch.Tensor = None
     scale: Optional[torch.Tensor] = None
+    defer_to: Optional["SparseAutoEncoder"] = None  # module whose optimiser consumes factored weight gradients
+
+
+class SparseRowGrad:
+    """Gradient of a feature-major [F, d] weight in factored form:
+    g[f, :] = sum over feature f's slots of coef[slot] * dense[token(slot), :].
+    Produced by the fused backward when the optimiser can consume it directly (HipAdam), so the
+    dense gradient never has to be written to HBM.  `dense()` materialises it on demand."""
+
+    def __init__(self, fi: ops.FeatureIndex, coef: torch.Tensor, dense_operand: torch.Tensor, n_features: int,
+                 bias_param: Optional[torch.Tensor] = None):
+        self.fi, self.coef, self.dense_operand, self.n_features, self.bias_param = fi, coef, dense_operand, n_features, bias_param
+
+    def dense(self):
+        """(rows [F, d] fp32, bias gradient [F] or None)"""
+        return ops.sparse_grad_rows(self.fi, self.coef, self.dense_operand, self.n_features,
+                                    want_bias=self.bias_param is not None)
 
 
 class _FusedTopKLoss(torch.autograd.Function):
@@ -67,6 +84,7 @@ class _FusedTopKLoss(torch.autograd.Function):
         ctx.code, ctx.x_op, ctx.grad_recon, ctx.dval = code, x_op, grad_recon, dval
         ctx.w_enc_op, ctx.w_dec_op = w_enc_op, w_dec_op
         ctx.has_b_D = b_D is not None
+        ctx.defer_to = holder.defer_to
         ctx.mark_non_differentiable(recon)
         return loss, recon
 
@@ -78,15 +96,32 @@ class _FusedTopKLoss(torch.autograd.Function):
         g = g_loss.to(torch.float32)
         coef_dec = code.val * g          # dW_D[f] = sum val * grad_recon[token]
         coef_enc = ctx.dval * g          # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
-        dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_recon, F)
-        dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_op, F, want_bias=True)
         db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
+        sae = ctx.defer_to
+        if sae is not None and getattr(sae.W_D, "_sparse_grad", None) is None and sae.W_D.grad is None \
+                and getattr(sae.W_E, "_sparse_grad", None) is None and sae.W_E.grad is None:
+            # hand the factored gradients to the optimiser; b_E's gradient is a by-product of its W_E pass
+            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, ctx.grad_recon, F)
+            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, ctx.x_op, F, bias_param=sae.b_E)
+            dW_D = dW_Et = db_E = None
+        else:
+            if sae is not None:  # a second backward before the optimiser ran: fall back to dense accumulation
+                for prm in (sae.W_D, sae.W_E):
+                    sg = getattr(prm, "_sparse_grad", None)
+                    if sg is not None:
+                        rows, bias = sg.dense()
+                        prm.grad = rows if prm is sae.W_D else rows.t()
+                        if bias is not None:
+                            sg.bias_param.grad = bias if sg.bias_param.grad is None else sg.bias_param.grad + bias
+                        prm._sparse_grad = None
+            dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_recon, F)
+            dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_op, F, want_bias=True)
         dx = None
         if ctx.needs_input_grad[0]:
             import dataclasses
             dx = ops.sparse_decode_fwd(dataclasses.replace(code, val=coef_enc), ctx.w_enc_op, None)
         dlabel = -ctx.grad_recon * g if ctx.needs_input_grad[1] else None
-        return dx, dlabel, None, dW_Et.t(), db_E, dW_D, db_D, None, None, None, None, None
+        return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None, None, None
 
 
 @register_sae_model("sae")
@@ -109,6 +144,9 @@ class SparseAutoEncoder(SparseDictionary):
         self.hook_reconstructed = HookPoint()
         # derived operands (bf16 shadows, row norms) keyed by name -> (param version, tensor)
         self._derived: dict[str, tuple[int, torch.Tensor]] = {}
+        # set by an optimiser that consumes SparseRowGrad (HipAdam): the fused backward then leaves W_E.grad /
+        # W_D.grad unset and attaches the factored gradient as `param._sparse_grad` instead
+        self.defer_weight_grads = False
 
     # ---- derived operands, refreshed when the parameter's version counter moves ----
     def _derive(self, name: str, param: torch.Tensor, make) -> torch.Tensor:
@@ -291,6 +329,7 @@ class SparseAutoEncoder(SparseDictionary):
             tok_w = m / m.sum()
         scale = self._decoder_norm_nograd() if self.cfg.sparsity_include_decoder_norm else None
         holder = _Holder()
+        holder.defer_to = self if self.defer_weight_grads and torch.is_grad_enabled() else None
         loss, recon = _FusedTopKLoss.apply(
             x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x,
             label.to(torch.float32).contiguous(), tok_w, self.W_E, self.b_E, self.W_D,

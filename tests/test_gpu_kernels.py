@@ -343,3 +343,31 @@ def test_adam_step_matches_torch(pkg, dev, n, row_len):
             assert rel_err(norms, p.cpu().view(-1, row_len).double().norm(dim=1)) < 1e-6
     st = opt.state[ref]
     assert rel_err(m, st["exp_avg"]) < 1e-6 and rel_err(v, st["exp_avg_sq"]) < 1e-6
+
+
+@pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (128, 4096, 512, 4), (40, 5120, 96, 3)])
+@pytest.mark.parametrize("dense_dtype", [torch.float32, torch.bfloat16])
+def test_adam_step_sparse_rows_equals_grad_rows_then_adam(pkg, dev, B, d, F, k, dense_dtype):
+    """the gradient-free route (rows rebuilt inside the Adam pass) gives the same bits as writing the
+    dense gradient rows first and running the plain Adam kernel on them"""
+    print(f"adam sparse rows B={B} d={d} F={F} k={k} {dense_dtype}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=d + B + 1)
+    fi = pkg.ops.build_feature_index(code)
+    g = torch.Generator().manual_seed(8)
+    dense = torch.randn(B, d, generator=g).to(dense_dtype).to(dev)
+    coef = torch.randn(code.n_slots, generator=g).to(dev)
+    p0 = torch.randn(F, d, generator=g).to(dev)
+    hyper = dict(lr=4e-4, beta1=0.9, beta2=0.999, eps=1e-8)
+    pa, ma, va = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    pb, mb, vb = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    sha, shb = torch.empty(F, d, dtype=torch.bfloat16, device=dev), torch.empty(F, d, dtype=torch.bfloat16, device=dev)
+    na, nb = torch.empty(F, device=dev), torch.empty(F, device=dev)
+    bias_b = torch.empty(F, device=dev)
+    for step in (1, 2):
+        rows, bias_a = pkg.ops.sparse_grad_rows(fi, coef, dense, F, want_bias=True)
+        pkg.ops.adam_step(pa, rows, ma, va, step=step, shadow_bf16=sha, row_norm_out=na, row_len=d, **hyper)
+        pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=step, shadow_bf16=shb, row_norm_out=nb,
+                                      bias_grad_out=bias_b, **hyper)
+        assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
+        assert torch.equal(sha, shb) and torch.equal(na, nb) and torch.equal(bias_a, bias_b)
+    assert not torch.equal(pa, p0)

@@ -161,3 +161,53 @@ def test_fused_step_then_adam_matches_oracle_adam(pkg, oracle, dev):
     want, got = ref.W_D.detach(), sae.W_D.detach().cpu()
     unchanged = (want == before["W_D"]).all(dim=1)
     assert unchanged.any() and torch.equal(got[unchanged], before["W_D"][unchanged])
+
+
+@pytest.mark.parametrize("amp", [False, True])
+def test_factored_gradients_match_dense_gradients(pkg, oracle, dev, amp):
+    """HipAdam consuming the factored weight gradients (no dense dW in memory) ends at the same
+    parameters, moments and derived operands as HipAdam fed dense gradients from autograd."""
+    results = []
+    for defer in (True, False):
+        sae, _, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=5, include_norm=True)
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae, defer_weight_grads=defer)
+        assert sae.defer_weight_grads == defer
+        gbatch = {k: v.to(dev) for k, v in batch.items()}
+        for _ in range(3):
+            if amp:
+                with torch.autocast("cuda", dtype=torch.bfloat16):
+                    loss = sae.compute_loss(gbatch, return_aux_data=False)
+            else:
+                loss = sae.compute_loss(gbatch, return_aux_data=False)
+            loss.backward()
+            if defer:
+                assert sae.W_D.grad is None and sae.W_E.grad is None and sae.W_D._sparse_grad is not None
+            else:
+                assert sae.W_D.grad is not None and sae.W_E.grad.shape == sae.W_E.shape
+            opt.step()
+            opt.zero_grad()
+            assert sae.W_D.grad is None and getattr(sae.W_D, "_sparse_grad", None) is None
+        results.append(({n: p.detach().clone() for n, p in sae.named_parameters()}, loss.item(),
+                        {n: opt.state[p]["exp_avg_sq"].clone() for n, p in sae.named_parameters()}))
+    (pa, la, va), (pb, lb, vb) = results
+    assert la == lb
+    for n in pa:
+        assert torch.equal(pa[n], pb[n]), n
+        assert torch.equal(va[n], vb[n]), n
+
+
+def test_materialize_grads_and_second_backward(pkg, oracle, dev):
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=6, include_norm=False)
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae)
+    gbatch = {k: v.to(dev) for k, v in batch.items()}
+    sae.compute_loss(gbatch)["loss"].backward()
+    opt.materialize_grads()
+    g1 = {n: p.grad.clone() for n, p in sae.named_parameters()}
+    assert g1["W_E"].shape == sae.W_E.shape and g1["W_E"].stride() == sae.W_E.stride()
+    opt.zero_grad()
+    # two backward passes before a step accumulate, as autograd would
+    sae.compute_loss(gbatch)["loss"].backward()
+    sae.compute_loss(gbatch)["loss"].backward()
+    opt.materialize_grads()
+    for n, p in sae.named_parameters():
+        assert torch.allclose(p.grad, 2 * g1[n], rtol=1e-6, atol=1e-12), n
