@@ -41,6 +41,9 @@ def algorithmic_work(B: int) -> dict:
         "sparse_grad_rows[bf16 dense]": ("hbm", F * d * 4),              # dW_E^T: likewise
         "adam_step[matrix]": ("hbm", F * d * 30),                        # g,p,m,v read; p,m,v written; bf16 shadow written
         "adam_step[vector]": ("hbm", (F + d) / 2 * 28),                  # the two biases, averaged
+        # Adam with the gradient rows rebuilt in registers: p,m,v read; p,m,v written; bf16 shadow written
+        "adam_step_sparse_rows[f32 dense]": ("hbm", F * d * 26),
+        "adam_step_sparse_rows[bf16 dense]": ("hbm", F * d * 26),
         "build_feature_index": ("hbm", B * k * 16 + F * 12),
         "cast_f32_to_bf16": ("hbm", B * d * 6),
         "col_sum": ("hbm", B * d * 4),

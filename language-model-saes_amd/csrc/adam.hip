@@ -25,20 +25,20 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
   const int64_t n4 = n >> 2;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    float4 pp = reinterpret_cast<float4 *>(p)[i];
-    const float4 gg = reinterpret_cast<const float4 *>(g)[i];
-    float4 mm = reinterpret_cast<float4 *>(m)[i];
-    float4 vv = reinterpret_cast<float4 *>(v)[i];
+    float4 pp = load_stream(p, i);
+    const float4 gg = load_stream(g, i);
+    float4 mm = load_stream(m, i);
+    float4 vv = load_stream(v, i);
     adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
     adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
-    reinterpret_cast<float4 *>(p)[i] = pp;
-    reinterpret_cast<float4 *>(m)[i] = mm;
-    reinterpret_cast<float4 *>(v)[i] = vv;
+    store_stream(p, i, pp);
+    store_stream(m, i, mm);
+    store_stream(v, i, vv);
     if (shadow) {
       uint2 o;
       o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
       o.y = (uint32_t)f32_to_bf16_bits(pp.z) | ((uint32_t)f32_to_bf16_bits(pp.w) << 16);
-      reinterpret_cast<uint2 *>(shadow)[i] = o;
+      store_stream(shadow, i, o);
     }
   }
   const int64_t t = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -60,21 +60,21 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
   float sq = 0.f;
   for (int i = threadIdx.x; i < (row_len >> 2); i += 256) {
     const int64_t q = base4 + i;
-    float4 pp = reinterpret_cast<float4 *>(p)[q];
-    const float4 gg = reinterpret_cast<const float4 *>(g)[q];
-    float4 mm = reinterpret_cast<float4 *>(m)[q];
-    float4 vv = reinterpret_cast<float4 *>(v)[q];
+    float4 pp = load_stream(p, q);
+    const float4 gg = load_stream(g, q);
+    float4 mm = load_stream(m, q);
+    float4 vv = load_stream(v, q);
     adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
     adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
-    reinterpret_cast<float4 *>(p)[q] = pp;
-    reinterpret_cast<float4 *>(m)[q] = mm;
-    reinterpret_cast<float4 *>(v)[q] = vv;
+    store_stream(p, q, pp);
+    store_stream(m, q, mm);
+    store_stream(v, q, vv);
     sq = fmaf(pp.x, pp.x, sq); sq = fmaf(pp.y, pp.y, sq); sq = fmaf(pp.z, pp.z, sq); sq = fmaf(pp.w, pp.w, sq);
     if (shadow) {
       uint2 o;
       o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
       o.y = (uint32_t)f32_to_bf16_bits(pp.z) | ((uint32_t)f32_to_bf16_bits(pp.w) << 16);
-      reinterpret_cast<uint2 *>(shadow)[q] = o;
+      store_stream(shadow, q, o);
     }
   }
   const float tot = block_sum<4>(sq, red);
@@ -163,9 +163,9 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < 4; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
-        pp[u] = reinterpret_cast<const float4 *>(p)[base4 + seg];
-        mm[u] = reinterpret_cast<const float4 *>(m)[base4 + seg];
-        vv[u] = reinterpret_cast<const float4 *>(v)[base4 + seg];
+        pp[u] = load_stream(p, base4 + seg);
+        mm[u] = load_stream(m, base4 + seg);
+        vv[u] = load_stream(v, base4 + seg);
       }
       g[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
@@ -196,16 +196,16 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       if (seg < n_seg) {
         adam_one(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_one(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
         adam_one(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_one(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
-        reinterpret_cast<float4 *>(p)[base4 + seg] = pp[u];
-        reinterpret_cast<float4 *>(m)[base4 + seg] = mm[u];
-        reinterpret_cast<float4 *>(v)[base4 + seg] = vv[u];
+        store_stream(p, base4 + seg, pp[u]);
+        store_stream(m, base4 + seg, mm[u]);
+        store_stream(v, base4 + seg, vv[u]);
         sq = fmaf(pp[u].x, pp[u].x, sq); sq = fmaf(pp[u].y, pp[u].y, sq);
         sq = fmaf(pp[u].z, pp[u].z, sq); sq = fmaf(pp[u].w, pp[u].w, sq);
         if (shadow) {
           uint2 o;
           o.x = (uint32_t)f32_to_bf16_bits(pp[u].x) | ((uint32_t)f32_to_bf16_bits(pp[u].y) << 16);
           o.y = (uint32_t)f32_to_bf16_bits(pp[u].z) | ((uint32_t)f32_to_bf16_bits(pp[u].w) << 16);
-          reinterpret_cast<uint2 *>(shadow)[base4 + seg] = o;
+          store_stream(shadow, base4 + seg, o);
         }
       }
     }

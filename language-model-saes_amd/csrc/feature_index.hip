@@ -4,7 +4,7 @@
 // weight gradients need the transpose: for every feature, the slots that name it.
 //
 //   count   one global atomic per valid slot into counts[F]; also records slot -> token
-//   scan    exclusive prefix sum over counts -> feat_ptr[F + 1]
+//   scan    exclusive prefix sum over counts -> feat_ptr[F + 1] (tile sums, scan of sums, finish)
 //   fill    slot ids dropped into their feature's segment through a per-feature cursor
 //   order   every segment is put into ascending slot order, so the result (and every sum
 //           taken over a segment afterwards) is independent of the order in which the
@@ -44,33 +44,75 @@ __global__ __launch_bounds__(FI_THREADS) void fi_count_kernel(const int32_t *__r
   }
 }
 
-// Single-workgroup exclusive scan: thread t owns a contiguous run of ceil(F/1024) counters.
-__global__ __launch_bounds__(1024) void fi_scan_kernel(const int32_t *__restrict__ counts, int F,
-                                                       int32_t *__restrict__ feat_ptr,
-                                                       int32_t *__restrict__ cursor) {
-  __shared__ int32_t part[1024];
-  const int tid = threadIdx.x;
-  const int per = (F + 1023) / 1024;
-  const int lo = tid * per, hi = min(F, lo + per);
-  int s = 0;
-  for (int i = lo; i < hi; ++i) s += counts[i];
-  part[tid] = s;
+// Exclusive scan of counts[F] in three small launches: per-tile sums (1024 counters per
+// workgroup, coalesced), a one-workgroup scan of the tile sums, per-tile scan + tile offset.
+constexpr int SCAN_TILE = 1024;  // counters per workgroup (256 threads x 4)
+
+__device__ __forceinline__ int block_excl_scan_256(int v, int *lds_wave, int &total) {
+  // exclusive scan over 256 threads; lds_wave holds 4 ints
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += t;
+  }
   __syncthreads();
-  // Hillis-Steele inclusive scan over 1024 partials
-  for (int o = 1; o < 1024; o <<= 1) {
-    const int v = tid >= o ? part[tid - o] : 0;
-    __syncthreads();
-    part[tid] += v;
+  if (lane == 63) lds_wave[w] = incl;
+  __syncthreads();
+  int base = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) base += (i < w) ? lds_wave[i] : 0;
+  total = lds_wave[0] + lds_wave[1] + lds_wave[2] + lds_wave[3];
+  return base + incl - v;
+}
+
+__global__ __launch_bounds__(256) void fi_tile_sum_kernel(const int32_t *__restrict__ counts, int F,
+                                                          int32_t *__restrict__ tile_sums) {
+  __shared__ int lds_wave[4];
+  const int base = blockIdx.x * SCAN_TILE + threadIdx.x * 4;
+  int s = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) s += (base + e < F) ? counts[base + e] : 0;
+  int total;
+  block_excl_scan_256(s, lds_wave, total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// one workgroup; n_tiles is small (F / 1024), handled in chunks of 256
+__global__ __launch_bounds__(256) void fi_tile_scan_kernel(int32_t *__restrict__ tile_sums, int n_tiles,
+                                                           int32_t *__restrict__ feat_ptr, int F) {
+  __shared__ int lds_wave[4];
+  int carry = 0;
+  for (int c0 = 0; c0 < n_tiles; c0 += 256) {
+    const int i = c0 + threadIdx.x;
+    const int v = i < n_tiles ? tile_sums[i] : 0;
+    int total;
+    const int ex = block_excl_scan_256(v, lds_wave, total);
+    if (i < n_tiles) tile_sums[i] = carry + ex;
+    carry += total;
     __syncthreads();
   }
-  int run = part[tid] - s;  // exclusive prefix of my run
-  for (int i = lo; i < hi; ++i) {
-    const int c = counts[i];
-    feat_ptr[i] = run;
-    cursor[i] = run;
-    run += c;
+  if (threadIdx.x == 0) feat_ptr[F] = carry;
+}
+
+__global__ __launch_bounds__(256) void fi_tile_finish_kernel(const int32_t *__restrict__ counts, int F,
+                                                             const int32_t *__restrict__ tile_offsets,
+                                                             int32_t *__restrict__ feat_ptr,
+                                                             int32_t *__restrict__ cursor) {
+  __shared__ int lds_wave[4];
+  const int base = blockIdx.x * SCAN_TILE + threadIdx.x * 4;
+  int c[4];
+  int s = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { c[e] = (base + e < F) ? counts[base + e] : 0; s += c[e]; }
+  int total;
+  int run = tile_offsets[blockIdx.x] + block_excl_scan_256(s, lds_wave, total);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (base + e < F) { feat_ptr[base + e] = run; cursor[base + e] = run; }
+    run += c[e];
   }
-  if (tid == 1023) feat_ptr[F] = part[1023];
 }
 
 __global__ __launch_bounds__(FI_THREADS) void fi_fill_kernel(const int32_t *__restrict__ idx,
@@ -214,8 +256,8 @@ __global__ __launch_bounds__(FI_THREADS) void sparse_grad_rows_kernel(
 extern "C" int64_t sae_feature_index_workspace_bytes(int64_t B, int64_t F, int64_t n_slots) {
   (void)B;
   if (F <= 0 || n_slots <= 0) return 0;
-  // counts[F] + cursor[F] + ordering scratch[n_slots]
-  return (int64_t)sizeof(int32_t) * (2 * F + n_slots) + 256;
+  // counts[F] + cursor[F] + unordered slots[n_slots] + scan tile sums[ceil(F / 1024)]
+  return (int64_t)sizeof(int32_t) * (2 * F + n_slots + (F + 1023) / 1024) + 256;
 }
 
 extern "C" int sae_build_feature_index(const int32_t *idx, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
@@ -234,11 +276,15 @@ extern "C" int sae_build_feature_index(const int32_t *idx, const int64_t *row_of
   int32_t *counts = reinterpret_cast<int32_t *>(workspace);
   int32_t *cursor = counts + F;
   int32_t *unordered = cursor + F;
+  int32_t *tile_sums = unordered + n_slots;
   hipLaunchKernelGGL(fi_zero_kernel, dim3((unsigned)((F + 255) / 256)), dim3(256), 0, st, counts, F);
   const unsigned tok_blocks = (unsigned)((B + (FI_THREADS / 64) - 1) / (FI_THREADS / 64));
   hipLaunchKernelGGL(fi_count_kernel, dim3(tok_blocks), dim3(FI_THREADS), 0, st, idx, row_off, row_nnz, (int)B, (int)F,
                      counts, slot_tok);
-  hipLaunchKernelGGL(fi_scan_kernel, dim3(1), dim3(1024), 0, st, counts, (int)F, feat_ptr, cursor);
+  const int n_tiles = (int)((F + SCAN_TILE - 1) / SCAN_TILE);
+  hipLaunchKernelGGL(fi_tile_sum_kernel, dim3(n_tiles), dim3(256), 0, st, counts, (int)F, tile_sums);
+  hipLaunchKernelGGL(fi_tile_scan_kernel, dim3(1), dim3(256), 0, st, tile_sums, n_tiles, feat_ptr, (int)F);
+  hipLaunchKernelGGL(fi_tile_finish_kernel, dim3(n_tiles), dim3(256), 0, st, counts, (int)F, tile_sums, feat_ptr, cursor);
   hipLaunchKernelGGL(fi_fill_kernel, dim3(tok_blocks), dim3(FI_THREADS), 0, st, idx, row_off, row_nnz, (int)B, (int)F,
                      cursor, unordered);
   const unsigned feat_blocks = (unsigned)((F + (FI_THREADS / 64) - 1) / (FI_THREADS / 64));
