@@ -79,7 +79,7 @@ int sae_col_sum(const float *src, float *out, int64_t B, int64_t n, int accumula
  * x [B, d] and w_enc_t [F, d] share in_dtype (SAE_BF16: bf16 operands, fp32 accumulate;
  * SAE_F32: fp32 MFMA).  pre [B, F] is written as out_dtype; SAE_BF16 rounds the fp32
  * accumulator to bf16, which is what the autocast matmul returns.
- * Requires d % 32 == 0 (bf16) / d % 16 == 0 (fp32); B and F arbitrary (edge tiles masked).
+ * Requires d % 64 == 0 (bf16) / d % 32 == 0 (fp32); B and F arbitrary (edge tiles masked).
  * Replaces `x @ self.W_E` (models/sae.py:324). */
 int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, int64_t B, int64_t d, int64_t F,
                      int in_dtype, int out_dtype, void *stream);

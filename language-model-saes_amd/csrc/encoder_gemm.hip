@@ -4,19 +4,24 @@
 // (or 4 fp32) one lane feeds to a matrix-core instruction.
 //
 // Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile and
-// walks K in stages of 64 bytes per row (32 bf16 / 16 fp32).  Waves are arranged 2 x 4: each owns
-// 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32 accumulators per lane).
+// walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32): a full cache line per row, which the
+// L2 serves at twice the rate of half lines (measured 27 vs 13 TB/s aggregate L2->LDS).  Waves are
+// arranged 2 x 4: each owns 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32
+// accumulators per lane).
 //
-// Pipeline: four stages of (256 + 256) rows x 64 bytes = 32 KiB live in LDS (128 of the CU's
-// 160 KiB).  Stages are filled by LDS-direct loads (global_load_lds_dwordx4: the data never
-// passes through VGPRs), three stages ahead of the one being consumed; one s_waitcnt vmcnt(8) +
-// s_barrier per stage both publishes the stage that just landed and frees the one just consumed.
-// The loads are issued through inline assembly so that the compiler's wait-count insertion does
-// not serialise them against the LDS reads of the other stages.
+// Pipeline: LDS (all 160 KiB of the CU) is a ring of five 32 KiB slots; a slot holds one operand's
+// slab (256 rows x 128 bytes).  Load units alternate W slab j, x slab j, W slab j+1, ...; unit t
+// lives in slot t % 5.  Slots are filled by LDS-direct loads (global_load_lds_dwordx4: the data
+// never passes through VGPRs).  While slab j is consumed, x slab j+1 and W slab j+2 are in flight:
+// the weights, which come from HBM, get the longer lead; the activations mostly hit L2 / Infinity
+// Cache.  One s_waitcnt vmcnt(4) + s_barrier per slab publishes the slab that just landed and
+// frees the two slots of the slab just consumed.  The loads are issued through inline assembly so
+// that the compiler's wait-count insertion does not serialise them against LDS reads of other
+// slots.
 //
-// LDS layout: row r of a stage is 64 bytes = 4 chunks of 16 bytes; chunk c is stored at physical
-// chunk c ^ ((r >> 2) & 3).  A group of 16 lanes then covers 256 distinct bytes when MFMA
-// fragments are read (16 rows, one logical chunk): zero bank conflicts (SQ_LDS_BANK_CONFLICT = 0).
+// LDS layout: row r of a slot is 128 bytes = 8 chunks of 16 bytes; chunk c is stored at physical
+// chunk c ^ ((r >> 1) & 7).  A group of 16 lanes then covers 256 distinct bytes when MFMA
+// fragments are read (16 rows, one logical chunk): no bank conflicts (SQ_LDS_BANK_CONFLICT = 0).
 // An LDS-direct load writes 1 KiB linearly (lane l -> base + 16 l), so the swizzle is applied on
 // the global side: lane l fetches the logical chunk that belongs at its physical slot.
 //
@@ -24,9 +29,9 @@
 // which leaves every lane holding 4 consecutive features of one token: the epilogue packs them
 // into one 8-byte (bf16) or 16-byte (fp32) store.
 //
-// Workgroups are numbered so that consecutive ids land on the 8 XCDs round-robin, and the
-// workgroups of one XCD walk all token tiles of one feature tile before moving on: a W_E stage
-// is pulled from HBM once per XCD-L2 and shared by the token tiles.
+// Workgroup order: consecutive ids land on the 8 XCDs round-robin; within an XCD, 32 consecutive
+// workgroups (one per CU) cover 8 token tiles x 4 feature tiles, so every slab in an XCD's L2 is
+// shared by 4 or 8 resident workgroups (best measured of 16x2, 8x4).
 //
 // Rows beyond B or F are clamped to the last valid row when loading (their products land in
 // accumulators that the epilogue never stores), so the main loop has no bounds checks.
@@ -34,7 +39,7 @@
 
 namespace sae {
 
-#define WAITCNT_VM8 ((8 & 0xf) | (0x7 << 4) | (0xf << 8) | ((8 >> 4) << 14))
+#define WAITCNT_VM4 ((4 & 0xf) | (0x7 << 4) | (0xf << 8) | ((4 >> 4) << 14))
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -42,12 +47,13 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 constexpr int GEMM_BM = 256;       // tokens per workgroup tile
 constexpr int GEMM_BN = 256;       // features per workgroup tile
-constexpr int GEMM_SLAB = 64;      // bytes of K per row per stage
-constexpr int GEMM_STAGES = 4;
+constexpr int GEMM_SLAB = 128;     // bytes of K per row per slab
+constexpr int GEMM_SLOTS = 5;      // ring of 32 KiB slots, each holding one operand's slab
 constexpr int GEMM_THREADS = 512;
-constexpr int GEMM_LDS_BYTES = GEMM_STAGES * (GEMM_BM + GEMM_BN) * GEMM_SLAB;
+constexpr int GEMM_SLOT_BYTES = 256 * GEMM_SLAB;
+constexpr int GEMM_LDS_BYTES = GEMM_SLOTS * GEMM_SLOT_BYTES;
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 2) & 3)) << 4); }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 template <bool BF16_IN>
 __device__ __forceinline__ void mma_chunk(const u32x4 &wf, const u32x4 &xf, f32x16_t &acc) {
@@ -71,25 +77,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     int row_bytes /* d * sizeof(elem) */, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   // [x slab 0][x slab 1][w slab 0][w slab 1]
-  constexpr int X_BYTES = GEMM_BM * GEMM_SLAB, W_BYTES = GEMM_BN * GEMM_SLAB;
 
   // ---- XCD-aware tile assignment ----
   const int bid = blockIdx.x;
-  const int total = tiles_m * tiles_n;
   int tile_m, tile_n;
   {
     const int xcd = bid & 7, slot = bid >> 3;
-    const int full = (tiles_n >> 3) << 3;  // feature tiles that split evenly over 8 XCDs
-    const int lin_limit = full * tiles_m;
-    if (bid < lin_limit) {
-      tile_n = (slot / tiles_m) * 8 + xcd;
-      tile_m = slot % tiles_m;
-    } else {  // remainder: plain row-major walk
-      const int r = bid - lin_limit;
-      tile_n = full + r / tiles_m;
-      tile_m = r % tiles_m;
-    }
-    (void)total;
+    // per XCD: groups of 32 consecutive workgroups cover 8 token tiles x 4 feature tiles
+    const int grp = slot >> 5, in = slot & 31;
+    const int m_groups = (tiles_m + 7) >> 3;           // groups of 8 token tiles (last one may be partial)
+    const int n_grp = grp / m_groups, m_half = grp % m_groups;
+    tile_m = m_half * 8 + (in & 7);
+    tile_n = (n_grp * 4 + (in >> 3)) * 8 + xcd;
+    if (tile_n >= tiles_n || tile_m >= tiles_m) return;
   }
   const int m0 = tile_m * GEMM_BM, n0 = tile_n * GEMM_BN;
 
@@ -97,20 +97,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
   const int wm = wave >> 2, wn = wave & 3;
 
   // ---- global -> LDS staging assignment: 8 lanes cover one 128-byte row slab ----
-  const int ld_phys = lane & 3;  // physical 16-byte chunk this lane fills
-  const char *xg[2];
-  const char *wg[2];
-  bool xok[2], wok[2];
-  int lds_off[2];
+  const int ld_phys = lane & 7;  // physical 16-byte chunk this lane fills
+  const char *xg[4];
+  const char *wg[4];
+  bool xok[4], wok[4];
+  int lds_off[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = wave * 32 + i * 16 + (lane >> 2);
-    const int ld_chunk = ld_phys ^ ((r >> 2) & 3);  // logical chunk that lives at this physical slot
+  for (int i = 0; i < 4; ++i) {
+    const int r = wave * 32 + i * 8 + (lane >> 3);
+    const int ld_chunk = ld_phys ^ ((r >> 1) & 7);  // logical chunk that lives at this physical slot
     xok[i] = (m0 + r) < M;
     wok[i] = (n0 + r) < N;
     xg[i] = x + (size_t)(xok[i] ? (m0 + r) : (M - 1)) * row_bytes + ld_chunk * 16;
     wg[i] = w + (size_t)(wok[i] ? (n0 + r) : (N - 1)) * row_bytes + ld_chunk * 16;
-    lds_off[i] = (wave * 32 + i * 16) * GEMM_SLAB;  // wave-uniform base of the 1 KiB this load fills
+    lds_off[i] = (wave * 32 + i * 8) * GEMM_SLAB;  // wave-uniform base of the 1 KiB this load fills
   }
 
   f32x16_t acc[2][4];  // [feature sub-tile][token sub-tile]
@@ -131,29 +131,36 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
 #else
 #define LDS_DMA16(GPTR, LDSADDR) ((void)0)
 #endif
-#define LOAD_SLAB_TO_LDS(SLAB, BUF)                                                                      \
-  _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                       \
-    LDS_DMA16(xg[i] + (size_t)(SLAB) * GEMM_SLAB, lds_base + (BUF) * X_BYTES + lds_off[i]);             \
-    LDS_DMA16(wg[i] + (size_t)(SLAB) * GEMM_SLAB, lds_base + GEMM_STAGES * X_BYTES + (BUF) * W_BYTES + lds_off[i]); \
+  // unit t of the load sequence: t even -> W slab t/2, t odd -> x slab (t-1)/2; it lives in slot t % 5
+#define LOAD_UNIT(T)                                                                                     \
+  {                                                                                                      \
+    const int t_ = (T);                                                                                  \
+    int slab_ = t_ >> 1;                                                                                 \
+    slab_ = slab_ < n_slabs ? slab_ : n_slabs - 1; /* tail: harmless re-read */                          \
+    const uint32_t slot_ = lds_base + (uint32_t)(t_ % GEMM_SLOTS) * GEMM_SLOT_BYTES;                     \
+    if (t_ & 1) {                                                                                        \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) LDS_DMA16(xg[i] + (size_t)slab_ * GEMM_SLAB, slot_ + lds_off[i]); \
+    } else {                                                                                             \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) LDS_DMA16(wg[i] + (size_t)slab_ * GEMM_SLAB, slot_ + lds_off[i]); \
+    }                                                                                                    \
   }
-  // prologue: stages 0..2 in flight
-  LOAD_SLAB_TO_LDS(0, 0)
-  LOAD_SLAB_TO_LDS(n_slabs > 1 ? 1 : 0, 1)
-  LOAD_SLAB_TO_LDS(n_slabs > 2 ? 2 : 0, 2)
+  // prologue: W0 x0 W1 x1 W2 in flight
+  LOAD_UNIT(0) LOAD_UNIT(1) LOAD_UNIT(2) LOAD_UNIT(3) LOAD_UNIT(4)
 
   const int frag_row = lane & 31, frag_half = lane >> 5;
   for (int slab = 0; slab < n_slabs; ++slab) {
-    const int buf = slab & (GEMM_STAGES - 1);
-    // my loads of this slab have landed when at most the two younger stages (8 loads) are outstanding
-    __builtin_amdgcn_s_waitcnt(WAITCNT_VM8);
-    __builtin_amdgcn_s_barrier();  // everyone's part of this slab landed; everyone is done reading the previous slab
-    const int nxt = slab + 3 < n_slabs ? slab + 3 : n_slabs - 1;  // tail re-reads the last slab (never used)
-    LOAD_SLAB_TO_LDS(nxt, (slab + 3) & (GEMM_STAGES - 1))
+    // units 2*slab and 2*slab+1 must have landed; at most one younger unit (4 loads) may be outstanding
+    __builtin_amdgcn_s_waitcnt(WAITCNT_VM4);
+    __builtin_amdgcn_s_barrier();  // everyone's part landed; everyone is done with the previous slab's two slots
+    if (slab >= 1) {
+      LOAD_UNIT(2 * slab + 3)  // x slab+1  -> slot freed by W slab-1
+      LOAD_UNIT(2 * slab + 4)  // W slab+2  -> slot freed by x slab-1
+    }
     __builtin_amdgcn_sched_barrier(0);
-    const char *lx = lds + buf * X_BYTES;
-    const char *lw = lds + GEMM_STAGES * X_BYTES + buf * W_BYTES;
+    const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
+    const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {  // 2 MFMA k-steps per stage (32 bytes of K each)
+    for (int s = 0; s < 4; ++s) {  // 4 MFMA k-steps per slab (32 bytes of K each)
       const int chunk = 2 * s + frag_half;
       u32x4 wf[2], xf[4];
 #pragma unroll
@@ -224,7 +231,9 @@ static int launch_gemm(const void *x, const void *w, void *out, int64_t B, int64
                                      hipGetErrorString(e));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
+  // grid: 8 XCDs x (token tiles padded to 8) x (feature tiles per XCD padded to 4); padding workgroups exit at once
+  const int m_pad = (tiles_m + 7) / 8 * 8, n_local_pad = ((tiles_n + 7) / 8 + 3) / 4 * 4;
+  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
                      (const char *)w, out, (int)B, (int)F, (int)(d * esz), tiles_m, tiles_n);
   return check_launch("encoder_gemm");
 }
@@ -239,7 +248,7 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
   SAE_REQUIRE(in_dtype == SAE_F32 || in_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad in_dtype %d", in_dtype);
   SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm: bad out_dtype %d", out_dtype);
   SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm: size too large");
-  const int64_t per_slab = in_dtype == SAE_BF16 ? 32 : 16;  // elements in one 64-byte stage row
+  const int64_t per_slab = in_dtype == SAE_BF16 ? 64 : 32;
   SAE_REQUIRE(d % per_slab == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm: d_model=%lld must be a multiple of %lld",
               (long long)d, (long long)per_slab);
   SAE_REQUIRE((((uintptr_t)x | (uintptr_t)w_enc_t | (uintptr_t)pre) & 15) == 0, SAE_ERR_INVALID_ARG,

@@ -30,7 +30,7 @@ def code_to_rows(code):
 # encoder GEMM
 # ---------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (64, 768, 6144), (1, 64, 8), (513, 256, 260), (40, 16, 24), (70, 48, 300)])
+@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (64, 768, 6144), (1, 64, 8), (513, 256, 260), (40, 32, 24), (70, 96, 300), (2100, 64, 520), (300, 32, 9000)])
 def test_encoder_gemm_fp32(pkg, dev, B, d, F):
     print(f"gemm fp32 B={B} d={d} F={F}", flush=True)
     g = torch.Generator().manual_seed(B * 7 + F)
@@ -41,7 +41,7 @@ def test_encoder_gemm_fp32(pkg, dev, B, d, F):
     assert rel_err(pre, want) < FP32_TOL
 
 
-@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (512, 2048, 4096), (33, 64, 72), (20, 32, 16), (100, 96, 520)])
+@pytest.mark.parametrize("B,d,F", [(256, 64, 256), (300, 128, 1000), (512, 2048, 4096), (33, 64, 72), (20, 64, 16), (100, 192, 520), (2304, 128, 300)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_encoder_gemm_bf16(pkg, dev, B, d, F, out_dtype):
     print(f"gemm bf16 B={B} d={d} F={F} out={out_dtype}", flush=True)
