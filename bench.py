@@ -74,7 +74,8 @@ def gpu_step_bench(args):
         sae.b_E.zero_()
         sae.b_D.copy_(x.mean(0))
     batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
-    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae)
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae,
+                       overlap_decoder_update=args.overlap)
 
     def step():
         with torch.autocast("cuda", dtype=torch.bfloat16):
@@ -145,6 +146,7 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=512)
     ap.add_argument("--cpu-sample-features", type=int, default=32768)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overlap", action="store_true", help="run the decoder Adam pass on a second stream, overlapping the next GEMM")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives are part of it); run with --gpus 1",

@@ -152,16 +152,30 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     // units 2*slab and 2*slab+1 must have landed; at most one younger unit (4 loads) may be outstanding
     __builtin_amdgcn_s_waitcnt(WAITCNT_VM4);
     __builtin_amdgcn_s_barrier();  // everyone's part landed; everyone is done with the previous slab's two slots
-    if (slab >= 1) {
-      LOAD_UNIT(2 * slab + 3)  // x slab+1  -> slot freed by W slab-1
-      LOAD_UNIT(2 * slab + 4)  // W slab+2  -> slot freed by x slab-1
-    }
+    // units issued while this slab is consumed: x slab+1 -> slot freed by W slab-1, W slab+2 -> slot freed by
+    // x slab-1.  Two of the eight loads per k-step, so that requests trickle instead of bursting.
+    const int tA = 2 * slab + 3, tB = 2 * slab + 4;
+    int sA = tA >> 1; sA = sA < n_slabs ? sA : n_slabs - 1;
+    int sB = tB >> 1; sB = sB < n_slabs ? sB : n_slabs - 1;
+    const uint32_t slotA = lds_base + (uint32_t)(tA % GEMM_SLOTS) * GEMM_SLOT_BYTES;
+    const uint32_t slotB = lds_base + (uint32_t)(tB % GEMM_SLOTS) * GEMM_SLOT_BYTES;
     __builtin_amdgcn_sched_barrier(0);
     const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
     const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {  // 4 MFMA k-steps per slab (32 bytes of K each)
       const int chunk = 2 * s + frag_half;
+      if (slab >= 1) {
+        // x unit in k-steps 0-1, W unit in k-steps 2-3: the W loads stay the four youngest, which is what
+        // the vmcnt(4) at the top of the next slab relies on
+        if (s < 2) {
+          LDS_DMA16(xg[2 * s] + (size_t)sA * GEMM_SLAB, slotA + lds_off[2 * s]);
+          LDS_DMA16(xg[2 * s + 1] + (size_t)sA * GEMM_SLAB, slotA + lds_off[2 * s + 1]);
+        } else {
+          LDS_DMA16(wg[2 * s - 4] + (size_t)sB * GEMM_SLAB, slotB + lds_off[2 * s - 4]);
+          LDS_DMA16(wg[2 * s - 3] + (size_t)sB * GEMM_SLAB, slotB + lds_off[2 * s - 3]);
+        }
+      }
       u32x4 wf[2], xf[4];
 #pragma unroll
       for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));

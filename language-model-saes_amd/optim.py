@@ -20,6 +20,14 @@ from torch.optim import Optimizer
 from . import ops
 
 
+class _null_ctx:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
 def _flat_view(p: torch.Tensor) -> torch.Tensor:
     """A contiguous view over p's memory (p itself, or its transpose for feature-major 2-D weights)."""
     if p.is_contiguous():
@@ -31,7 +39,7 @@ def _flat_view(p: torch.Tensor) -> torch.Tensor:
 
 class HipAdam(Optimizer):
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, model=None,
-                 defer_weight_grads: bool = True):
+                 defer_weight_grads: bool = True, overlap_decoder_update: bool = False):
         if lr < 0.0 or eps < 0.0 or not (0.0 <= betas[0] < 1.0) or not (0.0 <= betas[1] < 1.0):
             raise ValueError("invalid Adam hyper-parameters")
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps))
@@ -44,6 +52,17 @@ class HipAdam(Optimizer):
                     self._roles[id(p)] = name
             if defer_weight_grads and hasattr(model, "defer_weight_grads"):
                 model.defer_weight_grads = True
+        # Optional pipelining: the decoder's update (HBM-bound) runs on a second stream and overlaps the
+        # next step's encoder GEMM (matrix-core / L2-bound), which reads only W_E.  The model waits for it
+        # before anything of its own reads W_D, its bf16 copy or its row norms; code that touches W_D
+        # outside the model must call `join()` first.
+        self._overlap = bool(overlap_decoder_update) and model is not None and hasattr(model, "set_pending_update")
+        self._side_stream = None
+
+    def join(self) -> None:
+        """Make the current stream wait for an overlapped decoder update still in flight."""
+        if self._model is not None and hasattr(self._model, "wait_pending_update"):
+            self._model.wait_pending_update()
 
     def zero_grad(self, set_to_none: bool = True):
         super().zero_grad(set_to_none=set_to_none)
@@ -103,29 +122,47 @@ class HipAdam(Optimizer):
             with torch.enable_grad():
                 loss = closure()
         # pass 1: weights whose gradient arrives in factored form (also yields the encoder-bias gradient)
+        deferred = []
         for group in self.param_groups:
-            b1, b2 = group["betas"]
             for p in group["params"]:
-                sg = getattr(p, "_sparse_grad", None)
-                if sg is None:
-                    continue
-                if p.grad is not None:
-                    raise RuntimeError("parameter has both a dense and a factored gradient")
-                st = self._state(p)
-                st["step"] += 1
-                pv = _flat_view(p)
-                mv, vv = _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"])
-                role, shadow, norm_out = self._by_products(p, pv)
-                bias_out = None
-                if sg.bias_param is not None:
-                    bias_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
+                if getattr(p, "_sparse_grad", None) is not None:
+                    deferred.append((group, p))
+        # the decoder goes last so that, when overlapped, it has the stream's tail to itself
+        deferred.sort(key=lambda gp: self._roles.get(id(gp[1])) == "W_D")
+        for group, p in deferred:
+            b1, b2 = group["betas"]
+            sg = p._sparse_grad
+            if p.grad is not None:
+                raise RuntimeError("parameter has both a dense and a factored gradient")
+            st = self._state(p)
+            st["step"] += 1
+            pv = _flat_view(p)
+            mv, vv = _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"])
+            role, shadow, norm_out = self._by_products(p, pv)
+            bias_out = None
+            if sg.bias_param is not None:
+                bias_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
+            side = None
+            if self._overlap and role == "W_D" and bias_out is None:
+                if self._side_stream is None:
+                    self._side_stream = torch.cuda.Stream(device=p.device)
+                side = self._side_stream
+                side.wait_stream(torch.cuda.current_stream(p.device))
+                for t in (sg.fi.feat_ptr, sg.fi.feat_slot, sg.fi.slot_tok, sg.coef, sg.dense_operand):
+                    t.record_stream(side)  # step-local tensors: keep their memory until the side stream is done
+            with torch.cuda.stream(side) if side is not None else _null_ctx():
                 ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
                                           eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
                                           row_norm_out=norm_out, bias_grad_out=bias_out)
-                if bias_out is not None:
-                    sg.bias_param.grad = bias_out if sg.bias_param.grad is None else sg.bias_param.grad + bias_out
-                p._sparse_grad = None
-                self._publish(p, role, shadow, norm_out)
+                if side is not None:
+                    ev = torch.cuda.Event()
+                    ev.record(side)
+            if bias_out is not None:
+                sg.bias_param.grad = bias_out if sg.bias_param.grad is None else sg.bias_param.grad + bias_out
+            p._sparse_grad = None
+            self._publish(p, role, shadow, norm_out)
+            if side is not None:
+                self._model.set_pending_update(ev)
         # pass 2: everything with a dense gradient
         for group in self.param_groups:
             b1, b2 = group["betas"]

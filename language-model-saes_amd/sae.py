@@ -41,6 +41,7 @@ class _Holder:
     pre: torch.Tensor = None
     scale: Optional[torch.Tensor] = None
     defer_to: Optional["SparseAutoEncoder"] = None  # module whose optimiser consumes factored weight gradients
+    model: Optional["SparseAutoEncoder"] = None
 
 
 class SparseRowGrad:
@@ -69,14 +70,19 @@ class _FusedTopKLoss(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, x, label, tok_w, W_E, b_E, W_D, b_D, w_enc_op, w_dec_op, scale, k, holder):
-        amp = w_enc_op.dtype == torch.bfloat16
+    def forward(ctx, x, label, tok_w, W_E, b_E, W_D, b_D, k, amp, holder):
+        sae = holder.model
+        w_enc_op = sae._w_enc_operand(amp)
         if amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)
         else:
             x_op = x.contiguous()
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.float32)
+        # decoder-side operands are fetched after the GEMM is enqueued: an overlapped decoder update of the
+        # previous step (see HipAdam) is waited for here, not before the GEMM
+        scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
+        w_dec_op = sae._w_dec_operand(amp)
         code = ops.select_topk_row(pre, b_E, scale, k)
         recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, b_D, label, tok_w)
         loss = loss_tok.sum()
@@ -121,7 +127,7 @@ class _FusedTopKLoss(torch.autograd.Function):
             import dataclasses
             dx = ops.sparse_decode_fwd(dataclasses.replace(code, val=coef_enc), ctx.w_enc_op, None)
         dlabel = -ctx.grad_recon * g if ctx.needs_input_grad[1] else None
-        return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None, None, None
+        return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
 @register_sae_model("sae")
@@ -147,6 +153,16 @@ class SparseAutoEncoder(SparseDictionary):
         # set by an optimiser that consumes SparseRowGrad (HipAdam): the fused backward then leaves W_E.grad /
         # W_D.grad unset and attaches the factored gradient as `param._sparse_grad` instead
         self.defer_weight_grads = False
+
+    # ---- an optimiser may still be updating W_D on another stream (see HipAdam.overlap_decoder_update) ----
+    def set_pending_update(self, event) -> None:
+        self._pending_update = event
+
+    def wait_pending_update(self) -> None:
+        ev = getattr(self, "_pending_update", None)
+        if ev is not None:
+            torch.cuda.current_stream(self.W_D.device).wait_event(ev)
+            self._pending_update = None
 
     # ---- derived operands, refreshed when the parameter's version counter moves ----
     def _derive(self, name: str, param: torch.Tensor, make) -> torch.Tensor:
@@ -179,12 +195,14 @@ class SparseAutoEncoder(SparseDictionary):
         return self._derive("W_E.bf16", self.W_E, lambda old: ops.cast_bf16(wt, old))
 
     def _w_dec_operand(self, amp: bool) -> torch.Tensor:
+        self.wait_pending_update()
         w = self.W_D.detach()
         if not amp or w.dtype == torch.bfloat16:
             return w
         return self._derive("W_D.bf16", self.W_D, lambda old: ops.cast_bf16(w, old))
 
     def _decoder_norm_nograd(self) -> torch.Tensor:
+        self.wait_pending_update()
         return self._derive("W_D.norm", self.W_D, lambda old: ops.row_norm(self.W_D.detach().float(), old))
 
     # ---- norms (models/sae.py:136-188, 209-212) ----
@@ -192,6 +210,7 @@ class SparseAutoEncoder(SparseDictionary):
         return torch.norm(self.W_E, p=2, dim=0, keepdim=keepdim)
 
     def decoder_norm(self, keepdim: bool = False) -> torch.Tensor:
+        self.wait_pending_update()
         return torch.norm(self.W_D, p=2, dim=1, keepdim=keepdim)
 
     def decoder_bias_norm(self) -> torch.Tensor:
@@ -327,18 +346,17 @@ class SparseAutoEncoder(SparseDictionary):
         else:
             m = mask.to(torch.float32)
             tok_w = m / m.sum()
-        scale = self._decoder_norm_nograd() if self.cfg.sparsity_include_decoder_norm else None
         holder = _Holder()
+        holder.model = self
         holder.defer_to = self if self.defer_weight_grads and torch.is_grad_enabled() else None
         loss, recon = _FusedTopKLoss.apply(
             x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x,
             label.to(torch.float32).contiguous(), tok_w, self.W_E, self.b_E, self.W_D,
-            self.b_D if self.cfg.use_decoder_bias else None,
-            self._w_enc_operand(amp), self._w_dec_operand(amp), scale, int(self.current_k), holder)
+            self.b_D if self.cfg.use_decoder_bias else None, int(self.current_k), amp, holder)
         if not return_aux_data:
             return loss
 
-        code, pre, b_E = holder.code, holder.pre, self.b_E.detach()
+        code, pre, b_E, scale = holder.code, holder.pre, self.b_E.detach(), holder.scale
 
         def dense_hidden_pre():
             h0 = pre.float() + b_E

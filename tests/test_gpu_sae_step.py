@@ -211,3 +211,30 @@ def test_materialize_grads_and_second_backward(pkg, oracle, dev):
     opt.materialize_grads()
     for n, p in sae.named_parameters():
         assert torch.allclose(p.grad, 2 * g1[n], rtol=1e-6, atol=1e-12), n
+
+
+def test_overlapped_decoder_update_gives_identical_training(pkg, oracle, dev):
+    """Running the decoder's Adam pass on a second stream (overlapping the next step's GEMM) must not
+    change a single bit of a multi-step run."""
+    results = []
+    for overlap in (False, True):
+        sae, _, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=7, include_norm=True)
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae, overlap_decoder_update=overlap)
+        gbatch = {k: v.to(dev) for k, v in batch.items()}
+        losses = []
+        for _ in range(6):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                loss = sae.compute_loss(gbatch, return_aux_data=False)
+            loss.backward()
+            opt.step()
+            opt.zero_grad()
+            losses.append(loss)
+        opt.join()
+        torch.cuda.synchronize()
+        results.append(([l.item() for l in losses], {n: p.detach().clone() for n, p in sae.named_parameters()},
+                        sae.decoder_norm().detach().clone()))
+    (la, pa, na), (lb, pb, nb) = results
+    assert la == lb and la[-1] < la[0]
+    for n in pa:
+        assert torch.equal(pa[n], pb[n]), n
+    assert torch.equal(na, nb)
