@@ -85,6 +85,15 @@ def gpu_step_bench(args):
         opt.zero_grad()
         return loss
 
+    if args.calibrate_copy:
+        # a plain device copy of known size (1 GiB read + 1 GiB written), for scaling rocprofv3's
+        # FETCH_SIZE / WRITE_SIZE counters when they are collected over this command
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -146,6 +155,7 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=512)
     ap.add_argument("--cpu-sample-features", type=int, default=32768)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
     ap.add_argument("--overlap", action="store_true", help="run the decoder Adam pass on a second stream, overlapping the next GEMM")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -30,8 +30,9 @@
 // into one 8-byte (bf16) or 16-byte (fp32) store.
 //
 // Workgroup order: consecutive ids land on the 8 XCDs round-robin; within an XCD, 32 consecutive
-// workgroups (one per CU) cover 8 token tiles x 4 feature tiles, so every slab in an XCD's L2 is
-// shared by 4 or 8 resident workgroups (best measured of 16x2, 8x4).
+// workgroups (one per CU) cover 4 token tiles x 8 feature tiles, so every slab in an XCD's L2 is
+// shared by 8 or 4 resident workgroups (measured at the headline shape: 16x2 978, 8x4 1084, 4x8 1189,
+// 2x16 1107, 1x32 923 TFLOP/s).
 //
 // Rows beyond B or F are clamped to the last valid row when loading (their products land in
 // accumulators that the epilogue never stores), so the main loop has no bounds checks.
@@ -83,12 +84,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
   int tile_m, tile_n;
   {
     const int xcd = bid & 7, slot = bid >> 3;
-    // per XCD: groups of 32 consecutive workgroups cover 8 token tiles x 4 feature tiles
+    // per XCD: groups of 32 consecutive workgroups cover 4 token tiles x 8 feature tiles
     const int grp = slot >> 5, in = slot & 31;
-    const int m_groups = (tiles_m + 7) >> 3;           // groups of 8 token tiles (last one may be partial)
+    const int m_groups = (tiles_m + 3) >> 2;           // groups of 4 token tiles (last one may be partial)
     const int n_grp = grp / m_groups, m_half = grp % m_groups;
-    tile_m = m_half * 8 + (in & 7);
-    tile_n = (n_grp * 4 + (in >> 3)) * 8 + xcd;
+    tile_m = m_half * 4 + (in & 3);
+    tile_n = (n_grp * 8 + (in >> 2)) * 8 + xcd;
     if (tile_n >= tiles_n || tile_m >= tiles_m) return;
   }
   const int m0 = tile_m * GEMM_BM, n0 = tile_n * GEMM_BN;
@@ -245,8 +246,8 @@ static int launch_gemm(const void *x, const void *w, void *out, int64_t B, int64
                                      hipGetErrorString(e));
     attr_set = true;
   }
-  // grid: 8 XCDs x (token tiles padded to 8) x (feature tiles per XCD padded to 4); padding workgroups exit at once
-  const int m_pad = (tiles_m + 7) / 8 * 8, n_local_pad = ((tiles_n + 7) / 8 + 3) / 4 * 4;
+  // grid: 8 XCDs x (token tiles padded to 4) x (feature tiles per XCD padded to 8); padding workgroups exit at once
+  const int m_pad = (tiles_m + 3) / 4 * 4, n_local_pad = ((tiles_n + 7) / 8 + 7) / 8 * 8;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
                      (const char *)w, out, (int)B, (int)F, (int)(d * esz), tiles_m, tiles_n);
   return check_launch("encoder_gemm");
