@@ -107,6 +107,25 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
                            int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
                            int32_t *row_nnz, int cand_cap, void *stream);
 
+/* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
+ * (h0, h1 as above); ties at the threshold -> lowest flattened index b * F + f.  If fewer than
+ * k_total entries are positive, all positives are kept.
+ *   feat_mask (nullable, fp32 0/1 [F]): the aux-k form, h1 = ((h0 * scale) / scale) * feat_mask * scale,
+ *     i.e. `hidden_pre * is_dead * decoder_norm` op for op;
+ *   k_total_dev (nullable): read k_total from device memory instead (k' * B with k' known only there);
+ *   idx/val have room for `capacity` entries (entries beyond it are dropped; k_total is the
+ *     natural capacity); row_off/row_nnz [B] describe the variable-length rows; total_out
+ *     (nullable, device int64) receives the number of kept entries.
+ * workspace: sae_select_topk_batch_workspace_bytes(B, F), 256-byte aligned.
+ * Replaces the batchtopk closure (models/sparse_dictionary.py:761-794) + utils/math.py:81-171
+ * with dim=(-2,-1), and the dead-latent select of the aux-k loss (sparse_dictionary.py:952-972). */
+int64_t sae_select_topk_batch_workspace_bytes(int64_t B, int64_t F);
+int sae_select_topk_batch(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                          const float *feat_mask, int64_t B, int64_t F, int64_t k_total,
+                          const int64_t *k_total_dev, int32_t *idx, float *val, int64_t capacity,
+                          int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+
 /* ---- sparse decoder --------------------------------------------------------------- */
 
 /* recon[b, :] = sum_s val[s] * W_D[idx[s], :] + b_dec,  s over token b's slots.

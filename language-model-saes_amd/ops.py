@@ -220,6 +220,50 @@ def select_topk_row(
     return SparseCode(idx, val, row_off, row_nnz, B, F)
 
 
+def select_topk_batch(
+    pre: torch.Tensor,
+    b_enc: Optional[torch.Tensor],
+    scale: Optional[torch.Tensor],
+    k_total,
+    feat_mask: Optional[torch.Tensor] = None,
+    capacity: Optional[int] = None,
+) -> SparseCode:
+    """Batch-global TopK.  `k_total` is an int, or a device int64 tensor (then `capacity` is required)."""
+    _req(pre, "pre", ndim=2)
+    B, F = pre.shape
+    for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
+        if t is not None:
+            _req(t, name, torch.float32, 1)
+            if t.numel() != F:
+                raise ValueError(f"{name} must have {F} elements")
+    dev = pre.device
+    k_dev = None
+    if isinstance(k_total, torch.Tensor):
+        _req(k_total, "k_total", torch.int64)
+        if capacity is None:
+            raise ValueError("capacity is required when k_total lives on the device")
+        k_dev, k_host = k_total, 0
+    else:
+        k_host = int(k_total)
+        if capacity is None:
+            capacity = max(min(k_host, B * F), 1)
+    idx = torch.zeros(capacity, dtype=torch.int32, device=dev)
+    val = torch.zeros(capacity, dtype=torch.float32, device=dev)
+    row_off = torch.empty(B, dtype=torch.int64, device=dev)
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.sae_select_topk_batch_workspace_bytes(B, F)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with _timed("select_topk_batch"):
+        check(
+            lib.sae_select_topk_batch(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
+                                      _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
+                                      row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre)),
+            "select_topk_batch",
+        )
+    return SparseCode(idx, val, row_off, row_nnz, B, F)
+
+
 # ---- sparse decoder -------------------------------------------------------------------------
 
 def _check_code(code: SparseCode, w_dec: torch.Tensor):

@@ -371,3 +371,80 @@ def test_adam_step_sparse_rows_equals_grad_rows_then_adam(pkg, dev, B, d, F, k, 
         assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
         assert torch.equal(sha, shb) and torch.equal(na, nb) and torch.equal(bias_a, bias_b)
     assert not torch.equal(pa, p0)
+
+
+# ---------------------------------------------------------------------------------------------
+# BatchTopK select
+# ---------------------------------------------------------------------------------------------
+
+def oracle_batchtopk_dense(oracle, pre, b_enc, scale, k_total, feat_mask=None):
+    """dense [B, F] feature activations by the oracle's rule (global top-k_total, ties -> lowest flat index)"""
+    h0 = pre.float() + (b_enc if b_enc is not None else 0.0)
+    h1 = h0 * scale if scale is not None else h0
+    if feat_mask is not None:
+        h1 = ((h1 / scale) * feat_mask) * scale if scale is not None else h1 * feat_mask
+    r = h1 * h1.gt(0).to(h1.dtype)
+    a = oracle.topk(r, k=min(k_total, r.numel()), dim=(-2, -1)) if k_total > 0 else torch.zeros_like(r)
+    return a / scale if scale is not None else a
+
+
+def check_batch_select(pkg, oracle, dev, pre, b_enc, scale, k_total, feat_mask=None, k_on_device=False):
+    to = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    if k_on_device:
+        code = pkg.ops.select_topk_batch(pre.to(dev), to(b_enc), to(scale), torch.tensor(k_total, dtype=torch.int64, device=dev),
+                                         to(feat_mask), capacity=max(k_total, 1))
+    else:
+        code = pkg.ops.select_topk_batch(pre.to(dev), to(b_enc), to(scale), k_total, to(feat_mask))
+    want = oracle_batchtopk_dense(oracle, pre, b_enc, scale, k_total, feat_mask)
+    got = code.to_dense().cpu()
+    assert torch.equal(got != 0, want != 0), "kept sets differ"
+    assert torch.equal(got, want), "kept values differ"
+    # structure: offsets are the running sum of the row lengths; indices ascend inside a row
+    nnz = code.row_nnz.cpu().long()
+    assert torch.equal(code.row_off.cpu(), torch.cumsum(nnz, 0) - nnz)
+    assert nnz.sum().item() == (want != 0).sum().item()
+    for (ri, _) in code_to_rows(code):
+        assert np.all(np.diff(ri) > 0)
+    return code
+
+
+@pytest.mark.parametrize("B,F,k", [(9, 1000, 5), (64, 4096, 32), (8, 32768, 64), (3, 37, 4), (300, 512, 7)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_select_topk_batch_random(pkg, oracle, dev, B, F, k, dtype):
+    print(f"batchtopk B={B} F={F} k={k} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(F + k)
+    pre = torch.randn(B, F, generator=g).to(dtype)
+    b_enc = 0.1 * torch.randn(F, generator=g)
+    scale = 0.5 + torch.rand(F, generator=g)
+    code = check_batch_select(pkg, oracle, dev, pre, b_enc, scale, k * B)
+    assert code.row_nnz.sum().item() == k * B
+    check_batch_select(pkg, oracle, dev, pre, None, None, k * B, k_on_device=True)
+
+
+def test_select_topk_batch_ties_and_degenerate(pkg, oracle, dev):
+    B, F = 6, 2000
+    g = torch.Generator().manual_seed(0)
+    pre = torch.randint(0, 4, (B, F), generator=g).float()      # four levels: the threshold sits inside a huge tie
+    for k_total in (1, 17, 3000, 5000, B * F):
+        check_batch_select(pkg, oracle, dev, pre, None, None, k_total)
+    check_batch_select(pkg, oracle, dev, torch.full((B, F), 2.0), None, None, 2500)   # all equal: first 2500 flat indices
+    check_batch_select(pkg, oracle, dev, -torch.ones(B, F), None, None, 100)          # nothing positive
+    few = torch.zeros(B, F); few[1, 5] = 1.0; few[4, 1999] = 3.0
+    code = check_batch_select(pkg, oracle, dev, few, None, None, 100)                 # fewer positives than k_total
+    assert code.row_nnz.cpu().tolist() == [0, 1, 0, 0, 1, 0]
+    check_batch_select(pkg, oracle, dev, pre, None, None, 0)                          # k_total = 0 keeps nothing
+    bfq = torch.randn(B, F, generator=g).bfloat16()                                   # bf16-quantised: natural ties
+    check_batch_select(pkg, oracle, dev, bfq, None, None, 64 * B)
+
+
+def test_select_topk_batch_feature_mask(pkg, oracle, dev):
+    """aux-k form: only masked-in (dead) features compete"""
+    B, F = 16, 3000
+    g = torch.Generator().manual_seed(4)
+    pre = torch.randn(B, F, generator=g)
+    b_enc = 0.1 * torch.randn(F, generator=g)
+    scale = 0.5 + torch.rand(F, generator=g)
+    mask = (torch.rand(F, generator=g) < 0.1).float()
+    code = check_batch_select(pkg, oracle, dev, pre, b_enc, scale, 8 * B, feat_mask=mask)
+    assert (mask[code.idx.cpu().long()[: code.row_nnz.sum().item()]] == 1).all()
+    check_batch_select(pkg, oracle, dev, pre, b_enc, scale, 8 * B, feat_mask=torch.zeros(F))  # nothing is dead
