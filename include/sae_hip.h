@@ -99,12 +99,14 @@ int sae_select_topk_row(const void *pre, int pre_dtype, const float *b_enc, cons
                         int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
                         int32_t *row_nnz, void *stream);
 
-/* Same, with the capacity of the in-LDS candidate list exposed (0..4096).  A token whose
- * candidates do not fit takes the general path (radix histograms over the whole row), which
- * returns the identical result; cand_cap = 0 forces it for every token.  For testing and
- * tuning; no counterpart in the reference. */
+/* Same, with two more knobs.
+ *   feat_mask (nullable, fp32 0/1 [F]): the aux-k form, h1 = ((h0 * scale) / scale) * feat_mask * scale,
+ *     i.e. `hidden_pre * is_dead * decoder_norm` op for op (models/sparse_dictionary.py:952-972);
+ *   cand_cap (0..4096): capacity of the in-LDS candidate list.  A token whose candidates do not
+ *     fit takes the general path (radix histograms over the whole row), which returns the
+ *     identical result; cand_cap = 0 forces it for every token (testing and tuning). */
 int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
-                           int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
+                           const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
                            int32_t *row_nnz, int cand_cap, void *stream);
 
 /* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
@@ -212,6 +214,22 @@ int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot,
                               float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                               double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                               float *bias_grad_out, void *stream);
+
+/* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
+ * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and
+ *   p -= lr * sqrt(1 - b2^t) / (1 - b1^t) * m / (sqrt(v) + eps);
+ * a gradient that is zero everywhere leaves p, m, v and the step counter untouched.
+ * step_state: device float[1], the number of steps taken so far (in/out; t = step_state + 1);
+ * flag_workspace: device int32[1] scratch.  No host synchronisation (the reference's
+ * `if not grad.any(): continue` is evaluated on the device). */
+int sae_sparse_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
+                         double beta2, double eps, float *step_state, int32_t *flag_workspace,
+                         void *shadow_bf16, void *stream);
+
+/* acc[0] += sum_i g[i]^2, acc[1] += #{i : g[i] != 0}, both accumulated in fp64 (acc: device double[2],
+ * cleared by the caller before the first tensor).  The two quantities behind
+ * compute_grad_norm (optim.py:257-277): ||g|| / sqrt(#non-zero). */
+int sae_grad_sq_nnz(const float *g, int64_t n, double *acc, void *stream);
 
 #ifdef __cplusplus
 }

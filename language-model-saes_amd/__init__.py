@@ -16,3 +16,8 @@ from .sae import SparseAutoEncoder  # noqa: E402,F401
 from .optim import HipAdam  # noqa: E402,F401
 
 __all__ += ["SAEConfig", "SparseDictionaryConfig", "JumpReLU", "SparseDictionary", "SparseAutoEncoder", "HipAdam"]
+
+from .optim import HipSparseAdam, clip_grad_norm, compute_grad_norm  # noqa: E402,F401
+from .trainer import Trainer, TrainerConfig, get_scheduler  # noqa: E402,F401
+
+__all__ += ["HipSparseAdam", "clip_grad_norm", "compute_grad_norm", "Trainer", "TrainerConfig", "get_scheduler"]

@@ -28,7 +28,7 @@ SIGNATURES = {
     "sae_col_sum": (_I, [_P, _P, _L, _L, _I, _P, _L, _P]),
     "sae_encoder_gemm": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "sae_select_topk_row": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
-    "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),
+    "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),
     "sae_select_topk_batch_workspace_bytes": (_L, [_L, _L]),
     "sae_select_topk_batch": (_I, [_P, _I, _P, _P, _P, _L, _L, _L, _P, _P, _P, _L, _P, _P, _P, _P, _L, _P]),
     "sae_sparse_decode_fwd": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _L, _P]),
@@ -38,6 +38,8 @@ SIGNATURES = {
     "sae_build_feature_index": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P]),
     "sae_sparse_grad_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _P]),
     "sae_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _L, _P, _P, _L, _P]),
+    "sae_sparse_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _P, _P, _P, _P]),
+    "sae_grad_sq_nnz": (_I, [_P, _L, _P, _P]),
     "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P]),
 }
 

@@ -248,3 +248,100 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
                        coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out);
   return check_launch("adam_step_sparse_rows");
 }
+
+// ---------------------------------------------------------------------------------------------
+// SparseAdam (masked-momentum Adam) and the gradient-norm diagnostic.
+// ---------------------------------------------------------------------------------------------
+namespace sae {
+
+__global__ __launch_bounds__(256) void any_nonzero_kernel(const float *__restrict__ g, int64_t n, int32_t *flag) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int hit = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) hit |= g[i] != 0.f;
+  hit = wave_sum_i(hit);
+  if ((threadIdx.x & 63) == 0 && hit) atomicOr(flag, 1);
+}
+
+// moments decay everywhere; gradient contributions and the parameter move only where g != 0;
+// nothing at all happens (and the step counter stays) when the whole gradient is zero
+__global__ __launch_bounds__(256) void sparse_adam_kernel(float *__restrict__ p, const float *__restrict__ g,
+                                                          float *__restrict__ m, float *__restrict__ v, int64_t n,
+                                                          double lr, double beta1, double beta2, float eps,
+                                                          const float *__restrict__ step_state,
+                                                          const int32_t *__restrict__ flag, uint16_t *__restrict__ shadow) {
+  if (*flag == 0) return;
+  const double t = (double)step_state[0] + 1.0;
+  const float step_size = (float)(lr * sqrt(1.0 - pow(beta2, t)) / (1.0 - pow(beta1, t)));
+  const float b1 = (float)beta1, b2 = (float)beta2, omb1 = (float)(1.0 - beta1), omb2 = (float)(1.0 - beta2);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const float gg = g[i];
+    float mm = m[i] * b1, vv = v[i] * b2, pp = p[i];
+    if (gg != 0.f) {
+      mm = mm + omb1 * gg;
+      vv = vv + omb2 * gg * gg;
+      pp = pp - step_size * mm / (sqrtf(vv) + eps);
+      p[i] = pp;
+    }
+    m[i] = mm;
+    v[i] = vv;
+    if (shadow) shadow[i] = f32_to_bf16_bits(pp);
+  }
+}
+
+__global__ void sparse_adam_advance_kernel(float *step_state, const int32_t *flag) {
+  if (threadIdx.x == 0 && blockIdx.x == 0 && *flag) step_state[0] += 1.f;
+}
+
+// acc[0] += sum g^2 (fp64), acc[1] += #(g != 0) (fp64 count)
+__global__ __launch_bounds__(256) void grad_sq_nnz_kernel(const float *__restrict__ g, int64_t n, double *acc) {
+  __shared__ double red[8];
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  double sq = 0.0;
+  int nz = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const float x = g[i];
+    sq += (double)x * (double)x;
+    nz += x != 0.f;
+  }
+  double cnt = (double)nz;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { sq += __shfl_xor(sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) { red[w] = sq; red[4 + w] = cnt; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    atomicAdd(&acc[0], red[0] + red[1] + red[2] + red[3]);
+    atomicAdd(&acc[1], red[4] + red[5] + red[6] + red[7]);
+  }
+}
+
+}  // namespace sae
+
+extern "C" int sae_sparse_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
+                                    double beta2, double eps, float *step_state, int32_t *flag_workspace,
+                                    void *shadow_bf16, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(p && g && m && v && step_state && flag_workspace, SAE_ERR_INVALID_ARG, "sparse_adam_step: null pointer");
+  SAE_REQUIRE(n > 0, SAE_ERR_INVALID_ARG, "sparse_adam_step: n must be positive");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = zero_fill(flag_workspace, 4, st);
+  if (rc) return rc;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 32768) blocks = 32768;
+  hipLaunchKernelGGL(any_nonzero_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g, n, flag_workspace);
+  hipLaunchKernelGGL(sparse_adam_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, lr, beta1, beta2,
+                     (float)eps, step_state, flag_workspace, reinterpret_cast<uint16_t *>(shadow_bf16));
+  hipLaunchKernelGGL(sparse_adam_advance_kernel, dim3(1), dim3(64), 0, st, step_state, flag_workspace);
+  return check_launch("sparse_adam_step");
+}
+
+extern "C" int sae_grad_sq_nnz(const float *g, int64_t n, double *acc, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(g && acc, SAE_ERR_INVALID_ARG, "grad_sq_nnz: null pointer");
+  SAE_REQUIRE(n > 0, SAE_ERR_INVALID_ARG, "grad_sq_nnz: n must be positive");
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(grad_sq_nnz_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, g, n, acc);
+  return check_launch("grad_sq_nnz");
+}

@@ -38,8 +38,9 @@ struct SelShared {
   int32_t digit_found;
 };
 
-__device__ __forceinline__ uint32_t key_of(float pre, float b, float s) {
-  const float h1 = (pre + b) * s;
+__device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm, bool has_mask) {
+  float h1 = (pre + b) * s;
+  if (has_mask) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
 
@@ -102,12 +103,13 @@ struct RowReader {
   const void *row;
   const float *b_enc;
   const float *scale;
+  const float *fmask;
   int F;
   // calls fn(index, key) for every element of the row, vectorised when the row allows it
   template <typename Fn>
   __device__ __forceinline__ void for_each(Fn fn) const {
     constexpr int V = BF16 ? 8 : 4;  // elements per 16-byte load
-    const bool vec_ok = (F % V == 0) && (((((uintptr_t)row) | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0);
+    const bool vec_ok = (F % V == 0) && (((((uintptr_t)row) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
     if (vec_ok) {
       const int n_chunks = F / V;
       for (int c = threadIdx.x; c < n_chunks; c += SEL_THREADS) {
@@ -125,7 +127,17 @@ struct RowReader {
           pre[2] = __uint_as_float(raw.z); pre[3] = __uint_as_float(raw.w);
         }
         const int base = c * V;
-        float bb[V], ss[V];
+        float bb[V], ss[V], mm[V];
+        if (fmask) {
+#pragma unroll
+          for (int q = 0; q < V / 4; ++q) {
+            const float4 t = reinterpret_cast<const float4 *>(fmask + base)[q];
+            mm[4 * q] = t.x; mm[4 * q + 1] = t.y; mm[4 * q + 2] = t.z; mm[4 * q + 3] = t.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) mm[e] = 1.f;
+        }
         if (b_enc) {
 #pragma unroll
           for (int q = 0; q < V / 4; ++q) {
@@ -147,14 +159,14 @@ struct RowReader {
           for (int e = 0; e < V; ++e) ss[e] = 1.f;
         }
 #pragma unroll
-        for (int e = 0; e < V; ++e) fn(base + e, key_of(pre[e], bb[e], ss[e]));
+        for (int e = 0; e < V; ++e) fn(base + e, key_of(pre[e], bb[e], ss[e], mm[e], fmask != nullptr));
       }
     } else {
       for (int i = threadIdx.x; i < F; i += SEL_THREADS) {
         float pre;
         if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
         else pre = reinterpret_cast<const float *>(row)[i];
-        fn(i, key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f));
+        fn(i, key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr));
       }
     }
   }
@@ -182,7 +194,8 @@ __device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<B
 
 template <bool BF16>
 __global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
-    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale, int F, int k,
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
+    const float *__restrict__ fmask, int F, int k,
     int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
     int32_t *__restrict__ row_nnz, int cand_cap) {
   __shared__ SelShared sh;
@@ -192,6 +205,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
   rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
   rr.scale = scale;
+  rr.fmask = fmask;
   rr.F = F;
 
   // ---- pass 1: per-thread maximum key and number of positive elements ----
@@ -353,8 +367,8 @@ __global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
 
 }  // namespace sae
 
-extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale, int64_t B,
-                                      int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
+extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                                      const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
                                       int cand_cap, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
@@ -367,10 +381,10 @@ extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const floa
   (void)kk;
   hipStream_t st = (hipStream_t)stream;
   if (pre_dtype == SAE_BF16)
-    hipLaunchKernelGGL(select_topk_row_kernel<true>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,
+    hipLaunchKernelGGL(select_topk_row_kernel<true>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale, feat_mask,
                        (int)F, k, idx, val, row_off, row_nnz, cand_cap);
   else
-    hipLaunchKernelGGL(select_topk_row_kernel<false>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,
+    hipLaunchKernelGGL(select_topk_row_kernel<false>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale, feat_mask,
                        (int)F, k, idx, val, row_off, row_nnz, cand_cap);
   return check_launch("select_topk_row");
 }
@@ -378,5 +392,5 @@ extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const floa
 extern "C" int sae_select_topk_row(const void *pre, int pre_dtype, const float *b_enc, const float *scale, int64_t B,
                                    int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
                                    void *stream) {
-  return sae_select_topk_row_ex(pre, pre_dtype, b_enc, scale, B, F, k, idx, val, row_off, row_nnz, sae::SEL_CAP, stream);
+  return sae_select_topk_row_ex(pre, pre_dtype, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, sae::SEL_CAP, stream);
 }

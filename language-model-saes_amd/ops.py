@@ -112,6 +112,16 @@ class SparseCode:
         return out
 
 
+def stack_codes(a: SparseCode, b: SparseCode) -> SparseCode:
+    """The code of 2B virtual tokens: a's tokens first, then b's (same feature space).  Used to hand
+    two sparse codes with different dense operands to the gradient-row kernels in one piece."""
+    if a.d_sae != b.d_sae:
+        raise ValueError("codes address different dictionaries")
+    return SparseCode(torch.cat([a.idx, b.idx]), torch.cat([a.val, b.val]),
+                      torch.cat([a.row_off, b.row_off + a.n_slots]), torch.cat([a.row_nnz, b.row_nnz]),
+                      a.n_tokens + b.n_tokens, a.d_sae)
+
+
 @dataclass
 class FeatureIndex:
     feat_ptr: torch.Tensor   # int32 [F + 1]
@@ -192,10 +202,11 @@ def select_topk_row(
     scale: Optional[torch.Tensor],
     k: int,
     cand_cap: Optional[int] = None,
+    feat_mask: Optional[torch.Tensor] = None,
 ) -> SparseCode:
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
-    for name, t in (("b_enc", b_enc), ("scale", scale)):
+    for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
         if t is not None:
             _req(t, name, torch.float32, 1)
             if t.numel() != F:
@@ -209,12 +220,13 @@ def select_topk_row(
     lib = _lib.load()
     _t = _timed("select_topk_row")
     _t.__enter__()
-    if cand_cap is None:
+    if cand_cap is None and feat_mask is None:
         rc = lib.sae_select_topk_row(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
                                      val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     else:
-        rc = lib.sae_select_topk_row_ex(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
-                                        val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), int(cand_cap), _stream(pre))
+        rc = lib.sae_select_topk_row_ex(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k,
+                                        idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(),
+                                        4096 if cand_cap is None else int(cand_cap), _stream(pre))
     _t.__exit__()
     check(rc, "select_topk_row")
     return SparseCode(idx, val, row_off, row_nnz, B, F)
@@ -421,3 +433,35 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                                                   _ptr(row_norm_out), _ptr(bias_grad_out), _stream(p)),
             "adam_step_sparse_rows",
         )
+
+
+def sparse_adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, step_state: torch.Tensor, *,
+                     lr: float, beta1: float, beta2: float, eps: float, shadow_bf16: Optional[torch.Tensor] = None) -> None:
+    """SparseAdam on contiguous fp32 storage; `step_state` is a device float tensor [1] (steps taken so far)."""
+    for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
+        _req(t, name, torch.float32)
+        if t.numel() != p.numel():
+            raise ValueError(f"{name} must have {p.numel()} elements")
+    _req(step_state, "step_state", torch.float32)
+    flag = torch.empty(1, dtype=torch.int32, device=p.device)
+    with _timed("sparse_adam_step"):
+        check(
+            _lib.load().sae_sparse_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1,
+                                             beta2, eps, step_state.data_ptr(), flag.data_ptr(), _ptr(shadow_bf16), _stream(p)),
+            "sparse_adam_step",
+        )
+
+
+def grad_sq_nnz(grads) -> torch.Tensor:
+    """device double[2]: (sum of squares, number of non-zero entries) over a list of fp32 tensors."""
+    grads = [g for g in grads if g is not None]
+    assert len(grads) > 0, "No gradients found"
+    acc = torch.zeros(2, dtype=torch.float64, device=grads[0].device)
+    lib = _lib.load()
+    for g in grads:
+        if not g.is_contiguous():
+            g = g.t() if g.ndim == 2 and g.t().is_contiguous() else g.contiguous()
+        _req(g, "grad", torch.float32)
+        with _timed("grad_sq_nnz"):
+            check(lib.sae_grad_sq_nnz(g.data_ptr(), g.numel(), acc.data_ptr(), _stream(g)), "grad_sq_nnz")
+    return acc

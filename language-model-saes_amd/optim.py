@@ -185,3 +185,72 @@ class HipAdam(Optimizer):
                               row_len=pv.shape[1] if norm_out is not None else 0)
                 self._publish(p, role, shadow, norm_out)
         return loss
+
+
+class HipSparseAdam(Optimizer):
+    """SparseAdam of the reference (src/llamascopium/optim.py:142-254) with the per-parameter update in
+    one kernel: moments decay everywhere, gradient contributions and the parameter move only where
+    the gradient is non-zero, a parameter whose gradient is entirely zero is skipped (its step counter
+    too).  That test runs on the device, so `step()` never synchronises.  Factored weight gradients
+    are materialised first (the masked update needs the element-wise gradient)."""
+
+    def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, weight_decay: float = 0, model=None):
+        if lr < 0.0 or eps < 0.0 or not (0.0 <= betas[0] < 1.0) or not (0.0 <= betas[1] < 1.0) or weight_decay < 0.0:
+            raise ValueError("invalid SparseAdam hyper-parameters")
+        if weight_decay != 0:
+            raise NotImplementedError("weight decay is not part of the kernel (the reference's trainer never sets it)")
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        self._model = model
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for group in self.param_groups:
+            b1, b2 = group["betas"]
+            for p in group["params"]:
+                sg = getattr(p, "_sparse_grad", None)
+                if sg is not None:
+                    rows, bias = sg.dense()
+                    p.grad = rows if p.is_contiguous() else rows.t()
+                    if bias is not None:
+                        sg.bias_param.grad = bias
+                    p._sparse_grad = None
+        for group in self.param_groups:
+            b1, b2 = group["betas"]
+            for p in group["params"]:
+                if p.grad is None:
+                    continue
+                st = self.state[p]
+                if len(st) == 0:
+                    st["step"] = torch.zeros(1, dtype=torch.float32, device=p.device)
+                    st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                    st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                pv = _flat_view(p)
+                gv = _flat_view(p.grad) if p.grad.stride() == p.stride() else _flat_view(p.grad.contiguous())
+                ops.sparse_adam_step(pv, gv, _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"]), st["step"],
+                                     lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"])
+                torch.autograd.graph.increment_version(p)
+        return loss
+
+
+def compute_grad_norm(params) -> torch.Tensor:
+    """||g||_2 over all gradients divided by sqrt(number of non-zero gradient entries)
+    (src/llamascopium/optim.py:257-277), as a device scalar.  Factored gradients must be materialised first."""
+    grads = [p.grad for p in params if p.grad is not None]
+    acc = ops.grad_sq_nnz(grads)
+    return (acc[0].sqrt() / acc[1].sqrt()).to(torch.float32)
+
+
+def clip_grad_norm(params, max_norm: float) -> torch.Tensor:
+    """src/llamascopium/optim.py:280-292 without the host round trip: gradients are scaled by
+    max_norm / (norm + 1e-6) when the norm exceeds max_norm, decided on the device."""
+    params = [p for p in params if p.grad is not None]
+    norm = compute_grad_norm(params)
+    if max_norm != float("inf"):
+        factor = torch.where(norm > max_norm, max_norm / (norm + 1e-6), torch.ones_like(norm))
+        for p in params:
+            p.grad.mul_(factor)
+    return norm

@@ -42,6 +42,9 @@ class _Holder:
     scale: Optional[torch.Tensor] = None
     defer_to: Optional["SparseAutoEncoder"] = None  # module whose optimiser consumes factored weight gradients
     model: Optional["SparseAutoEncoder"] = None
+    aux: Optional[dict] = None      # aux-k request: {"is_dead": callable(code) -> bool [F], "k_aux": int, "coefficient": float}
+    aux_code: ops.SparseCode = None
+    l_aux: Optional[torch.Tensor] = None
 
 
 class SparseRowGrad:
@@ -60,13 +63,20 @@ class SparseRowGrad:
                                     want_bias=self.bias_param is not None)
 
 
-class _FusedTopKLoss(torch.autograd.Function):
-    """encode -> TopK -> decode -> masked-mean squared error, forward and backward, in kernels.
+class _FusedSparseStep(torch.autograd.Function):
+    """encode -> TopK / BatchTopK -> decode -> masked-mean squared error (+ aux-k), forward and backward,
+    in kernels.
 
-    forward : GEMM, select (bias + norm scale fused), decode + loss + grad_recon + d val (fused)
-    backward: feature index, dW_D / dW_E^T rows, db_E, db_D; no dense [B, F] tensor is formed.
-    The decoder-norm scale enters as act(h * n) / n; its two derivative terms with respect to n
-    cancel analytically, so no gradient flows to W_D through n.
+    forward : GEMM, select (bias + norm scale fused), decode + loss + grad_recon + d val
+    backward: feature index, dW_D / dW_E^T rows (or their factored form), db_E, db_D; no dense [B, F]
+              tensor is formed.
+    The decoder-norm scale enters as act(h * n) / n; its two derivative terms with respect to n cancel
+    analytically, so no gradient flows to W_D through n.
+
+    aux-k (models/sparse_dictionary.py:940-991): a second select restricted to dead features, decoded
+    without bias; l_aux = alpha * mean_b |(label - recon) - aux_recon|^2 with the residual carrying
+    gradient.  The two codes are stacked into one code over 2B virtual tokens so that a single feature
+    index serves both gradients.
     """
 
     @staticmethod
@@ -83,12 +93,53 @@ class _FusedTopKLoss(torch.autograd.Function):
         # previous step (see HipAdam) is waited for here, not before the GEMM
         scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
         w_dec_op = sae._w_dec_operand(amp)
-        code = ops.select_topk_row(pre, b_E, scale, k)
-        recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, b_D, label, tok_w)
-        loss = loss_tok.sum()
-        holder.code, holder.pre, holder.scale = code, pre, scale
-        ctx.code, ctx.x_op, ctx.grad_recon, ctx.dval = code, x_op, grad_recon, dval
-        ctx.w_enc_op, ctx.w_dec_op = w_enc_op, w_dec_op
+        B = x.shape[0]
+        batch_wide = sae.cfg.act_fn.lower() == "batchtopk"
+        if batch_wide:
+            code = ops.select_topk_batch(pre, b_E, scale, k * B)
+        else:
+            code = ops.select_topk_row(pre, b_E, scale, k)
+        aux = holder.aux
+        if aux is None:
+            recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, b_D, label, tok_w)
+            loss = loss_tok.sum()
+            l_aux = None
+            grad_code, grad_dense_D, grad_coef_E, x_rows = code, grad_recon, dval, x_op
+        else:
+            dead = aux["is_dead"](code)                       # bool [F], from the caller's dead statistics
+            dead_f = dead.to(torch.float32)
+            n_dead = dead.sum()
+            k_aux = int(aux["k_aux"])
+            if batch_wide:
+                k_dev = (torch.clamp(n_dead, max=k_aux) * B).to(torch.int64)
+                aux_code = ops.select_topk_batch(pre, b_E, scale, k_dev, feat_mask=dead_f, capacity=k_aux * B)
+            else:
+                # min(k_aux, #dead) needs no host value: at most #dead entries can be positive
+                aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f)
+            recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
+            aux_recon = ops.sparse_decode_fwd(aux_code, w_dec_op, None)
+            has_dead = (n_dead > 0).to(torch.float32)
+            w = tok_w[:, None]
+            diff = recon - label
+            r = (label - recon) - aux_recon
+            alpha = float(aux["coefficient"]) * has_dead
+            l_rec = (w * diff * diff).sum()
+            l_aux = alpha * (w * r * r).sum()
+            loss = l_rec + l_aux
+            g_aux = (-2.0 * alpha) * w * r                     # d loss / d aux_recon
+            grad_recon = 2.0 * w * diff + g_aux                # d loss / d recon (the residual is not detached)
+            dval = ops.sparse_decode_bwd_dval(code, grad_recon, w_dec_op)
+            dval_aux = ops.sparse_decode_bwd_dval(aux_code, g_aux, w_dec_op)
+            grad_code = ops.stack_codes(code, aux_code)
+            grad_dense_D = torch.cat([grad_recon, g_aux])
+            grad_coef_E = torch.cat([dval, dval_aux])
+            x_rows = torch.cat([x_op, x_op])
+            holder.aux_code = aux_code
+        holder.code, holder.pre, holder.scale, holder.l_aux = code, pre, scale, l_aux
+        ctx.grad_code, ctx.x_rows, ctx.grad_dense_D, ctx.grad_coef_E = grad_code, x_rows, grad_dense_D, grad_coef_E
+        ctx.grad_recon = grad_recon
+        ctx.n_tokens = B
+        ctx.w_enc_op = w_enc_op
         ctx.has_b_D = b_D is not None
         ctx.defer_to = holder.defer_to
         ctx.mark_non_differentiable(recon)
@@ -96,19 +147,19 @@ class _FusedTopKLoss(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, _g_recon):
-        code = ctx.code
+        code = ctx.grad_code
         F = code.d_sae
         fi = ops.build_feature_index(code)
         g = g_loss.to(torch.float32)
         coef_dec = code.val * g          # dW_D[f] = sum val * grad_recon[token]
-        coef_enc = ctx.dval * g          # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
+        coef_enc = ctx.grad_coef_E * g   # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
         db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
         sae = ctx.defer_to
         if sae is not None and getattr(sae.W_D, "_sparse_grad", None) is None and sae.W_D.grad is None \
                 and getattr(sae.W_E, "_sparse_grad", None) is None and sae.W_E.grad is None:
             # hand the factored gradients to the optimiser; b_E's gradient is a by-product of its W_E pass
-            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, ctx.grad_recon, F)
-            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, ctx.x_op, F, bias_param=sae.b_E)
+            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, ctx.grad_dense_D, F)
+            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, ctx.x_rows, F, bias_param=sae.b_E)
             dW_D = dW_Et = db_E = None
         else:
             if sae is not None:  # a second backward before the optimiser ran: fall back to dense accumulation
@@ -120,13 +171,17 @@ class _FusedTopKLoss(torch.autograd.Function):
                         if bias is not None:
                             sg.bias_param.grad = bias if sg.bias_param.grad is None else sg.bias_param.grad + bias
                         prm._sparse_grad = None
-            dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_recon, F)
-            dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_op, F, want_bias=True)
+            dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_dense_D, F)
+            dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_rows, F, want_bias=True)
         dx = None
         if ctx.needs_input_grad[0]:
             import dataclasses
             dx = ops.sparse_decode_fwd(dataclasses.replace(code, val=coef_enc), ctx.w_enc_op, None)
-        dlabel = -ctx.grad_recon * g if ctx.needs_input_grad[1] else None
+            if dx.shape[0] != ctx.n_tokens:  # stacked code: fold the aux half back onto its tokens
+                dx = dx[: ctx.n_tokens] + dx[ctx.n_tokens:]
+        dlabel = None
+        if ctx.needs_input_grad[1]:
+            dlabel = -ctx.grad_recon * g
         return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
@@ -317,10 +372,10 @@ class SparseAutoEncoder(SparseDictionary):
     # ---- fused train-step loss ----
     def _fused_eligible(self, x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
         return (
-            self.cfg.act_fn.lower() == "topk"
+            self.cfg.act_fn.lower() in ("topk", "batchtopk")
             and x.is_cuda and x.ndim == 2 and label.ndim == 2
             and not self.cfg.use_glu_encoder
-            and sparsity_loss_type is None and not (lp_coefficient > 0.0) and not (auxk_coefficient > 0.0)
+            and sparsity_loss_type is None and not (lp_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
             and self.W_E.dtype == torch.float32
         )
@@ -348,8 +403,18 @@ class SparseAutoEncoder(SparseDictionary):
             tok_w = m / m.sum()
         holder = _Holder()
         holder.model = self
+        if auxk_coefficient > 0.0:
+            assert update_dead_statistics is not None, "update_dead_statistics must be set when auxk_coefficient > 0.0"
+
+            def is_dead(code, _upd=update_dead_statistics, _mask=mask):
+                sparse_upd = getattr(getattr(_upd, "__self__", None), "update_dead_statistics_sparse", None)
+                if sparse_upd is not None:
+                    return sparse_upd(code, _mask)
+                return _upd(code.to_dense(), _mask, ("batch", "sae"))  # a callable that only knows dense activations
+
+            holder.aux = {"is_dead": is_dead, "k_aux": k_aux, "coefficient": auxk_coefficient}
         holder.defer_to = self if self.defer_weight_grads and torch.is_grad_enabled() else None
-        loss, recon = _FusedTopKLoss.apply(
+        loss, recon = _FusedSparseStep.apply(
             x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x,
             label.to(torch.float32).contiguous(), tok_w, self.W_E, self.b_E, self.W_D,
             self.b_D if self.cfg.use_decoder_bias else None, int(self.current_k), amp, holder)
@@ -362,8 +427,10 @@ class SparseAutoEncoder(SparseDictionary):
             h0 = pre.float() + b_E
             return (h0 * scale) / scale if scale is not None else h0
 
+        l_aux = holder.l_aux
         eager = {
-            "loss": loss, "l_rec": loss, "l_s": None, "l_p": None, "l_aux": None, "label": label, "mask": mask,
+            "loss": loss, "l_rec": loss if l_aux is None else (loss - l_aux).detach(), "l_s": None, "l_p": None,
+            "l_aux": l_aux, "label": label, "mask": mask,
             "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
             "auxk_coefficient": auxk_coefficient, "sparse_code": code,
         }

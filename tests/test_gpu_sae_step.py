@@ -238,3 +238,92 @@ def test_overlapped_decoder_update_gives_identical_training(pkg, oracle, dev):
     for n in pa:
         assert torch.equal(pa[n], pb[n]), n
     assert torch.equal(na, nb)
+
+
+# ---------------------------------------------------------------------------------------------
+# BatchTopK and aux-k through the fused step
+# ---------------------------------------------------------------------------------------------
+
+def make_pair_act(pkg, oracle, dev, act_fn, **kw):
+    sae, ref, batch = make_pair(pkg, oracle, dev, **kw)
+    sae.cfg.act_fn = act_fn
+    sae.activation_function = sae.activation_function_factory(None)
+    ref.act_fn = act_fn
+    ref.activation_function = ref._make_activation()
+    return sae, ref, batch
+
+
+@pytest.mark.parametrize("amp", [False, True])
+def test_fused_batchtopk_step_matches_oracle(pkg, oracle, dev, amp):
+    print(f"fused batchtopk amp={amp}", flush=True)
+    sae, ref, batch = make_pair_act(pkg, oracle, dev, "batchtopk", d=256, F=2048, k=16, B=192, r=8, seed=11,
+                                    include_norm=True)
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=amp, substitute=True)
+    tol = BF16_TOL if amp else FP32_TOL
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert (rctx["feature_acts"] != 0).sum().item() == 16 * 192
+    assert (rctx["feature_acts"] != 0).sum(-1).float().std().item() > 0  # rows really differ in length
+    assert rel_err(ctx["reconstructed"], rctx["reconstructed"]) < tol
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < tol
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        assert rel_err(getattr(sae, name).grad, getattr(ref, name).grad) < tol, name
+
+
+@pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
+@pytest.mark.parametrize("include_norm", [False, True])
+def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm):
+    print(f"fused aux-k {act_fn} include_norm={include_norm}", flush=True)
+    B, F, k, k_aux = 192, 2048, 16, 24
+    sae, ref, batch = make_pair_act(pkg, oracle, dev, act_fn, d=256, F=F, k=k, B=B, r=8, seed=12, include_norm=include_norm,
+                                    mask_frac=0.2)
+    trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=1 / 32, k_aux=k_aux, dead_threshold=float(B)))
+    trainer._initialize_dead_statistics(sae)
+    stats = oracle.DeadStatistics(F, dead_threshold=float(B))
+    # one earlier batch so that the counters are not all zero
+    warm = torch.zeros(B, F); warm[:, ::7] = 1.0
+    trainer.update_dead_statistics(warm.to(dev), None, ("batch", "sae"))
+    stats.update(warm, None, 1)
+
+    gbatch = {k_: v.to(dev) for k_, v in batch.items()}
+    kw = dict(auxk_coefficient=1 / 32, k_aux=k_aux)
+    ctx = sae.compute_loss(gbatch, update_dead_statistics=trainer.update_dead_statistics, **kw)
+    ctx["loss"].backward()
+    # oracle with the HIP GEMM's forward values (see run_both)
+    sae_pre = pkg.ops.encoder_gemm(gbatch["in"].contiguous(), sae._w_enc_operand(False), torch.float32).cpu()
+
+    def encode_sub(x, return_hidden_pre=False, **_):
+        mm = _SubstitutedMatmul.apply(x, ref.W_E, sae_pre)
+        hp = mm + ref.b_E
+        if ref.sparsity_include_decoder_norm:
+            hp = hp * ref.decoder_norm()
+        fa = ref.activation_function(hp)
+        if ref.sparsity_include_decoder_norm:
+            fa = fa / ref.decoder_norm()
+            hp = hp / ref.decoder_norm()
+        return (fa, hp) if return_hidden_pre else fa
+
+    ref.encode = encode_sub
+    rctx = ref.compute_loss(batch, update_dead_statistics=stats.update, **kw)
+    rctx["loss"].backward()
+
+    assert torch.equal(trainer.is_dead.cpu(), stats.is_dead)
+    assert torch.equal(trainer.tokens_since_last_activation.cpu(), stats.tokens_since_last_activation)
+    assert stats.is_dead.sum().item() > k_aux  # plenty of dead features: the aux select really truncates
+    assert rctx["l_aux"].item() > 0
+    assert abs(ctx["l_aux"].item() - rctx["l_aux"].item()) / rctx["l_aux"].item() < FP32_TOL
+    assert abs(ctx["l_rec"].item() - rctx["l_rec"].item()) / rctx["l_rec"].item() < FP32_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < FP32_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        assert rel_err(getattr(sae, name).grad, getattr(ref, name).grad) < FP32_TOL, name
+    assert sae.current_k == k and ref.current_k == k
+
+
+def test_fused_auxk_without_dead_features_is_plain_loss(pkg, oracle, dev):
+    sae, ref, batch = make_pair_act(pkg, oracle, dev, "topk", d=256, F=2048, k=16, B=192, r=8, seed=13, include_norm=True)
+    trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=0.5, k_aux=8, dead_threshold=1e9))
+    trainer._initialize_dead_statistics(sae)
+    gbatch = {k_: v.to(dev) for k_, v in batch.items()}
+    ctx = sae.compute_loss(gbatch, auxk_coefficient=0.5, k_aux=8, update_dead_statistics=trainer.update_dead_statistics)
+    plain = sae.compute_loss(gbatch)
+    assert ctx["l_aux"].item() == 0.0
+    assert abs(ctx["loss"].item() - plain["loss"].item()) <= 1e-6 * plain["loss"].item()

@@ -162,3 +162,48 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_lr_schedules_hand_values(pkg):
+    p = torch.nn.Parameter(torch.zeros(1))
+
+    def lrs(name, n, **kw):
+        opt = torch.optim.SGD([p], lr=1.0)
+        sch = pkg.get_scheduler(name, opt, **kw)
+        out = []
+        for _ in range(n):
+            out.append(opt.param_groups[0]["lr"])
+            opt.step(); sch.step()
+        return out
+
+    assert lrs("constant", 3) == [1.0, 1.0, 1.0]
+    got = lrs("constantwithwarmup", 10, warm_up_steps=4, cool_down_steps=2, training_steps=10, lr_end_ratio=0.0)
+    assert got[:4] == [0.25, 0.5, 0.75, 1.0] and got[4:9] == [1.0] * 5 and got[9] == 0.5
+    got = lrs("linearwarmupdecay", 6, warm_up_steps=2, training_steps=6)
+    assert got == [0.5, 1.0, 1.0, 0.75, 0.5, 0.25]
+    got = lrs("cosineannealingwarmup", 5, warm_up_steps=1, training_steps=5, lr_end=0.0)
+    assert got[0] == 1.0 and abs(got[3] - 0.5 * (1 + math.cos(math.pi * 2 / 4))) < 1e-12
+    got = lrs("exponentialwarmup", 4, warm_up_steps=1, training_steps=4, lr_end=1 / 8)
+    assert abs(got[2] - (1 / 8) ** (1 / 3)) < 1e-12
+    with pytest.raises(ValueError):
+        pkg.get_scheduler("nope", torch.optim.SGD([p], lr=1.0), training_steps=3)
+
+
+def test_trainer_config_defaults_follow_the_reference(pkg):
+    c = pkg.TrainerConfig()
+    assert c.l1_coefficient == 8e-5 and c.l1_coefficient_warmup_steps == 0.1 and c.lr == 4e-4 and c.betas == (0.9, 0.999)
+    assert c.k_aux == 512 and c.dead_threshold == 1e7 and c.amp_dtype == torch.bfloat16 and c.clip_grad_norm == 0.0
+    assert c.lr_scheduler_name == "constantwithwarmup" and c.lr_warm_up_steps == 5000 and c.lr_end_ratio == 1 / 32
+    assert c.optimizer_class == "adam" and c.tanh_stretch_coefficient == 4.0 and c.frequency_scale == 0.01
+
+
+def test_trainer_dead_statistics_dense_form_on_cpu(pkg, oracle):
+    t = pkg.Trainer(pkg.TrainerConfig(dead_threshold=5))
+    t.tokens_since_last_activation = torch.zeros(3, dtype=torch.long)
+    t.is_dead = torch.zeros(3, dtype=torch.bool)
+    ref = oracle.DeadStatistics(3, dead_threshold=5)
+    for acts, mask in [(torch.tensor([[1.0, 0, 0], [0, 0, 0]]), None), (torch.tensor([[1.0, 0, 0], [0, 0, 0]]), torch.tensor([1.0, 0.0])),
+                       (torch.tensor([[0, 2.0, 0], [0, 0, 0]]), None)]:
+        a = t.update_dead_statistics(acts, mask, ("batch", "sae")); b = ref.update(acts, mask, 1)
+        assert torch.equal(a, b) and torch.equal(t.tokens_since_last_activation, ref.tokens_since_last_activation)
+    assert t.is_dead.tolist() == [False, False, True]
