@@ -21,3 +21,10 @@ from .optim import HipSparseAdam, clip_grad_norm, compute_grad_norm  # noqa: E40
 from .trainer import Trainer, TrainerConfig, get_scheduler  # noqa: E402,F401
 
 __all__ += ["HipSparseAdam", "clip_grad_norm", "compute_grad_norm", "Trainer", "TrainerConfig", "get_scheduler"]
+
+from .config import CLTConfig, CrosscoderConfig, LorsaConfig  # noqa: E402,F401
+from .crosscoder import Crosscoder  # noqa: E402,F401
+from .clt import CrossLayerTranscoder  # noqa: E402,F401
+from .lorsa import LowRankSparseAttention  # noqa: E402,F401
+
+__all__ += ["CrosscoderConfig", "CLTConfig", "LorsaConfig", "Crosscoder", "CrossLayerTranscoder", "LowRankSparseAttention"]

@@ -1,0 +1,399 @@
+"""Cross-layer transcoder on the HIP path.
+
+API of the reference's CLT (src/llamascopium/models/clt.py:124-1125): L encoders `W_E [L, d, F]`,
+`b_E [L, F]`; decoder groups `W_D[j] [j+1, F, d]` (sources 0..j writing to layer j) with biases
+`b_D[j] [d]`; output layer j is  y_j = sum_{i<=j} f_i @ W_D[j][i] + b_D[j].
+
+Memory layout: `W_E` has the reference's shape but each layer is stored feature-major (a permuted
+view of a contiguous [L, F, d] buffer), so every layer's encoder is one call of the encoder GEMM.
+A decoder group is contiguous, so `W_D[j]` read as a [(j+1)*F, d] matrix is the decoder of the
+concatenated feature space of layers 0..j.
+
+Fused path (TopK family): the activations of all layers are held as ONE sparse code over the
+concatenated L*F feature space with every token's entries in ascending (layer, feature) order.
+Output layer j then decodes the per-token PREFIX of that code (the entries of layers <= j) against
+`W_D[j]`, i.e. the 78 dense [B, F] x [F, d] products of a 12-layer CLT become 12 sparse decodes, and
+one feature index of the whole code serves every weight gradient (a feature range of it is the
+index of a layer, a feature prefix the index of a decoder group).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Any, Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .activation_functions import JumpReLU, _topk_mask_lowest_index, topk_dense
+from .config import CLTConfig, register_sae_model
+from .sae import _autocast_dtype
+from .sparse_dictionary import LazyDict, SparseDictionary
+
+_TOPK_FAMILY = ("topk", "layertopk", "batchtopk", "batchlayertopk")
+
+
+def _slot_tokens(code: ops.SparseCode):
+    """(token of every slot [n_slots] int64, slot-is-inside-its-row [n_slots] bool)."""
+    slots = torch.arange(code.n_slots, device=code.idx.device)
+    tok = torch.searchsorted(code.row_off, slots, right=True) - 1
+    tok = tok.clamp_(min=0)
+    valid = (slots - code.row_off[tok]) < code.row_nnz[tok]
+    return tok, valid
+
+
+def merge_layer_codes(codes: list[ops.SparseCode]) -> tuple[ops.SparseCode, torch.Tensor]:
+    """Per-layer codes over F features each -> one code over L*F features (feature l*F + f), every
+    token's entries sorted by (layer, feature); also the per-token per-layer entry counts [B, L]."""
+    L, B, F = len(codes), codes[0].n_tokens, codes[0].d_sae
+    keys, vals = [], []
+    sentinel = torch.iinfo(torch.int64).max
+    for l, c in enumerate(codes):
+        tok, valid = _slot_tokens(c)
+        key = tok * (L * F) + (l * F) + c.idx.long()
+        keys.append(torch.where(valid, key, torch.full_like(key, sentinel)))
+        vals.append(c.val)
+    key, perm = torch.sort(torch.cat(keys))
+    val = torch.cat(vals)[perm]
+    layer_cnt = torch.stack([c.row_nnz for c in codes], dim=1)                     # [B, L]
+    row_nnz = layer_cnt.sum(dim=1).to(torch.int32)
+    row_off = torch.cumsum(row_nnz, 0, dtype=torch.int64) - row_nnz
+    idx = torch.where(key == sentinel, torch.zeros_like(key), key % (L * F)).to(torch.int32)
+    return ops.SparseCode(idx, val.contiguous(), row_off, row_nnz, B, L * F), layer_cnt
+
+
+def layer_counts(code: ops.SparseCode, L: int, F: int) -> torch.Tensor:
+    """Entries per (token, layer) [B, L] of a code over L*F features."""
+    tok, valid = _slot_tokens(code)
+    cell = tok * L + torch.div(code.idx.long(), F, rounding_mode="floor")
+    cell = torch.where(valid, cell, torch.zeros_like(cell))     # slots outside their row add 0 to cell 0
+    cnt = torch.zeros(code.n_tokens * L, dtype=torch.int32, device=code.idx.device)
+    cnt.scatter_add_(0, cell, valid.to(torch.int32))
+    return cnt.view(code.n_tokens, L)
+
+
+class _FusedCLTStep(torch.autograd.Function):
+    """L encoder GEMMs -> TopK-family select -> L prefix decodes + squared error, forward and backward
+    in kernels.  Arguments after `holder` are the parameters: W_E, b_E, W_D[0..L-1], b_D[0..L-1]."""
+
+    @staticmethod
+    def forward(ctx, x, label, amp, holder, W_E, b_E, *dec):
+        m: "CrossLayerTranscoder" = holder["model"]
+        B, L, d = x.shape
+        F = m.cfg.d_sae
+        k = int(m.current_k)
+        act = m.cfg.act_fn.lower()
+        w_enc_op = m._w_enc_operand(amp)                                   # [L, F, d]
+        x_l = x.permute(1, 0, 2).contiguous()                              # [L, B, d]
+        if amp:
+            x_op = ops.cast_bf16(x_l.view(L * B, d)).view(L, B, d) if x_l.dtype != torch.bfloat16 else x_l
+        else:
+            x_op = x_l
+        out_dtype = torch.bfloat16 if amp else torch.float32
+        pres = [ops.encoder_gemm(x_op[l], w_enc_op[l], out_dtype) for l in range(L)]
+        norms = m._norm_per_feature_nograd() if m.cfg.sparsity_include_decoder_norm else None     # [L, F]
+        b_enc = b_E.detach().float().contiguous()
+        if act in ("topk", "batchtopk"):
+            sel = (lambda p, b, s: ops.select_topk_row(p, b, s, min(k, F))) if act == "topk" else \
+                  (lambda p, b, s: ops.select_topk_batch(p, b, s, k * B))
+            codes = [sel(pres[l], b_enc[l], None if norms is None else norms[l]) for l in range(L)]
+            cat, layer_cnt = merge_layer_codes(codes)
+        else:
+            pre_cat = torch.stack(pres, dim=1).view(B, L * F)
+            flat = lambda t: None if t is None else t.reshape(L * F)      # noqa: E731
+            if act == "layertopk":
+                cat = ops.select_topk_row(pre_cat, flat(b_enc), flat(norms), min(k, L * F))
+            else:
+                cat = ops.select_topk_batch(pre_cat, flat(b_enc), flat(norms), k * B)
+            layer_cnt = layer_counts(cat, L, F)
+        prefix = torch.cumsum(layer_cnt, dim=1).to(torch.int32)           # entries of layers <= j, per token
+        _, valid = _slot_tokens(cat)
+        slot_layer = torch.div(cat.idx, F, rounding_mode="floor")
+        tok_w = torch.full((B,), 1.0 / (L * B), dtype=torch.float32, device=x.device)
+        w_dec_ops = m._w_dec_operands(amp)
+        b_D = dec[L:]
+        recons, grads = [], []
+        dval = torch.zeros(cat.n_slots, dtype=torch.float32, device=x.device)
+        loss = None
+        for j in range(L):
+            code_j = dataclasses.replace(cat, row_nnz=prefix[:, j].contiguous(), d_sae=(j + 1) * F)
+            recon, loss_tok, grad_recon, dval_j = ops.sparse_decode_mse_fused(
+                code_j, w_dec_ops[j].view((j + 1) * F, d), b_D[j].detach(), label[j].contiguous(), tok_w)
+            dval = dval + torch.where(valid & (slot_layer <= j), dval_j, torch.zeros_like(dval_j))
+            recons.append(recon); grads.append(grad_recon)
+            loss = loss_tok.sum() if loss is None else loss + loss_tok.sum()
+        recon = torch.stack(recons, dim=0)
+        holder.update(code=cat, pres=pres, norms=norms, layer_cnt=layer_cnt)
+        ctx.cat, ctx.grads, ctx.dval, ctx.x_op, ctx.w_enc_op = cat, grads, dval, x_op, w_enc_op
+        ctx.shape = (B, L, d, F)
+        ctx.mark_non_differentiable(recon)
+        return loss, recon
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_recon):
+        B, L, d, F = ctx.shape
+        g = g_loss.to(torch.float32)
+        cat = ctx.cat
+        fi = ops.build_feature_index(cat)
+        coef_dec = cat.val * g
+        coef_enc = ctx.dval * g
+        dW_D, db_D, dW_E, db_E = [], [], [], []
+        for j in range(L):
+            fi_j = ops.FeatureIndex(fi.feat_ptr[: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)      # features of layers <= j
+            rows, _ = ops.sparse_grad_rows(fi_j, coef_dec, ctx.grads[j], (j + 1) * F)
+            dW_D.append(rows.view(j + 1, F, d))
+            db_D.append(ops.col_sum(ctx.grads[j]) * g)
+            fi_l = ops.FeatureIndex(fi.feat_ptr[j * F: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)  # features of layer j
+            rows_e, bias_e = ops.sparse_grad_rows(fi_l, coef_enc, ctx.x_op[j], F, want_bias=True)
+            dW_E.append(rows_e); db_E.append(bias_e)
+        dW_E = torch.stack(dW_E).permute(0, 2, 1)                       # [L, F, d] buffer seen as [L, d, F]
+        dx = dlabel = None
+        if ctx.needs_input_grad[0]:
+            # d x[:, l] = sum over layer l's kept entries of d(pre) * W_E[l][:, f]
+            w_all = ctx.w_enc_op.reshape(L * F, d)
+            parts = []
+            slot_layer = torch.div(cat.idx, F, rounding_mode="floor")
+            for l in range(L):
+                c = dataclasses.replace(cat, val=torch.where(slot_layer == l, coef_enc, torch.zeros_like(coef_enc)))
+                parts.append(ops.sparse_decode_fwd(c, w_all, None))
+            dx = torch.stack(parts, dim=1)
+        if ctx.needs_input_grad[1]:
+            dlabel = -torch.stack(ctx.grads, dim=0) * g
+        return (dx, dlabel, None, None, dW_E, torch.stack(db_E), *dW_D, *db_D)
+
+
+@register_sae_model("clt")
+class CrossLayerTranscoder(SparseDictionary):
+    def __init__(self, cfg: CLTConfig, device_mesh=None):
+        super().__init__(cfg, device_mesh=device_mesh)
+        self.cfg = cfg
+        L, d, F = cfg.n_layers, cfg.d_model, cfg.d_sae
+        kw = dict(device=cfg.device, dtype=cfg.dtype)
+        self.W_E = nn.Parameter(torch.empty(L, F, d, **kw).permute(0, 2, 1))   # shape [L, d, F], per-layer feature-major
+        self.b_E = nn.Parameter(torch.empty(L, F, **kw))
+        self.W_D = nn.ParameterList([nn.Parameter(torch.empty(i + 1, F, d, **kw)) for i in range(L)])
+        self.b_D = nn.ParameterList([nn.Parameter(torch.empty(d, **kw)) for _ in range(L)])
+        self._norm_cache: Optional[tuple[tuple[int, ...], torch.Tensor]] = None
+
+    # ---- activations (clt.py:232-387): the selection scope depends on the name ----
+    def activation_function_factory(self, device_mesh=None):
+        act = self.cfg.act_fn.lower()
+        assert act in ["relu", "topk", "jumprelu", "batchtopk", "layertopk", "batchlayertopk"], (
+            f"Not implemented activation function {self.cfg.act_fn}")
+        if act == "relu":
+            return lambda x: x * x.gt(0).to(x.dtype)
+        if act == "jumprelu":
+            return JumpReLU(self.cfg.jumprelu_threshold_window, shape=(self.cfg.n_layers, self.cfg.d_sae),
+                            dims_to_keep_in_bwd=(-2, -1), device=self.cfg.device, dtype=self.cfg.dtype)
+        if act == "topk":
+            def topk_activation(x: torch.Tensor):
+                if x.is_cuda:
+                    return topk_dense(x, self.current_k)
+                raise RuntimeError("the TopK activation runs on the GPU only (no CPU fallback in this build)")
+            return topk_activation
+
+        def scoped(x: torch.Tensor):
+            # dense form of the wider scopes: positive part, then keep the k (or k * batch) largest of every
+            # group; a group's members are flattened in the order the reference permutes them (selected dims last,
+            # in the order named), so ties fall to the same element
+            r = x * x.gt(0).to(x.dtype)
+            B, L, F = r.shape
+            if act == "layertopk":
+                groups, kk = r.reshape(B, L * F), self.current_k
+            elif act == "batchtopk":
+                groups, kk = r.permute(1, 0, 2).reshape(L, B * F), self.current_k * B
+            else:  # batchlayertopk: dims (0, -1, -2) -> batch, feature, layer
+                groups, kk = r.permute(0, 2, 1).reshape(1, B * F * L), self.current_k * B
+            with torch.no_grad():
+                mask = _topk_mask_lowest_index(groups, kk)
+                if act == "layertopk":
+                    mask = mask.view(B, L, F)
+                elif act == "batchtopk":
+                    mask = mask.view(L, B, F).permute(1, 0, 2)
+                else:
+                    mask = mask.view(B, F, L).permute(0, 2, 1)
+            return r * mask.to(r.dtype)
+        return scoped
+
+    # ---- kernel operands ----
+    def _w_enc_operand(self, amp: bool) -> torch.Tensor:
+        wt = self.W_E.detach().permute(0, 2, 1)
+        wt = wt if wt.is_contiguous() else wt.contiguous()
+        if not amp or wt.dtype == torch.bfloat16:
+            return wt
+        L, d, F = self.cfg.n_layers, self.cfg.d_model, self.cfg.d_sae
+        return self._derive("W_E.bf16", self.W_E, lambda old: ops.cast_bf16(
+            wt.view(L * F, d), None if old is None else old.view(L * F, d))).view(L, F, d)
+
+    def _w_dec_operands(self, amp: bool) -> list[torch.Tensor]:
+        out = []
+        for j, w in enumerate(self.W_D):
+            wd = w.detach()
+            if amp and wd.dtype != torch.bfloat16:
+                F, d = self.cfg.d_sae, self.cfg.d_model
+                wd = self._derive(f"W_D.{j}.bf16", w, lambda old, wd=wd, j=j: ops.cast_bf16(
+                    wd.view((j + 1) * F, d), None if old is None else old.view((j + 1) * F, d))).view(j + 1, F, d)
+            out.append(wd)
+        return out
+
+    def _norm_per_feature_nograd(self) -> torch.Tensor:
+        """decoder_norm_per_feature() through the row-norm kernel, cached until a decoder group changes."""
+        vers = tuple(w._version for w in self.W_D)
+        if self._norm_cache is not None and self._norm_cache[0] == vers and self._norm_cache[1].device == self.W_D[0].device:
+            return self._norm_cache[1]
+        L, d, F = self.cfg.n_layers, self.cfg.d_model, self.cfg.d_sae
+        with torch.no_grad():
+            sq = torch.zeros(L, F, dtype=torch.float32, device=self.W_D[0].device)
+            for j, w in enumerate(self.W_D):
+                n = ops.row_norm(w.detach().float().view((j + 1) * F, d)).view(j + 1, F)
+                sq[: j + 1] += n * n
+            norms = sq.sqrt_()
+        self._norm_cache = (vers, norms)
+        return norms
+
+    # ---- norms (clt.py:801-907) ----
+    def decoder_norm(self, keepdim: bool = False):
+        return torch.ones(self.cfg.n_decoders, device=self.W_E.device, dtype=self.cfg.dtype)
+
+    def encoder_norm(self, keepdim: bool = False):
+        return torch.norm(self.W_E, p=2, dim=1, keepdim=keepdim)
+
+    def decoder_bias_norm(self):
+        return torch.ones(self.cfg.n_layers, device=self.W_E.device, dtype=self.cfg.dtype)
+
+    @torch.no_grad()
+    def decoder_norm_per_feature(self, layer: Optional[int] = None) -> torch.Tensor:
+        L, F = self.cfg.n_layers, self.cfg.d_sae
+        norms = torch.zeros(L, F, dtype=self.cfg.dtype, device=self.W_E.device)
+        if layer is not None:
+            for layer_to in range(layer, L):
+                norms[layer_to] = self.W_D[layer_to][layer].pow(2).sum(dim=-1).sqrt()
+            return norms
+        for layer_to, w in enumerate(self.W_D):
+            norms[: layer_to + 1] = norms[: layer_to + 1] + w.pow(2).sum(dim=-1)
+        return norms.sqrt()
+
+    @torch.no_grad()
+    def decoder_norm_per_decoder(self) -> torch.Tensor:
+        return torch.cat([torch.norm(w, p=2, dim=(1, 2)) for w in self.W_D])
+
+    def get_decoder_weights(self, layer_to: int) -> torch.Tensor:
+        return self.W_D[layer_to]
+
+    @torch.no_grad()
+    def init_parameters(self, **kwargs):
+        """clt.py:390-467: encoders U(+-1/sqrt(F)), every decoder U(+-1/sqrt(L d)), zero biases."""
+        super().init_parameters(**kwargs)
+        eb = 1.0 / math.sqrt(self.cfg.d_sae)
+        db = 1.0 / math.sqrt(self.cfg.n_layers * self.cfg.d_model)
+        self.W_E.uniform_(-eb, eb)
+        self.b_E.zero_()
+        for w in self.W_D:
+            w.uniform_(-db, db)
+            if self.cfg.init_cross_layer_decoder_all_zero:
+                w[:-1] = 0
+        for b in self.b_D:
+            b.zero_()
+
+    @torch.no_grad()
+    def standardize_parameters_of_dataset_norm(self):
+        """clt.py:908-937: fold the per-layer dataset norms into the weights."""
+        assert self.cfg.norm_activation == "dataset-wise"
+        assert self.dataset_average_activation_norm is not None
+        fin = lambda l: math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_points_in[l]]    # noqa: E731
+        fout = lambda l: math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_points_out[l]]  # noqa: E731
+        for l in range(self.cfg.n_layers):
+            self.W_E.data[l].mul_(fin(l))
+        for layer_to in range(self.cfg.n_layers):
+            self.W_D[layer_to].div_(fout(layer_to))
+            self.b_D[layer_to].div_(fout(layer_to))
+        self.cfg.norm_activation = "inference"
+
+    # ---- API path over dense tensors (clt.py:527-709) ----
+    def encode(self, x: torch.Tensor, return_hidden_pre: bool = False, **kwargs):
+        hidden_pre = torch.einsum("...ld,lds->...ls", x, self.W_E) + self.b_E
+        if self.cfg.sparsity_include_decoder_norm:
+            hidden_pre = hidden_pre * self.decoder_norm_per_feature()
+        feature_acts = self.activation_function(hidden_pre)
+        if self.cfg.sparsity_include_decoder_norm:
+            feature_acts = feature_acts / self.decoder_norm_per_feature()
+        return (feature_acts, hidden_pre) if return_hidden_pre else feature_acts
+
+    def decode(self, feature_acts: torch.Tensor, batch_first: bool = False, **kwargs):
+        out = []
+        for layer_to in range(self.cfg.n_layers):
+            contribution = (feature_acts[..., : layer_to + 1, :].permute(1, 0, 2) @ self.W_D[layer_to]).sum(0)
+            out.append(contribution + self.b_D[layer_to])
+        return torch.stack(out, dim=1 if batch_first else 0)
+
+    def prepare_input(self, batch: dict[str, torch.Tensor], **kwargs) -> tuple[torch.Tensor, dict[str, Any], dict[str, Any]]:
+        xs = []
+        for hp in self.cfg.hook_points_in:
+            if hp not in batch:
+                raise ValueError(f"Missing hook point {hp} in batch")
+            xs.append(batch[hp])
+        return torch.stack(xs, dim=xs[0].ndim - 1), {}, {}
+
+    def prepare_label(self, batch: dict[str, torch.Tensor], **kwargs) -> torch.Tensor:
+        ys = []
+        for hp in self.cfg.hook_points_out:
+            if hp not in batch:
+                raise ValueError(f"Missing hook point {hp} in batch")
+            ys.append(batch[hp])
+        return torch.stack(ys, dim=0)
+
+    # ---- loss (clt.py:1024-1104) ----
+    def _fused_eligible(self, x, sparsity_loss_type) -> bool:
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        return (self.cfg.act_fn.lower() in _TOPK_FAMILY and x.is_cuda and x.ndim == 3 and sparsity_loss_type is None
+                and self.W_E.dtype == torch.float32 and self.cfg.d_model % (64 if amp else 32) == 0)
+
+    def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,
+                     frequency_scale: float = 0.01, p: int = 1, l1_coefficient: float = 1.0, return_aux_data: bool = True,
+                     **kwargs):
+        x, enc_kw, dec_kw = self.prepare_input(batch)
+        label = self.prepare_label(batch, **kwargs)
+        mask = batch.get("mask")
+        n_tokens = (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item()))
+        if self._fused_eligible(x, sparsity_loss_type):
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            holder: dict[str, Any] = {"model": self}
+            xin = x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x
+            loss, recon = _FusedCLTStep.apply(xin, label.to(torch.float32), amp, holder, self.W_E, self.b_E,
+                                              *self.W_D, *self.b_D)
+            if not return_aux_data:
+                return loss
+            B, L, F = x.shape[0], self.cfg.n_layers, self.cfg.d_sae
+            eager = {"loss": loss, "l_rec": loss, "l_s": None, "label": label, "mask": mask, "reconstructed": recon,
+                     "sparse_code": holder["code"]}
+            lazy = {"n_tokens": n_tokens, "feature_acts": lambda: holder["code"].to_dense().view(B, L, F)}
+            return LazyDict(eager, lazy)
+
+        feature_acts = self.encode(x, **enc_kw)
+        reconstructed = self.decode(feature_acts, **dec_kw)
+        l_rec = (reconstructed - label).pow(2).sum(dim=-1).mean()
+        loss_dict: dict[str, Optional[torch.Tensor]] = {"l_rec": l_rec}
+        loss = l_rec
+        if sparsity_loss_type is not None:
+            n = self.decoder_norm_per_feature()
+            if sparsity_loss_type == "power":
+                l_s = torch.norm(feature_acts * n, p=p, dim=-1)
+            elif sparsity_loss_type == "tanh":
+                l_s = torch.tanh(tanh_stretch_coefficient * feature_acts * n).sum(dim=-1)
+            elif sparsity_loss_type == "tanh-quad":
+                t = torch.tanh(tanh_stretch_coefficient * feature_acts * n)
+                freq = t.mean(dim=tuple(range(t.ndim - 1)))
+                l_s = (freq * (1 + freq / frequency_scale)).sum(dim=-1)
+            else:
+                raise ValueError(f"sparsity_loss_type f{sparsity_loss_type} not supported.")
+            l_s = l1_coefficient * l_s
+            loss_dict["l_s"] = l_s
+            loss = loss + l_s.mean()
+        else:
+            loss_dict["l_s"] = None
+        if not return_aux_data:
+            return loss
+        return {"loss": loss, **loss_dict, "label": label, "mask": mask, "n_tokens": n_tokens(),
+                "feature_acts": feature_acts, "reconstructed": reconstructed}

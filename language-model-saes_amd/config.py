@@ -107,3 +107,121 @@ class SAEConfig(SparseDictionaryConfig):
     @property
     def hooks_out(self) -> list[str]:
         return [self.hook_point_out]
+
+
+@register_sae_config("crosscoder")
+class CrosscoderConfig(SparseDictionaryConfig):
+    """models/crosscoder.py:60-81: one head per hook point; reads and writes the same hook points."""
+
+    sae_type: str = "crosscoder"
+    hook_points: list[str]
+
+    @property
+    def associated_hook_points(self) -> list[str]:
+        return self.hook_points
+
+    @property
+    def hooks_in(self) -> list[str]:
+        return self.hook_points
+
+    @property
+    def hooks_out(self) -> list[str]:
+        return self.hook_points
+
+    @property
+    def n_heads(self) -> int:
+        return len(self.hook_points)
+
+
+@register_sae_config("clt")
+class CLTConfig(SparseDictionaryConfig):
+    """models/clt.py:67-121: L encoders, L(L+1)/2 decoders (layer i writes to layers i..L-1)."""
+
+    sae_type: str = "clt"
+    act_fn: Literal["relu", "jumprelu", "topk", "batchtopk", "batchlayertopk", "layertopk"] = "relu"
+    init_cross_layer_decoder_all_zero: bool = False
+    hook_points_in: list[str]
+    hook_points_out: list[str]
+    # Kept for config compatibility: the reference switches its decode to torch CSR matrices with these;
+    # here the sparse decode kernel is used whenever the activation is of the TopK family.
+    decode_with_csr: bool = False
+    sparsity_threshold_for_csr: float = 0.05
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.hook_points_in)
+
+    @property
+    def n_decoders(self) -> int:
+        return self.n_layers * (self.n_layers + 1) // 2
+
+    @property
+    def associated_hook_points(self) -> list[str]:
+        return self.hook_points_in + self.hook_points_out
+
+    @property
+    def hooks_in(self) -> list[str]:
+        return self.hook_points_in
+
+    @property
+    def hooks_out(self) -> list[str]:
+        return self.hook_points_out
+
+    def model_post_init(self, __context):
+        super().model_post_init(__context)
+        assert len(self.hook_points_in) == len(self.hook_points_out), "Number of input and output hook points must match"
+
+
+@register_sae_config("lorsa")
+class LorsaConfig(SparseDictionaryConfig):
+    """models/lorsa.py:45-106: every dictionary feature is a rank-1 value/output head; groups of
+    d_sae / n_qk_heads features share one query/key head."""
+
+    sae_type: str = "lorsa"
+    hook_point_in: str
+    hook_point_out: str
+    n_qk_heads: int
+    d_qk_head: int
+    positional_embedding_type: Literal["rotary", "none"] = "rotary"
+    rotary_dim: int
+    rotary_base: int = 10000
+    rotary_adjacent_pairs: bool = True
+    rotary_scale: int = 1
+    use_NTK_by_parts_rope: bool = False
+    NTK_by_parts_factor: float = 1.0
+    NTK_by_parts_low_freq_factor: float = 1.0
+    NTK_by_parts_high_freq_factor: float = 1.0
+    old_context_len: int = 2048
+    n_ctx: int
+    attn_scale: Optional[float] = None
+    use_post_qk_ln: bool = False
+    normalization_type: Optional[Literal["LN", "RMS"]] = None
+    eps: float = 1e-6
+
+    @property
+    def n_ov_heads(self) -> int:
+        return self.d_sae
+
+    @property
+    def ov_group_size(self) -> int:
+        return self.n_ov_heads // self.n_qk_heads
+
+    @property
+    def associated_hook_points(self) -> list[str]:
+        return [self.hook_point_in, self.hook_point_out]
+
+    @property
+    def hooks_in(self) -> list[str]:
+        return [self.hook_point_in]
+
+    @property
+    def hooks_out(self) -> list[str]:
+        return [self.hook_point_out]
+
+    def model_post_init(self, __context):
+        super().model_post_init(__context)
+        assert self.hook_point_in is not None and self.hook_point_out is not None, "hook_point_in and hook_point_out must be set"
+        assert self.hook_point_in != self.hook_point_out, "hook_point_in and hook_point_out must be different"
+        assert self.n_ov_heads % self.n_qk_heads == 0, "n_ov_heads must be divisible by n_qk_heads"
+        if self.attn_scale is None:
+            self.attn_scale = self.d_qk_head ** 0.5

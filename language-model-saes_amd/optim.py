@@ -28,13 +28,20 @@ class _null_ctx:
         return False
 
 
-def _flat_view(p: torch.Tensor) -> torch.Tensor:
-    """A contiguous view over p's memory (p itself, or its transpose for feature-major 2-D weights)."""
+def _flat_order(p: torch.Tensor):
+    """Permutation of p's dims under which its memory is contiguous (None if there is none)."""
     if p.is_contiguous():
-        return p
-    if p.ndim == 2 and p.t().is_contiguous():
-        return p.t()
-    raise ValueError(f"parameter with strides {p.stride()} is neither contiguous nor a transposed contiguous matrix")
+        return tuple(range(p.ndim))
+    order = tuple(sorted(range(p.ndim), key=lambda i: -p.stride(i)))
+    return order if p.permute(order).is_contiguous() else None
+
+
+def _flat_view(p: torch.Tensor) -> torch.Tensor:
+    """A contiguous view over p's memory (p itself, or the permutation that undoes a feature-major layout)."""
+    order = _flat_order(p)
+    if order is None:
+        raise ValueError(f"parameter with strides {p.stride()} is not a permuted contiguous tensor")
+    return p if order == tuple(range(p.ndim)) else p.permute(order)
 
 
 class HipAdam(Optimizer):
@@ -177,7 +184,7 @@ class HipAdam(Optimizer):
                 same_layout = lambda t: _flat_view(t) if t.stride() == p.stride() else None  # noqa: E731
                 gv, mv, vv = same_layout(p.grad), same_layout(st["exp_avg"]), same_layout(st["exp_avg_sq"])
                 if gv is None:
-                    gv = _flat_view(p.grad.contiguous()) if p.is_contiguous() else p.grad.t().contiguous()
+                    gv = p.grad.permute(_flat_order(p)).contiguous()
                 assert mv is not None and vv is not None, "optimizer state must share the parameter's layout"
                 role, shadow, norm_out = self._by_products(p, pv)
                 ops.adam_step(pv, gv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"],
@@ -229,7 +236,7 @@ class HipSparseAdam(Optimizer):
                     st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 pv = _flat_view(p)
-                gv = _flat_view(p.grad) if p.grad.stride() == p.stride() else _flat_view(p.grad.contiguous())
+                gv = _flat_view(p.grad) if p.grad.stride() == p.stride() else p.grad.permute(_flat_order(p)).contiguous()
                 ops.sparse_adam_step(pv, gv, _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"]), st["step"],
                                      lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"])
                 torch.autograd.graph.increment_version(p)

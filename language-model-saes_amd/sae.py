@@ -203,8 +203,6 @@ class SparseAutoEncoder(SparseDictionary):
         self.hook_hidden_pre = HookPoint()
         self.hook_feature_acts = HookPoint()
         self.hook_reconstructed = HookPoint()
-        # derived operands (bf16 shadows, row norms) keyed by name -> (param version, tensor)
-        self._derived: dict[str, tuple[int, torch.Tensor]] = {}
         # set by an optimiser that consumes SparseRowGrad (HipAdam): the fused backward then leaves W_E.grad /
         # W_D.grad unset and attaches the factored gradient as `param._sparse_grad` instead
         self.defer_weight_grads = False
@@ -218,25 +216,6 @@ class SparseAutoEncoder(SparseDictionary):
         if ev is not None:
             torch.cuda.current_stream(self.W_D.device).wait_event(ev)
             self._pending_update = None
-
-    # ---- derived operands, refreshed when the parameter's version counter moves ----
-    def _derive(self, name: str, param: torch.Tensor, make) -> torch.Tensor:
-        ver = param._version
-        hit = self._derived.get(name)
-        if hit is not None and hit[0] == ver and hit[1].device == param.device:
-            return hit[1]
-        with torch.no_grad():
-            t = make(hit[1] if hit is not None and hit[1].device == param.device else None)
-        self._derived[name] = (ver, t)
-        return t
-
-    def set_derived(self, name: str, param: torch.Tensor, tensor: torch.Tensor) -> None:
-        """Called by the fused optimiser after it wrote a fresh shadow / norm itself."""
-        self._derived[name] = (param._version, tensor)
-
-    def get_derived_buffer(self, name: str) -> Optional[torch.Tensor]:
-        hit = self._derived.get(name)
-        return None if hit is None else hit[1]
 
     def w_enc_t(self) -> torch.Tensor:
         """Contiguous [F, d] view of the encoder weight."""

@@ -78,6 +78,27 @@ class SparseDictionary(nn.Module):
         self.dataset_average_activation_norm: dict[str, float] | None = None
         self.device_mesh = None
         self.activation_function = self.activation_function_factory(None)
+        # derived operands (bf16 shadows, row norms) keyed by name -> (param version, tensor)
+        self._derived: dict[str, tuple[int, torch.Tensor]] = {}
+
+    # ---- derived operands, refreshed when the parameter's version counter moves ----
+    def _derive(self, name: str, param: torch.Tensor, make) -> torch.Tensor:
+        ver = param._version
+        hit = self._derived.get(name)
+        if hit is not None and hit[0] == ver and hit[1].device == param.device:
+            return hit[1]
+        with torch.no_grad():
+            t = make(hit[1] if hit is not None and hit[1].device == param.device else None)
+        self._derived[name] = (ver, t)
+        return t
+
+    def set_derived(self, name: str, param: torch.Tensor, tensor: torch.Tensor) -> None:
+        """Called by the fused optimiser after it wrote a fresh shadow / norm itself."""
+        self._derived[name] = (param._version, tensor)
+
+    def get_derived_buffer(self, name: str) -> Optional[torch.Tensor]:
+        hit = self._derived.get(name)
+        return None if hit is None else hit[1]
 
     # ---- small state setters (sparse_dictionary.py:248-260) ----
     @torch.no_grad()

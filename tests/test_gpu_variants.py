@@ -1,0 +1,285 @@
+"""Parity of the kernel-backed crosscoder / CLT / Lorsa train steps against their CPU oracles.
+
+fp32 runs are compared at 1e-5 relative (gradients 1e-4: they are sums of many fp32 terms
+accumulated in a different order than the CPU's GEMMs).  bf16 autocast runs are compared at the
+2e-2 relative bound on the loss and reconstruction only: the oracle on CPU rounds its GEMMs
+differently in bf16, so an entry close to the k-th value can legitimately fall on the other side.
+"""
+
+import importlib
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+GRAD_TOL = 1e-4
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def vo(oracle):
+    return importlib.import_module("oracle.variants_oracle")
+
+
+def rel_err(got, want):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def frob_err(got, want):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).norm() / want.norm()).item()
+
+
+def copy_params(dst, src):
+    s = {k.replace("ln_q_w", "ln_q.w").replace("ln_k_w", "ln_k.w"): v for k, v in src.named_parameters()}
+    with torch.no_grad():
+        for k, p in dst.named_parameters():
+            p.copy_(s[k].to(p.device, p.dtype))
+
+
+def check_grads(model, ref, tol=GRAD_TOL):
+    rp = {k.replace("ln_q_w", "ln_q.w").replace("ln_k_w", "ln_k.w"): v for k, v in ref.named_parameters()}
+    scale = max(v.grad.abs().max().item() for v in rp.values())
+    for n, p in model.named_parameters():
+        assert p.grad is not None, n
+        assert tuple(p.grad.shape) == tuple(p.shape), n
+        if rp[n].grad.abs().max().item() < 1e-5 * scale:
+            # analytically zero (a key bias shifts every score of a softmax row alike): both sides hold rounding noise
+            assert p.grad.abs().max().item() < 1e-4 * scale, n
+            continue
+        assert rel_err(p.grad, rp[n].grad) < tol, (n, rel_err(p.grad, rp[n].grad))
+
+
+# ---- crosscoder ----------------------------------------------------------------------------------
+
+def make_crosscoder(pkg, vo, dev, H, d, F, k, seed):
+    ref = vo.init_uniform_(vo.CrosscoderOracle(H, d, F, act_fn="topk", top_k=k), seed=seed, bound=0.3)
+    with torch.no_grad():   # spread the decoder norms so that the heads select differently
+        g = torch.Generator().manual_seed(seed + 7)
+        ref.W_D.mul_(0.25 + 1.5 * torch.rand(H, F, 1, generator=g))
+    hooks = [f"h{i}" for i in range(H)]
+    cfg = pkg.CrosscoderConfig(hook_points=hooks, d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                               norm_activation="inference", device="cuda", dtype=torch.float32)
+    m = pkg.Crosscoder(cfg)
+    copy_params(m, ref)
+    return m, ref, hooks
+
+
+@pytest.mark.parametrize("H,d,F,k,B", [(2, 64, 512, 8, 96), (3, 32, 384, 5, 130), (4, 64, 1024, 16, 64)])
+def test_crosscoder_fused_step_fp32(pkg, vo, dev, H, d, F, k, B):
+    m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=31)
+    g = torch.Generator().manual_seed(32)
+    batch = {h: torch.randn(B, d, generator=g) for h in hooks}
+    batch["tokens"] = torch.zeros(B, dtype=torch.long)
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    out = m.compute_loss(gb)
+    assert "sparse_codes" in out, "the kernel path did not run"
+    want = ref.compute_loss(batch, hooks)
+    assert torch.equal((out["feature_acts"] > 0).cpu(), want["feature_acts"] > 0)           # same selection, every head
+    assert not torch.equal(want["feature_acts"][:, 0] > 0, want["feature_acts"][:, 1] > 0)   # and the heads do differ
+    assert rel_err(out["feature_acts"], want["feature_acts"]) < FP32_TOL
+    assert rel_err(out["hidden_pre"], want["hidden_pre"]) < FP32_TOL
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
+    assert rel_err(out["loss"], want["loss"]) < FP32_TOL
+    out["loss"].backward(); want["loss"].backward()
+    check_grads(m, ref)
+
+
+def test_crosscoder_mask_and_adam_step(pkg, vo, dev):
+    H, d, F, k, B = 2, 64, 512, 8, 80
+    m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=33)
+    g = torch.Generator().manual_seed(34)
+    batch = {h: torch.randn(B, d, generator=g) for h in hooks}
+    batch["tokens"] = torch.zeros(B, dtype=torch.long)
+    mask = (torch.rand(B, H, generator=g) > 0.3).float()
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    gb["mask"] = mask.to(dev)
+    opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
+    ropt = torch.optim.Adam(ref.parameters(), lr=1e-3)
+    before = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    loss = m.compute_loss(gb, return_aux_data=False)
+    want = ref.compute_loss(batch, hooks, mask=mask)["loss"]
+    assert rel_err(loss, want) < FP32_TOL
+    loss.backward(); want.backward()
+    check_grads(m, ref)
+    opt.step(); ropt.step()
+    rp = dict(ref.named_parameters())
+    for n, p in m.named_parameters():   # the move itself, relative to its own size
+        move, want_move = p.detach().cpu() - before[n], rp[n].detach() - before[n]
+        assert rel_err(move, want_move) < 1e-3, n
+    assert m.W_E.permute(2, 0, 1).is_contiguous()      # the update kept the feature-major layout
+
+
+def test_crosscoder_fused_step_bf16(pkg, vo, dev):
+    H, d, F, k, B = 2, 64, 1024, 16, 128
+    m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=35)
+    g = torch.Generator().manual_seed(36)
+    batch = {h: torch.randn(B, d, generator=g) for h in hooks}
+    batch["tokens"] = torch.zeros(B, dtype=torch.long)
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = m.compute_loss(gb)
+    want = ref.compute_loss(batch, hooks)
+    assert rel_err(out["loss"], want["loss"]) < BF16_TOL
+    # bf16 rounding of the GEMM legitimately flips near-ties against the fp32 oracle, so the step is checked
+    # stage by stage: the pre-activation within the bf16 bound, the selection exact on the kernel's OWN
+    # pre-activation, and the decode within the bf16 bound of the oracle's decode of the kernel's code
+    hp, acts = out["hidden_pre"].cpu(), out["feature_acts"].cpu()
+    assert rel_err(hp, want["hidden_pre"]) < BF16_TOL
+    with torch.no_grad():
+        n = ref.decoder_norm()
+        own = ref.activation_function(hp * n) / n
+        assert torch.equal(own > 0, acts > 0)
+        assert rel_err(acts, own) < FP32_TOL
+        assert rel_err(out["reconstructed"], ref.decode(acts)) < BF16_TOL
+    out["loss"].backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+
+
+# ---- CLT -----------------------------------------------------------------------------------------
+
+def make_clt(pkg, vo, dev, act_fn, L, d, F, k, seed, include_norm=True):
+    ref = vo.init_uniform_(vo.CLTOracle(L, d, F, act_fn=act_fn, top_k=k, sparsity_include_decoder_norm=include_norm),
+                           seed=seed, bound=0.3)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(seed + 7)
+        for w in ref.W_D:
+            w.mul_(0.25 + 1.5 * torch.rand(w.shape[0], F, 1, generator=g))
+    hin, hout = [f"i{l}" for l in range(L)], [f"o{l}" for l in range(L)]
+    cfg = pkg.CLTConfig(hook_points_in=hin, hook_points_out=hout, d_model=d, expansion_factor=F / d, act_fn=act_fn, top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=include_norm, device="cuda",
+                        dtype=torch.float32)
+    m = pkg.CrossLayerTranscoder(cfg)
+    copy_params(m, ref)
+    return m, ref, hin, hout
+
+
+def clt_batch(L, B, d, seed):
+    g = torch.Generator().manual_seed(seed)
+    batch = {f"i{l}": torch.randn(B, d, generator=g) for l in range(L)}
+    batch.update({f"o{l}": torch.randn(B, d, generator=g) for l in range(L)})
+    batch["tokens"] = torch.zeros(B, dtype=torch.long)
+    return batch
+
+
+@pytest.mark.parametrize("act_fn", ["topk", "layertopk", "batchtopk", "batchlayertopk"])
+@pytest.mark.parametrize("L,d,F,k,B,include_norm", [(3, 64, 256, 4, 64, True), (4, 32, 192, 6, 50, False)])
+def test_clt_fused_step_fp32(pkg, vo, dev, act_fn, L, d, F, k, B, include_norm):
+    m, ref, hin, hout = make_clt(pkg, vo, dev, act_fn, L, d, F, k, seed=41, include_norm=include_norm)
+    batch = clt_batch(L, B, d, seed=42)
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    out = m.compute_loss(gb)
+    assert "sparse_code" in out, "the kernel path did not run"
+    want = ref.compute_loss(batch, hin, hout)
+    code = out["sparse_code"]
+    # every token's entries ascend in (layer, feature): the prefix decode relies on it
+    idx, off, nnz = code.idx.cpu(), code.row_off.cpu(), code.row_nnz.cpu()
+    for b in range(B):
+        row = idx[off[b]: off[b] + nnz[b]]
+        assert torch.all(row[1:] > row[:-1])
+    assert torch.equal((out["feature_acts"] > 0).cpu(), want["feature_acts"] > 0)
+    assert rel_err(out["feature_acts"], want["feature_acts"]) < FP32_TOL
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
+    assert rel_err(out["loss"], want["loss"]) < FP32_TOL
+    out["loss"].backward(); want["loss"].backward()
+    check_grads(m, ref)
+
+
+def test_clt_fused_matches_own_dense_path_and_adam(pkg, vo, dev):
+    """The sparse prefix decode against the module's own dense API path (same weights, same device), then
+    one optimiser step over the ParameterList against torch.optim.Adam on the oracle."""
+    L, d, F, k, B = 3, 64, 256, 4, 48
+    m, ref, hin, hout = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=43)
+    batch = clt_batch(L, B, d, seed=44)
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    x, _, _ = m.prepare_input(gb)
+    dense = m.decode(m.encode(x))
+    out = m.compute_loss(gb)
+    assert rel_err(out["reconstructed"], dense) < FP32_TOL
+    opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
+    ropt = torch.optim.Adam(ref.parameters(), lr=1e-3)
+    before = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    out["loss"].backward()
+    ref.compute_loss(batch, hin, hout)["loss"].backward()
+    opt.step(); ropt.step()
+    rp = dict(ref.named_parameters())
+    for n, p in m.named_parameters():
+        assert rel_err(p.detach().cpu() - before[n], rp[n].detach() - before[n]) < 1e-3, n
+    # second step: the cached norms and operands must follow the update
+    opt.zero_grad(); ropt.zero_grad()
+    out2 = m.compute_loss(gb)
+    want2 = ref.compute_loss(batch, hin, hout)
+    assert rel_err(out2["loss"], want2["loss"]) < 1e-4
+
+
+def test_clt_fused_step_bf16(pkg, vo, dev):
+    L, d, F, k, B = 3, 64, 512, 8, 96
+    m, ref, hin, hout = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=45)
+    batch = clt_batch(L, B, d, seed=46)
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = m.compute_loss(gb)
+    want = ref.compute_loss(batch, hin, hout)
+    assert rel_err(out["loss"], want["loss"]) < BF16_TOL
+    agree = ((out["feature_acts"] > 0).cpu() == (want["feature_acts"] > 0)).float().mean().item()
+    assert agree > 0.999
+    out["loss"].backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+
+
+# ---- Lorsa ---------------------------------------------------------------------------------------
+
+def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, **kw):
+    ref = vo.init_uniform_(vo.LorsaOracle(d_model=d, d_sae=F, n_qk_heads=h, d_qk_head=dq, n_ctx=n_ctx, act_fn="topk", top_k=k,
+                                          **kw), seed=seed, bound=0.3)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(seed + 7)
+        ref.W_O.mul_(0.25 + 1.5 * torch.rand(F, 1, generator=g))
+    ckw = dict(kw)
+    ckw.setdefault("rotary_dim", dq)
+    cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
+                          d_qk_head=dq, n_ctx=n_ctx, act_fn="topk", top_k=k, norm_activation="inference", device="cuda",
+                          dtype=torch.float32, **ckw)
+    m = pkg.LowRankSparseAttention(cfg)
+    copy_params(m, ref)
+    return m, ref
+
+
+@pytest.mark.parametrize("kw", [dict(positional_embedding_type="none"),
+                                dict(positional_embedding_type="rotary", rotary_dim=16),
+                                dict(positional_embedding_type="none", sparsity_include_decoder_norm=False)])
+def test_lorsa_fused_step_fp32(pkg, vo, dev, kw):
+    d, F, h, dq, s, b, k = 64, 256, 4, 16, 16, 3, 8
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, 32, k, seed=51, **kw)
+    g = torch.Generator().manual_seed(52)
+    batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+    mask = (torch.rand(b, s, generator=g) > 0.2).float()
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    gb["mask"] = mask.to(dev)
+    out = m.compute_loss(gb)
+    assert "sparse_code" in out, "the kernel path did not run"
+    want = ref.compute_loss(batch, mask=mask)
+    assert rel_err(out["hidden_pre"], want["hidden_pre"]) < FP32_TOL
+    assert torch.equal((out["feature_acts"] > 0).cpu(), want["feature_acts"] > 0)
+    assert rel_err(out["feature_acts"], want["feature_acts"]) < FP32_TOL
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
+    assert rel_err(out["loss"], want["loss"]) < FP32_TOL
+    out["loss"].backward(); want["loss"].backward()
+    check_grads(m, ref)
+
+
+def test_lorsa_fused_step_bf16(pkg, vo, dev):
+    d, F, h, dq, s, b, k = 64, 512, 4, 16, 32, 2, 8
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, 32, k, seed=53, positional_embedding_type="none")
+    g = torch.Generator().manual_seed(54)
+    batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = m.compute_loss(gb)
+    want = ref.compute_loss(batch)
+    assert rel_err(out["loss"], want["loss"]) < BF16_TOL
+    out["loss"].backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
