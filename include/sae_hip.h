@@ -231,6 +231,40 @@ int sae_sparse_adam_step(float *p, const float *g, float *m, float *v, int64_t n
  * compute_grad_norm (optim.py:257-277): ||g|| / sqrt(#non-zero). */
 int sae_grad_sq_nnz(const float *g, int64_t n, double *acc, void *stream);
 
+/* ---- JumpReLU with straight-through threshold gradient --------------------------------------------
+ * Replaces STEFunction / JumpReLU (activation_functions.py:15-140) as the SAE encoder applies it
+ * (models/sae.py:136-160: scale by the decoder norm, activate, unscale) together with the sparsity
+ * terms that read the same [B, F] data: the tanh penalty (models/sparse_dictionary.py:893-894) and the
+ * Lp penalty (models/sparse_dictionary.py:927-938).
+ * With h = pre + b_enc, s = scale[f] (1 when scale is NULL), u = h * s, n = pen_norm[f] (1 when NULL;
+ * the decoder norm the penalties weigh by, whether or not the activation is scaled by it):
+ *   acts[b, f]   = u > theta[f] ? u / s : 0                       (dtype of `pre`)
+ *   tanh_tok[b]  = sum_f tanh(tanh_c * acts * n)                  (optional)
+ *   lp_tok[b]    = sum_f relu(theta - h) * n                      (optional)
+ *   l0_tok[b]    = number of kept features                        (optional)
+ * pre, acts: [B, F] row-major, SAE_F32 or SAE_BF16; F must be a multiple of 8. */
+int sae_jumprelu_fwd(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
+                     const float *theta, int64_t B, int64_t F, double tanh_c, void *acts, float *tanh_tok, float *lp_tok, float *l0_tok,
+                     void *stream);
+
+int64_t sae_jumprelu_bwd_workspace_bytes(int64_t B, int64_t F);
+
+/* Backward of the above.  d_acts [B, F] is the gradient arriving at acts; g_tanh [B] / g_lp [B] are the
+ * gradients arriving at tanh_tok / lp_tok (NULL when that term is unused).  With
+ * ga = d_acts + g_tanh[b] * tanh_c * n * (1 - tanh^2):
+ *   d_pre[b, f]  = (u > theta ? ga : 0) - (theta > h ? g_lp[b] * n : 0)
+ *   d_bias[f]    = sum_b d_pre
+ *   d_theta[f]   = sum_b [ |u - theta| < window / 2 and u > 0 ] * (ga / s) * (-theta / window)  +  sum_b [theta > h] g_lp[b] n
+ *                  (the rectangle-window estimator of activation_functions.py:45-61; the gradient of
+ *                  log theta is d_theta * theta)
+ *   d_pen_norm[f] = sum_b g_tanh[b] tanh_c acts (1 - tanh^2) + sum_b g_lp[b] relu(theta - h)     (optional;
+ *                  the derivative terms of acts with respect to `scale` cancel, so `scale` gets no gradient)
+ * The per-feature sums are reduced in a fixed order (deterministic). */
+int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
+                     const float *theta, const void *d_acts, const float *g_tanh, double tanh_c, const float *g_lp, double window,
+                     int64_t B, int64_t F, void *d_pre, float *d_bias, float *d_theta, float *d_pen_norm,
+                     void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,253 @@
+// JumpReLU activation with its straight-through threshold gradient and the sparsity penalties that read
+// the same [B, F] data, as two streaming passes (forward, backward).  Both are HBM-bound: the forward
+// reads the pre-activation and writes the activation once; the backward reads the pre-activation and
+// the incoming gradient once, writes the pre-activation gradient once, and reduces three per-feature
+// sums (bias, threshold, decoder-norm gradients) through per-row-group partials that a second kernel
+// adds in a fixed order, so results do not depend on scheduling.
+//
+// Per element, with h = pre + b_enc, s = scale (decoder norm, 1 when absent), u = h * s:
+//   keep = u > theta                      activation  a = keep ? h : 0   ( = jumprelu(u) / s )
+// and with n = pen_norm (the decoder norm the penalties weigh by, 1 when absent; it is the same vector as
+// `scale` when the activation includes the decoder norm, but the penalties use it either way):
+//   tanh term   t = tanh(c * a * n)       lp term  relu(theta - h) * n
+// and for the backward, with ga = d_acts + g_tanh[b] * c * n * (1 - t^2):
+//   d_pre    = keep ? ga : 0   - (theta > h ? g_lp[b] * n : 0)
+//   d_theta += (|u - theta| < window/2 and u > 0) ? (ga / s) * (-theta / window) : 0   + (theta > h ? g_lp[b] * n : 0)
+//   d_pen_norm += g_tanh[b] * c * a * (1 - t^2) + g_lp[b] * relu(theta - h)
+//   d_bias  += d_pre
+// (the two derivative terms of a = jumprelu(h s) / s with respect to s cancel exactly).
+#include "common.h"
+
+namespace sae {
+
+constexpr int JR_THREADS = 256;
+constexpr int JR_ROWS = 64;  // rows per block of the backward pass (one partial per row group and feature)
+
+template <bool BF16>
+__device__ __forceinline__ void load8(const void *__restrict__ p, int64_t g, float (&v)[8]) {
+  if constexpr (BF16) {
+    const u32x4 r = reinterpret_cast<const u32x4 *>(p)[g];
+    v[0] = bf16_bits_to_f32((uint16_t)(r.x & 0xffffu)); v[1] = bf16_bits_to_f32((uint16_t)(r.x >> 16));
+    v[2] = bf16_bits_to_f32((uint16_t)(r.y & 0xffffu)); v[3] = bf16_bits_to_f32((uint16_t)(r.y >> 16));
+    v[4] = bf16_bits_to_f32((uint16_t)(r.z & 0xffffu)); v[5] = bf16_bits_to_f32((uint16_t)(r.z >> 16));
+    v[6] = bf16_bits_to_f32((uint16_t)(r.w & 0xffffu)); v[7] = bf16_bits_to_f32((uint16_t)(r.w >> 16));
+  } else {
+    const float4 a = reinterpret_cast<const float4 *>(p)[2 * g], b = reinterpret_cast<const float4 *>(p)[2 * g + 1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ void store8(void *__restrict__ p, int64_t g, const float (&v)[8]) {
+  if constexpr (BF16) {
+    u32x4 o;
+    o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+    o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+    o.z = (uint32_t)f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
+    o.w = (uint32_t)f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+    reinterpret_cast<u32x4 *>(p)[g] = o;
+  } else {
+    reinterpret_cast<float4 *>(p)[2 * g] = make_float4(v[0], v[1], v[2], v[3]);
+    reinterpret_cast<float4 *>(p)[2 * g + 1] = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
+__device__ __forceinline__ void load8_f32_or(const float *__restrict__ p, int64_t g, float fill, float (&v)[8]) {
+  if (p) {
+    load8<false>(p, g, v);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = fill;
+  }
+}
+
+// one block per token row
+template <bool BF16>
+__global__ __launch_bounds__(JR_THREADS) void jumprelu_fwd_kernel(
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
+    const float *__restrict__ pen, const float *__restrict__ theta, int64_t F, float tanh_c, void *__restrict__ acts,
+    float *__restrict__ tanh_tok,
+    float *__restrict__ lp_tok, float *__restrict__ l0_tok) {
+  __shared__ float red[JR_THREADS / 64];
+  const int64_t row = blockIdx.x;
+  const int64_t groups = F >> 3;
+  const int64_t rbase = row * groups;
+  float tsum = 0.f, lpsum = 0.f, cnt = 0.f;
+  for (int64_t g = threadIdx.x; g < groups; g += JR_THREADS) {
+    float p[8], b[8], s[8], np[8], th[8], a[8];
+    load8<BF16>(pre, rbase + g, p);
+    load8_f32_or(b_enc, g, 0.f, b);
+    load8_f32_or(scale, g, 1.f, s);
+    load8_f32_or(pen, g, 1.f, np);
+    load8<false>(theta, g, th);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float h = p[i] + b[i];
+      const float u = h * s[i];
+      const bool keep = u > th[i];
+      a[i] = keep ? (scale ? u / s[i] : h) : 0.f;
+      cnt += keep ? 1.f : 0.f;
+      if (tanh_tok && keep) tsum += tanhf(tanh_c * a[i] * np[i]);
+      if (lp_tok) lpsum += fmaxf(th[i] - h, 0.f) * np[i];
+    }
+    store8<BF16>(acts, rbase + g, a);
+  }
+  if (tanh_tok) {
+    const float t = block_sum<JR_THREADS / 64>(tsum, red);
+    if (threadIdx.x == 0) tanh_tok[row] = t;
+  }
+  if (lp_tok) {
+    const float t = block_sum<JR_THREADS / 64>(lpsum, red);
+    if (threadIdx.x == 0) lp_tok[row] = t;
+  }
+  if (l0_tok) {
+    const float t = block_sum<JR_THREADS / 64>(cnt, red);
+    if (threadIdx.x == 0) l0_tok[row] = t;
+  }
+}
+
+// grid (ceil(F / 2048), ceil(B / JR_ROWS)); a thread owns 8 adjacent features for JR_ROWS rows
+template <bool BF16>
+__global__ __launch_bounds__(JR_THREADS) void jumprelu_bwd_kernel(
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
+    const float *__restrict__ pen, const float *__restrict__ theta, const void *__restrict__ d_acts,
+    const float *__restrict__ g_tanh, float tanh_c,
+    const float *__restrict__ g_lp, float window, int64_t B, int64_t F, void *__restrict__ d_pre,
+    float *__restrict__ part_bias, float *__restrict__ part_theta, float *__restrict__ part_scale) {
+  const int64_t groups = F >> 3;
+  const int64_t g = (int64_t)blockIdx.x * JR_THREADS + threadIdx.x;
+  if (g >= groups) return;
+  float b[8], s[8], np[8], th[8];
+  load8_f32_or(b_enc, g, 0.f, b);
+  load8_f32_or(scale, g, 1.f, s);
+  load8_f32_or(pen, g, 1.f, np);
+  load8<false>(theta, g, th);
+  float acc_b[8], acc_t[8], acc_s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc_b[i] = acc_t[i] = acc_s[i] = 0.f;
+  const float half_w = 0.5f * window;
+  const int64_t r0 = (int64_t)blockIdx.y * JR_ROWS;
+  const int64_t r1 = (r0 + JR_ROWS < B) ? r0 + JR_ROWS : B;
+#pragma unroll 2
+  for (int64_t r = r0; r < r1; ++r) {
+    float p[8], ga[8], dp[8];
+    load8<BF16>(pre, r * groups + g, p);
+    load8<BF16>(d_acts, r * groups + g, ga);
+    const float gt = g_tanh ? g_tanh[r] * tanh_c : 0.f;
+    const float gl = g_lp ? g_lp[r] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float h = p[i] + b[i];
+      const float u = h * s[i];
+      const bool keep = u > th[i];
+      float gtot = ga[i];
+      if (g_tanh) {
+        const float a = keep ? (scale ? u / s[i] : h) : 0.f;
+        const float t = keep ? tanhf(tanh_c * a * np[i]) : 0.f;
+        const float sech2 = 1.f - t * t;
+        gtot += gt * np[i] * sech2;
+        acc_s[i] += gt * a * sech2;
+      }
+      float d = keep ? gtot : 0.f;
+      const bool in_window = (fabsf(u - th[i]) < half_w) && (u > 0.f);
+      if (in_window) acc_t[i] += (gtot / s[i]) * (-th[i] / window);
+      if (g_lp && th[i] > h) {
+        d -= gl * np[i];
+        acc_t[i] += gl * np[i];
+        acc_s[i] += gl * (th[i] - h);
+      }
+      dp[i] = d;
+      acc_b[i] += d;
+    }
+    store8<BF16>(d_pre, r * groups + g, dp);
+  }
+  const int64_t off = (int64_t)blockIdx.y * groups + g;
+  store8<false>(part_bias, off, acc_b);
+  store8<false>(part_theta, off, acc_t);
+  if (part_scale) store8<false>(part_scale, off, acc_s);
+}
+
+// out[f] = sum over row groups of part[group][f], in group order
+__global__ __launch_bounds__(256) void jumprelu_reduce_kernel(const float *__restrict__ part, int n_groups, int64_t F,
+                                                              float *__restrict__ out) {
+  const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (f >= F) return;
+  float s = 0.f;
+  for (int j = 0; j < n_groups; ++j) s += part[(int64_t)j * F + f];
+  out[f] = s;
+}
+
+static int check_shape(const char *who, const void *pre, int dtype, const float *theta, const float *b_enc,
+                       const float *scale, int64_t B, int64_t F) {
+  SAE_REQUIRE(pre && theta, SAE_ERR_INVALID_ARG, "%s: null pointer", who);
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F < (1LL << 31), SAE_ERR_INVALID_ARG, "%s: bad shape", who);
+  SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "%s: bad dtype %d", who, dtype);
+  SAE_REQUIRE(F % 8 == 0, SAE_ERR_UNSUPPORTED, "%s: d_sae=%lld must be a multiple of 8", who, (long long)F);
+  SAE_REQUIRE(((((uintptr_t)pre) | ((uintptr_t)theta) | ((uintptr_t)b_enc) | ((uintptr_t)scale)) & 15) == 0,
+              SAE_ERR_INVALID_ARG, "%s: pre, theta, b_enc and scale must be 16-byte aligned", who);
+  return SAE_OK;
+}
+
+}  // namespace sae
+
+using namespace sae;
+
+extern "C" int sae_jumprelu_fwd(const void *pre, int dtype, const float *b_enc, const float *scale,
+                                const float *pen_norm, const float *theta, int64_t B, int64_t F, double tanh_c_d, void *acts, float *tanh_tok, float *lp_tok,
+                                float *l0_tok, void *stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float tanh_c = (float)tanh_c_d;
+  int rc = check_shape("jumprelu_fwd", pre, dtype, theta, b_enc, scale, B, F);
+  if (rc) return rc;
+  SAE_REQUIRE(acts && (((uintptr_t)acts) & 15) == 0, SAE_ERR_INVALID_ARG, "jumprelu_fwd: acts must be a 16-byte aligned buffer");
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(jumprelu_fwd_kernel<true>, dim3((unsigned)B), dim3(JR_THREADS), 0, st, pre, b_enc, scale, pen_norm, theta, F,
+                       tanh_c, acts, tanh_tok, lp_tok, l0_tok);
+  else
+    hipLaunchKernelGGL(jumprelu_fwd_kernel<false>, dim3((unsigned)B), dim3(JR_THREADS), 0, st, pre, b_enc, scale, pen_norm, theta, F,
+                       tanh_c, acts, tanh_tok, lp_tok, l0_tok);
+  return check_launch("jumprelu_fwd");
+}
+
+extern "C" int64_t sae_jumprelu_bwd_workspace_bytes(int64_t B, int64_t F) {
+  const int64_t n_groups = (B + JR_ROWS - 1) / JR_ROWS;
+  return 3 * n_groups * F * (int64_t)sizeof(float);
+}
+
+extern "C" int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float *scale,
+                                const float *pen_norm, const float *theta, const void *d_acts, const float *g_tanh, double tanh_c_d, const float *g_lp,
+                                double window_d, int64_t B, int64_t F, void *d_pre, float *d_bias, float *d_theta,
+                                float *d_pen_norm, void *workspace, int64_t workspace_bytes, void *stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float tanh_c = (float)tanh_c_d, window = (float)window_d;
+  int rc = check_shape("jumprelu_bwd", pre, dtype, theta, b_enc, scale, B, F);
+  if (rc) return rc;
+  SAE_REQUIRE(d_acts && d_pre && d_bias && d_theta, SAE_ERR_INVALID_ARG, "jumprelu_bwd: null pointer");
+  SAE_REQUIRE(((((uintptr_t)d_acts) | ((uintptr_t)d_pre)) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "jumprelu_bwd: d_acts and d_pre must be 16-byte aligned");
+  SAE_REQUIRE(window > 0.f, SAE_ERR_INVALID_ARG, "jumprelu_bwd: window must be positive");
+  SAE_REQUIRE(!d_pen_norm || pen_norm, SAE_ERR_INVALID_ARG, "jumprelu_bwd: d_pen_norm needs pen_norm");
+  SAE_REQUIRE((((uintptr_t)pen_norm) & 15) == 0, SAE_ERR_INVALID_ARG, "jumprelu_bwd: pen_norm must be 16-byte aligned");
+  SAE_REQUIRE(workspace && workspace_bytes >= sae_jumprelu_bwd_workspace_bytes(B, F) && (((uintptr_t)workspace) & 15) == 0,
+              SAE_ERR_WORKSPACE, "jumprelu_bwd: workspace too small or misaligned");
+  const int64_t n_groups = (B + JR_ROWS - 1) / JR_ROWS;
+  float *part_bias = reinterpret_cast<float *>(workspace);
+  float *part_theta = part_bias + n_groups * F;
+  float *part_scale = d_pen_norm ? part_theta + n_groups * F : nullptr;
+  const int64_t groups = F >> 3;
+  const dim3 grid((unsigned)((groups + JR_THREADS - 1) / JR_THREADS), (unsigned)n_groups);
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(jumprelu_bwd_kernel<true>, grid, dim3(JR_THREADS), 0, st, pre, b_enc, scale, pen_norm, theta, d_acts, g_tanh,
+                       tanh_c, g_lp, window, B, F, d_pre, part_bias, part_theta, part_scale);
+  else
+    hipLaunchKernelGGL(jumprelu_bwd_kernel<false>, grid, dim3(JR_THREADS), 0, st, pre, b_enc, scale, pen_norm, theta, d_acts, g_tanh,
+                       tanh_c, g_lp, window, B, F, d_pre, part_bias, part_theta, part_scale);
+  rc = check_launch("jumprelu_bwd");
+  if (rc) return rc;
+  const unsigned rb = (unsigned)((F + 255) / 256);
+  hipLaunchKernelGGL(jumprelu_reduce_kernel, dim3(rb), dim3(256), 0, st, part_bias, (int)n_groups, F, d_bias);
+  hipLaunchKernelGGL(jumprelu_reduce_kernel, dim3(rb), dim3(256), 0, st, part_theta, (int)n_groups, F, d_theta);
+  if (d_pen_norm)
+    hipLaunchKernelGGL(jumprelu_reduce_kernel, dim3(rb), dim3(256), 0, st, part_scale, (int)n_groups, F, d_pen_norm);
+  return check_launch("jumprelu_bwd(reduce)");
+}

@@ -465,3 +465,57 @@ def grad_sq_nnz(grads) -> torch.Tensor:
         with _timed("grad_sq_nnz"):
             check(lib.sae_grad_sq_nnz(g.data_ptr(), g.numel(), acc.data_ptr(), _stream(g)), "grad_sq_nnz")
     return acc
+
+
+# ---- JumpReLU ---------------------------------------------------------------------------------
+
+def jumprelu_fwd(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], theta: torch.Tensor,
+                 tanh_c: float = 0.0, pen_norm: Optional[torch.Tensor] = None, want_tanh: bool = False, want_lp: bool = False, want_l0: bool = False):
+    """acts [B, F] (dtype of pre) and the requested per-token sums (tanh penalty, Lp penalty, L0), each [B] or None."""
+    _req(pre, "pre", ndim=2)
+    B, F = pre.shape
+    for name, v in (("b_enc", b_enc), ("scale", scale), ("theta", theta), ("pen_norm", pen_norm)):
+        if v is not None:
+            _req(v, name, torch.float32, 1)
+            if v.numel() != F:
+                raise ValueError(f"{name} must have {F} elements")
+    dev = pre.device
+    acts = torch.empty_like(pre)
+    mk = lambda want: torch.empty(B, dtype=torch.float32, device=dev) if want else None  # noqa: E731
+    tanh_tok, lp_tok, l0_tok = mk(want_tanh), mk(want_lp), mk(want_l0)
+    with _timed("jumprelu_fwd"):
+        check(_lib.load().sae_jumprelu_fwd(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(pen_norm), theta.data_ptr(), B, F,
+                                           float(tanh_c), acts.data_ptr(), _ptr(tanh_tok), _ptr(lp_tok), _ptr(l0_tok),
+                                           _stream(pre)), "jumprelu_fwd")
+    return acts, tanh_tok, lp_tok, l0_tok
+
+
+def jumprelu_bwd(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], theta: torch.Tensor,
+                 d_acts: torch.Tensor, g_tanh: Optional[torch.Tensor], tanh_c: float, g_lp: Optional[torch.Tensor],
+                 window: float, pen_norm: Optional[torch.Tensor] = None, want_norm_grad: bool = False):
+    """(d_pre [B, F], d_bias [F], d_theta [F], d_pen_norm [F] or None)"""
+    _req(pre, "pre", ndim=2)
+    _req(d_acts, "d_acts", pre.dtype, 2)
+    if d_acts.shape != pre.shape:
+        raise ValueError("d_acts must have the shape of pre")
+    B, F = pre.shape
+    for name, v in (("g_tanh", g_tanh), ("g_lp", g_lp)):
+        if v is not None:
+            _req(v, name, torch.float32, 1)
+            if v.numel() != B:
+                raise ValueError(f"{name} must have {B} elements")
+    dev = pre.device
+    lib = _lib.load()
+    d_pre = torch.empty_like(pre)
+    d_bias = torch.empty(F, dtype=torch.float32, device=dev)
+    d_theta = torch.empty(F, dtype=torch.float32, device=dev)
+    d_scale = torch.empty(F, dtype=torch.float32, device=dev) if want_norm_grad else None
+    ws_bytes = lib.sae_jumprelu_bwd_workspace_bytes(B, F)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with _timed("jumprelu_bwd"):
+        check(lib.sae_jumprelu_bwd(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(pen_norm), theta.data_ptr(),
+                                   d_acts.data_ptr(),
+                                   _ptr(g_tanh), float(tanh_c), _ptr(g_lp), float(window), B, F, d_pre.data_ptr(),
+                                   d_bias.data_ptr(), d_theta.data_ptr(), _ptr(d_scale), ws.data_ptr(), ws_bytes,
+                                   _stream(pre)), "jumprelu_bwd")
+    return d_pre, d_bias, d_theta, d_scale

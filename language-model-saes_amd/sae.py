@@ -185,6 +185,61 @@ class _FusedSparseStep(torch.autograd.Function):
         return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
+class _EncoderGemm(torch.autograd.Function):
+    """pre = x @ W_E through the GEMM kernel, for activations whose output is dense (JumpReLU): the incoming
+    gradient is then dense as well and both backward products are plain library GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, W_E, w_op, amp):
+        if amp:
+            x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())
+            pre = ops.encoder_gemm(x_op, w_op, torch.bfloat16)
+        else:
+            x_op = x.float().contiguous()
+            pre = ops.encoder_gemm(x_op, w_op, torch.float32)
+        ctx.save_for_backward(x_op, w_op)
+        ctx.x_dtype = x.dtype
+        return pre
+
+    @staticmethod
+    def backward(ctx, g):
+        x_op, w_op = ctx.saved_tensors
+        gg = g.to(w_op.dtype)
+        dx = (gg @ w_op).to(ctx.x_dtype) if ctx.needs_input_grad[0] else None
+        dW = (gg.t() @ x_op).t().float() if ctx.needs_input_grad[1] else None     # [d, F] with feature-major strides
+        return dx, dW, None, None
+
+
+class _JumpReLUStep(torch.autograd.Function):
+    """bias + decoder-norm scale + JumpReLU + the tanh / Lp penalty sums in one pass over [B, F]; the backward
+    is one more pass that also yields the bias, threshold and decoder-norm gradients.  `norm` is the decoder
+    norm; `scaled` says whether the activation is applied to h * norm (the penalties weigh by it either way)."""
+
+    @staticmethod
+    def forward(ctx, pre, b_E, norm, theta, scaled, tanh_c, window, want_tanh, want_lp):
+        b = b_E.detach().float().contiguous()
+        n = None if norm is None else norm.detach().float().contiguous()
+        th = theta.detach().float().contiguous()
+        acts, tanh_tok, lp_tok, _ = ops.jumprelu_fwd(pre.contiguous(), b, n if scaled else None, th, tanh_c, pen_norm=n,
+                                                     want_tanh=want_tanh, want_lp=want_lp)
+        ctx.save_for_backward(pre, b, th, *(() if n is None else (n,)))
+        ctx.has_norm, ctx.scaled, ctx.tanh_c, ctx.window = n is not None, scaled, tanh_c, window
+        ctx.b_dtype, ctx.th_dtype = b_E.dtype, theta.dtype
+        return acts, tanh_tok, lp_tok
+
+    @staticmethod
+    def backward(ctx, g_acts, g_tanh, g_lp):
+        pre, b, th, *rest = ctx.saved_tensors
+        n = rest[0] if ctx.has_norm else None
+        if g_acts is None:
+            g_acts = torch.zeros_like(pre)
+        fix = lambda g: None if g is None else g.float().contiguous()   # noqa: E731
+        d_pre, d_bias, d_theta, d_norm = ops.jumprelu_bwd(
+            pre.contiguous(), b, n if ctx.scaled else None, th, g_acts.to(pre.dtype).contiguous(), fix(g_tanh), ctx.tanh_c,
+            fix(g_lp), ctx.window, pen_norm=n, want_norm_grad=ctx.has_norm and ctx.needs_input_grad[2])
+        return d_pre, d_bias.to(ctx.b_dtype), d_norm, d_theta.to(ctx.th_dtype), None, None, None, None, None
+
+
 @register_sae_model("sae")
 class SparseAutoEncoder(SparseDictionary):
     def __init__(self, cfg: SAEConfig, device_mesh=None):
@@ -359,12 +414,62 @@ class SparseAutoEncoder(SparseDictionary):
             and self.W_E.dtype == torch.float32
         )
 
+    # ---- JumpReLU train-step loss: dense activations, so encoder kernel + one fused element-wise pass each way,
+    # with the dense decoder products left to the library GEMM ----
+    def _jumprelu_eligible(self, x, label, sparsity_loss_type, auxk_coefficient) -> bool:
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        return (
+            self.cfg.act_fn.lower() == "jumprelu" and x.is_cuda and x.ndim == 2 and label.ndim == 2
+            and not self.cfg.use_glu_encoder and sparsity_loss_type in (None, "tanh") and not (auxk_coefficient > 0.0)
+            and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
+            and self.W_E.dtype == torch.float32 and self.cfg.d_sae % 8 == 0 and self.cfg.d_model % (64 if amp else 32) == 0
+        )
+
+    def _jumprelu_loss(self, batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient, lp_coefficient,
+                       auxk_coefficient, return_aux_data):
+        from .sparse_dictionary import apply_token_mask
+
+        mask = batch.get("mask")
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        jr = self.activation_function
+        pre = _EncoderGemm.apply(x, self.W_E, self._w_enc_operand(amp), amp)
+        want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
+        scaled = bool(self.cfg.sparsity_include_decoder_norm)
+        n = self.decoder_norm() if (scaled or want_tanh or want_lp) else None
+        acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
+                                                     float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
+                                                     want_tanh, want_lp)
+        reconstructed = acts @ self.W_D
+        if self.cfg.use_decoder_bias:
+            reconstructed = reconstructed + self.b_D
+        l_rec = apply_token_mask((reconstructed - label).pow(2).sum(dim=-1), 1, mask, "mean")
+        loss = l_rec
+        l_s = l_p = None
+        if want_tanh:
+            l_s = l1_coefficient * tanh_tok
+            loss = loss + apply_token_mask(l_s, 1, mask, "mean")
+        if want_lp:
+            l_p = apply_token_mask(lp_coefficient * lp_tok, 1, mask, "mean")
+            loss = loss + l_p
+        if not return_aux_data:
+            return loss
+        b_E = self.b_E.detach()
+        eager = {"loss": loss, "l_rec": l_rec, "l_s": l_s, "l_p": l_p, "l_aux": None, "label": label, "mask": mask,
+                 "feature_acts": acts, "reconstructed": reconstructed, "l1_coefficient": l1_coefficient,
+                 "lp_coefficient": lp_coefficient, "auxk_coefficient": auxk_coefficient}
+        lazy = {"n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
+                "hidden_pre": lambda: pre.detach().float() + b_E}
+        return LazyDict(eager, lazy)
+
     def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,
                      frequency_scale: float = 0.01, p: int = 1, l1_coefficient: float = 1.0,
                      lp_coefficient: float = 0.0, auxk_coefficient: float = 0.0, k_aux: int = 512,
                      update_dead_statistics=None, return_aux_data: bool = True, **kwargs):
         x, _, _ = self.prepare_input(batch)
         label = self.prepare_label(batch, **kwargs)
+        if self._jumprelu_eligible(x, label, sparsity_loss_type, auxk_coefficient):
+            return self._jumprelu_loss(batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient,
+                                       lp_coefficient, auxk_coefficient, return_aux_data)
         if not self._fused_eligible(x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient):
             return super().compute_loss(
                 batch, sparsity_loss_type=sparsity_loss_type, tanh_stretch_coefficient=tanh_stretch_coefficient,

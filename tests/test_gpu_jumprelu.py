@@ -1,0 +1,215 @@
+"""JumpReLU kernels (forward, straight-through backward, tanh / Lp penalty sums) and the JumpReLU train
+step of the SAE module against the oracle.
+
+Kernel level: the oracle's STEFunction / JumpReLU under autograd on CPU, composed exactly as the
+reference's encoder and loss compose them (scale by the decoder norm, activate, unscale; tanh and Lp
+penalties), is differentiated with respect to the pre-activation, bias, threshold and norm.
+Step level: SAEOracle with act_fn="jumprelu" against the module's compute_loss.
+"""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+GRAD_TOL = 1e-4
+BF16_TOL = 2e-2
+
+
+def rel_err(got, want):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def oracle_terms(oracle, pre, b, n, log_theta, window, c, pen=None):
+    """acts, tanh_tok, lp_tok as the reference composes them (models/sae.py:136-160,
+    models/sparse_dictionary.py:893-894, 927-938)."""
+    jr = oracle.JumpReLU(window, (pre.shape[1],))
+    jr.log_jumprelu_threshold = log_theta
+    h = pre + b
+    u = h * n if n is not None else h
+    acts = jr(u)
+    if n is not None:
+        acts = acts / n
+        hidden_pre = u / n
+    else:
+        hidden_pre = u
+    one = pen if pen is not None else torch.ones_like(b)
+    tanh_tok = torch.tanh(c * acts * one).sum(-1)
+    lp_tok = (torch.nn.functional.relu(jr.get_jumprelu_threshold() - hidden_pre) * one).sum(-1)
+    return acts, tanh_tok, lp_tok
+
+
+@pytest.mark.parametrize("B,F", [(70, 512), (129, 1024), (64, 2056)])
+@pytest.mark.parametrize("with_scale", [True, False])
+def test_jumprelu_kernels_fp32(pkg, oracle, dev, B, F, with_scale):
+    ops = pkg.ops
+    g = torch.Generator().manual_seed(B + F)
+    pre = torch.randn(B, F, generator=g).requires_grad_()
+    b = (0.1 * torch.randn(F, generator=g)).requires_grad_()
+    pen = (0.5 + torch.rand(F, generator=g)).requires_grad_()       # the decoder norm: always weighs the penalties,
+    n = pen if with_scale else None                                  # scales the activation only when configured
+    log_theta = torch.nn.Parameter(torch.log(0.05 + 0.5 * torch.rand(F, generator=g)))
+    window, c = 0.4, 1.7
+    acts, tanh_tok, lp_tok = oracle_terms(oracle, pre, b, n, log_theta, window, c, pen=pen)
+    d_acts = torch.randn(B, F, generator=g)
+    g_tanh, g_lp = torch.rand(B, generator=g), torch.rand(B, generator=g)
+    ((acts * d_acts).sum() + (tanh_tok * g_tanh).sum() + (lp_tok * g_lp).sum()).backward()
+
+    to = lambda t: None if t is None else t.detach().to(dev).contiguous()  # noqa: E731
+    theta = log_theta.detach().exp()
+    a, tt, lt, l0 = ops.jumprelu_fwd(to(pre), to(b), to(n), to(theta), c, pen_norm=to(pen), want_tanh=True, want_lp=True,
+                                     want_l0=True)
+    assert torch.equal((a > 0).cpu(), acts.detach() > 0) or torch.equal((a != 0).cpu(), acts.detach() != 0)
+    assert rel_err(a, acts) < FP32_TOL
+    assert rel_err(tt, tanh_tok) < FP32_TOL and rel_err(lt, lp_tok) < FP32_TOL
+    assert torch.equal(l0.cpu(), (acts.detach() != 0).sum(-1).float())
+    d_pre, d_bias, d_theta, d_norm = ops.jumprelu_bwd(to(pre), to(b), to(n), to(theta), to(d_acts), to(g_tanh), c, to(g_lp),
+                                                      window, pen_norm=to(pen), want_norm_grad=True)
+    assert rel_err(d_pre, pre.grad) < FP32_TOL
+    assert rel_err(d_bias, b.grad) < GRAD_TOL
+    assert rel_err(d_theta * theta.to(dev), log_theta.grad) < GRAD_TOL      # chain rule through exp()
+    assert (log_theta.grad != 0).float().mean() > 0.5                         # the window did catch entries
+    assert rel_err(d_norm, pen.grad) < GRAD_TOL      # penalty terms only: the activation's two norm terms cancel
+    # without the penalty terms: plain STE
+    pre.grad = b.grad = log_theta.grad = None
+    acts2, _, _ = oracle_terms(oracle, pre, b, pen.detach() if with_scale else None, log_theta, window, c)
+    (acts2 * d_acts).sum().backward()
+    d_pre2, d_bias2, d_theta2, _ = ops.jumprelu_bwd(to(pre), to(b), to(n), to(theta), to(d_acts), None, 0.0, None, window)
+    assert rel_err(d_pre2, pre.grad) < FP32_TOL
+    assert rel_err(d_theta2 * theta.to(dev), log_theta.grad) < GRAD_TOL
+
+
+def test_jumprelu_special_cases(pkg, dev):
+    """Closed forms of the estimator: no entry inside the window -> zero threshold gradient; non-positive
+    inputs never contribute to it; kept entries pass the gradient unchanged, dropped entries block it."""
+    ops = pkg.ops
+    F = 16
+    theta = torch.full((F,), 0.5, device=dev)
+    pre = torch.tensor([[2.0] * 8 + [-3.0] * 8, [0.55] * 8 + [0.45] * 8], device=dev)      # row 0 far away, row 1 inside
+    d_acts = torch.ones(2, F, device=dev)
+    a, _, _, _ = ops.jumprelu_fwd(pre, None, None, theta)
+    assert torch.equal(a, torch.where(pre > 0.5, pre, torch.zeros_like(pre)))
+    d_pre, d_bias, d_theta, _ = ops.jumprelu_bwd(pre[:1].contiguous(), None, None, theta, d_acts[:1].contiguous(), None, 0.0,
+                                                 None, 0.2)
+    assert torch.all(d_theta == 0) and torch.equal(d_pre, (pre[:1] > 0.5).float())
+    d_pre, d_bias, d_theta, _ = ops.jumprelu_bwd(pre, None, None, theta, d_acts, None, 0.0, None, 0.2)
+    assert torch.allclose(d_theta, torch.full((F,), -0.5 / 0.2, device=dev))               # one in-window row: -theta / eps
+    assert torch.equal(d_bias, torch.tensor([2.0] * 8 + [0.0] * 8, device=dev))
+    neg = torch.full((1, F), -0.01, device=dev)      # within the window of a tiny threshold but not positive
+    _, _, d_theta, _ = ops.jumprelu_bwd(neg, None, None, torch.full((F,), 0.001, device=dev), d_acts[:1].contiguous(), None,
+                                        0.0, None, 0.1)
+    assert torch.all(d_theta == 0)
+    with pytest.raises(RuntimeError):
+        ops.jumprelu_fwd(torch.zeros(2, 12, device=dev), None, None, torch.zeros(12, device=dev))   # F not a multiple of 8
+
+
+def test_jumprelu_kernels_bf16(pkg, oracle, dev):
+    ops = pkg.ops
+    B, F = 96, 1024
+    g = torch.Generator().manual_seed(7)
+    pre = torch.randn(B, F, generator=g).bfloat16()
+    b = 0.1 * torch.randn(F, generator=g)
+    n = 0.5 + torch.rand(F, generator=g)
+    theta = 0.05 + 0.5 * torch.rand(F, generator=g)
+    d_acts = torch.randn(B, F, generator=g).bfloat16()
+    pre32 = pre.float().requires_grad_()
+    log_theta = torch.nn.Parameter(theta.log())
+    acts, _, _ = oracle_terms(oracle, pre32, b, n, log_theta, 0.4, 1.0, pen=n)
+    (acts * d_acts.float()).sum().backward()
+    a, _, _, _ = ops.jumprelu_fwd(pre.to(dev), b.to(dev), n.to(dev), theta.to(dev))
+    assert a.dtype == torch.bfloat16 and rel_err(a, acts) < BF16_TOL
+    d_pre, d_bias, d_theta, _ = ops.jumprelu_bwd(pre.to(dev), b.to(dev), n.to(dev), theta.to(dev), d_acts.to(dev), None, 0.0,
+                                                 None, 0.4)
+    assert d_pre.dtype == torch.bfloat16 and rel_err(d_pre, pre32.grad) < BF16_TOL
+    assert rel_err(d_theta * theta.to(dev), log_theta.grad) < GRAD_TOL       # sums are fp32 on both sides
+
+
+def make_pair(pkg, oracle, dev, d, F, B, seed, include_norm, window):
+    from lm_saes_amd import synthetic
+
+    x = synthetic.activations(B, d, 8, seed)
+    w = synthetic.sae_weights(d, F, x, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    W_D = (w[2] * (0.5 + torch.rand(F, 1, generator=g))).contiguous()
+    b_E = 0.02 * torch.randn(F, generator=g)
+    w = (w[0], b_E, W_D, w[3])
+    log_theta = torch.log(0.02 + 0.3 * torch.rand(F, generator=g))
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=window, norm_activation="inference",
+                        sparsity_include_decoder_norm=include_norm, device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    synthetic.load_weights(sae, *[t.to(dev) for t in w])
+    ref = oracle.SAEOracle(d, F, act_fn="jumprelu", jumprelu_threshold_window=window,
+                           sparsity_include_decoder_norm=include_norm)
+    synthetic.load_weights(ref, *w)
+    with torch.no_grad():
+        sae.activation_function.log_jumprelu_threshold.copy_(log_theta.to(dev))
+        ref.activation_function.log_jumprelu_threshold.copy_(log_theta)
+    y = x + 0.1 * torch.randn(B, d, generator=g)
+    batch = {"in": x, "out": y, "tokens": torch.zeros(B, dtype=torch.long),
+             "mask": (torch.rand(B, generator=g) > 0.25).float()}
+    return sae, ref, batch
+
+
+def named_grads(m):
+    out = {n: p.grad for n, p in m.named_parameters()}
+    return {k.replace("activation_function.", ""): v for k, v in out.items()}
+
+
+@pytest.mark.parametrize("include_norm", [True, False])
+@pytest.mark.parametrize("kw", [dict(), dict(sparsity_loss_type="tanh", l1_coefficient=0.05, tanh_stretch_coefficient=2.0),
+                                dict(sparsity_loss_type="tanh", l1_coefficient=0.05, lp_coefficient=0.01)])
+def test_jumprelu_step_fp32_matches_oracle(pkg, oracle, dev, include_norm, kw):
+    d, F, B = 64, 512, 96
+    sae, ref, batch = make_pair(pkg, oracle, dev, d, F, B, seed=11, include_norm=include_norm, window=0.3)
+    gb = {k: v.to(dev) for k, v in batch.items()}
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
+    out = sae.compute_loss(gb, **kw)
+    out["loss"].backward()
+    torch.cuda.synchronize()
+    pkg.ops.set_kernel_timer(None)
+    ran = set(timer.summary())
+    assert {"encoder_gemm", "jumprelu_fwd", "jumprelu_bwd"} <= ran, ran      # the kernel path, not the generic one
+    want = ref.compute_loss(batch, **kw)
+    want["loss"].backward()
+    assert torch.equal((out["feature_acts"] != 0).cpu(), want["feature_acts"] != 0)
+    for key in ("feature_acts", "hidden_pre", "reconstructed", "loss", "l_rec"):
+        assert rel_err(out[key], want[key]) < FP32_TOL, key
+    for key in ("l_s", "l_p"):
+        assert (out[key] is None) == (want[key] is None)
+        if want[key] is not None:
+            assert rel_err(out[key], want[key]) < FP32_TOL, key
+    got, exp = named_grads(sae), named_grads(ref)
+    for n in exp:
+        assert got[n] is not None, n
+        assert rel_err(got[n], exp[n]) < GRAD_TOL, (n, rel_err(got[n], exp[n]))
+    assert (exp["log_jumprelu_threshold"] != 0).float().mean() > 0.3
+
+
+def test_jumprelu_step_bf16_and_adam(pkg, oracle, dev):
+    d, F, B = 64, 1024, 128
+    sae, ref, batch = make_pair(pkg, oracle, dev, d, F, B, seed=12, include_norm=True, window=0.3)
+    gb = {k: v.to(dev) for k, v in batch.items()}
+    groups = sae.get_parameters()
+    opt = pkg.HipAdam([{"params": groups[0]["params"]}, {"params": groups[1]["params"], "lr": 2e-3}], lr=1e-3, model=sae)
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=0.05)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(gb, **kw)
+    assert out["feature_acts"].dtype == torch.bfloat16
+    want = ref.compute_loss(batch, **kw)
+    assert rel_err(out["loss"], want["loss"]) < BF16_TOL
+    assert rel_err(out["l_s"], want["l_s"]) < BF16_TOL
+    agree = ((out["feature_acts"] != 0).cpu() == (want["feature_acts"] != 0)).float().mean().item()
+    assert agree > 0.995
+    out["loss"].backward()
+    before = {n: p.detach().clone() for n, p in sae.named_parameters()}
+    opt.step()
+    for n, p in sae.named_parameters():
+        assert torch.isfinite(p).all() and not torch.equal(p, before[n]), n
+    # the operands cached for the next step follow the update
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out2 = sae.compute_loss(gb, **kw)
+    assert torch.isfinite(out2["loss"]) and out2["loss"].item() != out["loss"].item()
