@@ -1,23 +1,28 @@
 #!/usr/bin/env python3
 """Headline benchmark: train tokens/s of the TopK SAE step on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--workload NAME]
 
 A "step" is one pass of the hot path over one batch of synthetic activations that already sit in
 HBM: compute_loss under bf16 autocast (encoder GEMM -> bias + TopK select -> sparse decode + MSE
 and its backward) -> loss.backward() (feature index, dW_D / dW_E rows, bias gradients) ->
-HipAdam.step() -> zero_grad().  Workload: d_model 4096, d_sae 131072, k 64, fp32 master weights with
-bf16 GEMM / gather operands (the reference's default mixed precision), B tokens per step.
+HipAdam.step() -> zero_grad().  Default workload: d_model 4096, d_sae 131072, k 64, fp32 master
+weights with bf16 GEMM / gather operands (the reference's default mixed precision), 4096 tokens per
+step.  `--workload` runs the same step on the other model configurations (BatchTopK with aux-k,
+JumpReLU with the tanh penalty, cross-layer transcoder, Lorsa) for profiling; their lines carry their
+own workload name.
 
-Prints ONE JSON line.  `roofline` describes the kernel with the largest share of the step, timed
-with HIP events inside the timed region; `cpu_baseline` is the oracle (a CPU restatement of the
-reference's eager path) timed on this host on a reduced batch of the same shape.
+Prints ONE JSON line.  `roofline` describes the kernel of this library with the largest share of
+the step, timed with HIP events inside the timed region; `cpu_baseline` (default workload only) is
+the oracle (a CPU restatement of the reference's eager path) timed on this host on a reduced batch
+of the same shape.
 """
 
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -29,14 +34,25 @@ D_MODEL, D_SAE, TOP_K = 4096, 131072, 64
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# Measured HBM bytes per launch (fetched + written, in GB) of the default workload's kernels, from two
+# rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE) of this file, scaled by what the same counters read for
+# transfers of known size in the same runs: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this machine.
+HBM_TRAFFIC_GB = {
+    "encoder_gemm": 8.51, "adam_step_sparse_rows[f32 dense]": 18.14, "adam_step_sparse_rows[bf16 dense]": 16.01,
+    "sparse_decode_mse_fused": 4.39, "select_topk_row": 2.31,
+}
 
-def algorithmic_work(B: int) -> dict:
-    """Per-launch algorithmic work of every kernel of the step (bytes unless noted)."""
-    d, F, k = D_MODEL, D_SAE, TOP_K
+
+def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
+    """Per-launch algorithmic work of the library's kernels (bytes unless noted) for B tokens of a
+    d -> F dictionary with k active features per token."""
     return {
         "encoder_gemm": ("mfma", 2.0 * B * d * F),                       # flop
         "select_topk_row": ("hbm", B * F * 2 + B * k * 8),               # read bf16 pre once, write idx+val
+        "select_topk_batch": ("hbm", 3 * B * F * 2 + B * k * 8),         # three radix passes over bf16 pre + ordered emit
         "sparse_decode_mse_fused": ("hbm", 2 * B * k * d * 2 + 3 * B * d * 4),  # rows for recon and for d val; label, recon, grad
+        "sparse_decode_fwd": ("hbm", B * k * d * 2 + B * d * 4),
+        "sparse_decode_bwd_dval": ("hbm", B * k * d * 2 + B * d * 4),
         "sparse_grad_rows[f32 dense]": ("hbm", F * d * 4),               # dW_D: one full fp32 gradient matrix written
         "sparse_grad_rows[bf16 dense]": ("hbm", F * d * 4),              # dW_E^T: likewise
         "adam_step[matrix]": ("hbm", F * d * 30),                        # g,p,m,v read; p,m,v written; bf16 shadow written
@@ -47,7 +63,165 @@ def algorithmic_work(B: int) -> dict:
         "build_feature_index": ("hbm", B * k * 16 + F * 12),
         "cast_f32_to_bf16": ("hbm", B * d * 6),
         "col_sum": ("hbm", B * d * 4),
+        "jumprelu_fwd": ("hbm", B * F * 4),                              # bf16 pre read, bf16 acts written
+        "jumprelu_bwd": ("hbm", B * F * 6),                              # bf16 pre and d_acts read, bf16 d_pre written
     }
+
+
+# ---- workloads ------------------------------------------------------------------------------------
+
+def _autocast_step(model, batch, opt, loss_kwargs):
+    import torch
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            loss = model.compute_loss(batch, return_aux_data=False, **loss_kwargs)
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        return loss
+    return step
+
+
+def _init_sae_on_device(sae, x, d, seed=4):
+    import torch
+
+    with torch.no_grad():
+        g = torch.Generator(device=x.device).manual_seed(seed)
+        wt = sae.W_E.t()
+        wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
+        sae.W_D.copy_(wt / wt.norm(dim=1, keepdim=True))
+        sae.b_E.zero_()
+        sae.b_D.copy_(x.mean(0))
+
+
+def build_topk(pkg, dev, args):
+    """The headline workload: TopK SAE d=4096, F=131072, k=64."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = args.batch or 4096, D_MODEL, D_SAE, TOP_K
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
+                        dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, 64, seed=4).to(dev)    # activations G(d, r=64, seed 4); weights drawn on the device
+    _init_sae_on_device(sae, x, d)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae,
+                      overlap_decoder_update=args.overlap)
+    name = f"topk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} fp32-master/bf16-operands adam"
+    return _autocast_step(sae, batch, opt, {}), B, name, (B, d, F, k)
+
+
+class _FixedDead:
+    """Stands in for the trainer's dead-feature statistics: a fixed set of features counts as dead."""
+
+    def __init__(self, is_dead):
+        self.is_dead = is_dead
+
+    def update_dead_statistics(self, feature_acts, mask, specs):
+        return self.is_dead
+
+    def update_dead_statistics_sparse(self, code, mask):
+        return self.is_dead
+
+
+def build_batchtopk(pkg, dev, args):
+    """BatchTopK SAE d=2048, F=32768, 8192 tokens, global top 64 x 8192, aux-k on the top 512 dead features."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = args.batch or 8192, 2048, 32768, 64
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="batchtopk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
+                        dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, 32, seed=4).to(dev)
+    _init_sae_on_device(sae, x, d)
+    g = torch.Generator(device=dev).manual_seed(5)
+    dead = _FixedDead(torch.rand(F, device=dev, generator=g) < 0.1)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae)
+    kw = dict(auxk_coefficient=1.0 / 32, k_aux=512, update_dead_statistics=dead.update_dead_statistics)
+    name = f"batchtopk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} aux-k=512 (10% of features dead) bf16 adam"
+    return _autocast_step(sae, batch, opt, kw), B, name, (B, d, F, k)
+
+
+def build_jumprelu(pkg, dev, args):
+    """JumpReLU SAE d=4096, F=131072, 4096 tokens: Gaussian rows with 4 outlier dimensions x50, threshold
+    log(0.001), rectangle window 0.001, tanh penalty coefficient 5."""
+    import torch
+
+    B, d, F = args.batch or 4096, D_MODEL, D_SAE
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=0.001, norm_activation="inference", sparsity_include_decoder_norm=True,
+                        device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(B, d, device=dev, generator=g)
+    x[:, [7, 511, 1024, 3000]] *= 50.0
+    _init_sae_on_device(sae, x, d)
+    with torch.no_grad():
+        sae.activation_function.log_jumprelu_threshold.fill_(math.log(0.001))
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    groups = sae.get_parameters()
+    opt = pkg.HipAdam([{"params": groups[0]["params"]}, {"params": groups[1]["params"]}], lr=4e-4, model=sae)
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=5.0)
+    name = f"jumprelu_sae_train_step d_model={d} d_sae={F} batch={B} window=0.001 tanh-penalty=5 bf16 adam"
+    return _autocast_step(sae, batch, opt, kw), B, name, (B, d, F, F // 2)
+
+
+def build_clt(pkg, dev, args):
+    """Cross-layer transcoder: 12 layers, d=768, 12288 features per layer, k=64 per layer, 2048 tokens;
+    targets y_j = tanh(A_j x_j) with seeded A_j ~ N(0, 1) / sqrt(768)."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, L, d, F, k = args.batch or 2048, 12, 768, 12288, 64
+    hin, hout = [f"in{l}" for l in range(L)], [f"out{l}" for l in range(L)]
+    cfg = pkg.CLTConfig(hook_points_in=hin, hook_points_out=hout, d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda", dtype=torch.float32)
+    clt = pkg.CrossLayerTranscoder(cfg)
+    clt.init_parameters()
+    g = torch.Generator(device=dev).manual_seed(4)
+    batch = {"tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    for l in range(L):
+        x = synthetic.activations(B, d, 16, seed=4 + l).to(dev)
+        A = torch.randn(d, d, device=dev, generator=g) / d ** 0.5
+        batch[hin[l]], batch[hout[l]] = x, torch.tanh(x @ A)
+    opt = pkg.HipAdam(clt.get_parameters()[0]["params"], lr=4e-4, model=clt)
+    name = f"clt_train_step layers={L} d_model={d} d_sae={F} k={k}/layer batch={B} bf16 adam"
+    return _autocast_step(clt, batch, opt, {}), B, name, (B, d, F, k)
+
+
+def build_lorsa(pkg, dev, args):
+    """Lorsa: d=768, 16 sequences x 1024 tokens, 64 query/key heads of width 64, 8192 value/output heads
+    (128 per query/key head), k=64; target = causal softmax attention of a seeded rank-64 head set."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    nb, s, d, F, h, dq, k = 16, 1024, 768, 8192, 64, 64, 64
+    cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
+                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type="none", act_fn="topk", top_k=k,
+                          norm_activation="inference", device="cuda", dtype=torch.float32)
+    m = pkg.LowRankSparseAttention(cfg)
+    m.init_parameters()
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = synthetic.activations(nb * s, d, 64, seed=4).to(dev).view(nb, s, d)
+    with torch.no_grad():
+        wq, wk = (torch.randn(d, 64, device=dev, generator=g) / d ** 0.5 for _ in range(2))
+        wvo = (torch.randn(d, 64, device=dev, generator=g) @ torch.randn(64, d, device=dev, generator=g)) / (8 * d ** 0.5)
+        y = torch.nn.functional.scaled_dot_product_attention((x @ wq)[:, None], (x @ wk)[:, None], (x @ wvo)[:, None],
+                                                             is_causal=True, scale=1 / 8)[:, 0]
+    batch = {"in": x, "out": y.contiguous(), "tokens": torch.zeros(nb, s, dtype=torch.long, device=dev)}
+    opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=4e-4, model=m)
+    name = f"lorsa_train_step d_model={d} sequences={nb}x{s} qk_heads={h}x{dq} ov_heads={F} k={k} bf16 adam"
+    return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
+
+
+WORKLOADS = {"topk": build_topk, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+             "lorsa": build_lorsa}
 
 
 def gpu_step_bench(args):
@@ -55,35 +229,8 @@ def gpu_step_bench(args):
     from __graft_entry__ import load_package
 
     pkg = load_package()
-    from lm_saes_amd import synthetic
-
     dev = torch.device("cuda:0")
-    B = args.batch
-    d, F, k = D_MODEL, D_SAE, TOP_K
-    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
-                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
-                        dtype=torch.float32)
-    sae = pkg.SparseAutoEncoder(cfg)
-    # N* recipe: activations G(d, r=64, seed 4); weights drawn on the device (1.07e9 parameters)
-    x = synthetic.activations(B, d, 64, seed=4).to(dev)
-    with torch.no_grad():
-        g = torch.Generator(device=dev).manual_seed(4)
-        wt = sae.W_E.t()
-        wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
-        sae.W_D.copy_(wt / wt.norm(dim=1, keepdim=True))
-        sae.b_E.zero_()
-        sae.b_D.copy_(x.mean(0))
-    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
-    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae,
-                       overlap_decoder_update=args.overlap)
-
-    def step():
-        with torch.autocast("cuda", dtype=torch.bfloat16):
-            loss = sae.compute_loss(batch, return_aux_data=False)
-        loss.backward()
-        opt.step()
-        opt.zero_grad()
-        return loss
+    step, tokens, name, shape = WORKLOADS[args.workload](pkg, dev, args)
 
     if args.calibrate_copy:
         # a plain device copy of known size (1 GiB read + 1 GiB written), for scaling rocprofv3's
@@ -107,8 +254,7 @@ def gpu_step_bench(args):
     t1 = time.perf_counter()
     pkg.ops.set_kernel_timer(None)
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernels = timer.summary()
-    return ms_per_step, kernels, float(loss.item())
+    return ms_per_step, timer.summary(), float(loss.item()), tokens, name, shape
 
 
 def cpu_baseline(sample_batch: int, sample_features: int):
@@ -151,7 +297,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=4096)
+    ap.add_argument("--batch", type=int, default=0, help="tokens per step (0: the workload's own size)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="topk")
     ap.add_argument("--cpu-sample-batch", type=int, default=512)
     ap.add_argument("--cpu-sample-features", type=int, default=32768)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -163,9 +310,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    ms_per_step, kernels, loss = gpu_step_bench(args)
-    B = args.batch
-    work = algorithmic_work(B)
+    ms_per_step, kernels, loss, tokens, name, shape = gpu_step_bench(args)
+    work = algorithmic_work(*shape)
     dominant = max(kernels, key=lambda n: kernels[n]["total_ms"])
     bound, per_launch = work.get(dominant, ("hbm", 0.0))
     avg_ms = kernels[dominant]["avg_ms"]
@@ -173,33 +319,40 @@ def main():
         achieved, peak, unit = per_launch / avg_ms / 1e9, PEAK_BF16_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = per_launch / avg_ms / 1e6, PEAK_HBM_GBS, "GB/s"
+    traffic = HBM_TRAFFIC_GB.get(dominant) if args.workload == "topk" else None
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-        "frac": round(achieved / peak, 4), "traffic": None, "avg_ms": round(avg_ms, 4),
+        "frac": round(achieved / peak, 4), "traffic": None if traffic is None else traffic * 1e9, "avg_ms": round(avg_ms, 4),
         "launches_per_step": kernels[dominant]["calls"] / args.steps,
     }
     per_kernel = {}
-    for name, st in kernels.items():
-        bnd, w = work.get(name, ("hbm", 0.0))
+    uniform = args.workload in ("topk", "batchtopk", "jumprelu")     # one dictionary shape for every launch
+    for kname, st in kernels.items():
+        bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None
-        per_kernel[name] = {
-            "ms_per_step": round(st["total_ms"] / args.steps, 4), "avg_ms": round(st["avg_ms"], 4), "bound": bnd,
+        per_kernel[kname] = {
+            "ms_per_step": round(st["total_ms"] / args.steps, 4), "avg_ms": round(st["avg_ms"], 4),
+            "launches_per_step": st["calls"] / args.steps, "bound": bnd,
             "achieved": None if rate is None else round(rate, 1),
             "frac": None if rate is None else round(rate / (PEAK_BF16_TFLOPS if bnd == "mfma" else PEAK_HBM_GBS), 4),
         }
+    if not uniform:
+        roofline.update(achieved=None, frac=None)   # launches of different shapes share a label: no single per-launch figure
+    headline = args.workload == "topk"
     out = {
-        "metric": "train tokens/s, TopK SAE d=4096 F=131072 k=64 bf16; % MFMA / HBM roofline",
-        "value": round(B / (ms_per_step / 1e3), 1),
+        "metric": "train tokens/s, TopK SAE d=4096 F=131072 k=64 bf16; % MFMA / HBM roofline" if headline
+                  else f"train tokens/s, {args.workload} workload (not the headline metric)",
+        "value": round(tokens / (ms_per_step / 1e3), 1),
         "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"topk_sae_train_step d_model={D_MODEL} d_sae={D_SAE} k={TOP_K} batch={B} "
-                               "fp32-master/bf16-operands adam", "batch_tokens": B},
+        "config": {"workload": name, "batch_tokens": tokens},
         "roofline": roofline,
         "kernels": per_kernel,
+        "kernel_ms_per_step": round(sum(v["ms_per_step"] for v in per_kernel.values()), 4),
         "final_loss": loss,
     }
-    if not args.no_cpu_baseline:
+    if headline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, args.cpu_sample_features)
     print(json.dumps(out))
 

@@ -213,8 +213,9 @@ def select_topk_row(
                 raise ValueError(f"{name} must have {F} elements")
     k = int(k)
     dev = pre.device
-    idx = torch.empty(B * k, dtype=torch.int32, device=dev)
-    val = torch.empty(B * k, dtype=torch.float32, device=dev)
+    # zero-filled: slots a row does not use (fewer than k positive entries) then hold feature 0 with value 0
+    idx = torch.zeros(B * k, dtype=torch.int32, device=dev)
+    val = torch.zeros(B * k, dtype=torch.float32, device=dev)
     row_off = torch.empty(B, dtype=torch.int64, device=dev)
     row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
     lib = _lib.load()

@@ -170,10 +170,11 @@ class Trainer:
         slots = torch.arange(code.n_slots, device=code.val.device)
         tok = torch.searchsorted(code.row_off, slots, right=True) - 1
         valid_slot = (slots - code.row_off[tok]) < code.row_nnz[tok]
-        vals = code.val * valid_slot
+        vals = torch.where(valid_slot, code.val, torch.zeros_like(code.val))
         if mask is not None:
             vals = vals * mask.reshape(-1).to(vals)[tok]
-        acts_sum = torch.zeros(code.d_sae, dtype=torch.float32, device=vals.device).index_add_(0, code.idx.long(), vals)
+        acts_sum = torch.zeros(code.d_sae, dtype=torch.float32, device=vals.device).index_add_(
+            0, torch.where(valid_slot, code.idx.long(), torch.zeros_like(tok)), vals)
         valid = mask.sum() if mask is not None else B
         return self._advance_dead_statistics(acts_sum.gt(0), valid)
 
