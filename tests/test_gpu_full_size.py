@@ -1,0 +1,396 @@
+"""The benchmark configurations at their full sizes.
+
+The CPU oracle cannot finish these shapes in seconds, so the kernel path is checked here through
+size-independent properties and against an independent dense recomputation with torch's library
+routines ON THE GPU (matmul, topk, sort): given the kernel's own pre-activation, the selection must
+be exactly the k largest with lowest-index ties; given the selection, reconstruction, loss and every
+gradient must equal what dense GEMMs give; the optimiser move must equal the closed-form first Adam
+step.  The small-shape tests elsewhere tie the same kernels to the CPU oracle.
+"""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(got, want):
+    return ((got.double() - want.double()).abs().max() / want.double().abs().max().clamp_min(1e-30)).item()
+
+
+def dense_mask(code):
+    """bool [B, F]: the positions a sparse code holds."""
+    B, F = code.n_tokens, code.d_sae
+    slots = torch.arange(code.n_slots, device=code.idx.device)
+    tok = (torch.searchsorted(code.row_off, slots, right=True) - 1).clamp_(min=0)
+    valid = (slots - code.row_off[tok]) < code.row_nnz[tok]
+    m = torch.zeros(B * F, dtype=torch.bool, device=code.idx.device)
+    m[(tok * F + code.idx.long())[valid]] = True
+    return m.view(B, F)
+
+
+def check_threshold_selection(score, kept, per_row: bool):
+    """kept must be the largest entries of `score` (per row, or over the whole batch), ties at the
+    threshold going to the lowest (flattened) index."""
+    if not per_row:
+        score, kept = score.reshape(1, -1), kept.reshape(1, -1)
+    lo = score.masked_fill(~kept, float("inf")).min(dim=1).values          # smallest kept
+    hi = score.masked_fill(kept, float("-inf")).max(dim=1).values          # largest dropped
+    assert torch.all(lo >= hi), "a dropped entry is larger than a kept one"
+    assert torch.all(lo > 0), "a non-positive entry was kept"
+    tied = lo == hi
+    if tied.any():
+        n = score.shape[1]
+        pos = torch.arange(n, device=score.device).expand_as(score)
+        at_t = score == lo[:, None]
+        last_kept = torch.where(at_t & kept, pos, torch.full_like(pos, -1)).max(dim=1).values
+        first_dropped = torch.where(at_t & ~kept, pos, torch.full_like(pos, n)).min(dim=1).values
+        assert torch.all(last_kept[tied] < first_dropped[tied]), "a tie at the threshold did not go to the lowest index"
+    return int(tied.sum().item())
+
+
+def build_sae(pkg, dev, d, F, k, B, r, act_fn="topk", seed=4):
+    from lm_saes_amd import synthetic
+
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn=act_fn, top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, r, seed=seed).to(dev)
+    with torch.no_grad():
+        g = torch.Generator(device=dev).manual_seed(seed)
+        wt = sae.W_E.t()
+        wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
+        sae.W_D.copy_(wt / wt.norm(dim=1, keepdim=True) * (0.5 + torch.rand(F, 1, device=dev, generator=g)))
+        sae.b_E.copy_(0.01 * torch.randn(F, device=dev, generator=g))
+        sae.b_D.copy_(x.mean(0))
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    return sae, batch
+
+
+def own_scores(pkg, sae, x):
+    """(h, n): the pre-activation plus bias exactly as the select kernel forms it (the encoder kernel is
+    deterministic, so running it again gives the same bits) and the decoder norms it scales by."""
+    pre = pkg.ops.encoder_gemm(pkg.ops.cast_bf16(x.contiguous()), sae._w_enc_operand(True), torch.bfloat16)
+    return pre.float() + sae.b_E.detach(), sae._decoder_norm_nograd()
+
+
+def dense_backward(sae, x_bf, kept, val, recon, label, w):
+    """Gradients of sum_b w_b |recon_b - label_b|^2 by dense library GEMMs, given the selection `kept`, the kept
+    values `val` ([B, F] dense) and bf16-rounded operands (the rounding the kernels' operands carry)."""
+    Wd = sae._w_dec_operand(True).float()
+    grad_recon = 2.0 * w[:, None] * (recon - label)
+    dW_D = val.t() @ grad_recon
+    d_pre = (grad_recon @ Wd.t()) * kept
+    dW_Et = d_pre.t() @ x_bf.float()
+    return dW_D, dW_Et, d_pre.sum(0), grad_recon.sum(0)
+
+
+def test_headline_shape_step_properties(pkg, dev):
+    """TopK SAE d=4096, F=131072, k=64, 4096 tokens, bf16 operands: the benchmark's own configuration."""
+    d, F, k, B = 4096, 131072, 64, 4096
+    sae, batch = build_sae(pkg, dev, d, F, k, B, r=64)
+    x = batch["in"]
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(batch)
+    code = out["sparse_code"]
+    # --- the code: k entries per row, ascending, in range
+    assert torch.all(code.row_nnz == k) and torch.equal(code.row_off, torch.arange(B, device=dev) * k)
+    idx = code.idx.view(B, k)
+    assert torch.all(idx[:, 1:] > idx[:, :-1]) and idx.min() >= 0 and idx.max() < F
+    # --- selection = k largest of the kernel's own scaled pre-activation, lowest index on ties
+    hp, n = own_scores(pkg, sae, x)                         # (pre + b_E) as the kernel formed it, [B, F] fp32
+    assert rel_err(out["hidden_pre"], hp) < 1e-6
+    x_bf = x.bfloat16()
+    assert rel_err(hp, x_bf.float() @ sae._w_enc_operand(True).float().t() + sae.b_E.detach()) < 2e-2     # bf16 output rounding
+    kept = dense_mask(code)
+    ties = check_threshold_selection(hp * n, kept, per_row=True)
+    print(f"rows with a tie at the threshold: {ties}", flush=True)
+    val = torch.zeros(B, F, device=dev).masked_scatter_(kept, code.val)        # both in (row, ascending index) order
+    assert rel_err(val[kept], ((hp * n) / n)[kept]) < 1e-6                      # kept values: scaled, selected, unscaled again
+    # --- decode, loss
+    Wd = sae._w_dec_operand(True).float()
+    recon = val @ Wd + sae.b_D.detach()
+    assert rel_err(out["reconstructed"], recon) < 1e-4
+    w = torch.full((B,), 1.0 / B, device=dev)
+    assert abs(out["loss"].item() - ((recon - x).pow(2).sum(-1) * w).sum().item()) < 1e-4 * out["loss"].item()
+    doubled = pkg.ops.sparse_decode_fwd(pkg.ops.SparseCode(code.idx, 2 * code.val, code.row_off, code.row_nnz, B, F),
+                                        sae._w_dec_operand(True), sae.b_D.detach())
+    assert rel_err(doubled - sae.b_D.detach(), 2 * (out["reconstructed"] - sae.b_D.detach())) < 1e-6   # linear in the values
+    # --- backward against dense GEMMs
+    out["loss"].backward()
+    dW_D, dW_Et, db_E, db_D = dense_backward(sae, x_bf, kept, val, out["reconstructed"], x, w)
+    assert rel_err(sae.W_D.grad, dW_D) < 1e-4
+    assert rel_err(sae.W_E.grad.t(), dW_Et) < 1e-4
+    assert rel_err(sae.b_E.grad, db_E) < 1e-4 and rel_err(sae.b_D.grad, db_D) < 1e-4
+    # --- the optimiser consuming factored gradients: closed-form first Adam step, fresh shadows and norms
+    g_D, g_Et = sae.W_D.grad.clone(), sae.W_E.grad.t().clone()
+    p_D, p_Et = sae.W_D.detach().clone(), sae.W_E.detach().t().clone()
+    for p in sae.parameters():
+        p.grad = None
+    lr, eps = 4e-4, 1e-8
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=lr, eps=eps, model=sae)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        loss = sae.compute_loss(batch, return_aux_data=False)
+    loss.backward()
+    assert sae.W_D.grad is None and sae.W_D._sparse_grad is not None      # no dense gradient matrix was written
+    opt.step()
+    for p_new, p_old, g in ((sae.W_D.detach(), p_D, g_D), (sae.W_E.detach().t(), p_Et, g_Et)):
+        want = -lr * g / (g.abs() + eps)           # m_hat = g, v_hat = g^2 on the first step
+        assert ((p_new - p_old) - want).abs().max().item() < 2e-3 * lr
+    assert torch.equal(sae.get_derived_buffer("W_D.bf16"), sae.W_D.detach().bfloat16())
+    assert torch.equal(sae.get_derived_buffer("W_E.bf16"), sae.W_E.detach().t().bfloat16())
+    assert rel_err(sae.get_derived_buffer("W_D.norm"), sae.W_D.detach().norm(dim=1)) < 1e-6
+
+
+class _FixedDead:
+    def __init__(self, is_dead):
+        self.is_dead = is_dead
+
+    def update_dead_statistics(self, feature_acts, mask, specs):
+        return self.is_dead
+
+    def update_dead_statistics_sparse(self, code, mask):
+        return self.is_dead
+
+
+def test_batchtopk_auxk_shape_step_properties(pkg, dev):
+    """BatchTopK SAE d=2048, F=32768, 8192 tokens, global top 64 x 8192, aux-k over the top 512 dead features."""
+    d, F, k, B, k_aux, alpha = 2048, 32768, 64, 8192, 512, 1 / 32
+    sae, batch = build_sae(pkg, dev, d, F, k, B, r=32, act_fn="batchtopk")
+    x = batch["in"]
+    g = torch.Generator(device=dev).manual_seed(5)
+    is_dead = torch.rand(F, device=dev, generator=g) < 0.1
+    dead = _FixedDead(is_dead)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(batch, auxk_coefficient=alpha, k_aux=k_aux, update_dead_statistics=dead.update_dead_statistics)
+    code = out["sparse_code"]
+    assert int(code.row_nnz.sum().item()) == k * B                                  # exactly k x B survive, batch-wide
+    assert code.row_nnz.float().std().item() > 0
+    hp, n = own_scores(pkg, sae, x)
+    kept = dense_mask(code)
+    assert int(kept.sum().item()) == k * B
+    check_threshold_selection(hp * n, kept, per_row=False)
+    # rows ascend in index
+    val = torch.zeros(B, F, device=dev).masked_scatter_(kept, code.val[: k * B])
+    assert rel_err(val[kept], hp[kept]) < 1e-6
+    # the aux selection, recomputed densely: the k_aux x B largest of the dead features' scaled pre-activations
+    n_dead = int(is_dead.sum().item())
+    kk = min(k_aux, n_dead) * B
+    dead_score = torch.where(is_dead[None, :], hp * n, torch.zeros_like(hp)).clamp_min(0)
+    thr = torch.topk(dead_score.flatten(), kk).values[-1]
+    aux_kept = dead_score > thr                                                       # strict: ties at the threshold aside
+    Wd = sae._w_dec_operand(True).float()
+    recon = val @ Wd + sae.b_D.detach()
+    assert rel_err(out["reconstructed"], recon) < 1e-4
+    w = torch.full((B,), 1.0 / B, device=dev)
+    l_rec = ((recon - x).pow(2).sum(-1) * w).sum()
+    aux_val = torch.where(aux_kept, hp, torch.zeros_like(hp))
+    resid = (x - recon) - aux_val @ Wd
+    l_aux = alpha * (resid.pow(2).sum(-1) * w).sum()
+    assert abs(out["l_rec"].item() - l_rec.item()) < 1e-4 * l_rec.item()
+    assert abs(out["l_aux"].item() - l_aux.item()) < 1e-3 * l_aux.item()            # a handful of threshold ties may differ
+    out["loss"].backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in sae.parameters())
+    # gradient of the decoder bias: column sums of d loss / d recon, with the residual carrying gradient
+    g_recon = 2.0 * w[:, None] * (recon - x) - 2.0 * alpha * w[:, None] * resid
+    assert rel_err(sae.b_D.grad, g_recon.sum(0)) < 1e-3
+    # dead features only ever receive aux gradient rows; live unselected features none at all
+    untouched = ~(kept.any(0) | (is_dead & (dead_score > 0).any(0)))
+    assert torch.all(sae.W_D.grad[untouched] == 0)
+
+
+def test_reference_cpu_configuration_full_size_against_oracle(pkg, oracle, dev):
+    """The configuration the reference's CPU path runs: d=768, F=6144, k=32, 4096 tokens, fp32, one step with
+    Adam (lr 4e-4), against the oracle itself (its encoder product takes the kernel's forward values so that
+    last-bit differences of the two GEMMs cannot flip a selection)."""
+    from lm_saes_amd import synthetic
+
+    d, F, k, B = 768, 6144, 32, 4096
+    x = synthetic.activations(B, d, 16, seed=4)
+    w = synthetic.sae_weights(d, F, x, seed=4)
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    synthetic.load_weights(sae, *[t.to(dev) for t in w])
+    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=True)
+    synthetic.load_weights(ref, *w)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long)}
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae)
+    ropt = oracle.make_adam(ref, lr=4e-4)
+    out = sae.compute_loss(gb)
+    out["loss"].backward()
+    pre = pkg.ops.encoder_gemm(gb["in"].contiguous(), sae._w_enc_operand(False), torch.float32).cpu()
+
+    class Sub(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, xx, W):
+            ctx.save_for_backward(xx, W)
+            return pre.clone()
+
+        @staticmethod
+        def backward(ctx, gg):
+            xx, W = ctx.saved_tensors
+            return gg @ W.t(), xx.t() @ gg
+
+    def encode_sub(xx, return_hidden_pre=False, **_):
+        hp = (Sub.apply(xx, ref.W_E) + ref.b_E) * ref.decoder_norm()
+        fa = ref.activation_function(hp) / ref.decoder_norm()
+        return (fa, hp / ref.decoder_norm()) if return_hidden_pre else fa
+
+    ref.encode = encode_sub
+    want = ref.compute_loss(batch)
+    want["loss"].backward()
+    assert torch.equal((out["feature_acts"] != 0).cpu(), want["feature_acts"] != 0)          # bit-exact index sets
+    assert rel_err(out["feature_acts"].cpu(), want["feature_acts"]) < 1e-5
+    assert rel_err(out["reconstructed"].cpu(), want["reconstructed"]) < 1e-5
+    assert abs(out["loss"].item() - want["loss"].item()) < 1e-5 * want["loss"].item()
+    opt.materialize_grads()
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        assert rel_err(getattr(sae, name).grad.cpu(), getattr(ref, name).grad) < 1e-5, name
+    before = {n_: p.detach().clone() for n_, p in ref.named_parameters()}
+    grads = {n_: p.grad.detach().clone() for n_, p in ref.named_parameters()}
+    opt.step(); ropt.step()
+    for n_, p in sae.named_parameters():
+        move, want_move = p.detach().cpu() - before[n_], dict(ref.named_parameters())[n_].detach() - before[n_]
+        # the first Adam step is g / (|g| + eps): where |g| is within rounding of zero the two sides may differ in
+        # sign, so the move is compared where the gradient is resolved, and bounded by lr everywhere
+        resolved = grads[n_].abs() > 1e-3 * grads[n_].abs().max()
+        assert (move - want_move)[resolved].abs().max().item() < 2e-3 * 4e-4, n_
+        assert move.abs().max().item() <= 4e-4 * (1 + 1e-5), n_
+
+
+def test_clt_shape_fused_step_against_dense_path(pkg, dev):
+    """CLT, 12 layers, d=768, 12288 features per layer, k=64 per layer, 2048 tokens, fp32: the prefix decode
+    of the concatenated sparse code against the module's dense path (78 library GEMMs), forward and backward."""
+    from lm_saes_amd import synthetic
+
+    L, d, F, k, B = 12, 768, 12288, 64, 2048
+    hin, hout = [f"in{l}" for l in range(L)], [f"out{l}" for l in range(L)]
+    cfg = pkg.CLTConfig(hook_points_in=hin, hook_points_out=hout, d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda", dtype=torch.float32)
+    clt = pkg.CrossLayerTranscoder(cfg)
+    clt.init_parameters()
+    g = torch.Generator(device=dev).manual_seed(4)
+    batch = {"tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    for l in range(L):
+        x = synthetic.activations(B, d, 16, seed=4 + l).to(dev)
+        batch[hin[l]], batch[hout[l]] = x, torch.tanh(x @ (torch.randn(d, d, device=dev, generator=g) / d ** 0.5))
+    out = clt.compute_loss(batch)
+    code = out["sparse_code"]
+    assert torch.all(code.row_nnz == L * k)
+    out["loss"].backward()
+    fused = {n_: p.grad.clone() for n_, p in clt.named_parameters()}
+    for p in clt.parameters():
+        p.grad = None
+    # dense path on the kernel's own selection (a second encoder product by the library GEMM would differ in
+    # the last bit and could flip near-ties): decode through the 78 dense blocks, autograd for the decoder side
+    xs, _, _ = clt.prepare_input(batch)
+    label = clt.prepare_label(batch)
+    feature_acts = out["feature_acts"].clone().requires_grad_()
+    kept = feature_acts.detach() != 0
+    assert int(kept.sum().item()) == B * L * k
+    recon = clt.decode(feature_acts)
+    loss = (recon - label).pow(2).sum(-1).mean()
+    assert rel_err(out["reconstructed"], recon) < 1e-4
+    assert abs(out["loss"].item() - loss.item()) < 1e-5 * loss.item()
+    loss.backward()
+    for n_, p in clt.named_parameters():
+        if n_.startswith("W_D") or n_.startswith("b_D"):
+            assert rel_err(fused[n_], p.grad) < 2e-4, n_
+    # encoder side: TopK passes the gradient of kept entries unchanged (the decoder-norm factors cancel)
+    d_pre = feature_acts.grad * kept
+    assert rel_err(fused["W_E"], torch.einsum("bld,blf->ldf", xs, d_pre)) < 2e-4
+    assert rel_err(fused["b_E"], d_pre.sum(0)) < 2e-4
+    # and the values the code holds are the unscaled pre-activations of its own encoder product
+    hp = torch.stack([pkg.ops.encoder_gemm(xs[:, l].contiguous(), clt._w_enc_operand(False)[l], torch.float32)
+                      for l in range(L)], dim=1) + clt.b_E.detach()
+    assert rel_err(feature_acts.detach()[kept], hp[kept]) < 1e-6
+    score = (hp * clt._norm_per_feature_nograd()).view(B * L, F)
+    check_threshold_selection(score, kept.view(B * L, F), per_row=True)
+
+
+def test_lorsa_shape_fused_step_against_dense_path(pkg, dev):
+    """Lorsa, d=768, 16 x 1024 tokens, 64 query/key heads of width 64, 8192 value/output heads, k=64, fp32:
+    the sparse tail (select, sparse decode, W_O rows, scatter of the value gradients) against the dense path."""
+    from lm_saes_amd import synthetic
+
+    nb, s, d, F, h, dq, k = 16, 1024, 768, 8192, 64, 64, 64
+    cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
+                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type="none", act_fn="topk", top_k=k,
+                          norm_activation="inference", device="cuda", dtype=torch.float32)
+    m = pkg.LowRankSparseAttention(cfg)
+    m.init_parameters()
+    x = synthetic.activations(nb * s, d, 64, seed=4).to(dev).view(nb, s, d)
+    y = torch.roll(x, 1, dims=1) * 0.5
+    batch = {"in": x, "out": y, "tokens": torch.zeros(nb, s, dtype=torch.long, device=dev)}
+    out = m.compute_loss(batch)
+    assert "sparse_code" in out and torch.all(out["sparse_code"].row_nnz == k)
+    out["loss"].backward()
+    fused = {n_: p.grad.clone() for n_, p in m.named_parameters()}
+    for p in m.parameters():
+        p.grad = None
+    want = pkg.SparseDictionary.compute_loss(m, batch)          # the generic dense op sequence
+    assert torch.equal(want["feature_acts"] != 0, out["feature_acts"] != 0)
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < 1e-4
+    assert abs(out["loss"].item() - want["loss"].item()) < 1e-5 * want["loss"].item()
+    want["loss"].backward()
+    scale = max(p.grad.abs().max().item() for p in m.parameters())
+    for n_, p in m.named_parameters():
+        if p.grad.abs().max().item() < 1e-5 * scale:        # analytically zero (key bias): rounding noise on both sides
+            continue
+        assert rel_err(fused[n_], p.grad) < 2e-4, n_
+
+
+def test_jumprelu_shape_fused_step_against_dense_path(pkg, dev):
+    """JumpReLU SAE d=4096, F=131072, 4096 tokens, threshold 0.001, window 0.001, tanh penalty 5, fp32: the fused
+    element-wise kernels against the generic dense op sequence fed the same encoder product."""
+    d, F, B = 4096, 131072, 4096
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=0.001, norm_activation="inference", sparsity_include_decoder_norm=True,
+                        device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(B, d, device=dev, generator=g)
+    x[:, [7, 511, 1024, 3000]] *= 50.0
+    with torch.no_grad():
+        wt = sae.W_E.t()
+        wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
+        sae.W_D.copy_(wt / wt.norm(dim=1, keepdim=True))
+        sae.b_E.zero_()
+        sae.b_D.copy_(x.mean(0))
+        sae.activation_function.log_jumprelu_threshold.fill_(math.log(0.001))
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=5.0)
+    out = sae.compute_loss(batch, **kw)
+    out["loss"].backward()
+    fused = {n_: p.grad.clone() for n_, p in sae.named_parameters()}
+    acts_mask, loss_f, l_s_f = out["feature_acts"] != 0, out["loss"].item(), out["l_s"].mean().item()
+    pre = out["hidden_pre"] - sae.b_E.detach()
+    del out
+    for p in sae.parameters():
+        p.grad = None
+
+    class Sub(torch.autograd.Function):      # the kernel's encoder product as the forward value, matmul backward
+        @staticmethod
+        def forward(ctx, xx, W):
+            ctx.save_for_backward(xx, W)
+            return pre.clone()
+
+        @staticmethod
+        def backward(ctx, gg):
+            xx, W = ctx.saved_tensors
+            return gg @ W.t(), xx.t() @ gg
+
+    sae._matmul_enc = lambda xx, W: Sub.apply(xx, W)
+    want = pkg.SparseDictionary.compute_loss(sae, batch, **kw)
+    assert torch.equal(want["feature_acts"] != 0, acts_mask)
+    assert 0.3 < acts_mask.float().mean().item() < 0.7               # about half of all features fire at this threshold
+    assert abs(loss_f - want["loss"].item()) < 1e-5 * want["loss"].item()
+    assert abs(l_s_f - want["l_s"].mean().item()) < 1e-5 * want["l_s"].mean().item()
+    want["loss"].backward()
+    for n_, p in sae.named_parameters():
+        assert rel_err(fused[n_], p.grad) < 2e-4, n_
+    assert (fused["activation_function.log_jumprelu_threshold"] != 0).float().mean().item() > 0.5
