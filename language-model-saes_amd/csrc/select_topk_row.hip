@@ -9,8 +9,12 @@
 //   1. every thread takes the maximum key of the elements it owns; the k-th largest of those
 //      1024 maxima is a lower bound L of the k-th largest key of the row, because k distinct
 //      elements are >= L;
-//   2. the row is read again (it sits in L2 now) and every element with key >= L is appended
-//      to a candidate list in LDS -- for i.i.d. data about k + a few elements;
+//   2. every element with key >= L is appended to a candidate list in LDS -- for i.i.d. data about
+//      k + a few elements.  Rows of up to 131072 elements are not read again for this: pass 1 keeps
+//      the largest key of every 16-byte chunk in registers, which is enough to rule out all but a
+//      handful of chunks, and only those are re-formed from memory (the bias and scale vectors
+//      cost four times the row's own bytes per pass, so a second pass over memory is what the
+//      kernel's time would otherwise go to).  Longer rows are read a second time;
 //   3. an exact radix select over the candidates in LDS yields the threshold key T; among
 //      the candidates with key == T the lowest indices win (a second radix select over the
 //      indices); the kept elements are ranked by index and written in ascending order.
@@ -105,69 +109,81 @@ struct RowReader {
   const float *scale;
   const float *fmask;
   int F;
+  static constexpr int V = BF16 ? 8 : 4;  // elements per 16-byte load
+  __device__ __forceinline__ bool vec_ok() const {
+    return (F % V == 0) && (((((uintptr_t)row) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
+  }
+  // keys of the V elements of 16-byte chunk c
+  __device__ __forceinline__ u32x4 load_raw(int c) const { return reinterpret_cast<const u32x4 *>(row)[c]; }
+  __device__ __forceinline__ void chunk_keys(int c, uint32_t (&keys)[V]) const { keys_from_raw(c, load_raw(c), keys); }
+  __device__ __forceinline__ void keys_from_raw(int c, const u32x4 &raw, uint32_t (&keys)[V]) const {
+    float pre[V];
+    if constexpr (BF16) {
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        pre[2 * q] = __uint_as_float(w[q] << 16);
+        pre[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u);
+      }
+    } else {
+      pre[0] = __uint_as_float(raw.x); pre[1] = __uint_as_float(raw.y);
+      pre[2] = __uint_as_float(raw.z); pre[3] = __uint_as_float(raw.w);
+    }
+    const int base = c * V;
+    float bb[V], ss[V], mm[V];
+    if (fmask) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        const float4 t = reinterpret_cast<const float4 *>(fmask + base)[q];
+        mm[4 * q] = t.x; mm[4 * q + 1] = t.y; mm[4 * q + 2] = t.z; mm[4 * q + 3] = t.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) mm[e] = 1.f;
+    }
+    if (b_enc) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        const float4 t = reinterpret_cast<const float4 *>(b_enc + base)[q];
+        bb[4 * q] = t.x; bb[4 * q + 1] = t.y; bb[4 * q + 2] = t.z; bb[4 * q + 3] = t.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) bb[e] = 0.f;
+    }
+    if (scale) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        const float4 t = reinterpret_cast<const float4 *>(scale + base)[q];
+        ss[4 * q] = t.x; ss[4 * q + 1] = t.y; ss[4 * q + 2] = t.z; ss[4 * q + 3] = t.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss[e] = 1.f;
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) keys[e] = key_of(pre[e], bb[e], ss[e], mm[e], fmask != nullptr);
+  }
+  // key of one element
+  __device__ __forceinline__ uint32_t key_at(int i) const {
+    float pre;
+    if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
+    else pre = reinterpret_cast<const float *>(row)[i];
+    return key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr);
+  }
   // calls fn(index, key) for every element of the row, vectorised when the row allows it
   template <typename Fn>
   __device__ __forceinline__ void for_each(Fn fn) const {
-    constexpr int V = BF16 ? 8 : 4;  // elements per 16-byte load
-    const bool vec_ok = (F % V == 0) && (((((uintptr_t)row) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
-    if (vec_ok) {
+    if (vec_ok()) {
       const int n_chunks = F / V;
       for (int c = threadIdx.x; c < n_chunks; c += SEL_THREADS) {
-        const u32x4 raw = reinterpret_cast<const u32x4 *>(row)[c];
-        float pre[V];
-        if constexpr (BF16) {
-          const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        uint32_t keys[V];
+        chunk_keys(c, keys);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            pre[2 * q] = __uint_as_float(w[q] << 16);
-            pre[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u);
-          }
-        } else {
-          pre[0] = __uint_as_float(raw.x); pre[1] = __uint_as_float(raw.y);
-          pre[2] = __uint_as_float(raw.z); pre[3] = __uint_as_float(raw.w);
-        }
-        const int base = c * V;
-        float bb[V], ss[V], mm[V];
-        if (fmask) {
-#pragma unroll
-          for (int q = 0; q < V / 4; ++q) {
-            const float4 t = reinterpret_cast<const float4 *>(fmask + base)[q];
-            mm[4 * q] = t.x; mm[4 * q + 1] = t.y; mm[4 * q + 2] = t.z; mm[4 * q + 3] = t.w;
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < V; ++e) mm[e] = 1.f;
-        }
-        if (b_enc) {
-#pragma unroll
-          for (int q = 0; q < V / 4; ++q) {
-            const float4 t = reinterpret_cast<const float4 *>(b_enc + base)[q];
-            bb[4 * q] = t.x; bb[4 * q + 1] = t.y; bb[4 * q + 2] = t.z; bb[4 * q + 3] = t.w;
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < V; ++e) bb[e] = 0.f;
-        }
-        if (scale) {
-#pragma unroll
-          for (int q = 0; q < V / 4; ++q) {
-            const float4 t = reinterpret_cast<const float4 *>(scale + base)[q];
-            ss[4 * q] = t.x; ss[4 * q + 1] = t.y; ss[4 * q + 2] = t.z; ss[4 * q + 3] = t.w;
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < V; ++e) ss[e] = 1.f;
-        }
-#pragma unroll
-        for (int e = 0; e < V; ++e) fn(base + e, key_of(pre[e], bb[e], ss[e], mm[e], fmask != nullptr));
+        for (int e = 0; e < V; ++e) fn(c * V + e, keys[e]);
       }
     } else {
-      for (int i = threadIdx.x; i < F; i += SEL_THREADS) {
-        float pre;
-        if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
-        else pre = reinterpret_cast<const float *>(row)[i];
-        fn(i, key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr));
-      }
+      for (int i = threadIdx.x; i < F; i += SEL_THREADS) fn(i, key_at(i));
     }
   }
 };
@@ -192,8 +208,15 @@ __device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<B
   }
 }
 
-template <bool BF16>
-__global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
+// STASH: the row has at most SEL_STASH_ELEMS elements per thread and is 16-byte addressable.  Pass 1 then
+// keeps the largest key of every 16-byte chunk it reads in a register (16 or 32 per thread), and pass 2
+// walks those registers instead of reading the row, its bias and its scale a second time: a chunk can only
+// contribute to the candidate list if its largest key is >= the bound, and only those chunks (k plus a
+// handful per row) are formed again from memory.
+constexpr int SEL_STASH_ELEMS = 128;  // per thread: rows up to 131072 elements
+
+template <bool BF16, bool STASH>
+__global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
     int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
@@ -211,10 +234,43 @@ __global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
   // ---- pass 1: per-thread maximum key and number of positive elements ----
   uint32_t my_max = 0u;
   int my_pos = 0;
-  rr.for_each([&](int, uint32_t key) {
-    my_max = key > my_max ? key : my_max;
-    my_pos += key != 0u;
-  });
+  constexpr int V = RowReader<BF16>::V;
+  constexpr int NCH = SEL_STASH_ELEMS / V;            // chunks per thread when stashing
+  uint32_t cmax[STASH ? NCH : 1];                     // largest key of each of this thread's chunks
+  if constexpr (STASH) {
+    const int n_chunks = F / V;
+    constexpr int G = 1;   // row chunks requested together (more than one costs registers the two-workgroup occupancy needs)
+#pragma unroll
+    for (int j0 = 0; j0 < NCH; j0 += G) {
+      u32x4 raw[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int c = tid + (j0 + g) * SEL_THREADS;
+        raw[g] = rr.load_raw(c < n_chunks ? c : tid);     // clamped: a valid address, result unused
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int c = tid + (j0 + g) * SEL_THREADS;
+        uint32_t m = 0u;
+        if (c < n_chunks) {
+          uint32_t keys[V];
+          rr.keys_from_raw(c, raw[g], keys);
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            m = keys[e] > m ? keys[e] : m;
+            my_pos += keys[e] != 0u;
+          }
+        }
+        cmax[j0 + g] = m;
+        my_max = m > my_max ? m : my_max;
+      }
+    }
+  } else {
+    rr.for_each([&](int, uint32_t key) {
+      my_max = key > my_max ? key : my_max;
+      my_pos += key != 0u;
+    });
+  }
   sh.tmax[tid] = my_max;
   if (tid == 0) sh.count = 0;
   // total positives in the row
@@ -255,12 +311,27 @@ __global__ __launch_bounds__(SEL_THREADS) void select_topk_row_kernel(
   if (!general) {
     // ---- pass 2: gather candidates with key >= L (and key > 0) into LDS ----
     const uint32_t L = (n_pos <= k) ? 1u : (T == 0u ? 1u : T);
-    rr.for_each([&](int i, uint32_t key) {
+    auto consider = [&](int i, uint32_t key) {
       if (key >= L) {
         const int slot = atomicAdd(&sh.count, 1);
         if (slot < cand_cap) { sh.cand_key[slot] = key; sh.cand_idx[slot] = i; }
       }
-    });
+    };
+    if constexpr (STASH) {
+      // only chunks whose largest key reaches L can contribute: k plus a handful per row; those are read again
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) {
+        if (cmax[j] >= L) {
+          const int c = tid + j * SEL_THREADS;
+          uint32_t keys[V];
+          rr.chunk_keys(c, keys);
+#pragma unroll
+          for (int e = 0; e < V; ++e) consider(c * V + e, keys[e]);
+        }
+      }
+    } else {
+      rr.for_each(consider);
+    }
     __syncthreads();
     n_cand = sh.count;
     if (n_cand > cand_cap) general = true;
@@ -380,12 +451,20 @@ extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const floa
   const int kk = k > F ? (int)F : k;
   (void)kk;
   hipStream_t st = (hipStream_t)stream;
-  if (pre_dtype == SAE_BF16)
-    hipLaunchKernelGGL(select_topk_row_kernel<true>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale, feat_mask,
-                       (int)F, k, idx, val, row_off, row_nnz, cand_cap);
-  else
-    hipLaunchKernelGGL(select_topk_row_kernel<false>, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale, feat_mask,
-                       (int)F, k, idx, val, row_off, row_nnz, cand_cap);
+  const int V = pre_dtype == SAE_BF16 ? 8 : 4;
+  const size_t row_bytes = (size_t)F * (pre_dtype == SAE_BF16 ? 2 : 4);
+  // every row 16-byte addressable and short enough for the register stash
+  const bool stash = (F % V == 0) && F <= (int64_t)SEL_STASH_ELEMS * SEL_THREADS && (row_bytes % 16 == 0) &&
+                     (((((uintptr_t)pre) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)feat_mask) & 15) == 0);
+#define SAE_LAUNCH_SELECT(BF, ST)                                                                                          \
+  hipLaunchKernelGGL((select_topk_row_kernel<BF, ST>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,       \
+                     feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap)
+  if (pre_dtype == SAE_BF16) {
+    if (stash) SAE_LAUNCH_SELECT(true, true); else SAE_LAUNCH_SELECT(true, false);
+  } else {
+    if (stash) SAE_LAUNCH_SELECT(false, true); else SAE_LAUNCH_SELECT(false, false);
+  }
+#undef SAE_LAUNCH_SELECT
   return check_launch("select_topk_row");
 }
 
