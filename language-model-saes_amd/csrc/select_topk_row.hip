@@ -239,31 +239,21 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   uint32_t cmax[STASH ? NCH : 1];                     // largest key of each of this thread's chunks
   if constexpr (STASH) {
     const int n_chunks = F / V;
-    constexpr int G = 1;   // row chunks requested together (more than one costs registers the two-workgroup occupancy needs)
 #pragma unroll
-    for (int j0 = 0; j0 < NCH; j0 += G) {
-      u32x4 raw[G];
+    for (int j = 0; j < NCH; ++j) {
+      const int c = tid + j * SEL_THREADS;
+      uint32_t m = 0u;
+      if (c < n_chunks) {
+        uint32_t keys[V];
+        rr.chunk_keys(c, keys);
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const int c = tid + (j0 + g) * SEL_THREADS;
-        raw[g] = rr.load_raw(c < n_chunks ? c : tid);     // clamped: a valid address, result unused
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const int c = tid + (j0 + g) * SEL_THREADS;
-        uint32_t m = 0u;
-        if (c < n_chunks) {
-          uint32_t keys[V];
-          rr.keys_from_raw(c, raw[g], keys);
-#pragma unroll
-          for (int e = 0; e < V; ++e) {
-            m = keys[e] > m ? keys[e] : m;
-            my_pos += keys[e] != 0u;
-          }
+        for (int e = 0; e < V; ++e) {
+          m = keys[e] > m ? keys[e] : m;
+          my_pos += keys[e] != 0u;
         }
-        cmax[j0 + g] = m;
-        my_max = m > my_max ? m : my_max;
       }
+      cmax[j] = m;
+      my_max = m > my_max ? m : my_max;
     }
   } else {
     rr.for_each([&](int, uint32_t key) {

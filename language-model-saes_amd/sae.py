@@ -135,6 +135,10 @@ class _FusedSparseStep(torch.autograd.Function):
             grad_coef_E = torch.cat([dval, dval_aux])
             x_rows = torch.cat([x_op, x_op])
             holder.aux_code = aux_code
+        if amp:
+            # the decoder's weight gradient pairs the activations with the bf16-rounded output gradient, as the
+            # backward of an autocast matmul does; the gather of those rows then moves half the bytes
+            grad_dense_D = ops.cast_bf16(grad_dense_D.contiguous())
         holder.code, holder.pre, holder.scale, holder.l_aux = code, pre, scale, l_aux
         ctx.grad_code, ctx.x_rows, ctx.grad_dense_D, ctx.grad_coef_E = grad_code, x_rows, grad_dense_D, grad_coef_E
         ctx.grad_recon = grad_recon
