@@ -63,6 +63,10 @@ def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
         "build_feature_index": ("hbm", B * k * 16 + F * 12),
         "cast_f32_to_bf16": ("hbm", B * d * 6),
         "col_sum": ("hbm", B * d * 4),
+        "sparse_rows_grad_sq_nnz": ("hbm", B * k * d * 2 + B * k * 12 + F * 24),  # gathered bf16 rows (cache hits), index, partials
+        "code_stats": ("hbm", B * k * 8 + B * 12),
+        "recon_stats": ("hbm", 2 * B * d * 4),
+        "grad_sq_nnz": ("hbm", (F + d) / 2 * 4),
         "jumprelu_fwd": ("hbm", B * F * 4),                              # bf16 pre read, bf16 acts written
         "jumprelu_bwd": ("hbm", B * F * 6),                              # bf16 pre and d_acts read, bf16 d_pre written
     }
@@ -112,6 +116,30 @@ def build_topk(pkg, dev, args):
                       overlap_decoder_update=args.overlap)
     name = f"topk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} fp32-master/bf16-operands adam"
     return _autocast_step(sae, batch, opt, {}), B, name, (B, d, F, k)
+
+
+def build_topk_trainer(pkg, dev, args):
+    """The headline shape driven through `Trainer.train_one_step`: the step plus what the reference's loop
+    adds around it every step (gradient norm over all parameters, the eight logging metrics, LR schedule)."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = args.batch or 4096, D_MODEL, D_SAE, TOP_K
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
+                        dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, 64, seed=4).to(dev)
+    _init_sae_on_device(sae, x, d)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    tcfg = pkg.TrainerConfig(lr=4e-4, total_training_tokens=B * 1_000_000, amp_dtype=torch.bfloat16, l1_coefficient=None,
+                             skip_metrics_calculation=False, log_frequency=1000, clip_grad_norm=args.clip, k_warmup_steps=0,
+                             lr_warm_up_steps=100)
+    trainer = pkg.Trainer(tcfg)
+    trainer.prepare(sae, batch)
+    name = (f"topk_sae Trainer.train_one_step d_model={d} d_sae={F} k={k} batch={B} fp32-master/bf16-operands adam, "
+            f"grad norm + metrics every step, clip_grad_norm={args.clip}")
+    return (lambda: trainer.train_one_step(sae, batch)["loss"]), B, name, (B, d, F, k)
 
 
 class _FixedDead:
@@ -220,7 +248,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "topk_trainer": build_topk_trainer, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
@@ -303,6 +331,7 @@ def main():
     ap.add_argument("--cpu-sample-features", type=int, default=32768)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
+    ap.add_argument("--clip", type=float, default=0.0, help="clip_grad_norm of the topk_trainer workload (0: norm only)")
     ap.add_argument("--overlap", action="store_true", help="run the decoder Adam pass on a second stream, overlapping the next GEMM")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -319,14 +348,14 @@ def main():
         achieved, peak, unit = per_launch / avg_ms / 1e9, PEAK_BF16_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = per_launch / avg_ms / 1e6, PEAK_HBM_GBS, "GB/s"
-    traffic = HBM_TRAFFIC_GB.get(dominant) if args.workload == "topk" else None
+    traffic = HBM_TRAFFIC_GB.get(dominant) if args.workload in ("topk", "topk_trainer") else None
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
         "frac": round(achieved / peak, 4), "traffic": None if traffic is None else traffic * 1e9, "avg_ms": round(avg_ms, 4),
         "launches_per_step": kernels[dominant]["calls"] / args.steps,
     }
     per_kernel = {}
-    uniform = args.workload in ("topk", "batchtopk", "jumprelu")     # one dictionary shape for every launch
+    uniform = args.workload in ("topk", "topk_trainer", "batchtopk", "jumprelu")     # one dictionary shape for every launch
     for kname, st in kernels.items():
         bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None

@@ -206,14 +206,16 @@ int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, doubl
  * consumed at once; no dense gradient is stored.  Same update rule, scalars and by-products
  * (shadow_bf16, row_norm_out) as sae_adam_step; bias_grad_out (nullable) receives
  * sum_{s in segment f} coef[s], the gradient of the per-feature bias.  Bit-identical to
- * sae_sparse_grad_rows followed by sae_adam_step.
+ * sae_sparse_grad_rows followed by sae_adam_step.  grad_scale (nullable): device float[1]; the
+ * row gradient and bias_grad_out are multiplied by it before use, which is clip_grad_norm's
+ * `grad.mul_(factor)` (optim.py:280-292) with the factor left on the device.
  * Replaces loss.backward()'s dense `f^T @ grad` / `x^T @ dh` GEMMs together with
  * torch.optim.Adam.step for W_D / W_E (trainer.py:627-647). */
 int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
                               const float *coef, const void *dense, int dense_dtype, float *p, float *m,
                               float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                               double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                              float *bias_grad_out, void *stream);
+                              float *bias_grad_out, const float *grad_scale, void *stream);
 
 /* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
  * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and
@@ -230,6 +232,45 @@ int sae_sparse_adam_step(float *p, const float *g, float *m, float *v, int64_t n
  * cleared by the caller before the first tensor).  The two quantities behind
  * compute_grad_norm (optim.py:257-277): ||g|| / sqrt(#non-zero). */
 int sae_grad_sq_nnz(const float *g, int64_t n, double *acc, void *stream);
+
+int64_t sae_sparse_rows_grad_sq_nnz_workspace_bytes(int64_t F);
+
+/* The same two sums for a weight gradient held in factored form (see sae_adam_step_sparse_rows): every
+ * feature's row is rebuilt in registers and reduced, the dense gradient is never stored.  This is what
+ * the trainer's every-step clip_grad_norm / grad-norm diagnostic (trainer.py:629-639, optim.py:257-292)
+ * needs from W_E and W_D.  acc as in sae_grad_sq_nnz (accumulated into, in a fixed order);
+ * bias_grad_out (nullable) receives sum_{s in segment f} coef[s]; workspace: device memory of
+ * sae_sparse_rows_grad_sq_nnz_workspace_bytes(F) bytes, 16-byte aligned. */
+int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                const float *coef, const void *dense, int dense_dtype, int64_t F, int64_t d,
+                                double *acc, float *bias_grad_out, void *workspace, int64_t workspace_bytes,
+                                void *stream);
+
+/* ---- Training metrics from the sparse code ----------------------------------------------------------
+ * The per-step quantities behind FrequencyMetric, MeanFeatureActMetric and L0Metric (metrics.py:102-127,
+ * 189-204, 258-288), which the reference computes from the dense [B, F] feature_acts:
+ *   freq_acc[f] += sum_b w_b [acts[b, f] > 0]        (act_freq_scores; w_b = tok_w[b], 1 when tok_w is NULL)
+ *   l0_tok[b]    = #{f : acts[b, f] > 0}             (nullable)
+ *   totals[0]   += sum of all kept values            (feature_acts.sum())
+ *   totals[1]   += #{(b, f) : acts[b, f] > 0}        (feature_acts.gt(0).sum(), unmasked as in the reference)
+ *   totals[2]   += sum_b w_b l0_tok[b]               (the masked L0 sum)
+ * idx / val / row_off / row_nnz: a sparse code as the select kernels emit it.  freq_acc (float[F], nullable)
+ * and totals (double[3], nullable) are accumulated into, so a running sum over steps needs no extra pass. */
+int sae_code_stats(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
+                   const float *tok_w, int64_t B, int64_t F, float *freq_acc, float *l0_tok, double *totals,
+                   void *stream);
+
+/* ExplainedVarianceMetric and L2NormErrorMetric (metrics.py:207-255, 291-314) from label / recon [B, d] fp32 and the
+ * (masked) column mean of label:  with se_b = |recon_b - label_b|^2, var_b = |label_b - mean|^2 and
+ * <.> = sum_b w_b (.) / sum_b w_b,
+ *   acc[0] += 1 - <se> / <var>         explained_variance
+ *   acc[1] += <1 - se / var>           explained_variance_legacy
+ *   acc[2] += <sqrt(se)>               l2_norm_error
+ *   acc[3] += <sqrt(se)> / <|label|>   l2_norm_error_ratio
+ * acc: device double[4], accumulated into; step_out (nullable): device float[4], this step's values;
+ * tok_workspace: device float[3 B]. */
+int sae_recon_stats(const float *label, const float *recon, const float *label_mean, const float *tok_w,
+                    int64_t B, int64_t d, float *tok_workspace, double *acc, float *step_out, void *stream);
 
 /* ---- JumpReLU with straight-through threshold gradient --------------------------------------------
  * Replaces STEFunction / JumpReLU (activation_functions.py:15-140) as the SAE encoder applies it

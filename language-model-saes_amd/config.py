@@ -76,6 +76,43 @@ class SparseDictionaryConfig(BaseModelConfig):
     def d_sae(self) -> int:
         return int(self.d_model * self.expansion_factor)
 
+    @classmethod
+    def from_pretrained(cls, pretrained_name_or_path: str, strict_loading: bool = True, **kwargs):
+        """Read `<path>/config.json` as the reference writes it (models/sparse_dictionary.py:156-186) and build
+        the config class its `sae_type` names; `kwargs` (device, dtype, ...) override the file.  A path to a
+        weights file stands for its directory.  Hub names are not resolved here."""
+        import json
+        import os
+
+        root = pretrained_name_or_path
+        if os.path.isfile(root):
+            root = os.path.dirname(root)
+            if os.path.basename(root) == "checkpoints" and not os.path.exists(os.path.join(root, "config.json")):
+                root = os.path.dirname(root)
+        path = os.path.join(root, "config.json")
+        if not os.path.exists(path):
+            raise FileNotFoundError(f"no config.json under {root!r} (only local directories are supported)")
+        with open(path, "r") as f:
+            d = json.load(f)
+        d["sae_pretrained_name_or_path"] = pretrained_name_or_path
+        d["strict_loading"] = strict_loading
+        if cls is SparseDictionaryConfig:
+            cls = SAE_TYPE_TO_CONFIG_CLASS[d["sae_type"]]
+        return cls.model_validate({**d, **kwargs})
+
+    def save_hyperparameters(self, sae_path, remove_loading_info: bool = True) -> None:
+        """Write `<sae_path>/config.json` (models/sparse_dictionary.py:188-196)."""
+        import json
+        import os
+
+        assert os.path.exists(sae_path), f"{sae_path} does not exist. Unable to save hyperparameters."
+        d = self.model_dump()
+        if remove_loading_info:
+            d.pop("sae_pretrained_name_or_path", None)
+            d.pop("strict_loading", None)
+        with open(os.path.join(sae_path, "config.json"), "w") as f:
+            json.dump(d, f, indent=4)
+
     @property
     def associated_hook_points(self) -> list[str]:
         raise NotImplementedError

@@ -139,9 +139,11 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
     float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
-    uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad) {
+    uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad,
+    const float *__restrict__ grad_scale) {
   __shared__ float red[4];
   const int f = blockIdx.x, tid = threadIdx.x;
+  const float gs = grad_scale ? grad_scale[0] : 1.f;
   const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
   const int n_seg = d >> 2;
   const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     float s = 0.f;
     for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
     s = wave_sum(s);
-    if (tid == 0) bias_grad[f] = s;
+    if (tid == 0) bias_grad[f] = grad_scale ? s * gs : s;
   }
 
   float sq = 0.f;
@@ -194,6 +196,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < 4; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
+        if (grad_scale) { g[u].x *= gs; g[u].y *= gs; g[u].z *= gs; g[u].w *= gs; }
         adam_one(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_one(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
         adam_one(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_one(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
         store_stream(p, base4 + seg, pp[u]);
@@ -222,7 +225,7 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
                                          const float *coef, const void *dense, int dense_dtype, float *p, float *m,
                                          float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                                          double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                                         float *bias_grad_out, void *stream) {
+                                         float *bias_grad_out, const float *grad_scale, void *stream) {
   using namespace sae;
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: null pointer");
@@ -242,10 +245,10 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
   hipStream_t st = (hipStream_t)stream;
   if (dense_dtype == SAE_BF16)
     hipLaunchKernelGGL(adam_sparse_rows_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale);
   else
     hipLaunchKernelGGL(adam_sparse_rows_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale);
   return check_launch("adam_step_sparse_rows");
 }
 
@@ -334,6 +337,127 @@ extern "C" int sae_sparse_adam_step(float *p, const float *g, float *m, float *v
                      (float)eps, step_state, flag_workspace, reinterpret_cast<uint16_t *>(shadow_bf16));
   hipLaunchKernelGGL(sparse_adam_advance_kernel, dim3(1), dim3(64), 0, st, step_state, flag_workspace);
   return check_launch("sparse_adam_step");
+}
+
+namespace sae {
+
+// One workgroup per feature: rebuilds the feature's gradient row exactly as adam_sparse_rows_kernel does
+// (same accumulation order, so the same bits) and reduces sum g^2 and #(g != 0) into partial[2 f], partial[2 f + 1].
+template <bool DENSE_BF16>
+__global__ __launch_bounds__(256) void sparse_rows_sq_nnz_kernel(
+    const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot, const int32_t *__restrict__ slot_tok,
+    const float *__restrict__ coef, const void *__restrict__ dense, int d, double *__restrict__ partial,
+    float *__restrict__ bias_grad) {
+  __shared__ double red[8];
+  const int f = blockIdx.x, tid = threadIdx.x;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  if (bias_grad && tid < 64) {
+    float s = 0.f;
+    for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
+    s = wave_sum(s);
+    if (tid == 0) bias_grad[f] = s;
+  }
+  if (lo == hi) {  // no token used this feature: the row gradient is exactly zero
+    if (tid == 0) { partial[2 * (size_t)f] = 0.0; partial[2 * (size_t)f + 1] = 0.0; }
+    return;
+  }
+  const int n_seg = d >> 2;
+  const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
+  const char *dbase = reinterpret_cast<const char *>(dense);
+  double sq = 0.0;
+  int nz = 0;
+  for (int seg0 = tid; seg0 < n_seg; seg0 += 256 * 4) {
+    float4 g[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) g[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = lo; i < hi; ++i) {
+      const int s = feat_slot[i];
+      const float c = coef[s];
+      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int seg = seg0 + u * 256;
+        if (seg < n_seg) {
+          float4 x;
+          if constexpr (DENSE_BF16) {
+            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
+            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
+            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
+          } else {
+            x = reinterpret_cast<const float4 *>(row)[seg];
+          }
+          g[u].x = fmaf(c, x.x, g[u].x); g[u].y = fmaf(c, x.y, g[u].y);
+          g[u].z = fmaf(c, x.z, g[u].z); g[u].w = fmaf(c, x.w, g[u].w);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float s4 = g[u].x * g[u].x;   // a 4-element fp32 partial keeps the fp64 adds off the critical path
+      s4 = fmaf(g[u].y, g[u].y, s4); s4 = fmaf(g[u].z, g[u].z, s4); s4 = fmaf(g[u].w, g[u].w, s4);
+      sq += (double)s4;
+      nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
+    }
+  }
+  double cnt = (double)nz;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { sq += __shfl_xor(sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
+  const int lane = tid & 63, w = tid >> 6;
+  if (lane == 0) { red[w] = sq; red[4 + w] = cnt; }
+  __syncthreads();
+  if (tid == 0) {
+    partial[2 * (size_t)f] = red[0] + red[1] + red[2] + red[3];
+    partial[2 * (size_t)f + 1] = red[4] + red[5] + red[6] + red[7];
+  }
+}
+
+// acc[0] += sum of partial[2 f], acc[1] += sum of partial[2 f + 1], in a fixed order (one workgroup)
+__global__ __launch_bounds__(1024) void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc) {
+  __shared__ double red[32];
+  double sq = 0.0, cnt = 0.0;
+  for (int64_t f = threadIdx.x; f < F; f += 1024) { sq += partial[2 * f]; cnt += partial[2 * f + 1]; }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { sq += __shfl_xor(sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) { red[w] = sq; red[16 + w] = cnt; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double a = 0.0, b = 0.0;
+    for (int i = 0; i < 16; ++i) { a += red[i]; b += red[16 + i]; }
+    acc[0] += a;
+    acc[1] += b;
+  }
+}
+
+}  // namespace sae
+
+extern "C" int64_t sae_sparse_rows_grad_sq_nnz_workspace_bytes(int64_t F) { return F > 0 ? 16 * F : 0; }
+
+extern "C" int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                           const float *coef, const void *dense, int dense_dtype, int64_t F, int64_t d,
+                                           double *acc, float *bias_grad_out, void *workspace, int64_t workspace_bytes,
+                                           void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && acc && workspace, SAE_ERR_INVALID_ARG,
+              "sparse_rows_grad_sq_nnz: null pointer");
+  SAE_REQUIRE(F > 0 && d > 0, SAE_ERR_INVALID_ARG, "sparse_rows_grad_sq_nnz: bad sizes");
+  SAE_REQUIRE(dense_dtype == SAE_F32 || dense_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "sparse_rows_grad_sq_nnz: bad dtype %d", dense_dtype);
+  SAE_REQUIRE(d % 4 == 0 && F < (1LL << 31) && d < (1LL << 31), SAE_ERR_UNSUPPORTED,
+              "sparse_rows_grad_sq_nnz: d_model=%lld must be a multiple of 4", (long long)d);
+  SAE_REQUIRE((((uintptr_t)dense | (uintptr_t)workspace) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "sparse_rows_grad_sq_nnz: 16-byte alignment required");
+  SAE_REQUIRE(workspace_bytes >= 16 * F, SAE_ERR_INVALID_ARG, "sparse_rows_grad_sq_nnz: workspace of %lld bytes, %lld needed",
+              (long long)workspace_bytes, (long long)(16 * F));
+  hipStream_t st = (hipStream_t)stream;
+  double *partial = reinterpret_cast<double *>(workspace);
+  if (dense_dtype == SAE_BF16)
+    hipLaunchKernelGGL(sparse_rows_sq_nnz_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, coef,
+                       dense, (int)d, partial, bias_grad_out);
+  else
+    hipLaunchKernelGGL(sparse_rows_sq_nnz_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, coef,
+                       dense, (int)d, partial, bias_grad_out);
+  hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, acc);
+  return check_launch("sparse_rows_grad_sq_nnz");
 }
 
 extern "C" int sae_grad_sq_nnz(const float *g, int64_t n, double *acc, void *stream) {

@@ -413,8 +413,9 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
 def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, p: torch.Tensor, m: torch.Tensor,
                           v: torch.Tensor, *, lr: float, beta1: float, beta2: float, eps: float, step: int,
                           shadow_bf16: Optional[torch.Tensor] = None, row_norm_out: Optional[torch.Tensor] = None,
-                          bias_grad_out: Optional[torch.Tensor] = None) -> None:
-    """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense)."""
+                          bias_grad_out: Optional[torch.Tensor] = None, grad_scale: Optional[torch.Tensor] = None) -> None:
+    """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense);
+    `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping)."""
     for name, t in (("p", p), ("m", m), ("v", v)):
         _req(t, name, torch.float32, 2)
     _req(coef, "coef", torch.float32, 1)
@@ -426,13 +427,35 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
         raise ValueError("feature index was built for a different number of features")
     if shadow_bf16 is not None:
         _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
+    if grad_scale is not None:
+        _req(grad_scale, "grad_scale", torch.float32)
     with _timed("adam_step_sparse_rows[bf16 dense]" if dense.dtype == torch.bfloat16 else "adam_step_sparse_rows[f32 dense]"):
         check(
             _lib.load().sae_adam_step_sparse_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
                                                   coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),
                                                   v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step), _ptr(shadow_bf16),
-                                                  _ptr(row_norm_out), _ptr(bias_grad_out), _stream(p)),
+                                                  _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale), _stream(p)),
             "adam_step_sparse_rows",
+        )
+
+
+def sparse_rows_grad_sq_nnz(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, acc: torch.Tensor,
+                            bias_grad_out: Optional[torch.Tensor] = None) -> None:
+    """acc (device double[2]) += (sum of squares, number of non-zero entries) of the [F, d] gradient that
+    (fi, coef, dense) stand for; optionally writes the per-feature bias gradient as well."""
+    _req(coef, "coef", torch.float32, 1)
+    _req(dense, "dense", ndim=2)
+    _req(acc, "acc", torch.float64, 1)
+    F, d = fi.feat_ptr.numel() - 1, dense.shape[1]
+    lib = _lib.load()
+    nbytes = lib.sae_sparse_rows_grad_sq_nnz_workspace_bytes(F)
+    ws = torch.empty(nbytes // 8, dtype=torch.float64, device=dense.device)
+    with _timed("sparse_rows_grad_sq_nnz"):
+        check(
+            lib.sae_sparse_rows_grad_sq_nnz(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
+                                            coef.data_ptr(), dense.data_ptr(), _dt(dense), F, d, acc.data_ptr(),
+                                            _ptr(bias_grad_out), ws.data_ptr(), nbytes, _stream(dense)),
+            "sparse_rows_grad_sq_nnz",
         )
 
 
@@ -520,3 +543,55 @@ def jumprelu_bwd(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Option
                                    d_bias.data_ptr(), d_theta.data_ptr(), _ptr(d_scale), ws.data_ptr(), ws_bytes,
                                    _stream(pre)), "jumprelu_bwd")
     return d_pre, d_bias, d_theta, d_scale
+
+
+def code_stats(code: SparseCode, tok_w: Optional[torch.Tensor] = None, freq_acc: Optional[torch.Tensor] = None,
+               totals: Optional[torch.Tensor] = None, want_l0: bool = False) -> Optional[torch.Tensor]:
+    """Activation statistics of a sparse code without densifying it: `freq_acc` (float [F]) += per-feature
+    count of (masked) tokens with a positive activation; `totals` (double [3]) += (sum of values, number of
+    positive values, masked number of positive values); returns the per-token L0 when asked for."""
+    _req(code.idx, "code.idx", torch.int32)
+    _req(code.val, "code.val", torch.float32)
+    if tok_w is not None:
+        _req(tok_w, "tok_w", torch.float32, 1)
+        if tok_w.numel() != code.n_tokens:
+            raise ValueError("tok_w must hold one weight per token")
+    if freq_acc is not None:
+        _req(freq_acc, "freq_acc", torch.float32, 1)
+        if freq_acc.numel() != code.d_sae:
+            raise ValueError("freq_acc must hold one entry per feature")
+    if totals is not None:
+        _req(totals, "totals", torch.float64, 1)
+    l0 = torch.empty(code.n_tokens, dtype=torch.float32, device=code.val.device) if want_l0 else None
+    with _timed("code_stats"):
+        check(
+            _lib.load().sae_code_stats(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(),
+                                       _ptr(tok_w), code.n_tokens, code.d_sae, _ptr(freq_acc), _ptr(l0), _ptr(totals),
+                                       _stream(code.val)),
+            "code_stats",
+        )
+    return l0
+
+
+def recon_stats(label: torch.Tensor, recon: torch.Tensor, label_mean: torch.Tensor, acc: torch.Tensor,
+                tok_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """acc (double [4]) += this step's (explained variance, legacy explained variance, L2 error, L2 error
+    ratio); returns the step's four values (float [4])."""
+    _req(label, "label", torch.float32, 2)
+    _req(recon, "recon", torch.float32, 2)
+    _req(label_mean, "label_mean", torch.float32, 1)
+    _req(acc, "acc", torch.float64, 1)
+    B, d = label.shape
+    if recon.shape != label.shape or label_mean.numel() != d or acc.numel() < 4:
+        raise ValueError("shape mismatch")
+    if tok_w is not None:
+        _req(tok_w, "tok_w", torch.float32, 1)
+    ws = torch.empty(3 * B, dtype=torch.float32, device=label.device)
+    out = torch.empty(4, dtype=torch.float32, device=label.device)
+    with _timed("recon_stats"):
+        check(
+            _lib.load().sae_recon_stats(label.data_ptr(), recon.data_ptr(), label_mean.data_ptr(), _ptr(tok_w), B, d,
+                                        ws.data_ptr(), acc.data_ptr(), out.data_ptr(), _stream(label)),
+            "recon_stats",
+        )
+    return out

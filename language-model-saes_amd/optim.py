@@ -155,12 +155,13 @@ class HipAdam(Optimizer):
                     self._side_stream = torch.cuda.Stream(device=p.device)
                 side = self._side_stream
                 side.wait_stream(torch.cuda.current_stream(p.device))
-                for t in (sg.fi.feat_ptr, sg.fi.feat_slot, sg.fi.slot_tok, sg.coef, sg.dense_operand):
-                    t.record_stream(side)  # step-local tensors: keep their memory until the side stream is done
+                for t in (sg.fi.feat_ptr, sg.fi.feat_slot, sg.fi.slot_tok, sg.coef, sg.dense_operand, sg.scale):
+                    if t is not None:
+                        t.record_stream(side)  # step-local tensors: keep their memory until the side stream is done
             with torch.cuda.stream(side) if side is not None else _null_ctx():
                 ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
                                           eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
-                                          row_norm_out=norm_out, bias_grad_out=bias_out)
+                                          row_norm_out=norm_out, bias_grad_out=bias_out, grad_scale=sg.scale)
                 if side is not None:
                     ev = torch.cuda.Event()
                     ev.record(side)
@@ -243,21 +244,62 @@ class HipSparseAdam(Optimizer):
         return loss
 
 
+def _grad_sq_nnz(params) -> torch.Tensor:
+    """device double[2] = (sum g^2, #non-zero g) over dense `.grad`s and factored weight gradients alike.
+    A factored gradient is reduced by a kernel that rebuilds its rows in registers; the bias gradient it
+    carries is produced on the way and becomes an ordinary `.grad` (so it is counted, clipped and stepped
+    like any other).  The two sums of a factored gradient are cached on it: the second norm of a step (the
+    after-clipping diagnostic) costs nothing."""
+    params = list(params)
+    acc = None
+    for p in params:
+        sg = getattr(p, "_sparse_grad", None)
+        if sg is None:
+            continue
+        if acc is None:
+            acc = torch.zeros(2, dtype=torch.float64, device=p.device)
+        if sg.sq_nnz is None:
+            own = torch.zeros(2, dtype=torch.float64, device=p.device)
+            bias_out = None
+            if sg.bias_param is not None:
+                bias_out = torch.empty(sg.n_features, dtype=torch.float32, device=p.device)
+            ops.sparse_rows_grad_sq_nnz(sg.fi, sg.coef, sg.dense_operand, own, bias_grad_out=bias_out)
+            if bias_out is not None:
+                bp = sg.bias_param
+                bp.grad = bias_out if bp.grad is None else bp.grad + bias_out
+                sg.bias_param = None
+            sg.sq_nnz = own
+        own = sg.sq_nnz
+        if sg.scale is not None:
+            own = own * torch.stack([sg.scale.double().square().reshape(()), torch.ones((), dtype=torch.float64, device=p.device)])
+        acc += own
+    dense = [p.grad for p in params if p.grad is not None]
+    if dense:
+        d = ops.grad_sq_nnz(dense)
+        acc = d if acc is None else acc + d
+    assert acc is not None, "No gradients found"
+    return acc
+
+
 def compute_grad_norm(params) -> torch.Tensor:
     """||g||_2 over all gradients divided by sqrt(number of non-zero gradient entries)
-    (src/llamascopium/optim.py:257-277), as a device scalar.  Factored gradients must be materialised first."""
-    grads = [p.grad for p in params if p.grad is not None]
-    acc = ops.grad_sq_nnz(grads)
+    (src/llamascopium/optim.py:257-277), as a device scalar.  Dense and factored gradients both count."""
+    acc = _grad_sq_nnz(params)
     return (acc[0].sqrt() / acc[1].sqrt()).to(torch.float32)
 
 
 def clip_grad_norm(params, max_norm: float) -> torch.Tensor:
     """src/llamascopium/optim.py:280-292 without the host round trip: gradients are scaled by
-    max_norm / (norm + 1e-6) when the norm exceeds max_norm, decided on the device."""
-    params = [p for p in params if p.grad is not None]
+    max_norm / (norm + 1e-6) when the norm exceeds max_norm, decided on the device.  A factored weight
+    gradient is not rewritten: the factor is attached to it and applied where its rows are formed."""
+    params = list(params)   # not filtered yet: a bias gradient carried by a factored weight gradient appears below
     norm = compute_grad_norm(params)
     if max_norm != float("inf"):
         factor = torch.where(norm > max_norm, max_norm / (norm + 1e-6), torch.ones_like(norm))
         for p in params:
-            p.grad.mul_(factor)
+            if p.grad is not None:
+                p.grad.mul_(factor)
+            sg = getattr(p, "_sparse_grad", None)
+            if sg is not None:
+                sg.scale = factor.reshape(1) if sg.scale is None else sg.scale * factor
     return norm

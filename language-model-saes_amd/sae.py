@@ -56,11 +56,18 @@ class SparseRowGrad:
     def __init__(self, fi: ops.FeatureIndex, coef: torch.Tensor, dense_operand: torch.Tensor, n_features: int,
                  bias_param: Optional[torch.Tensor] = None):
         self.fi, self.coef, self.dense_operand, self.n_features, self.bias_param = fi, coef, dense_operand, n_features, bias_param
+        self.scale: Optional[torch.Tensor] = None    # device float[1] from gradient clipping, applied where rows are formed
+        self.sq_nnz: Optional[torch.Tensor] = None   # cached (sum g^2, #non-zero) of the unscaled rows
 
     def dense(self):
         """(rows [F, d] fp32, bias gradient [F] or None)"""
-        return ops.sparse_grad_rows(self.fi, self.coef, self.dense_operand, self.n_features,
-                                    want_bias=self.bias_param is not None)
+        rows, bias = ops.sparse_grad_rows(self.fi, self.coef, self.dense_operand, self.n_features,
+                                          want_bias=self.bias_param is not None)
+        if self.scale is not None:
+            rows.mul_(self.scale)
+            if bias is not None:
+                bias.mul_(self.scale)
+        return rows, bias
 
 
 class _FusedSparseStep(torch.autograd.Function):

@@ -20,6 +20,9 @@ from .activation_functions import JumpReLU, batch_topk_dense, topk_dense
 from .config import SAE_TYPE_TO_MODEL_CLASS, SparseDictionaryConfig
 
 
+CHECKPOINT_VERSION = "lm-saes-amd-1"
+
+
 def apply_token_mask(t: torch.Tensor, n_token_dims: int, mask: Optional[torch.Tensor], reduction: str = "sum"):
     """Reduce the leading token dims (batch[, context]) of `t`, optionally weighted by a 0/1 mask.
     Same results as utils/tensor_specs.py:64-84."""
@@ -165,6 +168,25 @@ class SparseDictionary(nn.Module):
         return {k: v / scale_factors[k] for k, v in batch.items()}
 
     # ---- optimiser groups (sparse_dictionary.py:501-510) ----
+    def log_statistics(self) -> dict[str, Any]:
+        """models/sparse_dictionary.py:698-711: weight-norm means, the current k, the mean JumpReLU threshold."""
+        out: dict[str, Any] = {}
+        if hasattr(self, "encoder_norm") and hasattr(self, "decoder_norm"):
+            with torch.no_grad():
+                out["metrics/encoder_norm"] = self.encoder_norm().mean().item()
+                out["metrics/decoder_norm"] = self.decoder_norm().mean().item()
+                if self.cfg.use_decoder_bias and hasattr(self, "decoder_bias_norm"):
+                    out["metrics/decoder_bias_norm"] = self.decoder_bias_norm().mean().item()
+        if "topk" in self.cfg.act_fn:
+            out["sparsity/k"] = self.current_k
+        if isinstance(self.activation_function, JumpReLU):
+            out["metrics/mean_jumprelu_threshold"] = self.activation_function.log_jumprelu_threshold.detach().exp().mean().item()
+        return out
+
+    def compute_training_metrics(self, **kwargs) -> dict[str, float]:
+        """Model-specific training metrics (models/sparse_dictionary.py:1029-1039); none for the base class."""
+        return {}
+
     def get_parameters(self) -> list[dict[str, Any]]:
         jr = list(self.activation_function.parameters()) if isinstance(self.activation_function, JumpReLU) else []
         others = [p for p in self.parameters() if not any(p is q for q in jr)]
@@ -193,7 +215,86 @@ class SparseDictionary(nn.Module):
     def from_config(cls, cfg: SparseDictionaryConfig, device_mesh=None):
         if cls is SparseDictionary:
             cls = SAE_TYPE_TO_MODEL_CLASS[cfg.sae_type]
+        if cfg.sae_pretrained_name_or_path is not None:
+            return cls.from_pretrained(cfg.sae_pretrained_name_or_path, strict_loading=cfg.strict_loading,
+                                       device=cfg.device, dtype=cfg.dtype)
         return cls(cfg, device_mesh)
+
+    # ---- checkpoint files in the reference's format (sparse_dictionary.py:280-331, 558-665) ----
+    @torch.no_grad()
+    def save_checkpoint(self, ckpt_path) -> None:
+        """`.safetensors`: the full state dict (reference key names and shapes, W_E as [d_model, d_sae]
+        row-major, plus the `dataset_average_activation_norm.*` scalars) with a `version` metadata entry;
+        `.pt`: `{"sae": state_dict, "version": ...}`."""
+        import os
+
+        sd = {k: v.detach().contiguous() for k, v in self.full_state_dict().items()}
+        suffix = os.path.splitext(str(ckpt_path))[1]
+        if suffix == ".safetensors":
+            import safetensors.torch as safe
+
+            safe.save_file({k: v.cpu() for k, v in sd.items()}, str(ckpt_path), {"version": CHECKPOINT_VERSION})
+        elif suffix == ".pt":
+            torch.save({"sae": sd, "version": CHECKPOINT_VERSION}, str(ckpt_path))
+        else:
+            raise ValueError(f"Invalid checkpoint path {ckpt_path}. Currently only supports .safetensors and .pt formats.")
+
+    @torch.no_grad()
+    def save_pretrained(self, save_path, fold_activation_scale: bool = False) -> None:
+        import os
+
+        os.makedirs(str(save_path), exist_ok=True)
+        if fold_activation_scale:
+            assert hasattr(self, "standardize_parameters_of_dataset_norm"), (
+                f"{type(self).__name__} does not support dataset norm standardization")
+            self.standardize_parameters_of_dataset_norm()
+        self.save_checkpoint(os.path.join(str(save_path), "sae_weights.safetensors"))
+
+    @classmethod
+    def from_local(cls, path: str, device_mesh=None, strict_loading: bool = True, fold_activation_scale: bool = False,
+                   **kwargs):
+        """Load `<path>/config.json` and the first weights file found in the reference's priority order
+        (sae_weights, checkpoints/pruned, checkpoints/final; safetensors before pt); `path` may also name
+        a weights file directly.  The `.pt` form is read with `weights_only=True`."""
+        import os
+
+        path = str(path)
+        cfg = SparseDictionaryConfig.from_pretrained(path, strict_loading=strict_loading, **kwargs)
+        cfg.sae_pretrained_name_or_path = None
+        model = cls.from_config(cfg, device_mesh=device_mesh)
+        if path.endswith((".pt", ".safetensors")):
+            ckpt_path = path
+        else:
+            for rel in ("sae_weights.safetensors", "sae_weights.pt", "checkpoints/pruned.safetensors", "checkpoints/pruned.pt",
+                        "checkpoints/final.safetensors", "checkpoints/final.pt"):
+                ckpt_path = os.path.join(path, rel)
+                if os.path.exists(ckpt_path):
+                    break
+            else:
+                raise FileNotFoundError(f"Pretrained model not found at {path}")
+        if ckpt_path.endswith(".safetensors"):
+            import safetensors.torch as safe
+
+            state_dict = safe.load_file(ckpt_path, device=cfg.device)
+        else:
+            state_dict = torch.load(ckpt_path, map_location=cfg.device, weights_only=True)["sae"]
+        model.load_full_state_dict(state_dict, strict=strict_loading)
+        if fold_activation_scale:
+            assert hasattr(model, "standardize_parameters_of_dataset_norm"), (
+                f"{type(model).__name__} does not support dataset norm standardization")
+            model.standardize_parameters_of_dataset_norm()
+        return model
+
+    @classmethod
+    def from_pretrained(cls, pretrained_name_or_path: str, *, device_mesh=None, fold_activation_scale: bool = False,
+                        strict_loading: bool = True, **kwargs):
+        """Local directories and files only: hub repositories and SAELens names are outside this path."""
+        import os
+
+        if not os.path.exists(str(pretrained_name_or_path)):
+            raise ValueError(f"{pretrained_name_or_path!r} is not a local path; hub downloads are not part of this library")
+        return cls.from_local(str(pretrained_name_or_path), device_mesh=device_mesh, strict_loading=strict_loading,
+                              fold_activation_scale=fold_activation_scale, **kwargs)
 
     # ---- to be provided by subclasses ----
     def encode(self, x, return_hidden_pre: bool = False, **kwargs):

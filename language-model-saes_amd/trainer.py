@@ -19,6 +19,7 @@ from torch.optim import lr_scheduler
 
 from . import ops
 from .config import TorchDtype
+from .metrics import default_metrics
 from .optim import HipAdam, HipSparseAdam, clip_grad_norm
 from .sparse_dictionary import SparseDictionary, apply_token_mask
 
@@ -107,6 +108,9 @@ class Trainer:
         self.scheduler = None
         self.tokens_since_last_activation: Optional[torch.Tensor] = None
         self.is_dead: Optional[torch.Tensor] = None
+        self.metrics: list = []
+        self.log_sink: Optional[Callable[[int, dict], None]] = None   # receives (step, metrics) every log_frequency steps
+        self.last_logged: Optional[dict] = None
 
     # ---- trainer.py:310-346 ----
     def _initialize_trainer(self, sae: SparseDictionary, first_batch: dict):
@@ -204,6 +208,32 @@ class Trainer:
             frequency_scale=self.cfg.frequency_scale, k_aux=self.cfg.k_aux,
             update_dead_statistics=self.update_dead_statistics if auxk > 0.0 else None)
 
+    # ---- trainer.py:512-562 ----
+    @torch.no_grad()
+    def _log(self, sae: SparseDictionary, ctx: dict) -> None:
+        """Update every metric with this step's context; every `log_frequency` steps reduce them to
+        numbers (the only host synchronisation of the logging path) and hand them to `log_sink`."""
+        if not self.metrics:
+            self.metrics = default_metrics(sae)
+        for metric in self.metrics:
+            ctx.update(metric.update(ctx))
+        if (self.cur_step + 1) % self.cfg.log_frequency == 0:
+            out: dict = {}
+            for metric in self.metrics:
+                out.update(metric.compute())
+            out.update({
+                "details/current_learning_rate": self.optimizer.param_groups[0]["lr"],
+                "details/n_training_tokens": self.cur_tokens,
+                "details/l1_coefficient": ctx.get("l1_coefficient"),
+                "details/lp_coefficient": ctx.get("lp_coefficient"),
+                "details/auxk_coefficient": ctx.get("auxk_coefficient"),
+            })
+            if hasattr(sae, "log_statistics"):
+                out.update(sae.log_statistics())
+            self.last_logged = out
+            if self.log_sink is not None:
+                self.log_sink(self.cur_step + 1, out)
+
     # ---- trainer.py:576-671 (loop body; no progress bar, files or wandb) ----
     def fit(self, sae: SparseDictionary, activation_stream: Iterable[dict],
             on_step: Optional[Callable[[int, dict], None]] = None) -> Optional[bool]:
@@ -212,39 +242,48 @@ class Trainer:
             batch = next(stream)
         except StopIteration:
             return True
-        if self.optimizer is None:
-            self._initialize_trainer(sae, batch)
-            self._initialize_optimizer(sae)
-        if self.cfg.auxk_coefficient is not None and self.cfg.auxk_coefficient > 0.0 and self.is_dead is None:
-            self._initialize_dead_statistics(sae)
-        device_type = next(sae.parameters()).device.type
+        self.prepare(sae, batch)
         try:
             while True:
-                batch = sae.normalize_activations(batch)
-                sae.train()
-                if self.cfg.amp_dtype is not None and self.cfg.amp_dtype != torch.float32:
-                    with torch.autocast(device_type=device_type, dtype=self.cfg.amp_dtype):
-                        ctx = self._training_step(sae, batch)
-                else:
-                    ctx = self._training_step(sae, batch)
-                ctx["loss"].backward()
-                if not self.cfg.skip_metrics_calculation or self.cfg.clip_grad_norm > 0:
-                    # the reference computes this every step; it needs element-wise gradients
-                    if hasattr(self.optimizer, "materialize_grads"):
-                        self.optimizer.materialize_grads()
-                    ctx["grad_norm_before_clipping"] = clip_grad_norm(
-                        [p for n, p in sae.named_parameters() if p.grad is not None and "log_jumprelu_threshold" not in n],
-                        max_norm=self.cfg.clip_grad_norm if self.cfg.clip_grad_norm > 0 else math.inf)
-                if on_step is not None:
-                    on_step(self.cur_step, ctx)
-                self.optimizer.step()
-                self.optimizer.zero_grad()
-                self.scheduler.step()
-                self.cur_step += 1
-                self.cur_tokens += batch["tokens"].numel() if batch.get("mask") is None else int(batch["mask"].sum().item())
+                self.train_one_step(sae, batch, on_step)
                 if self.cur_step >= self.total_training_steps:
                     break
                 batch = next(stream)
         except StopIteration:
             return True
         return None
+
+    def prepare(self, sae: SparseDictionary, first_batch: dict) -> None:
+        """What `fit` sets up before its first step: step counts, optimizer, scheduler, dead statistics."""
+        if self.optimizer is None:
+            self._initialize_trainer(sae, first_batch)
+            self._initialize_optimizer(sae)
+        if self.cfg.auxk_coefficient is not None and self.cfg.auxk_coefficient > 0.0 and self.is_dead is None:
+            self._initialize_dead_statistics(sae)
+
+    def train_one_step(self, sae: SparseDictionary, batch: dict,
+                       on_step: Optional[Callable[[int, dict], None]] = None) -> dict:
+        """The body of the reference's loop (trainer.py:605-660) for one batch."""
+        batch = sae.normalize_activations(batch)
+        sae.train()
+        if self.cfg.amp_dtype is not None and self.cfg.amp_dtype != torch.float32:
+            with torch.autocast(device_type=next(sae.parameters()).device.type, dtype=self.cfg.amp_dtype):
+                ctx = self._training_step(sae, batch)
+        else:
+            ctx = self._training_step(sae, batch)
+        ctx["loss"].backward()
+        # every step, as the reference does (trainer.py:629-639); factored weight gradients are
+        # reduced where they are, nothing dense is materialised; the jumprelu threshold is excluded
+        ctx["grad_norm_before_clipping"] = clip_grad_norm(
+            [p for n, p in sae.named_parameters() if "log_jumprelu_threshold" not in n],
+            max_norm=self.cfg.clip_grad_norm if self.cfg.clip_grad_norm > 0 else math.inf)
+        if not self.cfg.skip_metrics_calculation:
+            self._log(sae, ctx)
+        if on_step is not None:
+            on_step(self.cur_step, ctx)
+        self.optimizer.step()
+        self.optimizer.zero_grad()
+        self.scheduler.step()
+        self.cur_step += 1
+        self.cur_tokens += batch["tokens"].numel() if batch.get("mask") is None else int(batch["mask"].sum().item())
+        return ctx
