@@ -246,6 +246,17 @@ int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slo
                                 double *acc, float *bias_grad_out, void *workspace, int64_t workspace_bytes,
                                 void *stream);
 
+/* ---- Activation batches from a shuffle buffer -----------------------------------------------------------
+ * dst[i, :] = cast(scale * src[row_idx[i], :]) for i < n_rows: one batch drawn from a token buffer that
+ * stays where it is in HBM.  Replaces ActivationBuffer.shuffle / yield_batch
+ * (activation/processors/activation.py:96-164), which permute and re-concatenate the whole buffer for every
+ * refill and every batch; here a shuffle permutes indices only and a batch is this one gather, with the
+ * dtype override (activation/processors/activation.py:397-410) and a normalisation factor folded in.
+ * src: [n_src_rows, d], dst: [n_rows, d], SAE_F32 or SAE_BF16 each; row_idx: device int64[n_rows], every
+ * entry in [0, n_src_rows) (an entry outside leaves its output row untouched). */
+int sae_gather_rows(const void *src, int src_dtype, const int64_t *row_idx, int64_t n_src_rows, int64_t n_rows,
+                    int64_t d, void *dst, int dst_dtype, double scale, void *stream);
+
 /* ---- Training metrics from the sparse code ----------------------------------------------------------
  * The per-step quantities behind FrequencyMetric, MeanFeatureActMetric and L0Metric (metrics.py:102-127,
  * 189-204, 258-288), which the reference computes from the dense [B, F] feature_acts:

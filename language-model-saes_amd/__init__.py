@@ -28,3 +28,14 @@ from .clt import CrossLayerTranscoder  # noqa: E402,F401
 from .lorsa import LowRankSparseAttention  # noqa: E402,F401
 
 __all__ += ["CrosscoderConfig", "CLTConfig", "LorsaConfig", "Crosscoder", "CrossLayerTranscoder", "LowRankSparseAttention"]
+
+from . import metrics  # noqa: E402,F401
+from .activation import (  # noqa: E402,F401
+    ActivationBatchler, ActivationTransformer, ActivationWriter, ActivationWriterConfig, BufferShuffleConfig,
+    CachedActivationLoader, ChunkInfo, cached_activation_stream,
+)
+from .initializer import Initializer, InitializerConfig, calculate_activation_norm  # noqa: E402,F401
+
+__all__ += ["metrics", "ActivationBatchler", "ActivationTransformer", "ActivationWriter", "ActivationWriterConfig",
+            "BufferShuffleConfig", "CachedActivationLoader", "ChunkInfo", "cached_activation_stream", "Initializer",
+            "InitializerConfig", "calculate_activation_norm"]

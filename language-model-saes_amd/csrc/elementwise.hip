@@ -97,7 +97,81 @@ __global__ __launch_bounds__(256) void col_sum_final_kernel(const float *__restr
   out[j] = accumulate ? out[j] + s : s;
 }
 
+// dst[i, :] = cast(scale * src[row_idx[i], :]).  One workgroup per output row, 8 elements per thread per
+// trip (16-byte loads from bf16 rows, 2 x 16 from fp32 rows); rows whose byte length is not a multiple of
+// 16 take the element-wise tail path for the whole row.
+template <bool SRC_BF16, bool DST_BF16>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const void *__restrict__ src, const int64_t *__restrict__ row_idx,
+                                                          int64_t n_src_rows, int d, void *__restrict__ dst, float scale) {
+  const int64_t i = blockIdx.x;
+  const int64_t r = row_idx[i];
+  if (r < 0 || r >= n_src_rows) return;   // the host validates indices it generated; a foreign index writes nothing
+  const size_t s_es = SRC_BF16 ? 2 : 4, d_es = DST_BF16 ? 2 : 4;
+  const char *srow = reinterpret_cast<const char *>(src) + (size_t)r * d * s_es;
+  char *drow = reinterpret_cast<char *>(dst) + (size_t)i * d * d_es;
+  const bool vec = (d & 7) == 0 && ((reinterpret_cast<uintptr_t>(srow) | reinterpret_cast<uintptr_t>(drow)) & 15) == 0;
+  if (vec) {
+    for (int c = threadIdx.x; c < (d >> 3); c += 256) {
+      float v[8];
+      if constexpr (SRC_BF16) {
+        const u32x4 q = reinterpret_cast<const u32x4 *>(srow)[c];
+        v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+        v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+        v[4] = __uint_as_float(q.z << 16); v[5] = __uint_as_float(q.z & 0xffff0000u);
+        v[6] = __uint_as_float(q.w << 16); v[7] = __uint_as_float(q.w & 0xffff0000u);
+      } else {
+        const float4 a = reinterpret_cast<const float4 *>(srow)[2 * c], b = reinterpret_cast<const float4 *>(srow)[2 * c + 1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+      }
+      if (scale != 1.f) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= scale;
+      }
+      if constexpr (DST_BF16) {
+        u32x4 o;
+        o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+        o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+        o.z = (uint32_t)f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
+        o.w = (uint32_t)f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+        reinterpret_cast<u32x4 *>(drow)[c] = o;
+      } else {
+        reinterpret_cast<float4 *>(drow)[2 * c] = make_float4(v[0], v[1], v[2], v[3]);
+        reinterpret_cast<float4 *>(drow)[2 * c + 1] = make_float4(v[4], v[5], v[6], v[7]);
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < d; c += 256) {
+      float x = SRC_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(srow)[c]) : reinterpret_cast<const float *>(srow)[c];
+      if (scale != 1.f) x *= scale;
+      if constexpr (DST_BF16) reinterpret_cast<uint16_t *>(drow)[c] = f32_to_bf16_bits(x);
+      else reinterpret_cast<float *>(drow)[c] = x;
+    }
+  }
+}
+
 }  // namespace sae
+
+extern "C" int sae_gather_rows(const void *src, int src_dtype, const int64_t *row_idx, int64_t n_src_rows, int64_t n_rows,
+                               int64_t d, void *dst, int dst_dtype, double scale, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(src && row_idx && dst, SAE_ERR_INVALID_ARG, "gather_rows: null pointer");
+  SAE_REQUIRE(n_rows > 0 && d > 0 && n_src_rows > 0 && d < (1LL << 31) && n_rows < (1LL << 31), SAE_ERR_INVALID_ARG,
+              "gather_rows: bad sizes");
+  SAE_REQUIRE((src_dtype == SAE_F32 || src_dtype == SAE_BF16) && (dst_dtype == SAE_F32 || dst_dtype == SAE_BF16),
+              SAE_ERR_INVALID_ARG, "gather_rows: bad dtype %d -> %d", src_dtype, dst_dtype);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)n_rows), block(256);
+  const float sc = (float)scale;
+  if (src_dtype == SAE_BF16 && dst_dtype == SAE_BF16)
+    hipLaunchKernelGGL((gather_rows_kernel<true, true>), grid, block, 0, st, src, row_idx, n_src_rows, (int)d, dst, sc);
+  else if (src_dtype == SAE_BF16)
+    hipLaunchKernelGGL((gather_rows_kernel<true, false>), grid, block, 0, st, src, row_idx, n_src_rows, (int)d, dst, sc);
+  else if (dst_dtype == SAE_BF16)
+    hipLaunchKernelGGL((gather_rows_kernel<false, true>), grid, block, 0, st, src, row_idx, n_src_rows, (int)d, dst, sc);
+  else
+    hipLaunchKernelGGL((gather_rows_kernel<false, false>), grid, block, 0, st, src, row_idx, n_src_rows, (int)d, dst, sc);
+  return check_launch("gather_rows");
+}
 
 extern "C" int sae_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {
   using namespace sae;

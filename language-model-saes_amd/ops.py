@@ -595,3 +595,27 @@ def recon_stats(label: torch.Tensor, recon: torch.Tensor, label_mean: torch.Tens
             "recon_stats",
         )
     return out
+
+
+def gather_rows(src: torch.Tensor, row_idx: torch.Tensor, out_dtype: Optional[torch.dtype] = None, scale: float = 1.0,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i] = cast(scale * src[row_idx[i]]) for a [N, d] fp32 / bf16 buffer and int64 row indices."""
+    _req(src, "src", ndim=2)
+    _req(row_idx, "row_idx", torch.int64, 1)
+    out_dtype = out_dtype or src.dtype
+    n, d = row_idx.numel(), src.shape[1]
+    if out is None:
+        out = torch.empty(n, d, dtype=out_dtype, device=src.device)
+    else:
+        _req(out, "out", out_dtype, 2)
+        if tuple(out.shape) != (n, d):
+            raise ValueError("out has the wrong shape")
+    if n == 0:
+        return out
+    with _timed("gather_rows"):
+        check(
+            _lib.load().sae_gather_rows(src.data_ptr(), _dt(src), row_idx.data_ptr(), src.shape[0], n, d, out.data_ptr(), _dt(out),
+                                        float(scale), _stream(src)),
+            "gather_rows",
+        )
+    return out

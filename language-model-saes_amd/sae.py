@@ -351,6 +351,13 @@ class SparseAutoEncoder(SparseDictionary):
         self.W_E.copy_(self.W_D.t() * factor)
 
     @torch.no_grad()
+    def init_encoder_bias_with_mean_hidden_pre(self, batch: dict[str, torch.Tensor]):
+        """models/sae.py:511-515."""
+        x = self.prepare_input(batch)[0]
+        _, hidden_pre = self.encode(x, return_hidden_pre=True)
+        self.b_E.sub_(hidden_pre.mean(dim=0).to(self.b_E.dtype))
+
+    @torch.no_grad()
     def init_parameters(self, **kwargs):
         """models/sae.py:400-436: uniform encoder/decoder, zero biases."""
         super().init_parameters(**kwargs)
