@@ -67,6 +67,7 @@ def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
         "code_stats": ("hbm", B * k * 8 + B * 12),
         "recon_stats": ("hbm", 2 * B * d * 4),
         "grad_sq_nnz": ("hbm", (F + d) / 2 * 4),
+        "gather_rows": ("hbm", B * d * 6),                               # fp32 rows read, bf16 rows written
         "jumprelu_fwd": ("hbm", B * F * 4),                              # bf16 pre read, bf16 acts written
         "jumprelu_bwd": ("hbm", B * F * 6),                              # bf16 pre and d_acts read, bf16 d_pre written
     }
@@ -140,6 +141,25 @@ def build_topk_trainer(pkg, dev, args):
     name = (f"topk_sae Trainer.train_one_step d_model={d} d_sae={F} k={k} batch={B} fp32-master/bf16-operands adam, "
             f"grad norm + metrics every step, clip_grad_norm={args.clip}")
     return (lambda: trainer.train_one_step(sae, batch)["loss"]), B, name, (B, d, F, k)
+
+
+def build_activation_stream(pkg, dev, args):
+    """Not a train step: one batch drawn from the shuffling batchler (4096 tokens of d_model=4096, fp32 rows in a
+    131072-token HBM buffer, handed out as bf16), refills and shuffles included."""
+    import torch
+
+    B, d, chunk = args.batch or 4096, D_MODEL, 32768
+    src = torch.randn(chunk, d, device=dev)
+
+    def chunks():
+        while True:
+            yield {"in": src, "tokens": torch.zeros(chunk, dtype=torch.long, device=dev)}
+
+    batchler = pkg.ActivationBatchler(B, buffer_size=131072, buffer_shuffle_config=pkg.BufferShuffleConfig(),
+                                      override_dtype=torch.bfloat16)
+    it = batchler.process(chunks())
+    name = f"activation_batchler batch={B} d_model={d} buffer=131072 tokens fp32 -> bf16"
+    return (lambda: next(it)["in"].sum()), B, name, (B, d, D_SAE, TOP_K)
 
 
 class _FixedDead:
@@ -248,7 +268,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "topk_trainer": build_topk_trainer, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
@@ -355,7 +375,7 @@ def main():
         "launches_per_step": kernels[dominant]["calls"] / args.steps,
     }
     per_kernel = {}
-    uniform = args.workload in ("topk", "topk_trainer", "batchtopk", "jumprelu")     # one dictionary shape for every launch
+    uniform = args.workload in ("topk", "topk_trainer", "batchtopk", "jumprelu", "activation_stream")     # one dictionary shape for every launch
     for kname, st in kernels.items():
         bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None

@@ -308,8 +308,13 @@ class _RowStore:
             bigger[: self.data.shape[0]] = self.data
             self.data = bigger
 
-    def put(self, rows: torch.Tensor, first: int) -> None:
-        self.data[first:first + rows.shape[0]] = rows
+    def put(self, rows: torch.Tensor, slots_host: torch.Tensor) -> None:
+        n = rows.shape[0]
+        first = int(slots_host[0])
+        if int(slots_host[-1]) - first == n - 1:      # slots are handed out ascending: contiguous means a plain slice
+            self.data[first:first + n] = rows
+        else:
+            self.data.index_copy_(0, slots_host.to(self.data.device), rows.to(self.data.dtype))
 
     def take(self, idx_host: torch.Tensor, out_dtype: Optional[torch.dtype], scale: float) -> torch.Tensor:
         d = self.data
@@ -347,45 +352,25 @@ class ActivationBatchler:
         stores: dict[str, _RowStore] = {}
         lists: dict[str, list] = {}          # non-tensor fields travel in arrival order (no shuffling with them)
         order = torch.empty(0, dtype=torch.int64)   # slab rows in logical order
-        free: list[tuple[int, int]] = []     # free slab ranges [first, last)
+        free = torch.empty(0, dtype=torch.int64)    # slab rows not in use, ascending
         capacity = 0
 
-        def alloc(n: int) -> int:
-            """First row of a free range of n slab rows (the slabs grow when none is large enough)."""
-            nonlocal capacity
-            for j, (a, b) in enumerate(free):
-                if b - a >= n:
-                    free[j] = (a + n, b)
-                    if free[j][0] == free[j][1]:
-                        free.pop(j)
-                    return a
-            first = capacity
-            capacity = capacity + max(n, capacity // 2, self.buffer_size or 0, self.batch_size)
-            for s in stores.values():
-                s.grow(capacity)
-            if capacity - (first + n) > 0:
-                free.append((first + n, capacity))
-            return first
+        def alloc(n: int) -> torch.Tensor:
+            """n free slab rows, ascending (the slabs grow when too few are free)."""
+            nonlocal capacity, free
+            if free.numel() < n:
+                grown = capacity + max(n - free.numel(), capacity // 2, self.buffer_size or 0, self.batch_size)
+                for s in stores.values():
+                    s.grow(grown)
+                free = torch.cat([free, torch.arange(capacity, grown, dtype=torch.int64)])
+                capacity = grown
+            slots, free = free[:n], free[n:]
+            return slots
 
         def release(rows: torch.Tensor) -> None:
-            if rows.numel() == 0:
-                return
-            r = rows.sort().values.tolist()
-            start = prev = r[0]
-            for x in r[1:]:
-                if x != prev + 1:
-                    free.append((start, prev + 1))
-                    start = x
-                prev = x
-            free.append((start, prev + 1))
-            free.sort()
-            merged: list[tuple[int, int]] = []
-            for a, b in free:
-                if merged and merged[-1][1] == a:
-                    merged[-1] = (merged[-1][0], b)
-                else:
-                    merged.append((a, b))
-            free[:] = merged
+            nonlocal free
+            if rows.numel():
+                free = torch.cat([free, rows]).sort().values
 
         def take(n: int) -> dict[str, Any]:
             nonlocal order
@@ -405,13 +390,13 @@ class ActivationBatchler:
                 for k, v in tensors.items():
                     if k not in stores:
                         stores[k] = _RowStore(v, capacity)
-                first = alloc(n)
+                slots = alloc(n)
                 for k, v in tensors.items():
-                    stores[k].put(v, first)
+                    stores[k].put(v, slots)
                 for k, v in d.items():
                     if not isinstance(v, torch.Tensor):
                         lists.setdefault(k, []).extend(v)
-                order = torch.cat([order, torch.arange(first, first + n, dtype=torch.int64)])
+                order = torch.cat([order, slots])
             if self.buffer_size is not None:
                 if order.numel() >= self.buffer_size:
                     assert not lists, "All data must be tensors to perform shuffling"
