@@ -415,7 +415,16 @@ __global__ __launch_bounds__(256) void sparse_rows_sq_nnz_kernel(
 __global__ __launch_bounds__(1024) void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc) {
   __shared__ double red[32];
   double sq = 0.0, cnt = 0.0;
-  for (int64_t f = threadIdx.x; f < F; f += 1024) { sq += partial[2 * f]; cnt += partial[2 * f + 1]; }
+  // four independent 16-byte loads in flight per thread; the order of the additions is fixed by the indexing
+  typedef __attribute__((ext_vector_type(2))) double f64x2;
+  const f64x2 *pairs = reinterpret_cast<const f64x2 *>(partial);
+  int64_t f = threadIdx.x;
+  for (; f + 3 * 1024 < F; f += 4 * 1024) {
+    const f64x2 a = pairs[f], b = pairs[f + 1024], c = pairs[f + 2048], d = pairs[f + 3072];
+    sq += (a[0] + b[0]) + (c[0] + d[0]);
+    cnt += (a[1] + b[1]) + (c[1] + d[1]);
+  }
+  for (; f < F; f += 1024) { const f64x2 a = pairs[f]; sq += a[0]; cnt += a[1]; }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) { sq += __shfl_xor(sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;

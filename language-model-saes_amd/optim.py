@@ -12,6 +12,7 @@ kernel scales by: both are by-products of data already in registers.
 
 from __future__ import annotations
 
+import weakref
 from typing import Optional
 
 import torch
@@ -248,16 +249,14 @@ def _grad_sq_nnz(params) -> torch.Tensor:
     """device double[2] = (sum g^2, #non-zero g) over dense `.grad`s and factored weight gradients alike.
     A factored gradient is reduced by a kernel that rebuilds its rows in registers; the bias gradient it
     carries is produced on the way and becomes an ordinary `.grad` (so it is counted, clipped and stepped
-    like any other).  The two sums of a factored gradient are cached on it: the second norm of a step (the
-    after-clipping diagnostic) costs nothing."""
+    like any other).  The sums are cached (on the factored gradient; on a dense gradient tensor together with
+    its version counter): the second norm of a step, the after-clipping diagnostic, launches almost nothing."""
     params = list(params)
-    acc = None
+    parts = []
     for p in params:
         sg = getattr(p, "_sparse_grad", None)
         if sg is None:
             continue
-        if acc is None:
-            acc = torch.zeros(2, dtype=torch.float64, device=p.device)
         if sg.sq_nnz is None:
             own = torch.zeros(2, dtype=torch.float64, device=p.device)
             bias_out = None
@@ -271,14 +270,27 @@ def _grad_sq_nnz(params) -> torch.Tensor:
             sg.sq_nnz = own
         own = sg.sq_nnz
         if sg.scale is not None:
-            own = own * torch.stack([sg.scale.double().square().reshape(()), torch.ones((), dtype=torch.float64, device=p.device)])
-        acc += own
+            own = torch.stack([own[0] * sg.scale.double().square().reshape(()), own[1]])
+        parts.append(own)
     dense = [p.grad for p in params if p.grad is not None]
     if dense:
-        d = ops.grad_sq_nnz(dense)
-        acc = d if acc is None else acc + d
-    assert acc is not None, "No gradients found"
-    return acc
+        parts.append(_dense_sq_nnz(dense))
+    assert parts, "No gradients found"
+    return parts[0] if len(parts) == 1 else torch.stack(parts).sum(0)
+
+
+_dense_cache: dict = {"refs": (), "versions": (), "sums": None}
+
+
+def _dense_sq_nnz(grads) -> torch.Tensor:
+    """Joint (sum g^2, #non-zero) of a list of dense gradients, remembered while the same tensor objects
+    stay unmodified (weak references and version counters decide)."""
+    refs, versions = _dense_cache["refs"], _dense_cache["versions"]
+    if len(refs) == len(grads) and all(r() is g and v == g._version for r, v, g in zip(refs, versions, grads)):
+        return _dense_cache["sums"]
+    sums = ops.grad_sq_nnz(grads)
+    _dense_cache.update(refs=tuple(weakref.ref(g) for g in grads), versions=tuple(g._version for g in grads), sums=sums)
+    return sums
 
 
 def compute_grad_norm(params) -> torch.Tensor:

@@ -154,12 +154,24 @@ class SparseDictionary(nn.Module):
             assert self.dataset_average_activation_norm is not None, (
                 "dataset_average_activation_norm must be provided from Initializer"
             )
-            return torch.tensor(math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[hook_point],
-                                device=x.device, dtype=x.dtype)
-        return torch.tensor(1.0, device=x.device, dtype=x.dtype)
+            return self._scalar(math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[hook_point], x)
+        return self._scalar(1.0, x)
+
+    def _scalar(self, value: float, like: torch.Tensor) -> torch.Tensor:
+        """0-dim tensor of `value` on like's device in like's dtype, built once (a host-to-device copy per call otherwise)."""
+        cache = self.__dict__.setdefault("_scalar_cache", {})
+        key = (value, like.device, like.dtype)
+        t = cache.get(key)
+        if t is None:
+            if len(cache) > 64:
+                cache.clear()
+            t = cache[key] = torch.tensor(value, device=like.device, dtype=like.dtype)
+        return t
 
     def normalize_activations(self, batch: dict[str, torch.Tensor], *, return_scale_factor: bool = False):
         hooks = self.cfg.associated_hook_points
+        if self.cfg.norm_activation == "inference" and not return_scale_factor:
+            return dict(batch)    # every factor is the constant 1: no pass over the activations
         scale = {k: self.compute_norm_factor(v, hook_point=k) for k, v in batch.items() if k in hooks}
         out = {k: (v * scale[k] if k in scale else v) for k, v in batch.items()}
         return (out, scale) if return_scale_factor else out
