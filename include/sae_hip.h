@@ -209,13 +209,18 @@ int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, doubl
  * sae_sparse_grad_rows followed by sae_adam_step.  grad_scale (nullable): device float[1]; the
  * row gradient and bias_grad_out are multiplied by it before use, which is clip_grad_norm's
  * `grad.mul_(factor)` (optim.py:280-292) with the factor left on the device.
+ * grad_sq_nnz_acc (nullable): device double[2]; sum g^2 and #(g != 0) of the gradient this call consumes are
+ * added to it (the sums of sae_sparse_rows_grad_sq_nnz, as a by-product: the every-step gradient-norm
+ * diagnostic of trainer.py:629-639 then costs no pass of its own).  It needs `workspace`, device memory of
+ * sae_sparse_rows_grad_sq_nnz_workspace_bytes(F) bytes, 16-byte aligned; both may be NULL / 0 otherwise.
  * Replaces loss.backward()'s dense `f^T @ grad` / `x^T @ dh` GEMMs together with
  * torch.optim.Adam.step for W_D / W_E (trainer.py:627-647). */
 int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
                               const float *coef, const void *dense, int dense_dtype, float *p, float *m,
                               float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                               double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                              float *bias_grad_out, const float *grad_scale, void *stream);
+                              float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
+                              void *workspace, int64_t workspace_bytes, void *stream);
 
 /* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
  * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and

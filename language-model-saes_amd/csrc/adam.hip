@@ -134,14 +134,17 @@ extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64
 // ---------------------------------------------------------------------------------------------
 namespace sae {
 
+__global__ void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc);  // defined below
+
 template <bool DENSE_BF16>
 __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
     float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
     uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad,
-    const float *__restrict__ grad_scale) {
+    const float *__restrict__ grad_scale, double *__restrict__ sq_nnz_partial) {
   __shared__ float red[4];
+  __shared__ double red_d[8];
   const int f = blockIdx.x, tid = threadIdx.x;
   const float gs = grad_scale ? grad_scale[0] : 1.f;
   const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
@@ -158,6 +161,8 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
   }
 
   float sq = 0.f;
+  double g_sq = 0.0;
+  int g_nz = 0;
   for (int seg0 = tid; seg0 < n_seg; seg0 += 256 * 4) {
     // issue the streaming reads of p, m, v first: they are the HBM traffic; the gradient operands hit cache
     float4 pp[4], mm[4], vv[4], g[4];
@@ -197,6 +202,12 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
         if (grad_scale) { g[u].x *= gs; g[u].y *= gs; g[u].z *= gs; g[u].w *= gs; }
+        if (sq_nnz_partial) {  // the same 4-element fp32 partials as sparse_rows_sq_nnz_kernel
+          float s4 = g[u].x * g[u].x;
+          s4 = fmaf(g[u].y, g[u].y, s4); s4 = fmaf(g[u].z, g[u].z, s4); s4 = fmaf(g[u].w, g[u].w, s4);
+          g_sq += (double)s4;
+          g_nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
+        }
         adam_one(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_one(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
         adam_one(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_one(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
         store_stream(p, base4 + seg, pp[u]);
@@ -217,6 +228,18 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const float tot = block_sum<4>(sq, red);
     if (tid == 0) row_norm[f] = sqrtf(tot);
   }
+  if (sq_nnz_partial) {
+    double cnt = (double)g_nz;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { g_sq += __shfl_xor(g_sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
+    const int lane = tid & 63, w = tid >> 6;
+    if (lane == 0) { red_d[w] = g_sq; red_d[4 + w] = cnt; }
+    __syncthreads();
+    if (tid == 0) {
+      sq_nnz_partial[2 * (size_t)f] = red_d[0] + red_d[1] + red_d[2] + red_d[3];
+      sq_nnz_partial[2 * (size_t)f + 1] = red_d[4] + red_d[5] + red_d[6] + red_d[7];
+    }
+  }
 }
 
 }  // namespace sae
@@ -225,10 +248,14 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
                                          const float *coef, const void *dense, int dense_dtype, float *p, float *m,
                                          float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                                          double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                                         float *bias_grad_out, const float *grad_scale, void *stream) {
+                                         float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
+                                         void *workspace, int64_t workspace_bytes, void *stream) {
   using namespace sae;
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: null pointer");
+  SAE_REQUIRE(!grad_sq_nnz_acc || (workspace && workspace_bytes >= 16 * F && ((uintptr_t)workspace & 15) == 0),
+              SAE_ERR_WORKSPACE, "adam_step_sparse_rows: the gradient sums need an aligned workspace of %lld bytes",
+              (long long)(16 * F));
   SAE_REQUIRE(F > 0 && d > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step_sparse_rows: bad sizes / step");
   SAE_REQUIRE(dense_dtype == SAE_F32 || dense_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "adam_step_sparse_rows: bad dtype %d", dense_dtype);
   SAE_REQUIRE(d % 4 == 0 && F < (1LL << 31) && d < (1LL << 31), SAE_ERR_UNSUPPORTED,
@@ -243,12 +270,14 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(1.0 - pow(beta2, (double)step)));
   a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
+  double *partial = grad_sq_nnz_acc ? reinterpret_cast<double *>(workspace) : nullptr;
   if (dense_dtype == SAE_BF16)
     hipLaunchKernelGGL(adam_sparse_rows_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial);
   else
     hipLaunchKernelGGL(adam_sparse_rows_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial);
+  if (partial) hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, grad_sq_nnz_acc);
   return check_launch("adam_step_sparse_rows");
 }
 

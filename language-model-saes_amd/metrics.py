@@ -92,22 +92,36 @@ def _code_totals(ctx, freq_acc: Optional[torch.Tensor] = None) -> torch.Tensor:
 
 
 class GradientNormMetric(Metric):
-    """metrics.py:78-99.  Both norms stay device scalars until `compute()`."""
+    """metrics.py:78-99.  Both norms stay device scalars until `compute()`.  A norm marked as deferred in the
+    context is a tensor that the coming optimizer step fills in; it is folded into the running maxima at the
+    next call, when it holds its value (the trainer never defers on a step that reports)."""
 
     def __init__(self, sae):
         self.sae = sae
         self.gradient_norm = Record("max")
         self.gradient_norm_before_clipping = Record("max")
+        self._pending: Optional[torch.Tensor] = None
+
+    def _fold(self) -> None:
+        if self._pending is not None:
+            self.gradient_norm_before_clipping.update(self._pending)
+            self.gradient_norm.update(self._pending)
+            self._pending = None
 
     def update(self, ctx):
+        self._fold()
         before = ctx.get("grad_norm_before_clipping")
         assert before is not None, "Gradient norm before clipping must be provided"
+        if ctx.get("grad_norm_is_deferred"):
+            self._pending = before      # one value for both: nothing was clipped and no parameter was left out
+            return {"gradient_norm_per_param": before, "gradient_norm_before_clipping": before}
         self.gradient_norm_before_clipping.update(before)
         norm = compute_grad_norm(self.sae.parameters())
         self.gradient_norm.update(norm)
         return {"gradient_norm_per_param": norm, "gradient_norm_before_clipping": before}
 
     def compute(self):
+        assert self._pending is None, "a deferred gradient norm cannot be reported in the step that defers it"
         return {
             "metrics/gradient_norm_per_param": item(self.gradient_norm.compute()),
             "metrics/gradient_norm_before_clipping": item(self.gradient_norm_before_clipping.compute()),

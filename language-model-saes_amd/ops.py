@@ -413,9 +413,11 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
 def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, p: torch.Tensor, m: torch.Tensor,
                           v: torch.Tensor, *, lr: float, beta1: float, beta2: float, eps: float, step: int,
                           shadow_bf16: Optional[torch.Tensor] = None, row_norm_out: Optional[torch.Tensor] = None,
-                          bias_grad_out: Optional[torch.Tensor] = None, grad_scale: Optional[torch.Tensor] = None) -> None:
+                          bias_grad_out: Optional[torch.Tensor] = None, grad_scale: Optional[torch.Tensor] = None,
+                          grad_sq_nnz_acc: Optional[torch.Tensor] = None) -> None:
     """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense);
-    `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping)."""
+    `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping);
+    `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed."""
     for name, t in (("p", p), ("m", m), ("v", v)):
         _req(t, name, torch.float32, 2)
     _req(coef, "coef", torch.float32, 1)
@@ -429,12 +431,18 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
         _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
     if grad_scale is not None:
         _req(grad_scale, "grad_scale", torch.float32)
+    ws, ws_bytes = None, 0
+    if grad_sq_nnz_acc is not None:
+        _req(grad_sq_nnz_acc, "grad_sq_nnz_acc", torch.float64, 1)
+        ws_bytes = 16 * F
+        ws = torch.empty(2 * F, dtype=torch.float64, device=p.device)
     with _timed("adam_step_sparse_rows[bf16 dense]" if dense.dtype == torch.bfloat16 else "adam_step_sparse_rows[f32 dense]"):
         check(
             _lib.load().sae_adam_step_sparse_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
                                                   coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),
                                                   v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step), _ptr(shadow_bf16),
-                                                  _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale), _stream(p)),
+                                                  _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale),
+                                                  _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, _stream(p)),
             "adam_step_sparse_rows",
         )
 

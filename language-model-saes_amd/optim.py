@@ -66,6 +66,20 @@ class HipAdam(Optimizer):
         # outside the model must call `join()` first.
         self._overlap = bool(overlap_decoder_update) and model is not None and hasattr(model, "set_pending_update")
         self._side_stream = None
+        self._norm_request = None   # (params, out): a gradient norm to be produced as a by-product of the next step()
+
+    def deferred_grad_norm(self, params) -> torch.Tensor:
+        """`compute_grad_norm(params)` as a device scalar that the next `step()` fills in: the sums of a factored
+        weight gradient then come out of the Adam kernel that consumes it, at no extra pass.  For callers that do
+        not need the value before the step (a logged diagnostic; clipping does).  Reading the tensor before
+        `step()` has run gives garbage."""
+        params = list(params)
+        dev = next((p.device for p in params), torch.device("cuda"))
+        if self._overlap or self._norm_request is not None:
+            return compute_grad_norm(params)     # a second stream would race on the sums: take the direct route
+        out = torch.empty((), dtype=torch.float32, device=dev)
+        self._norm_request = (params, out)
+        return out
 
     def join(self) -> None:
         """Make the current stream wait for an overlapped decoder update still in flight."""
@@ -129,6 +143,11 @@ class HipAdam(Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        req, acc, wanted = self._norm_request, None, ()
+        self._norm_request = None
+        if req is not None:
+            wanted = {id(p) for p in req[0]}
+            acc = torch.zeros(2, dtype=torch.float64, device=req[1].device)
         # pass 1: weights whose gradient arrives in factored form (also yields the encoder-bias gradient)
         deferred = []
         for group in self.param_groups:
@@ -150,6 +169,13 @@ class HipAdam(Optimizer):
             bias_out = None
             if sg.bias_param is not None:
                 bias_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
+            sums_out = None
+            if id(p) in wanted:
+                if sg.sq_nnz is not None:     # already reduced by a direct norm call: reuse
+                    acc += sg.sq_nnz if sg.scale is None else torch.stack(
+                        [sg.sq_nnz[0] * sg.scale.double().square().reshape(()), sg.sq_nnz[1]])
+                else:
+                    sums_out = acc
             side = None
             if self._overlap and role == "W_D" and bias_out is None:
                 if self._side_stream is None:
@@ -162,7 +188,8 @@ class HipAdam(Optimizer):
             with torch.cuda.stream(side) if side is not None else _null_ctx():
                 ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
                                           eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
-                                          row_norm_out=norm_out, bias_grad_out=bias_out, grad_scale=sg.scale)
+                                          row_norm_out=norm_out, bias_grad_out=bias_out, grad_scale=sg.scale,
+                                          grad_sq_nnz_acc=sums_out)
                 if side is not None:
                     ev = torch.cuda.Event()
                     ev.record(side)
@@ -172,6 +199,11 @@ class HipAdam(Optimizer):
             self._publish(p, role, shadow, norm_out)
             if side is not None:
                 self._model.set_pending_update(ev)
+        if req is not None:
+            dense = [p.grad for p in req[0] if p.grad is not None]
+            if dense:
+                acc = acc + _dense_sq_nnz(dense)
+            req[1].copy_(acc[0].sqrt() / acc[1].sqrt())
         # pass 2: everything with a dense gradient
         for group in self.param_groups:
             b1, b2 = group["betas"]

@@ -272,11 +272,20 @@ class Trainer:
         else:
             ctx = self._training_step(sae, batch)
         ctx["loss"].backward()
-        # every step, as the reference does (trainer.py:629-639); factored weight gradients are
-        # reduced where they are, nothing dense is materialised; the jumprelu threshold is excluded
-        ctx["grad_norm_before_clipping"] = clip_grad_norm(
-            [p for n, p in sae.named_parameters() if "log_jumprelu_threshold" not in n],
-            max_norm=self.cfg.clip_grad_norm if self.cfg.clip_grad_norm > 0 else math.inf)
+        # every step, as the reference does (trainer.py:629-639); factored weight gradients are reduced where they
+        # are, nothing dense is materialised; the jumprelu threshold is excluded.  Without clipping the value is only
+        # logged, so it is taken as a by-product of the optimizer step (valid once `optimizer.step()` has run).
+        named = list(sae.named_parameters())
+        clipped = [p for n, p in named if "log_jumprelu_threshold" not in n]
+        reports = not self.cfg.skip_metrics_calculation and (self.cur_step + 1) % self.cfg.log_frequency == 0
+        can_defer = (self.cfg.clip_grad_norm <= 0 and hasattr(self.optimizer, "deferred_grad_norm") and not reports
+                     and on_step is None and len(clipped) == len(named))
+        if can_defer:
+            ctx["grad_norm_before_clipping"] = self.optimizer.deferred_grad_norm(clipped)
+            ctx["grad_norm_is_deferred"] = True
+        else:
+            ctx["grad_norm_before_clipping"] = clip_grad_norm(
+                clipped, max_norm=self.cfg.clip_grad_norm if self.cfg.clip_grad_norm > 0 else math.inf)
         if not self.cfg.skip_metrics_calculation:
             self._log(sae, ctx)
         if on_step is not None:

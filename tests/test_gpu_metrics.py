@@ -221,3 +221,32 @@ def test_trainer_log_matches_the_oracle_metrics(pkg, oracle, mo, dev, masked, au
             else:
                 assert got[key] == pytest.approx(v, rel=2e-3, abs=1e-6), (key, got[key], v)
         assert got["sparsity/k"] == k and "metrics/decoder_norm" in got and got["details/current_learning_rate"] > 0
+
+
+def test_deferred_grad_norm_comes_out_of_the_optimizer_step(pkg, oracle, dev):
+    """The norm produced as a by-product of HipAdam.step() equals the direct one, and the step itself is unchanged."""
+    from lm_saes_amd import synthetic
+
+    d, F, k, B = 128, 1024, 8, 96
+    x = synthetic.activations(B, d, 8, seed=41)
+    batch = {"in": x.to(dev), "out": x.to(dev), "tokens": torch.zeros(B, device=dev)}
+    results = []
+    for deferred in (False, True):
+        sae, w = _small_sae(pkg, dev, d, F, k, x, seed=41)
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=1e-3, model=sae)
+        norms = []
+        for _ in range(3):
+            sae.compute_loss(batch, return_aux_data=False).backward()
+            params = list(sae.parameters())
+            norms.append(opt.deferred_grad_norm(params) if deferred else pkg.compute_grad_norm(params))
+            opt.step(); opt.zero_grad()
+        results.append(([n.item() for n in norms], [p.detach().clone() for p in sae.parameters()]))
+    (direct, p_direct), (by_product, p_by) = results
+    for a, b in zip(direct, by_product):
+        assert b == pytest.approx(a, rel=1e-6)
+    for a, b in zip(p_direct, p_by):
+        assert torch.equal(a, b)
+    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k)
+    synthetic.load_weights(ref, *w)
+    ref.compute_loss({"in": x, "out": x, "tokens": torch.zeros(B)})["loss"].backward()
+    assert by_product[0] == pytest.approx(oracle.compute_grad_norm([p.grad for p in ref.parameters()]).item(), rel=1e-5)
