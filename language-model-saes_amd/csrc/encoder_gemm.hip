@@ -72,6 +72,15 @@ __device__ __forceinline__ void mma_chunk(const u32x4 &wf, const u32x4 &xf, f32x
   }
 }
 
+// two floats -> two bf16 (round to nearest even, NaN stays a quiet NaN) without a branch
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+  const uint32_t ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16, rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) >> 16;
+  const uint32_t ha = (ua & 0x7fffffffu) > 0x7f800000u ? ((ua >> 16) | 0x0040u) : ra;
+  const uint32_t hb = (ub & 0x7fffffffu) > 0x7f800000u ? ((ub >> 16) | 0x0040u) : rb;
+  return (ha & 0xffffu) | (hb << 16);
+}
+
 template <bool BF16_IN, bool BF16_OUT>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
@@ -193,6 +202,40 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
 
   // ---- epilogue: lane holds, per (i, j, g): 4 consecutive features of one token ----
   // D[row = feature, col = token]: token = lane % 32, feature = 8*g + 4*(lane/32) + r
+  if constexpr (BF16_OUT) {
+    // Full tiles go through LDS (free now) so that global stores are whole 128-byte lines: every wave transposes
+    // its own 128-token x 64-feature block in a private region, rows padded to 136 bytes (the 8-byte writes of a
+    // half-wave then fall on 64 distinct banks), and writes it out 8 token rows per instruction.
+    if (m0 + GEMM_BM <= M && n0 + GEMM_BN <= N && (N & 63) == 0) {
+      constexpr int PITCH = 136;
+      __builtin_amdgcn_s_barrier();  // every wave is done reading operand slabs (and its own loads have landed)
+      char *stage = lds + wave * (128 * PITCH);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            uint2 pk;
+            pk.x = pack_bf16x2(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+            pk.y = pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+            *reinterpret_cast<uint2 *>(stage + (j * 32 + frag_row) * PITCH + (i * 32 + 8 * g + 4 * frag_half) * 2) = pk;
+          }
+      // the region is private to the wave: no barrier, the compiler's wait on the LDS writes is enough
+      uint16_t *obase = reinterpret_cast<uint16_t *>(out) + (size_t)(m0 + wm * 128) * N + n0 + wn * 64;
+      const int r_in = lane >> 3, c16 = lane & 7;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = q * 8 + r_in;
+        const char *src = stage + row * PITCH + c16 * 16;
+        const uint2 lo = *reinterpret_cast<const uint2 *>(src), hi = *reinterpret_cast<const uint2 *>(src + 8);
+        u32x4 v;
+        v.x = lo.x; v.y = lo.y; v.z = hi.x; v.w = hi.y;
+        *reinterpret_cast<u32x4 *>(obase + (size_t)row * N + c16 * 8) = v;
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int tok = m0 + wm * 128 + j * 32 + frag_row;
