@@ -26,8 +26,9 @@
 // the global side: lane l fetches the logical chunk that belongs at its physical slot.
 //
 // The matrix cores compute D = Wtile * xtile^T (features along the 32 "rows" of the instruction),
-// which leaves every lane holding 4 consecutive features of one token: the epilogue packs them
-// into one 8-byte (bf16) or 16-byte (fp32) store.
+// which leaves every lane holding 4 consecutive features of one token.  For bf16 output a full tile is
+// transposed through LDS, wave by wave, and leaves as whole 128-byte lines; edge tiles and fp32 output
+// store each lane's 4 features directly (8 or 16 bytes).
 //
 // Workgroup order: consecutive ids land on the 8 XCDs round-robin; within an XCD, 32 consecutive
 // workgroups (one per CU) cover 4 token tiles x 8 feature tiles, so every slab in an XCD's L2 is
