@@ -29,7 +29,7 @@ from torch import nn
 from . import ops
 from .activation_functions import JumpReLU, _topk_mask_lowest_index, topk_dense
 from .config import CLTConfig, register_sae_model
-from .sae import _autocast_dtype
+from .sae import SparseRowGrad, SparseRowGradPieces, _autocast_dtype
 from .sparse_dictionary import LazyDict, SparseDictionary
 
 _TOPK_FAMILY = ("topk", "layertopk", "batchtopk", "batchlayertopk")
@@ -128,6 +128,8 @@ class _FusedCLTStep(torch.autograd.Function):
         holder.update(code=cat, pres=pres, norms=norms, layer_cnt=layer_cnt)
         ctx.cat, ctx.grads, ctx.dval, ctx.x_op, ctx.w_enc_op = cat, grads, dval, x_op, w_enc_op
         ctx.shape = (B, L, d, F)
+        ctx.amp = bool(amp)
+        ctx.defer_to = m if holder.get("defer") else None
         ctx.mark_non_differentiable(recon)
         return loss, recon
 
@@ -139,16 +141,33 @@ class _FusedCLTStep(torch.autograd.Function):
         fi = ops.build_feature_index(cat)
         coef_dec = cat.val * g
         coef_enc = ctx.dval * g
+        m = ctx.defer_to
+        dec_params = None if m is None else list(m.W_D)
+        defer = (m is not None and m.W_E.grad is None and getattr(m.W_E, "_sparse_grad", None) is None
+                 and all(w.grad is None and getattr(w, "_sparse_grad", None) is None for w in dec_params))
         dW_D, db_D, dW_E, db_E = [], [], [], []
+        enc_pieces = []
         for j in range(L):
             fi_j = ops.FeatureIndex(fi.feat_ptr[: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)      # features of layers <= j
+            fi_l = ops.FeatureIndex(fi.feat_ptr[j * F: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)  # features of layer j
+            db_D.append(ops.col_sum(ctx.grads[j]) * g)
+            if defer:
+                # the optimiser rebuilds the rows where it consumes them; nothing dense is written here
+                gd = ops.cast_bf16(ctx.grads[j]) if ctx.amp else ctx.grads[j]
+                dec_params[j]._sparse_grad = SparseRowGrad(fi_j, coef_dec, gd, (j + 1) * F)
+                enc_pieces.append((j * F, SparseRowGrad(fi_l, coef_enc, ctx.x_op[j], F)))
+                dW_D.append(None)
+                continue
             rows, _ = ops.sparse_grad_rows(fi_j, coef_dec, ctx.grads[j], (j + 1) * F)
             dW_D.append(rows.view(j + 1, F, d))
-            db_D.append(ops.col_sum(ctx.grads[j]) * g)
-            fi_l = ops.FeatureIndex(fi.feat_ptr[j * F: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)  # features of layer j
             rows_e, bias_e = ops.sparse_grad_rows(fi_l, coef_enc, ctx.x_op[j], F, want_bias=True)
             dW_E.append(rows_e); db_E.append(bias_e)
-        dW_E = torch.stack(dW_E).permute(0, 2, 1)                       # [L, F, d] buffer seen as [L, d, F]
+        if defer:
+            m.W_E._sparse_grad = SparseRowGradPieces(enc_pieces, L * F, bias_param=m.b_E)
+            dW_E = db_E = None
+        else:
+            dW_E = torch.stack(dW_E).permute(0, 2, 1)                   # [L, F, d] buffer seen as [L, d, F]
+            db_E = torch.stack(db_E)
         dx = dlabel = None
         if ctx.needs_input_grad[0]:
             # d x[:, l] = sum over layer l's kept entries of d(pre) * W_E[l][:, f]
@@ -161,7 +180,7 @@ class _FusedCLTStep(torch.autograd.Function):
             dx = torch.stack(parts, dim=1)
         if ctx.needs_input_grad[1]:
             dlabel = -torch.stack(ctx.grads, dim=0) * g
-        return (dx, dlabel, None, None, dW_E, torch.stack(db_E), *dW_D, *db_D)
+        return (dx, dlabel, None, None, dW_E, db_E, *dW_D, *db_D)
 
 
 @register_sae_model("clt")
@@ -176,6 +195,9 @@ class CrossLayerTranscoder(SparseDictionary):
         self.W_D = nn.ParameterList([nn.Parameter(torch.empty(i + 1, F, d, **kw)) for i in range(L)])
         self.b_D = nn.ParameterList([nn.Parameter(torch.empty(d, **kw)) for _ in range(L)])
         self._norm_cache: Optional[tuple[tuple[int, ...], torch.Tensor]] = None
+        # set by an optimiser that consumes factored gradients (HipAdam): the fused backward then attaches them to
+        # W_E / W_D[j] as `_sparse_grad` instead of writing dense gradient rows
+        self.defer_weight_grads = False
 
     # ---- activations (clt.py:232-387): the selection scope depends on the name ----
     def activation_function_factory(self, device_mesh=None):
@@ -359,7 +381,7 @@ class CrossLayerTranscoder(SparseDictionary):
         n_tokens = (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item()))
         if self._fused_eligible(x, sparsity_loss_type):
             amp = _autocast_dtype("cuda") == torch.bfloat16
-            holder: dict[str, Any] = {"model": self}
+            holder: dict[str, Any] = {"model": self, "defer": self.defer_weight_grads and torch.is_grad_enabled()}
             xin = x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x
             loss, recon = _FusedCLTStep.apply(xin, label.to(torch.float32), amp, holder, self.W_E, self.b_E,
                                               *self.W_D, *self.b_D)

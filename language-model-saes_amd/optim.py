@@ -45,6 +45,21 @@ def _flat_view(p: torch.Tensor) -> torch.Tensor:
     return p if order == tuple(range(p.ndim)) else p.permute(order)
 
 
+def _grad_like(p: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """A [rows, d] gradient of p's contiguous storage, viewed with p's shape and strides."""
+    order = _flat_order(p)
+    g = rows.view([p.shape[i] for i in order])
+    inv = [0] * len(order)
+    for pos, dim in enumerate(order):
+        inv[dim] = pos
+    return g.permute(inv)
+
+
+def _pieces(sg):
+    """(first_row, SparseRowGrad) pairs of a factored gradient, single or in row blocks."""
+    return sg.pieces if hasattr(sg, "pieces") else [(0, sg)]
+
+
 class HipAdam(Optimizer):
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, model=None,
                  defer_weight_grads: bool = True, overlap_decoder_update: bool = False):
@@ -56,7 +71,10 @@ class HipAdam(Optimizer):
         if model is not None:
             for name in ("W_E", "W_D"):
                 p = getattr(model, name, None)
-                if p is not None:
+                if isinstance(p, torch.nn.ParameterList):
+                    for j, q in enumerate(p):
+                        self._roles[id(q)] = f"{name}.{j}"
+                elif p is not None:
                     self._roles[id(p)] = name
             if defer_weight_grads and hasattr(model, "defer_weight_grads"):
                 model.defer_weight_grads = True
@@ -103,9 +121,9 @@ class HipAdam(Optimizer):
                 if sg is None:
                     continue
                 rows, bias = sg.dense()
-                p.grad = rows if p.is_contiguous() else rows.t()
+                p.grad = _grad_like(p, rows)
                 if bias is not None:
-                    sg.bias_param.grad = bias
+                    sg.bias_param.grad = bias.view(sg.bias_param.shape)
                 p._sparse_grad = None
 
     def _state(self, p):
@@ -137,6 +155,48 @@ class HipAdam(Optimizer):
             if norm_out is not None:
                 self._model.set_derived("W_D.norm", p, norm_out)
 
+    def _step_row_blocks(self, group, p, sg, st, pv, mv, vv, acc) -> None:
+        """A weight whose [rows, d] view is updated block by block (a cross-layer transcoder's stacked layers):
+        one kernel per block with a factored gradient, a plain zero-gradient Adam pass over rows no block covers."""
+        b1, b2 = group["betas"]
+        d = pv.shape[-1]
+        p2, m2, v2 = pv.reshape(-1, d), mv.reshape(-1, d), vv.reshape(-1, d)
+        role = self._roles.get(id(p))
+        shadow = self._model.get_derived_buffer(f"{role}.bf16") if role is not None else None
+        if shadow is not None and (shadow.numel() != p2.numel() or shadow.dtype != torch.bfloat16):
+            shadow = None
+        sh2 = shadow.view(-1, d) if shadow is not None else None
+        bias_param = getattr(sg, "bias_param", None)
+        bias_buf = torch.zeros(p2.shape[0], dtype=torch.float32, device=p.device) if bias_param is not None else None
+        step = int(st["step"].item())
+        covered = 0
+        for r0, piece in sorted(_pieces(sg), key=lambda rp: rp[0]):
+            n = piece.n_features
+            if r0 != covered:
+                raise NotImplementedError("row blocks of a factored gradient must tile the parameter")
+            sums_out = None
+            if acc is not None:
+                if piece.sq_nnz is not None:
+                    acc += piece.sq_nnz if piece.scale is None else torch.stack(
+                        [piece.sq_nnz[0] * piece.scale.double().square().reshape(()), piece.sq_nnz[1]])
+                else:
+                    sums_out = acc
+            ops.adam_step_sparse_rows(piece.fi, piece.coef, piece.dense_operand, p2[r0:r0 + n], m2[r0:r0 + n], v2[r0:r0 + n],
+                                      lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"], step=step,
+                                      shadow_bf16=None if sh2 is None else sh2[r0:r0 + n],
+                                      bias_grad_out=None if bias_buf is None else bias_buf[r0:r0 + n],
+                                      grad_scale=piece.scale, grad_sq_nnz_acc=sums_out)
+            covered = r0 + n
+        if covered != p2.shape[0]:
+            raise NotImplementedError("row blocks of a factored gradient must tile the parameter")
+        if bias_buf is not None:
+            g = bias_buf.view(bias_param.shape)
+            bias_param.grad = g if bias_param.grad is None else bias_param.grad + g
+        p._sparse_grad = None
+        torch.autograd.graph.increment_version(p)
+        if shadow is not None:
+            self._model.set_derived(f"{role}.bf16", p, shadow)
+
     @torch.no_grad()
     def step(self, closure=None):
         loss = None
@@ -165,6 +225,9 @@ class HipAdam(Optimizer):
             st["step"] += 1
             pv = _flat_view(p)
             mv, vv = _flat_view(st["exp_avg"]), _flat_view(st["exp_avg_sq"])
+            if hasattr(sg, "pieces") or pv.ndim != 2:
+                self._step_row_blocks(group, p, sg, st, pv, mv, vv, acc if id(p) in wanted else None)
+                continue
             role, shadow, norm_out = self._by_products(p, pv)
             bias_out = None
             if sg.bias_param is not None:
@@ -255,9 +318,9 @@ class HipSparseAdam(Optimizer):
                 sg = getattr(p, "_sparse_grad", None)
                 if sg is not None:
                     rows, bias = sg.dense()
-                    p.grad = rows if p.is_contiguous() else rows.t()
+                    p.grad = _grad_like(p, rows)
                     if bias is not None:
-                        sg.bias_param.grad = bias
+                        sg.bias_param.grad = bias.view(sg.bias_param.shape)
                     p._sparse_grad = None
         for group in self.param_groups:
             b1, b2 = group["betas"]
@@ -286,24 +349,31 @@ def _grad_sq_nnz(params) -> torch.Tensor:
     params = list(params)
     parts = []
     for p in params:
-        sg = getattr(p, "_sparse_grad", None)
-        if sg is None:
+        whole = getattr(p, "_sparse_grad", None)
+        if whole is None:
             continue
-        if sg.sq_nnz is None:
-            own = torch.zeros(2, dtype=torch.float64, device=p.device)
-            bias_out = None
-            if sg.bias_param is not None:
-                bias_out = torch.empty(sg.n_features, dtype=torch.float32, device=p.device)
-            ops.sparse_rows_grad_sq_nnz(sg.fi, sg.coef, sg.dense_operand, own, bias_grad_out=bias_out)
-            if bias_out is not None:
-                bp = sg.bias_param
-                bp.grad = bias_out if bp.grad is None else bp.grad + bias_out
+        bias_param = getattr(whole, "bias_param", None)
+        bias_buf = None
+        for r0, sg in _pieces(whole):
+            if sg.sq_nnz is None:
+                own = torch.zeros(2, dtype=torch.float64, device=p.device)
+                bias_out = None
+                if bias_param is not None:
+                    if bias_buf is None:
+                        bias_buf = torch.zeros(bias_param.numel(), dtype=torch.float32, device=p.device)
+                    bias_out = bias_buf[r0:r0 + sg.n_features]
+                ops.sparse_rows_grad_sq_nnz(sg.fi, sg.coef, sg.dense_operand, own, bias_grad_out=bias_out)
+                sg.sq_nnz = own
+            own = sg.sq_nnz
+            if sg.scale is not None:
+                own = torch.stack([own[0] * sg.scale.double().square().reshape(()), own[1]])
+            parts.append(own)
+        if bias_buf is not None:
+            g = bias_buf.view(bias_param.shape)
+            bias_param.grad = g if bias_param.grad is None else bias_param.grad + g
+            whole.bias_param = None
+            for _, sg in _pieces(whole):
                 sg.bias_param = None
-            sg.sq_nnz = own
-        own = sg.sq_nnz
-        if sg.scale is not None:
-            own = torch.stack([own[0] * sg.scale.double().square().reshape(()), own[1]])
-        parts.append(own)
     dense = [p.grad for p in params if p.grad is not None]
     if dense:
         parts.append(_dense_sq_nnz(dense))
@@ -343,7 +413,8 @@ def clip_grad_norm(params, max_norm: float) -> torch.Tensor:
         for p in params:
             if p.grad is not None:
                 p.grad.mul_(factor)
-            sg = getattr(p, "_sparse_grad", None)
-            if sg is not None:
-                sg.scale = factor.reshape(1) if sg.scale is None else sg.scale * factor
+            whole = getattr(p, "_sparse_grad", None)
+            if whole is not None:
+                for _, sg in _pieces(whole):
+                    sg.scale = factor.reshape(1) if sg.scale is None else sg.scale * factor
     return norm

@@ -70,6 +70,34 @@ class SparseRowGrad:
         return rows, bias
 
 
+class SparseRowGradPieces:
+    """Factored gradient of a weight whose contiguous [rows, d] view splits into row blocks with separate
+    feature indices or dense operands (the L encoder layers of a cross-layer transcoder): `pieces` is a list
+    of (first_row, SparseRowGrad).  Rows outside every piece have zero gradient.  `bias_param` (optional) is
+    the per-row bias whose gradient the pieces carry (flat index = row)."""
+
+    def __init__(self, pieces, n_rows: int, bias_param: Optional[torch.Tensor] = None):
+        self.pieces, self.n_rows, self.bias_param = list(pieces), int(n_rows), bias_param
+
+    def dense(self):
+        """(rows [n_rows, d] fp32, bias gradient [n_rows] or None)"""
+        first = self.pieces[0][1]
+        d = first.dense_operand.shape[1]
+        rows = torch.zeros(self.n_rows, d, dtype=torch.float32, device=first.coef.device)
+        bias = torch.zeros(self.n_rows, dtype=torch.float32, device=first.coef.device) if self.bias_param is not None else None
+        for r0, sg in self.pieces:
+            want = bias is not None
+            part, b = ops.sparse_grad_rows(sg.fi, sg.coef, sg.dense_operand, sg.n_features, want_bias=want)
+            if sg.scale is not None:
+                part.mul_(sg.scale)
+                if b is not None:
+                    b.mul_(sg.scale)
+            rows[r0:r0 + sg.n_features] = part
+            if b is not None:
+                bias[r0:r0 + sg.n_features] = b
+        return rows, bias
+
+
 class _FusedSparseStep(torch.autograd.Function):
     """encode -> TopK / BatchTopK -> decode -> masked-mean squared error (+ aux-k), forward and backward,
     in kernels.
