@@ -213,6 +213,11 @@ int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, doubl
  * added to it (the sums of sae_sparse_rows_grad_sq_nnz, as a by-product: the every-step gradient-norm
  * diagnostic of trainer.py:629-639 then costs no pass of its own).  It needs `workspace`, device memory of
  * sae_sparse_rows_grad_sq_nnz_workspace_bytes(F) bytes, 16-byte aligned; both may be NULL / 0 otherwise.
+ * extra_map / extra_rows / extra_bias (nullable, the first two together): a block of gradient rows held densely,
+ * for features whose gradient is not worth factoring (the aux-k loss touches every dead feature from a large
+ * share of the tokens; its rows come from three small GEMMs).  extra_map: device int32[F], -1 or the row of
+ * extra_rows ([n, d] fp32, 16-byte aligned) that is added to feature f's gradient; extra_bias: fp32[n] added to
+ * bias_grad_out likewise.
  * Replaces loss.backward()'s dense `f^T @ grad` / `x^T @ dh` GEMMs together with
  * torch.optim.Adam.step for W_D / W_E (trainer.py:627-647). */
 int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
@@ -220,7 +225,8 @@ int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot,
                               float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                               double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                               float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
-                              void *workspace, int64_t workspace_bytes, void *stream);
+                              void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
+                              const float *extra_rows, const float *extra_bias, void *stream);
 
 /* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
  * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and
@@ -245,10 +251,12 @@ int64_t sae_sparse_rows_grad_sq_nnz_workspace_bytes(int64_t F);
  * the trainer's every-step clip_grad_norm / grad-norm diagnostic (trainer.py:629-639, optim.py:257-292)
  * needs from W_E and W_D.  acc as in sae_grad_sq_nnz (accumulated into, in a fixed order);
  * bias_grad_out (nullable) receives sum_{s in segment f} coef[s]; workspace: device memory of
- * sae_sparse_rows_grad_sq_nnz_workspace_bytes(F) bytes, 16-byte aligned. */
+ * sae_sparse_rows_grad_sq_nnz_workspace_bytes(F) bytes, 16-byte aligned; extra_map / extra_rows / extra_bias as in
+ * sae_adam_step_sparse_rows. */
 int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
                                 const float *coef, const void *dense, int dense_dtype, int64_t F, int64_t d,
                                 double *acc, float *bias_grad_out, void *workspace, int64_t workspace_bytes,
+                                const int32_t *extra_map, const float *extra_rows, const float *extra_bias,
                                 void *stream);
 
 /* ---- Activation batches from a shuffle buffer -----------------------------------------------------------

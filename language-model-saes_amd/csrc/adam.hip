@@ -142,11 +142,13 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
     float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
     uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad,
-    const float *__restrict__ grad_scale, double *__restrict__ sq_nnz_partial) {
+    const float *__restrict__ grad_scale, double *__restrict__ sq_nnz_partial,
+    const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows, const float *__restrict__ extra_bias) {
   __shared__ float red[4];
   __shared__ double red_d[8];
   const int f = blockIdx.x, tid = threadIdx.x;
   const float gs = grad_scale ? grad_scale[0] : 1.f;
+  const int xo = extra_map ? extra_map[f] : -1;   // row of the dense gradient block that adds to this feature, or -1
   const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
   const int n_seg = d >> 2;
   const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
@@ -157,6 +159,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     float s = 0.f;
     for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
     s = wave_sum(s);
+    if (xo >= 0 && extra_bias) s += extra_bias[xo];
     if (tid == 0) bias_grad[f] = grad_scale ? s * gs : s;
   }
 
@@ -174,7 +177,8 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
         mm[u] = load_stream(m, base4 + seg);
         vv[u] = load_stream(v, base4 + seg);
       }
-      g[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
+                                      : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     for (int i = lo; i < hi; ++i) {
       const int s = feat_slot[i];
@@ -249,10 +253,13 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
                                          float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
                                          double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                                          float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
-                                         void *workspace, int64_t workspace_bytes, void *stream) {
+                                         void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
+                                         const float *extra_rows, const float *extra_bias, void *stream) {
   using namespace sae;
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: null pointer");
+  SAE_REQUIRE((extra_map == nullptr) == (extra_rows == nullptr) && (((uintptr_t)extra_rows) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "adam_step_sparse_rows: extra_map and extra_rows go together (extra_rows 16-byte aligned)");
   SAE_REQUIRE(!grad_sq_nnz_acc || (workspace && workspace_bytes >= 16 * F && ((uintptr_t)workspace & 15) == 0),
               SAE_ERR_WORKSPACE, "adam_step_sparse_rows: the gradient sums need an aligned workspace of %lld bytes",
               (long long)(16 * F));
@@ -273,10 +280,12 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
   double *partial = grad_sq_nnz_acc ? reinterpret_cast<double *>(workspace) : nullptr;
   if (dense_dtype == SAE_BF16)
     hipLaunchKernelGGL(adam_sparse_rows_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial,
+                       extra_map, extra_rows, extra_bias);
   else
     hipLaunchKernelGGL(adam_sparse_rows_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial);
+                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial,
+                       extra_map, extra_rows, extra_bias);
   if (partial) hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, grad_sq_nnz_acc);
   return check_launch("adam_step_sparse_rows");
 }
@@ -376,17 +385,20 @@ template <bool DENSE_BF16>
 __global__ __launch_bounds__(256) void sparse_rows_sq_nnz_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot, const int32_t *__restrict__ slot_tok,
     const float *__restrict__ coef, const void *__restrict__ dense, int d, double *__restrict__ partial,
-    float *__restrict__ bias_grad) {
+    float *__restrict__ bias_grad, const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows,
+    const float *__restrict__ extra_bias) {
   __shared__ double red[8];
   const int f = blockIdx.x, tid = threadIdx.x;
   const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  const int xo = extra_map ? extra_map[f] : -1;
   if (bias_grad && tid < 64) {
     float s = 0.f;
     for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
     s = wave_sum(s);
+    if (xo >= 0 && extra_bias) s += extra_bias[xo];
     if (tid == 0) bias_grad[f] = s;
   }
-  if (lo == hi) {  // no token used this feature: the row gradient is exactly zero
+  if (lo == hi && xo < 0) {  // no token used this feature: the row gradient is exactly zero
     if (tid == 0) { partial[2 * (size_t)f] = 0.0; partial[2 * (size_t)f + 1] = 0.0; }
     return;
   }
@@ -398,7 +410,11 @@ __global__ __launch_bounds__(256) void sparse_rows_sq_nnz_kernel(
   for (int seg0 = tid; seg0 < n_seg; seg0 += 256 * 4) {
     float4 g[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) g[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int u = 0; u < 4; ++u) {
+      const int seg = seg0 + u * 256;
+      g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
+                                      : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     for (int i = lo; i < hi; ++i) {
       const int s = feat_slot[i];
       const float c = coef[s];
@@ -474,6 +490,7 @@ extern "C" int64_t sae_sparse_rows_grad_sq_nnz_workspace_bytes(int64_t F) { retu
 extern "C" int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
                                            const float *coef, const void *dense, int dense_dtype, int64_t F, int64_t d,
                                            double *acc, float *bias_grad_out, void *workspace, int64_t workspace_bytes,
+                                           const int32_t *extra_map, const float *extra_rows, const float *extra_bias,
                                            void *stream) {
   using namespace sae;
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && acc && workspace, SAE_ERR_INVALID_ARG,
@@ -490,10 +507,10 @@ extern "C" int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_
   double *partial = reinterpret_cast<double *>(workspace);
   if (dense_dtype == SAE_BF16)
     hipLaunchKernelGGL(sparse_rows_sq_nnz_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, coef,
-                       dense, (int)d, partial, bias_grad_out);
+                       dense, (int)d, partial, bias_grad_out, extra_map, extra_rows, extra_bias);
   else
     hipLaunchKernelGGL(sparse_rows_sq_nnz_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, coef,
-                       dense, (int)d, partial, bias_grad_out);
+                       dense, (int)d, partial, bias_grad_out, extra_map, extra_rows, extra_bias);
   hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, acc);
   return check_launch("sparse_rows_grad_sq_nnz");
 }

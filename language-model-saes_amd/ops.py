@@ -414,10 +414,11 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                           v: torch.Tensor, *, lr: float, beta1: float, beta2: float, eps: float, step: int,
                           shadow_bf16: Optional[torch.Tensor] = None, row_norm_out: Optional[torch.Tensor] = None,
                           bias_grad_out: Optional[torch.Tensor] = None, grad_scale: Optional[torch.Tensor] = None,
-                          grad_sq_nnz_acc: Optional[torch.Tensor] = None) -> None:
+                          grad_sq_nnz_acc: Optional[torch.Tensor] = None, extra: Optional["DenseRowBlock"] = None) -> None:
     """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense);
     `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping);
-    `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed."""
+    `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed;
+    `extra` adds a densely held block of gradient rows."""
     for name, t in (("p", p), ("m", m), ("v", v)):
         _req(t, name, torch.float32, 2)
     _req(coef, "coef", torch.float32, 1)
@@ -442,13 +443,35 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                                                   coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),
                                                   v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step), _ptr(shadow_bf16),
                                                   _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale),
-                                                  _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, _stream(p)),
+                                                  _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, *_extra_ptrs(extra, F, d), _stream(p)),
             "adam_step_sparse_rows",
         )
 
 
+@dataclass
+class DenseRowBlock:
+    """Gradient rows held densely for a subset of features: `row_map` int32 [F] (-1 or the row of `rows`),
+    `rows` fp32 [n, d], `bias` fp32 [n] or None (added to the per-feature bias gradient)."""
+
+    row_map: torch.Tensor
+    rows: torch.Tensor
+    bias: Optional[torch.Tensor] = None
+
+
+def _extra_ptrs(extra: Optional[DenseRowBlock], F: int, d: int):
+    if extra is None:
+        return None, None, None
+    _req(extra.row_map, "extra.row_map", torch.int32, 1)
+    _req(extra.rows, "extra.rows", torch.float32, 2)
+    if extra.row_map.numel() != F or extra.rows.shape[1] != d:
+        raise ValueError("dense row block does not fit the matrix")
+    if extra.bias is not None:
+        _req(extra.bias, "extra.bias", torch.float32, 1)
+    return extra.row_map.data_ptr(), extra.rows.data_ptr(), _ptr(extra.bias)
+
+
 def sparse_rows_grad_sq_nnz(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, acc: torch.Tensor,
-                            bias_grad_out: Optional[torch.Tensor] = None) -> None:
+                            bias_grad_out: Optional[torch.Tensor] = None, extra: Optional[DenseRowBlock] = None) -> None:
     """acc (device double[2]) += (sum of squares, number of non-zero entries) of the [F, d] gradient that
     (fi, coef, dense) stand for; optionally writes the per-feature bias gradient as well."""
     _req(coef, "coef", torch.float32, 1)
@@ -462,7 +485,7 @@ def sparse_rows_grad_sq_nnz(fi: FeatureIndex, coef: torch.Tensor, dense: torch.T
         check(
             lib.sae_sparse_rows_grad_sq_nnz(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
                                             coef.data_ptr(), dense.data_ptr(), _dt(dense), F, d, acc.data_ptr(),
-                                            _ptr(bias_grad_out), ws.data_ptr(), nbytes, _stream(dense)),
+                                            _ptr(bias_grad_out), ws.data_ptr(), nbytes, *_extra_ptrs(extra, F, d), _stream(dense)),
             "sparse_rows_grad_sq_nnz",
         )
 

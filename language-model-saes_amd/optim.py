@@ -185,7 +185,7 @@ class HipAdam(Optimizer):
                                       lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"], step=step,
                                       shadow_bf16=None if sh2 is None else sh2[r0:r0 + n],
                                       bias_grad_out=None if bias_buf is None else bias_buf[r0:r0 + n],
-                                      grad_scale=piece.scale, grad_sq_nnz_acc=sums_out)
+                                      grad_scale=piece.scale, grad_sq_nnz_acc=sums_out, extra=piece.extra)
             covered = r0 + n
         if covered != p2.shape[0]:
             raise NotImplementedError("row blocks of a factored gradient must tile the parameter")
@@ -245,14 +245,15 @@ class HipAdam(Optimizer):
                     self._side_stream = torch.cuda.Stream(device=p.device)
                 side = self._side_stream
                 side.wait_stream(torch.cuda.current_stream(p.device))
-                for t in (sg.fi.feat_ptr, sg.fi.feat_slot, sg.fi.slot_tok, sg.coef, sg.dense_operand, sg.scale):
+                extra_t = () if sg.extra is None else (sg.extra.row_map, sg.extra.rows, sg.extra.bias)
+                for t in (sg.fi.feat_ptr, sg.fi.feat_slot, sg.fi.slot_tok, sg.coef, sg.dense_operand, sg.scale, *extra_t):
                     if t is not None:
                         t.record_stream(side)  # step-local tensors: keep their memory until the side stream is done
             with torch.cuda.stream(side) if side is not None else _null_ctx():
                 ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
                                           eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
                                           row_norm_out=norm_out, bias_grad_out=bias_out, grad_scale=sg.scale,
-                                          grad_sq_nnz_acc=sums_out)
+                                          grad_sq_nnz_acc=sums_out, extra=sg.extra)
                 if side is not None:
                     ev = torch.cuda.Event()
                     ev.record(side)
@@ -362,7 +363,7 @@ def _grad_sq_nnz(params) -> torch.Tensor:
                     if bias_buf is None:
                         bias_buf = torch.zeros(bias_param.numel(), dtype=torch.float32, device=p.device)
                     bias_out = bias_buf[r0:r0 + sg.n_features]
-                ops.sparse_rows_grad_sq_nnz(sg.fi, sg.coef, sg.dense_operand, own, bias_grad_out=bias_out)
+                ops.sparse_rows_grad_sq_nnz(sg.fi, sg.coef, sg.dense_operand, own, bias_grad_out=bias_out, extra=sg.extra)
                 sg.sq_nnz = own
             own = sg.sq_nnz
             if sg.scale is not None:

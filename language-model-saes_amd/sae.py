@@ -54,15 +54,22 @@ class SparseRowGrad:
     dense gradient never has to be written to HBM.  `dense()` materialises it on demand."""
 
     def __init__(self, fi: ops.FeatureIndex, coef: torch.Tensor, dense_operand: torch.Tensor, n_features: int,
-                 bias_param: Optional[torch.Tensor] = None):
+                 bias_param: Optional[torch.Tensor] = None, extra: Optional[ops.DenseRowBlock] = None):
         self.fi, self.coef, self.dense_operand, self.n_features, self.bias_param = fi, coef, dense_operand, n_features, bias_param
+        self.extra = extra    # gradient rows held densely for some features (added to the factored part)
         self.scale: Optional[torch.Tensor] = None    # device float[1] from gradient clipping, applied where rows are formed
         self.sq_nnz: Optional[torch.Tensor] = None   # cached (sum g^2, #non-zero) of the unscaled rows
 
-    def dense(self):
+    def dense(self, want_bias: Optional[bool] = None):
         """(rows [F, d] fp32, bias gradient [F] or None)"""
         rows, bias = ops.sparse_grad_rows(self.fi, self.coef, self.dense_operand, self.n_features,
-                                          want_bias=self.bias_param is not None)
+                                          want_bias=self.bias_param is not None if want_bias is None else want_bias)
+        if self.extra is not None:
+            hit = self.extra.row_map >= 0
+            src = self.extra.row_map.clamp_min(0).long()
+            rows += torch.where(hit[:, None], self.extra.rows.index_select(0, src), torch.zeros_like(rows))
+            if bias is not None and self.extra.bias is not None:
+                bias += torch.where(hit, self.extra.bias.index_select(0, src), torch.zeros_like(bias))
         if self.scale is not None:
             rows.mul_(self.scale)
             if bias is not None:
@@ -96,6 +103,85 @@ class SparseRowGradPieces:
             if b is not None:
                 bias[r0:r0 + sg.n_features] = b
         return rows, bias
+
+
+def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux: int, batch_wide: bool, amp: bool):
+    """Forward half of the aux-k term on a compacted dead block.  Gathers the dead features' encoder / decoder
+    rows into [n, d] matrices (n = #dead padded to the GEMM's K granule), recomputes their pre-activations with
+    the encoder GEMM (same kernel, same accumulation order as the full product: identical values), selects among
+    them, scatters the kept values into a dense [B, n] matrix and decodes it with one more GEMM.
+    Returns None when the shapes do not fit the GEMM kernel or the block is too wide to pay; sizing the block
+    needs #dead on the host (one synchronisation per step, as the reference's `int(is_dead.sum().item())`)."""
+    B, d = x_op.shape
+    F = dead.numel()
+    gran = 64 if amp else 32
+    if B % gran != 0 or d % gran != 0:
+        return None
+    dead_idx = torch.nonzero(dead).squeeze(1)
+    nd = int(dead_idx.numel())
+    if nd == 0:
+        return {"n_dead": 0, "code": None}
+    if nd > 64 * max(k_aux, 1) or B * (nd + gran) >= 2 ** 31:
+        return None
+    ndp = (nd + gran - 1) // gran * gran
+    dev = x_op.device
+
+    def rows_of(w):   # [nd, d] gathered, zero rows up to ndp
+        out = torch.zeros(ndp, d, dtype=w.dtype, device=dev)
+        out[:nd] = w.index_select(0, dead_idx)
+        return out
+
+    W_Et, W_D = rows_of(w_enc_op), rows_of(w_dec_op)
+    b_d = torch.zeros(ndp, dtype=torch.float32, device=dev)
+    b_d[:nd] = b_E.detach().float().index_select(0, dead_idx)
+    s_d = None
+    if scale is not None:
+        s_d = torch.ones(ndp, dtype=torch.float32, device=dev)
+        s_d[:nd] = scale.index_select(0, dead_idx)
+    pre_d = ops.encoder_gemm(x_op, W_Et, pre_dtype)                                   # [B, ndp]
+    kk = min(k_aux, nd)
+    code_d = ops.select_topk_batch(pre_d, b_d, s_d, kk * B) if batch_wide else ops.select_topk_row(pre_d, b_d, s_d, kk)
+    # dense [B, ndp] activations of the block
+    tok, valid = _code_slot_tokens(code_d)
+    flat = tok.long() * ndp + code_d.idx.long()
+    vals = torch.where(valid, code_d.val, torch.zeros_like(code_d.val))
+    A = torch.zeros(B * ndp, dtype=torch.float32, device=dev).scatter_add_(0, flat, vals).view(B, ndp)
+    A_op = ops.cast_bf16(A) if amp else A
+    aux_recon = ops.encoder_gemm(A_op, W_D.t().contiguous(), torch.float32)            # [B, d] = A @ W_D[dead]
+    # the same code with the dictionary's own feature ids (for callers that look at it)
+    idx_full = torch.where(valid, dead_idx.index_select(0, code_d.idx.long().clamp_max(nd - 1)).to(torch.int32),
+                           torch.zeros_like(code_d.idx))
+    import dataclasses
+    code_full = dataclasses.replace(code_d, idx=idx_full, d_sae=F)
+    row_map = torch.full((F,), -1, dtype=torch.int32, device=dev)
+    row_map[dead_idx] = torch.arange(nd, dtype=torch.int32, device=dev)
+    return {"n_dead": nd, "ndp": ndp, "W_Et": W_Et, "W_D": W_D, "A": A, "A_op": A_op, "aux_recon": aux_recon,
+            "code": code_full, "row_map": row_map}
+
+
+def _code_slot_tokens(code: ops.SparseCode):
+    """(token of every slot, whether the slot is in use) for a sparse code."""
+    slots = torch.arange(code.n_slots, device=code.val.device)
+    tok = torch.searchsorted(code.row_off, slots, right=True) - 1
+    valid = (slots - code.row_off[tok]) < code.row_nnz[tok]
+    return tok, valid
+
+
+def _aux_dense_grads(blk, g_aux, x_op, amp: bool):
+    """Backward half: with G = d loss / d aux_recon [B, d] and A the block's activations [B, n],
+    d A = G W_D[dead]^T masked to the kept entries (the decoder-norm scale cancels as in the main path),
+    dW_D[dead] = A^T G, dW_E^T[dead] = dA^T x, db_E[dead] = column sums of dA: three GEMMs with K = d, B, B."""
+    nd = blk["n_dead"]
+    A, A_op = blk["A"], blk["A_op"]
+    G_op = ops.cast_bf16(g_aux.contiguous()) if amp else g_aux.contiguous()
+    dA = ops.encoder_gemm(G_op, blk["W_D"], torch.float32)                             # [B, ndp]
+    dpre = torch.where(A > 0, dA, torch.zeros_like(dA))
+    dpre_op = ops.cast_bf16(dpre) if amp else dpre
+    dW_D = ops.encoder_gemm(A_op.t().contiguous(), G_op.t().contiguous(), torch.float32)        # [ndp, d]
+    dW_Et = ops.encoder_gemm(dpre_op.t().contiguous(), x_op.t().contiguous(), torch.float32)    # [ndp, d]
+    db_E = ops.col_sum(dpre)
+    return {"row_map": blk["row_map"], "dW_D": dW_D[:nd].contiguous(), "dW_Et": dW_Et[:nd].contiguous(),
+            "db_E": db_E[:nd].contiguous(), "dpre": dpre, "W_Et": blk["W_Et"]}
 
 
 class _FusedSparseStep(torch.autograd.Function):
@@ -140,36 +226,67 @@ class _FusedSparseStep(torch.autograd.Function):
             loss = loss_tok.sum()
             l_aux = None
             grad_code, grad_dense_D, grad_coef_E, x_rows = code, grad_recon, dval, x_op
+            ctx.aux_dense = None
         else:
             dead = aux["is_dead"](code)                       # bool [F], from the caller's dead statistics
-            dead_f = dead.to(torch.float32)
-            n_dead = dead.sum()
             k_aux = int(aux["k_aux"])
-            if batch_wide:
-                k_dev = (torch.clamp(n_dead, max=k_aux) * B).to(torch.int64)
-                aux_code = ops.select_topk_batch(pre, b_E, scale, k_dev, feat_mask=dead_f, capacity=k_aux * B)
+            ctx.aux_dense = None
+            dense_block = None
+            if aux.get("dense", True):
+                dense_block = _aux_dense_block(x_op, pre.dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux, batch_wide, amp)
+            sae._last_aux_route = "dense" if dense_block is not None else "sparse"
+            if dense_block is not None:
+                # The dead block is small and hit by a large share of the tokens: its part of the step is three small
+                # GEMMs on a compacted [n_dead, d] copy of the two weight blocks instead of gathers per (token, feature).
+                blk = dense_block
+                recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
+                w = tok_w[:, None]
+                diff = recon - label
+                alpha = float(aux["coefficient"])
+                l_rec = (w * diff * diff).sum()
+                if blk["n_dead"] == 0:
+                    l_aux = torch.zeros_like(l_rec)
+                    g_aux = None
+                    grad_recon = 2.0 * w * diff
+                else:
+                    r = (label - recon) - blk["aux_recon"]
+                    l_aux = alpha * (w * r * r).sum()
+                    g_aux = (-2.0 * alpha) * w * r                 # d loss / d aux_recon
+                    grad_recon = 2.0 * w * diff + g_aux            # d loss / d recon (the residual is not detached)
+                loss = l_rec + l_aux
+                dval = ops.sparse_decode_bwd_dval(code, grad_recon, w_dec_op)
+                if g_aux is not None:
+                    ctx.aux_dense = _aux_dense_grads(blk, g_aux, x_op, amp)
+                grad_code, grad_dense_D, grad_coef_E, x_rows = code, grad_recon, dval, x_op
+                holder.aux_code = blk["code"]
             else:
-                # min(k_aux, #dead) needs no host value: at most #dead entries can be positive
-                aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f)
-            recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
-            aux_recon = ops.sparse_decode_fwd(aux_code, w_dec_op, None)
-            has_dead = (n_dead > 0).to(torch.float32)
-            w = tok_w[:, None]
-            diff = recon - label
-            r = (label - recon) - aux_recon
-            alpha = float(aux["coefficient"]) * has_dead
-            l_rec = (w * diff * diff).sum()
-            l_aux = alpha * (w * r * r).sum()
-            loss = l_rec + l_aux
-            g_aux = (-2.0 * alpha) * w * r                     # d loss / d aux_recon
-            grad_recon = 2.0 * w * diff + g_aux                # d loss / d recon (the residual is not detached)
-            dval = ops.sparse_decode_bwd_dval(code, grad_recon, w_dec_op)
-            dval_aux = ops.sparse_decode_bwd_dval(aux_code, g_aux, w_dec_op)
-            grad_code = ops.stack_codes(code, aux_code)
-            grad_dense_D = torch.cat([grad_recon, g_aux])
-            grad_coef_E = torch.cat([dval, dval_aux])
-            x_rows = torch.cat([x_op, x_op])
-            holder.aux_code = aux_code
+                dead_f = dead.to(torch.float32)
+                n_dead = dead.sum()
+                if batch_wide:
+                    k_dev = (torch.clamp(n_dead, max=k_aux) * B).to(torch.int64)
+                    aux_code = ops.select_topk_batch(pre, b_E, scale, k_dev, feat_mask=dead_f, capacity=k_aux * B)
+                else:
+                    # min(k_aux, #dead) needs no host value: at most #dead entries can be positive
+                    aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f)
+                recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
+                aux_recon = ops.sparse_decode_fwd(aux_code, w_dec_op, None)
+                has_dead = (n_dead > 0).to(torch.float32)
+                w = tok_w[:, None]
+                diff = recon - label
+                r = (label - recon) - aux_recon
+                alpha = float(aux["coefficient"]) * has_dead
+                l_rec = (w * diff * diff).sum()
+                l_aux = alpha * (w * r * r).sum()
+                loss = l_rec + l_aux
+                g_aux = (-2.0 * alpha) * w * r                     # d loss / d aux_recon
+                grad_recon = 2.0 * w * diff + g_aux                # d loss / d recon (the residual is not detached)
+                dval = ops.sparse_decode_bwd_dval(code, grad_recon, w_dec_op)
+                dval_aux = ops.sparse_decode_bwd_dval(aux_code, g_aux, w_dec_op)
+                grad_code = ops.stack_codes(code, aux_code)
+                grad_dense_D = torch.cat([grad_recon, g_aux])
+                grad_coef_E = torch.cat([dval, dval_aux])
+                x_rows = torch.cat([x_op, x_op])
+                holder.aux_code = aux_code
         if amp:
             # the decoder's weight gradient pairs the activations with the bf16-rounded output gradient, as the
             # backward of an autocast matmul does; the gather of those rows then moves half the bytes
@@ -193,12 +310,17 @@ class _FusedSparseStep(torch.autograd.Function):
         coef_dec = code.val * g          # dW_D[f] = sum val * grad_recon[token]
         coef_enc = ctx.grad_coef_E * g   # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
         db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
+        extra_D = extra_E = None
+        ad = ctx.aux_dense
+        if ad is not None:   # the dead block's rows, held densely
+            extra_D = ops.DenseRowBlock(ad["row_map"], ad["dW_D"] * g, None)
+            extra_E = ops.DenseRowBlock(ad["row_map"], ad["dW_Et"] * g, ad["db_E"] * g)
         sae = ctx.defer_to
         if sae is not None and getattr(sae.W_D, "_sparse_grad", None) is None and sae.W_D.grad is None \
                 and getattr(sae.W_E, "_sparse_grad", None) is None and sae.W_E.grad is None:
             # hand the factored gradients to the optimiser; b_E's gradient is a by-product of its W_E pass
-            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, ctx.grad_dense_D, F)
-            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, ctx.x_rows, F, bias_param=sae.b_E)
+            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, ctx.grad_dense_D, F, extra=extra_D)
+            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, ctx.x_rows, F, bias_param=sae.b_E, extra=extra_E)
             dW_D = dW_Et = db_E = None
         else:
             if sae is not None:  # a second backward before the optimiser ran: fall back to dense accumulation
@@ -210,14 +332,16 @@ class _FusedSparseStep(torch.autograd.Function):
                         if bias is not None:
                             sg.bias_param.grad = bias if sg.bias_param.grad is None else sg.bias_param.grad + bias
                         prm._sparse_grad = None
-            dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, ctx.grad_dense_D, F)
-            dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, ctx.x_rows, F, want_bias=True)
+            dW_D, _ = SparseRowGrad(fi, coef_dec, ctx.grad_dense_D, F, extra=extra_D).dense()
+            dW_Et, db_E = SparseRowGrad(fi, coef_enc, ctx.x_rows, F, extra=extra_E).dense(want_bias=True)
         dx = None
         if ctx.needs_input_grad[0]:
             import dataclasses
             dx = ops.sparse_decode_fwd(dataclasses.replace(code, val=coef_enc), ctx.w_enc_op, None)
             if dx.shape[0] != ctx.n_tokens:  # stacked code: fold the aux half back onto its tokens
                 dx = dx[: ctx.n_tokens] + dx[ctx.n_tokens:]
+            if ad is not None:
+                dx = dx + (ad["dpre"].to(ad["W_Et"].dtype) @ ad["W_Et"]).to(torch.float32) * g
         dlabel = None
         if ctx.needs_input_grad[1]:
             dlabel = -ctx.grad_recon * g
@@ -300,6 +424,9 @@ class SparseAutoEncoder(SparseDictionary):
         # set by an optimiser that consumes SparseRowGrad (HipAdam): the fused backward then leaves W_E.grad /
         # W_D.grad unset and attaches the factored gradient as `param._sparse_grad` instead
         self.defer_weight_grads = False
+        # aux-k: treat the dead features as a compact dense block (three small GEMMs) when shapes allow; False keeps
+        # the sparse route (dead-feature entries stacked onto the main code) for every shape
+        self.aux_dense_block = True
 
     # ---- an optimiser may still be updating W_D on another stream (see HipAdam.overlap_decoder_update) ----
     def set_pending_update(self, event) -> None:
@@ -542,7 +669,7 @@ class SparseAutoEncoder(SparseDictionary):
                     return sparse_upd(code, _mask)
                 return _upd(code.to_dense(), _mask, ("batch", "sae"))  # a callable that only knows dense activations
 
-            holder.aux = {"is_dead": is_dead, "k_aux": k_aux, "coefficient": auxk_coefficient}
+            holder.aux = {"is_dead": is_dead, "k_aux": k_aux, "coefficient": auxk_coefficient, "dense": self.aux_dense_block}
         holder.defer_to = self if self.defer_weight_grads and torch.is_grad_enabled() else None
         loss, recon = _FusedSparseStep.apply(
             x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x,

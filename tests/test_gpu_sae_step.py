@@ -271,11 +271,14 @@ def test_fused_batchtopk_step_matches_oracle(pkg, oracle, dev, amp):
 
 @pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
 @pytest.mark.parametrize("include_norm", [False, True])
-def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm):
-    print(f"fused aux-k {act_fn} include_norm={include_norm}", flush=True)
-    B, F, k, k_aux = 192, 2048, 16, 24
+@pytest.mark.parametrize("route", ["dense", "sparse"])
+def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm, route):
+    """Both routes of the aux-k term (dead features as a compact dense block / stacked onto the sparse code)."""
+    print(f"fused aux-k {act_fn} include_norm={include_norm} route={route}", flush=True)
+    B, F, k, k_aux = 192, 2048, 16, 32
     sae, ref, batch = make_pair_act(pkg, oracle, dev, act_fn, d=256, F=F, k=k, B=B, r=8, seed=12, include_norm=include_norm,
                                     mask_frac=0.2)
+    sae.aux_dense_block = route == "dense"
     trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=1 / 32, k_aux=k_aux, dead_threshold=float(B)))
     trainer._initialize_dead_statistics(sae)
     stats = oracle.DeadStatistics(F, dead_threshold=float(B))
@@ -306,6 +309,7 @@ def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm):
     rctx = ref.compute_loss(batch, update_dead_statistics=stats.update, **kw)
     rctx["loss"].backward()
 
+    assert sae._last_aux_route == route
     assert torch.equal(trainer.is_dead.cpu(), stats.is_dead)
     assert torch.equal(trainer.tokens_since_last_activation.cpu(), stats.tokens_since_last_activation)
     assert stats.is_dead.sum().item() > k_aux  # plenty of dead features: the aux select really truncates
