@@ -250,3 +250,38 @@ def test_deferred_grad_norm_comes_out_of_the_optimizer_step(pkg, oracle, dev):
     synthetic.load_weights(ref, *w)
     ref.compute_loss({"in": x, "out": x, "tokens": torch.zeros(B)})["loss"].backward()
     assert by_product[0] == pytest.approx(oracle.compute_grad_norm([p.grad for p in ref.parameters()]).item(), rel=1e-5)
+
+
+def test_dense_row_block_adds_to_the_factored_gradient(pkg, dev):
+    """`extra` (a densely held block of gradient rows) in the Adam row pass and in the factored norm: equal to the
+    same rows added to the materialised gradient."""
+    B, d, F, k, n = 64, 128, 600, 8, 37
+    g = torch.Generator().manual_seed(17)
+    code, _ = random_code(pkg, dev, B, F, k, seed=18)
+    fi = pkg.ops.build_feature_index(code)
+    coef = torch.randn(B * k, generator=g).to(dev)
+    dense_op = torch.randn(B, d, generator=g).to(dev)
+    ids = torch.randperm(F, generator=g)[:n].sort().values
+    row_map = torch.full((F,), -1, dtype=torch.int32); row_map[ids] = torch.arange(n, dtype=torch.int32)
+    block = pkg.ops.DenseRowBlock(row_map.to(dev), torch.randn(n, d, generator=g).to(dev), torch.randn(n, generator=g).to(dev))
+    rows, bias = pkg.ops.sparse_grad_rows(fi, coef, dense_op, F, want_bias=True)
+    rows_x = rows.clone(); rows_x[ids.to(dev)] = block.rows + rows[ids.to(dev)]      # the block is the accumulator's start value
+    bias_x = bias.clone(); bias_x[ids.to(dev)] += block.bias
+    p0 = torch.randn(F, d, generator=g).to(dev)
+    pa, ma, va = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    pb, mb, vb = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    bias_out = torch.empty(F, device=dev)
+    acc = torch.zeros(2, dtype=torch.float64, device=dev)
+    pkg.ops.adam_step(pa, rows_x, ma, va, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1)
+    pkg.ops.adam_step_sparse_rows(fi, coef, dense_op, pb, mb, vb, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1,
+                                  bias_grad_out=bias_out, grad_sq_nnz_acc=acc, extra=block)
+    assert (pa - pb).abs().max() <= 2e-6 * 1e-3 + 1e-7 and (ma - mb).abs().max() <= 1e-6 * ma.abs().max()
+    assert (bias_out - bias_x).abs().max() <= 1e-5 * bias_x.abs().max()
+    assert acc[1].item() == (rows_x != 0).sum().item()
+    assert acc[0].item() == pytest.approx(rows_x.double().pow(2).sum().item(), rel=1e-5)
+    acc2 = torch.zeros(2, dtype=torch.float64, device=dev)
+    pkg.ops.sparse_rows_grad_sq_nnz(fi, coef, dense_op, acc2, extra=block)
+    assert acc2[1].item() == acc[1].item() and acc2[0].item() == pytest.approx(acc[0].item(), rel=1e-9)
+    with pytest.raises(ValueError):
+        pkg.ops.adam_step_sparse_rows(fi, coef, dense_op, pb, mb, vb, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=2,
+                                      extra=pkg.ops.DenseRowBlock(row_map[:10].to(dev), block.rows, None))
