@@ -180,27 +180,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    for (int i = lo; i < hi; ++i) {
-      const int s = feat_slot[i];
-      const float c = coef[s];
-      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int seg = seg0 + u * 256;
-        if (seg < n_seg) {
-          float4 x;
-          if constexpr (DENSE_BF16) {
-            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
-            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
-            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
-          } else {
-            x = reinterpret_cast<const float4 *>(row)[seg];
-          }
-          g[u].x = fmaf(c, x.x, g[u].x); g[u].y = fmaf(c, x.y, g[u].y);
-          g[u].z = fmaf(c, x.z, g[u].z); g[u].w = fmaf(c, x.w, g[u].w);
-        }
-      }
-    }
+    gather_rows_fma<DENSE_BF16>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int seg = seg0 + u * 256;
@@ -415,27 +395,7 @@ __global__ __launch_bounds__(256) void sparse_rows_sq_nnz_kernel(
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    for (int i = lo; i < hi; ++i) {
-      const int s = feat_slot[i];
-      const float c = coef[s];
-      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int seg = seg0 + u * 256;
-        if (seg < n_seg) {
-          float4 x;
-          if constexpr (DENSE_BF16) {
-            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
-            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
-            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
-          } else {
-            x = reinterpret_cast<const float4 *>(row)[seg];
-          }
-          g[u].x = fmaf(c, x.x, g[u].x); g[u].y = fmaf(c, x.y, g[u].y);
-          g[u].z = fmaf(c, x.z, g[u].z); g[u].w = fmaf(c, x.w, g[u].w);
-        }
-      }
-    }
+    gather_rows_fma<DENSE_BF16>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       float s4 = g[u].x * g[u].x;   // a 4-element fp32 partial keeps the fp64 adds off the critical path

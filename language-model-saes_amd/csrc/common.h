@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <type_traits>
 
 #include "../../include/sae_hip.h"
 
@@ -88,5 +89,64 @@ __device__ __forceinline__ void store_stream(uint16_t *base, int64_t q, const ui
 struct __attribute__((aligned(16))) u32x4 {
   uint32_t x, y, z, w;
 };
+
+// g[u] += sum over the segment's (slot, token) pairs of coef[slot] * dense[token, 4-element piece seg0 + ROW_THREADS u], pairs
+// in ascending order (the order every route to these gradient rows uses, so all of them give the same bits).
+// A pair costs three dependent loads (slot, then coefficient and token, then the row): pairs are taken in groups
+// whose index and row loads are all issued before the first multiply-add, which hides that chain on long segments.
+template <bool DENSE_BF16, int ROW_THREADS = 256>
+__device__ __forceinline__ void gather_rows_fma(float4 (&g)[4], int lo, int hi, const int32_t *__restrict__ feat_slot,
+                                                const int32_t *__restrict__ slot_tok, const float *__restrict__ coef,
+                                                const char *dbase, size_t row_bytes, int seg0, int n_seg) {
+  constexpr int C = DENSE_BF16 ? 4 : 2;
+  typedef typename std::conditional<DENSE_BF16, uint2, float4>::type piece_t;
+  auto fma_piece = [&](float4 &acc, float c, const piece_t &r) {
+    float4 x;
+    if constexpr (DENSE_BF16) {
+      x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
+      x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
+    } else {
+      x = r;
+    }
+    acc.x = fmaf(c, x.x, acc.x); acc.y = fmaf(c, x.y, acc.y);
+    acc.z = fmaf(c, x.z, acc.z); acc.w = fmaf(c, x.w, acc.w);
+  };
+  int i = lo;
+  for (; i + C <= hi; i += C) {
+    int sl[C];
+#pragma unroll
+    for (int j = 0; j < C; ++j) sl[j] = feat_slot[i + j];
+    float c[C];
+    const piece_t *row[C];
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+      c[j] = coef[sl[j]];
+      row[j] = reinterpret_cast<const piece_t *>(dbase + (size_t)slot_tok[sl[j]] * row_bytes);
+    }
+    piece_t r[C][4];
+#pragma unroll
+    for (int j = 0; j < C; ++j)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int seg = seg0 + u * ROW_THREADS;
+        if (seg < n_seg) r[j][u] = row[j][seg];
+      }
+#pragma unroll
+    for (int j = 0; j < C; ++j)
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (seg0 + u * ROW_THREADS < n_seg) fma_piece(g[u], c[j], r[j][u]);
+  }
+  for (; i < hi; ++i) {
+    const int sl = feat_slot[i];
+    const float c = coef[sl];
+    const piece_t *row = reinterpret_cast<const piece_t *>(dbase + (size_t)slot_tok[sl] * row_bytes);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int seg = seg0 + u * ROW_THREADS;
+      if (seg < n_seg) fma_piece(g[u], c, row[seg]);
+    }
+  }
+}
 
 }  // namespace sae

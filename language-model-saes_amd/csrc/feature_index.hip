@@ -222,27 +222,7 @@ __global__ __launch_bounds__(FI_THREADS) void sparse_grad_rows_kernel(
     float4 acc[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) acc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = lo; i < hi; ++i) {
-      const int s = feat_slot[i];
-      const float c = coef[s];
-      const char *row = dbase + (size_t)slot_tok[s] * row_bytes;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int seg = seg0 + u * FI_THREADS;
-        if (seg < n_seg) {
-          float4 x;
-          if constexpr (DENSE_BF16) {
-            const uint2 r = reinterpret_cast<const uint2 *>(row)[seg];
-            x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
-            x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
-          } else {
-            x = reinterpret_cast<const float4 *>(row)[seg];
-          }
-          acc[u].x = fmaf(c, x.x, acc[u].x); acc[u].y = fmaf(c, x.y, acc[u].y);
-          acc[u].z = fmaf(c, x.z, acc[u].z); acc[u].w = fmaf(c, x.w, acc[u].w);
-        }
-      }
-    }
+    gather_rows_fma<DENSE_BF16, FI_THREADS>(acc, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int seg = seg0 + u * FI_THREADS;

@@ -24,7 +24,7 @@ from torch import nn
 from . import ops
 from .config import LorsaConfig, register_sae_model
 from .hooks import HookPoint
-from .sae import _autocast_dtype
+from .sae import SparseRowGrad, _autocast_dtype
 from .sparse_dictionary import LazyDict, SparseDictionary
 
 
@@ -91,6 +91,8 @@ class _SparseTail(torch.autograd.Function):
             code, w_op, None if b_D is None else b_D.detach(), label, tok_w)
         holder["code"] = code
         ctx.code, ctx.grad_recon, ctx.dval = code, grad_recon, dval
+        ctx.amp = bool(amp)
+        ctx.defer_to = m if holder.get("defer") else None
         ctx.has_b_D = b_D is not None
         ctx.in_dtype = hidden_pre.dtype
         ctx.mark_non_differentiable(recon)
@@ -102,7 +104,15 @@ class _SparseTail(torch.autograd.Function):
         T, F = code.n_tokens, code.d_sae
         g = g_loss.to(torch.float32)
         fi = ops.build_feature_index(code)
-        dW_O, _ = ops.sparse_grad_rows(fi, code.val * g, ctx.grad_recon, F)
+        m = ctx.defer_to
+        if m is not None and m.W_O.grad is None and getattr(m.W_O, "_sparse_grad", None) is None:
+            # the optimiser rebuilds the rows where it consumes them (under autocast from the bf16-rounded output
+            # gradient, as the backward of an autocast matmul pairs them)
+            gd = ops.cast_bf16(ctx.grad_recon.contiguous()) if ctx.amp else ctx.grad_recon
+            m.W_O._sparse_grad = SparseRowGrad(fi, code.val * g, gd, F)
+            dW_O = None
+        else:
+            dW_O, _ = ops.sparse_grad_rows(fi, code.val * g, ctx.grad_recon, F)
         db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
         d_hp = None
         if ctx.needs_input_grad[0]:
@@ -130,6 +140,9 @@ class LowRankSparseAttention(SparseDictionary):
         self.b_V = P(cfg.n_ov_heads)
         if cfg.use_decoder_bias:
             self.b_D = P(cfg.d_model)
+        # set by an optimiser that consumes factored gradients (HipAdam): W_O's gradient is then attached to it as
+        # `_sparse_grad` instead of being written as dense rows
+        self.defer_weight_grads = False
         self.register_buffer("mask", torch.tril(torch.ones((cfg.n_ctx, cfg.n_ctx), device=cfg.device).bool()))
         self.register_buffer("IGNORE", torch.tensor(-torch.inf, device=cfg.device))
         if cfg.use_post_qk_ln:
@@ -212,10 +225,10 @@ class LowRankSparseAttention(SparseDictionary):
         w = self.W_O.detach()
         if not amp or w.dtype == torch.bfloat16:
             return w
-        return self._derive("W_O.bf16", self.W_O, lambda old: ops.cast_bf16(w, old))
+        return self._derive("W_D.bf16", self.W_O, lambda old: ops.cast_bf16(w, old))
 
     def _decoder_norm_nograd(self) -> torch.Tensor:
-        return self._derive("W_O.norm", self.W_O, lambda old: ops.row_norm(self.W_O.detach().float(), old))
+        return self._derive("W_D.norm", self.W_O, lambda old: ops.row_norm(self.W_O.detach().float(), old))
 
     # ---- norms (lorsa.py:577-640, 946-958) ----
     def encoder_norm(self, keepdim: bool = False) -> torch.Tensor:
@@ -435,7 +448,7 @@ class LowRankSparseAttention(SparseDictionary):
             tok_w = mf / mf.sum()
         amp = _autocast_dtype("cuda") == torch.bfloat16
         hidden_pre = self.compute_hidden_pre(x)                                    # [b, s, F], autograd-tracked
-        holder: dict[str, Any] = {"model": self}
+        holder: dict[str, Any] = {"model": self, "defer": self.defer_weight_grads and torch.is_grad_enabled()}
         loss, recon = _SparseTail.apply(hidden_pre.reshape(T, F), label.to(torch.float32).reshape(T, d).contiguous(), tok_w,
                                         self.W_O, self.b_D if self.cfg.use_decoder_bias else None, int(self.current_k), amp,
                                         holder)

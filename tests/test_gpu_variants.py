@@ -313,3 +313,27 @@ def test_lorsa_fused_step_bf16(pkg, vo, dev):
     assert rel_err(out["loss"], want["loss"]) < BF16_TOL
     out["loss"].backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+
+
+def test_lorsa_adam_steps_with_factored_output_gradient(pkg, vo, dev):
+    """With HipAdam attached W_O's gradient stays factored; three steps against torch.optim.Adam on the oracle, and
+    the cached bf16 copy / row norms of W_O follow the update."""
+    d, F, h, dq, s, b, k = 64, 512, 4, 16, 32, 2, 8
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, 32, k, seed=55, positional_embedding_type="rotary", rotary_dim=16)
+    g = torch.Generator().manual_seed(56)
+    batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
+    ropt = torch.optim.Adam(ref.parameters(), lr=1e-3)
+    rp = {k_.replace("ln_q_w", "ln_q.w").replace("ln_k_w", "ln_k.w"): v for k_, v in ref.named_parameters()}
+    for step in range(3):
+        out = m.compute_loss(gb)
+        want = ref.compute_loss(batch)
+        assert rel_err(out["loss"], want["loss"]) < 1e-3, step
+        out["loss"].backward(); want["loss"].backward()
+        assert m.W_O.grad is None and m.W_O._sparse_grad is not None
+        opt.step(); ropt.step(); opt.zero_grad(); ropt.zero_grad()
+        for n, p in m.named_parameters():
+            q = rp[n].detach()
+            assert (p.detach().cpu() - q).abs().max() <= 5e-2 * 1e-3 * (step + 1) + 1e-6 * q.abs().max(), (step, n)
+    assert torch.allclose(m._decoder_norm_nograd().cpu(), m.W_O.detach().norm(dim=1).cpu(), rtol=1e-5)
