@@ -49,7 +49,7 @@ def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
     return {
         "encoder_gemm": ("mfma", 2.0 * B * d * F),                       # flop
         "select_topk_row": ("hbm", B * F * 2 + B * k * 8),               # read bf16 pre once, write idx+val
-        "select_topk_batch": ("hbm", 3 * B * F * 2 + B * k * 8),         # three radix passes over bf16 pre + ordered emit
+        "select_topk_batch": ("hbm", B * F * 2 + B * k * 8),             # read bf16 pre once, write idx+val
         "sparse_decode_mse_fused": ("hbm", 2 * B * k * d * 2 + 3 * B * d * 4),  # rows for recon and for d val; label, recon, grad
         "sparse_decode_fwd": ("hbm", B * k * d * 2 + B * d * 4),
         "sparse_decode_bwd_dval": ("hbm", B * k * d * 2 + B * d * 4),
@@ -375,7 +375,9 @@ def main():
         "launches_per_step": kernels[dominant]["calls"] / args.steps,
     }
     per_kernel = {}
-    uniform = args.workload in ("topk", "topk_trainer", "batchtopk", "jumprelu", "activation_stream")     # one dictionary shape for every launch
+    # one dictionary shape for every launch of a kernel (the aux-k branch of "batchtopk" runs the GEMM and the
+    # select on its compact block of dead features as well, CLT and Lorsa on several shapes)
+    uniform = args.workload in ("topk", "topk_trainer", "jumprelu", "activation_stream")
     for kname, st in kernels.items():
         bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None

@@ -4,15 +4,34 @@
 // (ties at the threshold: lowest flattened index b * F + f first) and emits the survivors as a
 // sparse code with one variable-length row per token, indices ascending.
 //
-//   hist x3   exact radix select of the k_total-th largest key over all B * F keys: three
-//             streaming passes build 11 + 11 + 9-bit digit histograms (per-wave private
-//             histograms in LDS, merged with one global atomic per bin and workgroup); a
-//             one-workgroup kernel after each pass picks the digit and narrows the prefix
-//   count     one workgroup per token: number of keys above the threshold and equal to it
+// The [B, F] matrix is read in full ONCE.  A row is cut into granules of 8 * V consecutive
+// elements (V = 8 bf16 / 4 fp32: the 128 bytes eight lanes read with one 16-byte load each).
+//
+//   first     the one full pass: the largest key of every granule, kept in the workspace, and the
+//             histogram of the top 11 bits of those maxima
+//   bound     one workgroup: at least as many keys as granule maxima reach any value, so the
+//             k_total-th largest maximum (rounded down to its histogram bin) is a lower bound on the
+//             threshold
+//   gather    per token: the keys at or above the lower bound (the candidates: about 1.5 k_total of
+//             them) with their features, token by token and in feature order, into a list; only
+//             granules whose largest key reaches the bound are read
+//   next x3   exact radix select of the k_total-th largest key: digit histograms of bits 30..20,
+//             19..9 and 8..0 of the candidates that match the prefix so far
+//   pick      after each: one workgroup picks the digit in which the running count from the top
+//             reaches the wanted rank (fewer positives than k_total: keep every positive, no search)
+//   count     per token: candidates above the threshold and equal to it
 //   plan      one workgroup: prefix sums over tokens -> row offsets, and how many of each token's
 //             threshold ties are kept (the first `need` ties in flattened order)
-//   emit      one workgroup per token walks its row in index order and compacts the kept
-//             elements with a block-wide prefix sum, so indices ascend without a sort
+//   emit      per token: walks the token's candidates in feature order and places the kept ones
+//             with an in-wave prefix sum, so indices ascend without a sort
+//
+// The candidate list holds B * F / 64 + 1024 entries.  When more keys reach the lower bound (a matrix
+// of few distinct values), next, count and emit read the matrix again instead, granule by granule
+// as gather does: same results, about twice the time.
+//
+// gather, next, count and emit give one WAVE to each token: it reads the token's granule maxima
+// 256 at a time, packs the surviving granules' numbers into a list, and reads them 32 at a time
+// (four loads in flight, each covering eight granules), with no workgroup barrier.
 //
 // Keys are the bit patterns of positive floats (unsigned order == float order); non-positive
 // entries have key 0 and are never kept, which is the reference's relu mask.  k_total may be
@@ -25,16 +44,32 @@ namespace sae {
 constexpr int BT_THREADS = 1024;
 constexpr int BT_WAVES = BT_THREADS / 64;
 constexpr int BT_BINS = 2048;
+constexpr uint32_t BT_KEEP_NOTHING = 0xffffffffu;
+constexpr int BT_GL = 8;                  // lanes that read one granule
+constexpr int BT_GPW = 64 / BT_GL;        // granules one wave-wide load covers
+constexpr int BT_LIVE = 256;              // granule maxima a wave examines at a time
 
 struct BatchSelState {      // lives in the workspace, one per call
   uint32_t prefix;          // bits of the threshold key decided so far
   uint32_t mask;            // which bits those are
   int64_t remaining;        // rank still to resolve inside the current prefix
   int64_t k_total;          // resolved k (min(k_total, #positives))
-  int64_t n_positive;
+  int64_t n_positive;       // number of positive keys when every one of them is a candidate, else -1
   int32_t done;             // 1 when the threshold needs no (further) search
   uint32_t threshold;       // final: keep key > threshold, plus the first `remaining` keys == threshold
+  uint32_t lower;           // a lower bound on the threshold, found from the granule maxima
+  unsigned long long cand_count;  // keys >= lower that the gather pass met (may exceed the list's capacity)
+  int32_t overflow;         // 1: they did not fit; the later passes read the matrix again instead
 };
+
+constexpr int BT_STASH = 512;   // candidates of one token a wave collects in LDS before it reserves their place
+
+// capacity of the candidate list for a [B, F] matrix: k_total is B * F / 512 for k = F / 512 per token, and about
+// twice k_total keys reach the lower bound, so this leaves a wide margin at 1/8 of a bf16 matrix's bytes
+__host__ __device__ inline int64_t bt_candidate_capacity(int64_t B, int64_t F) {
+  const int64_t c = B * F / 64 + 1024;
+  return c < 0x7fffffffLL ? c : 0x7fffffffLL;
+}
 
 __device__ __forceinline__ uint32_t bt_key(float pre, float b, float s, float fm, bool has_mask) {
   float h1 = (pre + b) * s;
@@ -42,287 +77,545 @@ __device__ __forceinline__ uint32_t bt_key(float pre, float b, float s, float fm
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
 
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { const uint32_t t = (uint32_t)__shfl_xor((int)v, o, 64); v = t > v ? t : v; }
+  return v;
+}
+
 template <bool BF16>
 struct BatchReader {
+  static constexpr int V = BF16 ? 8 : 4;
   const void *pre;
   const float *b_enc, *scale, *fmask;
   int F;
-  // fn(f, key) for every element of row b, in any order
-  template <typename Fn>
-  __device__ __forceinline__ void row_for_each(int b, Fn fn) const {
-    const char *row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
-    constexpr int V = BF16 ? 8 : 4;
-    const bool vec_ok = (F % V == 0) && ((((uintptr_t)row | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
-    if (vec_ok) {
-      for (int c = threadIdx.x; c < F / V; c += blockDim.x) chunk(row, c, fn);
-    } else {
-      for (int i = threadIdx.x; i < F; i += blockDim.x) fn(i, scalar_key(row, i));
-    }
+  int vec;    // rows, bias, scale and mask can be read as 16-byte vectors
+  int nseg;   // 64-lane segments per row (the full pass walks these)
+  int ngran;  // granules per row, rounded up to a multiple of 4 (the maxima past the row's end are 0)
+  __device__ __forceinline__ const char *row_ptr(int b) const {
+    return reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   }
-  __device__ __forceinline__ uint32_t scalar_key(const char *row, int i) const {
-    float p;
-    if constexpr (BF16) p = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
-    else p = reinterpret_cast<const float *>(row)[i];
-    return bt_key(p, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr);
+  // feature index of the first of this lane's V consecutive elements when its quarter wave reads granule g
+  __device__ __forceinline__ int lane_base(int g) const { return (g * BT_GL + (int)(threadIdx.x & (BT_GL - 1))) * V; }
+  // Loads under a per-lane condition are each followed by a wait for memory; the loads below are therefore
+  // issued by every lane, a lane with nothing to read (base < 0 or past the row's end) reading the row's first
+  // bytes instead, and its result is discarded when the keys are formed.
+  __device__ __forceinline__ int safe_base(int base) const { return (base >= 0 && base < F) ? base : 0; }
+  // the 16 bytes of row b at feature `base` (vector layout only)
+  __device__ __forceinline__ u32x4 load_raw(int b, int base) const {
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (vec) raw = reinterpret_cast<const u32x4 *>(row_ptr(b))[safe_base(base) / V];
+    return raw;
   }
-  template <typename Fn>
-  __device__ __forceinline__ void chunk(const char *row, int c, Fn fn) const {
-    constexpr int V = BF16 ? 8 : 4;
-    const u32x4 raw = reinterpret_cast<const u32x4 *>(row)[c];
-    float p[V], bb[V], ss[V], mm[V];
-    if constexpr (BF16) {
-      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  struct Params { float bb[V], ss[V], mm[V]; };  // bias, scale and mask of V consecutive features
+  __device__ __forceinline__ void load_params(int base, Params &pr) const {
+    auto load_vec = [&](const float *src, float (&dst)[V], float dflt) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) { p[2 * q] = __uint_as_float(w[q] << 16); p[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
-    } else {
-      p[0] = __uint_as_float(raw.x); p[1] = __uint_as_float(raw.y); p[2] = __uint_as_float(raw.z); p[3] = __uint_as_float(raw.w);
-    }
-    const int base = c * V;
-    auto load = [&](const float *src, float (&dst)[V], float dflt) {
-      if (src) {
+      for (int e = 0; e < V; ++e) dst[e] = dflt;
+      if (!src) return;
+      if (vec) {
+        const int sb = safe_base(base);
 #pragma unroll
         for (int q = 0; q < V / 4; ++q) {
-          const float4 t = reinterpret_cast<const float4 *>(src + base)[q];
+          const float4 t = reinterpret_cast<const float4 *>(src + sb)[q];
           dst[4 * q] = t.x; dst[4 * q + 1] = t.y; dst[4 * q + 2] = t.z; dst[4 * q + 3] = t.w;
         }
-      } else {
+      } else if (base >= 0) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) dst[e] = dflt;
+        for (int e = 0; e < V; ++e) if (base + e < F) dst[e] = src[base + e];
       }
     };
-    load(b_enc, bb, 0.f); load(scale, ss, 1.f); load(fmask, mm, 1.f);
+    load_vec(b_enc, pr.bb, 0.f); load_vec(scale, pr.ss, 1.f); load_vec(fmask, pr.mm, 1.f);
+  }
+  // keys of the V elements of row b from `base` on, with their bias, scale and mask already in registers
+  __device__ __forceinline__ void keys_with(int b, int base, const u32x4 &raw, const Params &pr, uint32_t (&keys)[V]) const {
+    float p[V];
+    if (vec) {
+      if constexpr (BF16) {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-    for (int e = 0; e < V; ++e) fn(base + e, bt_key(p[e], bb[e], ss[e], mm[e], fmask != nullptr));
+        for (int q = 0; q < 4; ++q) { p[2 * q] = __uint_as_float(w[q] << 16); p[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
+      } else {
+        p[0] = __uint_as_float(raw.x); p[1] = __uint_as_float(raw.y); p[2] = __uint_as_float(raw.z); p[3] = __uint_as_float(raw.w);
+      }
+    } else {
+      const char *row = row_ptr(b);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        p[e] = 0.f;
+        if (base >= 0 && base + e < F) {
+          if constexpr (BF16) p[e] = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[base + e]);
+          else p[e] = reinterpret_cast<const float *>(row)[base + e];
+        }
+      }
+    }
+    const bool inside = base >= 0 && base < F;
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      keys[e] = (inside && base + e < F) ? bt_key(p[e], pr.bb[e], pr.ss[e], pr.mm[e], fmask != nullptr) : 0u;
+  }
+  // the same, fetching bias, scale and mask
+  __device__ __forceinline__ void keys_of(int b, int base, const u32x4 &raw, uint32_t (&keys)[V]) const {
+    Params pr;
+    load_params(base, pr);
+    keys_with(b, base, raw, pr, keys);
+  }
+  // fn(base, keys) over the granules of row b whose largest key is >= bound, run by ONE wave: each call hands
+  // every lane the V keys from feature `base` on (base < 0: none, keys are 0) with bases ascending over the
+  // lanes and over the calls, and every lane takes part in every call, so fn may use cross-lane operations.
+  // `live` is BT_LIVE ints of LDS private to the wave.
+  template <typename Fn>
+  __device__ __forceinline__ void for_live_granules(int b, const uint32_t *__restrict__ gran_max_row, uint32_t bound,
+                                                    int *live, Fn fn) const {
+    const int lane = threadIdx.x & 63, part = lane / BT_GL;
+    for (int g0 = 0; g0 < ngran; g0 += BT_LIVE) {
+      // a lane looks at four consecutive granules; the list keeps them in ascending order
+      const int gl = g0 + lane * 4;
+      u32x4 mx = {0u, 0u, 0u, 0u};
+      if (gl < ngran) mx = *reinterpret_cast<const u32x4 *>(gran_max_row + gl);   // ngran is a multiple of 4
+      const bool a0 = mx.x >= bound, a1 = mx.y >= bound, a2 = mx.z >= bound, a3 = mx.w >= bound;   // bound >= 1
+      const unsigned long long m0 = __ballot(a0), m1 = __ballot(a1), m2 = __ballot(a2), m3 = __ballot(a3);
+      const unsigned long long below = (1ull << lane) - 1ull;
+      int r = __popcll(m0 & below) + __popcll(m1 & below) + __popcll(m2 & below) + __popcll(m3 & below);
+      if (a0) live[r++] = gl;
+      if (a1) live[r++] = gl + 1;
+      if (a2) live[r++] = gl + 2;
+      if (a3) live[r++] = gl + 3;   // same wave: LDS operations complete in order
+      const int n = __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+      __builtin_amdgcn_wave_barrier();
+      for (int i = 0; i < n; i += 4 * BT_GPW) {
+        int base[4];
+        u32x4 raw[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int j = i + BT_GPW * q + part;
+          base[q] = j < n ? lane_base(live[j]) : -1;
+          raw[q] = load_raw(b, base[q]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (i + BT_GPW * q < n) {
+            uint32_t keys[V];
+            keys_of(b, base[q], raw[q], keys);
+            fn(base[q], keys);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
 };
 
 __global__ void bt_init_kernel(BatchSelState *st, uint32_t *hist, int64_t k_host, const int64_t *k_dev) {
   for (int i = threadIdx.x; i < BT_BINS; i += blockDim.x) hist[i] = 0u;
   if (threadIdx.x == 0) {
-    st->prefix = 0u; st->mask = 0u; st->done = 0; st->n_positive = 0; st->threshold = 0u;
+    st->prefix = 0u; st->mask = 0u; st->done = 0; st->n_positive = 0; st->threshold = 0u; st->lower = 1u;
+    st->cand_count = 0ull; st->overflow = 0;
     st->k_total = k_dev ? *k_dev : k_host;
     st->remaining = st->k_total;
-    if (st->k_total <= 0) { st->done = 1; st->k_total = 0; st->remaining = 0; st->threshold = 0xffffffffu; }  // keep nothing
+    if (st->k_total <= 0) { st->done = 1; st->k_total = 0; st->remaining = 0; st->threshold = BT_KEEP_NOTHING; }
   }
 }
 
-// digit histogram of keys matching the current prefix; grid-stride over rows
+// The full pass: every granule's largest key and the histogram of the top 11 bits of those maxima.  At least as
+// many keys as granule maxima reach any given value, so the k_total-th largest maximum is a lower bound on the
+// k_total-th largest key.
 template <bool BF16>
-__global__ __launch_bounds__(BT_THREADS) void bt_hist_kernel(BatchReader<BF16> rd, int B, const BatchSelState *st,
-                                                             uint32_t *__restrict__ hist, int shift, int bits) {
-  extern __shared__ uint32_t bt_lds[];  // BT_WAVES private histograms of (1 << bits) bins
-  const int nb = 1 << bits;
-  if (st->done) return;
-  for (int i = threadIdx.x; i < nb * BT_WAVES; i += BT_THREADS) bt_lds[i] = 0u;
+__global__ __launch_bounds__(BT_THREADS) void bt_first_kernel(BatchReader<BF16> rd, int B, int rows_per_wg, const BatchSelState *st,
+                                                              uint32_t *__restrict__ hist, uint32_t *__restrict__ gran_max) {
+  __shared__ uint32_t h[BT_BINS];
+  constexpr int V = BatchReader<BF16>::V;
+  if (st->done) return;  // k_total <= 0: nothing is kept and the maxima are never read
+  for (int i = threadIdx.x; i < BT_BINS; i += BT_THREADS) h[i] = 0u;
   __syncthreads();
-  uint32_t *mine = bt_lds + (threadIdx.x >> 6) * nb;
-  const uint32_t prefix = st->prefix, mask = st->mask, dm = (uint32_t)nb - 1u;
-  for (int b = blockIdx.x; b < B; b += gridDim.x) {
-    rd.row_for_each(b, [&](int, uint32_t key) {
-      if (key != 0u && (key & mask) == prefix) atomicAdd(&mine[(key >> shift) & dm], 1u);
-    });
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // A wave owns ONE 64-lane segment of the columns and walks rows_per_wg rows of it, so bias, scale and mask
+  // are fetched once and stay in registers; four rows' loads are in flight at a time.
+  const int s = blockIdx.x * BT_WAVES + wave;
+  const int r0 = blockIdx.y * rows_per_wg, r1 = r0 + rows_per_wg < B ? r0 + rows_per_wg : B;
+  if (s < rd.nseg) {
+    const int base = (s * 64 + lane) * V;
+    const int g = s * BT_GPW + lane / BT_GL;
+    typename BatchReader<BF16>::Params pr;
+    rd.load_params(base, pr);
+    for (int r = r0; r < r1; r += 4) {
+      u32x4 raw[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) raw[q] = rd.load_raw(r + q < r1 ? r + q : r, base);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (r + q < r1) {
+          uint32_t keys[V];
+          rd.keys_with(r + q, base, raw[q], pr, keys);
+          uint32_t mx = 0u;
+#pragma unroll
+          for (int e = 0; e < V; ++e) mx = keys[e] > mx ? keys[e] : mx;
+#pragma unroll
+          for (int o = BT_GL / 2; o > 0; o >>= 1) { const uint32_t t = (uint32_t)__shfl_xor((int)mx, o, 64); mx = t > mx ? t : mx; }
+          if ((lane & (BT_GL - 1)) == 0 && g < rd.ngran) {
+            gran_max[(size_t)(r + q) * rd.ngran + g] = mx;
+            if (mx) atomicAdd(&h[mx >> 20], 1u);
+          }
+        }
+      }
+    }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += BT_THREADS) {
-    uint32_t s = 0;
+  for (int i = threadIdx.x; i < BT_BINS; i += BT_THREADS)
+    if (h[i]) atomicAdd(&hist[i], h[i]);
+}
+
+constexpr int BT_TOKENS_PER_WG = 4;  // gather, next, count, emit: one wave per token
+
+struct BatchCandidates {     // the keys >= lower, token by token, each token's in ascending feature order
+  uint32_t *key;
+  int32_t *feat;
+  uint32_t *tok_start;       // where token b's candidates begin
+  int32_t *tok_cnt;
+  int64_t cap;
+};
+
+// per token: the keys that reach the lower bound, with their features, appended to the candidate list.  The wave
+// collects them in LDS, reserves their place with one atomic and copies them out; a token with more than
+// BT_STASH of them walks its granules a second time and writes directly.
+template <bool BF16>
+__global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_gather_kernel(BatchReader<BF16> rd, int B, BatchSelState *st,
+                                                                          const uint32_t *__restrict__ gran_max,
+                                                                          BatchCandidates cd) {
+  __shared__ int live[BT_TOKENS_PER_WG * BT_LIVE];
+  __shared__ uint32_t stash_key[BT_TOKENS_PER_WG * BT_STASH];
+  __shared__ int32_t stash_feat[BT_TOKENS_PER_WG * BT_STASH];
+  constexpr int V = BatchReader<BF16>::V;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int b = blockIdx.x * BT_TOKENS_PER_WG + wave;
+  if (b >= B) return;
+  if (st->threshold == BT_KEEP_NOTHING) return;
+  const uint32_t lower = st->lower;   // 1 when every positive key is kept
+  uint32_t *my_key = stash_key + wave * BT_STASH;
+  int32_t *my_feat = stash_feat + wave * BT_STASH;
+  unsigned long long start = 0;
+  int n = 0;
+  for (int pass = 0; pass < 2; ++pass) {
+    n = 0;   // candidates of this token before the current call; the same in every lane
+    rd.for_live_granules(b, gran_max + (size_t)b * rd.ngran, lower, live + wave * BT_LIVE, [&](int base, const uint32_t (&keys)[V]) {
+      int mine = 0;
 #pragma unroll
-    for (int w = 0; w < BT_WAVES; ++w) s += bt_lds[w * nb + i];
-    if (s) atomicAdd(&hist[i], s);
+      for (int e = 0; e < V; ++e) mine += keys[e] >= lower;
+      int inc = mine;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += t;
+      }
+      int pos = n + inc - mine;
+      if (mine) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          if (keys[e] >= lower) {
+            if (pass == 0) {
+              if (pos < BT_STASH) { my_key[pos] = keys[e]; my_feat[pos] = base + e; }
+            } else {
+              cd.key[start + pos] = keys[e]; cd.feat[start + pos] = base + e;
+            }
+            ++pos;
+          }
+        }
+      }
+      n += __shfl(inc, 63, 64);
+    });
+    if (pass == 1) break;
+    if (lane == 0) start = atomicAdd(&st->cand_count, (unsigned long long)n);
+    start = __shfl((long long)start, 0, 64);
+    const bool fits = start + (unsigned long long)n <= (unsigned long long)cd.cap;
+    if (lane == 0) {
+      cd.tok_start[b] = fits ? (uint32_t)start : 0u;
+      cd.tok_cnt[b] = fits ? n : 0;
+      if (!fits) st->overflow = 1;
+    }
+    if (!fits) break;
+    if (n <= BT_STASH) {
+      __builtin_amdgcn_wave_barrier();
+      for (int i = lane; i < n; i += 64) { cd.key[start + i] = my_key[i]; cd.feat[start + i] = my_feat[i]; }
+      break;
+    }
   }
 }
 
-// one workgroup: choose the digit in which the running count (from the top bin down) reaches `remaining`
+// digit histogram of the keys matching the prefix found so far: over the candidate list, or, when that
+// overflowed, over the granules of the matrix that can hold such a key
+template <bool BF16>
+__global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_next_kernel(BatchReader<BF16> rd, int B, const BatchSelState *st,
+                                                                        uint32_t *__restrict__ hist,
+                                                                        const uint32_t *__restrict__ gran_max,
+                                                                        BatchCandidates cd, int shift, int bits) {
+  __shared__ uint32_t h[BT_BINS];
+  __shared__ int live[BT_TOKENS_PER_WG * BT_LIVE];
+  constexpr int V = BatchReader<BF16>::V;
+  if (st->done) return;
+  const int nb = 1 << bits;
+  for (int i = threadIdx.x; i < nb; i += blockDim.x) h[i] = 0u;
+  __syncthreads();
+  const uint32_t prefix = st->prefix, mask = st->mask, dm = (uint32_t)nb - 1u, lower = st->lower;
+  if (!st->overflow) {
+    // the list is short: a few workgroups read it (four keys in flight per thread), so that few partial
+    // histograms reach the global one
+    constexpr int LIST_WGS = 128;
+    if (blockIdx.x >= LIST_WGS) return;
+    const int64_t n = (int64_t)st->cand_count;
+    const int64_t stride = (int64_t)(gridDim.x < LIST_WGS ? gridDim.x : LIST_WGS) * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += 4 * stride) {
+      uint32_t key[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) key[q] = cd.key[i + q * stride < n ? i + q * stride : n - 1];   // unconditional loads
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (i + q * stride < n && (key[q] & mask) == prefix) atomicAdd(&h[(key[q] >> shift) & dm], 1u);
+    }
+  } else {
+    // every key that matches is >= prefix (its undecided bits are >= 0); keys below `lower` cannot be the threshold
+    const uint32_t bound = prefix > lower ? prefix : lower;
+    const int b = blockIdx.x * BT_TOKENS_PER_WG + (threadIdx.x >> 6);
+    if (b < B) {
+      rd.for_live_granules(b, gran_max + (size_t)b * rd.ngran, bound, live + (threadIdx.x >> 6) * BT_LIVE, [&](int, const uint32_t (&keys)[V]) {
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          if (keys[e] >= lower && (keys[e] & mask) == prefix) atomicAdd(&h[(keys[e] >> shift) & dm], 1u);
+      });
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nb; i += blockDim.x)
+    if (h[i]) atomicAdd(&hist[i], h[i]);
+}
+
+// inclusive prefix sum over the 1024 threads of a workgroup (wsum: BT_WAVES values of LDS)
+__device__ __forceinline__ int64_t bt_block_scan(int64_t v, int64_t *wsum) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int64_t t = __shfl_up((long long)v, o, 64);
+    if (lane >= o) v += t;
+  }
+  if (lane == 63) wsum[wave] = v;
+  __syncthreads();
+  int64_t base = 0;
+  for (int w = 0; w < wave; ++w) base += wsum[w];
+  __syncthreads();
+  return v + base;
+}
+
+// Walking the nb bins from the top down, the bin in which the running count reaches `target` (> 0), and the rank
+// wanted inside that bin; *bin stays -1 when the histogram holds fewer than `target`.  One workgroup of 1024.
+__device__ __forceinline__ void bt_find_from_top(const uint32_t *hist, int nb, int64_t target, int64_t *wsum, int *bin,
+                                                 int64_t *need_out) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *bin = -1;
+  const int per = (nb + 1023) / 1024;  // thread t owns the bins nb - 1 - (t * per + e)
+  int64_t local = 0;
+  for (int e = 0; e < per; ++e) { const int i = nb - 1 - (tid * per + e); if (i >= 0) local += hist[i]; }
+  const int64_t incl = bt_block_scan(local, wsum);  // its barriers also order the write of *bin above
+  const int64_t excl = incl - local;
+  if (excl < target && incl >= target) {
+    int64_t need = target - excl;
+    for (int e = 0; e < per; ++e) {
+      const int i = nb - 1 - (tid * per + e);
+      if (i < 0) break;
+      const int64_t c = hist[i];
+      if (c >= need) { *bin = i; *need_out = need; break; }
+      need -= c;
+    }
+  }
+  __syncthreads();
+}
+
+// one workgroup, after the full pass: the key from which the search starts
+__global__ __launch_bounds__(1024) void bt_bound_kernel(BatchSelState *st, uint32_t *hist) {
+  __shared__ int64_t wsum[BT_WAVES];
+  __shared__ int bin;
+  __shared__ int64_t need;
+  const int tid = threadIdx.x;
+  if (st->done) { for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u; return; }
+  bt_find_from_top(hist, BT_BINS, st->k_total, wsum, &bin, &need);
+  // k_total granules have a maximum in this bin or above, so the threshold is at least the bin's lower edge;
+  // with fewer positive maxima than k_total (bin < 0) every positive key is a candidate
+  if (tid == 0) st->lower = bin > 0 ? ((uint32_t)bin) << 20 : 1u;
+  for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u;  // the key histograms start from zero
+}
+
+// one workgroup: choose the digit in which the running count (from the top bin down) reaches `remaining`.
+// The first of the three also settles the case of fewer positives than k_total: then the lower bound is 1, the
+// gather pass has met every positive key, and all of them are kept.
 __global__ __launch_bounds__(1024) void bt_pick_kernel(BatchSelState *st, uint32_t *hist, int shift, int bits, int first) {
-  __shared__ int64_t part[1024];
-  __shared__ int chosen;
+  __shared__ int64_t wsum[BT_WAVES];
+  __shared__ int bin;
+  __shared__ int64_t need;
   const int nb = 1 << bits, tid = threadIdx.x;
   if (st->done) { for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u; return; }
-  // thread t owns bins [hi - 2t - 1 ... ] from the top: with 2048 bins and 1024 threads, 2 bins each
-  const int per = (nb + 1023) / 1024;
-  int64_t local = 0;
-  for (int e = 0; e < per; ++e) { const int bin = nb - 1 - (tid * per + e); if (bin >= 0) local += hist[bin]; }
-  part[tid] = local;
-  __syncthreads();
-  for (int o = 1; o < 1024; o <<= 1) {
-    const int64_t v = tid >= o ? part[tid - o] : 0;
-    __syncthreads();
-    part[tid] += v;
-    __syncthreads();
-  }
-  const int64_t total = part[1023];
-  if (tid == 0) chosen = -1;
-  __syncthreads();
-  // decisions taken by thread 0 travel through LDS (a global flag re-read by the other waves could come
-  // from a stale scalar-cache line)
-  __shared__ int sh_done;
-  __shared__ int64_t sh_remaining;
+  const int64_t n_cand = (int64_t)st->cand_count, k_total = st->k_total;
+  const bool keep_all = first && st->lower == 1u && n_cand <= k_total;   // the same in every thread
+  bt_find_from_top(hist, nb, st->remaining, wsum, &bin, &need);
   if (tid == 0) {
-    int done = 0;
-    if (first) {
-      st->n_positive = total;
-      if (total <= st->k_total) {  // fewer positives than k: keep every positive
-        st->done = 1; st->k_total = total; st->prefix = 0u; st->mask = 0u; st->remaining = 0; st->threshold = 0u;
-        done = 1;
-      }
-    }
-    sh_done = done;
-    sh_remaining = st->remaining;
-  }
-  __syncthreads();
-  if (!sh_done) {
-    const int64_t remaining = sh_remaining;
-    const int64_t excl = part[tid] - local;
-    if (excl < remaining && part[tid] >= remaining) {
-      int64_t need = remaining - excl;
-      for (int e = 0; e < per; ++e) {
-        const int bin = nb - 1 - (tid * per + e);
-        if (bin < 0) break;
-        const int64_t h = hist[bin];
-        if (h >= need) { chosen = bin; st->remaining = need; break; }
-        need -= h;
-      }
+    if (first) st->n_positive = st->lower == 1u ? n_cand : -1;   // known only when every positive is a candidate
+    if (keep_all) {
+      st->done = 1; st->k_total = n_cand; st->prefix = 0u; st->mask = 0u; st->remaining = 0; st->threshold = 0u;
+    } else if (bin >= 0) {
+      st->remaining = need;
+      st->prefix |= ((uint32_t)bin) << shift;
+      st->mask |= ((uint32_t)(nb - 1)) << shift;
+      if (shift == 0) st->threshold = st->prefix;
     }
   }
-  __syncthreads();
-  if (tid == 0 && chosen >= 0) {
-    st->prefix |= ((uint32_t)chosen) << shift;
-    st->mask |= ((uint32_t)(nb - 1)) << shift;
-    if (shift == 0) st->threshold = st->prefix;
-  }
-  __syncthreads();
   for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u;  // ready for the next pass
 }
 
 // per token: how many keys are above the threshold, how many equal it
 template <bool BF16>
-__global__ __launch_bounds__(BT_THREADS) void bt_count_kernel(BatchReader<BF16> rd, const BatchSelState *st,
-                                                              int32_t *__restrict__ n_gt, int32_t *__restrict__ n_tie) {
-  __shared__ int red[2 * BT_WAVES];
-  const int b = blockIdx.x;
+__global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_count_kernel(BatchReader<BF16> rd, int B, const BatchSelState *st,
+                                                                         const uint32_t *__restrict__ gran_max,
+                                                                         BatchCandidates cd, int32_t *__restrict__ n_gt,
+                                                                         int32_t *__restrict__ n_tie) {
+  __shared__ int live[BT_TOKENS_PER_WG * BT_LIVE];
+  constexpr int V = BatchReader<BF16>::V;
+  const int b = blockIdx.x * BT_TOKENS_PER_WG + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (b >= B) return;
   const uint32_t T = st->threshold;
   int gt = 0, tie = 0;
-  rd.row_for_each(b, [&](int, uint32_t key) { gt += key > T; tie += (key == T) && key != 0u; });
-  gt = wave_sum_i(gt); tie = wave_sum_i(tie);
-  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = gt; red[BT_WAVES + (threadIdx.x >> 6)] = tie; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int a = 0, c = 0;
-    for (int w = 0; w < BT_WAVES; ++w) { a += red[w]; c += red[BT_WAVES + w]; }
-    n_gt[b] = a; n_tie[b] = c;
+  if (T == BT_KEEP_NOTHING) {
+  } else if (!st->overflow) {
+    const uint32_t *keys = cd.key + cd.tok_start[b];
+    const int n = cd.tok_cnt[b];
+    for (int i = lane; i < n; i += 64) { const uint32_t k = keys[i]; gt += k > T; tie += k == T; }
+  } else {
+    rd.for_live_granules(b, gran_max + (size_t)b * rd.ngran, T ? T : 1u, live + (threadIdx.x >> 6) * BT_LIVE, [&](int, const uint32_t (&keys)[V]) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) { gt += keys[e] > T; tie += (keys[e] == T) && keys[e] != 0u; }
+    });
   }
+  gt = wave_sum_i(gt); tie = wave_sum_i(tie);
+  if (lane == 0) { n_gt[b] = gt; n_tie[b] = tie; }
 }
 
-// one workgroup: row offsets and per-token tie allowance (first `need` ties in flattened order)
+// one workgroup: row offsets and per-token tie allowance (first `need` ties in flattened order).
+// Thread t owns the tokens [t * per, (t + 1) * per).
 __global__ __launch_bounds__(1024) void bt_plan_kernel(const BatchSelState *st, const int32_t *__restrict__ n_gt,
                                                        const int32_t *__restrict__ n_tie, int B,
                                                        int32_t *__restrict__ tie_keep, int64_t *__restrict__ row_off,
                                                        int32_t *__restrict__ row_nnz, int64_t *__restrict__ total_out) {
-  __shared__ int64_t part[1024];
-  __shared__ int64_t carry_tie, carry_off;
+  __shared__ int64_t wsum[BT_WAVES];
   const int tid = threadIdx.x;
   const int64_t need = st->done ? 0 : st->remaining;  // threshold ties that belong to the top k_total
-  if (tid == 0) { carry_tie = 0; carry_off = 0; }
-  __syncthreads();
-  for (int b0 = 0; b0 < B; b0 += 1024) {
-    const int b = b0 + tid;
-    // exclusive scan of tie counts over this chunk of tokens
-    const int64_t t = b < B ? n_tie[b] : 0;
-    part[tid] = t;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) { const int64_t v = tid >= o ? part[tid - o] : 0; __syncthreads(); part[tid] += v; __syncthreads(); }
-    const int64_t ties_before = carry_tie + part[tid] - t;
-    const int64_t chunk_ties = part[1023];
-    __syncthreads();
-    int64_t keep = need - ties_before;
-    keep = keep < 0 ? 0 : (keep > t ? t : keep);
-    const int64_t nnz = b < B ? (int64_t)n_gt[b] + keep : 0;
-    part[tid] = nnz;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) { const int64_t v = tid >= o ? part[tid - o] : 0; __syncthreads(); part[tid] += v; __syncthreads(); }
-    if (b < B) { tie_keep[b] = (int32_t)keep; row_nnz[b] = (int32_t)nnz; row_off[b] = carry_off + part[tid] - nnz; }
-    const int64_t chunk_nnz = part[1023];
-    __syncthreads();
-    if (tid == 0) { carry_tie += chunk_ties; carry_off += chunk_nnz; }
-    __syncthreads();
+  const int64_t per = ((int64_t)B + 1023) / 1024;
+  const int lo = (int)(tid * per < B ? tid * per : B), hi = (int)(lo + per < B ? lo + per : B);
+  // The three walks below take a thread's tokens eight at a time.  Their loads are unconditional (a slot past
+  // the thread's range re-reads its last token and is masked afterwards): loads under a per-lane condition
+  // would each be followed by a wait for memory.
+  const int last = hi > lo ? hi - 1 : 0;   // B >= 1, so token 0 exists
+  int64_t ties = 0;
+  for (int c = lo; c < hi; c += 8) {
+    int32_t t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = n_tie[c + j < hi ? c + j : last];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ties += c + j < hi ? t[j] : 0;
   }
-  if (tid == 0 && total_out) *total_out = carry_off;
+  int64_t ties_before = bt_block_scan(ties, wsum) - ties;
+  int64_t nnz_sum = 0;
+  for (int c = lo; c < hi; c += 8) {
+    int32_t t[8], g[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { const int b = c + j < hi ? c + j : last; t[j] = n_tie[b]; g[j] = n_gt[b]; }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (c + j < hi) {
+        int64_t keep = need - ties_before;
+        keep = keep < 0 ? 0 : (keep > t[j] ? t[j] : keep);
+        ties_before += t[j];
+        const int64_t nnz = (int64_t)g[j] + keep;
+        tie_keep[c + j] = (int32_t)keep; row_nnz[c + j] = (int32_t)nnz;
+        nnz_sum += nnz;
+      }
+    }
+  }
+  const int64_t incl = bt_block_scan(nnz_sum, wsum);
+  int64_t off = incl - nnz_sum;
+  for (int c = lo; c < hi; c += 8) {
+    int32_t z[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z[j] = row_nnz[c + j < hi ? c + j : last];   // this thread's own stores above
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { if (c + j < hi) { row_off[c + j] = off; off += z[j]; } }
+  }
+  if (tid == 1023 && total_out) *total_out = incl;
 }
 
 // per token: ordered compaction of the kept elements
 template <bool BF16>
-__global__ __launch_bounds__(BT_THREADS) void bt_emit_kernel(BatchReader<BF16> rd, const BatchSelState *st,
-                                                             const int32_t *__restrict__ tie_keep,
-                                                             const int64_t *__restrict__ row_off,
-                                                             int32_t *__restrict__ idx_out, float *__restrict__ val_out,
-                                                             int64_t capacity) {
-  __shared__ int wsum_sel[BT_WAVES], wsum_tie[BT_WAVES];
-  __shared__ int run_sel, run_tie;
-  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_emit_kernel(BatchReader<BF16> rd, int B, const BatchSelState *st,
+                                                                        const uint32_t *__restrict__ gran_max,
+                                                                        BatchCandidates cd,
+                                                                        const int32_t *__restrict__ tie_keep,
+                                                                        const int64_t *__restrict__ row_off,
+                                                                        int32_t *__restrict__ idx_out,
+                                                                        float *__restrict__ val_out, int64_t capacity) {
+  __shared__ int live[BT_TOKENS_PER_WG * BT_LIVE];
+  constexpr int V = BatchReader<BF16>::V;
+  const int b = blockIdx.x * BT_TOKENS_PER_WG + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (b >= B) return;
   const uint32_t T = st->threshold;
+  if (T == BT_KEEP_NOTHING) return;
   const int keep_ties = tie_keep[b];
   const int64_t off = row_off[b];
-  const char *row = reinterpret_cast<const char *>(rd.pre) + (size_t)b * rd.F * (BF16 ? 2 : 4);
-  if (tid == 0) { run_sel = 0; run_tie = 0; }
-  __syncthreads();
-  constexpr int V = BF16 ? 8 : 4;
-  const int F = rd.F;
-  const bool vec_ok = (F % V == 0) && ((((uintptr_t)row | (uintptr_t)rd.b_enc | (uintptr_t)rd.scale | (uintptr_t)rd.fmask) & 15) == 0);
-  const int per_thread = vec_ok ? V : 1;
-  const int chunk_elems = BT_THREADS * per_thread;
-  for (int c0 = 0; c0 < F; c0 += chunk_elems) {
-    // thread tid owns elements [c0 + tid * per_thread, + per_thread): contiguous, so thread order == index order
-    uint32_t keys[V];
-    int n_mine = 0;
-    const int base = c0 + tid * per_thread;
-    if (vec_ok) {
-      if (base < F) { rd.chunk(row, base / V, [&](int i, uint32_t k) { keys[i - base] = k; }); n_mine = V; }
-    } else if (base < F) { keys[0] = rd.scalar_key(row, base); n_mine = 1; }
-    int my_gt_or_tie = 0, my_tie = 0;
-    for (int e = 0; e < n_mine; ++e) { my_tie += keys[e] == T && keys[e] != 0u; my_gt_or_tie += keys[e] > T; }
-    // block-wide exclusive scans (ties, and strictly-greater) in thread order
-    int inc_t = my_tie, inc_g = my_gt_or_tie;
+  int run_gt = 0, run_tie = 0;  // of this token, before the elements of the current call
+  // One call places up to 64 * N keys; lane l holds keys[e] with features feat0 + e, ascending over e, lanes and calls.
+  auto place = [&](int feat0, const auto &keys, auto n_const) {
+    constexpr int N = decltype(n_const)::value;
+    int mine = 0;  // keys above the threshold in the low half, ties in the high half (one call holds <= 512 keys)
+#pragma unroll
+    for (int e = 0; e < N; ++e) mine += (int)(keys[e] > T) + ((int)(keys[e] == T && keys[e] != 0u) << 16);
+    int inc = mine;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
-      const int a = __shfl_up(inc_t, o, 64), g = __shfl_up(inc_g, o, 64);
-      if (lane >= o) { inc_t += a; inc_g += g; }
+      const int a = __shfl_up(inc, o, 64);
+      if (lane >= o) inc += a;
     }
-    if (lane == 63) { wsum_tie[wave] = inc_t; wsum_sel[wave] = inc_g; }
-    __syncthreads();
-    int base_t = run_tie, base_g = 0, tot_t = 0, tot_g = 0;
+    const int total = __shfl(inc, 63, 64);
+    const int before = inc - mine;
+    int tie_rank = run_tie + (before >> 16);  // ties of this token before my first element
+    // kept elements before my first one: every greater key, and the first keep_ties ties
+    int pos = run_gt + (before & 0xffff) + (tie_rank < keep_ties ? tie_rank : keep_ties);
+    if (mine) {
 #pragma unroll
-    for (int w = 0; w < BT_WAVES; ++w) {
-      if (w < wave) { base_t += wsum_tie[w]; base_g += wsum_sel[w]; }
-      tot_t += wsum_tie[w]; tot_g += wsum_sel[w];
-    }
-    int tie_rank = base_t + inc_t - my_tie;   // ties of this token seen before my first element
-    // position among kept elements = kept greater-than before me + kept ties before me (+ row running total)
-    int gt_before = base_g + inc_g - my_gt_or_tie;
-    const int ties_kept_before = tie_rank < keep_ties ? tie_rank : keep_ties;
-    int pos = run_sel + gt_before + (ties_kept_before - (run_tie < keep_ties ? run_tie : keep_ties));
-    for (int e = 0; e < n_mine; ++e) {
-      const uint32_t k = keys[e];
-      bool keep = k > T;
-      if (k == T && k != 0u) { keep = tie_rank < keep_ties; ++tie_rank; }
-      if (keep) {
-        const int64_t o = off + pos;
-        if (o < capacity) {
-          const int f = base + e;
-          const float h1 = __uint_as_float(k);
-          idx_out[o] = f;
-          val_out[o] = rd.scale ? h1 / rd.scale[f] : h1;
+      for (int e = 0; e < N; ++e) {
+        const uint32_t k = keys[e];
+        bool keep = k > T;
+        if (k == T && k != 0u) { keep = tie_rank < keep_ties; ++tie_rank; }
+        if (keep) {
+          const int64_t o = off + pos;
+          if (o < capacity) {
+            const int f = feat0 + e;
+            const float h1 = __uint_as_float(k);
+            idx_out[o] = f;
+            val_out[o] = rd.scale ? h1 / rd.scale[f] : h1;
+          }
+          ++pos;
         }
-        ++pos;
       }
     }
-    __syncthreads();
-    if (tid == 0) {
-      const int kept_t_before = run_tie < keep_ties ? run_tie : keep_ties;
-      const int new_tie = run_tie + tot_t;
-      const int kept_t_after = new_tie < keep_ties ? new_tie : keep_ties;
-      run_sel += tot_g + (kept_t_after - kept_t_before);
-      run_tie = new_tie;
+    run_gt += total & 0xffff;
+    run_tie += total >> 16;
+  };
+  if (!st->overflow) {
+    const uint32_t *ck = cd.key + cd.tok_start[b];
+    const int32_t *cf = cd.feat + cd.tok_start[b];
+    const int n = cd.tok_cnt[b];
+    for (int i0 = 0; i0 < n; i0 += 64) {
+      const int i = i0 + lane;
+      const uint32_t one[1] = {i < n ? ck[i] : 0u};
+      place(i < n ? cf[i] : 0, one, std::integral_constant<int, 1>{});
     }
-    __syncthreads();
+  } else {
+    rd.for_live_granules(b, gran_max + (size_t)b * rd.ngran, T ? T : 1u, live + (threadIdx.x >> 6) * BT_LIVE,
+                         [&](int base, const uint32_t (&keys)[V]) { place(base, keys, std::integral_constant<int, V>{}); });
   }
 }
 
@@ -331,42 +624,55 @@ static int run_batch_select(const void *pre, const float *b_enc, const float *sc
                             int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
                             int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
                             hipStream_t st) {
+  constexpr int V = BatchReader<BF16>::V;
   char *ws = reinterpret_cast<char *>(workspace);
   BatchSelState *state = reinterpret_cast<BatchSelState *>(ws);
+  const bool vec = (F % V == 0) &&
+                   ((((uintptr_t)pre | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
+  const int nseg = (int)((F + 64 * V - 1) / (64 * V)), ngran = (int)((F + BT_GL * V - 1) / (BT_GL * V) + 3) / 4 * 4;
   uint32_t *hist = reinterpret_cast<uint32_t *>(ws + 256);
-  int32_t *n_gt = reinterpret_cast<int32_t *>(ws + 256 + BT_BINS * 4);
+  uint32_t *gran_max = reinterpret_cast<uint32_t *>(ws + 256 + BT_BINS * 4);   // 16-byte aligned rows
+  int32_t *n_gt = reinterpret_cast<int32_t *>(gran_max + B * ngran);
   int32_t *n_tie = n_gt + B;
   int32_t *tie_keep = n_tie + B;
-  BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F};
+  BatchCandidates cd;
+  cd.tok_start = reinterpret_cast<uint32_t *>(tie_keep + B);
+  cd.tok_cnt = reinterpret_cast<int32_t *>(cd.tok_start + B);
+  cd.cap = bt_candidate_capacity(B, F);
+  cd.key = reinterpret_cast<uint32_t *>(cd.tok_cnt + B);
+  cd.feat = reinterpret_cast<int32_t *>(cd.key + cd.cap);
+  BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F, vec ? 1 : 0, nseg, ngran};
   hipLaunchKernelGGL(bt_init_kernel, dim3(1), dim3(256), 0, st, state, hist, k_total, k_total_dev);
-  const unsigned hist_grid = (unsigned)(B < 1024 ? B : 1024);
+  const int rows_per_wg = (int)(B / 65535 > 16 ? B / 65535 + 1 : 16);
+  hipLaunchKernelGGL(bt_first_kernel<BF16>, dim3((unsigned)((nseg + BT_WAVES - 1) / BT_WAVES), (unsigned)((B + rows_per_wg - 1) / rows_per_wg)),
+                     dim3(BT_THREADS), 0, st, rd, (int)B, rows_per_wg, state, hist, gran_max);
+  hipLaunchKernelGGL(bt_bound_kernel, dim3(1), dim3(1024), 0, st, state, hist);
+  const unsigned token_grid = (unsigned)((B + BT_TOKENS_PER_WG - 1) / BT_TOKENS_PER_WG);
+  const dim3 token_block(BT_TOKENS_PER_WG * 64);
+  hipLaunchKernelGGL(bt_gather_kernel<BF16>, dim3(token_grid), token_block, 0, st, rd, (int)B, state, gran_max, cd);
   const int shifts[3] = {20, 9, 0}, bits[3] = {11, 11, 9};  // bits 30..20, 19..9, 8..0 (bit 31 is the sign: always 0)
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bt_hist_kernel<BF16>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (BT_WAVES << 11) * 4);
-    if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "select_topk_batch: LDS reservation failed: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
   for (int p = 0; p < 3; ++p) {
-    hipLaunchKernelGGL(bt_hist_kernel<BF16>, dim3(hist_grid), dim3(BT_THREADS), (size_t)(BT_WAVES << bits[p]) * 4, st, rd,
-                       (int)B, state, hist, shifts[p], bits[p]);
+    hipLaunchKernelGGL(bt_next_kernel<BF16>, dim3(token_grid), token_block, 0, st, rd, (int)B, state, hist, gran_max, cd,
+                       shifts[p], bits[p]);
     hipLaunchKernelGGL(bt_pick_kernel, dim3(1), dim3(1024), 0, st, state, hist, shifts[p], bits[p], p == 0 ? 1 : 0);
   }
-  hipLaunchKernelGGL(bt_count_kernel<BF16>, dim3((unsigned)B), dim3(BT_THREADS), 0, st, rd, state, n_gt, n_tie);
+  hipLaunchKernelGGL(bt_count_kernel<BF16>, dim3(token_grid), token_block, 0, st, rd, (int)B, state, gran_max, cd, n_gt, n_tie);
   hipLaunchKernelGGL(bt_plan_kernel, dim3(1), dim3(1024), 0, st, state, n_gt, n_tie, (int)B, tie_keep, row_off, row_nnz,
                      total_out);
-  hipLaunchKernelGGL(bt_emit_kernel<BF16>, dim3((unsigned)B), dim3(BT_THREADS), 0, st, rd, state, tie_keep, row_off, idx,
-                     val, capacity);
+  hipLaunchKernelGGL(bt_emit_kernel<BF16>, dim3(token_grid), token_block, 0, st, rd, (int)B, state, gran_max, cd, tie_keep,
+                     row_off, idx, val, capacity);
   return check_launch("select_topk_batch");
 }
 
 }  // namespace sae
 
 extern "C" int64_t sae_select_topk_batch_workspace_bytes(int64_t B, int64_t F) {
-  (void)F;
-  if (B <= 0) return 0;
-  return 256 + sae::BT_BINS * 4 + 3 * B * (int64_t)sizeof(int32_t) + 256;
+  if (B <= 0 || F <= 0) return 0;
+  // state, histogram, 5 per-token counters, the candidate list (key and feature), and one largest key per 256
+  // bytes of a row (sized for the shorter fp32 granules of 64 elements)
+  const int64_t ngran = ((F + sae::BT_GL * 4 - 1) / (sae::BT_GL * 4) + 3) / 4 * 4;
+  return 256 + sae::BT_BINS * 4 + 5 * B * (int64_t)sizeof(int32_t) + 8 * sae::bt_candidate_capacity(B, F) +
+         B * ngran * 4 + 256;
 }
 
 extern "C" int sae_select_topk_batch(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
@@ -376,7 +682,7 @@ extern "C" int sae_select_topk_batch(const void *pre, int pre_dtype, const float
                                      int64_t workspace_bytes, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_batch: null pointer");
-  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F < (1LL << 31), SAE_ERR_INVALID_ARG, "select_topk_batch: bad shape");
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F <= (1LL << 30), SAE_ERR_INVALID_ARG, "select_topk_batch: bad shape");
   SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_batch: bad dtype %d", pre_dtype);
   SAE_REQUIRE(k_total_dev || k_total >= 0, SAE_ERR_INVALID_ARG, "select_topk_batch: k_total must be >= 0");
   SAE_REQUIRE(capacity > 0, SAE_ERR_INVALID_ARG, "select_topk_batch: capacity must be positive");

@@ -408,7 +408,8 @@ def check_batch_select(pkg, oracle, dev, pre, b_enc, scale, k_total, feat_mask=N
     return code
 
 
-@pytest.mark.parametrize("B,F,k", [(9, 1000, 5), (64, 4096, 32), (8, 32768, 64), (3, 37, 4), (300, 512, 7)])
+@pytest.mark.parametrize("B,F,k", [(9, 1000, 5), (64, 4096, 32), (8, 32768, 64), (3, 37, 4), (300, 512, 7),
+                                   (2, 600064, 50), (2, 600001, 50)])   # more than 64 segments per wave; odd row length
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_select_topk_batch_random(pkg, oracle, dev, B, F, k, dtype):
     print(f"batchtopk B={B} F={F} k={k} {dtype}", flush=True)
@@ -435,6 +436,17 @@ def test_select_topk_batch_ties_and_degenerate(pkg, oracle, dev):
     check_batch_select(pkg, oracle, dev, pre, None, None, 0)                          # k_total = 0 keeps nothing
     bfq = torch.randn(B, F, generator=g).bfloat16()                                   # bf16-quantised: natural ties
     check_batch_select(pkg, oracle, dev, bfq, None, None, 64 * B)
+    # more keys at the threshold's level than the candidate list holds (B * F / 64 + 1024): the select then
+    # re-reads the matrix; one token alone holds more of them than a wave collects at a time (512)
+    wide = torch.randint(0, 3, (40, 8192), generator=g).float()
+    wide[7] = 2.0
+    for k_total in (50, 9000, 120000):
+        check_batch_select(pkg, oracle, dev, wide, None, None, k_total)
+    # the list holds them, but one token has more than 512: it is walked twice
+    peaked = torch.randn(40, 8192, generator=g)
+    peaked[11, 1000:3000] += 10.0
+    check_batch_select(pkg, oracle, dev, peaked, None, None, 2500)
+    check_batch_select(pkg, oracle, dev, peaked.bfloat16(), None, None, 2500)
 
 
 def test_select_topk_batch_feature_mask(pkg, oracle, dev):
