@@ -118,7 +118,9 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
  *   idx/val have room for `capacity` entries (entries beyond it are dropped; k_total is the
  *     natural capacity); row_off/row_nnz [B] describe the variable-length rows; total_out
  *     (nullable, device int64) receives the number of kept entries.
- * workspace: sae_select_topk_batch_workspace_bytes(B, F), 256-byte aligned.
+ * workspace: sae_select_topk_batch_workspace_bytes(B, F) bytes, 256-byte aligned: about B * F / 4 bytes
+ *   (one largest key per 32 elements, and a candidate list of B * F / 64 + 1024 keys with their features);
+ *   F <= 2^30.
  * Replaces the batchtopk closure (models/sparse_dictionary.py:761-794) + utils/math.py:81-171
  * with dim=(-2,-1), and the dead-latent select of the aux-k loss (sparse_dictionary.py:952-972). */
 int64_t sae_select_topk_batch_workspace_bytes(int64_t B, int64_t F);
