@@ -261,6 +261,24 @@ int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slo
                                 const int32_t *extra_map, const float *extra_rows, const float *extra_bias,
                                 void *stream);
 
+/* [rows, cols] fp32 or bf16 -> bf16 [cols, rows] (round to nearest even).
+ *   mask (nullable, fp32 [rows, cols]): entries whose mask is not positive are written as 0;
+ *   col_part (nullable, fp32 [ceil(rows / 64), cols]): per 64-row tile, the column sums of the (masked) fp32
+ *     values, in a fixed order; summing its rows (sae_col_sum) gives the column sums of the masked matrix.
+ * The operands autograd transposes inside the backward of the aux-k products (`aux_acts @ W_D` and the encoder
+ * product over the dead features, models/sparse_dictionary.py:952-991): A^T, G^T, x^T for dW = A^T G, and
+ * d pre^T = (dA masked to the kept entries)^T with its column sums = the dead features' bias gradient. */
+int sae_transpose_to_bf16(const void *src, int src_dtype, const float *mask, int64_t rows, int64_t cols, void *dst,
+                          float *col_part, void *stream);
+
+/* Sparse code -> dense [B, n_cols] rows, in fp32 and / or bf16 (either pointer may be null, not both): token b's
+ * entries idx/val[row_off[b] .. row_off[b] + row_nnz[b]) at their columns, zeros elsewhere; indices outside
+ * [0, n_cols) are dropped.  A token's indices must be distinct.
+ * The reference's TopK / BatchTopK activation returns this dense matrix (utils/math.py:81-171 scatter); here it is
+ * wanted only for the compact block of dead features of the aux-k term (models/sparse_dictionary.py:952-972). */
+int sae_code_to_dense(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
+                      int64_t n_cols, float *dense_f32, void *dense_bf16, void *stream);
+
 /* ---- Activation batches from a shuffle buffer -----------------------------------------------------------
  * dst[i, :] = cast(scale * src[row_idx[i], :]) for i < n_rows: one batch drawn from a token buffer that
  * stays where it is in HBM.  Replaces ActivationBuffer.shuffle / yield_batch

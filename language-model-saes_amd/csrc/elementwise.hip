@@ -149,6 +149,122 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const void *__restrict
   }
 }
 
+// [rows, cols] fp32 or bf16 -> bf16 [cols, rows] through a 64 x 64 LDS tile.  With `mask` (fp32 [rows, cols]) an
+// entry whose mask is not positive is written as 0.  With `col_part` the tile's column sums of the (masked)
+// fp32 values go to col_part[tile_row, col]: summing those rows gives the column sums in a fixed order.
+// VEC: rows and cols are multiples of 8 and the pointers 16-byte aligned, so every access is a whole vector.
+template <bool SRC_BF16, bool VEC>
+__global__ __launch_bounds__(256) void transpose_to_bf16_kernel(const void *__restrict__ src, const float *__restrict__ mask,
+                                                                int64_t rows, int64_t cols, uint16_t *__restrict__ dst,
+                                                                float *__restrict__ col_part) {
+  __shared__ float tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const int tid = threadIdx.x;
+  if constexpr (VEC) {
+    constexpr int W = SRC_BF16 ? 8 : 4;          // elements per 16-byte load
+    constexpr int TX = 64 / W, RP = 256 / TX;    // threads across a tile row, tile rows per pass
+    const int tx = tid % TX, ty = tid / TX;
+#pragma unroll
+    for (int p = 0; p < 64 / RP; ++p) {
+      const int i = ty + p * RP;
+      const int64_t r = r0 + i, c = c0 + tx * W;
+      float v[W];
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = 0.f;
+      if (r < rows && c < cols) {
+        const u32x4 raw = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(src) + (r * cols + c) * (SRC_BF16 ? 2 : 4));
+        if constexpr (SRC_BF16) {
+          const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) { v[2 * q] = __uint_as_float(w[q] << 16); v[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
+        } else {
+          v[0] = __uint_as_float(raw.x); v[1] = __uint_as_float(raw.y); v[2] = __uint_as_float(raw.z); v[3] = __uint_as_float(raw.w);
+        }
+        if (mask) {
+#pragma unroll
+          for (int q = 0; q < W / 4; ++q) {
+            const float4 m = *reinterpret_cast<const float4 *>(mask + r * cols + c + 4 * q);
+            if (!(m.x > 0.f)) v[4 * q] = 0.f;
+            if (!(m.y > 0.f)) v[4 * q + 1] = 0.f;
+            if (!(m.z > 0.f)) v[4 * q + 2] = 0.f;
+            if (!(m.w > 0.f)) v[4 * q + 3] = 0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < W; ++e) tile[i][tx * W + e] = v[e];
+    }
+  } else {
+    const int tx = tid & 63, ty = tid >> 6;
+    for (int i = ty; i < 64; i += 4) {
+      const int64_t r = r0 + i, c = c0 + tx;
+      float v = 0.f;
+      if (r < rows && c < cols) {
+        if constexpr (SRC_BF16) v = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(src)[r * cols + c]);
+        else v = reinterpret_cast<const float *>(src)[r * cols + c];
+        if (mask && !(mask[r * cols + c] > 0.f)) v = 0.f;
+      }
+      tile[i][tx] = v;
+    }
+  }
+  __syncthreads();
+  if (col_part && tid < 64 && c0 + tid < cols) {
+    float s = 0.f;
+#pragma unroll 8
+    for (int i = 0; i < 64; ++i) s += tile[i][tid];   // rows past the matrix hold 0
+    col_part[(int64_t)blockIdx.y * cols + c0 + tid] = s;
+  }
+  if constexpr (VEC) {
+    const int tx = tid & 7, ty = tid >> 3;   // 8 threads write the 64 bf16 of one output row
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const int cc = ty + 32 * p;
+      const int64_t c = c0 + cc, r = r0 + tx * 8;
+      if (c < cols && r < rows) {
+        u32x4 o;
+        o.x = ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 0][cc]) | ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 1][cc]) << 16));
+        o.y = ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 2][cc]) | ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 3][cc]) << 16));
+        o.z = ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 4][cc]) | ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 5][cc]) << 16));
+        o.w = ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 6][cc]) | ((uint32_t)f32_to_bf16_bits(tile[tx * 8 + 7][cc]) << 16));
+        *reinterpret_cast<u32x4 *>(dst + c * rows + r) = o;
+      }
+    }
+  } else {
+    const int tx = tid & 63, ty = tid >> 6;
+    for (int i = ty; i < 64; i += 4) {
+      const int64_t c = c0 + i, r = r0 + tx;
+      if (c < cols && r < rows) dst[c * rows + r] = f32_to_bf16_bits(tile[tx][i]);
+    }
+  }
+}
+
+// One workgroup per token: the token's sparse row (idx, val in slots row_off[b] .. + row_nnz[b]) written out as a
+// dense row of n_cols entries, in fp32 and / or bf16.  The row is assembled in LDS 8192 columns at a time, so every
+// global write is coalesced; indices outside [0, n_cols) are dropped.
+constexpr int C2D_CHUNK = 8192;
+__global__ __launch_bounds__(256) void code_to_dense_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
+                                                            const int64_t *__restrict__ row_off,
+                                                            const int32_t *__restrict__ row_nnz, int64_t n_cols,
+                                                            float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
+  __shared__ float row[C2D_CHUNK];
+  const int64_t b = blockIdx.x;
+  const int64_t off = row_off[b];
+  const int n = row_nnz[b], tid = threadIdx.x;
+  for (int64_t c0 = 0; c0 < n_cols; c0 += C2D_CHUNK) {
+    const int w = (int)(n_cols - c0 < C2D_CHUNK ? n_cols - c0 : C2D_CHUNK);
+    for (int i = tid; i < w; i += 256) row[i] = 0.f;
+    __syncthreads();
+    for (int s = tid; s < n; s += 256) {
+      const int64_t j = (int64_t)idx[off + s] - c0;
+      if (j >= 0 && j < w) row[j] = val[off + s];   // a token's indices are distinct
+    }
+    __syncthreads();
+    if (out_f32) for (int i = tid; i < w; i += 256) out_f32[b * n_cols + c0 + i] = row[i];
+    if (out_bf16) for (int i = tid; i < w; i += 256) out_bf16[b * n_cols + c0 + i] = f32_to_bf16_bits(row[i]);
+    __syncthreads();
+  }
+}
+
 }  // namespace sae
 
 extern "C" int sae_gather_rows(const void *src, int src_dtype, const int64_t *row_idx, int64_t n_src_rows, int64_t n_rows,
@@ -171,6 +287,40 @@ extern "C" int sae_gather_rows(const void *src, int src_dtype, const int64_t *ro
   else
     hipLaunchKernelGGL((gather_rows_kernel<false, false>), grid, block, 0, st, src, row_idx, n_src_rows, (int)d, dst, sc);
   return check_launch("gather_rows");
+}
+
+extern "C" int sae_transpose_to_bf16(const void *src, int src_dtype, const float *mask, int64_t rows, int64_t cols,
+                                     void *dst, float *col_part, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(src && dst, SAE_ERR_INVALID_ARG, "transpose_to_bf16: null pointer");
+  SAE_REQUIRE(rows > 0 && cols > 0, SAE_ERR_INVALID_ARG, "transpose_to_bf16: bad shape");
+  SAE_REQUIRE(src_dtype == SAE_F32 || src_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "transpose_to_bf16: bad dtype %d", src_dtype);
+  const int64_t gx = (cols + 63) / 64, gy = (rows + 63) / 64;
+  SAE_REQUIRE(gy <= 65535, SAE_ERR_UNSUPPORTED, "transpose_to_bf16: rows=%lld above %d", (long long)rows, 65535 * 64);
+  const bool vec = rows % 8 == 0 && cols % 8 == 0 &&
+                   ((((uintptr_t)src | (uintptr_t)dst | (uintptr_t)mask) & 15) == 0);
+  const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  uint16_t *out = reinterpret_cast<uint16_t *>(dst);
+  if (src_dtype == SAE_BF16) {
+    if (vec) hipLaunchKernelGGL((transpose_to_bf16_kernel<true, true>), grid, block, 0, st, src, mask, rows, cols, out, col_part);
+    else hipLaunchKernelGGL((transpose_to_bf16_kernel<true, false>), grid, block, 0, st, src, mask, rows, cols, out, col_part);
+  } else {
+    if (vec) hipLaunchKernelGGL((transpose_to_bf16_kernel<false, true>), grid, block, 0, st, src, mask, rows, cols, out, col_part);
+    else hipLaunchKernelGGL((transpose_to_bf16_kernel<false, false>), grid, block, 0, st, src, mask, rows, cols, out, col_part);
+  }
+  return check_launch("transpose_to_bf16");
+}
+
+extern "C" int sae_code_to_dense(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
+                                 int64_t B, int64_t n_cols, float *dense_f32, void *dense_bf16, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "code_to_dense: null pointer");
+  SAE_REQUIRE(dense_f32 || dense_bf16, SAE_ERR_INVALID_ARG, "code_to_dense: no output");
+  SAE_REQUIRE(B > 0 && n_cols > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "code_to_dense: bad shape");
+  hipLaunchKernelGGL(code_to_dense_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, idx, val, row_off, row_nnz,
+                     n_cols, dense_f32, reinterpret_cast<uint16_t *>(dense_bf16));
+  return check_launch("code_to_dense");
 }
 
 extern "C" int sae_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {

@@ -206,13 +206,16 @@ struct BatchReader {
   }
 };
 
-__global__ void bt_init_kernel(BatchSelState *st, uint32_t *hist, int64_t k_host, const int64_t *k_dev) {
+__global__ void bt_init_kernel(BatchSelState *st, uint32_t *hist, int64_t k_host, const int64_t *k_dev, int64_t cand_cap) {
   for (int i = threadIdx.x; i < BT_BINS; i += blockDim.x) hist[i] = 0u;
   if (threadIdx.x == 0) {
     st->prefix = 0u; st->mask = 0u; st->done = 0; st->n_positive = 0; st->threshold = 0u; st->lower = 1u;
-    st->cand_count = 0ull; st->overflow = 0;
+    st->cand_count = 0ull;
     st->k_total = k_dev ? *k_dev : k_host;
     st->remaining = st->k_total;
+    // k_total keys or more reach the lower bound (or every positive key does): a list shorter than k_total is
+    // not worth trying, and the gather pass is skipped
+    st->overflow = st->k_total > cand_cap;
     if (st->k_total <= 0) { st->done = 1; st->k_total = 0; st->remaining = 0; st->threshold = BT_KEEP_NOTHING; }
   }
 }
@@ -290,6 +293,7 @@ __global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_gather_kernel(BatchR
   const int b = blockIdx.x * BT_TOKENS_PER_WG + wave;
   if (b >= B) return;
   if (st->threshold == BT_KEEP_NOTHING) return;
+  if (st->overflow) return;           // known beforehand (k_total beyond the list), or found by a token before this one
   const uint32_t lower = st->lower;   // 1 when every positive key is kept
   uint32_t *my_key = stash_key + wave * BT_STASH;
   int32_t *my_feat = stash_feat + wave * BT_STASH;
@@ -405,9 +409,10 @@ __device__ __forceinline__ int64_t bt_block_scan(int64_t v, int64_t *wsum) {
 }
 
 // Walking the nb bins from the top down, the bin in which the running count reaches `target` (> 0), and the rank
-// wanted inside that bin; *bin stays -1 when the histogram holds fewer than `target`.  One workgroup of 1024.
+// wanted inside that bin; *bin stays -1 when the histogram holds fewer than `target`; *total_out is the
+// histogram's total.  One workgroup of 1024; the results (in LDS) are visible to every thread on return.
 __device__ __forceinline__ void bt_find_from_top(const uint32_t *hist, int nb, int64_t target, int64_t *wsum, int *bin,
-                                                 int64_t *need_out) {
+                                                 int64_t *need_out, int64_t *total_out) {
   const int tid = threadIdx.x;
   if (tid == 0) *bin = -1;
   const int per = (nb + 1023) / 1024;  // thread t owns the bins nb - 1 - (t * per + e)
@@ -415,6 +420,7 @@ __device__ __forceinline__ void bt_find_from_top(const uint32_t *hist, int nb, i
   for (int e = 0; e < per; ++e) { const int i = nb - 1 - (tid * per + e); if (i >= 0) local += hist[i]; }
   const int64_t incl = bt_block_scan(local, wsum);  // its barriers also order the write of *bin above
   const int64_t excl = incl - local;
+  if (tid == 1023) *total_out = incl;
   if (excl < target && incl >= target) {
     int64_t need = target - excl;
     for (int e = 0; e < per; ++e) {
@@ -432,10 +438,10 @@ __device__ __forceinline__ void bt_find_from_top(const uint32_t *hist, int nb, i
 __global__ __launch_bounds__(1024) void bt_bound_kernel(BatchSelState *st, uint32_t *hist) {
   __shared__ int64_t wsum[BT_WAVES];
   __shared__ int bin;
-  __shared__ int64_t need;
+  __shared__ int64_t need, total;
   const int tid = threadIdx.x;
   if (st->done) { for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u; return; }
-  bt_find_from_top(hist, BT_BINS, st->k_total, wsum, &bin, &need);
+  bt_find_from_top(hist, BT_BINS, st->k_total, wsum, &bin, &need, &total);
   // k_total granules have a maximum in this bin or above, so the threshold is at least the bin's lower edge;
   // with fewer positive maxima than k_total (bin < 0) every positive key is a candidate
   if (tid == 0) st->lower = bin > 0 ? ((uint32_t)bin) << 20 : 1u;
@@ -444,20 +450,19 @@ __global__ __launch_bounds__(1024) void bt_bound_kernel(BatchSelState *st, uint3
 
 // one workgroup: choose the digit in which the running count (from the top bin down) reaches `remaining`.
 // The first of the three also settles the case of fewer positives than k_total: then the lower bound is 1, the
-// gather pass has met every positive key, and all of them are kept.
+// first histogram holds every positive key, and all of them are kept.
 __global__ __launch_bounds__(1024) void bt_pick_kernel(BatchSelState *st, uint32_t *hist, int shift, int bits, int first) {
   __shared__ int64_t wsum[BT_WAVES];
   __shared__ int bin;
-  __shared__ int64_t need;
+  __shared__ int64_t need, total;
   const int nb = 1 << bits, tid = threadIdx.x;
   if (st->done) { for (int i = tid; i < BT_BINS; i += 1024) hist[i] = 0u; return; }
-  const int64_t n_cand = (int64_t)st->cand_count, k_total = st->k_total;
-  const bool keep_all = first && st->lower == 1u && n_cand <= k_total;   // the same in every thread
-  bt_find_from_top(hist, nb, st->remaining, wsum, &bin, &need);
+  bt_find_from_top(hist, nb, st->remaining, wsum, &bin, &need, &total);
   if (tid == 0) {
-    if (first) st->n_positive = st->lower == 1u ? n_cand : -1;   // known only when every positive is a candidate
-    if (keep_all) {
-      st->done = 1; st->k_total = n_cand; st->prefix = 0u; st->mask = 0u; st->remaining = 0; st->threshold = 0u;
+    const bool all_counted = first && st->lower == 1u;   // the histogram's total is the number of positive keys
+    if (first) st->n_positive = all_counted ? total : -1;
+    if (all_counted && total <= st->k_total) {
+      st->done = 1; st->k_total = total; st->prefix = 0u; st->mask = 0u; st->remaining = 0; st->threshold = 0u;
     } else if (bin >= 0) {
       st->remaining = need;
       st->prefix |= ((uint32_t)bin) << shift;
@@ -642,7 +647,7 @@ static int run_batch_select(const void *pre, const float *b_enc, const float *sc
   cd.key = reinterpret_cast<uint32_t *>(cd.tok_cnt + B);
   cd.feat = reinterpret_cast<int32_t *>(cd.key + cd.cap);
   BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F, vec ? 1 : 0, nseg, ngran};
-  hipLaunchKernelGGL(bt_init_kernel, dim3(1), dim3(256), 0, st, state, hist, k_total, k_total_dev);
+  hipLaunchKernelGGL(bt_init_kernel, dim3(1), dim3(256), 0, st, state, hist, k_total, k_total_dev, bt_candidate_capacity(B, F));
   const int rows_per_wg = (int)(B / 65535 > 16 ? B / 65535 + 1 : 16);
   hipLaunchKernelGGL(bt_first_kernel<BF16>, dim3((unsigned)((nseg + BT_WAVES - 1) / BT_WAVES), (unsigned)((B + rows_per_wg - 1) / rows_per_wg)),
                      dim3(BT_THREADS), 0, st, rd, (int)B, rows_per_wg, state, hist, gran_max);

@@ -173,6 +173,40 @@ def col_sum(src: torch.Tensor, out: Optional[torch.Tensor] = None, accumulate: b
     return out
 
 
+def transpose_to_bf16(src: torch.Tensor, mask: Optional[torch.Tensor] = None, col_sums: bool = False):
+    """bf16 [cols, rows] = src[rows, cols]^T (fp32 or bf16 source), entries whose `mask` (fp32, same shape) is not
+    positive written as 0.  With `col_sums` also returns the fp32 column sums of the masked source (summed tile by
+    tile in a fixed order); otherwise the second value is None."""
+    _req(src, "src", ndim=2)
+    if src.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"src must be fp32 or bf16, not {src.dtype}")
+    r, c = src.shape
+    if mask is not None:
+        _req(mask, "mask", torch.float32, 2)
+        if tuple(mask.shape) != (r, c):
+            raise ValueError("mask must have the source's shape")
+    out = torch.empty(c, r, dtype=torch.bfloat16, device=src.device)
+    part = torch.empty((r + 63) // 64, c, dtype=torch.float32, device=src.device) if col_sums else None
+    with _timed("transpose_to_bf16"):
+        check(_lib.load().sae_transpose_to_bf16(src.data_ptr(), _dt(src), _ptr(mask), r, c, out.data_ptr(), _ptr(part),
+                                                _stream(src)), "transpose_to_bf16")
+    return out, (col_sum(part) if col_sums else None)
+
+
+def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_bf16: bool = False):
+    """Dense [n_tokens, n_cols] rows of a sparse code, in fp32 and / or bf16 -> (f32 or None, bf16 or None)."""
+    if not (want_f32 or want_bf16):
+        raise ValueError("no output requested")
+    B, dev = code.n_tokens, code.val.device
+    f32 = torch.empty(B, n_cols, dtype=torch.float32, device=dev) if want_f32 else None
+    b16 = torch.empty(B, n_cols, dtype=torch.bfloat16, device=dev) if want_bf16 else None
+    with _timed("code_to_dense"):
+        check(_lib.load().sae_code_to_dense(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                            code.row_nnz.data_ptr(), B, int(n_cols), _ptr(f32), _ptr(b16), _stream(code.val)),
+              "code_to_dense")
+    return f32, b16
+
+
 # ---- encoder --------------------------------------------------------------------------------
 
 def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

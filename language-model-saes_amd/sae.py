@@ -141,14 +141,15 @@ def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_au
     pre_d = ops.encoder_gemm(x_op, W_Et, pre_dtype)                                   # [B, ndp]
     kk = min(k_aux, nd)
     code_d = ops.select_topk_batch(pre_d, b_d, s_d, kk * B) if batch_wide else ops.select_topk_row(pre_d, b_d, s_d, kk)
-    # dense [B, ndp] activations of the block
-    tok, valid = _code_slot_tokens(code_d)
-    flat = tok.long() * ndp + code_d.idx.long()
-    vals = torch.where(valid, code_d.val, torch.zeros_like(code_d.val))
-    A = torch.zeros(B * ndp, dtype=torch.float32, device=dev).scatter_add_(0, flat, vals).view(B, ndp)
-    A_op = ops.cast_bf16(A) if amp else A
-    aux_recon = ops.encoder_gemm(A_op, W_D.t().contiguous(), torch.float32)            # [B, d] = A @ W_D[dead]
-    # the same code with the dictionary's own feature ids (for callers that look at it)
+    # dense [B, ndp] activations of the block: fp32 (the mask of the backward pass) and, under autocast, bf16
+    A, A_b16 = ops.code_to_dense(code_d, ndp, want_f32=True, want_bf16=amp)
+    A_op = A_b16 if amp else A
+    W_D_T = ops.transpose_to_bf16(W_D)[0] if amp else W_D.t().contiguous()
+    aux_recon = ops.encoder_gemm(A_op, W_D_T, torch.float32)                          # [B, d] = A @ W_D[dead]
+    # the same code with the dictionary's own feature ids (for callers that look at it); slots past the last
+    # token's end are unused and keep index 0
+    n_used = code_d.row_off[-1] + code_d.row_nnz[-1]
+    valid = torch.arange(code_d.n_slots, device=dev) < n_used
     idx_full = torch.where(valid, dead_idx.index_select(0, code_d.idx.long().clamp_max(nd - 1)).to(torch.int32),
                            torch.zeros_like(code_d.idx))
     import dataclasses
@@ -173,15 +174,23 @@ def _aux_dense_grads(blk, g_aux, x_op, amp: bool):
     dW_D[dead] = A^T G, dW_E^T[dead] = dA^T x, db_E[dead] = column sums of dA: three GEMMs with K = d, B, B."""
     nd = blk["n_dead"]
     A, A_op = blk["A"], blk["A_op"]
-    G_op = ops.cast_bf16(g_aux.contiguous()) if amp else g_aux.contiguous()
-    dA = ops.encoder_gemm(G_op, blk["W_D"], torch.float32)                             # [B, ndp]
-    dpre = torch.where(A > 0, dA, torch.zeros_like(dA))
-    dpre_op = ops.cast_bf16(dpre) if amp else dpre
-    dW_D = ops.encoder_gemm(A_op.t().contiguous(), G_op.t().contiguous(), torch.float32)        # [ndp, d]
-    dW_Et = ops.encoder_gemm(dpre_op.t().contiguous(), x_op.t().contiguous(), torch.float32)    # [ndp, d]
-    db_E = ops.col_sum(dpre)
+    g_aux = g_aux.contiguous()
+    if amp:
+        # bf16 operands; the transposes round the fp32 sources themselves, so each equals cast-then-transpose
+        G_op = ops.cast_bf16(g_aux)
+        dA = ops.encoder_gemm(G_op, blk["W_D"], torch.float32)                         # [B, ndp]
+        dpre_T, db_E = ops.transpose_to_bf16(dA, mask=A, col_sums=True)                 # d pre = dA where A > 0
+        dW_D = ops.encoder_gemm(ops.transpose_to_bf16(A_op)[0], ops.transpose_to_bf16(g_aux)[0], torch.float32)   # [ndp, d]
+        dW_Et = ops.encoder_gemm(dpre_T, ops.transpose_to_bf16(x_op)[0], torch.float32)                            # [ndp, d]
+        dpre = None   # formed on demand (only the gradient with respect to x wants it in this layout)
+    else:
+        dA = ops.encoder_gemm(g_aux, blk["W_D"], torch.float32)
+        dpre = torch.where(A > 0, dA, torch.zeros_like(dA))
+        dW_D = ops.encoder_gemm(A_op.t().contiguous(), g_aux.t().contiguous(), torch.float32)
+        dW_Et = ops.encoder_gemm(dpre.t().contiguous(), x_op.t().contiguous(), torch.float32)
+        db_E = ops.col_sum(dpre)
     return {"row_map": blk["row_map"], "dW_D": dW_D[:nd].contiguous(), "dW_Et": dW_Et[:nd].contiguous(),
-            "db_E": db_E[:nd].contiguous(), "dpre": dpre, "W_Et": blk["W_Et"]}
+            "db_E": db_E[:nd].contiguous(), "dpre": dpre, "dA": dA, "A": A, "W_Et": blk["W_Et"]}
 
 
 class _FusedSparseStep(torch.autograd.Function):
@@ -341,7 +350,8 @@ class _FusedSparseStep(torch.autograd.Function):
             if dx.shape[0] != ctx.n_tokens:  # stacked code: fold the aux half back onto its tokens
                 dx = dx[: ctx.n_tokens] + dx[ctx.n_tokens:]
             if ad is not None:
-                dx = dx + (ad["dpre"].to(ad["W_Et"].dtype) @ ad["W_Et"]).to(torch.float32) * g
+                dpre = ad["dpre"] if ad["dpre"] is not None else torch.where(ad["A"] > 0, ad["dA"], torch.zeros_like(ad["dA"]))
+                dx = dx + (dpre.to(ad["W_Et"].dtype) @ ad["W_Et"]).to(torch.float32) * g
         dlabel = None
         if ctx.needs_input_grad[1]:
             dlabel = -ctx.grad_recon * g

@@ -312,6 +312,42 @@ def test_cast_rownorm_transpose_colsum(pkg, dev):
     assert rel_err(pkg.ops.row_norm(b.to(dev)), b.double().norm(dim=1)) < 1e-6
 
 
+@pytest.mark.parametrize("rows,cols", [(256, 192), (301, 520), (64, 8), (8, 64), (77, 13), (1, 1)])
+@pytest.mark.parametrize("src_dtype", [torch.float32, torch.bfloat16])
+def test_transpose_to_bf16(pkg, dev, rows, cols, src_dtype):
+    """bit-exact against cast-then-transpose; the mask zeroes entries; the column sums are those of the masked source"""
+    print(f"transpose_to_bf16 {rows}x{cols} {src_dtype}", flush=True)
+    g = torch.Generator().manual_seed(rows * 1000 + cols)
+    a = torch.randn(rows, cols, generator=g).to(src_dtype)
+    out, sums = pkg.ops.transpose_to_bf16(a.to(dev))
+    assert sums is None and torch.equal(out.cpu(), a.bfloat16().t().contiguous())
+    mask = torch.randn(rows, cols, generator=g)          # about half not positive, some exactly 0
+    mask[0, 0] = 0.0
+    masked = torch.where(mask > 0, a.float(), torch.zeros(()))
+    out, sums = pkg.ops.transpose_to_bf16(a.to(dev), mask=mask.to(dev), col_sums=True)
+    assert torch.equal(out.cpu(), masked.bfloat16().t().contiguous())
+    assert torch.allclose(sums.cpu().double(), masked.double().sum(0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("B,n_cols,k", [(5, 100, 7), (64, 3328, 512), (3, 20000, 40), (2, 8192, 1)])
+def test_code_to_dense(pkg, oracle, dev, B, n_cols, k):
+    """a BatchTopK code (ragged rows, unused tail slots) and a TopK code written out densely, fp32 and bf16"""
+    print(f"code_to_dense B={B} n={n_cols} k={k}", flush=True)
+    g = torch.Generator().manual_seed(B + n_cols)
+    pre = torch.randn(B, n_cols, generator=g)
+    pre[0] = -1.0                                        # a token that keeps nothing
+    for code in (pkg.ops.select_topk_batch(pre.to(dev), None, None, k * B), pkg.ops.select_topk_row(pre.to(dev), None, None, k)):
+        want = code.to_dense().cpu()
+        f32, b16 = pkg.ops.code_to_dense(code, n_cols, want_f32=True, want_bf16=True)
+        assert torch.equal(f32.cpu(), want)
+        assert torch.equal(b16.cpu(), want.bfloat16())
+        only_b16 = pkg.ops.code_to_dense(code, n_cols, want_f32=False, want_bf16=True)
+        assert only_b16[0] is None and torch.equal(only_b16[1].cpu(), want.bfloat16())
+    # indices at or beyond n_cols are dropped
+    f32, _ = pkg.ops.code_to_dense(code, n_cols // 2)
+    assert torch.equal(f32.cpu(), want[:, : n_cols // 2])
+
+
 def test_row_norm_reference_fixture(pkg, dev):
     """decoder norms of the reference's test fixture (tests/unit/test_sae.py:31-55): closed forms"""
     W_D = torch.tensor([[1.0, 5.0], [2.0, 6.0], [3.0, 7.0], [4.0, 8.0]])
@@ -433,6 +469,9 @@ def test_select_topk_batch_ties_and_degenerate(pkg, oracle, dev):
     few = torch.zeros(B, F); few[1, 5] = 1.0; few[4, 1999] = 3.0
     code = check_batch_select(pkg, oracle, dev, few, None, None, 100)                 # fewer positives than k_total
     assert code.row_nnz.cpu().tolist() == [0, 1, 0, 0, 1, 0]
+    code = check_batch_select(pkg, oracle, dev, few, None, None, 5000)                # the same with k_total beyond the candidate list
+    assert code.row_nnz.cpu().tolist() == [0, 1, 0, 0, 1, 0]
+    check_batch_select(pkg, oracle, dev, pre, None, None, 5000, k_on_device=True)     # k_total read on the device, beyond the list
     check_batch_select(pkg, oracle, dev, pre, None, None, 0)                          # k_total = 0 keeps nothing
     bfq = torch.randn(B, F, generator=g).bfloat16()                                   # bf16-quantised: natural ties
     check_batch_select(pkg, oracle, dev, bfq, None, None, 64 * B)
