@@ -10,11 +10,14 @@ struct AdamScalars {
   float beta1, beta2, one_minus_beta1, one_minus_beta2, step_size, inv_bc2_sqrt, eps;
 };
 
+// Every multiply-add is written out as a fused one, so that no kernel that inlines this leaves the choice of
+// what to fuse to the compiler: the kernels that promise identical bits (the plain passes, the passes that rebuild
+// the gradient rows) then really compute the same thing.
 __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v, const AdamScalars &a) {
-  m = m + a.one_minus_beta1 * (g - m);               // lerp, as torch does
-  v = a.beta2 * v + a.one_minus_beta2 * g * g;
-  const float denom = sqrtf(v) * a.inv_bc2_sqrt + a.eps;
-  p = p - a.step_size * (m / denom);
+  m = fmaf(a.one_minus_beta1, __fsub_rn(g, m), m);   // lerp, as torch does
+  v = fmaf(a.beta2, v, __fmul_rn(__fmul_rn(a.one_minus_beta2, g), g));
+  const float denom = fmaf(sqrtf(v), a.inv_bc2_sqrt, a.eps);
+  p = fmaf(-a.step_size, m / denom, p);
   return p;
 }
 
@@ -136,7 +139,7 @@ namespace sae {
 
 __global__ void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc);  // defined below
 
-template <bool DENSE_BF16>
+template <bool DENSE_BF16, int U>
 __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
@@ -146,6 +149,8 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows, const float *__restrict__ extra_bias) {
   __shared__ float red[4];
   __shared__ double red_d[8];
+  __shared__ float s_coef[256];
+  __shared__ int32_t s_tok[256];
   const int f = blockIdx.x, tid = threadIdx.x;
   const float gs = grad_scale ? grad_scale[0] : 1.f;
   const int xo = extra_map ? extra_map[f] : -1;   // row of the dense gradient block that adds to this feature, or -1
@@ -166,11 +171,14 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
   float sq = 0.f;
   double g_sq = 0.0;
   int g_nz = 0;
-  for (int seg0 = tid; seg0 < n_seg; seg0 += 256 * 4) {
+  // U pieces of 4 elements per thread and pass: a row of up to 1024 U elements takes one pass (the same for every
+  // thread of the workgroup, which gathers the gradient row together)
+  for (int seg_base = 0; seg_base < n_seg; seg_base += 256 * U) {
+    const int seg0 = seg_base + tid;
     // issue the streaming reads of p, m, v first: they are the HBM traffic; the gradient operands hit cache
-    float4 pp[4], mm[4], vv[4], g[4];
+    float4 pp[U], mm[U], vv[U], g[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
         pp[u] = load_stream(p, base4 + seg);
@@ -180,12 +188,15 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    gather_rows_fma<DENSE_BF16>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg);
+    gather_rows_staged<DENSE_BF16, 256, U>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg, s_coef, s_tok);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
-        if (grad_scale) { g[u].x *= gs; g[u].y *= gs; g[u].z *= gs; g[u].w *= gs; }
+        if (grad_scale) {   // rounded products, as when the scaled gradient is written out before the step
+          g[u].x = __fmul_rn(g[u].x, gs); g[u].y = __fmul_rn(g[u].y, gs);
+          g[u].z = __fmul_rn(g[u].z, gs); g[u].w = __fmul_rn(g[u].w, gs);
+        }
         if (sq_nnz_partial) {  // the same 4-element fp32 partials as sparse_rows_sq_nnz_kernel
           float s4 = g[u].x * g[u].x;
           s4 = fmaf(g[u].y, g[u].y, s4); s4 = fmaf(g[u].z, g[u].z, s4); s4 = fmaf(g[u].w, g[u].w, s4);
@@ -258,14 +269,20 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
   a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
   double *partial = grad_sq_nnz_acc ? reinterpret_cast<double *>(workspace) : nullptr;
-  if (dense_dtype == SAE_BF16)
-    hipLaunchKernelGGL(adam_sparse_rows_kernel<true>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial,
-                       extra_map, extra_rows, extra_bias);
-  else
-    hipLaunchKernelGGL(adam_sparse_rows_kernel<false>, dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok,
-                       coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, bias_grad_out, grad_scale, partial,
-                       extra_map, extra_rows, extra_bias);
+  {
+#define SAE_ADAM_ROWS(BF, UU)                                                                                              \
+  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
+                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,            \
+                     bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias)
+    // pieces of 4 elements per thread: short rows keep fewer registers, so more rows are in flight per CU
+    const int u = d <= 1024 ? 1 : (d <= 2048 ? 2 : 4);
+    if (dense_dtype == SAE_BF16) {
+      if (u == 1) SAE_ADAM_ROWS(true, 1); else if (u == 2) SAE_ADAM_ROWS(true, 2); else SAE_ADAM_ROWS(true, 4);
+    } else {
+      if (u == 1) SAE_ADAM_ROWS(false, 1); else if (u == 2) SAE_ADAM_ROWS(false, 2); else SAE_ADAM_ROWS(false, 4);
+    }
+#undef SAE_ADAM_ROWS
+  }
   if (partial) hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, grad_sq_nnz_acc);
   return check_launch("adam_step_sparse_rows");
 }

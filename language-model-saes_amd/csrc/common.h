@@ -149,4 +149,66 @@ __device__ __forceinline__ void gather_rows_fma(float4 (&g)[4], int lo, int hi, 
   }
 }
 
+// The same sum, computed by a whole workgroup of ROW_THREADS threads for ONE segment (every thread calls it; a
+// thread whose pieces lie past the row passes seg0 >= n_seg and only helps).  The segment's coefficients and
+// tokens are first staged in LDS, ROW_THREADS pairs at a time and one pair per thread, so the two dependent
+// index loads are paid once per chunk instead of once per group of pairs; the rows of a group of pairs are then
+// all requested before the first multiply-add.  U pieces per thread (piece u at seg0 + ROW_THREADS u); pairs in
+// ascending order as above, so the bits are the same.  s_coef / s_tok: ROW_THREADS entries of LDS each.
+template <bool DENSE_BF16, int ROW_THREADS, int U>
+__device__ __forceinline__ void gather_rows_staged(float4 (&g)[U], int lo, int hi, const int32_t *__restrict__ feat_slot,
+                                                   const int32_t *__restrict__ slot_tok, const float *__restrict__ coef,
+                                                   const char *dbase, size_t row_bytes, int seg0, int n_seg,
+                                                   float *s_coef, int32_t *s_tok) {
+  constexpr int C = (DENSE_BF16 ? 8 : 4) / (U == 4 ? 2 : 1);   // pairs whose rows are in flight together
+  typedef typename std::conditional<DENSE_BF16, uint2, float4>::type piece_t;
+  auto fma_piece = [&](float4 &acc, float c, const piece_t &r) {
+    float4 x;
+    if constexpr (DENSE_BF16) {
+      x.x = __uint_as_float(r.x << 16); x.y = __uint_as_float(r.x & 0xffff0000u);
+      x.z = __uint_as_float(r.y << 16); x.w = __uint_as_float(r.y & 0xffff0000u);
+    } else {
+      x = r;
+    }
+    acc.x = fmaf(c, x.x, acc.x); acc.y = fmaf(c, x.y, acc.y);
+    acc.z = fmaf(c, x.z, acc.z); acc.w = fmaf(c, x.w, acc.w);
+  };
+  const int tid = threadIdx.x;
+  for (int c0 = lo; c0 < hi; c0 += ROW_THREADS) {
+    const int n = hi - c0 < ROW_THREADS ? hi - c0 : ROW_THREADS;
+    __syncthreads();   // the previous chunk (or the previous call) has been consumed
+    if (tid < n) {
+      const int sl = feat_slot[c0 + tid];
+      s_coef[tid] = coef[sl];
+      s_tok[tid] = slot_tok[sl];
+    }
+    __syncthreads();
+    int i = 0;
+    for (; i + C <= n; i += C) {
+      piece_t r[C][U];
+#pragma unroll
+      for (int j = 0; j < C; ++j) {
+        const piece_t *row = reinterpret_cast<const piece_t *>(dbase + (size_t)s_tok[i + j] * row_bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (seg0 + u * ROW_THREADS < n_seg) r[j][u] = row[seg0 + u * ROW_THREADS];
+      }
+#pragma unroll
+      for (int j = 0; j < C; ++j) {
+        const float c = s_coef[i + j];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (seg0 + u * ROW_THREADS < n_seg) fma_piece(g[u], c, r[j][u]);
+      }
+    }
+    for (; i < n; ++i) {
+      const float c = s_coef[i];
+      const piece_t *row = reinterpret_cast<const piece_t *>(dbase + (size_t)s_tok[i] * row_bytes);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (seg0 + u * ROW_THREADS < n_seg) fma_piece(g[u], c, row[seg0 + u * ROW_THREADS]);
+    }
+  }
+}
+
 }  // namespace sae
