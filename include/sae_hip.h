@@ -261,6 +261,19 @@ int sae_sparse_rows_grad_sq_nnz(const int32_t *feat_ptr, const int32_t *feat_slo
                                 const int32_t *extra_map, const float *extra_rows, const float *extra_bias,
                                 void *stream);
 
+/* Reconstruction loss, aux-k loss and the two output gradients of a step whose aux reconstruction is dense, one
+ * pass over [B, d] (d a multiple of 4, 16-byte aligned rows):
+ *   rec_tok[b] = w_b sum_j (recon - label)^2                      (l_rec = sum_b rec_tok, w_b = tok_w[b] or 1)
+ *   aux_tok[b] = w_b sum_j ((label - recon) - aux_recon)^2        (l_aux = alpha sum_b aux_tok)
+ *   g_aux      = (-2 alpha w_b) ((label - recon) - aux_recon)     = d loss / d aux_recon
+ *   grad_recon = (2 w_b) (recon - label) + g_aux                  = d loss / d recon (the residual carries gradient)
+ * aux_recon may be null (no dead feature: aux_tok and g_aux are then not written and grad_recon is the first term);
+ * grad_recon_bf16 (nullable) receives grad_recon rounded to bf16.
+ * Replaces models/sparse_dictionary.py:871-886 (l_rec) and :973-991 (the aux-k residual loss) with their autograd twins. */
+int sae_mse_auxk_fused(const float *recon, const float *label, const float *aux_recon, const float *tok_w, double alpha,
+                       int64_t B, int64_t d, float *rec_tok, float *aux_tok, float *g_aux, float *grad_recon,
+                       void *grad_recon_bf16, void *stream);
+
 /* [rows, cols] fp32 or bf16 -> bf16 [cols, rows] (round to nearest even).
  *   mask (nullable, fp32 [rows, cols]): entries whose mask is not positive are written as 0;
  *   col_part (nullable, fp32 [ceil(rows / 64), cols]): per 64-row tile, the column sums of the (masked) fp32

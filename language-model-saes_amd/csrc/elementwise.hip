@@ -265,6 +265,59 @@ __global__ __launch_bounds__(256) void code_to_dense_kernel(const int32_t *__res
   }
 }
 
+// One workgroup per token: squared error, aux-k residual and both output gradients in one pass over the row.
+//   diff = recon - label            rec_tok[b] = w_b * sum diff^2
+//   r = (label - recon) - aux       aux_tok[b] = w_b * sum r^2                       (aux given)
+//   g_aux = (-2 alpha w_b) r        grad_recon = (2 w_b) diff + g_aux                (g_aux = 0 without aux)
+// grad_recon is also written as bf16 when asked (the operand of the decoder's factored gradient under autocast).
+__global__ __launch_bounds__(256) void mse_auxk_kernel(const float *__restrict__ recon, const float *__restrict__ label,
+                                                       const float *__restrict__ aux, const float *__restrict__ tok_w,
+                                                       float alpha, int d, float *__restrict__ rec_tok,
+                                                       float *__restrict__ aux_tok, float *__restrict__ g_aux,
+                                                       float *__restrict__ grad_recon, uint16_t *__restrict__ grad_bf16) {
+  __shared__ float red[4];
+  const int64_t b = blockIdx.x;
+  const int tid = threadIdx.x, n4 = d >> 2;
+  const float w = tok_w ? tok_w[b] : 1.f;
+  const float ca = __fmul_rn(-2.f * alpha, w), cr = __fmul_rn(2.f, w);
+  const float4 *rp = reinterpret_cast<const float4 *>(recon + b * d), *lp = reinterpret_cast<const float4 *>(label + b * d);
+  const float4 *ap = aux ? reinterpret_cast<const float4 *>(aux + b * d) : nullptr;
+  float sq_rec = 0.f, sq_aux = 0.f;
+  for (int i = tid; i < n4; i += 256) {
+    const float4 rc = rp[i], lb = lp[i];
+    const float4 ax = ap ? ap[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float rv[4] = {rc.x, rc.y, rc.z, rc.w}, lv[4] = {lb.x, lb.y, lb.z, lb.w}, av[4] = {ax.x, ax.y, ax.z, ax.w};
+    float go[4], ga[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float diff = __fsub_rn(rv[e], lv[e]);
+      sq_rec = fmaf(diff, diff, sq_rec);
+      ga[e] = 0.f;
+      if (ap) {
+        const float r = __fsub_rn(__fsub_rn(lv[e], rv[e]), av[e]);
+        sq_aux = fmaf(r, r, sq_aux);
+        ga[e] = __fmul_rn(ca, r);
+      }
+      go[e] = __fadd_rn(__fmul_rn(cr, diff), ga[e]);
+    }
+    reinterpret_cast<float4 *>(grad_recon + b * d)[i] = make_float4(go[0], go[1], go[2], go[3]);
+    if (ap && g_aux) reinterpret_cast<float4 *>(g_aux + b * d)[i] = make_float4(ga[0], ga[1], ga[2], ga[3]);
+    if (grad_bf16) {
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16_bits(go[0]) | ((uint32_t)f32_to_bf16_bits(go[1]) << 16);
+      o.y = (uint32_t)f32_to_bf16_bits(go[2]) | ((uint32_t)f32_to_bf16_bits(go[3]) << 16);
+      reinterpret_cast<uint2 *>(grad_bf16 + b * d)[i] = o;
+    }
+  }
+  const float tr = block_sum<4>(sq_rec, red);
+  __syncthreads();
+  const float ta = block_sum<4>(sq_aux, red);
+  if (tid == 0) {
+    rec_tok[b] = w * tr;
+    if (aux_tok) aux_tok[b] = w * ta;
+  }
+}
+
 }  // namespace sae
 
 extern "C" int sae_gather_rows(const void *src, int src_dtype, const int64_t *row_idx, int64_t n_src_rows, int64_t n_rows,
@@ -321,6 +374,22 @@ extern "C" int sae_code_to_dense(const int32_t *idx, const float *val, const int
   hipLaunchKernelGGL(code_to_dense_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, idx, val, row_off, row_nnz,
                      n_cols, dense_f32, reinterpret_cast<uint16_t *>(dense_bf16));
   return check_launch("code_to_dense");
+}
+
+extern "C" int sae_mse_auxk_fused(const float *recon, const float *label, const float *aux_recon, const float *tok_w,
+                                  double alpha, int64_t B, int64_t d, float *rec_tok, float *aux_tok, float *g_aux,
+                                  float *grad_recon, void *grad_recon_bf16, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(recon && label && rec_tok && grad_recon, SAE_ERR_INVALID_ARG, "mse_auxk_fused: null pointer");
+  SAE_REQUIRE(!aux_recon || (aux_tok && g_aux), SAE_ERR_INVALID_ARG, "mse_auxk_fused: aux_tok and g_aux go with aux_recon");
+  SAE_REQUIRE(B > 0 && d > 0 && d % 4 == 0 && d < (1LL << 31) && B < (1LL << 31), SAE_ERR_INVALID_ARG,
+              "mse_auxk_fused: bad shape (d must be a multiple of 4)");
+  SAE_REQUIRE((((uintptr_t)recon | (uintptr_t)label | (uintptr_t)aux_recon | (uintptr_t)g_aux | (uintptr_t)grad_recon |
+                (uintptr_t)grad_recon_bf16) & 15) == 0, SAE_ERR_INVALID_ARG, "mse_auxk_fused: 16-byte alignment required");
+  hipLaunchKernelGGL(mse_auxk_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, recon, label, aux_recon, tok_w,
+                     (float)alpha, (int)d, rec_tok, aux_recon ? aux_tok : nullptr, g_aux, grad_recon,
+                     reinterpret_cast<uint16_t *>(grad_recon_bf16));
+  return check_launch("mse_auxk_fused");
 }
 
 extern "C" int sae_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {

@@ -207,6 +207,35 @@ def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_b
     return f32, b16
 
 
+def mse_auxk_fused(recon: torch.Tensor, label: torch.Tensor, aux_recon: Optional[torch.Tensor],
+                   tok_w: Optional[torch.Tensor], alpha: float, want_bf16: bool = False):
+    """-> (rec_tok [B], aux_tok [B] or None, g_aux [B, d] or None, grad_recon [B, d], grad_recon in bf16 or None):
+    the per-token weighted squared error, the per-token weighted squared aux-k residual (l_aux = alpha * its sum),
+    d loss / d aux_recon and d loss / d recon."""
+    _req(recon, "recon", torch.float32, 2)
+    _req(label, "label", torch.float32, 2)
+    B, d = recon.shape
+    if tuple(label.shape) != (B, d):
+        raise ValueError("label must have recon's shape")
+    if aux_recon is not None:
+        _req(aux_recon, "aux_recon", torch.float32, 2)
+        if tuple(aux_recon.shape) != (B, d):
+            raise ValueError("aux_recon must have recon's shape")
+    if tok_w is not None:
+        _req(tok_w, "tok_w", torch.float32, 1)
+    dev = recon.device
+    rec_tok = torch.empty(B, dtype=torch.float32, device=dev)
+    aux_tok = torch.empty(B, dtype=torch.float32, device=dev) if aux_recon is not None else None
+    g_aux = torch.empty(B, d, dtype=torch.float32, device=dev) if aux_recon is not None else None
+    grad = torch.empty(B, d, dtype=torch.float32, device=dev)
+    grad16 = torch.empty(B, d, dtype=torch.bfloat16, device=dev) if want_bf16 else None
+    with _timed("mse_auxk_fused"):
+        check(_lib.load().sae_mse_auxk_fused(recon.data_ptr(), label.data_ptr(), _ptr(aux_recon), _ptr(tok_w), float(alpha), B, d,
+                                             rec_tok.data_ptr(), _ptr(aux_tok), _ptr(g_aux), grad.data_ptr(), _ptr(grad16),
+                                             _stream(recon)), "mse_auxk_fused")
+    return rec_tok, aux_tok, g_aux, grad, grad16
+
+
 # ---- encoder --------------------------------------------------------------------------------
 
 def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

@@ -230,6 +230,7 @@ class _FusedSparseStep(torch.autograd.Function):
         else:
             code = ops.select_topk_row(pre, b_E, scale, k)
         aux = holder.aux
+        grad_recon_b16 = None   # set by the route that already has grad_recon in bf16
         if aux is None:
             recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, b_D, label, tok_w)
             loss = loss_tok.sum()
@@ -249,19 +250,12 @@ class _FusedSparseStep(torch.autograd.Function):
                 # GEMMs on a compacted [n_dead, d] copy of the two weight blocks instead of gathers per (token, feature).
                 blk = dense_block
                 recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
-                w = tok_w[:, None]
-                diff = recon - label
                 alpha = float(aux["coefficient"])
-                l_rec = (w * diff * diff).sum()
-                if blk["n_dead"] == 0:
-                    l_aux = torch.zeros_like(l_rec)
-                    g_aux = None
-                    grad_recon = 2.0 * w * diff
-                else:
-                    r = (label - recon) - blk["aux_recon"]
-                    l_aux = alpha * (w * r * r).sum()
-                    g_aux = (-2.0 * alpha) * w * r                 # d loss / d aux_recon
-                    grad_recon = 2.0 * w * diff + g_aux            # d loss / d recon (the residual is not detached)
+                # squared error, aux-k residual (the residual is not detached), d loss / d aux_recon and d loss / d recon
+                rec_tok, aux_tok, g_aux, grad_recon, grad_recon_b16 = ops.mse_auxk_fused(
+                    recon, label, blk["aux_recon"] if blk["n_dead"] else None, tok_w, alpha, want_bf16=amp)
+                l_rec = rec_tok.sum()
+                l_aux = alpha * aux_tok.sum() if aux_tok is not None else torch.zeros_like(l_rec)
                 loss = l_rec + l_aux
                 dval = ops.sparse_decode_bwd_dval(code, grad_recon, w_dec_op)
                 if g_aux is not None:
@@ -299,7 +293,7 @@ class _FusedSparseStep(torch.autograd.Function):
         if amp:
             # the decoder's weight gradient pairs the activations with the bf16-rounded output gradient, as the
             # backward of an autocast matmul does; the gather of those rows then moves half the bytes
-            grad_dense_D = ops.cast_bf16(grad_dense_D.contiguous())
+            grad_dense_D = grad_recon_b16 if grad_recon_b16 is not None else ops.cast_bf16(grad_dense_D.contiguous())
         holder.code, holder.pre, holder.scale, holder.l_aux = code, pre, scale, l_aux
         ctx.grad_code, ctx.x_rows, ctx.grad_dense_D, ctx.grad_coef_E = grad_code, x_rows, grad_dense_D, grad_coef_E
         ctx.grad_recon = grad_recon

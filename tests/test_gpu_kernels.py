@@ -348,6 +348,28 @@ def test_code_to_dense(pkg, oracle, dev, B, n_cols, k):
     assert torch.equal(f32.cpu(), want[:, : n_cols // 2])
 
 
+@pytest.mark.parametrize("B,d", [(7, 64), (300, 768), (64, 4096)])
+def test_mse_auxk_fused(pkg, dev, B, d):
+    """the four outputs against the formulas of the aux-k loss in fp64 (fp32 bar: 1e-5 relative)"""
+    g = torch.Generator().manual_seed(B + d)
+    recon, label, aux = (torch.randn(B, d, generator=g) for _ in range(3))
+    w = torch.rand(B, generator=g) / B
+    alpha = 1.0 / 32
+    rec_tok, aux_tok, g_aux, grad, grad16 = pkg.ops.mse_auxk_fused(recon.to(dev), label.to(dev), aux.to(dev), w.to(dev), alpha,
+                                                                   want_bf16=True)
+    R, L, A, W = recon.double(), label.double(), aux.double(), w.double()[:, None]
+    r = (L - R) - A
+    assert rel_err(rec_tok, (W * (R - L) ** 2).sum(1)) < 1e-5
+    assert rel_err(aux_tok, (W * r ** 2).sum(1)) < 1e-5
+    assert rel_err(g_aux, -2 * alpha * W * r) < 1e-5
+    assert rel_err(grad, 2 * W * (R - L) - 2 * alpha * W * r) < 1e-5
+    assert torch.equal(grad16.cpu(), grad.cpu().bfloat16())
+    # without an aux reconstruction (no dead feature) and without token weights
+    rec_tok, aux_tok, g_aux, grad2, grad16 = pkg.ops.mse_auxk_fused(recon.to(dev), label.to(dev), None, None, alpha)
+    assert aux_tok is None and g_aux is None and grad16 is None
+    assert rel_err(rec_tok, ((R - L) ** 2).sum(1)) < 1e-5 and rel_err(grad2, 2 * (R - L)) < 1e-5
+
+
 def test_row_norm_reference_fixture(pkg, dev):
     """decoder norms of the reference's test fixture (tests/unit/test_sae.py:31-55): closed forms"""
     W_D = torch.tensor([[1.0, 5.0], [2.0, 6.0], [3.0, 7.0], [4.0, 8.0]])
