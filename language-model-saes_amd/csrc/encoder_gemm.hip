@@ -6,8 +6,10 @@
 // Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile and
 // walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32): a full cache line per row, which the
 // L2 serves at twice the rate of half lines (measured 27 vs 13 TB/s aggregate L2->LDS).  Waves are
-// arranged 2 x 4: each owns 128 tokens x 64 features = 4 x 2 MFMA tiles of 32x32 (128 fp32
-// accumulators per lane).
+// arranged 2 x 4: each owns 128 tokens x 64 features (128 fp32 accumulators per lane): 8 x 4 tiles of
+// v_mfma_f32_16x16x32_bf16 for bf16 operands (two k-steps of 64 bytes per slab, a quarter wave per
+// 16-byte chunk; measured 1.28-1.30 against 1.22-1.23 PFLOP/s for 4 x 2 tiles of 32x32x16 at the
+// headline shape), 4 x 2 tiles of v_mfma_f32_32x32x2f32 for fp32 operands.
 //
 // Pipeline: LDS (all 160 KiB of the CU) is a ring of five 32 KiB slots; a slot holds one operand's
 // slab (256 rows x 128 bytes).  Load units alternate W slab j, x slab j, W slab j+1, ...; unit t
@@ -25,7 +27,7 @@
 // An LDS-direct load writes 1 KiB linearly (lane l -> base + 16 l), so the swizzle is applied on
 // the global side: lane l fetches the logical chunk that belongs at its physical slot.
 //
-// The matrix cores compute D = Wtile * xtile^T (features along the 32 "rows" of the instruction),
+// The matrix cores compute D = Wtile * xtile^T (features along the "rows" of the instruction),
 // which leaves every lane holding 4 consecutive features of one token.  For bf16 output a full tile is
 // transposed through LDS, wave by wave, and leaves as whole 128-byte lines; edge tiles and fp32 output
 // store each lane's 4 features directly (8 or 16 bytes).
@@ -124,13 +126,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     lds_off[i] = (wave * 32 + i * 8) * GEMM_SLAB;  // wave-uniform base of the 1 KiB this load fills
   }
 
-  f32x16_t acc[2][4];  // [feature sub-tile][token sub-tile]
+  f32x16_t acc[BF16_IN ? 1 : 2][BF16_IN ? 1 : 4];  // fp32 operands: [feature sub-tile of 32][token sub-tile of 32]
+  f32x4_t acc16[BF16_IN ? 4 : 1][BF16_IN ? 8 : 1];  // bf16 operands: [feature sub-tile of 16][token sub-tile of 16]
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < (BF16_IN ? 1 : 2); ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < (BF16_IN ? 1 : 4); ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+#pragma unroll
+  for (int i = 0; i < (BF16_IN ? 4 : 1); ++i)
+#pragma unroll
+    for (int j = 0; j < (BF16_IN ? 8 : 1); ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc16[i][j][v] = 0.f;
 
   const int n_slabs = row_bytes / GEMM_SLAB;
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -164,7 +173,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     __builtin_amdgcn_s_waitcnt(WAITCNT_VM4);
     __builtin_amdgcn_s_barrier();  // everyone's part landed; everyone is done with the previous slab's two slots
     // units issued while this slab is consumed: x slab+1 -> slot freed by W slab-1, W slab+2 -> slot freed by
-    // x slab-1.  Two of the eight loads per k-step, so that requests trickle instead of bursting.
+    // x slab-1.  Two of the eight loads per phase, so that requests trickle instead of bursting.
     const int tA = 2 * slab + 3, tB = 2 * slab + 4;
     int sA = tA >> 1; sA = sA < n_slabs ? sA : n_slabs - 1;
     int sB = tB >> 1; sB = sB < n_slabs ? sB : n_slabs - 1;
@@ -173,11 +182,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     __builtin_amdgcn_sched_barrier(0);
     const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
     const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
+    u32x4 wf16[4];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {  // 4 MFMA k-steps per slab (32 bytes of K each)
+    for (int s = 0; s < 4; ++s) {  // 4 phases per slab, each with a quarter of the slab's loads and matrix-core work
       const int chunk = 2 * s + frag_half;
       if (slab >= 1) {
-        // x unit in k-steps 0-1, W unit in k-steps 2-3: the W loads stay the four youngest, which is what
+        // x unit in phases 0-1, W unit in phases 2-3: the W loads stay the four youngest, which is what
         // the vmcnt(4) at the top of the next slab relies on
         if (s < 2) {
           LDS_DMA16(xg[2 * s] + (size_t)sA * GEMM_SLAB, slotA + lds_off[2 * s]);
@@ -187,15 +197,38 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
           LDS_DMA16(wg[2 * s - 3] + (size_t)sB * GEMM_SLAB, slotB + lds_off[2 * s - 3]);
         }
       }
-      u32x4 wf[2], xf[4];
+      if constexpr (BF16_IN) {
+        // 16x16x32 instructions: a k-step is 64 bytes of K (4 chunks, one per quarter wave); phase s covers
+        // k-step s / 2 and the token sub-tiles 4 (s & 1) .. + 4; the W fragments of a k-step are read in its first phase
+        const int c16 = 4 * (s >> 1) + (lane >> 4);
+        if ((s & 1) == 0) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));
+          for (int i = 0; i < 4; ++i) wf16[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 16 + (lane & 15), c16));
+        }
+        u32x4 xf16[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 32 + frag_row, chunk));
+        for (int j = 0; j < 4; ++j)
+          xf16[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + ((s & 1) * 4 + j) * 16 + (lane & 15), c16));
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) mma_chunk<BF16_IN>(wf[i], xf[j], acc[i][j]);
+          for (int j = 0; j < 4; ++j) {
+            bf16x8_t a = __builtin_bit_cast(bf16x8_t, wf16[i]);
+            bf16x8_t b = __builtin_bit_cast(bf16x8_t, xf16[j]);
+            acc16[i][(s & 1) * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc16[i][(s & 1) * 4 + j], 0, 0, 0);
+          }
+      } else {
+        // 32x32x2 fp32 instructions: phase s covers 32 bytes of K (two chunks, one per half wave)
+        u32x4 wf[2], xf[4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 32 + frag_row, chunk));
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mma_chunk<BF16_IN>(wf[i], xf[j], acc[i][j]);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -211,6 +244,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
       constexpr int PITCH = 136;
       __builtin_amdgcn_s_barrier();  // every wave is done reading operand slabs (and its own loads have landed)
       char *stage = lds + wave * (128 * PITCH);
+      if constexpr (BF16_IN) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint2 pk;
+            pk.x = pack_bf16x2(acc16[i][j][0], acc16[i][j][1]);
+            pk.y = pack_bf16x2(acc16[i][j][2], acc16[i][j][3]);
+            *reinterpret_cast<uint2 *>(stage + (j * 16 + (lane & 15)) * PITCH + (i * 16 + 4 * (lane >> 4)) * 2) = pk;
+          }
+      } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -222,6 +266,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
             pk.y = pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
             *reinterpret_cast<uint2 *>(stage + (j * 32 + frag_row) * PITCH + (i * 32 + 8 * g + 4 * frag_half) * 2) = pk;
           }
+      }
       // the region is private to the wave: no barrier, the compiler's wait on the LDS writes is enough
       uint16_t *obase = reinterpret_cast<uint16_t *>(out) + (size_t)(m0 + wm * 128) * N + n0 + wn * 64;
       const int r_in = lane >> 3, c16 = lane & 7;
@@ -237,17 +282,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
       return;
     }
   }
+  constexpr int SUB = BF16_IN ? 16 : 32, NJ = 128 / SUB, NI = 64 / SUB, NG = BF16_IN ? 1 : 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int tok = m0 + wm * 128 + j * 32 + frag_row;
+  for (int j = 0; j < NJ; ++j) {
+    const int tok = m0 + wm * 128 + j * SUB + (BF16_IN ? (lane & 15) : frag_row);
     if (tok >= M) continue;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int f = n0 + wn * 64 + i * 32 + 8 * g + 4 * frag_half;
-        const float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
-        const float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+      for (int g = 0; g < NG; ++g) {
+        const int f = n0 + wn * 64 + i * SUB + (BF16_IN ? 4 * (lane >> 4) : 8 * g + 4 * frag_half);
+        float v0, v1, v2, v3;
+        if constexpr (BF16_IN) { v0 = acc16[i][j][0]; v1 = acc16[i][j][1]; v2 = acc16[i][j][2]; v3 = acc16[i][j][3]; }
+        else { v0 = acc[i][j][4 * g + 0]; v1 = acc[i][j][4 * g + 1]; v2 = acc[i][j][4 * g + 2]; v3 = acc[i][j][4 * g + 3]; }
         if constexpr (BF16_OUT) {
           uint16_t *o = reinterpret_cast<uint16_t *>(out) + (size_t)tok * N + f;
           if (f + 3 < N && (N & 3) == 0) {
