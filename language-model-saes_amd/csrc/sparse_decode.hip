@@ -39,14 +39,15 @@ __device__ __forceinline__ void load8(const void *row, int seg, float (&o)[8]) {
 
 // FWD: compute recon.  LOSS: also loss / grad_recon (implies FWD).  DVAL: compute dval from
 // grad_recon (own, when LOSS; read from memory otherwise).
-template <bool W_BF16, int SEGS, bool FWD, bool LOSS, bool DVAL>
-__global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
+template <bool W_BF16, int SEGS, bool FWD, bool LOSS, bool DVAL, int THREADS = DEC_THREADS>
+__global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
     const int32_t *__restrict__ idx, const float *__restrict__ val, const int64_t *__restrict__ row_off,
     const int32_t *__restrict__ row_nnz, const void *__restrict__ w_dec, const float *__restrict__ b_dec,
     const float *__restrict__ label, const float *__restrict__ tok_w, float *__restrict__ recon,
     float *__restrict__ loss_tok, float *__restrict__ grad_recon, float *__restrict__ dval, int d) {
   extern __shared__ __attribute__((aligned(16))) float g_lds[];  // [d] when DVAL
-  __shared__ float red[DEC_WAVES];
+  constexpr int WAVES = THREADS / 64;
+  __shared__ float red[WAVES];
   const int b = blockIdx.x, tid = threadIdx.x;
   const int64_t off = row_off[b];
   const int nnz = row_nnz[b];
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
         const char *row = wbase + (size_t)f * row_bytes;
 #pragma unroll
         for (int s = 0; s < SEGS; ++s) {
-          const int seg = tid + s * DEC_THREADS;
+          const int seg = tid + s * THREADS;
           if (seg < n_seg) load8<W_BF16>(row, seg, w[u][s]);
         }
       }
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
       const char *row = wbase + (size_t)f * row_bytes;
 #pragma unroll
       for (int s = 0; s < SEGS; ++s) {
-        const int seg = tid + s * DEC_THREADS;
+        const int seg = tid + s * THREADS;
         if (seg < n_seg) {
           float w[8];
           load8<W_BF16>(row, seg, w);
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
     const float tw = LOSS ? (tok_w ? tok_w[b] : 1.f) : 0.f;
 #pragma unroll
     for (int s = 0; s < SEGS; ++s) {
-      const int seg = tid + s * DEC_THREADS;
+      const int seg = tid + s * THREADS;
       if (seg < n_seg) {
         const size_t o = (size_t)b * d + (size_t)seg * 8;
         float r[8];
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
       }
     }
     if constexpr (LOSS) {
-      const float tot = block_sum<DEC_WAVES>(sq, red);
+      const float tot = block_sum<WAVES>(sq, red);
       if (tid == 0) loss_tok[b] = tw * tot;
     }
   }
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
   if constexpr (DVAL) {
     if constexpr (!LOSS) {
       // grad_recon comes from memory
-      for (int seg = tid; seg < n_seg; seg += DEC_THREADS) {
+      for (int seg = tid; seg < n_seg; seg += THREADS) {
         const float4 a = reinterpret_cast<const float4 *>(grad_recon + (size_t)b * d)[2 * seg];
         const float4 c = reinterpret_cast<const float4 *>(grad_recon + (size_t)b * d)[2 * seg + 1];
         reinterpret_cast<float4 *>(g_lds + seg * 8)[0] = a;
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
     }
     __syncthreads();
     const int lane = tid & 63, wave = tid >> 6;
-    for (int j = wave; j < nnz; j += DEC_WAVES) {
+    for (int j = wave; j < nnz; j += WAVES) {
       const int f = idx[off + j];
       const char *row = wbase + (size_t)f * row_bytes;
       float dot = 0.f;
@@ -190,7 +191,8 @@ __global__ __launch_bounds__(DEC_THREADS) void sparse_decode_kernel(
 template <bool W_BF16, bool FWD, bool LOSS, bool DVAL>
 static int launch_decode(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
                          const void *w_dec, const float *b_dec, const float *label, const float *tok_w, float *recon,
-                         float *loss_tok, float *grad_recon, float *dval, int64_t B, int64_t d, hipStream_t st) {
+                         float *loss_tok, float *grad_recon, float *dval, int64_t B, int64_t d, hipStream_t st,
+                         int64_t n_slots = 0) {
   const int n_seg = (int)(d / 8);
   const size_t lds = DVAL ? (size_t)d * sizeof(float) : 0;
   const int segs = (n_seg + DEC_THREADS - 1) / DEC_THREADS;
@@ -205,7 +207,16 @@ static int launch_decode(const int32_t *idx, const float *val, const int64_t *ro
     hipLaunchKernelGGL(kern, dim3((unsigned)B), dim3(DEC_THREADS), lds, st, idx, val, row_off, row_nnz, w_dec,    \
                        b_dec, label, tok_w, recon, loss_tok, grad_recon, dval, (int)d);                           \
   } while (0)
-  if (!FWD) SAE_DEC_LAUNCH(1);
+  // Short rows (d <= 1024): two waves per token, so that most lanes own a segment and twice as many tokens are
+  // resident per CU (the gathers' latency is hidden by resident tokens).  Not when the d val phase has long row
+  // lists to walk (more than 128 slots per token on average): there each wave takes one row at a time and four
+  // waves per token finish sooner (Lorsa's 64-row tokens 0.43 -> 0.30 ms with two waves, the CLT's up to 768-row
+  // prefix codes 4.7 -> 6.1 ms).
+  if (n_seg <= 128 && (!DVAL || n_slots <= 128 * B)) {
+    auto kern = sparse_decode_kernel<W_BF16, 1, FWD, LOSS, DVAL, 128>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)B), dim3(128), lds, st, idx, val, row_off, row_nnz, w_dec, b_dec, label,
+                       tok_w, recon, loss_tok, grad_recon, dval, (int)d);
+  } else if (!FWD) SAE_DEC_LAUNCH(1);
   else if (segs <= 1) SAE_DEC_LAUNCH(1);
   else if (segs <= 2) SAE_DEC_LAUNCH(2);
   else if (segs <= 4) SAE_DEC_LAUNCH(4);
@@ -255,9 +266,9 @@ extern "C" int sae_sparse_decode_bwd_dval(const int32_t *idx, const int64_t *row
   if (rc) return rc;
   if (w_dtype == SAE_BF16)
     return launch_decode<true, false, false, true>(idx, nullptr, row_off, row_nnz, w_dec, nullptr, nullptr, nullptr,
-                                                   nullptr, nullptr, const_cast<float *>(grad_recon), dval, B, d, st);
+                                                   nullptr, nullptr, const_cast<float *>(grad_recon), dval, B, d, st, n_slots);
   return launch_decode<false, false, false, true>(idx, nullptr, row_off, row_nnz, w_dec, nullptr, nullptr, nullptr,
-                                                  nullptr, nullptr, const_cast<float *>(grad_recon), dval, B, d, st);
+                                                  nullptr, nullptr, const_cast<float *>(grad_recon), dval, B, d, st, n_slots);
 }
 
 extern "C" int sae_sparse_decode_mse_fused(const int32_t *idx, const float *val, const int64_t *row_off,
@@ -275,7 +286,7 @@ extern "C" int sae_sparse_decode_mse_fused(const int32_t *idx, const float *val,
   if (rc) return rc;
   if (w_dtype == SAE_BF16)
     return launch_decode<true, true, true, true>(idx, val, row_off, row_nnz, w_dec, b_dec, label, tok_w, recon,
-                                                 loss_tok, grad_recon, dval, B, d, st);
+                                                 loss_tok, grad_recon, dval, B, d, st, n_slots);
   return launch_decode<false, true, true, true>(idx, val, row_off, row_nnz, w_dec, b_dec, label, tok_w, recon,
-                                                loss_tok, grad_recon, dval, B, d, st);
+                                                loss_tok, grad_recon, dval, B, d, st, n_slots);
 }
