@@ -39,7 +39,7 @@ __device__ __forceinline__ void load8(const void *row, int seg, float (&o)[8]) {
 
 // FWD: compute recon.  LOSS: also loss / grad_recon (implies FWD).  DVAL: compute dval from
 // grad_recon (own, when LOSS; read from memory otherwise).
-template <bool W_BF16, int SEGS, bool FWD, bool LOSS, bool DVAL, int THREADS = DEC_THREADS>
+template <bool W_BF16, int SEGS, bool FWD, bool LOSS, bool DVAL, int THREADS = DEC_THREADS, bool SHORT_LISTS = false>
 __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
     const int32_t *__restrict__ idx, const float *__restrict__ val, const int64_t *__restrict__ row_off,
     const int32_t *__restrict__ row_nnz, const void *__restrict__ w_dec, const float *__restrict__ b_dec,
@@ -158,6 +158,39 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
     }
     __syncthreads();
     const int lane = tid & 63, wave = tid >> 6;
+    if constexpr (SHORT_LISTS) {
+      // short rows (n_seg <= 128) and short row lists: a wave takes two rows at a time (four 16-byte loads in flight
+      // per lane instead of two); a lane's products run over its segments in ascending order as below, so a row's
+      // dot product has the same bits.  A separate instantiation: with long lists (the CLT's prefix codes) this
+      // path is slower (4.7 -> 6.4 ms), and its registers alone cost the other path residency (4.7 -> 7.2 ms).
+      for (int j0 = wave * 2; j0 < nnz; j0 += WAVES * 2) {
+        const bool two = j0 + 1 < nnz;
+        const int f0 = idx[off + j0], f1 = idx[off + (two ? j0 + 1 : j0)];
+        const char *row0 = wbase + (size_t)f0 * row_bytes, *row1 = wbase + (size_t)f1 * row_bytes;
+        float w0[2][8], w1[2][8];
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {
+          const int sg = lane + 64 * l;
+          if (sg < n_seg) { load8<W_BF16>(row0, sg, w0[l]); load8<W_BF16>(row1, sg, w1[l]); }
+        }
+        float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {
+          const int sg = lane + 64 * l;
+          if (sg < n_seg) {
+            const float4 g0 = reinterpret_cast<const float4 *>(g_lds + sg * 8)[0];
+            const float4 g1 = reinterpret_cast<const float4 *>(g_lds + sg * 8)[1];
+            d0 = fmaf(g0.x, w0[l][0], d0); d0 = fmaf(g0.y, w0[l][1], d0); d0 = fmaf(g0.z, w0[l][2], d0); d0 = fmaf(g0.w, w0[l][3], d0);
+            d0 = fmaf(g1.x, w0[l][4], d0); d0 = fmaf(g1.y, w0[l][5], d0); d0 = fmaf(g1.z, w0[l][6], d0); d0 = fmaf(g1.w, w0[l][7], d0);
+            d1 = fmaf(g0.x, w1[l][0], d1); d1 = fmaf(g0.y, w1[l][1], d1); d1 = fmaf(g0.z, w1[l][2], d1); d1 = fmaf(g0.w, w1[l][3], d1);
+            d1 = fmaf(g1.x, w1[l][4], d1); d1 = fmaf(g1.y, w1[l][5], d1); d1 = fmaf(g1.z, w1[l][6], d1); d1 = fmaf(g1.w, w1[l][7], d1);
+          }
+        }
+        d0 = wave_sum(d0); d1 = wave_sum(d1);
+        if (lane == 0) { dval[off + j0] = d0; if (two) dval[off + j0 + 1] = d1; }
+      }
+      return;
+    }
     for (int j = wave; j < nnz; j += WAVES) {
       const int f = idx[off + j];
       const char *row = wbase + (size_t)f * row_bytes;
@@ -212,8 +245,9 @@ static int launch_decode(const int32_t *idx, const float *val, const int64_t *ro
   // lists to walk (more than 128 slots per token on average): there each wave takes one row at a time and four
   // waves per token finish sooner (Lorsa's 64-row tokens 0.43 -> 0.30 ms with two waves, the CLT's up to 768-row
   // prefix codes 4.7 -> 6.1 ms).
-  if (n_seg <= 128 && (!DVAL || n_slots <= 128 * B)) {
-    auto kern = sparse_decode_kernel<W_BF16, 1, FWD, LOSS, DVAL, 128>;
+  const bool short_lists = n_slots <= 128 * B;   // also when the caller gave no slot count (forward only)
+  if (n_seg <= 128 && (!DVAL || short_lists)) {
+    auto kern = sparse_decode_kernel<W_BF16, 1, FWD, LOSS, DVAL, 128, true>;
     hipLaunchKernelGGL(kern, dim3((unsigned)B), dim3(128), lds, st, idx, val, row_off, row_nnz, w_dec, b_dec, label,
                        tok_w, recon, loss_tok, grad_recon, dval, (int)d);
   } else if (!FWD) SAE_DEC_LAUNCH(1);
