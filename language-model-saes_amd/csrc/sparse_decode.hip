@@ -62,8 +62,9 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[s][e] = 0.f;
 
-    // rows in flight per step, bounded so the staging registers stay below ~64 per lane
-    constexpr int U = SEGS <= 2 ? 4 : (SEGS == 4 ? 2 : 1);
+    // rows in flight per step.  Few: what hides the gathers' latency is the number of tokens resident on a CU, and
+    // the staging registers decide that (d = 4096: two rows, 8 waves per SIMD, 0.59 ms; four rows, 5 waves, 0.72 ms)
+    constexpr int U = SEGS == 1 ? 4 : (SEGS <= 4 ? 2 : 1);
     int j = 0;
     for (; j + U <= nnz; j += U) {
       float w[U][SEGS][8];
