@@ -197,10 +197,14 @@ int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, cons
  * (torch.optim.Adam, no weight decay, no amsgrad: trainer.py:375-390).  step = t >= 1.
  * shadow_bf16 (nullable) receives bf16(p) for the next step's GEMM / gather operands.
  * row_norm_out (nullable, requires row_len > 0 and n % row_len == 0) receives the L2 norm
- * of every updated row of length row_len, i.e. the next step's decoder_norm(). */
+ * of every updated row of length row_len, i.e. the next step's decoder_norm().
+ * row_grad_coef (nullable, fp32 [n / row_len], same requirement on row_len): the gradient of row r is
+ * g + row_grad_coef[r] * p.  This is how the gradient that reaches W_D through decoder_norm()
+ * (models/sae.py:136-147: d W_D[f, :] += (d n_f / n_f) W_D[f, :], e.g. from the tanh sparsity penalty,
+ * models/sparse_dictionary.py:897-906) is applied without a pass over [F, d] of its own. */
 int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
                   double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                  int64_t row_len, void *stream);
+                  int64_t row_len, const float *row_grad_coef, void *stream);
 
 /* Adam on a feature-major weight matrix [F, d] whose gradient is given in factored form:
  *   g[f, :] = sum_{s in segment f of the feature index} coef[s] * dense[slot_tok[s], :]

@@ -14,8 +14,8 @@ struct AdamScalars {
 // what to fuse to the compiler: the kernels that promise identical bits (the plain passes, the passes that rebuild
 // the gradient rows) then really compute the same thing.
 __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v, const AdamScalars &a) {
-  m = fmaf(a.one_minus_beta1, __fsub_rn(g, m), m);   // lerp, as torch does
-  v = fmaf(a.beta2, v, __fmul_rn(__fmul_rn(a.one_minus_beta2, g), g));
+  m = fmaf(a.one_minus_beta1, sub_rn(g, m), m);   // lerp, as torch does
+  v = fmaf(a.beta2, v, mul_rn(mul_rn(a.one_minus_beta2, g), g));
   const float denom = fmaf(sqrtf(v), a.inv_bc2_sqrt, a.eps);
   p = fmaf(-a.step_size, m / denom, p);
   return p;
@@ -53,20 +53,27 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
   }
 }
 
-// row-wise: one workgroup per row of row_len (a multiple of 4) elements; also emits the row norm
+// row-wise: one workgroup per row of row_len (a multiple of 4) elements; also emits the row norm.  With row_coef
+// the gradient of row r is g + row_coef[r] * p (product and sum rounded separately, as when that term is added to
+// the gradient tensor beforehand): the gradient that reaches a weight through its row norms, d n / n times the row.
 __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, const float *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int row_len,
                                                         AdamScalars a, uint16_t *__restrict__ shadow,
-                                                        float *__restrict__ row_norm) {
+                                                        float *__restrict__ row_norm, const float *__restrict__ row_coef) {
   __shared__ float red[4];
   const int64_t base4 = (int64_t)blockIdx.x * (row_len >> 2);
+  const float rc = row_coef ? row_coef[blockIdx.x] : 0.f;
   float sq = 0.f;
   for (int i = threadIdx.x; i < (row_len >> 2); i += 256) {
     const int64_t q = base4 + i;
     float4 pp = load_stream(p, q);
-    const float4 gg = load_stream(g, q);
+    float4 gg = load_stream(g, q);
     float4 mm = load_stream(m, q);
     float4 vv = load_stream(v, q);
+    if (row_coef) {
+      gg.x = add_rn(gg.x, mul_rn(rc, pp.x)); gg.y = add_rn(gg.y, mul_rn(rc, pp.y));
+      gg.z = add_rn(gg.z, mul_rn(rc, pp.z)); gg.w = add_rn(gg.w, mul_rn(rc, pp.w));
+    }
     adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
     adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
     store_stream(p, q, pp);
@@ -80,15 +87,17 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
       store_stream(shadow, q, o);
     }
   }
-  const float tot = block_sum<4>(sq, red);
-  if (threadIdx.x == 0) row_norm[blockIdx.x] = sqrtf(tot);
+  if (row_norm) {
+    const float tot = block_sum<4>(sq, red);
+    if (threadIdx.x == 0) row_norm[blockIdx.x] = sqrtf(tot);
+  }
 }
 
 }  // namespace sae
 
 extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
                              double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                             int64_t row_len, void *stream) {
+                             int64_t row_len, const float *row_grad_coef, void *stream) {
   using namespace sae;
   SAE_REQUIRE(p && g && m && v, SAE_ERR_INVALID_ARG, "adam_step: null pointer");
   SAE_REQUIRE(n > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step: n must be positive and step >= 1");
@@ -105,13 +114,13 @@ extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(bc2));
   a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
-  if (row_norm_out) {
+  if (row_norm_out || row_grad_coef) {
     SAE_REQUIRE(row_len > 0 && row_len % 4 == 0 && n % row_len == 0 && row_len < (1LL << 31), SAE_ERR_INVALID_ARG,
-                "adam_step: row_norm_out needs row_len %% 4 == 0 dividing n");
+                "adam_step: row_norm_out / row_grad_coef need row_len %% 4 == 0 dividing n");
     const int64_t rows = n / row_len;
     SAE_REQUIRE(rows < (1LL << 31), SAE_ERR_UNSUPPORTED, "adam_step: too many rows");
     hipLaunchKernelGGL(adam_rows_kernel, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
-                       reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out);
+                       reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
   } else {
     int64_t blocks = ((n >> 2) + 255) / 256;
     if (blocks < 1) blocks = 1;
@@ -194,8 +203,8 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
         if (grad_scale) {   // rounded products, as when the scaled gradient is written out before the step
-          g[u].x = __fmul_rn(g[u].x, gs); g[u].y = __fmul_rn(g[u].y, gs);
-          g[u].z = __fmul_rn(g[u].z, gs); g[u].w = __fmul_rn(g[u].w, gs);
+          g[u].x = mul_rn(g[u].x, gs); g[u].y = mul_rn(g[u].y, gs);
+          g[u].z = mul_rn(g[u].z, gs); g[u].w = mul_rn(g[u].w, gs);
         }
         if (sq_nnz_partial) {  // the same 4-element fp32 partials as sparse_rows_sq_nnz_kernel
           float s4 = g[u].x * g[u].x;

@@ -41,6 +41,25 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// ---- single operations that stay single ----------------------------------------------------
+// The compiler may fuse a product with a following sum into one fused multiply-add (and HIP's __fmul_rn /
+// __fadd_rn are plain operators, so they do not prevent it).  Where a result has to have the bits of two
+// separately rounded operations (kernels that promise the same bits as another route, or as the framework's
+// element-wise kernels), the operations go through these: an operation compiled with contraction off is never
+// fused, also after inlining.
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+
 // ---- wave (64 lanes) and block reductions ---------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -279,7 +279,7 @@ __global__ __launch_bounds__(256) void mse_auxk_kernel(const float *__restrict__
   const int64_t b = blockIdx.x;
   const int tid = threadIdx.x, n4 = d >> 2;
   const float w = tok_w ? tok_w[b] : 1.f;
-  const float ca = __fmul_rn(-2.f * alpha, w), cr = __fmul_rn(2.f, w);
+  const float ca = mul_rn(-2.f * alpha, w), cr = mul_rn(2.f, w);
   const float4 *rp = reinterpret_cast<const float4 *>(recon + b * d), *lp = reinterpret_cast<const float4 *>(label + b * d);
   const float4 *ap = aux ? reinterpret_cast<const float4 *>(aux + b * d) : nullptr;
   float sq_rec = 0.f, sq_aux = 0.f;
@@ -290,15 +290,15 @@ __global__ __launch_bounds__(256) void mse_auxk_kernel(const float *__restrict__
     float go[4], ga[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float diff = __fsub_rn(rv[e], lv[e]);
+      const float diff = sub_rn(rv[e], lv[e]);
       sq_rec = fmaf(diff, diff, sq_rec);
       ga[e] = 0.f;
       if (ap) {
-        const float r = __fsub_rn(__fsub_rn(lv[e], rv[e]), av[e]);
+        const float r = sub_rn(sub_rn(lv[e], rv[e]), av[e]);
         sq_aux = fmaf(r, r, sq_aux);
-        ga[e] = __fmul_rn(ca, r);
+        ga[e] = mul_rn(ca, r);
       }
-      go[e] = __fadd_rn(__fmul_rn(cr, diff), ga[e]);
+      go[e] = add_rn(mul_rn(cr, diff), ga[e]);
     }
     reinterpret_cast<float4 *>(grad_recon + b * d)[i] = make_float4(go[0], go[1], go[2], go[3]);
     if (ap && g_aux) reinterpret_cast<float4 *>(g_aux + b * d)[i] = make_float4(ga[0], ga[1], ga[2], ga[3]);

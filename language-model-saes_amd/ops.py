@@ -458,17 +458,25 @@ def sparse_grad_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Tensor, 
 
 def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, *, lr: float, beta1: float,
               beta2: float, eps: float, step: int, shadow_bf16: Optional[torch.Tensor] = None,
-              row_norm_out: Optional[torch.Tensor] = None, row_len: int = 0) -> None:
+              row_norm_out: Optional[torch.Tensor] = None, row_len: int = 0,
+              row_grad_coef: Optional[torch.Tensor] = None) -> None:
+    """One Adam update; with `row_grad_coef` (fp32, one value per row of `row_len` elements) the gradient of row r
+    is g + row_grad_coef[r] * p."""
     for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
         _req(t, name, torch.float32)
         if t.numel() != p.numel():
             raise ValueError(f"{name} must have {p.numel()} elements")
     if shadow_bf16 is not None:
         _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
+    if row_grad_coef is not None:
+        _req(row_grad_coef, "row_grad_coef", torch.float32, 1)
+        if row_len <= 0 or row_grad_coef.numel() * row_len != p.numel():
+            raise ValueError("row_grad_coef needs row_len > 0 and one value per row")
     with _timed("adam_step[matrix]" if p.ndim == 2 else "adam_step[vector]"):
         check(
             _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
-                                      eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _stream(p)),
+                                      eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _ptr(row_grad_coef),
+                                      _stream(p)),
             "adam_step",
         )
 

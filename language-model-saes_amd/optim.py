@@ -110,12 +110,15 @@ class HipAdam(Optimizer):
             for p in group["params"]:
                 if getattr(p, "_sparse_grad", None) is not None:
                     p._sparse_grad = None
+                if getattr(p, "_row_grad_coef", None) is not None:
+                    p._row_grad_coef = None
 
     @torch.no_grad()
     def materialize_grads(self) -> None:
         """Turn factored weight gradients into ordinary dense `.grad` tensors (for gradient clipping,
         the grad-norm diagnostic, or a different optimiser)."""
         for group in self.param_groups:
+            fold_row_grad_coef(group["params"])
             for p in group["params"]:
                 sg = getattr(p, "_sparse_grad", None)
                 if sg is None:
@@ -206,6 +209,7 @@ class HipAdam(Optimizer):
         req, acc, wanted = self._norm_request, None, ()
         self._norm_request = None
         if req is not None:
+            fold_row_grad_coef(req[0])   # the norm is over the element-wise gradient
             wanted = {id(p) for p in req[0]}
             acc = torch.zeros(2, dtype=torch.float64, device=req[1].device)
         # pass 1: weights whose gradient arrives in factored form (also yields the encoder-bias gradient)
@@ -272,6 +276,11 @@ class HipAdam(Optimizer):
         for group in self.param_groups:
             b1, b2 = group["betas"]
             for p in group["params"]:
+                row_coef = getattr(p, "_row_grad_coef", None)
+                if row_coef is not None and (p.grad is None or p.ndim != 2 or p.shape[1] % 4 != 0 or not p.is_contiguous()
+                                             or not p.grad.is_contiguous()):
+                    fold_row_grad_coef([p])     # no row-wise kernel for this layout: add the term to the gradient
+                    row_coef = None
                 if p.grad is None:
                     continue
                 if p.dtype != torch.float32:
@@ -287,7 +296,9 @@ class HipAdam(Optimizer):
                 role, shadow, norm_out = self._by_products(p, pv)
                 ops.adam_step(pv, gv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"],
                               step=int(st["step"].item()), shadow_bf16=shadow, row_norm_out=norm_out,
-                              row_len=pv.shape[1] if norm_out is not None else 0)
+                              row_len=pv.shape[1] if (norm_out is not None or row_coef is not None) else 0,
+                              row_grad_coef=row_coef)
+                p._row_grad_coef = None
                 self._publish(p, role, shadow, norm_out)
         return loss
 
@@ -341,6 +352,19 @@ class HipSparseAdam(Optimizer):
         return loss
 
 
+def fold_row_grad_coef(params) -> None:
+    """Add a weight's pending row-norm gradient (`_row_grad_coef`: d n / n per row, left by the decoder-norm
+    Function for the optimiser) to its dense `.grad` as coef[:, None] * W, for consumers of the element-wise
+    gradient (norm, clipping, SparseAdam).  HipAdam.step applies it inside its update kernel instead."""
+    for p in params:
+        coef = getattr(p, "_row_grad_coef", None)
+        if coef is None:
+            continue
+        term = coef.view(-1, *([1] * (p.ndim - 1))) * p.detach()
+        p.grad = term if p.grad is None else p.grad + term
+        p._row_grad_coef = None
+
+
 def _grad_sq_nnz(params) -> torch.Tensor:
     """device double[2] = (sum g^2, #non-zero g) over dense `.grad`s and factored weight gradients alike.
     A factored gradient is reduced by a kernel that rebuilds its rows in registers; the bias gradient it
@@ -348,6 +372,7 @@ def _grad_sq_nnz(params) -> torch.Tensor:
     like any other).  The sums are cached (on the factored gradient; on a dense gradient tensor together with
     its version counter): the second norm of a step, the after-clipping diagnostic, launches almost nothing."""
     params = list(params)
+    fold_row_grad_coef(params)
     parts = []
     for p in params:
         whole = getattr(p, "_sparse_grad", None)

@@ -377,6 +377,48 @@ class _EncoderGemm(torch.autograd.Function):
         return dx, dW, None, None
 
 
+class _RowNormDeferred(torch.autograd.Function):
+    """n[f] = ||W[f, :]||_2 with the value taken from the cache the optimiser keeps.  Its gradient,
+    d W[f, :] = (d n_f / n_f) W[f, :] (what `torch.norm(W, dim=1)` sends back), is a per-row multiple of W: when
+    `owner` is given it is left on the parameter as `_row_grad_coef` for HipAdam, which applies it inside its
+    update kernel, instead of being formed as a dense [F, d] tensor and added to the other gradient."""
+
+    @staticmethod
+    def forward(ctx, W, n_value, owner):
+        ctx.save_for_backward(n_value)
+        ctx.param, ctx.owner = W, owner
+        return n_value.clone()
+
+    @staticmethod
+    def backward(ctx, g_n):
+        (n,) = ctx.saved_tensors
+        W = ctx.param
+        coef = torch.where(n > 0, g_n.to(torch.float32) / n, torch.zeros_like(n))
+        if ctx.owner is not None:
+            prev = getattr(W, "_row_grad_coef", None)
+            W._row_grad_coef = coef if prev is None else prev + coef
+            return None, None, None
+        return (coef[:, None] * W.detach()).to(W.dtype), None, None
+
+
+class _DenseDecode(torch.autograd.Function):
+    """acts @ W_D on the bf16 copy of W_D that the optimiser maintains, so that autocast's per-step cast of the
+    fp32 master (and its backward) is not run; the products are those of an autocast matmul (models/sae.py:367)."""
+
+    @staticmethod
+    def forward(ctx, acts, W_D, w_op):
+        ctx.save_for_backward(acts, w_op)
+        return acts @ w_op
+
+    @staticmethod
+    def backward(ctx, g):
+        acts, w_op = ctx.saved_tensors
+        gg = g.to(w_op.dtype)
+        d_acts = gg @ w_op.t() if ctx.needs_input_grad[0] else None
+        dW = (acts.t() @ gg).float() if ctx.needs_input_grad[1] else None
+        return d_acts, dW, None
+
+
 class _JumpReLUStep(torch.autograd.Function):
     """bias + decoder-norm scale + JumpReLU + the tanh / Lp penalty sums in one pass over [B, F]; the backward
     is one more pass that also yields the bias, threshold and decoder-norm gradients.  `norm` is the decoder
@@ -612,11 +654,17 @@ class SparseAutoEncoder(SparseDictionary):
         pre = _EncoderGemm.apply(x, self.W_E, self._w_enc_operand(amp), amp)
         want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
         scaled = bool(self.cfg.sparsity_include_decoder_norm)
-        n = self.decoder_norm() if (scaled or want_tanh or want_lp) else None
+        n = None
+        if scaled or want_tanh or want_lp:
+            defer = self if (self.defer_weight_grads and torch.is_grad_enabled()) else None
+            n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), defer)
         acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
                                                      float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
                                                      want_tanh, want_lp)
-        reconstructed = acts @ self.W_D
+        if amp and acts.dtype == torch.bfloat16:
+            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(True))
+        else:
+            reconstructed = acts @ self.W_D
         if self.cfg.use_decoder_bias:
             reconstructed = reconstructed + self.b_D
         l_rec = apply_token_mask((reconstructed - label).pow(2).sum(dim=-1), 1, mask, "mean")

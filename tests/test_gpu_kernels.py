@@ -403,6 +403,28 @@ def test_adam_step_matches_torch(pkg, dev, n, row_len):
     assert rel_err(m, st["exp_avg"]) < 1e-6 and rel_err(v, st["exp_avg_sq"]) < 1e-6
 
 
+def test_adam_step_row_grad_coef_equals_adding_the_term_first(pkg, dev):
+    """g + coef[r] * p applied inside the update kernel gives the bits of adding coef[:, None] * p to g beforehand"""
+    g0 = torch.Generator().manual_seed(21)
+    F, d = 300, 768
+    p0 = torch.randn(F, d, generator=g0).to(dev)
+    grad = torch.randn(F, d, generator=g0).to(dev)
+    coef = (0.1 * torch.randn(F, generator=g0)).to(dev)
+    hyper = dict(lr=4e-4, beta1=0.9, beta2=0.999, eps=1e-8)
+    pa, ma, va = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    pb, mb, vb = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    na, nb = torch.empty(F, device=dev), torch.empty(F, device=dev)
+    for step in (1, 2, 3):
+        pkg.ops.adam_step(pa, grad + coef[:, None] * pa, ma, va, step=step, row_norm_out=na, row_len=d, **hyper)
+        pkg.ops.adam_step(pb, grad, mb, vb, step=step, row_norm_out=nb, row_len=d, row_grad_coef=coef, **hyper)
+        assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb) and torch.equal(na, nb)
+    pkg.ops.adam_step(pb, grad, mb, vb, step=4, row_len=d, row_grad_coef=coef, **hyper)      # without the norm output
+    pkg.ops.adam_step(pa, grad + coef[:, None] * pa, ma, va, step=4, **hyper)
+    assert torch.equal(pa, pb)
+    with pytest.raises(ValueError):
+        pkg.ops.adam_step(pb, grad, mb, vb, step=5, row_grad_coef=coef, **hyper)               # row_len missing
+
+
 @pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (128, 4096, 512, 4), (40, 5120, 96, 3)])
 @pytest.mark.parametrize("dense_dtype", [torch.float32, torch.bfloat16])
 def test_adam_step_sparse_rows_equals_grad_rows_then_adam(pkg, dev, B, d, F, k, dense_dtype):
