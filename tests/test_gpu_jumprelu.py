@@ -213,3 +213,35 @@ def test_jumprelu_step_bf16_and_adam(pkg, oracle, dev):
     with torch.autocast("cuda", dtype=torch.bfloat16):
         out2 = sae.compute_loss(gb, **kw)
     assert torch.isfinite(out2["loss"]) and out2["loss"].item() != out["loss"].item()
+
+
+def test_jumprelu_norm_gradient_inside_the_adam_kernel_equals_the_dense_route(pkg, oracle, dev):
+    """The gradient that reaches W_D through decoder_norm() is applied as a per-row coefficient inside the Adam
+    kernel when the optimiser owns the model; with that switched off it is a dense tensor added to the other
+    gradient.  Same bits after several steps, and the gradient norm (which needs the element-wise gradient) agrees."""
+    d, F, B = 64, 1024, 128
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=0.05)
+    models = []
+    for defer in (True, False):
+        sae, _, batch = make_pair(pkg, oracle, dev, d, F, B, seed=13, include_norm=True, window=0.3)
+        gb = {k: v.to(dev) for k, v in batch.items()}
+        groups = sae.get_parameters()
+        opt = pkg.HipAdam([{"params": groups[0]["params"]}, {"params": groups[1]["params"], "lr": 2e-3}], lr=1e-3,
+                          model=sae, defer_weight_grads=defer)
+        norms = []
+        for step in range(3):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                out = sae.compute_loss(gb, **kw)
+            out["loss"].backward()
+            if step == 0:
+                assert (getattr(sae.W_D, "_row_grad_coef", None) is not None) == defer
+            if step == 2:
+                norms.append(pkg.optim.compute_grad_norm([p for g in opt.param_groups for p in g["params"]]))
+                assert getattr(sae.W_D, "_row_grad_coef", None) is None      # folded into .grad for the norm
+            opt.step()
+            opt.zero_grad()
+        models.append((sae, norms))
+    (a, na), (b, nb) = models
+    for (n, p), (_, q) in zip(a.named_parameters(), b.named_parameters()):
+        assert torch.equal(p, q), n
+    assert torch.equal(na[0], nb[0])
