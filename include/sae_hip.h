@@ -195,6 +195,8 @@ int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, cons
  *   m = b1*m + (1-b1)*g;  v = b2*v + (1-b2)*g*g;
  *   p -= lr / (1 - b1^t) * m / (sqrt(v) / sqrt(1 - b2^t) + eps)
  * (torch.optim.Adam, no weight decay, no amsgrad: trainer.py:375-390).  step = t >= 1.
+ * g is fp32 or bf16 (g_dtype): the weight gradient of an autocast matmul is a bf16 tensor that the framework
+ * widens to fp32 in a pass of its own before torch.optim.Adam reads it; here it is widened as it is read.
  * shadow_bf16 (nullable) receives bf16(p) for the next step's GEMM / gather operands.
  * row_norm_out (nullable, requires row_len > 0 and n % row_len == 0) receives the L2 norm
  * of every updated row of length row_len, i.e. the next step's decoder_norm().
@@ -202,7 +204,7 @@ int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat_slot, cons
  * g + row_grad_coef[r] * p.  This is how the gradient that reaches W_D through decoder_norm()
  * (models/sae.py:136-147: d W_D[f, :] += (d n_f / n_f) W_D[f, :], e.g. from the tanh sparsity penalty,
  * models/sparse_dictionary.py:897-906) is applied without a pass over [F, d] of its own. */
-int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
+int sae_adam_step(float *p, const void *g, int g_dtype, float *m, float *v, int64_t n, double lr, double beta1,
                   double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                   int64_t row_len, const float *row_grad_coef, void *stream);
 

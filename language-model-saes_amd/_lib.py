@@ -37,7 +37,7 @@ SIGNATURES = {
     "sae_feature_index_workspace_bytes": (_L, [_L, _L, _L]),
     "sae_build_feature_index": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P]),
     "sae_sparse_grad_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _P]),
-    "sae_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _L, _P, _P, _L, _P, _P]),
+    "sae_adam_step": (_I, [_P, _P, _I, _P, _P, _L, _F, _F, _F, _F, _L, _P, _P, _L, _P, _P]),
     "sae_sparse_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _P, _P, _P, _P]),
     "sae_grad_sq_nnz": (_I, [_P, _L, _P, _P]),
     "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P]),

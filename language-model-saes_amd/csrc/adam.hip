@@ -21,15 +21,33 @@ __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v,
   return p;
 }
 
+// four gradient elements from group q of an fp32 or a bf16 gradient (a bf16 value widens exactly)
+template <bool G_BF16>
+__device__ __forceinline__ float4 load_grad4(const void *g, int64_t q) {
+  if constexpr (G_BF16) {
+    const nt_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x2 *>(g) + q);
+    return make_float4(__uint_as_float(t[0] << 16), __uint_as_float(t[0] & 0xffff0000u), __uint_as_float(t[1] << 16),
+                       __uint_as_float(t[1] & 0xffff0000u));
+  } else {
+    return load_stream(reinterpret_cast<const float *>(g), q);
+  }
+}
+template <bool G_BF16>
+__device__ __forceinline__ float load_grad1(const void *g, int64_t i) {
+  if constexpr (G_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(g)[i]);
+  else return reinterpret_cast<const float *>(g)[i];
+}
+
 // flat: grid-stride over float4 groups
-__global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, const float *__restrict__ g,
+template <bool G_BF16>
+__global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, const void *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int64_t n,
                                                         AdamScalars a, uint16_t *__restrict__ shadow) {
   const int64_t n4 = n >> 2;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
     float4 pp = load_stream(p, i);
-    const float4 gg = load_stream(g, i);
+    const float4 gg = load_grad4<G_BF16>(g, i);
     float4 mm = load_stream(m, i);
     float4 vv = load_stream(v, i);
     adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
@@ -47,7 +65,7 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
   const int64_t t = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t < n) {
     float pp = p[t], mm = m[t], vv = v[t];
-    adam_one(pp, g[t], mm, vv, a);
+    adam_one(pp, load_grad1<G_BF16>(g, t), mm, vv, a);
     p[t] = pp; m[t] = mm; v[t] = vv;
     if (shadow) shadow[t] = f32_to_bf16_bits(pp);
   }
@@ -56,7 +74,8 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
 // row-wise: one workgroup per row of row_len (a multiple of 4) elements; also emits the row norm.  With row_coef
 // the gradient of row r is g + row_coef[r] * p (product and sum rounded separately, as when that term is added to
 // the gradient tensor beforehand): the gradient that reaches a weight through its row norms, d n / n times the row.
-__global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, const float *__restrict__ g,
+template <bool G_BF16>
+__global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, const void *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int row_len,
                                                         AdamScalars a, uint16_t *__restrict__ shadow,
                                                         float *__restrict__ row_norm, const float *__restrict__ row_coef) {
@@ -67,7 +86,7 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
   for (int i = threadIdx.x; i < (row_len >> 2); i += 256) {
     const int64_t q = base4 + i;
     float4 pp = load_stream(p, q);
-    float4 gg = load_stream(g, q);
+    float4 gg = load_grad4<G_BF16>(g, q);
     float4 mm = load_stream(m, q);
     float4 vv = load_stream(v, q);
     if (row_coef) {
@@ -95,11 +114,12 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
 
 }  // namespace sae
 
-extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64_t n, double lr, double beta1,
-                             double beta2, double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                             int64_t row_len, const float *row_grad_coef, void *stream) {
+extern "C" int sae_adam_step(float *p, const void *g, int g_dtype, float *m, float *v, int64_t n, double lr,
+                             double beta1, double beta2, double eps, int64_t step, void *shadow_bf16,
+                             float *row_norm_out, int64_t row_len, const float *row_grad_coef, void *stream) {
   using namespace sae;
   SAE_REQUIRE(p && g && m && v, SAE_ERR_INVALID_ARG, "adam_step: null pointer");
+  SAE_REQUIRE(g_dtype == SAE_F32 || g_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "adam_step: bad gradient dtype %d", g_dtype);
   SAE_REQUIRE(n > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step: n must be positive and step >= 1");
   SAE_REQUIRE((((uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v) & 15) == 0, SAE_ERR_INVALID_ARG,
               "adam_step: 16-byte alignment required");
@@ -119,14 +139,22 @@ extern "C" int sae_adam_step(float *p, const float *g, float *m, float *v, int64
                 "adam_step: row_norm_out / row_grad_coef need row_len %% 4 == 0 dividing n");
     const int64_t rows = n / row_len;
     SAE_REQUIRE(rows < (1LL << 31), SAE_ERR_UNSUPPORTED, "adam_step: too many rows");
-    hipLaunchKernelGGL(adam_rows_kernel, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
-                       reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
+    if (g_dtype == SAE_BF16)
+      hipLaunchKernelGGL(adam_rows_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
+                         reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
+    else
+      hipLaunchKernelGGL(adam_rows_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
+                         reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
   } else {
     int64_t blocks = ((n >> 2) + 255) / 256;
     if (blocks < 1) blocks = 1;
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(adam_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
-                       reinterpret_cast<uint16_t *>(shadow_bf16));
+    if (g_dtype == SAE_BF16)
+      hipLaunchKernelGGL(adam_flat_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
+                         reinterpret_cast<uint16_t *>(shadow_bf16));
+    else
+      hipLaunchKernelGGL(adam_flat_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
+                         reinterpret_cast<uint16_t *>(shadow_bf16));
   }
   return check_launch("adam_step");
 }

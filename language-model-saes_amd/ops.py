@@ -460,10 +460,13 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
               beta2: float, eps: float, step: int, shadow_bf16: Optional[torch.Tensor] = None,
               row_norm_out: Optional[torch.Tensor] = None, row_len: int = 0,
               row_grad_coef: Optional[torch.Tensor] = None) -> None:
-    """One Adam update; with `row_grad_coef` (fp32, one value per row of `row_len` elements) the gradient of row r
-    is g + row_grad_coef[r] * p."""
+    """One Adam update; `g` may be bf16 (widened as it is read); with `row_grad_coef` (fp32, one value per row of
+    `row_len` elements) the gradient of row r is g + row_grad_coef[r] * p."""
     for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
-        _req(t, name, torch.float32)
+        if name == "g" and t.dtype == torch.bfloat16:
+            _req(t, name, torch.bfloat16)
+        else:
+            _req(t, name, torch.float32)
         if t.numel() != p.numel():
             raise ValueError(f"{name} must have {p.numel()} elements")
     if shadow_bf16 is not None:
@@ -474,7 +477,7 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
             raise ValueError("row_grad_coef needs row_len > 0 and one value per row")
     with _timed("adam_step[matrix]" if p.ndim == 2 else "adam_step[vector]"):
         check(
-            _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
+            _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), _dt(g), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
                                       eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _ptr(row_grad_coef),
                                       _stream(p)),
             "adam_step",

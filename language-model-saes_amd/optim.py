@@ -112,6 +112,8 @@ class HipAdam(Optimizer):
                     p._sparse_grad = None
                 if getattr(p, "_row_grad_coef", None) is not None:
                     p._row_grad_coef = None
+                if getattr(p, "_lowp_grad", None) is not None:
+                    p._lowp_grad = None
 
     @torch.no_grad()
     def materialize_grads(self) -> None:
@@ -276,12 +278,16 @@ class HipAdam(Optimizer):
         for group in self.param_groups:
             b1, b2 = group["betas"]
             for p in group["params"]:
-                row_coef = getattr(p, "_row_grad_coef", None)
-                if row_coef is not None and (p.grad is None or p.ndim != 2 or p.shape[1] % 4 != 0 or not p.is_contiguous()
-                                             or not p.grad.is_contiguous()):
+                row_coef, lowp = getattr(p, "_row_grad_coef", None), getattr(p, "_lowp_grad", None)
+                if lowp is not None and (p.grad is not None or tuple(lowp.shape) != tuple(_flat_view(p).shape)
+                                         or not lowp.is_contiguous()):
+                    fold_row_grad_coef([p])     # a second, fp32 gradient as well (or an unexpected layout): one dense sum
+                    row_coef = lowp = None
+                if row_coef is not None and ((p.grad is None and lowp is None) or p.ndim != 2 or p.shape[1] % 4 != 0
+                                             or not p.is_contiguous() or (p.grad is not None and not p.grad.is_contiguous())):
                     fold_row_grad_coef([p])     # no row-wise kernel for this layout: add the term to the gradient
-                    row_coef = None
-                if p.grad is None:
+                    row_coef = lowp = None
+                if p.grad is None and lowp is None:
                     continue
                 if p.dtype != torch.float32:
                     raise TypeError("HipAdam updates fp32 master parameters")
@@ -289,7 +295,8 @@ class HipAdam(Optimizer):
                 st["step"] += 1
                 pv = _flat_view(p)
                 same_layout = lambda t: _flat_view(t) if t.stride() == p.stride() else None  # noqa: E731
-                gv, mv, vv = same_layout(p.grad), same_layout(st["exp_avg"]), same_layout(st["exp_avg_sq"])
+                mv, vv = same_layout(st["exp_avg"]), same_layout(st["exp_avg_sq"])
+                gv = lowp if lowp is not None else same_layout(p.grad)
                 if gv is None:
                     gv = p.grad.permute(_flat_order(p)).contiguous()
                 assert mv is not None and vv is not None, "optimizer state must share the parameter's layout"
@@ -298,7 +305,7 @@ class HipAdam(Optimizer):
                               step=int(st["step"].item()), shadow_bf16=shadow, row_norm_out=norm_out,
                               row_len=pv.shape[1] if (norm_out is not None or row_coef is not None) else 0,
                               row_grad_coef=row_coef)
-                p._row_grad_coef = None
+                p._row_grad_coef = p._lowp_grad = None
                 self._publish(p, role, shadow, norm_out)
         return loss
 
@@ -353,10 +360,16 @@ class HipSparseAdam(Optimizer):
 
 
 def fold_row_grad_coef(params) -> None:
-    """Add a weight's pending row-norm gradient (`_row_grad_coef`: d n / n per row, left by the decoder-norm
-    Function for the optimiser) to its dense `.grad` as coef[:, None] * W, for consumers of the element-wise
-    gradient (norm, clipping, SparseAdam).  HipAdam.step applies it inside its update kernel instead."""
+    """Bring what the backward left on a weight for HipAdam into its dense fp32 `.grad`, for consumers of the
+    element-wise gradient (norm, clipping, SparseAdam): a bf16 gradient over the parameter's storage
+    (`_lowp_grad`, widened), and the row-norm gradient (`_row_grad_coef`: d n / n per row, added as
+    coef[:, None] * W).  HipAdam.step otherwise takes both inside its update kernel."""
     for p in params:
+        lowp = getattr(p, "_lowp_grad", None)
+        if lowp is not None:
+            term = _grad_like(p, lowp.float())
+            p.grad = term if p.grad is None else p.grad + term
+            p._lowp_grad = None
         coef = getattr(p, "_row_grad_coef", None)
         if coef is None:
             continue

@@ -357,7 +357,7 @@ class _EncoderGemm(torch.autograd.Function):
     gradient is then dense as well and both backward products are plain library GEMMs."""
 
     @staticmethod
-    def forward(ctx, x, W_E, w_op, amp):
+    def forward(ctx, x, W_E, w_op, amp, defer=False):
         if amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())
             pre = ops.encoder_gemm(x_op, w_op, torch.bfloat16)
@@ -366,6 +366,8 @@ class _EncoderGemm(torch.autograd.Function):
             pre = ops.encoder_gemm(x_op, w_op, torch.float32)
         ctx.save_for_backward(x_op, w_op)
         ctx.x_dtype = x.dtype
+        # a bf16 weight gradient can stay bf16 until the optimiser reads it, when the parameter is stored feature-major
+        ctx.param = W_E if (defer and amp and W_E.ndim == 2 and W_E.stride() == (1, W_E.shape[0])) else None
         return pre
 
     @staticmethod
@@ -373,8 +375,21 @@ class _EncoderGemm(torch.autograd.Function):
         x_op, w_op = ctx.saved_tensors
         gg = g.to(w_op.dtype)
         dx = (gg @ w_op).to(ctx.x_dtype) if ctx.needs_input_grad[0] else None
-        dW = (gg.t() @ x_op).t().float() if ctx.needs_input_grad[1] else None     # [d, F] with feature-major strides
-        return dx, dW, None, None
+        dW = None
+        if ctx.needs_input_grad[1]:
+            rows = gg.t() @ x_op                                                   # [F, d]
+            if ctx.param is not None:
+                _leave_lowp_grad(ctx.param, rows)
+            else:
+                dW = rows.t().float()                                              # [d, F] with feature-major strides
+        return dx, dW, None, None, None
+
+
+def _leave_lowp_grad(param, rows: torch.Tensor) -> None:
+    """Leave a bf16 weight gradient ([rows, d] over the parameter's storage) on the parameter for HipAdam, which
+    widens it as its kernel reads it, instead of returning an fp32 copy to autograd."""
+    prev = getattr(param, "_lowp_grad", None)
+    param._lowp_grad = rows if prev is None else prev + rows
 
 
 class _RowNormDeferred(torch.autograd.Function):
@@ -406,8 +421,9 @@ class _DenseDecode(torch.autograd.Function):
     fp32 master (and its backward) is not run; the products are those of an autocast matmul (models/sae.py:367)."""
 
     @staticmethod
-    def forward(ctx, acts, W_D, w_op):
+    def forward(ctx, acts, W_D, w_op, defer=False):
         ctx.save_for_backward(acts, w_op)
+        ctx.param = W_D if (defer and W_D.is_contiguous()) else None
         return acts @ w_op
 
     @staticmethod
@@ -415,8 +431,14 @@ class _DenseDecode(torch.autograd.Function):
         acts, w_op = ctx.saved_tensors
         gg = g.to(w_op.dtype)
         d_acts = gg @ w_op.t() if ctx.needs_input_grad[0] else None
-        dW = (acts.t() @ gg).float() if ctx.needs_input_grad[1] else None
-        return d_acts, dW, None
+        dW = None
+        if ctx.needs_input_grad[1]:
+            rows = acts.t() @ gg                                                   # [F, d] bf16
+            if ctx.param is not None:
+                _leave_lowp_grad(ctx.param, rows)
+            else:
+                dW = rows.float()
+        return d_acts, dW, None, None
 
 
 class _JumpReLUStep(torch.autograd.Function):
@@ -651,18 +673,18 @@ class SparseAutoEncoder(SparseDictionary):
         mask = batch.get("mask")
         amp = _autocast_dtype("cuda") == torch.bfloat16
         jr = self.activation_function
-        pre = _EncoderGemm.apply(x, self.W_E, self._w_enc_operand(amp), amp)
+        defer = bool(self.defer_weight_grads and torch.is_grad_enabled())
+        pre = _EncoderGemm.apply(x, self.W_E, self._w_enc_operand(amp), amp, defer)
         want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
         scaled = bool(self.cfg.sparsity_include_decoder_norm)
         n = None
         if scaled or want_tanh or want_lp:
-            defer = self if (self.defer_weight_grads and torch.is_grad_enabled()) else None
-            n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), defer)
+            n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), self if defer else None)
         acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
                                                      float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
                                                      want_tanh, want_lp)
         if amp and acts.dtype == torch.bfloat16:
-            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(True))
+            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(True), defer)
         else:
             reconstructed = acts @ self.W_D
         if self.cfg.use_decoder_bias:

@@ -423,6 +423,20 @@ def test_adam_step_row_grad_coef_equals_adding_the_term_first(pkg, dev):
     assert torch.equal(pa, pb)
     with pytest.raises(ValueError):
         pkg.ops.adam_step(pb, grad, mb, vb, step=5, row_grad_coef=coef, **hyper)               # row_len missing
+    # a bf16 gradient is widened as it is read: the bits of converting it first (row-wise and flat kernels, odd tail)
+    g16 = grad.bfloat16()
+    for kwargs in (dict(row_norm_out=nb, row_len=d, row_grad_coef=coef), dict()):
+        pkg.ops.adam_step(pb, g16, mb, vb, step=5, **kwargs, **hyper)
+        kwargs_a = dict(kwargs, row_norm_out=na) if kwargs else {}
+        pkg.ops.adam_step(pa, g16.float(), ma, va, step=5, **kwargs_a, **hyper)
+        assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
+    q0 = torch.randn(1003, generator=g0).to(dev)
+    gq = torch.randn(1003, generator=g0).to(dev).bfloat16()
+    qa, qb = q0.clone(), q0.clone()
+    z = lambda: torch.zeros_like(q0)  # noqa: E731
+    pkg.ops.adam_step(qa, gq.float(), z(), z(), step=1, **hyper)
+    pkg.ops.adam_step(qb, gq, z(), z(), step=1, **hyper)
+    assert torch.equal(qa, qb)
 
 
 @pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (128, 4096, 512, 4), (40, 5120, 96, 3)])
