@@ -277,8 +277,8 @@ def select_topk_row(
     k = int(k)
     dev = pre.device
     # zero-filled: slots a row does not use (fewer than k positive entries) then hold feature 0 with value 0
-    idx = torch.zeros(B * k, dtype=torch.int32, device=dev)
-    val = torch.zeros(B * k, dtype=torch.float32, device=dev)
+    idx = torch.empty(B * k, dtype=torch.int32, device=dev)     # the kernel writes every slot (zeros in unused ones)
+    val = torch.empty(B * k, dtype=torch.float32, device=dev)
     row_off = torch.empty(B, dtype=torch.int64, device=dev)
     row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
     lib = _lib.load()
