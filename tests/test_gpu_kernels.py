@@ -546,6 +546,30 @@ def test_select_topk_batch_ties_and_degenerate(pkg, oracle, dev):
     check_batch_select(pkg, oracle, dev, peaked.bfloat16(), None, None, 2500)
 
 
+def test_select_topk_batch_random_sweep(pkg, oracle, dev):
+    """many small random cases against the oracle: shapes around the granule (64 / 32 elements) and list-capacity
+    boundaries, quantised values (ties at the threshold), all three k regimes, bias / scale / mask on and off"""
+    rng = np.random.default_rng(7)
+    g = torch.Generator().manual_seed(7)
+    for case in range(60):
+        B = int(rng.integers(1, 40))
+        F = int(rng.choice([1, 7, 31, 32, 33, 63, 64, 65, 127, 128, 200, 511, 512, 513, 1000, 2048, 4097]))
+        dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float32
+        levels = int(rng.choice([0, 0, 3, 17]))                        # 0: continuous values
+        pre = torch.randn(B, F, generator=g)
+        if levels:
+            pre = torch.round(pre * levels / 3) * 3 / levels          # few distinct values
+        pre = pre.to(dtype)
+        b_enc = 0.1 * torch.randn(F, generator=g) if rng.random() < 0.6 else None
+        scale = 0.5 + torch.rand(F, generator=g) if rng.random() < 0.6 else None
+        mask = (torch.rand(F, generator=g) < 0.5).float() if (scale is not None and rng.random() < 0.3) else None
+        k_total = int(rng.choice([0, 1, B, max(1, B * F // 50), B * F // 3, B * F]))
+        print(f"sweep case {case}: B={B} F={F} {dtype} levels={levels} k_total={k_total} "
+              f"bias={b_enc is not None} scale={scale is not None} mask={mask is not None}", flush=True)
+        check_batch_select(pkg, oracle, dev, pre, b_enc, scale, k_total, feat_mask=mask,
+                           k_on_device=bool(k_total > 0 and rng.random() < 0.3))
+
+
 def test_select_topk_batch_feature_mask(pkg, oracle, dev):
     """aux-k form: only masked-in (dead) features compete"""
     B, F = 16, 3000
