@@ -38,8 +38,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE) of this file, scaled by what the same counters read for
 # transfers of known size in the same runs: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this machine.
 HBM_TRAFFIC_GB = {
-    "encoder_gemm": 7.72, "adam_step_sparse_rows[f32 dense]": 18.14, "adam_step_sparse_rows[bf16 dense]": 16.01,
-    "sparse_decode_mse_fused": 4.39, "select_topk_row": 1.50,
+    "encoder_gemm": 7.61, "adam_step_sparse_rows[f32 dense]": 18.14, "adam_step_sparse_rows[bf16 dense]": 16.00,
+    "sparse_decode_mse_fused": 4.38, "select_topk_row": 1.50,
 }
 
 
