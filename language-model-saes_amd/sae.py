@@ -302,10 +302,13 @@ class _FusedSparseStep(torch.autograd.Function):
         ctx.has_b_D = b_D is not None
         ctx.defer_to = holder.defer_to
         ctx.mark_non_differentiable(recon)
+        ctx.set_materialize_grads(False)   # no [B, d] tensor of zeros for the output that carries no gradient
         return loss, recon
 
     @staticmethod
     def backward(ctx, g_loss, _g_recon):
+        if g_loss is None:
+            return (None,) * 10
         code = ctx.grad_code
         F = code.d_sae
         fi = ops.build_feature_index(code)
