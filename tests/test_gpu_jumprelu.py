@@ -245,3 +245,34 @@ def test_jumprelu_norm_gradient_inside_the_adam_kernel_equals_the_dense_route(pk
     for (n, p), (_, q) in zip(a.named_parameters(), b.named_parameters()):
         assert torch.equal(p, q), n
     assert torch.equal(na[0], nb[0])
+
+
+@pytest.mark.parametrize("clip", [0.0, 0.05])
+def test_jumprelu_trainer_steps_with_and_without_deferred_terms(pkg, oracle, dev, clip):
+    """`Trainer.train_one_step` on a JumpReLU SAE under bf16 autocast (gradient norm every step, clipping on or off):
+    the run whose optimiser takes the norm gradient and the bf16 weight gradients inside its kernels ends with the
+    bits of the run that gets them as dense fp32 gradients."""
+    d, F, B, steps = 64, 1024, 128, 4
+    finals = []
+    for defer in (True, False):
+        sae, _, batch = make_pair(pkg, oracle, dev, d, F, B, seed=14, include_norm=True, window=0.3)
+        gb = {k: v.to(dev) for k, v in batch.items()}
+        tcfg = pkg.TrainerConfig(lr=1e-3, lr_warm_up_steps=2, lr_cool_down_steps=1, total_training_tokens=B * steps,
+                                 amp_dtype=torch.bfloat16, sparsity_loss_type="tanh", l1_coefficient=0.05,
+                                 skip_metrics_calculation=True, log_frequency=2, clip_grad_norm=clip, k_warmup_steps=0,
+                                 l1_coefficient_warmup_steps=2)
+        trainer = pkg.Trainer(tcfg)
+        trainer.prepare(sae, gb)
+        assert sae.defer_weight_grads          # the trainer's optimiser owns the model
+        if not defer:
+            sae.defer_weight_grads = False
+        norms = []
+        for _ in range(steps):
+            out = trainer.train_one_step(sae, gb)
+            norms.append(float(out["grad_norm_before_clipping"]))
+        finals.append(({n: p.detach().clone() for n, p in sae.named_parameters()}, norms))
+    (a, na), (b, nb) = finals
+    for n in a:
+        assert torch.isfinite(a[n]).all()
+        assert torch.equal(a[n], b[n]), n
+    assert na == nb
