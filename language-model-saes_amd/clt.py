@@ -269,7 +269,9 @@ class CrossLayerTranscoder(SparseDictionary):
         with torch.no_grad():
             sq = torch.zeros(L, F, dtype=torch.float32, device=self.W_D[0].device)
             for j, w in enumerate(self.W_D):
-                n = ops.row_norm(w.detach().float().view((j + 1) * F, d)).view(j + 1, F)
+                # the optimiser's row pass leaves a group's row norms behind; otherwise one pass of the row-norm kernel
+                n = self._derive(f"W_D.{j}.norm", w, lambda old, w=w, j=j: ops.row_norm(
+                    w.detach().float().view((j + 1) * F, d), old)).view(j + 1, F)
                 sq[: j + 1] += n * n
             norms = sq.sqrt_()
         self._norm_cache = (vers, norms)

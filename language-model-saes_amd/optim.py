@@ -173,6 +173,14 @@ class HipAdam(Optimizer):
         sh2 = shadow.view(-1, d) if shadow is not None else None
         bias_param = getattr(sg, "bias_param", None)
         bias_buf = torch.zeros(p2.shape[0], dtype=torch.float32, device=p.device) if bias_param is not None else None
+        # a decoder group held as one block (a cross-layer transcoder's W_D[j]) also yields its row norms
+        want_norm = (role is not None and role.startswith("W_D.") and not hasattr(sg, "pieces") and d % 4 == 0
+                     and hasattr(self._model, "set_derived"))
+        norm_buf = None
+        if want_norm:
+            norm_buf = self._model.get_derived_buffer(f"{role}.norm")
+            if norm_buf is None or norm_buf.numel() != p2.shape[0]:
+                norm_buf = torch.empty(p2.shape[0], dtype=torch.float32, device=p.device)
         step = int(st["step"].item())
         covered = 0
         for r0, piece in sorted(_pieces(sg), key=lambda rp: rp[0]):
@@ -189,6 +197,7 @@ class HipAdam(Optimizer):
             ops.adam_step_sparse_rows(piece.fi, piece.coef, piece.dense_operand, p2[r0:r0 + n], m2[r0:r0 + n], v2[r0:r0 + n],
                                       lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"], step=step,
                                       shadow_bf16=None if sh2 is None else sh2[r0:r0 + n],
+                                      row_norm_out=None if norm_buf is None else norm_buf[r0:r0 + n],
                                       bias_grad_out=None if bias_buf is None else bias_buf[r0:r0 + n],
                                       grad_scale=piece.scale, grad_sq_nnz_acc=sums_out, extra=piece.extra)
             covered = r0 + n
@@ -201,6 +210,8 @@ class HipAdam(Optimizer):
         torch.autograd.graph.increment_version(p)
         if shadow is not None:
             self._model.set_derived(f"{role}.bf16", p, shadow)
+        if norm_buf is not None:
+            self._model.set_derived(f"{role}.norm", p, norm_buf)
 
     @torch.no_grad()
     def step(self, closure=None):
