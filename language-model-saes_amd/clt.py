@@ -109,8 +109,6 @@ class _FusedCLTStep(torch.autograd.Function):
                 cat = ops.select_topk_batch(pre_cat, flat(b_enc), flat(norms), k * B)
             layer_cnt = layer_counts(cat, L, F)
         prefix = torch.cumsum(layer_cnt, dim=1).to(torch.int32)           # entries of layers <= j, per token
-        _, valid = _slot_tokens(cat)
-        slot_layer = torch.div(cat.idx, F, rounding_mode="floor")
         tok_w = torch.full((B,), 1.0 / (L * B), dtype=torch.float32, device=x.device)
         w_dec_ops = m._w_dec_operands(amp)
         b_D = dec[L:]
@@ -121,7 +119,9 @@ class _FusedCLTStep(torch.autograd.Function):
             code_j = dataclasses.replace(cat, row_nnz=prefix[:, j].contiguous(), d_sae=(j + 1) * F)
             recon, loss_tok, grad_recon, dval_j = ops.sparse_decode_mse_fused(
                 code_j, w_dec_ops[j].view((j + 1) * F, d), b_D[j].detach(), label[j].contiguous(), tok_w)
-            dval = dval + torch.where(valid & (slot_layer <= j), dval_j, torch.zeros_like(dval_j))
+            # the merged code is sorted by layer inside a token, so a token's first prefix[b, j] slots are its entries of
+            # layers <= j; the kernel writes exactly those and leaves every other slot at 0
+            dval += dval_j
             recons.append(recon); grads.append(grad_recon)
             loss = loss_tok.sum() if loss is None else loss + loss_tok.sum()
         recon = torch.stack(recons, dim=0)
