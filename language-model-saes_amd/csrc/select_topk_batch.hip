@@ -26,8 +26,9 @@
 //             with an in-wave prefix sum, so indices ascend without a sort
 //
 // The candidate list holds B * F / 64 + 1024 entries.  When more keys reach the lower bound (a matrix
-// of few distinct values), next, count and emit read the matrix again instead, granule by granule
-// as gather does: same results, about twice the time.
+// of few distinct values, or k_total itself beyond the list: then gather is skipped), next, count and
+// emit read the matrix again instead, granule by granule as gather does: same results, about twice
+// the time.
 //
 // gather, next, count and emit give one WAVE to each token: it reads the token's granule maxima
 // 256 at a time, packs the surviving granules' numbers into a list, and reads them 32 at a time
@@ -75,12 +76,6 @@ __device__ __forceinline__ uint32_t bt_key(float pre, float b, float s, float fm
   float h1 = (pre + b) * s;
   if (has_mask) h1 = ((h1 / s) * fm) * s;   // aux-k: hidden_pre * dead * scale, op for op
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
-}
-
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { const uint32_t t = (uint32_t)__shfl_xor((int)v, o, 64); v = t > v ? t : v; }
-  return v;
 }
 
 template <bool BF16>
