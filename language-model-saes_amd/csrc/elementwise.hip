@@ -83,8 +83,17 @@ __global__ __launch_bounds__(256) void col_sum_partial_kernel(const float *__res
   const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (j >= n) return;
   const int64_t b0 = (int64_t)blockIdx.y * rows_per, b1 = min(B, b0 + rows_per);
+  // eight loads are issued before their sums (same order of additions): the loop is otherwise one load latency per row
   float s = 0.f;
-  for (int64_t b = b0; b < b1; ++b) s += src[b * n + j];
+  int64_t b = b0;
+  for (; b + 8 <= b1; b += 8) {
+    float t[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) t[q] = src[(b + q) * n + j];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) s += t[q];
+  }
+  for (; b < b1; ++b) s += src[b * n + j];
   part[(int64_t)blockIdx.y * n + j] = s;
 }
 
@@ -93,7 +102,15 @@ __global__ __launch_bounds__(256) void col_sum_final_kernel(const float *__restr
   const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (j >= n) return;
   float s = 0.f;
-  for (int c = 0; c < chunks; ++c) s += part[(int64_t)c * n + j];
+  int c = 0;
+  for (; c + 8 <= chunks; c += 8) {
+    float t[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) t[q] = part[(int64_t)(c + q) * n + j];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) s += t[q];
+  }
+  for (; c < chunks; ++c) s += part[(int64_t)c * n + j];
   out[j] = accumulate ? out[j] + s : s;
 }
 
