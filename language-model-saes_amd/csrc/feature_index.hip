@@ -151,51 +151,68 @@ __global__ __launch_bounds__(FI_THREADS) void fi_order_kernel(const int32_t *__r
   if (lane < len) feat_slot[lo + rank] = mine;
 }
 
-// Segments longer than 64 slots: one workgroup per feature runs a counting sort keyed by
-// token.  A feature occurs at most once per token, so a bitmap over the B tokens plus a
-// prefix popcount gives every slot its rank.  LDS: bitmap[ceil(B/32)] + prefix[ceil(B/32)].
-__global__ __launch_bounds__(FI_THREADS) void fi_order_long_kernel(const int32_t *__restrict__ feat_ptr,
+// Segments longer than 64 slots: a workgroup runs a counting sort keyed by token.  A feature occurs at most once
+// per token, so a bitmap over the B tokens plus a prefix popcount gives every slot its rank.
+// LDS: bitmap[ceil(B/32)] + prefix[ceil(B/32)].  Workgroup w looks at features w, w + gridDim.x, ... (FI_THREADS
+// of them per round, one per thread), lists the long ones in LDS and sorts them one after another: a sparse code
+// has few long segments, and a grid of one workgroup per feature spent its time starting workgroups that left
+// at once.
+constexpr int FI_LONG_GRID = 16384;
+__global__ __launch_bounds__(FI_THREADS) void fi_order_long_kernel(const int32_t *__restrict__ feat_ptr, int F,
                                                                    const int32_t *__restrict__ unordered,
                                                                    const int32_t *__restrict__ slot_tok, int B,
                                                                    int32_t *__restrict__ feat_slot) {
   extern __shared__ uint32_t fi_lds[];
-  __shared__ int32_t part[FI_THREADS];
-  const int f = blockIdx.x, tid = threadIdx.x;
-  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
-  if (hi - lo <= 64) return;
+  __shared__ int32_t part[FI_THREADS / 64];
+  __shared__ int32_t long_list[FI_THREADS];
+  __shared__ int32_t n_long;
+  const int tid = threadIdx.x;
   const int W = (B + 31) >> 5;
   uint32_t *bitmap = fi_lds;
   uint32_t *prefix = fi_lds + W;
-  for (int w = tid; w < W; w += FI_THREADS) bitmap[w] = 0u;
-  __syncthreads();
-  for (int i = lo + tid; i < hi; i += FI_THREADS) {
-    const int t = slot_tok[unordered[i]];
-    atomicOr(&bitmap[t >> 5], 1u << (t & 31));
-  }
-  __syncthreads();
-  const int per = (W + FI_THREADS - 1) / FI_THREADS;
-  const int wlo = tid * per, whi = min(W, wlo + per);
-  int s = 0;
-  for (int w = wlo; w < whi; ++w) s += __popc(bitmap[w]);
-  part[tid] = s;
-  __syncthreads();
-  for (int o = 1; o < FI_THREADS; o <<= 1) {
-    const int v = tid >= o ? part[tid - o] : 0;
+  for (int64_t first = blockIdx.x; first < F; first += (int64_t)gridDim.x * FI_THREADS) {
+    if (tid == 0) n_long = 0;
     __syncthreads();
-    part[tid] += v;
+    const int64_t mine = first + (int64_t)tid * gridDim.x;
+    if (mine < F && feat_ptr[mine + 1] - feat_ptr[mine] > 64) long_list[atomicAdd(&n_long, 1)] = (int32_t)mine;
     __syncthreads();
-  }
-  int run = part[tid] - s;
-  for (int w = wlo; w < whi; ++w) {
-    prefix[w] = (uint32_t)run;
-    run += __popc(bitmap[w]);
-  }
-  __syncthreads();
-  for (int i = lo + tid; i < hi; i += FI_THREADS) {
-    const int slot = unordered[i];
-    const int t = slot_tok[slot];
-    const int rank = (int)prefix[t >> 5] + __popc(bitmap[t >> 5] & ((1u << (t & 31)) - 1u));
-    feat_slot[lo + rank] = slot;
+    const int nl = n_long;
+    for (int q = 0; q < nl; ++q) {
+      const int f = long_list[q];
+      const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+      for (int w = tid; w < W; w += FI_THREADS) bitmap[w] = 0u;
+      __syncthreads();
+      for (int i = lo + tid; i < hi; i += FI_THREADS) {
+        const int t = slot_tok[unordered[i]];
+        atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+      }
+      __syncthreads();
+      const int per = (W + FI_THREADS - 1) / FI_THREADS;
+      const int wlo = tid * per, whi = min(W, wlo + per);
+      int s = 0;
+      for (int w = wlo; w < whi; ++w) s += __popc(bitmap[w]);
+      int incl = s;   // inclusive scan inside the wave, then the waves' totals through LDS
+      for (int o = 1; o < 64; o <<= 1) {
+        const int v = __shfl_up(incl, o);
+        if ((tid & 63) >= o) incl += v;
+      }
+      if ((tid & 63) == 63) part[tid >> 6] = incl;
+      __syncthreads();
+      int run = incl - s;
+      for (int w = 0; w < (tid >> 6); ++w) run += part[w];
+      for (int w = wlo; w < whi; ++w) {
+        prefix[w] = (uint32_t)run;
+        run += __popc(bitmap[w]);
+      }
+      __syncthreads();
+      for (int i = lo + tid; i < hi; i += FI_THREADS) {
+        const int slot = unordered[i];
+        const int t = slot_tok[slot];
+        const int rank = (int)prefix[t >> 5] + __popc(bitmap[t >> 5] & ((1u << (t & 31)) - 1u));
+        feat_slot[lo + rank] = slot;
+      }
+      __syncthreads();   // the bitmap is cleared again for the next feature
+    }
   }
 }
 
@@ -270,8 +287,8 @@ extern "C" int sae_build_feature_index(const int32_t *idx, const int64_t *row_of
   const unsigned feat_blocks = (unsigned)((F + (FI_THREADS / 64) - 1) / (FI_THREADS / 64));
   hipLaunchKernelGGL(fi_order_kernel, dim3(feat_blocks), dim3(FI_THREADS), 0, st, feat_ptr, (int)F, unordered, feat_slot);
   const size_t bitmap_lds = (size_t)2 * ((B + 31) / 32) * sizeof(uint32_t);
-  hipLaunchKernelGGL(fi_order_long_kernel, dim3((unsigned)F), dim3(FI_THREADS), bitmap_lds, st, feat_ptr, unordered,
-                     slot_tok, (int)B, feat_slot);
+  hipLaunchKernelGGL(fi_order_long_kernel, dim3((unsigned)(F < FI_LONG_GRID ? F : FI_LONG_GRID)), dim3(FI_THREADS), bitmap_lds,
+                     st, feat_ptr, (int)F, unordered, slot_tok, (int)B, feat_slot);
   return check_launch("build_feature_index");
 }
 
