@@ -305,6 +305,25 @@ def gpu_step_bench(args):
     return ms_per_step, timer.summary(), float(loss.item()), tokens, name, shape
 
 
+def mfma_probe() -> dict:
+    """Rate of back-to-back v_mfma_f32_16x16x32_bf16 from registers: the matrix cores' ceiling on this card at
+    the clock it grants, next to the published 2.5 PFLOP/s."""
+    import torch
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    dev = torch.device("cuda:0")
+    pkg.ops.mfma_probe(dev, 4096, 256)   # warm-up
+    best = 0.0
+    runs = []
+    for _ in range(5):
+        flop, ms = pkg.ops.mfma_probe(dev, 4096, 8192)
+        runs.append(round(flop / ms / 1e9, 1))
+        best = max(best, flop / ms / 1e9)
+    return {"probe": "v_mfma_f32_16x16x32_bf16 from registers, 4096 workgroups x 4 waves x 8192 x 32 instructions",
+            "tflops_best": round(best, 1), "tflops_runs": runs, "published_peak_tflops": 2500.0}
+
+
 def cpu_baseline(sample_batch: int, sample_features: int):
     """Oracle (the reference's eager op sequence on CPU) on a bounded sample of the workload:
     same d_model and k, `sample_features` of the 131072 dictionary features, `sample_batch` tokens.
@@ -357,6 +376,8 @@ def main():
     ap.add_argument("--cpu-sample-features", type=int, default=32768)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of a train step: the rate of register-only bf16 MFMA loops (one JSON line)")
     ap.add_argument("--clip", type=float, default=0.0, help="clip_grad_norm of the topk_trainer workload (0: norm only)")
     ap.add_argument("--overlap", action="store_true", help="run the decoder Adam pass on a second stream, overlapping the next GEMM")
     args = ap.parse_args()
@@ -364,6 +385,10 @@ def main():
         print("bench.py: this build measures one GPU only (no collectives are part of it); run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+
+    if args.mfma_probe:
+        print(json.dumps(mfma_probe()))
+        return
 
     ms_per_step, kernels, loss, tokens, name, shape = gpu_step_bench(args)
     work = algorithmic_work(*shape)

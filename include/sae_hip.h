@@ -369,6 +369,12 @@ int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float
                      int64_t B, int64_t F, void *d_pre, float *d_bias, float *d_theta, float *d_pen_norm,
                      void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Measurement aid, no counterpart in the reference: n_workgroups x 4 waves each issue iters x 32
+ * v_mfma_f32_16x16x32_bf16 from registers (no memory traffic in the loop) and write one float per lane to
+ * out [n_workgroups * 256].  *flop_out (host, optional) receives the flop count of the launch.  The rate it
+ * reaches is the matrix cores' ceiling on the card at the clock it runs at, which sae_encoder_gemm is read against. */
+int sae_mfma_probe(float *out, int64_t n_workgroups, int64_t iters, double *flop_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -7,7 +7,7 @@ synchronising.  torch is used for device memory and streams only.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -700,6 +700,21 @@ def recon_stats(label: torch.Tensor, recon: torch.Tensor, label_mean: torch.Tens
             "recon_stats",
         )
     return out
+
+
+def mfma_probe(device: torch.device, n_workgroups: int = 4096, iters: int = 4096) -> Tuple[float, float]:
+    """Run the register-only MFMA loop (`sae_mfma_probe`) once and return (flop of the launch, milliseconds)."""
+    import ctypes
+
+    out = torch.empty(n_workgroups * 256, dtype=torch.float32, device=device)
+    flop = ctypes.c_double(0.0)
+    lib = _lib.load()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    check(lib.sae_mfma_probe(out.data_ptr(), n_workgroups, iters, ctypes.addressof(flop), _stream(out)), "mfma_probe")
+    end.record()
+    end.synchronize()
+    return flop.value, start.elapsed_time(end)
 
 
 def gather_rows(src: torch.Tensor, row_idx: torch.Tensor, out_dtype: Optional[torch.dtype] = None, scale: float = 1.0,

@@ -581,3 +581,12 @@ def test_select_topk_batch_feature_mask(pkg, oracle, dev):
     code = check_batch_select(pkg, oracle, dev, pre, b_enc, scale, 8 * B, feat_mask=mask)
     assert (mask[code.idx.cpu().long()[: code.row_nnz.sum().item()]] == 1).all()
     check_batch_select(pkg, oracle, dev, pre, b_enc, scale, 8 * B, feat_mask=torch.zeros(F))  # nothing is dead
+
+
+@pytest.mark.gpu
+def test_mfma_probe_runs_and_counts_its_flop(pkg, dev):
+    flop, ms = pkg.ops.mfma_probe(dev, n_workgroups=64, iters=16)
+    assert flop == 2.0 * 16 * 16 * 32 * 32 * 16 * 4 * 64
+    assert ms > 0.0
+    with pytest.raises(RuntimeError):
+        pkg.ops.mfma_probe(dev, n_workgroups=0, iters=16)
