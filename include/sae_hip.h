@@ -236,6 +236,23 @@ int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot,
                               void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
                               const float *extra_rows, const float *extra_bias, void *stream);
 
+/* The two Adam entry points above for a dictionary whose dtype is bfloat16 (config.py:39 `dtype`; parameters,
+ * gradients and both moments are then bf16 tensors and torch.optim.Adam, trainer.py:375-390, updates them with its
+ * multi-tensor element-wise operations): p_bf16, m_bf16, v_bf16 are bf16 arrays, there is no shadow copy (the
+ * parameter is its own bf16 operand), and the update rounds to bf16 after every element-wise operation torch
+ * performs -- the gradient itself; lerp for m; mul, then addcmul for v; sqrt, the division by sqrt(1 - beta2^t)
+ * and the addition of eps for the denominator; addcdiv for p.  row_norm_out is the fp32 norm of the updated bf16
+ * rows.  No dense extra block (aux-k on a bf16 dictionary takes the reference's dense route). */
+int sae_adam_step_lowp(void *p_bf16, const void *g, int g_dtype, void *m_bf16, void *v_bf16, int64_t n, double lr,
+                       double beta1, double beta2, double eps, int64_t step, float *row_norm_out, int64_t row_len,
+                       const float *row_grad_coef, void *stream);
+int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                   const float *coef, const void *dense, int dense_dtype, void *p_bf16, void *m_bf16,
+                                   void *v_bf16, int64_t F, int64_t d, double lr, double beta1, double beta2,
+                                   double eps, int64_t step, float *row_norm_out, float *bias_grad_out,
+                                   const float *grad_scale, double *grad_sq_nnz_acc, void *workspace,
+                                   int64_t workspace_bytes, void *stream);
+
 /* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
  * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and
  *   p -= lr * sqrt(1 - b2^t) / (1 - b1^t) * m / (sqrt(v) + eps);

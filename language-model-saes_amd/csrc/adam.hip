@@ -7,7 +7,7 @@
 namespace sae {
 
 struct AdamScalars {
-  float beta1, beta2, one_minus_beta1, one_minus_beta2, step_size, inv_bc2_sqrt, eps;
+  float beta1, beta2, one_minus_beta1, one_minus_beta2, step_size, inv_bc2_sqrt, eps, bc2_sqrt;
 };
 
 // Every multiply-add is written out as a fused one, so that no kernel that inlines this leaves the choice of
@@ -19,6 +19,61 @@ __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v,
   const float denom = fmaf(sqrtf(v), a.inv_bc2_sqrt, a.eps);
   p = fmaf(-a.step_size, m / denom, p);
   return p;
+}
+
+// The update of a parameter held in bf16 with bf16 moments, as torch's multi-tensor Adam computes it on such
+// tensors (the reference's optimizer when the dictionary's dtype is bfloat16, trainer.py:375-390): every
+// element-wise operation works in fp32 and rounds its result to bf16 -- lerp for m; mul then addcmul for v;
+// sqrt, division by sqrt(bias correction 2) and the addition of eps for the denominator; addcdiv for p.  (With
+// beta2 = 0.999 the product v * beta2 mostly rounds back to v: that is what the reference's arithmetic does.)
+__device__ __forceinline__ float bf16_round(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+__device__ __forceinline__ float adam_one_lowp(float &p, float g, float &m, float &v, const AdamScalars &a) {
+  m = bf16_round(fmaf(a.one_minus_beta1, sub_rn(g, m), m));
+  v = bf16_round(mul_rn(v, a.beta2));
+  v = bf16_round(fmaf(mul_rn(a.one_minus_beta2, g), g, v));
+  float denom = bf16_round(sqrtf(v));
+  denom = bf16_round(denom / a.bc2_sqrt);
+  denom = bf16_round(add_rn(denom, a.eps));
+  p = bf16_round(fmaf(-a.step_size, m / denom, p));
+  return p;
+}
+template <bool S_BF16>
+__device__ __forceinline__ float adam_any(float &p, float g, float &m, float &v, const AdamScalars &a) {
+  if constexpr (S_BF16) return adam_one_lowp(p, bf16_round(g), m, v, a);
+  else return adam_one(p, g, m, v, a);
+}
+
+// four elements of group q of a parameter or moment array: fp32, or bf16 (widened exactly / rounded on the way out)
+template <bool S_BF16>
+__device__ __forceinline__ float4 load_state4(const float *base, int64_t q) {
+  if constexpr (S_BF16) {
+    const nt_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x2 *>(base) + q);
+    return make_float4(__uint_as_float(t[0] << 16), __uint_as_float(t[0] & 0xffff0000u), __uint_as_float(t[1] << 16),
+                       __uint_as_float(t[1] & 0xffff0000u));
+  } else {
+    return load_stream(base, q);
+  }
+}
+template <bool S_BF16>
+__device__ __forceinline__ void store_state4(float *base, int64_t q, const float4 &x) {
+  if constexpr (S_BF16) {
+    uint2 o;   // the values are bf16-representable already
+    o.x = (__float_as_uint(x.x) >> 16) | (__float_as_uint(x.y) & 0xffff0000u);
+    o.y = (__float_as_uint(x.z) >> 16) | (__float_as_uint(x.w) & 0xffff0000u);
+    store_stream(reinterpret_cast<uint16_t *>(base), q, o);
+  } else {
+    store_stream(base, q, x);
+  }
+}
+template <bool S_BF16>
+__device__ __forceinline__ float load_state1(const float *base, int64_t i) {
+  if constexpr (S_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(base)[i]);
+  else return base[i];
+}
+template <bool S_BF16>
+__device__ __forceinline__ void store_state1(float *base, int64_t i, float x) {
+  if constexpr (S_BF16) reinterpret_cast<uint16_t *>(base)[i] = (uint16_t)(__float_as_uint(x) >> 16);
+  else base[i] = x;
 }
 
 // four gradient elements from group q of an fp32 or a bf16 gradient (a bf16 value widens exactly)
@@ -38,23 +93,24 @@ __device__ __forceinline__ float load_grad1(const void *g, int64_t i) {
   else return reinterpret_cast<const float *>(g)[i];
 }
 
-// flat: grid-stride over float4 groups
-template <bool G_BF16>
+// flat: grid-stride over groups of four elements.  S_BF16: p, m, v point to bf16 arrays (the pointer type is
+// nominal) and the update is the low-precision one above.
+template <bool G_BF16, bool S_BF16 = false>
 __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, const void *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int64_t n,
                                                         AdamScalars a, uint16_t *__restrict__ shadow) {
   const int64_t n4 = n >> 2;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    float4 pp = load_stream(p, i);
+    float4 pp = load_state4<S_BF16>(p, i);
     const float4 gg = load_grad4<G_BF16>(g, i);
-    float4 mm = load_stream(m, i);
-    float4 vv = load_stream(v, i);
-    adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
-    adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
-    store_stream(p, i, pp);
-    store_stream(m, i, mm);
-    store_stream(v, i, vv);
+    float4 mm = load_state4<S_BF16>(m, i);
+    float4 vv = load_state4<S_BF16>(v, i);
+    adam_any<S_BF16>(pp.x, gg.x, mm.x, vv.x, a); adam_any<S_BF16>(pp.y, gg.y, mm.y, vv.y, a);
+    adam_any<S_BF16>(pp.z, gg.z, mm.z, vv.z, a); adam_any<S_BF16>(pp.w, gg.w, mm.w, vv.w, a);
+    store_state4<S_BF16>(p, i, pp);
+    store_state4<S_BF16>(m, i, mm);
+    store_state4<S_BF16>(v, i, vv);
     if (shadow) {
       uint2 o;
       o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
@@ -64,9 +120,9 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
   }
   const int64_t t = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t < n) {
-    float pp = p[t], mm = m[t], vv = v[t];
-    adam_one(pp, load_grad1<G_BF16>(g, t), mm, vv, a);
-    p[t] = pp; m[t] = mm; v[t] = vv;
+    float pp = load_state1<S_BF16>(p, t), mm = load_state1<S_BF16>(m, t), vv = load_state1<S_BF16>(v, t);
+    adam_any<S_BF16>(pp, load_grad1<G_BF16>(g, t), mm, vv, a);
+    store_state1<S_BF16>(p, t, pp); store_state1<S_BF16>(m, t, mm); store_state1<S_BF16>(v, t, vv);
     if (shadow) shadow[t] = f32_to_bf16_bits(pp);
   }
 }
@@ -74,7 +130,7 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
 // row-wise: one workgroup per row of row_len (a multiple of 4) elements; also emits the row norm.  With row_coef
 // the gradient of row r is g + row_coef[r] * p (product and sum rounded separately, as when that term is added to
 // the gradient tensor beforehand): the gradient that reaches a weight through its row norms, d n / n times the row.
-template <bool G_BF16>
+template <bool G_BF16, bool S_BF16 = false>
 __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, const void *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int row_len,
                                                         AdamScalars a, uint16_t *__restrict__ shadow,
@@ -85,19 +141,24 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
   float sq = 0.f;
   for (int i = threadIdx.x; i < (row_len >> 2); i += 256) {
     const int64_t q = base4 + i;
-    float4 pp = load_stream(p, q);
+    float4 pp = load_state4<S_BF16>(p, q);
     float4 gg = load_grad4<G_BF16>(g, q);
-    float4 mm = load_stream(m, q);
-    float4 vv = load_stream(v, q);
+    float4 mm = load_state4<S_BF16>(m, q);
+    float4 vv = load_state4<S_BF16>(v, q);
     if (row_coef) {
-      gg.x = add_rn(gg.x, mul_rn(rc, pp.x)); gg.y = add_rn(gg.y, mul_rn(rc, pp.y));
-      gg.z = add_rn(gg.z, mul_rn(rc, pp.z)); gg.w = add_rn(gg.w, mul_rn(rc, pp.w));
+      if constexpr (S_BF16) {   // both gradient terms exist as bf16 tensors before they are added
+        gg.x = add_rn(bf16_round(gg.x), bf16_round(mul_rn(rc, pp.x))); gg.y = add_rn(bf16_round(gg.y), bf16_round(mul_rn(rc, pp.y)));
+        gg.z = add_rn(bf16_round(gg.z), bf16_round(mul_rn(rc, pp.z))); gg.w = add_rn(bf16_round(gg.w), bf16_round(mul_rn(rc, pp.w)));
+      } else {
+        gg.x = add_rn(gg.x, mul_rn(rc, pp.x)); gg.y = add_rn(gg.y, mul_rn(rc, pp.y));
+        gg.z = add_rn(gg.z, mul_rn(rc, pp.z)); gg.w = add_rn(gg.w, mul_rn(rc, pp.w));
+      }
     }
-    adam_one(pp.x, gg.x, mm.x, vv.x, a); adam_one(pp.y, gg.y, mm.y, vv.y, a);
-    adam_one(pp.z, gg.z, mm.z, vv.z, a); adam_one(pp.w, gg.w, mm.w, vv.w, a);
-    store_stream(p, q, pp);
-    store_stream(m, q, mm);
-    store_stream(v, q, vv);
+    adam_any<S_BF16>(pp.x, gg.x, mm.x, vv.x, a); adam_any<S_BF16>(pp.y, gg.y, mm.y, vv.y, a);
+    adam_any<S_BF16>(pp.z, gg.z, mm.z, vv.z, a); adam_any<S_BF16>(pp.w, gg.w, mm.w, vv.w, a);
+    store_state4<S_BF16>(p, q, pp);
+    store_state4<S_BF16>(m, q, mm);
+    store_state4<S_BF16>(v, q, vv);
     sq = fmaf(pp.x, pp.x, sq); sq = fmaf(pp.y, pp.y, sq); sq = fmaf(pp.z, pp.z, sq); sq = fmaf(pp.w, pp.w, sq);
     if (shadow) {
       uint2 o;
@@ -114,10 +175,10 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
 
 }  // namespace sae
 
-extern "C" int sae_adam_step(float *p, const void *g, int g_dtype, float *m, float *v, int64_t n, double lr,
-                             double beta1, double beta2, double eps, int64_t step, void *shadow_bf16,
-                             float *row_norm_out, int64_t row_len, const float *row_grad_coef, void *stream) {
-  using namespace sae;
+namespace sae {
+static int adam_step_impl(bool lowp, float *p, const void *g, int g_dtype, float *m, float *v, int64_t n, double lr,
+                          double beta1, double beta2, double eps, int64_t step, void *shadow_bf16,
+                          float *row_norm_out, int64_t row_len, const float *row_grad_coef, void *stream) {
   SAE_REQUIRE(p && g && m && v, SAE_ERR_INVALID_ARG, "adam_step: null pointer");
   SAE_REQUIRE(g_dtype == SAE_F32 || g_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "adam_step: bad gradient dtype %d", g_dtype);
   SAE_REQUIRE(n > 0 && step >= 1, SAE_ERR_INVALID_ARG, "adam_step: n must be positive and step >= 1");
@@ -132,6 +193,7 @@ extern "C" int sae_adam_step(float *p, const void *g, int g_dtype, float *m, flo
   const double bc2 = 1.0 - pow(beta2, (double)step);
   a.step_size = (float)(lr / bc1);
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(bc2));
+  a.bc2_sqrt = (float)sqrt(bc2);
   a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
   if (row_norm_out || row_grad_coef) {
@@ -139,24 +201,40 @@ extern "C" int sae_adam_step(float *p, const void *g, int g_dtype, float *m, flo
                 "adam_step: row_norm_out / row_grad_coef need row_len %% 4 == 0 dividing n");
     const int64_t rows = n / row_len;
     SAE_REQUIRE(rows < (1LL << 31), SAE_ERR_UNSUPPORTED, "adam_step: too many rows");
-    if (g_dtype == SAE_BF16)
-      hipLaunchKernelGGL(adam_rows_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
-                         reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
-    else
-      hipLaunchKernelGGL(adam_rows_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a,
-                         reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef);
+#define SAE_ADAM_DENSE_ROWS(GB, SB)                                                                                  \
+  hipLaunchKernelGGL((adam_rows_kernel<GB, SB>), dim3((unsigned)rows), dim3(256), 0, st, p, g, m, v, (int)row_len, a, \
+                     reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out, row_grad_coef)
+    if (lowp) { if (g_dtype == SAE_BF16) SAE_ADAM_DENSE_ROWS(true, true); else SAE_ADAM_DENSE_ROWS(false, true); }
+    else { if (g_dtype == SAE_BF16) SAE_ADAM_DENSE_ROWS(true, false); else SAE_ADAM_DENSE_ROWS(false, false); }
+#undef SAE_ADAM_DENSE_ROWS
   } else {
     int64_t blocks = ((n >> 2) + 255) / 256;
     if (blocks < 1) blocks = 1;
     if (blocks > 65536) blocks = 65536;
-    if (g_dtype == SAE_BF16)
-      hipLaunchKernelGGL(adam_flat_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
-                         reinterpret_cast<uint16_t *>(shadow_bf16));
-    else
-      hipLaunchKernelGGL(adam_flat_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a,
-                         reinterpret_cast<uint16_t *>(shadow_bf16));
+#define SAE_ADAM_FLAT(GB, SB)                                                                                 \
+  hipLaunchKernelGGL((adam_flat_kernel<GB, SB>), dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a, \
+                     reinterpret_cast<uint16_t *>(shadow_bf16))
+    if (lowp) { if (g_dtype == SAE_BF16) SAE_ADAM_FLAT(true, true); else SAE_ADAM_FLAT(false, true); }
+    else { if (g_dtype == SAE_BF16) SAE_ADAM_FLAT(true, false); else SAE_ADAM_FLAT(false, false); }
+#undef SAE_ADAM_FLAT
   }
   return check_launch("adam_step");
+}
+}  // namespace sae
+
+extern "C" int sae_adam_step(float *p, const void *g, int g_dtype, float *m, float *v, int64_t n, double lr,
+                             double beta1, double beta2, double eps, int64_t step, void *shadow_bf16,
+                             float *row_norm_out, int64_t row_len, const float *row_grad_coef, void *stream) {
+  return sae::adam_step_impl(false, p, g, g_dtype, m, v, n, lr, beta1, beta2, eps, step, shadow_bf16, row_norm_out, row_len,
+                             row_grad_coef, stream);
+}
+
+extern "C" int sae_adam_step_lowp(void *p_bf16, const void *g, int g_dtype, void *m_bf16, void *v_bf16, int64_t n, double lr,
+                                  double beta1, double beta2, double eps, int64_t step, float *row_norm_out,
+                                  int64_t row_len, const float *row_grad_coef, void *stream) {
+  return sae::adam_step_impl(true, reinterpret_cast<float *>(p_bf16), g, g_dtype, reinterpret_cast<float *>(m_bf16),
+                             reinterpret_cast<float *>(v_bf16), n, lr, beta1, beta2, eps, step, nullptr, row_norm_out,
+                             row_len, row_grad_coef, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -176,7 +254,7 @@ namespace sae {
 
 __global__ void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc);  // defined below
 
-template <bool DENSE_BF16, int U>
+template <bool DENSE_BF16, int U, bool S_BF16 = false>
 __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
@@ -218,9 +296,9 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
-        pp[u] = load_stream(p, base4 + seg);
-        mm[u] = load_stream(m, base4 + seg);
-        vv[u] = load_stream(v, base4 + seg);
+        pp[u] = load_state4<S_BF16>(p, base4 + seg);
+        mm[u] = load_state4<S_BF16>(m, base4 + seg);
+        vv[u] = load_state4<S_BF16>(v, base4 + seg);
       }
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -230,6 +308,9 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
+        if constexpr (S_BF16) {   // the gradient is a bf16 tensor before anything reads it
+          g[u].x = bf16_round(g[u].x); g[u].y = bf16_round(g[u].y); g[u].z = bf16_round(g[u].z); g[u].w = bf16_round(g[u].w);
+        }
         if (grad_scale) {   // rounded products, as when the scaled gradient is written out before the step
           g[u].x = mul_rn(g[u].x, gs); g[u].y = mul_rn(g[u].y, gs);
           g[u].z = mul_rn(g[u].z, gs); g[u].w = mul_rn(g[u].w, gs);
@@ -240,11 +321,11 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
           g_sq += (double)s4;
           g_nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
         }
-        adam_one(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_one(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
-        adam_one(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_one(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
-        store_stream(p, base4 + seg, pp[u]);
-        store_stream(m, base4 + seg, mm[u]);
-        store_stream(v, base4 + seg, vv[u]);
+        adam_any<S_BF16>(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_any<S_BF16>(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
+        adam_any<S_BF16>(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_any<S_BF16>(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
+        store_state4<S_BF16>(p, base4 + seg, pp[u]);
+        store_state4<S_BF16>(m, base4 + seg, mm[u]);
+        store_state4<S_BF16>(v, base4 + seg, vv[u]);
         sq = fmaf(pp[u].x, pp[u].x, sq); sq = fmaf(pp[u].y, pp[u].y, sq);
         sq = fmaf(pp[u].z, pp[u].z, sq); sq = fmaf(pp[u].w, pp[u].w, sq);
         if (shadow) {
@@ -276,14 +357,14 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
 
 }  // namespace sae
 
-extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
-                                         const float *coef, const void *dense, int dense_dtype, float *p, float *m,
-                                         float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
-                                         double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
-                                         float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
-                                         void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
-                                         const float *extra_rows, const float *extra_bias, void *stream) {
-  using namespace sae;
+namespace sae {
+static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                      const float *coef, const void *dense, int dense_dtype, float *p, float *m,
+                                      float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
+                                      double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                                      float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
+                                      void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
+                                      const float *extra_rows, const float *extra_bias, void *stream) {
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: null pointer");
   SAE_REQUIRE((extra_map == nullptr) == (extra_rows == nullptr) && (((uintptr_t)extra_rows) & 15) == 0, SAE_ERR_INVALID_ARG,
@@ -303,25 +384,59 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
   a.one_minus_beta2 = (float)(1.0 - beta2);
   a.step_size = (float)(lr / (1.0 - pow(beta1, (double)step)));
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(1.0 - pow(beta2, (double)step)));
+  a.bc2_sqrt = (float)sqrt(1.0 - pow(beta2, (double)step));
   a.eps = (float)eps;
   hipStream_t st = (hipStream_t)stream;
   double *partial = grad_sq_nnz_acc ? reinterpret_cast<double *>(workspace) : nullptr;
   {
-#define SAE_ADAM_ROWS(BF, UU)                                                                                              \
-  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
-                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,            \
+#define SAE_ADAM_ROWS(BF, UU, SB)                                                                                              \
+  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU, SB>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
+                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,                \
                      bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias)
     // pieces of 4 elements per thread: short rows keep fewer registers, so more rows are in flight per CU
     const int u = d <= 1024 ? 1 : (d <= 2048 ? 2 : 4);
-    if (dense_dtype == SAE_BF16) {
-      if (u == 1) SAE_ADAM_ROWS(true, 1); else if (u == 2) SAE_ADAM_ROWS(true, 2); else SAE_ADAM_ROWS(true, 4);
+    if (lowp) {
+      if (dense_dtype == SAE_BF16) {
+        if (u == 1) SAE_ADAM_ROWS(true, 1, true); else if (u == 2) SAE_ADAM_ROWS(true, 2, true); else SAE_ADAM_ROWS(true, 4, true);
+      } else {
+        if (u == 1) SAE_ADAM_ROWS(false, 1, true); else if (u == 2) SAE_ADAM_ROWS(false, 2, true); else SAE_ADAM_ROWS(false, 4, true);
+      }
+    } else if (dense_dtype == SAE_BF16) {
+      if (u == 1) SAE_ADAM_ROWS(true, 1, false); else if (u == 2) SAE_ADAM_ROWS(true, 2, false); else SAE_ADAM_ROWS(true, 4, false);
     } else {
-      if (u == 1) SAE_ADAM_ROWS(false, 1); else if (u == 2) SAE_ADAM_ROWS(false, 2); else SAE_ADAM_ROWS(false, 4);
+      if (u == 1) SAE_ADAM_ROWS(false, 1, false); else if (u == 2) SAE_ADAM_ROWS(false, 2, false); else SAE_ADAM_ROWS(false, 4, false);
     }
 #undef SAE_ADAM_ROWS
   }
   if (partial) hipLaunchKernelGGL(sq_nnz_finish_kernel, dim3(1), dim3(1024), 0, st, partial, F, grad_sq_nnz_acc);
   return check_launch("adam_step_sparse_rows");
+}
+}  // namespace sae
+
+extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                         const float *coef, const void *dense, int dense_dtype, float *p, float *m,
+                                         float *v, int64_t F, int64_t d, double lr, double beta1, double beta2,
+                                         double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
+                                         float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
+                                         void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
+                                         const float *extra_rows, const float *extra_bias, void *stream) {
+  return sae::adam_step_sparse_rows_impl(false, feat_ptr, feat_slot, slot_tok, coef, dense, dense_dtype, p, m, v, F, d, lr,
+                                         beta1, beta2, eps, step, shadow_bf16, row_norm_out, bias_grad_out, grad_scale,
+                                         grad_sq_nnz_acc, workspace, workspace_bytes, extra_map, extra_rows, extra_bias,
+                                         stream);
+}
+
+extern "C" int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
+                                              const float *coef, const void *dense, int dense_dtype, void *p_bf16,
+                                              void *m_bf16, void *v_bf16, int64_t F, int64_t d, double lr, double beta1,
+                                              double beta2, double eps, int64_t step, float *row_norm_out,
+                                              float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
+                                              void *workspace, int64_t workspace_bytes, void *stream) {
+  return sae::adam_step_sparse_rows_impl(true, feat_ptr, feat_slot, slot_tok, coef, dense, dense_dtype,
+                                         reinterpret_cast<float *>(p_bf16), reinterpret_cast<float *>(m_bf16),
+                                         reinterpret_cast<float *>(v_bf16), F, d, lr, beta1, beta2, eps, step, nullptr,
+                                         row_norm_out, bias_grad_out, grad_scale, grad_sq_nnz_acc, workspace,
+                                         workspace_bytes, nullptr, nullptr, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -461,21 +461,33 @@ def adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor
               row_norm_out: Optional[torch.Tensor] = None, row_len: int = 0,
               row_grad_coef: Optional[torch.Tensor] = None) -> None:
     """One Adam update; `g` may be bf16 (widened as it is read); with `row_grad_coef` (fp32, one value per row of
-    `row_len` elements) the gradient of row r is g + row_grad_coef[r] * p."""
+    `row_len` elements) the gradient of row r is g + row_grad_coef[r] * p.  A bf16 `p` (with bf16 `m`, `v`) takes the
+    low-precision update that rounds after every element-wise operation, as torch's Adam does on bf16 tensors."""
+    lowp = p.dtype == torch.bfloat16
     for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
         if name == "g" and t.dtype == torch.bfloat16:
             _req(t, name, torch.bfloat16)
         else:
-            _req(t, name, torch.float32)
+            _req(t, name, torch.bfloat16 if lowp and name != "g" else torch.float32)
         if t.numel() != p.numel():
             raise ValueError(f"{name} must have {p.numel()} elements")
     if shadow_bf16 is not None:
+        if lowp:
+            raise ValueError("a bf16 parameter has no shadow copy")
         _req(shadow_bf16, "shadow_bf16", torch.bfloat16)
     if row_grad_coef is not None:
         _req(row_grad_coef, "row_grad_coef", torch.float32, 1)
         if row_len <= 0 or row_grad_coef.numel() * row_len != p.numel():
             raise ValueError("row_grad_coef needs row_len > 0 and one value per row")
     with _timed("adam_step[matrix]" if p.ndim == 2 else "adam_step[vector]"):
+        if lowp:
+            check(
+                _lib.load().sae_adam_step_lowp(p.data_ptr(), g.data_ptr(), _dt(g), m.data_ptr(), v.data_ptr(), p.numel(), lr,
+                                               beta1, beta2, eps, int(step), _ptr(row_norm_out), int(row_len),
+                                               _ptr(row_grad_coef), _stream(p)),
+                "adam_step_lowp",
+            )
+            return
         check(
             _lib.load().sae_adam_step(p.data_ptr(), g.data_ptr(), _dt(g), m.data_ptr(), v.data_ptr(), p.numel(), lr, beta1, beta2,
                                       eps, int(step), _ptr(shadow_bf16), _ptr(row_norm_out), int(row_len), _ptr(row_grad_coef),
@@ -492,9 +504,13 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
     """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense);
     `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping);
     `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed;
-    `extra` adds a densely held block of gradient rows."""
+    `extra` adds a densely held block of gradient rows.  A bf16 `p` (with bf16 `m`, `v`) takes the low-precision
+    update (no shadow copy, no extra block)."""
+    lowp = p.dtype == torch.bfloat16
     for name, t in (("p", p), ("m", m), ("v", v)):
-        _req(t, name, torch.float32, 2)
+        _req(t, name, torch.bfloat16 if lowp else torch.float32, 2)
+    if lowp and (shadow_bf16 is not None or extra is not None):
+        raise ValueError("the low-precision update takes neither a shadow copy nor a dense row block")
     _req(coef, "coef", torch.float32, 1)
     _req(dense, "dense", ndim=2)
     F, d = p.shape
@@ -512,6 +528,16 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
         ws_bytes = 16 * F
         ws = torch.empty(2 * F, dtype=torch.float64, device=p.device)
     with _timed("adam_step_sparse_rows[bf16 dense]" if dense.dtype == torch.bfloat16 else "adam_step_sparse_rows[f32 dense]"):
+        if lowp:
+            check(
+                _lib.load().sae_adam_step_sparse_rows_lowp(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
+                                                           coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(),
+                                                           m.data_ptr(), v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step),
+                                                           _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale),
+                                                           _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, _stream(p)),
+                "adam_step_sparse_rows_lowp",
+            )
+            return
         check(
             _lib.load().sae_adam_step_sparse_rows(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), fi.slot_tok.data_ptr(),
                                                   coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),

@@ -467,6 +467,61 @@ def test_adam_step_sparse_rows_equals_grad_rows_then_adam(pkg, dev, B, d, F, k, 
     assert not torch.equal(pa, p0)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,row_len", [(4096 * 3, 0), (1003, 0), (512 * 768, 768)])
+def test_adam_step_on_bf16_tensors_follows_torch_adam(pkg, dev, n, row_len):
+    """bf16 parameter, gradient and moments: the oracle is the library routine itself, torch.optim.Adam on CPU
+    bf16 tensors (every element-wise op rounds to bf16).  Tolerance 2e-2 relative (bf16); nearly every element
+    agrees to the bit."""
+    print(f"adam lowp n={n} row_len={row_len}", flush=True)
+    g = torch.Generator().manual_seed(n)
+    p0 = torch.randn(n, generator=g).bfloat16()
+    ref_p = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.Adam([ref_p], lr=1e-2, betas=(0.9, 0.999), eps=1e-8, foreach=False)
+    p, m, v = p0.clone().to(dev), torch.zeros(n, dtype=torch.bfloat16, device=dev), torch.zeros(n, dtype=torch.bfloat16, device=dev)
+    norm = torch.empty(n // row_len, device=dev) if row_len else None
+    for step in range(1, 6):
+        grad = (torch.randn(n, generator=g) * 0.1).bfloat16()
+        ref_p.grad = grad.clone()
+        opt.step()
+        pkg.ops.adam_step(p, grad.to(dev), m, v, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, step=step,
+                          row_norm_out=norm, row_len=row_len)
+        st = opt.state[ref_p]
+        for name, got, want in (("p", p, ref_p.data), ("m", m, st["exp_avg"]), ("v", v, st["exp_avg_sq"])):
+            got, want = got.cpu().float(), want.float()
+            assert torch.allclose(got, want, rtol=2e-2, atol=1e-6), f"{name} at step {step}"
+            assert (got == want).float().mean().item() > 0.97, f"{name} at step {step}: too few identical elements"
+    assert not torch.equal(p.cpu(), p0)
+    if row_len:
+        assert torch.allclose(norm.cpu(), p.cpu().float().view(-1, row_len).norm(dim=1), rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 8), (300, 768, 1000, 16), (40, 5120, 96, 3)])
+def test_adam_step_sparse_rows_on_bf16_tensors_equals_grad_rows_then_adam(pkg, dev, B, d, F, k):
+    """bf16 state: rows rebuilt inside the pass == dense rows written out, rounded to bf16, then the plain pass"""
+    print(f"adam lowp sparse rows B={B} d={d} F={F} k={k}", flush=True)
+    code = random_code(pkg, dev, B, F, k, seed=d + B + 2)
+    fi = pkg.ops.build_feature_index(code)
+    g = torch.Generator().manual_seed(9)
+    dense = torch.randn(B, d, generator=g).bfloat16().to(dev)
+    coef = torch.randn(code.n_slots, generator=g).to(dev)
+    p0 = torch.randn(F, d, generator=g).bfloat16().to(dev)
+    hyper = dict(lr=4e-4, beta1=0.9, beta2=0.999, eps=1e-8)
+    z = lambda: torch.zeros(F, d, dtype=torch.bfloat16, device=dev)  # noqa: E731
+    pa, ma, va, pb, mb, vb = p0.clone(), z(), z(), p0.clone(), z(), z()
+    na, nb, bias_b = torch.empty(F, device=dev), torch.empty(F, device=dev), torch.empty(F, device=dev)
+    for step in (1, 2):
+        rows, bias_a = pkg.ops.sparse_grad_rows(fi, coef, dense, F, want_bias=True)
+        pkg.ops.adam_step(pa, rows.bfloat16(), ma, va, step=step, row_norm_out=na, row_len=d, **hyper)
+        pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=step, row_norm_out=nb, bias_grad_out=bias_b, **hyper)
+        assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
+        assert torch.equal(na, nb) and torch.equal(bias_a, bias_b)
+    assert not torch.equal(pa, p0)
+    with pytest.raises(ValueError):
+        pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=3, shadow_bf16=z(), **hyper)
+
+
 # ---------------------------------------------------------------------------------------------
 # BatchTopK select
 # ---------------------------------------------------------------------------------------------
