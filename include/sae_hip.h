@@ -109,6 +109,13 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
                            const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
                            int32_t *row_nnz, int cand_cap, void *stream);
 
+/* sae_select_topk_row for a dictionary whose dtype is bfloat16 (config.py:39): pre is bf16, and the sum with the
+ * bias, the product with the scale and the final quotient are each rounded to bf16, as the bf16 tensors
+ * `x @ W_E + b_E`, `hidden_pre * decoder_norm()` and `feature_acts / decoder_norm()` are (models/sae.py:324-341).
+ * b_enc / scale are fp32 copies of the bf16 bias / norms.  Keys then collide often; ties -> lowest feature index. */
+int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int k,
+                             int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream);
+
 /* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
  * (h0, h1 as above); ties at the threshold -> lowest flattened index b * F + f.  If fewer than
  * k_total entries are positive, all positives are kept.

@@ -28,6 +28,7 @@ SIGNATURES = {
     "sae_col_sum": (_I, [_P, _P, _L, _L, _I, _P, _L, _P]),
     "sae_encoder_gemm": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "sae_select_topk_row": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
+    "sae_select_topk_row_lowp": (_I, [_P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),
     "sae_select_topk_batch_workspace_bytes": (_L, [_L, _L]),
     "sae_select_topk_batch": (_I, [_P, _I, _P, _P, _P, _L, _L, _L, _P, _P, _P, _L, _P, _P, _P, _P, _L, _P]),

@@ -42,9 +42,19 @@ struct SelShared {
   int32_t digit_found;
 };
 
+// LOWP: the arithmetic of a dictionary whose parameters are bf16 tensors -- the sum with the bias and the product
+// with the norm are each rounded to bf16, as the tensors `x @ W_E + b_E` and `hidden_pre * decoder_norm()` are
+// (models/sae.py:324-335 with cfg.dtype = bfloat16); the bias and scale arrive as fp32 copies of bf16 values.
+__device__ __forceinline__ float sel_bf16_round(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+template <bool LOWP>
 __device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm, bool has_mask) {
-  float h1 = (pre + b) * s;
-  if (has_mask) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
+  float h1;
+  if constexpr (LOWP) {
+    h1 = sel_bf16_round(mul_rn(sel_bf16_round(add_rn(pre, b)), s));
+  } else {
+    h1 = (pre + b) * s;
+    if (has_mask) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
+  }
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
 
@@ -102,7 +112,7 @@ __device__ __forceinline__ void lds_kth_largest(SelShared *sh, int n, int k, Key
   }
 }
 
-template <bool BF16>
+template <bool BF16, bool LOWP = false>
 struct RowReader {
   const void *row;
   const float *b_enc;
@@ -162,14 +172,14 @@ struct RowReader {
       for (int e = 0; e < V; ++e) ss[e] = 1.f;
     }
 #pragma unroll
-    for (int e = 0; e < V; ++e) keys[e] = key_of(pre[e], bb[e], ss[e], mm[e], fmask != nullptr);
+    for (int e = 0; e < V; ++e) keys[e] = key_of<LOWP>(pre[e], bb[e], ss[e], mm[e], fmask != nullptr);
   }
   // key of one element
   __device__ __forceinline__ uint32_t key_at(int i) const {
     float pre;
     if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
     else pre = reinterpret_cast<const float *>(row)[i];
-    return key_of(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr);
+    return key_of<LOWP>(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr);
   }
   // calls fn(index, key) for every element of the row, vectorised when the row allows it
   template <typename Fn>
@@ -189,8 +199,8 @@ struct RowReader {
 };
 
 // Exact k-th largest over the whole row in global memory (general path).
-template <bool BF16>
-__device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<BF16> &rr, int k) {
+template <bool BF16, bool LOWP>
+__device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<BF16, LOWP> &rr, int k) {
   if (threadIdx.x == 0) { sh->prefix = 0u; sh->remaining = k; }
   uint32_t mask = 0u;
 #pragma unroll 1
@@ -215,7 +225,7 @@ __device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<B
 // handful per row) are formed again from memory.
 constexpr int SEL_STASH_ELEMS = 128;  // per thread: rows up to 131072 elements
 
-template <bool BF16, bool STASH>
+template <bool BF16, bool STASH, bool LOWP = false>
 __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   __shared__ SelShared sh;
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
-  RowReader<BF16> rr;
+  RowReader<BF16, LOWP> rr;
   rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
   rr.scale = scale;
@@ -234,7 +244,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   // ---- pass 1: per-thread maximum key and number of positive elements ----
   uint32_t my_max = 0u;
   int my_pos = 0;
-  constexpr int V = RowReader<BF16>::V;
+  constexpr int V = RowReader<BF16, LOWP>::V;
   constexpr int NCH = SEL_STASH_ELEMS / V;            // chunks per thread when stashing
   uint32_t cmax[STASH ? NCH : 1];                     // largest key of each of this thread's chunks
   if constexpr (STASH) {
@@ -330,7 +340,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   if (general) {
     // ---- general path: exact threshold over the whole row ----
     __syncthreads();
-    row_kth_largest<BF16>(&sh, rr, k_eff);
+    row_kth_largest<BF16, LOWP>(&sh, rr, k_eff);
     T = sh.prefix;
     need = sh.remaining;  // elements equal to T that are kept
     __syncthreads();
@@ -419,7 +429,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const float s = scale ? scale[my_idx] : 1.f;
     if (rank < k) {
       idx_out[(size_t)b * k + rank] = my_idx;
-      val_out[(size_t)b * k + rank] = scale ? h1 / s : h1;
+      val_out[(size_t)b * k + rank] = scale ? (LOWP ? sel_bf16_round(h1 / s) : h1 / s) : h1;
     }
   }
   for (int i = k_eff + tid; i < k; i += SEL_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
@@ -428,10 +438,10 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
 
 }  // namespace sae
 
-extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
-                                      const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
-                                      int cand_cap, void *stream) {
-  using namespace sae;
+namespace sae {
+static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                                const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,
+                                int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream) {
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
   SAE_REQUIRE(B > 0 && F > 0, SAE_ERR_INVALID_ARG, "select_topk_row: B and F must be positive");
   SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_row: bad dtype %d", pre_dtype);
@@ -446,16 +456,32 @@ extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const floa
   // every row 16-byte addressable and short enough for the register stash
   const bool stash = (F % V == 0) && F <= (int64_t)SEL_STASH_ELEMS * SEL_THREADS && (row_bytes % 16 == 0) &&
                      (((((uintptr_t)pre) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)feat_mask) & 15) == 0);
-#define SAE_LAUNCH_SELECT(BF, ST)                                                                                          \
-  hipLaunchKernelGGL((select_topk_row_kernel<BF, ST>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, scale,       \
-                     feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap)
-  if (pre_dtype == SAE_BF16) {
+#define SAE_LAUNCH_SELECT(BF, ST, ...)                                                                                     \
+  hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
+                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap)
+  if (lowp) {
+    if (stash) SAE_LAUNCH_SELECT(true, true, true); else SAE_LAUNCH_SELECT(true, false, true);
+  } else if (pre_dtype == SAE_BF16) {
     if (stash) SAE_LAUNCH_SELECT(true, true); else SAE_LAUNCH_SELECT(true, false);
   } else {
     if (stash) SAE_LAUNCH_SELECT(false, true); else SAE_LAUNCH_SELECT(false, false);
   }
 #undef SAE_LAUNCH_SELECT
   return check_launch("select_topk_row");
+}
+}  // namespace sae
+
+extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
+                                      const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,
+                                      int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream) {
+  return sae::select_topk_row_impl(false, pre, pre_dtype, b_enc, scale, feat_mask, B, F, k, idx, val, row_off, row_nnz, cand_cap,
+                                   stream);
+}
+
+extern "C" int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
+                                        int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
+  return sae::select_topk_row_impl(true, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz,
+                                   sae::SEL_CAP, stream);
 }
 
 extern "C" int sae_select_topk_row(const void *pre, int pre_dtype, const float *b_enc, const float *scale, int64_t B,

@@ -266,9 +266,14 @@ def select_topk_row(
     k: int,
     cand_cap: Optional[int] = None,
     feat_mask: Optional[torch.Tensor] = None,
+    lowp: bool = False,
 ) -> SparseCode:
+    """Per-token TopK of (pre + b_enc) * scale.  `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the
+    arithmetic of a dictionary whose parameters are bf16 tensors)."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
+    if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None or feat_mask is not None):
+        raise ValueError("lowp select takes a bf16 pre and neither cand_cap nor feat_mask")
     for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
         if t is not None:
             _req(t, name, torch.float32, 1)
@@ -284,7 +289,10 @@ def select_topk_row(
     lib = _lib.load()
     _t = _timed("select_topk_row")
     _t.__enter__()
-    if cand_cap is None and feat_mask is None:
+    if lowp:
+        rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(), val.data_ptr(),
+                                          row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+    elif cand_cap is None and feat_mask is None:
         rc = lib.sae_select_topk_row(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
                                      val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     else:

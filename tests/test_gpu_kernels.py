@@ -163,6 +163,29 @@ def test_select_topk_row_matches_torch_topk_when_tie_free(pkg, dev):
     assert torch.equal(code.idx.view(-1, k).cpu().long(), want)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,F,k", [(5, 4096, 16), (16, 24576, 64), (3, 1001, 8), (4, 131072, 64)])
+def test_select_topk_row_in_bf16_arithmetic(pkg, oracle, dev, B, F, k):
+    """a dictionary held in bf16: bias sum, norm product and final quotient are bf16 tensors in the reference
+    (models/sae.py:324-341).  The expected code is that op sequence on CPU bf16 tensors with the oracle's TopK."""
+    print(f"select lowp B={B} F={F} k={k}", flush=True)
+    g = torch.Generator().manual_seed(F + k + 1)
+    pre = torch.randn(B, F, generator=g).bfloat16()
+    b_enc = (0.1 * torch.randn(F, generator=g)).bfloat16()
+    norm = (0.5 + torch.rand(F, generator=g)).bfloat16()
+    h1 = (pre + b_enc) * norm
+    want = oracle.topk(h1 * h1.gt(0).to(h1.dtype), k=k, dim=-1) / norm
+    assert want.dtype == torch.bfloat16
+    code = pkg.ops.select_topk_row(pre.to(dev), b_enc.float().to(dev), norm.float().to(dev), k, lowp=True)
+    got = code.to_dense().cpu()
+    assert torch.equal(got != 0, want != 0), "kept sets differ"
+    assert torch.equal(got, want.float()), "kept values differ"
+    # the rounding makes ties at the threshold common; the plain arithmetic keeps another set
+    plain = pkg.ops.select_topk_row(pre.to(dev), b_enc.float().to(dev), norm.float().to(dev), k).to_dense().cpu()
+    if F >= 24576:
+        assert not torch.equal(plain != 0, want != 0)
+
+
 # ---------------------------------------------------------------------------------------------
 # sparse decode, fused loss, d val
 # ---------------------------------------------------------------------------------------------
