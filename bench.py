@@ -119,6 +119,26 @@ def build_topk(pkg, dev, args):
     return _autocast_step(sae, batch, opt, {}), B, name, (B, d, F, k)
 
 
+def build_topk_bf16_params(pkg, dev, args):
+    """The headline shape with the dictionary itself held in bf16 (cfg.dtype = bfloat16: bf16 parameters,
+    gradients and Adam moments, as the reference trains with that dtype).  A secondary figure: the reference's
+    default, and the headline, is fp32 parameters under bf16 autocast."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = args.batch or 4096, D_MODEL, args.d_sae or D_SAE, TOP_K
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
+                        dtype=torch.bfloat16)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, 64, seed=4).to(dev)
+    _init_sae_on_device(sae, x, d)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae)
+    name = f"topk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} bf16-parameters adam"
+    return _autocast_step(sae, batch, opt, {}), B, name, (B, d, F, k)
+
+
 def build_topk_trainer(pkg, dev, args):
     """The headline shape driven through `Trainer.train_one_step`: the step plus what the reference's loop
     adds around it every step (gradient norm over all parameters, the eight logging metrics, LR schedule)."""
@@ -268,7 +288,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
@@ -392,6 +412,9 @@ def main():
 
     ms_per_step, kernels, loss, tokens, name, shape = gpu_step_bench(args)
     work = algorithmic_work(*shape)
+    if args.workload == "topk_bf16_params":   # bf16 p, m, v read and written; no shadow copy
+        work["adam_step_sparse_rows[bf16 dense]"] = ("hbm", shape[1] * shape[2] * 12)
+        work["adam_step[vector]"] = ("hbm", (shape[1] + shape[2]) / 2 * 14)
     dominant = max(kernels, key=lambda n: kernels[n]["total_ms"])
     bound, per_launch = work.get(dominant, ("hbm", 0.0))
     avg_ms = kernels[dominant]["avg_ms"]
@@ -408,7 +431,7 @@ def main():
     per_kernel = {}
     # one dictionary shape for every launch of a kernel (the aux-k branch of "batchtopk" runs the GEMM and the
     # select on its compact block of dead features as well, CLT and Lorsa on several shapes)
-    uniform = args.workload in ("topk", "topk_trainer", "jumprelu", "activation_stream")
+    uniform = args.workload in ("topk", "topk_bf16_params", "topk_trainer", "jumprelu", "activation_stream")
     for kname, st in kernels.items():
         bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None

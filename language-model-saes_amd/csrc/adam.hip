@@ -26,21 +26,61 @@ __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v,
 // element-wise operation works in fp32 and rounds its result to bf16 -- lerp for m; mul then addcmul for v;
 // sqrt, division by sqrt(bias correction 2) and the addition of eps for the denominator; addcdiv for p.  (With
 // beta2 = 0.999 the product v * beta2 mostly rounds back to v: that is what the reference's arithmetic does.)
-__device__ __forceinline__ float bf16_round(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
-__device__ __forceinline__ float adam_one_lowp(float &p, float g, float &m, float &v, const AdamScalars &a) {
-  m = bf16_round(fmaf(a.one_minus_beta1, sub_rn(g, m), m));
-  v = bf16_round(mul_rn(v, a.beta2));
-  v = bf16_round(fmaf(mul_rn(a.one_minus_beta2, g), g, v));
-  float denom = bf16_round(sqrtf(v));
-  denom = bf16_round(denom / a.bc2_sqrt);
-  denom = bf16_round(add_rn(denom, a.eps));
-  p = bf16_round(fmaf(-a.step_size, m / denom, p));
-  return p;
+// Rounding goes through the hardware's packed conversion (two values per instruction); the square root, the
+// division by sqrt(bias correction 2) and the quotient m / denominator use the single-instruction forms (1 ulp in
+// fp32), whose error disappears in the rounding to bf16 that follows each of them except on rare boundary cases:
+// with IEEE division and square root sequences the pass is bound by its arithmetic, not by memory.
+typedef __attribute__((ext_vector_type(2))) float adam_f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 adam_bf16x2;
+__device__ __forceinline__ void bf16_round2(float &x, float &y) {
+  const adam_f32x2 in = {x, y};
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(in, adam_bf16x2));
+  x = __uint_as_float(packed << 16);
+  y = __uint_as_float(packed & 0xffff0000u);
+}
+__device__ __forceinline__ float bf16_round(float x) {
+  float y = x;
+  bf16_round2(x, y);
+  return x;
+}
+// two elements at a time; both lanes of a pair see exactly the scalar sequence
+__device__ __forceinline__ void adam_two_lowp(float &p0, float &p1, float g0, float g1, float &m0, float &m1, float &v0,
+                                              float &v1, const AdamScalars &a) {
+  bf16_round2(g0, g1);
+  m0 = fmaf(a.one_minus_beta1, sub_rn(g0, m0), m0); m1 = fmaf(a.one_minus_beta1, sub_rn(g1, m1), m1);
+  bf16_round2(m0, m1);
+  v0 = mul_rn(v0, a.beta2); v1 = mul_rn(v1, a.beta2);
+  bf16_round2(v0, v1);
+  v0 = fmaf(mul_rn(a.one_minus_beta2, g0), g0, v0); v1 = fmaf(mul_rn(a.one_minus_beta2, g1), g1, v1);
+  bf16_round2(v0, v1);
+  float d0 = __builtin_amdgcn_sqrtf(v0), d1 = __builtin_amdgcn_sqrtf(v1);
+  bf16_round2(d0, d1);
+  d0 = mul_rn(d0, a.inv_bc2_sqrt); d1 = mul_rn(d1, a.inv_bc2_sqrt);
+  bf16_round2(d0, d1);
+  d0 = add_rn(d0, a.eps); d1 = add_rn(d1, a.eps);
+  bf16_round2(d0, d1);
+  p0 = fmaf(-a.step_size, mul_rn(m0, __builtin_amdgcn_rcpf(d0)), p0);
+  p1 = fmaf(-a.step_size, mul_rn(m1, __builtin_amdgcn_rcpf(d1)), p1);
+  bf16_round2(p0, p1);
 }
 template <bool S_BF16>
-__device__ __forceinline__ float adam_any(float &p, float g, float &m, float &v, const AdamScalars &a) {
-  if constexpr (S_BF16) return adam_one_lowp(p, bf16_round(g), m, v, a);
-  else return adam_one(p, g, m, v, a);
+__device__ __forceinline__ void adam_any(float &p, float g, float &m, float &v, const AdamScalars &a) {
+  if constexpr (S_BF16) {
+    float p1 = p, m1 = m, v1 = v;
+    adam_two_lowp(p, p1, g, g, m, m1, v, v1, a);
+  } else {
+    adam_one(p, g, m, v, a);
+  }
+}
+template <bool S_BF16>
+__device__ __forceinline__ void adam_any4(float4 &p, const float4 &g, float4 &m, float4 &v, const AdamScalars &a) {
+  if constexpr (S_BF16) {
+    adam_two_lowp(p.x, p.y, g.x, g.y, m.x, m.y, v.x, v.y, a);
+    adam_two_lowp(p.z, p.w, g.z, g.w, m.z, m.w, v.z, v.w, a);
+  } else {
+    adam_one(p.x, g.x, m.x, v.x, a); adam_one(p.y, g.y, m.y, v.y, a);
+    adam_one(p.z, g.z, m.z, v.z, a); adam_one(p.w, g.w, m.w, v.w, a);
+  }
 }
 
 // four elements of group q of a parameter or moment array: fp32, or bf16 (widened exactly / rounded on the way out)
@@ -106,8 +146,7 @@ __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, c
     const float4 gg = load_grad4<G_BF16>(g, i);
     float4 mm = load_state4<S_BF16>(m, i);
     float4 vv = load_state4<S_BF16>(v, i);
-    adam_any<S_BF16>(pp.x, gg.x, mm.x, vv.x, a); adam_any<S_BF16>(pp.y, gg.y, mm.y, vv.y, a);
-    adam_any<S_BF16>(pp.z, gg.z, mm.z, vv.z, a); adam_any<S_BF16>(pp.w, gg.w, mm.w, vv.w, a);
+    adam_any4<S_BF16>(pp, gg, mm, vv, a);
     store_state4<S_BF16>(p, i, pp);
     store_state4<S_BF16>(m, i, mm);
     store_state4<S_BF16>(v, i, vv);
@@ -154,8 +193,7 @@ __global__ __launch_bounds__(256) void adam_rows_kernel(float *__restrict__ p, c
         gg.z = add_rn(gg.z, mul_rn(rc, pp.z)); gg.w = add_rn(gg.w, mul_rn(rc, pp.w));
       }
     }
-    adam_any<S_BF16>(pp.x, gg.x, mm.x, vv.x, a); adam_any<S_BF16>(pp.y, gg.y, mm.y, vv.y, a);
-    adam_any<S_BF16>(pp.z, gg.z, mm.z, vv.z, a); adam_any<S_BF16>(pp.w, gg.w, mm.w, vv.w, a);
+    adam_any4<S_BF16>(pp, gg, mm, vv, a);
     store_state4<S_BF16>(p, q, pp);
     store_state4<S_BF16>(m, q, mm);
     store_state4<S_BF16>(v, q, vv);
@@ -321,8 +359,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
           g_sq += (double)s4;
           g_nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
         }
-        adam_any<S_BF16>(pp[u].x, g[u].x, mm[u].x, vv[u].x, a); adam_any<S_BF16>(pp[u].y, g[u].y, mm[u].y, vv[u].y, a);
-        adam_any<S_BF16>(pp[u].z, g[u].z, mm[u].z, vv[u].z, a); adam_any<S_BF16>(pp[u].w, g[u].w, mm[u].w, vv[u].w, a);
+        adam_any4<S_BF16>(pp[u], g[u], mm[u], vv[u], a);
         store_state4<S_BF16>(p, base4 + seg, pp[u]);
         store_state4<S_BF16>(m, base4 + seg, mm[u]);
         store_state4<S_BF16>(v, base4 + seg, vv[u]);

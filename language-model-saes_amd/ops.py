@@ -616,7 +616,8 @@ def sparse_adam_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch
 
 
 def grad_sq_nnz(grads) -> torch.Tensor:
-    """device double[2]: (sum of squares, number of non-zero entries) over a list of fp32 tensors."""
+    """device double[2]: (sum of squares, number of non-zero entries) over a list of fp32 tensors (bf16 ones
+    are widened first: the small parameters of a dictionary held in bf16)."""
     grads = [g for g in grads if g is not None]
     assert len(grads) > 0, "No gradients found"
     acc = torch.zeros(2, dtype=torch.float64, device=grads[0].device)
@@ -624,6 +625,8 @@ def grad_sq_nnz(grads) -> torch.Tensor:
     for g in grads:
         if not g.is_contiguous():
             g = g.t() if g.ndim == 2 and g.t().is_contiguous() else g.contiguous()
+        if g.dtype == torch.bfloat16:
+            g = g.float()
         _req(g, "grad", torch.float32)
         with _timed("grad_sq_nnz"):
             check(lib.sae_grad_sq_nnz(g.data_ptr(), g.numel(), acc.data_ptr(), _stream(g)), "grad_sq_nnz")

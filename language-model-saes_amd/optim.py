@@ -126,9 +126,9 @@ class HipAdam(Optimizer):
                 if sg is None:
                     continue
                 rows, bias = sg.dense()
-                p.grad = _grad_like(p, rows)
+                p.grad = _grad_like(p, rows.to(p.dtype))
                 if bias is not None:
-                    sg.bias_param.grad = bias.view(sg.bias_param.shape)
+                    sg.bias_param.grad = bias.view(sg.bias_param.shape).to(sg.bias_param.dtype)
                 p._sparse_grad = None
 
     def _state(self, p):
@@ -204,7 +204,7 @@ class HipAdam(Optimizer):
         if covered != p2.shape[0]:
             raise NotImplementedError("row blocks of a factored gradient must tile the parameter")
         if bias_buf is not None:
-            g = bias_buf.view(bias_param.shape)
+            g = bias_buf.view(bias_param.shape).to(bias_param.dtype)
             bias_param.grad = g if bias_param.grad is None else bias_param.grad + g
         p._sparse_grad = None
         torch.autograd.graph.increment_version(p)
@@ -275,6 +275,7 @@ class HipAdam(Optimizer):
                     ev = torch.cuda.Event()
                     ev.record(side)
             if bias_out is not None:
+                bias_out = bias_out.to(sg.bias_param.dtype)
                 sg.bias_param.grad = bias_out if sg.bias_param.grad is None else sg.bias_param.grad + bias_out
             p._sparse_grad = None
             self._publish(p, role, shadow, norm_out)
@@ -300,8 +301,8 @@ class HipAdam(Optimizer):
                     row_coef = lowp = None
                 if p.grad is None and lowp is None:
                     continue
-                if p.dtype != torch.float32:
-                    raise TypeError("HipAdam updates fp32 master parameters")
+                if p.dtype not in (torch.float32, torch.bfloat16):
+                    raise TypeError("HipAdam updates fp32 or bf16 parameters")
                 st = self._state(p)
                 st["step"] += 1
                 pv = _flat_view(p)
@@ -378,13 +379,13 @@ def fold_row_grad_coef(params) -> None:
     for p in params:
         lowp = getattr(p, "_lowp_grad", None)
         if lowp is not None:
-            term = _grad_like(p, lowp.float())
+            term = _grad_like(p, lowp.to(p.dtype))
             p.grad = term if p.grad is None else p.grad + term
             p._lowp_grad = None
         coef = getattr(p, "_row_grad_coef", None)
         if coef is None:
             continue
-        term = coef.view(-1, *([1] * (p.ndim - 1))) * p.detach()
+        term = (coef.view(-1, *([1] * (p.ndim - 1))) * p.detach()).to(p.dtype)
         p.grad = term if p.grad is None else p.grad + term
         p._row_grad_coef = None
 
@@ -419,7 +420,7 @@ def _grad_sq_nnz(params) -> torch.Tensor:
                 own = torch.stack([own[0] * sg.scale.double().square().reshape(()), own[1]])
             parts.append(own)
         if bias_buf is not None:
-            g = bias_buf.view(bias_param.shape)
+            g = bias_buf.view(bias_param.shape).to(bias_param.dtype)
             bias_param.grad = g if bias_param.grad is None else bias_param.grad + g
             whole.bias_param = None
             for _, sg in _pieces(whole):

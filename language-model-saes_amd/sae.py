@@ -212,7 +212,14 @@ class _FusedSparseStep(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, label, tok_w, W_E, b_E, W_D, b_D, k, amp, holder):
         sae = holder.model
+        # a dictionary held in bf16 (cfg.dtype = bfloat16): the weights are their own bf16 operands, and the bias
+        # sum, norm product and quotient around the select are bf16 tensors in the reference
+        lowp = W_E.dtype == torch.bfloat16
+        amp = amp or lowp
         w_enc_op = sae._w_enc_operand(amp)
+        if lowp:
+            b_E = b_E.float()
+            b_D = b_D.float() if b_D is not None else None
         if amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)
@@ -222,13 +229,15 @@ class _FusedSparseStep(torch.autograd.Function):
         # decoder-side operands are fetched after the GEMM is enqueued: an overlapped decoder update of the
         # previous step (see HipAdam) is waited for here, not before the GEMM
         scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
+        if lowp and scale is not None:
+            scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
         w_dec_op = sae._w_dec_operand(amp)
         B = x.shape[0]
         batch_wide = sae.cfg.act_fn.lower() == "batchtopk"
         if batch_wide:
             code = ops.select_topk_batch(pre, b_E, scale, k * B)
         else:
-            code = ops.select_topk_row(pre, b_E, scale, k)
+            code = ops.select_topk_row(pre, b_E, scale, k, lowp=lowp)
         aux = holder.aux
         grad_recon_b16 = None   # set by the route that already has grad_recon in bf16
         if aux is None:
@@ -300,6 +309,7 @@ class _FusedSparseStep(torch.autograd.Function):
         ctx.n_tokens = B
         ctx.w_enc_op = w_enc_op
         ctx.has_b_D = b_D is not None
+        ctx.param_dtype = W_E.dtype
         ctx.defer_to = holder.defer_to
         ctx.mark_non_differentiable(recon)
         ctx.set_materialize_grads(False)   # no [B, d] tensor of zeros for the output that carries no gradient
@@ -334,8 +344,10 @@ class _FusedSparseStep(torch.autograd.Function):
                     sg = getattr(prm, "_sparse_grad", None)
                     if sg is not None:
                         rows, bias = sg.dense()
+                        rows = rows.to(prm.dtype)
                         prm.grad = rows if prm is sae.W_D else rows.t()
                         if bias is not None:
+                            bias = bias.to(sg.bias_param.dtype)
                             sg.bias_param.grad = bias if sg.bias_param.grad is None else sg.bias_param.grad + bias
                         prm._sparse_grad = None
             dW_D, _ = SparseRowGrad(fi, coef_dec, ctx.grad_dense_D, F, extra=extra_D).dense()
@@ -352,6 +364,9 @@ class _FusedSparseStep(torch.autograd.Function):
         dlabel = None
         if ctx.needs_input_grad[1]:
             dlabel = -ctx.grad_recon * g
+        pd = ctx.param_dtype
+        if pd != torch.float32:   # gradients of bf16 parameters are bf16 tensors
+            dW_Et, db_E, dW_D, db_D = (None if t is None else t.to(pd) for t in (dW_Et, db_E, dW_D, db_D))
         return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
@@ -655,7 +670,9 @@ class SparseAutoEncoder(SparseDictionary):
             and not self.cfg.use_glu_encoder
             and sparsity_loss_type is None and not (lp_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
-            and self.W_E.dtype == torch.float32
+            and (self.W_E.dtype == torch.float32
+                 or (self.W_E.dtype == torch.bfloat16 and self.cfg.act_fn.lower() == "topk" and not (auxk_coefficient > 0.0)
+                     and self.cfg.d_model % 64 == 0))
         )
 
     # ---- JumpReLU train-step loss: dense activations, so encoder kernel + one fused element-wise pass each way,

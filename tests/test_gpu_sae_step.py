@@ -35,7 +35,7 @@ class _SubstitutedMatmul(torch.autograd.Function):
         return (g.to(W.dtype) @ W.t()).to(x.dtype), (x.t().to(g.dtype) @ g).to(W.dtype), None
 
 
-def make_pair(pkg, oracle, dev, d, F, k, B, r, seed, include_norm, mask_frac=0.0):
+def make_pair(pkg, oracle, dev, d, F, k, B, r, seed, include_norm, mask_frac=0.0, dtype=torch.float32):
     from lm_saes_amd import synthetic
 
     x = synthetic.activations(B, d, r, seed)
@@ -47,10 +47,10 @@ def make_pair(pkg, oracle, dev, d, F, k, B, r, seed, include_norm, mask_frac=0.0
     w = (w[0], b_E, W_D.contiguous(), w[3])
     cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
                         top_k=k, norm_activation="inference", sparsity_include_decoder_norm=include_norm,
-                        device="cuda", dtype=torch.float32)
+                        device="cuda", dtype=dtype)
     sae = pkg.SparseAutoEncoder(cfg)
     synthetic.load_weights(sae, *[t.to(dev) for t in w])
-    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=include_norm)
+    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=include_norm, dtype=dtype)
     synthetic.load_weights(ref, *w)
     batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long)}
     if mask_frac > 0:
@@ -129,6 +129,69 @@ def test_fused_step_bf16_matches_oracle(pkg, oracle, dev, include_norm):
     for name in ("W_E", "b_E", "W_D", "b_D"):
         got, want = getattr(sae, name).grad, getattr(ref, name).grad
         assert got.dtype == torch.float32 and rel_err(got, want) < BF16_TOL, name
+
+
+@pytest.mark.parametrize("include_norm", [False, True])
+def test_fused_step_with_bf16_parameters_matches_oracle(pkg, oracle, dev, include_norm):
+    """cfg.dtype = bfloat16: parameters, gradients and the tensors around the select are bf16 in the reference.
+    The select must keep the same set (its arithmetic rounds where the reference's tensors do); the
+    reconstruction is compared to bf16 tolerance (the kernel keeps it in fp32, the reference rounds it)."""
+    print(f"fused step, bf16 parameters, include_norm={include_norm}", flush=True)
+    sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=7, include_norm=include_norm,
+                                dtype=torch.bfloat16)
+    assert sae.W_E.dtype == torch.bfloat16 and ref.W_E.dtype == torch.bfloat16
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=True, substitute=True)
+    assert "sparse_code" in ctx, "the fused route was not taken"
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert torch.equal(ctx["feature_acts"].cpu(), rctx["feature_acts"].float()), "kept values differ"
+    assert rel_err(ctx["reconstructed"], rctx["reconstructed"]) < BF16_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < BF16_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = getattr(sae, name).grad, getattr(ref, name).grad
+        assert got.dtype == torch.bfloat16 and got.shape == want.shape
+        assert rel_err(got, want) < BF16_TOL, name
+
+
+def test_bf16_parameters_step_with_adam_follows_torch_adam(pkg, oracle, dev):
+    """three steps of fused loss + HipAdam on a bf16 dictionary against the oracle + torch.optim.Adam on CPU bf16
+    tensors; factored gradients (no dense dW) and dense ones end at the same bits"""
+    finals = []
+    for defer in (True, False):
+        sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=8, include_norm=True,
+                                    dtype=torch.bfloat16)
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae, defer_weight_grads=defer)
+        gbatch = {k: v.to(dev) for k, v in batch.items()}
+        for _ in range(3):
+            loss = sae.compute_loss(gbatch, return_aux_data=False)
+            loss.backward()
+            if defer:
+                assert sae.W_D.grad is None and sae.W_D._sparse_grad is not None
+            opt.step()
+            opt.zero_grad()
+        for n, p in sae.named_parameters():
+            assert p.dtype == torch.bfloat16 and opt.state[p]["exp_avg"].dtype == torch.bfloat16, n
+        finals.append(({n: p.detach().clone() for n, p in sae.named_parameters()}, loss.item()))
+    (pa, la), (pb, lb) = finals
+    assert la == lb
+    for n in pa:
+        assert torch.equal(pa[n], pb[n]), n
+    # the oracle: same three steps with torch's Adam; selections may differ in a few near-ties (its matmul rounds
+    # differently), so the comparison is in tolerance
+    ropt = oracle.make_adam(ref, lr=4e-4)
+    before = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    for _ in range(3):
+        rloss = ref.compute_loss(batch)["loss"]
+        rloss.backward()
+        ropt.step(); ropt.zero_grad()
+    assert abs(la - rloss.item()) / rloss.item() < BF16_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = pa[name].cpu().float(), getattr(ref, name).detach().float()
+        assert (want != before[name].float()).any(), name
+        # an entry whose gradient differs (a selection flipped at a near-tie) moves the other way: bounded by a few
+        # times steps * lr, and rare
+        moved = (want - before[name].float()).abs().max().item()
+        assert (got - want).abs().max().item() <= 4 * moved, name
+        assert ((got - want).abs() > 0.5 * moved).float().mean().item() < 2e-2, name
 
 
 def test_fused_step_unsubstituted_agrees_statistically(pkg, oracle, dev):
