@@ -292,7 +292,7 @@ namespace sae {
 
 __global__ void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc);  // defined below
 
-template <bool DENSE_BF16, int U, bool S_BF16 = false>
+template <bool DENSE_BF16, int U>
 __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
@@ -334,9 +334,9 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
-        pp[u] = load_state4<S_BF16>(p, base4 + seg);
-        mm[u] = load_state4<S_BF16>(m, base4 + seg);
-        vv[u] = load_state4<S_BF16>(v, base4 + seg);
+        pp[u] = load_state4<false>(p, base4 + seg);
+        mm[u] = load_state4<false>(m, base4 + seg);
+        vv[u] = load_state4<false>(v, base4 + seg);
       }
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -346,9 +346,6 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
-        if constexpr (S_BF16) {   // the gradient is a bf16 tensor before anything reads it
-          g[u].x = bf16_round(g[u].x); g[u].y = bf16_round(g[u].y); g[u].z = bf16_round(g[u].z); g[u].w = bf16_round(g[u].w);
-        }
         if (grad_scale) {   // rounded products, as when the scaled gradient is written out before the step
           g[u].x = mul_rn(g[u].x, gs); g[u].y = mul_rn(g[u].y, gs);
           g[u].z = mul_rn(g[u].z, gs); g[u].w = mul_rn(g[u].w, gs);
@@ -359,10 +356,10 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
           g_sq += (double)s4;
           g_nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
         }
-        adam_any4<S_BF16>(pp[u], g[u], mm[u], vv[u], a);
-        store_state4<S_BF16>(p, base4 + seg, pp[u]);
-        store_state4<S_BF16>(m, base4 + seg, mm[u]);
-        store_state4<S_BF16>(v, base4 + seg, vv[u]);
+        adam_any4<false>(pp[u], g[u], mm[u], vv[u], a);
+        store_state4<false>(p, base4 + seg, pp[u]);
+        store_state4<false>(m, base4 + seg, mm[u]);
+        store_state4<false>(v, base4 + seg, vv[u]);
         sq = fmaf(pp[u].x, pp[u].x, sq); sq = fmaf(pp[u].y, pp[u].y, sq);
         sq = fmaf(pp[u].z, pp[u].z, sq); sq = fmaf(pp[u].w, pp[u].w, sq);
         if (shadow) {
@@ -388,6 +385,140 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     if (tid == 0) {
       sq_nnz_partial[2 * (size_t)f] = red_d[0] + red_d[1] + red_d[2] + red_d[3];
       sq_nnz_partial[2 * (size_t)f + 1] = red_d[4] + red_d[5] + red_d[6] + red_d[7];
+    }
+  }
+}
+
+}  // namespace sae
+
+namespace sae {
+
+// The same pass in persistent form, used for bf16 p, m, v.  A row is 6 bytes per parameter there, so a workgroup
+// per row keeps too few bytes in flight to fill the memory system while it waits for its index loads and gathers
+// (3.3 TB/s).  Here a workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ... in units of 256 U pieces, and
+// requests the next unit's p, m, v (as they lie in memory: 6 registers per piece) before it gathers and updates
+// the current one: 4.4 TB/s.  Arithmetic and summation order are those of the kernel above, so the dense route
+// over rounded gradient rows gives the same bits.  For fp32 state (S_BF16 = false compiles, and passes the same
+// tests) this form is slower than a workgroup per row, 2.86 against 2.51 ms at the headline shape, whatever the
+// grid: it is not dispatched.  Five waves per SIMD are asked for: at 98 registers (104 allocated) only four fit,
+// and the pass falls from 1.46 to 1.69 ms.
+template <bool DENSE_BF16, int U, bool S_BF16>
+__global__ __launch_bounds__(256, 5) void adam_sparse_rows_persistent_kernel(
+    const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
+    const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
+    float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int F, int d, AdamScalars a,
+    uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad,
+    const float *__restrict__ grad_scale, double *__restrict__ sq_nnz_partial,
+    const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows, const float *__restrict__ extra_bias) {
+  __shared__ float red[4];
+  __shared__ double red_d[8];
+  __shared__ float s_coef[256];
+  __shared__ int32_t s_tok[256];
+  const int tid = threadIdx.x;
+  const float gs = grad_scale ? grad_scale[0] : 1.f;
+  const int n_seg = d >> 2;
+  const int passes = (n_seg + 256 * U - 1) / (256 * U);
+  const size_t row_bytes = (size_t)d * (DENSE_BF16 ? 2 : 4);
+  const char *dbase = reinterpret_cast<const char *>(dense);
+  typedef typename std::conditional<S_BF16, nt_u32x2, nt_f32x4>::type raw_t;   // four elements as they lie in memory
+  struct Raw { raw_t p[U], m[U], v[U]; };
+  auto request = [&](Raw &r, int row, int pass) {
+    const int64_t base4 = (int64_t)row * n_seg;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int seg = pass * 256 * U + tid + u * 256;
+      if (seg < n_seg) {
+        r.p[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(p) + base4 + seg);
+        r.m[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(m) + base4 + seg);
+        r.v[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(v) + base4 + seg);
+      }
+    }
+  };
+  auto widen = [](const raw_t &t) {
+    if constexpr (S_BF16)
+      return make_float4(__uint_as_float(t[0] << 16), __uint_as_float(t[0] & 0xffff0000u), __uint_as_float(t[1] << 16),
+                         __uint_as_float(t[1] & 0xffff0000u));
+    else
+      return make_float4(t[0], t[1], t[2], t[3]);
+  };
+  Raw next;
+  if ((int)blockIdx.x < F) request(next, blockIdx.x, 0);
+  for (int f = blockIdx.x; f < F; f += gridDim.x) {
+    const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+    const int xo = extra_map ? extra_map[f] : -1;   // row of the dense gradient block that adds to this feature, or -1
+    const int64_t base4 = (int64_t)f * n_seg;
+    if (bias_grad && tid < 64) {
+      float s = 0.f;
+      for (int i = lo + tid; i < hi; i += 64) s += coef[feat_slot[i]];
+      s = wave_sum(s);
+      if (xo >= 0 && extra_bias) s += extra_bias[xo];
+      if (tid == 0) bias_grad[f] = grad_scale ? s * gs : s;
+    }
+    float sq = 0.f;
+    double g_sq = 0.0;
+    int g_nz = 0;
+    for (int pass = 0; pass < passes; ++pass) {
+      const Raw cur = next;
+      if (pass + 1 < passes) request(next, f, pass + 1);
+      else if (f + (int)gridDim.x < F) request(next, f + gridDim.x, 0);
+      const int seg0 = pass * 256 * U + tid;
+      float4 g[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int seg = seg0 + u * 256;
+        g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
+                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      gather_rows_staged<DENSE_BF16, 256, U>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg, s_coef, s_tok);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int seg = seg0 + u * 256;
+        if (seg < n_seg) {
+          if constexpr (S_BF16) {   // the gradient is a bf16 tensor before anything reads it
+            g[u].x = bf16_round(g[u].x); g[u].y = bf16_round(g[u].y); g[u].z = bf16_round(g[u].z); g[u].w = bf16_round(g[u].w);
+          }
+          if (grad_scale) {
+            g[u].x = mul_rn(g[u].x, gs); g[u].y = mul_rn(g[u].y, gs);
+            g[u].z = mul_rn(g[u].z, gs); g[u].w = mul_rn(g[u].w, gs);
+          }
+          if (sq_nnz_partial) {
+            float s4 = g[u].x * g[u].x;
+            s4 = fmaf(g[u].y, g[u].y, s4); s4 = fmaf(g[u].z, g[u].z, s4); s4 = fmaf(g[u].w, g[u].w, s4);
+            g_sq += (double)s4;
+            g_nz += (g[u].x != 0.f) + (g[u].y != 0.f) + (g[u].z != 0.f) + (g[u].w != 0.f);
+          }
+          float4 pp = widen(cur.p[u]), mm = widen(cur.m[u]), vv = widen(cur.v[u]);
+          adam_any4<S_BF16>(pp, g[u], mm, vv, a);
+          store_state4<S_BF16>(p, base4 + seg, pp);
+          store_state4<S_BF16>(m, base4 + seg, mm);
+          store_state4<S_BF16>(v, base4 + seg, vv);
+          if (!S_BF16 && shadow) {
+            uint2 o;
+            o.x = (uint32_t)f32_to_bf16_bits(pp.x) | ((uint32_t)f32_to_bf16_bits(pp.y) << 16);
+            o.y = (uint32_t)f32_to_bf16_bits(pp.z) | ((uint32_t)f32_to_bf16_bits(pp.w) << 16);
+            store_stream(shadow, base4 + seg, o);
+          }
+          sq = fmaf(pp.x, pp.x, sq); sq = fmaf(pp.y, pp.y, sq);
+          sq = fmaf(pp.z, pp.z, sq); sq = fmaf(pp.w, pp.w, sq);
+        }
+      }
+    }
+    if (row_norm) {
+      const float tot = block_sum<4>(sq, red);
+      if (tid == 0) row_norm[f] = sqrtf(tot);
+    }
+    if (sq_nnz_partial) {
+      double cnt = (double)g_nz;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) { g_sq += __shfl_xor(g_sq, o, 64); cnt += __shfl_xor(cnt, o, 64); }
+      const int lane = tid & 63, w = tid >> 6;
+      __syncthreads();   // red_d of the previous row has been read
+      if (lane == 0) { red_d[w] = g_sq; red_d[4 + w] = cnt; }
+      __syncthreads();
+      if (tid == 0) {
+        sq_nnz_partial[2 * (size_t)f] = red_d[0] + red_d[1] + red_d[2] + red_d[3];
+        sq_nnz_partial[2 * (size_t)f + 1] = red_d[4] + red_d[5] + red_d[6] + red_d[7];
+      }
     }
   }
 }
@@ -426,22 +557,34 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
   hipStream_t st = (hipStream_t)stream;
   double *partial = grad_sq_nnz_acc ? reinterpret_cast<double *>(workspace) : nullptr;
   {
-#define SAE_ADAM_ROWS(BF, UU, SB)                                                                                              \
-  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU, SB>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
-                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,                \
+#define SAE_ADAM_ROWS(BF, UU)                                                                                              \
+  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
+                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,            \
                      bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias)
     // pieces of 4 elements per thread: short rows keep fewer registers, so more rows are in flight per CU
     const int u = d <= 1024 ? 1 : (d <= 2048 ? 2 : 4);
     if (lowp) {
+      // persistent form: at most two pieces per thread and unit (95-102 registers: five workgroups per CU), and two
+      // rounds of resident workgroups -- a grid that is not a multiple of what is resident leaves a tail
+      // (1536 workgroups on 256 CUs: 1.84 ms against 1.47 ms with 1280 or 2560)
+      int dev = 0, cus = 256;
+      if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      const int64_t gmax = (int64_t)(cus > 0 ? cus : 256) * (d <= 1024 ? 14 : 10);   // 7 resident per CU at 66 registers
+      const unsigned grid = (unsigned)(F < gmax ? F : gmax);
+#define SAE_ADAM_ROWS_LOWP(BF, UU)                                                                                      \
+  hipLaunchKernelGGL((adam_sparse_rows_persistent_kernel<BF, UU, true>), dim3(grid), dim3(256), 0, st, feat_ptr, feat_slot, \
+                     slot_tok, coef, dense, p, m, v, (int)F, (int)d, a, nullptr, row_norm_out, bias_grad_out, grad_scale,  \
+                     partial, nullptr, nullptr, nullptr)
       if (dense_dtype == SAE_BF16) {
-        if (u == 1) SAE_ADAM_ROWS(true, 1, true); else if (u == 2) SAE_ADAM_ROWS(true, 2, true); else SAE_ADAM_ROWS(true, 4, true);
+        if (d <= 1024) SAE_ADAM_ROWS_LOWP(true, 1); else SAE_ADAM_ROWS_LOWP(true, 2);
       } else {
-        if (u == 1) SAE_ADAM_ROWS(false, 1, true); else if (u == 2) SAE_ADAM_ROWS(false, 2, true); else SAE_ADAM_ROWS(false, 4, true);
+        if (d <= 1024) SAE_ADAM_ROWS_LOWP(false, 1); else SAE_ADAM_ROWS_LOWP(false, 2);
       }
+#undef SAE_ADAM_ROWS_LOWP
     } else if (dense_dtype == SAE_BF16) {
-      if (u == 1) SAE_ADAM_ROWS(true, 1, false); else if (u == 2) SAE_ADAM_ROWS(true, 2, false); else SAE_ADAM_ROWS(true, 4, false);
+      if (u == 1) SAE_ADAM_ROWS(true, 1); else if (u == 2) SAE_ADAM_ROWS(true, 2); else SAE_ADAM_ROWS(true, 4);
     } else {
-      if (u == 1) SAE_ADAM_ROWS(false, 1, false); else if (u == 2) SAE_ADAM_ROWS(false, 2, false); else SAE_ADAM_ROWS(false, 4, false);
+      if (u == 1) SAE_ADAM_ROWS(false, 1); else if (u == 2) SAE_ADAM_ROWS(false, 2); else SAE_ADAM_ROWS(false, 4);
     }
 #undef SAE_ADAM_ROWS
   }
