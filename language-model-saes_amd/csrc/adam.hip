@@ -30,19 +30,6 @@ __device__ __forceinline__ float adam_one(float &p, float g, float &m, float &v,
 // division by sqrt(bias correction 2) and the quotient m / denominator use the single-instruction forms (1 ulp in
 // fp32), whose error disappears in the rounding to bf16 that follows each of them except on rare boundary cases:
 // with IEEE division and square root sequences the pass is bound by its arithmetic, not by memory.
-typedef __attribute__((ext_vector_type(2))) float adam_f32x2;
-typedef __attribute__((ext_vector_type(2))) __bf16 adam_bf16x2;
-__device__ __forceinline__ void bf16_round2(float &x, float &y) {
-  const adam_f32x2 in = {x, y};
-  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(in, adam_bf16x2));
-  x = __uint_as_float(packed << 16);
-  y = __uint_as_float(packed & 0xffff0000u);
-}
-__device__ __forceinline__ float bf16_round(float x) {
-  float y = x;
-  bf16_round2(x, y);
-  return x;
-}
 // two elements at a time; both lanes of a pair see exactly the scalar sequence
 __device__ __forceinline__ void adam_two_lowp(float &p0, float &p1, float g0, float g1, float &m0, float &m1, float &v0,
                                               float &v1, const AdamScalars &a) {

@@ -41,6 +41,21 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// Round-to-nearest-even to bf16 precision through the packed hardware conversion (two values per instruction).
+typedef __attribute__((ext_vector_type(2))) float cvt_f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 cvt_bf16x2;
+__device__ __forceinline__ void bf16_round2(float &x, float &y) {
+  const cvt_f32x2 in = {x, y};
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(in, cvt_bf16x2));
+  x = __uint_as_float(packed << 16);
+  y = __uint_as_float(packed & 0xffff0000u);
+}
+__device__ __forceinline__ float bf16_round(float x) {
+  float y = x;
+  bf16_round2(x, y);
+  return x;
+}
+
 // ---- single operations that stay single ----------------------------------------------------
 // The compiler may fuse a product with a following sum into one fused multiply-add (and HIP's __fmul_rn /
 // __fadd_rn are plain operators, so they do not prevent it).  Where a result has to have the bits of two

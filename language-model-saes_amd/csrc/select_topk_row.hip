@@ -45,7 +45,7 @@ struct SelShared {
 // LOWP: the arithmetic of a dictionary whose parameters are bf16 tensors -- the sum with the bias and the product
 // with the norm are each rounded to bf16, as the tensors `x @ W_E + b_E` and `hidden_pre * decoder_norm()` are
 // (models/sae.py:324-335 with cfg.dtype = bfloat16); the bias and scale arrive as fp32 copies of bf16 values.
-__device__ __forceinline__ float sel_bf16_round(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+__device__ __forceinline__ float sel_bf16_round(float x) { return bf16_round(x); }
 template <bool LOWP>
 __device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm, bool has_mask) {
   float h1;
