@@ -386,8 +386,8 @@ namespace sae {
 // requests the next unit's p, m, v (as they lie in memory: 6 registers per piece) before it gathers and updates
 // the current one: 4.4 TB/s.  Arithmetic and summation order are those of the kernel above, so the dense route
 // over rounded gradient rows gives the same bits.  For fp32 state (S_BF16 = false compiles, and passes the same
-// tests) this form is slower than a workgroup per row, 2.86 against 2.51 ms at the headline shape, whatever the
-// grid: it is not dispatched.  Five waves per SIMD are asked for: at 98 registers (104 allocated) only four fit,
+// tests) this form is slower than a workgroup per row, 2.86 against 2.51 ms at the headline shape and 6.3 against
+// 4.9 ms over a cross-layer transcoder's rows of 768, whatever the grid: it is not dispatched.  Five waves per SIMD are asked for: at 98 registers (104 allocated) only four fit,
 // and the pass falls from 1.46 to 1.69 ms.
 template <bool DENSE_BF16, int U, bool S_BF16>
 __global__ __launch_bounds__(256, 5) void adam_sparse_rows_persistent_kernel(
