@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # transfers of known size in the same runs: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this machine.
 HBM_TRAFFIC_GB = {
     "encoder_gemm": 7.61, "adam_step_sparse_rows[f32 dense]": 18.14, "adam_step_sparse_rows[bf16 dense]": 16.00,
-    "sparse_decode_mse_fused": 4.38, "select_topk_row": 1.50,
+    "sparse_decode_mse_fused": 4.38, "select_topk_row": 1.19,
 }
 
 

@@ -46,14 +46,17 @@ struct SelShared {
 // with the norm are each rounded to bf16, as the tensors `x @ W_E + b_E` and `hidden_pre * decoder_norm()` are
 // (models/sae.py:324-335 with cfg.dtype = bfloat16); the bias and scale arrive as fp32 copies of bf16 values.
 __device__ __forceinline__ float sel_bf16_round(float x) { return bf16_round(x); }
-template <bool LOWP>
-__device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm, bool has_mask) {
+// ARITH selects the arithmetic at compile time: the masked (aux-k) form costs registers that the plain form,
+// which runs every step, should not pay for (with one kernel for both, 14 registers per lane were spilled).
+constexpr int SEL_PLAIN = 0, SEL_LOWP = 1, SEL_MASKED = 2;
+template <int ARITH>
+__device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm) {
   float h1;
-  if constexpr (LOWP) {
+  if constexpr (ARITH == SEL_LOWP) {
     h1 = sel_bf16_round(mul_rn(sel_bf16_round(add_rn(pre, b)), s));
   } else {
     h1 = (pre + b) * s;
-    if (has_mask) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
+    if constexpr (ARITH == SEL_MASKED) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
   }
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
@@ -112,7 +115,7 @@ __device__ __forceinline__ void lds_kth_largest(SelShared *sh, int n, int k, Key
   }
 }
 
-template <bool BF16, bool LOWP = false>
+template <bool BF16, int ARITH = SEL_PLAIN>
 struct RowReader {
   const void *row;
   const float *b_enc;
@@ -141,7 +144,7 @@ struct RowReader {
     }
     const int base = c * V;
     float bb[V], ss[V], mm[V];
-    if (fmask) {
+    if constexpr (ARITH == SEL_MASKED) {
 #pragma unroll
       for (int q = 0; q < V / 4; ++q) {
         const float4 t = reinterpret_cast<const float4 *>(fmask + base)[q];
@@ -172,14 +175,14 @@ struct RowReader {
       for (int e = 0; e < V; ++e) ss[e] = 1.f;
     }
 #pragma unroll
-    for (int e = 0; e < V; ++e) keys[e] = key_of<LOWP>(pre[e], bb[e], ss[e], mm[e], fmask != nullptr);
+    for (int e = 0; e < V; ++e) keys[e] = key_of<ARITH>(pre[e], bb[e], ss[e], mm[e]);
   }
   // key of one element
   __device__ __forceinline__ uint32_t key_at(int i) const {
     float pre;
     if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
     else pre = reinterpret_cast<const float *>(row)[i];
-    return key_of<LOWP>(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, fmask ? fmask[i] : 1.f, fmask != nullptr);
+    return key_of<ARITH>(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, ARITH == SEL_MASKED ? fmask[i] : 1.f);
   }
   // calls fn(index, key) for every element of the row, vectorised when the row allows it
   template <typename Fn>
@@ -199,8 +202,8 @@ struct RowReader {
 };
 
 // Exact k-th largest over the whole row in global memory (general path).
-template <bool BF16, bool LOWP>
-__device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<BF16, LOWP> &rr, int k) {
+template <bool BF16, int ARITH>
+__device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<BF16, ARITH> &rr, int k) {
   if (threadIdx.x == 0) { sh->prefix = 0u; sh->remaining = k; }
   uint32_t mask = 0u;
 #pragma unroll 1
@@ -225,7 +228,7 @@ __device__ __forceinline__ void row_kth_largest(SelShared *sh, const RowReader<B
 // handful per row) are formed again from memory.
 constexpr int SEL_STASH_ELEMS = 128;  // per thread: rows up to 131072 elements
 
-template <bool BF16, bool STASH, bool LOWP = false>
+template <bool BF16, bool STASH, int ARITH = SEL_PLAIN>
 __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
@@ -234,7 +237,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   __shared__ SelShared sh;
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
-  RowReader<BF16, LOWP> rr;
+  RowReader<BF16, ARITH> rr;
   rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
   rr.scale = scale;
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   // ---- pass 1: per-thread maximum key and number of positive elements ----
   uint32_t my_max = 0u;
   int my_pos = 0;
-  constexpr int V = RowReader<BF16, LOWP>::V;
+  constexpr int V = RowReader<BF16, ARITH>::V;
   constexpr int NCH = SEL_STASH_ELEMS / V;            // chunks per thread when stashing
   uint32_t cmax[STASH ? NCH : 1];                     // largest key of each of this thread's chunks
   if constexpr (STASH) {
@@ -340,7 +343,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
   if (general) {
     // ---- general path: exact threshold over the whole row ----
     __syncthreads();
-    row_kth_largest<BF16, LOWP>(&sh, rr, k_eff);
+    row_kth_largest<BF16, ARITH>(&sh, rr, k_eff);
     T = sh.prefix;
     need = sh.remaining;  // elements equal to T that are kept
     __syncthreads();
@@ -429,7 +432,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const float s = scale ? scale[my_idx] : 1.f;
     if (rank < k) {
       idx_out[(size_t)b * k + rank] = my_idx;
-      val_out[(size_t)b * k + rank] = scale ? (LOWP ? sel_bf16_round(h1 / s) : h1 / s) : h1;
+      val_out[(size_t)b * k + rank] = scale ? (ARITH == SEL_LOWP ? sel_bf16_round(h1 / s) : h1 / s) : h1;
     }
   }
   for (int i = k_eff + tid; i < k; i += SEL_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
@@ -460,7 +463,13 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
   hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
                      scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap)
   if (lowp) {
-    if (stash) SAE_LAUNCH_SELECT(true, true, true); else SAE_LAUNCH_SELECT(true, false, true);
+    if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP);
+  } else if (feat_mask) {
+    if (pre_dtype == SAE_BF16) {
+      if (stash) SAE_LAUNCH_SELECT(true, true, SEL_MASKED); else SAE_LAUNCH_SELECT(true, false, SEL_MASKED);
+    } else {
+      if (stash) SAE_LAUNCH_SELECT(false, true, SEL_MASKED); else SAE_LAUNCH_SELECT(false, false, SEL_MASKED);
+    }
   } else if (pre_dtype == SAE_BF16) {
     if (stash) SAE_LAUNCH_SELECT(true, true); else SAE_LAUNCH_SELECT(true, false);
   } else {
