@@ -551,6 +551,7 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
     // pieces of 4 elements per thread: short rows keep fewer registers, so more rows are in flight per CU
     const int u = d <= 1024 ? 1 : (d <= 2048 ? 2 : 4);
     if (lowp) {
+      SAE_REQUIRE(F < (1LL << 31) - (1 << 20), SAE_ERR_UNSUPPORTED, "adam_step_sparse_rows_lowp: F too large");
       // persistent form: at most two pieces per thread and unit (95-102 registers: five workgroups per CU), and two
       // rounds of resident workgroups -- a grid that is not a multiple of what is resident leaves a tail
       // (1536 workgroups on 256 CUs: 1.84 ms against 1.47 ms with 1280 or 2560)
