@@ -194,6 +194,41 @@ def test_bf16_parameters_step_with_adam_follows_torch_adam(pkg, oracle, dev):
         assert ((got - want).abs() > 0.5 * moved).float().mean().item() < 2e-2, name
 
 
+@pytest.mark.parametrize("clip", [0.0, 0.02])
+def test_bf16_parameters_through_the_trainer_shell(pkg, oracle, dev, clip):
+    """`Trainer.train_one_step` on a bf16 dictionary: gradient norm every step (and clipping), metrics on; the loss
+    goes down and everything stays bf16 and finite.  Factored and dense weight gradients agree on the norm to bf16
+    tolerance (the factored one is summed over unrounded rows) and, without clipping, end at the same parameters."""
+    d, F, k, B, steps = 256, 2048, 16, 192, 5
+    runs = []
+    for defer in (True, False):
+        sae, _, batch = make_pair(pkg, oracle, dev, d=d, F=F, k=k, B=B, r=8, seed=9, include_norm=True, dtype=torch.bfloat16)
+        gb = {kk: v.to(dev) for kk, v in batch.items()}
+        gb["mask"] = torch.ones(B, device=dev)
+        tcfg = pkg.TrainerConfig(lr=2e-3, lr_warm_up_steps=1, lr_cool_down_steps=1, total_training_tokens=B * steps,
+                                 amp_dtype=torch.bfloat16, skip_metrics_calculation=False, log_frequency=1,
+                                 clip_grad_norm=clip, k_warmup_steps=0, l1_coefficient_warmup_steps=2)
+        trainer = pkg.Trainer(tcfg)
+        trainer.prepare(sae, gb)
+        if not defer:
+            sae.defer_weight_grads = False
+        losses, norms = [], []
+        for _ in range(steps):
+            out = trainer.train_one_step(sae, gb)
+            losses.append(float(out["loss"].detach()))
+            norms.append(float(out["grad_norm_before_clipping"]))
+        for n, p in sae.named_parameters():
+            assert p.dtype == torch.bfloat16 and torch.isfinite(p).all(), n
+        assert losses[-1] < losses[0]
+        runs.append(({n: p.detach().clone() for n, p in sae.named_parameters()}, losses, norms))
+    (pa, la, na), (pb, lb, nb) = runs
+    assert abs(na[0] - nb[0]) / nb[0] < BF16_TOL
+    if clip == 0.0:
+        assert la == lb
+        for n in pa:
+            assert torch.equal(pa[n], pb[n]), n
+
+
 def test_fused_step_unsubstituted_agrees_statistically(pkg, oracle, dev):
     """No substitution: the two GEMMs round differently, so a few near-tie selections may flip."""
     sae, ref, batch = make_pair(pkg, oracle, dev, d=256, F=2048, k=16, B=192, r=8, seed=2, include_norm=True)
