@@ -325,7 +325,11 @@ class _FusedSparseStep(torch.autograd.Function):
         g = g_loss.to(torch.float32)
         coef_dec = code.val * g          # dW_D[f] = sum val * grad_recon[token]
         coef_enc = ctx.grad_coef_E * g   # dW_E^T[f] = sum d(pre) * x[token]; kept entries are positive, so d(pre) = d val
-        db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
+        db_D = None
+        if ctx.has_b_D:
+            # a bf16 dictionary's reconstruction is a bf16 tensor, so the gradient summed for b_D is the bf16-rounded one
+            gr = ctx.grad_recon if ctx.param_dtype == torch.float32 else ctx.grad_dense_D.float()
+            db_D = ops.col_sum(gr) * g
         extra_D = extra_E = None
         ad = ctx.aux_dense
         if ad is not None:   # the dead block's rows, held densely
