@@ -119,6 +119,63 @@ def build_topk(pkg, dev, args):
     return _autocast_step(sae, batch, opt, {}), B, name, (B, d, F, k)
 
 
+C1 = dict(d=768, F=6144, k=32, B=4096, r=16, seed=0)   # the reference's CPU-runnable configuration: fp32, MSE only
+
+
+def build_c1_fp32(pkg, dev, args):
+    """TopK SAE d=768 -> 6144, k=32, B=4096 in fp32 (no autocast), Adam lr 4e-4: the configuration the CPU path runs
+    at full shape, so `cpu_baseline` of this workload is the oracle on exactly the same step."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = C1["B"], C1["d"], C1["F"], C1["k"]
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
+                        dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    x = synthetic.activations(B, d, C1["r"], seed=C1["seed"]).to(dev)
+    _init_sae_on_device(sae, x, d, seed=C1["seed"])
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae)
+
+    def step():
+        loss = sae.compute_loss(batch, return_aux_data=False)
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        return loss
+    return step, B, f"topk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} fp32 adam", (B, d, F, k)
+
+
+def cpu_baseline_c1():
+    """The oracle on the full C1 step (same shape, fp32, same optimizer), all host threads."""
+    import torch
+    from __graft_entry__ import load_oracle, load_package
+
+    oracle = load_oracle()
+    load_package()
+    from lm_saes_amd import synthetic
+
+    B, d, F, k = C1["B"], C1["d"], C1["F"], C1["k"]
+    m = oracle.SAEOracle(d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=True)
+    with torch.no_grad():
+        m.W_E.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5)
+        m.W_D.copy_(m.W_E.t())
+        m.W_D.div_(m.W_D.norm(dim=1, keepdim=True))
+    x = synthetic.activations(B, d, C1["r"], seed=C1["seed"])
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long)}
+    opt = oracle.make_adam(m, lr=4e-4)
+    oracle.train_step(m, opt, batch)
+    n_timed, t0 = 0, time.perf_counter()
+    while n_timed < 3 or (time.perf_counter() - t0 < 12.0 and n_timed < 20):
+        oracle.train_step(m, opt, batch)
+        n_timed += 1
+    dt = (time.perf_counter() - t0) / n_timed
+    return {"value": round(B / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 warm-up + {n_timed} timed steps of the full step (d_model={d} d_sae={F} k={k} B={B}, fp32) on CPU, "
+                      f"torch {torch.__version__}, {dt:.2f} s per step"}
+
+
 def build_topk_bf16_params(pkg, dev, args):
     """The headline shape with the dictionary itself held in bf16 (cfg.dtype = bfloat16: bf16 parameters,
     gradients and Adam moments, as the reference trains with that dtype).  A secondary figure: the reference's
@@ -288,7 +345,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
@@ -459,6 +516,9 @@ def main():
     }
     if headline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, args.cpu_sample_features)
+    if args.workload == "c1_fp32" and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_c1()
+        out["dtype"] = "f32"
     print(json.dumps(out))
 
 
