@@ -73,6 +73,15 @@ int64_t sae_col_sum_workspace_bytes(int64_t B, int64_t n);
 int sae_col_sum(const float *src, float *out, int64_t B, int64_t n, int accumulate, void *workspace,
                 int64_t workspace_bytes, void *stream);
 
+/* sae_col_sum for callers that cannot allocate a workspace (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The partial sums live in a fixed
+ * 4 MiB device array inside the library (one copy per GPU, held until the process ends), so the call allocates
+ * nothing; n is limited to SAE_COL_SUM_STATIC_MAX_N columns (larger n: SAE_ERR_UNSUPPORTED; use sae_col_sum).
+ * Same kernels and order of additions as sae_col_sum: identical bits.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (different streams) race; calls on one stream are ordered and safe. */
+#define SAE_COL_SUM_STATIC_MAX_N 16384
+int sae_col_sum_static(const float *src, float *out, int64_t B, int64_t n, int accumulate, void *stream);
+
 /* ---- encoder ---------------------------------------------------------------------- */
 
 /* pre[b, f] = sum_j x[b, j] * w_enc_t[f, j]          (no bias: the select kernels add it)

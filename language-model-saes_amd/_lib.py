@@ -26,6 +26,7 @@ SIGNATURES = {
     "sae_transpose_f32": (_I, [_P, _P, _L, _L, _P]),
     "sae_col_sum_workspace_bytes": (_L, [_L, _L]),
     "sae_col_sum": (_I, [_P, _P, _L, _L, _I, _P, _L, _P]),
+    "sae_col_sum_static": (_I, [_P, _P, _L, _L, _I, _P]),
     "sae_encoder_gemm": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "sae_select_topk_row": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_lowp": (_I, [_P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),

@@ -2,6 +2,8 @@
 // All are HBM-bound single passes with 16-byte accesses where the shape allows.
 #include "common.h"
 
+#include <mutex>
+
 namespace sae {
 
 __global__ void zero_fill_kernel(uint32_t *p, size_t n_words) {
@@ -460,4 +462,54 @@ extern "C" int sae_col_sum(const float *src, float *out, int64_t B, int64_t n, i
   hipLaunchKernelGGL(col_sum_partial_kernel, dim3(gx, (unsigned)chunks), dim3(256), 0, (hipStream_t)stream, src, part, B, n, rows_per);
   hipLaunchKernelGGL(col_sum_final_kernel, dim3(gx), dim3(256), 0, (hipStream_t)stream, part, out, n, chunks, accumulate);
   return check_launch("col_sum");
+}
+
+// ---- column sums with the partial sums in a fixed device array --------------------------------------
+// The partial sums of sae_col_sum live in caller-supplied workspace.  Callers that cannot allocate one
+// (code under graph capture, serving loops) use this array instead: 64 chunks x SAE_COL_SUM_STATIC_MAX_N
+// floats = 4 MiB, held by every device the library runs on until the process ends.
+static __device__ __align__(256) float scratch[64 * SAE_COL_SUM_STATIC_MAX_N];
+
+namespace {
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices] = {nullptr};   // device address of `scratch`, one per device
+std::mutex g_scratch_mutex;
+
+// Device address of this device's copy of `scratch` (the array's name is a host-side handle, not an address).
+int scratch_address(float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return sae::fail(SAE_ERR_LAUNCH, "col_sum_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return sae::fail(SAE_ERR_UNSUPPORTED, "col_sum_static: device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float *ptr = nullptr;
+    e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return sae::fail(SAE_ERR_LAUNCH, "col_sum_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return SAE_OK;
+}
+}  // namespace
+
+extern "C" int sae_col_sum_static(const float *src, float *out, int64_t B, int64_t n, int accumulate, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(src && out, SAE_ERR_INVALID_ARG, "col_sum_static: null pointer");
+  SAE_REQUIRE(B > 0 && n > 0, SAE_ERR_INVALID_ARG, "col_sum_static: bad shape");
+  SAE_REQUIRE(n <= SAE_COL_SUM_STATIC_MAX_N, SAE_ERR_UNSUPPORTED,
+              "col_sum_static: n = %lld exceeds the fixed scratch array's %d columns; use sae_col_sum with a workspace",
+              (long long)n, (int)SAE_COL_SUM_STATIC_MAX_N);
+  float *part = nullptr;
+  const int rc = scratch_address(&part);
+  if (rc != SAE_OK) return rc;
+  // Same grid, chunking and order of additions as sae_col_sum, so the bits are the same.  Every partial the
+  // second kernel reads (chunks x n) is written by the first, so nothing left by an earlier call is seen.
+  const int chunks = (int)(B < 64 ? B : 64);
+  const int rows_per = (int)((B + chunks - 1) / chunks);
+  const unsigned gx = (unsigned)((n + 255) / 256);
+  hipLaunchKernelGGL(col_sum_partial_kernel, dim3(gx, (unsigned)chunks), dim3(256), 0, (hipStream_t)stream, src, part, B, n, rows_per);
+  hipLaunchKernelGGL(col_sum_final_kernel, dim3(gx), dim3(256), 0, (hipStream_t)stream, part, out, n, chunks, accumulate);
+  return check_launch("col_sum_static");
 }
