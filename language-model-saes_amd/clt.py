@@ -323,16 +323,26 @@ class CrossLayerTranscoder(SparseDictionary):
 
     @torch.no_grad()
     def standardize_parameters_of_dataset_norm(self):
-        """clt.py:908-937: fold the per-layer dataset norms into the weights."""
+        """clt.py:908-937: fold the per-layer dataset norms into the parameters so that raw activations can be fed.
+        With fin(l) = sqrt(d) / norm_in(l) and fout(l) = sqrt(d) / norm_out(l): the encoder weights stay, the encoder
+        bias (and a JumpReLU threshold) of layer l is divided by fin(l) (features come out in raw-input units),
+        W_D[layer_to][layer_from] is multiplied by fin(layer_from) / fout(layer_to) and b_D[layer_to] is divided by
+        fout(layer_to).  In-place operations on the parameters themselves (not on `.data`), so the version counters
+        move and cached bf16 copies / norms are rebuilt on their next use."""
         assert self.cfg.norm_activation == "dataset-wise"
         assert self.dataset_average_activation_norm is not None
-        fin = lambda l: math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_points_in[l]]    # noqa: E731
-        fout = lambda l: math.sqrt(self.cfg.d_model) / self.dataset_average_activation_norm[self.cfg.hook_points_out[l]]  # noqa: E731
-        for l in range(self.cfg.n_layers):
-            self.W_E.data[l].mul_(fin(l))
+        norms = self.dataset_average_activation_norm
+        fin = lambda l: math.sqrt(self.cfg.d_model) / norms[self.cfg.hook_points_in[l]]    # noqa: E731
+        fout = lambda l: math.sqrt(self.cfg.d_model) / norms[self.cfg.hook_points_out[l]]  # noqa: E731
+        for layer_from in range(self.cfg.n_layers):
+            self.b_E[layer_from].div_(fin(layer_from))
+            if self.cfg.act_fn.lower() == "jumprelu":
+                log_thr = self.activation_function.log_jumprelu_threshold
+                log_thr[layer_from] = torch.log(log_thr[layer_from].exp() / fin(layer_from))
         for layer_to in range(self.cfg.n_layers):
-            self.W_D[layer_to].div_(fout(layer_to))
             self.b_D[layer_to].div_(fout(layer_to))
+            for layer_from in range(layer_to + 1):
+                self.W_D[layer_to][layer_from].mul_(fin(layer_from) / fout(layer_to))
         self.cfg.norm_activation = "inference"
 
     # ---- API path over dense tensors (clt.py:527-709) ----

@@ -154,6 +154,52 @@ def test_clt_dense_loss_matches_oracle(pkg, vo, act_fn, loss_type):
         assert torch.allclose(p.grad, rp[n].grad, rtol=1e-4, atol=1e-6), n
 
 
+@pytest.mark.parametrize("act_fn", ["relu", "jumprelu"])
+def test_clt_standardize_folds_dataset_norms_as_the_reference_does(pkg, vo, act_fn):
+    """clt.py:908-937.  Closed form per parameter (W_E untouched; b_E[l] and the threshold / fin(l);
+    W_D[to][from] * fin(from) / fout(to); b_D[to] / fout(to)) and the property the fold exists for: the folded
+    model on raw activations gives the normalised model's features / fin(l) and reconstruction / fout(l)."""
+    import math
+    # without the decoder-norm scale around the activation: a threshold on h * norm is not invariant under the
+    # fold (the norms change with W_D), in the reference either
+    m, _, hin, hout = make_clt(pkg, vo, act_fn, sparsity_include_decoder_norm=False)
+    L, d = 3, 4
+    if act_fn == "jumprelu":
+        with torch.no_grad():
+            m.activation_function.log_jumprelu_threshold.copy_(torch.linspace(-2.0, -0.5, 24).view(3, 8))
+    norms = {**{h: 1.5 + 0.5 * l for l, h in enumerate(hin)}, **{h: 0.7 + 0.3 * l for l, h in enumerate(hout)}}
+    fin = [math.sqrt(d) / norms[h] for h in hin]
+    fout = [math.sqrt(d) / norms[h] for h in hout]
+    m.cfg.norm_activation = "dataset-wise"
+    m.set_dataset_average_activation_norm(norms)
+    raw = torch.randn(7, L, d, generator=torch.Generator().manual_seed(5))
+    x_n = raw * torch.tensor(fin).view(1, L, 1)
+    with torch.no_grad():
+        acts_n = m.encode(x_n)
+        rec_n = m.decode(acts_n, batch_first=True)
+    before = {n: p.detach().clone() for n, p in m.named_parameters()}
+    versions = {n: p._version for n, p in m.named_parameters()}
+    m.standardize_parameters_of_dataset_norm()
+    assert m.cfg.norm_activation == "inference"
+    after = dict(m.named_parameters())
+    assert torch.equal(after["W_E"], before["W_E"])
+    for l in range(L):
+        assert torch.allclose(after["b_E"][l], before["b_E"][l] / fin[l])
+        assert torch.allclose(after[f"b_D.{l}"], before[f"b_D.{l}"] / fout[l])
+        for lf in range(l + 1):
+            assert torch.allclose(after[f"W_D.{l}"][lf], before[f"W_D.{l}"][lf] * (fin[lf] / fout[l]))
+        if act_fn == "jumprelu":
+            n = "activation_function.log_jumprelu_threshold"
+            assert torch.allclose(after[n][l].exp(), before[n][l].exp() / fin[l])
+    # every touched parameter's version moved, so cached bf16 copies and norms are rebuilt
+    assert all(after[n]._version > versions[n] for n in after if n != "W_E")
+    with torch.no_grad():
+        acts = m.encode(raw)
+        rec = m.decode(acts, batch_first=True)
+    assert torch.allclose(acts, acts_n / torch.tensor(fin).view(1, L, 1), rtol=1e-5, atol=1e-7)
+    assert torch.allclose(rec, rec_n / torch.tensor(fout).view(1, L, 1), rtol=1e-5, atol=1e-6)
+
+
 # ---- Lorsa ---------------------------------------------------------------------------------------
 
 def make_lorsa(pkg, vo, act_fn="relu", **kw):
