@@ -213,12 +213,23 @@ class CachedActivationLoader:
             for k, v in chunk.items():
                 if isinstance(v, torch.Tensor):
                     staged[k] = v.to(self.device, non_blocking=True)
-                    staged[k].record_stream(torch.cuda.current_stream(self.device))
                 else:
                     staged[k] = v
             done = torch.cuda.Event()
             done.record(stream)
         return staged, (done, chunk)   # the pinned source stays referenced until the copy has been waited for
+
+    @staticmethod
+    def _hand_over(staged: dict[str, Any], done, consumer) -> dict[str, Any]:
+        """Give a staged chunk to the stream that will read it.  The tensors were allocated on the copy stream, so
+        the caching allocator would reuse their blocks for a later host-to-device copy as soon as the consumer drops
+        them, while kernels queued on the consumer stream may still be reading: `record_stream(consumer)` defers that
+        reuse until the consumer's queued work has passed."""
+        consumer.wait_event(done)
+        for v in staged.values():
+            if isinstance(v, torch.Tensor):
+                v.record_stream(consumer)
+        return staged
 
     def process(self, data: None = None, **kwargs) -> Iterator[dict[str, Any]]:
         hook_chunks = {hp: self._get_sorted_chunks(hp) for hp in self.cache_dirs}
@@ -257,8 +268,7 @@ class CachedActivationLoader:
                 nxt = self._to_device(payload, copy_stream) if kind == "chunk" else None
                 if pending is not None:
                     staged, (done, _host) = pending
-                    torch.cuda.current_stream(self.device).wait_event(done)
-                    yield staged
+                    yield self._hand_over(staged, done, torch.cuda.current_stream(self.device))
                 pending = nxt
                 if kind == "end":
                     break

@@ -668,9 +668,14 @@ class SparseAutoEncoder(SparseDictionary):
 
     # ---- fused train-step loss ----
     def _fused_eligible(self, x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
+        amp = _autocast_dtype("cuda") == torch.bfloat16 or self.W_E.dtype == torch.bfloat16
+        # what the kernels are built for: the GEMM's K granule, 16-byte decoder rows, and the feature index's token
+        # limit (the sparse aux-k route stacks a second code onto the token axis); other shapes take the dense route
+        shapes_fit = (self.cfg.d_model % (64 if amp else 32) == 0
+                      and x.shape[0] * (2 if auxk_coefficient > 0.0 else 1) <= 131072)
         return (
             self.cfg.act_fn.lower() in ("topk", "batchtopk")
-            and x.is_cuda and x.ndim == 2 and label.ndim == 2
+            and x.is_cuda and x.ndim == 2 and label.ndim == 2 and shapes_fit
             and not self.cfg.use_glu_encoder
             and sparsity_loss_type is None and not (lp_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)

@@ -75,6 +75,24 @@ def get_scheduler(scheduler_name: Optional[str], optimizer, **kwargs):
             optimizer,
             lr_lambda=lambda steps: min(1.0, (steps + 1) / warm, end + (1 - end) / cool * max(total - steps, 1)),
         )
+    if name == "constantwithwarmupsmooth":
+        # two-piece warm-up (a line up to gamma * warm, then a parabola that lands flat on 1 at warm), a plateau,
+        # and a cosine decay to 0 over the last 1.5 * warm steps; gamma = 0.5
+        gamma = 0.5
+        cool_from = total - int(1.5 * warm)
+
+        def smooth(steps):
+            if steps < gamma * warm:
+                return 2 * (steps + 1) / (warm * (1 + gamma))
+            if steps < warm:
+                return 1 - ((steps / warm - 1) ** 2) / (1 - gamma ** 2)
+            if steps < cool_from:
+                return 1.0
+            return 0.5 * (1 + math.cos(math.pi * (steps - cool_from) / (total - cool_from)))
+        return lr_scheduler.LambdaLR(optimizer, smooth)
+    if name == "cosineannealingwarmrestarts":
+        return lr_scheduler.CosineAnnealingWarmRestarts(optimizer, T_0=total // kwargs.get("num_cycles", 1),
+                                                        eta_min=kwargs.get("lr_end", 0))
     if name == "linearwarmupdecay":
         return lr_scheduler.LambdaLR(
             optimizer, lambda steps: (steps + 1) / warm if steps < warm else (total - steps) / (total - warm))

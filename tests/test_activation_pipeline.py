@@ -207,3 +207,25 @@ def test_cached_activation_stream_end_to_end_on_cpu(pkg, tmp_path):
     got = torch.cat([b["in"] for b in batches])
     assert torch.equal(got, kept) and all(b["in"].shape[0] == 10 for b in batches[:-1])
     assert torch.equal(torch.cat([b["tokens"] for b in batches]), torch.cat([t[m.bool()] for t, m, _ in want]))
+
+
+def test_staged_chunk_is_tied_to_the_consumer_stream(pkg):
+    """A chunk copied on the side stream is handed over by waiting for the copy on the consumer's stream and by
+    recording that stream on every tensor, so the allocator cannot recycle the blocks under queued readers."""
+    calls = []
+
+    class FakeStream:
+        def wait_event(self, ev):
+            calls.append(("wait", ev))
+
+    class FakeTensor(torch.Tensor):
+        def record_stream(self, stream):
+            calls.append(("record", stream))
+
+    consumer, done = FakeStream(), object()
+    staged = {"a": torch.zeros(2).as_subclass(FakeTensor), "tokens": torch.zeros(2, dtype=torch.long).as_subclass(FakeTensor),
+              "meta": [{"x": 1}]}
+    out = pkg.activation.CachedActivationLoader._hand_over(staged, done, consumer)
+    assert out is staged
+    assert calls[0] == ("wait", done)
+    assert [c for c in calls[1:]] == [("record", consumer), ("record", consumer)]

@@ -185,6 +185,12 @@ def test_lr_schedules_hand_values(pkg):
     assert got[0] == 1.0 and abs(got[3] - 0.5 * (1 + math.cos(math.pi * 2 / 4))) < 1e-12
     got = lrs("exponentialwarmup", 4, warm_up_steps=1, training_steps=4, lr_end=1 / 8)
     assert abs(got[2] - (1 / 8) ** (1 / 3)) < 1e-12
+    # smooth warm-up (optim.py:35-51, 95-102): line to gamma * warm, parabola to 1 at warm, plateau, cosine over the last 1.5 warm
+    got = lrs("constantwithwarmupsmooth", 20, warm_up_steps=4, training_steps=20)
+    want = [1 / 3, 2 / 3, 2 / 3, 1 - 0.0625 / 0.75] + [1.0] * 11 + [0.5 * (1 + math.cos(math.pi * k / 6)) for k in range(1, 6)]
+    assert all(abs(a - b) < 1e-12 for a, b in zip(got, want)), got
+    got = lrs("cosineannealingwarmrestarts", 9, training_steps=8, num_cycles=2, lr_end=0.0)
+    assert abs(got[0] - 1.0) < 1e-12 and abs(got[2] - 0.5) < 1e-12 and abs(got[4] - 1.0) < 1e-12 and abs(got[6] - 0.5) < 1e-12
     with pytest.raises(ValueError):
         pkg.get_scheduler("nope", torch.optim.SGD([p], lr=1.0), training_steps=3)
 
