@@ -60,6 +60,28 @@ def _pieces(sg):
     return sg.pieces if hasattr(sg, "pieces") else [(0, sg)]
 
 
+def _relayout_loaded_state(opt: Optimizer, step_on_device: bool) -> None:
+    """After Optimizer.load_state_dict: give `exp_avg` / `exp_avg_sq` the strides, dtype and device of their
+    parameter (a checkpoint holds them contiguous in the logical shape; a feature-major W_E is not), and put the
+    step counter where the optimiser keeps it (a host scalar for HipAdam, a device float[1] for HipSparseAdam)."""
+    for group in opt.param_groups:
+        for prm in group["params"]:
+            st = opt.state.get(prm)
+            if not st:
+                continue
+            for k in ("exp_avg", "exp_avg_sq"):
+                t = st[k]
+                if tuple(t.shape) != tuple(prm.shape):
+                    raise ValueError(f"optimizer state {k} has shape {tuple(t.shape)}, parameter {tuple(prm.shape)}")
+                if t.stride() != prm.stride() or t.dtype != prm.dtype or t.device != prm.device:
+                    laid = torch.empty_like(prm, memory_format=torch.preserve_format)
+                    laid.copy_(t)
+                    st[k] = laid
+            step = st.get("step", 0)
+            step = step.detach().float() if torch.is_tensor(step) else torch.tensor(float(step), dtype=torch.float32)
+            st["step"] = step.reshape(1).to(prm.device) if step_on_device else step.reshape(()).cpu()
+
+
 class HipAdam(Optimizer):
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, model=None,
                  defer_weight_grads: bool = True, overlap_decoder_update: bool = False):
@@ -138,6 +160,23 @@ class HipAdam(Optimizer):
             st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
             st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
         return st
+
+    # ---- checkpoint interchange with torch.optim.Adam (trainer.py:198-209, 272-278) ----
+    def state_dict(self):
+        """torch.optim.Adam's layout: `step`, `exp_avg`, `exp_avg_sq` per parameter index, the two moments as
+        contiguous tensors of the parameter's logical shape (a feature-major W_E's moments leave as [d, F])."""
+        sd = super().state_dict()
+        for st in sd["state"].values():
+            for k in ("exp_avg", "exp_avg_sq"):
+                if k in st and not st[k].is_contiguous():
+                    st[k] = st[k].contiguous()
+        return sd
+
+    def load_state_dict(self, state_dict):
+        """Accepts a torch.optim.Adam state dict (or this class's own): the moments are brought to each parameter's
+        memory layout, which the update kernels address as one flat array together with the parameter."""
+        super().load_state_dict(state_dict)
+        _relayout_loaded_state(self, step_on_device=False)
 
     def _by_products(self, p, pv):
         """(role, bf16 shadow buffer or None, row-norm buffer or None) for the two weight matrices."""
@@ -336,6 +375,18 @@ class HipSparseAdam(Optimizer):
             raise NotImplementedError("weight decay is not part of the kernel (the reference's trainer never sets it)")
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
         self._model = model
+
+    def state_dict(self):
+        sd = super().state_dict()
+        for st in sd["state"].values():
+            for k in ("exp_avg", "exp_avg_sq"):
+                if k in st and not st[k].is_contiguous():
+                    st[k] = st[k].contiguous()
+        return sd
+
+    def load_state_dict(self, state_dict):
+        super().load_state_dict(state_dict)
+        _relayout_loaded_state(self, step_on_device=True)
 
     @torch.no_grad()
     def step(self, closure=None):

@@ -3,14 +3,17 @@
 The parts of the reference's `Trainer` (src/llamascopium/trainer.py) that sit on the hot loop:
 the k-annealing schedule and l1 warm-up of `_training_step` (:457-510), the dead-latent statistics
 behind the aux-k loss (:403-454), optimizer / LR-schedule construction (:349-401, optim.py:23-139)
-and the loop body of `fit` (:605-665).  Logging sinks, wandb, checkpoint files and the progress bar
-are not part of this path; `fit` reports through an optional callback instead, and never forces a
+the loop body of `fit` (:605-665) and complete checkpoints with resuming (:155-307).  Logging sinks, wandb and the
+progress bar are not part of this path; `fit` reports through an optional callback instead, and never forces a
 device synchronisation on its own (the reference syncs every step for its progress bar).
 """
 
 from __future__ import annotations
 
+import json
 import math
+import os
+from pathlib import Path
 from typing import Callable, Iterable, Literal, Optional, Tuple
 
 import torch
@@ -49,8 +52,9 @@ class TrainerConfig(BaseModel):
     # "adam" / "sparseadam" as in the reference; both map to the HIP kernels
     optimizer_class: Literal["adam", "sparseadam"] = "adam"
     optimizer_foreach: bool = True
-    lr_scheduler_name: Literal["constant", "constantwithwarmup", "linearwarmupdecay", "cosineannealing",
-                               "cosineannealingwarmup", "exponentialwarmup"] = "constantwithwarmup"
+    lr_scheduler_name: Literal["constant", "constantwithwarmup", "constantwithwarmupsmooth", "linearwarmupdecay",
+                               "cosineannealing", "cosineannealingwarmup", "cosineannealingwarmrestarts",
+                               "exponentialwarmup"] = "constantwithwarmup"
     lr_end_ratio: float = 1 / 32
     lr_warm_up_steps: int | float = 5000
     lr_cool_down_steps: int | float = 0.2
@@ -58,6 +62,17 @@ class TrainerConfig(BaseModel):
     clip_grad_norm: float = 0.0
     total_training_tokens: int = 300_000_000
     log_frequency: int = 1000
+    # checkpoints (trainer.py:107-124): model weights at `n_checkpoints` thresholds under exp_result_path/checkpoints;
+    # a directory written by `Trainer.save_checkpoint` is resumed from with `from_pretrained_path`
+    n_checkpoints: int = 0
+    check_point_save_mode: Literal["log", "linear"] = "log"
+    from_pretrained_path: Optional[str] = None
+    exp_result_path: str = "results"
+
+    def model_post_init(self, __context):
+        assert self.lr_end_ratio <= 1, "lr_end_ratio must be in 0 to 1 (inclusive)."
+        if self.from_pretrained_path is not None:
+            assert os.path.exists(self.from_pretrained_path), f"from_pretrained_path {self.from_pretrained_path} does not exist"
 
 
 def get_scheduler(scheduler_name: Optional[str], optimizer, **kwargs):
@@ -116,6 +131,7 @@ def get_scheduler(scheduler_name: Optional[str], optimizer, **kwargs):
 class Trainer:
     def __init__(self, cfg: TrainerConfig):
         self.cfg = cfg
+        self.checkpoint_thresholds: list[int] = []
         self.cur_step = 0
         self.cur_tokens = 0
         self.total_training_steps = 0
@@ -146,6 +162,71 @@ class Trainer:
         self.k_warmup_steps = steps(self.cfg.k_warmup_steps)
         self.k_cold_booting_steps = steps(self.cfg.k_cold_booting_steps)
         self.l1_coefficient_warmup_steps = steps(self.cfg.l1_coefficient_warmup_steps)
+        if self.cfg.n_checkpoints > 0:
+            n, total = self.cfg.n_checkpoints, self.total_training_steps
+            if self.cfg.check_point_save_mode == "linear":
+                self.checkpoint_thresholds = list(range(0, total, total // n))[1:]
+            else:   # "log": the reference multiplies these step counts by the batch size (trainer.py:339-343) and
+                # compares them with the step counter; kept as it is
+                self.checkpoint_thresholds = [math.ceil(2 ** (i / n * math.log2(total))) * bs for i in range(1, n)]
+
+    # ---- trainer.py:155-307: a complete checkpoint (model, optimizer, scheduler, trainer state) and resuming ----
+    _STATE_KEYS = ("cur_step", "cur_tokens", "total_training_steps", "lr_warm_up_steps", "lr_cool_down_steps",
+                   "k_warmup_steps", "k_cold_booting_steps", "l1_coefficient_warmup_steps", "checkpoint_thresholds")
+
+    def save_checkpoint(self, sae: SparseDictionary, checkpoint_path) -> Path:
+        """Writes <checkpoint_path>/checkpoints/step_<cur_step>/ with the reference's file set: the model's
+        hyper-parameters and `sae_weights.safetensors`, `trainer.pt`, `optimizer.pt`, `scheduler.pt`.  `trainer.pt`
+        holds the trainer's counters and its config as a plain dict (the reference pickles the config object, which
+        only its own package can read back); the optimizer file is a torch.optim.Adam state dict.  Returns the
+        directory."""
+        ckpt = Path(checkpoint_path) / "checkpoints" / f"step_{self.cur_step}"
+        os.makedirs(ckpt, exist_ok=True)
+        if self.optimizer is not None and hasattr(self.optimizer, "join"):
+            self.optimizer.join()
+        sae.cfg.save_hyperparameters(ckpt)
+        sae.save_checkpoint(ckpt / "sae_weights.safetensors")
+        state = {k: getattr(self, k) for k in self._STATE_KEYS}
+        state["cfg"] = self.cfg.model_dump()
+        state["amp_dtype"] = None if self.cfg.amp_dtype is None else str(self.cfg.amp_dtype)
+        torch.save(state, ckpt / "trainer.pt")
+        if self.optimizer is not None:
+            torch.save(self.optimizer.state_dict(), ckpt / "optimizer.pt")
+        if self.scheduler is not None:
+            torch.save(self.scheduler.state_dict(), ckpt / "scheduler.pt")
+        return ckpt
+
+    @classmethod
+    def from_checkpoint(cls, sae: SparseDictionary, checkpoint_path) -> "Trainer":
+        """A trainer that continues where `save_checkpoint` stopped: counters and config from `trainer.pt`, a fresh
+        optimizer and scheduler for `sae` (whose weights the caller loads from the same directory) with their saved
+        states loaded.  `fit` then skips its own initialisation (cfg.from_pretrained_path is set)."""
+        ckpt = Path(checkpoint_path)
+        if not os.path.exists(ckpt / "trainer.pt"):
+            raise ValueError(f"Trainer checkpoint not found at {ckpt / 'trainer.pt'}")
+        state = torch.load(ckpt / "trainer.pt", map_location="cpu", weights_only=True)
+        cfg = state.get("cfg")
+        if cfg is None:
+            raise ValueError("Checkpoint does not contain trainer config")
+        cfg = dict(cfg)
+        amp = state.get("amp_dtype")
+        cfg["amp_dtype"] = None if amp is None else getattr(torch, str(amp).replace("torch.", ""))
+        cfg["from_pretrained_path"] = str(checkpoint_path)
+        trainer = cls(TrainerConfig(**cfg))
+        for k in cls._STATE_KEYS:
+            setattr(trainer, k, state[k])
+        trainer._initialize_optimizer(sae)
+        trainer.optimizer.load_state_dict(torch.load(ckpt / "optimizer.pt", map_location="cpu", weights_only=True))
+        trainer.scheduler.load_state_dict(torch.load(ckpt / "scheduler.pt", map_location="cpu", weights_only=True))
+        return trainer
+
+    def _maybe_save_sae_checkpoint(self, sae: SparseDictionary) -> None:
+        """trainer.py:563-574: the model's weights each time the step counter passes the next threshold."""
+        if self.checkpoint_thresholds and self.cur_step >= self.checkpoint_thresholds[0]:
+            path = os.path.join(self.cfg.exp_result_path, "checkpoints", f"{self.cur_step}.safetensors")
+            os.makedirs(os.path.dirname(path), exist_ok=True)
+            sae.save_checkpoint(path)
+            self.checkpoint_thresholds.pop(0)
 
     # ---- trainer.py:349-401 ----
     def _initialize_optimizer(self, sae: SparseDictionary):
@@ -264,6 +345,7 @@ class Trainer:
         try:
             while True:
                 self.train_one_step(sae, batch, on_step)
+                self._maybe_save_sae_checkpoint(sae)
                 if self.cur_step >= self.total_training_steps:
                     break
                 batch = next(stream)

@@ -140,3 +140,79 @@ def test_variant_checkpoints_round_trip(pkg, tmp_path, kind):
         for k in f.keys():
             if not k.startswith("dataset_average_activation_norm."):
                 assert tuple(f.get_tensor(k).shape) == tuple(model.state_dict()[k].shape), k
+
+
+# ---- trainer checkpoints (trainer.py:155-307) and optimizer-state interchange with torch.optim.Adam ----
+
+def _tiny_sae(pkg, device="cpu"):
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=8, expansion_factor=2, act_fn="topk", top_k=2,
+                        norm_activation="inference", device=device, dtype=torch.float32)
+    m = pkg.SparseAutoEncoder(cfg)
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(torch.randn(p.shape, generator=g))
+    return m
+
+
+def test_adam_state_crosses_between_torch_adam_and_hip_adam(pkg):
+    """A torch.optim.Adam state dict (moments contiguous in the reference's [d, F] shape for W_E) loads into HipAdam
+    with the moments re-laid to the parameter's feature-major strides, and HipAdam's own state dict goes back."""
+    m = _tiny_sae(pkg)
+    twin = {n: torch.nn.Parameter(p.detach().clone().contiguous()) for n, p in m.named_parameters()}
+    topt = torch.optim.Adam(list(twin.values()), lr=1e-3)
+    g = torch.Generator().manual_seed(4)
+    for _ in range(2):
+        for p in twin.values():
+            p.grad = torch.randn(p.shape, generator=g)
+        topt.step()
+    sd = topt.state_dict()
+    assert sd["state"][0]["exp_avg"].is_contiguous()
+    hopt = pkg.HipAdam(list(m.parameters()), lr=1e-3, model=m)
+    hopt.load_state_dict(sd)
+    for (n, p), q in zip(m.named_parameters(), twin.values()):
+        st = hopt.state[p]
+        assert st["exp_avg"].stride() == p.stride() and st["exp_avg_sq"].stride() == p.stride(), n
+        assert torch.equal(st["exp_avg"], topt.state[q]["exp_avg"]) and torch.equal(st["exp_avg_sq"], topt.state[q]["exp_avg_sq"])
+        assert st["step"].device.type == "cpu" and float(st["step"]) == 2.0
+    assert m.W_E.stride() == (1, 8) and hopt.state[m.W_E]["exp_avg"].t().is_contiguous()
+    back = hopt.state_dict()
+    assert all(s["exp_avg"].is_contiguous() and s["exp_avg_sq"].is_contiguous() for s in back["state"].values())
+    topt2 = torch.optim.Adam([torch.nn.Parameter(p.detach().clone().contiguous()) for p in m.parameters()], lr=1e-3)
+    topt2.load_state_dict(back)
+    for a, b in zip(topt2.state.values(), topt.state.values()):
+        assert torch.equal(a["exp_avg"], b["exp_avg"]) and torch.equal(a["exp_avg_sq"], b["exp_avg_sq"]) and float(a["step"]) == 2.0
+    with pytest.raises(ValueError, match="shape"):
+        bad = topt.state_dict()
+        bad["state"][0]["exp_avg"] = torch.zeros(3, 3)
+        pkg.HipAdam(list(m.parameters()), lr=1e-3).load_state_dict(bad)
+
+
+def test_trainer_checkpoint_file_set_and_resume_state(pkg, tmp_path):
+    """The reference's directory layout and the counters a resumed trainer starts from."""
+    m = _tiny_sae(pkg)
+    cfg = pkg.TrainerConfig(total_training_tokens=40, lr=1e-3, lr_warm_up_steps=2, lr_cool_down_steps=2, amp_dtype=None,
+                            k_warmup_steps=0, l1_coefficient=None, n_checkpoints=2, check_point_save_mode="linear",
+                            exp_result_path=str(tmp_path / "results"))
+    tr = pkg.Trainer(cfg)
+    tr._initialize_trainer(m, {"tokens": torch.zeros(4)})
+    assert tr.total_training_steps == 10 and tr.checkpoint_thresholds == [5]
+    tr._initialize_optimizer(m)
+    for _ in range(3):     # the counters and the LR schedule move as in three steps (no kernel runs on the CPU)
+        tr.scheduler.step(); tr.cur_step += 1; tr.cur_tokens += 4
+    ckpt = tr.save_checkpoint(m, tmp_path / "run")
+    assert ckpt == tmp_path / "run" / "checkpoints" / "step_3"
+    assert sorted(p.name for p in ckpt.iterdir()) == ["config.json", "optimizer.pt", "sae_weights.safetensors", "scheduler.pt", "trainer.pt"]
+    m2 = pkg.SparseDictionary.from_pretrained(str(ckpt), device="cpu", dtype=torch.float32)
+    assert all(torch.equal(a, b) for a, b in zip(m.parameters(), m2.parameters()))
+    tr2 = pkg.Trainer.from_checkpoint(m2, str(ckpt))
+    assert (tr2.cur_step, tr2.cur_tokens, tr2.total_training_steps, tr2.checkpoint_thresholds) == (3, 12, 10, [5])
+    assert tr2.cfg.from_pretrained_path == str(ckpt) and tr2.cfg.amp_dtype is None and tr2.cfg.lr == 1e-3
+    assert tr2.scheduler.last_epoch == 3 and tr2.optimizer.param_groups[0]["lr"] == tr.optimizer.param_groups[0]["lr"]
+    with pytest.raises(ValueError, match="not found"):
+        pkg.Trainer.from_checkpoint(m2, str(tmp_path))
+    # "log" thresholds as the reference computes them (trainer.py:339-343)
+    tr3 = pkg.Trainer(pkg.TrainerConfig(total_training_tokens=4096, n_checkpoints=4, exp_result_path=str(tmp_path / "r3")))
+    tr3._initialize_trainer(m, {"tokens": torch.zeros(4)})
+    import math
+    assert tr3.checkpoint_thresholds == [math.ceil(2 ** (i / 4 * 10)) * 4 for i in (1, 2, 3)]

@@ -47,3 +47,89 @@ def test_reference_layout_checkpoint_trains_on_the_hip_path_and_back(pkg, oracle
     assert abs(got - want) < 1e-5 * want
     for n, p in ref.named_parameters():
         assert (back[n] - p.detach()).abs().max() <= 2e-2 * 3e-3 + 1e-6 * p.detach().abs().max(), n
+
+
+def _stream(x, B, n, dev):
+    for i in range(n):
+        rows = x[(i * B) % x.shape[0]:][:B]
+        yield {"in": rows.to(dev), "out": rows.to(dev), "tokens": torch.zeros(B, device=dev),
+               "mask": torch.ones(B, device=dev)}
+
+
+def test_trainer_resumes_bit_identically_from_a_complete_checkpoint(pkg, dev, tmp_path):
+    """trainer.py:155-307: three steps, a checkpoint, two more steps -- against loading the checkpoint into a fresh
+    model + `Trainer.from_checkpoint` and running the same two steps: parameters and moments agree to the bit."""
+    from lm_saes_amd import synthetic
+
+    d, F, k, B = 128, 1024, 8, 96
+    x = synthetic.activations(5 * B, d, 8, seed=41)
+    w = synthetic.sae_weights(d, F, x, seed=41)
+
+    def fresh():
+        cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                            top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
+        m = pkg.SparseAutoEncoder(cfg)
+        synthetic.load_weights(m, *[t.to(dev) for t in w])
+        return m
+
+    tcfg = pkg.TrainerConfig(total_training_tokens=5 * B, lr=1e-3, lr_warm_up_steps=2, lr_cool_down_steps=2, amp_dtype=None,
+                             k_warmup_steps=0, l1_coefficient=None, skip_metrics_calculation=True,
+                             exp_result_path=str(tmp_path / "results"))
+    sae, tr = fresh(), pkg.Trainer(tcfg)
+    batches = list(_stream(x, B, 5, dev))
+    tr.prepare(sae, batches[0])
+    for b in batches[:3]:
+        tr.train_one_step(sae, b)
+    ckpt = tr.save_checkpoint(sae, tmp_path / "run")
+    for b in batches[3:]:
+        tr.train_one_step(sae, b)
+
+    sae2 = pkg.SparseDictionary.from_pretrained(str(ckpt), device="cuda", dtype=torch.float32)
+    tr2 = pkg.Trainer.from_checkpoint(sae2, str(ckpt))
+    assert tr2.cur_step == 3 and tr2.optimizer.param_groups[0]["lr"] == pytest.approx(1e-3)
+    assert tr2.fit(sae2, iter(batches[3:])) is None and tr2.cur_step == 5
+    torch.cuda.synchronize()
+    for (n, p), q in zip(sae.named_parameters(), sae2.parameters()):
+        assert torch.equal(p, q), n
+        a, b = tr.optimizer.state[p], tr2.optimizer.state[q]
+        assert torch.equal(a["exp_avg"], b["exp_avg"]) and torch.equal(a["exp_avg_sq"], b["exp_avg_sq"]), n
+        assert float(a["step"]) == float(b["step"]) == 5.0
+
+
+def test_torch_adam_state_continues_on_hip_adam(pkg, oracle, dev):
+    """Optimizer state written by torch.optim.Adam on the reference layout (the oracle model, W_E moments [d, F]
+    contiguous) is loaded into HipAdam; both then take the same two steps and stay together."""
+    from lm_saes_amd import synthetic
+
+    d, F, k, B = 128, 1024, 8, 96
+    x = synthetic.activations(B, d, 8, seed=43)
+    w = synthetic.sae_weights(d, F, x, seed=43)
+    ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k)
+    synthetic.load_weights(ref, *w)
+    ropt = oracle.make_adam(ref, lr=1e-3)
+    cpu_batch = {"in": x, "out": x, "tokens": torch.zeros(B)}
+    for _ in range(2):
+        oracle.train_step(ref, ropt, cpu_batch)
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                        top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    sae.load_state_dict({n: p.detach().to(dev) for n, p in ref.named_parameters()})
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=1e-3, model=sae)
+    # the oracle's parameter order is the module's: map its state onto HipAdam's parameters by name
+    order = {id(p): i for i, p in enumerate(opt.param_groups[0]["params"])}
+    by_name = dict(sae.named_parameters())
+    sd = ropt.state_dict()
+    ref_idx = {id(p): i for i, p in enumerate(q for g in ropt.param_groups for q in g["params"])}
+    state = {order[id(by_name[n])]: sd["state"][ref_idx[id(p)]] for n, p in ref.named_parameters()}
+    opt.load_state_dict({"state": state, "param_groups": opt.state_dict()["param_groups"]})
+    assert opt.state[sae.W_E]["exp_avg"].stride() == sae.W_E.stride()
+    batch = {k_: v.to(dev) for k_, v in cpu_batch.items()}
+    for _ in range(2):
+        loss = sae.compute_loss(batch, return_aux_data=False)
+        loss.backward(); opt.step(); opt.zero_grad()
+        oracle.train_step(ref, ropt, cpu_batch)
+    for n, p in ref.named_parameters():
+        got = by_name[n].detach().cpu()
+        assert (got - p.detach()).abs().max() <= 2e-2 * 2e-3 + 1e-6 * p.detach().abs().max(), n
+        m_ref = ropt.state[p]["exp_avg"]
+        assert (opt.state[by_name[n]]["exp_avg"].cpu() - m_ref).abs().max() <= 1e-4 * m_ref.abs().max() + 1e-9, n
