@@ -64,6 +64,19 @@ def merge_layer_codes(codes: list[ops.SparseCode]) -> tuple[ops.SparseCode, torc
     return ops.SparseCode(idx, val.contiguous(), row_off, row_nnz, B, L * F), layer_cnt
 
 
+def relabel_feature_major_code(code: ops.SparseCode, L: int, F: int) -> ops.SparseCode:
+    """A code whose feature ids are f * L + l (the columns of a [B, F, L] matrix) -> the same entries under
+    ids l * F + f, every token's entries re-sorted to ascend in (layer, feature).  Rows keep their extents."""
+    tok, valid = _slot_tokens(code)
+    raw = code.idx.long()
+    new = (raw % L) * F + torch.div(raw, L, rounding_mode="floor")
+    sentinel = torch.iinfo(torch.int64).max
+    key, perm = torch.sort(torch.where(valid, tok * (L * F) + new, torch.full_like(new, sentinel)))
+    idx = torch.where(key == sentinel, torch.zeros_like(key), key % (L * F)).to(torch.int32)
+    # valid slots are packed row after row from slot 0 on (the batch select's layout), so sorted position = slot
+    return dataclasses.replace(code, idx=idx, val=code.val[perm].contiguous())
+
+
 def layer_counts(code: ops.SparseCode, L: int, F: int) -> torch.Tensor:
     """Entries per (token, layer) [B, L] of a code over L*F features."""
     tok, valid = _slot_tokens(code)
@@ -101,12 +114,16 @@ class _FusedCLTStep(torch.autograd.Function):
             codes = [sel(pres[l], b_enc[l], None if norms is None else norms[l]) for l in range(L)]
             cat, layer_cnt = merge_layer_codes(codes)
         else:
-            pre_cat = torch.stack(pres, dim=1).view(B, L * F)
+            pre_cat = torch.stack(pres, dim=1).view(B, L * F) if act == "layertopk" else None
             flat = lambda t: None if t is None else t.reshape(L * F)      # noqa: E731
             if act == "layertopk":
                 cat = ops.select_topk_row(pre_cat, flat(b_enc), flat(norms), min(k, L * F))
             else:
-                cat = ops.select_topk_batch(pre_cat, flat(b_enc), flat(norms), k * B)
+                # the reference flattens this scope as (batch, feature, layer) (clt.py:312: dim=(0, -1, -2)), which is
+                # the order that decides ties at the threshold: select over the [B, F, L] arrangement, then relabel
+                tr = lambda t: None if t is None else t.t().reshape(F * L).contiguous()   # noqa: E731
+                cat = ops.select_topk_batch(torch.stack(pres, dim=2).view(B, F * L), tr(b_enc), tr(norms), k * B)
+                cat = relabel_feature_major_code(cat, L, F)
             layer_cnt = layer_counts(cat, L, F)
         prefix = torch.cumsum(layer_cnt, dim=1).to(torch.int32)           # entries of layers <= j, per token
         tok_w = torch.full((B,), 1.0 / (L * B), dtype=torch.float32, device=x.device)

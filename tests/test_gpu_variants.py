@@ -53,6 +53,29 @@ def check_grads(model, ref, tol=GRAD_TOL):
         assert rel_err(p.grad, rp[n].grad) < tol, (n, rel_err(p.grad, rp[n].grad))
 
 
+def check_bf16_grads_on_the_kernels_selection(model, ref, run_ref, kept_cpu):
+    """The oracle's backward under CPU bf16 autocast, its activation replaced by `h * kept` (the kernel's own
+    selection: TopK passes the gradient of kept entries and nothing else, so the autograd is the same), against
+    the kernel path's gradients at the bf16 bound.  Without the substitution an entry near the k-th value can fall
+    on the other side in the oracle's differently rounded product, and the gradients would differ by whole rows."""
+    ref.activation_function = lambda h: h * kept_cpu.to(h.dtype).reshape(h.shape)
+    for p in ref.parameters():
+        p.grad = None
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        want = run_ref()
+    want["loss"].backward()
+    rp = {k.replace("ln_q_w", "ln_q.w").replace("ln_k_w", "ln_k.w"): v for k, v in ref.named_parameters()}
+    scale = max(v.grad.abs().max().item() for v in rp.values())
+    errs = {}
+    for n, p in model.named_parameters():
+        assert p.grad is not None and tuple(p.grad.shape) == tuple(p.shape), n
+        if rp[n].grad.abs().max().item() < 1e-4 * scale:
+            continue     # analytically zero: rounding noise on both sides
+        errs[n] = rel_err(p.grad, rp[n].grad)
+    assert all(e < BF16_TOL for e in errs.values()), errs
+    return want
+
+
 # ---- crosscoder ----------------------------------------------------------------------------------
 
 def make_crosscoder(pkg, vo, dev, H, d, F, k, seed):
@@ -136,7 +159,7 @@ def test_crosscoder_fused_step_bf16(pkg, vo, dev):
         assert rel_err(acts, own) < FP32_TOL
         assert rel_err(out["reconstructed"], ref.decode(acts)) < BF16_TOL
     out["loss"].backward()
-    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+    check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch, hooks), acts > 0)
 
 
 # ---- CLT -----------------------------------------------------------------------------------------
@@ -186,6 +209,40 @@ def test_clt_fused_step_fp32(pkg, vo, dev, act_fn, L, d, F, k, B, include_norm):
     assert rel_err(out["loss"], want["loss"]) < FP32_TOL
     out["loss"].backward(); want["loss"].backward()
     check_grads(m, ref)
+
+
+def test_clt_batch_layer_scope_breaks_exact_ties_in_the_reference_order(pkg, vo, dev):
+    """The batch-and-layer-wide scope flattens (batch, feature, layer) in the reference (clt.py:312, dim=(0, -1, -2)),
+    so of two equal values at the threshold the one with the lower f * L + l inside the token is kept.  Layer 1 is
+    built as layer 0 with its features reversed and fed the same input, so every positive value occurs exactly
+    twice in a token, as (0, f) and (1, F - 1 - f); an odd k * B splits the pair at the threshold.  For f > F / 2 the
+    reference order keeps the layer-1 twin where a (batch, layer, feature) flattening would keep the layer-0 one."""
+    L, d, F = 2, 32, 64
+    decided_by_order = 0
+    for seed, k, B in [(61, 3, 7), (62, 5, 9), (63, 3, 11), (64, 7, 5), (65, 5, 13), (66, 3, 9)]:
+        m, ref, hin, hout = make_clt(pkg, vo, dev, "batchlayertopk", L, d, F, k, seed=seed, include_norm=False)
+        with torch.no_grad():
+            ref.W_E[1] = ref.W_E[0].flip(-1)
+            ref.b_E[1] = ref.b_E[0].flip(-1)
+        copy_params(m, ref)
+        batch = clt_batch(L, B, d, seed=seed + 100)
+        batch["i1"] = batch["i0"].clone()
+        gb = {k_: v.to(dev) for k_, v in batch.items()}
+        out = m.compute_loss(gb)
+        assert "sparse_code" in out, "the kernel path did not run"
+        want = ref.compute_loss(batch, hin, hout)
+        got_kept, want_kept = (out["feature_acts"] > 0).cpu(), want["feature_acts"] > 0
+        assert int(want_kept.sum()) == k * B
+        assert torch.equal(got_kept, want_kept), f"seed {seed}: selections differ"
+        assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
+        # which twin was kept at the split pair: layer 1's only if the reference order says so
+        twins = want_kept[:, 0, :] != want_kept[:, 1, :].flip(-1)           # [B, F]: pairs of which one member is kept
+        assert int(twins.sum()) == 1
+        b, f = [int(t) for t in twins.nonzero()[0]]
+        kept_layer = 0 if want_kept[b, 0, f] else 1
+        assert kept_layer == (0 if f * L < (F - 1 - f) * L + 1 else 1)
+        decided_by_order += int(kept_layer == 1)
+    assert decided_by_order > 0, "no case in which the two flattening orders disagree was drawn"
 
 
 def test_clt_fused_matches_own_dense_path_and_adam(pkg, vo, dev):
@@ -254,10 +311,12 @@ def test_clt_fused_step_bf16(pkg, vo, dev):
         out = m.compute_loss(gb)
     want = ref.compute_loss(batch, hin, hout)
     assert rel_err(out["loss"], want["loss"]) < BF16_TOL
-    agree = ((out["feature_acts"] > 0).cpu() == (want["feature_acts"] > 0)).float().mean().item()
+    kept = (out["feature_acts"] > 0).cpu()
+    agree = (kept == (want["feature_acts"] > 0)).float().mean().item()
     assert agree > 0.999
     out["loss"].backward()
-    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+    w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch, hin, hout), kept)
+    assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["loss"], w16["loss"]) < BF16_TOL
 
 
 # ---- Lorsa ---------------------------------------------------------------------------------------
@@ -312,7 +371,9 @@ def test_lorsa_fused_step_bf16(pkg, vo, dev):
     want = ref.compute_loss(batch)
     assert rel_err(out["loss"], want["loss"]) < BF16_TOL
     out["loss"].backward()
-    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+    kept = (out["feature_acts"] > 0).cpu()
+    w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch), kept)
+    assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["hidden_pre"], w16["hidden_pre"]) < BF16_TOL
 
 
 def test_lorsa_adam_steps_with_factored_output_gradient(pkg, vo, dev):
