@@ -402,6 +402,38 @@ int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float
                      int64_t B, int64_t F, void *d_pre, float *d_bias, float *d_theta, float *d_pen_norm,
                      void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- Causal attention with grouped value heads (low-rank sparse attention) -------------------------------
+ * Replaces F.scaled_dot_product_attention(query, key, value, scale, is_causal=True) as LowRankSparseAttention calls it
+ * (models/lorsa.py:650-660, 714-724) and its autograd backward: n_heads query/key heads of width d_qk, and per head a
+ * value of width d_v whose columns are the d_v rank-1 value heads (dictionary features) that share the head's pattern.
+ *   out[b, s, h, :] = sum_{s' <= s} softmax_{s'}(scale * q[b, s, h, :] . k[b, s', h, :]) * v[b, s', h, :]
+ * bf16 operands, fp32 accumulation, probabilities rounded to bf16 before they multiply the values (as the library's
+ * fused kernels do).  T = n_batch * seq, token t = b * seq + s.  Layouts: "natural" [T, n_heads * width] (heads side by
+ * side: what x @ W gives) and "transposed" [n_heads * width, T]; each operand is taken in the layout(s) whose
+ * contraction index is contiguous for the products that read it.
+ *   q, k      natural    [T, n_heads * d_qk]
+ *   vt        transposed [n_heads * d_v, T]
+ *   q_bias / k_bias [n_heads * d_qk], v_bias [n_heads * d_v]  fp32, nullable, 16-byte aligned: added to the bf16 operand
+ *             as it is loaded and rounded back to bf16 (the projections' `+ b_Q`, `+ b_K`, `+ b_V`, models/lorsa.py:793-813)
+ *   out       natural    [T, n_heads * d_v] bf16;  lse fp32 [n_batch, n_heads, seq] = log sum_{s'} exp(scale * q . k)
+ * Requires d_qk in {32, 64}, d_v in {32, 64, 128}, seq % 8 == 0. */
+int sae_attention_fwd(const void *q, const void *k, const void *vt, const float *q_bias, const float *k_bias,
+                      const float *v_bias, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v,
+                      double scale, void *out, float *lse, void *stream);
+
+/* Backward of sae_attention_fwd.  q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout (biases
+ * are added to q / qt, k / kt and v on load as in the forward pass); lse from the forward pass; dvec_workspace: device
+ * float[n_batch * n_heads * seq].  Outputs, bf16, transposed: dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T] (the
+ * gradients of the biased operands; a bias gradient is the row sum, sae_row_sum).  No atomics: reproducible. */
+int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
+                      const void *dout, const void *doutt, const float *q_bias, const float *k_bias, const float *v_bias,
+                      const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v, double scale,
+                      float *dvec_workspace, void *dqt, void *dkt, void *dvt, void *stream);
+
+/* out[r] = sum_c src[r, c] (fp32 sum, fixed order) for src [rows, cols] fp32 or bf16.  The bias gradients autograd forms by
+ * summing over tokens, for gradients held transposed ([features, tokens]). */
+int sae_row_sum(const void *src, int src_dtype, int64_t rows, int64_t cols, float *out, void *stream);
+
 /* Measurement aid, no counterpart in the reference: n_workgroups x 4 waves each issue iters x 32
  * v_mfma_f32_16x16x32_bf16 from registers (no memory traffic in the loop) and write one float per lane to
  * out [n_workgroups * 256].  *flop_out (host, optional) receives the flop count of the launch.  The rate it

@@ -5,11 +5,15 @@ heads `W_Q, W_K [h, d, q]`, and `d_sae` rank-1 value/output heads `W_V, W_O [F, 
 one dictionary feature; feature f mixes its values over key positions with the causal softmax
 pattern of query/key head f // (F / h).
 
-What runs where: the value projection is the encoder GEMM kernel (`W_V` is feature-major already);
-the query/key projections and the attention mixing are torch library routines (small GEMMs and
-scaled-dot-product attention); the TopK select, the sparse decode through `W_O`, the squared
-error, the `W_O` gradient rows and the scatter of the value gradients back to the dense
-pre-activation are the sparse kernels of the SAE path.
+What runs where under bf16 autocast (the reference's default precision): the three projections are the
+encoder GEMM kernel (`W_V` is feature-major already; the query / key weights are used through a
+[heads * width, d_model] bf16 copy), the causal attention mixing and its backward are the matrix-core
+attention kernels (no [s, s] matrix, no padding of the narrower query / key heads to the value width),
+the weight gradients of the projections are GEMM-kernel products over the token axis, and the TopK
+select, the sparse decode through `W_O`, the squared error, the `W_O` gradient rows and the scatter of
+the value gradients back to the dense pre-activation are the sparse kernels of the SAE path.  In fp32,
+with rotary embeddings or query / key norms, or with user hooks on the attention internals, the
+projections and the mixing are torch library routines.
 """
 
 from __future__ import annotations
@@ -74,6 +78,66 @@ class _ValueProjection(torch.autograd.Function):
         return gx, gw, None, None
 
 
+class _ProjectAndMix(torch.autograd.Function):
+    """x -> q, k, v projections -> causal attention mixing -> hidden_pre [T, F] (bf16), all on the GEMM and attention
+    kernels, for the configuration without rotary embedding and query / key norms.
+
+    forward : q = x W_Q, k = x W_K as [T, h dq] (natural), v^T = W_V x^T as [F, T] (the GEMM with its operands swapped
+              yields the transposed layout the mixing product contracts over); the biases are added as the attention
+              kernel loads its operands.
+    backward: the transposed copies q^T, k^T (swapped GEMMs), v (GEMM), dout^T (cast-transpose kernel); the attention
+              backward returns dq^T, dk^T, dv^T [., T], which are exactly the operands of the weight-gradient products
+              dW = d(.)^T x over the token axis; bias gradients are their row sums."""
+
+    @staticmethod
+    def forward(ctx, x2, W_Q, W_K, W_V, b_Q, b_K, b_V, model, seq):
+        cfg = model.cfg
+        T = x2.shape[0]
+        n_batch, h = T // seq, cfg.n_qk_heads
+        x_op = x2 if x2.dtype == torch.bfloat16 else ops.cast_bf16(x2.float().contiguous())
+        wq, wk, wv = model._w_qk_operand("W_Q"), model._w_qk_operand("W_K"), model._w_val_operand(True)
+        q = ops.encoder_gemm(x_op, wq, torch.bfloat16)                      # [T, h dq]
+        k = ops.encoder_gemm(x_op, wk, torch.bfloat16)
+        vt = ops.encoder_gemm(wv, x_op, torch.bfloat16)                     # [F, T]
+        scale = 1.0 / model.attn_scale
+        out, lse = ops.attention_fwd(q, k, vt, n_batch, seq, h, scale, b_Q, b_K, b_V)
+        ctx.save_for_backward(x_op, wq, wk, wv, q, k, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
+        ctx.dims = (n_batch, seq, h, scale)
+        ctx.shapes = (tuple(W_Q.shape), tuple(W_K.shape))
+        ctx.x_dtype = x2.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dz):
+        x_op, wq, wk, wv, q, k, out, lse, b_Q, b_K, b_V = ctx.saved_tensors
+        n_batch, seq, h, scale = ctx.dims
+        dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
+        qt = ops.encoder_gemm(wq, x_op, torch.bfloat16)                     # [h dq, T]
+        kt = ops.encoder_gemm(wk, x_op, torch.bfloat16)
+        v = ops.encoder_gemm(x_op, wv, torch.bfloat16)                      # [T, F]
+        dzt = ops.transpose_to_bf16(dz)[0]                                  # [F, T]
+        dqt, dkt, dvt = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale, b_Q, b_K, b_V)
+        xt = ops.transpose_to_bf16(x_op)[0]                                 # [d, T]
+        d = x_op.shape[1]
+        dq_w = q.shape[1] // h
+
+        def qk_weight_grad(gt, shape):
+            rows = ops.encoder_gemm(gt, xt, torch.float32)                  # [h dq, d] = d(.)^T x
+            return rows.view(h, dq_w, d).permute(0, 2, 1).contiguous().view(shape)
+
+        dW_Q = qk_weight_grad(dqt, ctx.shapes[0]) if ctx.needs_input_grad[1] else None
+        dW_K = qk_weight_grad(dkt, ctx.shapes[1]) if ctx.needs_input_grad[2] else None
+        dW_V = ops.encoder_gemm(dvt, xt, torch.float32) if ctx.needs_input_grad[3] else None
+        db_Q = ops.row_sum(dqt).view(b_Q.shape) if ctx.needs_input_grad[4] else None
+        db_K = ops.row_sum(dkt).view(b_K.shape) if ctx.needs_input_grad[5] else None
+        db_V = ops.row_sum(dvt).view(b_V.shape) if ctx.needs_input_grad[6] else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            # rare (activations do not carry gradients in training): library products on the transposed gradients
+            dx = (dqt.t().float() @ wq.float() + dkt.t().float() @ wk.float() + dvt.t().float() @ wv.float()).to(ctx.x_dtype)
+        return dx, dW_Q, dW_K, dW_V, db_Q, db_K, db_V, None, None
+
+
 class _SparseTail(torch.autograd.Function):
     """hidden_pre [T, F] -> TopK select (decoder-norm scale fused) -> sparse decode through W_O + b_D ->
     masked-mean squared error.  Backward: W_O gradient rows from the feature index, b_D from a column
@@ -115,7 +179,10 @@ class _SparseTail(torch.autograd.Function):
             dW_O, _ = ops.sparse_grad_rows(fi, code.val * g, ctx.grad_recon, F)
         db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
         d_hp = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and ctx.in_dtype == torch.bfloat16:
+            import dataclasses
+            d_hp = ops.code_to_dense(dataclasses.replace(code, val=ctx.dval * g), F, want_f32=False, want_bf16=True)[1]
+        elif ctx.needs_input_grad[0]:
             slots = torch.arange(code.n_slots, device=code.idx.device)
             tok = (torch.searchsorted(code.row_off, slots, right=True) - 1).clamp_(min=0)
             valid = (slots - code.row_off[tok]) < code.row_nnz[tok]
@@ -143,6 +210,8 @@ class LowRankSparseAttention(SparseDictionary):
         # set by an optimiser that consumes factored gradients (HipAdam): W_O's gradient is then attached to it as
         # `_sparse_grad` instead of being written as dense rows
         self.defer_weight_grads = False
+        # False sends projections and attention mixing to the torch library routines in every configuration
+        self.use_mix_kernels = True
         self.register_buffer("mask", torch.tril(torch.ones((cfg.n_ctx, cfg.n_ctx), device=cfg.device).bool()))
         self.register_buffer("IGNORE", torch.tensor(-torch.inf, device=cfg.device))
         if cfg.use_post_qk_ln:
@@ -220,6 +289,29 @@ class LowRankSparseAttention(SparseDictionary):
         if not amp or w.dtype == torch.bfloat16:
             return w
         return self._derive("W_V.bf16", self.W_V, lambda old: ops.cast_bf16(w, old))
+
+    def _w_qk_operand(self, name: str) -> torch.Tensor:
+        """bf16 [n_qk_heads * d_qk_head, d_model] copy of W_Q / W_K [h, d, q] (one head's output column = one row)."""
+        p = getattr(self, name)
+        h, d, dq = p.shape
+        return self._derive(f"{name}.rows.bf16", p, lambda old: ops.cast_bf16(
+            p.detach().float().permute(0, 2, 1).reshape(h * dq, d).contiguous(), old))
+
+    def _mix_kernel_eligible(self, x: torch.Tensor) -> bool:
+        """The projections + mixing run on the GEMM and attention kernels: bf16 autocast over fp32 parameters, no
+        rotary embedding or query / key norm between projection and scores, no user hook on the attention internals,
+        and shapes the kernels are built for."""
+        cfg = self.cfg
+        if not (self.use_mix_kernels and x.is_cuda and x.ndim == 3 and _autocast_dtype("cuda") == torch.bfloat16
+                and self.W_V.dtype == torch.float32):
+            return False
+        if cfg.positional_embedding_type == "rotary" or cfg.use_post_qk_ln:
+            return False
+        if any(getattr(self, f"hook_{n}").has_hooks for n in ("q", "k", "q_post_rot", "k_post_rot", "attn_pattern", "attn_score")):
+            return False
+        b, s, d = x.shape
+        return (ops.attention_shapes_supported(s, cfg.d_qk_head, cfg.ov_group_size) and d % 64 == 0 and (b * s) % 64 == 0
+                and cfg.d_sae == cfg.n_qk_heads * cfg.ov_group_size)
 
     def _w_dec_operand(self, amp: bool) -> torch.Tensor:
         w = self.W_O.detach()
@@ -347,7 +439,11 @@ class LowRankSparseAttention(SparseDictionary):
         return torch.einsum("hbqk,bkhr->bqhr", pattern, vg).reshape(b, -1, F)
 
     def compute_hidden_pre(self, x: torch.Tensor) -> torch.Tensor:
-        """lorsa.py:642-662: causal attention of every feature's value over key positions (library SDPA)."""
+        """lorsa.py:642-662: causal attention of every feature's value over key positions."""
+        if self._mix_kernel_eligible(x):
+            b, s, d = x.shape
+            z = _ProjectAndMix.apply(x.reshape(b * s, d), self.W_Q, self.W_K, self.W_V, self.b_Q, self.b_K, self.b_V, self, s)
+            return z.view(b, s, self.cfg.d_sae)
         q, k, v = self._compute_qkv(x)
         query, key = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3)
         value = v.reshape(*k.shape[:3], -1).permute(0, 2, 1, 3)

@@ -739,6 +739,90 @@ def recon_stats(label: torch.Tensor, recon: torch.Tensor, label_mean: torch.Tens
     return out
 
 
+# ---- causal attention with grouped value heads ------------------------------------------------------------
+
+ATTENTION_D_QK = (32, 64)
+ATTENTION_D_V = (32, 64, 128)
+
+
+def attention_shapes_supported(seq: int, d_qk: int, d_v: int) -> bool:
+    """Whether the attention kernels are built for these head widths and sequence length."""
+    return d_qk in ATTENTION_D_QK and d_v in ATTENTION_D_V and seq % 8 == 0
+
+
+def _att_check(name: str, t: torch.Tensor, shape: tuple) -> None:
+    _req(t, name, torch.bfloat16, 2)
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _att_bias(name: str, t: Optional[torch.Tensor], n: int) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    t = t.detach().reshape(-1)
+    _req(t, name, torch.float32, 1)
+    if t.numel() != n:
+        raise ValueError(f"{name} must have {n} elements")
+    return t
+
+
+def attention_fwd(q: torch.Tensor, k: torch.Tensor, vt: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
+                  q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
+                  v_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Causal softmax attention: q, k natural [T, n_heads * d_qk], vt transposed [n_heads * d_v, T] (bf16, T = n_batch * seq)
+    -> (out natural [T, n_heads * d_v] bf16, lse fp32 [n_batch, n_heads, seq]).  Biases (fp32) are added on load."""
+    T = n_batch * seq
+    d_qk, d_v = q.shape[1] // n_heads, vt.shape[0] // n_heads
+    _att_check("q", q, (T, n_heads * d_qk)); _att_check("k", k, (T, n_heads * d_qk)); _att_check("vt", vt, (n_heads * d_v, T))
+    bq, bk, bv = _att_bias("q_bias", q_bias, n_heads * d_qk), _att_bias("k_bias", k_bias, n_heads * d_qk), _att_bias("v_bias", v_bias, n_heads * d_v)
+    out = torch.empty(T, n_heads * d_v, dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty(n_batch, n_heads, seq, dtype=torch.float32, device=q.device)
+    with _timed("attention_fwd"):
+        check(_lib.load().sae_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), _ptr(bq), _ptr(bk), _ptr(bv), n_batch, seq,
+                                            n_heads, d_qk, d_v, float(scale), out.data_ptr(), lse.data_ptr(), _stream(q)),
+              "attention_fwd")
+    return out, lse
+
+
+def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
+                  dout: torch.Tensor, doutt: torch.Tensor, lse: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
+                  q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
+                  v_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Backward of attention_fwd -> (dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T]) in bf16, transposed layout.
+    q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout."""
+    T = n_batch * seq
+    d_qk, d_v = q.shape[1] // n_heads, v.shape[1] // n_heads
+    for name, t, shape in (("q", q, (T, n_heads * d_qk)), ("k", k, (T, n_heads * d_qk)), ("qt", qt, (n_heads * d_qk, T)),
+                           ("kt", kt, (n_heads * d_qk, T)), ("v", v, (T, n_heads * d_v)), ("out", out, (T, n_heads * d_v)),
+                           ("dout", dout, (T, n_heads * d_v)), ("doutt", doutt, (n_heads * d_v, T))):
+        _att_check(name, t, shape)
+    _req(lse, "lse", torch.float32, 3)
+    if tuple(lse.shape) != (n_batch, n_heads, seq):
+        raise ValueError("lse must be [n_batch, n_heads, seq]")
+    bq, bk, bv = _att_bias("q_bias", q_bias, n_heads * d_qk), _att_bias("k_bias", k_bias, n_heads * d_qk), _att_bias("v_bias", v_bias, n_heads * d_v)
+    dev = q.device
+    dqt = torch.empty(n_heads * d_qk, T, dtype=torch.bfloat16, device=dev)
+    dkt = torch.empty(n_heads * d_qk, T, dtype=torch.bfloat16, device=dev)
+    dvt = torch.empty(n_heads * d_v, T, dtype=torch.bfloat16, device=dev)
+    dvec = torch.empty(n_batch * n_heads * seq, dtype=torch.float32, device=dev)
+    with _timed("attention_bwd"):
+        check(_lib.load().sae_attention_bwd(q.data_ptr(), qt.data_ptr(), k.data_ptr(), kt.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                            dout.data_ptr(), doutt.data_ptr(), _ptr(bq), _ptr(bk), _ptr(bv), lse.data_ptr(), n_batch,
+                                            seq, n_heads, d_qk, d_v, float(scale), dvec.data_ptr(), dqt.data_ptr(), dkt.data_ptr(),
+                                            dvt.data_ptr(), _stream(q)), "attention_bwd")
+    return dqt, dkt, dvt
+
+
+def row_sum(src: torch.Tensor) -> torch.Tensor:
+    """fp32 [rows] = sum over the columns of a bf16 / fp32 matrix [rows, cols]."""
+    _req(src, "src", ndim=2)
+    r, c = src.shape
+    out = torch.empty(r, dtype=torch.float32, device=src.device)
+    with _timed("row_sum"):
+        check(_lib.load().sae_row_sum(src.data_ptr(), _dt(src), r, c, out.data_ptr(), _stream(src)), "row_sum")
+    return out
+
+
 def mfma_probe(device: torch.device, n_workgroups: int = 4096, iters: int = 4096) -> Tuple[float, float]:
     """Run the register-only MFMA loop (`sae_mfma_probe`) once and return (flop of the launch, milliseconds)."""
     import ctypes

@@ -60,6 +60,14 @@ def _pieces(sg):
     return sg.pieces if hasattr(sg, "pieces") else [(0, sg)]
 
 
+def _contiguous_moments(sd: dict) -> dict:
+    """A state dict whose moments are contiguous in the parameter's logical shape.  The per-parameter dicts that
+    Optimizer.state_dict() returns are the optimiser's live ones, so they are copied, not edited."""
+    sd["state"] = {i: {k: (v.contiguous() if k in ("exp_avg", "exp_avg_sq") and torch.is_tensor(v) else v)
+                       for k, v in st.items()} for i, st in sd["state"].items()}
+    return sd
+
+
 def _relayout_loaded_state(opt: Optimizer, step_on_device: bool) -> None:
     """After Optimizer.load_state_dict: give `exp_avg` / `exp_avg_sq` the strides, dtype and device of their
     parameter (a checkpoint holds them contiguous in the logical shape; a feature-major W_E is not), and put the
@@ -165,12 +173,7 @@ class HipAdam(Optimizer):
     def state_dict(self):
         """torch.optim.Adam's layout: `step`, `exp_avg`, `exp_avg_sq` per parameter index, the two moments as
         contiguous tensors of the parameter's logical shape (a feature-major W_E's moments leave as [d, F])."""
-        sd = super().state_dict()
-        for st in sd["state"].values():
-            for k in ("exp_avg", "exp_avg_sq"):
-                if k in st and not st[k].is_contiguous():
-                    st[k] = st[k].contiguous()
-        return sd
+        return _contiguous_moments(super().state_dict())
 
     def load_state_dict(self, state_dict):
         """Accepts a torch.optim.Adam state dict (or this class's own): the moments are brought to each parameter's
@@ -377,12 +380,7 @@ class HipSparseAdam(Optimizer):
         self._model = model
 
     def state_dict(self):
-        sd = super().state_dict()
-        for st in sd["state"].values():
-            for k in ("exp_avg", "exp_avg_sq"):
-                if k in st and not st[k].is_contiguous():
-                    st[k] = st[k].contiguous()
-        return sd
+        return _contiguous_moments(super().state_dict())
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)

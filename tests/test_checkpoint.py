@@ -177,6 +177,7 @@ def test_adam_state_crosses_between_torch_adam_and_hip_adam(pkg):
         assert st["step"].device.type == "cpu" and float(st["step"]) == 2.0
     assert m.W_E.stride() == (1, 8) and hopt.state[m.W_E]["exp_avg"].t().is_contiguous()
     back = hopt.state_dict()
+    assert hopt.state[m.W_E]["exp_avg"].stride() == m.W_E.stride()      # exporting left the live state as it was
     assert all(s["exp_avg"].is_contiguous() and s["exp_avg_sq"].is_contiguous() for s in back["state"].values())
     topt2 = torch.optim.Adam([torch.nn.Parameter(p.detach().clone().contiguous()) for p in m.parameters()], lr=1e-3)
     topt2.load_state_dict(back)

@@ -1,0 +1,136 @@
+"""The causal attention kernels (grouped value heads, bf16 operands on the matrix cores) through the C ABI against
+textbook attention in fp64 with an explicit [s, s] score matrix, on inputs that are exactly representable in bf16.
+
+What separates the kernel from exact arithmetic is then only its own roundings: the probabilities are rounded to
+bf16 before they multiply the values (2^-9 relative per term), dS likewise, and the outputs are bf16 tensors
+(2^-9).  The bounds below are therefore a few 2^-9 of each tensor's largest element; the log-sum-exp, which
+never leaves fp32, is held to 1e-5.  A wrong mask, head mapping, scale or a missing rescale of the running sums is
+off by tens of percent.
+"""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 8e-3        # bf16 output + bf16 probabilities
+GRAD_TOL = 2e-2       # bf16 gradients of sums of products of bf16-rounded factors
+LSE_TOL = 1e-5
+
+
+def bf16r(t):
+    return t.to(torch.bfloat16).to(torch.float64)
+
+
+def rel_max(got, want):
+    return ((got.double().cpu() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def rel_frob(got, want):
+    return ((got.double().cpu() - want).norm() / want.norm().clamp_min(1e-30)).item()
+
+
+def reference(q, k, v, nb, s, h, scale):
+    """q, k [T, h dq], v [T, h dv] fp64 leaves -> out [T, h dv], lse [nb, h, s]; causal softmax per (batch, head)."""
+    dq, dv = q.shape[1] // h, v.shape[1] // h
+    q4, k4, v4 = q.view(nb, s, h, dq), k.view(nb, s, h, dq), v.view(nb, s, h, dv)
+    scores = torch.einsum("bqhd,bkhd->bhqk", q4, k4) * scale
+    mask = torch.ones(s, s, dtype=torch.bool).tril()
+    scores = scores.masked_fill(~mask, float("-inf"))
+    lse = torch.logsumexp(scores, dim=-1)
+    out = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(scores, dim=-1), v4)
+    return out.reshape(nb * s, h * dv), lse
+
+
+def make_case(nb, s, h, dq, dv, seed, with_bias):
+    g = torch.Generator().manual_seed(seed)
+    T = nb * s
+    q = bf16r(torch.randn(T, h * dq, generator=g))
+    k = bf16r(torch.randn(T, h * dq, generator=g))
+    v = bf16r(torch.randn(T, h * dv, generator=g))
+    dout = bf16r(torch.randn(T, h * dv, generator=g))
+    if with_bias:
+        bq, bk, bv = (0.3 * torch.randn(h * dq, generator=g), 0.3 * torch.randn(h * dq, generator=g), 0.3 * torch.randn(h * dv, generator=g))
+    else:
+        bq = bk = bv = None
+    return q, k, v, dout, bq, bk, bv
+
+
+CASES = [
+    # nb, seq, heads, d_qk, d_v, bias
+    (2, 64, 2, 32, 32, False),
+    (1, 40, 3, 32, 64, True),          # ragged: one partial block
+    (2, 72, 2, 64, 64, False),         # ragged second block
+    (1, 200, 2, 64, 128, True),        # the benchmark's head widths, four blocks, ragged tail
+    (3, 128, 4, 64, 128, False),
+    (1, 8, 1, 64, 32, True),           # shortest sequence the kernels take
+]
+
+
+@pytest.mark.parametrize("nb,s,h,dq,dv,with_bias", CASES)
+def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv, with_bias):
+    print(f"attention case nb={nb} seq={s} heads={h} d_qk={dq} d_v={dv} bias={with_bias}", flush=True)
+    q, k, v, dout, bq, bk, bv = make_case(nb, s, h, dq, dv, seed=100 + s + dq + dv, with_bias=with_bias)
+    scale = 1.0 / math.sqrt(dq)
+    # what the kernel sees after it has added the biases: bf16(bf16 operand + fp32 bias)
+    eff = lambda t, b: t if b is None else bf16r((t.float() + b).double())     # noqa: E731
+    ql, kl, vl = (eff(q, bq).requires_grad_(), eff(k, bk).requires_grad_(), eff(v, bv).requires_grad_())
+    want_out, want_lse = reference(ql, kl, vl, nb, s, h, scale)
+    (want_out * dout).sum().backward()
+
+    to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
+    gq, gk, gv, gdo = to_dev(q), to_dev(k), to_dev(v), to_dev(dout)
+    gvt = gv.t().contiguous()
+    bias_dev = [None if b is None else b.to(dev) for b in (bq, bk, bv)]
+    out, lse = pkg.ops.attention_fwd(gq, gk, gvt, nb, s, h, scale, *bias_dev)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (nb * s, h * dv)
+    assert rel_max(out, want_out.detach()) < OUT_TOL, rel_max(out, want_out.detach())
+    assert (lse.double().cpu() - want_lse.detach()).abs().max().item() < LSE_TOL * max(1.0, want_lse.abs().max().item())
+
+    dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(), lse,
+                                          nb, s, h, scale, *bias_dev)
+    torch.cuda.synchronize()
+    errs = {"dq": (rel_max(dqt.t(), ql.grad), rel_frob(dqt.t(), ql.grad)),
+            "dk": (rel_max(dkt.t(), kl.grad), rel_frob(dkt.t(), kl.grad)),
+            "dv": (rel_max(dvt.t(), vl.grad), rel_frob(dvt.t(), vl.grad))}
+    assert all(e[0] < GRAD_TOL and e[1] < GRAD_TOL / 2 for e in errs.values()), errs
+
+
+def test_attention_is_causal_and_sequences_do_not_mix(pkg, dev):
+    """Changing a later position, or another sequence of the batch, leaves every earlier output bit-identical."""
+    nb, s, h, dq, dv = 2, 96, 2, 64, 128
+    q, k, v, _, _, _, _ = make_case(nb, s, h, dq, dv, seed=7, with_bias=False)
+    to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
+    gq, gk, gv = to_dev(q), to_dev(k), to_dev(v)
+    out0, lse0 = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, 0.125)
+    cut = 50
+    gk2, gv2 = gk.clone(), gv.clone()
+    gk2[cut:s] = 3.0          # later positions of sequence 0
+    gv2[cut:s] = -2.0
+    gk2[s + 10:] = 1.5        # and a stretch of sequence 1
+    out1, lse1 = pkg.ops.attention_fwd(gq, gk2, gv2.t().contiguous(), nb, s, h, 0.125)
+    assert torch.equal(out0[:cut], out1[:cut]) and torch.equal(lse0[0, :, :cut], lse1[0, :, :cut])
+    assert torch.equal(out0[s:s + 10], out1[s:s + 10])
+    assert not torch.equal(out0[cut:s], out1[cut:s])
+    # the first position attends to itself only
+    assert torch.equal(out0[0].float(), gv[0].float())
+
+
+def test_attention_rejects_shapes_it_is_not_built_for(pkg, dev):
+    z = torch.zeros(16, 48, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="d_qk"):
+        pkg.ops.attention_fwd(z, z, z.t().contiguous(), 1, 16, 1, 1.0)          # d_qk = 48
+    z = torch.zeros(12, 32, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        pkg.ops.attention_fwd(z, z, z.t().contiguous(), 1, 12, 1, 1.0)
+    assert not pkg.ops.attention_shapes_supported(12, 32, 32) and pkg.ops.attention_shapes_supported(1024, 64, 128)
+
+
+def test_row_sum(pkg, dev):
+    g = torch.Generator().manual_seed(3)
+    src = torch.randn(37, 1000, generator=g)
+    assert rel_max(pkg.ops.row_sum(src.to(dev)), src.double().sum(1)) < 1e-6
+    b = src.to(torch.bfloat16)
+    assert rel_max(pkg.ops.row_sum(b.to(dev)), b.double().sum(1)) < 1e-6

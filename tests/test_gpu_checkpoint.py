@@ -96,40 +96,59 @@ def test_trainer_resumes_bit_identically_from_a_complete_checkpoint(pkg, dev, tm
         assert float(a["step"]) == float(b["step"]) == 5.0
 
 
-def test_torch_adam_state_continues_on_hip_adam(pkg, oracle, dev):
-    """Optimizer state written by torch.optim.Adam on the reference layout (the oracle model, W_E moments [d, F]
-    contiguous) is loaded into HipAdam; both then take the same two steps and stay together."""
+def test_adam_state_round_trip_through_torch_adam_continues_bit_identically(pkg, oracle, dev):
+    """HipAdam's state after two steps is exported, loaded into a torch.optim.Adam over reference-layout parameters
+    (the oracle model: W_E and its moments [d, F] contiguous), exported from there and loaded into a second HipAdam
+    on a copy of the weights.  Both HIP models then take the same two steps: parameters and moments stay identical
+    to the bit, and torch's Adam accepts the state (it takes a step of its own on the oracle from it)."""
     from lm_saes_amd import synthetic
 
     d, F, k, B = 128, 1024, 8, 96
     x = synthetic.activations(B, d, 8, seed=43)
     w = synthetic.sae_weights(d, F, x, seed=43)
+
+    def fresh(weights):
+        cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                            top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
+        m = pkg.SparseAutoEncoder(cfg)
+        m.load_state_dict(weights)
+        return m, pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
+
+    def steps(m, opt, n):
+        for _ in range(n):
+            m.compute_loss(batch, return_aux_data=False).backward()
+            opt.step(); opt.zero_grad()
+
+    batch = {"in": x.to(dev), "out": x.to(dev), "tokens": torch.zeros(B, device=dev)}
+    a, opt_a = fresh(dict(zip(("W_E", "b_E", "W_D", "b_D"), [t.to(dev) for t in w])))
+    steps(a, opt_a, 2)
+    # -> torch.optim.Adam on the oracle (reference layout), by parameter name
     ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k)
-    synthetic.load_weights(ref, *w)
+    ref.load_state_dict({n: p.detach().cpu().contiguous() for n, p in a.named_parameters()})
     ropt = oracle.make_adam(ref, lr=1e-3)
-    cpu_batch = {"in": x, "out": x, "tokens": torch.zeros(B)}
-    for _ in range(2):
-        oracle.train_step(ref, ropt, cpu_batch)
-    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
-                        top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
-    sae = pkg.SparseAutoEncoder(cfg)
-    sae.load_state_dict({n: p.detach().to(dev) for n, p in ref.named_parameters()})
-    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=1e-3, model=sae)
-    # the oracle's parameter order is the module's: map its state onto HipAdam's parameters by name
-    order = {id(p): i for i, p in enumerate(opt.param_groups[0]["params"])}
-    by_name = dict(sae.named_parameters())
-    sd = ropt.state_dict()
-    ref_idx = {id(p): i for i, p in enumerate(q for g in ropt.param_groups for q in g["params"])}
-    state = {order[id(by_name[n])]: sd["state"][ref_idx[id(p)]] for n, p in ref.named_parameters()}
-    opt.load_state_dict({"state": state, "param_groups": opt.state_dict()["param_groups"]})
-    assert opt.state[sae.W_E]["exp_avg"].stride() == sae.W_E.stride()
-    batch = {k_: v.to(dev) for k_, v in cpu_batch.items()}
-    for _ in range(2):
-        loss = sae.compute_loss(batch, return_aux_data=False)
-        loss.backward(); opt.step(); opt.zero_grad()
-        oracle.train_step(ref, ropt, cpu_batch)
-    for n, p in ref.named_parameters():
-        got = by_name[n].detach().cpu()
-        assert (got - p.detach()).abs().max() <= 2e-2 * 2e-3 + 1e-6 * p.detach().abs().max(), n
-        m_ref = ropt.state[p]["exp_avg"]
-        assert (opt.state[by_name[n]]["exp_avg"].cpu() - m_ref).abs().max() <= 1e-4 * m_ref.abs().max() + 1e-9, n
+    names_a = {id(p): n for n, p in a.named_parameters()}
+    names_r = {id(p): n for n, p in ref.named_parameters()}
+    order_a = [names_a[id(p)] for g in opt_a.param_groups for p in g["params"]]
+    order_r = [names_r[id(p)] for g in ropt.param_groups for p in g["params"]]
+    sd_a = opt_a.state_dict()
+    by_name = {order_a[i]: st for i, st in sd_a["state"].items()}
+    assert by_name["W_E"]["exp_avg"].is_contiguous() and tuple(by_name["W_E"]["exp_avg"].shape) == (d, F)
+    ropt.load_state_dict({"state": {i: by_name[n] for i, n in enumerate(order_r)}, "param_groups": ropt.state_dict()["param_groups"]})
+    assert all(float(ropt.state[p]["step"]) == 2.0 for p in ref.parameters())
+    # <- and back into a second HipAdam
+    sd_r = ropt.state_dict()
+    back = {order_r[i]: st for i, st in sd_r["state"].items()}
+    b, opt_b = fresh({n: p.detach().clone() for n, p in a.named_parameters()})
+    order_b = [{id(p): n for n, p in b.named_parameters()}[id(p)] for g in opt_b.param_groups for p in g["params"]]
+    opt_b.load_state_dict({"state": {i: back[n] for i, n in enumerate(order_b)}, "param_groups": opt_b.state_dict()["param_groups"]})
+    assert opt_b.state[b.W_E]["exp_avg"].stride() == b.W_E.stride()
+    steps(a, opt_a, 2); steps(b, opt_b, 2)
+    torch.cuda.synchronize()
+    for (n, p), q in zip(a.named_parameters(), b.parameters()):
+        assert torch.equal(p, q), n
+        assert torch.equal(opt_a.state[p]["exp_avg"], opt_b.state[q]["exp_avg"]), n
+        assert torch.equal(opt_a.state[p]["exp_avg_sq"], opt_b.state[q]["exp_avg_sq"]), n
+        assert float(opt_a.state[p]["step"]) == float(opt_b.state[q]["step"]) == 4.0
+    before = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    oracle.train_step(ref, ropt, {"in": x, "out": x, "tokens": torch.zeros(B)})
+    assert all(torch.isfinite(p).all() and not torch.equal(p.detach(), before[n]) for n, p in ref.named_parameters())

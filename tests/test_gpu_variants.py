@@ -69,10 +69,10 @@ def check_bf16_grads_on_the_kernels_selection(model, ref, run_ref, kept_cpu):
     errs = {}
     for n, p in model.named_parameters():
         assert p.grad is not None and tuple(p.grad.shape) == tuple(p.shape), n
-        if rp[n].grad.abs().max().item() < 1e-4 * scale:
-            continue     # analytically zero: rounding noise on both sides
+        if rp[n].grad.abs().max().item() < 1e-2 * scale:
+            continue     # analytically zero (a key bias shifts a softmax row alike) or below the bf16 noise of the step
         errs[n] = rel_err(p.grad, rp[n].grad)
-    assert all(e < BF16_TOL for e in errs.values()), errs
+    assert all(e < BF16_TOL for e in errs.values()), sorted(errs.items(), key=lambda kv: -kv[1])[:4]
     return want
 
 
@@ -360,14 +360,26 @@ def test_lorsa_fused_step_fp32(pkg, vo, dev, kw):
     check_grads(m, ref)
 
 
-def test_lorsa_fused_step_bf16(pkg, vo, dev):
-    d, F, h, dq, s, b, k = 64, 512, 4, 16, 32, 2, 8
-    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, 32, k, seed=53, positional_embedding_type="none")
+@pytest.mark.parametrize("d,F,h,dq,s,b", [(64, 512, 4, 32, 32, 2),      # value width 128, one block
+                                          (64, 256, 4, 64, 96, 2),      # width 64 / 64, a ragged second block
+                                          (128, 256, 8, 32, 64, 3)])    # value width 32
+def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b):
+    """bf16 autocast: projections on the GEMM kernel, causal mixing and its backward on the attention kernels."""
+    k = 8
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=53, positional_embedding_type="none")
     g = torch.Generator().manual_seed(54)
+    with torch.no_grad():      # non-zero projection biases, so that the kernels' bias path is exercised
+        for n in ("b_Q", "b_K", "b_V"):
+            getattr(ref, n).copy_(0.2 * torch.randn(getattr(ref, n).shape, generator=g))
+    copy_params(m, ref)
     batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
     gb = {k_: v.to(dev) for k_, v in batch.items()}
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
     with torch.autocast("cuda", dtype=torch.bfloat16):
         out = m.compute_loss(gb)
+    pkg.ops.set_kernel_timer(None)
+    assert "attention_fwd" in timer.records, "the attention kernel did not run"
     want = ref.compute_loss(batch)
     assert rel_err(out["loss"], want["loss"]) < BF16_TOL
     out["loss"].backward()
