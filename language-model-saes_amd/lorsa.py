@@ -85,9 +85,9 @@ class _ProjectAndMix(torch.autograd.Function):
     forward : q = x W_Q, k = x W_K as [T, h dq] (natural), v^T = W_V x^T as [F, T] (the GEMM with its operands swapped
               yields the transposed layout the mixing product contracts over); the biases are added as the attention
               kernel loads its operands.
-    backward: the transposed copies q^T, k^T (swapped GEMMs), v (GEMM), dout^T (cast-transpose kernel); the attention
-              backward returns dq^T, dk^T, dv^T [., T], which are exactly the operands of the weight-gradient products
-              dW = d(.)^T x over the token axis; bias gradients are their row sums."""
+    backward: the transposed copies q^T, k^T, v, dout^T (cast-transpose kernel); the attention backward returns
+              dq^T, dk^T, dv^T [., T] in one buffer, which is exactly the operand of the weight-gradient product
+              dW = d(.)^T x over the token axis (one GEMM for the three); bias gradients are its row sums."""
 
     @staticmethod
     def forward(ctx, x2, W_Q, W_K, W_V, b_Q, b_K, b_V, model, seq):
@@ -101,7 +101,7 @@ class _ProjectAndMix(torch.autograd.Function):
         vt = ops.encoder_gemm(wv, x_op, torch.bfloat16)                     # [F, T]
         scale = 1.0 / model.attn_scale
         out, lse = ops.attention_fwd(q, k, vt, n_batch, seq, h, scale, b_Q, b_K, b_V)
-        ctx.save_for_backward(x_op, wq, wk, wv, q, k, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
+        ctx.save_for_backward(x_op, wq, wk, wv, q, k, vt, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
         ctx.dims = (n_batch, seq, h, scale)
         ctx.shapes = (tuple(W_Q.shape), tuple(W_K.shape))
         ctx.x_dtype = x2.dtype
@@ -109,28 +109,31 @@ class _ProjectAndMix(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dz):
-        x_op, wq, wk, wv, q, k, out, lse, b_Q, b_K, b_V = ctx.saved_tensors
+        x_op, wq, wk, wv, q, k, vt, out, lse, b_Q, b_K, b_V = ctx.saved_tensors
         n_batch, seq, h, scale = ctx.dims
         dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
-        qt = ops.encoder_gemm(wq, x_op, torch.bfloat16)                     # [h dq, T]
-        kt = ops.encoder_gemm(wk, x_op, torch.bfloat16)
-        v = ops.encoder_gemm(x_op, wv, torch.bfloat16)                      # [T, F]
+        qt, kt, v = ops.transpose_to_bf16(q)[0], ops.transpose_to_bf16(k)[0], ops.transpose_to_bf16(vt)[0]
         dzt = ops.transpose_to_bf16(dz)[0]                                  # [F, T]
-        dqt, dkt, dvt = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale, b_Q, b_K, b_V)
+        dqt, dkt, dvt, stacked = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale, b_Q, b_K, b_V,
+                                                   return_stacked=True)
         xt = ops.transpose_to_bf16(x_op)[0]                                 # [d, T]
         d = x_op.shape[1]
-        dq_w = q.shape[1] // h
+        n_qk = q.shape[1]
+        dq_w = n_qk // h
+        # the three weight gradients d(.)^T x in one product over the token axis: the gradients share one buffer
+        # [2 h dq + F, T], and a single launch fills the chip where three would each leave most of it idle
+        rows = ops.encoder_gemm(stacked, xt, torch.float32)                 # [2 h dq + F, d]
+        sums = ops.row_sum(stacked)
 
-        def qk_weight_grad(gt, shape):
-            rows = ops.encoder_gemm(gt, xt, torch.float32)                  # [h dq, d] = d(.)^T x
-            return rows.view(h, dq_w, d).permute(0, 2, 1).contiguous().view(shape)
+        def qk_weight_grad(part, shape):
+            return part.view(h, dq_w, d).permute(0, 2, 1).contiguous().view(shape)
 
-        dW_Q = qk_weight_grad(dqt, ctx.shapes[0]) if ctx.needs_input_grad[1] else None
-        dW_K = qk_weight_grad(dkt, ctx.shapes[1]) if ctx.needs_input_grad[2] else None
-        dW_V = ops.encoder_gemm(dvt, xt, torch.float32) if ctx.needs_input_grad[3] else None
-        db_Q = ops.row_sum(dqt).view(b_Q.shape) if ctx.needs_input_grad[4] else None
-        db_K = ops.row_sum(dkt).view(b_K.shape) if ctx.needs_input_grad[5] else None
-        db_V = ops.row_sum(dvt).view(b_V.shape) if ctx.needs_input_grad[6] else None
+        dW_Q = qk_weight_grad(rows[:n_qk], ctx.shapes[0]) if ctx.needs_input_grad[1] else None
+        dW_K = qk_weight_grad(rows[n_qk: 2 * n_qk], ctx.shapes[1]) if ctx.needs_input_grad[2] else None
+        dW_V = rows[2 * n_qk:] if ctx.needs_input_grad[3] else None
+        db_Q = sums[:n_qk].view(b_Q.shape) if ctx.needs_input_grad[4] else None
+        db_K = sums[n_qk: 2 * n_qk].view(b_K.shape) if ctx.needs_input_grad[5] else None
+        db_V = sums[2 * n_qk:].view(b_V.shape) if ctx.needs_input_grad[6] else None
         dx = None
         if ctx.needs_input_grad[0]:
             # rare (activations do not carry gradients in training): library products on the transposed gradients

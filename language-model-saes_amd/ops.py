@@ -787,9 +787,10 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, vt: torch.Tensor, n_batch: i
 def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
                   dout: torch.Tensor, doutt: torch.Tensor, lse: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
                   q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
-                  v_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                  v_bias: Optional[torch.Tensor] = None, return_stacked: bool = False):
     """Backward of attention_fwd -> (dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T]) in bf16, transposed layout.
-    q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout."""
+    q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout.  The three are row blocks of one
+    buffer [n_heads * (2 d_qk + d_v), T], returned as a fourth value with `return_stacked`."""
     T = n_batch * seq
     d_qk, d_v = q.shape[1] // n_heads, v.shape[1] // n_heads
     for name, t, shape in (("q", q, (T, n_heads * d_qk)), ("k", k, (T, n_heads * d_qk)), ("qt", qt, (n_heads * d_qk, T)),
@@ -801,16 +802,16 @@ def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.
         raise ValueError("lse must be [n_batch, n_heads, seq]")
     bq, bk, bv = _att_bias("q_bias", q_bias, n_heads * d_qk), _att_bias("k_bias", k_bias, n_heads * d_qk), _att_bias("v_bias", v_bias, n_heads * d_v)
     dev = q.device
-    dqt = torch.empty(n_heads * d_qk, T, dtype=torch.bfloat16, device=dev)
-    dkt = torch.empty(n_heads * d_qk, T, dtype=torch.bfloat16, device=dev)
-    dvt = torch.empty(n_heads * d_v, T, dtype=torch.bfloat16, device=dev)
+    # one buffer, so that a caller can also treat the three gradients as one [2 h d_qk + h d_v, T] matrix
+    grads = torch.empty(n_heads * (2 * d_qk + d_v), T, dtype=torch.bfloat16, device=dev)
+    dqt, dkt, dvt = grads[: n_heads * d_qk], grads[n_heads * d_qk: 2 * n_heads * d_qk], grads[2 * n_heads * d_qk:]
     dvec = torch.empty(n_batch * n_heads * seq, dtype=torch.float32, device=dev)
     with _timed("attention_bwd"):
         check(_lib.load().sae_attention_bwd(q.data_ptr(), qt.data_ptr(), k.data_ptr(), kt.data_ptr(), v.data_ptr(), out.data_ptr(),
                                             dout.data_ptr(), doutt.data_ptr(), _ptr(bq), _ptr(bk), _ptr(bv), lse.data_ptr(), n_batch,
                                             seq, n_heads, d_qk, d_v, float(scale), dvec.data_ptr(), dqt.data_ptr(), dkt.data_ptr(),
                                             dvt.data_ptr(), _stream(q)), "attention_bwd")
-    return dqt, dkt, dvt
+    return (dqt, dkt, dvt, grads) if return_stacked else (dqt, dkt, dvt)
 
 
 def row_sum(src: torch.Tensor) -> torch.Tensor:

@@ -66,6 +66,8 @@ CASES = [
     (1, 200, 2, 64, 128, True),        # the benchmark's head widths, four blocks, ragged tail
     (3, 128, 4, 64, 128, False),
     (1, 8, 1, 64, 32, True),           # shortest sequence the kernels take
+    (2, 136, 4, 64, 128, True),        # 8 (sequence, head) pairs: the XCD-aware workgroup order, ragged tail
+    (4, 72, 4, 32, 64, False),         # 16 pairs
 ]
 
 
