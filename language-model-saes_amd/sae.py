@@ -374,9 +374,29 @@ class _FusedSparseStep(torch.autograd.Function):
         return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
+def _transposed(t: torch.Tensor) -> torch.Tensor:
+    """[r, c] -> contiguous [c, r] in the same dtype (bf16 or fp32) through the transpose kernels."""
+    t = t.contiguous()
+    return ops.transpose_to_bf16(t)[0] if t.dtype == torch.bfloat16 else ops.transpose(t)
+
+
+def _gemm_k_ok(k: int, dtype: torch.dtype) -> bool:
+    """Whether the GEMM kernel takes a contraction of length k for this operand dtype."""
+    return k % (64 if dtype == torch.bfloat16 else 32) == 0
+
+
+def _rows_over_tokens(left: torch.Tensor, right: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """left^T @ right for left [B, m], right [B, n] -> [m, n]: a product over the token axis (a weight gradient).  The
+    GEMM kernel contracts over the contiguous axis of both operands, so both are transposed first."""
+    if _gemm_k_ok(left.shape[0], left.dtype):
+        return ops.encoder_gemm(_transposed(left), _transposed(right), out_dtype)
+    return (left.t() @ right).to(out_dtype)       # a token count the kernel's K granule does not divide
+
+
 class _EncoderGemm(torch.autograd.Function):
     """pre = x @ W_E through the GEMM kernel, for activations whose output is dense (JumpReLU): the incoming
-    gradient is then dense as well and both backward products are plain library GEMMs."""
+    gradient is then dense as well, and the weight gradient d(pre)^T x is a product over the token axis on the same
+    kernel."""
 
     @staticmethod
     def forward(ctx, x, W_E, w_op, amp, defer=False):
@@ -396,10 +416,11 @@ class _EncoderGemm(torch.autograd.Function):
     def backward(ctx, g):
         x_op, w_op = ctx.saved_tensors
         gg = g.to(w_op.dtype)
+        # the input's gradient is rarely wanted (activations carry none in training): a library product
         dx = (gg @ w_op).to(ctx.x_dtype) if ctx.needs_input_grad[0] else None
         dW = None
         if ctx.needs_input_grad[1]:
-            rows = gg.t() @ x_op                                                   # [F, d]
+            rows = _rows_over_tokens(gg, x_op, w_op.dtype)                         # [F, d]
             if ctx.param is not None:
                 _leave_lowp_grad(ctx.param, rows)
             else:
@@ -439,28 +460,31 @@ class _RowNormDeferred(torch.autograd.Function):
 
 
 class _DenseDecode(torch.autograd.Function):
-    """acts @ W_D on the bf16 copy of W_D that the optimiser maintains, so that autocast's per-step cast of the
-    fp32 master (and its backward) is not run; the products are those of an autocast matmul (models/sae.py:367)."""
+    """acts @ W_D for dense activations on the GEMM kernel (models/sae.py:367).  `w_op` is W_D [F, d] as the kernels
+    read it (under autocast the bf16 copy the optimiser maintains, so that the per-step cast of the fp32 master and
+    its backward are not run), `w_t` the same matrix transposed [d, F]: the forward product contracts over features.
+    Backward: d acts = g W_D^T contracts over d_model (W_D as it is), dW_D = acts^T g over the tokens."""
 
     @staticmethod
-    def forward(ctx, acts, W_D, w_op, defer=False):
+    def forward(ctx, acts, W_D, w_op, w_t, defer=False):
+        acts = acts.contiguous()
         ctx.save_for_backward(acts, w_op)
-        ctx.param = W_D if (defer and W_D.is_contiguous()) else None
-        return acts @ w_op
+        ctx.param = W_D if (defer and W_D.is_contiguous() and w_op.dtype == torch.bfloat16) else None
+        return ops.encoder_gemm(acts, w_t, acts.dtype)
 
     @staticmethod
     def backward(ctx, g):
         acts, w_op = ctx.saved_tensors
-        gg = g.to(w_op.dtype)
-        d_acts = gg @ w_op.t() if ctx.needs_input_grad[0] else None
+        gg = g.to(w_op.dtype).contiguous()
+        d_acts = ops.encoder_gemm(gg, w_op, w_op.dtype) if ctx.needs_input_grad[0] else None
         dW = None
         if ctx.needs_input_grad[1]:
-            rows = acts.t() @ gg                                                   # [F, d] bf16
+            rows = _rows_over_tokens(acts, gg, w_op.dtype)                         # [F, d]
             if ctx.param is not None:
                 _leave_lowp_grad(ctx.param, rows)
             else:
                 dW = rows.float()
-        return d_acts, dW, None, None
+        return d_acts, dW, None, None, None
 
 
 class _JumpReLUStep(torch.autograd.Function):
@@ -545,6 +569,11 @@ class SparseAutoEncoder(SparseDictionary):
         if not amp or w.dtype == torch.bfloat16:
             return w
         return self._derive("W_D.bf16", self.W_D, lambda old: ops.cast_bf16(w, old))
+
+    def _w_dec_t_operand(self, amp: bool) -> torch.Tensor:
+        """W_D^T [d, F] in the operand dtype: what a dense `acts @ W_D` on the GEMM kernel contracts against."""
+        w = self._w_dec_operand(amp)
+        return self._derive("W_D.t.bf16" if w.dtype == torch.bfloat16 else "W_D.t.f32", self.W_D, lambda old: _transposed(w))
 
     def _decoder_norm_nograd(self) -> torch.Tensor:
         self.wait_pending_update()
@@ -684,8 +713,8 @@ class SparseAutoEncoder(SparseDictionary):
                      and self.cfg.d_model % 64 == 0))
         )
 
-    # ---- JumpReLU train-step loss: dense activations, so encoder kernel + one fused element-wise pass each way,
-    # with the dense decoder products left to the library GEMM ----
+    # ---- JumpReLU train-step loss: dense activations, so the GEMM kernel for all five dense products (two of them
+    # over the token axis, on transposed operands) + one fused element-wise pass each way ----
     def _jumprelu_eligible(self, x, label, sparsity_loss_type, auxk_coefficient) -> bool:
         amp = _autocast_dtype("cuda") == torch.bfloat16
         return (
@@ -712,8 +741,8 @@ class SparseAutoEncoder(SparseDictionary):
         acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
                                                      float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
                                                      want_tanh, want_lp)
-        if amp and acts.dtype == torch.bfloat16:
-            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(True), defer)
+        if _gemm_k_ok(self.cfg.d_sae, acts.dtype) and self.cfg.d_model % 8 == 0:
+            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(amp), self._w_dec_t_operand(amp), defer)
         else:
             reconstructed = acts @ self.W_D
         if self.cfg.use_decoder_bias:
