@@ -331,6 +331,18 @@ int sae_transpose_to_bf16(const void *src, int src_dtype, const float *mask, int
 int sae_code_to_dense(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
                       int64_t n_cols, float *dense_f32, void *dense_bf16, void *stream);
 
+/* ---- Dense feature activations -> sparse code ----------------------------------------------------------------
+ * The conversion in front of the sparse decoder kernels when a caller hands over a dense [B, F] activation matrix
+ * (fp32 or bf16): get_sparse_representation (kernels/kernels.py:14-58: nonzero, bincount, cumsum, scatter into a padded
+ * [B, nnz_max] pair) as two passes.
+ *   sae_dense_row_nnz: row_nnz[b] = #{f : dense[b, f] != 0}.
+ *   sae_dense_to_code: given row_off (int64 [B], e.g. the exclusive prefix sum of row_nnz), token b's non-zero entries
+ *     are written in ascending feature order to idx / val [capacity] from slot row_off[b] on; slots at or past
+ *     `capacity` are dropped.  (row_off, row_nnz, idx, val) is then a sparse code as the select entry points emit it. */
+int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_t F, int32_t *row_nnz, void *stream);
+int sae_dense_to_code(const void *dense, int dtype, int64_t B, int64_t F, const int64_t *row_off, int32_t *idx, float *val,
+                      int64_t capacity, void *stream);
+
 /* ---- Activation batches from a shuffle buffer -----------------------------------------------------------
  * dst[i, :] = cast(scale * src[row_idx[i], :]) for i < n_rows: one batch drawn from a token buffer that
  * stays where it is in HBM.  Replaces ActivationBuffer.shuffle / yield_batch

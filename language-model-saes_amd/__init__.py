@@ -29,7 +29,7 @@ from .lorsa import LowRankSparseAttention  # noqa: E402,F401
 
 __all__ += ["CrosscoderConfig", "CLTConfig", "LorsaConfig", "Crosscoder", "CrossLayerTranscoder", "LowRankSparseAttention"]
 
-from . import metrics  # noqa: E402,F401
+from . import kernels, metrics  # noqa: E402,F401
 from .activation import (  # noqa: E402,F401
     ActivationBatchler, ActivationTransformer, ActivationWriter, ActivationWriterConfig, BufferShuffleConfig,
     CachedActivationLoader, ChunkInfo, cached_activation_stream,

@@ -96,9 +96,28 @@ def _topk_mask_lowest_index(x_flat: torch.Tensor, k: int) -> torch.Tensor:
     return mask
 
 
+class _BatchTopKDense(torch.autograd.Function):
+    """Dense [B, F] -> dense [B, F] batch-wide TopK through the batch select kernel: the k_total largest positive
+    entries of the whole batch (ties -> lowest flattened index) keep their values and their gradient."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, k_total: int):
+        x2 = (x if x.dtype in (torch.float32, torch.bfloat16) else x.float()).contiguous()
+        code = ops.select_topk_batch(x2, None, None, min(int(k_total), x2.numel()))
+        ctx.code, ctx.in_dtype = code, x.dtype
+        return code.to_dense().to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        mask = ctx.code.to_dense() > 0
+        return (g * mask).to(ctx.in_dtype), None
+
+
 def batch_topk_dense(x: torch.Tensor, k_total: int) -> torch.Tensor:
-    """Keep the k_total largest positive entries of the whole [B, F] batch (ties -> lowest
-    flattened index).  Device-side sort; the BatchTopK select kernel replaces it on the hot path."""
+    """Keep the k_total largest positive entries of the whole [B, F] batch (ties -> lowest flattened index): the batch
+    select kernel on GPU tensors it takes (F <= 2^30), a stable sort elsewhere."""
+    if x.is_cuda and x.ndim == 2 and x.shape[1] <= 2 ** 30 and x.shape[0] <= 131072:
+        return _BatchTopKDense.apply(x, k_total)
     r = x * x.gt(0).to(x.dtype)
     with torch.no_grad():
         mask = _topk_mask_lowest_index(r.reshape(1, -1), k_total).reshape(r.shape)

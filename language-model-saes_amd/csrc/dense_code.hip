@@ -1,0 +1,132 @@
+// Dense [B, F] feature activations -> sparse code (the layout the select kernels emit), in two passes:
+// count the non-zeros of every token, then, given the row offsets, write each token's (feature, value) pairs in
+// ascending feature order.  What get_sparse_representation does with nonzero / bincount / cumsum / scatter
+// (kernels/kernels.py:14-58) before the sparse decoder kernels can run on a dense activation matrix.
+#include "common.h"
+
+namespace sae {
+
+template <bool BF16>
+__device__ __forceinline__ void load8(const void *__restrict__ row, int64_t col, int64_t F, float (&x)[8]) {
+  if constexpr (BF16) {
+    const uint16_t *r = reinterpret_cast<const uint16_t *>(row);
+    if (col + 8 <= F && ((F & 7) == 0)) {
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(r + col);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[2 * j] = __uint_as_float(w[j] << 16);
+        x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = col + j < F ? bf16_bits_to_f32(r[col + j]) : 0.f;
+    }
+  } else {
+    const float *r = reinterpret_cast<const float *>(row);
+    if (col + 8 <= F && ((F & 3) == 0)) {
+      const float4 a = *reinterpret_cast<const float4 *>(r + col), b = *reinterpret_cast<const float4 *>(r + col + 4);
+      x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = col + j < F ? r[col + j] : 0.f;
+    }
+  }
+}
+
+// one workgroup per token: row_nnz[b] = #{f : dense[b, f] != 0}
+template <bool BF16>
+__global__ __launch_bounds__(256) void dense_row_nnz_kernel(const void *__restrict__ dense, int64_t F, int32_t *__restrict__ row_nnz) {
+  __shared__ float red[4];
+  const int64_t b = blockIdx.x;
+  const char *row = reinterpret_cast<const char *>(dense) + b * F * (BF16 ? 2 : 4);
+  int cnt = 0;
+  for (int64_t col = (int64_t)threadIdx.x * 8; col < F; col += 256 * 8) {
+    float x[8];
+    load8<BF16>(row, col, F, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cnt += x[j] != 0.f;
+  }
+  const float total = block_sum<4>((float)cnt, red);     // exact: at most 2^24 non-zeros per row are countable this way
+  if (threadIdx.x == 0) row_nnz[b] = (int32_t)total;
+}
+
+// one workgroup per token: the non-zeros of the row, in ascending feature order, to idx / val from row_off[b] on
+template <bool BF16>
+__global__ __launch_bounds__(256) void dense_to_code_kernel(const void *__restrict__ dense, int64_t F, const int64_t *__restrict__ row_off,
+                                                            int32_t *__restrict__ idx, float *__restrict__ val, int64_t capacity) {
+  __shared__ int wave_tot[4];
+  const int64_t b = blockIdx.x;
+  const char *row = reinterpret_cast<const char *>(dense) + b * F * (BF16 ? 2 : 4);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t run = row_off[b];
+  for (int64_t base = 0; base < F; base += 256 * 8) {
+    const int64_t col = base + (int64_t)threadIdx.x * 8;
+    float x[8];
+    if (col < F) {
+      load8<BF16>(row, col, F, x);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = 0.f;
+    }
+    int cnt = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cnt += x[j] != 0.f;
+    int incl = cnt;                                   // inclusive prefix over the wave's lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    __syncthreads();                                  // the previous chunk's totals have been read
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int t = wave_tot[w];
+      before += w < wave ? t : 0;
+      total += t;
+    }
+    int64_t pos = run + before + incl - cnt;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (x[j] != 0.f) {
+        if (pos < capacity) {
+          idx[pos] = (int32_t)(col + j);
+          val[pos] = x[j];
+        }
+        ++pos;
+      }
+    }
+    run += total;
+  }
+}
+
+}  // namespace sae
+
+extern "C" int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_t F, int32_t *row_nnz, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(dense && row_nnz, SAE_ERR_INVALID_ARG, "dense_row_nnz: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < ((int64_t)1 << 31) && F < ((int64_t)1 << 31), SAE_ERR_INVALID_ARG, "dense_row_nnz: bad shape");
+  SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "dense_row_nnz: bad dtype");
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(dense_row_nnz_kernel<true>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_nnz);
+  else
+    hipLaunchKernelGGL(dense_row_nnz_kernel<false>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_nnz);
+  return check_launch("dense_row_nnz");
+}
+
+extern "C" int sae_dense_to_code(const void *dense, int dtype, int64_t B, int64_t F, const int64_t *row_off, int32_t *idx,
+                                 float *val, int64_t capacity, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(dense && row_off && idx && val, SAE_ERR_INVALID_ARG, "dense_to_code: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < ((int64_t)1 << 31) && F < ((int64_t)1 << 31) && capacity >= 0, SAE_ERR_INVALID_ARG,
+              "dense_to_code: bad shape");
+  SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "dense_to_code: bad dtype");
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(dense_to_code_kernel<true>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity);
+  else
+    hipLaunchKernelGGL(dense_to_code_kernel<false>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity);
+  return check_launch("dense_to_code");
+}

@@ -1,0 +1,142 @@
+"""The kernel operators of the reference's `kernels` package (src/llamascopium/kernels/__init__.py:1-6,
+kernels/entrypoints.py:16-90) on the HIP path: the sparse decoder product a model switches to with
+`cfg.use_triton_kernel` once its activations are sparse enough, and the encoder product whose backward goes sparse
+when the incoming gradient is.  Same call signatures; the Triton-named entry points are aliases, so code written
+against the reference keeps working.
+
+    decode_with_hip_spmm_kernel(feature_acts [.., d_sae], decoder_weight)  -> [.., d_model]
+    encode_with_hip_spmm_kernel(x [B, L, d], W_E [L, d, F], b_E [L, F], sparsity_threshold) -> [B, L, F]
+    get_sparse_representation(x [B, d_sae]) -> (indices [B, nnz_max] int64, values [B, nnz_max])
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+from . import ops
+
+
+def _autocast_bf16() -> bool:
+    return torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16
+
+
+def get_sparse_representation(x: torch.Tensor, pad_val: int = 0):
+    """kernels/kernels.py:14-58: the padded [B, nnz_max] index / value pair of a dense [B, d_sae] tensor (non-zeros of
+    each row in ascending column order, `pad_val` / 0 behind them; a batch without non-zeros gives [B, 1] of zeros).
+    The kernels here work on the packed sparse code (`ops.dense_to_code`); this form is kept for callers of the
+    reference's helper."""
+    code = ops.dense_to_code(x.contiguous() if x.dtype in (torch.float32, torch.bfloat16) else x.float().contiguous())
+    B = code.n_tokens
+    nnz_max = max(int(code.row_nnz.max().item()), 1)
+    pos = torch.arange(nnz_max, device=x.device)[None, :]
+    valid = pos < code.row_nnz[:, None]
+    src = (code.row_off[:, None] + pos).clamp_max(code.n_slots - 1)
+    indices = torch.where(valid, code.idx.long()[src], torch.full((B, nnz_max), pad_val, dtype=torch.long, device=x.device))
+    values = torch.where(valid, code.val[src], torch.zeros(B, nnz_max, device=x.device)).to(x.dtype)
+    return indices, values
+
+
+class _SparseDecode(torch.autograd.Function):
+    """out = feature_acts @ W for a dense feature_acts whose rows are mostly zero: dense -> sparse code -> gather of the
+    active decoder rows (TritonDecoderAutogradTopK's role, kernels/kernels.py:542-566).  Backward: the gradient of the
+    activations at their non-zero positions (zero elsewhere, as the reference masks it), and the decoder gradient rows
+    from the feature index of the code."""
+
+    @staticmethod
+    def forward(ctx, feature_acts, weight, w_op, capacity):
+        fa = feature_acts if feature_acts.dtype in (torch.float32, torch.bfloat16) else feature_acts.float()
+        code = ops.dense_to_code(fa.contiguous(), capacity)
+        ctx.code, ctx.w_op = code, w_op
+        ctx.in_dtype, ctx.w_dtype = feature_acts.dtype, weight.dtype
+        return ops.sparse_decode_fwd(code, w_op, None)
+
+    @staticmethod
+    def backward(ctx, g):
+        code, w_op = ctx.code, ctx.w_op
+        g = g.float().contiguous()
+        d_acts = d_w = None
+        if ctx.needs_input_grad[0]:
+            dval = ops.sparse_decode_bwd_dval(code, g, w_op)
+            d_acts = ops.code_to_dense(dataclasses.replace(code, val=dval), code.d_sae)[0].to(ctx.in_dtype)
+        if ctx.needs_input_grad[1]:
+            fi = ops.build_feature_index(code)
+            d_w = ops.sparse_grad_rows(fi, code.val, g, code.d_sae)[0].to(ctx.w_dtype)
+        return d_acts, d_w, None, None
+
+
+def decode_with_hip_spmm_kernel(feature_acts: torch.Tensor, decoder_weight: torch.Tensor, *,
+                                w_operand: Optional[torch.Tensor] = None, capacity: Optional[int] = None) -> torch.Tensor:
+    """kernels/entrypoints.py:16-40.  feature_acts [.., d_sae] dense (or a torch sparse COO tensor), decoder_weight
+    [d_sae, d_model]; the [d_model, d_sae] tensor the reference's own call site passes (`W_D.T.contiguous()`,
+    models/sae.py:363) is recognised by its shape and read as its transpose.  Returns feature_acts @ decoder_weight in
+    fp32.  `w_operand`: a prepared copy of the weight for the gather (e.g. the bf16 copy under autocast)."""
+    if feature_acts.is_sparse:
+        feature_acts = feature_acts.to_dense()
+    F = feature_acts.shape[-1]
+    if decoder_weight.shape[0] != F and decoder_weight.shape[-1] == F:
+        decoder_weight = decoder_weight.t()
+    if decoder_weight.shape[0] != F:
+        raise ValueError(f"decoder_weight {tuple(decoder_weight.shape)} does not match d_sae = {F}")
+    if w_operand is None:
+        w = decoder_weight.detach()
+        w_operand = w if w.is_contiguous() else w.contiguous()
+        if w_operand.dtype not in (torch.float32, torch.bfloat16):
+            w_operand = w_operand.float()
+    lead = feature_acts.shape[:-1]
+    out = _SparseDecode.apply(feature_acts.reshape(-1, F), decoder_weight, w_operand, capacity)
+    return out.view(*lead, out.shape[-1])
+
+
+class _EncodeLayer(torch.autograd.Function):
+    """x @ W_E + b_E on the GEMM kernel; in the backward pass, a gradient that is sparse enough (a TopK-family
+    activation passes on only its kept entries) goes through the sparse kernels: d x gathers the active encoder rows,
+    d W_E / d b_E come from the feature index of the gradient's code (TritonEncoderAutogradDynamicK,
+    kernels/kernels.py:439-539)."""
+
+    @staticmethod
+    def forward(ctx, x, W_E, b_E, sparsity_threshold):
+        amp = _autocast_bf16()
+        wt = W_E.detach().t()
+        wt = wt if wt.is_contiguous() else wt.contiguous()                      # [F, d]
+        if amp and wt.dtype == torch.float32:
+            x_op, w_op, out_dtype = ops.cast_bf16(x.float().contiguous()), ops.cast_bf16(wt), torch.bfloat16
+        else:
+            x_op, w_op, out_dtype = x.to(wt.dtype).contiguous(), wt, wt.dtype
+        pre = ops.encoder_gemm(x_op, w_op, out_dtype)
+        ctx.save_for_backward(x_op, w_op)
+        ctx.thr, ctx.x_dtype, ctx.w_dtype, ctx.b_dtype = float(sparsity_threshold), x.dtype, W_E.dtype, b_E.dtype
+        return pre + b_E
+
+    @staticmethod
+    def backward(ctx, g):
+        x_op, w_op = ctx.saved_tensors
+        g = g.contiguous()
+        sparse = (g == 0).float().mean().item() > ctx.thr       # the reference decides on the host as well
+        if sparse:
+            code = ops.dense_to_code(g if g.dtype in (torch.float32, torch.bfloat16) else g.float())
+            fi = ops.build_feature_index(code)
+            dx = ops.sparse_decode_fwd(code, w_op, None).to(ctx.x_dtype) if ctx.needs_input_grad[0] else None
+            rows, bias = ops.sparse_grad_rows(fi, code.val, x_op, code.d_sae, want_bias=True)
+            dW = rows.t().to(ctx.w_dtype) if ctx.needs_input_grad[1] else None
+            db = bias.to(ctx.b_dtype) if ctx.needs_input_grad[2] else None
+            return dx, dW, db, None
+        gg = g.to(w_op.dtype)
+        dx = (gg @ w_op).to(ctx.x_dtype) if ctx.needs_input_grad[0] else None
+        dW = (gg.t() @ x_op).t().to(ctx.w_dtype) if ctx.needs_input_grad[1] else None
+        db = g.float().sum(0).to(ctx.b_dtype) if ctx.needs_input_grad[2] else None
+        return dx, dW, db, None
+
+
+def encode_with_hip_spmm_kernel(x: torch.Tensor, W_E: torch.Tensor, b_E: torch.Tensor,
+                                sparsity_threshold: float = 0.996) -> torch.Tensor:
+    """kernels/entrypoints.py:43-90: "bld,lds->bls" layer by layer, + b_E."""
+    B, L, _ = x.shape
+    return torch.stack([_EncodeLayer.apply(x[:, l, :], W_E[l], b_E[l], sparsity_threshold) for l in range(L)], dim=1)
+
+
+# the reference's names
+decode_with_triton_spmm_kernel = decode_with_hip_spmm_kernel
+encode_with_triton_spmm_kernel = encode_with_hip_spmm_kernel

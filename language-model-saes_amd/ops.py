@@ -207,6 +207,37 @@ def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_b
     return f32, b16
 
 
+def dense_row_nnz(dense: torch.Tensor) -> torch.Tensor:
+    """int32 [B]: the number of non-zero entries of every row of a dense [B, F] matrix (fp32 or bf16)."""
+    _req(dense, "dense", ndim=2)
+    B, F = dense.shape
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dense.device)
+    with _timed("dense_row_nnz"):
+        check(_lib.load().sae_dense_row_nnz(dense.data_ptr(), _dt(dense), B, F, row_nnz.data_ptr(), _stream(dense)), "dense_row_nnz")
+    return row_nnz
+
+
+def dense_to_code(dense: torch.Tensor, capacity: Optional[int] = None) -> "SparseCode":
+    """Sparse code of a dense [B, F] activation matrix (fp32 or bf16): every token's non-zero entries in ascending
+    feature order, rows packed one after the other.  Without `capacity` the number of non-zeros is read back from the
+    device to size the code (one synchronisation, as the reference's `nnz_max.item()`); with it (an upper bound the
+    caller knows, e.g. k * B after a TopK activation) nothing is read back and entries past it would be dropped."""
+    _req(dense, "dense", ndim=2)
+    B, F = dense.shape
+    lib = _lib.load()
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dense.device)
+    with _timed("dense_to_code"):
+        check(lib.sae_dense_row_nnz(dense.data_ptr(), _dt(dense), B, F, row_nnz.data_ptr(), _stream(dense)), "dense_row_nnz")
+        incl = torch.cumsum(row_nnz, 0, dtype=torch.int64)
+        row_off = incl - row_nnz
+        cap = int(incl[-1].item()) if capacity is None else int(capacity)
+        idx = torch.zeros(max(cap, 1), dtype=torch.int32, device=dense.device)
+        val = torch.zeros(max(cap, 1), dtype=torch.float32, device=dense.device)
+        check(lib.sae_dense_to_code(dense.data_ptr(), _dt(dense), B, F, row_off.data_ptr(), idx.data_ptr(), val.data_ptr(), cap,
+                                    _stream(dense)), "dense_to_code")
+    return SparseCode(idx, val, row_off, row_nnz, B, F)
+
+
 def mse_auxk_fused(recon: torch.Tensor, label: torch.Tensor, aux_recon: Optional[torch.Tensor],
                    tok_w: Optional[torch.Tensor], alpha: float, want_bf16: bool = False):
     """-> (rec_tok [B], aux_tok [B] or None, g_aux [B, d] or None, grad_recon [B, d], grad_recon in bf16 or None):

@@ -407,7 +407,7 @@ class _EncoderGemm(torch.autograd.Function):
             x_op = x.float().contiguous()
             pre = ops.encoder_gemm(x_op, w_op, torch.float32)
         ctx.save_for_backward(x_op, w_op)
-        ctx.x_dtype = x.dtype
+        ctx.x_dtype, ctx.w_dtype = x.dtype, W_E.dtype
         # a bf16 weight gradient can stay bf16 until the optimiser reads it, when the parameter is stored feature-major
         ctx.param = W_E if (defer and amp and W_E.ndim == 2 and W_E.stride() == (1, W_E.shape[0])) else None
         return pre
@@ -424,7 +424,7 @@ class _EncoderGemm(torch.autograd.Function):
             if ctx.param is not None:
                 _leave_lowp_grad(ctx.param, rows)
             else:
-                dW = rows.t().float()                                              # [d, F] with feature-major strides
+                dW = rows.t().to(ctx.w_dtype)                                      # [d, F] with feature-major strides
         return dx, dW, None, None, None
 
 
@@ -647,6 +647,21 @@ class SparseAutoEncoder(SparseDictionary):
 
     # ---- API path over dense tensors (models/sae.py:288-377) ----
     def _matmul_enc(self, x: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
+        """x @ W for an encoder weight (W_E or the GLU gate): the GEMM kernel on GPU tensors whose shapes it takes,
+        with its weight gradient as a product over the token axis on the same kernel; a library product otherwise."""
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        d = W.shape[0]
+        if (x.is_cuda and W.is_cuda and W.ndim == 2 and x.shape[-1] == d and W.dtype in (torch.float32, torch.bfloat16)
+                and _gemm_k_ok(d, torch.bfloat16 if (amp or W.dtype == torch.bfloat16) else torch.float32)):
+            wt = W.detach().t()
+            wt = wt if wt.is_contiguous() else wt.contiguous()          # [F, d]; a view for feature-major weights
+            low = amp or wt.dtype == torch.bfloat16
+            if low and wt.dtype != torch.bfloat16:
+                name = "W_E.bf16" if W is self.W_E else ("W_E_glu.bf16" if W is getattr(self, "W_E_glu", None) else None)
+                wt = self._derive(name, W, lambda old: ops.cast_bf16(wt, old)) if name is not None else ops.cast_bf16(wt)
+            lead = x.shape[:-1]
+            pre = _EncoderGemm.apply(x.reshape(-1, d), W, wt, low)
+            return pre.view(*lead, pre.shape[-1])
         return x @ W
 
     def encode(self, x: torch.Tensor, return_hidden_pre: bool = False, **kwargs):
@@ -671,7 +686,20 @@ class SparseAutoEncoder(SparseDictionary):
             reconstructed = ops.sparse_decode_fwd(feature_acts, self._w_dec_operand(amp),
                                                   self.b_D.detach() if self.cfg.use_decoder_bias else None)
             return self.hook_reconstructed(reconstructed)
-        reconstructed = feature_acts @ self.W_D
+        reconstructed = None
+        if self.cfg.use_triton_kernel and feature_acts.is_cuda and self.cfg.d_model % 8 == 0 and self.W_D.dtype == torch.float32:
+            # models/sae.py:355-367: the sparse decoder kernel once every token's activations are sparse enough
+            # (and not all empty); the count is read on the host, as in the reference
+            from .kernels import decode_with_hip_spmm_kernel
+
+            fa2 = feature_acts.reshape(-1, feature_acts.shape[-1])
+            nnz = ops.dense_row_nnz((fa2 if fa2.dtype in (torch.float32, torch.bfloat16) else fa2.float()).contiguous())
+            max_l0 = int(nnz.max().item())
+            if 0 < max_l0 < self.cfg.d_sae * (1 - self.cfg.sparsity_threshold_for_triton_spmm_kernel):
+                amp = _autocast_dtype("cuda") == torch.bfloat16
+                reconstructed = decode_with_hip_spmm_kernel(feature_acts, self.W_D, w_operand=self._w_dec_operand(amp))
+        if reconstructed is None:
+            reconstructed = feature_acts @ self.W_D
         if self.cfg.use_decoder_bias:
             reconstructed = reconstructed + self.b_D
         return self.hook_reconstructed(reconstructed)

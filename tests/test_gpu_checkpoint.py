@@ -111,7 +111,10 @@ def test_adam_state_round_trip_through_torch_adam_continues_bit_identically(pkg,
         cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
                             top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
         m = pkg.SparseAutoEncoder(cfg)
-        m.load_state_dict(weights)
+        if isinstance(weights, dict):
+            m.load_state_dict(weights)
+        else:
+            synthetic.load_weights(m, *weights)
         return m, pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
 
     def steps(m, opt, n):
@@ -120,7 +123,7 @@ def test_adam_state_round_trip_through_torch_adam_continues_bit_identically(pkg,
             opt.step(); opt.zero_grad()
 
     batch = {"in": x.to(dev), "out": x.to(dev), "tokens": torch.zeros(B, device=dev)}
-    a, opt_a = fresh(dict(zip(("W_E", "b_E", "W_D", "b_D"), [t.to(dev) for t in w])))
+    a, opt_a = fresh([t.to(dev) for t in w])
     steps(a, opt_a, 2)
     # -> torch.optim.Adam on the oracle (reference layout), by parameter name
     ref = oracle.SAEOracle(d, F, act_fn="topk", top_k=k)
