@@ -63,7 +63,8 @@ def _pieces(sg):
 def _contiguous_moments(sd: dict) -> dict:
     """A state dict whose moments are contiguous in the parameter's logical shape.  The per-parameter dicts that
     Optimizer.state_dict() returns are the optimiser's live ones, so they are copied, not edited."""
-    sd["state"] = {i: {k: (v.contiguous() if k in ("exp_avg", "exp_avg_sq") and torch.is_tensor(v) else v)
+    sd["state"] = {i: {k: (v.contiguous() if k in ("exp_avg", "exp_avg_sq") and torch.is_tensor(v)
+                           else (v.clone() if torch.is_tensor(v) else v))
                        for k, v in st.items()} for i, st in sd["state"].items()}
     return sd
 
@@ -86,7 +87,9 @@ def _relayout_loaded_state(opt: Optimizer, step_on_device: bool) -> None:
                     laid.copy_(t)
                     st[k] = laid
             step = st.get("step", 0)
-            step = step.detach().float() if torch.is_tensor(step) else torch.tensor(float(step), dtype=torch.float32)
+            # a copy of its own: Optimizer.load_state_dict passes a `step` tensor through as it is, so two optimisers
+            # loaded from one in-memory state dict would otherwise count on the same tensor
+            step = step.detach().float().clone() if torch.is_tensor(step) else torch.tensor(float(step), dtype=torch.float32)
             st["step"] = step.reshape(1).to(prm.device) if step_on_device else step.reshape(()).cpu()
 
 

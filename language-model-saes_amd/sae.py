@@ -747,13 +747,14 @@ class SparseAutoEncoder(SparseDictionary):
         amp = _autocast_dtype("cuda") == torch.bfloat16
         return (
             self.cfg.act_fn.lower() == "jumprelu" and x.is_cuda and x.ndim == 2 and label.ndim == 2
-            and not self.cfg.use_glu_encoder and sparsity_loss_type in (None, "tanh") and not (auxk_coefficient > 0.0)
+            and not self.cfg.use_glu_encoder and sparsity_loss_type in (None, "tanh", "power", "tanh-quad")
+            and not (auxk_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
             and self.W_E.dtype == torch.float32 and self.cfg.d_sae % 8 == 0 and self.cfg.d_model % (64 if amp else 32) == 0
         )
 
     def _jumprelu_loss(self, batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient, lp_coefficient,
-                       auxk_coefficient, return_aux_data):
+                       auxk_coefficient, return_aux_data, frequency_scale: float = 0.01, p: int = 1):
         from .sparse_dictionary import apply_token_mask
 
         mask = batch.get("mask")
@@ -764,7 +765,8 @@ class SparseAutoEncoder(SparseDictionary):
         want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
         scaled = bool(self.cfg.sparsity_include_decoder_norm)
         n = None
-        if scaled or want_tanh or want_lp:
+        want_dense_pen = sparsity_loss_type in ("power", "tanh-quad")
+        if scaled or want_tanh or want_lp or want_dense_pen:
             n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), self if defer else None)
         acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
                                                      float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
@@ -781,6 +783,18 @@ class SparseAutoEncoder(SparseDictionary):
         if want_tanh:
             l_s = l1_coefficient * tanh_tok
             loss = loss + apply_token_mask(l_s, 1, mask, "mean")
+        elif want_dense_pen:
+            # models/sparse_dictionary.py:888-925.  The products of the step stay on the GEMM kernel; these two penalties
+            # are element-wise framework operations on the activations (their gradient joins the decoder's on the
+            # way into the activation kernel's backward, and reaches W_D through the norm as a per-row coefficient)
+            weighted = acts.float() * n
+            if sparsity_loss_type == "power":
+                l_s = torch.norm(weighted, p=p, dim=-1)
+            else:
+                freq = torch.tanh(tanh_stretch_coefficient * weighted).mean(dim=0)
+                l_s = (freq * (1 + freq / frequency_scale)).sum(dim=-1)
+            l_s = l1_coefficient * l_s
+            loss = loss + apply_token_mask(l_s, min(1, l_s.ndim), mask if l_s.ndim else None, "mean")
         if want_lp:
             l_p = apply_token_mask(lp_coefficient * lp_tok, 1, mask, "mean")
             loss = loss + l_p
@@ -802,7 +816,7 @@ class SparseAutoEncoder(SparseDictionary):
         label = self.prepare_label(batch, **kwargs)
         if self._jumprelu_eligible(x, label, sparsity_loss_type, auxk_coefficient):
             return self._jumprelu_loss(batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient,
-                                       lp_coefficient, auxk_coefficient, return_aux_data)
+                                       lp_coefficient, auxk_coefficient, return_aux_data, frequency_scale, p)
         if not self._fused_eligible(x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient):
             return super().compute_loss(
                 batch, sparsity_loss_type=sparsity_loss_type, tanh_stretch_coefficient=tanh_stretch_coefficient,

@@ -122,9 +122,15 @@ def test_sparsity_losses_match_the_oracle(pkg, oracle, dev, loss_type, kw, act_f
     batch = {"in": x, "out": x + 0.1 * torch.randn(x.shape, generator=g), "tokens": torch.zeros(x.shape[0], dtype=torch.long),
              "mask": (torch.rand(x.shape[0], generator=g) > 0.25).float()}
     args = dict(sparsity_loss_type=loss_type, l1_coefficient=0.05, tanh_stretch_coefficient=2.0, **kw)
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
     out = sae.compute_loss({k_: v.to(dev) for k_, v in batch.items()}, **args)
     want = ref.compute_loss(batch, **args)
     out["loss"].backward(); want["loss"].backward()
+    torch.cuda.synchronize()
+    pkg.ops.set_kernel_timer(None)
+    if act_fn == "jumprelu":    # the step's own route: activation kernel each way, five products on the GEMM kernel
+        assert {"jumprelu_fwd", "jumprelu_bwd"} <= set(timer.records) and len(timer.records["encoder_gemm"]) == 5, set(timer.records)
     for key in ("loss", "l_rec", "l_s", "feature_acts", "reconstructed"):
         assert rel_err(out[key], want[key]) < FP32_TOL, key
     got, exp = named_grads(sae), named_grads(ref)
