@@ -34,13 +34,35 @@ D_MODEL, D_SAE, TOP_K = 4096, 131072, 64
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# Measured HBM bytes per launch (fetched + written, in GB) of the default workload's kernels, from two
-# rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE) of this file, scaled by what the same counters read for
-# transfers of known size in the same runs: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this machine.
-HBM_TRAFFIC_GB = {
-    "encoder_gemm": 7.61, "adam_step_sparse_rows[f32 dense]": 18.14, "adam_step_sparse_rows[bf16 dense]": 16.00,
-    "sparse_decode_mse_fused": 4.38, "select_topk_row": 1.19,
-}
+# Measured HBM bytes per launch of the default workload's kernels are not typed in here: they are read from the table
+# "Scaled HBM traffic per launch" of the committed counter summary (two rocprofv3 runs, FETCH_SIZE and WRITE_SIZE, scaled
+# by what the same counters read for transfers of known size in the same runs).
+HBM_TRAFFIC_FILE = os.path.join("profiles", "train_step_topk_d4096_F131072_k64_B4096_hbm_counters.md")
+HBM_TRAFFIC_ROWS = {"encoder_gemm": "encoder_gemm", "adam_step_sparse_rows[f32 dense]": "adam_sparse_rows",
+                    "adam_step_sparse_rows[bf16 dense]": "adam_sparse_rows", "sparse_decode_mse_fused": "sparse_decode_mse_fused",
+                    "select_topk_row": "select_topk_row"}
+# launches that move so little that their duration is the launch / dependency latency, not a bandwidth
+LATENCY_BOUND = {"build_feature_index", "adam_step[vector]", "col_sum", "cast_f32_to_bf16", "code_stats", "recon_stats",
+                 "grad_sq_nnz", "gather_rows", "row_sum", "row_norm"}
+
+
+def measured_traffic_gb(kernel: str):
+    """Total HBM GB per launch of `kernel` from the committed counter summary, or None."""
+    label = HBM_TRAFFIC_ROWS.get(kernel)
+    path = os.path.join(ROOT, HBM_TRAFFIC_FILE)
+    if label is None or not os.path.exists(path):
+        return None
+    in_table = False
+    for line in open(path):
+        if line.startswith("## "):
+            in_table = line.startswith("## Scaled HBM traffic per launch")
+        elif in_table and line.startswith("| " + label):
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            try:
+                return float(cells[3])        # kernel | fetched GB | written GB | total GB | ...
+            except (IndexError, ValueError):
+                return None
+    return None
 
 
 def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
@@ -402,11 +424,9 @@ def mfma_probe() -> dict:
 
 
 def cpu_baseline(sample_batch: int, sample_features: int):
-    """Oracle (the reference's eager op sequence on CPU) on a bounded sample of the workload:
-    same d_model and k, `sample_features` of the 131072 dictionary features, `sample_batch` tokens.
-    Per-step CPU cost is close to linear in the number of features (GEMMs, [B, F] temporaries and
-    Adam all scale with F), so the full dictionary would take 131072 / sample_features times longer
-    per token; the reported value is the measured one, not an extrapolation."""
+    """Oracle (the reference's eager op sequence on CPU) on a bounded sample of the headline workload: the full
+    dictionary (d_model, d_sae, k as on the GPU), `sample_batch` tokens per step instead of 4096 (the host cannot
+    finish the full batch in the time a default run has); the reported value is measured, not extrapolated."""
     import torch
     from __graft_entry__ import load_oracle, load_package
 
@@ -425,16 +445,17 @@ def cpu_baseline(sample_batch: int, sample_features: int):
     batch = {"in": x, "out": x, "tokens": torch.zeros(sample_batch, dtype=torch.long)}
     opt = oracle.make_adam(m, lr=4e-4)
     oracle.train_step(m, opt, batch, amp_dtype=torch.bfloat16)  # warm-up (allocates Adam state)
-    # timed steps until about 12 s of CPU work have been spent (at least 2, at most 20)
+    # timed steps until about 12 s of CPU work have been spent (at least 3, at most 20)
     n_timed, t0 = 0, time.perf_counter()
-    while n_timed < 2 or (time.perf_counter() - t0 < 12.0 and n_timed < 20):
+    while n_timed < 3 or (time.perf_counter() - t0 < 12.0 and n_timed < 20):
         oracle.train_step(m, opt, batch, amp_dtype=torch.bfloat16)
         n_timed += 1
     dt = (time.perf_counter() - t0) / n_timed
     return {
         "value": round(sample_batch / dt, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
-        "sample": f"1 warm-up + {n_timed} timed steps of the TopK SAE train step at d_model={d} k={k} with {F} of the "
-                  f"{D_SAE} features (1/{D_SAE // F} of the dictionary) and B={sample_batch} tokens, fp32 master "
+        "sample": f"1 warm-up + {n_timed} timed steps of the TopK SAE train step at d_model={d} k={k} d_sae={F}"
+                  + ("" if F == D_SAE else f" ({F} of the {D_SAE} features)")
+                  + f" with B={sample_batch} tokens per step (the GPU step has 4096), fp32 master "
                   f"weights + bf16 autocast on CPU, torch {torch.__version__}, {dt:.2f} s per step",
     }
 
@@ -450,7 +471,8 @@ def main():
                     help="dictionary size of the topk workload (0: 131072, the headline; a smaller one keeps the 32-bit "
                          "hardware counters of a profiling run from saturating and is never the headline metric)")
     ap.add_argument("--cpu-sample-batch", type=int, default=512)
-    ap.add_argument("--cpu-sample-features", type=int, default=32768)
+    ap.add_argument("--cpu-sample-features", type=int, default=D_SAE,
+                    help="dictionary size of the CPU baseline (default: the full 131072 features)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
     ap.add_argument("--mfma-probe", action="store_true",
@@ -479,10 +501,11 @@ def main():
         achieved, peak, unit = per_launch / avg_ms / 1e9, PEAK_BF16_TFLOPS, "TFLOP/s"
     else:
         achieved, peak, unit = per_launch / avg_ms / 1e6, PEAK_HBM_GBS, "GB/s"
-    traffic = HBM_TRAFFIC_GB.get(dominant) if args.workload in ("topk", "topk_trainer") else None
+    traffic = measured_traffic_gb(dominant) if args.workload in ("topk", "topk_trainer") and not args.d_sae and not args.batch else None
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-        "frac": round(achieved / peak, 4), "traffic": None if traffic is None else traffic * 1e9, "avg_ms": round(avg_ms, 4),
+        "frac": round(achieved / peak, 4), "traffic": None if traffic is None else traffic * 1e9,
+        "traffic_source": None if traffic is None else HBM_TRAFFIC_FILE, "avg_ms": round(avg_ms, 4),
         "launches_per_step": kernels[dominant]["calls"] / args.steps,
     }
     per_kernel = {}
@@ -491,6 +514,8 @@ def main():
     uniform = args.workload in ("topk", "topk_bf16_params", "topk_trainer", "jumprelu", "activation_stream")
     for kname, st in kernels.items():
         bnd, w = work.get(kname, ("hbm", 0.0)) if uniform else ("hbm", 0.0)
+        if kname in LATENCY_BOUND:
+            bnd, w = "latency", 0.0
         rate = w / st["avg_ms"] / (1e9 if bnd == "mfma" else 1e6) if w else None
         per_kernel[kname] = {
             "ms_per_step": round(st["total_ms"] / args.steps, 4), "avg_ms": round(st["avg_ms"], 4),
@@ -516,6 +541,7 @@ def main():
     }
     if headline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, args.cpu_sample_features)
+        out["cpu_baseline_c1"] = cpu_baseline_c1()   # the configuration the reference's CPU path runs at full shape
     if args.workload == "c1_fp32" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_c1()
         out["dtype"] = "f32"
