@@ -242,6 +242,8 @@ int sae_adam_step(float *p, const void *g, int g_dtype, float *m, float *v, int6
  * share of the tokens; its rows come from three small GEMMs).  extra_map: device int32[F], -1 or the row of
  * extra_rows ([n, d] fp32, 16-byte aligned) that is added to feature f's gradient; extra_bias: fp32[n] added to
  * bias_grad_out likewise.
+ * row_grad_coef (nullable, fp32 [F]): as in sae_adam_step, the gradient of row f is g + row_grad_coef[f] * p[f, :] (product
+ * and sum rounded separately): the gradient that reaches W_D through decoder_norm().
  * Replaces loss.backward()'s dense `f^T @ grad` / `x^T @ dh` GEMMs together with
  * torch.optim.Adam.step for W_D / W_E (trainer.py:627-647). */
 int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
@@ -250,7 +252,7 @@ int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot,
                               double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                               float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
                               void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
-                              const float *extra_rows, const float *extra_bias, void *stream);
+                              const float *extra_rows, const float *extra_bias, const float *row_grad_coef, void *stream);
 
 /* The two Adam entry points above for a dictionary whose dtype is bfloat16 (config.py:39 `dtype`; parameters,
  * gradients and both moments are then bf16 tensors and torch.optim.Adam, trainer.py:375-390, updates them with its
@@ -445,6 +447,32 @@ int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *
 /* out[r] = sum_c src[r, c] (fp32 sum, fixed order) for src [rows, cols] fp32 or bf16.  The bias gradients autograd forms by
  * summing over tokens, for gradients held transposed ([features, tokens]). */
 int sae_row_sum(const void *src, int src_dtype, int64_t rows, int64_t cols, float *out, void *stream);
+
+/* The sparse form of the JumpReLU step, for dictionaries whose activations have become sparse (what the reference
+ * reaches for with its sparsity gate, models/sae.py:355-367, and the sparsity-gated backward of
+ * kernels/kernels.py:475-539): instead of a dense [B, F] activation, a sparse code of every token's kept features
+ * (u > theta: value u / s, in_window as below) and of the features inside the straight-through window that are not kept
+ * (|u - theta| < window / 2 and u > 0: value 0, in_window 1), with h, s, u, n as for sae_jumprelu_fwd.
+ *   sae_jumprelu_select_count: row_nnz[b] = number of such entries of token b.
+ *   sae_jumprelu_select_emit:  given row_off (int64 [B], the exclusive prefix sum of row_nnz), writes token b's entries in
+ *     ascending feature order to idx / val / in_window [capacity] from slot row_off[b] on (entries at or past `capacity`
+ *     are dropped), and per token tanh_tok[b] = sum over kept features of tanh(tanh_c * value * n) and l0_tok[b] = number
+ *     of kept features (both nullable).
+ * (row_off, row_nnz, idx, val) is a sparse code as the TopK select emits it: sae_sparse_decode_mse_fused gives the value
+ * gradients of all entries (the flagged ones included: their threshold gradient needs them), sae_build_feature_index and
+ * the factored optimizer pass take it as it is.  F must be a multiple of 8. */
+int sae_jumprelu_select_count(const void *pre, int dtype, const float *b_enc, const float *scale, const float *theta,
+                              double window, int64_t B, int64_t F, int32_t *row_nnz, void *stream);
+int sae_jumprelu_select_emit(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
+                             const float *theta, double window, double tanh_c, int64_t B, int64_t F, const int64_t *row_off,
+                             int32_t *idx, float *val, float *in_window, int64_t capacity, float *tanh_tok, float *l0_tok,
+                             void *stream);
+
+/* out_a[f] = sum over the slots of feature f (feat_ptr / feat_slot of sae_build_feature_index) of a[slot], and the same
+ * for b -> out_b (b, out_b nullable): the per-feature sums autograd forms by summing a dense [B, F] gradient over the
+ * tokens (threshold and decoder-norm gradients of the sparse JumpReLU step), in a fixed order. */
+int sae_feature_segment_sums(const int32_t *feat_ptr, const int32_t *feat_slot, const float *a, const float *b, int64_t F,
+                             float *out_a, float *out_b, void *stream);
 
 /* Measurement aid, no counterpart in the reference: n_workgroups x 4 waves each issue iters x 32
  * v_mfma_f32_16x16x32_bf16 from registers (no memory traffic in the loop) and write one float per lane to

@@ -42,7 +42,7 @@ SIGNATURES = {
     "sae_adam_step": (_I, [_P, _P, _I, _P, _P, _L, _F, _F, _F, _F, _L, _P, _P, _L, _P, _P]),
     "sae_sparse_adam_step": (_I, [_P, _P, _P, _P, _L, _F, _F, _F, _F, _P, _P, _P, _P]),
     "sae_grad_sq_nnz": (_I, [_P, _L, _P, _P]),
-    "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P]),
+    "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P]),
     "sae_adam_step_lowp": (_I, [_P, _P, _I, _P, _P, _L, _F, _F, _F, _F, _L, _P, _L, _P, _P]),
     "sae_adam_step_sparse_rows_lowp": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _L, _P]),
     "sae_gather_rows": (_I, [_P, _I, _P, _L, _L, _L, _P, _I, _F, _P]),
@@ -60,6 +60,9 @@ SIGNATURES = {
     "sae_row_sum": (_I, [_P, _I, _L, _L, _P, _P]),
     "sae_dense_row_nnz": (_I, [_P, _I, _L, _L, _P, _P]),
     "sae_dense_to_code": (_I, [_P, _I, _L, _L, _P, _P, _P, _L, _P]),
+    "sae_jumprelu_select_count": (_I, [_P, _I, _P, _P, _P, _F, _L, _L, _P, _P]),
+    "sae_jumprelu_select_emit": (_I, [_P, _I, _P, _P, _P, _P, _F, _F, _L, _L, _P, _P, _P, _P, _L, _P, _P, _P]),
+    "sae_feature_segment_sums": (_I, [_P, _P, _P, _P, _L, _P, _P, _P]),
     "sae_mfma_probe": (_I, [_P, _L, _L, _P, _P]),
     "sae_jumprelu_bwd": (_I, [_P, _I, _P, _P, _P, _P, _P, _P, _F, _P, _F, _L, _L, _P, _P, _P, _P, _P, _L, _P]),
 }

@@ -286,13 +286,15 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
     uint16_t *__restrict__ shadow, float *__restrict__ row_norm, float *__restrict__ bias_grad,
     const float *__restrict__ grad_scale, double *__restrict__ sq_nnz_partial,
-    const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows, const float *__restrict__ extra_bias) {
+    const int32_t *__restrict__ extra_map, const float *__restrict__ extra_rows, const float *__restrict__ extra_bias,
+    const float *__restrict__ row_grad_coef) {
   __shared__ float red[4];
   __shared__ double red_d[8];
   __shared__ float s_coef[256];
   __shared__ int32_t s_tok[256];
   const int f = blockIdx.x, tid = threadIdx.x;
   const float gs = grad_scale ? grad_scale[0] : 1.f;
+  const float rc = row_grad_coef ? row_grad_coef[f] : 0.f;   // the row's gradient through its L2 norm: rc * p[f, :]
   const int xo = extra_map ? extra_map[f] : -1;   // row of the dense gradient block that adds to this feature, or -1
   const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
   const int n_seg = d >> 2;
@@ -333,6 +335,10 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     for (int u = 0; u < U; ++u) {
       const int seg = seg0 + u * 256;
       if (seg < n_seg) {
+        if (row_grad_coef) {   // product and sum rounded separately, as when the term is added to a stored gradient
+          g[u].x = add_rn(g[u].x, mul_rn(rc, pp[u].x)); g[u].y = add_rn(g[u].y, mul_rn(rc, pp[u].y));
+          g[u].z = add_rn(g[u].z, mul_rn(rc, pp[u].z)); g[u].w = add_rn(g[u].w, mul_rn(rc, pp[u].w));
+        }
         if (grad_scale) {   // rounded products, as when the scaled gradient is written out before the step
           g[u].x = mul_rn(g[u].x, gs); g[u].y = mul_rn(g[u].y, gs);
           g[u].z = mul_rn(g[u].z, gs); g[u].w = mul_rn(g[u].w, gs);
@@ -519,9 +525,11 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
                                       double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                                       float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
                                       void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
-                                      const float *extra_rows, const float *extra_bias, void *stream) {
+                                      const float *extra_rows, const float *extra_bias, const float *row_grad_coef,
+                                      void *stream) {
   SAE_REQUIRE(feat_ptr && feat_slot && slot_tok && coef && dense && p && m && v, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: null pointer");
+  SAE_REQUIRE(!(lowp && row_grad_coef), SAE_ERR_UNSUPPORTED, "adam_step_sparse_rows_lowp: no row_grad_coef for bf16 state");
   SAE_REQUIRE((extra_map == nullptr) == (extra_rows == nullptr) && (((uintptr_t)extra_rows) & 15) == 0, SAE_ERR_INVALID_ARG,
               "adam_step_sparse_rows: extra_map and extra_rows go together (extra_rows 16-byte aligned)");
   SAE_REQUIRE(!grad_sq_nnz_acc || (workspace && workspace_bytes >= 16 * F && ((uintptr_t)workspace & 15) == 0),
@@ -547,7 +555,7 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
 #define SAE_ADAM_ROWS(BF, UU)                                                                                              \
   hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, UU>), dim3((unsigned)F), dim3(256), 0, st, feat_ptr, feat_slot, slot_tok, \
                      coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,            \
-                     bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias)
+                     bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias, row_grad_coef)
     // pieces of 4 elements per thread: short rows keep fewer registers, so more rows are in flight per CU
     const int u = d <= 1024 ? 1 : (d <= 2048 ? 2 : 4);
     if (lowp) {
@@ -587,11 +595,12 @@ extern "C" int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t 
                                          double eps, int64_t step, void *shadow_bf16, float *row_norm_out,
                                          float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
                                          void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
-                                         const float *extra_rows, const float *extra_bias, void *stream) {
+                                         const float *extra_rows, const float *extra_bias, const float *row_grad_coef,
+                                         void *stream) {
   return sae::adam_step_sparse_rows_impl(false, feat_ptr, feat_slot, slot_tok, coef, dense, dense_dtype, p, m, v, F, d, lr,
                                          beta1, beta2, eps, step, shadow_bf16, row_norm_out, bias_grad_out, grad_scale,
                                          grad_sq_nnz_acc, workspace, workspace_bytes, extra_map, extra_rows, extra_bias,
-                                         stream);
+                                         row_grad_coef, stream);
 }
 
 extern "C" int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int32_t *feat_slot, const int32_t *slot_tok,
@@ -604,7 +613,7 @@ extern "C" int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int
                                          reinterpret_cast<float *>(p_bf16), reinterpret_cast<float *>(m_bf16),
                                          reinterpret_cast<float *>(v_bf16), F, d, lr, beta1, beta2, eps, step, nullptr,
                                          row_norm_out, bias_grad_out, grad_scale, grad_sq_nnz_acc, workspace,
-                                         workspace_bytes, nullptr, nullptr, nullptr, stream);
+                                         workspace_bytes, nullptr, nullptr, nullptr, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -311,3 +311,39 @@ extern "C" int sae_sparse_grad_rows(const int32_t *feat_ptr, const int32_t *feat
                        slot_tok, coef, dense, out, bias_out, (int)d);
   return check_launch("sparse_grad_rows");
 }
+
+namespace sae {
+
+// out_x[f] = sum over feature f's slots of x[slot], for up to two per-slot arrays at once; one wave per feature,
+// lane-strided partial sums added in a fixed order.
+__global__ __launch_bounds__(256) void fi_segment_sums_kernel(const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
+                                                              const float *__restrict__ a, const float *__restrict__ b, int F,
+                                                              float *__restrict__ out_a, float *__restrict__ out_b) {
+  const int f = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (f >= F) return;
+  const int lo = feat_ptr[f], hi = feat_ptr[f + 1];
+  float sa = 0.f, sb = 0.f;
+  for (int i = lo + lane; i < hi; i += 64) {
+    const int sl = feat_slot[i];
+    sa += a[sl];
+    if (b) sb += b[sl];
+  }
+  sa = wave_sum(sa);
+  if (b) sb = wave_sum(sb);
+  if (lane == 0) {
+    out_a[f] = sa;
+    if (b) out_b[f] = sb;
+  }
+}
+
+}  // namespace sae
+
+extern "C" int sae_feature_segment_sums(const int32_t *feat_ptr, const int32_t *feat_slot, const float *a, const float *b, int64_t F,
+                                        float *out_a, float *out_b, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(feat_ptr && feat_slot && a && out_a && (!b || out_b), SAE_ERR_INVALID_ARG, "feature_segment_sums: null pointer");
+  SAE_REQUIRE(F > 0 && F < (1LL << 31), SAE_ERR_INVALID_ARG, "feature_segment_sums: bad F");
+  hipLaunchKernelGGL(fi_segment_sums_kernel, dim3((unsigned)((F + 3) / 4)), dim3(256), 0, (hipStream_t)stream, feat_ptr, feat_slot, a, b,
+                     (int)F, out_a, out_b);
+  return check_launch("feature_segment_sums");
+}

@@ -226,6 +226,164 @@ static int check_shape(const char *who, const void *pre, int dtype, const float 
 
 using namespace sae;
 
+namespace sae {
+
+// ---- the sparse route: threshold select -> sparse code --------------------------------------------------------
+// A trained JumpReLU dictionary keeps a few dozen of its features per token.  The step then needs, per token, the
+// kept features (u > theta: value u / s) and the features inside the straight-through window that are not kept
+// (|u - theta| < window / 2, u > 0: value 0, flagged): the former carry the reconstruction, both carry a threshold
+// gradient.  Two passes over the pre-activation (count, then emit in ascending feature order at the row offsets the
+// caller derives from the counts) give a sparse code in the layout the TopK select emits, which the sparse decoder,
+// the feature index and the factored optimizer pass consume as they are.  Same arithmetic per element as the dense
+// kernels above.
+template <bool BF16>
+__device__ __forceinline__ void jr_classify(const void *__restrict__ pre, const float *__restrict__ b_enc,
+                                            const float *__restrict__ scale, const float *__restrict__ theta, int64_t rbase,
+                                            int64_t g, float half_w, float (&a)[8], bool (&keep)[8], bool (&win)[8]) {
+  float p[8], b[8], s[8], th[8];
+  load8<BF16, false>(pre, rbase + g, p);
+  load8_f32_or(b_enc, g, 0.f, b);
+  load8_f32_or(scale, g, 1.f, s);
+  load8<false>(theta, g, th);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float h = p[i] + b[i];
+    const float u = h * s[i];
+    keep[i] = u > th[i];
+    win[i] = (fabsf(u - th[i]) < half_w) && (u > 0.f);
+    a[i] = keep[i] ? (scale ? u / s[i] : h) : 0.f;
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(JR_THREADS) void jumprelu_select_count_kernel(
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
+    const float *__restrict__ theta, int64_t F, float half_w, int32_t *__restrict__ row_nnz) {
+  __shared__ float red[JR_THREADS / 64];
+  const int64_t row = blockIdx.x, groups = F >> 3;
+  int cnt = 0;
+  for (int64_t g = threadIdx.x; g < groups; g += JR_THREADS) {
+    float a[8];
+    bool keep[8], win[8];
+    jr_classify<BF16>(pre, b_enc, scale, theta, row * groups, g, half_w, a, keep, win);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cnt += (keep[i] || win[i]) ? 1 : 0;
+  }
+  const float t = block_sum<JR_THREADS / 64>((float)cnt, red);
+  if (threadIdx.x == 0) row_nnz[row] = (int32_t)t;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(JR_THREADS) void jumprelu_select_emit_kernel(
+    const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
+    const float *__restrict__ pen, const float *__restrict__ theta, int64_t F, float half_w, float tanh_c,
+    const int64_t *__restrict__ row_off, int32_t *__restrict__ idx, float *__restrict__ val, float *__restrict__ in_window,
+    int64_t capacity, float *__restrict__ tanh_tok, float *__restrict__ l0_tok) {
+  __shared__ float red[JR_THREADS / 64];
+  __shared__ int wave_tot[JR_THREADS / 64];
+  const int64_t row = blockIdx.x, groups = F >> 3;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t run = row_off[row];
+  float tsum = 0.f, kept = 0.f;
+  for (int64_t g0 = 0; g0 < groups; g0 += JR_THREADS) {
+    const int64_t g = g0 + threadIdx.x;
+    float a[8];
+    bool keep[8], win[8];
+    int cnt = 0;
+    if (g < groups) {
+      jr_classify<BF16>(pre, b_enc, scale, theta, row * groups, g, half_w, a, keep, win);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) cnt += (keep[i] || win[i]) ? 1 : 0;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { a[i] = 0.f; keep[i] = win[i] = false; }
+    }
+    int incl = cnt;                                   // inclusive prefix over the wave's lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    __syncthreads();                                  // the previous chunk's totals have been read
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < JR_THREADS / 64; ++w) {
+      const int t = wave_tot[w];
+      before += w < wave ? t : 0;
+      total += t;
+    }
+    int64_t pos = run + before + incl - cnt;
+    if (cnt) {
+      float np[8];
+      load8_f32_or(pen, g, 1.f, np);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (keep[i] || win[i]) {
+          if (pos < capacity) {
+            idx[pos] = (int32_t)(g * 8 + i);
+            val[pos] = a[i];
+            in_window[pos] = win[i] ? 1.f : 0.f;
+          }
+          ++pos;
+        }
+        if (keep[i]) {
+          kept += 1.f;
+          if (tanh_tok) tsum += tanh_pos(tanh_c * a[i] * np[i]);
+        }
+      }
+    }
+    run += total;
+  }
+  if (tanh_tok) {
+    const float t = block_sum<JR_THREADS / 64>(tsum, red);
+    if (threadIdx.x == 0) tanh_tok[row] = t;
+  }
+  if (l0_tok) {
+    const float t = block_sum<JR_THREADS / 64>(kept, red);
+    if (threadIdx.x == 0) l0_tok[row] = t;
+  }
+}
+
+}  // namespace sae
+
+extern "C" int sae_jumprelu_select_count(const void *pre, int dtype, const float *b_enc, const float *scale, const float *theta,
+                                         double window, int64_t B, int64_t F, int32_t *row_nnz, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre && theta && row_nnz, SAE_ERR_INVALID_ARG, "jumprelu_select_count: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && (F & 7) == 0 && B < ((int64_t)1 << 31), SAE_ERR_INVALID_ARG,
+              "jumprelu_select_count: B > 0 and F a positive multiple of 8 expected");
+  SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "jumprelu_select_count: bad dtype");
+  const float hw = 0.5f * (float)window;
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(jumprelu_select_count_kernel<true>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
+                       scale, theta, F, hw, row_nnz);
+  else
+    hipLaunchKernelGGL(jumprelu_select_count_kernel<false>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
+                       scale, theta, F, hw, row_nnz);
+  return check_launch("jumprelu_select_count");
+}
+
+extern "C" int sae_jumprelu_select_emit(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
+                                        const float *theta, double window, double tanh_c, int64_t B, int64_t F,
+                                        const int64_t *row_off, int32_t *idx, float *val, float *in_window, int64_t capacity,
+                                        float *tanh_tok, float *l0_tok, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre && theta && row_off && idx && val && in_window, SAE_ERR_INVALID_ARG, "jumprelu_select_emit: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && (F & 7) == 0 && B < ((int64_t)1 << 31) && capacity >= 0, SAE_ERR_INVALID_ARG,
+              "jumprelu_select_emit: B > 0 and F a positive multiple of 8 expected");
+  SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "jumprelu_select_emit: bad dtype");
+  const float hw = 0.5f * (float)window;
+  if (dtype == SAE_BF16)
+    hipLaunchKernelGGL(jumprelu_select_emit_kernel<true>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
+                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok);
+  else
+    hipLaunchKernelGGL(jumprelu_select_emit_kernel<false>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
+                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok);
+  return check_launch("jumprelu_select_emit");
+}
+
 extern "C" int sae_jumprelu_fwd(const void *pre, int dtype, const float *b_enc, const float *scale,
                                 const float *pen_norm, const float *theta, int64_t B, int64_t F, double tanh_c_d, void *acts, float *tanh_tok, float *lp_tok,
                                 float *l0_tok, void *stream) {

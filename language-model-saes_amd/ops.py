@@ -539,8 +539,10 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                           v: torch.Tensor, *, lr: float, beta1: float, beta2: float, eps: float, step: int,
                           shadow_bf16: Optional[torch.Tensor] = None, row_norm_out: Optional[torch.Tensor] = None,
                           bias_grad_out: Optional[torch.Tensor] = None, grad_scale: Optional[torch.Tensor] = None,
-                          grad_sq_nnz_acc: Optional[torch.Tensor] = None, extra: Optional["DenseRowBlock"] = None) -> None:
+                          grad_sq_nnz_acc: Optional[torch.Tensor] = None, extra: Optional["DenseRowBlock"] = None,
+                          row_grad_coef: Optional[torch.Tensor] = None) -> None:
     """Adam on a feature-major [F, d] matrix whose gradient rows are rebuilt from (fi, coef, dense);
+    `row_grad_coef` (fp32 [F]) adds row_grad_coef[f] * p[f, :] to row f's gradient (the gradient through the row norm);
     `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping);
     `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed;
     `extra` adds a densely held block of gradient rows.  A bf16 `p` (with bf16 `m`, `v`) takes the low-precision
@@ -548,8 +550,12 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
     lowp = p.dtype == torch.bfloat16
     for name, t in (("p", p), ("m", m), ("v", v)):
         _req(t, name, torch.bfloat16 if lowp else torch.float32, 2)
-    if lowp and (shadow_bf16 is not None or extra is not None):
-        raise ValueError("the low-precision update takes neither a shadow copy nor a dense row block")
+    if lowp and (shadow_bf16 is not None or extra is not None or row_grad_coef is not None):
+        raise ValueError("the low-precision update takes neither a shadow copy, a dense row block nor a row coefficient")
+    if row_grad_coef is not None:
+        _req(row_grad_coef, "row_grad_coef", torch.float32, 1)
+        if row_grad_coef.numel() != p.shape[0]:
+            raise ValueError("row_grad_coef must have one entry per row")
     _req(coef, "coef", torch.float32, 1)
     _req(dense, "dense", ndim=2)
     F, d = p.shape
@@ -582,7 +588,8 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                                                   coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(), m.data_ptr(),
                                                   v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step), _ptr(shadow_bf16),
                                                   _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale),
-                                                  _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, *_extra_ptrs(extra, F, d), _stream(p)),
+                                                  _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, *_extra_ptrs(extra, F, d),
+                                                  _ptr(row_grad_coef), _stream(p)),
             "adam_step_sparse_rows",
         )
 
@@ -716,6 +723,54 @@ def jumprelu_bwd(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Option
                                    d_bias.data_ptr(), d_theta.data_ptr(), _ptr(d_scale), ws.data_ptr(), ws_bytes,
                                    _stream(pre)), "jumprelu_bwd")
     return d_pre, d_bias, d_theta, d_scale
+
+
+def jumprelu_select(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], theta: torch.Tensor,
+                    window: float, tanh_c: float = 0.0, pen_norm: Optional[torch.Tensor] = None, want_tanh: bool = False,
+                    max_entries: Optional[int] = None):
+    """Sparse form of the JumpReLU activation: the code of every token's kept features (value u / s) and of the features
+    inside the straight-through window that are not kept (value 0) -> (code, in_window fp32 [n_slots], tanh_tok [B] or
+    None, l0_tok [B]), or None when the batch holds no such entry or more than `max_entries` of them (the caller then
+    takes the dense route).  The entry count is read back from the device to size the code: one synchronisation per call, as the
+    reference's sparsity gate (models/sae.py:355-358)."""
+    _req(pre, "pre", ndim=2)
+    B, F = pre.shape
+    lib = _lib.load()
+    row_nnz = torch.empty(B, dtype=torch.int32, device=pre.device)
+    with _timed("jumprelu_select"):
+        check(lib.sae_jumprelu_select_count(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), theta.data_ptr(), float(window), B, F,
+                                            row_nnz.data_ptr(), _stream(pre)), "jumprelu_select_count")
+        incl = torch.cumsum(row_nnz, 0, dtype=torch.int64)
+        total = int(incl[-1].item())
+        if total == 0 or (max_entries is not None and total > max_entries):
+            return None
+        row_off = incl - row_nnz
+        cap = max(total, 1)
+        idx = torch.zeros(cap, dtype=torch.int32, device=pre.device)
+        val = torch.zeros(cap, dtype=torch.float32, device=pre.device)
+        win = torch.zeros(cap, dtype=torch.float32, device=pre.device)
+        tanh_tok = torch.empty(B, dtype=torch.float32, device=pre.device) if want_tanh else None
+        l0_tok = torch.empty(B, dtype=torch.float32, device=pre.device)
+        check(lib.sae_jumprelu_select_emit(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(pen_norm), theta.data_ptr(),
+                                           float(window), float(tanh_c), B, F, row_off.data_ptr(), idx.data_ptr(), val.data_ptr(),
+                                           win.data_ptr(), total, _ptr(tanh_tok), l0_tok.data_ptr(), _stream(pre)),
+              "jumprelu_select_emit")
+    return SparseCode(idx, val, row_off, row_nnz, B, F), win, tanh_tok, l0_tok
+
+
+def feature_segment_sums(fi: FeatureIndex, a: torch.Tensor, b: Optional[torch.Tensor] = None):
+    """Per-feature sums of one or two per-slot fp32 arrays over the feature index -> (fp32 [F], fp32 [F] or None)."""
+    _req(a, "a", torch.float32, 1)
+    F = fi.feat_ptr.numel() - 1
+    out_a = torch.empty(F, dtype=torch.float32, device=a.device)
+    out_b = None
+    if b is not None:
+        _req(b, "b", torch.float32, 1)
+        out_b = torch.empty(F, dtype=torch.float32, device=a.device)
+    with _timed("feature_segment_sums"):
+        check(_lib.load().sae_feature_segment_sums(fi.feat_ptr.data_ptr(), fi.feat_slot.data_ptr(), a.data_ptr(), _ptr(b), F,
+                                                   out_a.data_ptr(), _ptr(out_b), _stream(a)), "feature_segment_sums")
+    return out_a, out_b
 
 
 def code_stats(code: SparseCode, tok_w: Optional[torch.Tensor] = None, freq_acc: Optional[torch.Tensor] = None,

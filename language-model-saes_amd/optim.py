@@ -267,7 +267,7 @@ class HipAdam(Optimizer):
         req, acc, wanted = self._norm_request, None, ()
         self._norm_request = None
         if req is not None:
-            fold_row_grad_coef(req[0])   # the norm is over the element-wise gradient
+            fold_row_grad_coef(req[0], keep_factored=True)   # the norm is over the element-wise gradient
             wanted = {id(p) for p in req[0]}
             acc = torch.zeros(2, dtype=torch.float64, device=req[1].device)
         # pass 1: weights whose gradient arrives in factored form (also yields the encoder-bias gradient)
@@ -291,6 +291,10 @@ class HipAdam(Optimizer):
                 self._step_row_blocks(group, p, sg, st, pv, mv, vv, acc if id(p) in wanted else None)
                 continue
             role, shadow, norm_out = self._by_products(p, pv)
+            row_coef = getattr(p, "_row_grad_coef", None)     # the gradient through the row norm, added where rows are rebuilt
+            if row_coef is not None and (p.dtype != torch.float32 or sg.sq_nnz is not None):
+                raise RuntimeError("a row-norm gradient term cannot join this factored gradient")
+            p._row_grad_coef = None
             bias_out = None
             if sg.bias_param is not None:
                 bias_out = torch.empty(pv.shape[0], dtype=torch.float32, device=p.device)
@@ -315,7 +319,7 @@ class HipAdam(Optimizer):
                 ops.adam_step_sparse_rows(sg.fi, sg.coef, sg.dense_operand, pv, mv, vv, lr=group["lr"], beta1=b1, beta2=b2,
                                           eps=group["eps"], step=int(st["step"].item()), shadow_bf16=shadow,
                                           row_norm_out=norm_out, bias_grad_out=bias_out, grad_scale=sg.scale,
-                                          grad_sq_nnz_acc=sums_out, extra=sg.extra)
+                                          grad_sq_nnz_acc=sums_out, extra=sg.extra, row_grad_coef=row_coef)
                 if side is not None:
                     ev = torch.cuda.Event()
                     ev.record(side)
@@ -423,7 +427,7 @@ class HipSparseAdam(Optimizer):
         return loss
 
 
-def fold_row_grad_coef(params) -> None:
+def fold_row_grad_coef(params, keep_factored: bool = False) -> None:
     """Bring what the backward left on a weight for HipAdam into its dense fp32 `.grad`, for consumers of the
     element-wise gradient (norm, clipping, SparseAdam): a bf16 gradient over the parameter's storage
     (`_lowp_grad`, widened), and the row-norm gradient (`_row_grad_coef`: d n / n per row, added as
@@ -437,6 +441,17 @@ def fold_row_grad_coef(params) -> None:
         coef = getattr(p, "_row_grad_coef", None)
         if coef is None:
             continue
+        sg = getattr(p, "_sparse_grad", None)
+        if sg is not None:
+            if keep_factored and not hasattr(sg, "pieces"):
+                continue        # HipAdam's factored pass adds the term to the rows it rebuilds
+            # an element-wise consumer of a gradient that is factored AND has a row-norm term: both become dense
+            rows, bias = sg.dense()
+            p.grad = _grad_like(p, rows.to(p.dtype))
+            if bias is not None:
+                g = bias.view(sg.bias_param.shape).to(sg.bias_param.dtype)
+                sg.bias_param.grad = g if sg.bias_param.grad is None else sg.bias_param.grad + g
+            p._sparse_grad = None
         term = (coef.view(-1, *([1] * (p.ndim - 1))) * p.detach()).to(p.dtype)
         p.grad = term if p.grad is None else p.grad + term
         p._row_grad_coef = None

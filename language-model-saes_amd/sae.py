@@ -399,8 +399,10 @@ class _EncoderGemm(torch.autograd.Function):
     kernel."""
 
     @staticmethod
-    def forward(ctx, x, W_E, w_op, amp, defer=False):
-        if amp:
+    def forward(ctx, x, W_E, w_op, amp, defer=False, given=None):
+        if given is not None:             # (x operand, product) computed by the caller already
+            x_op, pre = given
+        elif amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())
             pre = ops.encoder_gemm(x_op, w_op, torch.bfloat16)
         else:
@@ -425,7 +427,7 @@ class _EncoderGemm(torch.autograd.Function):
                 _leave_lowp_grad(ctx.param, rows)
             else:
                 dW = rows.t().to(ctx.w_dtype)                                      # [d, F] with feature-major strides
-        return dx, dW, None, None, None
+        return dx, dW, None, None, None, None
 
 
 def _leave_lowp_grad(param, rows: torch.Tensor) -> None:
@@ -517,6 +519,82 @@ class _JumpReLUStep(torch.autograd.Function):
         return d_pre, d_bias.to(ctx.b_dtype), d_norm, d_theta.to(ctx.th_dtype), None, None, None, None, None
 
 
+class _JumpReLUSparseStep(torch.autograd.Function):
+    """The JumpReLU step of a dictionary whose activations are sparse: threshold select -> sparse decode + squared error
+    (+ tanh penalty) forward, and backward through the feature index of the code, like the TopK step.  The code holds
+    every token's kept features and, with value 0, the features inside the straight-through window that are not kept;
+    `dval` (the decoder's gradient at every entry) is what both the pre-activation gradient of kept entries and the
+    threshold gradient of window entries start from.  With ga = dval + l1 w_b c n (1 - tanh^2(c a n)):
+        d pre   = ga at kept entries                              -> dW_E^T rows, db_E (factored)
+        d theta = sum over window entries of (ga / s) (-theta / window)
+        d n     = sum over kept entries of l1 w_b c a (1 - tanh^2)
+    exactly the sums the dense backward kernel forms over [B, F] (the two derivative terms of act(h s) / s with
+    respect to s cancel)."""
+
+    @staticmethod
+    def forward(ctx, theta, norm, W_E, b_E, W_D, b_D, label, tok_w, holder):
+        sae, code = holder["model"], holder["code"]
+        amp = holder["amp"]
+        w_dec_op = sae._w_dec_operand(amp)
+        recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, w_dec_op, None if b_D is None else b_D.detach(),
+                                                                        label, tok_w)
+        loss = loss_tok.sum()
+        l_s = None
+        if holder["want_tanh"]:
+            l_s = holder["l1"] * holder["tanh_tok"]
+            loss = loss + (tok_w * l_s).sum()
+        holder["l_s"], holder["l_rec"] = l_s, loss_tok.sum()
+        ctx.save_for_backward(theta.detach().float(), tok_w, grad_recon, dval, *(() if norm is None else (norm.detach().float(),)))
+        ctx.holder, ctx.has_norm, ctx.has_b_D = holder, norm is not None, b_D is not None
+        ctx.th_dtype = theta.dtype
+        ctx.mark_non_differentiable(recon)
+        ctx.set_materialize_grads(False)
+        return loss, recon
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_recon):
+        if g_loss is None:
+            return (None,) * 9
+        theta, tok_w, grad_recon, dval, *rest = ctx.saved_tensors
+        norm = rest[0] if ctx.has_norm else None
+        h = ctx.holder
+        sae, code, win = h["model"], h["code"], h["win"]
+        F = code.d_sae
+        g = g_loss.to(torch.float32)
+        fi = ops.build_feature_index(code)
+        idx = code.idx.long()
+        val = code.val
+        th_f = theta[idx]
+        s_f = norm[idx] if (norm is not None and h["scaled"]) else None
+        ga, dn_slot = dval, None
+        if h["want_tanh"]:
+            n_f = norm[idx]
+            c = h["tanh_c"]
+            t = torch.tanh(c * val * n_f)
+            sech2 = 1.0 - t * t
+            gt = (h["l1"] * c) * tok_w[fi.slot_tok.long()]
+            ga = dval + gt * n_f * sech2
+            dn_slot = (gt * val * sech2).contiguous()
+        d_pre = torch.where(val > 0, ga, torch.zeros_like(ga))
+        dth_slot = win * (ga if s_f is None else ga / s_f) * (-th_f / h["window"])
+        d_theta, d_norm = ops.feature_segment_sums(fi, dth_slot.contiguous(), dn_slot)
+        coef_dec, coef_enc = val * g, d_pre * g
+        x_op = h["x_op"]
+        grad_dense_D = ops.cast_bf16(grad_recon) if h["amp"] else grad_recon
+        db_D = ops.col_sum(grad_recon) * g if ctx.has_b_D else None
+        defer = h["defer"]
+        if defer and all(getattr(p, "_sparse_grad", None) is None and p.grad is None for p in (sae.W_D, sae.W_E)):
+            sae.W_D._sparse_grad = SparseRowGrad(fi, coef_dec, grad_dense_D, F)
+            sae.W_E._sparse_grad = SparseRowGrad(fi, coef_enc, x_op, F, bias_param=sae.b_E)
+            dW_D = dW_E = db_E = None
+        else:
+            dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, grad_dense_D, F)
+            dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, x_op, F, want_bias=True)
+            dW_E = dW_Et.t()
+        return ((d_theta * g).to(ctx.th_dtype), None if d_norm is None or not ctx.needs_input_grad[1] else d_norm * g,
+                dW_E, db_E, dW_D, db_D, None, None, None)
+
+
 @register_sae_model("sae")
 class SparseAutoEncoder(SparseDictionary):
     def __init__(self, cfg: SAEConfig, device_mesh=None):
@@ -541,6 +619,13 @@ class SparseAutoEncoder(SparseDictionary):
         # aux-k: treat the dead features as a compact dense block (three small GEMMs) when shapes allow; False keeps
         # the sparse route (dead-feature entries stacked onto the main code) for every shape
         self.aux_dense_block = True
+        # JumpReLU: take the sparse form of the step when the batch's activations are sparse enough (at most a fraction
+        # 1 - cfg.sparsity_threshold_for_triton_spmm_kernel of [B, F] kept or inside the threshold window).  Looking
+        # costs one pass over the pre-activation and one read-back; while the dictionary is dense it is done every
+        # `jumprelu_sparse_probe_every` steps only.
+        self.jumprelu_sparse_route = True
+        self.jumprelu_sparse_probe_every = 16
+        self._jr_dense_steps = 0
 
     # ---- an optimiser may still be updating W_D on another stream (see HipAdam.overlap_decoder_update) ----
     def set_pending_update(self, event) -> None:
@@ -761,9 +846,30 @@ class SparseAutoEncoder(SparseDictionary):
         amp = _autocast_dtype("cuda") == torch.bfloat16
         jr = self.activation_function
         defer = bool(self.defer_weight_grads and torch.is_grad_enabled())
-        pre = _EncoderGemm.apply(x, self.W_E, self._w_enc_operand(amp), amp, defer)
         want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
         scaled = bool(self.cfg.sparsity_include_decoder_norm)
+        w_enc_op = self._w_enc_operand(amp)
+        given = None
+        B = x.shape[0]
+        if (self.jumprelu_sparse_route and sparsity_loss_type in (None, "tanh") and not want_lp and B <= 131072
+                and self.cfg.d_model % 8 == 0 and self._jr_dense_steps % max(1, self.jumprelu_sparse_probe_every) == 0):
+            with torch.no_grad():
+                x_op = (x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())) if amp else x.float().contiguous()
+                pre_raw = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16 if amp else torch.float32)
+                given = (x_op, pre_raw)
+                n_raw = self._decoder_norm_nograd() if (scaled or want_tanh) else None
+                th_raw = jr.get_jumprelu_threshold().detach().float().contiguous()
+                budget = int(B * self.cfg.d_sae * (1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel))
+                picked = ops.jumprelu_select(pre_raw, self.b_E.detach().float(), n_raw if scaled else None, th_raw,
+                                             float(jr.jumprelu_threshold_window), float(tanh_stretch_coefficient), pen_norm=n_raw,
+                                             want_tanh=want_tanh, max_entries=budget)
+            if picked is not None:
+                self._jr_dense_steps = 0
+                return self._jumprelu_sparse_loss(batch, x, label, mask, picked, x_op, amp, defer, scaled, want_tanh,
+                                                  float(tanh_stretch_coefficient), float(l1_coefficient), lp_coefficient,
+                                                  auxk_coefficient, return_aux_data, pre_raw)
+        self._jr_dense_steps += 1
+        pre = _EncoderGemm.apply(x, self.W_E, w_enc_op, amp, defer, given)
         n = None
         want_dense_pen = sparsity_loss_type in ("power", "tanh-quad")
         if scaled or want_tanh or want_lp or want_dense_pen:
@@ -806,6 +912,36 @@ class SparseAutoEncoder(SparseDictionary):
                  "lp_coefficient": lp_coefficient, "auxk_coefficient": auxk_coefficient}
         lazy = {"n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
                 "hidden_pre": lambda: pre.detach().float() + b_E}
+        return LazyDict(eager, lazy)
+
+    def _jumprelu_sparse_loss(self, batch, x, label, mask, picked, x_op, amp, defer, scaled, want_tanh, tanh_c, l1_coefficient,
+                              lp_coefficient, auxk_coefficient, return_aux_data, pre_raw):
+        code, win, tanh_tok, l0_tok = picked
+        jr = self.activation_function
+        B = x.shape[0]
+        if mask is None:
+            tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=x.device)
+        else:
+            m = mask.to(torch.float32)
+            tok_w = m / m.sum()
+        n = None
+        if scaled or want_tanh:
+            n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), self if defer else None)
+        holder = {"model": self, "code": code, "win": win, "tanh_tok": tanh_tok, "x_op": x_op, "amp": amp, "defer": defer,
+                  "scaled": scaled, "want_tanh": want_tanh, "tanh_c": tanh_c, "l1": l1_coefficient,
+                  "window": float(jr.jumprelu_threshold_window)}
+        loss, recon = _JumpReLUSparseStep.apply(jr.get_jumprelu_threshold(), n, self.W_E, self.b_E, self.W_D,
+                                                self.b_D if self.cfg.use_decoder_bias else None,
+                                                label.to(torch.float32).contiguous(), tok_w, holder)
+        if not return_aux_data:
+            return loss
+        b_E = self.b_E.detach()
+        eager = {"loss": loss, "l_rec": holder["l_rec"], "l_s": holder["l_s"], "l_p": None, "l_aux": None, "label": label,
+                 "mask": mask, "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
+                 "auxk_coefficient": auxk_coefficient, "sparse_code": code}
+        lazy = {"n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
+                "feature_acts": code.to_dense,
+                "hidden_pre": lambda: pre_raw.float() + b_E}
         return LazyDict(eager, lazy)
 
     def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,

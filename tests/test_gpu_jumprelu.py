@@ -276,3 +276,141 @@ def test_jumprelu_trainer_steps_with_and_without_deferred_terms(pkg, oracle, dev
         assert torch.isfinite(a[n]).all()
         assert torch.equal(a[n], b[n]), n
     assert na == nb
+
+
+# ---- the sparse form of the step: threshold select -> sparse code -> sparse decode / factored gradients ----------
+
+def make_sparse_pair(pkg, oracle, dev, d, F, B, seed, include_norm, window=0.3, theta_lo=1.7, theta_hi=2.3, budget=0.99):
+    """Thresholds around 2 on pre-activations of unit scale: a few entries per thousand are kept, about as many more
+    lie inside the straight-through window."""
+    from lm_saes_amd import synthetic
+
+    x = synthetic.activations(B, d, 8, seed)
+    w = synthetic.sae_weights(d, F, x, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    W_D = (w[2] * (0.5 + torch.rand(F, 1, generator=g))).contiguous()
+    w = (w[0], 0.02 * torch.randn(F, generator=g), W_D, w[3])
+    log_theta = torch.log(theta_lo + (theta_hi - theta_lo) * torch.rand(F, generator=g))
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=window, norm_activation="inference", sparsity_include_decoder_norm=include_norm,
+                        sparsity_threshold_for_triton_spmm_kernel=budget, device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    synthetic.load_weights(sae, *[t.to(dev) for t in w])
+    ref = oracle.SAEOracle(d, F, act_fn="jumprelu", jumprelu_threshold_window=window, sparsity_include_decoder_norm=include_norm)
+    synthetic.load_weights(ref, *w)
+    with torch.no_grad():
+        sae.activation_function.log_jumprelu_threshold.copy_(log_theta.to(dev))
+        ref.activation_function.log_jumprelu_threshold.copy_(log_theta)
+    y = x + 0.1 * torch.randn(B, d, generator=g)
+    batch = {"in": x, "out": y, "tokens": torch.zeros(B, dtype=torch.long), "mask": (torch.rand(B, generator=g) > 0.25).float()}
+    return sae, ref, batch
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_scale", [True, False])
+def test_jumprelu_select_lists_kept_and_window_entries(pkg, dev, dtype, with_scale):
+    """sae_jumprelu_select_count / _emit against the definition on the CPU: kept = u > theta (value u / s), window =
+    |u - theta| < window / 2 and u > 0; every token's entries in ascending feature order; per-token tanh sums and L0."""
+    g = torch.Generator().manual_seed(31)
+    B, F, window, c = 37, 1024, 0.4, 2.0
+    pre = torch.randn(B, F, generator=g).to(dtype)
+    b = 0.1 * torch.randn(F, generator=g)
+    s = (0.5 + torch.rand(F, generator=g)) if with_scale else None
+    theta = 1.5 + torch.rand(F, generator=g)
+    got = pkg.ops.jumprelu_select(pre.to(dev), b.to(dev), None if s is None else s.to(dev), theta.to(dev), window, c,
+                                  pen_norm=None if s is None else s.to(dev), want_tanh=True)
+    code, win, tanh_tok, l0 = got
+    h = pre.float() + b
+    u = h * s if s is not None else h
+    keep = u > theta
+    inwin = ((u - theta).abs() < 0.5 * window) & (u > 0)
+    listed = keep | inwin
+    assert torch.equal(code.row_nnz.cpu().long(), listed.sum(1))
+    rows, cols = listed.nonzero(as_tuple=True)
+    assert code.n_slots == len(cols) and torch.equal(code.idx.cpu().long(), cols)
+    acts = torch.where(keep, (u / s) if s is not None else h, torch.zeros_like(h))
+    want_val = acts[rows, cols]
+    assert torch.equal(code.val.cpu(), want_val)
+    assert torch.equal(win.cpu(), inwin[rows, cols].float())
+    assert torch.equal(l0.cpu(), keep.sum(1).float())
+    n = s if s is not None else torch.ones(F)
+    want_tanh = torch.tanh(c * acts * n).sum(1)
+    assert ((tanh_tok.cpu() - want_tanh).abs().max() / want_tanh.abs().max()).item() < 1e-5
+    # the budget: more entries than allowed -> None (the caller's dense route); none at all -> None
+    assert pkg.ops.jumprelu_select(pre.to(dev), b.to(dev), None, theta.to(dev), window, max_entries=3) is None
+    assert pkg.ops.jumprelu_select(pre.to(dev), None, None, (theta + 100).to(dev), window) is None
+
+
+@pytest.mark.parametrize("include_norm", [True, False])
+@pytest.mark.parametrize("kw", [dict(), dict(sparsity_loss_type="tanh", l1_coefficient=0.05, tanh_stretch_coefficient=2.0)])
+def test_sparse_jumprelu_step_fp32_matches_oracle(pkg, oracle, dev, include_norm, kw):
+    d, F, B = 64, 4096, 96
+    sae, ref, batch = make_sparse_pair(pkg, oracle, dev, d, F, B, seed=21, include_norm=include_norm)
+    gb = {k: v.to(dev) for k, v in batch.items()}
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
+    out = sae.compute_loss(gb, **kw)
+    out["loss"].backward()
+    torch.cuda.synchronize()
+    pkg.ops.set_kernel_timer(None)
+    ran = set(timer.records)
+    assert "jumprelu_select" in ran and "sparse_decode_mse_fused" in ran and "jumprelu_fwd" not in ran, ran
+    want = ref.compute_loss(batch, **kw)
+    want["loss"].backward()
+    density = (want["feature_acts"] != 0).float().mean().item()
+    assert 0 < density < 0.01, density
+    assert torch.equal((out["feature_acts"] != 0).cpu(), want["feature_acts"] != 0)
+    for key in ("feature_acts", "hidden_pre", "reconstructed", "loss", "l_rec"):
+        assert rel_err(out[key], want[key]) < FP32_TOL, key
+    if want["l_s"] is not None:
+        assert rel_err(out["l_s"], want["l_s"]) < FP32_TOL
+    got, exp = named_grads(sae), named_grads(ref)
+    for n in exp:
+        assert got[n] is not None, n
+        assert rel_err(got[n], exp[n]) < GRAD_TOL, (n, rel_err(got[n], exp[n]))
+    assert (exp["log_jumprelu_threshold"] != 0).sum() > 20       # window entries exist and carry threshold gradient
+
+
+def test_sparse_jumprelu_adam_steps_follow_the_oracle_and_fall_back_when_dense(pkg, oracle, dev):
+    """Three optimizer steps on the sparse route with the tanh penalty: the factored weight gradients and the decoder-norm
+    term go into the Adam kernel (`row_grad_coef`), and the parameters follow torch.optim.Adam on the oracle (fp32: under
+    bf16 the first Adam steps, which move every touched weight by +-lr whatever the gradient's size, turn rounding noise on
+    near-zero gradient elements into full steps on either side).  One more step under bf16 autocast agrees in its loss.
+    Then the thresholds are lowered: the same model takes the dense route again."""
+    d, F, B = 64, 4096, 128
+    sae, ref, batch = make_sparse_pair(pkg, oracle, dev, d, F, B, seed=23, include_norm=True)
+    gb = {k: v.to(dev) for k, v in batch.items()}
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=0.05)
+    groups = sae.get_parameters()
+    opt = pkg.HipAdam([{"params": groups[0]["params"]}, {"params": groups[1]["params"], "lr": 2e-3}], lr=1e-3, model=sae)
+    ropt = oracle.make_adam(ref, lr=1e-3, jumprelu_lr_factor=2.0)
+    rp = {k.replace("activation_function.", ""): v for k, v in ref.named_parameters()}
+    for step in range(3):
+        out = sae.compute_loss(gb, **kw)
+        assert "sparse_code" in out, "the sparse route did not run"
+        out["loss"].backward()
+        assert sae.W_D._sparse_grad is not None and sae.W_D._row_grad_coef is not None and sae.W_D.grad is None
+        opt.step(); opt.zero_grad()
+        rctx = oracle.train_step(ref, ropt, batch, **kw)
+        assert rel_err(out["loss"], rctx["loss"]) < 1e-4, step
+        for n, p in sae.named_parameters():
+            q = rp[n.replace("activation_function.", "")].detach()
+            assert (p.detach().cpu() - q).abs().max() <= 2e-2 * 2e-3 * (step + 1) + 1e-6 * q.abs().max(), (step, n)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(gb, **kw)
+    assert "sparse_code" in out
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        want = ref.compute_loss(batch, **kw)
+    assert rel_err(out["loss"], want["loss"]) < BF16_TOL
+    out["loss"].backward()
+    opt.step(); opt.zero_grad()
+    assert all(torch.isfinite(p).all() for p in sae.parameters())
+    with torch.no_grad():
+        sae.activation_function.log_jumprelu_threshold.fill_(-3.0)
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        dense = sae.compute_loss(gb, **kw)
+    pkg.ops.set_kernel_timer(None)
+    assert "jumprelu_fwd" in timer.records and "sparse_code" not in dense
+    assert len(timer.records["encoder_gemm"]) == 2      # the probe's encoder product is reused, not recomputed
