@@ -319,6 +319,34 @@ def build_jumprelu(pkg, dev, args):
     return _autocast_step(sae, batch, opt, kw), B, name, (B, d, F, F // 2)
 
 
+def build_jumprelu_sparse(pkg, dev, args):
+    """The JumpReLU configuration as it looks once trained: the same shapes and data, thresholds raised so that about 64 of
+    the 131072 features pass per token (log-threshold log(3.5), window 0.1).  The step then takes its sparse form."""
+    import torch
+
+    B, d, F = args.batch or 4096, D_MODEL, D_SAE
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=0.1, norm_activation="inference", sparsity_include_decoder_norm=True,
+                        device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(B, d, device=dev, generator=g)
+    x[:, [7, 511, 1024, 3000]] *= 50.0
+    _init_sae_on_device(sae, x, d)
+    with torch.no_grad():
+        sae.activation_function.log_jumprelu_threshold.fill_(math.log(3.5))
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    groups = sae.get_parameters()
+    opt = pkg.HipAdam([{"params": groups[0]["params"]}, {"params": groups[1]["params"]}], lr=4e-4, model=sae)
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=5.0)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(batch, **kw)
+    l0 = float(out["sparse_code"].row_nnz.float().mean().item()) if "sparse_code" in out else float("nan")
+    name = (f"jumprelu_sae_train_step (sparse form, {l0:.0f} kept-or-window entries per token) d_model={d} d_sae={F} batch={B} "
+            f"window=0.1 tanh-penalty=5 bf16 adam")
+    return _autocast_step(sae, batch, opt, kw), B, name, (B, d, F, max(1, int(l0) if l0 == l0 else 64))
+
+
 def build_clt(pkg, dev, args):
     """Cross-layer transcoder: 12 layers, d=768, 12288 features per layer, k=64 per layer, 2048 tokens;
     targets y_j = tanh(A_j x_j) with seeded A_j ~ N(0, 1) / sqrt(768)."""
@@ -367,7 +395,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
