@@ -117,7 +117,7 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_fwd_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float h = p[i] + b[i];
-      const float u = h * s[i];
+      const float u = mul_rn(h, s[i]);
       const bool keep = u > th[i];
       a[i] = keep ? (scale ? u / s[i] : h) : 0.f;
       cnt += keep ? 1.f : 0.f;
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_bwd_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float h = p[i] + b[i];
-      const float u = h * s[i];
+      const float u = mul_rn(h, s[i]);
       const bool keep = u > th[i];
       float gtot = ga[i];
       if (g_tanh) {
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_bwd_kernel(
         acc_s[i] += gt * a * sech2;
       }
       float d = keep ? gtot : 0.f;
-      const bool in_window = (fabsf(u - th[i]) < half_w) && (u > 0.f);
+      const bool in_window = (fabsf(sub_rn(u, th[i])) < half_w) && (u > 0.f);
       if (in_window) acc_t[i] += (gtot / s[i]) * (-th[i] / window);
       if (g_lp && th[i] > h) {
         d -= gl * np[i];
@@ -248,9 +248,9 @@ __device__ __forceinline__ void jr_classify(const void *__restrict__ pre, const 
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float h = p[i] + b[i];
-    const float u = h * s[i];
+    const float u = mul_rn(h, s[i]);      // a rounded product, as the tensor h * norm is: never fused into u - theta
     keep[i] = u > th[i];
-    win[i] = (fabsf(u - th[i]) < half_w) && (u > 0.f);
+    win[i] = (fabsf(sub_rn(u, th[i])) < half_w) && (u > 0.f);
     a[i] = keep[i] ? (scale ? u / s[i] : h) : 0.f;
   }
 }

@@ -103,3 +103,91 @@ def test_random_sweep(pkg, oracle, dev, sweep_seed, budget_s=12.0):
                 pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=step, **hy)
                 assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
     assert n > 100
+
+
+@pytest.mark.parametrize("sweep_seed", [3])
+def test_random_sweep_attention_and_code_conversions(pkg, oracle, dev, sweep_seed, budget_s=10.0):
+    """The same kind of sweep for the attention kernels (forward + backward against fp64 attention on bf16-representable
+    inputs), the dense -> code conversion, the JumpReLU threshold select (both to the bit against their definitions) and
+    the factored Adam pass with a row-norm coefficient (to the bit against the dense route)."""
+    import math
+
+    rng = random.Random(sweep_seed)
+    t0 = time.time()
+    n = 0
+    bf = lambda t: t.to(torch.bfloat16)                                          # noqa: E731
+    while time.time() - t0 < budget_s:
+        n += 1
+        kind = rng.choice(["attention", "dense_code", "jr_select", "adam_rowcoef"])
+        seed = rng.randrange(1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        if kind == "attention":
+            nb = rng.choice([1, 2, 3, 8]); s = 8 * rng.choice([1, 3, 8, 9, 16, 25]); h = rng.choice([1, 2, 4, 8])
+            dq = rng.choice([32, 64]); dv = rng.choice([32, 64, 128]); bias = rng.random() < 0.5
+            print(f"[{n}] attention seed={seed} nb={nb} s={s} h={h} dq={dq} dv={dv} bias={bias}", flush=True)
+            T = nb * s
+            q, k, v, do = (bf(torch.randn(T, h * w, generator=g)) for w in (dq, dq, dv, dv))
+            bq, bk, bv = ((0.3 * torch.randn(h * w, generator=g)) if bias else None for w in (dq, dq, dv))
+            eff = lambda t, b: (t.double() if b is None else bf(t.float() + b).double()).requires_grad_()   # noqa: E731
+            ql, kl, vl = eff(q, bq), eff(k, bk), eff(v, bv)
+            scale = 1.0 / math.sqrt(dq)
+            sc = torch.einsum("bqhd,bkhd->bhqk", ql.view(nb, s, h, dq), kl.view(nb, s, h, dq)) * scale
+            sc = sc.masked_fill(~torch.ones(s, s, dtype=torch.bool).tril(), float("-inf"))
+            want = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(sc, -1), vl.view(nb, s, h, dv)).reshape(T, h * dv)
+            (want * do.double()).sum().backward()
+            dv_ = lambda t: None if t is None else t.to(dev)                                               # noqa: E731
+            gq, gk, gv, gdo = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
+            out, lse = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
+            rel = lambda a, b: ((a.double().cpu() - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()  # noqa: E731
+            assert rel(out, want.detach()) < 8e-3
+            dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(),
+                                                  lse, nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
+            assert rel(dqt.t(), ql.grad) < 2e-2 and rel(dkt.t(), kl.grad) < 2e-2 and rel(dvt.t(), vl.grad) < 2e-2
+        elif kind == "dense_code":
+            B = rng.choice([1, 5, 40]); F = rng.choice([8, 100, 2047, 4096, 20000, 131072]); dt = rng.choice([torch.float32, torch.bfloat16])
+            dens = rng.choice([0.0, 0.001, 0.05, 0.6])
+            print(f"[{n}] dense_code seed={seed} B={B} F={F} {dt} density={dens}", flush=True)
+            x = (torch.randn(B, F, generator=g) * (torch.rand(B, F, generator=g) < dens)).to(dt)
+            code = pkg.ops.dense_to_code(x.to(dev))
+            rows, cols = (x != 0).nonzero(as_tuple=True)
+            assert torch.equal(code.row_nnz.cpu().long(), (x != 0).sum(1))
+            assert torch.equal(code.idx.cpu().long()[: len(cols)], cols) and torch.equal(code.val.cpu()[: len(cols)], x[rows, cols].float())
+        elif kind == "jr_select":
+            B = rng.choice([1, 7, 33]); F = 8 * rng.choice([1, 13, 128, 512, 2048, 16384]); dt = rng.choice([torch.float32, torch.bfloat16])
+            window = rng.choice([1e-3, 0.1, 0.5]); use_s = rng.random() < 0.6
+            print(f"[{n}] jr_select seed={seed} B={B} F={F} {dt} window={window} scale={use_s}", flush=True)
+            pre = torch.randn(B, F, generator=g).to(dt)
+            b = 0.1 * torch.randn(F, generator=g)
+            s_ = 0.5 + torch.rand(F, generator=g) if use_s else None
+            theta = rng.choice([0.5, 1.5, 2.5]) + 0.5 * torch.rand(F, generator=g)
+            got = pkg.ops.jumprelu_select(pre.to(dev), b.to(dev), None if s_ is None else s_.to(dev), theta.to(dev), window)
+            hh = pre.float() + b
+            u = hh * s_ if use_s else hh
+            keep = u > theta
+            listed = keep | (((u - theta).abs() < 0.5 * window) & (u > 0))
+            if not listed.any():
+                assert got is None
+                continue
+            code, win, _, l0 = got
+            rows, cols = listed.nonzero(as_tuple=True)
+            acts = torch.where(keep, (u / s_) if use_s else hh, torch.zeros_like(hh))
+            assert torch.equal(code.idx.cpu().long(), cols) and torch.equal(code.val.cpu(), acts[rows, cols])
+            assert torch.equal(win.cpu(), (listed & (((u - theta).abs() < 0.5 * window) & (u > 0)))[rows, cols].float())
+            assert torch.equal(l0.cpu(), keep.sum(1).float())
+        else:
+            B = rng.choice([16, 64, 300]); d = rng.choice([64, 256, 768, 2048, 4096]); F = rng.choice([96, 256, 1000]); k = rng.choice([3, 8, 16])
+            dd = rng.choice([torch.float32, torch.bfloat16])
+            print(f"[{n}] adam_rowcoef seed={seed} B={B} d={d} F={F} k={k} {dd}", flush=True)
+            code = tk.random_code(pkg, dev, B, F, k, seed=seed)
+            fi = pkg.ops.build_feature_index(code)
+            dense = torch.randn(B, d, generator=g).to(dd).to(dev); coef = torch.randn(code.n_slots, generator=g).to(dev)
+            rc = (0.1 * torch.randn(F, generator=g)).to(dev)
+            p0 = torch.randn(F, d, generator=g).to(dev)
+            hy = dict(lr=4e-4, beta1=0.9, beta2=0.999, eps=1e-8)
+            pa, ma, va = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0); pb, mb, vb = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+            for step in (1, 2):
+                rows, _ = pkg.ops.sparse_grad_rows(fi, coef, dense, F, want_bias=True)
+                pkg.ops.adam_step(pa, rows, ma, va, step=step, row_len=d, row_grad_coef=rc, **hy)
+                pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=step, row_grad_coef=rc, **hy)
+                assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
+    assert n > 30
