@@ -88,8 +88,7 @@ template <bool BF16_IN, bool BF16_OUT>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
     int row_bytes /* d * sizeof(elem) */, int tiles_m, int tiles_n) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  // [x slab 0][x slab 1][w slab 0][w slab 1]
+  extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
 
   // ---- XCD-aware tile assignment ----
   const int bid = blockIdx.x;
@@ -329,14 +328,12 @@ static int launch_gemm(const void *x, const void *w, void *out, int64_t B, int64
   const int esz = BF16_IN ? 2 : 4;
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
   auto kern = encoder_gemm_kernel<BF16_IN, BF16_OUT>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       GEMM_LDS_BYTES);
-    if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "encoder_gemm: cannot reserve %d bytes of LDS: %s", GEMM_LDS_BYTES,
-                                     hipGetErrorString(e));
-    attr_set = true;
-  }
+  // asked for on every launch (a host-side table lookup): the attribute belongs to the kernel on the current device, and
+  // a cached "done" flag would be neither per device nor safe between threads
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     GEMM_LDS_BYTES);
+  if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "encoder_gemm: cannot reserve %d bytes of LDS: %s", GEMM_LDS_BYTES,
+                                   hipGetErrorString(e));
   // grid: 8 XCDs x (token tiles padded to 4) x (feature tiles per XCD padded to 8); padding workgroups exit at once
   const int m_pad = (tiles_m + 3) / 4 * 4, n_local_pad = ((tiles_n + 7) / 8 + 7) / 8 * 8;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,

@@ -451,8 +451,6 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
   SAE_REQUIRE(k >= 1 && k <= SEL_MAX_K, SAE_ERR_UNSUPPORTED, "select_topk_row: k=%d outside [1, %d]", k, SEL_MAX_K);
   SAE_REQUIRE(F < (1LL << 31) && B < (1LL << 31), SAE_ERR_UNSUPPORTED, "select_topk_row: size too large");
   SAE_REQUIRE(cand_cap >= 0 && cand_cap <= SEL_CAP, SAE_ERR_INVALID_ARG, "select_topk_row: cand_cap outside [0, %d]", SEL_CAP);
-  const int kk = k > F ? (int)F : k;
-  (void)kk;
   hipStream_t st = (hipStream_t)stream;
   const int V = pre_dtype == SAE_BF16 ? 8 : 4;
   const size_t row_bytes = (size_t)F * (pre_dtype == SAE_BF16 ? 2 : 4);
