@@ -3,23 +3,36 @@
 // Both operands are K-contiguous ("NT" GEMM), so a 16-byte piece of a row is exactly the 8 bf16
 // (or 4 fp32) one lane feeds to a matrix-core instruction.
 //
-// Tiling: one workgroup of 512 threads (8 waves of 64) owns a 256-token x 256-feature tile and
+// Tiling: one workgroup of 512 threads (8 waves of 64, two per SIMD) owns a 256-token x 256-feature tile and
 // walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32): a full cache line per row, which the
 // L2 serves at twice the rate of half lines (measured 27 vs 13 TB/s aggregate L2->LDS).  Waves are
 // arranged 2 x 4: each owns 128 tokens x 64 features (128 fp32 accumulators per lane): 8 x 4 tiles of
 // v_mfma_f32_16x16x32_bf16 for bf16 operands (two k-steps of 64 bytes per slab, a quarter wave per
-// 16-byte chunk; measured 1.28-1.30 against 1.22-1.23 PFLOP/s for 4 x 2 tiles of 32x32x16 at the
-// headline shape), 4 x 2 tiles of v_mfma_f32_32x32x2f32 for fp32 operands.
+// 16-byte chunk), 4 x 2 tiles of v_mfma_f32_32x32x2f32 for fp32 operands.
 //
-// Pipeline: LDS (all 160 KiB of the CU) is a ring of five 32 KiB slots; a slot holds one operand's
+// LDS (all 160 KiB of the CU) is a ring of five 32 KiB slots; a slot holds one operand's
 // slab (256 rows x 128 bytes).  Load units alternate W slab j, x slab j, W slab j+1, ...; unit t
 // lives in slot t % 5.  Slots are filled by LDS-direct loads (global_load_lds_dwordx4: the data
-// never passes through VGPRs).  While slab j is consumed, x slab j+1 and W slab j+2 are in flight:
-// the weights, which come from HBM, get the longer lead; the activations mostly hit L2 / Infinity
-// Cache.  One s_waitcnt vmcnt(4) + s_barrier per slab publishes the slab that just landed and
-// frees the two slots of the slab just consumed.  The loads are issued through inline assembly so
-// that the compiler's wait-count insertion does not serialise them against LDS reads of other
-// slots.
+// never passes through VGPRs), issued through inline assembly so that the compiler's wait-count
+// insertion does not serialise them against LDS reads of other slots.  While slab j is consumed, x slab j+1
+// and W slab j+2 are in flight: the weights, which come from HBM, get the longer lead; the activations
+// mostly hit L2 / Infinity Cache.
+//
+// bf16 operands, the schedule ("ping-pong"): the four waves that own tokens 0-127 of the tile (one per SIMD) and
+// the four that own tokens 128-255 alternate between a memory phase -- the 12 fragment reads of one k-step from
+// LDS plus 4 LDS-direct loads of 1 KiB -- and a matrix-core phase -- the k-step's 32 instructions.  A workgroup
+// barrier ends every phase and the second group runs one phase behind the first, so on every SIMD one wave
+// feeds the matrix cores while the other waits on LDS.  With all eight waves in the same phase (one barrier per
+// slab, loads and fragment reads interleaved with the matrix-core instructions by the compiler) the matrix cores
+// were busy 60 % of the cycles and each ingredient added its own time; with the phases they are busy 77 %
+// (3.49 -> 3.05 ms at B = d = 4096, F = 131072 on random operands).  What remains is the engine clock: it falls
+// as the matrix cores get busier (2.0 -> 1.8 GHz), the card is at its power limit.
+// A slab is read in phases 4j .. 4j+3 (phase numbers of the early group; the late group's step s runs in phase
+// 4j+s+1).  Early waves issue their quarter of x slab j+1 in phase 4j and of W slab j+2 in phase 4j+2, late
+// waves theirs in phases 4j+1 and 4j+3, into the slots slab j-1 left; every wave waits for all but its 4
+// youngest loads at the end of phase 4j+3, and the barrier that ends that phase publishes slab j+1.
+// fp32 operands keep the older schedule (one barrier per slab, four sub-phases, all waves in step): their
+// matrix-core time per byte is 16 times longer and hides everything else.
 //
 // LDS layout: row r of a slot is 128 bytes = 8 chunks of 16 bytes; chunk c is stored at physical
 // chunk c ^ ((r >> 1) & 7).  A group of 16 lanes then covers 256 distinct bytes when MFMA
@@ -33,9 +46,9 @@
 // store each lane's 4 features directly (8 or 16 bytes).
 //
 // Workgroup order: consecutive ids land on the 8 XCDs round-robin; within an XCD, 32 consecutive
-// workgroups (one per CU) cover 4 token tiles x 8 feature tiles, so every slab in an XCD's L2 is
-// shared by 8 or 4 resident workgroups (measured at the headline shape: 16x2 978, 8x4 1084, 4x8 1189,
-// 2x16 1107, 1x32 923 TFLOP/s).
+// workgroups (one per CU) cover RM token tiles x 32 / RM feature tiles, so every slab in an XCD's L2 is
+// shared by the resident workgroups (bf16: RM = 8 when there are at least 8 token tiles, 3.05 against 3.09 ms
+// for RM = 4 and 3.3 for RM = 2; fp32: RM = 4).
 //
 // Rows beyond B or F are clamped to the last valid row when loading (their products land in
 // accumulators that the epilogue never stores), so the main loop has no bounds checks.
@@ -59,20 +72,14 @@ constexpr int GEMM_LDS_BYTES = GEMM_SLOTS * GEMM_SLOT_BYTES;
 
 __device__ __forceinline__ int swz(int row, int chunk) { return row * GEMM_SLAB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
-template <bool BF16_IN>
-__device__ __forceinline__ void mma_chunk(const u32x4 &wf, const u32x4 &xf, f32x16_t &acc) {
-  if constexpr (BF16_IN) {
-    bf16x8_t a = __builtin_bit_cast(bf16x8_t, wf);
-    bf16x8_t b = __builtin_bit_cast(bf16x8_t, xf);
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
-  } else {
-    f32x4_t a = __builtin_bit_cast(f32x4_t, wf);
-    f32x4_t b = __builtin_bit_cast(f32x4_t, xf);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
-  }
+// one 16-byte chunk of K (4 fp32) of a 32 x 32 tile
+__device__ __forceinline__ void mma_chunk_f32(const u32x4 &wf, const u32x4 &xf, f32x16_t &acc) {
+  f32x4_t a = __builtin_bit_cast(f32x4_t, wf);
+  f32x4_t b = __builtin_bit_cast(f32x4_t, xf);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
 }
 
 // two floats -> two bf16 (round to nearest even, NaN stays a quiet NaN) without a branch
@@ -84,10 +91,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return (ha & 0xffffu) | (hb << 16);
 }
 
-template <bool BF16_IN, bool BF16_OUT>
-__global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
+// ---- fp32 operands ---------------------------------------------------------------------------------------------
+template <bool BF16_OUT>
+__global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
-    int row_bytes /* d * sizeof(elem) */, int tiles_m, int tiles_n) {
+    int row_bytes /* d * 4 */, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
 
   // ---- XCD-aware tile assignment ----
@@ -125,20 +133,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     lds_off[i] = (wave * 32 + i * 8) * GEMM_SLAB;  // wave-uniform base of the 1 KiB this load fills
   }
 
-  f32x16_t acc[BF16_IN ? 1 : 2][BF16_IN ? 1 : 4];  // fp32 operands: [feature sub-tile of 32][token sub-tile of 32]
-  f32x4_t acc16[BF16_IN ? 4 : 1][BF16_IN ? 8 : 1];  // bf16 operands: [feature sub-tile of 16][token sub-tile of 16]
+  f32x16_t acc[2][4];  // [feature sub-tile of 32][token sub-tile of 32]
 #pragma unroll
-  for (int i = 0; i < (BF16_IN ? 1 : 2); ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < (BF16_IN ? 1 : 4); ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-#pragma unroll
-  for (int i = 0; i < (BF16_IN ? 4 : 1); ++i)
-#pragma unroll
-    for (int j = 0; j < (BF16_IN ? 8 : 1); ++j)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) acc16[i][j][v] = 0.f;
 
   const int n_slabs = row_bytes / GEMM_SLAB;
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -181,7 +182,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
     __builtin_amdgcn_sched_barrier(0);
     const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
     const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
-    u32x4 wf16[4];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {  // 4 phases per slab, each with a quarter of the slab's loads and matrix-core work
       const int chunk = 2 * s + frag_half;
@@ -196,38 +196,16 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
           LDS_DMA16(wg[2 * s - 3] + (size_t)sB * GEMM_SLAB, slotB + lds_off[2 * s - 3]);
         }
       }
-      if constexpr (BF16_IN) {
-        // 16x16x32 instructions: a k-step is 64 bytes of K (4 chunks, one per quarter wave); phase s covers
-        // k-step s / 2 and the token sub-tiles 4 (s & 1) .. + 4; the W fragments of a k-step are read in its first phase
-        const int c16 = 4 * (s >> 1) + (lane >> 4);
-        if ((s & 1) == 0) {
+      // 32x32x2 fp32 instructions: phase s covers 32 bytes of K (two chunks, one per half wave)
+      u32x4 wf[2], xf[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) wf16[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 16 + (lane & 15), c16));
-        }
-        u32x4 xf16[4];
+      for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          xf16[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + ((s & 1) * 4 + j) * 16 + (lane & 15), c16));
+      for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 32 + frag_row, chunk));
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            bf16x8_t a = __builtin_bit_cast(bf16x8_t, wf16[i]);
-            bf16x8_t b = __builtin_bit_cast(bf16x8_t, xf16[j]);
-            acc16[i][(s & 1) * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc16[i][(s & 1) * 4 + j], 0, 0, 0);
-          }
-      } else {
-        // 32x32x2 fp32 instructions: phase s covers 32 bytes of K (two chunks, one per half wave)
-        u32x4 wf[2], xf[4];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 32 + frag_row, chunk));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 32 + frag_row, chunk));
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) mma_chunk<BF16_IN>(wf[i], xf[j], acc[i][j]);
-      }
+        for (int j = 0; j < 4; ++j) mma_chunk_f32(wf[i], xf[j], acc[i][j]);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -243,17 +221,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
       constexpr int PITCH = 136;
       __builtin_amdgcn_s_barrier();  // every wave is done reading operand slabs (and its own loads have landed)
       char *stage = lds + wave * (128 * PITCH);
-      if constexpr (BF16_IN) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            uint2 pk;
-            pk.x = pack_bf16x2(acc16[i][j][0], acc16[i][j][1]);
-            pk.y = pack_bf16x2(acc16[i][j][2], acc16[i][j][3]);
-            *reinterpret_cast<uint2 *>(stage + (j * 16 + (lane & 15)) * PITCH + (i * 16 + 4 * (lane >> 4)) * 2) = pk;
-          }
-      } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -265,7 +232,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
             pk.y = pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
             *reinterpret_cast<uint2 *>(stage + (j * 32 + frag_row) * PITCH + (i * 32 + 8 * g + 4 * frag_half) * 2) = pk;
           }
-      }
       // the region is private to the wave: no barrier, the compiler's wait on the LDS writes is enough
       uint16_t *obase = reinterpret_cast<uint16_t *>(out) + (size_t)(m0 + wm * 128) * N + n0 + wn * 64;
       const int r_in = lane >> 3, c16 = lane & 7;
@@ -281,19 +247,16 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
       return;
     }
   }
-  constexpr int SUB = BF16_IN ? 16 : 32, NJ = 128 / SUB, NI = 64 / SUB, NG = BF16_IN ? 1 : 4;
 #pragma unroll
-  for (int j = 0; j < NJ; ++j) {
-    const int tok = m0 + wm * 128 + j * SUB + (BF16_IN ? (lane & 15) : frag_row);
+  for (int j = 0; j < 4; ++j) {
+    const int tok = m0 + wm * 128 + j * 32 + frag_row;
     if (tok >= M) continue;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
+    for (int i = 0; i < 2; ++i) {
 #pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const int f = n0 + wn * 64 + i * SUB + (BF16_IN ? 4 * (lane >> 4) : 8 * g + 4 * frag_half);
-        float v0, v1, v2, v3;
-        if constexpr (BF16_IN) { v0 = acc16[i][j][0]; v1 = acc16[i][j][1]; v2 = acc16[i][j][2]; v3 = acc16[i][j][3]; }
-        else { v0 = acc[i][j][4 * g + 0]; v1 = acc[i][j][4 * g + 1]; v2 = acc[i][j][4 * g + 2]; v3 = acc[i][j][4 * g + 3]; }
+      for (int g = 0; g < 4; ++g) {
+        const int f = n0 + wn * 64 + i * 32 + 8 * g + 4 * frag_half;
+        const float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
         if constexpr (BF16_OUT) {
           uint16_t *o = reinterpret_cast<uint16_t *>(out) + (size_t)tok * N + f;
           if (f + 3 < N && (N & 3) == 0) {
@@ -323,21 +286,231 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_kernel(
   }
 }
 
-template <bool BF16_IN, bool BF16_OUT>
-static int launch_gemm(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, hipStream_t st) {
-  const int esz = BF16_IN ? 2 : 4;
-  const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
-  auto kern = encoder_gemm_kernel<BF16_IN, BF16_OUT>;
+// ---- bf16 operands ---------------------------------------------------------------------------------------------
+#define WAITCNT_VM(N) (((N) & 0xf) | (0x7 << 4) | (0xf << 8) | (((N) >> 4) << 14))
+#define WAITCNT_LGKM0 (0xf | (0x7 << 4) | (0x0 << 8) | (0x3 << 14))
+#define PHASE_BARRIER()                   \
+  __builtin_amdgcn_sched_barrier(0);      \
+  __builtin_amdgcn_s_barrier();           \
+  __builtin_amdgcn_sched_barrier(0)
+
+template <bool BF16_OUT>
+__global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
+    const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
+    int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
+
+  // ---- XCD-aware tile assignment: 32 consecutive workgroups of an XCD cover 2^rm_log2 token tiles x the rest in feature tiles
+  int tile_m, tile_n;
+  {
+    const int bid = blockIdx.x, xcd = bid & 7, slot = bid >> 3;
+    const int grp = slot >> 5, in = slot & 31;
+    const int rm = 1 << rm_log2, rn = 32 >> rm_log2;
+    const int m_groups = (tiles_m + rm - 1) >> rm_log2;
+    const int n_grp = grp / m_groups, m_part = grp % m_groups;
+    tile_m = m_part * rm + (in & (rm - 1));
+    tile_n = (n_grp * rn + (in >> rm_log2)) * 8 + xcd;
+    if (tile_n >= tiles_n || tile_m >= tiles_m) return;     // the whole workgroup leaves: no barrier is left short
+  }
+  const int m0 = tile_m * GEMM_BM, n0 = tile_n * GEMM_BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const bool late = wm != 0;          // the group that runs one phase behind
+
+  // ---- global -> LDS: every wave fills 32 rows of each operand slab with 4 loads of 1 KiB (8 lanes per 128-byte row,
+  // the chunk swizzle applied on the global side)
+  const char *xg[4], *wg[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = wave * 32 + i * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+    xg[i] = x + (size_t)(m0 + r < M ? m0 + r : M - 1) * row_bytes + chunk * 16;
+    wg[i] = w + (size_t)(n0 + r < N ? n0 + r : N - 1) * row_bytes + chunk * 16;
+  }
+  const uint32_t ld_base = (uint32_t)(wave * 32) * GEMM_SLAB;
+
+  f32x4_t acc[4][8];   // [feature sub-tile of 16][token sub-tile of 16]
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+  const int n_slabs = row_bytes / GEMM_SLAB;
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  // unit t of the load sequence: t even -> W slab t / 2, t odd -> x slab (t - 1) / 2; it lives in slot t % 5
+#define ISSUE_UNIT(UNIT, SLAB)                                                                                      \
+  {                                                                                                                 \
+    const uint32_t slot_ = lds_base + (uint32_t)((UNIT) % GEMM_SLOTS) * GEMM_SLOT_BYTES + ld_base;                  \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
+        LDS_DMA16(((UNIT) & 1 ? xg[i] : wg[i]) + (size_t)(SLAB) * GEMM_SLAB, slot_ + i * 1024);                     \
+  }
+  // at the end of the phase in which the last fragments of a slab are read, the next slab (x issued this slab, W a
+  // slab ago) must be in LDS: everything but this wave's 4 youngest loads (W two slabs ahead, if there is one)
+#define WAIT_NEXT_SLAB()                                                                 \
+  if (slab + 2 < n_slabs) __builtin_amdgcn_s_waitcnt(WAITCNT_VM(4));                     \
+  else __builtin_amdgcn_s_waitcnt(WAITCNT_VM(0))
+  ISSUE_UNIT(0, 0)
+  ISSUE_UNIT(1, 0)
+  if (n_slabs > 1) {
+    ISSUE_UNIT(2, 1)
+    __builtin_amdgcn_s_waitcnt(WAITCNT_VM(4));
+  } else {
+    __builtin_amdgcn_s_waitcnt(WAITCNT_VM(0));
+  }
+  PHASE_BARRIER();                      // slab 0 is in LDS
+  if (late) { PHASE_BARRIER(); }        // the late group sits out the first phase (the early group the last one)
+
+  const int frow = lane & 15, fq = lane >> 4;
+  u32x4 wf[4], xf[8];
+  // a k-step is 64 bytes of K: 4 chunks, one per quarter wave
+#define READ_FRAGS(KS)                                                                                              \
+  {                                                                                                                 \
+    const int c16_ = 4 * (KS) + fq;                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
+        wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 16 + frow, c16_));                          \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                                   \
+        xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 16 + frow, c16_));                         \
+  }
+#define MMA_STEP()                                                                                                  \
+  _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                                     \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                     \
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i]),                      \
+                                                          __builtin_bit_cast(bf16x8_t, xf[j]), acc[i][j], 0, 0, 0);
+
+  for (int slab = 0; slab < n_slabs; ++slab) {
+    const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
+    const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
+    // memory phase, k-step 0; x of the next slab goes into the slot the previous slab's W left
+    READ_FRAGS(0)
+    if (slab + 1 < n_slabs) ISSUE_UNIT(2 * slab + 3, slab + 1)
+    __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+    PHASE_BARRIER();
+    MMA_STEP()
+    PHASE_BARRIER();
+    // memory phase, k-step 1; W two slabs ahead goes into the slot the previous slab's x left
+    READ_FRAGS(1)
+    if (slab + 2 < n_slabs) ISSUE_UNIT(2 * slab + 4, slab + 2)
+    if (late) { WAIT_NEXT_SLAB(); }     // the late group's last reads of the slab: the phase the early group computes in
+    __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+    PHASE_BARRIER();
+    MMA_STEP()
+    if (!late) { WAIT_NEXT_SLAB(); }
+    PHASE_BARRIER();
+  }
+#undef ISSUE_UNIT
+#undef WAIT_NEXT_SLAB
+#undef READ_FRAGS
+#undef MMA_STEP
+  // The early group has one barrier to go (the late group's last matrix-core phase).  No wave reads operand slabs any
+  // more and every load has landed, so LDS is free: the early waves stage and store their output under that phase.
+
+  // ---- epilogue: lane holds, per (i, j): features 4 (lane / 16) .. + 3 of sub-tile i for token lane % 16 of sub-tile j
+  bool stored = false;
+  if constexpr (BF16_OUT) {
+    // Full tiles go through LDS so that global stores are whole 128-byte lines: every wave transposes its own
+    // 128-token x 64-feature block in a private region, rows padded to 136 bytes (the 8-byte writes of a quarter
+    // wave pair then fall on distinct banks), and writes it out 8 token rows per instruction.
+    if (m0 + GEMM_BM <= M && n0 + GEMM_BN <= N && (N & 63) == 0) {
+      constexpr int PITCH = 136;
+      char *stage = lds + wave * (128 * PITCH);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          uint2 pk;
+          pk.x = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+          pk.y = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+          *reinterpret_cast<uint2 *>(stage + (j * 16 + frow) * PITCH + (i * 16 + 4 * fq) * 2) = pk;
+        }
+      // the region is private to the wave: no barrier, the compiler's wait on the LDS writes is enough
+      uint16_t *obase = reinterpret_cast<uint16_t *>(out) + (size_t)(m0 + wm * 128) * N + n0 + wn * 64;
+      const int r_in = lane >> 3, c16 = lane & 7;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = q * 8 + r_in;
+        const char *src = stage + row * PITCH + c16 * 16;
+        const uint2 lo = *reinterpret_cast<const uint2 *>(src), hi = *reinterpret_cast<const uint2 *>(src + 8);
+        u32x4 v;
+        v.x = lo.x; v.y = lo.y; v.z = hi.x; v.w = hi.y;
+        *reinterpret_cast<u32x4 *>(obase + (size_t)row * N + c16 * 8) = v;
+      }
+      stored = true;
+    }
+  }
+  if (!stored) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int tok = m0 + wm * 128 + j * 16 + frow;
+      if (tok >= M) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int f = n0 + wn * 64 + i * 16 + 4 * fq;
+        const float v0 = acc[i][j][0], v1 = acc[i][j][1], v2 = acc[i][j][2], v3 = acc[i][j][3];
+        if constexpr (BF16_OUT) {
+          uint16_t *o = reinterpret_cast<uint16_t *>(out) + (size_t)tok * N + f;
+          if (f + 3 < N && (N & 3) == 0) {
+            uint2 pk;
+            pk.x = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+            pk.y = (uint32_t)f32_to_bf16_bits(v2) | ((uint32_t)f32_to_bf16_bits(v3) << 16);
+            *reinterpret_cast<uint2 *>(o) = pk;
+          } else {
+            if (f + 0 < N) o[0] = f32_to_bf16_bits(v0);
+            if (f + 1 < N) o[1] = f32_to_bf16_bits(v1);
+            if (f + 2 < N) o[2] = f32_to_bf16_bits(v2);
+            if (f + 3 < N) o[3] = f32_to_bf16_bits(v3);
+          }
+        } else {
+          float *o = reinterpret_cast<float *>(out) + (size_t)tok * N + f;
+          if (f + 3 < N && (N & 3) == 0) {
+            *reinterpret_cast<float4 *>(o) = make_float4(v0, v1, v2, v3);
+          } else {
+            if (f + 0 < N) o[0] = v0;
+            if (f + 1 < N) o[1] = v1;
+            if (f + 2 < N) o[2] = v2;
+            if (f + 3 < N) o[3] = v3;
+          }
+        }
+      }
+    }
+  }
+  if (!late) { PHASE_BARRIER(); }       // pairs with the late group's last phase
+}
+
+// grid: 8 XCDs x (token tiles padded to rm) x (feature tiles per XCD padded to 32 / rm); padding workgroups exit at once
+static int reserve_lds(const void *kern) {
   // asked for on every launch (a host-side table lookup): the attribute belongs to the kernel on the current device, and
   // a cached "done" flag would be neither per device nor safe between threads
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     GEMM_LDS_BYTES);
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);
   if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "encoder_gemm: cannot reserve %d bytes of LDS: %s", GEMM_LDS_BYTES,
                                    hipGetErrorString(e));
-  // grid: 8 XCDs x (token tiles padded to 4) x (feature tiles per XCD padded to 8); padding workgroups exit at once
+  return SAE_OK;
+}
+
+template <bool BF16_OUT>
+static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, hipStream_t st) {
+  const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
+  auto kern = encoder_gemm_f32_kernel<BF16_OUT>;
+  const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
+  if (rc != SAE_OK) return rc;
   const int m_pad = (tiles_m + 3) / 4 * 4, n_local_pad = ((tiles_n + 7) / 8 + 7) / 8 * 8;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
-                     (const char *)w, out, (int)B, (int)F, (int)(d * esz), tiles_m, tiles_n);
+                     (const char *)w, out, (int)B, (int)F, (int)(d * 4), tiles_m, tiles_n);
+  return check_launch("encoder_gemm");
+}
+
+template <bool BF16_OUT>
+static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, hipStream_t st) {
+  const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
+  auto kern = encoder_gemm_bf16_kernel<BF16_OUT>;
+  const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
+  if (rc != SAE_OK) return rc;
+  const int rm_log2 = tiles_m >= 8 ? 3 : 2, rm = 1 << rm_log2, rn = 32 >> rm_log2;
+  const int m_pad = (tiles_m + rm - 1) / rm * rm, n_local_pad = ((tiles_n + 7) / 8 + rn - 1) / rn * rn;
+  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
+                     (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2);
   return check_launch("encoder_gemm");
 }
 
@@ -358,9 +531,9 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
               "encoder_gemm: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   if (in_dtype == SAE_BF16) {
-    return out_dtype == SAE_BF16 ? launch_gemm<true, true>(x, w_enc_t, pre, B, d, F, st)
-                                 : launch_gemm<true, false>(x, w_enc_t, pre, B, d, F, st);
+    return out_dtype == SAE_BF16 ? launch_gemm_bf16<true>(x, w_enc_t, pre, B, d, F, st)
+                                 : launch_gemm_bf16<false>(x, w_enc_t, pre, B, d, F, st);
   }
-  return out_dtype == SAE_BF16 ? launch_gemm<false, true>(x, w_enc_t, pre, B, d, F, st)
-                               : launch_gemm<false, false>(x, w_enc_t, pre, B, d, F, st);
+  return out_dtype == SAE_BF16 ? launch_gemm_f32<true>(x, w_enc_t, pre, B, d, F, st)
+                               : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
 }
