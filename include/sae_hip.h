@@ -125,6 +125,23 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
 int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int k,
                              int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream);
 
+/* The encoder product and the per-token TopK with the row read only where it matters.
+ * sae_encoder_gemm_granule_max: sae_encoder_gemm for bf16 operands and bf16 output (F % 64 == 0) whose epilogue
+ *   also writes granule_max [B, F / 64] (uint32): for every token and every aligned granule of 64 features the
+ *   largest select key of the granule, the key of an element being the bit pattern of
+ *   h1 = (bf16(pre) + b_enc) * scale when h1 > 0 and 0 otherwise (b_enc / scale nullable: 0 / 1).
+ * sae_select_topk_row_granule: the result of sae_select_topk_row (same outputs, bit for bit) from pre and
+ *   granule_max: the k-th largest granule maximum bounds the k-th largest key from below, so only the ~k granules
+ *   that reach it are read from pre.  F % 64 == 0, F <= 262144, k <= 512; rows whose candidates do not fit the
+ *   in-LDS list (mass ties) are redone from the whole row by a second launch of the general kernel.
+ * Together they replace `hidden_pre = x @ W_E + b_E` followed by the TopK of `hidden_pre * decoder_norm`
+ * (models/sae.py:324-341, utils/math.py:81-171). */
+int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d, int64_t F,
+                                 const float *b_enc, const float *scale, uint32_t *granule_max, void *stream);
+int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
+                                int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
+                                void *stream);
+
 /* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
  * (h0, h1 as above); ties at the threshold -> lowest flattened index b * F + f.  If fewer than
  * k_total entries are positive, all positives are kept.

@@ -82,6 +82,14 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Ordering key of one pre-activation in the TopK selects: the bit pattern of h1 = (pre + b_enc) * scale when h1 > 0 and
+// 0 otherwise (for positive floats unsigned-integer order equals float order; non-positive entries are never kept).
+// One definition for the select kernels and for the GEMM epilogue that emits per-granule maxima of these keys.
+__device__ __forceinline__ uint32_t select_key_plain(float pre, float b, float s) {
+  const float h1 = (pre + b) * s;
+  return h1 > 0.f ? __float_as_uint(h1) : 0u;
+}
+
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

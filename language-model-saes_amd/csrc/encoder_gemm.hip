@@ -82,13 +82,10 @@ __device__ __forceinline__ void mma_chunk_f32(const u32x4 &wf, const u32x4 &xf, 
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
 }
 
-// two floats -> two bf16 (round to nearest even, NaN stays a quiet NaN) without a branch
+// two floats -> two bf16, round to nearest even: the packed hardware conversion
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
-  const uint32_t ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16, rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) >> 16;
-  const uint32_t ha = (ua & 0x7fffffffu) > 0x7f800000u ? ((ua >> 16) | 0x0040u) : ra;
-  const uint32_t hb = (ub & 0x7fffffffu) > 0x7f800000u ? ((ub >> 16) | 0x0040u) : rb;
-  return (ha & 0xffffu) | (hb << 16);
+  const cvt_f32x2 in = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, cvt_bf16x2));
 }
 
 // ---- fp32 operands ---------------------------------------------------------------------------------------------
@@ -294,10 +291,14 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
   __builtin_amdgcn_s_barrier();           \
   __builtin_amdgcn_sched_barrier(0)
 
-template <bool BF16_OUT>
+// GMAX (bf16 output, N a multiple of 64): the epilogue also writes, for every token and every aligned granule of 64
+// features, the largest select key of the granule's rounded outputs to gmax[token][N / 64]; the wave's 64 features are
+// one granule.
+template <bool BF16_OUT, bool GMAX>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
-    int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2) {
+    int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
+    const float *__restrict__ scale, uint32_t *__restrict__ gmax) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
 
   // ---- XCD-aware tile assignment: 32 consecutive workgroups of an XCD cover 2^rm_log2 token tiles x the rest in feature tiles
@@ -380,6 +381,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i]),                      \
                                                           __builtin_bit_cast(bf16x8_t, xf[j]), acc[i][j], 0, 0, 0);
 
+  // GMAX: this lane's 16 bias and 16 scale values, asked for here so that the epilogue does not wait for them
+  float bb[GMAX ? 4 : 1][4], ss[GMAX ? 4 : 1][4];
+  if constexpr (GMAX) {
+    const int f0 = n0 + wn * 64;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int f = f0 + i * 16 + 4 * fq;
+      const bool ok = f0 < N;
+      const float4 b4 = b_enc && ok ? *reinterpret_cast<const float4 *>(b_enc + f) : make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 s4 = scale && ok ? *reinterpret_cast<const float4 *>(scale + f) : make_float4(1.f, 1.f, 1.f, 1.f);
+      bb[i][0] = b4.x; bb[i][1] = b4.y; bb[i][2] = b4.z; bb[i][3] = b4.w;
+      ss[i][0] = s4.x; ss[i][1] = s4.y; ss[i][2] = s4.z; ss[i][3] = s4.w;
+    }
+  }
   for (int slab = 0; slab < n_slabs; ++slab) {
     const char *lw = lds + ((2 * slab) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
     const char *lx = lds + ((2 * slab + 1) % GEMM_SLOTS) * GEMM_SLOT_BYTES;
@@ -408,6 +423,31 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
   // more and every load has landed, so LDS is free: the early waves stage and store their output under that phase.
 
   // ---- epilogue: lane holds, per (i, j): features 4 (lane / 16) .. + 3 of sub-tile i for token lane % 16 of sub-tile j
+  if constexpr (GMAX) {
+    const int f0 = n0 + wn * 64;
+    if (f0 < N) {
+      const int ng = N >> 6;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        // positive floats order like their bit patterns, so the largest key is the key of the largest h1; the maximum
+        // starts at 0 and v_max ignores NaN operands, as the key of a NaN (0) is ignored
+        float hmax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // the accumulators take their rounded values here, so the stores below write exactly what the keys were formed from
+          const uint32_t lo = pack_bf16x2(acc[i][j][0], acc[i][j][1]), hi = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+          acc[i][j][0] = __uint_as_float(lo << 16); acc[i][j][1] = __uint_as_float(lo & 0xffff0000u);
+          acc[i][j][2] = __uint_as_float(hi << 16); acc[i][j][3] = __uint_as_float(hi & 0xffff0000u);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) hmax = fmaxf(hmax, (acc[i][j][r] + bb[i][r]) * ss[i][r]);   // h1 of select_key_plain
+        }
+        hmax = fmaxf(hmax, __shfl_xor(hmax, 16, 64));
+        hmax = fmaxf(hmax, __shfl_xor(hmax, 32, 64));
+        const int tok = m0 + wm * 128 + j * 16 + frow;
+        if (fq == 0 && tok < M) gmax[(size_t)tok * ng + (f0 >> 6)] = hmax > 0.f ? __float_as_uint(hmax) : 0u;
+      }
+    }
+  }
   bool stored = false;
   if constexpr (BF16_OUT) {
     // Full tiles go through LDS so that global stores are whole 128-byte lines: every wave transposes its own
@@ -501,16 +541,17 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
   return check_launch("encoder_gemm");
 }
 
-template <bool BF16_OUT>
-static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, hipStream_t st) {
+template <bool BF16_OUT, bool GMAX>
+static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
+                            const float *scale, uint32_t *gmax, hipStream_t st) {
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
-  auto kern = encoder_gemm_bf16_kernel<BF16_OUT>;
+  auto kern = encoder_gemm_bf16_kernel<BF16_OUT, GMAX>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
   if (rc != SAE_OK) return rc;
   const int rm_log2 = tiles_m >= 8 ? 3 : 2, rm = 1 << rm_log2, rn = 32 >> rm_log2;
   const int m_pad = (tiles_m + rm - 1) / rm * rm, n_local_pad = ((tiles_n + 7) / 8 + rn - 1) / rn * rn;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
-                     (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2);
+                     (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale, gmax);
   return check_launch("encoder_gemm");
 }
 
@@ -531,9 +572,24 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
               "encoder_gemm: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   if (in_dtype == SAE_BF16) {
-    return out_dtype == SAE_BF16 ? launch_gemm_bf16<true>(x, w_enc_t, pre, B, d, F, st)
-                                 : launch_gemm_bf16<false>(x, w_enc_t, pre, B, d, F, st);
+    return out_dtype == SAE_BF16 ? launch_gemm_bf16<true, false>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st)
+                                 : launch_gemm_bf16<false, false>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st);
   }
   return out_dtype == SAE_BF16 ? launch_gemm_f32<true>(x, w_enc_t, pre, B, d, F, st)
                                : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
+}
+
+extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d,
+                                            int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
+                                            void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x_bf16 && w_enc_t_bf16 && pre_bf16 && granule_max, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: B, d, F must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: size too large");
+  SAE_REQUIRE(d % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: d_model=%lld must be a multiple of 64", (long long)d);
+  SAE_REQUIRE(F % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: F=%lld must be a multiple of 64 (whole granules)",
+              (long long)F);
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_enc_t_bf16 | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0,
+              SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: pointers must be 16-byte aligned");
+  return launch_gemm_bf16<true, true>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream);
 }

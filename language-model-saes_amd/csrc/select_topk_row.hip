@@ -30,6 +30,7 @@ constexpr int SEL_THREADS = 1024;
 constexpr int SEL_WAVES = SEL_THREADS / 64;
 constexpr int SEL_CAP = 4096;      // candidate capacity == largest supported k
 constexpr int SEL_MAX_K = 4096;
+constexpr int SEL_ROW_FLAG = -1;   // row_nnz of a row the granule kernel left to the general kernel
 
 struct SelShared {
   uint32_t cand_key[SEL_CAP];
@@ -51,19 +52,21 @@ __device__ __forceinline__ float sel_bf16_round(float x) { return bf16_round(x);
 constexpr int SEL_PLAIN = 0, SEL_LOWP = 1, SEL_MASKED = 2;
 template <int ARITH>
 __device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm) {
+  if constexpr (ARITH == SEL_PLAIN) return select_key_plain(pre, b, s);
   float h1;
   if constexpr (ARITH == SEL_LOWP) {
     h1 = sel_bf16_round(mul_rn(sel_bf16_round(add_rn(pre, b)), s));
   } else {
     h1 = (pre + b) * s;
-    if constexpr (ARITH == SEL_MASKED) h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
+    h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
   }
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
 
 // Scan hist[255..0] from the top and find the bin where the running count reaches
 // `remaining`.  Executed by wave 0; results go to sh->prefix / sh->remaining.
-__device__ __forceinline__ void pick_digit(SelShared *sh, int shift) {
+template <typename SH>
+__device__ __forceinline__ void pick_digit(SH *sh, int shift) {
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     // lane 0 owns the top four bins (255..252), lane 63 the bottom four
@@ -95,8 +98,8 @@ __device__ __forceinline__ void pick_digit(SelShared *sh, int shift) {
 // Exact k-th largest of `n` keys held in LDS (n >= k >= 1).  On return (after the final
 // barrier) sh->prefix is that key and sh->remaining the number of elements equal to it that
 // belong to the top k.  `xform` maps a stored key to the ordering key.
-template <typename KeyAt>
-__device__ __forceinline__ void lds_kth_largest(SelShared *sh, int n, int k, KeyAt key_at) {
+template <int THREADS = SEL_THREADS, typename SH, typename KeyAt>
+__device__ __forceinline__ void lds_kth_largest(SH *sh, int n, int k, KeyAt key_at) {
   if (threadIdx.x == 0) { sh->prefix = 0u; sh->remaining = k; }
   uint32_t mask = 0u;
 #pragma unroll 1
@@ -104,7 +107,7 @@ __device__ __forceinline__ void lds_kth_largest(SelShared *sh, int n, int k, Key
     if (threadIdx.x < 256) sh->hist[threadIdx.x] = 0u;
     __syncthreads();
     const uint32_t prefix = sh->prefix;
-    for (int i = threadIdx.x; i < n; i += SEL_THREADS) {
+    for (int i = threadIdx.x; i < n; i += THREADS) {
       const uint32_t key = key_at(i);
       if ((key & mask) == prefix) atomicAdd(&sh->hist[(key >> shift) & 255u], 1u);
     }
@@ -233,10 +236,11 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
     int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
-    int32_t *__restrict__ row_nnz, int cand_cap) {
+    int32_t *__restrict__ row_nnz, int cand_cap, int only_flagged) {
   __shared__ SelShared sh;
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
+  if (only_flagged && row_nnz[b] != SEL_ROW_FLAG) return;     // the pass after the granule kernel: rows it gave up on
   RowReader<BF16, ARITH> rr;
   rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
@@ -444,7 +448,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
 namespace sae {
 static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const float *b_enc, const float *scale,
                                 const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,
-                                int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream) {
+                                int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream, int only_flagged = 0) {
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
   SAE_REQUIRE(B > 0 && F > 0, SAE_ERR_INVALID_ARG, "select_topk_row: B and F must be positive");
   SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_row: bad dtype %d", pre_dtype);
@@ -459,7 +463,7 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
                      (((((uintptr_t)pre) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)feat_mask) & 15) == 0);
 #define SAE_LAUNCH_SELECT(BF, ST, ...)                                                                                     \
   hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
-                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap)
+                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged)
   if (lowp) {
     if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP);
   } else if (feat_mask) {
@@ -476,7 +480,165 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
 #undef SAE_LAUNCH_SELECT
   return check_launch("select_topk_row");
 }
+// ---- select from per-granule maxima -----------------------------------------------------------------------------
+// The encoder GEMM can leave, next to pre [B, F] (bf16), the largest key of every aligned granule of 64 features
+// (gmax [B, F / 64]).  The k-th largest granule maximum is a lower bound L of the row's k-th largest key (k distinct
+// elements reach it), and only granules whose maximum reaches L can hold a kept element: about k of them.  One
+// workgroup of 256 threads per token reads the granule maxima (F / 16 bytes instead of the row's 2 F), radix-selects
+// L among them in LDS, re-forms the keys of the qualifying granules from memory and finishes like the kernel above:
+// exact threshold among the candidates, lowest indices among ties, ascending order.  Rows whose candidates do not fit
+// (mass ties) are flagged in row_nnz and redone by the general kernel in a second launch that skips every other row.
+constexpr int GS_THREADS = 256;
+constexpr int GS_CAP = 1024;            // candidates per row
+constexpr int GS_QCAP = 1024;           // qualifying granules per row
+constexpr int GS_MAX_K = 512;
+constexpr int GS_MAX_GRANULES = 4096;   // F <= 262144
+
+struct GsShared {
+  uint32_t cand_key[GS_CAP];
+  int32_t cand_idx[GS_CAP];
+  uint16_t q[GS_QCAP];
+  uint32_t hist[256];
+  int32_t count, qcount, gpos;
+  uint32_t prefix;
+  int32_t remaining, digit_found;
+};
+
+__global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
+    const uint16_t *__restrict__ pre, const uint32_t *__restrict__ gmax, const float *__restrict__ b_enc,
+    const float *__restrict__ scale, int F, int k, int32_t *__restrict__ idx_out, float *__restrict__ val_out,
+    int64_t *__restrict__ row_off, int32_t *__restrict__ row_nnz) {
+  __shared__ GsShared sh;
+  extern __shared__ __attribute__((aligned(16))) uint32_t gk[];   // the row's granule maxima
+  const int b = blockIdx.x, tid = threadIdx.x, ng = F >> 6;
+  RowReader<true, SEL_PLAIN> rr;
+  rr.row = pre + (size_t)b * F;
+  rr.b_enc = b_enc;
+  rr.scale = scale;
+  rr.fmask = nullptr;
+  rr.F = F;
+  if (tid == 0) { sh.count = 0; sh.qcount = 0; sh.gpos = 0; }
+  __syncthreads();
+  int my_pos = 0;
+  const uint32_t *grow = gmax + (size_t)b * ng;
+  for (int g = tid; g < ng; g += GS_THREADS) {
+    const uint32_t key = grow[g];
+    gk[g] = key;
+    my_pos += key != 0u;
+  }
+  my_pos = wave_sum_i(my_pos);
+  if ((tid & 63) == 0 && my_pos) atomicAdd(&sh.gpos, my_pos);
+  __syncthreads();
+  const int n_gpos = sh.gpos;
+  if (n_gpos == 0) {        // no positive element in the row
+    if (tid == 0) { row_off[b] = (int64_t)b * k; row_nnz[b] = 0; }
+    for (int i = tid; i < k; i += GS_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
+    return;
+  }
+  // with fewer than k positive granules every positive element is a candidate (their count decides how many are kept)
+  uint32_t L = 1u;
+  if (n_gpos >= k) {
+    lds_kth_largest<GS_THREADS>(&sh, ng, k, [&](int i) { return gk[i]; });
+    L = sh.prefix;
+    __syncthreads();
+  }
+  for (int g = tid; g < ng; g += GS_THREADS) {
+    if (gk[g] >= L) {
+      const int slot = atomicAdd(&sh.qcount, 1);
+      if (slot < GS_QCAP) sh.q[slot] = (uint16_t)g;
+    }
+  }
+  __syncthreads();
+  const int nq = sh.qcount;
+  bool give_up = nq > GS_QCAP;
+  if (!give_up) {
+    for (int p = tid; p < nq * 8; p += GS_THREADS) {     // one 16-byte chunk of a qualifying granule per thread and round
+      const int c = (int)sh.q[p >> 3] * 8 + (p & 7);
+      uint32_t keys[8];
+      rr.chunk_keys(c, keys);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (keys[e] >= L) {
+          const int slot = atomicAdd(&sh.count, 1);
+          if (slot < GS_CAP) { sh.cand_key[slot] = keys[e]; sh.cand_idx[slot] = c * 8 + e; }
+        }
+      }
+    }
+    __syncthreads();
+    give_up = sh.count > GS_CAP;
+  }
+  if (give_up) {
+    if (tid == 0) row_nnz[b] = SEL_ROW_FLAG;
+    return;
+  }
+  const int n_cand = sh.count;
+  const int k_eff = n_cand < k ? n_cand : k;
+  if (n_cand > k_eff) {
+    // ---- exact threshold among the candidates ----
+    lds_kth_largest<GS_THREADS>(&sh, n_cand, k_eff, [&](int i) { return sh.cand_key[i]; });
+    const uint32_t T = sh.prefix;
+    const int need = sh.remaining;
+    __syncthreads();
+    int my_ties = 0;
+    for (int i = tid; i < n_cand; i += GS_THREADS) my_ties += sh.cand_key[i] == T;
+    if (tid == 0) sh.count = 0;
+    __syncthreads();
+    my_ties = wave_sum_i(my_ties);
+    if ((tid & 63) == 0 && my_ties) atomicAdd(&sh.count, my_ties);
+    __syncthreads();
+    const int n_ties = sh.count;
+    __syncthreads();
+    uint32_t idx_limit = 0xffffffffu;
+    if (n_ties > need) {     // ties at the threshold: the lowest indices are kept
+      lds_kth_largest<GS_THREADS>(&sh, n_cand, need, [&](int i) { return sh.cand_key[i] == T ? ~(uint32_t)sh.cand_idx[i] : 0u; });
+      idx_limit = ~sh.prefix;
+      __syncthreads();
+    }
+    for (int i = tid; i < n_cand; i += GS_THREADS) {
+      const uint32_t key = sh.cand_key[i];
+      const bool keep = key > T || (key == T && (uint32_t)sh.cand_idx[i] <= idx_limit);
+      if (!keep) sh.cand_key[i] = 0u;
+    }
+    __syncthreads();
+  }
+  // ---- rank the kept candidates by index and write them out in ascending order ----
+  for (int i = tid; i < n_cand; i += GS_THREADS) {
+    const uint32_t key = sh.cand_key[i];
+    if (key == 0u) continue;
+    const int my_idx = sh.cand_idx[i];
+    int rank = 0;
+    for (int j = 0; j < n_cand; ++j) rank += (sh.cand_key[j] != 0u) && (sh.cand_idx[j] < my_idx);
+    const float h1 = __uint_as_float(key);
+    if (rank < k) {
+      idx_out[(size_t)b * k + rank] = my_idx;
+      val_out[(size_t)b * k + rank] = scale ? h1 / scale[my_idx] : h1;
+    }
+  }
+  for (int i = k_eff + tid; i < k; i += GS_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
+  if (tid == 0) { row_off[b] = (int64_t)b * k; row_nnz[b] = k_eff; }
+}
+
 }  // namespace sae
+
+extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                           const float *scale, int64_t B, int64_t F, int k, int32_t *idx, float *val,
+                                           int64_t *row_off, int32_t *row_nnz, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre_bf16 && granule_max && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row_granule: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "select_topk_row_granule: bad sizes");
+  SAE_REQUIRE(F % 64 == 0 && F / 64 <= GS_MAX_GRANULES, SAE_ERR_UNSUPPORTED,
+              "select_topk_row_granule: F=%lld must be a multiple of 64, at most %d", (long long)F, 64 * GS_MAX_GRANULES);
+  SAE_REQUIRE(k >= 1 && k <= GS_MAX_K, SAE_ERR_UNSUPPORTED, "select_topk_row_granule: k=%d outside [1, %d]", k, GS_MAX_K);
+  SAE_REQUIRE((((uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "select_topk_row_granule: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(select_topk_row_granule_kernel, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
+                     (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz);
+  const int rc = check_launch("select_topk_row_granule");
+  if (rc != SAE_OK) return rc;
+  // rows the granule kernel flagged (mass ties) are redone from the whole row; every other workgroup leaves at once
+  return select_topk_row_impl(false, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1);
+}
 
 extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
                                       const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,

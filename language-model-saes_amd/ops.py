@@ -288,6 +288,39 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     return pre
 
 
+GRANULE = 64                 # features per granule of the granule-maximum route
+GRANULE_MAX_F = 64 * 4096
+GRANULE_MAX_K = 512
+
+
+def granule_route_supported(d: int, F: int, k: int) -> bool:
+    """Shapes `encoder_gemm_granule_max` + `select_topk_row(..., granule_max=...)` take."""
+    return d % 64 == 0 and F % GRANULE == 0 and F <= GRANULE_MAX_F and 1 <= k <= GRANULE_MAX_K
+
+
+def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Optional[torch.Tensor],
+                             scale: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16 pre[B, F] = x @ w_enc_t^T plus granule_max [B, F / 64] (int32 holding uint32 keys): per token and aligned
+    granule of 64 features the largest select key, i.e. the bits of (pre + b_enc) * scale where that is positive."""
+    _req(x, "x", torch.bfloat16, 2)
+    _req(w_enc_t, "w_enc_t", torch.bfloat16, 2)
+    B, d = x.shape
+    F, d2 = w_enc_t.shape
+    if d != d2:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
+    for name, t in (("b_enc", b_enc), ("scale", scale)):
+        if t is not None:
+            _req(t, name, torch.float32, 1)
+            if t.numel() != F:
+                raise ValueError(f"{name} must have {F} elements")
+    pre = torch.empty(B, F, dtype=torch.bfloat16, device=x.device)
+    gmax = torch.empty(B, max(F // GRANULE, 1), dtype=torch.int32, device=x.device)
+    with _timed("encoder_gemm"):
+        check(_lib.load().sae_encoder_gemm_granule_max(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _ptr(b_enc),
+                                                       _ptr(scale), gmax.data_ptr(), _stream(x)), "encoder_gemm_granule_max")
+    return pre, gmax
+
+
 # ---- select ---------------------------------------------------------------------------------
 
 def select_topk_row(
@@ -298,13 +331,22 @@ def select_topk_row(
     cand_cap: Optional[int] = None,
     feat_mask: Optional[torch.Tensor] = None,
     lowp: bool = False,
+    granule_max: Optional[torch.Tensor] = None,
 ) -> SparseCode:
     """Per-token TopK of (pre + b_enc) * scale.  `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the
-    arithmetic of a dictionary whose parameters are bf16 tensors)."""
+    arithmetic of a dictionary whose parameters are bf16 tensors).  `granule_max`: the second output of
+    `encoder_gemm_granule_max` for the same pre, b_enc and scale; the row is then read only where a kept element
+    can be (same result)."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
     if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None or feat_mask is not None):
         raise ValueError("lowp select takes a bf16 pre and neither cand_cap nor feat_mask")
+    if granule_max is not None:
+        if lowp or cand_cap is not None or feat_mask is not None or pre.dtype != torch.bfloat16:
+            raise ValueError("the granule route takes a bf16 pre and none of lowp, cand_cap, feat_mask")
+        _req(granule_max, "granule_max", torch.int32, 2)
+        if tuple(granule_max.shape) != (B, F // GRANULE) or F % GRANULE:
+            raise ValueError(f"granule_max must be [{B}, {F}/{GRANULE}]")
     for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
         if t is not None:
             _req(t, name, torch.float32, 1)
@@ -320,7 +362,10 @@ def select_topk_row(
     lib = _lib.load()
     _t = _timed("select_topk_row")
     _t.__enter__()
-    if lowp:
+    if granule_max is not None:
+        rc = lib.sae_select_topk_row_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k,
+                                             idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+    elif lowp:
         rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(), val.data_ptr(),
                                           row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     elif cand_cap is None and feat_mask is None:

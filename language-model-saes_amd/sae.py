@@ -220,24 +220,35 @@ class _FusedSparseStep(torch.autograd.Function):
         if lowp:
             b_E = b_E.float()
             b_D = b_D.float() if b_D is not None else None
-        if amp:
+        B = x.shape[0]
+        batch_wide = sae.cfg.act_fn.lower() == "batchtopk"
+        # per-token TopK on bf16 operands: the GEMM's epilogue leaves the largest select key of every 64-feature granule,
+        # and the select reads the row only in the granules that can hold a kept element.  The keys need the decoder
+        # norms, so this route fetches them before the GEMM (and waits there for an overlapped decoder update).
+        granule = (amp and not lowp and not batch_wide and getattr(sae, "granule_select", True)
+                   and not sae._update_pending() and ops.granule_route_supported(x.shape[1], w_enc_op.shape[0], int(k)))
+        gmax = None
+        if granule:
+            x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
+            scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
+            pre, gmax = ops.encoder_gemm_granule_max(x_op, w_enc_op, b_E, scale)
+        elif amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)
         else:
             x_op = x.contiguous()
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.float32)
-        # decoder-side operands are fetched after the GEMM is enqueued: an overlapped decoder update of the
-        # previous step (see HipAdam) is waited for here, not before the GEMM
-        scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
-        if lowp and scale is not None:
-            scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
+        if not granule:
+            # decoder-side operands are fetched after the GEMM is enqueued: an overlapped decoder update of the
+            # previous step (see HipAdam) is waited for here, not before the GEMM
+            scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
+            if lowp and scale is not None:
+                scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
         w_dec_op = sae._w_dec_operand(amp)
-        B = x.shape[0]
-        batch_wide = sae.cfg.act_fn.lower() == "batchtopk"
         if batch_wide:
             code = ops.select_topk_batch(pre, b_E, scale, k * B)
         else:
-            code = ops.select_topk_row(pre, b_E, scale, k, lowp=lowp)
+            code = ops.select_topk_row(pre, b_E, scale, k, lowp=lowp, granule_max=gmax)
         aux = holder.aux
         grad_recon_b16 = None   # set by the route that already has grad_recon in bf16
         if aux is None:
@@ -630,6 +641,9 @@ class SparseAutoEncoder(SparseDictionary):
     # ---- an optimiser may still be updating W_D on another stream (see HipAdam.overlap_decoder_update) ----
     def set_pending_update(self, event) -> None:
         self._pending_update = event
+
+    def _update_pending(self) -> bool:
+        return getattr(self, "_pending_update", None) is not None
 
     def wait_pending_update(self) -> None:
         ev = getattr(self, "_pending_update", None)

@@ -1,0 +1,135 @@
+"""The granule route of the per-token TopK: the encoder GEMM's per-granule key maxima and the select that reads the
+row only where those maxima allow a kept element, against the kernels they stand in for.  Everything here is
+integer-exact: the same pre-activations (bit for bit), the same keys, the same kept indices and values."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, d, F, seed, dev, scale_kind="random", bias=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(F, d, generator=g) / d ** 0.5).to(torch.bfloat16).to(dev)
+    b = (0.1 * torch.randn(F, generator=g)).to(dev) if bias else None
+    s = None
+    if scale_kind == "random":
+        s = (0.5 + torch.rand(F, generator=g)).to(dev)
+    return x, w, b, s
+
+
+def _keys(pre, b, s):
+    h1 = pre.float()
+    if b is not None:
+        h1 = h1 + b
+    if s is not None:
+        h1 = h1 * s
+    bits = h1.contiguous().view(torch.int32)
+    return torch.where(h1 > 0, bits, torch.zeros_like(bits))
+
+
+@pytest.mark.parametrize("B,d,F", [(300, 128, 1024), (256, 256, 4096), (77, 64, 192), (512, 64, 64)])
+@pytest.mark.parametrize("bias,scale_kind", [(True, "random"), (False, None)])
+def test_gemm_granule_max_matches_keys_of_its_own_output(pkg, dev, B, d, F, bias, scale_kind):
+    x, w, b, s = _inputs(B, d, F, seed=B + F, dev=dev, scale_kind=scale_kind, bias=bias)
+    pre, gmax = pkg.ops.encoder_gemm_granule_max(x, w, b, s)
+    want_pre = pkg.ops.encoder_gemm(x, w, torch.bfloat16)
+    assert torch.equal(pre, want_pre)
+    want = _keys(pre, b, s).view(B, F // 64, 64).max(dim=2).values     # positive-float bits order like ints
+    assert torch.equal(gmax, want)
+
+
+CASES = [
+    # B, d, F, k
+    (128, 128, 2048, 16),
+    (300, 128, 8192, 64),
+    (64, 64, 64, 8),          # one granule
+    (96, 128, 1024, 512),     # the largest k the route takes
+    (50, 256, 16384, 100),
+]
+
+
+@pytest.mark.parametrize("B,d,F,k", CASES)
+def test_granule_select_equals_row_select(pkg, dev, B, d, F, k):
+    x, w, b, s = _inputs(B, d, F, seed=3 * B + k, dev=dev)
+    pre, gmax = pkg.ops.encoder_gemm_granule_max(x, w, b, s)
+    got = pkg.ops.select_topk_row(pre, b, s, k, granule_max=gmax)
+    want = pkg.ops.select_topk_row(pre, b, s, k)
+    assert torch.equal(got.row_nnz, want.row_nnz) and torch.equal(got.row_off, want.row_off)
+    assert torch.equal(got.idx, want.idx) and torch.equal(got.val, want.val)
+
+
+def _granule_max_of(pre, b, s):
+    B, F = pre.shape
+    return _keys(pre, b, s).view(B, F // 64, 64).max(dim=2).values.contiguous()
+
+
+def test_granule_select_degenerate_rows(pkg, dev):
+    """Rows with no positive entry, with fewer positive entries than k (spread over few granules and over many), rows
+    of one repeated value (mass ties: the candidate list overflows and the general kernel redoes the row), and ties
+    at the threshold inside and across granules.  The granule maxima are formed here from the same keys."""
+    B, F, k = 12, 4096, 32
+    g = torch.Generator().manual_seed(11)
+    pre = torch.randn(B, F, generator=g)
+    pre[0] = -pre[0].abs()                                   # nothing positive
+    pre[1] = -pre[1].abs(); pre[1, 5:15] = 1.0               # 10 positives, all equal, one granule
+    pre[2] = -pre[2].abs(); pre[2, ::300] = torch.arange(1, 15).float()   # 14 positives over 14 granules
+    pre[3] = 0.75                                            # every entry equal: 4096 ties
+    pre[4] = -1.0; pre[4, 100:1500] = 2.0                    # 1400 ties: more than the candidate list holds
+    pre[5] = pre[5].abs(); pre[5, 64:64 + 40] = 9.0          # 40 ties above everything, one granule: k - 40 more from the rest
+    pre[6] = -1.0; pre[6, 0::64] = 3.0                       # one tie per granule, 64 granules: lowest 32 indices win
+    pre[7] = -1.0; pre[7, 63::64] = 3.0; pre[7, 10] = 3.0
+    pre = pre.to(torch.bfloat16).to(dev)
+    b = torch.zeros(F, device=dev)
+    s = torch.ones(F, device=dev)
+    gmax = _granule_max_of(pre, b, s)
+    got = pkg.ops.select_topk_row(pre, b, s, k, granule_max=gmax)
+    want = pkg.ops.select_topk_row(pre, b, s, k)
+    assert torch.equal(got.row_nnz, want.row_nnz), (got.row_nnz, want.row_nnz)
+    assert torch.equal(got.idx, want.idx) and torch.equal(got.val, want.val)
+    nnz = got.row_nnz.tolist()
+    assert nnz[0] == 0 and nnz[1] == 10 and nnz[2] == 14 and nnz[3] == k and nnz[4] == k
+    assert got.idx.view(B, k)[6].tolist() == list(range(0, 64 * k, 64))
+    assert got.idx.view(B, k)[3].tolist() == list(range(k))
+
+
+def test_granule_route_is_what_the_fused_step_runs_and_changes_nothing(pkg, dev):
+    from lm_saes_amd import synthetic
+
+    d, F, k, B = 128, 2048, 16, 256
+    x = synthetic.activations(B, d, 8, seed=5)
+    w = synthetic.sae_weights(d, F, x, seed=5)
+
+    calls = []
+    real = pkg.ops.encoder_gemm_granule_max
+
+    def spy(*a, **kw):
+        calls.append(1)
+        return real(*a, **kw)
+
+    def run(granule):
+        cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                            top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
+        m = pkg.SparseAutoEncoder(cfg)
+        synthetic.load_weights(m, *[t.to(dev) for t in w])
+        m.granule_select = granule
+        batch = {"in": x.to(dev), "out": x.to(dev), "tokens": torch.zeros(B, device=dev)}
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            loss = m.compute_loss(batch, return_aux_data=False)
+        loss.backward()
+        return loss.detach(), {n: p.grad for n, p in m.named_parameters()}
+
+    pkg.ops.encoder_gemm_granule_max = spy
+    try:
+        la, ga = run(True)
+        assert len(calls) == 1
+        lb, gb = run(False)
+        assert len(calls) == 1
+    finally:
+        pkg.ops.encoder_gemm_granule_max = real
+    assert torch.equal(la, lb)
+    for n in ga:
+        assert (ga[n] is None) == (gb[n] is None), n
+        if ga[n] is not None:
+            assert torch.equal(ga[n], gb[n]), n
