@@ -43,7 +43,9 @@ HBM_TRAFFIC_ROWS = {"encoder_gemm": "encoder_gemm", "adam_step_sparse_rows[f32 d
                     "select_topk_row": "select_topk_row"}
 # launches that move so little that their duration is the launch / dependency latency, not a bandwidth
 LATENCY_BOUND = {"build_feature_index", "adam_step[vector]", "col_sum", "cast_f32_to_bf16", "code_stats", "recon_stats",
-                 "grad_sq_nnz", "gather_rows", "row_sum", "row_norm"}
+                 "grad_sq_nnz", "gather_rows", "row_sum", "row_norm",
+                 # one workgroup per token: a radix select over F / 64 keys in LDS (a dozen barriers) and ~k scattered granules
+                 "select_topk_row[granule]"}
 
 
 def measured_traffic_gb(kernel: str):
@@ -71,6 +73,7 @@ def algorithmic_work(B: int, d: int, F: int, k: int) -> dict:
     return {
         "encoder_gemm": ("mfma", 2.0 * B * d * F),                       # flop
         "select_topk_row": ("hbm", B * F * 2 + B * k * 8),               # read bf16 pre once, write idx+val
+        "select_topk_row[granule]": ("hbm", B * (F // 64) * 4 + B * k * (128 + 8)),   # granule maxima, ~k granules of pre, idx+val
         "select_topk_batch": ("hbm", B * F * 2 + B * k * 8),             # read bf16 pre once, write idx+val
         "sparse_decode_mse_fused": ("hbm", 2 * B * k * d * 2 + 3 * B * d * 4),  # rows for recon and for d val; label, recon, grad
         "sparse_decode_fwd": ("hbm", B * k * d * 2 + B * d * 4),

@@ -134,13 +134,27 @@ int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const flo
  *   granule_max: the k-th largest granule maximum bounds the k-th largest key from below, so only the ~k granules
  *   that reach it are read from pre.  F % 64 == 0, F <= 262144, k <= 512; rows whose candidates do not fit the
  *   in-LDS list (mass ties) are redone from the whole row by a second launch of the general kernel.
+ * n_groups > 1: that many independent products of one shape in one launch, every array stacked group after group
+ *   (x [G, B, d], w_enc_t [G, F, d], pre [G, B, F], b_enc / scale [G, F], granule_max [G, B, F / 64]); the select
+ *   then takes all G * B rows at once with rows_per_group = B (0: one group), so that row r uses the bias and scale
+ *   of group r / B.
  * Together they replace `hidden_pre = x @ W_E + b_E` followed by the TopK of `hidden_pre * decoder_norm`
  * (models/sae.py:324-341, utils/math.py:81-171). */
-int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d, int64_t F,
-                                 const float *b_enc, const float *scale, uint32_t *granule_max, void *stream);
+int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups, int64_t B,
+                                 int64_t d, int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
+                                 void *stream);
 int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
-                                int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
-                                void *stream);
+                                int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val, int64_t *row_off,
+                                int32_t *row_nnz, void *stream);
+
+/* Per-layer codes -> one code over L * F features (the cross-layer transcoder's per-layer TopK, models/clt.py:232-387:
+ * each layer keeps its own k, the decoders read all layers' entries of a token).  idx / val [L * B * k] and row_nnz
+ * [L * B] are the outputs of one stacked select (row l * B + b: layer l, token b; slots row * k ..; ascending features).
+ * out_idx / out_val [B * L * k], out_row_off / out_row_nnz [B]: token b's entries in slots b * L * k .., layer after
+ * layer, feature ids l * F + f (ascending), unused slots zeroed; layer_cnt [B, L] = entries per (token, layer). */
+int sae_merge_layer_codes(const int32_t *idx, const float *val, const int32_t *row_nnz, int64_t L, int64_t B, int64_t k,
+                          int64_t F, int32_t *out_idx, float *out_val, int64_t *out_row_off, int32_t *out_row_nnz,
+                          int32_t *layer_cnt, void *stream);
 
 /* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
  * (h0, h1 as above); ties at the threshold -> lowest flattened index b * F + f.  If fewer than

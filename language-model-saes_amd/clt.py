@@ -105,15 +105,27 @@ class _FusedCLTStep(torch.autograd.Function):
         else:
             x_op = x_l
         out_dtype = torch.bfloat16 if amp else torch.float32
-        pres = [ops.encoder_gemm(x_op[l], w_enc_op[l], out_dtype) for l in range(L)]
         norms = m._norm_per_feature_nograd() if m.cfg.sparsity_include_decoder_norm else None     # [L, F]
         b_enc = b_E.detach().float().contiguous()
-        if act in ("topk", "batchtopk"):
+        if (act == "topk" and amp and getattr(m, "granule_select", True) and w_enc_op.dtype == torch.bfloat16
+                and ops.granule_route_supported(d, F, min(k, F))):
+            # per-layer TopK on bf16 operands: the L encoder products in one launch whose epilogue leaves the per-granule
+            # key maxima, one select over the L * B stacked rows that reads a row only where those maxima allow a kept
+            # entry, and one kernel that strings every token's layers together
+            pre_all, gmax = ops.encoder_gemm_granule_max(x_op.contiguous(), w_enc_op, b_enc,
+                                                         None if norms is None else norms.contiguous())
+            stacked = ops.select_topk_row(pre_all.view(L * B, F), b_enc, None if norms is None else norms.contiguous(),
+                                          min(k, F), granule_max=gmax.view(L * B, -1), rows_per_group=B)
+            cat, layer_cnt = ops.merge_layer_codes(stacked, L)
+            pres = list(pre_all.unbind(0))
+        elif act in ("topk", "batchtopk"):
+            pres = [ops.encoder_gemm(x_op[l], w_enc_op[l], out_dtype) for l in range(L)]
             sel = (lambda p, b, s: ops.select_topk_row(p, b, s, min(k, F))) if act == "topk" else \
                   (lambda p, b, s: ops.select_topk_batch(p, b, s, k * B))
             codes = [sel(pres[l], b_enc[l], None if norms is None else norms[l]) for l in range(L)]
             cat, layer_cnt = merge_layer_codes(codes)
         else:
+            pres = [ops.encoder_gemm(x_op[l], w_enc_op[l], out_dtype) for l in range(L)]
             pre_cat = torch.stack(pres, dim=1).view(B, L * F) if act == "layertopk" else None
             flat = lambda t: None if t is None else t.reshape(L * F)      # noqa: E731
             if act == "layertopk":

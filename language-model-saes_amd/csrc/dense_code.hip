@@ -103,6 +103,39 @@ __global__ __launch_bounds__(256) void dense_to_code_kernel(const void *__restri
   }
 }
 
+
+// Per-layer codes of one shape, stacked layer after layer (row l * B + b holds at most k entries of layer l for token b,
+// ascending features, in slots [row * k, row * k + row_nnz)), -> one code over L * F features (feature l * F + f) with
+// L * k slots per token: a token's entries are its layers' entries one layer after the other, which is ascending order of
+// l * F + f.  One thread per slot: it moves its own entry (if its slot holds one) and zeroes the output slot of the same
+// number if that lies past the token's entries, so every output slot is written exactly once.
+__global__ __launch_bounds__(256) void merge_layer_codes_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
+                                                                const int32_t *__restrict__ row_nnz, int L, int B, int k, int F,
+                                                                int32_t *__restrict__ out_idx, float *__restrict__ out_val,
+                                                                int64_t *__restrict__ out_row_off, int32_t *__restrict__ out_row_nnz,
+                                                                int32_t *__restrict__ layer_cnt) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_tok = L * k;
+  if (t >= (int64_t)B * per_tok) return;
+  const int b = (int)(t / per_tok), s = (int)(t % per_tok), l = s / k, j = s % k;
+  int before = 0, total = 0, mine = 0;
+  for (int q = 0; q < L; ++q) {
+    const int n = row_nnz[(size_t)q * B + b];
+    before += q < l ? n : 0;
+    mine = q == l ? n : mine;
+    total += n;
+  }
+  const size_t base = (size_t)b * per_tok;
+  if (j < mine) {
+    const size_t src = ((size_t)l * B + b) * k + j;
+    out_idx[base + before + j] = idx[src] + l * F;
+    out_val[base + before + j] = val[src];
+  }
+  if (s >= total) { out_idx[base + s] = 0; out_val[base + s] = 0.f; }
+  if (j == 0) layer_cnt[(size_t)b * L + l] = mine;
+  if (s == 0) { out_row_off[b] = (int64_t)base; out_row_nnz[b] = total; }
+}
+
 }  // namespace sae
 
 extern "C" int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_t F, int32_t *row_nnz, void *stream) {
@@ -129,4 +162,19 @@ extern "C" int sae_dense_to_code(const void *dense, int dtype, int64_t B, int64_
   else
     hipLaunchKernelGGL(dense_to_code_kernel<false>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity);
   return check_launch("dense_to_code");
+}
+
+extern "C" int sae_merge_layer_codes(const int32_t *idx, const float *val, const int32_t *row_nnz, int64_t L, int64_t B, int64_t k,
+                                     int64_t F, int32_t *out_idx, float *out_val, int64_t *out_row_off, int32_t *out_row_nnz,
+                                     int32_t *layer_cnt, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(idx && val && row_nnz && out_idx && out_val && out_row_off && out_row_nnz && layer_cnt, SAE_ERR_INVALID_ARG,
+              "merge_layer_codes: null pointer");
+  SAE_REQUIRE(L > 0 && B > 0 && k > 0 && F > 0, SAE_ERR_INVALID_ARG, "merge_layer_codes: sizes must be positive");
+  SAE_REQUIRE(L * F < ((int64_t)1 << 31) && L * k < ((int64_t)1 << 31) && B < ((int64_t)1 << 31) &&
+                  B * L * k < ((int64_t)1 << 39), SAE_ERR_UNSUPPORTED, "merge_layer_codes: too large");
+  const int64_t n = B * L * k;
+  hipLaunchKernelGGL(merge_layer_codes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, idx, val, row_nnz,
+                     (int)L, (int)B, (int)k, (int)F, out_idx, out_val, out_row_off, out_row_nnz, layer_cnt);
+  return check_launch("merge_layer_codes");
 }

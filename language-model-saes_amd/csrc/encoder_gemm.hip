@@ -300,6 +300,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
     const float *__restrict__ scale, uint32_t *__restrict__ gmax) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
+  if (blockIdx.y) {      // group g of a batch of independent products of one shape, each operand stacked group after group
+    const size_t g = blockIdx.y;
+    x += g * (size_t)M * row_bytes;
+    w += g * (size_t)N * row_bytes;
+    out = reinterpret_cast<char *>(out) + g * (size_t)M * N * (BF16_OUT ? 2 : 4);
+    if constexpr (GMAX) {
+      if (b_enc) b_enc += g * (size_t)N;
+      if (scale) scale += g * (size_t)N;
+      gmax += g * (size_t)M * (N >> 6);
+    }
+  }
 
   // ---- XCD-aware tile assignment: 32 consecutive workgroups of an XCD cover 2^rm_log2 token tiles x the rest in feature tiles
   int tile_m, tile_n;
@@ -543,15 +554,16 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
 
 template <bool BF16_OUT, bool GMAX>
 static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
-                            const float *scale, uint32_t *gmax, hipStream_t st) {
+                            const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1) {
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
   auto kern = encoder_gemm_bf16_kernel<BF16_OUT, GMAX>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
   if (rc != SAE_OK) return rc;
   const int rm_log2 = tiles_m >= 8 ? 3 : 2, rm = 1 << rm_log2, rn = 32 >> rm_log2;
   const int m_pad = (tiles_m + rm - 1) / rm * rm, n_local_pad = ((tiles_n + 7) / 8 + rn - 1) / rn * rn;
-  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, (const char *)x,
-                     (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale, gmax);
+  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)n_groups), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st,
+                     (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale,
+                     gmax);
   return check_launch("encoder_gemm");
 }
 
@@ -579,17 +591,19 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
                                : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
 }
 
-extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d,
-                                            int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
-                                            void *stream) {
+extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups,
+                                            int64_t B, int64_t d, int64_t F, const float *b_enc, const float *scale,
+                                            uint32_t *granule_max, void *stream) {
   using namespace sae;
   SAE_REQUIRE(x_bf16 && w_enc_t_bf16 && pre_bf16 && granule_max, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: null pointer");
-  SAE_REQUIRE(B > 0 && d > 0 && F > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: B, d, F must be positive");
-  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: size too large");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0 && n_groups > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: sizes must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28) && n_groups <= 65535, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_granule_max: size too large");
   SAE_REQUIRE(d % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: d_model=%lld must be a multiple of 64", (long long)d);
   SAE_REQUIRE(F % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_granule_max: F=%lld must be a multiple of 64 (whole granules)",
               (long long)F);
   SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_enc_t_bf16 | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0,
               SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: pointers must be 16-byte aligned");
-  return launch_gemm_bf16<true, true>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream);
+  return launch_gemm_bf16<true, true>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream,
+                                      n_groups);
 }

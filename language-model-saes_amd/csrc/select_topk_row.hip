@@ -236,11 +236,16 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
     int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
-    int32_t *__restrict__ row_nnz, int cand_cap, int only_flagged) {
+    int32_t *__restrict__ row_nnz, int cand_cap, int only_flagged, int rows_per_group) {
   __shared__ SelShared sh;
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
-  if (only_flagged && row_nnz[b] != SEL_ROW_FLAG) return;     // the pass after the granule kernel: rows it gave up on
+  if (only_flagged) {     // the pass after the granule kernel: the rows it gave up on, with their group's bias / scale
+    if (row_nnz[b] != SEL_ROW_FLAG) return;
+    const size_t grp = (size_t)(b / rows_per_group);
+    if (b_enc) b_enc += grp * F;
+    if (scale) scale += grp * F;
+  }
   RowReader<BF16, ARITH> rr;
   rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
@@ -448,7 +453,8 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
 namespace sae {
 static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const float *b_enc, const float *scale,
                                 const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,
-                                int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream, int only_flagged = 0) {
+                                int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream, int only_flagged = 0,
+                                int rows_per_group = 1) {
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
   SAE_REQUIRE(B > 0 && F > 0, SAE_ERR_INVALID_ARG, "select_topk_row: B and F must be positive");
   SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_row: bad dtype %d", pre_dtype);
@@ -463,7 +469,7 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
                      (((((uintptr_t)pre) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)feat_mask) & 15) == 0);
 #define SAE_LAUNCH_SELECT(BF, ST, ...)                                                                                     \
   hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
-                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged)
+                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged, rows_per_group)
   if (lowp) {
     if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP);
   } else if (feat_mask) {
@@ -507,10 +513,15 @@ struct GsShared {
 __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     const uint16_t *__restrict__ pre, const uint32_t *__restrict__ gmax, const float *__restrict__ b_enc,
     const float *__restrict__ scale, int F, int k, int32_t *__restrict__ idx_out, float *__restrict__ val_out,
-    int64_t *__restrict__ row_off, int32_t *__restrict__ row_nnz) {
+    int64_t *__restrict__ row_off, int32_t *__restrict__ row_nnz, int rows_per_group) {
   __shared__ GsShared sh;
   extern __shared__ __attribute__((aligned(16))) uint32_t gk[];   // the row's granule maxima
   const int b = blockIdx.x, tid = threadIdx.x, ng = F >> 6;
+  {   // rows are stacked group after group, each group with a bias / scale vector of its own
+    const size_t grp = (size_t)(b / rows_per_group);
+    if (b_enc) b_enc += grp * F;
+    if (scale) scale += grp * F;
+  }
   RowReader<true, SEL_PLAIN> rr;
   rr.row = pre + (size_t)b * F;
   rr.b_enc = b_enc;
@@ -621,11 +632,14 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
 }  // namespace sae
 
 extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
-                                           const float *scale, int64_t B, int64_t F, int k, int32_t *idx, float *val,
-                                           int64_t *row_off, int32_t *row_nnz, void *stream) {
+                                           const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                           int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre_bf16 && granule_max && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row_granule: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "select_topk_row_granule: bad sizes");
+  if (rows_per_group <= 0) rows_per_group = B;
+  SAE_REQUIRE(B % rows_per_group == 0, SAE_ERR_INVALID_ARG, "select_topk_row_granule: B=%lld is not a multiple of rows_per_group=%lld",
+              (long long)B, (long long)rows_per_group);
   SAE_REQUIRE(F % 64 == 0 && F / 64 <= GS_MAX_GRANULES, SAE_ERR_UNSUPPORTED,
               "select_topk_row_granule: F=%lld must be a multiple of 64, at most %d", (long long)F, 64 * GS_MAX_GRANULES);
   SAE_REQUIRE(k >= 1 && k <= GS_MAX_K, SAE_ERR_UNSUPPORTED, "select_topk_row_granule: k=%d outside [1, %d]", k, GS_MAX_K);
@@ -633,11 +647,12 @@ extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t 
               "select_topk_row_granule: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(select_topk_row_granule_kernel, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
-                     (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz);
+                     (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
   const int rc = check_launch("select_topk_row_granule");
   if (rc != SAE_OK) return rc;
   // rows the granule kernel flagged (mass ties) are redone from the whole row; every other workgroup leaves at once
-  return select_topk_row_impl(false, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1);
+  return select_topk_row_impl(false, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1,
+                              (int)rows_per_group);
 }
 
 extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,

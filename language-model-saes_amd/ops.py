@@ -301,24 +301,49 @@ def granule_route_supported(d: int, F: int, k: int) -> bool:
 def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Optional[torch.Tensor],
                              scale: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
     """bf16 pre[B, F] = x @ w_enc_t^T plus granule_max [B, F / 64] (int32 holding uint32 keys): per token and aligned
-    granule of 64 features the largest select key, i.e. the bits of (pre + b_enc) * scale where that is positive."""
-    _req(x, "x", torch.bfloat16, 2)
-    _req(w_enc_t, "w_enc_t", torch.bfloat16, 2)
-    B, d = x.shape
-    F, d2 = w_enc_t.shape
-    if d != d2:
+    granule of 64 features the largest select key, i.e. the bits of (pre + b_enc) * scale where that is positive.
+    With a leading group dimension on every argument (x [G, B, d], w_enc_t [G, F, d], b_enc / scale [G, F]) the G
+    products run in one launch and the outputs are [G, B, F] and [G, B, F / 64]."""
+    grouped = x.dim() == 3
+    _req(x, "x", torch.bfloat16, 3 if grouped else 2)
+    _req(w_enc_t, "w_enc_t", torch.bfloat16, 3 if grouped else 2)
+    G = x.shape[0] if grouped else 1
+    B, d = x.shape[-2:]
+    F, d2 = w_enc_t.shape[-2:]
+    if d != d2 or (grouped and w_enc_t.shape[0] != G):
         raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
     for name, t in (("b_enc", b_enc), ("scale", scale)):
         if t is not None:
-            _req(t, name, torch.float32, 1)
-            if t.numel() != F:
-                raise ValueError(f"{name} must have {F} elements")
-    pre = torch.empty(B, F, dtype=torch.bfloat16, device=x.device)
-    gmax = torch.empty(B, max(F // GRANULE, 1), dtype=torch.int32, device=x.device)
+            _req(t, name, torch.float32, 2 if grouped else 1)
+            if t.numel() != G * F:
+                raise ValueError(f"{name} must have {G * F} elements")
+    lead = (G,) if grouped else ()
+    pre = torch.empty(*lead, B, F, dtype=torch.bfloat16, device=x.device)
+    gmax = torch.empty(*lead, B, max(F // GRANULE, 1), dtype=torch.int32, device=x.device)
     with _timed("encoder_gemm"):
-        check(_lib.load().sae_encoder_gemm_granule_max(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _ptr(b_enc),
+        check(_lib.load().sae_encoder_gemm_granule_max(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), G, B, d, F, _ptr(b_enc),
                                                        _ptr(scale), gmax.data_ptr(), _stream(x)), "encoder_gemm_granule_max")
     return pre, gmax
+
+
+def merge_layer_codes(code: SparseCode, L: int) -> Tuple[SparseCode, torch.Tensor]:
+    """`code`: one select over L * B stacked rows (row l * B + b, at most k entries each, F features) -> the code over
+    L * F features with L * k slots per token (feature l * F + f, ascending) and the entry counts [B, L]."""
+    rows, F = code.n_tokens, code.d_sae
+    if rows % L:
+        raise ValueError(f"{rows} rows are not {L} layers of equally many tokens")
+    B, k = rows // L, code.idx.numel() // rows
+    dev = code.idx.device
+    idx = torch.empty(B * L * k, dtype=torch.int32, device=dev)
+    val = torch.empty(B * L * k, dtype=torch.float32, device=dev)
+    row_off = torch.empty(B, dtype=torch.int64, device=dev)
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
+    layer_cnt = torch.empty(B, L, dtype=torch.int32, device=dev)
+    with _timed("merge_layer_codes"):
+        check(_lib.load().sae_merge_layer_codes(code.idx.data_ptr(), code.val.data_ptr(), code.row_nnz.data_ptr(), L, B, k, F,
+                                                idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(),
+                                                layer_cnt.data_ptr(), _stream(code.idx)), "merge_layer_codes")
+    return SparseCode(idx, val, row_off, row_nnz, B, L * F), layer_cnt
 
 
 # ---- select ---------------------------------------------------------------------------------
@@ -332,13 +357,18 @@ def select_topk_row(
     feat_mask: Optional[torch.Tensor] = None,
     lowp: bool = False,
     granule_max: Optional[torch.Tensor] = None,
+    rows_per_group: int = 0,
 ) -> SparseCode:
     """Per-token TopK of (pre + b_enc) * scale.  `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the
     arithmetic of a dictionary whose parameters are bf16 tensors).  `granule_max`: the second output of
     `encoder_gemm_granule_max` for the same pre, b_enc and scale; the row is then read only where a kept element
-    can be (same result)."""
+    can be (same result).  On that route `rows_per_group` > 0 says that pre stacks groups of that many rows and that
+    b_enc / scale hold one vector of F per group."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
+    n_vec = F * (B // rows_per_group if rows_per_group else 1)
+    if rows_per_group and (granule_max is None or B % rows_per_group):
+        raise ValueError("rows_per_group needs the granule route and must divide the number of rows")
     if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None or feat_mask is not None):
         raise ValueError("lowp select takes a bf16 pre and neither cand_cap nor feat_mask")
     if granule_max is not None:
@@ -349,9 +379,9 @@ def select_topk_row(
             raise ValueError(f"granule_max must be [{B}, {F}/{GRANULE}]")
     for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
         if t is not None:
-            _req(t, name, torch.float32, 1)
-            if t.numel() != F:
-                raise ValueError(f"{name} must have {F} elements")
+            _req(t, name, torch.float32)
+            if t.numel() != (F if name == "feat_mask" else n_vec):
+                raise ValueError(f"{name} must have {n_vec} elements")
     k = int(k)
     dev = pre.device
     # zero-filled: slots a row does not use (fewer than k positive entries) then hold feature 0 with value 0
@@ -360,11 +390,12 @@ def select_topk_row(
     row_off = torch.empty(B, dtype=torch.int64, device=dev)
     row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
     lib = _lib.load()
-    _t = _timed("select_topk_row")
+    _t = _timed("select_topk_row[granule]" if granule_max is not None else "select_topk_row")
     _t.__enter__()
     if granule_max is not None:
         rc = lib.sae_select_topk_row_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k,
-                                             idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+                                             int(rows_per_group), idx.data_ptr(), val.data_ptr(), row_off.data_ptr(),
+                                             row_nnz.data_ptr(), _stream(pre))
     elif lowp:
         rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(), val.data_ptr(),
                                           row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))

@@ -133,3 +133,39 @@ def test_granule_route_is_what_the_fused_step_runs_and_changes_nothing(pkg, dev)
         assert (ga[n] is None) == (gb[n] is None), n
         if ga[n] is not None:
             assert torch.equal(ga[n], gb[n]), n
+
+
+def test_grouped_gemm_select_and_merge_equal_the_per_layer_route(pkg, dev):
+    """L products in one launch, one select over the L * B stacked rows with a bias / scale vector per group, and the
+    merge kernel -- against L separate products and selects merged through a sort of (token, layer, feature) keys."""
+    from lm_saes_amd.clt import merge_layer_codes
+
+    L, B, d, F, k = 5, 200, 128, 1024, 24
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(L, B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(L, F, d, generator=g) / d ** 0.5).to(torch.bfloat16).to(dev)
+    b = (0.1 * torch.randn(L, F, generator=g)).to(dev)
+    s = (0.5 + torch.rand(L, F, generator=g)).to(dev)
+    x[2, 7] = 0          # a token with nothing positive in layer 2 but for the bias
+    b[3] = -5.0          # a layer that keeps (almost) nothing
+    pre_all, gmax = pkg.ops.encoder_gemm_granule_max(x, w, b, s)
+    for l in range(L):
+        assert torch.equal(pre_all[l], pkg.ops.encoder_gemm(x[l], w[l], torch.bfloat16))
+    stacked = pkg.ops.select_topk_row(pre_all.view(L * B, F), b, s, k, granule_max=gmax.view(L * B, -1), rows_per_group=B)
+    codes = [pkg.ops.select_topk_row(pre_all[l], b[l], s[l], k) for l in range(L)]
+    for l, c in enumerate(codes):
+        assert torch.equal(stacked.row_nnz[l * B:(l + 1) * B], c.row_nnz)
+        assert torch.equal(stacked.idx[l * B * k:(l + 1) * B * k], c.idx) and torch.equal(stacked.val[l * B * k:(l + 1) * B * k], c.val)
+    got, got_cnt = pkg.ops.merge_layer_codes(stacked, L)
+    want, want_cnt = merge_layer_codes(codes)
+    assert torch.equal(got_cnt, want_cnt) and torch.equal(got.row_nnz, want.row_nnz)
+    assert got.d_sae == want.d_sae == L * F and got.n_tokens == B
+    # the two lay their rows out differently (fixed L * k slots per token against packed rows): compare row by row
+    gi, gv = got.idx.view(B, L * k), got.val.view(B, L * k)
+    nnz = got.row_nnz.tolist()
+    off = want.row_off.tolist()
+    for t in range(B):
+        assert torch.equal(gi[t, :nnz[t]], want.idx[off[t]:off[t] + nnz[t]]), t
+        assert torch.equal(gv[t, :nnz[t]], want.val[off[t]:off[t] + nnz[t]]), t
+        assert not gi[t, nnz[t]:].any() and not gv[t, nnz[t]:].any()
+    assert got.row_off.tolist() == [t * L * k for t in range(B)]

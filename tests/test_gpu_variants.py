@@ -319,6 +319,25 @@ def test_clt_fused_step_bf16(pkg, vo, dev):
     assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["loss"], w16["loss"]) < BF16_TOL
 
 
+def test_clt_granule_route_changes_nothing(pkg, vo, dev):
+    """Per-layer TopK under autocast: the grouped product + granule select + merge kernel against the per-layer
+    products, row selects and sort-based merge.  Same kept entries in the same order, so the same bits everywhere."""
+    L, d, F, k, B = 4, 64, 512, 8, 160
+    batch = {k_: v.to(dev) for k_, v in clt_batch(L, B, d, seed=48).items()}
+    outs = []
+    for granule in (True, False):
+        m, _, _, _ = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=47)
+        m.granule_select = granule
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = m.compute_loss(batch)
+        out["loss"].backward()
+        outs.append((out["loss"].detach(), out["feature_acts"].detach(), {n: p.grad for n, p in m.named_parameters()}))
+    (la, fa, ga), (lb, fb, gb) = outs
+    assert torch.equal(la, lb) and torch.equal(fa, fb)
+    for n in ga:
+        assert torch.equal(ga[n], gb[n]), n
+
+
 # ---- Lorsa ---------------------------------------------------------------------------------------
 
 def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, **kw):
