@@ -147,6 +147,11 @@ int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_ma
                                 int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val, int64_t *row_off,
                                 int32_t *row_nnz, void *stream);
 
+/* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product
+ * (Lorsa's head activations): one streaming read of pre.  rows_per_group as in sae_select_topk_row_granule. */
+int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int64_t rows_per_group,
+                    uint32_t *granule_max, void *stream);
+
 /* Per-layer codes -> one code over L * F features (the cross-layer transcoder's per-layer TopK, models/clt.py:232-387:
  * each layer keeps its own k, the decoders read all layers' entries of a token).  idx / val [L * B * k] and row_nnz
  * [L * B] are the outputs of one stacked select (row l * B + b: layer l, token b; slots row * k ..; ascending features).

@@ -31,6 +31,7 @@ SIGNATURES = {
     "sae_select_topk_row": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_encoder_gemm_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P]),
     "sae_select_topk_row_granule": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _P, _P, _P, _P, _P]),
+    "sae_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _P, _P]),
     "sae_merge_layer_codes": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_lowp": (_I, [_P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),

@@ -629,6 +629,37 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
   if (tid == 0) { row_off[b] = (int64_t)b * k; row_nnz[b] = k_eff; }
 }
 
+// Granule maxima of rows that no GEMM epilogue left them for: eight lanes per granule (one 16-byte chunk each), eight
+// granules per wave and step.
+__global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__restrict__ pre, const float *__restrict__ b_enc,
+                                                          const float *__restrict__ scale, int F, int64_t n_granules,
+                                                          int rows_per_group, uint32_t *__restrict__ gmax) {
+  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+  const int part = threadIdx.x & 7, ng = F >> 6;
+  uint32_t m = 0u;
+  if (g < n_granules) {
+    const int64_t row = g / ng;
+    const int gi = (int)(g % ng);
+    RowReader<true, SEL_PLAIN> rr;
+    const size_t grp = (size_t)(row / rows_per_group);
+    rr.row = pre + (size_t)row * F;
+    rr.b_enc = b_enc ? b_enc + grp * F : nullptr;
+    rr.scale = scale ? scale + grp * F : nullptr;
+    rr.fmask = nullptr;
+    rr.F = F;
+    uint32_t keys[8];
+    rr.chunk_keys(gi * 8 + part, keys);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = keys[e] > m ? keys[e] : m;
+  }
+#pragma unroll
+  for (int o = 1; o < 8; o <<= 1) {
+    const uint32_t t = (uint32_t)__shfl_xor((int)m, o, 64);
+    m = t > m ? t : m;
+  }
+  if (part == 0 && g < n_granules) gmax[g] = m;
+}
+
 }  // namespace sae
 
 extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
@@ -672,4 +703,22 @@ extern "C" int sae_select_topk_row(const void *pre, int pre_dtype, const float *
                                    int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
                                    void *stream) {
   return sae_select_topk_row_ex(pre, pre_dtype, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, sae::SEL_CAP, stream);
+}
+
+extern "C" int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
+                               int64_t rows_per_group, uint32_t *granule_max, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre_bf16 && granule_max, SAE_ERR_INVALID_ARG, "granule_max: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F < (1LL << 31), SAE_ERR_INVALID_ARG, "granule_max: bad sizes");
+  SAE_REQUIRE(F % 64 == 0, SAE_ERR_UNSUPPORTED, "granule_max: F=%lld must be a multiple of 64", (long long)F);
+  if (rows_per_group <= 0) rows_per_group = B;
+  SAE_REQUIRE(B % rows_per_group == 0, SAE_ERR_INVALID_ARG, "granule_max: B=%lld is not a multiple of rows_per_group=%lld",
+              (long long)B, (long long)rows_per_group);
+  SAE_REQUIRE((((uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "granule_max: pointers must be 16-byte aligned");
+  const int64_t n = B * (F / 64);
+  SAE_REQUIRE((n * 8 + 255) / 256 < (1LL << 31), SAE_ERR_UNSUPPORTED, "granule_max: too large");
+  hipLaunchKernelGGL(granule_max_kernel, dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t *)pre_bf16, b_enc, scale, (int)F, n, (int)rows_per_group, granule_max);
+  return check_launch("granule_max");
 }

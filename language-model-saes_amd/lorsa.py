@@ -152,7 +152,13 @@ class _SparseTail(torch.autograd.Function):
         m: "LowRankSparseAttention" = holder["model"]
         scale = m._decoder_norm_nograd() if m.cfg.sparsity_include_decoder_norm else None
         hp = hidden_pre if hidden_pre.dtype in (torch.float32, torch.bfloat16) else hidden_pre.float()
-        code = ops.select_topk_row(hp.contiguous(), None, scale, k)
+        hp = hp.contiguous()
+        if hp.dtype == torch.bfloat16 and getattr(m, "granule_select", True) and ops.granule_route_supported(64, hp.shape[1], int(k)):
+            # short rows: one streaming pass for the per-granule key maxima, then a select that reads a row only where a
+            # kept entry can be, instead of one 1024-thread workgroup walking every row twice
+            code = ops.select_topk_row(hp, None, scale, k, granule_max=ops.granule_max(hp, None, scale))
+        else:
+            code = ops.select_topk_row(hp, None, scale, k)
         w_op = m._w_dec_operand(amp)
         recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(
             code, w_op, None if b_D is None else b_D.detach(), label, tok_w)

@@ -326,6 +326,23 @@ def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Opti
     return pre, gmax
 
 
+def granule_max(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], rows_per_group: int = 0) -> torch.Tensor:
+    """The granule maxima `encoder_gemm_granule_max` leaves, for a bf16 pre [B, F] from elsewhere."""
+    _req(pre, "pre", torch.bfloat16, 2)
+    B, F = pre.shape
+    n_vec = F * (B // rows_per_group if rows_per_group else 1)
+    for name, t in (("b_enc", b_enc), ("scale", scale)):
+        if t is not None:
+            _req(t, name, torch.float32)
+            if t.numel() != n_vec:
+                raise ValueError(f"{name} must have {n_vec} elements")
+    gmax = torch.empty(B, max(F // GRANULE, 1), dtype=torch.int32, device=pre.device)
+    with _timed("granule_max"):
+        check(_lib.load().sae_granule_max(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, int(rows_per_group), gmax.data_ptr(),
+                                          _stream(pre)), "granule_max")
+    return gmax
+
+
 def merge_layer_codes(code: SparseCode, L: int) -> Tuple[SparseCode, torch.Tensor]:
     """`code`: one select over L * B stacked rows (row l * B + b, at most k entries each, F features) -> the code over
     L * F features with L * k slots per token (feature l * F + f, ascending) and the entry counts [B, L]."""

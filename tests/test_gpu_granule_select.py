@@ -169,3 +169,28 @@ def test_grouped_gemm_select_and_merge_equal_the_per_layer_route(pkg, dev):
         assert torch.equal(gv[t, :nnz[t]], want.val[off[t]:off[t] + nnz[t]]), t
         assert not gi[t, nnz[t]:].any() and not gv[t, nnz[t]:].any()
     assert got.row_off.tolist() == [t * L * k for t in range(B)]
+
+
+@pytest.mark.parametrize("B,F,groups", [(300, 1024, 1), (64, 8192, 1), (96, 256, 3)])
+def test_standalone_granule_max(pkg, dev, B, F, groups):
+    g = torch.Generator().manual_seed(B + F)
+    pre = torch.randn(B, F, generator=g).to(torch.bfloat16).to(dev)
+    b = (0.1 * torch.randn(groups, F, generator=g)).to(dev)
+    s = (0.5 + torch.rand(groups, F, generator=g)).to(dev)
+    rpg = B // groups
+    got = pkg.ops.granule_max(pre, b.view(-1) if groups == 1 else b, s.view(-1) if groups == 1 else s, rows_per_group=0 if groups == 1 else rpg)
+    rows_b = b.repeat_interleave(rpg, dim=0)
+    rows_s = s.repeat_interleave(rpg, dim=0)
+    h1 = (pre.float() + rows_b) * rows_s
+    bits = h1.contiguous().view(torch.int32)
+    want = torch.where(h1 > 0, bits, torch.zeros_like(bits)).view(B, F // 64, 64).max(dim=2).values
+    assert torch.equal(got, want)
+    # and with neither bias nor scale
+    got0 = pkg.ops.granule_max(pre, None, None)
+    h0 = pre.float()
+    want0 = torch.where(h0 > 0, h0.contiguous().view(torch.int32), torch.zeros(B, F, dtype=torch.int32, device=dev)).view(B, F // 64, 64).max(dim=2).values
+    assert torch.equal(got0, want0)
+    k = 16
+    a = pkg.ops.select_topk_row(pre, None, None, k, granule_max=got0)
+    w = pkg.ops.select_topk_row(pre, None, None, k)
+    assert torch.equal(a.idx, w.idx) and torch.equal(a.val, w.val) and torch.equal(a.row_nnz, w.row_nnz)
