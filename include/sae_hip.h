@@ -125,6 +125,14 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
 int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int k,
                              int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream);
 
+/* out[b, f] = bf16(float(bf16(sum_j x[b, j] * w_t[f, j])) + col_bias[f] + row_bias[b])      (bf16 operands and output)
+ * What `(x @ W) + bias` is under bf16 autocast: the product a bf16 tensor, the bias an fp32 parameter, the sum cast to
+ * bf16 by the next autocast op.  col_bias [F] / row_bias [B] nullable (row_bias serves the swapped-operand call that
+ * writes a transposed projection).  d % 64 == 0.  Replaces Lorsa's q / k / v projections with their biases
+ * (models/lorsa.py:784-829). */
+int sae_encoder_gemm_bias(const void *x_bf16, const void *w_t_bf16, void *out_bf16, int64_t B, int64_t d, int64_t F,
+                          const float *col_bias, const float *row_bias, void *stream);
+
 /* The encoder product and the per-token TopK with the row read only where it matters.
  * sae_encoder_gemm_granule_max: sae_encoder_gemm for bf16 operands and bf16 output (F % 64 == 0) whose epilogue
  *   also writes granule_max [B, F / 64] (uint32): for every token and every aligned granule of 64 features the

@@ -29,6 +29,7 @@ SIGNATURES = {
     "sae_col_sum_static": (_I, [_P, _P, _L, _L, _I, _P]),
     "sae_encoder_gemm": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "sae_select_topk_row": (_I, [_P, _I, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
+    "sae_encoder_gemm_bias": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P]),
     "sae_encoder_gemm_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P]),
     "sae_select_topk_row_granule": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _P, _P, _P, _P, _P]),
     "sae_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _P, _P]),

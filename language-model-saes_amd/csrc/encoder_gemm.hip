@@ -291,10 +291,14 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
   __builtin_amdgcn_s_barrier();           \
   __builtin_amdgcn_sched_barrier(0)
 
-// GMAX (bf16 output, N a multiple of 64): the epilogue also writes, for every token and every aligned granule of 64
+// EPI_GMAX (bf16 output, N a multiple of 64): the epilogue also writes, for every token and every aligned granule of 64
 // features, the largest select key of the granule's rounded outputs to gmax[token][N / 64]; the wave's 64 features are
 // one granule.
-template <bool BF16_OUT, bool GMAX>
+// EPI_BIAS (bf16 output): out = bf16(float(bf16(acc)) + bias), the value of `(x @ w) + bias` when the product is a bf16
+// tensor and the bias an fp32 one; `b_enc` then holds a bias per output column (nullable), `scale` one per output row
+// (nullable).
+constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2;
+template <bool BF16_OUT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
     int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
@@ -305,7 +309,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     x += g * (size_t)M * row_bytes;
     w += g * (size_t)N * row_bytes;
     out = reinterpret_cast<char *>(out) + g * (size_t)M * N * (BF16_OUT ? 2 : 4);
-    if constexpr (GMAX) {
+    if constexpr (EPI == EPI_GMAX) {
       if (b_enc) b_enc += g * (size_t)N;
       if (scale) scale += g * (size_t)N;
       gmax += g * (size_t)M * (N >> 6);
@@ -392,18 +396,34 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i]),                      \
                                                           __builtin_bit_cast(bf16x8_t, xf[j]), acc[i][j], 0, 0, 0);
 
-  // GMAX: this lane's 16 bias and 16 scale values, asked for here so that the epilogue does not wait for them
-  float bb[GMAX ? 4 : 1][4], ss[GMAX ? 4 : 1][4];
-  if constexpr (GMAX) {
+  // EPI_GMAX: this lane's 16 bias and 16 scale values; EPI_BIAS: its 16 column biases and 8 row biases.  Asked for here
+  // so that the epilogue does not wait for them.
+  constexpr bool GMAX = EPI == EPI_GMAX, BIAS = EPI == EPI_BIAS;
+  float bb[EPI != EPI_NONE ? 4 : 1][4], ss[GMAX ? 4 : 1][4], rb[BIAS ? 8 : 1];
+  if constexpr (EPI != EPI_NONE) {
     const int f0 = n0 + wn * 64;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int f = f0 + i * 16 + 4 * fq;
-      const bool ok = f0 < N;
-      const float4 b4 = b_enc && ok ? *reinterpret_cast<const float4 *>(b_enc + f) : make_float4(0.f, 0.f, 0.f, 0.f);
-      const float4 s4 = scale && ok ? *reinterpret_cast<const float4 *>(scale + f) : make_float4(1.f, 1.f, 1.f, 1.f);
+      float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f), s4 = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (GMAX || (N & 3) == 0) {
+        if (b_enc && f + 3 < N) b4 = *reinterpret_cast<const float4 *>(b_enc + f);
+      } else if (b_enc) {     // a bias vector that is not 16-byte addressable at every f
+        b4.x = f < N ? b_enc[f] : 0.f; b4.y = f + 1 < N ? b_enc[f + 1] : 0.f;
+        b4.z = f + 2 < N ? b_enc[f + 2] : 0.f; b4.w = f + 3 < N ? b_enc[f + 3] : 0.f;
+      }
       bb[i][0] = b4.x; bb[i][1] = b4.y; bb[i][2] = b4.z; bb[i][3] = b4.w;
-      ss[i][0] = s4.x; ss[i][1] = s4.y; ss[i][2] = s4.z; ss[i][3] = s4.w;
+      if constexpr (GMAX) {
+        if (scale && f0 < N) s4 = *reinterpret_cast<const float4 *>(scale + f);
+        ss[i][0] = s4.x; ss[i][1] = s4.y; ss[i][2] = s4.z; ss[i][3] = s4.w;
+      }
+    }
+    if constexpr (BIAS) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int tok = m0 + wm * 128 + j * 16 + frow;
+        rb[j] = scale && tok < M ? scale[tok] : 0.f;
+      }
     }
   }
   for (int slab = 0; slab < n_slabs; ++slab) {
@@ -434,6 +454,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
   // more and every load has landed, so LDS is free: the early waves stage and store their output under that phase.
 
   // ---- epilogue: lane holds, per (i, j): features 4 (lane / 16) .. + 3 of sub-tile i for token lane % 16 of sub-tile j
+  if constexpr (BIAS) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = pack_bf16x2(acc[i][j][0], acc[i][j][1]), hi = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        acc[i][j][0] = (__uint_as_float(lo << 16) + bb[i][0]) + rb[j];
+        acc[i][j][1] = (__uint_as_float(lo & 0xffff0000u) + bb[i][1]) + rb[j];
+        acc[i][j][2] = (__uint_as_float(hi << 16) + bb[i][2]) + rb[j];
+        acc[i][j][3] = (__uint_as_float(hi & 0xffff0000u) + bb[i][3]) + rb[j];
+      }
+  }
   if constexpr (GMAX) {
     const int f0 = n0 + wn * 64;
     if (f0 < N) {
@@ -552,11 +584,11 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
   return check_launch("encoder_gemm");
 }
 
-template <bool BF16_OUT, bool GMAX>
+template <bool BF16_OUT, int EPI>
 static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
                             const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1) {
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
-  auto kern = encoder_gemm_bf16_kernel<BF16_OUT, GMAX>;
+  auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
   if (rc != SAE_OK) return rc;
   const int rm_log2 = tiles_m >= 8 ? 3 : 2, rm = 1 << rm_log2, rn = 32 >> rm_log2;
@@ -584,8 +616,8 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
               "encoder_gemm: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   if (in_dtype == SAE_BF16) {
-    return out_dtype == SAE_BF16 ? launch_gemm_bf16<true, false>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st)
-                                 : launch_gemm_bf16<false, false>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st);
+    return out_dtype == SAE_BF16 ? launch_gemm_bf16<true, EPI_NONE>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st)
+                                 : launch_gemm_bf16<false, EPI_NONE>(x, w_enc_t, pre, B, d, F, nullptr, nullptr, nullptr, st);
   }
   return out_dtype == SAE_BF16 ? launch_gemm_f32<true>(x, w_enc_t, pre, B, d, F, st)
                                : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
@@ -604,6 +636,18 @@ extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_en
               (long long)F);
   SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_enc_t_bf16 | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0,
               SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: pointers must be 16-byte aligned");
-  return launch_gemm_bf16<true, true>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream,
+  return launch_gemm_bf16<true, EPI_GMAX>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream,
                                       n_groups);
+}
+
+extern "C" int sae_encoder_gemm_bias(const void *x_bf16, const void *w_t_bf16, void *out_bf16, int64_t B, int64_t d, int64_t F,
+                                     const float *col_bias, const float *row_bias, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x_bf16 && w_t_bf16 && out_bf16, SAE_ERR_INVALID_ARG, "encoder_gemm_bias: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_bias: sizes must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm_bias: size too large");
+  SAE_REQUIRE(d % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_bias: d=%lld must be a multiple of 64", (long long)d);
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_t_bf16 | (uintptr_t)out_bf16 | (uintptr_t)col_bias) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "encoder_gemm_bias: pointers must be 16-byte aligned");
+  return launch_gemm_bf16<true, EPI_BIAS>(x_bf16, w_t_bf16, out_bf16, B, d, F, col_bias, row_bias, nullptr, (hipStream_t)stream);
 }

@@ -83,8 +83,8 @@ class _ProjectAndMix(torch.autograd.Function):
     kernels, for the configuration without rotary embedding and query / key norms.
 
     forward : q = x W_Q, k = x W_K as [T, h dq] (natural), v^T = W_V x^T as [F, T] (the GEMM with its operands swapped
-              yields the transposed layout the mixing product contracts over); the biases are added as the attention
-              kernel loads its operands.
+              yields the transposed layout the mixing product contracts over); the biases are added in the products'
+              epilogues.
     backward: the transposed copies q^T, k^T, v, dout^T (cast-transpose kernel); the attention backward returns
               dq^T, dk^T, dv^T [., T] in one buffer, which is exactly the operand of the weight-gradient product
               dW = d(.)^T x over the token axis (one GEMM for the three); bias gradients are its row sums."""
@@ -96,11 +96,15 @@ class _ProjectAndMix(torch.autograd.Function):
         n_batch, h = T // seq, cfg.n_qk_heads
         x_op = x2 if x2.dtype == torch.bfloat16 else ops.cast_bf16(x2.float().contiguous())
         wq, wk, wv = model._w_qk_operand("W_Q"), model._w_qk_operand("W_K"), model._w_val_operand(True)
-        q = ops.encoder_gemm(x_op, wq, torch.bfloat16)                      # [T, h dq]
-        k = ops.encoder_gemm(x_op, wk, torch.bfloat16)
-        vt = ops.encoder_gemm(wv, x_op, torch.bfloat16)                     # [F, T]
+        # the biases join in the products' epilogues (bf16 product + fp32 bias, rounded to bf16 again: what the attention
+        # gets under autocast); added per tile inside the attention kernels they would be re-added for every
+        # (query block, key block) pair and cost those kernels as many vector instructions as their softmax
+        flat = lambda b: b.detach().float().reshape(-1).contiguous()        # noqa: E731
+        q = ops.encoder_gemm_bias(x_op, wq, col_bias=flat(b_Q))             # [T, h dq]
+        k = ops.encoder_gemm_bias(x_op, wk, col_bias=flat(b_K))
+        vt = ops.encoder_gemm_bias(wv, x_op, row_bias=flat(b_V))            # [F, T]
         scale = 1.0 / model.attn_scale
-        out, lse = ops.attention_fwd(q, k, vt, n_batch, seq, h, scale, b_Q, b_K, b_V)
+        out, lse = ops.attention_fwd(q, k, vt, n_batch, seq, h, scale)
         ctx.save_for_backward(x_op, wq, wk, wv, q, k, vt, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
         ctx.dims = (n_batch, seq, h, scale)
         ctx.shapes = (tuple(W_Q.shape), tuple(W_K.shape))
@@ -114,7 +118,7 @@ class _ProjectAndMix(torch.autograd.Function):
         dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
         qt, kt, v = ops.transpose_to_bf16(q)[0], ops.transpose_to_bf16(k)[0], ops.transpose_to_bf16(vt)[0]
         dzt = ops.transpose_to_bf16(dz)[0]                                  # [F, T]
-        dqt, dkt, dvt, stacked = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale, b_Q, b_K, b_V,
+        dqt, dkt, dvt, stacked = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale,
                                                    return_stacked=True)
         xt = ops.transpose_to_bf16(x_op)[0]                                 # [d, T]
         d = x_op.shape[1]

@@ -288,6 +288,28 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     return pre
 
 
+def encoder_gemm_bias(x: torch.Tensor, w_t: torch.Tensor, col_bias: Optional[torch.Tensor] = None,
+                      row_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 out[B, F] = bf16(float(bf16(x @ w_t^T)) + col_bias[F] + row_bias[B]): a projection with its bias as a bf16
+    autocast product plus an fp32 bias gives it."""
+    _req(x, "x", torch.bfloat16, 2)
+    _req(w_t, "w_t", torch.bfloat16, 2)
+    B, d = x.shape
+    F, d2 = w_t.shape
+    if d != d2:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_t {tuple(w_t.shape)}")
+    for name, t, n in (("col_bias", col_bias, F), ("row_bias", row_bias, B)):
+        if t is not None:
+            _req(t, name, torch.float32)
+            if t.numel() != n:
+                raise ValueError(f"{name} must have {n} elements")
+    out = torch.empty(B, F, dtype=torch.bfloat16, device=x.device)
+    with _timed("encoder_gemm"):
+        check(_lib.load().sae_encoder_gemm_bias(x.data_ptr(), w_t.data_ptr(), out.data_ptr(), B, d, F, _ptr(col_bias),
+                                                _ptr(row_bias), _stream(x)), "encoder_gemm_bias")
+    return out
+
+
 GRANULE = 64                 # features per granule of the granule-maximum route
 GRANULE_MAX_F = 64 * 4096
 GRANULE_MAX_K = 512

@@ -668,3 +668,18 @@ def test_mfma_probe_runs_and_counts_its_flop(pkg, dev):
     assert ms > 0.0
     with pytest.raises(RuntimeError):
         pkg.ops.mfma_probe(dev, n_workgroups=0, iters=16)
+
+
+@pytest.mark.parametrize("B,d,F", [(300, 128, 520), (256, 64, 256), (70, 192, 1030)])
+def test_encoder_gemm_bias_epilogue(pkg, dev, B, d, F):
+    """out = bf16(float(bf16(x @ w^T)) + col_bias + row_bias): bit for bit the plain product followed by the sums."""
+    g = torch.Generator().manual_seed(B + F)
+    x = torch.randn(B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = torch.randn(F, d, generator=g).to(torch.bfloat16).to(dev)
+    cb = torch.randn(F, generator=g).to(dev)
+    rb = torch.randn(B, generator=g).to(dev)
+    plain = pkg.ops.encoder_gemm(x, w, torch.bfloat16).float()
+    assert torch.equal(pkg.ops.encoder_gemm_bias(x, w, col_bias=cb), (plain + cb).to(torch.bfloat16))
+    assert torch.equal(pkg.ops.encoder_gemm_bias(x, w, row_bias=rb), (plain + rb[:, None]).to(torch.bfloat16))
+    assert torch.equal(pkg.ops.encoder_gemm_bias(x, w, cb, rb), ((plain + cb) + rb[:, None]).to(torch.bfloat16))
+    assert torch.equal(pkg.ops.encoder_gemm_bias(x, w), plain.to(torch.bfloat16))
