@@ -191,3 +191,72 @@ def test_random_sweep_attention_and_code_conversions(pkg, oracle, dev, sweep_see
                 pkg.ops.adam_step_sparse_rows(fi, coef, dense, pb, mb, vb, step=step, row_grad_coef=rc, **hy)
                 assert torch.equal(pa, pb) and torch.equal(ma, mb) and torch.equal(va, vb)
     assert n > 30
+
+
+@pytest.mark.parametrize("sweep_seed", [4])
+def test_random_sweep_granule_route(pkg, oracle, dev, sweep_seed, budget_s=10.0):
+    """The granule route against the oracle's TopK, to the bit: granule maxima from the standalone pass or from the GEMM's
+    epilogue (then on the GEMM's own output), the granule select on single and grouped rows, and the layer merge against
+    the oracle's codes strung together.  Tie densities include rows of a single value (the flagged-row path)."""
+    rng = random.Random(sweep_seed)
+    t0 = time.time()
+    n = 0
+    while time.time() - t0 < budget_s:
+        n += 1
+        kind = rng.choice(["select", "select", "gemm_select", "grouped_merge"])
+        seed = rng.randrange(1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        if kind == "select":
+            B = rng.choice([1, 3, 9, 20]); F = 64 * rng.choice([1, 2, 7, 16, 64, 128, 192, 1024, 2048, 4096])
+            k = min(F, rng.choice([1, 4, 16, 32, 64, 128, 300, 512]))
+            ties = rng.choice([0, 0, 2, 16, 64])
+            pre = torch.randn(B, F, generator=g)
+            if ties: pre = quant(pre, ties)
+            if rng.random() < 0.2: pre[:, : F // 2] = -1.0
+            if rng.random() < 0.1: pre[rng.randrange(B)] = 0.5
+            if rng.random() < 0.1: pre[rng.randrange(B)] = -0.5
+            pre = pre.to(torch.bfloat16)
+            b = 0.1 * torch.randn(F, generator=g) if rng.random() < 0.7 else None
+            s = 0.5 + torch.rand(F, generator=g) if rng.random() < 0.7 else None
+            print(f"[{n}] granule select seed={seed} B={B} F={F} k={k} ties={ties} b={b is not None} s={s is not None}", flush=True)
+            dv = lambda t: None if t is None else t.to(dev)                      # noqa: E731
+            gmax = pkg.ops.granule_max(pre.to(dev), dv(b), dv(s))
+            code = pkg.ops.select_topk_row(pre.to(dev), dv(b), dv(s), k, granule_max=gmax)
+            got, want = tk.code_to_rows(code), tk.oracle_topk_code(oracle, pre, b, s, k)
+            for r, ((gi, gv), (wi, wv)) in enumerate(zip(got, want)):
+                assert (gi == wi).all() and (gv == wv).all(), f"row {r}"
+        elif kind == "gemm_select":
+            B = rng.choice([5, 64, 300]); d = 64 * rng.choice([1, 2, 4]); F = 64 * rng.choice([1, 3, 16, 40, 130])
+            k = min(F, rng.choice([1, 8, 32, 100]))
+            x = torch.randn(B, d, generator=g).to(torch.bfloat16); w = (torch.randn(F, d, generator=g) / d ** 0.5).to(torch.bfloat16)
+            b = 0.1 * torch.randn(F, generator=g) if rng.random() < 0.7 else None
+            s = 0.5 + torch.rand(F, generator=g) if rng.random() < 0.7 else None
+            print(f"[{n}] gemm + granule select seed={seed} B={B} d={d} F={F} k={k} b={b is not None} s={s is not None}", flush=True)
+            dv = lambda t: None if t is None else t.to(dev)                      # noqa: E731
+            pre, gmax = pkg.ops.encoder_gemm_granule_max(x.to(dev), w.to(dev), dv(b), dv(s))
+            assert torch.equal(gmax, pkg.ops.granule_max(pre, dv(b), dv(s)))
+            code = pkg.ops.select_topk_row(pre, dv(b), dv(s), k, granule_max=gmax)
+            got, want = tk.code_to_rows(code), tk.oracle_topk_code(oracle, pre.cpu(), b, s, k)
+            for r, ((gi, gv), (wi, wv)) in enumerate(zip(got, want)):
+                assert (gi == wi).all() and (gv == wv).all(), f"row {r}"
+        else:
+            L = rng.choice([1, 2, 5]); B = rng.choice([3, 40]); F = 64 * rng.choice([2, 16, 48]); k = min(F, rng.choice([2, 16, 64]))
+            pre = torch.randn(L * B, F, generator=g)
+            if rng.random() < 0.3: pre = quant(pre, 8)
+            if rng.random() < 0.3: pre[rng.randrange(L * B)] = -1.0
+            pre = pre.to(torch.bfloat16)
+            b = 0.1 * torch.randn(L, F, generator=g); s = 0.5 + torch.rand(L, F, generator=g)
+            print(f"[{n}] grouped select + merge seed={seed} L={L} B={B} F={F} k={k}", flush=True)
+            gmax = pkg.ops.granule_max(pre.to(dev), b.to(dev), s.to(dev), rows_per_group=B)
+            stacked = pkg.ops.select_topk_row(pre.to(dev), b.to(dev), s.to(dev), k, granule_max=gmax, rows_per_group=B)
+            merged, cnt = pkg.ops.merge_layer_codes(stacked, L)
+            mi, mv = merged.idx.view(B, L * k).cpu(), merged.val.view(B, L * k).cpu()
+            per_layer = [tk.oracle_topk_code(oracle, pre[l * B:(l + 1) * B], b[l], s[l], k) for l in range(L)]
+            for t in range(B):
+                wi = [i + l * F for l in range(L) for i in per_layer[l][t][0].tolist()]
+                wv = [v for l in range(L) for v in per_layer[l][t][1].tolist()]
+                assert mi[t, :len(wi)].tolist() == wi and mv[t, :len(wv)].tolist() == wv, f"token {t}"
+                assert merged.row_nnz[t].item() == len(wi) and not mi[t, len(wi):].any()
+                assert cnt[t].tolist() == [len(per_layer[l][t][0]) for l in range(L)]
+    print(f"{n} cases", flush=True)
+    assert n > 50
