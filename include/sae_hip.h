@@ -155,6 +155,15 @@ int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_ma
                                 int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val, int64_t *row_off,
                                 int32_t *row_nnz, void *stream);
 
+/* sae_select_topk_batch (bf16 pre, no feat_mask, F % 256 == 0) with the per-granule key maxima handed in
+ * (granule_max [B, F / 64] of sae_encoder_gemm_granule_max for the same pre, b_enc, scale): the select's one pass over
+ * the whole matrix shrinks to a histogram of the maxima; every later pass and the result are those of
+ * sae_select_topk_batch.  Same workspace. */
+int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
+                                  int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
+                                  int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
+                                  int64_t workspace_bytes, void *stream);
+
 /* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product
  * (Lorsa's head activations): one streaming read of pre.  rows_per_group as in sae_select_topk_row_granule. */
 int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int64_t rows_per_group,

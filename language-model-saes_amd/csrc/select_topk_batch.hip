@@ -263,6 +263,25 @@ __global__ __launch_bounds__(BT_THREADS) void bt_first_kernel(BatchReader<BF16> 
     if (h[i]) atomicAdd(&hist[i], h[i]);
 }
 
+// The full pass when the granule maxima already exist (the encoder GEMM's epilogue leaves them): only their histogram.
+__global__ __launch_bounds__(BT_THREADS) void bt_hist_kernel(const uint32_t *__restrict__ gran_max, int64_t n, const BatchSelState *st,
+                                                             uint32_t *__restrict__ hist) {
+  __shared__ uint32_t h[BT_BINS];
+  if (st->done) return;
+  for (int i = threadIdx.x; i < BT_BINS; i += BT_THREADS) h[i] = 0u;
+  __syncthreads();
+  for (int64_t i = ((int64_t)blockIdx.x * BT_THREADS + threadIdx.x) * 4; i < n; i += (int64_t)gridDim.x * BT_THREADS * 4) {
+    const u32x4 m = *reinterpret_cast<const u32x4 *>(gran_max + i);      // n is a multiple of 4
+    if (m.x) atomicAdd(&h[m.x >> 20], 1u);
+    if (m.y) atomicAdd(&h[m.y >> 20], 1u);
+    if (m.z) atomicAdd(&h[m.z >> 20], 1u);
+    if (m.w) atomicAdd(&h[m.w >> 20], 1u);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < BT_BINS; i += BT_THREADS)
+    if (h[i]) atomicAdd(&hist[i], h[i]);
+}
+
 constexpr int BT_TOKENS_PER_WG = 4;  // gather, next, count, emit: one wave per token
 
 struct BatchCandidates {     // the keys >= lower, token by token, each token's in ascending feature order
@@ -623,7 +642,7 @@ template <bool BF16>
 static int run_batch_select(const void *pre, const float *b_enc, const float *scale, const float *fmask, int64_t B,
                             int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
                             int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
-                            hipStream_t st) {
+                            hipStream_t st, const uint32_t *gran_max_given = nullptr) {
   constexpr int V = BatchReader<BF16>::V;
   char *ws = reinterpret_cast<char *>(workspace);
   BatchSelState *state = reinterpret_cast<BatchSelState *>(ws);
@@ -631,8 +650,10 @@ static int run_batch_select(const void *pre, const float *b_enc, const float *sc
                    ((((uintptr_t)pre | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)fmask) & 15) == 0);
   const int nseg = (int)((F + 64 * V - 1) / (64 * V)), ngran = (int)((F + BT_GL * V - 1) / (BT_GL * V) + 3) / 4 * 4;
   uint32_t *hist = reinterpret_cast<uint32_t *>(ws + 256);
-  uint32_t *gran_max = reinterpret_cast<uint32_t *>(ws + 256 + BT_BINS * 4);   // 16-byte aligned rows
-  int32_t *n_gt = reinterpret_cast<int32_t *>(gran_max + B * ngran);
+  uint32_t *gran_ws = reinterpret_cast<uint32_t *>(ws + 256 + BT_BINS * 4);   // 16-byte aligned rows
+  // maxima handed in (same granules, same keys: [B, F / 64] with F / 64 a multiple of 4) are read where they lie
+  const uint32_t *gran_max = gran_max_given ? gran_max_given : gran_ws;
+  int32_t *n_gt = reinterpret_cast<int32_t *>(gran_ws + B * ngran);
   int32_t *n_tie = n_gt + B;
   int32_t *tie_keep = n_tie + B;
   BatchCandidates cd;
@@ -644,8 +665,14 @@ static int run_batch_select(const void *pre, const float *b_enc, const float *sc
   BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F, vec ? 1 : 0, nseg, ngran};
   hipLaunchKernelGGL(bt_init_kernel, dim3(1), dim3(256), 0, st, state, hist, k_total, k_total_dev, bt_candidate_capacity(B, F));
   const int rows_per_wg = (int)(B / 65535 > 16 ? B / 65535 + 1 : 16);
-  hipLaunchKernelGGL(bt_first_kernel<BF16>, dim3((unsigned)((nseg + BT_WAVES - 1) / BT_WAVES), (unsigned)((B + rows_per_wg - 1) / rows_per_wg)),
-                     dim3(BT_THREADS), 0, st, rd, (int)B, rows_per_wg, state, hist, gran_max);
+  if (gran_max_given) {
+    const int64_t n = B * ngran;
+    const int64_t blocks = (n / 4 + BT_THREADS - 1) / BT_THREADS;
+    hipLaunchKernelGGL(bt_hist_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(BT_THREADS), 0, st, gran_max, n, state, hist);
+  } else {
+    hipLaunchKernelGGL(bt_first_kernel<BF16>, dim3((unsigned)((nseg + BT_WAVES - 1) / BT_WAVES), (unsigned)((B + rows_per_wg - 1) / rows_per_wg)),
+                       dim3(BT_THREADS), 0, st, rd, (int)B, rows_per_wg, state, hist, gran_ws);
+  }
   hipLaunchKernelGGL(bt_bound_kernel, dim3(1), dim3(1024), 0, st, state, hist);
   const unsigned token_grid = (unsigned)((B + BT_TOKENS_PER_WG - 1) / BT_TOKENS_PER_WG);
   const dim3 token_block(BT_TOKENS_PER_WG * 64);
@@ -695,4 +722,22 @@ extern "C" int sae_select_topk_batch(const void *pre, int pre_dtype, const float
                                   row_nnz, total_out, workspace, st);
   return run_batch_select<false>(pre, b_enc, scale, feat_mask, B, F, k_total, k_total_dev, idx, val, capacity, row_off,
                                  row_nnz, total_out, workspace, st);
+}
+
+extern "C" int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                             const float *scale, int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev,
+                                             int32_t *idx, float *val, int64_t capacity, int64_t *row_off, int32_t *row_nnz,
+                                             int64_t *total_out, void *workspace, int64_t workspace_bytes, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre_bf16 && granule_max && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_batch_granule: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F <= (1LL << 30), SAE_ERR_INVALID_ARG, "select_topk_batch_granule: bad shape");
+  SAE_REQUIRE(F % 256 == 0, SAE_ERR_UNSUPPORTED, "select_topk_batch_granule: F=%lld must be a multiple of 256", (long long)F);
+  SAE_REQUIRE(k_total_dev || k_total >= 0, SAE_ERR_INVALID_ARG, "select_topk_batch_granule: k_total must be >= 0");
+  SAE_REQUIRE(capacity > 0, SAE_ERR_INVALID_ARG, "select_topk_batch_granule: capacity must be positive");
+  SAE_REQUIRE(workspace && workspace_bytes >= sae_select_topk_batch_workspace_bytes(B, F), SAE_ERR_WORKSPACE,
+              "select_topk_batch_granule: workspace of %lld bytes needed", (long long)sae_select_topk_batch_workspace_bytes(B, F));
+  SAE_REQUIRE((((uintptr_t)workspace) & 255) == 0 && (((uintptr_t)granule_max | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0,
+              SAE_ERR_INVALID_ARG, "select_topk_batch_granule: workspace must be 256-byte, the other pointers 16-byte aligned");
+  return run_batch_select<true>(pre_bf16, b_enc, scale, nullptr, B, F, k_total, k_total_dev, idx, val, capacity, row_off, row_nnz,
+                                total_out, workspace, (hipStream_t)stream, granule_max);
 }

@@ -457,10 +457,19 @@ def select_topk_batch(
     k_total,
     feat_mask: Optional[torch.Tensor] = None,
     capacity: Optional[int] = None,
+    granule_max: Optional[torch.Tensor] = None,
 ) -> SparseCode:
-    """Batch-global TopK.  `k_total` is an int, or a device int64 tensor (then `capacity` is required)."""
+    """Batch-global TopK.  `k_total` is an int, or a device int64 tensor (then `capacity` is required).
+    `granule_max`: the second output of `encoder_gemm_granule_max` for the same bf16 pre, b_enc and scale (F a multiple
+    of 256, no feat_mask); the select's one full pass over the matrix then shrinks to a histogram of those maxima."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
+    if granule_max is not None:
+        if feat_mask is not None or pre.dtype != torch.bfloat16 or F % 256:
+            raise ValueError("granule_max needs a bf16 pre with F a multiple of 256 and no feat_mask")
+        _req(granule_max, "granule_max", torch.int32, 2)
+        if tuple(granule_max.shape) != (B, F // GRANULE):
+            raise ValueError(f"granule_max must be [{B}, {F // GRANULE}]")
     for name, t in (("b_enc", b_enc), ("scale", scale), ("feat_mask", feat_mask)):
         if t is not None:
             _req(t, name, torch.float32, 1)
@@ -485,12 +494,15 @@ def select_topk_batch(
     ws_bytes = lib.sae_select_topk_batch_workspace_bytes(B, F)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with _timed("select_topk_batch"):
-        check(
-            lib.sae_select_topk_batch(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
-                                      _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
-                                      row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre)),
-            "select_topk_batch",
-        )
+        if granule_max is not None:
+            rc = lib.sae_select_topk_batch_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k_host,
+                                                   _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
+                                                   row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
+        else:
+            rc = lib.sae_select_topk_batch(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
+                                           _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
+                                           row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
+        check(rc, "select_topk_batch")
     return SparseCode(idx, val, row_off, row_nnz, B, F)
 
 

@@ -222,11 +222,13 @@ class _FusedSparseStep(torch.autograd.Function):
             b_D = b_D.float() if b_D is not None else None
         B = x.shape[0]
         batch_wide = sae.cfg.act_fn.lower() == "batchtopk"
-        # per-token TopK on bf16 operands: the GEMM's epilogue leaves the largest select key of every 64-feature granule,
-        # and the select reads the row only in the granules that can hold a kept element.  The keys need the decoder
+        # TopK / BatchTopK on bf16 operands: the GEMM's epilogue leaves the largest select key of every 64-feature granule;
+        # the per-token select then reads a row only in the granules that can hold a kept element, and the batch-wide
+        # select is spared its one pass over the whole matrix.  The keys need the decoder
         # norms, so this route fetches them before the GEMM (and waits there for an overlapped decoder update).
-        granule = (amp and not lowp and not batch_wide and getattr(sae, "granule_select", True)
-                   and not sae._update_pending() and ops.granule_route_supported(x.shape[1], w_enc_op.shape[0], int(k)))
+        granule = (amp and not lowp and getattr(sae, "granule_select", True) and not sae._update_pending()
+                   and (ops.granule_route_supported(x.shape[1], w_enc_op.shape[0], int(k)) if not batch_wide
+                        else x.shape[1] % 64 == 0 and w_enc_op.shape[0] % 256 == 0))
         gmax = None
         if granule:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
@@ -246,7 +248,7 @@ class _FusedSparseStep(torch.autograd.Function):
                 scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
         w_dec_op = sae._w_dec_operand(amp)
         if batch_wide:
-            code = ops.select_topk_batch(pre, b_E, scale, k * B)
+            code = ops.select_topk_batch(pre, b_E, scale, k * B, granule_max=gmax)
         else:
             code = ops.select_topk_row(pre, b_E, scale, k, lowp=lowp, granule_max=gmax)
         aux = holder.aux

@@ -194,3 +194,19 @@ def test_standalone_granule_max(pkg, dev, B, F, groups):
     a = pkg.ops.select_topk_row(pre, None, None, k, granule_max=got0)
     w = pkg.ops.select_topk_row(pre, None, None, k)
     assert torch.equal(a.idx, w.idx) and torch.equal(a.val, w.val) and torch.equal(a.row_nnz, w.row_nnz)
+
+
+@pytest.mark.parametrize("B,d,F,k", [(64, 64, 256, 4), (300, 128, 1024, 16), (128, 64, 2048, 100)])
+def test_batch_select_with_granule_maxima_equals_batch_select(pkg, dev, B, d, F, k):
+    x, w, b, s = _inputs(B, d, F, seed=B + 5 * k, dev=dev)
+    pre, gmax = pkg.ops.encoder_gemm_granule_max(x, w, b, s)
+    got = pkg.ops.select_topk_batch(pre, b, s, k * B, granule_max=gmax)
+    want = pkg.ops.select_topk_batch(pre, b, s, k * B)
+    assert torch.equal(got.row_nnz, want.row_nnz) and torch.equal(got.row_off, want.row_off)
+    assert torch.equal(got.idx, want.idx) and torch.equal(got.val, want.val)
+    # nothing kept, and more asked for than there are positive entries
+    zero = pkg.ops.select_topk_batch(pre, b, s, 0, granule_max=gmax)
+    assert int(zero.row_nnz.sum()) == 0
+    every = pkg.ops.select_topk_batch(pre, b, s, B * F, granule_max=gmax)
+    ref = pkg.ops.select_topk_batch(pre, b, s, B * F)
+    assert torch.equal(every.row_nnz, ref.row_nnz) and torch.equal(every.idx, ref.idx) and torch.equal(every.val, ref.val)
