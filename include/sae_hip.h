@@ -513,13 +513,24 @@ int sae_row_sum(const void *src, int src_dtype, int64_t rows, int64_t cols, floa
  *     of kept features (both nullable).
  * (row_off, row_nnz, idx, val) is a sparse code as the TopK select emits it: sae_sparse_decode_mse_fused gives the value
  * gradients of all entries (the flagged ones included: their threshold gradient needs them), sae_build_feature_index and
- * the factored optimizer pass take it as it is.  F must be a multiple of 8. */
+ * the factored optimizer pass take it as it is.  F must be a multiple of 8.
+ * granule_margin (nullable; fp32 [B, F / 64], F % 64 == 0, F <= 262144): the second output of
+ * sae_encoder_gemm_jumprelu_margin for the same pre, b_enc, scale and theta.  Only granules whose margin reaches
+ * -window / 2 are then read from pre; the entries are the same (the per-token tanh sums add their terms in another order). */
 int sae_jumprelu_select_count(const void *pre, int dtype, const float *b_enc, const float *scale, const float *theta,
-                              double window, int64_t B, int64_t F, int32_t *row_nnz, void *stream);
+                              const float *granule_margin, double window, int64_t B, int64_t F, int32_t *row_nnz, void *stream);
 int sae_jumprelu_select_emit(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
-                             const float *theta, double window, double tanh_c, int64_t B, int64_t F, const int64_t *row_off,
-                             int32_t *idx, float *val, float *in_window, int64_t capacity, float *tanh_tok, float *l0_tok,
-                             void *stream);
+                             const float *theta, const float *granule_margin, double window, double tanh_c, int64_t B, int64_t F,
+                             const int64_t *row_off, int32_t *idx, float *val, float *in_window, int64_t capacity, float *tanh_tok,
+                             float *l0_tok, void *stream);
+
+/* sae_encoder_gemm (bf16 operands and output, d % 64 == 0, F % 64 == 0) whose epilogue also writes
+ * granule_margin [B, F / 64] (fp32): for every token and aligned granule of 64 features the largest
+ * (bf16(pre) + b_enc) * scale - theta, product and difference rounded separately as in the activation kernels
+ * (b_enc / scale nullable: 0 / 1).  Replaces `x @ W_E` ahead of the sparse JumpReLU select (models/sae.py:323-324). */
+int sae_encoder_gemm_jumprelu_margin(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d, int64_t F,
+                                     const float *b_enc, const float *scale, const float *theta, float *granule_margin,
+                                     void *stream);
 
 /* out_a[f] = sum over the slots of feature f (feat_ptr / feat_slot of sae_build_feature_index) of a[slot], and the same
  * for b -> out_b (b, out_b nullable): the per-feature sums autograd forms by summing a dense [B, F] gradient over the

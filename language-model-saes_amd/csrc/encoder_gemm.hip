@@ -297,19 +297,22 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
 // EPI_BIAS (bf16 output): out = bf16(float(bf16(acc)) + bias), the value of `(x @ w) + bias` when the product is a bf16
 // tensor and the bias an fp32 one; `b_enc` then holds a bias per output column (nullable), `scale` one per output row
 // (nullable).
-constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2;
+// EPI_MARGIN (bf16 output, N a multiple of 64): like EPI_GMAX, but what is written per token and granule is the largest
+// JumpReLU margin (out + bias) * scale - theta of the granule's rounded outputs (a float, each operation rounded on its
+// own as the activation kernels do): a granule holds an active or in-window entry only if that reaches -window / 2.
+constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2, EPI_MARGIN = 3;
 template <bool BF16_OUT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
     int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
-    const float *__restrict__ scale, uint32_t *__restrict__ gmax) {
+    const float *__restrict__ scale, uint32_t *__restrict__ gmax, const float *__restrict__ theta) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
   if (blockIdx.y) {      // group g of a batch of independent products of one shape, each operand stacked group after group
     const size_t g = blockIdx.y;
     x += g * (size_t)M * row_bytes;
     w += g * (size_t)N * row_bytes;
     out = reinterpret_cast<char *>(out) + g * (size_t)M * N * (BF16_OUT ? 2 : 4);
-    if constexpr (EPI == EPI_GMAX) {
+    if constexpr (EPI == EPI_GMAX || EPI == EPI_MARGIN) {
       if (b_enc) b_enc += g * (size_t)N;
       if (scale) scale += g * (size_t)N;
       gmax += g * (size_t)M * (N >> 6);
@@ -398,7 +401,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
 
   // EPI_GMAX: this lane's 16 bias and 16 scale values; EPI_BIAS: its 16 column biases and 8 row biases.  Asked for here
   // so that the epilogue does not wait for them.
-  constexpr bool GMAX = EPI == EPI_GMAX, BIAS = EPI == EPI_BIAS;
+  constexpr bool MARGIN = EPI == EPI_MARGIN, GMAX = EPI == EPI_GMAX || MARGIN, BIAS = EPI == EPI_BIAS;
   float bb[EPI != EPI_NONE ? 4 : 1][4], ss[GMAX ? 4 : 1][4], rb[BIAS ? 8 : 1];
   if constexpr (EPI != EPI_NONE) {
     const int f0 = n0 + wn * 64;
@@ -470,11 +473,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const int f0 = n0 + wn * 64;
     if (f0 < N) {
       const int ng = N >> 6;
+      float th[MARGIN ? 4 : 1][4];
+      if constexpr (MARGIN) {     // the thresholds are asked for here: the main loop's fragment registers are free now
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float4 t4 = *reinterpret_cast<const float4 *>(theta + f0 + i * 16 + 4 * fq);
+          th[i][0] = t4.x; th[i][1] = t4.y; th[i][2] = t4.z; th[i][3] = t4.w;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         // positive floats order like their bit patterns, so the largest key is the key of the largest h1; the maximum
         // starts at 0 and v_max ignores NaN operands, as the key of a NaN (0) is ignored
-        float hmax = 0.f;
+        float hmax = MARGIN ? -INFINITY : 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           // the accumulators take their rounded values here, so the stores below write exactly what the keys were formed from
@@ -482,12 +493,16 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
           acc[i][j][0] = __uint_as_float(lo << 16); acc[i][j][1] = __uint_as_float(lo & 0xffff0000u);
           acc[i][j][2] = __uint_as_float(hi << 16); acc[i][j][3] = __uint_as_float(hi & 0xffff0000u);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) hmax = fmaxf(hmax, (acc[i][j][r] + bb[i][r]) * ss[i][r]);   // h1 of select_key_plain
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (MARGIN) hmax = fmaxf(hmax, sub_rn(mul_rn(acc[i][j][r] + bb[i][r], ss[i][r]), th[i][r]));
+            else hmax = fmaxf(hmax, (acc[i][j][r] + bb[i][r]) * ss[i][r]);   // h1 of select_key_plain
+          }
         }
         hmax = fmaxf(hmax, __shfl_xor(hmax, 16, 64));
         hmax = fmaxf(hmax, __shfl_xor(hmax, 32, 64));
         const int tok = m0 + wm * 128 + j * 16 + frow;
-        if (fq == 0 && tok < M) gmax[(size_t)tok * ng + (f0 >> 6)] = hmax > 0.f ? __float_as_uint(hmax) : 0u;
+        if (fq == 0 && tok < M)
+          gmax[(size_t)tok * ng + (f0 >> 6)] = MARGIN ? __float_as_uint(hmax) : (hmax > 0.f ? __float_as_uint(hmax) : 0u);
       }
     }
   }
@@ -586,7 +601,8 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
 
 template <bool BF16_OUT, int EPI>
 static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
-                            const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1) {
+                            const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1,
+                            const float *theta = nullptr) {
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
   auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
@@ -595,7 +611,7 @@ static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, 
   const int m_pad = (tiles_m + rm - 1) / rm * rm, n_local_pad = ((tiles_n + 7) / 8 + rn - 1) / rn * rn;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)n_groups), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st,
                      (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale,
-                     gmax);
+                     gmax, theta);
   return check_launch("encoder_gemm");
 }
 
@@ -650,4 +666,20 @@ extern "C" int sae_encoder_gemm_bias(const void *x_bf16, const void *w_t_bf16, v
   SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_t_bf16 | (uintptr_t)out_bf16 | (uintptr_t)col_bias) & 15) == 0, SAE_ERR_INVALID_ARG,
               "encoder_gemm_bias: pointers must be 16-byte aligned");
   return launch_gemm_bf16<true, EPI_BIAS>(x_bf16, w_t_bf16, out_bf16, B, d, F, col_bias, row_bias, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int sae_encoder_gemm_jumprelu_margin(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t B, int64_t d,
+                                                int64_t F, const float *b_enc, const float *scale, const float *theta,
+                                                float *granule_margin, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x_bf16 && w_enc_t_bf16 && pre_bf16 && theta && granule_margin, SAE_ERR_INVALID_ARG,
+              "encoder_gemm_jumprelu_margin: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_jumprelu_margin: sizes must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28), SAE_ERR_UNSUPPORTED, "encoder_gemm_jumprelu_margin: size too large");
+  SAE_REQUIRE(d % 64 == 0 && F % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_jumprelu_margin: d=%lld and F=%lld must be multiples of 64",
+              (long long)d, (long long)F);
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_enc_t_bf16 | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale |
+                (uintptr_t)theta) & 15) == 0, SAE_ERR_INVALID_ARG, "encoder_gemm_jumprelu_margin: pointers must be 16-byte aligned");
+  return launch_gemm_bf16<true, EPI_MARGIN>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale,
+                                            reinterpret_cast<uint32_t *>(granule_margin), (hipStream_t)stream, 1, theta);
 }

@@ -255,17 +255,53 @@ __device__ __forceinline__ void jr_classify(const void *__restrict__ pre, const 
   }
 }
 
+// With the per-granule margins of the encoder product's epilogue (margin[row][F / 64] = the largest (h s - theta) of
+// the granule) only granules whose margin reaches -window / 2 can hold an entry: their numbers, ascending, are listed
+// in LDS and the kernels below walk the 16-byte chunks of those granules instead of the whole row.  Returns the number
+// of listed granules (the same in every thread).  `tot` is JR_THREADS / 64 ints of LDS.
+constexpr int JR_MAX_GRANULES = 4096;
+__device__ __forceinline__ int jr_live_granules(const float *__restrict__ margin_row, int n_gran, float half_w,
+                                                uint16_t *__restrict__ live, int *__restrict__ tot) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int run = 0;
+  for (int g0 = 0; g0 < n_gran; g0 += JR_THREADS) {
+    const int g = g0 + threadIdx.x;
+    const bool on = g < n_gran && margin_row[g] > -half_w;
+    const unsigned long long m = __ballot(on);
+    __syncthreads();                                  // the previous round's totals have been read
+    if (lane == 0) tot[wave] = __popcll(m);
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < JR_THREADS / 64; ++w) {
+      const int t = tot[w];
+      before += w < wave ? t : 0;
+      total += t;
+    }
+    if (on) live[run + before + __popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)g;
+    run += total;
+  }
+  __syncthreads();
+  return run;
+}
+
 template <bool BF16>
 __global__ __launch_bounds__(JR_THREADS) void jumprelu_select_count_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
-    const float *__restrict__ theta, int64_t F, float half_w, int32_t *__restrict__ row_nnz) {
+    const float *__restrict__ theta, int64_t F, float half_w, int32_t *__restrict__ row_nnz, const float *__restrict__ margin) {
   __shared__ float red[JR_THREADS / 64];
-  const int64_t row = blockIdx.x, groups = F >> 3;
+  __shared__ uint16_t live[JR_MAX_GRANULES];
+  __shared__ int tot[JR_THREADS / 64];
+  const int64_t row = blockIdx.x;
+  int64_t groups = F >> 3;
+  const int64_t rbase = row * groups;
+  if (margin) groups = 8 * (int64_t)jr_live_granules(margin + row * (F >> 6), (int)(F >> 6), half_w, live, tot);
   int cnt = 0;
-  for (int64_t g = threadIdx.x; g < groups; g += JR_THREADS) {
+  for (int64_t c = threadIdx.x; c < groups; c += JR_THREADS) {
+    const int64_t g = margin ? (int64_t)live[c >> 3] * 8 + (c & 7) : c;
     float a[8];
     bool keep[8], win[8];
-    jr_classify<BF16>(pre, b_enc, scale, theta, row * groups, g, half_w, a, keep, win);
+    jr_classify<BF16>(pre, b_enc, scale, theta, rbase, g, half_w, a, keep, win);
 #pragma unroll
     for (int i = 0; i < 8; ++i) cnt += (keep[i] || win[i]) ? 1 : 0;
   }
@@ -278,20 +314,27 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_select_emit_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ pen, const float *__restrict__ theta, int64_t F, float half_w, float tanh_c,
     const int64_t *__restrict__ row_off, int32_t *__restrict__ idx, float *__restrict__ val, float *__restrict__ in_window,
-    int64_t capacity, float *__restrict__ tanh_tok, float *__restrict__ l0_tok) {
+    int64_t capacity, float *__restrict__ tanh_tok, float *__restrict__ l0_tok, const float *__restrict__ margin) {
   __shared__ float red[JR_THREADS / 64];
   __shared__ int wave_tot[JR_THREADS / 64];
-  const int64_t row = blockIdx.x, groups = F >> 3;
+  __shared__ uint16_t live[JR_MAX_GRANULES];
+  const int64_t row = blockIdx.x;
+  int64_t groups = F >> 3;
+  const int64_t rbase = row * groups;
+  if (margin) groups = 8 * (int64_t)jr_live_granules(margin + row * (F >> 6), (int)(F >> 6), half_w, live, wave_tot);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int64_t run = row_off[row];
   float tsum = 0.f, kept = 0.f;
   for (int64_t g0 = 0; g0 < groups; g0 += JR_THREADS) {
-    const int64_t g = g0 + threadIdx.x;
+    const int64_t c = g0 + threadIdx.x;
+    // chunk c of the walk: of the row, or of the listed granules (ascending either way, so the entries come out in
+    // ascending feature order)
+    const int64_t g = (margin && c < groups) ? (int64_t)live[c >> 3] * 8 + (c & 7) : c;
     float a[8];
     bool keep[8], win[8];
     int cnt = 0;
-    if (g < groups) {
-      jr_classify<BF16>(pre, b_enc, scale, theta, row * groups, g, half_w, a, keep, win);
+    if (c < groups) {
+      jr_classify<BF16>(pre, b_enc, scale, theta, rbase, g, half_w, a, keep, win);
 #pragma unroll
       for (int i = 0; i < 8; ++i) cnt += (keep[i] || win[i]) ? 1 : 0;
     } else {
@@ -349,38 +392,44 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_select_emit_kernel(
 }  // namespace sae
 
 extern "C" int sae_jumprelu_select_count(const void *pre, int dtype, const float *b_enc, const float *scale, const float *theta,
-                                         double window, int64_t B, int64_t F, int32_t *row_nnz, void *stream) {
+                                         const float *granule_margin, double window, int64_t B, int64_t F, int32_t *row_nnz,
+                                         void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre && theta && row_nnz, SAE_ERR_INVALID_ARG, "jumprelu_select_count: null pointer");
+  SAE_REQUIRE(!granule_margin || (F % 64 == 0 && F / 64 <= JR_MAX_GRANULES), SAE_ERR_UNSUPPORTED,
+              "jumprelu_select_count: granule margins need F a multiple of 64, at most %d", 64 * JR_MAX_GRANULES);
   SAE_REQUIRE(B > 0 && F > 0 && (F & 7) == 0 && B < ((int64_t)1 << 31), SAE_ERR_INVALID_ARG,
               "jumprelu_select_count: B > 0 and F a positive multiple of 8 expected");
   SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "jumprelu_select_count: bad dtype");
   const float hw = 0.5f * (float)window;
   if (dtype == SAE_BF16)
     hipLaunchKernelGGL(jumprelu_select_count_kernel<true>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
-                       scale, theta, F, hw, row_nnz);
+                       scale, theta, F, hw, row_nnz, granule_margin);
   else
     hipLaunchKernelGGL(jumprelu_select_count_kernel<false>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
-                       scale, theta, F, hw, row_nnz);
+                       scale, theta, F, hw, row_nnz, granule_margin);
   return check_launch("jumprelu_select_count");
 }
 
 extern "C" int sae_jumprelu_select_emit(const void *pre, int dtype, const float *b_enc, const float *scale, const float *pen_norm,
-                                        const float *theta, double window, double tanh_c, int64_t B, int64_t F,
+                                        const float *theta, const float *granule_margin, double window, double tanh_c, int64_t B,
+                                        int64_t F,
                                         const int64_t *row_off, int32_t *idx, float *val, float *in_window, int64_t capacity,
                                         float *tanh_tok, float *l0_tok, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre && theta && row_off && idx && val && in_window, SAE_ERR_INVALID_ARG, "jumprelu_select_emit: null pointer");
+  SAE_REQUIRE(!granule_margin || (F % 64 == 0 && F / 64 <= JR_MAX_GRANULES), SAE_ERR_UNSUPPORTED,
+              "jumprelu_select_emit: granule margins need F a multiple of 64, at most %d", 64 * JR_MAX_GRANULES);
   SAE_REQUIRE(B > 0 && F > 0 && (F & 7) == 0 && B < ((int64_t)1 << 31) && capacity >= 0, SAE_ERR_INVALID_ARG,
               "jumprelu_select_emit: B > 0 and F a positive multiple of 8 expected");
   SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "jumprelu_select_emit: bad dtype");
   const float hw = 0.5f * (float)window;
   if (dtype == SAE_BF16)
     hipLaunchKernelGGL(jumprelu_select_emit_kernel<true>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
-                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok);
+                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok, granule_margin);
   else
     hipLaunchKernelGGL(jumprelu_select_emit_kernel<false>, dim3((unsigned)B), dim3(JR_THREADS), 0, (hipStream_t)stream, pre, b_enc,
-                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok);
+                       scale, pen_norm, theta, F, hw, (float)tanh_c, row_off, idx, val, in_window, capacity, tanh_tok, l0_tok, granule_margin);
   return check_launch("jumprelu_select_emit");
 }
 

@@ -365,6 +365,30 @@ def granule_max(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optiona
     return gmax
 
 
+def encoder_gemm_jumprelu_margin(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor],
+                                 theta: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16 pre[B, F] = x @ w_enc_t^T plus granule_margin [B, F / 64] fp32: per token and aligned granule of 64 features the
+    largest (pre + b_enc) * scale - theta (what `jumprelu_select(..., granule_margin=...)` prunes the row with)."""
+    _req(x, "x", torch.bfloat16, 2)
+    _req(w_enc_t, "w_enc_t", torch.bfloat16, 2)
+    B, d = x.shape
+    F, d2 = w_enc_t.shape
+    if d != d2:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
+    for name, t in (("b_enc", b_enc), ("scale", scale), ("theta", theta)):
+        if t is not None:
+            _req(t, name, torch.float32, 1)
+            if t.numel() != F:
+                raise ValueError(f"{name} must have {F} elements")
+    pre = torch.empty(B, F, dtype=torch.bfloat16, device=x.device)
+    margin = torch.empty(B, max(F // GRANULE, 1), dtype=torch.float32, device=x.device)
+    with _timed("encoder_gemm"):
+        check(_lib.load().sae_encoder_gemm_jumprelu_margin(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _ptr(b_enc),
+                                                           _ptr(scale), theta.data_ptr(), margin.data_ptr(), _stream(x)),
+              "encoder_gemm_jumprelu_margin")
+    return pre, margin
+
+
 def merge_layer_codes(code: SparseCode, L: int) -> Tuple[SparseCode, torch.Tensor]:
     """`code`: one select over L * B stacked rows (row l * B + b, at most k entries each, F features) -> the code over
     L * F features with L * k slots per token (feature l * F + f, ascending) and the entry counts [B, L]."""
@@ -854,19 +878,24 @@ def jumprelu_bwd(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Option
 
 def jumprelu_select(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], theta: torch.Tensor,
                     window: float, tanh_c: float = 0.0, pen_norm: Optional[torch.Tensor] = None, want_tanh: bool = False,
-                    max_entries: Optional[int] = None):
+                    max_entries: Optional[int] = None, granule_margin: Optional[torch.Tensor] = None):
     """Sparse form of the JumpReLU activation: the code of every token's kept features (value u / s) and of the features
     inside the straight-through window that are not kept (value 0) -> (code, in_window fp32 [n_slots], tanh_tok [B] or
     None, l0_tok [B]), or None when the batch holds no such entry or more than `max_entries` of them (the caller then
     takes the dense route).  The entry count is read back from the device to size the code: one synchronisation per call, as the
-    reference's sparsity gate (models/sae.py:355-358)."""
+    reference's sparsity gate (models/sae.py:355-358).  `granule_margin`: the second output of `encoder_gemm_jumprelu_margin`
+    for the same arguments; the kernels then read only the granules of `pre` that can hold an entry."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
+    if granule_margin is not None:
+        _req(granule_margin, "granule_margin", torch.float32, 2)
+        if tuple(granule_margin.shape) != (B, F // GRANULE) or F % GRANULE or F > GRANULE_MAX_F:
+            raise ValueError(f"granule_margin must be [{B}, {F}/{GRANULE}] with F a multiple of {GRANULE}, at most {GRANULE_MAX_F}")
     lib = _lib.load()
     row_nnz = torch.empty(B, dtype=torch.int32, device=pre.device)
     with _timed("jumprelu_select"):
-        check(lib.sae_jumprelu_select_count(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), theta.data_ptr(), float(window), B, F,
-                                            row_nnz.data_ptr(), _stream(pre)), "jumprelu_select_count")
+        check(lib.sae_jumprelu_select_count(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), theta.data_ptr(), _ptr(granule_margin),
+                                            float(window), B, F, row_nnz.data_ptr(), _stream(pre)), "jumprelu_select_count")
         incl = torch.cumsum(row_nnz, 0, dtype=torch.int64)
         total = int(incl[-1].item())
         if total == 0 or (max_entries is not None and total > max_entries):
@@ -879,7 +908,8 @@ def jumprelu_select(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Opt
         tanh_tok = torch.empty(B, dtype=torch.float32, device=pre.device) if want_tanh else None
         l0_tok = torch.empty(B, dtype=torch.float32, device=pre.device)
         check(lib.sae_jumprelu_select_emit(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(pen_norm), theta.data_ptr(),
-                                           float(window), float(tanh_c), B, F, row_off.data_ptr(), idx.data_ptr(), val.data_ptr(),
+                                           _ptr(granule_margin), float(window), float(tanh_c), B, F, row_off.data_ptr(),
+                                           idx.data_ptr(), val.data_ptr(),
                                            win.data_ptr(), total, _ptr(tanh_tok), l0_tok.data_ptr(), _stream(pre)),
               "jumprelu_select_emit")
     return SparseCode(idx, val, row_off, row_nnz, B, F), win, tanh_tok, l0_tok

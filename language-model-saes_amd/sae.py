@@ -871,14 +871,22 @@ class SparseAutoEncoder(SparseDictionary):
                 and self.cfg.d_model % 8 == 0 and self._jr_dense_steps % max(1, self.jumprelu_sparse_probe_every) == 0):
             with torch.no_grad():
                 x_op = (x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())) if amp else x.float().contiguous()
-                pre_raw = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16 if amp else torch.float32)
-                given = (x_op, pre_raw)
                 n_raw = self._decoder_norm_nograd() if (scaled or want_tanh) else None
                 th_raw = jr.get_jumprelu_threshold().detach().float().contiguous()
+                b_raw = self.b_E.detach().float()
+                margin = None
+                # once the route has been sparse, the product's epilogue also leaves every granule's largest margin over
+                # its thresholds, and the select reads the pre-activations only where an entry can be
+                if (amp and self._jr_dense_steps == 0 and getattr(self, "granule_select", True) and w_enc_op.dtype == torch.bfloat16
+                        and self.cfg.d_model % 64 == 0 and self.cfg.d_sae % ops.GRANULE == 0 and self.cfg.d_sae <= ops.GRANULE_MAX_F):
+                    pre_raw, margin = ops.encoder_gemm_jumprelu_margin(x_op, w_enc_op, b_raw, n_raw if scaled else None, th_raw)
+                else:
+                    pre_raw = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16 if amp else torch.float32)
+                given = (x_op, pre_raw)
                 budget = int(B * self.cfg.d_sae * (1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel))
-                picked = ops.jumprelu_select(pre_raw, self.b_E.detach().float(), n_raw if scaled else None, th_raw,
+                picked = ops.jumprelu_select(pre_raw, b_raw, n_raw if scaled else None, th_raw,
                                              float(jr.jumprelu_threshold_window), float(tanh_stretch_coefficient), pen_norm=n_raw,
-                                             want_tanh=want_tanh, max_entries=budget)
+                                             want_tanh=want_tanh, max_entries=budget, granule_margin=margin)
             if picked is not None:
                 self._jr_dense_steps = 0
                 return self._jumprelu_sparse_loss(batch, x, label, mask, picked, x_op, amp, defer, scaled, want_tanh,

@@ -341,6 +341,35 @@ def test_jumprelu_select_lists_kept_and_window_entries(pkg, dev, dtype, with_sca
     assert pkg.ops.jumprelu_select(pre.to(dev), None, None, (theta + 100).to(dev), window) is None
 
 
+@pytest.mark.parametrize("with_scale", [True, False])
+@pytest.mark.parametrize("B,d,F,theta0", [(70, 64, 1024, 1.5), (300, 128, 4096, 2.5), (33, 64, 64, 0.2)])
+def test_jumprelu_margin_route_lists_the_same_entries(pkg, dev, with_scale, B, d, F, theta0):
+    """sae_encoder_gemm_jumprelu_margin: the same pre-activations as the plain product, and per granule the largest
+    (pre + b) s - theta with product and difference rounded separately; the select that reads only the granules those
+    margins allow returns the code of the select that reads every row, bit for bit."""
+    g = torch.Generator().manual_seed(B + F)
+    x = torch.randn(B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(F, d, generator=g) / d ** 0.5).to(torch.bfloat16).to(dev)
+    b = (0.1 * torch.randn(F, generator=g)).to(dev)
+    s = (0.5 + torch.rand(F, generator=g)).to(dev) if with_scale else None
+    theta = (theta0 + 0.5 * torch.rand(F, generator=g)).to(dev)
+    window, c = 0.3, 2.0
+    pre, margin = pkg.ops.encoder_gemm_jumprelu_margin(x, w, b, s, theta)
+    assert torch.equal(pre, pkg.ops.encoder_gemm(x, w, torch.bfloat16))
+    h = pre.float() + b
+    u = h * s if s is not None else h
+    want_margin = (u - theta).view(B, F // 64, 64).max(dim=2).values
+    assert torch.equal(margin, want_margin)
+    got = pkg.ops.jumprelu_select(pre, b, s, theta, window, c, pen_norm=s, want_tanh=True, granule_margin=margin)
+    ref = pkg.ops.jumprelu_select(pre, b, s, theta, window, c, pen_norm=s, want_tanh=True)
+    assert (got is None) == (ref is None)
+    if ref is not None:
+        (gc, gw, gt, gl), (rc, rw, rt, rl) = got, ref
+        assert torch.equal(gc.row_nnz, rc.row_nnz) and torch.equal(gc.row_off, rc.row_off)
+        assert torch.equal(gc.idx, rc.idx) and torch.equal(gc.val, rc.val) and torch.equal(gw, rw) and torch.equal(gl, rl)
+        assert ((gt - rt).abs().max() / rt.abs().max().clamp_min(1e-30)).item() < 1e-5     # another summation order
+
+
 @pytest.mark.parametrize("include_norm", [True, False])
 @pytest.mark.parametrize("kw", [dict(), dict(sparsity_loss_type="tanh", l1_coefficient=0.05, tanh_stretch_coefficient=2.0)])
 def test_sparse_jumprelu_step_fp32_matches_oracle(pkg, oracle, dev, include_norm, kw):

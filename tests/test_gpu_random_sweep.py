@@ -133,16 +133,27 @@ def test_random_sweep_attention_and_code_conversions(pkg, oracle, dev, sweep_see
             scale = 1.0 / math.sqrt(dq)
             sc = torch.einsum("bqhd,bkhd->bhqk", ql.view(nb, s, h, dq), kl.view(nb, s, h, dq)) * scale
             sc = sc.masked_fill(~torch.ones(s, s, dtype=torch.bool).tril(), float("-inf"))
-            want = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(sc, -1), vl.view(nb, s, h, dv)).reshape(T, h * dv)
-            (want * do.double()).sum().backward()
+            P = torch.softmax(sc, -1).detach()
+            want = torch.einsum("bhqk,bkhd->bqhd", P, vl.detach().view(nb, s, h, dv)).reshape(T, h * dv)
             dv_ = lambda t: None if t is None else t.to(dev)                                               # noqa: E731
             gq, gk, gv, gdo = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
             out, lse = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
             rel = lambda a, b: ((a.double().cpu() - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()  # noqa: E731
-            assert rel(out, want.detach()) < 8e-3
+            assert rel(out, want) < 8e-3
             dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(),
                                                   lse, nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
-            assert rel(dqt.t(), ql.grad) < 2e-2 and rel(dkt.t(), kl.grad) < 2e-2 and rel(dvt.t(), vl.grad) < 2e-2
+            # The backward of a fused attention (this one and the library routine the reference calls) takes the SAVED
+            # output, a bf16 tensor, for D = rowsum(dout * out); on short sequences with wide value heads that rounding
+            # is not averaged away (seen: 3 % of max |dk| at s = 8, d_v = 128 against autograd through the exact output).
+            # The gradients are therefore checked against the exact formulas with D formed from the kernel's own output.
+            do4, v4 = do.double().view(nb, s, h, dv), vl.detach().view(nb, s, h, dv)
+            D = (do4 * out.double().cpu().view(nb, s, h, dv)).sum(-1).permute(0, 2, 1)                 # [nb, h, s]
+            dP = torch.einsum("bqhd,bkhd->bhqk", do4, v4)
+            dS = P * (dP - D[..., None])
+            want_dq = scale * torch.einsum("bhqk,bkhd->bqhd", dS, kl.detach().view(nb, s, h, dq)).reshape(T, h * dq)
+            want_dk = scale * torch.einsum("bhqk,bqhd->bkhd", dS, ql.detach().view(nb, s, h, dq)).reshape(T, h * dq)
+            want_dv = torch.einsum("bhqk,bqhd->bkhd", P, do4).reshape(T, h * dv)
+            assert rel(dqt.t(), want_dq) < 2e-2 and rel(dkt.t(), want_dk) < 2e-2 and rel(dvt.t(), want_dv) < 2e-2
         elif kind == "dense_code":
             B = rng.choice([1, 5, 40]); F = rng.choice([8, 100, 2047, 4096, 20000, 131072]); dt = rng.choice([torch.float32, torch.bfloat16])
             dens = rng.choice([0.0, 0.001, 0.05, 0.6])
