@@ -281,7 +281,7 @@ def test_jumprelu_trainer_steps_with_and_without_deferred_terms(pkg, oracle, dev
 # ---- the sparse form of the step: threshold select -> sparse code -> sparse decode / factored gradients ----------
 
 def make_sparse_pair(pkg, oracle, dev, d, F, B, seed, include_norm, window=0.3, theta_lo=1.7, theta_hi=2.3, budget=0.99):
-    """Thresholds around 2 on pre-activations of unit scale: a few entries per thousand are kept, about as many more
+    """Thresholds near 2.0 on pre-activations of unit scale: a few entries per thousand are kept, about as many more
     lie inside the straight-through window."""
     from lm_saes_amd import synthetic
 
