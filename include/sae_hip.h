@@ -232,6 +232,15 @@ int sae_sparse_decode_mse_fused(const int32_t *idx, const float *val, const int6
                                 float *recon, float *loss_tok, float *grad_recon, float *dval,
                                 int64_t B, int64_t d, int64_t F, int64_t n_slots, void *stream);
 
+/* sae_sparse_decode_mse_fused for a code that several decoders share (the cross-layer transcoder's prefix decodes,
+ * models/clt.py:630-709): the value gradients are ADDED to dval_acc [n_slots] (slots a call does not visit keep their
+ * value; the caller clears the array before the first call), so that the sum over the decoders needs no pass of its own.
+ * Each slot is written by the one wave that owns its token: no atomics, the additions happen in call order. */
+int sae_sparse_decode_mse_fused_acc(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
+                                    const void *w_dec, int w_dtype, const float *b_dec, const float *label, const float *tok_w,
+                                    float *recon, float *loss_tok, float *grad_recon, float *dval_acc, int64_t B, int64_t d,
+                                    int64_t F, int64_t n_slots, void *stream);
+
 /* ---- sparse backward -------------------------------------------------------------- */
 
 /* Feature-major index of a sparse code (a CSR transpose): for every feature f the list of

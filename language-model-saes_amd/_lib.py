@@ -42,6 +42,7 @@ SIGNATURES = {
     "sae_sparse_decode_fwd": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _L, _P]),
     "sae_sparse_decode_bwd_dval": (_I, [_P, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _P]),
     "sae_sparse_decode_mse_fused": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _P]),
+    "sae_sparse_decode_mse_fused_acc": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _P]),
     "sae_feature_index_workspace_bytes": (_L, [_L, _L, _L]),
     "sae_build_feature_index": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P]),
     "sae_sparse_grad_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _P]),

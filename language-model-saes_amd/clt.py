@@ -141,19 +141,22 @@ class _FusedCLTStep(torch.autograd.Function):
         tok_w = torch.full((B,), 1.0 / (L * B), dtype=torch.float32, device=x.device)
         w_dec_ops = m._w_dec_operands(amp)
         b_D = dec[L:]
-        recons, grads = [], []
+        grads = []
+        # the L decodes write their reconstructions and per-token losses into one buffer each and add their value gradients
+        # to one array: no stacking copy, no sum pass per layer
+        recon = torch.empty(L, B, d, dtype=torch.float32, device=x.device)
+        loss_toks = torch.empty(L, B, dtype=torch.float32, device=x.device)
         dval = torch.zeros(cat.n_slots, dtype=torch.float32, device=x.device)
-        loss = None
+        prefix_t = prefix.t().contiguous()                                # [L, B]
         for j in range(L):
-            code_j = dataclasses.replace(cat, row_nnz=prefix[:, j].contiguous(), d_sae=(j + 1) * F)
-            recon, loss_tok, grad_recon, dval_j = ops.sparse_decode_mse_fused(
-                code_j, w_dec_ops[j].view((j + 1) * F, d), b_D[j].detach(), label[j].contiguous(), tok_w)
             # the merged code is sorted by layer inside a token, so a token's first prefix[b, j] slots are its entries of
-            # layers <= j; the kernel writes exactly those and leaves every other slot at 0
-            dval += dval_j
-            recons.append(recon); grads.append(grad_recon)
-            loss = loss_tok.sum() if loss is None else loss + loss_tok.sum()
-        recon = torch.stack(recons, dim=0)
+            # layers <= j; the kernel visits exactly those
+            code_j = dataclasses.replace(cat, row_nnz=prefix_t[j], d_sae=(j + 1) * F)
+            _, _, grad_recon, _ = ops.sparse_decode_mse_fused(
+                code_j, w_dec_ops[j].view((j + 1) * F, d), b_D[j].detach(), label[j].contiguous(), tok_w,
+                recon_out=recon[j], loss_out=loss_toks[j], dval_acc=dval)
+            grads.append(grad_recon)
+        loss = loss_toks.sum()
         holder.update(code=cat, pres=pres, norms=norms, layer_cnt=layer_cnt)
         ctx.cat, ctx.grads, ctx.dval, ctx.x_op, ctx.w_enc_op = cat, grads, dval, x_op, w_enc_op
         ctx.shape = (B, L, d, F)

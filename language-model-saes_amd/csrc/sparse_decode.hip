@@ -44,7 +44,7 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
     const int32_t *__restrict__ idx, const float *__restrict__ val, const int64_t *__restrict__ row_off,
     const int32_t *__restrict__ row_nnz, const void *__restrict__ w_dec, const float *__restrict__ b_dec,
     const float *__restrict__ label, const float *__restrict__ tok_w, float *__restrict__ recon,
-    float *__restrict__ loss_tok, float *__restrict__ grad_recon, float *__restrict__ dval, int d) {
+    float *__restrict__ loss_tok, float *__restrict__ grad_recon, float *__restrict__ dval, int d, int acc_dval) {
   extern __shared__ __attribute__((aligned(16))) float g_lds[];  // [d] when DVAL
   constexpr int WAVES = THREADS / 64;
   __shared__ float red[WAVES];
@@ -167,6 +167,9 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
       for (int j0 = wave * 2; j0 < nnz; j0 += WAVES * 2) {
         const bool two = j0 + 1 < nnz;
         const int f0 = idx[off + j0], f1 = idx[off + (two ? j0 + 1 : j0)];
+        // the running sums these two results are added to, asked for together with the rows
+        const float prev0 = (acc_dval && lane == 0) ? dval[off + j0] : 0.f;
+        const float prev1 = (acc_dval && lane == 0 && two) ? dval[off + j0 + 1] : 0.f;
         const char *row0 = wbase + (size_t)f0 * row_bytes, *row1 = wbase + (size_t)f1 * row_bytes;
         float w0[2][8], w1[2][8];
 #pragma unroll
@@ -188,13 +191,17 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
           }
         }
         d0 = wave_sum(d0); d1 = wave_sum(d1);
-        if (lane == 0) { dval[off + j0] = d0; if (two) dval[off + j0 + 1] = d1; }
+        if (lane == 0) {
+          dval[off + j0] = acc_dval ? prev0 + d0 : d0;
+          if (two) dval[off + j0 + 1] = acc_dval ? prev1 + d1 : d1;
+        }
       }
       return;
     }
     for (int j = wave; j < nnz; j += WAVES) {
       const int f = idx[off + j];
       const char *row = wbase + (size_t)f * row_bytes;
+      const float prev = (acc_dval && lane == 0) ? dval[off + j] : 0.f;   // asked for together with the row
       float dot = 0.f;
       for (int seg = lane; seg < n_seg; seg += 64 * 4) {
         float w[4][8];
@@ -217,7 +224,7 @@ __global__ __launch_bounds__(THREADS) void sparse_decode_kernel(
         }
       }
       dot = wave_sum(dot);
-      if (lane == 0) dval[off + j] = dot;
+      if (lane == 0) dval[off + j] = acc_dval ? prev + dot : dot;
     }
   }
 }
@@ -226,7 +233,7 @@ template <bool W_BF16, bool FWD, bool LOSS, bool DVAL>
 static int launch_decode(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
                          const void *w_dec, const float *b_dec, const float *label, const float *tok_w, float *recon,
                          float *loss_tok, float *grad_recon, float *dval, int64_t B, int64_t d, hipStream_t st,
-                         int64_t n_slots = 0) {
+                         int64_t n_slots = 0, int acc_dval = 0) {
   const int n_seg = (int)(d / 8);
   const size_t lds = DVAL ? (size_t)d * sizeof(float) : 0;
   const int segs = (n_seg + DEC_THREADS - 1) / DEC_THREADS;
@@ -239,7 +246,7 @@ static int launch_decode(const int32_t *idx, const float *val, const int64_t *ro
       if (e != hipSuccess) return fail(SAE_ERR_LAUNCH, "sparse_decode: LDS reservation failed: %s", hipGetErrorString(e)); \
     }                                                                                                             \
     hipLaunchKernelGGL(kern, dim3((unsigned)B), dim3(DEC_THREADS), lds, st, idx, val, row_off, row_nnz, w_dec,    \
-                       b_dec, label, tok_w, recon, loss_tok, grad_recon, dval, (int)d);                           \
+                       b_dec, label, tok_w, recon, loss_tok, grad_recon, dval, (int)d, acc_dval);                 \
   } while (0)
   // Short rows (d <= 1024): two waves per token, so that most lanes own a segment and twice as many tokens are
   // resident per CU (the gathers' latency is hidden by resident tokens).  Not when the d val phase has long row
@@ -250,7 +257,7 @@ static int launch_decode(const int32_t *idx, const float *val, const int64_t *ro
   if (n_seg <= 128 && (!DVAL || short_lists)) {
     auto kern = sparse_decode_kernel<W_BF16, 1, FWD, LOSS, DVAL, 128, true>;
     hipLaunchKernelGGL(kern, dim3((unsigned)B), dim3(128), lds, st, idx, val, row_off, row_nnz, w_dec, b_dec, label,
-                       tok_w, recon, loss_tok, grad_recon, dval, (int)d);
+                       tok_w, recon, loss_tok, grad_recon, dval, (int)d, acc_dval);
   } else if (!FWD) SAE_DEC_LAUNCH(1);
   else if (segs <= 1) SAE_DEC_LAUNCH(1);
   else if (segs <= 2) SAE_DEC_LAUNCH(2);
@@ -324,4 +331,22 @@ extern "C" int sae_sparse_decode_mse_fused(const int32_t *idx, const float *val,
                                                  loss_tok, grad_recon, dval, B, d, st, n_slots);
   return launch_decode<false, true, true, true>(idx, val, row_off, row_nnz, w_dec, b_dec, label, tok_w, recon,
                                                 loss_tok, grad_recon, dval, B, d, st, n_slots);
+}
+
+extern "C" int sae_sparse_decode_mse_fused_acc(const int32_t *idx, const float *val, const int64_t *row_off,
+                                               const int32_t *row_nnz, const void *w_dec, int w_dtype, const float *b_dec,
+                                               const float *label, const float *tok_w, float *recon, float *loss_tok,
+                                               float *grad_recon, float *dval_acc, int64_t B, int64_t d, int64_t F,
+                                               int64_t n_slots, void *stream) {
+  using namespace sae;
+  int rc = check_common("sparse_decode_mse_fused_acc", idx, row_off, row_nnz, w_dec, w_dtype, B, d, F);
+  if (rc) return rc;
+  SAE_REQUIRE(val && label && loss_tok && grad_recon && dval_acc && n_slots > 0, SAE_ERR_INVALID_ARG,
+              "sparse_decode_mse_fused_acc: null pointer / n_slots");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_dtype == SAE_BF16)
+    return launch_decode<true, true, true, true>(idx, val, row_off, row_nnz, w_dec, b_dec, label, tok_w, recon,
+                                                 loss_tok, grad_recon, dval_acc, B, d, st, n_slots, 1);
+  return launch_decode<false, true, true, true>(idx, val, row_off, row_nnz, w_dec, b_dec, label, tok_w, recon,
+                                                loss_tok, grad_recon, dval_acc, B, d, st, n_slots, 1);
 }

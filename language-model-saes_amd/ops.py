@@ -576,8 +576,11 @@ def sparse_decode_bwd_dval(code: SparseCode, grad_recon: torch.Tensor, w_dec: to
 
 
 def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Optional[torch.Tensor], label: torch.Tensor,
-                            tok_w: Optional[torch.Tensor], want_recon: bool = True):
-    """Returns (recon or None, loss_tok [B], grad_recon [B, d], dval [n_slots])."""
+                            tok_w: Optional[torch.Tensor], want_recon: bool = True, recon_out: Optional[torch.Tensor] = None,
+                            loss_out: Optional[torch.Tensor] = None, dval_acc: Optional[torch.Tensor] = None):
+    """Returns (recon or None, loss_tok [B], grad_recon [B, d], dval [n_slots]).  `recon_out` [B, d] / `loss_out` [B]
+    (fp32, contiguous) receive those outputs in place of fresh tensors; `dval_acc` [n_slots] has the value gradients
+    added to it (and is returned as dval) instead of being overwritten: for a code several decoders share."""
     _check_code(code, w_dec)
     _req(label, "label", torch.float32, 2)
     F, d = w_dec.shape
@@ -587,17 +590,29 @@ def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Option
     if tok_w is not None:
         _req(tok_w, "tok_w", torch.float32, 1)
     dev = w_dec.device
-    recon = torch.empty(B, d, dtype=torch.float32, device=dev) if want_recon else None
-    loss_tok = torch.empty(B, dtype=torch.float32, device=dev)
+    if recon_out is not None:
+        _req(recon_out, "recon_out", torch.float32, 2)
+        if tuple(recon_out.shape) != (B, d):
+            raise ValueError(f"recon_out must be {(B, d)}")
+    if loss_out is not None:
+        _req(loss_out, "loss_out", torch.float32, 1)
+        if loss_out.numel() != B:
+            raise ValueError(f"loss_out must hold {B} values")
+    if dval_acc is not None:
+        _req(dval_acc, "dval_acc", torch.float32, 1)
+        if dval_acc.numel() != code.n_slots:
+            raise ValueError(f"dval_acc must hold {code.n_slots} values")
+    recon = recon_out if recon_out is not None else (torch.empty(B, d, dtype=torch.float32, device=dev) if want_recon else None)
+    loss_tok = loss_out if loss_out is not None else torch.empty(B, dtype=torch.float32, device=dev)
     grad_recon = torch.empty(B, d, dtype=torch.float32, device=dev)
-    dval = torch.empty(code.n_slots, dtype=torch.float32, device=dev)
+    dval = dval_acc if dval_acc is not None else torch.empty(code.n_slots, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    fn = lib.sae_sparse_decode_mse_fused_acc if dval_acc is not None else lib.sae_sparse_decode_mse_fused
     with _timed("sparse_decode_mse_fused"):
         check(
-            _lib.load().sae_sparse_decode_mse_fused(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
-                                                    code.row_nnz.data_ptr(), w_dec.data_ptr(), _dt(w_dec), _ptr(b_dec),
-                                                    label.data_ptr(), _ptr(tok_w), _ptr(recon), loss_tok.data_ptr(),
-                                                    grad_recon.data_ptr(), dval.data_ptr(), B, d, F, code.n_slots,
-                                                    _stream(w_dec)),
+            fn(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(), code.row_nnz.data_ptr(), w_dec.data_ptr(),
+               _dt(w_dec), _ptr(b_dec), label.data_ptr(), _ptr(tok_w), _ptr(recon), loss_tok.data_ptr(), grad_recon.data_ptr(),
+               dval.data_ptr(), B, d, F, code.n_slots, _stream(w_dec)),
             "sparse_decode_mse_fused",
         )
     return recon, loss_tok, grad_recon, dval

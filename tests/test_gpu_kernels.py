@@ -683,3 +683,29 @@ def test_encoder_gemm_bias_epilogue(pkg, dev, B, d, F):
     assert torch.equal(pkg.ops.encoder_gemm_bias(x, w, row_bias=rb), (plain + rb[:, None]).to(torch.bfloat16))
     assert torch.equal(pkg.ops.encoder_gemm_bias(x, w, cb, rb), ((plain + cb) + rb[:, None]).to(torch.bfloat16))
     assert torch.equal(pkg.ops.encoder_gemm_bias(x, w), plain.to(torch.bfloat16))
+
+
+def test_sparse_decode_fused_accumulates_value_gradients_and_writes_in_place(pkg, dev):
+    """sae_sparse_decode_mse_fused_acc: two decoders over prefixes of one code add their value gradients into one
+    array (bit for bit the sum of the two separate results, taken in call order) and write their reconstructions and
+    per-token losses into slices handed in."""
+    g = torch.Generator().manual_seed(77)
+    B, d, F, k = 50, 128, 600, 12
+    idx = torch.stack([torch.randperm(F, generator=g)[:k].sort().values for _ in range(B)]).to(torch.int32)
+    val = torch.rand(B, k, generator=g)
+    code = pkg.ops.SparseCode(idx.reshape(-1).to(dev), val.reshape(-1).to(dev), (torch.arange(B) * k).to(dev),
+                              torch.full((B,), k, dtype=torch.int32).to(dev), B, F)
+    import dataclasses
+    nnz_a = torch.randint(0, k + 1, (B,), generator=g).to(torch.int32).to(dev)
+    codes = [dataclasses.replace(code, row_nnz=nnz_a), code]
+    ws = [torch.randn(F, d, generator=g).to(dev) for _ in range(2)]
+    labels = [torch.randn(B, d, generator=g).to(dev) for _ in range(2)]
+    tok_w = torch.full((B,), 1.0 / B, device=dev)
+    sep = [pkg.ops.sparse_decode_mse_fused(c, w, None, y, tok_w) for c, w, y in zip(codes, ws, labels)]
+    recon = torch.empty(2, B, d, device=dev); loss = torch.empty(2, B, device=dev)
+    acc = torch.zeros(B * k, device=dev)
+    for j, (c, w, y) in enumerate(zip(codes, ws, labels)):
+        r, lt, gr, dv = pkg.ops.sparse_decode_mse_fused(c, w, None, y, tok_w, recon_out=recon[j], loss_out=loss[j], dval_acc=acc)
+        assert r.data_ptr() == recon[j].data_ptr() and dv.data_ptr() == acc.data_ptr()
+        assert torch.equal(gr, sep[j][2]) and torch.equal(recon[j], sep[j][0]) and torch.equal(loss[j], sep[j][1])
+    assert torch.equal(acc, sep[0][3] + sep[1][3])
