@@ -319,16 +319,23 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     }
   }
 
-  // ---- XCD-aware tile assignment: 32 consecutive workgroups of an XCD cover 2^rm_log2 token tiles x the rest in feature tiles
+  // ---- XCD-aware tile assignment.  One tile dimension is dealt round-robin to the 8 XCDs (the feature tiles, or, when
+  // there are fewer than 8 of those, the token tiles: rm_log2 < 0 says so and -rm_log2 - 1 takes its place); 32 consecutive
+  // workgroups of an XCD cover 2^rm_log2 tiles of the other dimension x the rest in tiles of the dealt one.
   int tile_m, tile_n;
   {
     const int bid = blockIdx.x, xcd = bid & 7, slot = bid >> 3;
     const int grp = slot >> 5, in = slot & 31;
-    const int rm = 1 << rm_log2, rn = 32 >> rm_log2;
-    const int m_groups = (tiles_m + rm - 1) >> rm_log2;
-    const int n_grp = grp / m_groups, m_part = grp % m_groups;
-    tile_m = m_part * rm + (in & (rm - 1));
-    tile_n = (n_grp * rn + (in >> rm_log2)) * 8 + xcd;
+    const bool deal_m = rm_log2 < 0;
+    const int ro_log2 = deal_m ? -rm_log2 - 1 : rm_log2;
+    const int tiles_o = deal_m ? tiles_n : tiles_m;        // the dimension kept whole inside an XCD
+    const int ro = 1 << ro_log2, rs = 32 >> ro_log2;
+    const int o_groups = (tiles_o + ro - 1) >> ro_log2;
+    const int s_grp = grp / o_groups, o_part = grp % o_groups;
+    const int tile_o = o_part * ro + (in & (ro - 1));
+    const int tile_s = (s_grp * rs + (in >> ro_log2)) * 8 + xcd;
+    tile_m = deal_m ? tile_s : tile_o;
+    tile_n = deal_m ? tile_o : tile_s;
     if (tile_n >= tiles_n || tile_m >= tiles_m) return;     // the whole workgroup leaves: no barrier is left short
   }
   const int m0 = tile_m * GEMM_BM, n0 = tile_n * GEMM_BN;
@@ -607,8 +614,12 @@ static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, 
   auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
   if (rc != SAE_OK) return rc;
-  const int rm_log2 = tiles_m >= 8 ? 3 : 2, rm = 1 << rm_log2, rn = 32 >> rm_log2;
-  const int m_pad = (tiles_m + rm - 1) / rm * rm, n_local_pad = ((tiles_n + 7) / 8 + rn - 1) / rn * rn;
+  // with fewer than 8 feature tiles most XCDs would sit idle if those were what is dealt to them: deal the token tiles
+  const bool deal_m = tiles_n < 8 && tiles_m > tiles_n;
+  const int tiles_o = deal_m ? tiles_n : tiles_m, tiles_s = deal_m ? tiles_m : tiles_n;
+  const int ro_log2 = tiles_o >= 8 ? 3 : (tiles_o > 2 ? 2 : (tiles_o > 1 ? 1 : 0)), ro = 1 << ro_log2, rs = 32 >> ro_log2;
+  const int rm_log2 = deal_m ? -ro_log2 - 1 : ro_log2;
+  const int m_pad = (tiles_o + ro - 1) / ro * ro, n_local_pad = ((tiles_s + 7) / 8 + rs - 1) / rs * rs;
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)n_groups), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st,
                      (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale,
                      gmax, theta);
