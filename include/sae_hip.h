@@ -489,22 +489,18 @@ int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float
  * contraction index is contiguous for the products that read it.
  *   q, k      natural    [T, n_heads * d_qk]
  *   vt        transposed [n_heads * d_v, T]
- *   q_bias / k_bias [n_heads * d_qk], v_bias [n_heads * d_v]  fp32, nullable, 16-byte aligned: added to the bf16 operand
- *             as it is loaded and rounded back to bf16 (the projections' `+ b_Q`, `+ b_K`, `+ b_V`, models/lorsa.py:793-813)
  *   out       natural    [T, n_heads * d_v] bf16;  lse fp32 [n_batch, n_heads, seq] = log sum_{s'} exp(scale * q . k)
  * Requires d_qk in {32, 64}, d_v in {32, 64, 128}, seq % 8 == 0. */
-int sae_attention_fwd(const void *q, const void *k, const void *vt, const float *q_bias, const float *k_bias,
-                      const float *v_bias, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v,
-                      double scale, void *out, float *lse, void *stream);
+int sae_attention_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk,
+                      int64_t d_v, double scale, void *out, float *lse, void *stream);
 
-/* Backward of sae_attention_fwd.  q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout (biases
- * are added to q / qt, k / kt and v on load as in the forward pass); lse from the forward pass; dvec_workspace: device
- * float[n_batch * n_heads * seq].  Outputs, bf16, transposed: dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T] (the
- * gradients of the biased operands; a bias gradient is the row sum, sae_row_sum).  No atomics: reproducible. */
+/* Backward of sae_attention_fwd.  q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout; lse from
+ * the forward pass; workspace: device float[2 * n_batch * n_heads * seq] (D = rowsum(dout * out), and the log-sum-exp in
+ * the log2 domain).  Outputs, bf16, transposed: dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T] (a projection bias's
+ * gradient is the row sum, sae_row_sum).  No atomics: reproducible. */
 int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                      const void *dout, const void *doutt, const float *q_bias, const float *k_bias, const float *v_bias,
-                      const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v, double scale,
-                      float *dvec_workspace, void *dqt, void *dkt, void *dvt, void *stream);
+                      const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads,
+                      int64_t d_qk, int64_t d_v, double scale, float *workspace, void *dqt, void *dkt, void *dvt, void *stream);
 
 /* out[r] = sum_c src[r, c] (fp32 sum, fixed order) for src [rows, cols] fp32 or bf16.  The bias gradients autograd forms by
  * summing over tokens, for gradients held transposed ([features, tokens]). */

@@ -1,5 +1,5 @@
 // Causal softmax attention with grouped value heads for gfx950 (bf16 operands, fp32 accumulation), forward and
-// backward, on the matrix cores (v_mfma_f32_16x16x32_bf16).
+// backward, on the matrix cores (v_mfma_f32_32x32x16_bf16).
 //
 // The mixing step of low-rank sparse attention: every query/key head h has d_qk-wide queries and keys and a
 // d_v-wide value whose columns are d_v separate rank-1 value heads (dictionary features h * d_v .. (h + 1) * d_v - 1)
@@ -14,150 +14,106 @@
 // products need; the transposed copies come for free from the projection GEMM with its operands swapped, or
 // from the cast-transpose kernel.
 //
-// Fragment convention of the instruction (D = A B, 16 x 16 x 32): lane l supplies A[m = l % 16][8 consecutive k of
-// group l / 16] and B[same k][n = l % 16], and receives D[m = 4 (l / 16) + i][n = l % 16], i < 4.  The contraction
-// slots of a lane group only have to mean the same index in A and B: a probability tile leaves the score product
-// as D (4 consecutive positions per lane), is packed to bf16 in registers and used as the B operand of the next
-// product with slots {4g + i} of one 16-position tile and {4g + i} of the next; the A operand is read from LDS
-// with the same two 8-byte pieces.  No probability ever goes through LDS or HBM.
+// Fragment convention of the instruction (D = A B, 32 x 32 x 16): lane l supplies A[m = l % 32][8 consecutive k of
+// half l / 32] and B[same k][n = l % 32], and receives D[m = 8 j + 4 (l / 32) + i][n = l % 32] in register 4 j + i
+// (i, j < 4).  A workgroup is 4 waves; a wave owns 32 positions (queries in the forward and dQ kernels, keys in the
+// dV and dK kernels) as the n index of every product, so that everything kept per position (running maximum and sum,
+// log-sum-exp, the accumulators' rescaling) is per lane.  A 32 x 32 tile of probabilities leaves the score product as
+// D (lane halves hold alternate groups of 4 positions of the contraction index of the next product); packed to bf16,
+// two v_permlane32_swap per 16 positions hand each half the 8 consecutive positions the B operand wants.  No
+// probability ever goes through LDS or HBM.
 //
-// Forward: one workgroup = 64 queries of one (batch, head); wave w owns queries 16 w .. 16 w + 15 and walks the
-// key blocks 0 .. diagonal with the online softmax (running maximum and sum per query in fp32, log2 domain).
-// Backward: D[q] = sum_dv dout * out (one small kernel); dV and dK each by a workgroup per 64 keys that walks the
-// query blocks diagonal .. last; dQ by a workgroup per 64 queries that walks the key blocks 0 .. diagonal.  All three
-// recompute the probabilities from q, k and the saved log-sum-exp.  No atomics: results are reproducible.
+// Tiles of the streamed operand (64 positions per iteration) go from global memory straight into LDS
+// (global_load_lds_dwordx4, two buffers: the loads of tile i + 1 are in flight while tile i is consumed; one
+// workgroup barrier per tile).  Such a load writes 1 KiB linearly (lane l -> base + 16 l), so the bank swizzle is
+// applied on the global side: a tile row of RB bytes holds its 16-byte chunk c at physical chunk
+// c ^ ((row * RB / 256) % (RB / 16)), which makes the 16 rows x one chunk of a fragment read cover 256 distinct bytes.
+//
+// Forward: one workgroup = 128 queries of one (batch, head), walking the key blocks 0 .. diagonal with the online
+// softmax (running maximum and sum per query in fp32, log2 domain; the accumulators are rescaled only when some
+// row's maximum has grown by more than 2^8, so probabilities are formed relative to a reference at most that far
+// below the true maximum: exact in real arithmetic, and bf16 keeps its relative precision at any magnitude).
+// Backward: D[q] = sum_dv dout * out (one small kernel, which also leaves the log-sum-exp in the log2 domain); dV and
+// dK each by a workgroup per 128 keys that walks the query blocks diagonal .. last; dQ by a workgroup per 128 queries
+// that walks the key blocks 0 .. diagonal.  All three recompute the probabilities from q, k and the saved
+// log-sum-exp.  No atomics: results are reproducible.
+//
+// Positions past the end of a sequence (seq not a multiple of the block sizes): loads repeat the last valid row or
+// 8-position piece, so every operand stays finite; their scores are masked (keys), zeroed (queries of the dV / dK
+// kernels) or never stored.
 #include "common.h"
 
 namespace sae {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 att_bf16x8;
-typedef __attribute__((ext_vector_type(4))) float att_f32x4;
+typedef __attribute__((ext_vector_type(16))) float att_f32x16;
 
-constexpr int ATT_BLOCK = 64;       // positions per workgroup and per inner iteration
 constexpr int ATT_THREADS = 256;
-constexpr int ATT_TPITCH = 144;     // bytes per LDS row of a transposed tile: 64 positions * 2 + 16 (bank spread)
+constexpr int ATT_OWN = 128;        // positions owned by a workgroup: 4 waves of 32
+constexpr int ATT_STEP = 64;        // positions of the streamed operand per iteration
 constexpr float ATT_LOG2E = 1.4426950408889634f;
+constexpr float ATT_RESCALE_STEP = 8.f;
 
-__device__ __forceinline__ constexpr int att_nat_pitch(int cols) { return cols * 2 + 16; }
+#define ATT_WAITCNT_VM(N) (((N) & 0xf) | (0x7 << 4) | (0xf << 8) | (((N) >> 4) << 14))
+#if defined(__HIP_DEVICE_COMPILE__)
+// LDS[LDSADDR + 16 lane] = 16 bytes at SBASE + VOFF (scalar base, per-lane byte offset); LDSADDR is wave-uniform
+#define ATT_DMA16(SBASE, VOFF, LDSADDR)                                                                        \
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(LDSADDR)), \
+               "v"(VOFF), "s"(SBASE)                                                                           \
+               : "memory")
+#define ATT_DMA4(SBASE, VOFF, LDSADDR)                                                                         \
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(LDSADDR)),   \
+               "v"(VOFF), "s"(SBASE)                                                                           \
+               : "memory")
+#else
+#define ATT_DMA16(SBASE, VOFF, LDSADDR) ((void)0)
+#define ATT_DMA4(SBASE, VOFF, LDSADDR) ((void)0)
+#endif
 
 __device__ __forceinline__ uint32_t att_pack2(float a, float b) {
   const cvt_f32x2 in = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, cvt_bf16x2));
 }
 
-__device__ __forceinline__ att_bf16x8 att_pack8(const att_f32x4 &lo, const att_f32x4 &hi) {
-  u32x4 r;
-  r.x = att_pack2(lo[0], lo[1]); r.y = att_pack2(lo[2], lo[3]);
-  r.z = att_pack2(hi[0], hi[1]); r.w = att_pack2(hi[2], hi[3]);
-  return __builtin_bit_cast(att_bf16x8, r);
+// byte offset of logical chunk `chunk` of row `row` in a tile whose rows are RB bytes
+template <int RB>
+__device__ __forceinline__ int att_swz(int row, int chunk) {
+  constexpr int CPR = RB / 16, RP = 256 / RB;
+  return row * RB + ((chunk ^ ((row / RP) & (CPR - 1))) << 4);
 }
 
-// 8 bf16 + 8 fp32 biases -> 8 bf16 (each sum rounded to nearest even: what `bf16_tensor + fp32_bias` cast back gives)
-__device__ __forceinline__ u32x4 att_add_bias8(const u32x4 &v, const float *__restrict__ bias) {
-  const float4 b0 = *reinterpret_cast<const float4 *>(bias), b1 = *reinterpret_cast<const float4 *>(bias + 4);
-  u32x4 r;
-  r.x = att_pack2(__uint_as_float(v.x << 16) + b0.x, __uint_as_float(v.x & 0xffff0000u) + b0.y);
-  r.y = att_pack2(__uint_as_float(v.y << 16) + b0.z, __uint_as_float(v.y & 0xffff0000u) + b0.w);
-  r.z = att_pack2(__uint_as_float(v.z << 16) + b1.x, __uint_as_float(v.z & 0xffff0000u) + b1.y);
-  r.w = att_pack2(__uint_as_float(v.w << 16) + b1.z, __uint_as_float(v.w & 0xffff0000u) + b1.w);
-  return r;
+// A operand: row `row` of a tile, contraction positions 16 st + 8 g .. + 7
+template <int RB>
+__device__ __forceinline__ att_bf16x8 att_frag(const char *tile, int row, int st, int g) {
+  return *reinterpret_cast<const att_bf16x8 *>(tile + att_swz<RB>(row, 2 * st + g));
 }
 
-__device__ __forceinline__ u32x4 att_add_bias1(const u32x4 &v, float b) {
-  u32x4 r;
-  r.x = att_pack2(__uint_as_float(v.x << 16) + b, __uint_as_float(v.x & 0xffff0000u) + b);
-  r.y = att_pack2(__uint_as_float(v.y << 16) + b, __uint_as_float(v.y & 0xffff0000u) + b);
-  r.z = att_pack2(__uint_as_float(v.z << 16) + b, __uint_as_float(v.z & 0xffff0000u) + b);
-  r.w = att_pack2(__uint_as_float(v.w << 16) + b, __uint_as_float(v.w & 0xffff0000u) + b);
-  return r;
-}
-
-// Tiles travel global -> registers -> LDS in two halves, so that the loads of the next tile are in flight while the
-// current one is consumed: att_load_* issues the 16-byte loads of a thread's pieces, att_store_* (an iteration later)
-// adds the bias, if any, and writes them to LDS.
-//
-// Natural layout: 64 consecutive tokens x COLS columns -> LDS rows of att_nat_pitch(COLS) bytes.  Rows at or past
-// `rows_valid` are zero.  `bias` (nullable) is indexed by absolute column.
-template <int COLS>
-__device__ __forceinline__ void att_load_nat(u32x4 (&regs)[COLS / 32], const uint16_t *__restrict__ g, int64_t ld, int64_t tok0,
-                                             int rows_valid, int col0) {
-  constexpr int CH = COLS / 8;
+// Per-lane byte offsets of a wave's NL loads of a tile (wave-load wl = wave * NL + i covers 1 KiB of it).
+// Natural tile: rows are consecutive tokens of a matrix with `ld` elements per token, RB bytes of each are taken;
+// rows at or past `rows_valid` repeat row rows_valid - 1.
+template <int RB, int NL>
+__device__ __forceinline__ void att_nat_offsets(uint32_t (&off)[NL], int wave, int lane, int ld, int rows_valid) {
+  constexpr int CPR = RB / 16, RPL = 1024 / RB, RP = 256 / RB;
 #pragma unroll
-  for (int j = 0; j < COLS / 32; ++j) {
-    const int c = threadIdx.x + j * ATT_THREADS;
-    const int r = c / CH, cc = c % CH;
-    regs[j] = u32x4{0u, 0u, 0u, 0u};
-    if (r < rows_valid) regs[j] = *reinterpret_cast<const u32x4 *>(g + (tok0 + r) * ld + col0 + cc * 8);
+  for (int i = 0; i < NL; ++i) {
+    const int row = (wave * NL + i) * RPL + lane / CPR, ch = (lane % CPR) ^ ((row / RP) & (CPR - 1));
+    off[i] = (uint32_t)(min(row, rows_valid - 1) * ld + ch * 8) * 2u;
   }
 }
-
-template <int COLS>
-__device__ __forceinline__ void att_store_nat(char *lds, const u32x4 (&regs)[COLS / 32], int rows_valid, int col0,
-                                              const float *__restrict__ bias) {
-  constexpr int CH = COLS / 8, PITCH = att_nat_pitch(COLS);
+// Transposed tile: row r is feature row r of a matrix with T tokens per row, 64 consecutive tokens (128 bytes) of each
+// are taken; 8-token pieces at or past `cols_valid` (a multiple of 8) repeat the last valid piece.
+template <int NL>
+__device__ __forceinline__ void att_tr_offsets(uint32_t (&off)[NL], int wave, int lane, int64_t T, int cols_valid) {
 #pragma unroll
-  for (int j = 0; j < COLS / 32; ++j) {
-    const int c = threadIdx.x + j * ATT_THREADS;
-    const int r = c / CH, cc = c % CH;
-    u32x4 v = regs[j];
-    if (bias && r < rows_valid) v = att_add_bias8(v, bias + col0 + cc * 8);
-    *reinterpret_cast<u32x4 *>(lds + r * PITCH + cc * 16) = v;
+  for (int i = 0; i < NL; ++i) {
+    const int row = (wave * NL + i) * 8 + (lane >> 3), ch = (lane & 7) ^ ((row >> 1) & 7);
+    off[i] = (uint32_t)((int64_t)row * T + min(ch * 8, cols_valid - 8)) * 2u;
   }
 }
-
-// Transposed layout: ROWS rows x 64 consecutive tokens -> LDS rows of ATT_TPITCH bytes.  Columns at or past
-// `cols_valid` (a multiple of 8) are zero.  `bias` (nullable) is indexed by absolute row.
-template <int ROWS>
-__device__ __forceinline__ void att_load_tr(u32x4 (&regs)[ROWS / 32], const uint16_t *__restrict__ gt, int64_t ld, int row0,
-                                            int64_t tok0, int cols_valid) {
+template <int NL>
+__device__ __forceinline__ void att_dma(const void *sbase, const uint32_t (&off)[NL], uint32_t lds_addr) {
 #pragma unroll
-  for (int j = 0; j < ROWS / 32; ++j) {
-    const int c = threadIdx.x + j * ATT_THREADS;
-    const int r = c >> 3, cc = c & 7;
-    regs[j] = u32x4{0u, 0u, 0u, 0u};
-    if (cc * 8 < cols_valid) regs[j] = *reinterpret_cast<const u32x4 *>(gt + (int64_t)(row0 + r) * ld + tok0 + cc * 8);
-  }
-}
-
-template <int ROWS>
-__device__ __forceinline__ void att_store_tr(char *lds, const u32x4 (&regs)[ROWS / 32], int row0, int cols_valid,
-                                             const float *__restrict__ bias) {
-#pragma unroll
-  for (int j = 0; j < ROWS / 32; ++j) {
-    const int c = threadIdx.x + j * ATT_THREADS;
-    const int r = c >> 3, cc = c & 7;
-    u32x4 v = regs[j];
-    if (bias && cc * 8 < cols_valid) v = att_add_bias1(v, bias[row0 + r]);
-    *reinterpret_cast<u32x4 *>(lds + r * ATT_TPITCH + cc * 16) = v;
-  }
-}
-
-// One token's row of a natural-layout matrix as the register fragments of a lane (8 columns of group g per 32-column step).
-template <int COLS>
-__device__ __forceinline__ void att_row_frags(att_bf16x8 (&f)[COLS / 32], const uint16_t *__restrict__ g, int64_t ld,
-                                              int64_t tok, bool valid, int col0, int grp, const float *__restrict__ bias) {
-#pragma unroll
-  for (int kk = 0; kk < COLS / 32; ++kk) {
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (valid) {
-      v = *reinterpret_cast<const u32x4 *>(g + tok * ld + col0 + kk * 32 + grp * 8);
-      if (bias) v = att_add_bias8(v, bias + col0 + kk * 32 + grp * 8);
-    }
-    f[kk] = __builtin_bit_cast(att_bf16x8, v);
-  }
-}
-
-__device__ __forceinline__ att_bf16x8 att_nat_frag(const char *lds, int pitch, int row, int kk, int grp) {
-  return *reinterpret_cast<const att_bf16x8 *>(lds + row * pitch + (kk * 32 + grp * 8) * 2);
-}
-
-// positions {32 u + 4 g + i} and {32 u + 16 + 4 g + i}, i < 4, of one row of a transposed tile
-__device__ __forceinline__ att_bf16x8 att_tr_frag(const char *lds, int row, int u, int grp) {
-  const uint2 lo = *reinterpret_cast<const uint2 *>(lds + row * ATT_TPITCH + (32 * u + 4 * grp) * 2);
-  const uint2 hi = *reinterpret_cast<const uint2 *>(lds + row * ATT_TPITCH + (32 * u + 16 + 4 * grp) * 2);
-  u32x4 r;
-  r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
-  return __builtin_bit_cast(att_bf16x8, r);
+  for (int i = 0; i < NL; ++i) ATT_DMA16(sbase, off[i], lds_addr + i * 1024);
 }
 
 // Workgroup id -> (position block, head, sequence).  The hardware deals consecutive workgroup ids round-robin to the 8
@@ -180,119 +136,199 @@ __device__ __forceinline__ void att_block_coords(int n_blocks, int n_heads, int 
   b = bh / n_heads;
 }
 
-__device__ __forceinline__ att_f32x4 att_mfma(const att_bf16x8 &a, const att_bf16x8 &b, const att_f32x4 &c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+__device__ __forceinline__ att_f32x16 att_mfma(const att_bf16x8 &a, const att_bf16x8 &b, const att_f32x16 &c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ att_f32x16 att_zero16() {
+  att_f32x16 z;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = 0.f;
+  return z;
 }
 
 __device__ __forceinline__ float att_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// both halves of the wave get max / sum of lane l and lane l ^ 32
+__device__ __forceinline__ float att_half_max(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float att_half_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// A lane's 16 values of a 32 x 32 tile (positions 8 j + 4 g + i of the tile's m index) -> the B operands of the two
+// 16-position steps of a product that contracts over m: half g of step c gets positions 16 c + 8 g .. + 7.  The swap
+// exchanges the upper half of its first operand with the lower half of its second.
+__device__ __forceinline__ void att_to_b_operands(const uint32_t (&pk)[8], att_bf16x8 (&b)[2]) {
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const auto w0 = __builtin_amdgcn_permlane32_swap(pk[4 * c], pk[4 * c + 2], false, false);
+    const auto w1 = __builtin_amdgcn_permlane32_swap(pk[4 * c + 1], pk[4 * c + 3], false, false);
+    u32x4 w;
+    w.x = w0[0]; w.y = w1[0]; w.z = w0[1]; w.w = w1[1];
+    b[c] = __builtin_bit_cast(att_bf16x8, w);
+  }
+}
+__device__ __forceinline__ void att_pack16(const att_f32x16 &x, uint32_t (&pk)[8]) {
+#pragma unroll
+  for (int r = 0; r < 8; ++r) pk[r] = att_pack2(x[2 * r], x[2 * r + 1]);
+}
+
+// One token's row of a natural-layout matrix as the B operands of a lane (8 columns of half g per 16-column step).
+template <int COLS>
+__device__ __forceinline__ void att_row_operands(att_bf16x8 (&f)[COLS / 16], const uint16_t *__restrict__ row, int g) {
+#pragma unroll
+  for (int st = 0; st < COLS / 16; ++st) f[st] = *reinterpret_cast<const att_bf16x8 *>(row + st * 16 + g * 8);
+}
+
+// A wave's 32 x ROWS accumulator tile set (acc[n] = rows 32 n .. 32 n + 31, this lane's token) -> transposed layout
+// dst[(row0 + row) * T + tok]
+template <int ROWS>
+__device__ __forceinline__ void att_store_transposed(uint16_t *__restrict__ dst, const att_f32x16 (&acc)[ROWS / 32], int row0, int64_t T,
+                                                     int64_t tok, int g) {
+#pragma unroll
+  for (int n = 0; n < ROWS / 32; ++n)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      dst[(int64_t)(row0 + n * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * T + tok] = (uint16_t)(att_pack2(acc[n][r], 0.f) & 0xffffu);
+}
+
 // ---- forward ---------------------------------------------------------------------------------------------
 template <int DQK, int DV>
-__global__ __launch_bounds__(ATT_THREADS) void attn_fwd_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ vt,
-    const float *__restrict__ bq, const float *__restrict__ bk, const float *__restrict__ bv, uint16_t *__restrict__ out,
+__global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ vt, uint16_t *__restrict__ out,
     float *__restrict__ lse, int seq, int n_heads, int n_batch, int64_t T, float sc2) {
-  constexpr int KP = att_nat_pitch(DQK);
-  __shared__ __attribute__((aligned(16))) char s_k[ATT_BLOCK * KP];
-  __shared__ __attribute__((aligned(16))) char s_vt[DV * ATT_TPITCH];
+  constexpr int KRB = DQK * 2;                                    // bytes of a key row
+  constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = DV * 128, BUF = K_BYTES + V_BYTES;
+  constexpr int KNL = K_BYTES / 4096, VNL = V_BYTES / 4096;      // loads per wave and tile
+  constexpr int OP = DV * 2 + 16;                                 // staging row pitch of the epilogue
+  constexpr int LDS_BYTES = 2 * BUF > 4 * 32 * OP ? 2 * BUF : 4 * 32 * OP;
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   int qb, h, b;
-  att_block_coords((seq + ATT_BLOCK - 1) / ATT_BLOCK, n_heads, n_batch, true, qb, h, b);     // long rows of work first
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, grp = lane >> 4;
+  att_block_coords((seq + ATT_OWN - 1) / ATT_OWN, n_heads, n_batch, true, qb, h, b);     // long rows of work first
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r32 = lane & 31, g = lane >> 5;
   const int64_t tok0 = (int64_t)b * seq;
-  const int64_t ldq = (int64_t)n_heads * DQK, ldv = (int64_t)n_heads * DV;
-  const int q_row = qb * ATT_BLOCK + wave * 16 + lr;
+  const int ldq = n_heads * DQK, ldv = n_heads * DV;
+  const int wq0 = qb * ATT_OWN + wave * 32, q_row = wq0 + r32;
 
-  att_bf16x8 qf[DQK / 32];
-  att_row_frags<DQK>(qf, q, ldq, tok0 + q_row, q_row < seq, h * DQK, grp, bq);
-  att_f32x4 o[DV / 16];
+  att_bf16x8 qf[DQK / 16];
+  att_row_operands<DQK>(qf, q + (tok0 + min(q_row, seq - 1)) * ldq + h * DQK, g);
+  att_f32x16 o[DV / 32];
 #pragma unroll
-  for (int n = 0; n < DV / 16; ++n) o[n] = att_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < DV / 32; ++n) o[n] = att_zero16();
   float m = -INFINITY, l = 0.f;
 
-  u32x4 rk[DQK / 32], rvt[DV / 32];
-  att_load_nat<DQK>(rk, k, ldq, tok0, min(ATT_BLOCK, seq), h * DQK);
-  att_load_tr<DV>(rvt, vt, T, h * DV, tok0, min(ATT_BLOCK, seq));
-  for (int kb = 0; kb <= qb; ++kb) {
-    const int valid = min(ATT_BLOCK, seq - kb * ATT_BLOCK);
-    __syncthreads();                       // every wave is done with the previous tile
-    att_store_nat<DQK>(s_k, rk, valid, h * DQK, bk);
-    att_store_tr<DV>(s_vt, rvt, h * DV, valid, bv);
-    __syncthreads();
-    if (kb < qb) {                         // the next tile's loads fly while this one is consumed
-      const int nvalid = min(ATT_BLOCK, seq - (kb + 1) * ATT_BLOCK);
-      att_load_nat<DQK>(rk, k, ldq, tok0 + (kb + 1) * ATT_BLOCK, nvalid, h * DQK);
-      att_load_tr<DV>(rvt, vt, T, h * DV, tok0 + (kb + 1) * ATT_BLOCK, nvalid);
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  const int n_kb = (min(seq, (qb + 1) * ATT_OWN) + ATT_STEP - 1) / ATT_STEP;
+  uint32_t koff[KNL], voff[VNL];
+  att_nat_offsets<KRB, KNL>(koff, wave, lane, ldq, ATT_STEP);
+  att_tr_offsets<VNL>(voff, wave, lane, T, ATT_STEP);
+  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *vbase = vt + (int64_t)h * DV * T + tok0;
+  auto issue = [&](int kb) {
+    const uint32_t buf = lds_base + (uint32_t)(kb & 1) * BUF;
+    const uint16_t *kt_ = kbase + (int64_t)kb * ATT_STEP * ldq, *vt_ = vbase + kb * ATT_STEP;
+    const int rem = seq - kb * ATT_STEP;
+    if (rem >= ATT_STEP) {
+      att_dma<KNL>(kt_, koff, buf + wave * KNL * 1024);
+      att_dma<VNL>(vt_, voff, buf + K_BYTES + wave * VNL * 1024);
+    } else {
+      uint32_t ko[KNL], vo[VNL];
+      att_nat_offsets<KRB, KNL>(ko, wave, lane, ldq, rem);
+      att_tr_offsets<VNL>(vo, wave, lane, T, rem);
+      att_dma<KNL>(kt_, ko, buf + wave * KNL * 1024);
+      att_dma<VNL>(vt_, vo, buf + K_BYTES + wave * VNL * 1024);
     }
-    att_f32x4 s[4];
+  };
+  issue(0);
+  for (int kb = 0; kb < n_kb; ++kb) {
+    __builtin_amdgcn_s_waitcnt(ATT_WAITCNT_VM(0));
+    __syncthreads();                       // tile kb is in LDS; every wave is done with the other buffer
+    if (kb + 1 < n_kb) issue(kb + 1);
+    const int key0 = kb * ATT_STEP;
+    if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
+    const char *sk = lds + (kb & 1) * BUF, *sv = sk + K_BYTES;
+    att_f32x16 s[2];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      s[t] = att_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < 2; ++t) {
+      s[t] = att_zero16();
 #pragma unroll
-      for (int kk = 0; kk < DQK / 32; ++kk) s[t] = att_mfma(att_nat_frag(s_k, KP, t * 16 + lr, kk, grp), qf[kk], s[t]);
+      for (int st = 0; st < DQK / 16; ++st) s[t] = att_mfma(att_frag<KRB>(sk, t * 32 + r32, st, g), qf[st], s[t]);
     }
-    if (kb == qb) {                       // only the diagonal block has keys after the query
+    if (key0 + ATT_STEP - 1 > wq0) {       // some key of the block lies after some query of the wave
+      const int thr = q_row - key0 - 4 * g;      // the lane's element at key offset 32 t + 8 j + i above this is masked
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (kb * ATT_BLOCK + t * 16 + 4 * grp + i > q_row) s[t][i] = -INFINITY;
+        for (int r = 0; r < 16; ++r) s[t][r] = (t * 32 + 8 * (r >> 2) + (r & 3) > thr) ? -INFINITY : s[t][r];
     }
     float mx = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[t][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    // every row meets at least one unmasked key in every block it visits, so m_new is finite; the scale is positive,
-    // so the maximum is taken over the raw scores and scaled once
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
+    mx = att_half_max(mx);
+    // key0 <= wq0 here (both are multiples of 32), so every row sees at least one key of the block and m_new is finite;
+    // the scale is positive, so the maximum is taken over the raw scores and scaled once
     const float m_new = fmaxf(m, mx * sc2);
-    if (__any(m_new > m)) {               // a running maximum that did not move leaves the sums as they are
+    if (__any(m_new > m + ATT_RESCALE_STEP)) {
       const float alpha = att_exp2(m - m_new);      // exp2(-inf) = 0 on the first block
       l *= alpha;
 #pragma unroll
-      for (int n = 0; n < DV / 16; ++n)
+      for (int n = 0; n < DV / 32; ++n)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[n][i] *= alpha;
+        for (int r = 0; r < 16; ++r) o[n][r] *= alpha;
       m = m_new;
     }
     float rs = 0.f;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 2; ++t) {
+      uint32_t pk[8];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = att_exp2(fmaf(s[t][i], sc2, -m));
-        s[t][i] = p;
-        rs += p;
+      for (int r = 0; r < 8; ++r) {
+        const float p0 = att_exp2(fmaf(s[t][2 * r], sc2, -m)), p1 = att_exp2(fmaf(s[t][2 * r + 1], sc2, -m));
+        rs += p0 + p1;
+        pk[r] = att_pack2(p0, p1);
       }
+      att_bf16x8 pb[2];
+      att_to_b_operands(pk, pb);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int n = 0; n < DV / 32; ++n) o[n] = att_mfma(att_frag<128>(sv, n * 32 + r32, 2 * t + c, g), pb[c], o[n]);
+    }
     l += rs;
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const att_bf16x8 pf = att_pack8(s[2 * u], s[2 * u + 1]);
-#pragma unroll
-      for (int n = 0; n < DV / 16; ++n) o[n] = att_mfma(att_tr_frag(s_vt, n * 16 + lr, u, grp), pf, o[n]);
-    }
   }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (q_row < seq) {
-    const float inv = 1.f / l;
-    uint16_t *orow = out + (tok0 + q_row) * ldv + h * DV + 4 * grp;
+  l = att_half_sum(l);
+  __syncthreads();                         // the tile buffers become the staging area of the epilogue
+  const float inv = 1.f / l;
+  char *so = lds + wave * 32 * OP;
 #pragma unroll
-    for (int n = 0; n < DV / 16; ++n) {
-      uint2 pk;
-      pk.x = att_pack2(o[n][0] * inv, o[n][1] * inv);
-      pk.y = att_pack2(o[n][2] * inv, o[n][3] * inv);
-      *reinterpret_cast<uint2 *>(orow + n * 16) = pk;
+  for (int n = 0; n < DV / 32; ++n)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint2 pkv;
+      pkv.x = att_pack2(o[n][4 * j] * inv, o[n][4 * j + 1] * inv);
+      pkv.y = att_pack2(o[n][4 * j + 2] * inv, o[n][4 * j + 3] * inv);
+      *reinterpret_cast<uint2 *>(so + r32 * OP + (n * 32 + 8 * j + 4 * g) * 2) = pkv;
     }
-    if (grp == 0) lse[((int64_t)b * n_heads + h) * seq + q_row] = (m + __log2f(l)) * 0.6931471805599453f;
+  constexpr int CH = DV / 8, ROWS_PER_PASS = 64 / CH;   // whole rows of the output leave as 16-byte pieces
+#pragma unroll
+  for (int ps = 0; ps < 32 / ROWS_PER_PASS; ++ps) {
+    const int row = ps * ROWS_PER_PASS + lane / CH, cc = lane % CH;
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(so + row * OP + cc * 16);
+    if (wq0 + row < seq) *reinterpret_cast<u32x4 *>(out + (tok0 + wq0 + row) * ldv + h * DV + cc * 8) = v;
   }
+  if (q_row < seq && g == 0) lse[((int64_t)b * n_heads + h) * seq + q_row] = (m + __log2f(l)) * 0.6931471805599453f;
 }
 
-// ---- backward: D[b, h, s] = sum_dv dout[t, h, dv] * out[t, h, dv] ---------------------------------------------
+// ---- backward: D[b, h, s] = sum_dv dout[t, h, dv] * out[t, h, dv], and the log-sum-exp in the log2 domain ------------
 template <int DV>
 __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const uint16_t *__restrict__ dout, const uint16_t *__restrict__ out,
-                                                            float *__restrict__ dvec, int seq, int n_heads, int64_t T) {
+                                                            const float *__restrict__ lse, float *__restrict__ dvec,
+                                                            float *__restrict__ lse2, int seq, int n_heads, int64_t T) {
   // 16 lanes per (token, head); a lane covers 8 columns per trip
   const int64_t pair = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
   const int sub = threadIdx.x & 15;
@@ -317,259 +353,232 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const uint16_t *__re
   if (pair < n_pairs && sub == 0) {
     const int64_t t = pair / n_heads;
     const int h = (int)(pair % n_heads);
-    dvec[((t / seq) * n_heads + h) * seq + (t % seq)] = acc;
+    const int64_t at = ((t / seq) * n_heads + h) * seq + (t % seq);
+    dvec[at] = acc;
+    lse2[at] = lse[at] * ATT_LOG2E;
   }
 }
 
-// ---- backward: dV^T (one workgroup per 64 keys) ------------------------------------------------------------------
-// dV^T[dv, key] = sum_q dout^T[dv, q] P[q, key].  (dK lives in a kernel of its own: fused, the two accumulators, the
-// four operand tiles and their fragments leave one wave per SIMD, and the kernel waits on its own barriers.)
-template <int DQK, int DV>
-__global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dv_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ doutt,
-    const float *__restrict__ bq, const float *__restrict__ bk, const float *__restrict__ lse, uint16_t *__restrict__ dvt,
-    int seq, int n_heads, int n_batch, int64_t T, float sc2) {
-  constexpr int QP = att_nat_pitch(DQK);
-  __shared__ __attribute__((aligned(16))) char s_q[ATT_BLOCK * QP];
-  __shared__ __attribute__((aligned(16))) char s_dot[DV * ATT_TPITCH];
-  __shared__ float s_lse[ATT_BLOCK];
-  const int nqb = (seq + ATT_BLOCK - 1) / ATT_BLOCK;
+// ---- backward: dV^T and dK^T (one workgroup per 128 keys, a wave per 32) -----------------------------------------------
+// P[q, key] = exp2(sc2 * q . k - lse2[q]) for q >= key.
+// WHAT = 0: dV^T[dv, key] = sum_q dout^T[dv, q] P[q, key].
+// WHAT = 1: dK^T[c, key] = sum_q q^T[c, q] dS[q, key],  dS = P (dP - D) scale,  dP[q, key] = dout[q, :] . v[key, :].
+// (One kernel for both would hold both accumulators, both register-resident rows and four streamed tiles: one wave per
+// SIMD, which waits on its own barriers.)
+template <int DQK, int DV, int WHAT>
+__global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_kernel(
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ qt, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+    const uint16_t *__restrict__ dout, const uint16_t *__restrict__ doutt, const float *__restrict__ lse2,
+    const float *__restrict__ dvec, uint16_t *__restrict__ dst, int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
+  constexpr bool DK = WHAT == 1;
+  constexpr int QRB = DQK * 2, ORB = DV * 2;
+  constexpr int Q_BYTES = ATT_STEP * QRB;                              // q natural (both)
+  constexpr int A_BYTES = DK ? DQK * 128 : DV * 128;                   // q^T (dK) or dout^T (dV): the accumulating product's A tile
+  constexpr int O_BYTES = DK ? ATT_STEP * ORB : 0;                     // dout natural (dK)
+  constexpr int VEC_BYTES = 512;                                       // 64 x (lse2, D)
+  constexpr int BUF = Q_BYTES + A_BYTES + O_BYTES + VEC_BYTES;
+  constexpr int QNL = Q_BYTES / 4096, ANL = A_BYTES / 4096, ONL = DK ? O_BYTES / 4096 : 1;
+  constexpr int ACC = DK ? DQK : DV;                                   // rows of the accumulated matrix
+  __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
+  const int n_qb = (seq + ATT_STEP - 1) / ATT_STEP;
   int kb, h, b;
-  att_block_coords(nqb, n_heads, n_batch, false, kb, h, b);     // key block 0 walks every query block: first
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, grp = lane >> 4;
+  att_block_coords((seq + ATT_OWN - 1) / ATT_OWN, n_heads, n_batch, false, kb, h, b);     // key block 0 walks every query block: first
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r32 = lane & 31, g = lane >> 5;
   const int64_t tok0 = (int64_t)b * seq;
-  const int64_t ldq = (int64_t)n_heads * DQK;
-  const int key_col = kb * ATT_BLOCK + wave * 16 + lr;
+  const int ldq = n_heads * DQK, ldv = n_heads * DV;
+  const int wk0 = kb * ATT_OWN + wave * 32, key = wk0 + r32;
 
-  att_bf16x8 kf[DQK / 32];
-  att_row_frags<DQK>(kf, k, ldq, tok0 + key_col, key_col < seq, h * DQK, grp, bk);
-  att_f32x4 dv[DV / 16];
+  att_bf16x8 kf[DQK / 16], vf[DK ? DV / 16 : 1];
+  att_row_operands<DQK>(kf, k + (tok0 + min(key, seq - 1)) * ldq + h * DQK, g);
+  if constexpr (DK) att_row_operands<DV>(vf, v + (tok0 + min(key, seq - 1)) * ldv + h * DV, g);
+  att_f32x16 acc[ACC / 32];
 #pragma unroll
-  for (int n = 0; n < DV / 16; ++n) dv[n] = att_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < ACC / 32; ++n) acc[n] = att_zero16();
 
-  u32x4 rq[DQK / 32], rdot[DV / 32];
-  float r_lse = INFINITY;                  // threads 0..63: one query's log-sum-exp in the log2 domain
-  auto load_tiles = [&](int qb) {
-    const int valid = min(ATT_BLOCK, seq - qb * ATT_BLOCK);
-    att_load_nat<DQK>(rq, q, ldq, tok0 + qb * ATT_BLOCK, valid, h * DQK);
-    att_load_tr<DV>(rdot, doutt, T, h * DV, tok0 + qb * ATT_BLOCK, valid);
-    if (threadIdx.x < ATT_BLOCK) {
-      const int qq = qb * ATT_BLOCK + threadIdx.x;
-      r_lse = qq < seq ? lse[((int64_t)b * n_heads + h) * seq + qq] * ATT_LOG2E : INFINITY;   // +inf: p = 0 past the sequence
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  uint32_t qoff[QNL], aoff[ANL], ooff[ONL];
+  att_nat_offsets<QRB, QNL>(qoff, wave, lane, ldq, ATT_STEP);
+  att_tr_offsets<ANL>(aoff, wave, lane, T, ATT_STEP);
+  if constexpr (DK) att_nat_offsets<ORB, ONL>(ooff, wave, lane, ldv, ATT_STEP);
+  const uint16_t *qbase = q + tok0 * ldq + h * DQK;
+  const uint16_t *abase = (DK ? qt + (int64_t)h * DQK * T : doutt + (int64_t)h * DV * T) + tok0;
+  const uint16_t *obase = dout + tok0 * ldv + h * DV;
+  const float *lbase = lse2 + ((int64_t)b * n_heads + h) * seq, *dbase = dvec + ((int64_t)b * n_heads + h) * seq;
+  auto issue = [&](int qb, int slot) {
+    const uint32_t buf = lds_base + (uint32_t)slot * BUF;
+    const int q0 = qb * ATT_STEP, rem = seq - q0;
+    const uint16_t *q_ = qbase + (int64_t)q0 * ldq, *a_ = abase + q0, *o_ = obase + (int64_t)q0 * ldv;
+    if (rem >= ATT_STEP) {
+      att_dma<QNL>(q_, qoff, buf + wave * QNL * 1024);
+      att_dma<ANL>(a_, aoff, buf + Q_BYTES + wave * ANL * 1024);
+      if constexpr (DK) att_dma<ONL>(o_, ooff, buf + Q_BYTES + A_BYTES + wave * ONL * 1024);
+    } else {
+      uint32_t qo[QNL], ao[ANL], oo[ONL];
+      att_nat_offsets<QRB, QNL>(qo, wave, lane, ldq, rem);
+      att_tr_offsets<ANL>(ao, wave, lane, T, rem);
+      att_dma<QNL>(q_, qo, buf + wave * QNL * 1024);
+      att_dma<ANL>(a_, ao, buf + Q_BYTES + wave * ANL * 1024);
+      if constexpr (DK) {
+        att_nat_offsets<ORB, ONL>(oo, wave, lane, ldv, rem);
+        att_dma<ONL>(o_, oo, buf + Q_BYTES + A_BYTES + wave * ONL * 1024);
+      }
     }
+    // the 64 queries' log-sum-exp (wave 0) and D (wave 1, dK only): 4 bytes per lane
+    const uint32_t voff = (uint32_t)min(lane, rem - 1) * 4u;
+    if (wave == 0) ATT_DMA4(lbase + q0, voff, buf + Q_BYTES + A_BYTES + O_BYTES);
+    if (DK && wave == 1) ATT_DMA4(dbase + q0, voff, buf + Q_BYTES + A_BYTES + O_BYTES + 256);
   };
-  load_tiles(kb);
-  for (int qb = kb; qb < nqb; ++qb) {
-    const int valid = min(ATT_BLOCK, seq - qb * ATT_BLOCK);
-    __syncthreads();
-    att_store_nat<DQK>(s_q, rq, valid, h * DQK, bq);
-    att_store_tr<DV>(s_dot, rdot, h * DV, valid, nullptr);
-    if (threadIdx.x < ATT_BLOCK) s_lse[threadIdx.x] = r_lse;
-    __syncthreads();
-    if (qb + 1 < nqb) load_tiles(qb + 1);
-    att_f32x4 p[4];
+  const int qb0 = kb * (ATT_OWN / ATT_STEP);
+  if (qb0 < n_qb) issue(qb0, 0);
+  for (int qb = qb0; qb < n_qb; ++qb) {
+    const int slot = (qb - qb0) & 1;
+    __builtin_amdgcn_s_waitcnt(ATT_WAITCNT_VM(0));
+    __syncthreads();                       // tile qb is in LDS; every wave is done with the other buffer
+    if (qb + 1 < n_qb) issue(qb + 1, slot ^ 1);
+    const int q0 = qb * ATT_STEP;
+    if (q0 + ATT_STEP - 1 < wk0) continue; // every query of this block lies before every key of this wave
+    const char *sq = lds + slot * BUF, *sa = sq + Q_BYTES, *so = sa + A_BYTES;
+    const float *svec = reinterpret_cast<const float *>(so + O_BYTES);
+    const bool diag = q0 < wk0 + 31;       // some query of the block lies before some key of the wave
+    const bool tail = q0 + ATT_STEP > seq; // some query of the block lies past the sequence
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      att_f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < 2; ++t) {
+      att_f32x16 s = att_zero16();
 #pragma unroll
-      for (int kk = 0; kk < DQK / 32; ++kk) s = att_mfma(att_nat_frag(s_q, QP, t * 16 + lr, kk, grp), kf[kk], s);
-      const att_f32x4 l4 = *reinterpret_cast<const att_f32x4 *>(s_lse + t * 16 + 4 * grp);
+      for (int st = 0; st < DQK / 16; ++st) s = att_mfma(att_frag<QRB>(sq, t * 32 + r32, st, g), kf[st], s);
+      att_f32x16 x;                        // P (dV) or dS (dK) of this lane's key and 16 of the tile's queries
+      if constexpr (DK) {
+        att_f32x16 dp = att_zero16();
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p[t][i] = att_exp2(fmaf(s[i], sc2, -l4[i]));
-    }
-    if (qb == kb) {                        // the diagonal block: queries before the key do not see it
+        for (int st = 0; st < DV / 16; ++st) dp = att_mfma(att_frag<ORB>(so, t * 32 + r32, st, g), vf[st], dp);
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int j = 0; j < 4; ++j) {
+          const float4 l4 = *reinterpret_cast<const float4 *>(svec + t * 32 + 8 * j + 4 * g);
+          const float4 d4 = *reinterpret_cast<const float4 *>(svec + 64 + t * 32 + 8 * j + 4 * g);
+          const float lj[4] = {l4.x, l4.y, l4.z, l4.w}, dj[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (key_col > qb * ATT_BLOCK + t * 16 + 4 * grp + i) p[t][i] = 0.f;
-    }
+          for (int i = 0; i < 4; ++i) x[4 * j + i] = att_exp2(fmaf(s[4 * j + i], sc2, -lj[i])) * ((dp[4 * j + i] - dj[i]) * scale);
+        }
+      } else {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const att_bf16x8 pf = att_pack8(p[2 * u], p[2 * u + 1]);
+        for (int j = 0; j < 4; ++j) {
+          const float4 l4 = *reinterpret_cast<const float4 *>(svec + t * 32 + 8 * j + 4 * g);
+          const float lj[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
-      for (int n = 0; n < DV / 16; ++n) dv[n] = att_mfma(att_tr_frag(s_dot, n * 16 + lr, u, grp), pf, dv[n]);
+          for (int i = 0; i < 4; ++i) x[4 * j + i] = att_exp2(fmaf(s[4 * j + i], sc2, -lj[i]));
+        }
+      }
+      if (diag || tail) {
+        // query offset 32 t + 8 j + 4 g + i: before the key -> 0; at or past the end of the sequence -> 0
+        const int lo = key - q0 - 4 * g, hi = seq - q0 - 4 * g;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qo = t * 32 + 8 * (r >> 2) + (r & 3);
+          x[r] = (qo < lo || qo >= hi) ? 0.f : x[r];
+        }
+      }
+      uint32_t pk[8];
+      att_pack16(x, pk);
+      att_bf16x8 xb[2];
+      att_to_b_operands(pk, xb);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int n = 0; n < ACC / 32; ++n) acc[n] = att_mfma(att_frag<128>(sa, n * 32 + r32, 2 * t + c, g), xb[c], acc[n]);
     }
   }
-  if (key_col < seq) {
-#pragma unroll
-    for (int n = 0; n < DV / 16; ++n)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        dvt[(int64_t)(h * DV + n * 16 + 4 * grp + i) * T + tok0 + key_col] = (uint16_t)(att_pack2(dv[n][i], 0.f) & 0xffffu);
-  }
+  if (key < seq) att_store_transposed<ACC>(dst, acc, h * ACC, T, tok0 + key, g);
 }
 
-// ---- backward: dK^T (one workgroup per 64 keys) ------------------------------------------------------------------
-// dK^T[dqk, key] = sum_q q^T[dqk, q] dS[q, key],  dS = P (dP - D) scale,  dP[q, key] = dout[q, :] . v[key, :].
+// ---- backward: dQ^T (one workgroup per 128 queries, a wave per 32) -------------------------------------------------------
+// dQ^T[c, q] = sum_key k^T[c, key] dS[q, key] over key <= q.
 template <int DQK, int DV>
-__global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dk_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ qt, const uint16_t *__restrict__ k,
-    const uint16_t *__restrict__ v, const uint16_t *__restrict__ dout, const float *__restrict__ bq,
-    const float *__restrict__ bk, const float *__restrict__ bv, const float *__restrict__ lse,
-    const float *__restrict__ dvec, uint16_t *__restrict__ dkt, int seq, int n_heads, int n_batch, int64_t T, float sc2,
-    float scale) {
-  constexpr int QP = att_nat_pitch(DQK), OP = att_nat_pitch(DV);
-  __shared__ __attribute__((aligned(16))) char s_q[ATT_BLOCK * QP];
-  __shared__ __attribute__((aligned(16))) char s_qt[DQK * ATT_TPITCH];
-  __shared__ __attribute__((aligned(16))) char s_do[ATT_BLOCK * OP];
-  __shared__ float s_lse[ATT_BLOCK], s_d[ATT_BLOCK];
-  const int nqb = (seq + ATT_BLOCK - 1) / ATT_BLOCK;
-  int kb, h, b;
-  att_block_coords(nqb, n_heads, n_batch, false, kb, h, b);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, grp = lane >> 4;
-  const int64_t tok0 = (int64_t)b * seq;
-  const int64_t ldq = (int64_t)n_heads * DQK, ldv = (int64_t)n_heads * DV;
-  const int key_col = kb * ATT_BLOCK + wave * 16 + lr;
-
-  att_bf16x8 kf[DQK / 32], vf[DV / 32];
-  att_row_frags<DQK>(kf, k, ldq, tok0 + key_col, key_col < seq, h * DQK, grp, bk);
-  att_row_frags<DV>(vf, v, ldv, tok0 + key_col, key_col < seq, h * DV, grp, bv);
-  att_f32x4 dk[DQK / 16];
-#pragma unroll
-  for (int n = 0; n < DQK / 16; ++n) dk[n] = att_f32x4{0.f, 0.f, 0.f, 0.f};
-
-  u32x4 rq[DQK / 32], rqt[DQK / 32], rdo[DV / 32];
-  float r_lse = INFINITY, r_d = 0.f;       // threads 0..63: one query's log-sum-exp (log2 domain) and D
-  auto load_tiles = [&](int qb) {
-    const int valid = min(ATT_BLOCK, seq - qb * ATT_BLOCK);
-    att_load_nat<DQK>(rq, q, ldq, tok0 + qb * ATT_BLOCK, valid, h * DQK);
-    att_load_tr<DQK>(rqt, qt, T, h * DQK, tok0 + qb * ATT_BLOCK, valid);
-    att_load_nat<DV>(rdo, dout, ldv, tok0 + qb * ATT_BLOCK, valid, h * DV);
-    if (threadIdx.x < ATT_BLOCK) {
-      const int qq = qb * ATT_BLOCK + threadIdx.x;
-      const int64_t at = ((int64_t)b * n_heads + h) * seq + qq;
-      r_lse = qq < seq ? lse[at] * ATT_LOG2E : INFINITY;   // +inf: a row past the sequence gets p = 0
-      r_d = qq < seq ? dvec[at] : 0.f;
-    }
-  };
-  load_tiles(kb);
-  for (int qb = kb; qb < nqb; ++qb) {
-    const int valid = min(ATT_BLOCK, seq - qb * ATT_BLOCK);
-    __syncthreads();
-    att_store_nat<DQK>(s_q, rq, valid, h * DQK, bq);
-    att_store_tr<DQK>(s_qt, rqt, h * DQK, valid, bq);
-    att_store_nat<DV>(s_do, rdo, valid, h * DV, nullptr);
-    if (threadIdx.x < ATT_BLOCK) {
-      s_lse[threadIdx.x] = r_lse;
-      s_d[threadIdx.x] = r_d;
-    }
-    __syncthreads();
-    if (qb + 1 < nqb) load_tiles(qb + 1);
-    att_f32x4 ds[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      att_f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < DQK / 32; ++kk) s = att_mfma(att_nat_frag(s_q, QP, t * 16 + lr, kk, grp), kf[kk], s);
-#pragma unroll
-      for (int kk = 0; kk < DV / 32; ++kk) dp = att_mfma(att_nat_frag(s_do, OP, t * 16 + lr, kk, grp), vf[kk], dp);
-      const att_f32x4 l4 = *reinterpret_cast<const att_f32x4 *>(s_lse + t * 16 + 4 * grp);
-      const att_f32x4 d4 = *reinterpret_cast<const att_f32x4 *>(s_d + t * 16 + 4 * grp);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ds[t][i] = att_exp2(fmaf(s[i], sc2, -l4[i])) * ((dp[i] - d4[i]) * scale);
-    }
-    if (qb == kb) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (key_col > qb * ATT_BLOCK + t * 16 + 4 * grp + i) ds[t][i] = 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const att_bf16x8 dsf = att_pack8(ds[2 * u], ds[2 * u + 1]);
-#pragma unroll
-      for (int n = 0; n < DQK / 16; ++n) dk[n] = att_mfma(att_tr_frag(s_qt, n * 16 + lr, u, grp), dsf, dk[n]);
-    }
-  }
-  if (key_col < seq) {
-#pragma unroll
-    for (int n = 0; n < DQK / 16; ++n)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        dkt[(int64_t)(h * DQK + n * 16 + 4 * grp + i) * T + tok0 + key_col] = (uint16_t)(att_pack2(dk[n][i], 0.f) & 0xffffu);
-  }
-}
-
-// ---- backward: dQ^T (one workgroup per 64 queries) -------------------------------------------------------------
-template <int DQK, int DV>
-__global__ __launch_bounds__(ATT_THREADS) void attn_bwd_dq_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ kt,
-    const uint16_t *__restrict__ v, const uint16_t *__restrict__ dout, const float *__restrict__ bq,
-    const float *__restrict__ bk, const float *__restrict__ bv, const float *__restrict__ lse,
-    const float *__restrict__ dvec, uint16_t *__restrict__ dqt, int seq, int n_heads, int n_batch, int64_t T, float sc2,
-    float scale) {
-  constexpr int KP = att_nat_pitch(DQK), VP = att_nat_pitch(DV);
-  __shared__ __attribute__((aligned(16))) char s_k[ATT_BLOCK * KP];
-  __shared__ __attribute__((aligned(16))) char s_kt[DQK * ATT_TPITCH];
-  __shared__ __attribute__((aligned(16))) char s_v[ATT_BLOCK * VP];
+__global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ kt, const uint16_t *__restrict__ v,
+    const uint16_t *__restrict__ dout, const float *__restrict__ lse2, const float *__restrict__ dvec, uint16_t *__restrict__ dqt,
+    int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
+  constexpr int KRB = DQK * 2, VRB = DV * 2;
+  constexpr int K_BYTES = ATT_STEP * KRB, KT_BYTES = DQK * 128, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + KT_BYTES + V_BYTES;
+  constexpr int KNL = K_BYTES / 4096, KTNL = KT_BYTES / 4096, VNL = V_BYTES / 4096;
+  __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
   int qb, h, b;
-  att_block_coords((seq + ATT_BLOCK - 1) / ATT_BLOCK, n_heads, n_batch, true, qb, h, b);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, grp = lane >> 4;
+  att_block_coords((seq + ATT_OWN - 1) / ATT_OWN, n_heads, n_batch, true, qb, h, b);
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r32 = lane & 31, g = lane >> 5;
   const int64_t tok0 = (int64_t)b * seq;
-  const int64_t ldq = (int64_t)n_heads * DQK, ldv = (int64_t)n_heads * DV;
-  const int q_row = qb * ATT_BLOCK + wave * 16 + lr;
-  const bool q_ok = q_row < seq;
+  const int ldq = n_heads * DQK, ldv = n_heads * DV;
+  const int wq0 = qb * ATT_OWN + wave * 32, q_row = wq0 + r32, q_ld = min(q_row, seq - 1);
 
-  att_bf16x8 qf[DQK / 32], dof[DV / 32];
-  att_row_frags<DQK>(qf, q, ldq, tok0 + q_row, q_ok, h * DQK, grp, bq);
-  att_row_frags<DV>(dof, dout, ldv, tok0 + q_row, q_ok, h * DV, grp, nullptr);
-  const int64_t at = ((int64_t)b * n_heads + h) * seq + q_row;
-  const float lse2 = q_ok ? lse[at] * ATT_LOG2E : INFINITY;
-  const float dq_sum = q_ok ? dvec[at] : 0.f;
-  att_f32x4 dq[DQK / 16];
+  att_bf16x8 qf[DQK / 16], dof[DV / 16];
+  att_row_operands<DQK>(qf, q + (tok0 + q_ld) * ldq + h * DQK, g);
+  att_row_operands<DV>(dof, dout + (tok0 + q_ld) * ldv + h * DV, g);
+  const int64_t at = ((int64_t)b * n_heads + h) * seq + q_ld;
+  const float l2 = lse2[at], dsum = dvec[at];
+  att_f32x16 dq[DQK / 32];
 #pragma unroll
-  for (int n = 0; n < DQK / 16; ++n) dq[n] = att_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < DQK / 32; ++n) dq[n] = att_zero16();
 
-  u32x4 rk[DQK / 32], rkt[DQK / 32], rv[DV / 32];
-  auto load_tiles = [&](int kb) {
-    const int valid = min(ATT_BLOCK, seq - kb * ATT_BLOCK);
-    att_load_nat<DQK>(rk, k, ldq, tok0 + kb * ATT_BLOCK, valid, h * DQK);
-    att_load_tr<DQK>(rkt, kt, T, h * DQK, tok0 + kb * ATT_BLOCK, valid);
-    att_load_nat<DV>(rv, v, ldv, tok0 + kb * ATT_BLOCK, valid, h * DV);
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  const int n_kb = (min(seq, (qb + 1) * ATT_OWN) + ATT_STEP - 1) / ATT_STEP;
+  uint32_t koff[KNL], ktoff[KTNL], voff[VNL];
+  att_nat_offsets<KRB, KNL>(koff, wave, lane, ldq, ATT_STEP);
+  att_tr_offsets<KTNL>(ktoff, wave, lane, T, ATT_STEP);
+  att_nat_offsets<VRB, VNL>(voff, wave, lane, ldv, ATT_STEP);
+  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *ktbase = kt + (int64_t)h * DQK * T + tok0, *vbase = v + tok0 * ldv + h * DV;
+  auto issue = [&](int kb) {
+    const uint32_t buf = lds_base + (uint32_t)(kb & 1) * BUF;
+    const int key0 = kb * ATT_STEP, rem = seq - key0;
+    const uint16_t *k_ = kbase + (int64_t)key0 * ldq, *kt_ = ktbase + key0, *v_ = vbase + (int64_t)key0 * ldv;
+    if (rem >= ATT_STEP) {
+      att_dma<KNL>(k_, koff, buf + wave * KNL * 1024);
+      att_dma<KTNL>(kt_, ktoff, buf + K_BYTES + wave * KTNL * 1024);
+      att_dma<VNL>(v_, voff, buf + K_BYTES + KT_BYTES + wave * VNL * 1024);
+    } else {
+      uint32_t ko[KNL], kto[KTNL], vo[VNL];
+      att_nat_offsets<KRB, KNL>(ko, wave, lane, ldq, rem);
+      att_tr_offsets<KTNL>(kto, wave, lane, T, rem);
+      att_nat_offsets<VRB, VNL>(vo, wave, lane, ldv, rem);
+      att_dma<KNL>(k_, ko, buf + wave * KNL * 1024);
+      att_dma<KTNL>(kt_, kto, buf + K_BYTES + wave * KTNL * 1024);
+      att_dma<VNL>(v_, vo, buf + K_BYTES + KT_BYTES + wave * VNL * 1024);
+    }
   };
-  load_tiles(0);
-  for (int kb = 0; kb <= qb; ++kb) {
-    const int valid = min(ATT_BLOCK, seq - kb * ATT_BLOCK);
+  issue(0);
+  for (int kb = 0; kb < n_kb; ++kb) {
+    __builtin_amdgcn_s_waitcnt(ATT_WAITCNT_VM(0));
     __syncthreads();
-    att_store_nat<DQK>(s_k, rk, valid, h * DQK, bk);
-    att_store_tr<DQK>(s_kt, rkt, h * DQK, valid, bk);
-    att_store_nat<DV>(s_v, rv, valid, h * DV, bv);
-    __syncthreads();
-    if (kb < qb) load_tiles(kb + 1);
-    att_f32x4 ds[4];
+    if (kb + 1 < n_kb) issue(kb + 1);
+    const int key0 = kb * ATT_STEP;
+    if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
+    const char *sk = lds + (kb & 1) * BUF, *skt = sk + K_BYTES, *sv = skt + KT_BYTES;
+    const bool diag = key0 + ATT_STEP - 1 > wq0;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      att_f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < 2; ++t) {
+      att_f32x16 s = att_zero16(), dp = att_zero16();
 #pragma unroll
-      for (int kk = 0; kk < DQK / 32; ++kk) s = att_mfma(att_nat_frag(s_k, KP, t * 16 + lr, kk, grp), qf[kk], s);
+      for (int st = 0; st < DQK / 16; ++st) s = att_mfma(att_frag<KRB>(sk, t * 32 + r32, st, g), qf[st], s);
 #pragma unroll
-      for (int kk = 0; kk < DV / 32; ++kk) dp = att_mfma(att_nat_frag(s_v, VP, t * 16 + lr, kk, grp), dof[kk], dp);
+      for (int st = 0; st < DV / 16; ++st) dp = att_mfma(att_frag<VRB>(sv, t * 32 + r32, st, g), dof[st], dp);
+      att_f32x16 ds;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ds[t][i] = att_exp2(fmaf(s[i], sc2, -lse2)) * ((dp[i] - dq_sum) * scale);
-    }
-    if (kb == qb) {                        // only the diagonal block has keys after the query
+      for (int r = 0; r < 16; ++r) ds[r] = att_exp2(fmaf(s[r], sc2, -l2)) * ((dp[r] - dsum) * scale);
+      if (diag) {
+        const int thr = q_row - key0 - 4 * g;
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int r = 0; r < 16; ++r) ds[r] = (t * 32 + 8 * (r >> 2) + (r & 3) > thr) ? 0.f : ds[r];
+      }
+      uint32_t pk[8];
+      att_pack16(ds, pk);
+      att_bf16x8 db[2];
+      att_to_b_operands(pk, db);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (kb * ATT_BLOCK + t * 16 + 4 * grp + i > q_row) ds[t][i] = 0.f;
-    }
+      for (int c = 0; c < 2; ++c)
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const att_bf16x8 dsf = att_pack8(ds[2 * u], ds[2 * u + 1]);
-#pragma unroll
-      for (int n = 0; n < DQK / 16; ++n) dq[n] = att_mfma(att_tr_frag(s_kt, n * 16 + lr, u, grp), dsf, dq[n]);
+        for (int n = 0; n < DQK / 32; ++n) dq[n] = att_mfma(att_frag<128>(skt, n * 32 + r32, 2 * t + c, g), db[c], dq[n]);
     }
   }
-  if (q_ok) {
-#pragma unroll
-    for (int n = 0; n < DQK / 16; ++n)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        dqt[(int64_t)(h * DQK + n * 16 + 4 * grp + i) * T + tok0 + q_row] = (uint16_t)(att_pack2(dq[n][i], 0.f) & 0xffffu);
-  }
+  if (q_row < seq) att_store_transposed<DQK>(dqt, dq, h * DQK, T, tok0 + q_row, g);
 }
 
 // out[r] = sum_c src[r, c] in fp32 for a bf16 or fp32 matrix [rows, cols]; one wave per row, fixed order; 16-byte
@@ -612,46 +621,49 @@ __global__ __launch_bounds__(256) void row_sum_kernel(const void *__restrict__ s
 }
 
 template <int DQK, int DV>
-static int launch_fwd(const void *q, const void *k, const void *vt, const float *bq, const float *bk, const float *bv,
-                      int64_t n_batch, int64_t seq, int64_t n_heads, double scale, void *out, float *lse, hipStream_t st) {
-  const dim3 grid((unsigned)(((seq + ATT_BLOCK - 1) / ATT_BLOCK) * n_heads * n_batch));
+static int launch_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads, double scale,
+                      void *out, float *lse, hipStream_t st) {
+  const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)vt, bq, bk, bv, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch, n_batch * seq,
+                     (const uint16_t *)vt, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch, n_batch * seq,
                      (float)(scale * 1.4426950408889634));
   return check_launch("attention_fwd");
 }
 
 template <int DQK, int DV>
 static int launch_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                      const void *dout, const void *doutt, const float *bq, const float *bk, const float *bv, const float *lse,
-                      int64_t n_batch, int64_t seq, int64_t n_heads, double scale, float *dvec, void *dqt, void *dkt, void *dvt,
-                      hipStream_t st) {
+                      const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads,
+                      double scale, float *workspace, void *dqt, void *dkt, void *dvt, hipStream_t st) {
   const int64_t T = n_batch * seq;
-  const dim3 grid((unsigned)(((seq + ATT_BLOCK - 1) / ATT_BLOCK) * n_heads * n_batch));
+  const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   const float sc2 = (float)(scale * 1.4426950408889634);
+  float *dvec = workspace, *lse2 = workspace + n_batch * n_heads * seq;
   const int64_t prep_blocks = (T * n_heads * 16 + 255) / 256;
   hipLaunchKernelGGL((attn_bwd_prep_kernel<DV>), dim3((unsigned)prep_blocks), dim3(256), 0, st, (const uint16_t *)dout,
-                     (const uint16_t *)out, dvec, (int)seq, (int)n_heads, T);
-  hipLaunchKernelGGL((attn_bwd_dv_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)doutt, bq, bk, lse, (uint16_t *)dvt, (int)seq, (int)n_heads, (int)n_batch, T, sc2);
-  hipLaunchKernelGGL((attn_bwd_dk_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)qt,
-                     (const uint16_t *)k, (const uint16_t *)v, (const uint16_t *)dout, bq, bk, bv, lse, dvec, (uint16_t *)dkt,
-                     (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
+                     (const uint16_t *)out, lse, dvec, lse2, (int)seq, (int)n_heads, T);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 0>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)qt,
+                     (const uint16_t *)k, (const uint16_t *)v, (const uint16_t *)dout, (const uint16_t *)doutt, lse2, dvec,
+                     (uint16_t *)dvt, (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 1>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)qt,
+                     (const uint16_t *)k, (const uint16_t *)v, (const uint16_t *)dout, (const uint16_t *)doutt, lse2, dvec,
+                     (uint16_t *)dkt, (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
   hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)kt, (const uint16_t *)v, (const uint16_t *)dout, bq, bk, bv, lse, dvec, (uint16_t *)dqt,
-                     (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
+                     (const uint16_t *)kt, (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dqt, (int)seq,
+                     (int)n_heads, (int)n_batch, T, sc2, (float)scale);
   return check_launch("attention_bwd");
 }
 
 static int check_shapes(const char *what, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v) {
   SAE_REQUIRE(n_batch > 0 && seq > 0 && n_heads > 0, SAE_ERR_INVALID_ARG, "%s: sizes must be positive", what);
-  SAE_REQUIRE(((seq + ATT_BLOCK - 1) / ATT_BLOCK) * n_heads * n_batch < ((int64_t)1 << 31), SAE_ERR_UNSUPPORTED,
+  SAE_REQUIRE(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch < ((int64_t)1 << 31), SAE_ERR_UNSUPPORTED,
               "%s: too many (block, head, sequence) workgroups", what);
   SAE_REQUIRE(seq % 8 == 0, SAE_ERR_UNSUPPORTED, "%s: seq = %lld must be a multiple of 8 (16-byte pieces of the transposed operands)",
               what, (long long)seq);
   SAE_REQUIRE((d_qk == 32 || d_qk == 64) && (d_v == 32 || d_v == 64 || d_v == 128), SAE_ERR_UNSUPPORTED,
               "%s: built for d_qk in {32, 64} and d_v in {32, 64, 128}, got %lld / %lld", what, (long long)d_qk, (long long)d_v);
-  SAE_REQUIRE(n_batch * seq * n_heads * (d_v > d_qk ? d_v : d_qk) < (int64_t)1 << 40, SAE_ERR_UNSUPPORTED, "%s: too large", what);
+  // a tile's per-lane offsets are 32-bit byte offsets from the tile's first element
+  SAE_REQUIRE(n_batch * seq * 128 * 2 < ((int64_t)1 << 32) && n_heads * 128 * 64 * 2 < ((int64_t)1 << 32), SAE_ERR_UNSUPPORTED,
+              "%s: more than 2^24 tokens or 2^18 heads", what);
   return SAE_OK;
 }
 
@@ -665,31 +677,28 @@ static int check_shapes(const char *what, int64_t n_batch, int64_t seq, int64_t 
   if (d_qk == 64 && d_v == 64) return CALL(64, 64);                             \
   return CALL(64, 128);
 
-extern "C" int sae_attention_fwd(const void *q, const void *k, const void *vt, const float *q_bias, const float *k_bias,
-                                 const float *v_bias, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v,
-                                 double scale, void *out, float *lse, void *stream) {
+extern "C" int sae_attention_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads,
+                                 int64_t d_qk, int64_t d_v, double scale, void *out, float *lse, void *stream) {
   using namespace sae;
   SAE_REQUIRE(q && k && vt && out && lse, SAE_ERR_INVALID_ARG, "attention_fwd: null pointer");
   const int rc = check_shapes("attention_fwd", n_batch, seq, n_heads, d_qk, d_v);
   if (rc != SAE_OK) return rc;
-#define ATT_FWD(A, B) launch_fwd<A, B>(q, k, vt, q_bias, k_bias, v_bias, n_batch, seq, n_heads, scale, out, lse, (hipStream_t)stream)
+#define ATT_FWD(A, B) launch_fwd<A, B>(q, k, vt, n_batch, seq, n_heads, scale, out, lse, (hipStream_t)stream)
   ATT_DISPATCH(ATT_FWD)
 #undef ATT_FWD
 }
 
 extern "C" int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                                 const void *dout, const void *doutt, const float *q_bias, const float *k_bias,
-                                 const float *v_bias, const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads,
-                                 int64_t d_qk, int64_t d_v, double scale, float *dvec_workspace, void *dqt, void *dkt, void *dvt,
-                                 void *stream) {
+                                 const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq,
+                                 int64_t n_heads, int64_t d_qk, int64_t d_v, double scale, float *workspace, void *dqt, void *dkt,
+                                 void *dvt, void *stream) {
   using namespace sae;
-  SAE_REQUIRE(q && qt && k && kt && v && out && dout && doutt && lse && dvec_workspace && dqt && dkt && dvt,
+  SAE_REQUIRE(q && qt && k && kt && v && out && dout && doutt && lse && workspace && dqt && dkt && dvt,
               SAE_ERR_INVALID_ARG, "attention_bwd: null pointer");
   const int rc = check_shapes("attention_bwd", n_batch, seq, n_heads, d_qk, d_v);
   if (rc != SAE_OK) return rc;
-#define ATT_BWD(A, B)                                                                                                        \
-  launch_bwd<A, B>(q, qt, k, kt, v, out, dout, doutt, q_bias, k_bias, v_bias, lse, n_batch, seq, n_heads, scale, dvec_workspace, \
-                   dqt, dkt, dvt, (hipStream_t)stream)
+#define ATT_BWD(A, B) \
+  launch_bwd<A, B>(q, qt, k, kt, v, out, dout, doutt, lse, n_batch, seq, n_heads, scale, workspace, dqt, dkt, dvt, (hipStream_t)stream)
   ATT_DISPATCH(ATT_BWD)
 #undef ATT_BWD
 }

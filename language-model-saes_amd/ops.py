@@ -1014,38 +1014,25 @@ def _att_check(name: str, t: torch.Tensor, shape: tuple) -> None:
         raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
-def _att_bias(name: str, t: Optional[torch.Tensor], n: int) -> Optional[torch.Tensor]:
-    if t is None:
-        return None
-    t = t.detach().reshape(-1)
-    _req(t, name, torch.float32, 1)
-    if t.numel() != n:
-        raise ValueError(f"{name} must have {n} elements")
-    return t
-
-
-def attention_fwd(q: torch.Tensor, k: torch.Tensor, vt: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
-                  q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
-                  v_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+def attention_fwd(q: torch.Tensor, k: torch.Tensor, vt: torch.Tensor, n_batch: int, seq: int, n_heads: int,
+                  scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
     """Causal softmax attention: q, k natural [T, n_heads * d_qk], vt transposed [n_heads * d_v, T] (bf16, T = n_batch * seq)
-    -> (out natural [T, n_heads * d_v] bf16, lse fp32 [n_batch, n_heads, seq]).  Biases (fp32) are added on load."""
+    -> (out natural [T, n_heads * d_v] bf16, lse fp32 [n_batch, n_heads, seq]).  Projection biases belong in the
+    products that form q, k and vt (`encoder_gemm_bias`)."""
     T = n_batch * seq
     d_qk, d_v = q.shape[1] // n_heads, vt.shape[0] // n_heads
     _att_check("q", q, (T, n_heads * d_qk)); _att_check("k", k, (T, n_heads * d_qk)); _att_check("vt", vt, (n_heads * d_v, T))
-    bq, bk, bv = _att_bias("q_bias", q_bias, n_heads * d_qk), _att_bias("k_bias", k_bias, n_heads * d_qk), _att_bias("v_bias", v_bias, n_heads * d_v)
     out = torch.empty(T, n_heads * d_v, dtype=torch.bfloat16, device=q.device)
     lse = torch.empty(n_batch, n_heads, seq, dtype=torch.float32, device=q.device)
     with _timed("attention_fwd"):
-        check(_lib.load().sae_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), _ptr(bq), _ptr(bk), _ptr(bv), n_batch, seq,
-                                            n_heads, d_qk, d_v, float(scale), out.data_ptr(), lse.data_ptr(), _stream(q)),
-              "attention_fwd")
+        check(_lib.load().sae_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), n_batch, seq, n_heads, d_qk, d_v,
+                                            float(scale), out.data_ptr(), lse.data_ptr(), _stream(q)), "attention_fwd")
     return out, lse
 
 
 def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
                   dout: torch.Tensor, doutt: torch.Tensor, lse: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
-                  q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
-                  v_bias: Optional[torch.Tensor] = None, return_stacked: bool = False):
+                  return_stacked: bool = False):
     """Backward of attention_fwd -> (dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T]) in bf16, transposed layout.
     q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout.  The three are row blocks of one
     buffer [n_heads * (2 d_qk + d_v), T], returned as a fourth value with `return_stacked`."""
@@ -1058,17 +1045,16 @@ def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.
     _req(lse, "lse", torch.float32, 3)
     if tuple(lse.shape) != (n_batch, n_heads, seq):
         raise ValueError("lse must be [n_batch, n_heads, seq]")
-    bq, bk, bv = _att_bias("q_bias", q_bias, n_heads * d_qk), _att_bias("k_bias", k_bias, n_heads * d_qk), _att_bias("v_bias", v_bias, n_heads * d_v)
     dev = q.device
     # one buffer, so that a caller can also treat the three gradients as one [2 h d_qk + h d_v, T] matrix
     grads = torch.empty(n_heads * (2 * d_qk + d_v), T, dtype=torch.bfloat16, device=dev)
     dqt, dkt, dvt = grads[: n_heads * d_qk], grads[n_heads * d_qk: 2 * n_heads * d_qk], grads[2 * n_heads * d_qk:]
-    dvec = torch.empty(n_batch * n_heads * seq, dtype=torch.float32, device=dev)
+    workspace = torch.empty(2 * n_batch * n_heads * seq, dtype=torch.float32, device=dev)
     with _timed("attention_bwd"):
         check(_lib.load().sae_attention_bwd(q.data_ptr(), qt.data_ptr(), k.data_ptr(), kt.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                            dout.data_ptr(), doutt.data_ptr(), _ptr(bq), _ptr(bk), _ptr(bv), lse.data_ptr(), n_batch,
-                                            seq, n_heads, d_qk, d_v, float(scale), dvec.data_ptr(), dqt.data_ptr(), dkt.data_ptr(),
-                                            dvt.data_ptr(), _stream(q)), "attention_bwd")
+                                            dout.data_ptr(), doutt.data_ptr(), lse.data_ptr(), n_batch, seq, n_heads, d_qk, d_v,
+                                            float(scale), workspace.data_ptr(), dqt.data_ptr(), dkt.data_ptr(), dvt.data_ptr(),
+                                            _stream(q)), "attention_bwd")
     return (dqt, dkt, dvt, grads) if return_stacked else (dqt, dkt, dvt)
 
 

@@ -44,55 +44,50 @@ def reference(q, k, v, nb, s, h, scale):
     return out.reshape(nb * s, h * dv), lse
 
 
-def make_case(nb, s, h, dq, dv, seed, with_bias):
+def make_case(nb, s, h, dq, dv, seed):
     g = torch.Generator().manual_seed(seed)
     T = nb * s
     q = bf16r(torch.randn(T, h * dq, generator=g))
     k = bf16r(torch.randn(T, h * dq, generator=g))
     v = bf16r(torch.randn(T, h * dv, generator=g))
     dout = bf16r(torch.randn(T, h * dv, generator=g))
-    if with_bias:
-        bq, bk, bv = (0.3 * torch.randn(h * dq, generator=g), 0.3 * torch.randn(h * dq, generator=g), 0.3 * torch.randn(h * dv, generator=g))
-    else:
-        bq = bk = bv = None
-    return q, k, v, dout, bq, bk, bv
+    return q, k, v, dout
 
 
 CASES = [
-    # nb, seq, heads, d_qk, d_v, bias
-    (2, 64, 2, 32, 32, False),
-    (1, 40, 3, 32, 64, True),          # ragged: one partial block
-    (2, 72, 2, 64, 64, False),         # ragged second block
-    (1, 200, 2, 64, 128, True),        # the benchmark's head widths, four blocks, ragged tail
-    (3, 128, 4, 64, 128, False),
-    (1, 8, 1, 64, 32, True),           # shortest sequence the kernels take
-    (2, 136, 4, 64, 128, True),        # 8 (sequence, head) pairs: the XCD-aware workgroup order, ragged tail
-    (4, 72, 4, 32, 64, False),         # 16 pairs
+    # nb, seq, heads, d_qk, d_v
+    (2, 64, 2, 32, 32),
+    (1, 40, 3, 32, 64),          # ragged: one partial block
+    (2, 72, 2, 64, 64),          # ragged second block
+    (1, 200, 2, 64, 128),        # the benchmark's head widths, four key blocks, ragged tail
+    (3, 128, 4, 64, 128),        # exactly one workgroup of queries per (sequence, head)
+    (1, 8, 1, 64, 32),           # shortest sequence the kernels take
+    (2, 136, 4, 64, 128),        # 8 (sequence, head) pairs: the XCD-aware workgroup order; a second workgroup of 8 queries
+    (4, 72, 4, 32, 64),          # 16 pairs
+    (1, 328, 2, 32, 128),        # three workgroups per head, ragged in both block sizes
+    (2, 256, 8, 64, 32),
 ]
 
 
-@pytest.mark.parametrize("nb,s,h,dq,dv,with_bias", CASES)
-def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv, with_bias):
-    print(f"attention case nb={nb} seq={s} heads={h} d_qk={dq} d_v={dv} bias={with_bias}", flush=True)
-    q, k, v, dout, bq, bk, bv = make_case(nb, s, h, dq, dv, seed=100 + s + dq + dv, with_bias=with_bias)
+@pytest.mark.parametrize("nb,s,h,dq,dv", CASES)
+def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv):
+    print(f"attention case nb={nb} seq={s} heads={h} d_qk={dq} d_v={dv}", flush=True)
+    q, k, v, dout = make_case(nb, s, h, dq, dv, seed=100 + s + dq + dv)
     scale = 1.0 / math.sqrt(dq)
-    # what the kernel sees after it has added the biases: bf16(bf16 operand + fp32 bias)
-    eff = lambda t, b: t if b is None else bf16r((t.float() + b).double())     # noqa: E731
-    ql, kl, vl = (eff(q, bq).requires_grad_(), eff(k, bk).requires_grad_(), eff(v, bv).requires_grad_())
+    ql, kl, vl = q.clone().requires_grad_(), k.clone().requires_grad_(), v.clone().requires_grad_()
     want_out, want_lse = reference(ql, kl, vl, nb, s, h, scale)
     (want_out * dout).sum().backward()
 
     to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
     gq, gk, gv, gdo = to_dev(q), to_dev(k), to_dev(v), to_dev(dout)
     gvt = gv.t().contiguous()
-    bias_dev = [None if b is None else b.to(dev) for b in (bq, bk, bv)]
-    out, lse = pkg.ops.attention_fwd(gq, gk, gvt, nb, s, h, scale, *bias_dev)
+    out, lse = pkg.ops.attention_fwd(gq, gk, gvt, nb, s, h, scale)
     assert out.dtype == torch.bfloat16 and tuple(out.shape) == (nb * s, h * dv)
     assert rel_max(out, want_out.detach()) < OUT_TOL, rel_max(out, want_out.detach())
     assert (lse.double().cpu() - want_lse.detach()).abs().max().item() < LSE_TOL * max(1.0, want_lse.abs().max().item())
 
     dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(), lse,
-                                          nb, s, h, scale, *bias_dev)
+                                          nb, s, h, scale)
     torch.cuda.synchronize()
     errs = {"dq": (rel_max(dqt.t(), ql.grad), rel_frob(dqt.t(), ql.grad)),
             "dk": (rel_max(dkt.t(), kl.grad), rel_frob(dkt.t(), kl.grad)),
@@ -103,7 +98,7 @@ def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv,
 def test_attention_is_causal_and_sequences_do_not_mix(pkg, dev):
     """Changing a later position, or another sequence of the batch, leaves every earlier output bit-identical."""
     nb, s, h, dq, dv = 2, 96, 2, 64, 128
-    q, k, v, _, _, _, _ = make_case(nb, s, h, dq, dv, seed=7, with_bias=False)
+    q, k, v, _ = make_case(nb, s, h, dq, dv, seed=7)
     to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
     gq, gk, gv = to_dev(q), to_dev(k), to_dev(v)
     out0, lse0 = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, 0.125)

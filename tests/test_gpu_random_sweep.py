@@ -122,26 +122,23 @@ def test_random_sweep_attention_and_code_conversions(pkg, oracle, dev, sweep_see
         seed = rng.randrange(1 << 30)
         g = torch.Generator().manual_seed(seed)
         if kind == "attention":
-            nb = rng.choice([1, 2, 3, 8]); s = 8 * rng.choice([1, 3, 8, 9, 16, 25]); h = rng.choice([1, 2, 4, 8])
-            dq = rng.choice([32, 64]); dv = rng.choice([32, 64, 128]); bias = rng.random() < 0.5
-            print(f"[{n}] attention seed={seed} nb={nb} s={s} h={h} dq={dq} dv={dv} bias={bias}", flush=True)
+            nb = rng.choice([1, 2, 3, 8]); s = 8 * rng.choice([1, 3, 8, 9, 16, 17, 25, 40]); h = rng.choice([1, 2, 4, 8])
+            dq = rng.choice([32, 64]); dv = rng.choice([32, 64, 128])
+            print(f"[{n}] attention seed={seed} nb={nb} s={s} h={h} dq={dq} dv={dv}", flush=True)
             T = nb * s
             q, k, v, do = (bf(torch.randn(T, h * w, generator=g)) for w in (dq, dq, dv, dv))
-            bq, bk, bv = ((0.3 * torch.randn(h * w, generator=g)) if bias else None for w in (dq, dq, dv))
-            eff = lambda t, b: (t.double() if b is None else bf(t.float() + b).double()).requires_grad_()   # noqa: E731
-            ql, kl, vl = eff(q, bq), eff(k, bk), eff(v, bv)
+            ql, kl, vl = q.double(), k.double(), v.double()
             scale = 1.0 / math.sqrt(dq)
             sc = torch.einsum("bqhd,bkhd->bhqk", ql.view(nb, s, h, dq), kl.view(nb, s, h, dq)) * scale
             sc = sc.masked_fill(~torch.ones(s, s, dtype=torch.bool).tril(), float("-inf"))
             P = torch.softmax(sc, -1).detach()
             want = torch.einsum("bhqk,bkhd->bqhd", P, vl.detach().view(nb, s, h, dv)).reshape(T, h * dv)
-            dv_ = lambda t: None if t is None else t.to(dev)                                               # noqa: E731
             gq, gk, gv, gdo = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
-            out, lse = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
+            out, lse = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, scale)
             rel = lambda a, b: ((a.double().cpu() - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()  # noqa: E731
             assert rel(out, want) < 8e-3
             dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(),
-                                                  lse, nb, s, h, scale, dv_(bq), dv_(bk), dv_(bv))
+                                                  lse, nb, s, h, scale)
             # The backward of a fused attention (this one and the library routine the reference calls) takes the SAVED
             # output, a bf16 tensor, for D = rowsum(dout * out); on short sequences with wide value heads that rounding
             # is not averaged away (seen: 3 % of max |dk| at s = 8, d_v = 128 against autograd through the exact output).
