@@ -38,6 +38,10 @@
 // that walks the key blocks 0 .. diagonal.  All three recompute the probabilities from q, k and the saved
 // log-sum-exp.  No atomics: results are reproducible.
 //
+// Between a block's first score product and its last accumulating product a wave runs at raised priority (s_setprio):
+// of the waves that share a SIMD, the one that can feed the matrix cores goes first, the ones in their vector-only
+// stretches (masking, running maximum, address arithmetic) fill in (6-8 % on every kernel).
+//
 // Positions past the end of a sequence (seq not a multiple of the block sizes): loads repeat the last valid row or
 // 8-position piece, so every operand stays finite; their scores are masked (keys), zeroed (queries of the dV / dK
 // kernels) or never stored.
@@ -251,12 +255,14 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
     if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
     const char *sk = lds + (kb & 1) * BUF, *sv = sk + K_BYTES;
     att_f32x16 s[2];
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       s[t] = att_zero16();
 #pragma unroll
       for (int st = 0; st < DQK / 16; ++st) s[t] = att_mfma(att_frag<KRB>(sk, t * 32 + r32, st, g), qf[st], s[t]);
     }
+    __builtin_amdgcn_s_setprio(0);
     if (key0 + ATT_STEP - 1 > wq0) {       // some key of the block lies after some query of the wave
       const int thr = q_row - key0 - 4 * g;      // the lane's element at key offset 32 t + 8 j + i above this is masked
 #pragma unroll
@@ -283,6 +289,7 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
       m = m_new;
     }
     float rs = 0.f;
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       uint32_t pk[8];
@@ -300,6 +307,7 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
         for (int n = 0; n < DV / 32; ++n) o[n] = att_mfma(att_frag<128>(sv, n * 32 + r32, 2 * t + c, g), pb[c], o[n]);
     }
     l += rs;
+    __builtin_amdgcn_s_setprio(0);
   }
   l = att_half_sum(l);
   __syncthreads();                         // the tile buffers become the staging area of the epilogue
@@ -442,6 +450,7 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
     const float *svec = reinterpret_cast<const float *>(so + O_BYTES);
     const bool diag = q0 < wk0 + 31;       // some query of the block lies before some key of the wave
     const bool tail = q0 + ATT_STEP > seq; // some query of the block lies past the sequence
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       att_f32x16 s = att_zero16();
@@ -487,6 +496,7 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 #pragma unroll
         for (int n = 0; n < ACC / 32; ++n) acc[n] = att_mfma(att_frag<128>(sa, n * 32 + r32, 2 * t + c, g), xb[c], acc[n]);
     }
+    __builtin_amdgcn_s_setprio(0);
   }
   if (key < seq) att_store_transposed<ACC>(dst, acc, h * ACC, T, tok0 + key, g);
 }
@@ -553,6 +563,7 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
     if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
     const char *sk = lds + (kb & 1) * BUF, *skt = sk + K_BYTES, *sv = skt + KT_BYTES;
     const bool diag = key0 + ATT_STEP - 1 > wq0;
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       att_f32x16 s = att_zero16(), dp = att_zero16();
@@ -577,6 +588,7 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
 #pragma unroll
         for (int n = 0; n < DQK / 32; ++n) dq[n] = att_mfma(att_frag<128>(skt, n * 32 + r32, 2 * t + c, g), db[c], dq[n]);
     }
+    __builtin_amdgcn_s_setprio(0);
   }
   if (q_row < seq) att_store_transposed<DQK>(dqt, dq, h * DQK, T, tok0 + q_row, g);
 }
