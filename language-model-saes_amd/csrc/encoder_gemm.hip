@@ -48,7 +48,9 @@
 // Workgroup order: consecutive ids land on the 8 XCDs round-robin; within an XCD, 32 consecutive
 // workgroups (one per CU) cover RM token tiles x 32 / RM feature tiles, so every slab in an XCD's L2 is
 // shared by the resident workgroups (bf16: RM = 8 when there are at least 8 token tiles, 3.05 against 3.09 ms
-// for RM = 4 and 3.3 for RM = 2; fp32: RM = 4).
+// for RM = 4 and 3.3 for RM = 2; fp32: RM = 4).  The feature tiles are the dimension dealt to the XCDs, unless there are
+// fewer than 8 of them and more token tiles than that: then the token tiles are dealt and an XCD's 32 workgroups cover
+// all feature tiles of 32 / (feature tiles) token tiles (a 768-feature product would otherwise run on 3 XCDs).
 //
 // Rows beyond B or F are clamped to the last valid row when loading (their products land in
 // accumulators that the epilogue never stores), so the main loop has no bounds checks.
