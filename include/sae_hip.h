@@ -485,22 +485,23 @@ int sae_jumprelu_bwd(const void *pre, int dtype, const float *b_enc, const float
  *   out[b, s, h, :] = sum_{s' <= s} softmax_{s'}(scale * q[b, s, h, :] . k[b, s', h, :]) * v[b, s', h, :]
  * bf16 operands, fp32 accumulation, probabilities rounded to bf16 before they multiply the values (as the library's
  * fused kernels do).  T = n_batch * seq, token t = b * seq + s.  Layouts: "natural" [T, n_heads * width] (heads side by
- * side: what x @ W gives) and "transposed" [n_heads * width, T]; each operand is taken in the layout(s) whose
- * contraction index is contiguous for the products that read it.
- *   q, k      natural    [T, n_heads * d_qk]
- *   vt        transposed [n_heads * d_v, T]
- *   out       natural    [T, n_heads * d_v] bf16;  lse fp32 [n_batch, n_heads, seq] = log sum_{s'} exp(scale * q . k)
- * Requires d_qk in {32, 64}, d_v in {32, 64, 128}, seq % 8 == 0. */
-int sae_attention_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk,
+ * side: what x @ W gives) and "transposed" [n_heads * width, T].
+ *   q, k      [T, n_heads * d_qk];  v [T, n_heads * d_v]   (natural: a product over positions reads its operand across
+ *             the rows of the LDS tile with transposing reads, so no transposed copies are taken)
+ *   out       [T, n_heads * d_v] bf16;  lse fp32 [n_batch, n_heads, seq] = log sum_{s'} exp(scale * q . k)
+ * Requires d_qk in {32, 64}, d_v in {32, 64, 128}, seq % 8 == 0, at most 2^24 tokens.  Projection biases belong in the
+ * products that form q, k, v (sae_encoder_gemm_bias). */
+int sae_attention_fwd(const void *q, const void *k, const void *v, int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk,
                       int64_t d_v, double scale, void *out, float *lse, void *stream);
 
-/* Backward of sae_attention_fwd.  q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout; lse from
- * the forward pass; workspace: device float[2 * n_batch * n_heads * seq] (D = rowsum(dout * out), and the log-sum-exp in
- * the log2 domain).  Outputs, bf16, transposed: dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T] (a projection bias's
- * gradient is the row sum, sae_row_sum).  No atomics: reproducible. */
-int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                      const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads,
-                      int64_t d_qk, int64_t d_v, double scale, float *workspace, void *dqt, void *dkt, void *dvt, void *stream);
+/* Backward of sae_attention_fwd.  q, k, v, out, dout natural; lse from the forward pass; workspace: device
+ * float[2 * n_batch * n_heads * seq] (D = rowsum(dout * out), and the log-sum-exp in the log2 domain).  Outputs, bf16,
+ * TRANSPOSED: dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T], the layout in which they are the left operand of the
+ * weight-gradient product over the token axis (a projection bias's gradient is the row sum, sae_row_sum).  No atomics:
+ * reproducible. */
+int sae_attention_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout, const float *lse,
+                      int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v, double scale, float *workspace,
+                      void *dqt, void *dkt, void *dvt, void *stream);
 
 /* out[r] = sum_c src[r, c] (fp32 sum, fixed order) for src [rows, cols] fp32 or bf16.  The bias gradients autograd forms by
  * summing over tokens, for gradients held transposed ([features, tokens]). */

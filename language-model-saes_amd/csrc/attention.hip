@@ -7,12 +7,12 @@
 //
 // Layouts (bf16 unless noted; T = n_batch * seq tokens, token t = b * seq + s):
 //   "natural"     [T, n_heads * width]   one token's heads side by side (what the projections x @ W produce),
-//   "transposed"  [n_heads * width, T]   the same matrix transposed (what the projections W @ x^T produce).
-// A matrix-core operand needs its contraction index contiguous in memory.  The scores contract over the head
-// width (natural q, k), the mixing contracts over key positions (transposed v), and the backward products
-// contract over positions or over widths in turn, so each kernel takes every operand in the layout(s) its
-// products need; the transposed copies come for free from the projection GEMM with its operands swapped, or
-// from the cast-transpose kernel.
+//   "transposed"  [n_heads * width, T]   the same matrix transposed.
+// Every operand is taken natural.  A matrix-core operand needs its contraction index in a lane's registers: the
+// scores contract over the head width (a row of a q / k tile: an ordinary 16-byte LDS read), the mixing and the
+// backward's accumulating products contract over positions (a column of a v / dout / q / k tile: ds_read_b64_tr_b16,
+// the LDS read that hands a lane 4 consecutive rows of one column).  The gradients leave transposed, which is the
+// layout in which they are the left operand of the weight-gradient product over the token axis.
 //
 // Fragment convention of the instruction (D = A B, 32 x 32 x 16): lane l supplies A[m = l % 32][8 consecutive k of
 // half l / 32] and B[same k][n = l % 32], and receives D[m = 8 j + 4 (l / 32) + i][n = l % 32] in register 4 j + i
@@ -26,8 +26,9 @@
 // Tiles of the streamed operand (64 positions per iteration) go from global memory straight into LDS
 // (global_load_lds_dwordx4, two buffers: the loads of tile i + 1 are in flight while tile i is consumed; one
 // workgroup barrier per tile).  Such a load writes 1 KiB linearly (lane l -> base + 16 l), so the bank swizzle is
-// applied on the global side: a tile row of RB bytes holds its 16-byte chunk c at physical chunk
-// c ^ ((row * RB / 256) % (RB / 16)), which makes the 16 rows x one chunk of a fragment read cover 256 distinct bytes.
+// applied on the global side: a tile row holds its 16-byte chunk c at physical chunk c ^ key(row), with a key such that
+// both access patterns cover 256 distinct bytes: 16 consecutive rows x one chunk (a fragment read along rows) and 4
+// consecutive rows x 4 consecutive chunks (a transposing read across rows).
 //
 // Forward: one workgroup = 128 queries of one (batch, head), walking the key blocks 0 .. diagonal with the online
 // softmax (running maximum and sum per query in fp32, log2 domain; the accumulators are rescaled only when some
@@ -80,10 +81,17 @@ __device__ __forceinline__ uint32_t att_pack2(float a, float b) {
 }
 
 // byte offset of logical chunk `chunk` of row `row` in a tile whose rows are RB bytes
+// chunk permutation of a row: any 16 consecutive rows x one chunk, and any 4 consecutive rows (from a multiple of 4) x 4
+// consecutive chunks (from a multiple of 4), cover 256 distinct bytes
+template <int RB>
+__device__ __forceinline__ int att_swz_key(int row) {
+  if constexpr (RB == 64) return (row >> 2) & 3;
+  else if constexpr (RB == 128) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  else return ((row & 3) << 2) | ((row >> 2) & 3);
+}
 template <int RB>
 __device__ __forceinline__ int att_swz(int row, int chunk) {
-  constexpr int CPR = RB / 16, RP = 256 / RB;
-  return row * RB + ((chunk ^ ((row / RP) & (CPR - 1))) << 4);
+  return row * RB + ((chunk ^ att_swz_key<RB>(row)) << 4);
 }
 
 // A operand: row `row` of a tile, contraction positions 16 st + 8 g .. + 7
@@ -92,26 +100,37 @@ __device__ __forceinline__ att_bf16x8 att_frag(const char *tile, int row, int st
   return *reinterpret_cast<const att_bf16x8 *>(tile + att_swz<RB>(row, 2 * st + g));
 }
 
+// A operand read ACROSS the rows of a natural tile: m = column col0 + lane % 32, contraction positions = rows
+// 16 st + 8 g .. + 7.  ds_read_b64_tr_b16 hands lane j of a group of 16 element j % 4 of the 8-byte pieces that lanes
+// 4 e + j / 4 (e < 4) point at; lane i therefore points at row 8 g + 4 hh + i / 4, columns 16 (group % 2) + 4 (i % 4) .. + 3.
+// att_tr_addr gives the per-lane byte offset for (col0, hh) at st = 0; a step adds 16 RB bytes (the permutation key of
+// a row does not depend on st).
+typedef __attribute__((ext_vector_type(4))) short att_i16x4;
+template <int RB>
+__device__ __forceinline__ int att_tr_addr(int lane, int col0, int hh) {
+  const int i = lane & 15, grp = lane >> 4;
+  const int row = 8 * (grp >> 1) + 4 * hh + (i >> 2), col = col0 + 16 * (grp & 1) + 4 * (i & 3);
+  return att_swz<RB>(row, col >> 3) + (col & 7) * 2;
+}
+__device__ __forceinline__ att_bf16x8 att_frag_tr(const char *tile, int addr0, int addr1, int step_bytes) {
+  typedef __attribute__((address_space(3))) att_i16x4 *lds_i16x4;
+  const att_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(tile + addr0 + step_bytes));
+  const att_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(tile + addr1 + step_bytes));
+  typedef __attribute__((ext_vector_type(8))) short i16x8;
+  const i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(att_bf16x8, v);
+}
+
 // Per-lane byte offsets of a wave's NL loads of a tile (wave-load wl = wave * NL + i covers 1 KiB of it).
 // Natural tile: rows are consecutive tokens of a matrix with `ld` elements per token, RB bytes of each are taken;
 // rows at or past `rows_valid` repeat row rows_valid - 1.
 template <int RB, int NL>
 __device__ __forceinline__ void att_nat_offsets(uint32_t (&off)[NL], int wave, int lane, int ld, int rows_valid) {
-  constexpr int CPR = RB / 16, RPL = 1024 / RB, RP = 256 / RB;
+  constexpr int CPR = RB / 16, RPL = 1024 / RB;
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int row = (wave * NL + i) * RPL + lane / CPR, ch = (lane % CPR) ^ ((row / RP) & (CPR - 1));
+    const int row = (wave * NL + i) * RPL + lane / CPR, ch = (lane % CPR) ^ att_swz_key<RB>(row);
     off[i] = (uint32_t)(min(row, rows_valid - 1) * ld + ch * 8) * 2u;
-  }
-}
-// Transposed tile: row r is feature row r of a matrix with T tokens per row, 64 consecutive tokens (128 bytes) of each
-// are taken; 8-token pieces at or past `cols_valid` (a multiple of 8) repeat the last valid piece.
-template <int NL>
-__device__ __forceinline__ void att_tr_offsets(uint32_t (&off)[NL], int wave, int lane, int64_t T, int cols_valid) {
-#pragma unroll
-  for (int i = 0; i < NL; ++i) {
-    const int row = (wave * NL + i) * 8 + (lane >> 3), ch = (lane & 7) ^ ((row >> 1) & 7);
-    off[i] = (uint32_t)((int64_t)row * T + min(ch * 8, cols_valid - 8)) * 2u;
   }
 }
 template <int NL>
@@ -202,10 +221,11 @@ __device__ __forceinline__ void att_store_transposed(uint16_t *__restrict__ dst,
 // ---- forward ---------------------------------------------------------------------------------------------
 template <int DQK, int DV>
 __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ vt, uint16_t *__restrict__ out,
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, uint16_t *__restrict__ out,
     float *__restrict__ lse, int seq, int n_heads, int n_batch, int64_t T, float sc2) {
   constexpr int KRB = DQK * 2;                                    // bytes of a key row
-  constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = DV * 128, BUF = K_BYTES + V_BYTES;
+  constexpr int VRB = DV * 2;
+  constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + V_BYTES;
   constexpr int KNL = K_BYTES / 4096, VNL = V_BYTES / 4096;      // loads per wave and tile
   constexpr int OP = DV * 2 + 16;                                 // staging row pitch of the epilogue
   constexpr int LDS_BYTES = 2 * BUF > 4 * 32 * OP ? 2 * BUF : 4 * 32 * OP;
@@ -229,23 +249,28 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
   const int n_kb = (min(seq, (qb + 1) * ATT_OWN) + ATT_STEP - 1) / ATT_STEP;
   uint32_t koff[KNL], voff[VNL];
   att_nat_offsets<KRB, KNL>(koff, wave, lane, ldq, ATT_STEP);
-  att_tr_offsets<VNL>(voff, wave, lane, T, ATT_STEP);
-  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *vbase = vt + (int64_t)h * DV * T + tok0;
+  att_nat_offsets<VRB, VNL>(voff, wave, lane, ldv, ATT_STEP);
+  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *vbase = v + tok0 * ldv + h * DV;
   auto issue = [&](int kb) {
     const uint32_t buf = lds_base + (uint32_t)(kb & 1) * BUF;
-    const uint16_t *kt_ = kbase + (int64_t)kb * ATT_STEP * ldq, *vt_ = vbase + kb * ATT_STEP;
+    const uint16_t *k_ = kbase + (int64_t)kb * ATT_STEP * ldq, *v_ = vbase + (int64_t)kb * ATT_STEP * ldv;
     const int rem = seq - kb * ATT_STEP;
     if (rem >= ATT_STEP) {
-      att_dma<KNL>(kt_, koff, buf + wave * KNL * 1024);
-      att_dma<VNL>(vt_, voff, buf + K_BYTES + wave * VNL * 1024);
+      att_dma<KNL>(k_, koff, buf + wave * KNL * 1024);
+      att_dma<VNL>(v_, voff, buf + K_BYTES + wave * VNL * 1024);
     } else {
       uint32_t ko[KNL], vo[VNL];
       att_nat_offsets<KRB, KNL>(ko, wave, lane, ldq, rem);
-      att_tr_offsets<VNL>(vo, wave, lane, T, rem);
-      att_dma<KNL>(kt_, ko, buf + wave * KNL * 1024);
-      att_dma<VNL>(vt_, vo, buf + K_BYTES + wave * VNL * 1024);
+      att_nat_offsets<VRB, VNL>(vo, wave, lane, ldv, rem);
+      att_dma<KNL>(k_, ko, buf + wave * KNL * 1024);
+      att_dma<VNL>(v_, vo, buf + K_BYTES + wave * VNL * 1024);
     }
   };
+  int vaddr[DV / 32][2];
+#pragma unroll
+  for (int n = 0; n < DV / 32; ++n)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) vaddr[n][hh] = att_tr_addr<VRB>(lane, n * 32, hh);
   issue(0);
   for (int kb = 0; kb < n_kb; ++kb) {
     __builtin_amdgcn_s_waitcnt(ATT_WAITCNT_VM(0));
@@ -304,7 +329,7 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int n = 0; n < DV / 32; ++n) o[n] = att_mfma(att_frag<128>(sv, n * 32 + r32, 2 * t + c, g), pb[c], o[n]);
+        for (int n = 0; n < DV / 32; ++n) o[n] = att_mfma(att_frag_tr(sv, vaddr[n][0], vaddr[n][1], (2 * t + c) * 16 * VRB), pb[c], o[n]);
     }
     l += rs;
     __builtin_amdgcn_s_setprio(0);
@@ -375,18 +400,17 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const uint16_t *__re
 // SIMD, which waits on its own barriers.)
 template <int DQK, int DV, int WHAT>
 __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ qt, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    const uint16_t *__restrict__ dout, const uint16_t *__restrict__ doutt, const float *__restrict__ lse2,
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+    const uint16_t *__restrict__ dout, const float *__restrict__ lse2,
     const float *__restrict__ dvec, uint16_t *__restrict__ dst, int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
   constexpr bool DK = WHAT == 1;
   constexpr int QRB = DQK * 2, ORB = DV * 2;
-  constexpr int Q_BYTES = ATT_STEP * QRB;                              // q natural (both)
-  constexpr int A_BYTES = DK ? DQK * 128 : DV * 128;                   // q^T (dK) or dout^T (dV): the accumulating product's A tile
-  constexpr int O_BYTES = DK ? ATT_STEP * ORB : 0;                     // dout natural (dK)
+  constexpr int Q_BYTES = ATT_STEP * QRB, O_BYTES = ATT_STEP * ORB;    // the streamed tiles: 64 queries' q and dout rows
   constexpr int VEC_BYTES = 512;                                       // 64 x (lse2, D)
-  constexpr int BUF = Q_BYTES + A_BYTES + O_BYTES + VEC_BYTES;
-  constexpr int QNL = Q_BYTES / 4096, ANL = A_BYTES / 4096, ONL = DK ? O_BYTES / 4096 : 1;
+  constexpr int BUF = Q_BYTES + O_BYTES + VEC_BYTES;
+  constexpr int QNL = Q_BYTES / 4096, ONL = O_BYTES / 4096;
   constexpr int ACC = DK ? DQK : DV;                                   // rows of the accumulated matrix
+  constexpr int ARB = DK ? QRB : ORB;                                  // row bytes of the tile the accumulating product reads across
   __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
   const int n_qb = (seq + ATT_STEP - 1) / ATT_STEP;
   int kb, h, b;
@@ -405,37 +429,35 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
-  uint32_t qoff[QNL], aoff[ANL], ooff[ONL];
+  uint32_t qoff[QNL], ooff[ONL];
   att_nat_offsets<QRB, QNL>(qoff, wave, lane, ldq, ATT_STEP);
-  att_tr_offsets<ANL>(aoff, wave, lane, T, ATT_STEP);
-  if constexpr (DK) att_nat_offsets<ORB, ONL>(ooff, wave, lane, ldv, ATT_STEP);
+  att_nat_offsets<ORB, ONL>(ooff, wave, lane, ldv, ATT_STEP);
+  int aaddr[ACC / 32][2];
+#pragma unroll
+  for (int n = 0; n < ACC / 32; ++n)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) aaddr[n][hh] = att_tr_addr<ARB>(lane, n * 32, hh);
   const uint16_t *qbase = q + tok0 * ldq + h * DQK;
-  const uint16_t *abase = (DK ? qt + (int64_t)h * DQK * T : doutt + (int64_t)h * DV * T) + tok0;
   const uint16_t *obase = dout + tok0 * ldv + h * DV;
   const float *lbase = lse2 + ((int64_t)b * n_heads + h) * seq, *dbase = dvec + ((int64_t)b * n_heads + h) * seq;
   auto issue = [&](int qb, int slot) {
     const uint32_t buf = lds_base + (uint32_t)slot * BUF;
     const int q0 = qb * ATT_STEP, rem = seq - q0;
-    const uint16_t *q_ = qbase + (int64_t)q0 * ldq, *a_ = abase + q0, *o_ = obase + (int64_t)q0 * ldv;
+    const uint16_t *q_ = qbase + (int64_t)q0 * ldq, *o_ = obase + (int64_t)q0 * ldv;
     if (rem >= ATT_STEP) {
       att_dma<QNL>(q_, qoff, buf + wave * QNL * 1024);
-      att_dma<ANL>(a_, aoff, buf + Q_BYTES + wave * ANL * 1024);
-      if constexpr (DK) att_dma<ONL>(o_, ooff, buf + Q_BYTES + A_BYTES + wave * ONL * 1024);
+      att_dma<ONL>(o_, ooff, buf + Q_BYTES + wave * ONL * 1024);
     } else {
-      uint32_t qo[QNL], ao[ANL], oo[ONL];
+      uint32_t qo[QNL], oo[ONL];
       att_nat_offsets<QRB, QNL>(qo, wave, lane, ldq, rem);
-      att_tr_offsets<ANL>(ao, wave, lane, T, rem);
+      att_nat_offsets<ORB, ONL>(oo, wave, lane, ldv, rem);
       att_dma<QNL>(q_, qo, buf + wave * QNL * 1024);
-      att_dma<ANL>(a_, ao, buf + Q_BYTES + wave * ANL * 1024);
-      if constexpr (DK) {
-        att_nat_offsets<ORB, ONL>(oo, wave, lane, ldv, rem);
-        att_dma<ONL>(o_, oo, buf + Q_BYTES + A_BYTES + wave * ONL * 1024);
-      }
+      att_dma<ONL>(o_, oo, buf + Q_BYTES + wave * ONL * 1024);
     }
     // the 64 queries' log-sum-exp (wave 0) and D (wave 1, dK only): 4 bytes per lane
     const uint32_t voff = (uint32_t)min(lane, rem - 1) * 4u;
-    if (wave == 0) ATT_DMA4(lbase + q0, voff, buf + Q_BYTES + A_BYTES + O_BYTES);
-    if (DK && wave == 1) ATT_DMA4(dbase + q0, voff, buf + Q_BYTES + A_BYTES + O_BYTES + 256);
+    if (wave == 0) ATT_DMA4(lbase + q0, voff, buf + Q_BYTES + O_BYTES);
+    if (DK && wave == 1) ATT_DMA4(dbase + q0, voff, buf + Q_BYTES + O_BYTES + 256);
   };
   const int qb0 = kb * (ATT_OWN / ATT_STEP);
   if (qb0 < n_qb) issue(qb0, 0);
@@ -446,7 +468,7 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
     if (qb + 1 < n_qb) issue(qb + 1, slot ^ 1);
     const int q0 = qb * ATT_STEP;
     if (q0 + ATT_STEP - 1 < wk0) continue; // every query of this block lies before every key of this wave
-    const char *sq = lds + slot * BUF, *sa = sq + Q_BYTES, *so = sa + A_BYTES;
+    const char *sq = lds + slot * BUF, *so = sq + Q_BYTES, *sa = DK ? sq : so;
     const float *svec = reinterpret_cast<const float *>(so + O_BYTES);
     const bool diag = q0 < wk0 + 31;       // some query of the block lies before some key of the wave
     const bool tail = q0 + ATT_STEP > seq; // some query of the block lies past the sequence
@@ -494,7 +516,7 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int n = 0; n < ACC / 32; ++n) acc[n] = att_mfma(att_frag<128>(sa, n * 32 + r32, 2 * t + c, g), xb[c], acc[n]);
+        for (int n = 0; n < ACC / 32; ++n) acc[n] = att_mfma(att_frag_tr(sa, aaddr[n][0], aaddr[n][1], (2 * t + c) * 16 * ARB), xb[c], acc[n]);
     }
     __builtin_amdgcn_s_setprio(0);
   }
@@ -505,12 +527,12 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 // dQ^T[c, q] = sum_key k^T[c, key] dS[q, key] over key <= q.
 template <int DQK, int DV>
 __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ kt, const uint16_t *__restrict__ v,
+    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     const uint16_t *__restrict__ dout, const float *__restrict__ lse2, const float *__restrict__ dvec, uint16_t *__restrict__ dqt,
     int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
   constexpr int KRB = DQK * 2, VRB = DV * 2;
-  constexpr int K_BYTES = ATT_STEP * KRB, KT_BYTES = DQK * 128, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + KT_BYTES + V_BYTES;
-  constexpr int KNL = K_BYTES / 4096, KTNL = KT_BYTES / 4096, VNL = V_BYTES / 4096;
+  constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + V_BYTES;
+  constexpr int KNL = K_BYTES / 4096, VNL = V_BYTES / 4096;
   __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
   int qb, h, b;
   att_block_coords((seq + ATT_OWN - 1) / ATT_OWN, n_heads, n_batch, true, qb, h, b);
@@ -531,27 +553,28 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
   const int n_kb = (min(seq, (qb + 1) * ATT_OWN) + ATT_STEP - 1) / ATT_STEP;
-  uint32_t koff[KNL], ktoff[KTNL], voff[VNL];
+  uint32_t koff[KNL], voff[VNL];
   att_nat_offsets<KRB, KNL>(koff, wave, lane, ldq, ATT_STEP);
-  att_tr_offsets<KTNL>(ktoff, wave, lane, T, ATT_STEP);
   att_nat_offsets<VRB, VNL>(voff, wave, lane, ldv, ATT_STEP);
-  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *ktbase = kt + (int64_t)h * DQK * T + tok0, *vbase = v + tok0 * ldv + h * DV;
+  int kaddr[DQK / 32][2];
+#pragma unroll
+  for (int n = 0; n < DQK / 32; ++n)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) kaddr[n][hh] = att_tr_addr<KRB>(lane, n * 32, hh);
+  const uint16_t *kbase = k + tok0 * ldq + h * DQK, *vbase = v + tok0 * ldv + h * DV;
   auto issue = [&](int kb) {
     const uint32_t buf = lds_base + (uint32_t)(kb & 1) * BUF;
     const int key0 = kb * ATT_STEP, rem = seq - key0;
-    const uint16_t *k_ = kbase + (int64_t)key0 * ldq, *kt_ = ktbase + key0, *v_ = vbase + (int64_t)key0 * ldv;
+    const uint16_t *k_ = kbase + (int64_t)key0 * ldq, *v_ = vbase + (int64_t)key0 * ldv;
     if (rem >= ATT_STEP) {
       att_dma<KNL>(k_, koff, buf + wave * KNL * 1024);
-      att_dma<KTNL>(kt_, ktoff, buf + K_BYTES + wave * KTNL * 1024);
-      att_dma<VNL>(v_, voff, buf + K_BYTES + KT_BYTES + wave * VNL * 1024);
+      att_dma<VNL>(v_, voff, buf + K_BYTES + wave * VNL * 1024);
     } else {
-      uint32_t ko[KNL], kto[KTNL], vo[VNL];
+      uint32_t ko[KNL], vo[VNL];
       att_nat_offsets<KRB, KNL>(ko, wave, lane, ldq, rem);
-      att_tr_offsets<KTNL>(kto, wave, lane, T, rem);
       att_nat_offsets<VRB, VNL>(vo, wave, lane, ldv, rem);
       att_dma<KNL>(k_, ko, buf + wave * KNL * 1024);
-      att_dma<KTNL>(kt_, kto, buf + K_BYTES + wave * KTNL * 1024);
-      att_dma<VNL>(v_, vo, buf + K_BYTES + KT_BYTES + wave * VNL * 1024);
+      att_dma<VNL>(v_, vo, buf + K_BYTES + wave * VNL * 1024);
     }
   };
   issue(0);
@@ -561,7 +584,7 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
     if (kb + 1 < n_kb) issue(kb + 1);
     const int key0 = kb * ATT_STEP;
     if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
-    const char *sk = lds + (kb & 1) * BUF, *skt = sk + K_BYTES, *sv = skt + KT_BYTES;
+    const char *sk = lds + (kb & 1) * BUF, *sv = sk + K_BYTES;
     const bool diag = key0 + ATT_STEP - 1 > wq0;
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
@@ -586,7 +609,7 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int n = 0; n < DQK / 32; ++n) dq[n] = att_mfma(att_frag<128>(skt, n * 32 + r32, 2 * t + c, g), db[c], dq[n]);
+        for (int n = 0; n < DQK / 32; ++n) dq[n] = att_mfma(att_frag_tr(sk, kaddr[n][0], kaddr[n][1], (2 * t + c) * 16 * KRB), db[c], dq[n]);
     }
     __builtin_amdgcn_s_setprio(0);
   }
@@ -633,19 +656,19 @@ __global__ __launch_bounds__(256) void row_sum_kernel(const void *__restrict__ s
 }
 
 template <int DQK, int DV>
-static int launch_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads, double scale,
+static int launch_fwd(const void *q, const void *k, const void *v, int64_t n_batch, int64_t seq, int64_t n_heads, double scale,
                       void *out, float *lse, hipStream_t st) {
   const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)vt, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch, n_batch * seq,
+                     (const uint16_t *)v, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch, n_batch * seq,
                      (float)(scale * 1.4426950408889634));
   return check_launch("attention_fwd");
 }
 
 template <int DQK, int DV>
-static int launch_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                      const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq, int64_t n_heads,
-                      double scale, float *workspace, void *dqt, void *dkt, void *dvt, hipStream_t st) {
+static int launch_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout, const float *lse,
+                      int64_t n_batch, int64_t seq, int64_t n_heads, double scale, float *workspace, void *dqt, void *dkt,
+                      void *dvt, hipStream_t st) {
   const int64_t T = n_batch * seq;
   const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   const float sc2 = (float)(scale * 1.4426950408889634);
@@ -653,15 +676,15 @@ static int launch_bwd(const void *q, const void *qt, const void *k, const void *
   const int64_t prep_blocks = (T * n_heads * 16 + 255) / 256;
   hipLaunchKernelGGL((attn_bwd_prep_kernel<DV>), dim3((unsigned)prep_blocks), dim3(256), 0, st, (const uint16_t *)dout,
                      (const uint16_t *)out, lse, dvec, lse2, (int)seq, (int)n_heads, T);
-  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 0>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)qt,
-                     (const uint16_t *)k, (const uint16_t *)v, (const uint16_t *)dout, (const uint16_t *)doutt, lse2, dvec,
-                     (uint16_t *)dvt, (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
-  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 1>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)qt,
-                     (const uint16_t *)k, (const uint16_t *)v, (const uint16_t *)dout, (const uint16_t *)doutt, lse2, dvec,
-                     (uint16_t *)dkt, (int)seq, (int)n_heads, (int)n_batch, T, sc2, (float)scale);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 0>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
+                     (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dvt, (int)seq, (int)n_heads,
+                     (int)n_batch, T, sc2, (float)scale);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 1>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
+                     (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dkt, (int)seq, (int)n_heads,
+                     (int)n_batch, T, sc2, (float)scale);
   hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)kt, (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dqt, (int)seq,
-                     (int)n_heads, (int)n_batch, T, sc2, (float)scale);
+                     (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dqt, (int)seq, (int)n_heads,
+                     (int)n_batch, T, sc2, (float)scale);
   return check_launch("attention_bwd");
 }
 
@@ -689,28 +712,27 @@ static int check_shapes(const char *what, int64_t n_batch, int64_t seq, int64_t 
   if (d_qk == 64 && d_v == 64) return CALL(64, 64);                             \
   return CALL(64, 128);
 
-extern "C" int sae_attention_fwd(const void *q, const void *k, const void *vt, int64_t n_batch, int64_t seq, int64_t n_heads,
+extern "C" int sae_attention_fwd(const void *q, const void *k, const void *v, int64_t n_batch, int64_t seq, int64_t n_heads,
                                  int64_t d_qk, int64_t d_v, double scale, void *out, float *lse, void *stream) {
   using namespace sae;
-  SAE_REQUIRE(q && k && vt && out && lse, SAE_ERR_INVALID_ARG, "attention_fwd: null pointer");
+  SAE_REQUIRE(q && k && v && out && lse, SAE_ERR_INVALID_ARG, "attention_fwd: null pointer");
   const int rc = check_shapes("attention_fwd", n_batch, seq, n_heads, d_qk, d_v);
   if (rc != SAE_OK) return rc;
-#define ATT_FWD(A, B) launch_fwd<A, B>(q, k, vt, n_batch, seq, n_heads, scale, out, lse, (hipStream_t)stream)
+#define ATT_FWD(A, B) launch_fwd<A, B>(q, k, v, n_batch, seq, n_heads, scale, out, lse, (hipStream_t)stream)
   ATT_DISPATCH(ATT_FWD)
 #undef ATT_FWD
 }
 
-extern "C" int sae_attention_bwd(const void *q, const void *qt, const void *k, const void *kt, const void *v, const void *out,
-                                 const void *dout, const void *doutt, const float *lse, int64_t n_batch, int64_t seq,
-                                 int64_t n_heads, int64_t d_qk, int64_t d_v, double scale, float *workspace, void *dqt, void *dkt,
-                                 void *dvt, void *stream) {
+extern "C" int sae_attention_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout, const float *lse,
+                                 int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v, double scale,
+                                 float *workspace, void *dqt, void *dkt, void *dvt, void *stream) {
   using namespace sae;
-  SAE_REQUIRE(q && qt && k && kt && v && out && dout && doutt && lse && workspace && dqt && dkt && dvt,
-              SAE_ERR_INVALID_ARG, "attention_bwd: null pointer");
+  SAE_REQUIRE(q && k && v && out && dout && lse && workspace && dqt && dkt && dvt, SAE_ERR_INVALID_ARG,
+              "attention_bwd: null pointer");
   const int rc = check_shapes("attention_bwd", n_batch, seq, n_heads, d_qk, d_v);
   if (rc != SAE_OK) return rc;
 #define ATT_BWD(A, B) \
-  launch_bwd<A, B>(q, qt, k, kt, v, out, dout, doutt, lse, n_batch, seq, n_heads, scale, workspace, dqt, dkt, dvt, (hipStream_t)stream)
+  launch_bwd<A, B>(q, k, v, out, dout, lse, n_batch, seq, n_heads, scale, workspace, dqt, dkt, dvt, (hipStream_t)stream)
   ATT_DISPATCH(ATT_BWD)
 #undef ATT_BWD
 }

@@ -82,12 +82,11 @@ class _ProjectAndMix(torch.autograd.Function):
     """x -> q, k, v projections -> causal attention mixing -> hidden_pre [T, F] (bf16), all on the GEMM and attention
     kernels, for the configuration without rotary embedding and query / key norms.
 
-    forward : q = x W_Q, k = x W_K as [T, h dq] (natural), v^T = W_V x^T as [F, T] (the GEMM with its operands swapped
-              yields the transposed layout the mixing product contracts over); the biases are added in the products'
-              epilogues.
-    backward: the transposed copies q^T, k^T, v, dout^T (cast-transpose kernel); the attention backward returns
-              dq^T, dk^T, dv^T [., T] in one buffer, which is exactly the operand of the weight-gradient product
-              dW = d(.)^T x over the token axis (one GEMM for the three); bias gradients are its row sums."""
+    forward : q = x W_Q, k = x W_K as [T, h dq], v = x W_V as [T, F]; the biases are added in the products' epilogues.
+    backward: the attention backward takes the same operands (products over positions read their tiles across the
+              rows) and returns dq^T, dk^T, dv^T [., T] in one buffer, which is exactly the operand of the
+              weight-gradient product dW = d(.)^T x over the token axis (one GEMM for the three); bias gradients are its
+              row sums."""
 
     @staticmethod
     def forward(ctx, x2, W_Q, W_K, W_V, b_Q, b_K, b_V, model, seq):
@@ -102,10 +101,10 @@ class _ProjectAndMix(torch.autograd.Function):
         flat = lambda b: b.detach().float().reshape(-1).contiguous()        # noqa: E731
         q = ops.encoder_gemm_bias(x_op, wq, col_bias=flat(b_Q))             # [T, h dq]
         k = ops.encoder_gemm_bias(x_op, wk, col_bias=flat(b_K))
-        vt = ops.encoder_gemm_bias(wv, x_op, row_bias=flat(b_V))            # [F, T]
+        v = ops.encoder_gemm_bias(x_op, wv, col_bias=flat(b_V))             # [T, F]
         scale = 1.0 / model.attn_scale
-        out, lse = ops.attention_fwd(q, k, vt, n_batch, seq, h, scale)
-        ctx.save_for_backward(x_op, wq, wk, wv, q, k, vt, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
+        out, lse = ops.attention_fwd(q, k, v, n_batch, seq, h, scale)
+        ctx.save_for_backward(x_op, wq, wk, wv, q, k, v, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
         ctx.dims = (n_batch, seq, h, scale)
         ctx.shapes = (tuple(W_Q.shape), tuple(W_K.shape))
         ctx.x_dtype = x2.dtype
@@ -113,13 +112,10 @@ class _ProjectAndMix(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dz):
-        x_op, wq, wk, wv, q, k, vt, out, lse, b_Q, b_K, b_V = ctx.saved_tensors
+        x_op, wq, wk, wv, q, k, v, out, lse, b_Q, b_K, b_V = ctx.saved_tensors
         n_batch, seq, h, scale = ctx.dims
         dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
-        qt, kt, v = ops.transpose_to_bf16(q)[0], ops.transpose_to_bf16(k)[0], ops.transpose_to_bf16(vt)[0]
-        dzt = ops.transpose_to_bf16(dz)[0]                                  # [F, T]
-        dqt, dkt, dvt, stacked = ops.attention_bwd(q, qt, k, kt, v, out, dz, dzt, lse, n_batch, seq, h, scale,
-                                                   return_stacked=True)
+        dqt, dkt, dvt, stacked = ops.attention_bwd(q, k, v, out, dz, lse, n_batch, seq, h, scale, return_stacked=True)
         xt = ops.transpose_to_bf16(x_op)[0]                                 # [d, T]
         d = x_op.shape[1]
         n_qk = q.shape[1]

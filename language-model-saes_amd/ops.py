@@ -1014,47 +1014,43 @@ def _att_check(name: str, t: torch.Tensor, shape: tuple) -> None:
         raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
-def attention_fwd(q: torch.Tensor, k: torch.Tensor, vt: torch.Tensor, n_batch: int, seq: int, n_heads: int,
+def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_batch: int, seq: int, n_heads: int,
                   scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Causal softmax attention: q, k natural [T, n_heads * d_qk], vt transposed [n_heads * d_v, T] (bf16, T = n_batch * seq)
-    -> (out natural [T, n_heads * d_v] bf16, lse fp32 [n_batch, n_heads, seq]).  Projection biases belong in the
-    products that form q, k and vt (`encoder_gemm_bias`)."""
+    """Causal softmax attention: q, k [T, n_heads * d_qk], v [T, n_heads * d_v] (bf16, T = n_batch * seq, a token's heads
+    side by side) -> (out [T, n_heads * d_v] bf16, lse fp32 [n_batch, n_heads, seq]).  Projection biases belong in the
+    products that form q, k and v (`encoder_gemm_bias`)."""
     T = n_batch * seq
-    d_qk, d_v = q.shape[1] // n_heads, vt.shape[0] // n_heads
-    _att_check("q", q, (T, n_heads * d_qk)); _att_check("k", k, (T, n_heads * d_qk)); _att_check("vt", vt, (n_heads * d_v, T))
+    d_qk, d_v = q.shape[1] // n_heads, v.shape[1] // n_heads
+    _att_check("q", q, (T, n_heads * d_qk)); _att_check("k", k, (T, n_heads * d_qk)); _att_check("v", v, (T, n_heads * d_v))
     out = torch.empty(T, n_heads * d_v, dtype=torch.bfloat16, device=q.device)
     lse = torch.empty(n_batch, n_heads, seq, dtype=torch.float32, device=q.device)
     with _timed("attention_fwd"):
-        check(_lib.load().sae_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), n_batch, seq, n_heads, d_qk, d_v,
+        check(_lib.load().sae_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), n_batch, seq, n_heads, d_qk, d_v,
                                             float(scale), out.data_ptr(), lse.data_ptr(), _stream(q)), "attention_fwd")
     return out, lse
 
 
-def attention_bwd(q: torch.Tensor, qt: torch.Tensor, k: torch.Tensor, kt: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
-                  dout: torch.Tensor, doutt: torch.Tensor, lse: torch.Tensor, n_batch: int, seq: int, n_heads: int, scale: float,
-                  return_stacked: bool = False):
-    """Backward of attention_fwd -> (dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T]) in bf16, transposed layout.
-    q, k, v, out, dout natural; qt, kt, doutt the transposed copies of q, k, dout.  The three are row blocks of one
-    buffer [n_heads * (2 d_qk + d_v), T], returned as a fourth value with `return_stacked`."""
+def attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
+                  n_batch: int, seq: int, n_heads: int, scale: float, return_stacked: bool = False):
+    """Backward of attention_fwd (operands as there, dout like out) -> (dqt, dkt [n_heads * d_qk, T], dvt [n_heads * d_v, T])
+    in bf16, TRANSPOSED: the three are row blocks of one buffer [n_heads * (2 d_qk + d_v), T], the left operand of a
+    weight-gradient product over the token axis, returned as a fourth value with `return_stacked`."""
     T = n_batch * seq
     d_qk, d_v = q.shape[1] // n_heads, v.shape[1] // n_heads
-    for name, t, shape in (("q", q, (T, n_heads * d_qk)), ("k", k, (T, n_heads * d_qk)), ("qt", qt, (n_heads * d_qk, T)),
-                           ("kt", kt, (n_heads * d_qk, T)), ("v", v, (T, n_heads * d_v)), ("out", out, (T, n_heads * d_v)),
-                           ("dout", dout, (T, n_heads * d_v)), ("doutt", doutt, (n_heads * d_v, T))):
+    for name, t, shape in (("q", q, (T, n_heads * d_qk)), ("k", k, (T, n_heads * d_qk)), ("v", v, (T, n_heads * d_v)),
+                           ("out", out, (T, n_heads * d_v)), ("dout", dout, (T, n_heads * d_v))):
         _att_check(name, t, shape)
     _req(lse, "lse", torch.float32, 3)
     if tuple(lse.shape) != (n_batch, n_heads, seq):
         raise ValueError("lse must be [n_batch, n_heads, seq]")
     dev = q.device
-    # one buffer, so that a caller can also treat the three gradients as one [2 h d_qk + h d_v, T] matrix
     grads = torch.empty(n_heads * (2 * d_qk + d_v), T, dtype=torch.bfloat16, device=dev)
     dqt, dkt, dvt = grads[: n_heads * d_qk], grads[n_heads * d_qk: 2 * n_heads * d_qk], grads[2 * n_heads * d_qk:]
     workspace = torch.empty(2 * n_batch * n_heads * seq, dtype=torch.float32, device=dev)
     with _timed("attention_bwd"):
-        check(_lib.load().sae_attention_bwd(q.data_ptr(), qt.data_ptr(), k.data_ptr(), kt.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                            dout.data_ptr(), doutt.data_ptr(), lse.data_ptr(), n_batch, seq, n_heads, d_qk, d_v,
-                                            float(scale), workspace.data_ptr(), dqt.data_ptr(), dkt.data_ptr(), dvt.data_ptr(),
-                                            _stream(q)), "attention_bwd")
+        check(_lib.load().sae_attention_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(),
+                                            lse.data_ptr(), n_batch, seq, n_heads, d_qk, d_v, float(scale), workspace.data_ptr(),
+                                            dqt.data_ptr(), dkt.data_ptr(), dvt.data_ptr(), _stream(q)), "attention_bwd")
     return (dqt, dkt, dvt, grads) if return_stacked else (dqt, dkt, dvt)
 
 

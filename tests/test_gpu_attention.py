@@ -80,14 +80,12 @@ def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv)
 
     to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
     gq, gk, gv, gdo = to_dev(q), to_dev(k), to_dev(v), to_dev(dout)
-    gvt = gv.t().contiguous()
-    out, lse = pkg.ops.attention_fwd(gq, gk, gvt, nb, s, h, scale)
+    out, lse = pkg.ops.attention_fwd(gq, gk, gv, nb, s, h, scale)
     assert out.dtype == torch.bfloat16 and tuple(out.shape) == (nb * s, h * dv)
     assert rel_max(out, want_out.detach()) < OUT_TOL, rel_max(out, want_out.detach())
     assert (lse.double().cpu() - want_lse.detach()).abs().max().item() < LSE_TOL * max(1.0, want_lse.abs().max().item())
 
-    dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gq.t().contiguous(), gk, gk.t().contiguous(), gv, out, gdo, gdo.t().contiguous(), lse,
-                                          nb, s, h, scale)
+    dqt, dkt, dvt = pkg.ops.attention_bwd(gq, gk, gv, out, gdo, lse, nb, s, h, scale)
     torch.cuda.synchronize()
     errs = {"dq": (rel_max(dqt.t(), ql.grad), rel_frob(dqt.t(), ql.grad)),
             "dk": (rel_max(dkt.t(), kl.grad), rel_frob(dkt.t(), kl.grad)),
@@ -101,13 +99,13 @@ def test_attention_is_causal_and_sequences_do_not_mix(pkg, dev):
     q, k, v, _ = make_case(nb, s, h, dq, dv, seed=7)
     to_dev = lambda t: t.to(torch.bfloat16).to(dev).contiguous()                # noqa: E731
     gq, gk, gv = to_dev(q), to_dev(k), to_dev(v)
-    out0, lse0 = pkg.ops.attention_fwd(gq, gk, gv.t().contiguous(), nb, s, h, 0.125)
+    out0, lse0 = pkg.ops.attention_fwd(gq, gk, gv, nb, s, h, 0.125)
     cut = 50
     gk2, gv2 = gk.clone(), gv.clone()
     gk2[cut:s] = 3.0          # later positions of sequence 0
     gv2[cut:s] = -2.0
     gk2[s + 10:] = 1.5        # and a stretch of sequence 1
-    out1, lse1 = pkg.ops.attention_fwd(gq, gk2, gv2.t().contiguous(), nb, s, h, 0.125)
+    out1, lse1 = pkg.ops.attention_fwd(gq, gk2, gv2, nb, s, h, 0.125)
     assert torch.equal(out0[:cut], out1[:cut]) and torch.equal(lse0[0, :, :cut], lse1[0, :, :cut])
     assert torch.equal(out0[s:s + 10], out1[s:s + 10])
     assert not torch.equal(out0[cut:s], out1[cut:s])
@@ -118,10 +116,10 @@ def test_attention_is_causal_and_sequences_do_not_mix(pkg, dev):
 def test_attention_rejects_shapes_it_is_not_built_for(pkg, dev):
     z = torch.zeros(16, 48, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="d_qk"):
-        pkg.ops.attention_fwd(z, z, z.t().contiguous(), 1, 16, 1, 1.0)          # d_qk = 48
+        pkg.ops.attention_fwd(z, z, z, 1, 16, 1, 1.0)          # d_qk = 48
     z = torch.zeros(12, 32, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="multiple of 8"):
-        pkg.ops.attention_fwd(z, z, z.t().contiguous(), 1, 12, 1, 1.0)
+        pkg.ops.attention_fwd(z, z, z, 1, 12, 1, 1.0)
     assert not pkg.ops.attention_shapes_supported(12, 32, 32) and pkg.ops.attention_shapes_supported(1024, 64, 128)
 
 
