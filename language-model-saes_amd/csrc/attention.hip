@@ -39,9 +39,10 @@
 // that walks the key blocks 0 .. diagonal.  All three recompute the probabilities from q, k and the saved
 // log-sum-exp.  No atomics: results are reproducible.
 //
-// Between a block's first score product and its last accumulating product a wave runs at raised priority (s_setprio):
-// of the waves that share a SIMD, the one that can feed the matrix cores goes first, the ones in their vector-only
-// stretches (masking, running maximum, address arithmetic) fill in (6-8 % on every kernel).
+// In the forward kernel a wave runs its score products and its exponentials / value products at raised priority
+// (s_setprio) and its masking, running maximum and address arithmetic at the base one: of the waves that share a
+// SIMD the one that can feed the matrix cores goes first (1-2 % in alternating runs; nothing measurable in the
+// backward kernels, which do without).
 //
 // Positions past the end of a sequence (seq not a multiple of the block sizes): loads repeat the last valid row or
 // 8-position piece, so every operand stays finite; their scores are masked (keys), zeroed (queries of the dV / dK
@@ -472,7 +473,6 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
     const float *svec = reinterpret_cast<const float *>(so + O_BYTES);
     const bool diag = q0 < wk0 + 31;       // some query of the block lies before some key of the wave
     const bool tail = q0 + ATT_STEP > seq; // some query of the block lies past the sequence
-    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       att_f32x16 s = att_zero16();
@@ -518,7 +518,6 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 #pragma unroll
         for (int n = 0; n < ACC / 32; ++n) acc[n] = att_mfma(att_frag_tr(sa, aaddr[n][0], aaddr[n][1], (2 * t + c) * 16 * ARB), xb[c], acc[n]);
     }
-    __builtin_amdgcn_s_setprio(0);
   }
   if (key < seq) att_store_transposed<ACC>(dst, acc, h * ACC, T, tok0 + key, g);
 }
@@ -586,7 +585,6 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
     if (key0 > wq0 + 31) continue;         // every key of this block lies after every query of this wave
     const char *sk = lds + (kb & 1) * BUF, *sv = sk + K_BYTES;
     const bool diag = key0 + ATT_STEP - 1 > wq0;
-    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       att_f32x16 s = att_zero16(), dp = att_zero16();
@@ -611,7 +609,6 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
 #pragma unroll
         for (int n = 0; n < DQK / 32; ++n) dq[n] = att_mfma(att_frag_tr(sk, kaddr[n][0], kaddr[n][1], (2 * t + c) * 16 * KRB), db[c], dq[n]);
     }
-    __builtin_amdgcn_s_setprio(0);
   }
   if (q_row < seq) att_store_transposed<DQK>(dqt, dq, h * DQK, T, tok0 + q_row, g);
 }
