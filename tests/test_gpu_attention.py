@@ -93,6 +93,33 @@ def test_attention_forward_and_backward_against_fp64(pkg, dev, nb, s, h, dq, dv)
     assert all(e[0] < GRAD_TOL and e[1] < GRAD_TOL / 2 for e in errs.values()), errs
 
 
+def test_attention_at_the_benchmark_shape_on_sampled_heads(pkg, dev):
+    """16 sequences x 1024 tokens, 64 heads of width 64 / 128 (8192 workgroups per kernel, every XCD slot used): forward
+    and the three gradients of a few (sequence, head) pairs against fp64 attention computed on the device."""
+    nb, s, h, dq, dv = 16, 1024, 64, 64, 128
+    g = torch.Generator(device=dev).manual_seed(11)
+    T = nb * s
+    q, k, v, do = (torch.randn(T, h * w, device=dev, generator=g).to(torch.bfloat16) for w in (dq, dq, dv, dv))
+    scale = 1.0 / math.sqrt(dq)
+    out, lse = pkg.ops.attention_fwd(q, k, v, nb, s, h, scale)
+    dqt, dkt, dvt = pkg.ops.attention_bwd(q, k, v, out, do, lse, nb, s, h, scale)
+    mask = torch.ones(s, s, dtype=torch.bool, device=dev).tril()
+    for b, hh in ((0, 0), (7, 33), (15, 63), (3, 8)):
+        rows = slice(b * s, (b + 1) * s)
+        ql = q[rows, hh * dq:(hh + 1) * dq].double().requires_grad_()
+        kl = k[rows, hh * dq:(hh + 1) * dq].double().requires_grad_()
+        vl = v[rows, hh * dv:(hh + 1) * dv].double().requires_grad_()
+        sc = (ql @ kl.t() * scale).masked_fill(~mask, float("-inf"))
+        want = torch.softmax(sc, -1) @ vl
+        (want * do[rows, hh * dv:(hh + 1) * dv].double()).sum().backward()
+        rel = lambda a, w: ((a.double() - w).abs().max() / w.abs().max()).item()     # noqa: E731
+        assert rel(out[rows, hh * dv:(hh + 1) * dv], want.detach()) < OUT_TOL
+        assert (lse[b, hh].double() - torch.logsumexp(sc.detach(), -1)).abs().max().item() < 1e-4
+        assert rel(dqt[hh * dq:(hh + 1) * dq, rows].t(), ql.grad) < GRAD_TOL
+        assert rel(dkt[hh * dq:(hh + 1) * dq, rows].t(), kl.grad) < GRAD_TOL
+        assert rel(dvt[hh * dv:(hh + 1) * dv, rows].t(), vl.grad) < GRAD_TOL
+
+
 def test_attention_is_causal_and_sequences_do_not_mix(pkg, dev):
     """Changing a later position, or another sequence of the batch, leaves every earlier output bit-identical."""
     nb, s, h, dq, dv = 2, 96, 2, 64, 128
