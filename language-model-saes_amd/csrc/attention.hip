@@ -223,7 +223,7 @@ __device__ __forceinline__ void att_store_transposed(uint16_t *__restrict__ dst,
 template <int DQK, int DV>
 __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
     const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, uint16_t *__restrict__ out,
-    float *__restrict__ lse, int seq, int n_heads, int n_batch, int64_t T, float sc2) {
+    float *__restrict__ lse, int seq, int n_heads, int n_batch, float sc2) {
   constexpr int KRB = DQK * 2;                                    // bytes of a key row
   constexpr int VRB = DV * 2;
   constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + V_BYTES;
@@ -657,7 +657,7 @@ static int launch_fwd(const void *q, const void *k, const void *v, int64_t n_bat
                       void *out, float *lse, hipStream_t st) {
   const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)v, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch, n_batch * seq,
+                     (const uint16_t *)v, (uint16_t *)out, lse, (int)seq, (int)n_heads, (int)n_batch,
                      (float)(scale * 1.4426950408889634));
   return check_launch("attention_fwd");
 }
