@@ -395,6 +395,13 @@ int sae_transpose_to_bf16(const void *src, int src_dtype, const float *mask, int
 int sae_code_to_dense(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
                       int64_t n_cols, float *dense_f32, void *dense_bf16, void *stream);
 
+/* The same matrix transposed and in bf16: dense_t_bf16 [n_cols, B] (cleared, then token b's entries written down column
+ * b).  The left operand of a dense weight-gradient product over the token axis, dW_D = acts^T grad_recon: what autograd
+ * forms for `feature_acts @ W_O` (models/lorsa.py:765-782), and cheaper than gathered gradient rows when the dictionary
+ * is small against the batch (d_sae / k below a few hundred). */
+int sae_code_to_dense_t(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
+                        int64_t n_cols, void *dense_t_bf16, void *stream);
+
 /* ---- Dense feature activations -> sparse code ----------------------------------------------------------------
  * The conversion in front of the sparse decoder kernels when a caller hands over a dense [B, F] activation matrix
  * (fp32 or bf16): get_sparse_representation (kernels/kernels.py:14-58: nonzero, bincount, cumsum, scatter into a padded

@@ -165,6 +165,7 @@ class _SparseTail(torch.autograd.Function):
         holder["code"] = code
         ctx.code, ctx.grad_recon, ctx.dval = code, grad_recon, dval
         ctx.amp = bool(amp)
+        ctx.dense_decoder_grad = bool(getattr(m, "dense_decoder_grad", True))
         ctx.defer_to = m if holder.get("defer") else None
         ctx.has_b_D = b_D is not None
         ctx.in_dtype = hidden_pre.dtype
@@ -176,9 +177,23 @@ class _SparseTail(torch.autograd.Function):
         code = ctx.code
         T, F = code.n_tokens, code.d_sae
         g = g_loss.to(torch.float32)
-        fi = ops.build_feature_index(code)
         m = ctx.defer_to
-        if m is not None and m.W_O.grad is None and getattr(m.W_O, "_sparse_grad", None) is None:
+        d_model = ctx.grad_recon.shape[1]
+        # A dictionary that is small against the batch (d_sae / k of a few hundred at most) gets its decoder gradient as
+        # the dense product acts^T grad_recon on the matrix cores, what autograd forms for `feature_acts @ W_O` under
+        # autocast: gathered gradient rows cost T k d_model bytes of gathers plus a feature index, the product T F d_model
+        # flop (16 x 1024 tokens, 8192 features, k = 64: 0.84 ms of index + row pass against ~0.45 ms)
+        if ctx.amp and ctx.dense_decoder_grad and T % 64 == 0 and d_model % 8 == 0 and F * T <= 400 * code.n_slots:
+            import dataclasses
+            acts_t = ops.code_to_dense_t(dataclasses.replace(code, val=code.val * g), F)           # [F, T] bf16
+            gd_t = ops.transpose_to_bf16(ctx.grad_recon.contiguous())[0]                          # [d, T] bf16
+            dW_O = ops.encoder_gemm(acts_t, gd_t, torch.float32)                                  # [F, d]
+            fi = None
+        else:
+            fi = ops.build_feature_index(code)
+        if fi is None:
+            pass
+        elif m is not None and m.W_O.grad is None and getattr(m.W_O, "_sparse_grad", None) is None:
             # the optimiser rebuilds the rows where it consumes them (under autocast from the bf16-rounded output
             # gradient, as the backward of an autocast matmul pairs them)
             gd = ops.cast_bf16(ctx.grad_recon.contiguous()) if ctx.amp else ctx.grad_recon
@@ -221,6 +236,8 @@ class LowRankSparseAttention(SparseDictionary):
         self.defer_weight_grads = False
         # False sends projections and attention mixing to the torch library routines in every configuration
         self.use_mix_kernels = True
+        # False keeps W_O's gradient in factored form (feature index + gathered rows) whatever the shape
+        self.dense_decoder_grad = True
         self.register_buffer("mask", torch.tril(torch.ones((cfg.n_ctx, cfg.n_ctx), device=cfg.device).bool()))
         self.register_buffer("IGNORE", torch.tensor(-torch.inf, device=cfg.device))
         if cfg.use_post_qk_ln:

@@ -207,6 +207,17 @@ def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_b
     return f32, b16
 
 
+def code_to_dense_t(code: "SparseCode", n_cols: int) -> torch.Tensor:
+    """bf16 [n_cols, n_tokens]: the dense matrix of a sparse code, transposed (the left operand of a product over tokens)."""
+    B = code.n_tokens
+    out = torch.empty(int(n_cols), B, dtype=torch.bfloat16, device=code.val.device)
+    with _timed("code_to_dense_t"):
+        check(_lib.load().sae_code_to_dense_t(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
+                                              code.row_nnz.data_ptr(), B, int(n_cols), out.data_ptr(), _stream(code.val)),
+              "code_to_dense_t")
+    return out
+
+
 def dense_row_nnz(dense: torch.Tensor) -> torch.Tensor:
     """int32 [B]: the number of non-zero entries of every row of a dense [B, F] matrix (fp32 or bf16)."""
     _req(dense, "dense", ndim=2)

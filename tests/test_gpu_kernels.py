@@ -709,3 +709,20 @@ def test_sparse_decode_fused_accumulates_value_gradients_and_writes_in_place(pkg
         assert r.data_ptr() == recon[j].data_ptr() and dv.data_ptr() == acc.data_ptr()
         assert torch.equal(gr, sep[j][2]) and torch.equal(recon[j], sep[j][0]) and torch.equal(loss[j], sep[j][1])
     assert torch.equal(acc, sep[0][3] + sep[1][3])
+
+
+def test_code_to_dense_transposed(pkg, dev):
+    """sae_code_to_dense_t: the dense matrix of a sparse code, transposed, in bf16; ragged and empty rows."""
+    g = torch.Generator().manual_seed(5)
+    B, F, k = 70, 333, 9
+    idx = torch.stack([torch.randperm(F, generator=g)[:k].sort().values for _ in range(B)]).to(torch.int32)
+    val = torch.randn(B, k, generator=g)
+    nnz = torch.randint(0, k + 1, (B,), generator=g).to(torch.int32)
+    nnz[3] = 0
+    code = pkg.ops.SparseCode(idx.reshape(-1).to(dev), val.reshape(-1).to(dev), (torch.arange(B) * k).to(dev), nnz.to(dev), B, F)
+    want = torch.zeros(B, F)
+    for r in range(B):
+        want[r, idx[r, : nnz[r]].long()] = val[r, : nnz[r]]
+    got = pkg.ops.code_to_dense_t(code, F)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (F, B)
+    assert torch.equal(got.cpu(), want.t().to(torch.bfloat16))

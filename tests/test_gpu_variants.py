@@ -379,13 +379,16 @@ def test_lorsa_fused_step_fp32(pkg, vo, dev, kw):
     check_grads(m, ref)
 
 
-@pytest.mark.parametrize("d,F,h,dq,s,b", [(64, 512, 4, 32, 32, 2),      # value width 128, one block
-                                          (64, 256, 4, 64, 96, 2),      # width 64 / 64, a ragged second block
-                                          (128, 256, 8, 32, 64, 3)])    # value width 32
-def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b):
-    """bf16 autocast: projections on the GEMM kernel, causal mixing and its backward on the attention kernels."""
+@pytest.mark.parametrize("d,F,h,dq,s,b,dense", [(64, 512, 4, 32, 32, 2, True),      # value width 128, one block
+                                                (64, 256, 4, 64, 96, 2, True),      # width 64 / 64, a ragged second block
+                                                (128, 256, 8, 32, 64, 3, True),     # value width 32
+                                                (64, 512, 4, 32, 32, 2, False)])    # W_O's gradient as gathered rows
+def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b, dense):
+    """bf16 autocast: projections on the GEMM kernel, causal mixing and its backward on the attention kernels; W_O's
+    gradient as the dense product acts^T grad_recon or as gathered rows."""
     k = 8
     m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=53, positional_embedding_type="none")
+    m.dense_decoder_grad = dense
     g = torch.Generator().manual_seed(54)
     with torch.no_grad():      # non-zero projection biases, so that the kernels' bias path is exercised
         for n in ("b_Q", "b_K", "b_V"):
@@ -397,11 +400,12 @@ def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b):
     pkg.ops.set_kernel_timer(timer)
     with torch.autocast("cuda", dtype=torch.bfloat16):
         out = m.compute_loss(gb)
-    pkg.ops.set_kernel_timer(None)
     assert "attention_fwd" in timer.records, "the attention kernel did not run"
     want = ref.compute_loss(batch)
     assert rel_err(out["loss"], want["loss"]) < BF16_TOL
     out["loss"].backward()
+    pkg.ops.set_kernel_timer(None)
+    assert ("code_to_dense_t" in timer.records) == dense
     kept = (out["feature_acts"] > 0).cpu()
     w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch), kept)
     assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["hidden_pre"], w16["hidden_pre"]) < BF16_TOL
