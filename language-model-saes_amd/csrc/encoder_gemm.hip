@@ -652,6 +652,25 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
                                : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
 }
 
+extern "C" int sae_encoder_gemm_grouped(const void *x_bf16, const void *w_t_bf16, void *out, int64_t n_groups, int64_t B, int64_t d,
+                                        int64_t F, int out_dtype, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x_bf16 && w_t_bf16 && out, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0 && n_groups > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: sizes must be positive");
+  SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: bad out_dtype %d", out_dtype);
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28) && n_groups <= 65535, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_grouped: size too large");
+  SAE_REQUIRE(d % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_grouped: d_model=%lld must be a multiple of 64", (long long)d);
+  SAE_REQUIRE((B * F * (out_dtype == SAE_BF16 ? 2 : 4)) % 16 == 0, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_grouped: a group's output must be a multiple of 16 bytes");
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_t_bf16 | (uintptr_t)out) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "encoder_gemm_grouped: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  return out_dtype == SAE_BF16
+             ? launch_gemm_bf16<true, EPI_NONE>(x_bf16, w_t_bf16, out, B, d, F, nullptr, nullptr, nullptr, st, n_groups)
+             : launch_gemm_bf16<false, EPI_NONE>(x_bf16, w_t_bf16, out, B, d, F, nullptr, nullptr, nullptr, st, n_groups);
+}
+
 extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups,
                                             int64_t B, int64_t d, int64_t F, const float *b_enc, const float *scale,
                                             uint32_t *granule_max, void *stream) {

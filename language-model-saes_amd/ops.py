@@ -207,13 +207,17 @@ def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_b
     return f32, b16
 
 
-def code_to_dense_t(code: "SparseCode", n_cols: int) -> torch.Tensor:
-    """bf16 [n_cols, n_tokens]: the dense matrix of a sparse code, transposed (the left operand of a product over tokens)."""
-    B = code.n_tokens
-    out = torch.empty(int(n_cols), B, dtype=torch.bfloat16, device=code.val.device)
+def code_to_dense_t(code: "SparseCode", n_cols: int, token_groups: int = 1) -> torch.Tensor:
+    """bf16 [n_cols, n_tokens]: the dense matrix of a sparse code, transposed (the left operand of a product over tokens).
+    With `token_groups` = G > 1 the token axis is cut into G runs, each a matrix of its own: [G, n_cols, n_tokens / G]."""
+    B, G = code.n_tokens, int(token_groups)
+    if G < 1 or B % G:
+        raise ValueError(f"{B} tokens do not split into {G} groups")
+    shape = (int(n_cols), B) if G == 1 else (G, int(n_cols), B // G)
+    out = torch.empty(*shape, dtype=torch.bfloat16, device=code.val.device)
     with _timed("code_to_dense_t"):
         check(_lib.load().sae_code_to_dense_t(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
-                                              code.row_nnz.data_ptr(), B, int(n_cols), out.data_ptr(), _stream(code.val)),
+                                              code.row_nnz.data_ptr(), B, int(n_cols), G, out.data_ptr(), _stream(code.val)),
               "code_to_dense_t")
     return out
 
@@ -297,6 +301,21 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
             "encoder_gemm",
         )
     return pre
+
+
+def encoder_gemm_grouped(x: torch.Tensor, w_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[g] = x[g] @ w_t[g]^T for bf16 x [G, B, d], w_t [G, F, d] -> [G, B, F], one launch."""
+    _req(x, "x", torch.bfloat16, 3)
+    _req(w_t, "w_t", torch.bfloat16, 3)
+    G, B, d = x.shape
+    G2, F, d2 = w_t.shape
+    if G != G2 or d != d2:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_t {tuple(w_t.shape)}")
+    out = torch.empty(G, B, F, dtype=out_dtype, device=x.device)
+    with _timed("encoder_gemm"):
+        check(_lib.load().sae_encoder_gemm_grouped(x.data_ptr(), w_t.data_ptr(), out.data_ptr(), G, B, d, F, _dt(out), _stream(x)),
+              "encoder_gemm_grouped")
+    return out
 
 
 def encoder_gemm_bias(x: torch.Tensor, w_t: torch.Tensor, col_bias: Optional[torch.Tensor] = None,

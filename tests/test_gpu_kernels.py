@@ -726,3 +726,19 @@ def test_code_to_dense_transposed(pkg, dev):
     got = pkg.ops.code_to_dense_t(code, F)
     assert got.dtype == torch.bfloat16 and tuple(got.shape) == (F, B)
     assert torch.equal(got.cpu(), want.t().to(torch.bfloat16))
+    # the token axis cut into runs, each a matrix of its own
+    for G in (2, 5, 7):
+        got = pkg.ops.code_to_dense_t(code, F, G)
+        assert tuple(got.shape) == (G, F, B // G)
+        assert torch.equal(got.cpu(), want.view(G, B // G, F).transpose(1, 2).to(torch.bfloat16))
+
+
+def test_encoder_gemm_grouped_equals_separate_products(pkg, dev):
+    g = torch.Generator().manual_seed(8)
+    G, B, d, F = 3, 200, 128, 300
+    x = torch.randn(G, B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = torch.randn(G, F, d, generator=g).to(torch.bfloat16).to(dev)
+    for dt in (torch.float32, torch.bfloat16):
+        got = pkg.ops.encoder_gemm_grouped(x, w, dt)
+        for i in range(G):
+            assert torch.equal(got[i], pkg.ops.encoder_gemm(x[i], w[i], dt))
