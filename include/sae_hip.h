@@ -93,12 +93,12 @@ int sae_col_sum_static(const float *src, float *out, int64_t B, int64_t n, int a
 int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, int64_t B, int64_t d, int64_t F,
                      int in_dtype, int out_dtype, void *stream);
 
-/* n_groups independent products of one shape in one launch, bf16 operands, every array stacked group after group:
- * x [G, B, d], w_t [G, F, d], out [G, B, F] (fp32 or bf16).  The per-layer products of models/clt.py:232-387 without an
- * epilogue, and the halves of a product over a long contraction axis whose few output tiles would leave most of the
- * chip idle (the caller sums the per-group results). */
-int sae_encoder_gemm_grouped(const void *x_bf16, const void *w_t_bf16, void *out, int64_t n_groups, int64_t B, int64_t d,
-                             int64_t F, int out_dtype, void *stream);
+/* Split-K form of sae_encoder_gemm for bf16 operands: slice s of the contraction axis (d / n_splits elements of every
+ * row) gives partials[s] (fp32 [n_splits, B, F]); their sum, which the caller forms in slice order, is the product.  For
+ * products with few output tiles and a long contraction (weight gradients over the token axis of a small dictionary),
+ * which would otherwise occupy a fraction of the chip.  d % (64 n_splits) == 0. */
+int sae_encoder_gemm_split_k(const void *x_bf16, const void *w_t_bf16, float *partials, int64_t n_splits, int64_t B, int64_t d,
+                             int64_t F, void *stream);
 
 /* ---- activation select ------------------------------------------------------------ */
 
@@ -402,14 +402,12 @@ int sae_transpose_to_bf16(const void *src, int src_dtype, const float *mask, int
 int sae_code_to_dense(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
                       int64_t n_cols, float *dense_f32, void *dense_bf16, void *stream);
 
-/* The same matrix transposed and in bf16: dense_t_bf16 [n_token_groups, n_cols, B / n_token_groups] (cleared, then token b's
- * entries written down column b % (B / groups) of matrix b / (B / groups); one group: [n_cols, B]).  The left operand of a
- * dense weight-gradient product over the token axis, dW_D = acts^T grad_recon: what autograd forms for
- * `feature_acts @ W_O` (models/lorsa.py:765-782), and cheaper than gathered gradient rows when the dictionary is small
- * against the batch (d_sae / k below a few hundred).  Token groups are the operands of sae_encoder_gemm_grouped, whose
- * per-group results the caller sums (a product with few output tiles then fills more of the chip). */
+/* The same matrix transposed and in bf16: dense_t_bf16 [n_cols, B] (cleared, then token b's entries written down column
+ * b).  The left operand of a dense weight-gradient product over the token axis, dW_D = acts^T grad_recon: what autograd
+ * forms for `feature_acts @ W_O` (models/lorsa.py:765-782), and cheaper than gathered gradient rows when the dictionary
+ * is small against the batch (d_sae / k below a few hundred). */
 int sae_code_to_dense_t(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz, int64_t B,
-                        int64_t n_cols, int64_t n_token_groups, void *dense_t_bf16, void *stream);
+                        int64_t n_cols, void *dense_t_bf16, void *stream);
 
 /* ---- Dense feature activations -> sparse code ----------------------------------------------------------------
  * The conversion in front of the sparse decoder kernels when a caller hands over a dense [B, F] activation matrix

@@ -284,21 +284,18 @@ __global__ __launch_bounds__(256) void code_to_dense_kernel(const int32_t *__res
   }
 }
 
-// The same matrix transposed, in bf16 (cleared beforehand): one wave per token scatters the token's entries down its
-// column.  The left operand of a product over the token axis (a dense weight gradient acts^T g).  The token axis may be
-// cut into groups of `per_group` tokens, each a matrix [n_cols, per_group] of its own, stacked group after group: the
-// operands of a grouped product whose partial results are then summed (split-K).
+// The same matrix transposed, [n_cols, B] in bf16 (cleared beforehand): one wave per token scatters the token's entries
+// down its column.  The left operand of a product over the token axis (a dense weight gradient acts^T g).
 __global__ __launch_bounds__(64) void code_to_dense_t_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
                                                              const int64_t *__restrict__ row_off,
-                                                             const int32_t *__restrict__ row_nnz, int64_t per_group,
-                                                             int64_t n_cols, uint16_t *__restrict__ out_t) {
+                                                             const int32_t *__restrict__ row_nnz, int64_t B, int64_t n_cols,
+                                                             uint16_t *__restrict__ out_t) {
   const int64_t b = blockIdx.x;
   const int64_t off = row_off[b];
   const int n = row_nnz[b];
-  uint16_t *col = out_t + (b / per_group) * n_cols * per_group + (b % per_group);
   for (int s = threadIdx.x; s < n; s += 64) {
     const int64_t j = idx[off + s];
-    if (j >= 0 && j < n_cols) col[j * per_group] = f32_to_bf16_bits(val[off + s]);
+    if (j >= 0 && j < n_cols) out_t[j * B + b] = f32_to_bf16_bits(val[off + s]);
   }
 }
 
@@ -414,16 +411,14 @@ extern "C" int sae_code_to_dense(const int32_t *idx, const float *val, const int
 }
 
 extern "C" int sae_code_to_dense_t(const int32_t *idx, const float *val, const int64_t *row_off, const int32_t *row_nnz,
-                                   int64_t B, int64_t n_cols, int64_t n_token_groups, void *dense_t_bf16, void *stream) {
+                                   int64_t B, int64_t n_cols, void *dense_t_bf16, void *stream) {
   using namespace sae;
   SAE_REQUIRE(idx && val && row_off && row_nnz && dense_t_bf16, SAE_ERR_INVALID_ARG, "code_to_dense_t: null pointer");
   SAE_REQUIRE(B > 0 && n_cols > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "code_to_dense_t: bad shape");
-  SAE_REQUIRE(n_token_groups > 0 && B % n_token_groups == 0, SAE_ERR_INVALID_ARG,
-              "code_to_dense_t: %lld tokens do not split into %lld groups", (long long)B, (long long)n_token_groups);
   const int rc = zero_fill(dense_t_bf16, (size_t)B * (size_t)n_cols * 2, (hipStream_t)stream);
   if (rc) return rc;
-  hipLaunchKernelGGL(code_to_dense_t_kernel, dim3((unsigned)B), dim3(64), 0, (hipStream_t)stream, idx, val, row_off, row_nnz,
-                     B / n_token_groups, n_cols, reinterpret_cast<uint16_t *>(dense_t_bf16));
+  hipLaunchKernelGGL(code_to_dense_t_kernel, dim3((unsigned)B), dim3(64), 0, (hipStream_t)stream, idx, val, row_off, row_nnz, B,
+                     n_cols, reinterpret_cast<uint16_t *>(dense_t_bf16));
   return check_launch("code_to_dense_t");
 }
 

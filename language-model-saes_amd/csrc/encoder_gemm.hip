@@ -306,13 +306,21 @@ constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2, EPI_MARGIN = 3;
 template <bool BF16_OUT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
-    int row_bytes /* d * 2 */, int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
+    int row_bytes /* contraction length * 2 */, int pitch_bytes /* bytes between operand rows */, int tiles_m, int tiles_n,
+    int rm_log2, const float *__restrict__ b_enc,
     const float *__restrict__ scale, uint32_t *__restrict__ gmax, const float *__restrict__ theta) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
-  if (blockIdx.y) {      // group g of a batch of independent products of one shape, each operand stacked group after group
+  if (blockIdx.y) {
+    // group g of a batch of independent products of one shape, each operand stacked group after group; or, when the rows
+    // are longer than the contraction, slice g of the contraction axis (split-K: the caller sums the groups' outputs)
     const size_t g = blockIdx.y;
-    x += g * (size_t)M * row_bytes;
-    w += g * (size_t)N * row_bytes;
+    if (pitch_bytes != row_bytes) {
+      x += g * (size_t)row_bytes;
+      w += g * (size_t)row_bytes;
+    } else {
+      x += g * (size_t)M * row_bytes;
+      w += g * (size_t)N * row_bytes;
+    }
     out = reinterpret_cast<char *>(out) + g * (size_t)M * N * (BF16_OUT ? 2 : 4);
     if constexpr (EPI == EPI_GMAX || EPI == EPI_MARGIN) {
       if (b_enc) b_enc += g * (size_t)N;
@@ -352,8 +360,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
   for (int i = 0; i < 4; ++i) {
     const int r = wave * 32 + i * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-    xg[i] = x + (size_t)(m0 + r < M ? m0 + r : M - 1) * row_bytes + chunk * 16;
-    wg[i] = w + (size_t)(n0 + r < N ? n0 + r : N - 1) * row_bytes + chunk * 16;
+    xg[i] = x + (size_t)(m0 + r < M ? m0 + r : M - 1) * pitch_bytes + chunk * 16;
+    wg[i] = w + (size_t)(n0 + r < N ? n0 + r : N - 1) * pitch_bytes + chunk * 16;
   }
   const uint32_t ld_base = (uint32_t)(wave * 32) * GEMM_SLAB;
 
@@ -611,7 +619,8 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
 template <bool BF16_OUT, int EPI>
 static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
                             const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1,
-                            const float *theta = nullptr) {
+                            const float *theta = nullptr, int64_t split_k = 1) {
+  // split_k > 1: d is the length of one slice of rows that are split_k * d long; the slices are the launch's groups
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
   auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
@@ -622,9 +631,9 @@ static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, 
   const int ro_log2 = tiles_o >= 8 ? 3 : (tiles_o > 2 ? 2 : (tiles_o > 1 ? 1 : 0)), ro = 1 << ro_log2, rs = 32 >> ro_log2;
   const int rm_log2 = deal_m ? -ro_log2 - 1 : ro_log2;
   const int m_pad = (tiles_o + ro - 1) / ro * ro, n_local_pad = ((tiles_s + 7) / 8 + rs - 1) / rs * rs;
-  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)n_groups), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st,
-                     (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2), tiles_m, tiles_n, rm_log2, b_enc, scale,
-                     gmax, theta);
+  hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)(split_k > 1 ? split_k : n_groups)), dim3(GEMM_THREADS),
+                     GEMM_LDS_BYTES, st, (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2),
+                     (int)(d * 2 * (split_k > 1 ? split_k : 1)), tiles_m, tiles_n, rm_log2, b_enc, scale, gmax, theta);
   return check_launch("encoder_gemm");
 }
 
@@ -652,23 +661,20 @@ extern "C" int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, i
                                : launch_gemm_f32<false>(x, w_enc_t, pre, B, d, F, st);
 }
 
-extern "C" int sae_encoder_gemm_grouped(const void *x_bf16, const void *w_t_bf16, void *out, int64_t n_groups, int64_t B, int64_t d,
-                                        int64_t F, int out_dtype, void *stream) {
+extern "C" int sae_encoder_gemm_split_k(const void *x_bf16, const void *w_t_bf16, float *partials, int64_t n_splits, int64_t B,
+                                        int64_t d, int64_t F, void *stream) {
   using namespace sae;
-  SAE_REQUIRE(x_bf16 && w_t_bf16 && out, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: null pointer");
-  SAE_REQUIRE(B > 0 && d > 0 && F > 0 && n_groups > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: sizes must be positive");
-  SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "encoder_gemm_grouped: bad out_dtype %d", out_dtype);
-  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28) && n_groups <= 65535, SAE_ERR_UNSUPPORTED,
-              "encoder_gemm_grouped: size too large");
-  SAE_REQUIRE(d % 64 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_grouped: d_model=%lld must be a multiple of 64", (long long)d);
-  SAE_REQUIRE((B * F * (out_dtype == SAE_BF16 ? 2 : 4)) % 16 == 0, SAE_ERR_UNSUPPORTED,
-              "encoder_gemm_grouped: a group's output must be a multiple of 16 bytes");
-  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_t_bf16 | (uintptr_t)out) & 15) == 0, SAE_ERR_INVALID_ARG,
-              "encoder_gemm_grouped: pointers must be 16-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
-  return out_dtype == SAE_BF16
-             ? launch_gemm_bf16<true, EPI_NONE>(x_bf16, w_t_bf16, out, B, d, F, nullptr, nullptr, nullptr, st, n_groups)
-             : launch_gemm_bf16<false, EPI_NONE>(x_bf16, w_t_bf16, out, B, d, F, nullptr, nullptr, nullptr, st, n_groups);
+  SAE_REQUIRE(x_bf16 && w_t_bf16 && partials, SAE_ERR_INVALID_ARG, "encoder_gemm_split_k: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0 && n_splits > 1, SAE_ERR_INVALID_ARG, "encoder_gemm_split_k: sizes must be positive, n_splits > 1");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28) && n_splits <= 64, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_split_k: size too large");
+  SAE_REQUIRE(d % (64 * n_splits) == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_split_k: d=%lld must be a multiple of 64 * n_splits",
+              (long long)d);
+  SAE_REQUIRE((B * F * 4) % 16 == 0, SAE_ERR_UNSUPPORTED, "encoder_gemm_split_k: a slice's output must be a multiple of 16 bytes");
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_t_bf16 | (uintptr_t)partials) & 15) == 0, SAE_ERR_INVALID_ARG,
+              "encoder_gemm_split_k: pointers must be 16-byte aligned");
+  return launch_gemm_bf16<false, EPI_NONE>(x_bf16, w_t_bf16, partials, B, d / n_splits, F, nullptr, nullptr, nullptr,
+                                           (hipStream_t)stream, 1, nullptr, n_splits);
 }
 
 extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups,

@@ -185,16 +185,9 @@ class _SparseTail(torch.autograd.Function):
         # flop (16 x 1024 tokens, 8192 features, k = 64: 0.84 ms of index + row pass against ~0.45 ms)
         if ctx.amp and ctx.dense_decoder_grad and T % 64 == 0 and d_model % 8 == 0 and F * T <= 400 * code.n_slots:
             import dataclasses
-            # F / 256 x d / 256 output tiles are few (96 at 8192 x 768): the token axis is cut in two and the halves' products
-            # run as one grouped launch, then are summed
-            G = 2 if T % 128 == 0 and (F // 256) * ((d_model + 255) // 256) <= 128 else 1
-            acts_t = ops.code_to_dense_t(dataclasses.replace(code, val=code.val * g), F, G)        # [G, F, T / G] bf16
-            gr = ctx.grad_recon.contiguous()
-            if G == 1:
-                dW_O = ops.encoder_gemm(acts_t, ops.transpose_to_bf16(gr)[0], torch.float32)       # [F, d]
-            else:
-                gd_t = torch.stack([ops.transpose_to_bf16(h)[0] for h in gr.view(G, T // G, d_model)])   # [G, d, T / G]
-                dW_O = ops.encoder_gemm_grouped(acts_t, gd_t, torch.float32).sum(0)
+            acts_t = ops.code_to_dense_t(dataclasses.replace(code, val=code.val * g), F)           # [F, T] bf16
+            gd_t = ops.transpose_to_bf16(ctx.grad_recon.contiguous())[0]                          # [d, T] bf16
+            dW_O = ops.encoder_gemm(acts_t, gd_t, torch.float32)        # [F, d]; few output tiles: the product splits its K
             fi = None
         else:
             fi = ops.build_feature_index(code)

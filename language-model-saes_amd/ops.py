@@ -207,17 +207,13 @@ def code_to_dense(code: "SparseCode", n_cols: int, want_f32: bool = True, want_b
     return f32, b16
 
 
-def code_to_dense_t(code: "SparseCode", n_cols: int, token_groups: int = 1) -> torch.Tensor:
-    """bf16 [n_cols, n_tokens]: the dense matrix of a sparse code, transposed (the left operand of a product over tokens).
-    With `token_groups` = G > 1 the token axis is cut into G runs, each a matrix of its own: [G, n_cols, n_tokens / G]."""
-    B, G = code.n_tokens, int(token_groups)
-    if G < 1 or B % G:
-        raise ValueError(f"{B} tokens do not split into {G} groups")
-    shape = (int(n_cols), B) if G == 1 else (G, int(n_cols), B // G)
-    out = torch.empty(*shape, dtype=torch.bfloat16, device=code.val.device)
+def code_to_dense_t(code: "SparseCode", n_cols: int) -> torch.Tensor:
+    """bf16 [n_cols, n_tokens]: the dense matrix of a sparse code, transposed (the left operand of a product over tokens)."""
+    B = code.n_tokens
+    out = torch.empty(int(n_cols), B, dtype=torch.bfloat16, device=code.val.device)
     with _timed("code_to_dense_t"):
         check(_lib.load().sae_code_to_dense_t(code.idx.data_ptr(), code.val.data_ptr(), code.row_off.data_ptr(),
-                                              code.row_nnz.data_ptr(), B, int(n_cols), G, out.data_ptr(), _stream(code.val)),
+                                              code.row_nnz.data_ptr(), B, int(n_cols), out.data_ptr(), _stream(code.val)),
               "code_to_dense_t")
     return out
 
@@ -294,6 +290,13 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     F, d2 = w_enc_t.shape
     if d != d2:
         raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
+    splits = gemm_split_k(B, d, F) if (x.dtype == torch.bfloat16 and out_dtype == torch.float32) else 1
+    if splits > 1:
+        partials = torch.empty(splits, B, F, dtype=torch.float32, device=x.device)
+        with _timed("encoder_gemm"):
+            check(_lib.load().sae_encoder_gemm_split_k(x.data_ptr(), w_enc_t.data_ptr(), partials.data_ptr(), splits, B, d, F,
+                                                       _stream(x)), "encoder_gemm_split_k")
+        return partials.sum(0)
     pre = torch.empty(B, F, dtype=out_dtype, device=x.device)
     with _timed("encoder_gemm"):
         check(
@@ -303,19 +306,18 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     return pre
 
 
-def encoder_gemm_grouped(x: torch.Tensor, w_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """out[g] = x[g] @ w_t[g]^T for bf16 x [G, B, d], w_t [G, F, d] -> [G, B, F], one launch."""
-    _req(x, "x", torch.bfloat16, 3)
-    _req(w_t, "w_t", torch.bfloat16, 3)
-    G, B, d = x.shape
-    G2, F, d2 = w_t.shape
-    if G != G2 or d != d2:
-        raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_t {tuple(w_t.shape)}")
-    out = torch.empty(G, B, F, dtype=out_dtype, device=x.device)
-    with _timed("encoder_gemm"):
-        check(_lib.load().sae_encoder_gemm_grouped(x.data_ptr(), w_t.data_ptr(), out.data_ptr(), G, B, d, F, _dt(out), _stream(x)),
-              "encoder_gemm_grouped")
-    return out
+def gemm_split_k(B: int, d: int, F: int) -> int:
+    """How many slices of the contraction axis a bf16 -> fp32 product [B, d] x [F, d]^T is cut into: products with few
+    256 x 256 output tiles and a long contraction (weight gradients over the token axis) would occupy a fraction of the
+    256 CUs; slices run as one launch and their fp32 results are summed in slice order (deterministic, and the same for
+    every caller of a shape).  1: no split."""
+    tiles = ((B + 255) // 256) * ((F + 255) // 256)
+    if tiles > 128 or d < 4096:
+        return 1
+    for g in (4, 3, 2):
+        if tiles * g <= 256 and d % (64 * g) == 0 and d // g >= 2048:
+            return g
+    return 1
 
 
 def encoder_gemm_bias(x: torch.Tensor, w_t: torch.Tensor, col_bias: Optional[torch.Tensor] = None,

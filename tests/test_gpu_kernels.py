@@ -726,19 +726,21 @@ def test_code_to_dense_transposed(pkg, dev):
     got = pkg.ops.code_to_dense_t(code, F)
     assert got.dtype == torch.bfloat16 and tuple(got.shape) == (F, B)
     assert torch.equal(got.cpu(), want.t().to(torch.bfloat16))
-    # the token axis cut into runs, each a matrix of its own
-    for G in (2, 5, 7):
-        got = pkg.ops.code_to_dense_t(code, F, G)
-        assert tuple(got.shape) == (G, F, B // G)
-        assert torch.equal(got.cpu(), want.view(G, B // G, F).transpose(1, 2).to(torch.bfloat16))
 
 
-def test_encoder_gemm_grouped_equals_separate_products(pkg, dev):
-    g = torch.Generator().manual_seed(8)
-    G, B, d, F = 3, 200, 128, 300
-    x = torch.randn(G, B, d, generator=g).to(torch.bfloat16).to(dev)
-    w = torch.randn(G, F, d, generator=g).to(torch.bfloat16).to(dev)
-    for dt in (torch.float32, torch.bfloat16):
-        got = pkg.ops.encoder_gemm_grouped(x, w, dt)
-        for i in range(G):
-            assert torch.equal(got[i], pkg.ops.encoder_gemm(x[i], w[i], dt))
+def test_encoder_gemm_split_k(pkg, dev):
+    """A bf16 -> fp32 product with few output tiles and a long contraction is cut along K: the slices' fp32 results summed
+    in slice order equal the sum of the separately computed slice products bit for bit, and the product within fp32
+    summation error of the unsplit kernel."""
+    g = torch.Generator().manual_seed(9)
+    B, d, F = 300, 8192, 520
+    G = pkg.ops.gemm_split_k(B, d, F)
+    assert G == 4 and pkg.ops.gemm_split_k(4096, 4096, 131072) == 1 and pkg.ops.gemm_split_k(300, 1024, 520) == 1
+    x = torch.randn(B, d, generator=g).to(torch.bfloat16).to(dev)
+    w = torch.randn(F, d, generator=g).to(torch.bfloat16).to(dev)
+    got = pkg.ops.encoder_gemm(x, w, torch.float32)
+    parts = [pkg.ops.encoder_gemm(x[:, i * d // G:(i + 1) * d // G].contiguous(), w[:, i * d // G:(i + 1) * d // G].contiguous(),
+                                  torch.float32) for i in range(G)]
+    assert torch.equal(got, torch.stack(parts).sum(0))
+    want = x.double() @ w.double().t()
+    assert ((got.double() - want).abs().max() / want.abs().max()).item() < 1e-5
