@@ -433,3 +433,33 @@ def test_lorsa_adam_steps_with_factored_output_gradient(pkg, vo, dev):
             q = rp[n].detach()
             assert (p.detach().cpu() - q).abs().max() <= 5e-2 * 1e-3 * (step + 1) + 1e-6 * q.abs().max(), (step, n)
     assert torch.allclose(m._decoder_norm_nograd().cpu(), m.W_O.detach().norm(dim=1).cpu(), rtol=1e-5)
+
+
+def test_lorsa_adam_steps_under_autocast_with_the_dense_output_gradient(pkg, vo, dev):
+    """bf16 autocast with HipAdam attached: the mixing runs on the attention kernels and W_O's gradient is the dense product
+    acts^T grad_recon, which the optimiser takes as an ordinary gradient; after every step the cached bf16 copy of W_O and
+    its row norms are those of the updated parameter, and three steps leave the loss where the same steps leave it with
+    the gradient in gathered-row form."""
+    d, F, h, dq, s, b, k = 64, 512, 4, 32, 32, 2, 8
+    losses = {}
+    for dense in (True, False):
+        m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=57, positional_embedding_type="none")
+        m.dense_decoder_grad = dense
+        g = torch.Generator().manual_seed(58)
+        batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+        gb = {k_: v.to(dev) for k_, v in batch.items()}
+        opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m)
+        seen = []
+        for step in range(3):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                out = m.compute_loss(gb)
+            out["loss"].backward()
+            assert (m.W_O.grad is not None) == dense
+            opt.step(); opt.zero_grad()
+            seen.append(out["loss"].item())
+            assert torch.equal(m._w_dec_operand(True), m.W_O.detach().to(torch.bfloat16)), step
+            assert torch.allclose(m._decoder_norm_nograd(), m.W_O.detach().norm(dim=1), rtol=1e-5), step
+        losses[dense] = seen
+    assert seen[2] < seen[0]
+    for a, c in zip(losses[True], losses[False]):
+        assert abs(a - c) <= 2e-2 * abs(c)
