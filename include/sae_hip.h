@@ -171,6 +171,16 @@ int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_
                                   int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
                                   int64_t workspace_bytes, void *stream);
 
+/* sae_select_topk_batch for a dictionary whose dtype is bfloat16 (config.py:39), as sae_select_topk_row_lowp is to
+ * sae_select_topk_row: pre is bf16, and the sum with the bias, the product with the scale and the final quotient are each
+ * rounded to bf16, as the bf16 tensors around the reference's batch_topk closure are (models/sae.py:324-341,
+ * models/sparse_dictionary.py:761-794).  b_enc / scale are fp32 copies of the bf16 bias / norms.  Many keys then share
+ * the threshold's value; ties keep the lowest flattened indices b * F + f.  No feat_mask.  Same workspace. */
+int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
+                               int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val, int64_t capacity,
+                               int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
+                               int64_t workspace_bytes, void *stream);
+
 /* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product
  * (Lorsa's head activations): one streaming read of pre.  rows_per_group as in sae_select_topk_row_granule. */
 int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int64_t rows_per_group,

@@ -72,9 +72,18 @@ __host__ __device__ inline int64_t bt_candidate_capacity(int64_t B, int64_t F) {
   return c < 0x7fffffffLL ? c : 0x7fffffffLL;
 }
 
-__device__ __forceinline__ uint32_t bt_key(float pre, float b, float s, float fm, bool has_mask) {
-  float h1 = (pre + b) * s;
-  if (has_mask) h1 = ((h1 / s) * fm) * s;   // aux-k: hidden_pre * dead * scale, op for op
+// lowp: the arithmetic of a dictionary whose parameters are bf16 tensors -- the sum with the bias and the product with
+// the norm are each rounded to bf16, as the tensors `x @ W_E + b_E` and `hidden_pre * decoder_norm()` are
+// (models/sae.py:324-335 with cfg.dtype = bfloat16); the bias and scale arrive as fp32 copies of bf16 values.  The flag
+// is the same for every lane of a launch.
+__device__ __forceinline__ uint32_t bt_key(float pre, float b, float s, float fm, bool has_mask, bool lowp) {
+  float h1;
+  if (lowp) {
+    h1 = bf16_round(mul_rn(bf16_round(add_rn(pre, b)), s));
+  } else {
+    h1 = (pre + b) * s;
+    if (has_mask) h1 = ((h1 / s) * fm) * s;   // aux-k: hidden_pre * dead * scale, op for op
+  }
   return h1 > 0.f ? __float_as_uint(h1) : 0u;
 }
 
@@ -87,6 +96,7 @@ struct BatchReader {
   int vec;    // rows, bias, scale and mask can be read as 16-byte vectors
   int nseg;   // 64-lane segments per row (the full pass walks these)
   int ngran;  // granules per row, rounded up to a multiple of 4 (the maxima past the row's end are 0)
+  int lowp;   // keys and values in bf16 arithmetic (see bt_key)
   __device__ __forceinline__ const char *row_ptr(int b) const {
     return reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
   }
@@ -147,7 +157,7 @@ struct BatchReader {
     const bool inside = base >= 0 && base < F;
 #pragma unroll
     for (int e = 0; e < V; ++e)
-      keys[e] = (inside && base + e < F) ? bt_key(p[e], pr.bb[e], pr.ss[e], pr.mm[e], fmask != nullptr) : 0u;
+      keys[e] = (inside && base + e < F) ? bt_key(p[e], pr.bb[e], pr.ss[e], pr.mm[e], fmask != nullptr, lowp != 0) : 0u;
   }
   // the same, fetching bias, scale and mask
   __device__ __forceinline__ void keys_of(int b, int base, const u32x4 &raw, uint32_t (&keys)[V]) const {
@@ -614,7 +624,9 @@ __global__ __launch_bounds__(BT_TOKENS_PER_WG * 64) void bt_emit_kernel(BatchRea
             const int f = feat0 + e;
             const float h1 = __uint_as_float(k);
             idx_out[o] = f;
-            val_out[o] = rd.scale ? h1 / rd.scale[f] : h1;
+            float v = h1;
+            if (rd.scale) { v = h1 / rd.scale[f]; if (rd.lowp) v = bf16_round(v); }   // the quotient is a bf16 tensor too
+            val_out[o] = v;
           }
           ++pos;
         }
@@ -642,7 +654,7 @@ template <bool BF16>
 static int run_batch_select(const void *pre, const float *b_enc, const float *scale, const float *fmask, int64_t B,
                             int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
                             int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
-                            hipStream_t st, const uint32_t *gran_max_given = nullptr) {
+                            hipStream_t st, const uint32_t *gran_max_given = nullptr, bool lowp = false) {
   constexpr int V = BatchReader<BF16>::V;
   char *ws = reinterpret_cast<char *>(workspace);
   BatchSelState *state = reinterpret_cast<BatchSelState *>(ws);
@@ -662,7 +674,7 @@ static int run_batch_select(const void *pre, const float *b_enc, const float *sc
   cd.cap = bt_candidate_capacity(B, F);
   cd.key = reinterpret_cast<uint32_t *>(cd.tok_cnt + B);
   cd.feat = reinterpret_cast<int32_t *>(cd.key + cd.cap);
-  BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F, vec ? 1 : 0, nseg, ngran};
+  BatchReader<BF16> rd{pre, b_enc, scale, fmask, (int)F, vec ? 1 : 0, nseg, ngran, lowp ? 1 : 0};
   hipLaunchKernelGGL(bt_init_kernel, dim3(1), dim3(256), 0, st, state, hist, k_total, k_total_dev, bt_candidate_capacity(B, F));
   const int rows_per_wg = (int)(B / 65535 > 16 ? B / 65535 + 1 : 16);
   if (gran_max_given) {
@@ -722,6 +734,22 @@ extern "C" int sae_select_topk_batch(const void *pre, int pre_dtype, const float
                                   row_nnz, total_out, workspace, st);
   return run_batch_select<false>(pre, b_enc, scale, feat_mask, B, F, k_total, k_total_dev, idx, val, capacity, row_off,
                                  row_nnz, total_out, workspace, st);
+}
+
+extern "C" int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
+                                          int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
+                                          int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out,
+                                          void *workspace, int64_t workspace_bytes, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(pre_bf16 && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: null pointer");
+  SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F <= (1LL << 30), SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: bad shape");
+  SAE_REQUIRE(k_total_dev || k_total >= 0, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: k_total must be >= 0");
+  SAE_REQUIRE(capacity > 0, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: capacity must be positive");
+  SAE_REQUIRE(workspace && workspace_bytes >= sae_select_topk_batch_workspace_bytes(B, F), SAE_ERR_WORKSPACE,
+              "select_topk_batch_lowp: workspace of %lld bytes needed", (long long)sae_select_topk_batch_workspace_bytes(B, F));
+  SAE_REQUIRE((((uintptr_t)workspace) & 255) == 0, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: workspace must be 256-byte aligned");
+  return run_batch_select<true>(pre_bf16, b_enc, scale, nullptr, B, F, k_total, k_total_dev, idx, val, capacity, row_off,
+                                row_nnz, total_out, workspace, (hipStream_t)stream, nullptr, true);
 }
 
 extern "C" int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,

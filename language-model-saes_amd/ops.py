@@ -514,12 +514,16 @@ def select_topk_batch(
     feat_mask: Optional[torch.Tensor] = None,
     capacity: Optional[int] = None,
     granule_max: Optional[torch.Tensor] = None,
+    lowp: bool = False,
 ) -> SparseCode:
     """Batch-global TopK.  `k_total` is an int, or a device int64 tensor (then `capacity` is required).
+    `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the arithmetic of a dictionary held in bf16).
     `granule_max`: the second output of `encoder_gemm_granule_max` for the same bf16 pre, b_enc and scale (F a multiple
     of 256, no feat_mask); the select's one full pass over the matrix then shrinks to a histogram of those maxima."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
+    if lowp and (pre.dtype != torch.bfloat16 or feat_mask is not None or granule_max is not None):
+        raise ValueError("lowp select takes a bf16 pre and neither feat_mask nor granule_max")
     if granule_max is not None:
         if feat_mask is not None or pre.dtype != torch.bfloat16 or F % 256:
             raise ValueError("granule_max needs a bf16 pre with F a multiple of 256 and no feat_mask")
@@ -554,6 +558,10 @@ def select_topk_batch(
             rc = lib.sae_select_topk_batch_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k_host,
                                                    _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
                                                    row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
+        elif lowp:
+            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k_host, _ptr(k_dev), idx.data_ptr(),
+                                                val.data_ptr(), capacity, row_off.data_ptr(), row_nnz.data_ptr(), None,
+                                                ws.data_ptr(), ws_bytes, _stream(pre))
         else:
             rc = lib.sae_select_topk_batch(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
                                            _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),

@@ -248,7 +248,7 @@ class _FusedSparseStep(torch.autograd.Function):
                 scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
         w_dec_op = sae._w_dec_operand(amp)
         if batch_wide:
-            code = ops.select_topk_batch(pre, b_E, scale, k * B, granule_max=gmax)
+            code = ops.select_topk_batch(pre, b_E, scale, k * B, granule_max=gmax, lowp=lowp)
         else:
             code = ops.select_topk_row(pre, b_E, scale, k, lowp=lowp, granule_max=gmax)
         aux = holder.aux
@@ -838,7 +838,7 @@ class SparseAutoEncoder(SparseDictionary):
             and sparsity_loss_type is None and not (lp_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
             and (self.W_E.dtype == torch.float32
-                 or (self.W_E.dtype == torch.bfloat16 and self.cfg.act_fn.lower() == "topk" and not (auxk_coefficient > 0.0)
+                 or (self.W_E.dtype == torch.bfloat16 and not (auxk_coefficient > 0.0)
                      and self.cfg.d_model % 64 == 0))
         )
 

@@ -662,6 +662,42 @@ def test_select_topk_batch_feature_mask(pkg, oracle, dev):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("B,F,k", [(5, 4096, 16), (16, 24576, 64), (3, 1001, 8), (40, 8192, 200), (64, 32768, 32)])
+def test_select_topk_batch_in_bf16_arithmetic(pkg, oracle, dev, B, F, k):
+    """BatchTopK of a dictionary held in bf16: bias sum, norm product and final quotient are bf16 tensors in the
+    reference (models/sae.py:324-341), and the closure's TopK runs over those bf16 values
+    (models/sparse_dictionary.py:761-794).  The expected code is that op sequence on CPU bf16 tensors with the oracle's
+    TopK over both axes; keys collide by the hundred at the threshold, where the lowest flattened indices are kept."""
+    print(f"batch select lowp B={B} F={F} k={k}", flush=True)
+    g = torch.Generator().manual_seed(F + k + 2)
+    pre = torch.randn(B, F, generator=g).bfloat16()
+    b_enc = (0.1 * torch.randn(F, generator=g)).bfloat16()
+    norm = (0.5 + torch.rand(F, generator=g)).bfloat16()
+    h1 = (pre + b_enc) * norm
+    h1 = h1 * h1.gt(0).to(h1.dtype)
+    want = oracle.topk(h1, k=k * B, dim=(-2, -1)) / norm
+    assert want.dtype == torch.bfloat16
+    for k_dev in (False, True):
+        kt = torch.tensor(k * B, dtype=torch.int64, device=dev) if k_dev else k * B
+        code = pkg.ops.select_topk_batch(pre.to(dev), b_enc.float().to(dev), norm.float().to(dev), kt, lowp=True,
+                                         capacity=k * B if k_dev else None)
+        got = code.to_dense().cpu()
+        assert int(code.row_nnz.sum()) == k * B
+        assert torch.equal(got != 0, want != 0), "kept sets differ"
+        assert torch.equal(got, want.float()), "kept values differ"
+    # the threshold's value is shared: a set of the same size with another tie order exists
+    thr = h1[want != 0].float().min()
+    if B * F >= 300000:
+        assert (h1.float() == thr).sum() > ((want != 0) & (h1.float() == thr)).sum()
+    # without bias and scale the arithmetic is the plain one
+    plain = pkg.ops.select_topk_batch(pre.to(dev), None, None, k * B)
+    lowp = pkg.ops.select_topk_batch(pre.to(dev), None, None, k * B, lowp=True)
+    assert torch.equal(plain.to_dense(), lowp.to_dense())
+    with pytest.raises(ValueError):
+        pkg.ops.select_topk_batch(pre.float().to(dev), None, None, k * B, lowp=True)
+
+
+@pytest.mark.gpu
 def test_mfma_probe_runs_and_counts_its_flop(pkg, dev):
     flop, ms = pkg.ops.mfma_probe(dev, n_workgroups=64, iters=16)
     assert flop == 2.0 * 16 * 16 * 32 * 32 * 16 * 4 * 64

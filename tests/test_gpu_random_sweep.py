@@ -28,7 +28,7 @@ def test_random_sweep(pkg, oracle, dev, sweep_seed, budget_s=12.0):
     n = 0
     while time.time() - t0 < budget_s:
         n += 1
-        kind = rng.choice(['row', 'row', 'row_lowp', 'row_mask', 'batch', 'batch', 'fi_adam', 'adam_lowp'])
+        kind = rng.choice(['row', 'row', 'row_lowp', 'row_mask', 'batch', 'batch', 'batch_lowp', 'fi_adam', 'adam_lowp'])
         seed = rng.randrange(1 << 30)
         g = torch.Generator().manual_seed(seed)
         if kind.startswith('row'):
@@ -71,6 +71,17 @@ def test_random_sweep(pkg, oracle, dev, sweep_seed, budget_s=12.0):
             fm = (torch.rand(F, generator=g) < 0.3).float() if (s is not None and rng.random() < 0.3) else None
             print(f'[{n}] batch seed={seed} B={B} F={F} k_total={k_total} {dt} ties={ties} mask={fm is not None}', flush=True)
             tk.check_batch_select(pkg, oracle, dev, pre, b, s, k_total, fm, k_on_device=rng.random() < 0.3)
+        elif kind == 'batch_lowp':
+            B = rng.choice([2, 5, 16, 33]); F = rng.choice([64, 1000, 4096, 8192, 32768]); k = rng.choice([1, 4, 32, 64])
+            k_total = min(B * F, k * B)
+            pre = torch.randn(B, F, generator=g).bfloat16()
+            bb = (0.1 * torch.randn(F, generator=g) if rng.random() < 0.7 else torch.zeros(F)).bfloat16()
+            nn = (0.5 + torch.rand(F, generator=g) if rng.random() < 0.7 else torch.ones(F)).bfloat16()
+            print(f'[{n}] batch_lowp seed={seed} B={B} F={F} k_total={k_total}', flush=True)
+            h1 = (pre + bb) * nn
+            want = oracle.topk(h1 * h1.gt(0).to(h1.dtype), k=k_total, dim=(-2, -1)) / nn
+            got = pkg.ops.select_topk_batch(pre.to(dev), bb.float().to(dev), nn.float().to(dev), k_total, lowp=True).to_dense().cpu()
+            assert torch.equal(got, want.float())
         elif kind == 'fi_adam':
             B = rng.choice([16, 64, 300]); d = rng.choice([64, 256, 768, 2048, 4096]); F = rng.choice([96, 256, 1000]); k = rng.choice([3, 8, 16])
             dd = rng.choice([torch.float32, torch.bfloat16])

@@ -367,6 +367,54 @@ def test_fused_batchtopk_step_matches_oracle(pkg, oracle, dev, amp):
         assert rel_err(getattr(sae, name).grad, getattr(ref, name).grad) < tol, name
 
 
+@pytest.mark.parametrize("include_norm", [False, True])
+def test_fused_batchtopk_step_with_bf16_parameters_matches_oracle(pkg, oracle, dev, include_norm):
+    """BatchTopK with cfg.dtype = bfloat16: the tensors around the batch-wide select are bf16 in the reference, so the
+    kept set and the kept values must be identical; reconstruction, loss and gradients to bf16 tolerance."""
+    print(f"fused batchtopk step, bf16 parameters, include_norm={include_norm}", flush=True)
+    sae, ref, batch = make_pair_act(pkg, oracle, dev, "batchtopk", d=256, F=2048, k=16, B=192, r=8, seed=12,
+                                    include_norm=include_norm, dtype=torch.bfloat16)
+    assert sae.W_E.dtype == torch.bfloat16 and ref.W_E.dtype == torch.bfloat16
+    ctx, rctx = run_both(pkg, oracle, dev, sae, ref, batch, amp=True, substitute=True)
+    assert "sparse_code" in ctx, "the fused route was not taken"
+    assert (rctx["feature_acts"] != 0).sum().item() == 16 * 192
+    assert (rctx["feature_acts"] != 0).sum(-1).float().std().item() > 0  # rows really differ in length
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert torch.equal(ctx["feature_acts"].cpu(), rctx["feature_acts"].float()), "kept values differ"
+    assert rel_err(ctx["reconstructed"], rctx["reconstructed"]) < BF16_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < BF16_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        got, want = getattr(sae, name).grad, getattr(ref, name).grad
+        assert got.dtype == torch.bfloat16 and got.shape == want.shape
+        assert rel_err(got, want) < BF16_TOL, name
+
+
+def test_batchtopk_bf16_parameters_adam_steps_factored_equals_dense(pkg, oracle, dev):
+    """three steps of the fused BatchTopK loss + HipAdam on a bf16 dictionary: the factored gradients and the dense
+    ones end at the same bits, and the loss falls"""
+    finals = []
+    for defer in (True, False):
+        sae, _, batch = make_pair_act(pkg, oracle, dev, "batchtopk", d=256, F=2048, k=16, B=192, r=8, seed=13,
+                                      include_norm=True, dtype=torch.bfloat16)
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae, defer_weight_grads=defer)
+        gbatch = {k: v.to(dev) for k, v in batch.items()}
+        losses = []
+        for _ in range(3):
+            loss = sae.compute_loss(gbatch, return_aux_data=False)
+            loss.backward()
+            if defer:
+                assert sae.W_D.grad is None and sae.W_D._sparse_grad is not None
+            opt.step()
+            opt.zero_grad()
+            losses.append(loss.item())
+        assert losses[-1] < losses[0]
+        finals.append(({n: p.detach().clone() for n, p in sae.named_parameters()}, losses))
+    (pa, la), (pb, lb) = finals
+    assert la == lb
+    for n in pa:
+        assert pa[n].dtype == torch.bfloat16 and torch.equal(pa[n], pb[n]), n
+
+
 @pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
 @pytest.mark.parametrize("include_norm", [False, True])
 @pytest.mark.parametrize("route", ["dense", "sparse"])
