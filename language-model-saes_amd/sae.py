@@ -140,7 +140,14 @@ def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_au
         s_d[:nd] = scale.index_select(0, dead_idx)
     pre_d = ops.encoder_gemm(x_op, W_Et, pre_dtype)                                   # [B, ndp]
     kk = min(k_aux, nd)
-    code_d = ops.select_topk_batch(pre_d, b_d, s_d, kk * B) if batch_wide else ops.select_topk_row(pre_d, b_d, s_d, kk)
+    # with a norm scale the keys are `hidden_pre * is_dead * decoder_norm` op for op, hidden_pre being the quotient the
+    # encoder returned (models/sparse_dictionary.py:958-966): the select's masked arithmetic with every block column in
+    if s_d is not None:
+        keep = torch.ones(ndp, dtype=torch.float32, device=dev)
+        code_d = (ops.select_topk_batch(pre_d, b_d, s_d, kk * B, feat_mask=keep) if batch_wide
+                  else ops.select_topk_row(pre_d, b_d, s_d, kk, feat_mask=keep))
+    else:
+        code_d = ops.select_topk_batch(pre_d, b_d, None, kk * B) if batch_wide else ops.select_topk_row(pre_d, b_d, None, kk)
     # dense [B, ndp] activations of the block: fp32 (the mask of the backward pass) and, under autocast, bf16
     A, A_b16 = ops.code_to_dense(code_d, ndp, want_f32=True, want_bf16=amp)
     A_op = A_b16 if amp else A
@@ -1025,6 +1032,8 @@ class SparseAutoEncoder(SparseDictionary):
             "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
             "auxk_coefficient": auxk_coefficient, "sparse_code": code,
         }
+        if holder.aux_code is not None:
+            eager["aux_sparse_code"] = holder.aux_code    # the aux-k term's selection among the dead features
         lazy = {
             "n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
             "feature_acts": code.to_dense,

@@ -7,6 +7,8 @@ here takes the GEMM's forward values from the HIP path (its backward stays the m
 second test runs the oracle untouched and checks agreement statistically.
 """
 
+import contextlib
+
 import pytest
 import torch
 
@@ -466,6 +468,46 @@ def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm, 
     for name in ("W_E", "b_E", "W_D", "b_D"):
         assert rel_err(getattr(sae, name).grad, getattr(ref, name).grad) < FP32_TOL, name
     assert sae.current_k == k and ref.current_k == k
+
+
+@pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
+@pytest.mark.parametrize("amp", [False, True])
+def test_auxk_selection_is_the_reference_op_sequence_on_both_routes(pkg, oracle, dev, act_fn, amp):
+    """The aux-k term's own selection among the dead features: `hidden_pre * is_dead * decoder_norm` with hidden_pre the
+    quotient the encoder returned (models/sparse_dictionary.py:958-970), evaluated op for op on the kernel's GEMM
+    output with the oracle's TopK.  The compact dense block and the stacked sparse code must keep exactly that set with
+    exactly those values."""
+    print(f"aux-k selection {act_fn} amp={amp}", flush=True)
+    B, F, k, k_aux = 192, 2048, 16, 32
+    codes = {}
+    for route in ("dense", "sparse"):
+        sae, ref, batch = make_pair_act(pkg, oracle, dev, act_fn, d=256, F=F, k=k, B=B, r=8, seed=14, include_norm=True)
+        sae.aux_dense_block = route == "dense"
+        trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=1 / 32, k_aux=k_aux, dead_threshold=float(B)))
+        trainer._initialize_dead_statistics(sae)
+        warm = torch.zeros(B, F); warm[:, ::7] = 1.0
+        trainer.update_dead_statistics(warm.to(dev), None, ("batch", "sae"))
+        gbatch = {k_: v.to(dev) for k_, v in batch.items()}
+        with (torch.autocast("cuda", dtype=torch.bfloat16) if amp else contextlib.nullcontext()):
+            ctx = sae.compute_loss(gbatch, update_dead_statistics=trainer.update_dead_statistics, auxk_coefficient=1 / 32,
+                                   k_aux=k_aux)
+        assert sae._last_aux_route == route
+        codes[route] = ctx["aux_sparse_code"].to_dense().cpu()
+        dead = trainer.is_dead.cpu()
+    # the reference's sequence on the same GEMM output
+    x_op = gbatch["in"].contiguous()
+    pre = (pkg.ops.encoder_gemm(pkg.ops.cast_bf16(x_op), sae._w_enc_operand(True), torch.bfloat16) if amp
+           else pkg.ops.encoder_gemm(x_op, sae._w_enc_operand(False), torch.float32)).cpu().float()
+    n = sae._decoder_norm_nograd().cpu()   # the norms the kernels read (the oracle's differ from them in the last bit)
+    hidden_pre = ((pre + sae.b_E.detach().cpu()) * n) / n
+    dead_pre = hidden_pre * dead * n
+    kk = min(k_aux, int(dead.sum()))
+    assert int(dead.sum()) > k_aux
+    relu = dead_pre * dead_pre.gt(0).to(dead_pre.dtype)
+    want = (oracle.topk(relu, k=kk, dim=-1) if act_fn == "topk" else oracle.topk(relu, k=kk * B, dim=(-2, -1))) / n
+    for route in ("dense", "sparse"):
+        assert torch.equal(codes[route] != 0, want != 0), f"{route}: kept sets differ"
+        assert torch.equal(codes[route], want), f"{route}: kept values differ"
 
 
 def test_fused_auxk_without_dead_features_is_plain_loss(pkg, oracle, dev):
