@@ -105,20 +105,51 @@ class SparseRowGradPieces:
         return rows, bias
 
 
-def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux: int, batch_wide: bool, amp: bool):
+class _DeadCount:
+    """#dead on its way to the host: the count and its copy into pinned memory are enqueued when this is made, and
+    `value()` waits for the copy only.  Kernels enqueued in between keep the GPU busy while the host waits and then
+    prepares the launches that depend on the count."""
+
+    def __init__(self, dead: torch.Tensor):
+        self.host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+        self.host.copy_(dead.sum().reshape(1), non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record()
+
+    def value(self) -> int:
+        self.event.synchronize()
+        return int(self.host[0])
+
+
+def _aux_block_fits(B: int, d: int, amp: bool) -> bool:
+    gran = 64 if amp else 32
+    return B % gran == 0 and d % gran == 0
+
+
+def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux: int, batch_wide: bool, amp: bool,
+                     n_dead: Optional[int] = None):
     """Forward half of the aux-k term on a compacted dead block.  Gathers the dead features' encoder / decoder
     rows into [n, d] matrices (n = #dead padded to the GEMM's K granule), recomputes their pre-activations with
     the encoder GEMM (same kernel, same accumulation order as the full product: identical values), selects among
     them, scatters the kept values into a dense [B, n] matrix and decodes it with one more GEMM.
     Returns None when the shapes do not fit the GEMM kernel or the block is too wide to pay; sizing the block
-    needs #dead on the host (one synchronisation per step, as the reference's `int(is_dead.sum().item())`)."""
+    needs #dead on the host (one synchronisation per step, as the reference's `int(is_dead.sum().item())`; `n_dead`
+    hands in a count the caller already fetched)."""
     B, d = x_op.shape
     F = dead.numel()
     gran = 64 if amp else 32
-    if B % gran != 0 or d % gran != 0:
+    if not _aux_block_fits(B, d, amp):
         return None
-    dead_idx = torch.nonzero(dead).squeeze(1)
-    nd = int(dead_idx.numel())
+    if n_dead is None:
+        dead_idx = torch.nonzero(dead).squeeze(1)
+        nd = int(dead_idx.numel())
+    else:
+        nd = int(n_dead)
+        # ascending indices of the dead features without another wait: each takes the place its rank gives it
+        rank = torch.cumsum(dead, 0) - 1
+        dead_idx = torch.empty(nd + 1, dtype=torch.int64, device=dead.device)
+        dead_idx.scatter_(0, torch.where(dead, rank, torch.full_like(rank, nd)), torch.arange(F, device=dead.device))
+        dead_idx = dead_idx[:nd]
     if nd == 0:
         return {"n_dead": 0, "code": None}
     if nd > 64 * max(k_aux, 1) or B * (nd + gran) >= 2 ** 31:
@@ -271,14 +302,19 @@ class _FusedSparseStep(torch.autograd.Function):
             k_aux = int(aux["k_aux"])
             ctx.aux_dense = None
             dense_block = None
-            if aux.get("dense", True):
-                dense_block = _aux_dense_block(x_op, pre.dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux, batch_wide, amp)
+            recon = None
+            if aux.get("dense", True) and _aux_block_fits(x_op.shape[0], x_op.shape[1], amp):
+                # the block is sized by #dead: the count is fetched while the main decode, which does not depend on
+                # it, runs
+                count = _DeadCount(dead)
+                recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
+                dense_block = _aux_dense_block(x_op, pre.dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux, batch_wide, amp,
+                                               n_dead=count.value())
             sae._last_aux_route = "dense" if dense_block is not None else "sparse"
             if dense_block is not None:
                 # The dead block is small and hit by a large share of the tokens: its part of the step is three small
                 # GEMMs on a compacted [n_dead, d] copy of the two weight blocks instead of gathers per (token, feature).
                 blk = dense_block
-                recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
                 alpha = float(aux["coefficient"])
                 # squared error, aux-k residual (the residual is not detached), d loss / d aux_recon and d loss / d recon
                 rec_tok, aux_tok, g_aux, grad_recon, grad_recon_b16 = ops.mse_auxk_fused(
@@ -300,7 +336,8 @@ class _FusedSparseStep(torch.autograd.Function):
                 else:
                     # min(k_aux, #dead) needs no host value: at most #dead entries can be positive
                     aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f)
-                recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
+                if recon is None:
+                    recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
                 aux_recon = ops.sparse_decode_fwd(aux_code, w_dec_op, None)
                 has_dead = (n_dead > 0).to(torch.float32)
                 w = tok_w[:, None]
