@@ -128,9 +128,13 @@ int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, c
 /* sae_select_topk_row for a dictionary whose dtype is bfloat16 (config.py:39): pre is bf16, and the sum with the
  * bias, the product with the scale and the final quotient are each rounded to bf16, as the bf16 tensors
  * `x @ W_E + b_E`, `hidden_pre * decoder_norm()` and `feature_acts / decoder_norm()` are (models/sae.py:324-341).
- * b_enc / scale are fp32 copies of the bf16 bias / norms.  Keys then collide often; ties -> lowest feature index. */
-int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int k,
-                             int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream);
+ * b_enc / scale are fp32 copies of the bf16 bias / norms.  Keys then collide often; ties -> lowest feature index.
+ * feat_mask (0/1 per feature, or NULL): the aux-k selection of such a dictionary, whose keys are
+ * `hidden_pre * is_dead * decoder_norm` with hidden_pre the bf16 quotient `encode` returned, i.e. two more roundings
+ * (models/sparse_dictionary.py:958-970). */
+int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, const float *feat_mask,
+                             int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz,
+                             void *stream);
 
 /* out[b, f] = bf16(float(bf16(sum_j x[b, j] * w_t[f, j])) + col_bias[f] + row_bias[b])      (bf16 operands and output)
  * What `(x @ W) + bias` is under bf16 autocast: the product a bf16 tensor, the bias an fp32 parameter, the sum cast to
@@ -175,10 +179,11 @@ int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_
  * sae_select_topk_row: pre is bf16, and the sum with the bias, the product with the scale and the final quotient are each
  * rounded to bf16, as the bf16 tensors around the reference's batch_topk closure are (models/sae.py:324-341,
  * models/sparse_dictionary.py:761-794).  b_enc / scale are fp32 copies of the bf16 bias / norms.  Many keys then share
- * the threshold's value; ties keep the lowest flattened indices b * F + f.  No feat_mask.  Same workspace. */
-int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
-                               int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val, int64_t capacity,
-                               int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
+ * the threshold's value; ties keep the lowest flattened indices b * F + f.  feat_mask as in sae_select_topk_row_lowp.
+ * Same workspace. */
+int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, const float *feat_mask,
+                               int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
+                               int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
                                int64_t workspace_bytes, void *stream);
 
 /* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product

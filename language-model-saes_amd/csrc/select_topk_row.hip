@@ -49,13 +49,21 @@ struct SelShared {
 __device__ __forceinline__ float sel_bf16_round(float x) { return bf16_round(x); }
 // ARITH selects the arithmetic at compile time: the masked (aux-k) form costs registers that the plain form,
 // which runs every step, should not pay for (with one kernel for both, 14 registers per lane were spilled).
-constexpr int SEL_PLAIN = 0, SEL_LOWP = 1, SEL_MASKED = 2;
+// LOWP_MASKED: the aux-k keys of such a dictionary, `hidden_pre * is_dead * decoder_norm` with hidden_pre the bf16
+// quotient the encoder returned (models/sparse_dictionary.py:958-966): one more rounding after each operation.
+constexpr int SEL_PLAIN = 0, SEL_LOWP = 1, SEL_MASKED = 2, SEL_LOWP_MASKED = 3;
+constexpr bool sel_has_mask(int arith) { return arith == SEL_MASKED || arith == SEL_LOWP_MASKED; }
+constexpr bool sel_is_lowp(int arith) { return arith == SEL_LOWP || arith == SEL_LOWP_MASKED; }
 template <int ARITH>
 __device__ __forceinline__ uint32_t key_of(float pre, float b, float s, float fm) {
   if constexpr (ARITH == SEL_PLAIN) return select_key_plain(pre, b, s);
   float h1;
   if constexpr (ARITH == SEL_LOWP) {
     h1 = sel_bf16_round(mul_rn(sel_bf16_round(add_rn(pre, b)), s));
+  } else if constexpr (ARITH == SEL_LOWP_MASKED) {
+    h1 = sel_bf16_round(mul_rn(sel_bf16_round(add_rn(pre, b)), s));
+    h1 = sel_bf16_round(h1 / s);
+    h1 = sel_bf16_round(mul_rn(sel_bf16_round(mul_rn(h1, fm)), s));
   } else {
     h1 = (pre + b) * s;
     h1 = ((h1 / s) * fm) * s;  // aux-k: hidden_pre * dead * scale, op for op
@@ -147,7 +155,7 @@ struct RowReader {
     }
     const int base = c * V;
     float bb[V], ss[V], mm[V];
-    if constexpr (ARITH == SEL_MASKED) {
+    if constexpr (sel_has_mask(ARITH)) {
 #pragma unroll
       for (int q = 0; q < V / 4; ++q) {
         const float4 t = reinterpret_cast<const float4 *>(fmask + base)[q];
@@ -185,7 +193,7 @@ struct RowReader {
     float pre;
     if constexpr (BF16) pre = bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(row)[i]);
     else pre = reinterpret_cast<const float *>(row)[i];
-    return key_of<ARITH>(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, ARITH == SEL_MASKED ? fmask[i] : 1.f);
+    return key_of<ARITH>(pre, b_enc ? b_enc[i] : 0.f, scale ? scale[i] : 1.f, sel_has_mask(ARITH) ? fmask[i] : 1.f);
   }
   // calls fn(index, key) for every element of the row, vectorised when the row allows it
   template <typename Fn>
@@ -441,7 +449,7 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const float s = scale ? scale[my_idx] : 1.f;
     if (rank < k) {
       idx_out[(size_t)b * k + rank] = my_idx;
-      val_out[(size_t)b * k + rank] = scale ? (ARITH == SEL_LOWP ? sel_bf16_round(h1 / s) : h1 / s) : h1;
+      val_out[(size_t)b * k + rank] = scale ? (sel_is_lowp(ARITH) ? sel_bf16_round(h1 / s) : h1 / s) : h1;
     }
   }
   for (int i = k_eff + tid; i < k; i += SEL_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
@@ -470,7 +478,9 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
 #define SAE_LAUNCH_SELECT(BF, ST, ...)                                                                                     \
   hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
                      scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged, rows_per_group)
-  if (lowp) {
+  if (lowp && feat_mask) {
+    if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP_MASKED); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP_MASKED);
+  } else if (lowp) {
     if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP);
   } else if (feat_mask) {
     if (pre_dtype == SAE_BF16) {
@@ -693,9 +703,10 @@ extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const floa
                                    stream);
 }
 
-extern "C" int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
-                                        int k, int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
-  return sae::select_topk_row_impl(true, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz,
+extern "C" int sae_select_topk_row_lowp(const void *pre_bf16, const float *b_enc, const float *scale, const float *feat_mask,
+                                        int64_t B, int64_t F, int k, int32_t *idx, float *val, int64_t *row_off,
+                                        int32_t *row_nnz, void *stream) {
+  return sae::select_topk_row_impl(true, pre_bf16, SAE_BF16, b_enc, scale, feat_mask, B, F, k, idx, val, row_off, row_nnz,
                                    sae::SEL_CAP, stream);
 }
 

@@ -455,7 +455,8 @@ def select_topk_row(
     rows_per_group: int = 0,
 ) -> SparseCode:
     """Per-token TopK of (pre + b_enc) * scale.  `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the
-    arithmetic of a dictionary whose parameters are bf16 tensors).  `granule_max`: the second output of
+    arithmetic of a dictionary whose parameters are bf16 tensors).  `feat_mask` (0/1 per feature): the aux-k selection
+    among the masked-in features, with the reference's key arithmetic for it.  `granule_max`: the second output of
     `encoder_gemm_granule_max` for the same pre, b_enc and scale; the row is then read only where a kept element
     can be (same result).  On that route `rows_per_group` > 0 says that pre stacks groups of that many rows and that
     b_enc / scale hold one vector of F per group."""
@@ -464,8 +465,8 @@ def select_topk_row(
     n_vec = F * (B // rows_per_group if rows_per_group else 1)
     if rows_per_group and (granule_max is None or B % rows_per_group):
         raise ValueError("rows_per_group needs the granule route and must divide the number of rows")
-    if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None or feat_mask is not None):
-        raise ValueError("lowp select takes a bf16 pre and neither cand_cap nor feat_mask")
+    if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None):
+        raise ValueError("lowp select takes a bf16 pre and no cand_cap")
     if granule_max is not None:
         if lowp or cand_cap is not None or feat_mask is not None or pre.dtype != torch.bfloat16:
             raise ValueError("the granule route takes a bf16 pre and none of lowp, cand_cap, feat_mask")
@@ -492,8 +493,8 @@ def select_topk_row(
                                              int(rows_per_group), idx.data_ptr(), val.data_ptr(), row_off.data_ptr(),
                                              row_nnz.data_ptr(), _stream(pre))
     elif lowp:
-        rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(), val.data_ptr(),
-                                          row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+        rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k, idx.data_ptr(),
+                                          val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     elif cand_cap is None and feat_mask is None:
         rc = lib.sae_select_topk_row(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), B, F, k, idx.data_ptr(),
                                      val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
@@ -522,8 +523,8 @@ def select_topk_batch(
     of 256, no feat_mask); the select's one full pass over the matrix then shrinks to a histogram of those maxima."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
-    if lowp and (pre.dtype != torch.bfloat16 or feat_mask is not None or granule_max is not None):
-        raise ValueError("lowp select takes a bf16 pre and neither feat_mask nor granule_max")
+    if lowp and (pre.dtype != torch.bfloat16 or granule_max is not None):
+        raise ValueError("lowp select takes a bf16 pre and no granule_max")
     if granule_max is not None:
         if feat_mask is not None or pre.dtype != torch.bfloat16 or F % 256:
             raise ValueError("granule_max needs a bf16 pre with F a multiple of 256 and no feat_mask")
@@ -559,9 +560,9 @@ def select_topk_batch(
                                                    _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
                                                    row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
         elif lowp:
-            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k_host, _ptr(k_dev), idx.data_ptr(),
-                                                val.data_ptr(), capacity, row_off.data_ptr(), row_nnz.data_ptr(), None,
-                                                ws.data_ptr(), ws_bytes, _stream(pre))
+            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
+                                                _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
+                                                row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
         else:
             rc = lib.sae_select_topk_batch(pre.data_ptr(), _dt(pre), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
                                            _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),

@@ -303,7 +303,8 @@ class _FusedSparseStep(torch.autograd.Function):
             ctx.aux_dense = None
             dense_block = None
             recon = None
-            if aux.get("dense", True) and _aux_block_fits(x_op.shape[0], x_op.shape[1], amp):
+            # (a dictionary held in bf16 takes the stacked sparse code: the dense block's kernels have no bf16 state)
+            if aux.get("dense", True) and not lowp and _aux_block_fits(x_op.shape[0], x_op.shape[1], amp):
                 # the block is sized by #dead: the count is fetched while the main decode, which does not depend on
                 # it, runs
                 count = _DeadCount(dead)
@@ -332,10 +333,10 @@ class _FusedSparseStep(torch.autograd.Function):
                 n_dead = dead.sum()
                 if batch_wide:
                     k_dev = (torch.clamp(n_dead, max=k_aux) * B).to(torch.int64)
-                    aux_code = ops.select_topk_batch(pre, b_E, scale, k_dev, feat_mask=dead_f, capacity=k_aux * B)
+                    aux_code = ops.select_topk_batch(pre, b_E, scale, k_dev, feat_mask=dead_f, capacity=k_aux * B, lowp=lowp)
                 else:
                     # min(k_aux, #dead) needs no host value: at most #dead entries can be positive
-                    aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f)
+                    aux_code = ops.select_topk_row(pre, b_E, scale, min(k_aux, pre.shape[1]), feat_mask=dead_f, lowp=lowp)
                 if recon is None:
                     recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
                 aux_recon = ops.sparse_decode_fwd(aux_code, w_dec_op, None)
@@ -385,7 +386,8 @@ class _FusedSparseStep(torch.autograd.Function):
         db_D = None
         if ctx.has_b_D:
             # a bf16 dictionary's reconstruction is a bf16 tensor, so the gradient summed for b_D is the bf16-rounded one
-            gr = ctx.grad_recon if ctx.param_dtype == torch.float32 else ctx.grad_dense_D.float()
+            # (of the tokens themselves: a stacked aux-k code appends the aux reconstruction's gradient, which has no bias)
+            gr = ctx.grad_recon if ctx.param_dtype == torch.float32 else ctx.grad_dense_D[: ctx.n_tokens].float()
             db_D = ops.col_sum(gr) * g
         extra_D = extra_E = None
         ad = ctx.aux_dense
@@ -882,8 +884,7 @@ class SparseAutoEncoder(SparseDictionary):
             and sparsity_loss_type is None and not (lp_coefficient > 0.0)
             and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
             and (self.W_E.dtype == torch.float32
-                 or (self.W_E.dtype == torch.bfloat16 and not (auxk_coefficient > 0.0)
-                     and self.cfg.d_model % 64 == 0))
+                 or (self.W_E.dtype == torch.bfloat16 and self.cfg.d_model % 64 == 0))
         )
 
     # ---- JumpReLU train-step loss: dense activations, so the GEMM kernel for all five dense products (two of them

@@ -698,6 +698,43 @@ def test_select_topk_batch_in_bf16_arithmetic(pkg, oracle, dev, B, F, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batch_wide", [False, True])
+@pytest.mark.parametrize("B,F,k,with_norm", [(5, 4096, 16, True), (16, 24576, 64, True), (3, 1001, 8, True), (12, 8192, 40, False)])
+def test_masked_select_in_bf16_arithmetic(pkg, oracle, dev, B, F, k, with_norm, batch_wide):
+    """aux-k selection of a dictionary held in bf16: the keys are `hidden_pre * is_dead * decoder_norm` on bf16 tensors,
+    hidden_pre being the quotient `encode` returned (models/sae.py:324-341, models/sparse_dictionary.py:958-970).  The
+    expected code is that op sequence on CPU bf16 tensors with the oracle's TopK."""
+    print(f"masked select lowp B={B} F={F} k={k} norm={with_norm} batch_wide={batch_wide}", flush=True)
+    g = torch.Generator().manual_seed(F + k + 3)
+    pre = torch.randn(B, F, generator=g).bfloat16()
+    b_enc = (0.1 * torch.randn(F, generator=g)).bfloat16()
+    norm = (0.5 + torch.rand(F, generator=g)).bfloat16() if with_norm else None
+    dead = torch.rand(F, generator=g) < 0.3
+    h1 = pre + b_enc
+    if with_norm:
+        h1 = h1 * norm
+        hidden_pre = h1 / norm
+        dead_pre = hidden_pre * dead * norm
+    else:
+        dead_pre = h1 * dead
+    assert dead_pre.dtype == torch.bfloat16
+    relu = dead_pre * dead_pre.gt(0).to(dead_pre.dtype)
+    want = oracle.topk(relu, k=k * B, dim=(-2, -1)) if batch_wide else oracle.topk(relu, k=k, dim=-1)
+    if with_norm:
+        want = want / norm
+    args = (pre.to(dev), b_enc.float().to(dev), None if norm is None else norm.float().to(dev))
+    fm = dead.float().to(dev)
+    if batch_wide:
+        code = pkg.ops.select_topk_batch(*args, k * B, feat_mask=fm, lowp=True)
+    else:
+        code = pkg.ops.select_topk_row(*args, k, feat_mask=fm, lowp=True)
+    got = code.to_dense().cpu()
+    assert torch.equal(got != 0, want != 0), "kept sets differ"
+    assert torch.equal(got, want.float()), "kept values differ"
+    assert not got[:, ~dead].any()
+
+
+@pytest.mark.gpu
 def test_mfma_probe_runs_and_counts_its_flop(pkg, dev):
     flop, ms = pkg.ops.mfma_probe(dev, n_workgroups=64, iters=16)
     assert flop == 2.0 * 16 * 16 * 32 * 32 * 16 * 4 * 64

@@ -48,8 +48,13 @@ def test_random_sweep(pkg, oracle, dev, sweep_seed, budget_s=12.0):
             elif kind == 'row_lowp':
                 pre = pre.bfloat16(); bb = (b if b is not None else torch.zeros(F)).bfloat16(); nn = (s if s is not None else torch.ones(F)).bfloat16()
                 h1 = (pre + bb) * nn
+                fm = None
+                if rng.random() < 0.4:
+                    fm = torch.rand(F, generator=g) < rng.choice([0.05, 0.3, 0.9])
+                    h1 = (h1 / nn) * fm * nn
                 want = oracle.topk(h1 * h1.gt(0).to(h1.dtype), k=k, dim=-1) / nn
-                got = pkg.ops.select_topk_row(pre.to(dev), bb.float().to(dev), nn.float().to(dev), k, lowp=True).to_dense().cpu()
+                got = pkg.ops.select_topk_row(pre.to(dev), bb.float().to(dev), nn.float().to(dev), k, lowp=True,
+                                              feat_mask=None if fm is None else fm.float().to(dev)).to_dense().cpu()
                 assert torch.equal(got, want.float())
             else:
                 fm = (torch.rand(F, generator=g) < rng.choice([0.01, 0.2, 0.9])).float()
@@ -79,8 +84,13 @@ def test_random_sweep(pkg, oracle, dev, sweep_seed, budget_s=12.0):
             nn = (0.5 + torch.rand(F, generator=g) if rng.random() < 0.7 else torch.ones(F)).bfloat16()
             print(f'[{n}] batch_lowp seed={seed} B={B} F={F} k_total={k_total}', flush=True)
             h1 = (pre + bb) * nn
+            fm = None
+            if rng.random() < 0.4:    # the aux-k form: the quotient the encoder returned, times the mask, times the norm
+                fm = torch.rand(F, generator=g) < rng.choice([0.05, 0.3, 0.9])
+                h1 = (h1 / nn) * fm * nn
             want = oracle.topk(h1 * h1.gt(0).to(h1.dtype), k=k_total, dim=(-2, -1)) / nn
-            got = pkg.ops.select_topk_batch(pre.to(dev), bb.float().to(dev), nn.float().to(dev), k_total, lowp=True).to_dense().cpu()
+            got = pkg.ops.select_topk_batch(pre.to(dev), bb.float().to(dev), nn.float().to(dev), k_total, lowp=True,
+                                            feat_mask=None if fm is None else fm.float().to(dev)).to_dense().cpu()
             assert torch.equal(got, want.float())
         elif kind == 'fi_adam':
             B = rng.choice([16, 64, 300]); d = rng.choice([64, 256, 768, 2048, 4096]); F = rng.choice([96, 256, 1000]); k = rng.choice([3, 8, 16])

@@ -471,6 +471,89 @@ def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm, 
 
 
 @pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
+def test_auxk_step_with_bf16_parameters(pkg, oracle, dev, act_fn):
+    """aux-k on a dictionary held in bf16 (the stacked sparse code): the aux selection is the reference's bf16 op sequence
+    exactly; losses and gradients agree with the oracle on CPU bf16 tensors to bf16 tolerance; three Adam steps with
+    factored and with dense gradients end at the same bits."""
+    print(f"aux-k step, bf16 parameters, {act_fn}", flush=True)
+    B, F, k, k_aux = 192, 2048, 16, 32
+    kw = dict(auxk_coefficient=1 / 32, k_aux=k_aux)
+
+    def fresh():
+        sae, ref, batch = make_pair_act(pkg, oracle, dev, act_fn, d=256, F=F, k=k, B=B, r=8, seed=15, include_norm=True,
+                                        dtype=torch.bfloat16)
+        trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=1 / 32, k_aux=k_aux, dead_threshold=float(B)))
+        trainer._initialize_dead_statistics(sae)
+        warm = torch.zeros(B, F); warm[:, ::7] = 1.0
+        trainer.update_dead_statistics(warm.to(dev), None, ("batch", "sae"))
+        stats = oracle.DeadStatistics(F, dead_threshold=float(B))
+        stats.update(warm, None, 1)
+        return sae, ref, batch, trainer, stats
+
+    sae, ref, batch, trainer, stats = fresh()
+    gbatch = {k_: v.to(dev) for k_, v in batch.items()}
+    ctx = sae.compute_loss(gbatch, update_dead_statistics=trainer.update_dead_statistics, **kw)
+    ctx["loss"].backward()
+    assert "sparse_code" in ctx and sae._last_aux_route == "sparse"
+    # the reference's sequence on bf16 tensors, from the kernel's own product
+    pre = pkg.ops.encoder_gemm(pkg.ops.cast_bf16(gbatch["in"].float().contiguous()), sae._w_enc_operand(True), torch.bfloat16).cpu()
+    n = sae._decoder_norm_nograd().cpu().bfloat16()
+    h1 = (pre + sae.b_E.detach().cpu()) * n
+    assert h1.dtype == torch.bfloat16
+    dead = trainer.is_dead.cpu()
+    dead_pre = (h1 / n) * dead * n
+    relu = dead_pre * dead_pre.gt(0).to(dead_pre.dtype)
+    kk = min(k_aux, int(dead.sum()))
+    assert int(dead.sum()) > k_aux
+    want = (oracle.topk(relu, k=kk, dim=-1) if act_fn == "topk" else oracle.topk(relu, k=kk * B, dim=(-2, -1))) / n
+    got = ctx["aux_sparse_code"].to_dense().cpu()
+    assert torch.equal(got != 0, want != 0), "aux-k kept sets differ"
+    assert torch.equal(got, want.float()), "aux-k kept values differ"
+
+    # the oracle on CPU bf16 tensors with the kernel's product handed in (see run_both)
+    def encode_sub(x, return_hidden_pre=False, **_):
+        mm = _SubstitutedMatmul.apply(x.to(torch.bfloat16), ref.W_E, pre)
+        hp = mm + ref.b_E
+        hp = hp * ref.decoder_norm()
+        fa = ref.activation_function(hp)
+        fa = fa / ref.decoder_norm()
+        hp = hp / ref.decoder_norm()
+        return (fa, hp) if return_hidden_pre else fa
+
+    ref.encode = encode_sub
+    rctx = ref.compute_loss(batch, update_dead_statistics=stats.update, **kw)
+    rctx["loss"].backward()
+    assert torch.equal(trainer.is_dead.cpu(), stats.is_dead)
+    assert torch.equal((ctx["feature_acts"] != 0).cpu(), rctx["feature_acts"] != 0), "selected index sets differ"
+    assert rctx["l_aux"].item() > 0
+    assert abs(ctx["l_aux"].item() - rctx["l_aux"].item()) / rctx["l_aux"].item() < BF16_TOL
+    assert abs(ctx["loss"].item() - rctx["loss"].item()) / rctx["loss"].item() < BF16_TOL
+    for name in ("W_E", "b_E", "W_D", "b_D"):
+        gotg, wantg = getattr(sae, name).grad, getattr(ref, name).grad
+        assert gotg.dtype == torch.bfloat16 and gotg.shape == wantg.shape
+        assert rel_err(gotg, wantg) < BF16_TOL, name
+
+    finals = []
+    for defer in (True, False):
+        sae, _, batch, trainer, _ = fresh()
+        opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, betas=(0.9, 0.999), model=sae, defer_weight_grads=defer)
+        losses = []
+        for _ in range(3):
+            loss = sae.compute_loss(gbatch, update_dead_statistics=trainer.update_dead_statistics, return_aux_data=False, **kw)
+            loss.backward()
+            if defer:
+                assert sae.W_D.grad is None and sae.W_D._sparse_grad is not None
+            opt.step()
+            opt.zero_grad()
+            losses.append(loss.item())
+        finals.append(({nm: p.detach().clone() for nm, p in sae.named_parameters()}, losses))
+    (pa, la), (pb, lb) = finals
+    assert la == lb and la[-1] < la[0]
+    for nm in pa:
+        assert pa[nm].dtype == torch.bfloat16 and torch.equal(pa[nm], pb[nm]), nm
+
+
+@pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
 @pytest.mark.parametrize("amp", [False, True])
 def test_auxk_selection_is_the_reference_op_sequence_on_both_routes(pkg, oracle, dev, act_fn, amp):
     """The aux-k term's own selection among the dead features: `hidden_pre * is_dead * decoder_norm` with hidden_pre the
