@@ -277,7 +277,7 @@ class _FixedDead:
         return self.is_dead
 
 
-def build_batchtopk(pkg, dev, args):
+def build_batchtopk(pkg, dev, args, bf16_params=False):
     """BatchTopK SAE d=2048, F=32768, 8192 tokens, global top 64 x 8192, aux-k on the top 512 dead features."""
     import torch
     from lm_saes_amd import synthetic
@@ -285,7 +285,7 @@ def build_batchtopk(pkg, dev, args):
     B, d, F, k = args.batch or 8192, 2048, 32768, 64
     cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="batchtopk",
                         top_k=k, norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda",
-                        dtype=torch.float32)
+                        dtype=torch.bfloat16 if bf16_params else torch.float32)
     sae = pkg.SparseAutoEncoder(cfg)
     x = synthetic.activations(B, d, 32, seed=4).to(dev)
     _init_sae_on_device(sae, x, d)
@@ -294,8 +294,14 @@ def build_batchtopk(pkg, dev, args):
     batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
     opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=4e-4, model=sae)
     kw = dict(auxk_coefficient=1.0 / 32, k_aux=512, update_dead_statistics=dead.update_dead_statistics)
-    name = f"batchtopk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} aux-k=512 (10% of features dead) bf16 adam"
+    name = (f"batchtopk_sae_train_step d_model={d} d_sae={F} k={k} batch={B} aux-k=512 (10% of features dead) "
+            + ("bf16-parameters adam" if bf16_params else "bf16 adam"))
     return _autocast_step(sae, batch, opt, kw), B, name, (B, d, F, k)
+
+
+def build_batchtopk_bf16_params(pkg, dev, args):
+    """The BatchTopK + aux-k workload with the dictionary itself held in bf16 (cfg.dtype = bfloat16): a secondary figure."""
+    return build_batchtopk(pkg, dev, args, bf16_params=True)
 
 
 def build_jumprelu(pkg, dev, args):
@@ -398,7 +404,7 @@ def build_lorsa(pkg, dev, args):
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
-WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
+WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "batchtopk_bf16_params": build_batchtopk_bf16_params, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
              "lorsa": build_lorsa}
 
 
@@ -522,7 +528,7 @@ def main():
 
     ms_per_step, kernels, loss, tokens, name, shape = gpu_step_bench(args)
     work = algorithmic_work(*shape)
-    if args.workload == "topk_bf16_params":   # bf16 p, m, v read and written; no shadow copy
+    if args.workload in ("topk_bf16_params", "batchtopk_bf16_params"):   # bf16 p, m, v read and written; no shadow copy
         work["adam_step_sparse_rows[bf16 dense]"] = ("hbm", shape[1] * shape[2] * 12)
         work["adam_step[vector]"] = ("hbm", (shape[1] + shape[2]) / 2 * 14)
     known = {}     # launches whose work is known although the workload runs other kernels on several shapes

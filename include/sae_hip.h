@@ -344,7 +344,8 @@ int sae_adam_step_sparse_rows(const int32_t *feat_ptr, const int32_t *feat_slot,
  * parameter is its own bf16 operand), and the update rounds to bf16 after every element-wise operation torch
  * performs -- the gradient itself; lerp for m; mul, then addcmul for v; sqrt, the division by sqrt(1 - beta2^t)
  * and the addition of eps for the denominator; addcdiv for p.  row_norm_out is the fp32 norm of the updated bf16
- * rows.  No dense extra block (aux-k on a bf16 dictionary takes the reference's dense route). */
+ * rows.  extra_map / extra_rows / extra_bias as in sae_adam_step_sparse_rows (fp32 rows, added before the gradient is
+ * rounded to bf16). */
 int sae_adam_step_lowp(void *p_bf16, const void *g, int g_dtype, void *m_bf16, void *v_bf16, int64_t n, double lr,
                        double beta1, double beta2, double eps, int64_t step, float *row_norm_out, int64_t row_len,
                        const float *row_grad_coef, void *stream);
@@ -353,7 +354,8 @@ int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int32_t *feat_
                                    void *v_bf16, int64_t F, int64_t d, double lr, double beta1, double beta2,
                                    double eps, int64_t step, float *row_norm_out, float *bias_grad_out,
                                    const float *grad_scale, double *grad_sq_nnz_acc, void *workspace,
-                                   int64_t workspace_bytes, void *stream);
+                                   int64_t workspace_bytes, const int32_t *extra_map, const float *extra_rows,
+                                   const float *extra_bias, void *stream);
 
 /* SparseAdam (optim.py:142-254) over n contiguous fp32 elements: m *= b1, v *= b2 everywhere;
  * where g != 0 also m += (1-b1) g, v += (1-b2) g^2 and

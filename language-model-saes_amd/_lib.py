@@ -52,7 +52,7 @@ SIGNATURES = {
     "sae_grad_sq_nnz": (_I, [_P, _L, _P, _P]),
     "sae_adam_step_sparse_rows": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P]),
     "sae_adam_step_lowp": (_I, [_P, _P, _I, _P, _P, _L, _F, _F, _F, _F, _L, _P, _L, _P, _P]),
-    "sae_adam_step_sparse_rows_lowp": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _L, _P]),
+    "sae_adam_step_sparse_rows_lowp": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _F, _F, _F, _F, _L, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P]),
     "sae_gather_rows": (_I, [_P, _I, _P, _L, _L, _L, _P, _I, _F, _P]),
     "sae_transpose_to_bf16": (_I, [_P, _I, _P, _L, _L, _P, _P, _P]),
     "sae_code_to_dense": (_I, [_P, _P, _P, _P, _L, _L, _P, _P, _P]),

@@ -570,7 +570,7 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
 #define SAE_ADAM_ROWS_LOWP(BF, UU)                                                                                      \
   hipLaunchKernelGGL((adam_sparse_rows_persistent_kernel<BF, UU, true>), dim3(grid), dim3(256), 0, st, feat_ptr, feat_slot, \
                      slot_tok, coef, dense, p, m, v, (int)F, (int)d, a, nullptr, row_norm_out, bias_grad_out, grad_scale,  \
-                     partial, nullptr, nullptr, nullptr)
+                     partial, extra_map, extra_rows, extra_bias)
       if (dense_dtype == SAE_BF16) {
         if (d <= 1024) SAE_ADAM_ROWS_LOWP(true, 1); else SAE_ADAM_ROWS_LOWP(true, 2);
       } else {
@@ -608,12 +608,13 @@ extern "C" int sae_adam_step_sparse_rows_lowp(const int32_t *feat_ptr, const int
                                               void *m_bf16, void *v_bf16, int64_t F, int64_t d, double lr, double beta1,
                                               double beta2, double eps, int64_t step, float *row_norm_out,
                                               float *bias_grad_out, const float *grad_scale, double *grad_sq_nnz_acc,
-                                              void *workspace, int64_t workspace_bytes, void *stream) {
+                                              void *workspace, int64_t workspace_bytes, const int32_t *extra_map,
+                                              const float *extra_rows, const float *extra_bias, void *stream) {
   return sae::adam_step_sparse_rows_impl(true, feat_ptr, feat_slot, slot_tok, coef, dense, dense_dtype,
                                          reinterpret_cast<float *>(p_bf16), reinterpret_cast<float *>(m_bf16),
                                          reinterpret_cast<float *>(v_bf16), F, d, lr, beta1, beta2, eps, step, nullptr,
                                          row_norm_out, bias_grad_out, grad_scale, grad_sq_nnz_acc, workspace,
-                                         workspace_bytes, nullptr, nullptr, nullptr, nullptr, stream);
+                                         workspace_bytes, extra_map, extra_rows, extra_bias, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -753,12 +753,12 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
     `grad_scale` (device float scalar) multiplies the gradient first (gradient clipping);
     `grad_sq_nnz_acc` (device double[2]) += (sum g^2, #non-zero g) of the gradient consumed;
     `extra` adds a densely held block of gradient rows.  A bf16 `p` (with bf16 `m`, `v`) takes the low-precision
-    update (no shadow copy, no extra block)."""
+    update (no shadow copy, no row coefficient)."""
     lowp = p.dtype == torch.bfloat16
     for name, t in (("p", p), ("m", m), ("v", v)):
         _req(t, name, torch.bfloat16 if lowp else torch.float32, 2)
-    if lowp and (shadow_bf16 is not None or extra is not None or row_grad_coef is not None):
-        raise ValueError("the low-precision update takes neither a shadow copy, a dense row block nor a row coefficient")
+    if lowp and (shadow_bf16 is not None or row_grad_coef is not None):
+        raise ValueError("the low-precision update takes neither a shadow copy nor a row coefficient")
     if row_grad_coef is not None:
         _req(row_grad_coef, "row_grad_coef", torch.float32, 1)
         if row_grad_coef.numel() != p.shape[0]:
@@ -786,7 +786,8 @@ def adam_step_sparse_rows(fi: FeatureIndex, coef: torch.Tensor, dense: torch.Ten
                                                            coef.data_ptr(), dense.data_ptr(), _dt(dense), p.data_ptr(),
                                                            m.data_ptr(), v.data_ptr(), F, d, lr, beta1, beta2, eps, int(step),
                                                            _ptr(row_norm_out), _ptr(bias_grad_out), _ptr(grad_scale),
-                                                           _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, _stream(p)),
+                                                           _ptr(grad_sq_nnz_acc), _ptr(ws), ws_bytes, *_extra_ptrs(extra, F, d),
+                                                           _stream(p)),
                 "adam_step_sparse_rows_lowp",
             )
             return

@@ -127,7 +127,7 @@ def _aux_block_fits(B: int, d: int, amp: bool) -> bool:
 
 
 def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux: int, batch_wide: bool, amp: bool,
-                     n_dead: Optional[int] = None):
+                     n_dead: Optional[int] = None, lowp: bool = False):
     """Forward half of the aux-k term on a compacted dead block.  Gathers the dead features' encoder / decoder
     rows into [n, d] matrices (n = #dead padded to the GEMM's K granule), recomputes their pre-activations with
     the encoder GEMM (same kernel, same accumulation order as the full product: identical values), selects among
@@ -173,12 +173,10 @@ def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_au
     kk = min(k_aux, nd)
     # with a norm scale the keys are `hidden_pre * is_dead * decoder_norm` op for op, hidden_pre being the quotient the
     # encoder returned (models/sparse_dictionary.py:958-966): the select's masked arithmetic with every block column in
-    if s_d is not None:
-        keep = torch.ones(ndp, dtype=torch.float32, device=dev)
-        code_d = (ops.select_topk_batch(pre_d, b_d, s_d, kk * B, feat_mask=keep) if batch_wide
-                  else ops.select_topk_row(pre_d, b_d, s_d, kk, feat_mask=keep))
-    else:
-        code_d = ops.select_topk_batch(pre_d, b_d, None, kk * B) if batch_wide else ops.select_topk_row(pre_d, b_d, None, kk)
+    # (`lowp`: a dictionary held in bf16, whose tensors around the select are bf16)
+    keep = torch.ones(ndp, dtype=torch.float32, device=dev) if s_d is not None else None
+    code_d = (ops.select_topk_batch(pre_d, b_d, s_d, kk * B, feat_mask=keep, lowp=lowp) if batch_wide
+              else ops.select_topk_row(pre_d, b_d, s_d, kk, feat_mask=keep, lowp=lowp))
     # dense [B, ndp] activations of the block: fp32 (the mask of the backward pass) and, under autocast, bf16
     A, A_b16 = ops.code_to_dense(code_d, ndp, want_f32=True, want_bf16=amp)
     A_op = A_b16 if amp else A
@@ -303,14 +301,13 @@ class _FusedSparseStep(torch.autograd.Function):
             ctx.aux_dense = None
             dense_block = None
             recon = None
-            # (a dictionary held in bf16 takes the stacked sparse code: the dense block's kernels have no bf16 state)
-            if aux.get("dense", True) and not lowp and _aux_block_fits(x_op.shape[0], x_op.shape[1], amp):
+            if aux.get("dense", True) and _aux_block_fits(x_op.shape[0], x_op.shape[1], amp):
                 # the block is sized by #dead: the count is fetched while the main decode, which does not depend on
                 # it, runs
                 count = _DeadCount(dead)
                 recon = ops.sparse_decode_fwd(code, w_dec_op, b_D)
                 dense_block = _aux_dense_block(x_op, pre.dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_aux, batch_wide, amp,
-                                               n_dead=count.value())
+                                               n_dead=count.value(), lowp=lowp)
             sae._last_aux_route = "dense" if dense_block is not None else "sparse"
             if dense_block is not None:
                 # The dead block is small and hit by a large share of the tokens: its part of the step is three small

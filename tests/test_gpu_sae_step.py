@@ -471,17 +471,19 @@ def test_fused_auxk_step_matches_oracle(pkg, oracle, dev, act_fn, include_norm, 
 
 
 @pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
-def test_auxk_step_with_bf16_parameters(pkg, oracle, dev, act_fn):
-    """aux-k on a dictionary held in bf16 (the stacked sparse code): the aux selection is the reference's bf16 op sequence
-    exactly; losses and gradients agree with the oracle on CPU bf16 tensors to bf16 tolerance; three Adam steps with
-    factored and with dense gradients end at the same bits."""
-    print(f"aux-k step, bf16 parameters, {act_fn}", flush=True)
+@pytest.mark.parametrize("route", ["dense", "sparse"])
+def test_auxk_step_with_bf16_parameters(pkg, oracle, dev, act_fn, route):
+    """aux-k on a dictionary held in bf16, on the compact dense block and on the stacked sparse code: the aux selection
+    is the reference's bf16 op sequence exactly; losses and gradients agree with the oracle on CPU bf16 tensors to bf16
+    tolerance; three Adam steps with factored and with dense gradients end at the same bits."""
+    print(f"aux-k step, bf16 parameters, {act_fn}, route={route}", flush=True)
     B, F, k, k_aux = 192, 2048, 16, 32
     kw = dict(auxk_coefficient=1 / 32, k_aux=k_aux)
 
     def fresh():
         sae, ref, batch = make_pair_act(pkg, oracle, dev, act_fn, d=256, F=F, k=k, B=B, r=8, seed=15, include_norm=True,
                                         dtype=torch.bfloat16)
+        sae.aux_dense_block = route == "dense"
         trainer = pkg.Trainer(pkg.TrainerConfig(auxk_coefficient=1 / 32, k_aux=k_aux, dead_threshold=float(B)))
         trainer._initialize_dead_statistics(sae)
         warm = torch.zeros(B, F); warm[:, ::7] = 1.0
@@ -494,7 +496,7 @@ def test_auxk_step_with_bf16_parameters(pkg, oracle, dev, act_fn):
     gbatch = {k_: v.to(dev) for k_, v in batch.items()}
     ctx = sae.compute_loss(gbatch, update_dead_statistics=trainer.update_dead_statistics, **kw)
     ctx["loss"].backward()
-    assert "sparse_code" in ctx and sae._last_aux_route == "sparse"
+    assert "sparse_code" in ctx and sae._last_aux_route == route
     # the reference's sequence on bf16 tensors, from the kernel's own product
     pre = pkg.ops.encoder_gemm(pkg.ops.cast_bf16(gbatch["in"].float().contiguous()), sae._w_enc_operand(True), torch.bfloat16).cpu()
     n = sae._decoder_norm_nograd().cpu().bfloat16()
