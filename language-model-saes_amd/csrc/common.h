@@ -50,6 +50,11 @@ __device__ __forceinline__ void bf16_round2(float &x, float &y) {
   x = __uint_as_float(packed << 16);
   y = __uint_as_float(packed & 0xffff0000u);
 }
+// two fp32 values rounded to bf16 (round-to-nearest-even) and packed, `lo` in the low half
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const cvt_f32x2 in = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, cvt_bf16x2));
+}
 __device__ __forceinline__ float bf16_round(float x) {
   float y = x;
   bf16_round2(x, y);

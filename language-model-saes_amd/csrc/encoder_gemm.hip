@@ -84,12 +84,6 @@ __device__ __forceinline__ void mma_chunk_f32(const u32x4 &wf, const u32x4 &xf, 
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
 }
 
-// two floats -> two bf16, round to nearest even: the packed hardware conversion
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  const cvt_f32x2 in = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, cvt_bf16x2));
-}
-
 // ---- fp32 operands ---------------------------------------------------------------------------------------------
 template <bool BF16_OUT>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(

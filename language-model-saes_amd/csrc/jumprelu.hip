@@ -1,5 +1,7 @@
 // JumpReLU activation with its straight-through threshold gradient and the sparsity penalties that read
-// the same [B, F] data, as two streaming passes (forward, backward).  Both are HBM-bound: the forward
+// the same [B, F] data, as two streaming passes (forward, backward).  Each element is read and written once, but at
+// bf16 the passes run at about half the memory system's rate: two dozen vector instructions per element (a division,
+// a tanh, conversions) and, in the forward, the per-feature vectors re-read from L2 set the pace.  The forward
 // reads the pre-activation and writes the activation once; the backward reads the pre-activation and
 // the incoming gradient once, writes the pre-activation gradient once, and reduces three per-feature
 // sums (bias, threshold, decoder-norm gradients) through per-row-group partials that a second kernel
@@ -57,10 +59,10 @@ template <bool BF16, bool STREAM = false>
 __device__ __forceinline__ void store8(void *__restrict__ p, int64_t g, const float (&v)[8]) {
   if constexpr (BF16) {
     u32x4 o;
-    o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
-    o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
-    o.z = (uint32_t)f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
-    o.w = (uint32_t)f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+    o.x = pack_bf16x2(v[0], v[1]);
+    o.y = pack_bf16x2(v[2], v[3]);
+    o.z = pack_bf16x2(v[4], v[5]);
+    o.w = pack_bf16x2(v[6], v[7]);
     if constexpr (STREAM) {
       const nt_u32x4 t = {o.x, o.y, o.z, o.w};
       __builtin_nontemporal_store(t, reinterpret_cast<nt_u32x4 *>(p) + g);
@@ -93,50 +95,82 @@ __device__ __forceinline__ float tanh_pos(float x) {
     return x * (1.f - x2 * (0.33333334f - 0.13333334f * x2));
   }
   const float e = __expf(2.f * x);
-  return 1.f - 2.f / (e + 1.f);
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);   // the reciprocal's 1 ulp is 1e-7 of the result at most
 }
 
-// one block per token row
+// u / s.  The fp32 instantiations keep the correctly rounded quotient; the bf16 ones, whose result is rounded to 8 bits
+// of mantissa right away, take the hardware reciprocal with one correction step (the passes are bound by their
+// arithmetic, and the IEEE sequence is a quarter of it).
+template <bool BF16>
+__device__ __forceinline__ float jr_div(float u, float s) {
+  if constexpr (BF16) {
+    const float r = __builtin_amdgcn_rcpf(s);
+    const float q = u * r;
+    return fmaf(fmaf(-q, s, u), r, q);
+  } else {
+    return u / s;
+  }
+}
+
+// one block per JR_FWD_ROWS token rows: the per-feature vectors (bias, scale, penalty norm, threshold: 128 bytes per
+// lane and step against 16 bytes of a bf16 row) are fetched once for all of them
+constexpr int JR_FWD_ROWS = 4;
 template <bool BF16>
 __global__ __launch_bounds__(JR_THREADS) void jumprelu_fwd_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ pen, const float *__restrict__ theta, int64_t B, int64_t F, float tanh_c,
     void *__restrict__ acts, float *__restrict__ tanh_tok, float *__restrict__ lp_tok, float *__restrict__ l0_tok) {
   __shared__ float red[JR_THREADS / 64];
-  const int64_t row = blockIdx.x;
+  constexpr int R = JR_FWD_ROWS;
+  const int64_t row0 = (int64_t)blockIdx.x * R;
+  const int n_rows = (int)((B - row0) < R ? (B - row0) : R);
   const int64_t groups = F >> 3;
-  const int64_t rbase = row * groups;
-  float tsum = 0.f, lpsum = 0.f, cnt = 0.f;
+  float tsum[R], lpsum[R], cnt[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) tsum[r] = lpsum[r] = cnt[r] = 0.f;
   for (int64_t g = threadIdx.x; g < groups; g += JR_THREADS) {
-    float p[8], b[8], s[8], np[8], th[8], a[8];
-    load8<BF16, true>(pre, rbase + g, p);
+    float p[R][8], b[8], s[8], np[8], th[8];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (r < n_rows) load8<BF16, true>(pre, (row0 + r) * groups + g, p[r]);
     load8_f32_or(b_enc, g, 0.f, b);
     load8_f32_or(scale, g, 1.f, s);
     load8_f32_or(pen, g, 1.f, np);
     load8<false>(theta, g, th);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float h = p[i] + b[i];
-      const float u = mul_rn(h, s[i]);
-      const bool keep = u > th[i];
-      a[i] = keep ? (scale ? u / s[i] : h) : 0.f;
-      cnt += keep ? 1.f : 0.f;
-      if (tanh_tok && keep) tsum += tanh_pos(tanh_c * a[i] * np[i]);
-      if (lp_tok) lpsum += fmaxf(th[i] - h, 0.f) * np[i];
+    for (int r = 0; r < R; ++r) {
+      if (r < n_rows) {
+        float a[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float h = p[r][i] + b[i];
+          const float u = mul_rn(h, s[i]);
+          const bool keep = u > th[i];
+          a[i] = keep ? (scale ? jr_div<BF16>(u, s[i]) : h) : 0.f;
+          cnt[r] += keep ? 1.f : 0.f;
+          if (tanh_tok && keep) tsum[r] += tanh_pos(tanh_c * a[i] * np[i]);
+          if (lp_tok) lpsum[r] += fmaxf(th[i] - h, 0.f) * np[i];
+        }
+        store8<BF16, true>(acts, (row0 + r) * groups + g, a);
+      }
     }
-    store8<BF16, true>(acts, rbase + g, a);
   }
-  if (tanh_tok) {
-    const float t = block_sum<JR_THREADS / 64>(tsum, red);
-    if (threadIdx.x == 0) tanh_tok[row] = t;
-  }
-  if (lp_tok) {
-    const float t = block_sum<JR_THREADS / 64>(lpsum, red);
-    if (threadIdx.x == 0) lp_tok[row] = t;
-  }
-  if (l0_tok) {
-    const float t = block_sum<JR_THREADS / 64>(cnt, red);
-    if (threadIdx.x == 0) l0_tok[row] = t;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r < n_rows) {   // uniform over the block
+      if (tanh_tok) {
+        const float t = block_sum<JR_THREADS / 64>(tsum[r], red);
+        if (threadIdx.x == 0) tanh_tok[row0 + r] = t;
+      }
+      if (lp_tok) {
+        const float t = block_sum<JR_THREADS / 64>(lpsum[r], red);
+        if (threadIdx.x == 0) lp_tok[row0 + r] = t;
+      }
+      if (l0_tok) {
+        const float t = block_sum<JR_THREADS / 64>(cnt[r], red);
+        if (threadIdx.x == 0) l0_tok[row0 + r] = t;
+      }
+    }
   }
 }
 
@@ -176,7 +210,7 @@ __global__ __launch_bounds__(JR_THREADS) void jumprelu_bwd_kernel(
       const bool keep = u > th[i];
       float gtot = ga[i];
       if (g_tanh) {
-        const float a = keep ? (scale ? u / s[i] : h) : 0.f;
+        const float a = keep ? (scale ? jr_div<BF16>(u, s[i]) : h) : 0.f;
         const float t = keep ? tanh_pos(tanh_c * a * np[i]) : 0.f;
         const float sech2 = 1.f - t * t;
         gtot += gt * np[i] * sech2;
@@ -441,7 +475,7 @@ extern "C" int sae_jumprelu_fwd(const void *pre, int dtype, const float *b_enc, 
   int rc = check_shape("jumprelu_fwd", pre, dtype, theta, b_enc, scale, B, F);
   if (rc) return rc;
   SAE_REQUIRE(acts && (((uintptr_t)acts) & 15) == 0, SAE_ERR_INVALID_ARG, "jumprelu_fwd: acts must be a 16-byte aligned buffer");
-  const unsigned fwd_blocks = (unsigned)B;
+  const unsigned fwd_blocks = (unsigned)((B + JR_FWD_ROWS - 1) / JR_FWD_ROWS);
   if (dtype == SAE_BF16)
     hipLaunchKernelGGL(jumprelu_fwd_kernel<true>, dim3(fwd_blocks), dim3(JR_THREADS), 0, st, pre, b_enc, scale, pen_norm,
                        theta, B, F, tanh_c, acts, tanh_tok, lp_tok, l0_tok);
