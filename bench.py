@@ -379,7 +379,7 @@ def build_clt(pkg, dev, args):
     return _autocast_step(clt, batch, opt, {}), B, name, (B, d, F, k)
 
 
-def build_lorsa(pkg, dev, args):
+def build_lorsa(pkg, dev, args, positional="none"):
     """Lorsa: d=768, 16 sequences x 1024 tokens, 64 query/key heads of width 64, 8192 value/output heads
     (128 per query/key head), k=64; target = causal softmax attention of a seeded rank-64 head set."""
     import torch
@@ -387,7 +387,7 @@ def build_lorsa(pkg, dev, args):
 
     nb, s, d, F, h, dq, k = 16, 1024, 768, 8192, 64, 64, 64
     cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
-                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type="none", act_fn="topk", top_k=k,
+                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type=positional, act_fn="topk", top_k=k,
                           norm_activation="inference", device="cuda", dtype=torch.float32)
     m = pkg.LowRankSparseAttention(cfg)
     m.init_parameters()
@@ -400,12 +400,19 @@ def build_lorsa(pkg, dev, args):
                                                              is_causal=True, scale=1 / 8)[:, 0]
     batch = {"in": x, "out": y.contiguous(), "tokens": torch.zeros(nb, s, dtype=torch.long, device=dev)}
     opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=4e-4, model=m)
-    name = f"lorsa_train_step d_model={d} sequences={nb}x{s} qk_heads={h}x{dq} ov_heads={F} k={k} bf16 adam"
+    name = (f"lorsa_train_step d_model={d} sequences={nb}x{s} qk_heads={h}x{dq} ov_heads={F} k={k} "
+            + ("rotary " if positional == "rotary" else "") + "bf16 adam")
     return _autocast_step(m, batch, opt, {}), nb * s, name, (nb * s, d, F, k)
 
 
+def build_lorsa_rotary(pkg, dev, args):
+    """The Lorsa workload with rotary embeddings on queries and keys (the reference's default; BASELINE's configuration has
+    none): a secondary figure."""
+    return build_lorsa(pkg, dev, args, positional="rotary")
+
+
 WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "batchtopk_bf16_params": build_batchtopk_bf16_params, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
-             "lorsa": build_lorsa}
+             "lorsa": build_lorsa, "lorsa_rotary": build_lorsa_rotary}
 
 
 def gpu_step_bench(args):
@@ -532,7 +539,7 @@ def main():
         work["adam_step_sparse_rows[bf16 dense]"] = ("hbm", shape[1] * shape[2] * 12)
         work["adam_step[vector]"] = ("hbm", (shape[1] + shape[2]) / 2 * 14)
     known = {}     # launches whose work is known although the workload runs other kernels on several shapes
-    if args.workload == "lorsa":
+    if args.workload in ("lorsa", "lorsa_rotary"):
         # causal attention of build_lorsa's shape: (query, key) pairs with key <= query, 2 flop per multiply-add;
         # forward = scores + weighted values; backward = scores again, dP, dV, dK, dQ (the algorithmic minimum: the
         # three backward kernels each recompute the scores they need)

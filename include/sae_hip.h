@@ -534,6 +534,22 @@ int sae_attention_bwd(const void *q, const void *k, const void *v, const void *o
                       int64_t n_batch, int64_t seq, int64_t n_heads, int64_t d_qk, int64_t d_v, double scale, float *workspace,
                       void *dqt, void *dkt, void *dvt, void *stream);
 
+/* Rotary positional embedding of Lorsa's queries / keys between projection and scores (models/lorsa.py:821-824, 864-904;
+ * tables as models/lorsa.py:525-575 builds them, cos / sin fp32 [n_ctx, rotary_dim]).  acc fp32 [T, n_heads d_head] holds
+ * the projection's accumulators, T = batches x seq tokens, a token's position is its index inside its sequence;
+ *   out = bf16(rotate(float(bf16(acc)) + bias)),
+ * i.e. the bf16 product plus the fp32 bias, rotated in fp32 and rounded once, as the reference's tensors are under bf16
+ * autocast.  The first rotary_dim elements of a head are rotated in pairs (adjacent_pairs: (2i, 2i+1), else
+ * (j, j + rotary_dim / 2)), the rest pass through.  rotary_dim a multiple of 16, d_head and seq multiples of 8. */
+int sae_rotary_fwd(const float *acc, const float *bias, const float *cos_tab, const float *sin_tab, int64_t n_ctx, int64_t T,
+                   int64_t seq, int64_t n_heads, int64_t d_head, int64_t rotary_dim, int adjacent_pairs, void *out_bf16,
+                   void *stream);
+/* The transpose of that rotation, in place on a gradient held transposed, grad_t bf16 [n_heads d_head, T] (what
+ * sae_attention_bwd leaves for queries and keys): rows in pairs, dx[a] = dy[a] cos[a] + dy[b] sin[b],
+ * dx[b] = dy[b] cos[b] - dy[a] sin[a], rounded to bf16.  cos_t / sin_t are the tables transposed, fp32 [rotary_dim, n_ctx]. */
+int sae_rotary_bwd_t(void *grad_t_bf16, const float *cos_t, const float *sin_t, int64_t n_ctx, int64_t T, int64_t seq,
+                     int64_t n_heads, int64_t d_head, int64_t rotary_dim, int adjacent_pairs, void *stream);
+
 /* out[r] = sum_c src[r, c] (fp32 sum, fixed order) for src [rows, cols] fp32 or bf16.  The bias gradients autograd forms by
  * summing over tokens, for gradients held transposed ([features, tokens]). */
 int sae_row_sum(const void *src, int src_dtype, int64_t rows, int64_t cols, float *out, void *stream);

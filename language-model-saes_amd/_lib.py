@@ -67,6 +67,8 @@ SIGNATURES = {
     "sae_jumprelu_bwd_workspace_bytes": (_L, [_L, _L]),
     "sae_attention_fwd": (_I, [_P, _P, _P, _L, _L, _L, _L, _L, _F, _P, _P, _P]),
     "sae_attention_bwd": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _F, _P, _P, _P, _P, _P]),
+    "sae_rotary_fwd": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _P, _P]),
+    "sae_rotary_bwd_t": (_I, [_P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _P]),
     "sae_row_sum": (_I, [_P, _I, _L, _L, _P, _P]),
     "sae_dense_row_nnz": (_I, [_P, _I, _L, _L, _P, _P]),
     "sae_dense_to_code": (_I, [_P, _I, _L, _L, _P, _P, _P, _L, _P]),

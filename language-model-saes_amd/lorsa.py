@@ -12,7 +12,7 @@ attention kernels (no [s, s] matrix, no padding of the narrower query / key head
 the weight gradients of the projections are GEMM-kernel products over the token axis, and the TopK
 select, the sparse decode through `W_O`, the squared error, the `W_O` gradient rows and the scatter of
 the value gradients back to the dense pre-activation are the sparse kernels of the SAE path.  In fp32,
-with rotary embeddings or query / key norms, or with user hooks on the attention internals, the
+with query / key norms, or with user hooks on the attention internals, the
 projections and the mixing are torch library routines.
 """
 
@@ -80,9 +80,11 @@ class _ValueProjection(torch.autograd.Function):
 
 class _ProjectAndMix(torch.autograd.Function):
     """x -> q, k, v projections -> causal attention mixing -> hidden_pre [T, F] (bf16), all on the GEMM and attention
-    kernels, for the configuration without rotary embedding and query / key norms.
+    kernels, for configurations without query / key norms.
 
     forward : q = x W_Q, k = x W_K as [T, h dq], v = x W_V as [T, F]; the biases are added in the products' epilogues.
+              With rotary embeddings q and k leave their products as fp32 accumulators, and one element-wise kernel
+              rounds them, adds the bias and rotates (`ops.rotary_fwd`); the backward un-rotates d q^T, d k^T in place.
     backward: the attention backward takes the same operands (products over positions read their tiles across the
               rows) and returns dq^T, dk^T, dv^T [., T] in one buffer, which is exactly the operand of the
               weight-gradient product dW = d(.)^T x over the token axis (one GEMM for the three); bias gradients are its
@@ -99,13 +101,22 @@ class _ProjectAndMix(torch.autograd.Function):
         # gets under autocast); added per tile inside the attention kernels they would be re-added for every
         # (query block, key block) pair and cost those kernels as many vector instructions as their softmax
         flat = lambda b: b.detach().float().reshape(-1).contiguous()        # noqa: E731
-        q = ops.encoder_gemm_bias(x_op, wq, col_bias=flat(b_Q))             # [T, h dq]
-        k = ops.encoder_gemm_bias(x_op, wk, col_bias=flat(b_K))
+        rot = model._rotary_tables() if cfg.positional_embedding_type == "rotary" else None
+        if rot is None:
+            q = ops.encoder_gemm_bias(x_op, wq, col_bias=flat(b_Q))         # [T, h dq]
+            k = ops.encoder_gemm_bias(x_op, wk, col_bias=flat(b_K))
+        else:
+            cos, sin = rot[0], rot[1]
+            q = ops.rotary_fwd(ops.encoder_gemm(x_op, wq, torch.float32), flat(b_Q), cos, sin, seq, h, cfg.rotary_dim,
+                               cfg.rotary_adjacent_pairs)
+            k = ops.rotary_fwd(ops.encoder_gemm(x_op, wk, torch.float32), flat(b_K), cos, sin, seq, h, cfg.rotary_dim,
+                               cfg.rotary_adjacent_pairs)
         v = ops.encoder_gemm_bias(x_op, wv, col_bias=flat(b_V))             # [T, F]
         scale = 1.0 / model.attn_scale
         out, lse = ops.attention_fwd(q, k, v, n_batch, seq, h, scale)
         ctx.save_for_backward(x_op, wq, wk, wv, q, k, v, out, lse, b_Q.detach(), b_K.detach(), b_V.detach())
         ctx.dims = (n_batch, seq, h, scale)
+        ctx.rotary = None if rot is None else (rot[2], rot[3], cfg.rotary_dim, cfg.rotary_adjacent_pairs)
         ctx.shapes = (tuple(W_Q.shape), tuple(W_K.shape))
         ctx.x_dtype = x2.dtype
         return out
@@ -120,6 +131,10 @@ class _ProjectAndMix(torch.autograd.Function):
         d = x_op.shape[1]
         n_qk = q.shape[1]
         dq_w = n_qk // h
+        if ctx.rotary is not None:   # the gradients arrive with respect to the rotated q, k
+            cos_t, sin_t, rdim, adjacent = ctx.rotary
+            ops.rotary_bwd_t(stacked[:n_qk], cos_t, sin_t, seq, h, rdim, adjacent)
+            ops.rotary_bwd_t(stacked[n_qk: 2 * n_qk], cos_t, sin_t, seq, h, rdim, adjacent)
         # the three weight gradients d(.)^T x in one product over the token axis: the gradients share one buffer
         # [2 h dq + F, T], and a single launch fills the chip where three would each leave most of it idle
         rows = ops.encoder_gemm(stacked, xt, torch.float32)                 # [2 h dq + F, d]
@@ -323,15 +338,31 @@ class LowRankSparseAttention(SparseDictionary):
         return self._derive(f"{name}.rows.bf16", p, lambda old: ops.cast_bf16(
             p.detach().float().permute(0, 2, 1).reshape(h * dq, d).contiguous(), old))
 
+    def _rotary_tables(self):
+        """(cos, sin [n_ctx, rotary_dim], cos^T, sin^T [rotary_dim, n_ctx]) fp32 on the buffers' device, as the rotary
+        kernels read them; the transposed copies are made once per buffer."""
+        cos, sin = self.rotary_cos, self.rotary_sin
+        key = (cos.data_ptr(), sin.data_ptr(), cos._version, sin._version)
+        cached = getattr(self, "_rotary_t", None)
+        if cached is None or cached[0] != key:
+            c32, s32 = cos.detach().float().contiguous(), sin.detach().float().contiguous()
+            cached = (key, (c32, s32, c32.t().contiguous(), s32.t().contiguous()))
+            self._rotary_t = cached
+        return cached[1]
+
     def _mix_kernel_eligible(self, x: torch.Tensor) -> bool:
         """The projections + mixing run on the GEMM and attention kernels: bf16 autocast over fp32 parameters, no
-        rotary embedding or query / key norm between projection and scores, no user hook on the attention internals,
-        and shapes the kernels are built for."""
+        query / key norm between projection and scores, no user hook on the attention internals, and shapes the kernels
+        (attention, and the rotary embedding when there is one) are built for."""
         cfg = self.cfg
         if not (self.use_mix_kernels and x.is_cuda and x.ndim == 3 and _autocast_dtype("cuda") == torch.bfloat16
                 and self.W_V.dtype == torch.float32):
             return False
-        if cfg.positional_embedding_type == "rotary" or cfg.use_post_qk_ln:
+        if cfg.use_post_qk_ln:
+            return False
+        if cfg.positional_embedding_type == "rotary" and not (
+                ops.rotary_supported(x.shape[1], cfg.d_qk_head, cfg.rotary_dim, cfg.rotary_scale)
+                and x.shape[1] <= self.rotary_cos.shape[0] and self.rotary_cos.is_cuda):
             return False
         if any(getattr(self, f"hook_{n}").has_hooks for n in ("q", "k", "q_post_rot", "k_post_rot", "attn_pattern", "attn_score")):
             return False

@@ -1096,6 +1096,54 @@ def attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.
     return (dqt, dkt, dvt, grads) if return_stacked else (dqt, dkt, dvt)
 
 
+def rotary_supported(seq: int, d_head: int, rotary_dim: int, rotary_scale: int = 1) -> bool:
+    """Shapes `rotary_fwd` / `rotary_bwd_t` take."""
+    return rotary_scale == 1 and seq % 8 == 0 and d_head % 8 == 0 and 0 < rotary_dim <= d_head and rotary_dim % 16 == 0
+
+
+def rotary_fwd(acc: torch.Tensor, bias: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor, seq: int, n_heads: int,
+               rotary_dim: int, adjacent_pairs: bool) -> torch.Tensor:
+    """bf16 [T, n_heads d_head] = rotate(float(bf16(acc)) + bias): the projection's fp32 accumulators `acc`, the bias
+    and the rotary embedding with tables cos / sin fp32 [n_ctx, rotary_dim]; a token's position is its index in its
+    sequence of `seq` tokens."""
+    _req(acc, "acc", torch.float32, 2)
+    T, width = acc.shape
+    for name, t in (("cos", cos), ("sin", sin)):
+        _req(t, name, torch.float32, 2)
+        if t.shape[1] != rotary_dim or t.shape != cos.shape:
+            raise ValueError(f"{name} must be [n_ctx, {rotary_dim}]")
+    if bias is not None:
+        _req(bias, "bias", torch.float32, 1)
+        if bias.numel() != width:
+            raise ValueError(f"bias must have {width} elements")
+    if width % n_heads:
+        raise ValueError("acc's width must be a multiple of n_heads")
+    out = torch.empty(T, width, dtype=torch.bfloat16, device=acc.device)
+    with _timed("rotary_fwd"):
+        check(_lib.load().sae_rotary_fwd(acc.data_ptr(), _ptr(bias), cos.data_ptr(), sin.data_ptr(), cos.shape[0], T, int(seq),
+                                         int(n_heads), width // n_heads, int(rotary_dim), int(bool(adjacent_pairs)),
+                                         out.data_ptr(), _stream(acc)), "rotary_fwd")
+    return out
+
+
+def rotary_bwd_t(grad_t: torch.Tensor, cos_t: torch.Tensor, sin_t: torch.Tensor, seq: int, n_heads: int, rotary_dim: int,
+                 adjacent_pairs: bool) -> None:
+    """In place on grad_t bf16 [n_heads d_head, T] (a gradient with respect to rotated queries / keys, transposed): the
+    gradient with respect to what was rotated.  cos_t / sin_t: the tables transposed, fp32 [rotary_dim, n_ctx]."""
+    _req(grad_t, "grad_t", torch.bfloat16, 2)
+    rows, T = grad_t.shape
+    for name, t in (("cos_t", cos_t), ("sin_t", sin_t)):
+        _req(t, name, torch.float32, 2)
+        if t.shape[0] != rotary_dim or t.shape != cos_t.shape:
+            raise ValueError(f"{name} must be [{rotary_dim}, n_ctx]")
+    if rows % n_heads:
+        raise ValueError("grad_t's rows must be a multiple of n_heads")
+    with _timed("rotary_bwd_t"):
+        check(_lib.load().sae_rotary_bwd_t(grad_t.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), cos_t.shape[1], T, int(seq),
+                                           int(n_heads), rows // n_heads, int(rotary_dim), int(bool(adjacent_pairs)),
+                                           _stream(grad_t)), "rotary_bwd_t")
+
+
 def row_sum(src: torch.Tensor) -> torch.Tensor:
     """fp32 [rows] = sum over the columns of a bf16 / fp32 matrix [rows, cols]."""
     _req(src, "src", ndim=2)

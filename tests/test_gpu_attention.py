@@ -156,3 +156,47 @@ def test_row_sum(pkg, dev):
     assert rel_max(pkg.ops.row_sum(src.to(dev)), src.double().sum(1)) < 1e-6
     b = src.to(torch.bfloat16)
     assert rel_max(pkg.ops.row_sum(b.to(dev)), b.double().sum(1)) < 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nb,seq,h,dq,rd,adjacent,with_bias", [(2, 16, 3, 32, 32, True, True), (2, 16, 3, 32, 32, False, True),
+                                                           (1, 40, 2, 64, 32, True, False), (3, 8, 5, 64, 48, False, True),
+                                                           (2, 24, 4, 16, 16, True, True), (16, 1024, 64, 64, 64, True, True)])
+def test_rotary_kernels_follow_the_reference_sequence(pkg, oracle, dev, nb, seq, h, dq, rd, adjacent, with_bias):
+    """models/lorsa.py:864-904 under bf16 autocast: the bf16 product plus the fp32 bias is an fp32 tensor, rotated in
+    fp32 (x * cos + flip(x) * sin), and the attention rounds it to bf16.  The expected values are that sequence with
+    torch on the CPU, its backward torch's autograd through it; both must be reproduced to the bit."""
+    import importlib
+    vo = importlib.import_module("oracle.variants_oracle")
+    print(f"rotary nb={nb} seq={seq} h={h} dq={dq} rd={rd} adjacent={adjacent} bias={with_bias}", flush=True)
+    n_ctx = seq + 8
+    g = torch.Generator().manual_seed(seq * dq + rd)
+    T = nb * seq
+    acc = torch.randn(T, h * dq, generator=g)
+    bias = 0.3 * torch.randn(h * dq, generator=g) if with_bias else None
+    sin, cos = vo.rotary_sin_cos(rd, n_ctx, 10000, adjacent)
+
+    def rotate(x4):      # [b, s, h, dq] fp32, the reference's sequence
+        x_rot, x_pass = x4[..., :rd], x4[..., rd:]
+        flip = x_rot.clone()
+        if adjacent:
+            flip[..., ::2] = -x_rot[..., 1::2]
+            flip[..., 1::2] = x_rot[..., ::2]
+        else:
+            n = rd // 2
+            flip[..., :n] = -x_rot[..., n:]
+            flip[..., n:] = x_rot[..., :n]
+        return torch.cat([x_rot * cos[None, :seq, None, :] + flip * sin[None, :seq, None, :], x_pass], dim=-1)
+
+    x = (acc.bfloat16().float() + (bias if with_bias else 0.0)).view(nb, seq, h, dq).requires_grad_(True)
+    y = rotate(x)
+    want = y.detach().bfloat16().view(T, h * dq)
+    got = pkg.ops.rotary_fwd(acc.to(dev), None if bias is None else bias.to(dev), cos.to(dev), sin.to(dev), seq, h, rd, adjacent)
+    assert torch.equal(got.cpu(), want)
+    # backward: a bf16 gradient with respect to y, held transposed [h dq, T]
+    dy = torch.randn(T, h * dq, generator=g).bfloat16()
+    y.backward(dy.float().view(nb, seq, h, dq))
+    want_dx_t = x.grad.view(T, h * dq).bfloat16().t().contiguous()
+    grad_t = dy.t().contiguous().to(dev)
+    pkg.ops.rotary_bwd_t(grad_t, cos.t().contiguous().to(dev), sin.t().contiguous().to(dev), seq, h, rd, adjacent)
+    assert torch.equal(grad_t.cpu(), want_dx_t)

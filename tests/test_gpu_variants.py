@@ -386,8 +386,21 @@ def test_lorsa_fused_step_fp32(pkg, vo, dev, kw):
 def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b, dense):
     """bf16 autocast: projections on the GEMM kernel, causal mixing and its backward on the attention kernels; W_O's
     gradient as the dense product acts^T grad_recon or as gathered rows."""
+    lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, positional_embedding_type="none")
+
+
+@pytest.mark.parametrize("dq,rotary_dim,adjacent", [(32, 32, True), (32, 32, False), (64, 32, True), (64, 48, False), (32, 16, True)])
+def test_lorsa_fused_step_bf16_with_rotary(pkg, vo, dev, dq, rotary_dim, adjacent):
+    """The same step with rotary embeddings (adjacent or half-split pairs, the whole head or its first elements): the
+    rotation and its transpose run in their own kernels around the attention kernels."""
+    timer = lorsa_bf16_step(pkg, vo, dev, 64, 256, 4, dq, 64, 2, True, positional_embedding_type="rotary",
+                            rotary_dim=rotary_dim, rotary_adjacent_pairs=adjacent)
+    assert "rotary_fwd" in timer.records and "rotary_bwd_t" in timer.records
+
+
+def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, **kw):
     k = 8
-    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=53, positional_embedding_type="none")
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=53, **kw)
     m.dense_decoder_grad = dense
     g = torch.Generator().manual_seed(54)
     with torch.no_grad():      # non-zero projection biases, so that the kernels' bias path is exercised
@@ -409,6 +422,7 @@ def test_lorsa_fused_step_bf16(pkg, vo, dev, d, F, h, dq, s, b, dense):
     kept = (out["feature_acts"] > 0).cpu()
     w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch), kept)
     assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["hidden_pre"], w16["hidden_pre"]) < BF16_TOL
+    return timer
 
 
 def test_lorsa_adam_steps_with_factored_output_gradient(pkg, vo, dev):
