@@ -11,9 +11,10 @@ encoder GEMM kernel (`W_V` is feature-major already; the query / key weights are
 attention kernels (no [s, s] matrix, no padding of the narrower query / key heads to the value width),
 the weight gradients of the projections are GEMM-kernel products over the token axis, and the TopK
 select, the sparse decode through `W_O`, the squared error, the `W_O` gradient rows and the scatter of
-the value gradients back to the dense pre-activation are the sparse kernels of the SAE path.  In fp32,
-with query / key norms, or with user hooks on the attention internals, the
-projections and the mixing are torch library routines.
+the value gradients back to the dense pre-activation are the sparse kernels of the SAE path.  With query / key
+norms, rotary shapes the rotary kernels do not take, or user hooks on q and k, those are formed by torch operations and
+the mixing alone runs on the attention kernels; in fp32, or with hooks on the scores or the pattern, the projections and
+the mixing are torch library routines.
 """
 
 from __future__ import annotations
@@ -154,6 +155,29 @@ class _ProjectAndMix(torch.autograd.Function):
             # rare (activations do not carry gradients in training): library products on the transposed gradients
             dx = (dqt.t().float() @ wq.float() + dkt.t().float() @ wk.float() + dvt.t().float() @ wv.float()).to(ctx.x_dtype)
         return dx, dW_Q, dW_K, dW_V, db_Q, db_K, db_V, None, None
+
+
+class _AttentionMix(torch.autograd.Function):
+    """Causal attention mixing of given bf16 q, k [T, h dq] and v [T, F] on the attention kernels.  For configurations
+    whose queries and keys are formed by other operations than `_ProjectAndMix` knows (query / key norms, rotary widths
+    its kernels do not take, user hooks on q or k): the library attention with its padded heads is still replaced; the
+    gradients go back in the operands' layout for autograd to carry on with."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, n_batch, seq, n_heads, scale):
+        out, lse = ops.attention_fwd(q, k, v, n_batch, seq, n_heads, scale)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.dims = (n_batch, seq, n_heads, scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, dz):
+        q, k, v, out, lse = ctx.saved_tensors
+        n_batch, seq, n_heads, scale = ctx.dims
+        dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
+        dqt, dkt, dvt = ops.attention_bwd(q, k, v, out, dz, lse, n_batch, seq, n_heads, scale)
+        back = lambda t: ops.transpose_to_bf16(t)[0]                        # noqa: E731   [w, T] -> [T, w]
+        return back(dqt), back(dkt), back(dvt), None, None, None, None
 
 
 class _SparseTail(torch.autograd.Function):
@@ -370,6 +394,20 @@ class LowRankSparseAttention(SparseDictionary):
         return (ops.attention_shapes_supported(s, cfg.d_qk_head, cfg.ov_group_size) and d % 64 == 0 and (b * s) % 64 == 0
                 and cfg.d_sae == cfg.n_qk_heads * cfg.ov_group_size)
 
+    def _attention_kernel_eligible(self, x: torch.Tensor) -> bool:
+        """The mixing alone runs on the attention kernels, q, k and v being formed by the general op sequence: what is
+        left when `_mix_kernel_eligible` declines for the way queries and keys are formed (query / key norms, other
+        rotary shapes, hooks on q or k).  Hooks on the scores or the pattern need the [s, s] matrices and keep the
+        library route."""
+        cfg = self.cfg
+        if not (self.use_mix_kernels and x.is_cuda and x.ndim == 3 and _autocast_dtype("cuda") == torch.bfloat16
+                and self.W_V.dtype == torch.float32):
+            return False
+        if self.hook_attn_pattern.has_hooks or self.hook_attn_score.has_hooks:
+            return False
+        return (ops.attention_shapes_supported(x.shape[1], cfg.d_qk_head, cfg.ov_group_size)
+                and cfg.d_sae == cfg.n_qk_heads * cfg.ov_group_size)
+
     def _w_dec_operand(self, amp: bool) -> torch.Tensor:
         w = self.W_O.detach()
         if not amp or w.dtype == torch.bfloat16:
@@ -502,6 +540,11 @@ class LowRankSparseAttention(SparseDictionary):
             z = _ProjectAndMix.apply(x.reshape(b * s, d), self.W_Q, self.W_K, self.W_V, self.b_Q, self.b_K, self.b_V, self, s)
             return z.view(b, s, self.cfg.d_sae)
         q, k, v = self._compute_qkv(x)
+        if self._attention_kernel_eligible(x):
+            b, s, _ = x.shape
+            flat = lambda t: t.reshape(b * s, -1).to(torch.bfloat16).contiguous()    # noqa: E731   (what the library casts to)
+            z = _AttentionMix.apply(flat(q), flat(k), flat(v), b, s, self.cfg.n_qk_heads, 1.0 / self.attn_scale)
+            return z.view(b, s, self.cfg.d_sae)
         query, key = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3)
         value = v.reshape(*k.shape[:3], -1).permute(0, 2, 1, 3)
         amp_dtype = _autocast_dtype(x.device.type)      # under autocast the library casts the three operands itself

@@ -341,8 +341,9 @@ def test_clt_granule_route_changes_nothing(pkg, vo, dev):
 # ---- Lorsa ---------------------------------------------------------------------------------------
 
 def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, **kw):
+    okw = {k_: v for k_, v in kw.items() if k_ != "normalization_type"}   # the oracle's query / key norm is the RMS one
     ref = vo.init_uniform_(vo.LorsaOracle(d_model=d, d_sae=F, n_qk_heads=h, d_qk_head=dq, n_ctx=n_ctx, act_fn="topk", top_k=k,
-                                          **kw), seed=seed, bound=0.3)
+                                          **okw), seed=seed, bound=0.3)
     with torch.no_grad():
         g = torch.Generator().manual_seed(seed + 7)
         ref.W_O.mul_(0.25 + 1.5 * torch.rand(F, 1, generator=g))
@@ -396,6 +397,17 @@ def test_lorsa_fused_step_bf16_with_rotary(pkg, vo, dev, dq, rotary_dim, adjacen
     timer = lorsa_bf16_step(pkg, vo, dev, 64, 256, 4, dq, 64, 2, True, positional_embedding_type="rotary",
                             rotary_dim=rotary_dim, rotary_adjacent_pairs=adjacent)
     assert "rotary_fwd" in timer.records and "rotary_bwd_t" in timer.records
+
+
+@pytest.mark.parametrize("kw", [dict(positional_embedding_type="none", use_post_qk_ln=True, normalization_type="RMS"),
+                                dict(positional_embedding_type="rotary", rotary_dim=8),
+                                dict(positional_embedding_type="rotary", rotary_dim=32, use_post_qk_ln=True,
+                                     normalization_type="RMS")])
+def test_lorsa_bf16_step_with_other_query_key_forms_runs_the_attention_kernels(pkg, vo, dev, kw):
+    """Query / key norms, or a rotary width the rotary kernels do not take: q, k, v come from the general op sequence
+    and the mixing still runs on the attention kernels (no library attention, no padded heads)."""
+    timer = lorsa_bf16_step(pkg, vo, dev, 64, 256, 4, 32, 64, 2, True, **kw)
+    assert "attention_bwd" in timer.records and "rotary_fwd" not in timer.records
 
 
 def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, **kw):
