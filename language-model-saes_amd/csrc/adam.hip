@@ -279,8 +279,11 @@ namespace sae {
 
 __global__ void sq_nnz_finish_kernel(const double *__restrict__ partial, int64_t F, double *acc);  // defined below
 
-template <bool DENSE_BF16, int U>
-__global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
+// NT threads: 256, or fewer for rows whose pieces do not fill four waves (a row of 768 elements has 192 pieces: a fourth
+// wave would hold a place on its SIMD and do nothing but help staging; a wave that owns no piece adds nothing to any sum,
+// so the results are the same bits)
+template <bool DENSE_BF16, int U, int NT = 256>
+__global__ __launch_bounds__(NT) void adam_sparse_rows_kernel(
     const int32_t *__restrict__ feat_ptr, const int32_t *__restrict__ feat_slot,
     const int32_t *__restrict__ slot_tok, const float *__restrict__ coef, const void *__restrict__ dense,
     float *__restrict__ p, float *__restrict__ m, float *__restrict__ v, int d, AdamScalars a,
@@ -290,8 +293,8 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     const float *__restrict__ row_grad_coef) {
   __shared__ float red[4];
   __shared__ double red_d[8];
-  __shared__ float s_coef[256];
-  __shared__ int32_t s_tok[256];
+  __shared__ float s_coef[NT];
+  __shared__ int32_t s_tok[NT];
   const int f = blockIdx.x, tid = threadIdx.x;
   const float gs = grad_scale ? grad_scale[0] : 1.f;
   const float rc = row_grad_coef ? row_grad_coef[f] : 0.f;   // the row's gradient through its L2 norm: rc * p[f, :]
@@ -315,13 +318,13 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
   int g_nz = 0;
   // U pieces of 4 elements per thread and pass: a row of up to 1024 U elements takes one pass (the same for every
   // thread of the workgroup, which gathers the gradient row together)
-  for (int seg_base = 0; seg_base < n_seg; seg_base += 256 * U) {
+  for (int seg_base = 0; seg_base < n_seg; seg_base += NT * U) {
     const int seg0 = seg_base + tid;
     // issue the streaming reads of p, m, v first: they are the HBM traffic; the gradient operands hit cache
     float4 pp[U], mm[U], vv[U], g[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int seg = seg0 + u * 256;
+      const int seg = seg0 + u * NT;
       if (seg < n_seg) {
         pp[u] = load_state4<false>(p, base4 + seg);
         mm[u] = load_state4<false>(m, base4 + seg);
@@ -330,10 +333,10 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
       g[u] = (xo >= 0 && seg < n_seg) ? reinterpret_cast<const float4 *>(extra_rows)[(int64_t)xo * n_seg + seg]
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    gather_rows_staged<DENSE_BF16, 256, U>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg, s_coef, s_tok);
+    gather_rows_staged<DENSE_BF16, NT, U>(g, lo, hi, feat_slot, slot_tok, coef, dbase, row_bytes, seg0, n_seg, s_coef, s_tok);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int seg = seg0 + u * 256;
+      const int seg = seg0 + u * NT;
       if (seg < n_seg) {
         if (row_grad_coef) {   // product and sum rounded separately, as when the term is added to a stored gradient
           g[u].x = add_rn(g[u].x, mul_rn(rc, pp[u].x)); g[u].y = add_rn(g[u].y, mul_rn(rc, pp[u].y));
@@ -365,7 +368,7 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     }
   }
   if (row_norm) {
-    const float tot = block_sum<4>(sq, red);
+    const float tot = block_sum<NT / 64>(sq, red);
     if (tid == 0) row_norm[f] = sqrtf(tot);
   }
   if (sq_nnz_partial) {
@@ -376,8 +379,11 @@ __global__ __launch_bounds__(256) void adam_sparse_rows_kernel(
     if (lane == 0) { red_d[w] = g_sq; red_d[4 + w] = cnt; }
     __syncthreads();
     if (tid == 0) {
-      sq_nnz_partial[2 * (size_t)f] = red_d[0] + red_d[1] + red_d[2] + red_d[3];
-      sq_nnz_partial[2 * (size_t)f + 1] = red_d[4] + red_d[5] + red_d[6] + red_d[7];
+      double s = red_d[0], c = red_d[4];
+#pragma unroll
+      for (int w2 = 1; w2 < NT / 64; ++w2) { s += red_d[w2]; c += red_d[4 + w2]; }
+      sq_nnz_partial[2 * (size_t)f] = s;
+      sq_nnz_partial[2 * (size_t)f + 1] = c;
     }
   }
 }
@@ -577,6 +583,13 @@ static int adam_step_sparse_rows_impl(bool lowp, const int32_t *feat_ptr, const 
         if (d <= 1024) SAE_ADAM_ROWS_LOWP(false, 1); else SAE_ADAM_ROWS_LOWP(false, 2);
       }
 #undef SAE_ADAM_ROWS_LOWP
+    } else if (u == 1 && d <= 768 && d > 512) {   // 129-192 pieces: three waves
+#define SAE_ADAM_ROWS_192(BF)                                                                                              \
+  hipLaunchKernelGGL((adam_sparse_rows_kernel<BF, 1, 192>), dim3((unsigned)F), dim3(192), 0, st, feat_ptr, feat_slot, slot_tok, \
+                     coef, dense, p, m, v, (int)d, a, reinterpret_cast<uint16_t *>(shadow_bf16), row_norm_out,            \
+                     bias_grad_out, grad_scale, partial, extra_map, extra_rows, extra_bias, row_grad_coef)
+      if (dense_dtype == SAE_BF16) SAE_ADAM_ROWS_192(true); else SAE_ADAM_ROWS_192(false);
+#undef SAE_ADAM_ROWS_192
     } else if (dense_dtype == SAE_BF16) {
       if (u == 1) SAE_ADAM_ROWS(true, 1); else if (u == 2) SAE_ADAM_ROWS(true, 2); else SAE_ADAM_ROWS(true, 4);
     } else {
