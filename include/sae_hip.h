@@ -165,6 +165,14 @@ int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, v
 int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
                                 int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val, int64_t *row_off,
                                 int32_t *row_nnz, void *stream);
+/* The two entry points above in the bf16 arithmetic of a dictionary held in bf16 (the keys of sae_select_topk_row_lowp:
+ * the sum with the bias and the product with the scale each rounded to bf16; values rounded after the division). */
+int sae_encoder_gemm_granule_max_lowp(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups, int64_t B,
+                                      int64_t d, int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
+                                      void *stream);
+int sae_select_topk_row_granule_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
+                                     int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val,
+                                     int64_t *row_off, int32_t *row_nnz, void *stream);
 
 /* sae_select_topk_batch (bf16 pre, no feat_mask, F % 256 == 0) with the per-granule key maxima handed in
  * (granule_max [B, F / 64] of sae_encoder_gemm_granule_max for the same pre, b_enc, scale): the select's one pass over
@@ -180,11 +188,12 @@ int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_
  * rounded to bf16, as the bf16 tensors around the reference's batch_topk closure are (models/sae.py:324-341,
  * models/sparse_dictionary.py:761-794).  b_enc / scale are fp32 copies of the bf16 bias / norms.  Many keys then share
  * the threshold's value; ties keep the lowest flattened indices b * F + f.  feat_mask as in sae_select_topk_row_lowp.
- * Same workspace. */
-int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, const float *feat_mask,
-                               int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx, float *val,
-                               int64_t capacity, int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
-                               int64_t workspace_bytes, void *stream);
+ * granule_max (or NULL): the maxima sae_encoder_gemm_granule_max_lowp left, as in sae_select_topk_batch_granule (no
+ * feat_mask then, F a multiple of 256).  Same workspace. */
+int sae_select_topk_batch_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
+                               const float *feat_mask, int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev,
+                               int32_t *idx, float *val, int64_t capacity, int64_t *row_off, int32_t *row_nnz,
+                               int64_t *total_out, void *workspace, int64_t workspace_bytes, void *stream);
 
 /* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product
  * (Lorsa's head activations): one streaming read of pre.  rows_per_group as in sae_select_topk_row_granule. */

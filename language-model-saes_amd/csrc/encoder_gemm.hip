@@ -296,7 +296,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
 // EPI_MARGIN (bf16 output, N a multiple of 64): like EPI_GMAX, but what is written per token and granule is the largest
 // JumpReLU margin (out + bias) * scale - theta of the granule's rounded outputs (a float, each operation rounded on its
 // own as the activation kernels do): a granule holds an active or in-window entry only if that reaches -window / 2.
-constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2, EPI_MARGIN = 3;
+// EPI_GMAX_LOWP: EPI_GMAX with the keys in the bf16 arithmetic of a dictionary held in bf16 (the sum with the bias and the
+// product with the scale each rounded to bf16: what sae_select_topk_row_lowp / sae_select_topk_batch_lowp form).
+constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2, EPI_MARGIN = 3, EPI_GMAX_LOWP = 4;
 template <bool BF16_OUT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
       w += g * (size_t)N * row_bytes;
     }
     out = reinterpret_cast<char *>(out) + g * (size_t)M * N * (BF16_OUT ? 2 : 4);
-    if constexpr (EPI == EPI_GMAX || EPI == EPI_MARGIN) {
+    if constexpr (EPI == EPI_GMAX || EPI == EPI_MARGIN || EPI == EPI_GMAX_LOWP) {
       if (b_enc) b_enc += g * (size_t)N;
       if (scale) scale += g * (size_t)N;
       gmax += g * (size_t)M * (N >> 6);
@@ -412,7 +414,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
 
   // EPI_GMAX: this lane's 16 bias and 16 scale values; EPI_BIAS: its 16 column biases and 8 row biases.  Asked for here
   // so that the epilogue does not wait for them.
-  constexpr bool MARGIN = EPI == EPI_MARGIN, GMAX = EPI == EPI_GMAX || MARGIN, BIAS = EPI == EPI_BIAS;
+  constexpr bool MARGIN = EPI == EPI_MARGIN, LOWPK = EPI == EPI_GMAX_LOWP, GMAX = EPI == EPI_GMAX || MARGIN || LOWPK, BIAS = EPI == EPI_BIAS;
   float bb[EPI != EPI_NONE ? 4 : 1][4], ss[GMAX ? 4 : 1][4], rb[BIAS ? 8 : 1];
   if constexpr (EPI != EPI_NONE) {
     const int f0 = n0 + wn * 64;
@@ -506,6 +508,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             if constexpr (MARGIN) hmax = fmaxf(hmax, sub_rn(mul_rn(acc[i][j][r] + bb[i][r], ss[i][r]), th[i][r]));
+            else if constexpr (LOWPK) hmax = fmaxf(hmax, bf16_round(mul_rn(bf16_round(add_rn(acc[i][j][r], bb[i][r])), ss[i][r])));
             else hmax = fmaxf(hmax, (acc[i][j][r] + bb[i][r]) * ss[i][r]);   // h1 of select_key_plain
           }
         }
@@ -686,6 +689,22 @@ extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_en
               SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max: pointers must be 16-byte aligned");
   return launch_gemm_bf16<true, EPI_GMAX>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max, (hipStream_t)stream,
                                       n_groups);
+}
+
+extern "C" int sae_encoder_gemm_granule_max_lowp(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups,
+                                                 int64_t B, int64_t d, int64_t F, const float *b_enc, const float *scale,
+                                                 uint32_t *granule_max, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(x_bf16 && w_enc_t_bf16 && pre_bf16 && granule_max, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max_lowp: null pointer");
+  SAE_REQUIRE(B > 0 && d > 0 && F > 0 && n_groups > 0, SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max_lowp: sizes must be positive");
+  SAE_REQUIRE(B < (1LL << 31) && F < (1LL << 31) && d < (1LL << 28) && n_groups <= 65535, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_granule_max_lowp: size too large");
+  SAE_REQUIRE(d % 64 == 0 && F % 64 == 0, SAE_ERR_UNSUPPORTED,
+              "encoder_gemm_granule_max_lowp: d_model=%lld and F=%lld must be multiples of 64", (long long)d, (long long)F);
+  SAE_REQUIRE((((uintptr_t)x_bf16 | (uintptr_t)w_enc_t_bf16 | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0,
+              SAE_ERR_INVALID_ARG, "encoder_gemm_granule_max_lowp: pointers must be 16-byte aligned");
+  return launch_gemm_bf16<true, EPI_GMAX_LOWP>(x_bf16, w_enc_t_bf16, pre_bf16, B, d, F, b_enc, scale, granule_max,
+                                           (hipStream_t)stream, n_groups);
 }
 
 extern "C" int sae_encoder_gemm_bias(const void *x_bf16, const void *w_t_bf16, void *out_bf16, int64_t B, int64_t d, int64_t F,

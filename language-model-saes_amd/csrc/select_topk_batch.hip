@@ -740,10 +740,11 @@ extern "C" int sae_select_topk_batch(const void *pre, int pre_dtype, const float
                                  row_nnz, total_out, workspace, st);
 }
 
-extern "C" int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_enc, const float *scale, const float *feat_mask,
-                                          int64_t B, int64_t F, int64_t k_total, const int64_t *k_total_dev, int32_t *idx,
-                                          float *val, int64_t capacity, int64_t *row_off, int32_t *row_nnz,
-                                          int64_t *total_out, void *workspace, int64_t workspace_bytes, void *stream) {
+extern "C" int sae_select_topk_batch_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                          const float *scale, const float *feat_mask, int64_t B, int64_t F, int64_t k_total,
+                                          const int64_t *k_total_dev, int32_t *idx, float *val, int64_t capacity,
+                                          int64_t *row_off, int32_t *row_nnz, int64_t *total_out, void *workspace,
+                                          int64_t workspace_bytes, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre_bf16 && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F <= (1LL << 30), SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: bad shape");
@@ -752,8 +753,11 @@ extern "C" int sae_select_topk_batch_lowp(const void *pre_bf16, const float *b_e
   SAE_REQUIRE(workspace && workspace_bytes >= sae_select_topk_batch_workspace_bytes(B, F), SAE_ERR_WORKSPACE,
               "select_topk_batch_lowp: workspace of %lld bytes needed", (long long)sae_select_topk_batch_workspace_bytes(B, F));
   SAE_REQUIRE((((uintptr_t)workspace) & 255) == 0, SAE_ERR_INVALID_ARG, "select_topk_batch_lowp: workspace must be 256-byte aligned");
+  SAE_REQUIRE(!granule_max || (!feat_mask && F % 256 == 0 &&
+                               (((uintptr_t)granule_max | (uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0),
+              SAE_ERR_UNSUPPORTED, "select_topk_batch_lowp: granule maxima need F a multiple of 256, 16-byte aligned pointers and no feat_mask");
   return run_batch_select<true>(pre_bf16, b_enc, scale, feat_mask, B, F, k_total, k_total_dev, idx, val, capacity, row_off,
-                                row_nnz, total_out, workspace, (hipStream_t)stream, nullptr, true);
+                                row_nnz, total_out, workspace, (hipStream_t)stream, granule_max, true);
 }
 
 extern "C" int sae_select_topk_batch_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,

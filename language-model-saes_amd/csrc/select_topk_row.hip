@@ -520,6 +520,8 @@ struct GsShared {
   int32_t remaining, digit_found;
 };
 
+// ARITH: SEL_PLAIN, or SEL_LOWP for maxima and keys in the bf16 arithmetic of a dictionary held in bf16
+template <int ARITH>
 __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     const uint16_t *__restrict__ pre, const uint32_t *__restrict__ gmax, const float *__restrict__ b_enc,
     const float *__restrict__ scale, int F, int k, int32_t *__restrict__ idx_out, float *__restrict__ val_out,
@@ -532,7 +534,7 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     if (b_enc) b_enc += grp * F;
     if (scale) scale += grp * F;
   }
-  RowReader<true, SEL_PLAIN> rr;
+  RowReader<true, ARITH> rr;
   rr.row = pre + (size_t)b * F;
   rr.b_enc = b_enc;
   rr.scale = scale;
@@ -632,7 +634,9 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     const float h1 = __uint_as_float(key);
     if (rank < k) {
       idx_out[(size_t)b * k + rank] = my_idx;
-      val_out[(size_t)b * k + rank] = scale ? h1 / scale[my_idx] : h1;
+      float v = h1;
+      if (scale) { v = h1 / scale[my_idx]; if (sel_is_lowp(ARITH)) v = sel_bf16_round(v); }
+      val_out[(size_t)b * k + rank] = v;
     }
   }
   for (int i = k_eff + tid; i < k; i += GS_THREADS) { idx_out[(size_t)b * k + i] = 0; val_out[(size_t)b * k + i] = 0.f; }
@@ -672,10 +676,10 @@ __global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__rest
 
 }  // namespace sae
 
-extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
-                                           const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
-                                           int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
-  using namespace sae;
+namespace sae {
+static int select_topk_row_granule_impl(bool lowp, const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                        const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                        int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
   SAE_REQUIRE(pre_bf16 && granule_max && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row_granule: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "select_topk_row_granule: bad sizes");
   if (rows_per_group <= 0) rows_per_group = B;
@@ -687,13 +691,32 @@ extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t 
   SAE_REQUIRE((((uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0, SAE_ERR_INVALID_ARG,
               "select_topk_row_granule: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(select_topk_row_granule_kernel, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
-                     (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
+  if (lowp)
+    hipLaunchKernelGGL(select_topk_row_granule_kernel<SEL_LOWP>, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
+                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
+  else
+    hipLaunchKernelGGL(select_topk_row_granule_kernel<SEL_PLAIN>, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
+                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
   const int rc = check_launch("select_topk_row_granule");
   if (rc != SAE_OK) return rc;
   // rows the granule kernel flagged (mass ties) are redone from the whole row; every other workgroup leaves at once
-  return select_topk_row_impl(false, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1,
+  return select_topk_row_impl(lowp, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1,
                               (int)rows_per_group);
+}
+}  // namespace sae
+
+extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                           const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                           int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
+  return sae::select_topk_row_granule_impl(false, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, idx, val, row_off,
+                                           row_nnz, stream);
+}
+
+extern "C" int sae_select_topk_row_granule_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
+                                                const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                                int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
+  return sae::select_topk_row_granule_impl(true, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, idx, val, row_off,
+                                           row_nnz, stream);
 }
 
 extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,

@@ -353,7 +353,7 @@ def granule_route_supported(d: int, F: int, k: int) -> bool:
 
 
 def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Optional[torch.Tensor],
-                             scale: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+                             scale: Optional[torch.Tensor], lowp: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """bf16 pre[B, F] = x @ w_enc_t^T plus granule_max [B, F / 64] (int32 holding uint32 keys): per token and aligned
     granule of 64 features the largest select key, i.e. the bits of (pre + b_enc) * scale where that is positive.
     With a leading group dimension on every argument (x [G, B, d], w_enc_t [G, F, d], b_enc / scale [G, F]) the G
@@ -374,9 +374,11 @@ def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Opti
     lead = (G,) if grouped else ()
     pre = torch.empty(*lead, B, F, dtype=torch.bfloat16, device=x.device)
     gmax = torch.empty(*lead, B, max(F // GRANULE, 1), dtype=torch.int32, device=x.device)
+    lib = _lib.load()
+    fn = lib.sae_encoder_gemm_granule_max_lowp if lowp else lib.sae_encoder_gemm_granule_max   # keys in bf16 arithmetic
     with _timed("encoder_gemm"):
-        check(_lib.load().sae_encoder_gemm_granule_max(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), G, B, d, F, _ptr(b_enc),
-                                                       _ptr(scale), gmax.data_ptr(), _stream(x)), "encoder_gemm_granule_max")
+        check(fn(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), G, B, d, F, _ptr(b_enc), _ptr(scale), gmax.data_ptr(),
+                 _stream(x)), "encoder_gemm_granule_max")
     return pre, gmax
 
 
@@ -468,8 +470,8 @@ def select_topk_row(
     if lowp and (pre.dtype != torch.bfloat16 or cand_cap is not None):
         raise ValueError("lowp select takes a bf16 pre and no cand_cap")
     if granule_max is not None:
-        if lowp or cand_cap is not None or feat_mask is not None or pre.dtype != torch.bfloat16:
-            raise ValueError("the granule route takes a bf16 pre and none of lowp, cand_cap, feat_mask")
+        if cand_cap is not None or feat_mask is not None or pre.dtype != torch.bfloat16:
+            raise ValueError("the granule route takes a bf16 pre and neither cand_cap nor feat_mask")
         _req(granule_max, "granule_max", torch.int32, 2)
         if tuple(granule_max.shape) != (B, F // GRANULE) or F % GRANULE:
             raise ValueError(f"granule_max must be [{B}, {F}/{GRANULE}]")
@@ -489,9 +491,9 @@ def select_topk_row(
     _t = _timed("select_topk_row[granule]" if granule_max is not None else "select_topk_row")
     _t.__enter__()
     if granule_max is not None:
-        rc = lib.sae_select_topk_row_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k,
-                                             int(rows_per_group), idx.data_ptr(), val.data_ptr(), row_off.data_ptr(),
-                                             row_nnz.data_ptr(), _stream(pre))
+        fn = lib.sae_select_topk_row_granule_lowp if lowp else lib.sae_select_topk_row_granule
+        rc = fn(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, int(rows_per_group), idx.data_ptr(),
+                val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     elif lowp:
         rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k, idx.data_ptr(),
                                           val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
@@ -523,8 +525,8 @@ def select_topk_batch(
     of 256, no feat_mask); the select's one full pass over the matrix then shrinks to a histogram of those maxima."""
     _req(pre, "pre", ndim=2)
     B, F = pre.shape
-    if lowp and (pre.dtype != torch.bfloat16 or granule_max is not None):
-        raise ValueError("lowp select takes a bf16 pre and no granule_max")
+    if lowp and pre.dtype != torch.bfloat16:
+        raise ValueError("lowp select takes a bf16 pre")
     if granule_max is not None:
         if feat_mask is not None or pre.dtype != torch.bfloat16 or F % 256:
             raise ValueError("granule_max needs a bf16 pre with F a multiple of 256 and no feat_mask")
@@ -555,12 +557,16 @@ def select_topk_batch(
     ws_bytes = lib.sae_select_topk_batch_workspace_bytes(B, F)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with _timed("select_topk_batch"):
-        if granule_max is not None:
+        if granule_max is not None and lowp:
+            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), None, B, F, k_host,
+                                                _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
+                                                row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
+        elif granule_max is not None:
             rc = lib.sae_select_topk_batch_granule(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k_host,
                                                    _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
                                                    row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
         elif lowp:
-            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
+            rc = lib.sae_select_topk_batch_lowp(pre.data_ptr(), None, _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k_host,
                                                 _ptr(k_dev), idx.data_ptr(), val.data_ptr(), capacity, row_off.data_ptr(),
                                                 row_nnz.data_ptr(), None, ws.data_ptr(), ws_bytes, _stream(pre))
         else:

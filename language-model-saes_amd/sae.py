@@ -262,14 +262,16 @@ class _FusedSparseStep(torch.autograd.Function):
         # the per-token select then reads a row only in the granules that can hold a kept element, and the batch-wide
         # select is spared its one pass over the whole matrix.  The keys need the decoder
         # norms, so this route fetches them before the GEMM (and waits there for an overlapped decoder update).
-        granule = (amp and not lowp and getattr(sae, "granule_select", True) and not sae._update_pending()
+        granule = (amp and getattr(sae, "granule_select", True) and not sae._update_pending()
                    and (ops.granule_route_supported(x.shape[1], w_enc_op.shape[0], int(k)) if not batch_wide
                         else x.shape[1] % 64 == 0 and w_enc_op.shape[0] % 256 == 0))
         gmax = None
         if granule:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
             scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
-            pre, gmax = ops.encoder_gemm_granule_max(x_op, w_enc_op, b_E, scale)
+            if lowp and scale is not None:
+                scale = scale.bfloat16().float()   # decoder_norm() of bf16 weights is a bf16 tensor
+            pre, gmax = ops.encoder_gemm_granule_max(x_op, w_enc_op, b_E, scale, lowp=lowp)
         elif amp:
             x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())
             pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)

@@ -60,6 +60,31 @@ def test_granule_select_equals_row_select(pkg, dev, B, d, F, k):
     assert torch.equal(got.idx, want.idx) and torch.equal(got.val, want.val)
 
 
+@pytest.mark.parametrize("B,d,F,k", [(128, 128, 2048, 16), (300, 128, 8192, 64), (64, 64, 256, 8), (256, 256, 16384, 100)])
+def test_granule_route_in_bf16_arithmetic(pkg, dev, B, d, F, k):
+    """A dictionary held in bf16: the product's epilogue forms the granule maxima from keys in bf16 arithmetic, and the
+    per-token and the batch-wide select that read them return what their full-row forms in that arithmetic return."""
+    x, w, b, s = _inputs(B, d, F, seed=5 * B + k, dev=dev)
+    b, s = b.bfloat16().float(), s.bfloat16().float()          # the bias and the norms of such a dictionary are bf16 values
+    pre, gmax = pkg.ops.encoder_gemm_granule_max(x, w, b, s, lowp=True)
+    assert torch.equal(pre, pkg.ops.encoder_gemm(x, w, torch.bfloat16))
+    h1 = ((pre + b.bfloat16()) * s.bfloat16()).float()        # bf16 tensors: each operation rounds
+    bits = h1.contiguous().view(torch.int32)
+    want_max = torch.where(h1 > 0, bits, torch.zeros_like(bits)).view(B, F // 64, 64).max(dim=2).values
+    assert torch.equal(gmax, want_max)
+    plain_max = pkg.ops.encoder_gemm_granule_max(x, w, b, s)[1]
+    assert not torch.equal(gmax, plain_max)                   # the fp32 keys are other numbers
+    got = pkg.ops.select_topk_row(pre, b, s, k, granule_max=gmax, lowp=True)
+    want = pkg.ops.select_topk_row(pre, b, s, k, lowp=True)
+    assert torch.equal(got.row_nnz, want.row_nnz) and torch.equal(got.idx, want.idx) and torch.equal(got.val, want.val)
+    if F % 256 == 0:
+        got = pkg.ops.select_topk_batch(pre, b, s, k * B, granule_max=gmax, lowp=True)
+        want = pkg.ops.select_topk_batch(pre, b, s, k * B, lowp=True)
+        assert torch.equal(got.row_nnz, want.row_nnz) and torch.equal(got.row_off, want.row_off)
+        n = int(want.row_nnz.sum())
+        assert n == k * B and torch.equal(got.idx[:n], want.idx[:n]) and torch.equal(got.val[:n], want.val[:n])
+
+
 def _granule_max_of(pre, b, s):
     B, F = pre.shape
     return _keys(pre, b, s).view(B, F // 64, 64).max(dim=2).values.contiguous()
