@@ -25,7 +25,7 @@ from torch import nn
 
 from . import ops
 from .config import CrosscoderConfig, register_sae_model
-from .sae import _autocast_dtype
+from .sae import SparseRowGrad, _autocast_dtype
 from .sparse_dictionary import LazyDict, SparseDictionary
 
 
@@ -67,6 +67,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         holder["codes"], holder["pre"], holder["norms"], holder["b_sum"] = codes, pre, norms, b_sum
         ctx.codes, ctx.grads, ctx.dvals, ctx.x_op, ctx.w_enc_op = codes, grads, dvals, x_op, w_enc_op
         ctx.shape = (B, H, d, F)
+        ctx.defer_to = m if holder.get("defer") else None
         ctx.mark_non_differentiable(recon)
         return loss, recon
 
@@ -74,18 +75,32 @@ class _FusedCrosscoderStep(torch.autograd.Function):
     def backward(ctx, g_loss, _g_recon):
         B, H, d, F = ctx.shape
         g = g_loss.to(torch.float32)
-        dW_D, db_D = [], []
-        for h in range(H):
-            fi = ops.build_feature_index(ctx.codes[h])
-            rows, _ = ops.sparse_grad_rows(fi, ctx.codes[h].val * g, ctx.grads[h], F)
-            dW_D.append(rows)
-            db_D.append(ops.col_sum(ctx.grads[h]) * g)
-        stacked = reduce(ops.stack_codes, ctx.codes)
+        m = ctx.defer_to
+        defer = (m is not None and all(w.grad is None and getattr(w, "_sparse_grad", None) is None for w in (m.W_E, m.W_D)))
+        db_D = [ops.col_sum(ctx.grads[h]) * g for h in range(H)]
+        stacked = reduce(ops.stack_codes, ctx.codes)          # the H codes on a virtual token axis: token h * B + b
         fi = ops.build_feature_index(stacked)
         fi = dataclasses.replace(fi, slot_tok=torch.remainder(fi.slot_tok, B).to(torch.int32))  # virtual token h*B + b -> row b of x
         coef = torch.cat(ctx.dvals) * g
-        dW_Et, db_sum = ops.sparse_grad_rows(fi, coef, ctx.x_op, F, want_bias=True)                    # [F, H*d], [F]
-        dW_E = dW_Et.view(F, H, d).permute(1, 2, 0)
+        if defer:
+            # The optimiser rebuilds the rows where it consumes them; nothing dense is written here.  The decoder
+            # [H, F, d] is one matrix of H F rows: head h's code addresses rows h F .. (h + 1) F of it, and its dense
+            # operand is head h's block of the stacked output gradients.
+            idx_cat = torch.cat([c.idx + h * F for h, c in enumerate(ctx.codes)])
+            cat_code = dataclasses.replace(stacked, idx=idx_cat, d_sae=H * F)
+            m.W_D._sparse_grad = SparseRowGrad(ops.build_feature_index(cat_code), stacked.val * g, torch.cat(ctx.grads), H * F)
+            m.W_E._sparse_grad = SparseRowGrad(fi, coef, ctx.x_op, F)
+            db_sum, _ = ops.feature_segment_sums(fi, coef)
+            dW_E = dW_D = None
+        else:
+            dW_D = []
+            for h in range(H):
+                fi_h = ops.build_feature_index(ctx.codes[h])
+                rows, _ = ops.sparse_grad_rows(fi_h, ctx.codes[h].val * g, ctx.grads[h], F)
+                dW_D.append(rows)
+            dW_D = torch.stack(dW_D)
+            dW_Et, db_sum = ops.sparse_grad_rows(fi, coef, ctx.x_op, F, want_bias=True)                # [F, H*d], [F]
+            dW_E = dW_Et.view(F, H, d).permute(1, 2, 0)
         db_E = db_sum.unsqueeze(0).expand(H, F)
         dx = dlabel = None
         if ctx.needs_input_grad[0]:
@@ -94,7 +109,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
             dx = reduce(torch.add, parts).view(B, H, d)
         if ctx.needs_input_grad[1]:
             dlabel = -torch.stack(ctx.grads, dim=1) * g
-        return dx, dlabel, None, dW_E, db_E, torch.stack(dW_D), torch.stack(db_D), None, None, None
+        return dx, dlabel, None, dW_E, db_E, dW_D, torch.stack(db_D), None, None, None
 
 
 @register_sae_model("crosscoder")
@@ -110,6 +125,9 @@ class Crosscoder(SparseDictionary):
         self.b_E = nn.Parameter(torch.empty(H, F, **kw))
         self.W_D = nn.Parameter(torch.empty(H, F, d, **kw))
         self.b_D = nn.Parameter(torch.empty(H, d, **kw))
+        # set by an optimiser that consumes factored gradients (HipAdam): the weight gradients are then attached to the
+        # parameters as `_sparse_grad` instead of being written as dense rows
+        self.defer_weight_grads = False
 
     # ---- kernel operands ----
     def _w_enc_operand(self, amp: bool) -> torch.Tensor:
@@ -246,7 +264,7 @@ class Crosscoder(SparseDictionary):
             mf = mask.to(torch.float32)
             tok_w = mf / mf.sum()
         amp = _autocast_dtype("cuda") == torch.bfloat16
-        holder: dict[str, Any] = {"model": self}
+        holder: dict[str, Any] = {"model": self, "defer": self.defer_weight_grads and torch.is_grad_enabled()}
         xin = x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x
         loss, recon = _FusedCrosscoderStep.apply(xin.contiguous(), label.to(torch.float32).contiguous(), tok_w, self.W_E,
                                                  self.b_E, self.W_D, self.b_D, int(self.current_k), amp, holder)

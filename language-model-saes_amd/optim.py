@@ -209,7 +209,11 @@ class HipAdam(Optimizer):
         """A weight whose [rows, d] view is updated block by block (a cross-layer transcoder's stacked layers):
         one kernel per block with a factored gradient, a plain zero-gradient Adam pass over rows no block covers."""
         b1, b2 = group["betas"]
-        d = pv.shape[-1]
+        # a row is as long as the dense operand's rows: the last axis of the storage (a cross-layer transcoder's layers),
+        # or several trailing axes taken together (a crosscoder's encoder, stored [F, H, d] with rows of H d)
+        d = int(_pieces(sg)[0][1].dense_operand.shape[1])
+        if pv.numel() % d != 0 or not pv.is_contiguous():
+            raise NotImplementedError("the factored gradient's rows do not tile the parameter's storage")
         p2, m2, v2 = pv.reshape(-1, d), mv.reshape(-1, d), vv.reshape(-1, d)
         role = self._roles.get(id(p))
         shadow = self._model.get_derived_buffer(f"{role}.bf16") if role is not None else None
@@ -219,7 +223,7 @@ class HipAdam(Optimizer):
         bias_param = getattr(sg, "bias_param", None)
         bias_buf = torch.zeros(p2.shape[0], dtype=torch.float32, device=p.device) if bias_param is not None else None
         # a decoder group held as one block (a cross-layer transcoder's W_D[j]) also yields its row norms
-        want_norm = (role is not None and role.startswith("W_D.") and not hasattr(sg, "pieces") and d % 4 == 0
+        want_norm = (role is not None and (role == "W_D" or role.startswith("W_D.")) and not hasattr(sg, "pieces") and d % 4 == 0
                      and hasattr(self._model, "set_derived"))
         norm_buf = None
         if want_norm:

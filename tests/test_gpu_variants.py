@@ -6,6 +6,7 @@ accumulated in a different order than the CPU's GEMMs).  bf16 autocast runs are 
 differently in bf16, so an entry close to the k-th value can legitimately fall on the other side.
 """
 
+import contextlib
 import importlib
 
 import pytest
@@ -127,6 +128,8 @@ def test_crosscoder_mask_and_adam_step(pkg, vo, dev):
     want = ref.compute_loss(batch, hooks, mask=mask)["loss"]
     assert rel_err(loss, want) < FP32_TOL
     loss.backward(); want.backward()
+    assert m.W_E.grad is None and m.W_E._sparse_grad is not None and m.W_D._sparse_grad is not None
+    opt.materialize_grads()             # the factored weight gradients as ordinary dense ones
     check_grads(m, ref)
     opt.step(); ropt.step()
     rp = dict(ref.named_parameters())
@@ -134,6 +137,49 @@ def test_crosscoder_mask_and_adam_step(pkg, vo, dev):
         move, want_move = p.detach().cpu() - before[n], rp[n].detach() - before[n]
         assert rel_err(move, want_move) < 1e-3, n
     assert m.W_E.permute(2, 0, 1).is_contiguous()      # the update kept the feature-major layout
+
+
+@pytest.mark.parametrize("amp", [False, True])
+def test_crosscoder_factored_gradients_over_adam_steps(pkg, vo, oracle, dev, amp):
+    """With HipAdam attached the crosscoder's backward leaves no dense weight gradient: the decoder [H, F, d] is updated
+    as one matrix of H F rows, the encoder (stored [F, H, d]) as F rows of H d.  Three steps end at the bits the dense
+    gradients end at; in fp32 they follow torch.optim.Adam on the oracle, and the gradient norm is the dense one."""
+    H, d, F, k, B = 3, 64, 512, 8, 96
+    finals = []
+    for defer in (True, False):
+        m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=37)
+        g = torch.Generator().manual_seed(38)
+        batch = {h: torch.randn(B, d, generator=g) for h in hooks}
+        batch["tokens"] = torch.zeros(B, dtype=torch.long)
+        gb = {k_: v.to(dev) for k_, v in batch.items()}
+        opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=1e-3, model=m, defer_weight_grads=defer)
+        ropt = torch.optim.Adam(ref.parameters(), lr=1e-3)
+        for step in range(3):
+            with (torch.autocast("cuda", dtype=torch.bfloat16) if amp else contextlib.nullcontext()):
+                loss = m.compute_loss(gb, return_aux_data=False)
+            loss.backward()
+            assert (m.W_E.grad is None and m.W_D.grad is None) == defer
+            if defer and not amp:
+                ref.compute_loss(batch, hooks)["loss"].backward()
+                want_norm = oracle.compute_grad_norm([p.grad for p in ref.parameters()]).item()
+                got_norm = pkg.compute_grad_norm(m.parameters()).item()
+                assert abs(got_norm - want_norm) < 1e-5 * want_norm
+                assert m.W_E.grad is None and m.W_E._sparse_grad is not None
+                ropt.step(); ropt.zero_grad()
+            opt.step(); opt.zero_grad()
+            if defer and not amp:
+                for (n, p), q in zip(m.named_parameters(), ref.parameters()):
+                    assert (p.detach().cpu() - q.detach()).abs().max() <= 2e-2 * 1e-3 * (step + 1) + 1e-6 * q.detach().abs().max(), (step, n)
+            if amp:      # the cached bf16 copies and row norms follow the update
+                assert torch.equal(m._w_dec_operand(True), m.W_D.detach().to(torch.bfloat16)), step
+                assert torch.equal(m._w_enc_operand(True), m.W_E.detach().permute(2, 0, 1).reshape(F, H * d).to(torch.bfloat16)), step
+            assert torch.allclose(m._decoder_norm_nograd(), m.W_D.detach().norm(dim=-1), rtol=1e-5), step
+        assert m.W_E.permute(2, 0, 1).is_contiguous()
+        finals.append(({n: p.detach().clone() for n, p in m.named_parameters()}, loss.item()))
+    (pa, la), (pb, lb) = finals
+    assert la == lb
+    for n in pa:
+        assert torch.equal(pa[n], pb[n]), n
 
 
 def test_crosscoder_fused_step_bf16(pkg, vo, dev):
