@@ -373,7 +373,8 @@ def test_lorsa_shape_fused_step_against_dense_path(pkg, dev):
         assert rel_err(fused[n_], p.grad) < 2e-4, n_
 
 
-def test_lorsa_shape_bf16_attention_kernels_against_library_path(pkg, dev):
+@pytest.mark.parametrize("rotary", [None, (16, False), (64, True)], ids=["no_rotary", "rotary16_halves", "rotary64_adjacent"])
+def test_lorsa_shape_bf16_attention_kernels_against_library_path(pkg, dev, rotary):
     """Lorsa at the benchmark shape under bf16 autocast (d=768, 16 x 1024 tokens, 64 query/key heads of width 64, 8192
     value/output heads in groups of 128, k=64): projections and causal mixing on the GEMM / attention kernels against
     the same module with those stages on torch's library routines (einsum + scaled_dot_product_attention).
@@ -382,9 +383,13 @@ def test_lorsa_shape_bf16_attention_kernels_against_library_path(pkg, dev):
     from lm_saes_amd import synthetic
 
     nb, s, d, F, h, dq, k = 16, 1024, 768, 8192, 64, 64, 64
+    # with rotary embeddings: the first 16 elements of a head in half-split pairs (the reference's own example,
+    # examples/train_pythia_lorsa_topk.py:32-34), or the whole head in adjacent pairs
+    pos = dict(positional_embedding_type="none", rotary_dim=dq) if rotary is None else dict(
+        positional_embedding_type="rotary", rotary_dim=rotary[0], rotary_adjacent_pairs=rotary[1])
     cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
-                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type="none", act_fn="topk", top_k=k,
-                          norm_activation="inference", device="cuda", dtype=torch.float32)
+                          d_qk_head=dq, n_ctx=s, act_fn="topk", top_k=k, norm_activation="inference", device="cuda",
+                          dtype=torch.float32, **pos)
     torch.manual_seed(0)
     m = pkg.LowRankSparseAttention(cfg)
     m.init_parameters()
@@ -403,6 +408,7 @@ def test_lorsa_shape_bf16_attention_kernels_against_library_path(pkg, dev):
     torch.cuda.synchronize()
     pkg.ops.set_kernel_timer(None)
     assert {"attention_fwd", "attention_bwd"} <= set(timer.records), set(timer.records)
+    assert ({"rotary_fwd", "rotary_bwd_t"} <= set(timer.records)) == (rotary is not None)
     fused = {n_: p.grad.clone() for n_, p in m.named_parameters()}
     hp = out["hidden_pre"]
     kept = dense_mask(out["sparse_code"])
