@@ -467,6 +467,41 @@ def mfma_probe() -> dict:
             "tflops_best": round(best, 1), "tflops_runs": runs, "published_peak_tflops": 2500.0}
 
 
+def gemm_operand_probe() -> dict:
+    """The headline encoder product (4096 x 4096 x 131072, bf16) timed with random, zero and constant operands: the same
+    kernel, launch and memory traffic each time, so what separates the figures is what the data costs the chip in
+    switching power, i.e. in clock."""
+    import torch
+    from __graft_entry__ import load_package
+
+    pkg = load_package()
+    dev = torch.device("cuda:0")
+    B, d, F = 4096, D_MODEL, D_SAE
+    g = torch.Generator(device=dev).manual_seed(4)
+    xr = torch.randn(B, d, device=dev, generator=g).bfloat16()
+    wr = (torch.randn(F, d, device=dev, generator=g) / d ** 0.5).bfloat16()
+
+    def timed(x, w, n=10):
+        for _ in range(3):
+            pkg.ops.encoder_gemm(x, w, torch.bfloat16)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(n):
+            pkg.ops.encoder_gemm(x, w, torch.bfloat16)
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) / n
+
+    cases = [("random", xr, wr), ("x zero", torch.zeros_like(xr), wr), ("both zero", torch.zeros_like(xr), torch.zeros_like(wr)),
+             ("both one", torch.ones_like(xr), torch.ones_like(wr)), ("random again", xr, wr)]
+    flop = 2.0 * B * d * F
+    out = {"probe": f"sae_encoder_gemm {B} x {d} x {F} bf16, 10 launches per case", "published_peak_tflops": PEAK_BF16_TFLOPS, "cases": {}}
+    for name, x, w in cases:
+        ms = timed(x, w)
+        out["cases"][name] = {"ms": round(ms, 3), "tflops": round(flop / ms / 1e9, 1)}
+    return out
+
+
 def cpu_baseline(sample_batch: int, sample_features: int):
     """Oracle (the reference's eager op sequence on CPU) on a bounded sample of the headline workload: the full
     dictionary (d_model, d_sae, k as on the GPU), `sample_batch` tokens per step instead of 4096 (the host cannot
@@ -519,6 +554,9 @@ def main():
                     help="dictionary size of the CPU baseline (default: the full 131072 features)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
+    ap.add_argument("--gemm-operand-probe", action="store_true",
+                    help="instead of a train step: the headline encoder product with random, zero and constant operands "
+                         "(one JSON line)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of a train step: the rate of register-only bf16 MFMA loops (one JSON line)")
     ap.add_argument("--clip", type=float, default=0.0, help="clip_grad_norm of the topk_trainer workload (0: norm only)")
@@ -529,6 +567,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.gemm_operand_probe:
+        print(json.dumps(gemm_operand_probe()))
+        return
     if args.mfma_probe:
         print(json.dumps(mfma_probe()))
         return
