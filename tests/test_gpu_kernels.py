@@ -214,7 +214,9 @@ def test_sparse_decode_fwd(pkg, dev, B, d, F, k, w_dtype):
     assert rel_err(recon_nb, want - b_dec.double()) < FP32_TOL
 
 
-@pytest.mark.parametrize("B,d,F,k", [(10, 64, 512, 8), (33, 768, 2048, 32), (6, 4096, 1024, 64)])
+@pytest.mark.parametrize("B,d,F,k", [(10, 64, 512, 8), (33, 768, 2048, 32), (6, 4096, 1024, 64),
+                                     # short rows with long row lists (a cross-layer transcoder's prefix codes)
+                                     (20, 768, 4096, 200), (9, 1024, 2048, 131), (12, 256, 1024, 150), (5, 8, 600, 133)])
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("masked", [False, True])
 def test_sparse_decode_mse_fused(pkg, dev, B, d, F, k, w_dtype, masked):
