@@ -209,27 +209,48 @@ class MeanFeatureActMetric(Metric):
         return {"metrics/mean_feature_act": item(self.mean_feature_act.compute())}
 
 
-def _recon_step_stats(ctx) -> torch.Tensor:
+def _layer_major(sae, ctx) -> bool:
+    """Whether label / reconstruction carry a leading layer axis that is no token axis: a cross-layer transcoder's
+    [layers, batch, d_model] (models/clt.py:54-69), whose metrics the reference forms per layer (the token mask spans
+    the batch axis only) and averages over layers when it reports."""
+    label, mask = ctx["label"], ctx.get("mask")
+    if label.ndim < 3 or not hasattr(getattr(sae, "cfg", None), "n_layers"):
+        return False
+    return label.shape[0] == sae.cfg.n_layers and (mask is None or tuple(mask.shape) == tuple(label.shape[1:-1]))
+
+
+def _recon_step_stats(ctx, layer_major: bool = False) -> torch.Tensor:
     """float[4] of this step: explained variance, legacy explained variance, L2 error, L2 error ratio
-    (one kernel pass over label and reconstruction; shared by the two metrics that read them)."""
+    (one kernel pass over label and reconstruction; shared by the two metrics that read them).  `layer_major`: one such
+    row per layer, float[layers, 4] transposed to [4, layers], so that index i is statistic i either way."""
     st = ctx.get("_recon_step_stats")
     if st is None:
         label, recon = ctx["label"].detach(), ctx["reconstructed"].detach()
-        label = label.reshape(-1, label.shape[-1]).to(torch.float32).contiguous()
-        recon = recon.reshape(-1, recon.shape[-1]).to(torch.float32).contiguous()
         w = _token_weights(ctx)
-        if w is None:
-            mean = ops.col_sum(label) / label.shape[0]
+
+        def one(lab, rec):
+            lab = lab.reshape(-1, lab.shape[-1]).to(torch.float32).contiguous()
+            rec = rec.reshape(-1, rec.shape[-1]).to(torch.float32).contiguous()
+            if w is None:
+                mean = ops.col_sum(lab) / lab.shape[0]
+            else:
+                mean = ops.col_sum(lab * w[:, None]) / w.sum()
+            acc = torch.zeros(4, dtype=torch.float64, device=lab.device)
+            return ops.recon_stats(lab, rec, mean.contiguous(), acc, tok_w=w)
+
+        if layer_major:
+            st = torch.stack([one(label[l], recon[l]) for l in range(label.shape[0])]).t().contiguous()
         else:
-            mean = ops.col_sum(label * w[:, None]) / w.sum()
-        acc = torch.zeros(4, dtype=torch.float64, device=label.device)
-        st = ops.recon_stats(label, recon, mean.contiguous(), acc, tok_w=w)
+            st = one(label, recon)
         ctx["_recon_step_stats"] = st
     return st
 
 
-def _dense_recon_stats(ctx):
+def _dense_recon_stats(ctx, layer_major: bool = False):
     label, recon, mask = ctx["label"], ctx["reconstructed"], ctx.get("mask")
+    if layer_major:     # per layer, as the reference's specs reduce (layers, batch, model) over the batch axis only
+        rows = [_dense_recon_stats({"label": label[l], "reconstructed": recon[l], "mask": mask}) for l in range(label.shape[0])]
+        return tuple(torch.stack([r[i] for r in rows]) for i in range(4))
     ntd = label.ndim - 1
     label_mean = apply_token_mask(label, ntd, mask, "mean")
     se = (recon - label).pow(2).sum(dim=-1)
@@ -239,6 +260,10 @@ def _dense_recon_stats(ctx):
     err = apply_token_mask(se.sqrt(), ntd, mask, "mean")
     ratio = err / apply_token_mask(label.norm(p=2, dim=-1), ntd, mask, "mean")
     return ev, legacy, err, ratio
+
+
+def _mean_if_vector(x):
+    return x.mean() if isinstance(x, torch.Tensor) and x.numel() > 1 else x
 
 
 def _on_gpu_2d(ctx) -> bool:
@@ -255,11 +280,12 @@ class ExplainedVarianceMetric(Metric):
         self.explained_variance_legacy = Record()
 
     def update(self, ctx):
+        lm = _layer_major(self.sae, ctx)
         if _on_gpu_2d(ctx):
-            st = _recon_step_stats(ctx)
+            st = _recon_step_stats(ctx, lm)
             ev, legacy = st[0], st[1]
         else:
-            ev, legacy, _, _ = _dense_recon_stats(ctx)
+            ev, legacy, _, _ = _dense_recon_stats(ctx, lm)
         self.explained_variance.update(ev)
         self.explained_variance_legacy.update(legacy)
         return {"explained_variance": ev, "explained_variance_legacy": legacy}
@@ -300,19 +326,22 @@ class L2NormErrorMetric(Metric):
         self.l2_norm_error_ratio = Record()
 
     def update(self, ctx):
+        lm = _layer_major(self.sae, ctx)
         if _on_gpu_2d(ctx):
-            st = _recon_step_stats(ctx)
+            st = _recon_step_stats(ctx, lm)
             err, ratio = st[2], st[3]
         else:
-            _, _, err, ratio = _dense_recon_stats(ctx)
+            _, _, err, ratio = _dense_recon_stats(ctx, lm)
         self.l2_norm_error.update(err)
         self.l2_norm_error_ratio.update(ratio)
         return {}
 
     def compute(self):
         return {
-            "metrics/l2_norm_error": item(self.l2_norm_error.compute()),
-            "metrics/l2_norm_error_ratio": item(self.l2_norm_error_ratio.compute()),
+            # a cross-layer transcoder has one value per layer here (the reference's `.item()` would refuse them):
+            # reported as their mean, as the explained variance is
+            "metrics/l2_norm_error": item(_mean_if_vector(self.l2_norm_error.compute())),
+            "metrics/l2_norm_error_ratio": item(_mean_if_vector(self.l2_norm_error_ratio.compute())),
         }
 
 

@@ -8,6 +8,7 @@ differently in bf16, so an entry close to the k-th value can legitimately fall o
 
 import contextlib
 import importlib
+import math
 
 import pytest
 import torch
@@ -535,3 +536,90 @@ def test_lorsa_adam_steps_under_autocast_with_the_dense_output_gradient(pkg, vo,
     assert seen[2] < seen[0]
     for a, c in zip(losses[True], losses[False]):
         assert abs(a - c) <= 2e-2 * abs(c)
+
+
+# ---- the trainer's step shell over the variants ---------------------------------------------------
+
+def _variant_case(pkg, vo, dev, kind):
+    g = torch.Generator().manual_seed(71)
+    if kind == "crosscoder":
+        H, d, F, k, B = 2, 64, 512, 8, 96
+        m, _, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=61)
+        batch = {h: torch.randn(B, d, generator=g) for h in hooks}
+        batch["tokens"] = torch.zeros(B, dtype=torch.long)
+        batch["mask"] = torch.ones(B, H)
+    elif kind == "clt":
+        L, d, F, k, B = 3, 64, 256, 4, 64
+        m, _, _, _ = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=62)
+        batch = clt_batch(L, B, d, seed=63)
+        batch["mask"] = torch.ones(B)
+    else:
+        d, F, h, dq, s, b, k = 64, 256, 4, 32, 64, 2, 8
+        m, _ = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=64, positional_embedding_type="rotary", rotary_dim=16,
+                          rotary_adjacent_pairs=False)
+        batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+        batch["mask"] = torch.ones(b, s)
+    return m, {k_: v.to(dev) for k_, v in batch.items()}
+
+
+@pytest.mark.parametrize("kind", ["crosscoder", "clt", "lorsa"])
+@pytest.mark.parametrize("clip", [0.0, 0.05])
+def test_variants_through_the_trainer_shell(pkg, vo, dev, kind, clip):
+    """`Trainer.train_one_step` (trainer.py:576-671) on the crosscoder, the cross-layer transcoder and Lorsa (with
+    rotary embeddings) under bf16 autocast: gradient norm every step (and clipping) over factored and dense gradients
+    alike, logging metrics on; the loss goes down, everything stays finite, the gradient norm is a positive number."""
+    print(f"trainer shell over {kind}, clip={clip}", flush=True)
+    m, gb = _variant_case(pkg, vo, dev, kind)
+    steps = 6
+    n_tok = int(gb["mask"].sum().item())
+    tcfg = pkg.TrainerConfig(lr=2e-3, lr_warm_up_steps=1, lr_cool_down_steps=1, total_training_tokens=n_tok * steps,
+                             amp_dtype=torch.bfloat16, skip_metrics_calculation=False, log_frequency=1,
+                             clip_grad_norm=clip, k_warmup_steps=0, l1_coefficient_warmup_steps=2)
+    trainer = pkg.Trainer(tcfg)
+    trainer.prepare(m, gb)
+    losses, norms = [], []
+    for _ in range(steps):
+        out = trainer.train_one_step(m, gb)
+        losses.append(float(out["loss"].detach()))
+        norms.append(float(out["grad_norm_before_clipping"]))
+    assert all(math.isfinite(v) for v in losses + norms) and all(n > 0 for n in norms)
+    assert losses[-1] < losses[0], losses
+    for n, p in m.named_parameters():
+        assert torch.isfinite(p).all(), n
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_clt_reconstruction_metrics_are_formed_per_layer(pkg, vo, oracle, dev, masked):
+    """A cross-layer transcoder's label / reconstruction are [layers, batch, d_model] and the token mask spans the batch
+    only (models/clt.py:54-69): the reference reduces over the batch axis, so explained variance and L2 error are one
+    value per layer (metrics.py:214-243, 297-303), each with that layer's own label mean, and the report is their mean."""
+    mo = importlib.import_module("oracle.metrics_oracle")
+    L, d, F, k, B = 3, 64, 256, 4, 64
+    m, _, _, _ = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=65)
+    batch = clt_batch(L, B, d, seed=66)
+    g = torch.Generator().manual_seed(67)
+    for l in range(L):      # layers with very different label means and scales: one pooled mean would be visibly wrong
+        batch[f"o{l}"] = batch[f"o{l}"] * (l + 1) + 3.0 * l
+    mask = (torch.rand(B, generator=g) > 0.3).float() if masked else None
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    if masked:
+        gb["mask"] = mask.to(dev)
+    ctx = m.compute_loss(gb)
+    label, recon = ctx["label"].detach().cpu(), ctx["reconstructed"].detach().cpu()
+    assert tuple(label.shape) == (L, B, d)
+    ev_m, l2_m = pkg.metrics.ExplainedVarianceMetric(m), pkg.metrics.L2NormErrorMetric(m)
+    step = dict(ctx)
+    got = ev_m.update(step)
+    l2_m.update(step)
+    want = [mo.explained_variance(label[l], recon[l], mask) for l in range(L)]
+    want_l2 = [mo.l2_norm_error(label[l], recon[l], mask) for l in range(L)]
+    assert tuple(got["explained_variance"].shape) == (L,)
+    for l in range(L):
+        assert abs(got["explained_variance"][l].item() - want[l][0].item()) < 1e-5 * max(1.0, abs(want[l][0].item()))
+        assert abs(got["explained_variance_legacy"][l].item() - want[l][1].item()) < 1e-4 * max(1.0, abs(want[l][1].item()))
+    rep, rep_l2 = ev_m.compute(), l2_m.compute()
+    assert rep["metrics/explained_variance"] == pytest.approx(sum(w[0].item() for w in want) / L, rel=1e-5, abs=1e-6)
+    assert rep_l2["metrics/l2_norm_error"] == pytest.approx(sum(w[0].item() for w in want_l2) / L, rel=1e-5)
+    assert rep_l2["metrics/l2_norm_error_ratio"] == pytest.approx(sum(w[1].item() for w in want_l2) / L, rel=1e-5)
+    pooled = mo.explained_variance(label.reshape(L * B, d), recon.reshape(L * B, d), None if mask is None else mask.repeat(L))[0].item()
+    assert abs(pooled - rep["metrics/explained_variance"]) > 1e-3      # the case does tell the two apart
