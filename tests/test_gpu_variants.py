@@ -623,3 +623,34 @@ def test_clt_reconstruction_metrics_are_formed_per_layer(pkg, vo, oracle, dev, m
     assert rep_l2["metrics/l2_norm_error_ratio"] == pytest.approx(sum(w[1].item() for w in want_l2) / L, rel=1e-5)
     pooled = mo.explained_variance(label.reshape(L * B, d), recon.reshape(L * B, d), None if mask is None else mask.repeat(L))[0].item()
     assert abs(pooled - rep["metrics/explained_variance"]) > 1e-3      # the case does tell the two apart
+
+
+@pytest.mark.parametrize("kind", ["crosscoder", "clt", "lorsa"])
+def test_variants_resume_bit_identically_from_a_trainer_checkpoint(pkg, vo, dev, kind, tmp_path):
+    """trainer.py:155-307 over the variants: three steps, a checkpoint, two more steps, against a fresh model loaded from
+    the checkpoint + `Trainer.from_checkpoint` taking the same two steps.  Parameters and Adam moments agree to the bit
+    (the moments of feature-major and stacked parameters go through torch's layout in the files)."""
+    m, gb = _variant_case(pkg, vo, dev, kind)
+    n_tok = int(gb["mask"].sum().item())
+    tcfg = pkg.TrainerConfig(total_training_tokens=5 * n_tok, lr=1e-3, lr_warm_up_steps=2, lr_cool_down_steps=2,
+                             amp_dtype=torch.bfloat16, k_warmup_steps=0, l1_coefficient=None, skip_metrics_calculation=True,
+                             exp_result_path=str(tmp_path / "results"))
+    tr = pkg.Trainer(tcfg)
+    tr.prepare(m, gb)
+    for _ in range(3):
+        tr.train_one_step(m, gb)
+    ckpt = tr.save_checkpoint(m, tmp_path / "run")
+    for _ in range(2):
+        tr.train_one_step(m, gb)
+    m2 = pkg.SparseDictionary.from_pretrained(str(ckpt), device="cuda", dtype=torch.float32)
+    assert type(m2) is type(m)
+    tr2 = pkg.Trainer.from_checkpoint(m2, str(ckpt))
+    assert tr2.cur_step == 3
+    tr2.fit(m2, iter([gb, gb]))
+    assert tr2.cur_step == 5
+    torch.cuda.synchronize()
+    for (n, p), q in zip(m.named_parameters(), m2.parameters()):
+        assert p.stride() == q.stride(), n
+        assert torch.equal(p, q), n
+        a, b = tr.optimizer.state[p], tr2.optimizer.state[q]
+        assert torch.equal(a["exp_avg"], b["exp_avg"]) and torch.equal(a["exp_avg_sq"], b["exp_avg_sq"]), n
