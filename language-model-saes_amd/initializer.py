@@ -68,6 +68,8 @@ class Initializer:
 
     def _init_encoder_side(self, sae: SparseDictionary, batch: dict) -> None:
         if self.cfg.init_encoder_with_decoder_transpose:
+            assert hasattr(sae, "init_encoder_with_decoder_transpose"), (
+                f"{type(sae).__name__} does not support encoder initialization from decoder")
             sae.init_encoder_with_decoder_transpose(self.cfg.init_encoder_with_decoder_transpose_factor)
         if self.cfg.init_encoder_bias_with_mean_hidden_pre:
             assert hasattr(sae, "init_encoder_bias_with_mean_hidden_pre"), (
@@ -94,7 +96,8 @@ class Initializer:
         batch = sae.normalize_activations(activation_batch)
         if self.cfg.bias_init_method == "geometric_median":
             assert sae.b_D is not None, "Decoder bias should exist if use_decoder_bias is True"
-            if hasattr(sae.cfg, "hook_points_out") and sae.b_D.ndim == 2:      # cross-layer transcoder: one bias per layer
+            # a cross-layer transcoder has one bias per layer (a list of vectors, or one [layers, d] tensor)
+            if hasattr(sae.cfg, "hook_points_out") and (not torch.is_tensor(sae.b_D) or sae.b_D.ndim == 2):
                 for i, hp in enumerate(sae.cfg.hook_points_out):
                     sae.b_D[i].copy_(batch[hp].mean(0))
             elif hasattr(sae.cfg, "hook_point_out"):

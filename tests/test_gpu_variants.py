@@ -654,3 +654,46 @@ def test_variants_resume_bit_identically_from_a_trainer_checkpoint(pkg, vo, dev,
         assert torch.equal(p, q), n
         a, b = tr.optimizer.state[p], tr2.optimizer.state[q]
         assert torch.equal(a["exp_avg"], b["exp_avg"]) and torch.equal(a["exp_avg_sq"], b["exp_avg_sq"]), n
+
+
+@pytest.mark.parametrize("kind", ["crosscoder", "clt", "lorsa"])
+def test_initializer_grid_search_over_the_variants(pkg, vo, dev, kind):
+    """initializer.py:115-148 on the variants: 70 forward passes, each after the decoder norms (and the encoder derived
+    from them) changed in place.  The norm it settles on is the argmin of the same losses taken on the generic op
+    sequence, and the kernel path's caches (bf16 copies, row norms) follow every in-place change: the loss after the
+    search equals the generic path's on the final weights."""
+    m, gb = _variant_case(pkg, vo, dev, kind)
+    gb = {k_: v for k_, v in gb.items() if k_ != "mask"}
+    if kind == "clt":    # no norm constraints on a cross-layer transcoder, in the reference as here: the bias start only
+        pkg.Initializer(pkg.InitializerConfig(grid_search_init_norm=False, bias_init_method="geometric_median",
+                                              init_encoder_with_decoder_transpose=False)).initialization_search(m, gb)
+        for i, hp in enumerate(m.cfg.hook_points_out):
+            assert torch.allclose(m.b_D[i].detach(), gb[hp].mean(0), atol=1e-6)
+        for bad in (dict(grid_search_init_norm=True, init_encoder_with_decoder_transpose=False),
+                    dict(grid_search_init_norm=False, init_encoder_with_decoder_transpose=True)):
+            with pytest.raises(AssertionError):
+                pkg.Initializer(pkg.InitializerConfig(**bad)).initialization_search(m, gb)
+        return
+    transpose = hasattr(m, "init_encoder_with_decoder_transpose")
+    # (the reference has no geometric-median bias start for a crosscoder either: initializer.py:95-113)
+    init = pkg.Initializer(pkg.InitializerConfig(grid_search_init_norm=True, init_encoder_with_decoder_transpose=transpose,
+                                                 bias_init_method="all_zero" if kind == "crosscoder" else "geometric_median"))
+    start = {n: p.detach().clone() for n, p in m.named_parameters()}
+    init.initialization_search(m, gb)
+    assert init.best_norm is not None and 0.0 < init.best_norm <= 5.1
+    with torch.no_grad():
+        got = m.compute_loss(gb)["l_rec"].mean().item()
+        want = pkg.SparseDictionary.compute_loss(m, gb)["l_rec"].mean().item()
+    assert abs(got - want) < 1e-4 * abs(want)
+    # the same search with every loss taken on the generic op sequence
+    with torch.no_grad():
+        for n, p in m.named_parameters():
+            p.copy_(start[n])
+    fused = type(m).compute_loss
+    try:
+        type(m).compute_loss = pkg.SparseDictionary.compute_loss
+        ref_init = pkg.Initializer(init.cfg)
+        ref_init.initialization_search(m, gb)
+    finally:
+        type(m).compute_loss = fused
+    assert ref_init.best_norm == pytest.approx(init.best_norm, abs=0.011)     # one step of the fine grid at most
