@@ -697,3 +697,38 @@ def test_initializer_grid_search_over_the_variants(pkg, vo, dev, kind):
     finally:
         type(m).compute_loss = fused
     assert ref_init.best_norm == pytest.approx(init.best_norm, abs=0.011)     # one step of the fine grid at most
+
+
+@pytest.mark.parametrize("kind", ["crosscoder", "clt", "lorsa"])
+@pytest.mark.parametrize("amp", [False, True])
+def test_variant_module_api_agrees_with_the_train_step(pkg, vo, dev, kind, amp):
+    """`encode` / `decode` / `forward` of the variants on GPU tensors (the reference's module API: dense feature
+    activations in, dense reconstructions out) against what `compute_loss` reports for the same batch: the same
+    selection, the same activations and reconstruction (fp32 1e-5; bf16 autocast at the bf16 bound, with the selection
+    compared where the two paths' pre-activations are not within rounding of the threshold)."""
+    m, gb = _variant_case(pkg, vo, dev, kind)
+    gb = {k_: v for k_, v in gb.items() if k_ != "mask"}
+    tol = BF16_TOL if amp else FP32_TOL
+    with (torch.autocast("cuda", dtype=torch.bfloat16) if amp else contextlib.nullcontext()), torch.no_grad():
+        ctx = m.compute_loss(gb)
+        x, enc_kw, dec_kw = m.prepare_input(gb)
+        acts, hidden = m.encode(x, return_hidden_pre=True, **enc_kw)
+        recon = m.decode(acts, **dec_kw)
+        out = m.forward(x, encoder_kwargs=enc_kw, decoder_kwargs=dec_kw)
+    want_acts, want_recon = ctx["feature_acts"].float(), ctx["reconstructed"].float()
+    assert acts.shape == want_acts.shape and recon.shape == want_recon.shape
+    if kind != "clt":        # a cross-layer transcoder's compute_loss reports no hidden_pre (models/clt.py:1024-1104)
+        assert rel_err(hidden.float(), ctx["hidden_pre"].float()) < tol
+    same = ((acts != 0) == (want_acts != 0)).float().mean().item()
+    assert same == 1.0 if not amp else same > 0.999, same
+    if not amp:
+        assert rel_err(acts.float(), want_acts) < tol
+    if amp:
+        # The op sequence rounds every head's product to bf16 before the sum over heads, the kernel path rounds the sum
+        # once: with these dense random inputs a few percent of the kept entries sit within that rounding of the k-th
+        # value and fall on the other side, and each moves its token's reconstruction by a whole decoder row.  The fp32
+        # runs above pin the values; here the two paths only have to agree in the large.
+        assert ((recon.float() - want_recon).norm() / want_recon.norm()).item() < 0.15
+    else:
+        assert rel_err(recon.float(), want_recon) < tol
+    assert rel_err(out.float(), recon.float()) < 1e-6
