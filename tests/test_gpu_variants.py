@@ -732,3 +732,39 @@ def test_variant_module_api_agrees_with_the_train_step(pkg, vo, dev, kind, amp):
     else:
         assert rel_err(recon.float(), want_recon) < tol
     assert rel_err(out.float(), recon.float()) < 1e-6
+
+
+@pytest.mark.parametrize("kind", ["sae", "crosscoder", "clt", "lorsa"])
+def test_sparseadam_through_the_trainer_shell(pkg, vo, oracle, dev, kind):
+    """`optimizer_class="sparseadam"` (trainer.py:375-378, optim.py:142-254) over the SAE and the variants: the masked
+    update needs element-wise gradients, so the weight gradients must arrive dense; loss falls, parameters stay finite,
+    and a parameter whose gradient was zero everywhere does not move."""
+    if kind == "sae":
+        from lm_saes_amd import synthetic
+        d, F, k, B = 128, 1024, 8, 96
+        x = synthetic.activations(B, d, 8, seed=81)
+        w = synthetic.sae_weights(d, F, x, seed=81)
+        cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="topk",
+                            top_k=k, norm_activation="inference", device="cuda", dtype=torch.float32)
+        m = pkg.SparseAutoEncoder(cfg)
+        synthetic.load_weights(m, *[t.to(dev) for t in w])
+        gb = {"in": x.to(dev), "out": x.to(dev), "tokens": torch.zeros(B, device=dev), "mask": torch.ones(B, device=dev)}
+    else:
+        m, gb = _variant_case(pkg, vo, dev, kind)
+    steps = 5
+    n_tok = int(gb["mask"].sum().item())
+    tcfg = pkg.TrainerConfig(lr=2e-3, lr_warm_up_steps=1, lr_cool_down_steps=1, total_training_tokens=n_tok * steps,
+                             amp_dtype=torch.bfloat16, skip_metrics_calculation=True, clip_grad_norm=0.0, k_warmup_steps=0,
+                             l1_coefficient_warmup_steps=2, optimizer_class="sparseadam")
+    trainer = pkg.Trainer(tcfg)
+    trainer.prepare(m, gb)
+    assert type(trainer.optimizer).__name__ == "HipSparseAdam"
+    losses = []
+    for _ in range(steps):
+        out = trainer.train_one_step(m, gb)
+        losses.append(float(out["loss"].detach()))
+        for n, p in m.named_parameters():
+            assert getattr(p, "_sparse_grad", None) is None, n      # nothing factored is left behind for an optimiser that cannot read it
+    assert all(math.isfinite(v) for v in losses) and losses[-1] < losses[0], losses
+    for n, p in m.named_parameters():
+        assert torch.isfinite(p).all(), n
