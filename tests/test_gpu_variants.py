@@ -768,3 +768,29 @@ def test_sparseadam_through_the_trainer_shell(pkg, vo, oracle, dev, kind):
     assert all(math.isfinite(v) for v in losses) and losses[-1] < losses[0], losses
     for n, p in m.named_parameters():
         assert torch.isfinite(p).all(), n
+
+
+@pytest.mark.parametrize("kind", ["crosscoder", "clt", "lorsa"])
+def test_k_annealing_reaches_the_variant_kernels(pkg, vo, dev, kind):
+    """trainer.py:462-485: `set_current_k` moves from `initial_k` down to `top_k` over the warm-up; the fused steps of
+    the variants must keep exactly the current number per token (and head / layer) at every step."""
+    m, gb = _variant_case(pkg, vo, dev, kind)
+    k = m.cfg.top_k
+    n_tok = int(gb["mask"].sum().item())
+    steps = 6
+    tcfg = pkg.TrainerConfig(lr=1e-3, lr_warm_up_steps=1, lr_cool_down_steps=1, total_training_tokens=n_tok * steps,
+                             amp_dtype=torch.bfloat16, skip_metrics_calculation=True, k_warmup_steps=4, initial_k=3 * k,
+                             k_schedule_type="linear", l1_coefficient_warmup_steps=2)
+    trainer = pkg.Trainer(tcfg)
+    trainer.prepare(m, gb)
+    seen = []
+    for _ in range(steps):
+        trainer.train_one_step(m, gb)
+        cur = int(m.current_k)
+        seen.append(cur)
+        with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+            ctx = m.compute_loss(gb)
+        acts = ctx["feature_acts"]
+        per_row = (acts != 0).sum(-1)
+        assert int(per_row.max()) == cur and int(per_row.min()) == cur, (kind, cur, int(per_row.min()), int(per_row.max()))
+    assert seen[0] > k and seen[-1] == k and all(a >= b for a, b in zip(seen, seen[1:])), seen
