@@ -1,13 +1,15 @@
-"""Randomized parity sweep over the crosscoder, the cross-layer transcoder and Lorsa in fp32: shapes, activation
-scopes, masks and positional embeddings are drawn from a seeded generator and every case's loss, outputs and
-parameter gradients are checked against the variants' oracle (crosscoder.py:221-469, clt.py:527-709, 837-876,
-lorsa.py:683-829).  Each case prints its parameters before it runs.
+"""Randomized parity sweep over the crosscoder, the cross-layer transcoder and Lorsa: shapes, activation scopes,
+masks and positional embeddings are drawn from a seeded generator and every case's loss, outputs and parameter
+gradients are checked against the variants' oracle (crosscoder.py:221-469, clt.py:527-709, 837-876,
+lorsa.py:683-829), in fp32 and under bf16 autocast (there with the stage-by-stage checks of the fixed-shape tests: the
+oracle's bf16 step on the kernels' own selection).  Each case prints its parameters before it runs.
 
 The GEMMs on the two sides add in different orders, so two pre-activations that differ in their last bits may swap
 places at the k-th rank: a case whose selections differ in a handful of entries is counted as a flip and its further
 comparisons are skipped; flips must stay rare, and a selection that differs by more than that fails."""
 
 import importlib.util
+import math
 import os
 import random
 
@@ -120,3 +122,32 @@ def test_lorsa_random_shapes(pkg, vo, dev, sweep_seed):
         want = ref.compute_loss(batch, mask=mask)
         flips += not compare(out, want, m, ref)
     few_flips(flips, N_CASES)
+
+
+N_BF16_CASES = 12
+
+
+@pytest.mark.parametrize("sweep_seed", [31, 41, 51])
+def test_bf16_steps_over_random_shapes(pkg, vo, dev, sweep_seed):
+    rng = random.Random(sweep_seed)
+    for n in range(N_BF16_CASES):
+        seed = rng.randrange(1 << 20)
+        H = rng.choice([2, 3, 4]); d = rng.choice([64, 128]); F = rng.choice([256, 512, 1024]); k = rng.choice([4, 16])
+        B = rng.choice([64, 96, 130])
+        print(f"[{n}] crosscoder bf16 seed={seed} H={H} d={d} F={F} k={k} B={B}", flush=True)
+        tv.crosscoder_bf16_step(pkg, vo, dev, H, d, F, k, B, seed=seed)
+    for n in range(N_BF16_CASES):
+        seed = rng.randrange(1 << 20)
+        act_fn = rng.choice(["topk", "topk", "layertopk", "batchtopk", "batchlayertopk"])
+        L = rng.choice([2, 3, 4]); d = rng.choice([64, 128]); F = rng.choice([256, 512]); k = rng.choice([4, 8]); B = rng.choice([64, 96, 160])
+        print(f"[{n}] clt bf16 seed={seed} {act_fn} L={L} d={d} F={F} k={k} B={B}", flush=True)
+        tv.clt_bf16_step(pkg, vo, dev, act_fn, L, d, F, k, B, seed=seed)
+    for n in range(N_BF16_CASES):
+        seed = rng.randrange(1 << 20)
+        d = rng.choice([64, 128]); h = rng.choice([2, 4, 8]); dv = rng.choice([32, 64, 128]); dq = rng.choice([32, 64])
+        s = rng.choice([8, 24, 64, 104]); b = (64 // math.gcd(s, 64)) * rng.choice([1, 2]); dense = rng.random() < 0.5
+        kw = rng.choice([dict(positional_embedding_type="none"),
+                         dict(positional_embedding_type="rotary", rotary_dim=rng.choice([16, 32, dq]),
+                              rotary_adjacent_pairs=rng.random() < 0.5)])
+        print(f"[{n}] lorsa bf16 seed={seed} d={d} h={h} dv={dv} dq={dq} s={s} b={b} dense={dense} {kw}", flush=True)
+        tv.lorsa_bf16_step(pkg, vo, dev, d, h * dv, h, dq, s, b, dense, seed=seed, **kw)

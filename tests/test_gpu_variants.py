@@ -74,8 +74,36 @@ def check_bf16_grads_on_the_kernels_selection(model, ref, run_ref, kept_cpu):
         if rp[n].grad.abs().max().item() < 1e-2 * scale:
             continue     # analytically zero (a key bias shifts a softmax row alike) or below the bf16 noise of the step
         errs[n] = rel_err(p.grad, rp[n].grad)
-    assert all(e < BF16_TOL for e in errs.values()), sorted(errs.items(), key=lambda kv: -kv[1])[:4]
+    far = [n for n, e in errs.items() if e >= BF16_TOL]
+    if far:
+        # two bf16 evaluations of a sum that nearly cancels (few tokens, a bias of the keys) can lie further from one
+        # another than either lies from the exact value: such a parameter is judged against the oracle's fp32 gradients
+        # on the same selection, where the kernel path may be no further off than 1.5 x the oracle's own bf16 step
+        g16 = {n: rp[n].grad.clone() for n in far}
+        for p in ref.parameters():
+            p.grad = None
+        run_ref()["loss"].backward()
+        mp = dict(model.named_parameters())
+        for n in far:
+            ours, theirs = rel_err(mp[n].grad, rp[n].grad), rel_err(g16[n], rp[n].grad)
+            assert ours <= max(BF16_TOL, 1.5 * theirs), (n, errs[n], ours, theirs)
     return want
+
+
+def assert_close_in_bf16(got, w16, run_ref_fp32, keys):
+    """`got[key]` against the oracle's bf16 step `w16[key]` at the bf16 bound; an output for which the two bf16
+    evaluations lie further apart (long softmax rows over large scores) is judged against the oracle's fp32 step on
+    the same selection, as the gradients are."""
+    w32 = None
+    for key in keys:
+        e = rel_err(got[key], w16[key])
+        if e < BF16_TOL:
+            continue
+        if w32 is None:
+            with torch.no_grad():
+                w32 = run_ref_fp32()
+        ours, theirs = rel_err(got[key], w32[key]), rel_err(w16[key], w32[key])
+        assert ours <= max(BF16_TOL, 1.5 * theirs), (key, e, ours, theirs)
 
 
 # ---- crosscoder ----------------------------------------------------------------------------------
@@ -184,9 +212,12 @@ def test_crosscoder_factored_gradients_over_adam_steps(pkg, vo, oracle, dev, amp
 
 
 def test_crosscoder_fused_step_bf16(pkg, vo, dev):
-    H, d, F, k, B = 2, 64, 1024, 16, 128
-    m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=35)
-    g = torch.Generator().manual_seed(36)
+    crosscoder_bf16_step(pkg, vo, dev, 2, 64, 1024, 16, 128, seed=35)
+
+
+def crosscoder_bf16_step(pkg, vo, dev, H, d, F, k, B, seed):
+    m, ref, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
     batch = {h: torch.randn(B, d, generator=g) for h in hooks}
     batch["tokens"] = torch.zeros(B, dtype=torch.long)
     gb = {k_: v.to(dev) for k_, v in batch.items()}
@@ -350,9 +381,12 @@ def test_clt_factored_gradients_follow_the_oracle_over_steps(pkg, vo, oracle, de
 
 
 def test_clt_fused_step_bf16(pkg, vo, dev):
-    L, d, F, k, B = 3, 64, 512, 8, 96
-    m, ref, hin, hout = make_clt(pkg, vo, dev, "topk", L, d, F, k, seed=45)
-    batch = clt_batch(L, B, d, seed=46)
+    clt_bf16_step(pkg, vo, dev, "topk", 3, 64, 512, 8, 96, seed=45)
+
+
+def clt_bf16_step(pkg, vo, dev, act_fn, L, d, F, k, B, seed, include_norm=True):
+    m, ref, hin, hout = make_clt(pkg, vo, dev, act_fn, L, d, F, k, seed=seed, include_norm=include_norm)
+    batch = clt_batch(L, B, d, seed=seed + 1)
     gb = {k_: v.to(dev) for k_, v in batch.items()}
     with torch.autocast("cuda", dtype=torch.bfloat16):
         out = m.compute_loss(gb)
@@ -363,7 +397,7 @@ def test_clt_fused_step_bf16(pkg, vo, dev):
     assert agree > 0.999
     out["loss"].backward()
     w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch, hin, hout), kept)
-    assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["loss"], w16["loss"]) < BF16_TOL
+    assert_close_in_bf16(out, w16, lambda: ref.compute_loss(batch, hin, hout), ("reconstructed", "loss"))
 
 
 def test_clt_granule_route_changes_nothing(pkg, vo, dev):
@@ -457,11 +491,11 @@ def test_lorsa_bf16_step_with_other_query_key_forms_runs_the_attention_kernels(p
     assert "attention_bwd" in timer.records and "rotary_fwd" not in timer.records
 
 
-def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, **kw):
+def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, seed=53, **kw):
     k = 8
-    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=53, **kw)
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=seed, **kw)
     m.dense_decoder_grad = dense
-    g = torch.Generator().manual_seed(54)
+    g = torch.Generator().manual_seed(seed + 1)
     with torch.no_grad():      # non-zero projection biases, so that the kernels' bias path is exercised
         for n in ("b_Q", "b_K", "b_V"):
             getattr(ref, n).copy_(0.2 * torch.randn(getattr(ref, n).shape, generator=g))
@@ -480,7 +514,7 @@ def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, **kw):
     assert ("code_to_dense_t" in timer.records) == dense
     kept = (out["feature_acts"] > 0).cpu()
     w16 = check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch), kept)
-    assert rel_err(out["reconstructed"], w16["reconstructed"]) < BF16_TOL and rel_err(out["hidden_pre"], w16["hidden_pre"]) < BF16_TOL
+    assert_close_in_bf16(out, w16, lambda: ref.compute_loss(batch), ("reconstructed", "hidden_pre"))
     return timer
 
 
