@@ -441,11 +441,13 @@ int sae_code_to_dense_t(const int32_t *idx, const float *val, const int64_t *row
  * [B, nnz_max] pair) as two passes.
  *   sae_dense_row_nnz: row_nnz[b] = #{f : dense[b, f] != 0}.
  *   sae_dense_to_code: given row_off (int64 [B], e.g. the exclusive prefix sum of row_nnz), token b's non-zero entries
- *     are written in ascending feature order to idx / val [capacity] from slot row_off[b] on; slots at or past
- *     `capacity` are dropped.  (row_off, row_nnz, idx, val) is then a sparse code as the select entry points emit it. */
+ *     are written in ascending feature order to idx / val [capacity] from slot row_off[b] on; entries that would land at
+ *     or past `capacity` are dropped, and `row_nnz` (nullable, int32 [B], rewritten) is cut to the number of entries that
+ *     were written for each token, so that a code with an undersized capacity stays walkable (truncated, never out of
+ *     bounds).  (row_off, row_nnz, idx, val) is then a sparse code as the select entry points emit it. */
 int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_t F, int32_t *row_nnz, void *stream);
 int sae_dense_to_code(const void *dense, int dtype, int64_t B, int64_t F, const int64_t *row_off, int32_t *idx, float *val,
-                      int64_t capacity, void *stream);
+                      int64_t capacity, int32_t *row_nnz, void *stream);
 
 /* ---- Activation batches from a shuffle buffer -----------------------------------------------------------
  * dst[i, :] = cast(scale * src[row_idx[i], :]) for i < n_rows: one batch drawn from a token buffer that

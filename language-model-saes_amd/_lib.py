@@ -73,7 +73,7 @@ SIGNATURES = {
     "sae_rotary_bwd_t": (_I, [_P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _P]),
     "sae_row_sum": (_I, [_P, _I, _L, _L, _P, _P]),
     "sae_dense_row_nnz": (_I, [_P, _I, _L, _L, _P, _P]),
-    "sae_dense_to_code": (_I, [_P, _I, _L, _L, _P, _P, _P, _L, _P]),
+    "sae_dense_to_code": (_I, [_P, _I, _L, _L, _P, _P, _P, _L, _P, _P]),
     "sae_jumprelu_select_count": (_I, [_P, _I, _P, _P, _P, _P, _F, _L, _L, _P, _P]),
     "sae_jumprelu_select_emit": (_I, [_P, _I, _P, _P, _P, _P, _P, _F, _F, _L, _L, _P, _P, _P, _P, _L, _P, _P, _P]),
     "sae_encoder_gemm_jumprelu_margin": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P]),

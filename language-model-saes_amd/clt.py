@@ -27,9 +27,9 @@ import torch
 from torch import nn
 
 from . import ops
-from .activation_functions import JumpReLU, _topk_mask_lowest_index, topk_dense
+from .activation_functions import JumpReLU, _topk_mask_lowest_index, batch_topk_dense, topk_dense
 from .config import CLTConfig, register_sae_model
-from .sae import SparseRowGrad, SparseRowGradPieces, _autocast_dtype
+from .sae import SparseRowGrad, SparseRowGradPieces, _autocast_dtype, _gemm_k_ok, _rows_over_tokens
 from .sparse_dictionary import LazyDict, SparseDictionary
 
 _TOPK_FAMILY = ("topk", "layertopk", "batchtopk", "batchlayertopk")
@@ -215,6 +215,84 @@ class _FusedCLTStep(torch.autograd.Function):
         return (dx, dlabel, None, None, dW_E, db_E, *dW_D, *db_D)
 
 
+class _LayerEncoderGemm(torch.autograd.Function):
+    """pre[b, l, :] = x[b, l, :] @ W_E[l] for every layer on the GEMM kernel (clt.py:559, "...ld,lds->...ls"): one launch
+    per layer into one [L, B, F] buffer, returned as its [B, L, F] view.  Backward: per layer the weight gradient
+    d(pre)^T x as a product over the token axis on the same kernel."""
+
+    @staticmethod
+    def forward(ctx, x, W_E, w_op, amp):
+        B, L, d = x.shape
+        F = w_op.shape[1]
+        x_l = x.permute(1, 0, 2).contiguous()                                    # [L, B, d]
+        if amp:
+            x_op = x_l if x_l.dtype == torch.bfloat16 else ops.cast_bf16(x_l.float().view(L * B, d)).view(L, B, d)
+        else:
+            x_op = x_l.float()
+        out_dtype = torch.bfloat16 if amp else torch.float32
+        pre = torch.empty(L, B, F, dtype=out_dtype, device=x.device)
+        for l in range(L):
+            ops.encoder_gemm(x_op[l], w_op[l], out_dtype, out=pre[l])
+        ctx.save_for_backward(x_op, w_op)
+        ctx.x_dtype, ctx.w_dtype = x.dtype, W_E.dtype
+        return pre.permute(1, 0, 2)
+
+    @staticmethod
+    def backward(ctx, g):
+        x_op, w_op = ctx.saved_tensors
+        L = x_op.shape[0]
+        gl = g.permute(1, 0, 2).to(w_op.dtype).contiguous()                     # [L, B, F]
+        dx = dW = None
+        if ctx.needs_input_grad[0]:   # rare (activations carry no gradient in training): library products
+            dx = torch.stack([gl[l] @ w_op[l] for l in range(L)], dim=1).to(ctx.x_dtype)
+        if ctx.needs_input_grad[1]:
+            rows = torch.stack([_rows_over_tokens(gl[l], x_op[l], w_op.dtype) for l in range(L)])      # [L, F, d]
+            dW = rows.permute(0, 2, 1).to(ctx.w_dtype)
+        return dx, dW, None, None
+
+
+class _PrefixDecode(torch.autograd.Function):
+    """out[j] = sum_{i <= j} feature_acts[:, i, :] @ W_D[j][i] for every output layer j (clt.py:630-709), for activations
+    given as one sparse code over the L F concatenated features (ascending (layer, feature) inside a token): output layer j
+    gathers the rows of W_D[j], read as [(j + 1) F, d], that the token's entries of layers <= j name.  Backward: the value
+    gradients of the L decodes summed and scattered back to the dense activations, and per decoder group the gradient rows
+    from the feature index (a feature prefix of the one index built for the whole code)."""
+
+    @staticmethod
+    def forward(ctx, acts2, code, prefix_t, dims, w_ops, *W_D):
+        L, F, d = dims
+        B = code.n_tokens
+        out = torch.empty(L, B, d, dtype=torch.float32, device=acts2.device)
+        for j in range(L):
+            code_j = dataclasses.replace(code, row_nnz=prefix_t[j], d_sae=(j + 1) * F)
+            out[j] = ops.sparse_decode_fwd(code_j, w_ops[j].view((j + 1) * F, d), None)
+        ctx.code, ctx.prefix_t, ctx.dims, ctx.w_ops = code, prefix_t, dims, w_ops
+        ctx.in_dtype, ctx.w_dtype = acts2.dtype, W_D[0].dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        L, F, d = ctx.dims
+        code, prefix_t, w_ops = ctx.code, ctx.prefix_t, ctx.w_ops
+        g = g.float().contiguous()
+        d_acts = None
+        if ctx.needs_input_grad[0]:
+            dval = None
+            for j in range(L):
+                code_j = dataclasses.replace(code, row_nnz=prefix_t[j], d_sae=(j + 1) * F)
+                dv = ops.sparse_decode_bwd_dval(code_j, g[j], w_ops[j].view((j + 1) * F, d))    # zero past the prefix
+                dval = dv if dval is None else dval.add_(dv)
+            d_acts = ops.code_to_dense(dataclasses.replace(code, val=dval), L * F)[0].to(ctx.in_dtype)
+        dW = [None] * L
+        if any(ctx.needs_input_grad[5:]):
+            fi = ops.build_feature_index(code)
+            for j in range(L):
+                if ctx.needs_input_grad[5 + j]:
+                    fi_j = ops.FeatureIndex(fi.feat_ptr[: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)
+                    dW[j] = ops.sparse_grad_rows(fi_j, code.val, g[j], (j + 1) * F)[0].view(j + 1, F, d).to(ctx.w_dtype)
+        return (d_acts, None, None, None, None, *dW)
+
+
 @register_sae_model("clt")
 class CrossLayerTranscoder(SparseDictionary):
     def __init__(self, cfg: CLTConfig, device_mesh=None):
@@ -230,6 +308,9 @@ class CrossLayerTranscoder(SparseDictionary):
         # set by an optimiser that consumes factored gradients (HipAdam): the fused backward then attaches them to
         # W_E / W_D[j] as `_sparse_grad` instead of writing dense gradient rows
         self.defer_weight_grads = False
+        # `decode` of dense activations takes the sparse decoder kernels when they are sparse enough; False keeps the
+        # dense products whatever the input
+        self.sparse_api_decode = True
 
     # ---- activations (clt.py:232-387): the selection scope depends on the name ----
     def activation_function_factory(self, device_mesh=None):
@@ -252,6 +333,16 @@ class CrossLayerTranscoder(SparseDictionary):
             # dense form of the wider scopes: positive part, then keep the k (or k * batch) largest of every
             # group; a group's members are flattened in the order the reference permutes them (selected dims last,
             # in the order named), so ties fall to the same element
+            if x.is_cuda and x.ndim == 3 and x.shape[0] <= 131072:
+                # the select kernels behind their dense-in / dense-out forms (lowest flattened index wins a tie, which is
+                # the order of the arrangement each scope is handed over in)
+                B, L, F = x.shape
+                if act == "layertopk":
+                    return topk_dense(x.reshape(B, L * F), self.current_k).view(B, L, F)
+                if act == "batchtopk":
+                    return torch.stack([batch_topk_dense(x[:, l, :].contiguous(), self.current_k * B) for l in range(L)], dim=1)
+                flat = batch_topk_dense(x.permute(0, 2, 1).reshape(B, F * L), self.current_k * B)
+                return flat.view(B, F, L).permute(0, 2, 1)
             r = x * x.gt(0).to(x.dtype)
             B, L, F = r.shape
             if act == "layertopk":
@@ -378,8 +469,21 @@ class CrossLayerTranscoder(SparseDictionary):
         self.cfg.norm_activation = "inference"
 
     # ---- API path over dense tensors (clt.py:527-709) ----
+    def _layer_products(self, x: torch.Tensor) -> torch.Tensor:
+        """einsum("...ld,lds->...ls", x, W_E) (clt.py:559): the GEMM kernel layer by layer on GPU tensors whose shapes it
+        takes, the library routine otherwise."""
+        L, d, F = self.cfg.n_layers, self.cfg.d_model, self.cfg.d_sae
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        low = amp or self.W_E.dtype == torch.bfloat16
+        if (x.is_cuda and self.W_E.is_cuda and tuple(x.shape[-2:]) == (L, d) and self.W_E.dtype in (torch.float32, torch.bfloat16)
+                and _gemm_k_ok(d, torch.bfloat16 if low else torch.float32)):
+            lead = x.shape[:-2]
+            pre = _LayerEncoderGemm.apply(x.reshape(-1, L, d).to(self.W_E.dtype), self.W_E, self._w_enc_operand(amp), low)
+            return pre.reshape(*lead, L, F)
+        return torch.einsum("...ld,lds->...ls", x, self.W_E)
+
     def encode(self, x: torch.Tensor, return_hidden_pre: bool = False, **kwargs):
-        hidden_pre = torch.einsum("...ld,lds->...ls", x, self.W_E) + self.b_E
+        hidden_pre = self._layer_products(x) + self.b_E
         if self.cfg.sparsity_include_decoder_norm:
             hidden_pre = hidden_pre * self.decoder_norm_per_feature()
         feature_acts = self.activation_function(hidden_pre)
@@ -388,11 +492,30 @@ class CrossLayerTranscoder(SparseDictionary):
         return (feature_acts, hidden_pre) if return_hidden_pre else feature_acts
 
     def decode(self, feature_acts: torch.Tensor, batch_first: bool = False, **kwargs):
-        out = []
-        for layer_to in range(self.cfg.n_layers):
-            contribution = (feature_acts[..., : layer_to + 1, :].permute(1, 0, 2) @ self.W_D[layer_to]).sum(0)
-            out.append(contribution + self.b_D[layer_to])
-        return torch.stack(out, dim=1 if batch_first else 0)
+        """feature_acts [.., L, F] -> [L, .., d] (clt.py:630-709).  Activations that are sparse enough (at most
+        cfg.sparsity_threshold_for_csr of the entries non-zero: the reference's own bound for its sparse decode, counted on
+        the device and read once) become one sparse code over the L F concatenated features and every output layer is a
+        sparse decode of its per-token prefix, with a sparse backward.  Denser activations take one 2-D product per
+        output layer, [.., (j + 1) F] x [(j + 1) F, d] (the reference's batched product over a permuted view, followed by a
+        sum over the source layers, is the same sum; a library batched bf16 product over such a view returned wrong
+        weight gradients for source layer 0 at 12 layers x 12288 features)."""
+        L, d, F = self.cfg.n_layers, self.cfg.d_model, self.cfg.d_sae
+        lead = feature_acts.shape[:-2]
+        acts2 = feature_acts.reshape(-1, L * F)
+        out = None
+        if (self._sparse_decode_allowed(feature_acts) and tuple(feature_acts.shape[-2:]) == (L, F) and d % 8 == 0
+                and self.W_D[0].dtype in (torch.float32, torch.bfloat16) and acts2.shape[0] <= 131072):
+            src = (acts2 if acts2.dtype in (torch.float32, torch.bfloat16) else acts2.float()).contiguous()
+            code = ops.dense_to_code(src, max_entries=int(self.cfg.sparsity_threshold_for_csr * src.numel()))
+            if code is not None:
+                amp = _autocast_dtype("cuda") == torch.bfloat16
+                prefix_t = torch.cumsum(layer_counts(code, L, F), dim=1).to(torch.int32).t().contiguous()    # [L, B]
+                out = _PrefixDecode.apply(acts2, code, prefix_t, (L, F, d), self._w_dec_operands(amp), *self.W_D)
+                out = out + torch.stack(list(self.b_D)).unsqueeze(1)
+        if out is None:
+            out = torch.stack([acts2[:, : (j + 1) * F] @ self.W_D[j].view((j + 1) * F, d) + self.b_D[j] for j in range(L)])
+        out = out.view(L, *lead, d)
+        return out.movedim(0, -2) if batch_first else out
 
     def prepare_input(self, batch: dict[str, torch.Tensor], **kwargs) -> tuple[torch.Tensor, dict[str, Any], dict[str, Any]]:
         xs = []

@@ -128,6 +128,9 @@ class Crosscoder(SparseDictionary):
         # set by an optimiser that consumes factored gradients (HipAdam): the weight gradients are then attached to the
         # parameters as `_sparse_grad` instead of being written as dense rows
         self.defer_weight_grads = False
+        # `decode` of dense activations takes the sparse decoder kernels when they are sparse enough; False keeps the
+        # reference's dense product whatever the input
+        self.sparse_api_decode = True
 
     # ---- kernel operands ----
     def _w_enc_operand(self, amp: bool) -> torch.Tensor:
@@ -213,16 +216,48 @@ class Crosscoder(SparseDictionary):
         return self.decoder_inner_product_matrices() / torch.einsum("is,js->sij", n, n)
 
     # ---- API path over dense tensors (crosscoder.py:221-469) ----
+    def _summed_encoding(self, x: torch.Tensor) -> torch.Tensor:
+        """sum_h (x_h @ W_E[h] + b_E[h]) [.., F] (crosscoder.py:222-275, 353-375): on GPU tensors ONE product of the GEMM
+        kernel over the concatenated model axis (K = H d, fp32 accumulation over all heads, one rounding under autocast
+        where the reference rounds every head's product), whose weight gradient is a product over the token axis on
+        the same kernel; the reference's op sequence otherwise."""
+        H, d, F = self.cfg.n_heads, self.cfg.d_model, self.cfg.d_sae
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        low = amp or self.W_E.dtype == torch.bfloat16
+        if (x.is_cuda and self.W_E.is_cuda and tuple(x.shape[-2:]) == (H, d) and self.W_E.dtype in (torch.float32, torch.bfloat16)
+                and (H * d) % (64 if low else 32) == 0):
+            from .sae import _EncoderGemm
+
+            lead = x.shape[:-2]
+            pre = _EncoderGemm.apply(x.reshape(-1, H * d).to(self.W_E.dtype), self.W_E, self._w_enc_operand(amp), low, False, None,
+                                     lambda rows: rows.view(F, H, d).permute(1, 2, 0))
+            return pre.view(*lead, F) + self.b_E.sum(dim=0)
+        return (torch.einsum("...hd,hdf->...hf", x, self.W_E) + self.b_E).sum(dim=-2)
+
     def encode(self, x: torch.Tensor, return_hidden_pre: bool = False, **kwargs):
         H, F = self.cfg.n_heads, self.cfg.d_sae
-        per_head = torch.einsum("...hd,hdf->...hf", x, self.W_E) + self.b_E
-        acc = per_head.sum(dim=-2)
+        acc = self._summed_encoding(x)
         acc = acc.unsqueeze(-2).expand(*acc.shape[:-1], H, F)
         n = self.decoder_norm()
         feature_acts = self.activation_function(acc * n) / n
         return (feature_acts, acc) if return_hidden_pre else feature_acts
 
     def decode(self, feature_acts: torch.Tensor, **kwargs):
+        """feature_acts [.., H, F] -> [.., H, d] (crosscoder.py:384-469).  Activations that are sparse enough (at most
+        1 - cfg.sparsity_threshold_for_triton_spmm_kernel of the entries non-zero, counted on the device and read once, as
+        the SAE's gate reads `max_l0`) go through the sparse decoder kernels, every head at once: row (token, head) of the
+        activations gathers its rows from head h's block of W_D [H F, d]; its backward is the sparse one as well."""
+        H, d, F = self.cfg.n_heads, self.cfg.d_model, self.cfg.d_sae
+        if (self._sparse_decode_allowed(feature_acts) and tuple(feature_acts.shape[-2:]) == (H, F) and d % 8 == 0
+                and self.W_D.dtype in (torch.float32, torch.bfloat16) and feature_acts.numel() < 2 ** 40):
+            from .kernels import sparse_decode_blocks
+
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            lead = feature_acts.shape[:-2]
+            out = sparse_decode_blocks(feature_acts.reshape(-1, F), self.W_D.view(H * F, d), self._w_dec_operand(amp).view(H * F, d),
+                                       n_blocks=H, max_density=1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel)
+            if out is not None:
+                return out.view(*lead, H, d) + self.b_D
         return torch.einsum("...hf,hfd->...hd", feature_acts, self.W_D) + self.b_D
 
     def prepare_input(self, batch: dict[str, torch.Tensor], **kwargs) -> tuple[torch.Tensor, dict[str, Any], dict[str, Any]]:

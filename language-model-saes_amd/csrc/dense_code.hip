@@ -51,10 +51,13 @@ __global__ __launch_bounds__(256) void dense_row_nnz_kernel(const void *__restri
   if (threadIdx.x == 0) row_nnz[b] = (int32_t)total;
 }
 
-// one workgroup per token: the non-zeros of the row, in ascending feature order, to idx / val from row_off[b] on
+// one workgroup per token: the non-zeros of the row, in ascending feature order, to idx / val from row_off[b] on; entries
+// that would land at or past `capacity` are not written, and `row_nnz` (optional) is cut to the entries that were, so
+// that no consumer of the code walks past the arrays
 template <bool BF16>
 __global__ __launch_bounds__(256) void dense_to_code_kernel(const void *__restrict__ dense, int64_t F, const int64_t *__restrict__ row_off,
-                                                            int32_t *__restrict__ idx, float *__restrict__ val, int64_t capacity) {
+                                                            int32_t *__restrict__ idx, float *__restrict__ val, int64_t capacity,
+                                                            int32_t *__restrict__ row_nnz) {
   __shared__ int wave_tot[4];
   const int64_t b = blockIdx.x;
   const char *row = reinterpret_cast<const char *>(dense) + b * F * (BF16 ? 2 : 4);
@@ -100,6 +103,10 @@ __global__ __launch_bounds__(256) void dense_to_code_kernel(const void *__restri
       }
     }
     run += total;
+  }
+  if (row_nnz && threadIdx.x == 0) {
+    const int64_t first = row_off[b], room = capacity > first ? capacity - first : 0, found = run - first;
+    row_nnz[b] = (int32_t)(found < room ? found : room);
   }
 }
 
@@ -151,16 +158,16 @@ extern "C" int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_
 }
 
 extern "C" int sae_dense_to_code(const void *dense, int dtype, int64_t B, int64_t F, const int64_t *row_off, int32_t *idx,
-                                 float *val, int64_t capacity, void *stream) {
+                                 float *val, int64_t capacity, int32_t *row_nnz, void *stream) {
   using namespace sae;
   SAE_REQUIRE(dense && row_off && idx && val, SAE_ERR_INVALID_ARG, "dense_to_code: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < ((int64_t)1 << 31) && F < ((int64_t)1 << 31) && capacity >= 0, SAE_ERR_INVALID_ARG,
               "dense_to_code: bad shape");
   SAE_REQUIRE(dtype == SAE_F32 || dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "dense_to_code: bad dtype");
   if (dtype == SAE_BF16)
-    hipLaunchKernelGGL(dense_to_code_kernel<true>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity);
+    hipLaunchKernelGGL(dense_to_code_kernel<true>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity, row_nnz);
   else
-    hipLaunchKernelGGL(dense_to_code_kernel<false>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity);
+    hipLaunchKernelGGL(dense_to_code_kernel<false>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dense, F, row_off, idx, val, capacity, row_nnz);
   return check_launch("dense_to_code");
 }
 

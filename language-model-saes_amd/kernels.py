@@ -40,16 +40,19 @@ def get_sparse_representation(x: torch.Tensor, pad_val: int = 0):
 
 
 class _SparseDecode(torch.autograd.Function):
-    """out = feature_acts @ W for a dense feature_acts whose rows are mostly zero: dense -> sparse code -> gather of the
-    active decoder rows (TritonDecoderAutogradTopK's role, kernels/kernels.py:542-566).  Backward: the gradient of the
-    activations at their non-zero positions (zero elsewhere, as the reference masks it), and the decoder gradient rows
-    from the feature index of the code."""
+    """out = feature_acts @ W for a dense feature_acts whose rows are mostly zero: the sparse code of the matrix ->
+    gather of the active decoder rows (TritonDecoderAutogradTopK's role, kernels/kernels.py:542-566).  Backward: the
+    gradient of the activations at their non-zero positions (zero elsewhere, as the reference masks it), and the decoder
+    gradient rows from the feature index of the code.
+
+    `code` addresses the rows of `w_op` (and of `weight`, the tensor the gradient goes to).  When the rows of
+    `feature_acts` are decoded by different blocks of `weight` (row r by block r % n_blocks: the heads of a crosscoder),
+    `code.idx` carries the block offset and `local_idx` the column inside feature_acts."""
 
     @staticmethod
-    def forward(ctx, feature_acts, weight, w_op, capacity):
-        fa = feature_acts if feature_acts.dtype in (torch.float32, torch.bfloat16) else feature_acts.float()
-        code = ops.dense_to_code(fa.contiguous(), capacity)
-        ctx.code, ctx.w_op = code, w_op
+    def forward(ctx, feature_acts, weight, w_op, code, local_idx=None):
+        ctx.code, ctx.w_op, ctx.local_idx = code, w_op, local_idx
+        ctx.n_cols = feature_acts.shape[-1]
         ctx.in_dtype, ctx.w_dtype = feature_acts.dtype, weight.dtype
         return ops.sparse_decode_fwd(code, w_op, None)
 
@@ -60,23 +63,58 @@ class _SparseDecode(torch.autograd.Function):
         d_acts = d_w = None
         if ctx.needs_input_grad[0]:
             dval = ops.sparse_decode_bwd_dval(code, g, w_op)
-            d_acts = ops.code_to_dense(dataclasses.replace(code, val=dval), code.d_sae)[0].to(ctx.in_dtype)
+            local = code if ctx.local_idx is None else dataclasses.replace(code, idx=ctx.local_idx, d_sae=ctx.n_cols)
+            d_acts = ops.code_to_dense(dataclasses.replace(local, val=dval), ctx.n_cols)[0].to(ctx.in_dtype)
         if ctx.needs_input_grad[1]:
             fi = ops.build_feature_index(code)
             d_w = ops.sparse_grad_rows(fi, code.val, g, code.d_sae)[0].to(ctx.w_dtype)
-        return d_acts, d_w, None, None
+        return d_acts, d_w, None, None, None
+
+
+def _as_code_source(feature_acts: torch.Tensor) -> torch.Tensor:
+    fa = feature_acts if feature_acts.dtype in (torch.float32, torch.bfloat16) else feature_acts.float()
+    return fa.contiguous()
+
+
+def sparse_decode_blocks(feature_acts: torch.Tensor, weight: torch.Tensor, w_operand: torch.Tensor, n_blocks: int = 1,
+                         max_density: Optional[float] = None) -> Optional[torch.Tensor]:
+    """feature_acts [rows, F] dense, weight / w_operand [n_blocks * F, d] (row r of feature_acts is decoded by block
+    r % n_blocks: with n_blocks = 1 a plain `feature_acts @ weight`) -> fp32 [rows, d] through the sparse decoder kernels,
+    differentiable in feature_acts and weight.  Returns None when more than `max_density` of the matrix is non-zero (the
+    count is read on the host, as the reference's own gate reads `max_l0`, models/sae.py:355-361)."""
+    fa = _as_code_source(feature_acts)
+    rows, F = fa.shape
+    limit = None if max_density is None else int(max_density * rows * F)
+    code = ops.dense_to_code(fa, max_entries=limit)
+    if code is None:
+        return None
+    local_idx = None
+    if n_blocks > 1:
+        slots = torch.arange(code.n_slots, device=fa.device)
+        row = (torch.searchsorted(code.row_off, slots, right=True) - 1).clamp_(min=0)
+        local_idx = code.idx
+        code = dataclasses.replace(code, idx=(code.idx + (row % n_blocks).to(torch.int32) * F), d_sae=n_blocks * F)
+    return _SparseDecode.apply(feature_acts, weight, w_operand, code, local_idx)
 
 
 def decode_with_hip_spmm_kernel(feature_acts: torch.Tensor, decoder_weight: torch.Tensor, *,
-                                w_operand: Optional[torch.Tensor] = None, capacity: Optional[int] = None) -> torch.Tensor:
+                                w_operand: Optional[torch.Tensor] = None, capacity: Optional[int] = None,
+                                transposed: Optional[bool] = None) -> torch.Tensor:
     """kernels/entrypoints.py:16-40.  feature_acts [.., d_sae] dense (or a torch sparse COO tensor), decoder_weight
     [d_sae, d_model]; the [d_model, d_sae] tensor the reference's own call site passes (`W_D.T.contiguous()`,
-    models/sae.py:363) is recognised by its shape and read as its transpose.  Returns feature_acts @ decoder_weight in
-    fp32.  `w_operand`: a prepared copy of the weight for the gather (e.g. the bf16 copy under autocast)."""
+    models/sae.py:363) is read as its transpose: `transposed=True` says so, `transposed=None` tells the two layouts apart
+    by shape and raises for a square weight, where the shape cannot tell.  Returns feature_acts @ decoder_weight in fp32.
+    `w_operand`: a prepared copy of the weight for the gather (e.g. the bf16 copy under autocast).  `capacity`: an upper
+    bound on the number of non-zeros (no read-back; entries past it are dropped)."""
     if feature_acts.is_sparse:
         feature_acts = feature_acts.to_dense()
     F = feature_acts.shape[-1]
-    if decoder_weight.shape[0] != F and decoder_weight.shape[-1] == F:
+    if transposed is None:
+        if decoder_weight.ndim == 2 and decoder_weight.shape[0] == decoder_weight.shape[1] == F and w_operand is None:
+            raise ValueError(f"decoder_weight is square ({F} x {F}): pass transposed=False for a [d_sae, d_model] weight or "
+                             "transposed=True for the [d_model, d_sae] form of the reference's call site")
+        transposed = decoder_weight.shape[0] != F and decoder_weight.shape[-1] == F
+    if transposed:
         decoder_weight = decoder_weight.t()
     if decoder_weight.shape[0] != F:
         raise ValueError(f"decoder_weight {tuple(decoder_weight.shape)} does not match d_sae = {F}")
@@ -86,7 +124,9 @@ def decode_with_hip_spmm_kernel(feature_acts: torch.Tensor, decoder_weight: torc
         if w_operand.dtype not in (torch.float32, torch.bfloat16):
             w_operand = w_operand.float()
     lead = feature_acts.shape[:-1]
-    out = _SparseDecode.apply(feature_acts.reshape(-1, F), decoder_weight, w_operand, capacity)
+    fa2 = feature_acts.reshape(-1, F)
+    code = ops.dense_to_code(_as_code_source(fa2), capacity)
+    out = _SparseDecode.apply(fa2, decoder_weight, w_operand, code, None)
     return out.view(*lead, out.shape[-1])
 
 

@@ -277,6 +277,9 @@ class LowRankSparseAttention(SparseDictionary):
         self.use_mix_kernels = True
         # False keeps W_O's gradient in factored form (feature index + gathered rows) whatever the shape
         self.dense_decoder_grad = True
+        # `decode` of dense activations takes the sparse decoder kernels when they are sparse enough; False keeps the
+        # reference's dense product whatever the input
+        self.sparse_api_decode = True
         self.register_buffer("mask", torch.tril(torch.ones((cfg.n_ctx, cfg.n_ctx), device=cfg.device).bool()))
         self.register_buffer("IGNORE", torch.tensor(-torch.inf, device=cfg.device))
         if cfg.use_post_qk_ln:
@@ -597,7 +600,21 @@ class LowRankSparseAttention(SparseDictionary):
             out = ops.sparse_decode_fwd(feature_acts, self._w_dec_operand(amp),
                                         self.b_D.detach() if self.cfg.use_decoder_bias else None)
             return self.hook_reconstructed(out)
-        out = torch.einsum("bps,sd->bpd", feature_acts, self.W_O)
+        out = None
+        F, d = self.cfg.d_sae, self.cfg.d_model
+        if (self._sparse_decode_allowed(feature_acts) and feature_acts.shape[-1] == F and d % 8 == 0
+                and self.W_O.dtype in (torch.float32, torch.bfloat16)):
+            # lorsa.py:765-782 for activations that are sparse enough (at most 1 - cfg.sparsity_threshold_for_triton_spmm_kernel
+            # of the entries non-zero, counted on the device and read once): the sparse decoder kernels, forward and backward
+            from .kernels import sparse_decode_blocks
+
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            out = sparse_decode_blocks(feature_acts.reshape(-1, F), self.W_O, self._w_dec_operand(amp),
+                                       max_density=1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel)
+            if out is not None:
+                out = out.view(*feature_acts.shape[:-1], d)
+        if out is None:
+            out = torch.einsum("bps,sd->bpd", feature_acts, self.W_O)
         if self.cfg.use_decoder_bias:
             out = out + self.b_D
         return self.hook_reconstructed(out)

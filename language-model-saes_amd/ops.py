@@ -228,11 +228,13 @@ def dense_row_nnz(dense: torch.Tensor) -> torch.Tensor:
     return row_nnz
 
 
-def dense_to_code(dense: torch.Tensor, capacity: Optional[int] = None) -> "SparseCode":
+def dense_to_code(dense: torch.Tensor, capacity: Optional[int] = None, max_entries: Optional[int] = None) -> Optional["SparseCode"]:
     """Sparse code of a dense [B, F] activation matrix (fp32 or bf16): every token's non-zero entries in ascending
     feature order, rows packed one after the other.  Without `capacity` the number of non-zeros is read back from the
-    device to size the code (one synchronisation, as the reference's `nnz_max.item()`); with it (an upper bound the
-    caller knows, e.g. k * B after a TopK activation) nothing is read back and entries past it would be dropped."""
+    device to size the code (one synchronisation, as the reference's `nnz_max.item()`); `max_entries` then makes the
+    call return None, before anything is written, when the matrix holds more non-zeros than that (the caller's sparsity
+    gate).  With `capacity` (an upper bound the caller knows, e.g. k * B after a TopK activation) nothing is read back;
+    entries past it are dropped and `row_nnz` is cut to what was written, so the code is truncated, never out of bounds."""
     _req(dense, "dense", ndim=2)
     B, F = dense.shape
     lib = _lib.load()
@@ -241,11 +243,16 @@ def dense_to_code(dense: torch.Tensor, capacity: Optional[int] = None) -> "Spars
         check(lib.sae_dense_row_nnz(dense.data_ptr(), _dt(dense), B, F, row_nnz.data_ptr(), _stream(dense)), "dense_row_nnz")
         incl = torch.cumsum(row_nnz, 0, dtype=torch.int64)
         row_off = incl - row_nnz
-        cap = int(incl[-1].item()) if capacity is None else int(capacity)
+        if capacity is None:
+            cap = int(incl[-1].item())
+            if max_entries is not None and cap > max_entries:
+                return None
+        else:
+            cap = int(capacity)
         idx = torch.zeros(max(cap, 1), dtype=torch.int32, device=dense.device)
         val = torch.zeros(max(cap, 1), dtype=torch.float32, device=dense.device)
         check(lib.sae_dense_to_code(dense.data_ptr(), _dt(dense), B, F, row_off.data_ptr(), idx.data_ptr(), val.data_ptr(), cap,
-                                    _stream(dense)), "dense_to_code")
+                                    row_nnz.data_ptr() if capacity is not None else None, _stream(dense)), "dense_to_code")
     return SparseCode(idx, val, row_off, row_nnz, B, F)
 
 
@@ -280,8 +287,8 @@ def mse_auxk_fused(recon: torch.Tensor, label: torch.Tensor, aux_recon: Optional
 
 # ---- encoder --------------------------------------------------------------------------------
 
-def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """pre[B, F] = x[B, d] @ w_enc_t[F, d]^T."""
+def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """pre[B, F] = x[B, d] @ w_enc_t[F, d]^T (`out`: a contiguous [B, F] tensor of `out_dtype` to write into)."""
     _req(x, "x", ndim=2)
     _req(w_enc_t, "w_enc_t", ndim=2)
     if x.dtype != w_enc_t.dtype:
@@ -290,14 +297,18 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype)
     F, d2 = w_enc_t.shape
     if d != d2:
         raise ValueError(f"shape mismatch: x {tuple(x.shape)} vs w_enc_t {tuple(w_enc_t.shape)}")
+    if out is not None:
+        _req(out, "out", out_dtype, 2)
+        if tuple(out.shape) != (B, F):
+            raise ValueError(f"out must be {(B, F)}, got {tuple(out.shape)}")
     splits = gemm_split_k(B, d, F) if (x.dtype == torch.bfloat16 and out_dtype == torch.float32) else 1
     if splits > 1:
         partials = torch.empty(splits, B, F, dtype=torch.float32, device=x.device)
         with _timed("encoder_gemm"):
             check(_lib.load().sae_encoder_gemm_split_k(x.data_ptr(), w_enc_t.data_ptr(), partials.data_ptr(), splits, B, d, F,
                                                        _stream(x)), "encoder_gemm_split_k")
-        return partials.sum(0)
-    pre = torch.empty(B, F, dtype=out_dtype, device=x.device)
+        return partials.sum(0) if out is None else torch.sum(partials, 0, out=out)
+    pre = out if out is not None else torch.empty(B, F, dtype=out_dtype, device=x.device)
     with _timed("encoder_gemm"):
         check(
             _lib.load().sae_encoder_gemm(x.data_ptr(), w_enc_t.data_ptr(), pre.data_ptr(), B, d, F, _dt(x), _dt(pre), _stream(x)),

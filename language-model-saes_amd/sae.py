@@ -457,7 +457,9 @@ class _EncoderGemm(torch.autograd.Function):
     kernel."""
 
     @staticmethod
-    def forward(ctx, x, W_E, w_op, amp, defer=False, given=None):
+    def forward(ctx, x, W_E, w_op, amp, defer=False, given=None, grad_view=None):
+        # grad_view: maps the gradient rows [F, K] (K = x's width) to the parameter's shape, for encoder weights that
+        # are not a [d, F] view of a [F, d] buffer (a crosscoder's [H, d, F] over [F, H, d])
         if given is not None:             # (x operand, product) computed by the caller already
             x_op, pre = given
         elif amp:
@@ -470,6 +472,7 @@ class _EncoderGemm(torch.autograd.Function):
         ctx.x_dtype, ctx.w_dtype = x.dtype, W_E.dtype
         # a bf16 weight gradient can stay bf16 until the optimiser reads it, when the parameter is stored feature-major
         ctx.param = W_E if (defer and amp and W_E.ndim == 2 and W_E.stride() == (1, W_E.shape[0])) else None
+        ctx.grad_view = grad_view
         return pre
 
     @staticmethod
@@ -483,9 +486,11 @@ class _EncoderGemm(torch.autograd.Function):
             rows = _rows_over_tokens(gg, x_op, w_op.dtype)                         # [F, d]
             if ctx.param is not None:
                 _leave_lowp_grad(ctx.param, rows)
+            elif ctx.grad_view is not None:
+                dW = ctx.grad_view(rows).to(ctx.w_dtype)
             else:
                 dW = rows.t().to(ctx.w_dtype)                                      # [d, F] with feature-major strides
-        return dx, dW, None, None, None, None
+        return dx, dW, None, None, None, None, None
 
 
 def _leave_lowp_grad(param, rows: torch.Tensor) -> None:
@@ -843,7 +848,7 @@ class SparseAutoEncoder(SparseDictionary):
             max_l0 = int(nnz.max().item())
             if 0 < max_l0 < self.cfg.d_sae * (1 - self.cfg.sparsity_threshold_for_triton_spmm_kernel):
                 amp = _autocast_dtype("cuda") == torch.bfloat16
-                reconstructed = decode_with_hip_spmm_kernel(feature_acts, self.W_D, w_operand=self._w_dec_operand(amp))
+                reconstructed = decode_with_hip_spmm_kernel(feature_acts, self.W_D, w_operand=self._w_dec_operand(amp), transposed=False)
         if reconstructed is None:
             reconstructed = feature_acts @ self.W_D
         if self.cfg.use_decoder_bias:

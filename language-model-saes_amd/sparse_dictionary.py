@@ -308,6 +308,17 @@ class SparseDictionary(nn.Module):
         return cls.from_local(str(pretrained_name_or_path), device_mesh=device_mesh, strict_loading=strict_loading,
                               fold_activation_scale=fold_activation_scale, **kwargs)
 
+    def _sparse_decode_allowed(self, feature_acts: torch.Tensor) -> bool:
+        """Whether `decode` may send dense activations through the sparse decoder kernels (models that set
+        `sparse_api_decode`).  Their backward returns the activation gradient at the non-zero entries only, as the
+        reference's sparse operator does (kernels/kernels.py:563): exact for TopK-family and ReLU activations, whose own
+        backward passes nothing else on, but a JumpReLU's threshold gradient also reads entries just below the
+        threshold, so a JumpReLU dictionary takes the route only where no gradient is asked of the activations."""
+        if not (getattr(self, "sparse_api_decode", False) and feature_acts.is_cuda):
+            return False
+        needs_grad = torch.is_grad_enabled() and feature_acts.requires_grad
+        return not (needs_grad and isinstance(self.activation_function, JumpReLU))
+
     # ---- to be provided by subclasses ----
     def encode(self, x, return_hidden_pre: bool = False, **kwargs):
         raise NotImplementedError

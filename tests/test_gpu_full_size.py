@@ -306,14 +306,9 @@ def test_clt_shape_fused_step_against_dense_path(pkg, dev, amp):
     feature_acts = out["feature_acts"].clone().requires_grad_()
     kept = feature_acts.detach() != 0
     assert int(kept.sum().item()) == B * L * k
+    clt.sparse_api_decode = False      # the module's dense products: one 2-D library product per output layer
     with _amp(amp):
-        if amp:
-            # block by block with 2-D products (the batched bf16 product over a permuted view, which `decode` uses,
-            # is not what this test wants to depend on)
-            recon = torch.stack([sum(feature_acts[:, lf, :] @ clt.W_D[lt][lf] for lf in range(lt + 1)) + clt.b_D[lt]
-                                 for lt in range(L)], dim=0)
-        else:
-            recon = clt.decode(feature_acts)
+        recon = clt.decode(feature_acts)
         loss = (recon.float() - label).pow(2).sum(-1).mean()
     assert rel_err(out["reconstructed"], recon) < tol_out
     assert abs(out["loss"].item() - loss.item()) < tol_loss * loss.item()
