@@ -15,7 +15,10 @@ own workload name.
 Prints ONE JSON line.  `roofline` describes the kernel of this library with the largest share of
 the step, timed with HIP events inside the timed region; `cpu_baseline` (default workload only) is
 the oracle (a CPU restatement of the reference's eager path) timed on this host on a reduced batch
-of the same shape.
+of the same shape.  After the headline's timed region a default run also times the other benchmark
+configurations for a few steps each (the reference's CPU configuration in fp32, BatchTopK with aux-k,
+JumpReLU dense and sparse, the cross-layer transcoder, Lorsa, a crosscoder) and reports them under
+`configs`; they never enter `value`.
 """
 
 from __future__ import annotations
@@ -316,7 +319,7 @@ def build_jumprelu(pkg, dev, args):
     sae = pkg.SparseAutoEncoder(cfg)
     g = torch.Generator(device=dev).manual_seed(4)
     x = torch.randn(B, d, device=dev, generator=g)
-    x[:, [7, 511, 1024, 3000]] *= 50.0
+    x[:, [7, 1029, 2050, 3071]] *= 50.0
     _init_sae_on_device(sae, x, d)
     with torch.no_grad():
         sae.activation_function.log_jumprelu_threshold.fill_(math.log(0.001))
@@ -340,7 +343,7 @@ def build_jumprelu_sparse(pkg, dev, args):
     sae = pkg.SparseAutoEncoder(cfg)
     g = torch.Generator(device=dev).manual_seed(4)
     x = torch.randn(B, d, device=dev, generator=g)
-    x[:, [7, 511, 1024, 3000]] *= 50.0
+    x[:, [7, 1029, 2050, 3071]] *= 50.0
     _init_sae_on_device(sae, x, d)
     with torch.no_grad():
         sae.activation_function.log_jumprelu_threshold.fill_(math.log(3.5))
@@ -411,17 +414,78 @@ def build_lorsa_rotary(pkg, dev, args):
     return build_lorsa(pkg, dev, args, positional="rotary")
 
 
+def build_crosscoder(pkg, dev, args):
+    """Crosscoder: 4 heads (hook points) of d=768, 24576 shared features, k=64 per head, 4096 tokens; head h reads
+    activations G(768, r=16, seed 20 + h); decoders start as unit-norm rows, encoders as their transposes."""
+    import torch
+    from lm_saes_amd import synthetic
+
+    B, H, d, F, k = args.batch or 4096, 4, 768, 24576, 64
+    hooks = [f"h{i}" for i in range(H)]
+    cfg = pkg.CrosscoderConfig(hook_points=hooks, d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                               norm_activation="inference", device="cuda", dtype=torch.float32)
+    m = pkg.Crosscoder(cfg)
+    batch = {"tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    for i, hp in enumerate(hooks):
+        batch[hp] = synthetic.activations(B, d, 16, seed=20 + i).to(dev)
+    with torch.no_grad():
+        g = torch.Generator(device=dev).manual_seed(4)
+        m.W_D.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
+        m.W_D.div_(m.W_D.norm(dim=-1, keepdim=True))
+        m.W_D.mul_(0.5 + torch.rand(H, F, 1, device=dev, generator=g))     # the heads' norms differ, so do their selections
+        m.init_encoder_with_decoder_transpose()
+        m.b_E.zero_()
+        m.b_D.copy_(torch.stack([batch[hp].mean(0) for hp in hooks]))
+    opt = pkg.HipAdam(m.get_parameters()[0]["params"], lr=4e-4, model=m)
+    name = f"crosscoder_train_step heads={H} d_model={d} d_sae={F} k={k} batch={B} bf16 adam"
+    return _autocast_step(m, batch, opt, {}), B, name, (B, d, F, k)
+
+
 WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "batchtopk_bf16_params": build_batchtopk_bf16_params, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
-             "lorsa": build_lorsa, "lorsa_rotary": build_lorsa_rotary}
+             "lorsa": build_lorsa, "lorsa_rotary": build_lorsa_rotary, "crosscoder": build_crosscoder}
+
+# the other benchmark configurations a default run times after the headline (a few steps each): BASELINE's five
+# configurations, the JumpReLU one in both of its forms, and a crosscoder
+CONFIG_RUNS = [("c1_topk_fp32", "c1_fp32", 10), ("c2_batchtopk_auxk", "batchtopk", 8), ("c3_jumprelu_dense", "jumprelu", 4),
+               ("c3_jumprelu_sparse", "jumprelu_sparse", 6), ("c4_clt", "clt", 6), ("c5_lorsa", "lorsa", 8),
+               ("crosscoder", "crosscoder", 8)]
 
 
-def gpu_step_bench(args):
+def step_work(workload: str, shape) -> dict:
+    """Algorithmic work PER STEP of kernels whose launches differ in shape inside one step of `workload` (label ->
+    (bound, flop or bytes)); a kernel's fraction of its roofline is then that work over its time per step."""
+    B, d, F, k = shape
+    if workload == "clt":
+        L = 12
+        blocks = L * (L + 1) // 2
+        return {"adam_step_sparse_rows[bf16 dense]": ("hbm", 26.0 * (L + blocks) * F * d),
+                "sparse_decode_mse_fused": ("hbm", sum(2.0 * B * (j + 1) * k * d * 2 + 3 * B * d * 4 for j in range(L))),
+                "encoder_gemm": ("mfma", 2.0 * B * d * F * L)}
+    if workload == "crosscoder":
+        H = 4
+        return {"adam_step_sparse_rows[bf16 dense]": ("hbm", 26.0 * 2 * H * F * d),
+                "sparse_decode_mse_fused": ("hbm", H * (2.0 * B * k * d * 2 + 3 * B * d * 4)),
+                "encoder_gemm": ("mfma", 2.0 * B * (H * d) * F)}
+    if workload in ("batchtopk", "jumprelu_sparse"):
+        return {"adam_step_sparse_rows[bf16 dense]": ("hbm", 26.0 * 2 * F * d)}
+    if workload in ("lorsa", "lorsa_rotary"):
+        nb, s, h, dq, dv = 16, 1024, 64, 64, 128
+        pairs = nb * h * s * (s + 1) // 2
+        return {"attention_fwd": ("mfma", 2.0 * pairs * (dq + dv)), "attention_bwd": ("mfma", 2.0 * pairs * (3 * dq + 2 * dv))}
+    return {}
+
+
+
+def gpu_step_bench(args, workload=None, steps=None, warmup=None):
     import torch
     from __graft_entry__ import load_package
 
     pkg = load_package()
     dev = torch.device("cuda:0")
-    step, tokens, name, shape = WORKLOADS[args.workload](pkg, dev, args)
+    workload = workload or args.workload
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
+    step, tokens, name, shape = WORKLOADS[workload](pkg, dev, args)
 
     if args.calibrate_copy:
         # a plain device copy of known size (1 GiB read + 1 GiB written), for scaling rocprofv3's
@@ -432,20 +496,56 @@ def gpu_step_bench(args):
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     timer = pkg.ops.KernelTimer()
     pkg.ops.set_kernel_timer(timer)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         loss = step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     pkg.ops.set_kernel_timer(None)
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = (t1 - t0) * 1e3 / steps
     return ms_per_step, timer.summary(), float(loss.item()), tokens, name, shape
+
+
+def config_run(args, key: str, workload: str, steps: int) -> dict:
+    """One of the other benchmark configurations, timed for a few steps in this process: its step time, throughput and
+    the library kernel with the largest share of the step (with its fraction of the roofline that bounds it where every
+    launch of it does known work)."""
+    import gc
+
+    import torch
+
+    batch, d_sae = args.batch, args.d_sae
+    args.batch, args.d_sae = 0, 0
+    try:
+        ms, kernels, loss, tokens, name, shape = gpu_step_bench(args, workload, steps, 2)
+    finally:
+        args.batch, args.d_sae = batch, d_sae
+    gc.collect()
+    torch.cuda.empty_cache()
+    dominant = max(kernels, key=lambda n: kernels[n]["total_ms"])
+    per_step = step_work(workload, shape)
+    uniform = workload in ("c1_fp32", "jumprelu")
+    bound = frac = None
+    if dominant in LATENCY_BOUND:
+        bound = "latency"
+    elif dominant in per_step:
+        bound, w = per_step[dominant]
+        rate = w / (kernels[dominant]["total_ms"] / steps)
+        frac = rate / 1e9 / PEAK_BF16_TFLOPS if bound == "mfma" else rate / 1e6 / PEAK_HBM_GBS
+    elif uniform and dominant in algorithmic_work(*shape):
+        bound, w = algorithmic_work(*shape)[dominant]
+        rate = w / kernels[dominant]["avg_ms"]
+        frac = rate / 1e9 / (157.3 if workload == "c1_fp32" else PEAK_BF16_TFLOPS) if bound == "mfma" else rate / 1e6 / PEAK_HBM_GBS
+    return {"workload": name, "steps": steps, "ms_per_step": round(ms, 4), "tokens_per_s": round(tokens / (ms / 1e3), 1),
+            "dominant_kernel": dominant, "dominant_ms_per_step": round(kernels[dominant]["total_ms"] / steps, 4),
+            "bound": bound, "frac": None if frac is None else round(frac, 4),
+            "kernel_ms_per_step": round(sum(v["total_ms"] for v in kernels.values()) / steps, 4), "final_loss": loss}
 
 
 def mfma_probe() -> dict:
@@ -553,6 +653,8 @@ def main():
     ap.add_argument("--cpu-sample-features", type=int, default=D_SAE,
                     help="dictionary size of the CPU baseline (default: the full 131072 features)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="headline run only: skip the short runs of the other benchmark configurations")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run three 1 GiB device copies (counter calibration)")
     ap.add_argument("--gemm-operand-probe", action="store_true",
                     help="instead of a train step: the headline encoder product with random, zero and constant operands "
@@ -633,6 +735,15 @@ def main():
         "kernel_ms_per_step": round(sum(v["ms_per_step"] for v in per_kernel.values()), 4),
         "final_loss": loss,
     }
+    if headline and not args.no_configs:
+        # the other configurations, a few steps each: not part of `value`, measured after its timed region
+        import gc
+
+        import torch
+
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["configs"] = {key: config_run(args, key, workload, steps) for key, workload, steps in CONFIG_RUNS}
     if headline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, args.cpu_sample_features)
         out["cpu_baseline_c1"] = cpu_baseline_c1()   # the configuration the reference's CPU path runs at full shape

@@ -155,7 +155,7 @@ class _FixedDead:
         return self.is_dead
 
 
-def test_batchtopk_auxk_shape_step_properties(pkg, dev):
+def test_batchtopk_auxk_shape_step_properties(pkg, oracle, dev):
     """BatchTopK SAE d=2048, F=32768, 8192 tokens, global top 64 x 8192, aux-k over the top 512 dead features."""
     d, F, k, B, k_aux, alpha = 2048, 32768, 64, 8192, 512, 1 / 32
     sae, batch = build_sae(pkg, dev, d, F, k, B, r=32, act_fn="batchtopk")
@@ -172,6 +172,12 @@ def test_batchtopk_auxk_shape_step_properties(pkg, dev):
     kept = dense_mask(code)
     assert int(kept.sum().item()) == k * B
     check_threshold_selection(hp * n, kept, per_row=False)
+    # the oracle's own BatchTopK (models/sparse_dictionary.py:761-794 restated: relu mask, then the k B largest over both
+    # axes by a stable sort on the CPU) on the kernel's scores: the same set of 524 288 positions, bit for bit
+    score_cpu = (hp * n).cpu()
+    want_kept = oracle.topk(score_cpu * score_cpu.gt(0).to(score_cpu.dtype), k=k * B, dim=(-2, -1), abs=True) != 0
+    assert torch.equal(want_kept, kept.cpu())
+    del score_cpu, want_kept
     # rows ascend in index
     val = torch.zeros(B, F, device=dev).masked_scatter_(kept, code.val[: k * B])
     assert rel_err(val[kept], hp[kept]) < 1e-6
@@ -443,7 +449,7 @@ def test_jumprelu_shape_fused_step_against_dense_path(pkg, dev, amp):
     sae = pkg.SparseAutoEncoder(cfg)
     g = torch.Generator(device=dev).manual_seed(4)
     x = torch.randn(B, d, device=dev, generator=g)
-    x[:, [7, 511, 1024, 3000]] *= 50.0
+    x[:, [7, 1029, 2050, 3071]] *= 50.0
     with torch.no_grad():
         wt = sae.W_E.t()
         wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)

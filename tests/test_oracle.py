@@ -345,6 +345,43 @@ def test_auxk_vs_numpy_and_special_cases(oracle):
     assert ctx2["l_aux"].item() == 0.0 and ctx2["loss"].item() == ctx2["l_rec"].item()
 
 
+def test_auxk_with_decoder_norm_scale_vs_numpy(oracle):
+    """The aux-k branch with `sparsity_include_decoder_norm=True` (models/sparse_dictionary.py:958-972): the dead features'
+    keys are hidden_pre * n (n = decoder row norms, spread here so that the ranking by h n differs from the ranking by h),
+    the kept values are divided by n again, so the aux reconstruction is built from hidden_pre itself.  Scalar loops."""
+    F, d, B, k = 12, 4, 9, 2
+    m = _dense_model(oracle, "topk", F=F, d=d, sparsity_include_decoder_norm=True)
+    with torch.no_grad():
+        m.W_D.mul_(torch.linspace(0.2, 3.0, F, dtype=torch.float64)[:, None])
+    m.current_k = k
+    x = torch.randn(B, d, dtype=torch.float64)
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B)}
+    stats = oracle.DeadStatistics(F, dead_threshold=B)
+    ctx = m.compute_loss(batch, auxk_coefficient=0.5, k_aux=3, update_dead_statistics=stats.update)
+    f = ctx["feature_acts"].detach().numpy()
+    fired = f.sum(0) > 0
+    hp = ctx["hidden_pre"].detach().numpy()
+    W_D = m.W_D.detach().numpy()
+    n = np.sqrt((W_D ** 2).sum(1))
+    e = (x - ctx["reconstructed"]).detach().numpy()
+    kk = min(3, int((~fired).sum()))
+    tot, by_h_differs = 0.0, False
+    for b in range(B):
+        key = np.where(~fired, hp[b] * n, 0.0)
+        order = sorted(range(F), key=lambda j: (-max(key[j], 0.0), j))[:kk]
+        plain = sorted(range(F), key=lambda j: (-max(np.where(~fired, hp[b], 0.0)[j], 0.0), j))[:kk]
+        by_h_differs |= set(j for j in order if key[j] > 0) != set(j for j in plain if hp[b][j] > 0 and not fired[j])
+        acts = np.zeros(F)
+        for j in order:
+            if key[j] > 0:
+                acts[j] = key[j] / n[j]
+        tot += ((e[b] - acts @ W_D) ** 2).sum()
+    want = 0.5 * tot / B
+    assert kk > 0 and by_h_differs          # the norm scale changes which dead features are picked
+    assert abs(ctx["l_aux"].item() - want) < 1e-10 * max(1.0, want)
+    assert abs(ctx["loss"].item() - ctx["l_rec"].item() - want) < 1e-10 * max(1.0, want)
+
+
 def test_dead_statistics_accumulate(oracle):
     st = oracle.DeadStatistics(3, dead_threshold=5)
     a = torch.tensor([[1.0, 0.0, 0.0], [0.0, 0.0, 0.0]])
