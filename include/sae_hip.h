@@ -100,6 +100,20 @@ int sae_encoder_gemm(const void *x, const void *w_enc_t, void *pre, int64_t B, i
 int sae_encoder_gemm_split_k(const void *x_bf16, const void *w_t_bf16, float *partials, int64_t n_splits, int64_t B, int64_t d,
                              int64_t F, void *stream);
 
+/* The same bf16 product for operands in either layout: out[m, n] = sum_k A[m, k] B[n, k], fp32 accumulation, out [M, N]
+ * written as out_dtype.  a_k_major / b_k_major = 0: the operand is stored [rows, K] (a row's K values side by side, as
+ * sae_encoder_gemm takes both); 1: it is stored [K, rows] (K-major: the rows' values side by side), read as it lies, with
+ * no transposed copy: its matrix-core fragments are read across the K-rows of the LDS tile.  That is the layout the products
+ * over the token axis find their operands in, and the dense decode its weight:
+ *   dW_E^T = d(pre)^T x and dW_D = acts^T d(recon)   (autograd of `x @ self.W_E` / `feature_acts @ self.W_D`,
+ *            models/sae.py:324, 367): A = d(pre) or acts [tokens, F], B = x or d(recon) [tokens, d], both K-major;
+ *   feature_acts @ W_D   (models/sae.py:367):          A = feature_acts [tokens, F], B = W_D [F, d] K-major.
+ * n_splits > 1 cuts the contraction into that many slices, run as one launch; out is then fp32 [n_splits, M, N] partial
+ * results, to be summed by the caller in slice order.  K % (64 n_splits) == 0; a K-major operand needs its row count
+ * (M or N) to be a multiple of 8; pointers 16-byte aligned. */
+int sae_gemm_bf16(const void *a, int a_k_major, const void *b, int b_k_major, void *out, int out_dtype, int64_t M, int64_t N,
+                  int64_t K, int64_t n_splits, void *stream);
+
 /* ---- activation select ------------------------------------------------------------ */
 
 /* Per-token TopK with fused bias and decoder-norm scale.

@@ -60,6 +60,7 @@ SIGNATURES = {
     "sae_code_to_dense": (_I, [_P, _P, _P, _P, _L, _L, _P, _P, _P]),
     "sae_code_to_dense_t": (_I, [_P, _P, _P, _P, _L, _L, _P, _P]),
     "sae_encoder_gemm_split_k": (_I, [_P, _P, _P, _L, _L, _L, _L, _P]),
+    "sae_gemm_bf16": (_I, [_P, _I, _P, _I, _P, _I, _L, _L, _L, _L, _P]),
     "sae_mse_auxk_fused": (_I, [_P, _P, _P, _P, _F, _L, _L, _P, _P, _P, _P, _P, _P]),
     "sae_code_stats": (_I, [_P, _P, _P, _P, _P, _L, _L, _P, _P, _P, _P]),
     "sae_recon_stats": (_I, [_P, _P, _P, _P, _L, _L, _P, _P, _P, _P]),

@@ -29,7 +29,7 @@ from torch import nn
 from . import ops
 from .activation_functions import JumpReLU, _topk_mask_lowest_index, batch_topk_dense, topk_dense
 from .config import CLTConfig, register_sae_model
-from .sae import SparseRowGrad, SparseRowGradPieces, _autocast_dtype, _gemm_k_ok, _rows_over_tokens
+from .sae import SparseRowGrad, SparseRowGradPieces, _autocast_dtype, _gemm_k_ok, _rows_over_tokens, dense_decode
 from .sparse_dictionary import LazyDict, SparseDictionary
 
 _TOPK_FAMILY = ("topk", "layertopk", "batchtopk", "batchlayertopk")
@@ -513,7 +513,18 @@ class CrossLayerTranscoder(SparseDictionary):
                 out = _PrefixDecode.apply(acts2, code, prefix_t, (L, F, d), self._w_dec_operands(amp), *self.W_D)
                 out = out + torch.stack(list(self.b_D)).unsqueeze(1)
         if out is None:
-            out = torch.stack([acts2[:, : (j + 1) * F] @ self.W_D[j].view((j + 1) * F, d) + self.b_D[j] for j in range(L)])
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            w_ops = self._w_dec_operands(amp) if feature_acts.is_cuda else None
+            outs = []
+            for j in range(L):
+                part = None
+                if w_ops is not None:   # the GEMM kernel on the layers' prefix (bf16 operands read W_D[j] as it lies)
+                    part = dense_decode(self, acts2[:, : (j + 1) * F], self.W_D[j].view((j + 1) * F, d),
+                                        w_ops[j].view((j + 1) * F, d), f"W_D.{j}.t.f32")
+                if part is None:
+                    part = acts2[:, : (j + 1) * F] @ self.W_D[j].view((j + 1) * F, d)
+                outs.append(part + self.b_D[j])
+            out = torch.stack(outs)
         out = out.view(L, *lead, d)
         return out.movedim(0, -2) if batch_first else out
 

@@ -258,6 +258,16 @@ class Crosscoder(SparseDictionary):
                                        n_blocks=H, max_density=1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel)
             if out is not None:
                 return out.view(*lead, H, d) + self.b_D
+        if feature_acts.is_cuda and tuple(feature_acts.shape[-2:]) == (H, F):
+            # denser activations: one product of the GEMM kernel per head (bf16 operands read W_D[h] as it lies)
+            from .sae import dense_decode
+
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            w_op = self._w_dec_operand(amp)
+            fa = feature_acts.reshape(-1, H, F)
+            outs = [dense_decode(self, fa[:, h], self.W_D[h], w_op[h], f"W_D.{h}.t.f32") for h in range(H)]
+            if all(o is not None for o in outs):
+                return torch.stack(outs, dim=1).view(*feature_acts.shape[:-2], H, d) + self.b_D
         return torch.einsum("...hf,hfd->...hd", feature_acts, self.W_D) + self.b_D
 
     def prepare_input(self, batch: dict[str, torch.Tensor], **kwargs) -> tuple[torch.Tensor, dict[str, Any], dict[str, Any]]:

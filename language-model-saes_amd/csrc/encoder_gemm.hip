@@ -299,20 +299,33 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_f32_kernel(
 // EPI_GMAX_LOWP: EPI_GMAX with the keys in the bf16 arithmetic of a dictionary held in bf16 (the sum with the bias and the
 // product with the scale each rounded to bf16: what sae_select_topk_row_lowp / sae_select_topk_batch_lowp form).
 constexpr int EPI_NONE = 0, EPI_GMAX = 1, EPI_BIAS = 2, EPI_MARGIN = 3, EPI_GMAX_LOWP = 4;
-template <bool BF16_OUT, int EPI>
+
+// Operand layouts.  The default is K-contiguous: row r of the operand (a token of x, a feature of w) holds its K values
+// side by side.  XT / WT say that the operand is stored the other way round, [K, rows] with the rows side by side (what a
+// product over the token axis finds: dW = d(pre)^T x reads d(pre) [tokens, features] and x [tokens, d_model] as they
+// are; acts @ W_D reads W_D [features, d_model] as it is).  A slab of such an operand is 64 K-rows of 256 values
+// (512 bytes each): the same 32 KiB slot, filled by the same 1 KiB LDS-direct loads (two K-rows per load), and its
+// matrix-core fragments (8 consecutive K values of one row) are read ACROSS the K-rows with ds_read_b64_tr_b16, two per
+// fragment: lane i of a group of 16 points at K-row 4 hh + i / 4, values 4 (i % 4) .. + 3 and receives the four K values
+// of value i.  Chunk c (16 bytes) of K-row r sits at chunk c ^ tkey(r), tkey(r) = 2 ((r & 3) | ((r >> 3) & 1) << 2): the
+// eight K-rows x 32 bytes that half a wave reads at once then fall on 256 distinct bytes.
+__device__ __forceinline__ int gemm_tkey(int krow) { return ((krow & 3) | (((krow >> 3) & 1) << 2)) << 1; }
+
+template <bool BF16_OUT, int EPI, bool XT = false, bool WT = false>
 __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
     const char *__restrict__ x, const char *__restrict__ w, void *__restrict__ out, int M, int N,
-    int row_bytes /* contraction length * 2 */, int pitch_bytes /* bytes between operand rows */, int tiles_m, int tiles_n,
-    int rm_log2, const float *__restrict__ b_enc,
+    int row_bytes /* contraction length * 2 */, int pitch_x, int pitch_w /* bytes between stored rows of x / w */,
+    int tiles_m, int tiles_n, int rm_log2, const float *__restrict__ b_enc,
     const float *__restrict__ scale, uint32_t *__restrict__ gmax, const float *__restrict__ theta) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // the ring of GEMM_SLOTS operand slabs
   if (blockIdx.y) {
     // group g of a batch of independent products of one shape, each operand stacked group after group; or, when the rows
-    // are longer than the contraction, slice g of the contraction axis (split-K: the caller sums the groups' outputs)
+    // are longer than the contraction (or an operand is stored [K, rows]), slice g of the contraction axis (split-K: the
+    // caller sums the groups' outputs)
     const size_t g = blockIdx.y;
-    if (pitch_bytes != row_bytes) {
-      x += g * (size_t)row_bytes;
-      w += g * (size_t)row_bytes;
+    if (XT || WT || pitch_x != row_bytes) {
+      x += XT ? g * (size_t)(row_bytes >> 1) * pitch_x : g * (size_t)row_bytes;
+      w += WT ? g * (size_t)(row_bytes >> 1) * pitch_w : g * (size_t)row_bytes;
     } else {
       x += g * (size_t)M * row_bytes;
       w += g * (size_t)N * row_bytes;
@@ -356,9 +369,23 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
   for (int i = 0; i < 4; ++i) {
     const int r = wave * 32 + i * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-    xg[i] = x + (size_t)(m0 + r < M ? m0 + r : M - 1) * pitch_bytes + chunk * 16;
-    wg[i] = w + (size_t)(n0 + r < N ? n0 + r : N - 1) * pitch_bytes + chunk * 16;
+    // stored [K, rows]: this load fills K-rows 8 wave + 2 i and + 1 of the slab, 32 chunks of 8 values each; values past
+    // the operand's last row repeat its last 8 (their products land in accumulators that are never stored)
+    const int kr = wave * 8 + i * 2 + (lane >> 5), tc = (lane & 31) ^ gemm_tkey(kr);
+    if constexpr (XT) {
+      const int m = m0 + tc * 8;
+      xg[i] = x + (size_t)kr * pitch_x + (size_t)(m + 8 <= M ? m : M - 8) * 2;
+    } else {
+      xg[i] = x + (size_t)(m0 + r < M ? m0 + r : M - 1) * pitch_x + chunk * 16;
+    }
+    if constexpr (WT) {
+      const int n = n0 + tc * 8;
+      wg[i] = w + (size_t)kr * pitch_w + (size_t)(n + 8 <= N ? n : N - 8) * 2;
+    } else {
+      wg[i] = w + (size_t)(n0 + r < N ? n0 + r : N - 1) * pitch_w + chunk * 16;
+    }
   }
+  const size_t x_adv = XT ? (size_t)64 * pitch_x : (size_t)GEMM_SLAB, w_adv = WT ? (size_t)64 * pitch_w : (size_t)GEMM_SLAB;
   const uint32_t ld_base = (uint32_t)(wave * 32) * GEMM_SLAB;
 
   f32x4_t acc[4][8];   // [feature sub-tile of 16][token sub-tile of 16]
@@ -377,7 +404,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
   {                                                                                                                 \
     const uint32_t slot_ = lds_base + (uint32_t)((UNIT) % GEMM_SLOTS) * GEMM_SLOT_BYTES + ld_base;                  \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
-        LDS_DMA16(((UNIT) & 1 ? xg[i] : wg[i]) + (size_t)(SLAB) * GEMM_SLAB, slot_ + i * 1024);                     \
+        LDS_DMA16(((UNIT) & 1 ? xg[i] + (size_t)(SLAB) * x_adv : wg[i] + (size_t)(SLAB) * w_adv), slot_ + i * 1024); \
   }
   // at the end of the phase in which the last fragments of a slab are read, the next slab (x issued this slab, W a
   // slab ago) must be in LDS: everything but this wave's 4 youngest loads (W two slabs ahead, if there is one)
@@ -397,14 +424,41 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
 
   const int frow = lane & 15, fq = lane >> 4;
   u32x4 wf[4], xf[8];
+  // stored [K, rows]: the lane's byte offset inside a slab for k-step 0, hh = 0 of every sub-tile (a k-step adds 32 K-rows =
+  // 16384 bytes, hh = 1 four K-rows = 2048 bytes; the chunk key depends on neither)
+  int xt_off[XT ? 8 : 1], wt_off[WT ? 4 : 1];
+  if constexpr (XT || WT) {
+    const int krow = 8 * fq + (frow >> 2), key = gemm_tkey(krow), sub = (frow & 3) >> 1, byte = (frow & 1) * 8;
+    if constexpr (XT) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) xt_off[j] = krow * 512 + (((wm * 16 + 2 * j + sub) ^ key) << 4) + byte;
+    }
+    if constexpr (WT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wt_off[i] = krow * 512 + (((wn * 8 + 2 * i + sub) ^ key) << 4) + byte;
+    }
+  }
+  typedef __attribute__((ext_vector_type(4))) short gemm_i16x4;
+  typedef __attribute__((address_space(3))) gemm_i16x4 *gemm_lds_i16x4;
+#define READ_TR(DST, BASE, OFF)                                                                                     \
+  {                                                                                                                 \
+    const gemm_i16x4 lo_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gemm_lds_i16x4)((BASE) + (OFF)));               \
+    const gemm_i16x4 hi_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gemm_lds_i16x4)((BASE) + (OFF) + 2048));        \
+    typedef __attribute__((ext_vector_type(8))) short i16x8_;                                                       \
+    DST = __builtin_bit_cast(u32x4, (i16x8_)__builtin_shufflevector(lo_, hi_, 0, 1, 2, 3, 4, 5, 6, 7));             \
+  }
   // a k-step is 64 bytes of K: 4 chunks, one per quarter wave
 #define READ_FRAGS(KS)                                                                                              \
   {                                                                                                                 \
     const int c16_ = 4 * (KS) + fq;                                                                                 \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
-        wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 16 + frow, c16_));                          \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                                   \
-        xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 16 + frow, c16_));                         \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                                 \
+      if constexpr (WT) READ_TR(wf[i], lw, wt_off[i] + (KS) * 16384)                                                \
+      else wf[i] = *reinterpret_cast<const u32x4 *>(lw + swz(wn * 64 + i * 16 + frow, c16_));                       \
+    }                                                                                                               \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                                                 \
+      if constexpr (XT) READ_TR(xf[j], lx, xt_off[j] + (KS) * 16384)                                                \
+      else xf[j] = *reinterpret_cast<const u32x4 *>(lx + swz(wm * 128 + j * 16 + frow, c16_));                      \
+    }                                                                                                               \
   }
 #define MMA_STEP()                                                                                                  \
   _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                                     \
@@ -465,6 +519,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void encoder_gemm_bf16_kernel(
 #undef ISSUE_UNIT
 #undef WAIT_NEXT_SLAB
 #undef READ_FRAGS
+#undef READ_TR
 #undef MMA_STEP
   // The early group has one barrier to go (the late group's last matrix-core phase).  No wave reads operand slabs any
   // more and every load has landed, so LDS is free: the early waves stage and store their output under that phase.
@@ -613,13 +668,13 @@ static int launch_gemm_f32(const void *x, const void *w, void *out, int64_t B, i
   return check_launch("encoder_gemm");
 }
 
-template <bool BF16_OUT, int EPI>
+template <bool BF16_OUT, int EPI, bool XT = false, bool WT = false>
 static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, int64_t d, int64_t F, const float *b_enc,
                             const float *scale, uint32_t *gmax, hipStream_t st, int64_t n_groups = 1,
                             const float *theta = nullptr, int64_t split_k = 1) {
-  // split_k > 1: d is the length of one slice of rows that are split_k * d long; the slices are the launch's groups
+  // split_k > 1: d is the length of one slice of a contraction that is split_k * d long; the slices are the launch's groups
   const int tiles_m = (int)((B + GEMM_BM - 1) / GEMM_BM), tiles_n = (int)((F + GEMM_BN - 1) / GEMM_BN);
-  auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI>;
+  auto kern = encoder_gemm_bf16_kernel<BF16_OUT, EPI, XT, WT>;
   const int rc = reserve_lds(reinterpret_cast<const void *>(kern));
   if (rc != SAE_OK) return rc;
   // with fewer than 8 feature tiles most XCDs would sit idle if those were what is dealt to them: deal the token tiles
@@ -628,9 +683,13 @@ static int launch_gemm_bf16(const void *x, const void *w, void *out, int64_t B, 
   const int ro_log2 = tiles_o >= 8 ? 3 : (tiles_o > 2 ? 2 : (tiles_o > 1 ? 1 : 0)), ro = 1 << ro_log2, rs = 32 >> ro_log2;
   const int rm_log2 = deal_m ? -ro_log2 - 1 : ro_log2;
   const int m_pad = (tiles_o + ro - 1) / ro * ro, n_local_pad = ((tiles_s + 7) / 8 + rs - 1) / rs * rs;
+  // bytes between stored rows: an operand stored [K, rows] has rows of `rows` values; a K-contiguous one rows of the whole
+  // contraction
+  const int64_t k_total = d * (split_k > 1 ? split_k : 1);
+  const int pitch_x = (int)((XT ? B : k_total) * 2), pitch_w = (int)((WT ? F : k_total) * 2);
   hipLaunchKernelGGL(kern, dim3(8 * m_pad * n_local_pad, (unsigned)(split_k > 1 ? split_k : n_groups)), dim3(GEMM_THREADS),
-                     GEMM_LDS_BYTES, st, (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2),
-                     (int)(d * 2 * (split_k > 1 ? split_k : 1)), tiles_m, tiles_n, rm_log2, b_enc, scale, gmax, theta);
+                     GEMM_LDS_BYTES, st, (const char *)x, (const char *)w, out, (int)B, (int)F, (int)(d * 2), pitch_x, pitch_w,
+                     tiles_m, tiles_n, rm_log2, b_enc, scale, gmax, theta);
   return check_launch("encoder_gemm");
 }
 
@@ -672,6 +731,34 @@ extern "C" int sae_encoder_gemm_split_k(const void *x_bf16, const void *w_t_bf16
               "encoder_gemm_split_k: pointers must be 16-byte aligned");
   return launch_gemm_bf16<false, EPI_NONE>(x_bf16, w_t_bf16, partials, B, d / n_splits, F, nullptr, nullptr, nullptr,
                                            (hipStream_t)stream, 1, nullptr, n_splits);
+}
+
+extern "C" int sae_gemm_bf16(const void *a, int a_k_major, const void *b, int b_k_major, void *out, int out_dtype, int64_t M,
+                             int64_t N, int64_t K, int64_t n_splits, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(a && b && out, SAE_ERR_INVALID_ARG, "gemm_bf16: null pointer");
+  SAE_REQUIRE(M > 0 && N > 0 && K > 0 && n_splits >= 1, SAE_ERR_INVALID_ARG, "gemm_bf16: sizes must be positive");
+  SAE_REQUIRE(out_dtype == SAE_F32 || out_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "gemm_bf16: bad out_dtype %d", out_dtype);
+  SAE_REQUIRE(M < (1LL << 30) && N < (1LL << 30) && K < (1LL << 28) && n_splits <= 64, SAE_ERR_UNSUPPORTED, "gemm_bf16: size too large");
+  SAE_REQUIRE(K % (64 * n_splits) == 0, SAE_ERR_UNSUPPORTED, "gemm_bf16: K=%lld must be a multiple of 64 * n_splits", (long long)K);
+  SAE_REQUIRE(n_splits == 1 || (out_dtype == SAE_F32 && (M * N * 4) % 16 == 0), SAE_ERR_UNSUPPORTED,
+              "gemm_bf16: split products write fp32 partial results of a multiple of 16 bytes each");
+  SAE_REQUIRE(!a_k_major || (M % 8 == 0), SAE_ERR_UNSUPPORTED, "gemm_bf16: an operand stored [K, M] needs M=%lld to be a multiple of 8",
+              (long long)M);
+  SAE_REQUIRE(!b_k_major || (N % 8 == 0), SAE_ERR_UNSUPPORTED, "gemm_bf16: an operand stored [K, N] needs N=%lld to be a multiple of 8",
+              (long long)N);
+  SAE_REQUIRE((((uintptr_t)a | (uintptr_t)b | (uintptr_t)out) & 15) == 0, SAE_ERR_INVALID_ARG, "gemm_bf16: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t ks = K / n_splits;
+#define SAE_GEMM_CASE(XT, WT)                                                                                                 \
+  return out_dtype == SAE_BF16                                                                                                \
+             ? launch_gemm_bf16<true, EPI_NONE, XT, WT>(a, b, out, M, ks, N, nullptr, nullptr, nullptr, st, 1, nullptr, n_splits) \
+             : launch_gemm_bf16<false, EPI_NONE, XT, WT>(a, b, out, M, ks, N, nullptr, nullptr, nullptr, st, 1, nullptr, n_splits)
+  if (a_k_major && b_k_major) { SAE_GEMM_CASE(true, true); }
+  if (a_k_major) { SAE_GEMM_CASE(true, false); }
+  if (b_k_major) { SAE_GEMM_CASE(false, true); }
+  SAE_GEMM_CASE(false, false);
+#undef SAE_GEMM_CASE
 }
 
 extern "C" int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups,

@@ -128,7 +128,6 @@ class _ProjectAndMix(torch.autograd.Function):
         n_batch, seq, h, scale = ctx.dims
         dz = dz.contiguous() if dz.dtype == torch.bfloat16 else ops.cast_bf16(dz.float().contiguous())
         dqt, dkt, dvt, stacked = ops.attention_bwd(q, k, v, out, dz, lse, n_batch, seq, h, scale, return_stacked=True)
-        xt = ops.transpose_to_bf16(x_op)[0]                                 # [d, T]
         d = x_op.shape[1]
         n_qk = q.shape[1]
         dq_w = n_qk // h
@@ -138,7 +137,7 @@ class _ProjectAndMix(torch.autograd.Function):
             ops.rotary_bwd_t(stacked[n_qk: 2 * n_qk], cos_t, sin_t, seq, h, rdim, adjacent)
         # the three weight gradients d(.)^T x in one product over the token axis: the gradients share one buffer
         # [2 h dq + F, T], and a single launch fills the chip where three would each leave most of it idle
-        rows = ops.encoder_gemm(stacked, xt, torch.float32)                 # [2 h dq + F, d]
+        rows = ops.gemm(stacked, x_op, torch.float32, b_k_major=True)       # [2 h dq + F, d]; x [T, d] read as it lies
         sums = ops.row_sum(stacked)
 
         def qk_weight_grad(part, shape):
@@ -225,8 +224,8 @@ class _SparseTail(torch.autograd.Function):
         if ctx.amp and ctx.dense_decoder_grad and T % 64 == 0 and d_model % 8 == 0 and F * T <= 400 * code.n_slots:
             import dataclasses
             acts_t = ops.code_to_dense_t(dataclasses.replace(code, val=code.val * g), F)           # [F, T] bf16
-            gd_t = ops.transpose_to_bf16(ctx.grad_recon.contiguous())[0]                          # [d, T] bf16
-            dW_O = ops.encoder_gemm(acts_t, gd_t, torch.float32)        # [F, d]; few output tiles: the product splits its K
+            gd = ops.cast_bf16(ctx.grad_recon.contiguous())                                       # [T, d] bf16, read as it lies
+            dW_O = ops.gemm(acts_t, gd, torch.float32, b_k_major=True)  # [F, d]; few output tiles: the product splits its K
             fi = None
         else:
             fi = ops.build_feature_index(code)
@@ -611,6 +610,14 @@ class LowRankSparseAttention(SparseDictionary):
             amp = _autocast_dtype("cuda") == torch.bfloat16
             out = sparse_decode_blocks(feature_acts.reshape(-1, F), self.W_O, self._w_dec_operand(amp),
                                        max_density=1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel)
+            if out is not None:
+                out = out.view(*feature_acts.shape[:-1], d)
+        if out is None and feature_acts.is_cuda and feature_acts.shape[-1] == F:
+            # denser activations: the GEMM kernel (bf16 operands read W_O as it lies)
+            from .sae import dense_decode
+
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            out = dense_decode(self, feature_acts.reshape(-1, F), self.W_O, self._w_dec_operand(amp), "W_O.t.f32")
             if out is not None:
                 out = out.view(*feature_acts.shape[:-1], d)
         if out is None:

@@ -317,6 +317,37 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype,
     return pre
 
 
+def gemm(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype, a_k_major: bool = False, b_k_major: bool = False,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = sum_k A[m, k] B[n, k] for bf16 operands in either layout: an operand is [rows, K] (its K values side by
+    side, what `encoder_gemm` takes) or, with its `*_k_major` flag, [K, rows], read as it lies with no transposed copy.
+    `gemm(g, x, dt, True, True)` is g^T @ x for g [tokens, m], x [tokens, n] (a weight gradient over the token axis);
+    `gemm(acts, W, dt, False, True)` is acts @ W for W [K, n] (a dense decode)."""
+    _req(a, "a", torch.bfloat16, 2)
+    _req(b, "b", torch.bfloat16, 2)
+    K, M = a.shape if a_k_major else (a.shape[1], a.shape[0])
+    Kb, N = b.shape if b_k_major else (b.shape[1], b.shape[0])
+    if K != Kb:
+        raise ValueError(f"contraction lengths differ: a {tuple(a.shape)} (k-major {a_k_major}) vs b {tuple(b.shape)} (k-major {b_k_major})")
+    if out is not None:
+        _req(out, "out", out_dtype, 2)
+        if tuple(out.shape) != (M, N):
+            raise ValueError(f"out must be {(M, N)}, got {tuple(out.shape)}")
+    splits = gemm_split_k(M, K, N) if out_dtype == torch.float32 and (M * N) % 4 == 0 else 1
+    lib = _lib.load()
+    if splits > 1:
+        partials = torch.empty(splits, M, N, dtype=torch.float32, device=a.device)
+        with _timed("encoder_gemm"):
+            check(lib.sae_gemm_bf16(a.data_ptr(), int(a_k_major), b.data_ptr(), int(b_k_major), partials.data_ptr(), SAE_F32, M, N, K,
+                                    splits, _stream(a)), "gemm_bf16")
+        return partials.sum(0) if out is None else torch.sum(partials, 0, out=out)
+    res = out if out is not None else torch.empty(M, N, dtype=out_dtype, device=a.device)
+    with _timed("encoder_gemm"):
+        check(lib.sae_gemm_bf16(a.data_ptr(), int(a_k_major), b.data_ptr(), int(b_k_major), res.data_ptr(), _dt(res), M, N, K, 1,
+                                _stream(a)), "gemm_bf16")
+    return res
+
+
 def gemm_split_k(B: int, d: int, F: int) -> int:
     """How many slices of the contraction axis a bf16 -> fp32 product [B, d] x [F, d]^T is cut into: products with few
     256 x 256 output tiles and a long contraction (weight gradients over the token axis) would occupy a fraction of the

@@ -180,8 +180,9 @@ def _aux_dense_block(x_op, pre_dtype, w_enc_op, w_dec_op, b_E, scale, dead, k_au
     # dense [B, ndp] activations of the block: fp32 (the mask of the backward pass) and, under autocast, bf16
     A, A_b16 = ops.code_to_dense(code_d, ndp, want_f32=True, want_bf16=amp)
     A_op = A_b16 if amp else A
-    W_D_T = ops.transpose_to_bf16(W_D)[0] if amp else W_D.t().contiguous()
-    aux_recon = ops.encoder_gemm(A_op, W_D_T, torch.float32)                          # [B, d] = A @ W_D[dead]
+    # [B, d] = A @ W_D[dead]: bf16 operands read the gathered decoder rows as they lie
+    aux_recon = (ops.gemm(A_op, W_D, torch.float32, b_k_major=True) if amp
+                 else ops.encoder_gemm(A_op, W_D.t().contiguous(), torch.float32))
     # the same code with the dictionary's own feature ids (for callers that look at it); slots past the last
     # token's end are unused and keep index 0
     n_used = code_d.row_off[-1] + code_d.row_nnz[-1]
@@ -212,12 +213,14 @@ def _aux_dense_grads(blk, g_aux, x_op, amp: bool):
     A, A_op = blk["A"], blk["A_op"]
     g_aux = g_aux.contiguous()
     if amp:
-        # bf16 operands; the transposes round the fp32 sources themselves, so each equals cast-then-transpose
+        # bf16 operands
         G_op = ops.cast_bf16(g_aux)
         dA = ops.encoder_gemm(G_op, blk["W_D"], torch.float32)                         # [B, ndp]
         dpre_T, db_E = ops.transpose_to_bf16(dA, mask=A, col_sums=True)                 # d pre = dA where A > 0
-        dW_D = ops.encoder_gemm(ops.transpose_to_bf16(A_op)[0], ops.transpose_to_bf16(g_aux)[0], torch.float32)   # [ndp, d]
-        dW_Et = ops.encoder_gemm(dpre_T, ops.transpose_to_bf16(x_op)[0], torch.float32)                            # [ndp, d]
+        # the two products over the token axis read A, G and x as they lie (stored [tokens, .]); d pre arrives transposed
+        # from the pass that masks it and sums its columns
+        dW_D = ops.gemm(A_op, G_op, torch.float32, a_k_major=True, b_k_major=True)                                # [ndp, d]
+        dW_Et = ops.gemm(dpre_T, x_op, torch.float32, b_k_major=True)                                              # [ndp, d]
         dpre = None   # formed on demand (only the gradient with respect to x wants it in this layout)
     else:
         dA = ops.encoder_gemm(g_aux, blk["W_D"], torch.float32)
@@ -444,8 +447,12 @@ def _gemm_k_ok(k: int, dtype: torch.dtype) -> bool:
 
 
 def _rows_over_tokens(left: torch.Tensor, right: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """left^T @ right for left [B, m], right [B, n] -> [m, n]: a product over the token axis (a weight gradient).  The
-    GEMM kernel contracts over the contiguous axis of both operands, so both are transposed first."""
+    """left^T @ right for left [B, m], right [B, n] -> [m, n]: a product over the token axis (a weight gradient).  bf16
+    operands are read as they lie (both are stored [K, rows] for this product); fp32 operands are transposed first, for
+    the fp32 kernel contracts over the contiguous axis of both."""
+    if (left.dtype == torch.bfloat16 and right.dtype == torch.bfloat16 and left.shape[0] % 64 == 0 and left.shape[1] % 8 == 0
+            and right.shape[1] % 8 == 0):
+        return ops.gemm(left.contiguous(), right.contiguous(), out_dtype, a_k_major=True, b_k_major=True)
     if _gemm_k_ok(left.shape[0], left.dtype):
         return ops.encoder_gemm(_transposed(left), _transposed(right), out_dtype)
     return (left.t() @ right).to(out_dtype)       # a token count the kernel's K granule does not divide
@@ -527,14 +534,18 @@ class _RowNormDeferred(torch.autograd.Function):
 class _DenseDecode(torch.autograd.Function):
     """acts @ W_D for dense activations on the GEMM kernel (models/sae.py:367).  `w_op` is W_D [F, d] as the kernels
     read it (under autocast the bf16 copy the optimiser maintains, so that the per-step cast of the fp32 master and
-    its backward are not run), `w_t` the same matrix transposed [d, F]: the forward product contracts over features.
+    its backward are not run).  The forward product contracts over features: bf16 operands read W_D as it lies ([K, d]
+    with K = features), fp32 operands a transposed copy `w_t` [d, F].
     Backward: d acts = g W_D^T contracts over d_model (W_D as it is), dW_D = acts^T g over the tokens."""
 
     @staticmethod
-    def forward(ctx, acts, W_D, w_op, w_t, defer=False):
+    def forward(ctx, acts, W_D, w_op, w_t=None, defer=False):
         acts = acts.contiguous()
         ctx.save_for_backward(acts, w_op)
         ctx.param = W_D if (defer and W_D.is_contiguous() and w_op.dtype == torch.bfloat16) else None
+        ctx.w_dtype = W_D.dtype
+        if w_t is None:
+            return ops.gemm(acts, w_op, acts.dtype, b_k_major=True)
         return ops.encoder_gemm(acts, w_t, acts.dtype)
 
     @staticmethod
@@ -548,8 +559,28 @@ class _DenseDecode(torch.autograd.Function):
             if ctx.param is not None:
                 _leave_lowp_grad(ctx.param, rows)
             else:
-                dW = rows.float()
+                dW = rows.to(ctx.w_dtype)
         return d_acts, dW, None, None, None
+
+
+def dense_decode(model, acts: torch.Tensor, W_D: torch.Tensor, w_op: torch.Tensor, w_t_name: str, defer: bool = False):
+    """acts [B, F] @ W_D [F, d] through `_DenseDecode` when the GEMM kernel takes the shapes, else None.  `w_op`: W_D as the
+    kernels read it; the activations are cast to its dtype (under autocast the bf16 copy: what the reference's autocast
+    matmul does to its operands).  A transposed fp32 copy is derived (and cached on `model` under `w_t_name`) only where
+    the fp32 kernel needs one."""
+    F, d = w_op.shape
+    if acts.ndim != 2 or acts.shape[-1] != F or not acts.is_cuda or w_op.dtype not in (torch.float32, torch.bfloat16):
+        return None
+    acts = acts.to(w_op.dtype)
+    # the forward contracts over F, the backward's d acts = g W_D^T over d: both must be whole slabs of the kernel
+    if w_op.dtype == torch.bfloat16:
+        if F % 64 == 0 and d % 64 == 0:
+            return _DenseDecode.apply(acts, W_D, w_op, None, defer)
+        return None
+    if w_op.dtype == torch.float32 and F % 32 == 0 and d % 32 == 0:
+        w_t = model._derive(w_t_name, W_D, lambda old: _transposed(w_op))
+        return _DenseDecode.apply(acts, W_D, w_op, w_t, defer)
+    return None
 
 
 class _JumpReLUStep(torch.autograd.Function):
@@ -721,11 +752,6 @@ class SparseAutoEncoder(SparseDictionary):
             return w
         return self._derive("W_D.bf16", self.W_D, lambda old: ops.cast_bf16(w, old))
 
-    def _w_dec_t_operand(self, amp: bool) -> torch.Tensor:
-        """W_D^T [d, F] in the operand dtype: what a dense `acts @ W_D` on the GEMM kernel contracts against."""
-        w = self._w_dec_operand(amp)
-        return self._derive("W_D.t.bf16" if w.dtype == torch.bfloat16 else "W_D.t.f32", self.W_D, lambda old: _transposed(w))
-
     def _decoder_norm_nograd(self) -> torch.Tensor:
         self.wait_pending_update()
         return self._derive("W_D.norm", self.W_D, lambda old: ops.row_norm(self.W_D.detach().float(), old))
@@ -849,6 +875,13 @@ class SparseAutoEncoder(SparseDictionary):
             if 0 < max_l0 < self.cfg.d_sae * (1 - self.cfg.sparsity_threshold_for_triton_spmm_kernel):
                 amp = _autocast_dtype("cuda") == torch.bfloat16
                 reconstructed = decode_with_hip_spmm_kernel(feature_acts, self.W_D, w_operand=self._w_dec_operand(amp), transposed=False)
+        if reconstructed is None and feature_acts.is_cuda:
+            # models/sae.py:367 on the GEMM kernel: bf16 operands read W_D as it lies, with the weight gradient as a product
+            # over the token axis on the same kernel
+            amp = _autocast_dtype("cuda") == torch.bfloat16
+            out = dense_decode(self, feature_acts.reshape(-1, feature_acts.shape[-1]), self.W_D, self._w_dec_operand(amp), "W_D.t.f32")
+            if out is not None:
+                reconstructed = out.view(*feature_acts.shape[:-1], out.shape[-1])
         if reconstructed is None:
             reconstructed = feature_acts @ self.W_D
         if self.cfg.use_decoder_bias:
@@ -950,9 +983,8 @@ class SparseAutoEncoder(SparseDictionary):
         acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
                                                      float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
                                                      want_tanh, want_lp)
-        if _gemm_k_ok(self.cfg.d_sae, acts.dtype) and self.cfg.d_model % 8 == 0:
-            reconstructed = _DenseDecode.apply(acts, self.W_D, self._w_dec_operand(amp), self._w_dec_t_operand(amp), defer)
-        else:
+        reconstructed = dense_decode(self, acts, self.W_D, self._w_dec_operand(amp), "W_D.t.f32", defer)
+        if reconstructed is None:
             reconstructed = acts @ self.W_D
         if self.cfg.use_decoder_bias:
             reconstructed = reconstructed + self.b_D

@@ -63,6 +63,43 @@ def test_encoder_gemm_bf16(pkg, dev, B, d, F, out_dtype):
         assert (diff == 0).float().mean() > 0.99
 
 
+@pytest.mark.parametrize("M,K,N", [(256, 64, 256), (264, 128, 1000), (512, 2048, 776), (40, 64, 72), (8, 64, 16), (2304, 192, 520),
+                                   (1000, 4096, 200), (776, 8192, 264)])
+@pytest.mark.parametrize("a_k_major,b_k_major", [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16_operand_layouts(pkg, dev, M, K, N, a_k_major, b_k_major, out_dtype):
+    """sae_gemm_bf16 with an operand stored [K, rows]: the product of the operands as they lie equals, BIT FOR BIT, the
+    K-contiguous kernel's product of their transposed copies (the same fragments reach the matrix cores in the same order),
+    and both match the exact product of the bf16 operands.  Shapes with edge tiles in both dimensions, one to 128 slabs of
+    K, and long contractions over few tiles (cut into slices for fp32 output, as for the K-contiguous kernel)."""
+    print(f"gemm layouts M={M} K={K} N={N} a_k_major={a_k_major} b_k_major={b_k_major} out={out_dtype}", flush=True)
+    g = torch.Generator().manual_seed(M * 13 + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    b = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16()
+    a_dev, b_dev = a.to(dev), b.to(dev)
+    a_arg = a_dev.t().contiguous() if a_k_major else a_dev
+    b_arg = b_dev.t().contiguous() if b_k_major else b_dev
+    got = pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major)
+    plain = pkg.ops.encoder_gemm(a_dev, b_dev, out_dtype)
+    assert got.shape == (M, N) and got.dtype == out_dtype
+    assert torch.equal(got, plain)
+    want = a.double() @ b.double().t()
+    assert rel_err(got, want) < (FP32_TOL if out_dtype == torch.float32 else 2 ** -7)
+    # into a given output tensor
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    assert pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major, out=out) is out
+    assert torch.equal(out, plain)
+
+
+def test_gemm_bf16_rejects_what_it_cannot_address(pkg, dev):
+    a = torch.zeros(64, 12, dtype=torch.bfloat16, device=dev)       # [K, M] with M = 12: not a multiple of 8
+    b = torch.zeros(16, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        pkg.ops.gemm(a, b, torch.float32, a_k_major=True)
+    with pytest.raises(ValueError, match="contraction"):
+        pkg.ops.gemm(b, torch.zeros(16, 128, dtype=torch.bfloat16, device=dev), torch.float32)
+
+
 def test_encoder_gemm_rejects_bad_shapes(pkg, dev):
     x = torch.randn(8, 40, device=dev)
     w = torch.randn(16, 40, device=dev)
