@@ -317,12 +317,26 @@ def encoder_gemm(x: torch.Tensor, w_enc_t: torch.Tensor, out_dtype: torch.dtype,
     return pre
 
 
+def _k_major_read_pays(rows: int, other_rows: int, K: int, a_side: bool) -> bool:
+    """Whether an operand stored [K, rows] is better read as it lies than copied into [rows, K] first.  Reading across
+    the K-rows of the LDS tile takes two 8-byte reads per fragment instead of one 16-byte read: measured +16 % of the
+    product's time for the operand whose rows are the output's rows (eight fragments per wave and k-step), +9 % for the
+    other (four); a transposed copy moves 4 bytes per element at about 4.7 TB/s behind a launch of its own.  Both routes
+    give the same bits."""
+    t_gemm = 2.0 * rows * other_rows * K / 1.4e15
+    extra = (0.16 if a_side else 0.09) * t_gemm
+    copy = rows * K * 4.0 / 4.7e12 + 8e-6
+    return extra <= copy
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype, a_k_major: bool = False, b_k_major: bool = False,
-         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+         out: Optional[torch.Tensor] = None, copy_when_faster: bool = True) -> torch.Tensor:
     """out[M, N] = sum_k A[m, k] B[n, k] for bf16 operands in either layout: an operand is [rows, K] (its K values side by
-    side, what `encoder_gemm` takes) or, with its `*_k_major` flag, [K, rows], read as it lies with no transposed copy.
-    `gemm(g, x, dt, True, True)` is g^T @ x for g [tokens, m], x [tokens, n] (a weight gradient over the token axis);
-    `gemm(acts, W, dt, False, True)` is acts @ W for W [K, n] (a dense decode)."""
+    side, what `encoder_gemm` takes) or, with its `*_k_major` flag, [K, rows].  `gemm(g, x, dt, True, True)` is g^T @ x for
+    g [tokens, m], x [tokens, n] (a weight gradient over the token axis); `gemm(acts, W, dt, False, True)` is acts @ W for
+    W [K, n] (a dense decode).  A [K, rows] operand is read as it lies, with no transposed copy, unless
+    `copy_when_faster` and a copy is the cheaper way for the shape (`_k_major_read_pays`); the result is the same bit
+    for bit."""
     _req(a, "a", torch.bfloat16, 2)
     _req(b, "b", torch.bfloat16, 2)
     K, M = a.shape if a_k_major else (a.shape[1], a.shape[0])
@@ -333,6 +347,11 @@ def gemm(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype, a_k_major: bo
         _req(out, "out", out_dtype, 2)
         if tuple(out.shape) != (M, N):
             raise ValueError(f"out must be {(M, N)}, got {tuple(out.shape)}")
+    if copy_when_faster:
+        if a_k_major and not _k_major_read_pays(M, N, K, True):
+            a, a_k_major = transpose_to_bf16(a)[0], False
+        if b_k_major and not _k_major_read_pays(N, M, K, False):
+            b, b_k_major = transpose_to_bf16(b)[0], False
     splits = gemm_split_k(M, K, N) if out_dtype == torch.float32 and (M * N) % 4 == 0 else 1
     lib = _lib.load()
     if splits > 1:

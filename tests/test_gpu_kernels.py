@@ -79,7 +79,7 @@ def test_gemm_bf16_operand_layouts(pkg, dev, M, K, N, a_k_major, b_k_major, out_
     a_dev, b_dev = a.to(dev), b.to(dev)
     a_arg = a_dev.t().contiguous() if a_k_major else a_dev
     b_arg = b_dev.t().contiguous() if b_k_major else b_dev
-    got = pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major)
+    got = pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major, copy_when_faster=False)
     plain = pkg.ops.encoder_gemm(a_dev, b_dev, out_dtype)
     assert got.shape == (M, N) and got.dtype == out_dtype
     assert torch.equal(got, plain)
@@ -87,15 +87,17 @@ def test_gemm_bf16_operand_layouts(pkg, dev, M, K, N, a_k_major, b_k_major, out_
     assert rel_err(got, want) < (FP32_TOL if out_dtype == torch.float32 else 2 ** -7)
     # into a given output tensor
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
-    assert pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major, out=out) is out
+    assert pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major, out=out, copy_when_faster=False) is out
     assert torch.equal(out, plain)
+    # with the choice between reading across the rows and a transposed copy left to the shape: the same bits
+    assert torch.equal(pkg.ops.gemm(a_arg, b_arg, out_dtype, a_k_major=a_k_major, b_k_major=b_k_major), plain)
 
 
 def test_gemm_bf16_rejects_what_it_cannot_address(pkg, dev):
     a = torch.zeros(64, 12, dtype=torch.bfloat16, device=dev)       # [K, M] with M = 12: not a multiple of 8
     b = torch.zeros(16, 64, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="multiple of 8"):
-        pkg.ops.gemm(a, b, torch.float32, a_k_major=True)
+        pkg.ops.gemm(a, b, torch.float32, a_k_major=True, copy_when_faster=False)
     with pytest.raises(ValueError, match="contraction"):
         pkg.ops.gemm(b, torch.zeros(16, 128, dtype=torch.bfloat16, device=dev), torch.float32)
 
