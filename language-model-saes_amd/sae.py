@@ -613,17 +613,38 @@ class _JumpReLUStep(torch.autograd.Function):
         return d_pre, d_bias.to(ctx.b_dtype), d_norm, d_theta.to(ctx.th_dtype), None, None, None, None, None
 
 
+def _code_penalty(code: ops.SparseCode, norm: torch.Tensor, kind: str, c: float, p: float, freq_scale: float, n_tokens: int):
+    """The sparsity penalty of a sparse code before its coefficient (models/sparse_dictionary.py:888-925 on a = f n at
+    the code's entries; entries that are zero add nothing to any of the three): per-token values [B] for "tanh" and
+    "power", one scalar for "tanh-quad"; plus what the backward needs (per-token power sums / per-feature frequencies)."""
+    tok, valid = _code_slot_tokens(code)
+    a = torch.where(valid, code.val * norm[code.idx.long()], torch.zeros_like(code.val))
+    B = code.n_tokens
+    if kind == "tanh":
+        pen = torch.zeros(B, dtype=torch.float32, device=a.device).index_add_(0, tok, torch.tanh(c * a))
+        return pen, None
+    if kind == "power":
+        S = torch.zeros(B, dtype=torch.float32, device=a.device).index_add_(0, tok, a.pow(p))
+        return S.pow(1.0 / p), S
+    if kind == "tanh-quad":
+        q = torch.zeros(code.d_sae, dtype=torch.float32, device=a.device).index_add_(0, code.idx.long(), torch.tanh(c * a)) / n_tokens
+        return (q * (1 + q / freq_scale)).sum(), q
+    raise ValueError(f"sparsity_loss_type f{kind} not supported.")
+
+
 class _JumpReLUSparseStep(torch.autograd.Function):
-    """The JumpReLU step of a dictionary whose activations are sparse: threshold select -> sparse decode + squared error
-    (+ tanh penalty) forward, and backward through the feature index of the code, like the TopK step.  The code holds
-    every token's kept features and, with value 0, the features inside the straight-through window that are not kept;
-    `dval` (the decoder's gradient at every entry) is what both the pre-activation gradient of kept entries and the
-    threshold gradient of window entries start from.  With ga = dval + l1 w_b c n (1 - tanh^2(c a n)):
+    """The step of a dictionary whose activations are a sparse code, with a sparsity penalty: sparse decode + squared error
+    (+ tanh / power / tanh-quad penalty) forward, and backward through the feature index of the code, like the plain TopK
+    step.  For a JumpReLU the code holds every token's kept features and, with value 0, the features inside the
+    straight-through window that are not kept (`win` flags them); for a TopK-family or ReLU dictionary it holds the
+    kept entries, `win` is zero and the threshold a vector of zeros.  `dval` (the decoder's gradient at every entry) is
+    what both the pre-activation gradient of kept entries and the threshold gradient of window entries start from.  With
+    a = f n the penalised quantity, P' = d penalty / d a at the entry, and ga = dval + P' n:
         d pre   = ga at kept entries                              -> dW_E^T rows, db_E (factored)
         d theta = sum over window entries of (ga / s) (-theta / window)
-        d n     = sum over kept entries of l1 w_b c a (1 - tanh^2)
-    exactly the sums the dense backward kernel forms over [B, F] (the two derivative terms of act(h s) / s with
-    respect to s cancel)."""
+        d n     = sum over kept entries of P' f
+    exactly the sums the dense backward forms over [B, F] (the two derivative terms of act(h s) / s with respect to s
+    cancel)."""
 
     @staticmethod
     def forward(ctx, theta, norm, W_E, b_E, W_D, b_D, label, tok_w, holder):
@@ -634,9 +655,15 @@ class _JumpReLUSparseStep(torch.autograd.Function):
                                                                         label, tok_w)
         loss = loss_tok.sum()
         l_s = None
-        if holder["want_tanh"]:
-            l_s = holder["l1"] * holder["tanh_tok"]
-            loss = loss + (tok_w * l_s).sum()
+        kind = holder.get("pen")
+        if kind is not None:
+            pen, aux = holder.get("pen_tok"), None
+            if pen is None:
+                pen, aux = _code_penalty(code, norm.detach().float(), kind, holder["tanh_c"], holder.get("p", 1),
+                                         holder.get("frequency_scale", 0.01), code.n_tokens)
+            l_s = holder["l1"] * pen
+            loss = loss + ((tok_w * l_s).sum() if l_s.ndim else l_s)
+            holder["pen_aux"] = aux
         holder["l_s"], holder["l_rec"] = l_s, loss_tok.sum()
         ctx.save_for_backward(theta.detach().float(), tok_w, grad_recon, dval, *(() if norm is None else (norm.detach().float(),)))
         ctx.holder, ctx.has_norm, ctx.has_b_D = holder, norm is not None, b_D is not None
@@ -658,20 +685,37 @@ class _JumpReLUSparseStep(torch.autograd.Function):
         fi = ops.build_feature_index(code)
         idx = code.idx.long()
         val = code.val
-        th_f = theta[idx]
         s_f = norm[idx] if (norm is not None and h["scaled"]) else None
         ga, dn_slot = dval, None
-        if h["want_tanh"]:
+        kind = h.get("pen")
+        if kind is not None:
             n_f = norm[idx]
-            c = h["tanh_c"]
-            t = torch.tanh(c * val * n_f)
-            sech2 = 1.0 - t * t
-            gt = (h["l1"] * c) * tok_w[fi.slot_tok.long()]
-            ga = dval + gt * n_f * sech2
-            dn_slot = (gt * val * sech2).contiguous()
+            a = val * n_f
+            if kind == "tanh":
+                c = h["tanh_c"]
+                t = torch.tanh(c * a)
+                dpen = (h["l1"] * c) * tok_w[fi.slot_tok.long()] * (1.0 - t * t)
+            elif kind == "power":
+                p, S = float(h.get("p", 1)), h["pen_aux"][fi.slot_tok.long()]
+                # d (sum a^p)^(1/p) / d a = S^(1/p - 1) a^(p - 1); torch's norm sends nothing to entries that are zero
+                dpen = torch.where(a > 0, h["l1"] * tok_w[fi.slot_tok.long()] * S.clamp_min(1e-30).pow(1.0 / p - 1.0) * a.pow(p - 1.0),
+                                   torch.zeros_like(a))
+            else:   # tanh-quad: q_f = mean over tokens of tanh(c a); l_s = l1 sum_f q_f (1 + q_f / scale)
+                c = h["tanh_c"]
+                t = torch.tanh(c * a)
+                q = h["pen_aux"][idx]
+                dpen = (h["l1"] * c / code.n_tokens) * (1.0 + 2.0 * q / h.get("frequency_scale", 0.01)) * (1.0 - t * t)
+            ga = dval + dpen * n_f
+            dn_slot = (dpen * val).contiguous()
         d_pre = torch.where(val > 0, ga, torch.zeros_like(ga))
-        dth_slot = win * (ga if s_f is None else ga / s_f) * (-th_f / h["window"])
-        d_theta, d_norm = ops.feature_segment_sums(fi, dth_slot.contiguous(), dn_slot)
+        d_theta = None
+        if h.get("has_theta", True):
+            th_f = theta[idx]
+            dth_slot = win * (ga if s_f is None else ga / s_f) * (-th_f / h["window"])
+            d_theta, d_norm = ops.feature_segment_sums(fi, dth_slot.contiguous(), dn_slot)
+            d_theta = (d_theta * g).to(ctx.th_dtype)
+        else:
+            d_norm = ops.feature_segment_sums(fi, dn_slot)[0] if dn_slot is not None else None
         coef_dec, coef_enc = val * g, d_pre * g
         x_op = h["x_op"]
         grad_dense_D = ops.cast_bf16(grad_recon) if h["amp"] else grad_recon
@@ -685,7 +729,7 @@ class _JumpReLUSparseStep(torch.autograd.Function):
             dW_D, _ = ops.sparse_grad_rows(fi, coef_dec, grad_dense_D, F)
             dW_Et, db_E = ops.sparse_grad_rows(fi, coef_enc, x_op, F, want_bias=True)
             dW_E = dW_Et.t()
-        return ((d_theta * g).to(ctx.th_dtype), None if d_norm is None or not ctx.needs_input_grad[1] else d_norm * g,
+        return (d_theta, None if d_norm is None or not ctx.needs_input_grad[1] else d_norm * g,
                 dW_E, db_E, dW_D, db_D, None, None, None)
 
 
@@ -908,33 +952,51 @@ class SparseAutoEncoder(SparseDictionary):
         return batch[self.cfg.hook_point_out]
 
     # ---- fused train-step loss ----
+    def _no_hooks(self) -> bool:
+        return not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
+
     def _fused_eligible(self, x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
+        """TopK / BatchTopK: the plain step (reconstruction loss, optionally aux-k) or, with a sparsity penalty, the step
+        with the penalty formed on the sparse code.  (An Lp coefficient is ignored for these activations, as the
+        reference's loss does: models/sparse_dictionary.py:927.)"""
         amp = _autocast_dtype("cuda") == torch.bfloat16 or self.W_E.dtype == torch.bfloat16
         # what the kernels are built for: the GEMM's K granule, 16-byte decoder rows, and the feature index's token
         # limit (the sparse aux-k route stacks a second code onto the token axis); other shapes take the dense route
         shapes_fit = (self.cfg.d_model % (64 if amp else 32) == 0
                       and x.shape[0] * (2 if auxk_coefficient > 0.0 else 1) <= 131072)
+        if sparsity_loss_type is not None and (auxk_coefficient > 0.0 or self.W_E.dtype != torch.float32
+                                               or sparsity_loss_type not in ("tanh", "power", "tanh-quad")):
+            return False
         return (
             self.cfg.act_fn.lower() in ("topk", "batchtopk")
             and x.is_cuda and x.ndim == 2 and label.ndim == 2 and shapes_fit
-            and not self.cfg.use_glu_encoder
-            and sparsity_loss_type is None and not (lp_coefficient > 0.0)
-            and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
+            and not self.cfg.use_glu_encoder and self._no_hooks()
             and (self.W_E.dtype == torch.float32
                  or (self.W_E.dtype == torch.bfloat16 and self.cfg.d_model % 64 == 0))
         )
 
-    # ---- JumpReLU train-step loss: dense activations, so the GEMM kernel for all five dense products (two of them
-    # over the token axis, on transposed operands) + one fused element-wise pass each way ----
+    # ---- JumpReLU / ReLU train-step loss: dense activations, so the GEMM kernel for all five dense products + one fused
+    # element-wise pass each way (a ReLU is the same kernels with a threshold of zero, which has no gradient) ----
     def _jumprelu_eligible(self, x, label, sparsity_loss_type, auxk_coefficient) -> bool:
         amp = _autocast_dtype("cuda") == torch.bfloat16
         return (
-            self.cfg.act_fn.lower() == "jumprelu" and x.is_cuda and x.ndim == 2 and label.ndim == 2
+            self.cfg.act_fn.lower() in ("jumprelu", "relu") and x.is_cuda and x.ndim == 2 and label.ndim == 2
             and not self.cfg.use_glu_encoder and sparsity_loss_type in (None, "tanh", "power", "tanh-quad")
-            and not (auxk_coefficient > 0.0)
-            and not (self.hook_hidden_pre.has_hooks or self.hook_feature_acts.has_hooks or self.hook_reconstructed.has_hooks)
+            and not (auxk_coefficient > 0.0) and self._no_hooks()
             and self.W_E.dtype == torch.float32 and self.cfg.d_sae % 8 == 0 and self.cfg.d_model % (64 if amp else 32) == 0
         )
+
+    def _threshold_and_window(self):
+        """(theta [F], window) of the activation: the JumpReLU's own, or zeros and any window for a ReLU (x > 0 is x > theta
+        with theta = 0, and d theta = g (-theta / window) vanishes)."""
+        jr = self.activation_function
+        if self.cfg.act_fn.lower() == "jumprelu":
+            return jr.get_jumprelu_threshold(), float(jr.jumprelu_threshold_window)
+        zero = self.__dict__.get("_zero_theta")
+        if zero is None or zero.device != self.b_E.device:
+            zero = torch.zeros(self.cfg.d_sae, dtype=torch.float32, device=self.b_E.device)
+            self.__dict__["_zero_theta"] = zero
+        return zero, 1.0
 
     def _jumprelu_loss(self, batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient, lp_coefficient,
                        auxk_coefficient, return_aux_data, frequency_scale: float = 0.01, p: int = 1):
@@ -942,19 +1004,20 @@ class SparseAutoEncoder(SparseDictionary):
 
         mask = batch.get("mask")
         amp = _autocast_dtype("cuda") == torch.bfloat16
-        jr = self.activation_function
+        is_jr = self.cfg.act_fn.lower() == "jumprelu"
+        theta, window = self._threshold_and_window()
         defer = bool(self.defer_weight_grads and torch.is_grad_enabled())
-        want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0
+        want_tanh, want_lp = sparsity_loss_type == "tanh", lp_coefficient > 0.0 and is_jr
         scaled = bool(self.cfg.sparsity_include_decoder_norm)
         w_enc_op = self._w_enc_operand(amp)
         given = None
         B = x.shape[0]
-        if (self.jumprelu_sparse_route and sparsity_loss_type in (None, "tanh") and not want_lp and B <= 131072
+        if (self.jumprelu_sparse_route and not want_lp and B <= 131072
                 and self.cfg.d_model % 8 == 0 and self._jr_dense_steps % max(1, self.jumprelu_sparse_probe_every) == 0):
             with torch.no_grad():
                 x_op = (x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())) if amp else x.float().contiguous()
-                n_raw = self._decoder_norm_nograd() if (scaled or want_tanh) else None
-                th_raw = jr.get_jumprelu_threshold().detach().float().contiguous()
+                n_raw = self._decoder_norm_nograd() if (scaled or sparsity_loss_type is not None) else None
+                th_raw = theta.detach().float().contiguous()
                 b_raw = self.b_E.detach().float()
                 margin = None
                 # once the route has been sparse, the product's epilogue also leaves every granule's largest margin over
@@ -966,22 +1029,22 @@ class SparseAutoEncoder(SparseDictionary):
                     pre_raw = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16 if amp else torch.float32)
                 given = (x_op, pre_raw)
                 budget = int(B * self.cfg.d_sae * (1.0 - self.cfg.sparsity_threshold_for_triton_spmm_kernel))
-                picked = ops.jumprelu_select(pre_raw, b_raw, n_raw if scaled else None, th_raw,
-                                             float(jr.jumprelu_threshold_window), float(tanh_stretch_coefficient), pen_norm=n_raw,
+                picked = ops.jumprelu_select(pre_raw, b_raw, n_raw if scaled else None, th_raw, window,
+                                             float(tanh_stretch_coefficient), pen_norm=n_raw,
                                              want_tanh=want_tanh, max_entries=budget, granule_margin=margin)
             if picked is not None:
                 self._jr_dense_steps = 0
-                return self._jumprelu_sparse_loss(batch, x, label, mask, picked, x_op, amp, defer, scaled, want_tanh,
-                                                  float(tanh_stretch_coefficient), float(l1_coefficient), lp_coefficient,
-                                                  auxk_coefficient, return_aux_data, pre_raw)
+                code, win, tanh_tok, _l0 = picked
+                return self._sparse_code_loss(batch, label, mask, code, win, x_op, pre_raw, amp, defer, theta, window,
+                                              sparsity_loss_type, tanh_tok, float(tanh_stretch_coefficient), float(l1_coefficient),
+                                              float(frequency_scale), p, lp_coefficient, auxk_coefficient, return_aux_data)
         self._jr_dense_steps += 1
         pre = _EncoderGemm.apply(x, self.W_E, w_enc_op, amp, defer, given)
         n = None
         want_dense_pen = sparsity_loss_type in ("power", "tanh-quad")
         if scaled or want_tanh or want_lp or want_dense_pen:
             n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), self if defer else None)
-        acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, jr.get_jumprelu_threshold(), scaled,
-                                                     float(tanh_stretch_coefficient), float(jr.jumprelu_threshold_window),
+        acts, tanh_tok, lp_tok = _JumpReLUStep.apply(pre, self.b_E, n, theta, scaled, float(tanh_stretch_coefficient), window,
                                                      want_tanh, want_lp)
         reconstructed = dense_decode(self, acts, self.W_D, self._w_dec_operand(amp), "W_D.t.f32", defer)
         if reconstructed is None:
@@ -1019,35 +1082,104 @@ class SparseAutoEncoder(SparseDictionary):
                 "hidden_pre": lambda: pre.detach().float() + b_E}
         return LazyDict(eager, lazy)
 
-    def _jumprelu_sparse_loss(self, batch, x, label, mask, picked, x_op, amp, defer, scaled, want_tanh, tanh_c, l1_coefficient,
-                              lp_coefficient, auxk_coefficient, return_aux_data, pre_raw):
-        code, win, tanh_tok, l0_tok = picked
-        jr = self.activation_function
-        B = x.shape[0]
+    def _sparse_code_loss(self, batch, label, mask, code, win, x_op, pre_raw, amp, defer, theta, window, sparsity_loss_type,
+                          pen_tok, tanh_c, l1_coefficient, frequency_scale, p, lp_coefficient, auxk_coefficient, return_aux_data):
+        """Loss of a step whose activations are the sparse code `code` (JumpReLU / ReLU above the sparsity gate, or a TopK
+        family selection) with an optional sparsity penalty, through `_JumpReLUSparseStep`."""
+        B = code.n_tokens
+        scaled = bool(self.cfg.sparsity_include_decoder_norm)
         if mask is None:
-            tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=x.device)
+            tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=label.device)
         else:
             m = mask.to(torch.float32)
             tok_w = m / m.sum()
         n = None
-        if scaled or want_tanh:
+        if scaled or sparsity_loss_type is not None:
             n = _RowNormDeferred.apply(self.W_D, self._decoder_norm_nograd(), self if defer else None)
-        holder = {"model": self, "code": code, "win": win, "tanh_tok": tanh_tok, "x_op": x_op, "amp": amp, "defer": defer,
-                  "scaled": scaled, "want_tanh": want_tanh, "tanh_c": tanh_c, "l1": l1_coefficient,
-                  "window": float(jr.jumprelu_threshold_window)}
-        loss, recon = _JumpReLUSparseStep.apply(jr.get_jumprelu_threshold(), n, self.W_E, self.b_E, self.W_D,
+        has_theta = self.cfg.act_fn.lower() == "jumprelu"
+        if win is None:
+            win = torch.zeros_like(code.val)
+        holder = {"model": self, "code": code, "win": win, "pen": sparsity_loss_type, "pen_tok": pen_tok, "x_op": x_op, "amp": amp,
+                  "defer": defer, "scaled": scaled, "tanh_c": tanh_c, "l1": l1_coefficient, "window": window, "p": p,
+                  "frequency_scale": frequency_scale, "has_theta": has_theta}
+        loss, recon = _JumpReLUSparseStep.apply(theta, n, self.W_E, self.b_E, self.W_D,
                                                 self.b_D if self.cfg.use_decoder_bias else None,
                                                 label.to(torch.float32).contiguous(), tok_w, holder)
         if not return_aux_data:
             return loss
         b_E = self.b_E.detach()
+        scale = self._decoder_norm_nograd() if scaled else None
+
+        def dense_hidden_pre():
+            h0 = pre_raw.float() + b_E
+            return (h0 * scale) / scale if scale is not None else h0
+
         eager = {"loss": loss, "l_rec": holder["l_rec"], "l_s": holder["l_s"], "l_p": None, "l_aux": None, "label": label,
                  "mask": mask, "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
                  "auxk_coefficient": auxk_coefficient, "sparse_code": code}
         lazy = {"n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
                 "feature_acts": code.to_dense,
-                "hidden_pre": lambda: pre_raw.float() + b_E}
+                "hidden_pre": dense_hidden_pre}
         return LazyDict(eager, lazy)
+
+    @torch.no_grad()
+    def _select_code(self, x: torch.Tensor, amp: bool):
+        """GEMM + TopK / BatchTopK select of an fp32 dictionary -> (x operand, pre, code): what the forward of the fused
+        step does, for the routes that continue from the code with other losses."""
+        w_enc_op = self._w_enc_operand(amp)
+        B, k = x.shape[0], int(self.current_k)
+        batch_wide = self.cfg.act_fn.lower() == "batchtopk"
+        b_E = self.b_E.detach().float()
+        scale = self._decoder_norm_nograd() if self.cfg.sparsity_include_decoder_norm else None
+        gmax = None
+        if amp:
+            x_op = x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.float().contiguous())
+            granule = (getattr(self, "granule_select", True)
+                       and (ops.granule_route_supported(x.shape[1], w_enc_op.shape[0], k) if not batch_wide
+                            else x.shape[1] % 64 == 0 and w_enc_op.shape[0] % 256 == 0))
+            if granule:
+                pre, gmax = ops.encoder_gemm_granule_max(x_op, w_enc_op, b_E, scale)
+            else:
+                pre = ops.encoder_gemm(x_op, w_enc_op, torch.bfloat16)
+        else:
+            x_op = x.float().contiguous()
+            pre = ops.encoder_gemm(x_op, w_enc_op, torch.float32)
+        if batch_wide:
+            code = ops.select_topk_batch(pre, b_E, scale, k * B, granule_max=gmax)
+        else:
+            code = ops.select_topk_row(pre, b_E, scale, k, granule_max=gmax)
+        return x_op, pre, code
+
+    def _flattened_loss(self, batch, x, label, kw):
+        """[batch, seq_len, d_model] activations (models/sae.py:288-345 takes both forms): every loss term is a (masked) mean
+        over all tokens, and BatchTopK flattens the two token axes itself, so the step runs on the [batch * seq_len, .]
+        views and the per-token outputs are given their two axes back."""
+        b, s, d = x.shape
+        mask = batch.get("mask")
+        flat = dict(batch)
+        flat[self.cfg.hook_point_in] = x.reshape(b * s, d)
+        flat[self.cfg.hook_point_out] = label.reshape(b * s, label.shape[-1])
+        if mask is not None:
+            flat["mask"] = mask.reshape(b * s)
+        if self.cfg.hook_point_in == self.cfg.hook_point_out:
+            flat[self.cfg.hook_point_out] = flat[self.cfg.hook_point_in]
+        out = self.compute_loss(flat, **kw)
+        if not kw.get("return_aux_data", True):
+            return out
+
+        def fix(v):
+            if torch.is_tensor(v) and v.ndim >= 1 and v.shape[0] == b * s:
+                return v.reshape(b, s, *v.shape[1:])
+            return v
+
+        if isinstance(out, LazyDict):
+            eager = {k_: fix(v) for k_, v in dict.items(out) if v is not LazyDict._PENDING}
+            lazy = {k_: (lambda f=f: fix(f())) for k_, f in out._lazy.items()}
+            res = LazyDict(eager, lazy)
+        else:
+            res = {k_: fix(v) for k_, v in out.items()}
+        res["label"], res["mask"] = label, mask
+        return res
 
     def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,
                      frequency_scale: float = 0.01, p: int = 1, l1_coefficient: float = 1.0,
@@ -1055,6 +1187,15 @@ class SparseAutoEncoder(SparseDictionary):
                      update_dead_statistics=None, return_aux_data: bool = True, **kwargs):
         x, _, _ = self.prepare_input(batch)
         label = self.prepare_label(batch, **kwargs)
+        if x.ndim == 3 and label.ndim == 3 and x.is_cuda and self._no_hooks():
+            x2, l2 = x.reshape(-1, x.shape[-1]), label.reshape(-1, label.shape[-1])
+            if (self._jumprelu_eligible(x2, l2, sparsity_loss_type, auxk_coefficient)
+                    or self._fused_eligible(x2, l2, sparsity_loss_type, lp_coefficient, auxk_coefficient)):
+                return self._flattened_loss(batch, x, label, dict(
+                    sparsity_loss_type=sparsity_loss_type, tanh_stretch_coefficient=tanh_stretch_coefficient,
+                    frequency_scale=frequency_scale, p=p, l1_coefficient=l1_coefficient, lp_coefficient=lp_coefficient,
+                    auxk_coefficient=auxk_coefficient, k_aux=k_aux, update_dead_statistics=update_dead_statistics,
+                    return_aux_data=return_aux_data, **kwargs))
         if self._jumprelu_eligible(x, label, sparsity_loss_type, auxk_coefficient):
             return self._jumprelu_loss(batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient,
                                        lp_coefficient, auxk_coefficient, return_aux_data, frequency_scale, p)
@@ -1068,6 +1209,17 @@ class SparseAutoEncoder(SparseDictionary):
         mask = batch.get("mask")
         B = x.shape[0]
         amp = _autocast_dtype("cuda") == torch.bfloat16
+        if sparsity_loss_type is not None:
+            # TopK / BatchTopK with a sparsity penalty: select as the plain step does, then decode, loss, penalty and the
+            # backward on the code (the penalty's gradient joins the decoder's at every kept entry and reaches W_D
+            # through the decoder norm)
+            x_op, pre, code = self._select_code(x, amp)
+            defer = bool(self.defer_weight_grads and torch.is_grad_enabled())
+            theta, window = self._threshold_and_window() if self.cfg.act_fn.lower() == "jumprelu" else (
+                torch.zeros(1, dtype=torch.float32, device=x.device), 1.0)
+            return self._sparse_code_loss(batch, label, mask, code, None, x_op, pre, amp, defer, theta, window, sparsity_loss_type,
+                                          None, float(tanh_stretch_coefficient), float(l1_coefficient), float(frequency_scale), p,
+                                          lp_coefficient, auxk_coefficient, return_aux_data)
         if mask is None:
             tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=x.device)
         else:
