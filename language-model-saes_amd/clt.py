@@ -550,6 +550,40 @@ class CrossLayerTranscoder(SparseDictionary):
         return (self.cfg.act_fn.lower() in _TOPK_FAMILY and x.is_cuda and x.ndim == 3 and sparsity_loss_type is None
                 and self.W_E.dtype == torch.float32 and self.cfg.d_model % (64 if amp else 32) == 0)
 
+    # ---- JumpReLU / ReLU: the activation on the threshold kernels, layer by layer ([L, F] thresholds, clt.py:247-257) ----
+    def _threshold_kernels_eligible(self, x, sparsity_loss_type) -> bool:
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        return (self.cfg.act_fn.lower() in ("jumprelu", "relu") and x.is_cuda and x.ndim == 3 and self.W_E.dtype == torch.float32
+                and self.cfg.d_sae % 8 == 0 and self.cfg.d_model % (64 if amp else 32) == 0
+                and sparsity_loss_type in (None, "tanh", "power", "tanh-quad"))
+
+    def _threshold_activations(self, x: torch.Tensor, want_tanh: bool, tanh_c: float):
+        """encode() for a JumpReLU or ReLU transcoder with the element-wise part on `sae_jumprelu_fwd / bwd`: the L encoder
+        products land in one [L, B, F] buffer, and each layer's slice takes one pass that adds the bias, scales by the
+        per-feature decoder norms (constants: the reference computes them without gradient, clt.py:836), applies the
+        layer's thresholds, divides again and, if asked, sums the tanh penalty per token; the backward pass is one kernel
+        per layer as well (pre-activation, bias and threshold gradients).  -> (feature_acts [B, L, F], tanh sums [B, L] or
+        None)."""
+        from .sae import _JumpReLUStep
+
+        L, d, F = self.cfg.n_layers, self.cfg.d_model, self.cfg.d_sae
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        pre = _LayerEncoderGemm.apply(x.to(self.W_E.dtype), self.W_E, self._w_enc_operand(amp), amp).permute(1, 0, 2)   # [L, B, F]
+        scaled = bool(self.cfg.sparsity_include_decoder_norm)
+        norms = self._norm_per_feature_nograd() if (scaled or want_tanh) else None
+        if self.cfg.act_fn.lower() == "jumprelu":
+            theta, window = self.activation_function.get_jumprelu_threshold(), float(self.activation_function.jumprelu_threshold_window)
+        else:
+            theta, window = torch.zeros(L, F, dtype=torch.float32, device=x.device), 1.0
+        acts, pens = [], []
+        for l in range(L):
+            a, t, _ = _JumpReLUStep.apply(pre[l], self.b_E[l], None if norms is None else norms[l], theta[l], scaled, tanh_c, window,
+                                          want_tanh, False)
+            acts.append(a)
+            pens.append(t)
+        feature_acts = torch.stack(acts, dim=1)
+        return feature_acts, (torch.stack(pens, dim=1) if want_tanh else None)
+
     def compute_loss(self, batch, label=None, *, sparsity_loss_type=None, tanh_stretch_coefficient: float = 4.0,
                      frequency_scale: float = 0.01, p: int = 1, l1_coefficient: float = 1.0, return_aux_data: bool = True,
                      **kwargs):
@@ -571,7 +605,11 @@ class CrossLayerTranscoder(SparseDictionary):
             lazy = {"n_tokens": n_tokens, "feature_acts": lambda: holder["code"].to_dense().view(B, L, F)}
             return LazyDict(eager, lazy)
 
-        feature_acts = self.encode(x, **enc_kw)
+        feature_acts = tanh_pen = None
+        if self._threshold_kernels_eligible(x, sparsity_loss_type):
+            feature_acts, tanh_pen = self._threshold_activations(x, sparsity_loss_type == "tanh", float(tanh_stretch_coefficient))
+        else:
+            feature_acts = self.encode(x, **enc_kw)
         reconstructed = self.decode(feature_acts, **dec_kw)
         l_rec = (reconstructed - label).pow(2).sum(dim=-1).mean()
         loss_dict: dict[str, Optional[torch.Tensor]] = {"l_rec": l_rec}
@@ -581,7 +619,7 @@ class CrossLayerTranscoder(SparseDictionary):
             if sparsity_loss_type == "power":
                 l_s = torch.norm(feature_acts * n, p=p, dim=-1)
             elif sparsity_loss_type == "tanh":
-                l_s = torch.tanh(tanh_stretch_coefficient * feature_acts * n).sum(dim=-1)
+                l_s = tanh_pen if tanh_pen is not None else torch.tanh(tanh_stretch_coefficient * feature_acts * n).sum(dim=-1)
             elif sparsity_loss_type == "tanh-quad":
                 t = torch.tanh(tanh_stretch_coefficient * feature_acts * n)
                 freq = t.mean(dim=tuple(range(t.ndim - 1)))

@@ -151,27 +151,34 @@ def test_clt_decode_backward_under_autocast_at_the_benchmark_shape(pkg, dev, rou
     assert rel_err(got_a, want_a) < BF16_TOL
 
 
-def test_clt_generic_loss_with_jumprelu_against_the_oracle(pkg, vo, dev):
-    """A JumpReLU cross-layer transcoder with a tanh penalty takes the generic `compute_loss` (clt.py:1024-1104) built
-    on `encode` and `decode`: loss and every gradient, the [L, F] thresholds' included, against the oracle in fp32; under
-    bf16 autocast the loss at 2e-2 and the decoder gradients on the same activations at 2e-2."""
-    L, d, F, B = 3, 64, 256, 72
-    m, ref, hin, hout = make_clt(pkg, vo, dev, "jumprelu", L, d, F, 4, seed=151)
-    with torch.no_grad():
-        ref.activation_function.log_jumprelu_threshold.add_(1.0)     # thresholds around 2.7: a minority of the entries fire
-    copy_params(m, ref)
+@pytest.mark.parametrize("act_fn", ["jumprelu", "relu"])
+@pytest.mark.parametrize("kw", [dict(sparsity_loss_type="tanh", l1_coefficient=0.3), dict(sparsity_loss_type="power", p=1, l1_coefficient=0.01),
+                                dict(sparsity_loss_type="tanh-quad", l1_coefficient=0.1, frequency_scale=0.05), {}],
+                         ids=["tanh", "l1", "tanh-quad", "mse"])
+def test_clt_threshold_activations_against_the_oracle(pkg, vo, dev, act_fn, kw):
+    """A JumpReLU (thresholds [L, F], clt.py:247-257) or ReLU cross-layer transcoder, with each sparsity penalty
+    (clt.py:1024-1104): the encoder products on the GEMM kernel, the activation and the tanh sums on the threshold
+    kernels layer by layer, the decode as dense products on the GEMM kernel; loss and every gradient, the thresholds'
+    included, against the oracle in fp32; under bf16 autocast the loss at 2e-2 and the decoder gradients on the same
+    activations at 2e-2."""
+    L, d, F, B = 3, 64, 256, 96
+    m, ref, hin, hout = make_clt(pkg, vo, dev, act_fn, L, d, F, 4, seed=151)
+    if act_fn == "jumprelu":
+        with torch.no_grad():
+            ref.activation_function.log_jumprelu_threshold.add_(1.0)     # thresholds around 2.7: a minority of the entries fire
+        copy_params(m, ref)
     batch = clt_batch(L, B, d, seed=152)
     gb = {k_: v.to(dev) for k_, v in batch.items()}
-    kw = dict(sparsity_loss_type="tanh", l1_coefficient=0.3)
     with kernel_names(pkg) as names:
         out = m.compute_loss(gb, **kw)
         out["loss"].backward()
-    assert "encoder_gemm" in names, set(names)
+    assert {"encoder_gemm", "jumprelu_fwd", "jumprelu_bwd"} <= set(names), set(names)
+    assert len(names["encoder_gemm"]) >= 2 * L + L      # L encoder products, L decodes, and their backward products
     want = ref.compute_loss(batch, hin, hout, **kw)
     want["loss"].backward()
     assert torch.equal((out["feature_acts"] != 0).cpu(), want["feature_acts"] != 0)
     density = (want["feature_acts"] != 0).float().mean().item()
-    assert 0.001 < density < 0.5, density
+    assert 0.001 < density < 0.6, density
     assert rel_err(out["loss"], want["loss"]) < FP32_TOL
     assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
     check_param_grads(m, ref, GRAD_TOL)
