@@ -358,41 +358,6 @@ __global__ __launch_bounds__(ATT_THREADS, 3) void attn_fwd_kernel(
   if (q_row < seq && g == 0) lse[((int64_t)b * n_heads + h) * seq + q_row] = (m + __log2f(l)) * 0.6931471805599453f;
 }
 
-// ---- backward: D[b, h, s] = sum_dv dout[t, h, dv] * out[t, h, dv], and the log-sum-exp in the log2 domain ------------
-template <int DV>
-__global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const uint16_t *__restrict__ dout, const uint16_t *__restrict__ out,
-                                                            const float *__restrict__ lse, float *__restrict__ dvec,
-                                                            float *__restrict__ lse2, int seq, int n_heads, int64_t T) {
-  // 16 lanes per (token, head); a lane covers 8 columns per trip
-  const int64_t pair = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
-  const int sub = threadIdx.x & 15;
-  const int64_t n_pairs = T * n_heads;
-  float acc = 0.f;
-  if (pair < n_pairs) {
-    const int64_t t = pair / n_heads;
-    const int h = (int)(pair % n_heads);
-    const int64_t base = t * ((int64_t)n_heads * DV) + (int64_t)h * DV;
-    for (int c = sub * 8; c < DV; c += 128) {
-      const u32x4 a = *reinterpret_cast<const u32x4 *>(dout + base + c), o = *reinterpret_cast<const u32x4 *>(out + base + c);
-      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, ow[4] = {o.x, o.y, o.z, o.w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc = fmaf(__uint_as_float(aw[j] << 16), __uint_as_float(ow[j] << 16), acc);
-        acc = fmaf(__uint_as_float(aw[j] & 0xffff0000u), __uint_as_float(ow[j] & 0xffff0000u), acc);
-      }
-    }
-  }
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (pair < n_pairs && sub == 0) {
-    const int64_t t = pair / n_heads;
-    const int h = (int)(pair % n_heads);
-    const int64_t at = ((t / seq) * n_heads + h) * seq + (t % seq);
-    dvec[at] = acc;
-    lse2[at] = lse[at] * ATT_LOG2E;
-  }
-}
-
 // ---- backward: dV^T and dK^T (one workgroup per 128 keys, a wave per 32) -----------------------------------------------
 // P[q, key] = exp2(sc2 * q . k - lse2[q]) for q >= key.
 // WHAT = 0: dV^T[dv, key] = sum_q dout^T[dv, q] P[q, key].
@@ -524,11 +489,14 @@ __global__ __launch_bounds__(ATT_THREADS, WHAT == 0 ? 3 : 2) void attn_bwd_dkv_k
 
 // ---- backward: dQ^T (one workgroup per 128 queries, a wave per 32) -------------------------------------------------------
 // dQ^T[c, q] = sum_key k^T[c, key] dS[q, key] over key <= q.
+// The kernel also forms, for its own queries, what the other two backward kernels read per query: D = sum_dv dout * out (from
+// the rows it holds anyway: each half of the wave has half of a row) and the log-sum-exp in the log2 domain, written to
+// dvec / lse2 [n_batch, n_heads, seq].  It is therefore launched first.
 template <int DQK, int DV>
 __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
     const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    const uint16_t *__restrict__ dout, const float *__restrict__ lse2, const float *__restrict__ dvec, uint16_t *__restrict__ dqt,
-    int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
+    const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, const float *__restrict__ lse, float *__restrict__ lse2,
+    float *__restrict__ dvec, uint16_t *__restrict__ dqt, int seq, int n_heads, int n_batch, int64_t T, float sc2, float scale) {
   constexpr int KRB = DQK * 2, VRB = DV * 2;
   constexpr int K_BYTES = ATT_STEP * KRB, V_BYTES = ATT_STEP * VRB, BUF = K_BYTES + V_BYTES;
   constexpr int KNL = K_BYTES / 4096, VNL = V_BYTES / 4096;
@@ -544,7 +512,26 @@ __global__ __launch_bounds__(ATT_THREADS, 2) void attn_bwd_dq_kernel(
   att_row_operands<DQK>(qf, q + (tok0 + q_ld) * ldq + h * DQK, g);
   att_row_operands<DV>(dof, dout + (tok0 + q_ld) * ldv + h * DV, g);
   const int64_t at = ((int64_t)b * n_heads + h) * seq + q_ld;
-  const float l2 = lse2[at], dsum = dvec[at];
+  const float l2 = lse[at] * ATT_LOG2E;
+  float dsum = 0.f;
+  {
+    const uint16_t *orow = out + (tok0 + q_ld) * ldv + h * DV;
+#pragma unroll
+    for (int st = 0; st < DV / 16; ++st) {
+      const u32x4 o4 = *reinterpret_cast<const u32x4 *>(orow + st * 16 + g * 8), a4 = __builtin_bit_cast(u32x4, dof[st]);
+      const uint32_t ow[4] = {o4.x, o4.y, o4.z, o4.w}, aw[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        dsum = fmaf(__uint_as_float(aw[j] << 16), __uint_as_float(ow[j] << 16), dsum);
+        dsum = fmaf(__uint_as_float(aw[j] & 0xffff0000u), __uint_as_float(ow[j] & 0xffff0000u), dsum);
+      }
+    }
+    dsum = att_half_sum(dsum);
+    if (q_row < seq && g == 0) {
+      lse2[at] = l2;
+      dvec[at] = dsum;
+    }
+  }
   att_f32x16 dq[DQK / 32];
 #pragma unroll
   for (int n = 0; n < DQK / 32; ++n) dq[n] = att_zero16();
@@ -670,17 +657,15 @@ static int launch_bwd(const void *q, const void *k, const void *v, const void *o
   const dim3 grid((unsigned)(((seq + ATT_OWN - 1) / ATT_OWN) * n_heads * n_batch));
   const float sc2 = (float)(scale * 1.4426950408889634);
   float *dvec = workspace, *lse2 = workspace + n_batch * n_heads * seq;
-  const int64_t prep_blocks = (T * n_heads * 16 + 255) / 256;
-  hipLaunchKernelGGL((attn_bwd_prep_kernel<DV>), dim3((unsigned)prep_blocks), dim3(256), 0, st, (const uint16_t *)dout,
-                     (const uint16_t *)out, lse, dvec, lse2, (int)seq, (int)n_heads, T);
+  // dQ first: it leaves D and the log2-domain log-sum-exp of every query for the two key-side kernels
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
+                     (const uint16_t *)v, (const uint16_t *)out, (const uint16_t *)dout, lse, lse2, dvec, (uint16_t *)dqt, (int)seq,
+                     (int)n_heads, (int)n_batch, T, sc2, (float)scale);
   hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 0>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
                      (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dvt, (int)seq, (int)n_heads,
                      (int)n_batch, T, sc2, (float)scale);
   hipLaunchKernelGGL((attn_bwd_dkv_kernel<DQK, DV, 1>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
                      (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dkt, (int)seq, (int)n_heads,
-                     (int)n_batch, T, sc2, (float)scale);
-  hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV>), grid, dim3(ATT_THREADS), 0, st, (const uint16_t *)q, (const uint16_t *)k,
-                     (const uint16_t *)v, (const uint16_t *)dout, lse2, dvec, (uint16_t *)dqt, (int)seq, (int)n_heads,
                      (int)n_batch, T, sc2, (float)scale);
   return check_launch("attention_bwd");
 }
