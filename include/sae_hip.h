@@ -171,22 +171,26 @@ int sae_encoder_gemm_bias(const void *x_bf16, const void *w_t_bf16, void *out_bf
  *   (x [G, B, d], w_enc_t [G, F, d], pre [G, B, F], b_enc / scale [G, F], granule_max [G, B, F / 64]); the select
  *   then takes all G * B rows at once with rows_per_group = B (0: one group), so that row r uses the bias and scale
  *   of group r / B.
+ * pre_rows (0: as many as rows): the groups may share ONE pre-activation matrix of pre_rows rows, row r then reading
+ *   pre row r % pre_rows (a crosscoder: every head selects from the same summed encoding under its own decoder norms,
+ *   models/crosscoder.py:353-382; the rows are then (head, token) and granule_max [n_heads * B, F / 64] comes from
+ *   sae_granule_max with the same arguments).
  * Together they replace `hidden_pre = x @ W_E + b_E` followed by the TopK of `hidden_pre * decoder_norm`
  * (models/sae.py:324-341, utils/math.py:81-171). */
 int sae_encoder_gemm_granule_max(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups, int64_t B,
                                  int64_t d, int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
                                  void *stream);
 int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
-                                int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val, int64_t *row_off,
-                                int32_t *row_nnz, void *stream);
+                                int64_t B, int64_t F, int k, int64_t rows_per_group, int64_t pre_rows, int32_t *idx, float *val,
+                                int64_t *row_off, int32_t *row_nnz, void *stream);
 /* The two entry points above in the bf16 arithmetic of a dictionary held in bf16 (the keys of sae_select_topk_row_lowp:
  * the sum with the bias and the product with the scale each rounded to bf16; values rounded after the division). */
 int sae_encoder_gemm_granule_max_lowp(const void *x_bf16, const void *w_enc_t_bf16, void *pre_bf16, int64_t n_groups, int64_t B,
                                       int64_t d, int64_t F, const float *b_enc, const float *scale, uint32_t *granule_max,
                                       void *stream);
 int sae_select_topk_row_granule_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc, const float *scale,
-                                     int64_t B, int64_t F, int k, int64_t rows_per_group, int32_t *idx, float *val,
-                                     int64_t *row_off, int32_t *row_nnz, void *stream);
+                                     int64_t B, int64_t F, int k, int64_t rows_per_group, int64_t pre_rows, int32_t *idx,
+                                     float *val, int64_t *row_off, int32_t *row_nnz, void *stream);
 
 /* sae_select_topk_batch (bf16 pre, no feat_mask, F % 256 == 0) with the per-granule key maxima handed in
  * (granule_max [B, F / 64] of sae_encoder_gemm_granule_max for the same pre, b_enc, scale): the select's one pass over
@@ -209,10 +213,11 @@ int sae_select_topk_batch_lowp(const void *pre_bf16, const uint32_t *granule_max
                                int32_t *idx, float *val, int64_t capacity, int64_t *row_off, int32_t *row_nnz,
                                int64_t *total_out, void *workspace, int64_t workspace_bytes, void *stream);
 
-/* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre [B, F] that did not come out of that product
- * (Lorsa's head activations): one streaming read of pre.  rows_per_group as in sae_select_topk_row_granule. */
+/* granule_max [B, F / 64] of sae_encoder_gemm_granule_max for a bf16 pre that did not come out of that product
+ * (Lorsa's head activations), or whose rows are shared by several groups of scales (a crosscoder's heads): one streaming
+ * read per row.  rows_per_group and pre_rows as in sae_select_topk_row_granule (B counts the rows of granule_max). */
 int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F, int64_t rows_per_group,
-                    uint32_t *granule_max, void *stream);
+                    int64_t pre_rows, uint32_t *granule_max, void *stream);
 
 /* Per-layer codes -> one code over L * F features (the cross-layer transcoder's per-layer TopK, models/clt.py:232-387:
  * each layer keeps its own k, the decoders read all layers' entries of a token).  idx / val [L * B * k] and row_nnz

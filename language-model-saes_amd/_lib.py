@@ -32,9 +32,9 @@ SIGNATURES = {
     "sae_encoder_gemm_bias": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P]),
     "sae_encoder_gemm_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P]),
     "sae_encoder_gemm_granule_max_lowp": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P]),
-    "sae_select_topk_row_granule": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _P, _P, _P, _P, _P]),
-    "sae_select_topk_row_granule_lowp": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _P, _P, _P, _P, _P]),
-    "sae_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _P, _P]),
+    "sae_select_topk_row_granule": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _L, _P, _P, _P, _P, _P]),
+    "sae_select_topk_row_granule_lowp": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _L, _P, _P, _P, _P, _P]),
+    "sae_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P]),
     "sae_merge_layer_codes": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_lowp": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),

@@ -57,8 +57,22 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         b_sum = b_E.detach().sum(dim=0)
         codes, recons, grads, dvals = [], [], [], []
         loss = None
+        stacked = None
+        if (amp and pre.dtype == torch.bfloat16 and getattr(m, "granule_select", True) and ops.granule_route_supported(64, F, int(k))):
+            # every head selects from the same summed encoding under its own decoder norms: ONE pass for the per-granule key
+            # maxima of the H * B (head, token) rows and ONE select over them, each row reading only the granules that can
+            # hold a kept entry, instead of H walks over whole rows; the rows come out head after head, which is the stacked
+            # code the backward wants
+            b_rep = b_sum.float().expand(H, F).contiguous()
+            n_rep = norms.contiguous()
+            gmax = ops.granule_max(pre, b_rep, n_rep, rows_per_group=B, n_rows=H * B)
+            stacked = ops.select_topk_row(pre, b_rep, n_rep, k, granule_max=gmax, rows_per_group=B, n_rows=H * B)
         for h in range(H):
-            code = ops.select_topk_row(pre, b_sum, norms[h], k)
+            if stacked is not None:
+                sl, rows = slice(h * B * k, (h + 1) * B * k), slice(h * B, (h + 1) * B)
+                code = ops.SparseCode(stacked.idx[sl], stacked.val[sl], stacked.row_off[rows] - h * B * k, stacked.row_nnz[rows], B, F)
+            else:
+                code = ops.select_topk_row(pre, b_sum, norms[h], k)
             recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(
                 code, w_dec_op[h], b_D.detach()[h].contiguous(), label[:, h].contiguous(), tok_w[:, h].contiguous())
             codes.append(code); recons.append(recon); grads.append(grad_recon); dvals.append(dval)
@@ -66,6 +80,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         recon = torch.stack(recons, dim=1)
         holder["codes"], holder["pre"], holder["norms"], holder["b_sum"] = codes, pre, norms, b_sum
         ctx.codes, ctx.grads, ctx.dvals, ctx.x_op, ctx.w_enc_op = codes, grads, dvals, x_op, w_enc_op
+        ctx.stacked = stacked
         ctx.shape = (B, H, d, F)
         ctx.defer_to = m if holder.get("defer") else None
         ctx.mark_non_differentiable(recon)
@@ -78,7 +93,8 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         m = ctx.defer_to
         defer = (m is not None and all(w.grad is None and getattr(w, "_sparse_grad", None) is None for w in (m.W_E, m.W_D)))
         db_D = [ops.col_sum(ctx.grads[h]) * g for h in range(H)]
-        stacked = reduce(ops.stack_codes, ctx.codes)          # the H codes on a virtual token axis: token h * B + b
+        # the H codes on a virtual token axis: token h * B + b
+        stacked = ctx.stacked if ctx.stacked is not None else reduce(ops.stack_codes, ctx.codes)
         fi = ops.build_feature_index(stacked)
         fi = dataclasses.replace(fi, slot_tok=torch.remainder(fi.slot_tok, B).to(torch.int32))  # virtual token h*B + b -> row b of x
         coef = torch.cat(ctx.dvals) * g

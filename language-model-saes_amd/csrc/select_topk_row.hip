@@ -244,18 +244,20 @@ __global__ __launch_bounds__(SEL_THREADS, 8) void select_topk_row_kernel(
     const void *__restrict__ pre, const float *__restrict__ b_enc, const float *__restrict__ scale,
     const float *__restrict__ fmask, int F, int k,
     int32_t *__restrict__ idx_out, float *__restrict__ val_out, int64_t *__restrict__ row_off,
-    int32_t *__restrict__ row_nnz, int cand_cap, int only_flagged, int rows_per_group) {
+    int32_t *__restrict__ row_nnz, int cand_cap, int only_flagged, int rows_per_group, int pre_rows) {
   __shared__ SelShared sh;
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
+  int src_row = b;
   if (only_flagged) {     // the pass after the granule kernel: the rows it gave up on, with their group's bias / scale
     if (row_nnz[b] != SEL_ROW_FLAG) return;
     const size_t grp = (size_t)(b / rows_per_group);
     if (b_enc) b_enc += grp * F;
     if (scale) scale += grp * F;
+    src_row = b % pre_rows;  // groups that share one matrix of pre_rows rows
   }
   RowReader<BF16, ARITH> rr;
-  rr.row = reinterpret_cast<const char *>(pre) + (size_t)b * F * (BF16 ? 2 : 4);
+  rr.row = reinterpret_cast<const char *>(pre) + (size_t)src_row * F * (BF16 ? 2 : 4);
   rr.b_enc = b_enc;
   rr.scale = scale;
   rr.fmask = fmask;
@@ -462,7 +464,7 @@ namespace sae {
 static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const float *b_enc, const float *scale,
                                 const float *feat_mask, int64_t B, int64_t F, int k, int32_t *idx, float *val,
                                 int64_t *row_off, int32_t *row_nnz, int cand_cap, void *stream, int only_flagged = 0,
-                                int rows_per_group = 1) {
+                                int rows_per_group = 1, int pre_rows = 1) {
   SAE_REQUIRE(pre && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row: null pointer");
   SAE_REQUIRE(B > 0 && F > 0, SAE_ERR_INVALID_ARG, "select_topk_row: B and F must be positive");
   SAE_REQUIRE(pre_dtype == SAE_F32 || pre_dtype == SAE_BF16, SAE_ERR_INVALID_ARG, "select_topk_row: bad dtype %d", pre_dtype);
@@ -477,7 +479,7 @@ static int select_topk_row_impl(bool lowp, const void *pre, int pre_dtype, const
                      (((((uintptr_t)pre) | (uintptr_t)b_enc | (uintptr_t)scale | (uintptr_t)feat_mask) & 15) == 0);
 #define SAE_LAUNCH_SELECT(BF, ST, ...)                                                                                     \
   hipLaunchKernelGGL((select_topk_row_kernel<BF, ST, ##__VA_ARGS__>), dim3((unsigned)B), dim3(SEL_THREADS), 0, st, pre, b_enc, \
-                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged, rows_per_group)
+                     scale, feat_mask, (int)F, k, idx, val, row_off, row_nnz, cand_cap, only_flagged, rows_per_group, pre_rows)
   if (lowp && feat_mask) {
     if (stash) SAE_LAUNCH_SELECT(true, true, SEL_LOWP_MASKED); else SAE_LAUNCH_SELECT(true, false, SEL_LOWP_MASKED);
   } else if (lowp) {
@@ -525,7 +527,7 @@ template <int ARITH>
 __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     const uint16_t *__restrict__ pre, const uint32_t *__restrict__ gmax, const float *__restrict__ b_enc,
     const float *__restrict__ scale, int F, int k, int32_t *__restrict__ idx_out, float *__restrict__ val_out,
-    int64_t *__restrict__ row_off, int32_t *__restrict__ row_nnz, int rows_per_group) {
+    int64_t *__restrict__ row_off, int32_t *__restrict__ row_nnz, int rows_per_group, int pre_rows) {
   __shared__ GsShared sh;
   extern __shared__ __attribute__((aligned(16))) uint32_t gk[];   // the row's granule maxima
   const int b = blockIdx.x, tid = threadIdx.x, ng = F >> 6;
@@ -535,7 +537,7 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
     if (scale) scale += grp * F;
   }
   RowReader<true, ARITH> rr;
-  rr.row = pre + (size_t)b * F;
+  rr.row = pre + (size_t)(b % pre_rows) * F;     // pre_rows < number of rows: the groups share one matrix of pre_rows rows
   rr.b_enc = b_enc;
   rr.scale = scale;
   rr.fmask = nullptr;
@@ -647,7 +649,7 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
 // granules per wave and step.
 __global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__restrict__ pre, const float *__restrict__ b_enc,
                                                           const float *__restrict__ scale, int F, int64_t n_granules,
-                                                          int rows_per_group, uint32_t *__restrict__ gmax) {
+                                                          int rows_per_group, int pre_rows, uint32_t *__restrict__ gmax) {
   const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
   const int part = threadIdx.x & 7, ng = F >> 6;
   uint32_t m = 0u;
@@ -656,7 +658,7 @@ __global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__rest
     const int gi = (int)(g % ng);
     RowReader<true, SEL_PLAIN> rr;
     const size_t grp = (size_t)(row / rows_per_group);
-    rr.row = pre + (size_t)row * F;
+    rr.row = pre + (size_t)(row % pre_rows) * F;
     rr.b_enc = b_enc ? b_enc + grp * F : nullptr;
     rr.scale = scale ? scale + grp * F : nullptr;
     rr.fmask = nullptr;
@@ -678,11 +680,14 @@ __global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__rest
 
 namespace sae {
 static int select_topk_row_granule_impl(bool lowp, const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
-                                        const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                        const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group, int64_t pre_rows,
                                         int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
   SAE_REQUIRE(pre_bf16 && granule_max && idx && val && row_off && row_nnz, SAE_ERR_INVALID_ARG, "select_topk_row_granule: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31), SAE_ERR_INVALID_ARG, "select_topk_row_granule: bad sizes");
   if (rows_per_group <= 0) rows_per_group = B;
+  if (pre_rows <= 0) pre_rows = B;
+  SAE_REQUIRE(pre_rows <= B && B % pre_rows == 0, SAE_ERR_INVALID_ARG, "select_topk_row_granule: B=%lld is not a multiple of pre_rows=%lld",
+              (long long)B, (long long)pre_rows);
   SAE_REQUIRE(B % rows_per_group == 0, SAE_ERR_INVALID_ARG, "select_topk_row_granule: B=%lld is not a multiple of rows_per_group=%lld",
               (long long)B, (long long)rows_per_group);
   SAE_REQUIRE(F % 64 == 0 && F / 64 <= GS_MAX_GRANULES, SAE_ERR_UNSUPPORTED,
@@ -693,30 +698,32 @@ static int select_topk_row_granule_impl(bool lowp, const void *pre_bf16, const u
   hipStream_t st = (hipStream_t)stream;
   if (lowp)
     hipLaunchKernelGGL(select_topk_row_granule_kernel<SEL_LOWP>, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
-                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
+                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group,
+                       (int)pre_rows);
   else
     hipLaunchKernelGGL(select_topk_row_granule_kernel<SEL_PLAIN>, dim3((unsigned)B), dim3(GS_THREADS), (size_t)(F / 64) * 4, st,
-                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group);
+                       (const uint16_t *)pre_bf16, granule_max, b_enc, scale, (int)F, k, idx, val, row_off, row_nnz, (int)rows_per_group,
+                       (int)pre_rows);
   const int rc = check_launch("select_topk_row_granule");
   if (rc != SAE_OK) return rc;
   // rows the granule kernel flagged (mass ties) are redone from the whole row; every other workgroup leaves at once
   return select_topk_row_impl(lowp, pre_bf16, SAE_BF16, b_enc, scale, nullptr, B, F, k, idx, val, row_off, row_nnz, SEL_CAP, stream, 1,
-                              (int)rows_per_group);
+                              (int)rows_per_group, (int)pre_rows);
 }
 }  // namespace sae
 
 extern "C" int sae_select_topk_row_granule(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
-                                           const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                           const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group, int64_t pre_rows,
                                            int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
-  return sae::select_topk_row_granule_impl(false, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, idx, val, row_off,
-                                           row_nnz, stream);
+  return sae::select_topk_row_granule_impl(false, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, pre_rows, idx, val,
+                                           row_off, row_nnz, stream);
 }
 
 extern "C" int sae_select_topk_row_granule_lowp(const void *pre_bf16, const uint32_t *granule_max, const float *b_enc,
-                                                const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group,
+                                                const float *scale, int64_t B, int64_t F, int k, int64_t rows_per_group, int64_t pre_rows,
                                                 int32_t *idx, float *val, int64_t *row_off, int32_t *row_nnz, void *stream) {
-  return sae::select_topk_row_granule_impl(true, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, idx, val, row_off,
-                                           row_nnz, stream);
+  return sae::select_topk_row_granule_impl(true, pre_bf16, granule_max, b_enc, scale, B, F, k, rows_per_group, pre_rows, idx, val,
+                                           row_off, row_nnz, stream);
 }
 
 extern "C" int sae_select_topk_row_ex(const void *pre, int pre_dtype, const float *b_enc, const float *scale,
@@ -740,7 +747,7 @@ extern "C" int sae_select_topk_row(const void *pre, int pre_dtype, const float *
 }
 
 extern "C" int sae_granule_max(const void *pre_bf16, const float *b_enc, const float *scale, int64_t B, int64_t F,
-                               int64_t rows_per_group, uint32_t *granule_max, void *stream) {
+                               int64_t rows_per_group, int64_t pre_rows, uint32_t *granule_max, void *stream) {
   using namespace sae;
   SAE_REQUIRE(pre_bf16 && granule_max, SAE_ERR_INVALID_ARG, "granule_max: null pointer");
   SAE_REQUIRE(B > 0 && F > 0 && B < (1LL << 31) && F < (1LL << 31), SAE_ERR_INVALID_ARG, "granule_max: bad sizes");
@@ -748,11 +755,14 @@ extern "C" int sae_granule_max(const void *pre_bf16, const float *b_enc, const f
   if (rows_per_group <= 0) rows_per_group = B;
   SAE_REQUIRE(B % rows_per_group == 0, SAE_ERR_INVALID_ARG, "granule_max: B=%lld is not a multiple of rows_per_group=%lld",
               (long long)B, (long long)rows_per_group);
+  if (pre_rows <= 0) pre_rows = B;
+  SAE_REQUIRE(pre_rows <= B && B % pre_rows == 0, SAE_ERR_INVALID_ARG, "granule_max: B=%lld is not a multiple of pre_rows=%lld",
+              (long long)B, (long long)pre_rows);
   SAE_REQUIRE((((uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0, SAE_ERR_INVALID_ARG,
               "granule_max: pointers must be 16-byte aligned");
   const int64_t n = B * (F / 64);
   SAE_REQUIRE((n * 8 + 255) / 256 < (1LL << 31), SAE_ERR_UNSUPPORTED, "granule_max: too large");
   hipLaunchKernelGGL(granule_max_kernel, dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t *)pre_bf16, b_enc, scale, (int)F, n, (int)rows_per_group, granule_max);
+                     (const uint16_t *)pre_bf16, b_enc, scale, (int)F, n, (int)rows_per_group, (int)pre_rows, granule_max);
   return check_launch("granule_max");
 }

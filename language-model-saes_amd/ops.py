@@ -443,19 +443,25 @@ def encoder_gemm_granule_max(x: torch.Tensor, w_enc_t: torch.Tensor, b_enc: Opti
     return pre, gmax
 
 
-def granule_max(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], rows_per_group: int = 0) -> torch.Tensor:
-    """The granule maxima `encoder_gemm_granule_max` leaves, for a bf16 pre [B, F] from elsewhere."""
+def granule_max(pre: torch.Tensor, b_enc: Optional[torch.Tensor], scale: Optional[torch.Tensor], rows_per_group: int = 0,
+                n_rows: Optional[int] = None) -> torch.Tensor:
+    """The granule maxima `encoder_gemm_granule_max` leaves, for a bf16 pre [B, F] from elsewhere.  `n_rows` (a multiple of
+    B) > B: the maxima of n_rows virtual rows that share pre's B rows (row r reads pre row r % B) under the bias / scale
+    vector of their group r / rows_per_group."""
     _req(pre, "pre", torch.bfloat16, 2)
     B, F = pre.shape
-    n_vec = F * (B // rows_per_group if rows_per_group else 1)
+    rows = B if n_rows is None else int(n_rows)
+    if rows % B:
+        raise ValueError(f"n_rows = {rows} is not a multiple of pre's {B} rows")
+    n_vec = F * (rows // rows_per_group if rows_per_group else 1)
     for name, t in (("b_enc", b_enc), ("scale", scale)):
         if t is not None:
             _req(t, name, torch.float32)
             if t.numel() != n_vec:
                 raise ValueError(f"{name} must have {n_vec} elements")
-    gmax = torch.empty(B, max(F // GRANULE, 1), dtype=torch.int32, device=pre.device)
+    gmax = torch.empty(rows, max(F // GRANULE, 1), dtype=torch.int32, device=pre.device)
     with _timed("granule_max"):
-        check(_lib.load().sae_granule_max(pre.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, int(rows_per_group), gmax.data_ptr(),
+        check(_lib.load().sae_granule_max(pre.data_ptr(), _ptr(b_enc), _ptr(scale), rows, F, int(rows_per_group), B, gmax.data_ptr(),
                                           _stream(pre)), "granule_max")
     return gmax
 
@@ -516,15 +522,21 @@ def select_topk_row(
     lowp: bool = False,
     granule_max: Optional[torch.Tensor] = None,
     rows_per_group: int = 0,
+    n_rows: Optional[int] = None,
 ) -> SparseCode:
     """Per-token TopK of (pre + b_enc) * scale.  `lowp`: bf16 `pre`, every intermediate rounded to bf16 (the
     arithmetic of a dictionary whose parameters are bf16 tensors).  `feat_mask` (0/1 per feature): the aux-k selection
     among the masked-in features, with the reference's key arithmetic for it.  `granule_max`: the second output of
     `encoder_gemm_granule_max` for the same pre, b_enc and scale; the row is then read only where a kept element
-    can be (same result).  On that route `rows_per_group` > 0 says that pre stacks groups of that many rows and that
-    b_enc / scale hold one vector of F per group."""
+    can be (same result).  On that route `rows_per_group` > 0 says that the rows come in groups of that many and that
+    b_enc / scale hold one vector of F per group; `n_rows` (a multiple of pre's row count) > that count says that the
+    groups share pre's rows (row r of the code reads pre row r % pre.shape[0]: a crosscoder's heads over one summed
+    encoding), granule_max then being `granule_max(pre, ..., n_rows=n_rows)`."""
     _req(pre, "pre", ndim=2)
-    B, F = pre.shape
+    pre_rows, F = pre.shape
+    B = pre_rows if n_rows is None else int(n_rows)
+    if B % pre_rows or (B != pre_rows and granule_max is None):
+        raise ValueError("n_rows needs the granule route and must be a multiple of pre's row count")
     n_vec = F * (B // rows_per_group if rows_per_group else 1)
     if rows_per_group and (granule_max is None or B % rows_per_group):
         raise ValueError("rows_per_group needs the granule route and must divide the number of rows")
@@ -553,8 +565,8 @@ def select_topk_row(
     _t.__enter__()
     if granule_max is not None:
         fn = lib.sae_select_topk_row_granule_lowp if lowp else lib.sae_select_topk_row_granule
-        rc = fn(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, int(rows_per_group), idx.data_ptr(),
-                val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
+        rc = fn(pre.data_ptr(), granule_max.data_ptr(), _ptr(b_enc), _ptr(scale), B, F, k, int(rows_per_group), pre_rows,
+                idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))
     elif lowp:
         rc = lib.sae_select_topk_row_lowp(pre.data_ptr(), _ptr(b_enc), _ptr(scale), _ptr(feat_mask), B, F, k, idx.data_ptr(),
                                           val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(), _stream(pre))

@@ -235,3 +235,25 @@ def test_batch_select_with_granule_maxima_equals_batch_select(pkg, dev, B, d, F,
     every = pkg.ops.select_topk_batch(pre, b, s, B * F, granule_max=gmax)
     ref = pkg.ops.select_topk_batch(pre, b, s, B * F)
     assert torch.equal(every.row_nnz, ref.row_nnz) and torch.equal(every.idx, ref.idx) and torch.equal(every.val, ref.val)
+
+
+@pytest.mark.parametrize("H,B,F,k", [(3, 70, 1024, 8), (4, 128, 4096, 32), (2, 33, 512, 64)])
+def test_groups_of_scales_over_one_shared_matrix(pkg, dev, H, B, F, k):
+    """`n_rows = H * B`: H groups of rows share ONE pre-activation matrix [B, F], each group selecting under a bias / scale
+    vector of its own (a crosscoder's heads).  The maxima equal those of the explicitly repeated matrix, and the one stacked
+    select equals, bit for bit, H selects of the row kernel."""
+    print(f"shared-matrix select H={H} B={B} F={F} k={k}", flush=True)
+    g = torch.Generator().manual_seed(H * 1000 + F + k)
+    pre = torch.randn(B, F, generator=g).bfloat16().to(dev)
+    bias = (0.1 * torch.randn(H, F, generator=g)).to(dev)
+    scale = (0.25 + 1.5 * torch.rand(H, F, generator=g)).to(dev)
+    gmax = pkg.ops.granule_max(pre, bias, scale, rows_per_group=B, n_rows=H * B)
+    want_gmax = pkg.ops.granule_max(pre.repeat(H, 1), bias, scale, rows_per_group=B)
+    assert torch.equal(gmax, want_gmax)
+    code = pkg.ops.select_topk_row(pre, bias, scale, k, granule_max=gmax, rows_per_group=B, n_rows=H * B)
+    assert code.n_tokens == H * B
+    for h in range(H):
+        want = pkg.ops.select_topk_row(pre, bias[h].contiguous(), scale[h].contiguous(), k)
+        sl, rows = slice(h * B * k, (h + 1) * B * k), slice(h * B, (h + 1) * B)
+        assert torch.equal(code.idx[sl], want.idx) and torch.equal(code.val[sl], want.val)
+        assert torch.equal(code.row_nnz[rows], want.row_nnz) and torch.equal(code.row_off[rows] - h * B * k, want.row_off)

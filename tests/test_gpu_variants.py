@@ -250,6 +250,33 @@ def crosscoder_bf16_step(pkg, vo, dev, H, d, F, k, B, seed):
     check_bf16_grads_on_the_kernels_selection(m, ref, lambda: ref.compute_loss(batch, hooks), acts > 0)
 
 
+def test_crosscoder_select_over_all_heads_equals_the_per_head_selects(pkg, vo, dev):
+    """Under autocast the fused crosscoder step forms the granule maxima of all (head, token) rows in one pass and selects
+    them in one launch; with `granule_select` off it runs one row select per head.  Same codes, losses and gradients."""
+    H, d, F, k, B = 3, 64, 1024, 16, 128
+    results = []
+    for granule in (True, False):
+        m, _, hooks = make_crosscoder(pkg, vo, dev, H, d, F, k, seed=37)
+        m.granule_select = granule
+        g = torch.Generator().manual_seed(38)
+        gb = {h: torch.randn(B, d, generator=g).to(dev) for h in hooks}
+        gb["tokens"] = torch.zeros(B, dtype=torch.long, device=dev)
+        timer = pkg.ops.KernelTimer()
+        pkg.ops.set_kernel_timer(timer)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = m.compute_loss(gb)
+        out["loss"].backward()
+        torch.cuda.synchronize()
+        pkg.ops.set_kernel_timer(None)
+        assert ("select_topk_row[granule]" in timer.records) == granule and ("granule_max" in timer.records) == granule
+        results.append((out["loss"].detach().clone(), [c.idx.clone() for c in out["sparse_codes"]], [c.val.clone() for c in out["sparse_codes"]],
+                        {n: p.grad.clone() for n, p in m.named_parameters()}))
+    (la, ia, va, ga), (lb, ib, vb, gb_) = results
+    assert torch.equal(la, lb)
+    assert all(torch.equal(x, y) for x, y in zip(ia, ib)) and all(torch.equal(x, y) for x, y in zip(va, vb))
+    assert all(torch.equal(ga[n], gb_[n]) for n in ga)
+
+
 # ---- CLT -----------------------------------------------------------------------------------------
 
 def make_clt(pkg, vo, dev, act_fn, L, d, F, k, seed, include_norm=True):
