@@ -191,7 +191,11 @@ class _SparseTail(torch.autograd.Function):
         scale = m._decoder_norm_nograd() if m.cfg.sparsity_include_decoder_norm else None
         hp = hidden_pre if hidden_pre.dtype in (torch.float32, torch.bfloat16) else hidden_pre.float()
         hp = hp.contiguous()
-        if hp.dtype == torch.bfloat16 and getattr(m, "granule_select", True) and ops.granule_route_supported(64, hp.shape[1], int(k)):
+        if m.cfg.act_fn.lower() == "batchtopk":
+            # the k * tokens largest over every token of the batch (the reference flattens batch and context first,
+            # models/sparse_dictionary.py:769-792)
+            code = ops.select_topk_batch(hp, None, scale, int(k) * hp.shape[0])
+        elif hp.dtype == torch.bfloat16 and getattr(m, "granule_select", True) and ops.granule_route_supported(64, hp.shape[1], int(k)):
             # short rows: one streaming pass for the per-granule key maxima, then a select that reads a row only where a
             # kept entry can be, instead of one 1024-thread workgroup walking every row twice
             code = ops.select_topk_row(hp, None, scale, k, granule_max=ops.granule_max(hp, None, scale))
@@ -646,7 +650,7 @@ class LowRankSparseAttention(SparseDictionary):
         return any(h.has_hooks for h in (self.hook_hidden_pre, self.hook_feature_acts, self.hook_reconstructed))
 
     def _fused_eligible(self, x, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
-        return (self.cfg.act_fn.lower() == "topk" and x.is_cuda and x.ndim == 3 and sparsity_loss_type is None
+        return (self.cfg.act_fn.lower() in ("topk", "batchtopk") and x.is_cuda and x.ndim == 3 and sparsity_loss_type is None
                 and not (lp_coefficient > 0.0) and not (auxk_coefficient > 0.0) and not self._has_hooks()
                 and self.W_O.dtype == torch.float32 and self.cfg.d_model % 8 == 0)
 

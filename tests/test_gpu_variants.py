@@ -458,9 +458,9 @@ def test_clt_granule_route_changes_nothing(pkg, vo, dev):
 
 # ---- Lorsa ---------------------------------------------------------------------------------------
 
-def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, **kw):
+def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, act_fn="topk", **kw):
     okw = {k_: v for k_, v in kw.items() if k_ != "normalization_type"}   # the oracle's query / key norm is the RMS one
-    ref = vo.init_uniform_(vo.LorsaOracle(d_model=d, d_sae=F, n_qk_heads=h, d_qk_head=dq, n_ctx=n_ctx, act_fn="topk", top_k=k,
+    ref = vo.init_uniform_(vo.LorsaOracle(d_model=d, d_sae=F, n_qk_heads=h, d_qk_head=dq, n_ctx=n_ctx, act_fn=act_fn, top_k=k,
                                           **okw), seed=seed, bound=0.3)
     with torch.no_grad():
         g = torch.Generator().manual_seed(seed + 7)
@@ -468,7 +468,7 @@ def make_lorsa(pkg, vo, dev, d, F, h, dq, n_ctx, k, seed, **kw):
     ckw = dict(kw)
     ckw.setdefault("rotary_dim", dq)
     cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
-                          d_qk_head=dq, n_ctx=n_ctx, act_fn="topk", top_k=k, norm_activation="inference", device="cuda",
+                          d_qk_head=dq, n_ctx=n_ctx, act_fn=act_fn, top_k=k, norm_activation="inference", device="cuda",
                           dtype=torch.float32, **ckw)
     m = pkg.LowRankSparseAttention(cfg)
     copy_params(m, ref)
@@ -528,9 +528,32 @@ def test_lorsa_bf16_step_with_other_query_key_forms_runs_the_attention_kernels(p
     assert "attention_bwd" in timer.records and "rotary_fwd" not in timer.records
 
 
-def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, seed=53, **kw):
+@pytest.mark.parametrize("amp", [False, True])
+def test_lorsa_fused_step_with_batchtopk(pkg, vo, dev, amp):
+    """BatchTopK over every token of the batch (k * tokens entries in all, rows of unequal length) on the same tail."""
+    d, F, h, dq, s, b, k = 64, 256, 4, 32, 32, 3, 8
+    if amp:
+        timer = lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, 2, True, act_fn="batchtopk", positional_embedding_type="none")
+        assert "select_topk_batch" in timer.records and "select_topk_row" not in timer.records
+        return
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=57, act_fn="batchtopk", positional_embedding_type="none")
+    g = torch.Generator().manual_seed(58)
+    batch = {"in": torch.randn(b, s, d, generator=g), "out": torch.randn(b, s, d, generator=g), "tokens": torch.zeros(b, s)}
+    out = m.compute_loss({k_: v.to(dev) for k_, v in batch.items()})
+    assert "sparse_code" in out, "the kernel path did not run"
+    want = ref.compute_loss(batch)
+    kept = (out["feature_acts"] > 0).cpu()
+    assert torch.equal(kept, want["feature_acts"] > 0) and int(kept.sum()) == k * b * s
+    assert len(set(kept.flatten(0, 1).sum(-1).tolist())) > 1, "rows of equal length: not a batch-wide selection"
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < FP32_TOL
+    assert rel_err(out["loss"], want["loss"]) < FP32_TOL
+    out["loss"].backward(); want["loss"].backward()
+    check_grads(m, ref)
+
+
+def lorsa_bf16_step(pkg, vo, dev, d, F, h, dq, s, b, dense, seed=53, act_fn="topk", **kw):
     k = 8
-    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=seed, **kw)
+    m, ref = make_lorsa(pkg, vo, dev, d, F, h, dq, s, k, seed=seed, act_fn=act_fn, **kw)
     m.dense_decoder_grad = dense
     g = torch.Generator().manual_seed(seed + 1)
     with torch.no_grad():      # non-zero projection biases, so that the kernels' bias path is exercised
