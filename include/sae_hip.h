@@ -228,6 +228,16 @@ int sae_merge_layer_codes(const int32_t *idx, const float *val, const int32_t *r
                           int64_t F, int32_t *out_idx, float *out_val, int64_t *out_row_off, int32_t *out_row_nnz,
                           int32_t *layer_cnt, void *stream);
 
+/* Codes of G groups over the same tokens and features -> one code holding every (token, feature) once (a crosscoder's
+ * heads select from one summed encoding, models/crosscoder.py:246-305, so d loss / d pre[b, f] is the sum of the heads'
+ * value gradients at (b, f) and the encoder's gradient rows need each pair once).  idx / val [G * B * k] and row_nnz
+ * [G * B] are one stacked select's outputs (row g * B + b: group g, token b; slots row * k ..).  out_idx / out_val
+ * [B * G * k], out_row_off / out_row_nnz [B]: token b's distinct features in slots b * G * k .., in order of first
+ * appearance, each with the sum of its values over the token's rows (added in group order); unused slots zeroed.
+ * G * k <= 1024. */
+int sae_union_group_codes(const int32_t *idx, const float *val, const int32_t *row_nnz, int64_t G, int64_t B, int64_t k,
+                          int32_t *out_idx, float *out_val, int64_t *out_row_off, int32_t *out_row_nnz, void *stream);
+
 /* Batch-global TopK (BatchTopK): keep the k_total largest h1 > 0 over the whole [B, F] batch
  * (h0, h1 as above); ties at the threshold -> lowest flattened index b * F + f.  If fewer than
  * k_total entries are positive, all positives are kept.

@@ -36,6 +36,7 @@ SIGNATURES = {
     "sae_select_topk_row_granule_lowp": (_I, [_P, _P, _P, _P, _L, _L, _I, _L, _L, _P, _P, _P, _P, _P]),
     "sae_granule_max": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P]),
     "sae_merge_layer_codes": (_I, [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P]),
+    "sae_union_group_codes": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_lowp": (_I, [_P, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _P]),
     "sae_select_topk_row_ex": (_I, [_P, _I, _P, _P, _P, _L, _L, _I, _P, _P, _P, _P, _I, _P]),
     "sae_select_topk_batch_workspace_bytes": (_L, [_L, _L]),

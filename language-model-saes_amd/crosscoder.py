@@ -81,6 +81,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         holder["codes"], holder["pre"], holder["norms"], holder["b_sum"] = codes, pre, norms, b_sum
         ctx.codes, ctx.grads, ctx.dvals, ctx.x_op, ctx.w_enc_op = codes, grads, dvals, x_op, w_enc_op
         ctx.stacked = stacked
+        ctx.amp = bool(amp)
         ctx.shape = (B, H, d, F)
         ctx.defer_to = m if holder.get("defer") else None
         ctx.mark_non_differentiable(recon)
@@ -95,16 +96,32 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         db_D = [ops.col_sum(ctx.grads[h]) * g for h in range(H)]
         # the H codes on a virtual token axis: token h * B + b
         stacked = ctx.stacked if ctx.stacked is not None else reduce(ops.stack_codes, ctx.codes)
-        fi = ops.build_feature_index(stacked)
-        fi = dataclasses.replace(fi, slot_tok=torch.remainder(fi.slot_tok, B).to(torch.int32))  # virtual token h*B + b -> row b of x
         coef = torch.cat(ctx.dvals) * g
+        k = stacked.idx.numel() // (H * B)
+        if stacked.idx.numel() == H * B * k and H * k <= 1024:
+            # the heads keep nearly the same features of a token (one encoding, H sets of norms): every (token, feature) once,
+            # with the heads' value gradients summed, so that the encoder's gradient rows gather a row of x once per pair
+            # instead of once per head
+            merged = ops.union_group_codes(dataclasses.replace(stacked, val=coef), H)
+            fi, coef = ops.build_feature_index(merged), merged.val
+        else:
+            fi = ops.build_feature_index(stacked)
+            fi = dataclasses.replace(fi, slot_tok=torch.remainder(fi.slot_tok, B).to(torch.int32))  # virtual token h*B + b -> row b of x
+        if ctx.amp:
+            # the decoder's weight gradient pairs the activations with the bf16-rounded output gradient, as the backward of
+            # an autocast product does; the gathered rows then move half the bytes
+            gd = torch.empty(H * B, d, dtype=torch.bfloat16, device=stacked.val.device)
+            for h in range(H):
+                ops.cast_bf16(ctx.grads[h], gd[h * B:(h + 1) * B])
+        else:
+            gd = torch.cat(ctx.grads)
         if defer:
             # The optimiser rebuilds the rows where it consumes them; nothing dense is written here.  The decoder
             # [H, F, d] is one matrix of H F rows: head h's code addresses rows h F .. (h + 1) F of it, and its dense
             # operand is head h's block of the stacked output gradients.
             idx_cat = torch.cat([c.idx + h * F for h, c in enumerate(ctx.codes)])
             cat_code = dataclasses.replace(stacked, idx=idx_cat, d_sae=H * F)
-            m.W_D._sparse_grad = SparseRowGrad(ops.build_feature_index(cat_code), stacked.val * g, torch.cat(ctx.grads), H * F)
+            m.W_D._sparse_grad = SparseRowGrad(ops.build_feature_index(cat_code), stacked.val * g, gd, H * F)
             m.W_E._sparse_grad = SparseRowGrad(fi, coef, ctx.x_op, F)
             db_sum, _ = ops.feature_segment_sums(fi, coef)
             dW_E = dW_D = None
@@ -112,7 +129,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
             dW_D = []
             for h in range(H):
                 fi_h = ops.build_feature_index(ctx.codes[h])
-                rows, _ = ops.sparse_grad_rows(fi_h, ctx.codes[h].val * g, ctx.grads[h], F)
+                rows, _ = ops.sparse_grad_rows(fi_h, ctx.codes[h].val * g, gd[h * B:(h + 1) * B], F)
                 dW_D.append(rows)
             dW_D = torch.stack(dW_D)
             dW_Et, db_sum = ops.sparse_grad_rows(fi, coef, ctx.x_op, F, want_bias=True)                # [F, H*d], [F]

@@ -143,6 +143,58 @@ __global__ __launch_bounds__(256) void merge_layer_codes_kernel(const int32_t *_
   if (s == 0) { out_row_off[b] = (int64_t)base; out_row_nnz[b] = total; }
 }
 
+
+// Codes of G groups over the same tokens and features, stacked group after group (row g * B + b: group g, token b, at most k
+// entries in slots [row * k, row * k + row_nnz)) -> one code with every (token, feature) once: token b's entries are the
+// distinct features of its G rows, in order of first appearance (group 0's entries first), each with the sum of the values
+// that feature carries in the token's rows, added in group order.  One wave per token; the token's G * k entries sit in
+// LDS and every entry is compared with all of them (G * k <= 1024: at most 16 passes of 1024 broadcast reads per lane).
+constexpr int UNION_MAX = 1024;
+__global__ __launch_bounds__(256) void union_group_codes_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
+                                                                const int32_t *__restrict__ row_nnz, int G, int B, int k,
+                                                                int32_t *__restrict__ out_idx, float *__restrict__ out_val,
+                                                                int64_t *__restrict__ out_row_off, int32_t *__restrict__ out_row_nnz) {
+  __shared__ int32_t s_idx[4][UNION_MAX];
+  __shared__ float s_val[4][UNION_MAX];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int b = blockIdx.x * 4 + wave;
+  const int per_tok = b < B ? G * k : 0;   // a wave past the last token does nothing but meet the barrier
+  int32_t *si = s_idx[wave];
+  float *sv = s_val[wave];
+  // slot s = g * k + j holds group g's j-th entry, or feature -1 past that row's entries
+  for (int s = lane; s < per_tok; s += 64) {
+    const int g = s / k, j = s - g * k;
+    const size_t row = (size_t)g * B + b;
+    const bool live = j < row_nnz[row];
+    si[s] = live ? idx[row * k + j] : -1;
+    sv[s] = live ? val[row * k + j] : 0.f;
+  }
+  __syncthreads();
+  if (b >= B) return;
+  const size_t base = (size_t)b * per_tok;
+  int written = 0;
+  for (int s0 = 0; s0 < per_tok; s0 += 64) {
+    const int s = s0 + lane;
+    const int mine = s < per_tok ? si[s] : -1;
+    float sum = 0.f;
+    bool first = mine >= 0;
+    for (int q = 0; q < per_tok; ++q) {
+      const bool same = si[q] == mine;
+      sum += same ? sv[q] : 0.f;
+      first = first && !(same && q < s);
+    }
+    const unsigned long long keep = __ballot(first);
+    if (first) {
+      const int pos = written + __popcll(keep & ((1ull << lane) - 1ull));
+      out_idx[base + pos] = mine;
+      out_val[base + pos] = sum;
+    }
+    written += __popcll(keep);
+  }
+  for (int s = written + lane; s < per_tok; s += 64) { out_idx[base + s] = 0; out_val[base + s] = 0.f; }
+  if (lane == 0) { out_row_off[b] = (int64_t)base; out_row_nnz[b] = written; }
+}
+
 }  // namespace sae
 
 extern "C" int sae_dense_row_nnz(const void *dense, int dtype, int64_t B, int64_t F, int32_t *row_nnz, void *stream) {
@@ -184,4 +236,17 @@ extern "C" int sae_merge_layer_codes(const int32_t *idx, const float *val, const
   hipLaunchKernelGGL(merge_layer_codes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, idx, val, row_nnz,
                      (int)L, (int)B, (int)k, (int)F, out_idx, out_val, out_row_off, out_row_nnz, layer_cnt);
   return check_launch("merge_layer_codes");
+}
+
+extern "C" int sae_union_group_codes(const int32_t *idx, const float *val, const int32_t *row_nnz, int64_t G, int64_t B, int64_t k,
+                                     int32_t *out_idx, float *out_val, int64_t *out_row_off, int32_t *out_row_nnz, void *stream) {
+  using namespace sae;
+  SAE_REQUIRE(idx && val && row_nnz && out_idx && out_val && out_row_off && out_row_nnz, SAE_ERR_INVALID_ARG,
+              "union_group_codes: null pointer");
+  SAE_REQUIRE(G > 0 && B > 0 && k > 0, SAE_ERR_INVALID_ARG, "union_group_codes: sizes must be positive");
+  SAE_REQUIRE(G * k <= UNION_MAX, SAE_ERR_UNSUPPORTED, "union_group_codes: more than 1024 entries per token");
+  SAE_REQUIRE(B < ((int64_t)1 << 31) && G * B < ((int64_t)1 << 31), SAE_ERR_UNSUPPORTED, "union_group_codes: too many rows");
+  hipLaunchKernelGGL(union_group_codes_kernel, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, (hipStream_t)stream, idx, val, row_nnz,
+                     (int)G, (int)B, (int)k, out_idx, out_val, out_row_off, out_row_nnz);
+  return check_launch("union_group_codes");
 }

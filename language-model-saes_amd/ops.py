@@ -510,6 +510,28 @@ def merge_layer_codes(code: SparseCode, L: int) -> Tuple[SparseCode, torch.Tenso
     return SparseCode(idx, val, row_off, row_nnz, B, L * F), layer_cnt
 
 
+def union_group_codes(code: SparseCode, groups: int) -> SparseCode:
+    """`code`: one select over groups * B stacked rows (row g * B + b, at most k entries each) -> the code over the B tokens
+    that holds every (token, feature) once, with the sum of the values it carries in the token's rows; groups * k slots per
+    token, distinct features in order of first appearance."""
+    rows = code.n_tokens
+    if rows % groups:
+        raise ValueError(f"{rows} rows are not {groups} groups of equally many tokens")
+    B, k = rows // groups, code.idx.numel() // rows
+    if code.idx.numel() != rows * k or groups * k > 1024:
+        raise ValueError("union_group_codes takes rows of equally many slots, at most 1024 per token in all")
+    dev = code.idx.device
+    idx = torch.empty(B * groups * k, dtype=torch.int32, device=dev)
+    val = torch.empty(B * groups * k, dtype=torch.float32, device=dev)
+    row_off = torch.empty(B, dtype=torch.int64, device=dev)
+    row_nnz = torch.empty(B, dtype=torch.int32, device=dev)
+    with _timed("union_group_codes"):
+        check(_lib.load().sae_union_group_codes(code.idx.data_ptr(), code.val.data_ptr(), code.row_nnz.data_ptr(), groups, B, k,
+                                                idx.data_ptr(), val.data_ptr(), row_off.data_ptr(), row_nnz.data_ptr(),
+                                                _stream(code.idx)), "union_group_codes")
+    return SparseCode(idx, val, row_off, row_nnz, B, code.d_sae)
+
+
 # ---- select ---------------------------------------------------------------------------------
 
 def select_topk_row(

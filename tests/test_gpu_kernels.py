@@ -858,3 +858,40 @@ def test_encoder_gemm_split_k(pkg, dev):
     assert torch.equal(got, torch.stack(parts).sum(0))
     want = x.double() @ w.double().t()
     assert ((got.double() - want).abs().max() / want.abs().max()).item() < 1e-5
+
+
+@pytest.mark.parametrize("G,B,k,F", [(4, 101, 16, 64), (1, 9, 8, 32), (3, 50, 64, 4096), (16, 7, 64, 256)])
+def test_union_group_codes(pkg, dev, G, B, k, F):
+    """Every (token, feature) of G stacked codes once, values summed in group order, order of first appearance; rows of
+    unequal length, a token with an empty row in every group, and 16 x 64 = 1024 entries per token (the limit)."""
+    g = torch.Generator().manual_seed(G * 1000 + B)
+    idx = torch.stack([torch.randperm(F, generator=g)[:k] for _ in range(G * B)]).to(torch.int32)    # distinct within a row
+    val = torch.randn(G * B, k, generator=g)
+    nnz = torch.randint(0, k + 1, (G * B,), generator=g, dtype=torch.int32)
+    nnz[torch.arange(G) * B + (B - 1)] = 0           # the last token keeps nothing anywhere
+    nnz[:B] = k                                      # group 0's rows are full
+    code = pkg.ops.SparseCode(idx.flatten().to(dev), val.flatten().to(dev), (torch.arange(G * B) * k).to(dev), nnz.to(dev), G * B, F)
+    got = pkg.ops.union_group_codes(code, G)
+    assert got.n_tokens == B and got.d_sae == F and got.row_off.tolist() == [t * G * k for t in range(B)]
+    gi, gv, gn = got.idx.view(B, G * k).cpu(), got.val.view(B, G * k).cpu(), got.row_nnz.tolist()
+    for t in range(B):
+        order, sums = [], {}
+        for q in range(G):
+            r = q * B + t
+            for j in range(int(nnz[r])):
+                f = int(idx[r, j])
+                if f not in sums:
+                    order.append(f)
+                    sums[f] = np.float32(0.0)
+                sums[f] = np.float32(sums[f] + np.float32(val[r, j]))
+        assert gn[t] == len(order), t
+        assert gi[t, :gn[t]].tolist() == order, t
+        assert np.array_equal(gv[t, :gn[t]].numpy(), np.array([sums[f] for f in order], dtype=np.float32)), t
+        assert not gi[t, gn[t]:].any() and not gv[t, gn[t]:].any()
+    with pytest.raises(ValueError):
+        pkg.ops.union_group_codes(code, G + 1)                       # rows that are not G + 1 groups of equally many tokens
+    if G * k == 1024:
+        wide = pkg.ops.SparseCode(torch.cat([code.idx, code.idx]), torch.cat([code.val, code.val]),
+                                  (torch.arange(2 * G * B) * k).to(dev), torch.cat([code.row_nnz, code.row_nnz]), 2 * G * B, F)
+        with pytest.raises(ValueError):
+            pkg.ops.union_group_codes(wide, 2 * G)                   # 2048 entries per token
