@@ -646,34 +646,58 @@ __global__ __launch_bounds__(GS_THREADS) void select_topk_row_granule_kernel(
 }
 
 // Granule maxima of rows that no GEMM epilogue left them for: eight lanes per granule (one 16-byte chunk each), eight
-// granules per wave and step.
+// granules per wave.  A lane keeps its chunk of bias and scale (64 bytes) for R consecutive rows of one group, so a row
+// costs its own 16 bytes of pre; the launch uses R = 8 when the groups are multiples of 8 rows and R = 1 otherwise.
+// With `groups` > 1 the rows are `groups` repeats of the same pre rows, one repeat per group of bias and scale (row
+// g * n_rows + r reads pre row r): the lane keeps its R chunks of pre and walks the groups, so pre is read once.
+template <int R>
 __global__ __launch_bounds__(256) void granule_max_kernel(const uint16_t *__restrict__ pre, const float *__restrict__ b_enc,
-                                                          const float *__restrict__ scale, int F, int64_t n_granules,
-                                                          int rows_per_group, int pre_rows, uint32_t *__restrict__ gmax) {
-  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+                                                          const float *__restrict__ scale, int F, int64_t n_rows, int64_t n_items,
+                                                          int rows_per_group, int pre_rows, int groups,
+                                                          uint32_t *__restrict__ gmax) {
+  const int64_t item = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;   // (block of R rows, granule)
+  if (item >= n_items) return;            // the eight lanes of an item leave together
   const int part = threadIdx.x & 7, ng = F >> 6;
-  uint32_t m = 0u;
-  if (g < n_granules) {
-    const int64_t row = g / ng;
-    const int gi = (int)(g % ng);
-    RowReader<true, SEL_PLAIN> rr;
-    const size_t grp = (size_t)(row / rows_per_group);
-    rr.row = pre + (size_t)(row % pre_rows) * F;
-    rr.b_enc = b_enc ? b_enc + grp * F : nullptr;
-    rr.scale = scale ? scale + grp * F : nullptr;
-    rr.fmask = nullptr;
-    rr.F = F;
-    uint32_t keys[8];
-    rr.chunk_keys(gi * 8 + part, keys);
+  const int64_t row0 = (item / ng) * R;
+  const int gi = (int)(item % ng);
+  const int c = gi * 8 + part;
+  u32x4 raw[R];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) m = keys[e] > m ? keys[e] : m;
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r < n_rows ? row0 + r : n_rows - 1;
+    raw[r] = reinterpret_cast<const u32x4 *>(pre + (size_t)(row % pre_rows) * F)[c];
+  }
+  for (int g = 0; g < groups; ++g) {
+  const size_t grp = groups > 1 ? (size_t)g : (size_t)(row0 / rows_per_group);
+  uint32_t *gout = gmax + (size_t)g * n_rows * ng;
+  float bb[8], ss[8];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const float4 zb = {0.f, 0.f, 0.f, 0.f}, os = {1.f, 1.f, 1.f, 1.f};
+    const float4 t = b_enc ? reinterpret_cast<const float4 *>(b_enc + grp * F + (size_t)c * 8)[q] : zb;
+    const float4 u = scale ? reinterpret_cast<const float4 *>(scale + grp * F + (size_t)c * 8)[q] : os;
+    bb[4 * q] = t.x; bb[4 * q + 1] = t.y; bb[4 * q + 2] = t.z; bb[4 * q + 3] = t.w;
+    ss[4 * q] = u.x; ss[4 * q + 1] = u.y; ss[4 * q + 2] = u.z; ss[4 * q + 3] = u.w;
   }
 #pragma unroll
-  for (int o = 1; o < 8; o <<= 1) {
-    const uint32_t t = (uint32_t)__shfl_xor((int)m, o, 64);
-    m = t > m ? t : m;
+  for (int r = 0; r < R; ++r) {
+    const uint32_t w[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+    uint32_t m = 0u;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t k0 = key_of<SEL_PLAIN>(__uint_as_float(w[q] << 16), bb[2 * q], ss[2 * q], 1.f);
+      const uint32_t k1 = key_of<SEL_PLAIN>(__uint_as_float(w[q] & 0xffff0000u), bb[2 * q + 1], ss[2 * q + 1], 1.f);
+      m = k0 > m ? k0 : m;
+      m = k1 > m ? k1 : m;
+    }
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) {
+      const uint32_t t = (uint32_t)__shfl_xor((int)m, o, 64);
+      m = t > m ? t : m;
+    }
+    if (part == 0 && row0 + r < n_rows) gout[(size_t)(row0 + r) * ng + gi] = m;
   }
-  if (part == 0 && g < n_granules) gmax[g] = m;
+  }
 }
 
 }  // namespace sae
@@ -760,9 +784,21 @@ extern "C" int sae_granule_max(const void *pre_bf16, const float *b_enc, const f
               (long long)B, (long long)pre_rows);
   SAE_REQUIRE((((uintptr_t)pre_bf16 | (uintptr_t)b_enc | (uintptr_t)scale) & 15) == 0, SAE_ERR_INVALID_ARG,
               "granule_max: pointers must be 16-byte aligned");
-  const int64_t n = B * (F / 64);
+  // rows of one block share a group's bias and scale: blocks of 8 rows when no block straddles two groups; groups that
+  // are repeats of the same pre rows are walked inside the kernel, over those rows once
+  const int R = rows_per_group % 8 == 0 ? 8 : 1;
+  const bool repeats = pre_rows < B && rows_per_group == pre_rows;
+  const int64_t rows = repeats ? pre_rows : B;
+  const int groups = repeats ? (int)(B / pre_rows) : 1;
+  const int64_t n = ((rows + R - 1) / R) * (F / 64);
   SAE_REQUIRE((n * 8 + 255) / 256 < (1LL << 31), SAE_ERR_UNSUPPORTED, "granule_max: too large");
-  hipLaunchKernelGGL(granule_max_kernel, dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t *)pre_bf16, b_enc, scale, (int)F, n, (int)rows_per_group, (int)pre_rows, granule_max);
+  if (R == 8)
+    hipLaunchKernelGGL(granule_max_kernel<8>, dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t *)pre_bf16, b_enc, scale, (int)F, rows, n, (int)rows_per_group, (int)pre_rows, groups,
+                       granule_max);
+  else
+    hipLaunchKernelGGL(granule_max_kernel<1>, dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t *)pre_bf16, b_enc, scale, (int)F, rows, n, (int)rows_per_group, (int)pre_rows, groups,
+                       granule_max);
   return check_launch("granule_max");
 }
