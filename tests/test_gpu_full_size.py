@@ -5,7 +5,8 @@ size-independent properties and against an independent dense recomputation with 
 routines ON THE GPU (matmul, topk, sort): given the kernel's own pre-activation, the selection must
 be exactly the k largest with lowest-index ties; given the selection, reconstruction, loss and every
 gradient must equal what dense GEMMs give; the optimiser move must equal the closed-form first Adam
-step.  The small-shape tests elsewhere tie the same kernels to the CPU oracle.
+step.  The small-shape tests elsewhere tie the same kernels to the CPU oracle, and the last three tests of this file
+run the oracle itself, with the full dictionaries, on a few tokens (or one sequence) of the full-size steps.
 """
 
 import math
@@ -496,3 +497,160 @@ def test_jumprelu_shape_fused_step_against_dense_path(pkg, dev, amp):
     for n_, p in sae.named_parameters():
         assert rel_err(fused[n_], p.grad) < tol_grad, n_
     assert (fused["activation_function.log_jumprelu_threshold"] != 0).float().mean().item() > 0.5
+
+
+# ---- the full-size steps against the CPU oracle on a few of their tokens ----------------------------------------------------
+# A token's forward pass does not depend on the batch's other tokens (per-token TopK, JumpReLU) or, for Lorsa, on other
+# sequences, so the oracle can afford the full dictionaries on a handful of tokens: the step runs on the GPU at its real
+# shape and the oracle recomputes some of its rows from the same parameters.
+
+def _copy_to_oracle(ref, model):
+    src = dict(model.named_parameters())
+    with torch.no_grad():
+        for n_, p in ref.named_parameters():
+            p.copy_(src[n_].detach().to("cpu", p.dtype))
+
+
+def test_clt_shape_rows_against_the_oracle(pkg, oracle, dev):
+    """C4 in fp32 (12 layers, d=768, 12288 features per layer, k=64, 2048 tokens): 32 of the tokens through the oracle's
+    encode (einsum + per-layer TopK) and its 78-block decode.  The two encoder products add in different orders, so an
+    entry within rounding of the k-th value may fall either way: such (token, layer) rows are counted and must be rare;
+    everything else agrees to fp32 rounding."""
+    import importlib
+
+    from lm_saes_amd import synthetic
+
+    vo = importlib.import_module("oracle.variants_oracle")
+    L, d, F, k, B = 12, 768, 12288, 64, 2048
+    hin, hout = [f"in{l}" for l in range(L)], [f"out{l}" for l in range(L)]
+    cfg = pkg.CLTConfig(hook_points_in=hin, hook_points_out=hout, d_model=d, expansion_factor=F / d, act_fn="topk", top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, device="cuda", dtype=torch.float32)
+    torch.manual_seed(0)
+    clt = pkg.CrossLayerTranscoder(cfg)
+    clt.init_parameters()
+    g = torch.Generator(device=dev).manual_seed(4)
+    batch = {"tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    for l in range(L):
+        x = synthetic.activations(B, d, 16, seed=4 + l).to(dev)
+        batch[hin[l]], batch[hout[l]] = x, torch.tanh(x @ (torch.randn(d, d, device=dev, generator=g) / d ** 0.5))
+    with torch.no_grad():
+        out = clt.compute_loss(batch)
+    assert "sparse_code" in out, "the kernel path did not run"
+    rows = torch.arange(5, B, 64, device=dev)
+    ref = vo.CLTOracle(L, d, F, act_fn="topk", top_k=k, sparsity_include_decoder_norm=True)
+    _copy_to_oracle(ref, clt)
+    sub = {n_: v[rows].cpu() for n_, v in batch.items()}
+    with torch.no_grad():
+        want = ref.compute_loss(sub, hin, hout)
+    # activations are [tokens, layers, features], reconstructions [layers, tokens, d] (the reference's layouts)
+    assert tuple(out["feature_acts"].shape) == (B, L, F) and tuple(out["reconstructed"].shape) == (L, B, d)
+    assert tuple(want["feature_acts"].shape) == (len(rows), L, F) and tuple(want["reconstructed"].shape) == (L, len(rows), d)
+    got_acts, got_recon = out["feature_acts"][rows].cpu(), out["reconstructed"][:, rows].cpu().transpose(0, 1)
+    want_recon = want["reconstructed"].transpose(0, 1)
+    same_rows = ((got_acts != 0) == (want["feature_acts"] != 0)).all(-1)            # [32, L]
+    assert same_rows.float().mean().item() > 0.99, same_rows.float().mean().item()
+    assert rel_err(got_acts[same_rows], want["feature_acts"][same_rows]) < 1e-5
+    # a token's reconstruction of layer j reads its layers 0..j: compared where all of those rows hold the same entries
+    prefix_ok = same_rows.cumprod(dim=1).bool()                                       # [32, L]
+    assert prefix_ok.float().mean().item() > 0.9
+    assert rel_err(got_recon[prefix_ok], want_recon[prefix_ok]) < 1e-4
+
+
+def test_lorsa_shape_sequence_against_the_oracle(pkg, oracle, dev):
+    """C5 under bf16 autocast (the attention, GEMM and select kernels): one of the 16 sequences through the fp32 oracle
+    (explicit causal softmax per head, dense TopK, dense decode), with the oracle's activation replaced by the kernel
+    path's own selection so that entries near the k-th value cannot fall differently; hidden_pre, the kept values and
+    the reconstruction agree at the bf16 bound."""
+    import importlib
+
+    from lm_saes_amd import synthetic
+
+    vo = importlib.import_module("oracle.variants_oracle")
+    nb, s, d, F, h, dq, k = 16, 1024, 768, 8192, 64, 64, 64
+    cfg = pkg.LorsaConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, n_qk_heads=h,
+                          d_qk_head=dq, n_ctx=s, rotary_dim=dq, positional_embedding_type="none", act_fn="topk", top_k=k,
+                          norm_activation="inference", device="cuda", dtype=torch.float32)
+    torch.manual_seed(0)
+    m = pkg.LowRankSparseAttention(cfg)
+    m.init_parameters()
+    with torch.no_grad():
+        for b_ in (m.b_Q, m.b_K, m.b_V):
+            b_.normal_(0, 0.05)
+    x = synthetic.activations(nb * s, d, 64, seed=4).to(dev).view(nb, s, d)
+    y = torch.roll(x, 1, dims=1) * 0.5
+    batch = {"in": x, "out": y, "tokens": torch.zeros(nb, s, dtype=torch.long, device=dev)}
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
+    with torch.no_grad(), _amp(True):
+        out = m.compute_loss(batch)
+    torch.cuda.synchronize()
+    pkg.ops.set_kernel_timer(None)
+    assert "attention_fwd" in timer.records, set(timer.records)
+    seq = 11
+    ref = vo.LorsaOracle(d_model=d, d_sae=F, n_qk_heads=h, d_qk_head=dq, n_ctx=s, act_fn="topk", top_k=k,
+                         positional_embedding_type="none")
+    _copy_to_oracle(ref, m)
+    for name, width in (("feature_acts", F), ("hidden_pre", F), ("reconstructed", d)):
+        assert tuple(out[name].shape) == (nb, s, width), (name, tuple(out[name].shape))
+    kept = (out["feature_acts"][seq] != 0).cpu()
+    assert torch.all(kept.sum(-1) == k)
+    ref.activation_function = lambda hp: hp * kept.to(hp.dtype).reshape(hp.shape)
+    sub = {"in": x[seq:seq + 1].cpu(), "out": y[seq:seq + 1].cpu(), "tokens": torch.zeros(1, s, dtype=torch.long)}
+    with torch.no_grad():
+        want = ref.compute_loss(sub)
+    assert rel_err(out["hidden_pre"][seq].cpu(), want["hidden_pre"][0]) < 2e-2
+    assert rel_err(out["feature_acts"][seq].cpu(), want["feature_acts"][0]) < 2e-2
+    assert rel_err(out["reconstructed"][seq].cpu(), want["reconstructed"][0]) < 2e-2
+    # and the kernel's selection is the oracle's own on all but near-tied entries
+    hp = want["hidden_pre"][0] * ref.decoder_norm()
+    own = torch.zeros_like(kept).scatter_(1, hp.topk(k, dim=-1).indices, True)
+    assert (own & kept).sum().item() > 0.9 * kept.sum().item()
+
+
+def test_jumprelu_shape_rows_against_the_oracle(pkg, oracle, dev):
+    """C3 in fp32 (d=4096, F=131072, 4096 tokens, threshold and window 0.001, tanh penalty): 48 of the tokens through the
+    oracle with the full dictionary.  A pre-activation within rounding of its threshold may fall either way between the two
+    encoder products: such entries are counted (a few of 6 M) and carry values of the threshold's size; activations,
+    reconstruction and the per-token penalty agree to fp32 rounding."""
+    d, F, B = 4096, 131072, 4096
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn="jumprelu",
+                        jumprelu_threshold_window=0.001, norm_activation="inference", sparsity_include_decoder_norm=True,
+                        device="cuda", dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(B, d, device=dev, generator=g)
+    x[:, [7, 1029, 2050, 3071]] *= 50.0
+    with torch.no_grad():
+        wt = sae.W_E.t()
+        wt.uniform_(-1.0 / d ** 0.5, 1.0 / d ** 0.5, generator=g)
+        sae.W_D.copy_(wt / wt.norm(dim=1, keepdim=True))
+        sae.b_E.zero_()
+        sae.b_D.copy_(x.mean(0))
+        sae.activation_function.log_jumprelu_threshold.fill_(math.log(0.001))
+    batch = {"in": x, "out": x, "tokens": torch.zeros(B, dtype=torch.long, device=dev)}
+    kw = dict(sparsity_loss_type="tanh", l1_coefficient=5.0)
+    timer = pkg.ops.KernelTimer()
+    pkg.ops.set_kernel_timer(timer)
+    with torch.no_grad():
+        out = sae.compute_loss(batch, **kw)
+    torch.cuda.synchronize()
+    pkg.ops.set_kernel_timer(None)
+    assert "jumprelu_fwd" in timer.records, set(timer.records)
+    rows = torch.arange(3, B, 86, device=dev)
+    assert tuple(out["feature_acts"].shape) == (B, F) and tuple(out["reconstructed"].shape) == (B, d) and tuple(out["l_s"].shape) == (B,)
+    got_acts, got_recon, got_ls = out["feature_acts"][rows].cpu(), out["reconstructed"][rows].cpu(), out["l_s"][rows].cpu()
+    del out
+    ref = oracle.SAEOracle(d, F, act_fn="jumprelu", jumprelu_threshold_window=0.001, sparsity_include_decoder_norm=True)
+    _copy_to_oracle(ref, sae)
+    sub = {"in": x[rows].cpu(), "out": x[rows].cpu(), "tokens": torch.zeros(len(rows), dtype=torch.long)}
+    with torch.no_grad():
+        want = ref.compute_loss(sub, **kw)
+    differ = (got_acts != 0) != (want["feature_acts"] != 0)
+    assert differ.sum().item() <= 1e-5 * differ.numel(), differ.sum().item()
+    assert 0.3 < (got_acts != 0).float().mean().item() < 0.7
+    # an entry that fell the other way holds a value of the threshold's size on one side and 0 on the other
+    both = got_acts - want["feature_acts"]
+    assert both[differ].abs().max().item() < 0.05 if differ.any() else True
+    assert rel_err(torch.where(differ, 0, got_acts), torch.where(differ, 0, want["feature_acts"])) < 1e-5
+    assert rel_err(got_recon, want["reconstructed"]) < 1e-4
+    assert rel_err(got_ls, want["l_s"]) < 1e-4
