@@ -120,15 +120,17 @@ __device__ __forceinline__ float load_grad1(const void *g, int64_t i) {
   else return reinterpret_cast<const float *>(g)[i];
 }
 
-// flat: grid-stride over groups of four elements.  S_BF16: p, m, v point to bf16 arrays (the pointer type is
-// nominal) and the update is the low-precision one above.
+// flat: a workgroup owns ADAM_FLAT_CHUNK consecutive groups of four elements (16 KB of each fp32 array: with a stride of
+// the whole grid between a thread's groups the same update ran 15 % slower on 537 M elements).  S_BF16: p, m, v point to
+// bf16 arrays (the pointer type is nominal) and the update is the low-precision one above.
+constexpr int ADAM_FLAT_CHUNK = 1024;
 template <bool G_BF16, bool S_BF16 = false>
 __global__ __launch_bounds__(256) void adam_flat_kernel(float *__restrict__ p, const void *__restrict__ g,
                                                         float *__restrict__ m, float *__restrict__ v, int64_t n,
                                                         AdamScalars a, uint16_t *__restrict__ shadow) {
   const int64_t n4 = n >> 2;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+  const int64_t first = (int64_t)blockIdx.x * ADAM_FLAT_CHUNK, last = first + ADAM_FLAT_CHUNK < n4 ? first + ADAM_FLAT_CHUNK : n4;
+  for (int64_t i = first + threadIdx.x; i < last; i += 256) {
     float4 pp = load_state4<S_BF16>(p, i);
     const float4 gg = load_grad4<G_BF16>(g, i);
     float4 mm = load_state4<S_BF16>(m, i);
@@ -233,9 +235,9 @@ static int adam_step_impl(bool lowp, float *p, const void *g, int g_dtype, float
     else { if (g_dtype == SAE_BF16) SAE_ADAM_DENSE_ROWS(true, false); else SAE_ADAM_DENSE_ROWS(false, false); }
 #undef SAE_ADAM_DENSE_ROWS
   } else {
-    int64_t blocks = ((n >> 2) + 255) / 256;
+    int64_t blocks = ((n >> 2) + ADAM_FLAT_CHUNK - 1) / ADAM_FLAT_CHUNK;
     if (blocks < 1) blocks = 1;
-    if (blocks > 65536) blocks = 65536;
+    SAE_REQUIRE(blocks < (1LL << 31), SAE_ERR_UNSUPPORTED, "adam_step: too many elements");
 #define SAE_ADAM_FLAT(GB, SB)                                                                                 \
   hipLaunchKernelGGL((adam_flat_kernel<GB, SB>), dim3((unsigned)blocks), dim3(256), 0, st, p, g, m, v, n, a, \
                      reinterpret_cast<uint16_t *>(shadow_bf16))
