@@ -8,6 +8,7 @@ import os
 import random
 import time
 
+import numpy as np
 import pytest
 import torch
 
@@ -231,11 +232,40 @@ def test_random_sweep_granule_route(pkg, oracle, dev, sweep_seed, budget_s=10.0)
     n = 0
     while time.time() - t0 < budget_s:
         n += 1
-        kind = rng.choice(["select", "select", "gemm_select", "grouped_merge"])
+        kind = rng.choice(["select", "select", "gemm_select", "grouped_merge", "shared_union"])
         seed = rng.randrange(1 << 30)
         g = torch.Generator().manual_seed(seed)
-        if kind == "select":
-            B = rng.choice([1, 3, 9, 20]); F = 64 * rng.choice([1, 2, 7, 16, 64, 128, 192, 1024, 2048, 4096])
+        if kind == "shared_union":
+            # H groups of bias / scale over ONE matrix (a crosscoder's heads), then every (token, feature) once
+            H = rng.choice([1, 2, 4, 7]); B = rng.choice([3, 8, 40]); F = 64 * rng.choice([2, 16, 48]); k = min(F, rng.choice([2, 16, 64]))
+            pre = torch.randn(B, F, generator=g)
+            if rng.random() < 0.3: pre = quant(pre, 8)
+            if rng.random() < 0.3: pre[rng.randrange(B)] = -1.0
+            pre = pre.to(torch.bfloat16)
+            b = 0.1 * torch.randn(H, F, generator=g); s = 0.8 + 0.4 * torch.rand(H, F, generator=g)
+            print(f"[{n}] shared-matrix select + union seed={seed} H={H} B={B} F={F} k={k}", flush=True)
+            gmax = pkg.ops.granule_max(pre.to(dev), b.to(dev), s.to(dev), rows_per_group=B, n_rows=H * B)
+            stacked = pkg.ops.select_topk_row(pre.to(dev), b.to(dev), s.to(dev), k, granule_max=gmax, rows_per_group=B, n_rows=H * B)
+            per_head = [tk.oracle_topk_code(oracle, pre, b[h], s[h], k) for h in range(H)]
+            got = tk.code_to_rows(stacked)
+            for h in range(H):
+                for t in range(B):
+                    (gi, gv), (wi, wv) = got[h * B + t], per_head[h][t]
+                    assert (gi == wi).all() and (gv == wv).all(), f"head {h} token {t}"
+            merged = pkg.ops.union_group_codes(stacked, H)
+            mi, mv, mn = merged.idx.view(B, H * k).cpu(), merged.val.view(B, H * k).cpu(), merged.row_nnz.tolist()
+            for t in range(B):
+                order, sums = [], {}
+                for h in range(H):
+                    for f, v in zip(per_head[h][t][0].tolist(), per_head[h][t][1]):
+                        if f not in sums:
+                            order.append(f); sums[f] = np.float32(0.0)
+                        sums[f] = np.float32(sums[f] + np.float32(v))
+                assert mn[t] == len(order) and mi[t, :mn[t]].tolist() == order, f"token {t}"
+                assert mv[t, :mn[t]].tolist() == [float(sums[f]) for f in order], f"token {t}"
+                assert not mi[t, mn[t]:].any() and not mv[t, mn[t]:].any()
+        elif kind == "select":
+            B = rng.choice([1, 3, 8, 9, 20, 24]); F = 64 * rng.choice([1, 2, 7, 16, 64, 128, 192, 1024, 2048, 4096])
             k = min(F, rng.choice([1, 4, 16, 32, 64, 128, 300, 512]))
             ties = rng.choice([0, 0, 2, 16, 64])
             pre = torch.randn(B, F, generator=g)
@@ -288,3 +318,30 @@ def test_random_sweep_granule_route(pkg, oracle, dev, sweep_seed, budget_s=10.0)
                 assert cnt[t].tolist() == [len(per_layer[l][t][0]) for l in range(L)]
     print(f"{n} cases", flush=True)
     assert n > 50
+
+
+@pytest.mark.parametrize("sweep_seed", [6])
+def test_random_sweep_gemm_operand_layouts(pkg, dev, sweep_seed, budget_s=8.0):
+    """sae_gemm_bf16 over drawn shapes (edge tiles in both dimensions, 1 to 64 slabs of K), layouts and output types:
+    bit for bit the K-contiguous kernel's product of the transposed copies, and the exact product to fp32 / bf16 rounding."""
+    rng = random.Random(sweep_seed)
+    t0 = time.time()
+    n = 0
+    while time.time() - t0 < budget_s:
+        n += 1
+        seed = rng.randrange(1 << 30)
+        g = torch.Generator().manual_seed(seed)
+        M = 8 * rng.randrange(1, 90); N = 8 * rng.randrange(1, 90); K = 64 * rng.choice([1, 2, 3, 5, 8, 16, 33, 64])
+        a_t, b_t = rng.choice([(False, True), (True, False), (True, True)])
+        out_dtype = rng.choice([torch.float32, torch.bfloat16])
+        print(f"[{n}] gemm layouts seed={seed} M={M} N={N} K={K} a_k_major={a_t} b_k_major={b_t} out={out_dtype}", flush=True)
+        a = torch.randn(M, K, generator=g).bfloat16(); b = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16()
+        a_dev, b_dev = a.to(dev), b.to(dev)
+        got = pkg.ops.gemm(a_dev.t().contiguous() if a_t else a_dev, b_dev.t().contiguous() if b_t else b_dev, out_dtype,
+                           a_k_major=a_t, b_k_major=b_t, copy_when_faster=False)
+        assert torch.equal(got, pkg.ops.encoder_gemm(a_dev, b_dev, out_dtype))
+        want = a.double() @ b.double().t()
+        err = ((got.double().cpu() - want).abs().max() / want.abs().max()).item()
+        assert err < (1e-5 if out_dtype == torch.float32 else 2 ** -7), err
+    print(f"{n} cases", flush=True)
+    assert n > 30
