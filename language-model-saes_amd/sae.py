@@ -435,6 +435,68 @@ class _FusedSparseStep(torch.autograd.Function):
         return dx, dlabel, None, None if dW_Et is None else dW_Et.t(), db_E, dW_D, db_D, None, None, None
 
 
+class _GluSparseStep(torch.autograd.Function):
+    """The TopK / BatchTopK step of a dictionary with a gated encoder (models/sae.py:326-331:
+    hidden_pre = (x W_E + b_E) * sigmoid(x W_E_glu + b_E_glu)): both encoder products on the GEMM kernel, the gate as
+    element-wise ops, then select, fused decode + loss and gradient rows as in the plain step.  Only kept entries carry a
+    gradient, so both encoders' weight gradients are gathered rows of x with one coefficient per kept entry:
+    d pre = d val * gate for W_E and d val * (x W_E + b_E) * gate * (1 - gate) for W_E_glu; no dense [B, F] gradient and
+    no dense backward product is formed."""
+
+    @staticmethod
+    def forward(ctx, x, label, tok_w, W_E, b_E, W_G, b_G, W_D, b_D, k, amp, holder):
+        sae = holder.model
+        w_enc_op, w_glu_op = sae._w_enc_operand(amp), sae._w_glu_operand(amp)
+        x_op = (x if x.dtype == torch.bfloat16 else ops.cast_bf16(x.contiguous())) if amp else x.contiguous()
+        out_dtype = torch.bfloat16 if amp else torch.float32
+        pre, pre_g = ops.encoder_gemm(x_op, w_enc_op, out_dtype), ops.encoder_gemm(x_op, w_glu_op, out_dtype)
+        lin = pre.float() + b_E
+        gate = torch.sigmoid(pre_g.float() + b_G)
+        hidden = lin * gate                                                        # [B, F] fp32, as the reference holds it
+        scale = sae._decoder_norm_nograd() if sae.cfg.sparsity_include_decoder_norm else None
+        B = x.shape[0]
+        if sae.cfg.act_fn.lower() == "batchtopk":
+            code = ops.select_topk_batch(hidden, None, scale, k * B)
+        else:
+            code = ops.select_topk_row(hidden, None, scale, k)
+        recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(code, sae._w_dec_operand(amp), b_D, label, tok_w)
+        tok, valid = _code_slot_tokens(code)
+        cell = torch.where(valid, tok * hidden.shape[1] + code.idx.long(), torch.zeros_like(tok))
+        zero = torch.zeros((), dtype=torch.float32, device=x.device)
+        ctx.lin = torch.where(valid, lin.flatten()[cell], zero)                    # per kept entry
+        ctx.gate = torch.where(valid, gate.flatten()[cell], zero)
+        ctx.code, ctx.x_op, ctx.grad_recon, ctx.dval, ctx.w_enc_op, ctx.w_glu_op = code, x_op, grad_recon, dval, w_enc_op, w_glu_op
+        ctx.amp, ctx.has_b_D = bool(amp), b_D is not None
+        holder.code, holder.hidden, holder.scale = code, hidden, scale
+        ctx.mark_non_differentiable(recon)
+        ctx.set_materialize_grads(False)
+        return loss_tok.sum(), recon
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_recon):
+        if g_loss is None:
+            return (None,) * 12
+        code = ctx.code
+        F = code.d_sae
+        g = g_loss.to(torch.float32)
+        fi = ops.build_feature_index(code)
+        # under autocast the decoder's weight gradient pairs the activations with the bf16-rounded output gradient
+        gd = ops.cast_bf16(ctx.grad_recon.contiguous()) if ctx.amp else ctx.grad_recon
+        dW_D, _ = ops.sparse_grad_rows(fi, code.val * g, gd, F)
+        d_hidden = ctx.dval * g                     # kept entries are positive and the norm's two terms cancel
+        c_enc, c_glu = d_hidden * ctx.gate, d_hidden * ctx.lin * ctx.gate * (1.0 - ctx.gate)
+        dW_Et, db_E = ops.sparse_grad_rows(fi, c_enc, ctx.x_op, F, want_bias=True)
+        dW_Gt, db_G = ops.sparse_grad_rows(fi, c_glu, ctx.x_op, F, want_bias=True)
+        db_D = ops.col_sum(ctx.grad_recon) * g if ctx.has_b_D else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            import dataclasses
+            dx = (ops.sparse_decode_fwd(dataclasses.replace(code, val=c_enc), ctx.w_enc_op, None)
+                  + ops.sparse_decode_fwd(dataclasses.replace(code, val=c_glu), ctx.w_glu_op, None))
+        dlabel = -ctx.grad_recon * g if ctx.needs_input_grad[1] else None
+        return dx, dlabel, None, dW_Et.t(), db_E, dW_Gt.t(), db_G, dW_D, db_D, None, None, None
+
+
 def _transposed(t: torch.Tensor) -> torch.Tensor:
     """[r, c] -> contiguous [c, r] in the same dtype (bf16 or fp32) through the transpose kernels."""
     t = t.contiguous()
@@ -789,6 +851,14 @@ class SparseAutoEncoder(SparseDictionary):
             return wt
         return self._derive("W_E.bf16", self.W_E, lambda old: ops.cast_bf16(wt, old))
 
+    def _w_glu_operand(self, amp: bool) -> torch.Tensor:
+        """[F, d] operand of the gate's product: the parameter's own buffer, or its bf16 copy under autocast."""
+        wt = self.W_E_glu.detach().t()
+        wt = wt if wt.is_contiguous() else wt.contiguous()
+        if not amp or wt.dtype == torch.bfloat16:
+            return wt
+        return self._derive("W_E_glu.bf16", self.W_E_glu, lambda old: ops.cast_bf16(wt, old))
+
     def _w_dec_operand(self, amp: bool) -> torch.Tensor:
         self.wait_pending_update()
         w = self.W_D.detach()
@@ -974,6 +1044,39 @@ class SparseAutoEncoder(SparseDictionary):
             and (self.W_E.dtype == torch.float32
                  or (self.W_E.dtype == torch.bfloat16 and self.cfg.d_model % 64 == 0))
         )
+
+    def _glu_eligible(self, x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient) -> bool:
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        return (self.cfg.use_glu_encoder and self.cfg.act_fn.lower() in ("topk", "batchtopk") and x.is_cuda and x.ndim == 2
+                and label.ndim == 2 and sparsity_loss_type is None and not (auxk_coefficient > 0.0) and self._no_hooks()
+                and self.W_E.dtype == torch.float32 and self.cfg.d_model % (64 if amp else 32) == 0
+                and self.cfg.d_model % 8 == 0 and x.shape[0] <= 131072)
+
+    def _glu_loss(self, batch, x, label, l1_coefficient, lp_coefficient, auxk_coefficient, return_aux_data):
+        mask = batch.get("mask")
+        B = x.shape[0]
+        amp = _autocast_dtype("cuda") == torch.bfloat16
+        if mask is None:
+            tok_w = torch.full((B,), 1.0 / B, dtype=torch.float32, device=x.device)
+        else:
+            m = mask.to(torch.float32)
+            tok_w = m / m.sum()
+        holder = _Holder()
+        holder.model = self
+        loss, recon = _GluSparseStep.apply(
+            x.to(torch.float32) if x.dtype not in (torch.float32, torch.bfloat16) else x, label.to(torch.float32).contiguous(),
+            tok_w, self.W_E, self.b_E, self.W_E_glu, self.b_E_glu, self.W_D, self.b_D if self.cfg.use_decoder_bias else None,
+            int(self.current_k), amp, holder)
+        if not return_aux_data:
+            return loss
+        code, hidden, scale = holder.code, holder.hidden, holder.scale
+        eager = {"loss": loss, "l_rec": loss, "l_s": None, "l_p": None, "l_aux": None, "label": label, "mask": mask,
+                 "reconstructed": recon, "l1_coefficient": l1_coefficient, "lp_coefficient": lp_coefficient,
+                 "auxk_coefficient": auxk_coefficient, "sparse_code": code}
+        lazy = {"n_tokens": (lambda: batch["tokens"].numel()) if mask is None else (lambda: int(mask.sum().item())),
+                "feature_acts": code.to_dense,
+                "hidden_pre": (lambda: (hidden * scale) / scale) if scale is not None else (lambda: hidden)}
+        return LazyDict(eager, lazy)
 
     # ---- JumpReLU / ReLU train-step loss: dense activations, so the GEMM kernel for all five dense products + one fused
     # element-wise pass each way (a ReLU is the same kernels with a threshold of zero, which has no gradient) ----
@@ -1196,6 +1299,8 @@ class SparseAutoEncoder(SparseDictionary):
                     frequency_scale=frequency_scale, p=p, l1_coefficient=l1_coefficient, lp_coefficient=lp_coefficient,
                     auxk_coefficient=auxk_coefficient, k_aux=k_aux, update_dead_statistics=update_dead_statistics,
                     return_aux_data=return_aux_data, **kwargs))
+        if self._glu_eligible(x, label, sparsity_loss_type, lp_coefficient, auxk_coefficient):
+            return self._glu_loss(batch, x, label, l1_coefficient, lp_coefficient, auxk_coefficient, return_aux_data)
         if self._jumprelu_eligible(x, label, sparsity_loss_type, auxk_coefficient):
             return self._jumprelu_loss(batch, x, label, sparsity_loss_type, tanh_stretch_coefficient, l1_coefficient,
                                        lp_coefficient, auxk_coefficient, return_aux_data, frequency_scale, p)

@@ -257,3 +257,107 @@ def test_topk_with_a_penalty_hands_factored_gradients_to_the_optimizer(pkg, orac
         g = rp[n].grad
         resolved = g.abs() > 1e-2 * g.abs().max()
         assert (moved - want)[resolved].abs().max().item() < 0.05 * 1e-3, n
+
+
+# ---- gated (GLU) encoder on the sparse step ----------------------------------------------------------------------------------
+
+def make_glu_models(pkg, oracle, dev, act_fn, d, F, k, B, seed):
+    from lm_saes_amd import synthetic
+
+    x = synthetic.activations(B, d, 8, seed)
+    w = synthetic.sae_weights(d, F, x, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    W_D = (w[2] * (0.5 + torch.rand(F, 1, generator=g))).contiguous()
+    w = (w[0], 0.02 * torch.randn(F, generator=g), W_D, w[3])
+    cfg = pkg.SAEConfig(hook_point_in="in", hook_point_out="out", d_model=d, expansion_factor=F / d, act_fn=act_fn, top_k=k,
+                        norm_activation="inference", sparsity_include_decoder_norm=True, use_glu_encoder=True, device="cuda",
+                        dtype=torch.float32)
+    sae = pkg.SparseAutoEncoder(cfg)
+    synthetic.load_weights(sae, *[t.to(dev) for t in w])
+    ref = oracle.SAEOracle(d, F, act_fn=act_fn, top_k=k, sparsity_include_decoder_norm=True, use_glu_encoder=True)
+    synthetic.load_weights(ref, *w)
+    with torch.no_grad():
+        wg, bg = torch.randn(d, F, generator=g) / d ** 0.5, 0.1 * torch.randn(F, generator=g)
+        sae.W_E_glu.copy_(wg.to(dev)); sae.b_E_glu.copy_(bg.to(dev))
+        ref.W_E_glu.copy_(wg); ref.b_E_glu.copy_(bg)
+    return sae, ref, x
+
+
+@pytest.mark.parametrize("act_fn", ["topk", "batchtopk"])
+def test_glu_encoder_takes_the_sparse_step_fp32(pkg, oracle, dev, act_fn):
+    """hidden_pre = (x W_E + b_E) * sigmoid(x W_E_glu + b_E_glu) (models/sae.py:326-331) with a token mask: select, fused
+    decode + loss and gathered gradient rows for W_E, W_E_glu and W_D; loss, outputs and all six gradients against the
+    oracle."""
+    d, F, k, B = 64, 512, 8, 96
+    sae, ref, x = make_glu_models(pkg, oracle, dev, act_fn, d, F, k, B, seed=71)
+    g = torch.Generator().manual_seed(72)
+    mask = (torch.rand(B, generator=g) > 0.2).float()
+    batch = {"in": x, "out": torch.tanh(x), "tokens": torch.zeros(B), "mask": mask}
+    with kernel_names(pkg) as names:
+        out = sae.compute_loss({k_: v.to(dev) for k_, v in batch.items()})
+        out["loss"].backward()
+    names = set(names)
+    assert {"sparse_decode_mse_fused", "build_feature_index"} <= names and any(n.startswith("sparse_grad_rows") for n in names), names
+    assert "sparse_code" in out
+    want = ref.compute_loss(batch)
+    want["loss"].backward()
+    assert torch.equal((out["feature_acts"] != 0).cpu(), want["feature_acts"] != 0)
+    if act_fn == "batchtopk":
+        assert len(set((out["feature_acts"] != 0).sum(-1).tolist())) > 1
+    for key in ("loss", "feature_acts", "hidden_pre", "reconstructed"):
+        assert rel_err(out[key], want[key]) < FP32_TOL, key
+    got, exp = dict(sae.named_parameters()), dict(ref.named_parameters())
+    assert set(got) == set(exp) and len(got) == 6
+    for n, p in exp.items():
+        assert got[n].grad is not None and tuple(got[n].grad.shape) == tuple(p.shape), n
+        assert rel_err(got[n].grad, p.grad) < GRAD_TOL, (n, rel_err(got[n].grad, p.grad))
+
+
+def test_glu_encoder_sparse_step_under_autocast(pkg, oracle, dev):
+    """bf16 autocast: the sparse step against the module's generic op sequence, whose two encoder products are the same
+    kernel launches (the same gated pre-activations, hence the same selection) and whose backward is dense bf16 products."""
+    d, F, k, B = 128, 1024, 16, 128
+    sae, _, x = make_glu_models(pkg, oracle, dev, "topk", d, F, k, B, seed=73)
+    batch = {"in": x.to(dev), "out": torch.tanh(x).to(dev), "tokens": torch.zeros(B, device=dev)}
+    with kernel_names(pkg) as names, torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sae.compute_loss(batch)
+        out["loss"].backward()
+    assert "sparse_decode_mse_fused" in set(names)
+    fused = {n: p.grad.clone() for n, p in sae.named_parameters()}
+    for p in sae.parameters():
+        p.grad = None
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        want = pkg.SparseDictionary.compute_loss(sae, batch)
+    want["loss"].backward()
+    assert torch.equal(out["feature_acts"] != 0, want["feature_acts"] != 0)
+    # (h n) / n with the norms of the row-norm kernel or of torch.norm: equal to a rounding of the product and the quotient
+    assert rel_err(out["hidden_pre"], want["hidden_pre"]) < 1e-6
+    assert rel_err(out["reconstructed"], want["reconstructed"]) < BF16_TOL
+    assert abs(out["loss"].item() - want["loss"].item()) < BF16_TOL * want["loss"].item()
+    for n, p in sae.named_parameters():
+        assert rel_err(fused[n], p.grad) < BF16_TOL, (n, rel_err(fused[n], p.grad))
+
+
+def test_glu_encoder_sparse_step_over_adam_steps(pkg, oracle, dev):
+    """Three optimisation steps of the gated dictionary with HipAdam (dense gradient rows from the sparse step; under autocast
+    the gate's bf16 operand is re-derived after every update) against torch.optim.Adam on the oracle."""
+    d, F, k, B = 64, 512, 8, 96
+    sae, ref, x = make_glu_models(pkg, oracle, dev, "topk", d, F, k, B, seed=75)
+    batch = {"in": x, "out": torch.tanh(x), "tokens": torch.zeros(B)}
+    gb = {k_: v.to(dev) for k_, v in batch.items()}
+    opt = pkg.HipAdam(sae.get_parameters()[0]["params"], lr=1e-3, model=sae)
+    ropt = oracle.make_adam(ref, lr=1e-3)
+    for step in range(3):
+        out = sae.compute_loss(gb)
+        assert "sparse_code" in out
+        out["loss"].backward()
+        want = ref.compute_loss(batch)
+        want["loss"].backward()
+        assert rel_err(out["loss"], want["loss"]) < 1e-4, step
+        opt.step(); opt.zero_grad()
+        ropt.step(); ropt.zero_grad()
+        for (n, p), q in zip(sae.named_parameters(), ref.parameters()):
+            assert (p.detach().cpu() - q.detach()).abs().max() <= 2e-2 * 1e-3 * (step + 1) + 1e-6 * q.detach().abs().max(), (step, n)
+    with torch.autocast("cuda", dtype=torch.bfloat16):      # the bf16 operands follow the updated weights
+        sae.compute_loss(gb, return_aux_data=False)
+    assert torch.equal(sae._w_glu_operand(True), sae.W_E_glu.detach().t().contiguous().to(torch.bfloat16))
