@@ -446,9 +446,9 @@ WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": b
 
 # the other benchmark configurations a default run times after the headline (a few steps each): BASELINE's five
 # configurations, the JumpReLU one in both of its forms, and a crosscoder
-CONFIG_RUNS = [("c1_topk_fp32", "c1_fp32", 10), ("c2_batchtopk_auxk", "batchtopk", 8), ("c3_jumprelu_dense", "jumprelu", 4),
-               ("c3_jumprelu_sparse", "jumprelu_sparse", 6), ("c4_clt", "clt", 6), ("c5_lorsa", "lorsa", 8),
-               ("crosscoder", "crosscoder", 8)]
+CONFIG_RUNS = [("c1_topk_fp32", "c1_fp32", 20), ("c2_batchtopk_auxk", "batchtopk", 12), ("c3_jumprelu_dense", "jumprelu", 5),
+               ("c3_jumprelu_sparse", "jumprelu_sparse", 10), ("c4_clt", "clt", 8), ("c5_lorsa", "lorsa", 12),
+               ("crosscoder", "crosscoder", 12)]
 
 
 def step_work(workload: str, shape) -> dict:
