@@ -34,10 +34,10 @@
 // softmax (running maximum and sum per query in fp32, log2 domain; the accumulators are rescaled only when some
 // row's maximum has grown by more than 2^8, so probabilities are formed relative to a reference at most that far
 // below the true maximum: exact in real arithmetic, and bf16 keeps its relative precision at any magnitude).
-// Backward: D[q] = sum_dv dout * out (one small kernel, which also leaves the log-sum-exp in the log2 domain); dV and
-// dK each by a workgroup per 128 keys that walks the query blocks diagonal .. last; dQ by a workgroup per 128 queries
-// that walks the key blocks 0 .. diagonal.  All three recompute the probabilities from q, k and the saved
-// log-sum-exp.  No atomics: results are reproducible.
+// Backward: dQ by a workgroup per 128 queries that walks the key blocks 0 .. diagonal; it is launched first and also
+// leaves, for its own queries, D[q] = sum_dv dout * out and the log-sum-exp in the log2 domain, which dV and dK (each by
+// a workgroup per 128 keys that walks the query blocks diagonal .. last) read per query.  All three recompute the
+// probabilities from q, k and the saved log-sum-exp.  No atomics: results are reproducible.
 //
 // In the forward kernel a wave runs its score products and its exponentials / value products at raised priority
 // (s_setprio) and its masking, running maximum and address arithmetic at the base one: of the waves that share a
