@@ -409,8 +409,8 @@ def build_lorsa(pkg, dev, args, positional="none"):
 
 
 def build_lorsa_rotary(pkg, dev, args):
-    """The Lorsa workload with rotary embeddings on queries and keys (the reference's default; BASELINE's configuration has
-    none): a secondary figure."""
+    """The Lorsa workload with rotary embeddings on queries and keys (the reference's default; the benchmarked Lorsa
+    configuration has none): a secondary figure."""
     return build_lorsa(pkg, dev, args, positional="rotary")
 
 
@@ -444,8 +444,8 @@ def build_crosscoder(pkg, dev, args):
 WORKLOADS = {"topk": build_topk, "c1_fp32": build_c1_fp32, "topk_bf16_params": build_topk_bf16_params, "topk_trainer": build_topk_trainer, "activation_stream": build_activation_stream, "batchtopk": build_batchtopk, "batchtopk_bf16_params": build_batchtopk_bf16_params, "jumprelu": build_jumprelu, "jumprelu_sparse": build_jumprelu_sparse, "clt": build_clt,
              "lorsa": build_lorsa, "lorsa_rotary": build_lorsa_rotary, "crosscoder": build_crosscoder}
 
-# the other benchmark configurations a default run times after the headline (a few steps each): BASELINE's five
-# configurations, the JumpReLU one in both of its forms, and a crosscoder
+# the other benchmark configurations a default run times after the headline (a few steps each): the five
+# benchmarked configurations, the JumpReLU one in both of its forms, and a crosscoder
 CONFIG_RUNS = [("c1_topk_fp32", "c1_fp32", 20), ("c2_batchtopk_auxk", "batchtopk", 12), ("c3_jumprelu_dense", "jumprelu", 5),
                ("c3_jumprelu_sparse", "jumprelu_sparse", 10), ("c4_clt", "clt", 8), ("c5_lorsa", "lorsa", 12),
                ("crosscoder", "crosscoder", 12)]
