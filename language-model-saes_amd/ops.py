@@ -20,14 +20,16 @@ def _stream(t: torch.Tensor) -> int:
 
 
 class KernelTimer:
-    """Collects HIP-event pairs around every library call made while it is installed.
+    """Collects HIP-event pairs around every library call made while it is installed, or, with `only`, around the calls
+    of those names (two event records per call cost host time and a few per cent of a step made of many short launches).
 
     Events are recorded on the stream the kernels are launched on (torch's current stream), so
     `elapsed_time` is the device-side duration of that call's kernels.  Read after a synchronize.
     """
 
-    def __init__(self):
+    def __init__(self, only=None):
         self.records: dict[str, list[tuple[torch.cuda.Event, torch.cuda.Event]]] = {}
+        self.only = None if only is None else frozenset(only)
 
     def summary(self) -> dict[str, dict[str, float]]:
         out = {}
@@ -50,16 +52,18 @@ class _timed:
         self.name = name
 
     def __enter__(self):
-        if _timer is not None:
+        t = _timer
+        self.timer = t if t is not None and (t.only is None or self.name in t.only) else None
+        if self.timer is not None:
             self.a = torch.cuda.Event(enable_timing=True)
             self.a.record()
         return self
 
     def __exit__(self, *exc):
-        if _timer is not None:
+        if self.timer is not None:
             b = torch.cuda.Event(enable_timing=True)
             b.record()
-            _timer.records.setdefault(self.name, []).append((self.a, b))
+            self.timer.records.setdefault(self.name, []).append((self.a, b))
         return False
 
 
