@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256) void merge_layer_codes_kernel(const int32_t *_
 // entries in slots [row * k, row * k + row_nnz)) -> one code with every (token, feature) once: token b's entries are the
 // distinct features of its G rows, in order of first appearance (group 0's entries first), each with the sum of the values
 // that feature carries in the token's rows, added in group order.  One wave per token; the token's G * k entries sit in
-// LDS and every entry is compared with all of them (G * k <= 1024: at most 16 passes of 1024 broadcast reads per lane).
+// LDS.  Rows whose features ascend (what the select kernels write) are searched by bisection, one search per entry and
+// other group; a token with a row that does not ascend has every entry compared with all of them instead (G * k <= 1024:
+// at most 16 passes of 1024 broadcast reads per lane).  Same result either way.
 constexpr int UNION_MAX = 1024;
 __global__ __launch_bounds__(256) void union_group_codes_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
                                                                 const int32_t *__restrict__ row_nnz, int G, int B, int k,
@@ -172,16 +174,43 @@ __global__ __launch_bounds__(256) void union_group_codes_kernel(const int32_t *_
   __syncthreads();
   if (b >= B) return;
   const size_t base = (size_t)b * per_tok;
+  // do the live entries of every row ascend?  (dead slots hold -1 and follow the live ones)
+  bool bad = false;
+  for (int s = lane; s < per_tok; s += 64) {
+    const int j = s % k;
+    bad = bad || (j > 0 && si[s] >= 0 && si[s - 1] >= si[s]);
+  }
+  const bool ascending = __ballot(bad) == 0ull;
   int written = 0;
   for (int s0 = 0; s0 < per_tok; s0 += 64) {
     const int s = s0 + lane;
     const int mine = s < per_tok ? si[s] : -1;
     float sum = 0.f;
     bool first = mine >= 0;
-    for (int q = 0; q < per_tok; ++q) {
-      const bool same = si[q] == mine;
-      sum += same ? sv[q] : 0.f;
-      first = first && !(same && q < s);
+    if (ascending) {
+      const int g = s / k;
+      if (mine >= 0) {
+        for (int q = 0; q < G; ++q) {
+          if (q == g) { sum += sv[s]; continue; }
+          // first slot of row q that is dead or holds a feature >= mine
+          int lo = q * k, hi = lo + k;
+          while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            const int v = si[mid];
+            if (v >= 0 && v < mine) lo = mid + 1; else hi = mid;
+          }
+          if (lo < (q + 1) * k && si[lo] == mine) {
+            sum += sv[lo];
+            first = first && q > g;
+          }
+        }
+      }
+    } else {
+      for (int q = 0; q < per_tok; ++q) {
+        const bool same = si[q] == mine;
+        sum += same ? sv[q] : 0.f;
+        first = first && !(same && q < s);
+      }
     }
     const unsigned long long keep = __ballot(first);
     if (first) {

@@ -860,16 +860,21 @@ def test_encoder_gemm_split_k(pkg, dev):
     assert ((got.double() - want).abs().max() / want.abs().max()).item() < 1e-5
 
 
+@pytest.mark.parametrize("ascending", [True, False])
 @pytest.mark.parametrize("G,B,k,F", [(4, 101, 16, 64), (1, 9, 8, 32), (3, 50, 64, 4096), (16, 7, 64, 256)])
-def test_union_group_codes(pkg, dev, G, B, k, F):
+def test_union_group_codes(pkg, dev, G, B, k, F, ascending):
     """Every (token, feature) of G stacked codes once, values summed in group order, order of first appearance; rows of
-    unequal length, a token with an empty row in every group, and 16 x 64 = 1024 entries per token (the limit)."""
+    unequal length, a token with an empty row in every group, and 16 x 64 = 1024 entries per token (the limit).  Rows in
+    ascending feature order (what the select kernels write: searched by bisection) and in any order (compared pairwise)."""
     g = torch.Generator().manual_seed(G * 1000 + B)
     idx = torch.stack([torch.randperm(F, generator=g)[:k] for _ in range(G * B)]).to(torch.int32)    # distinct within a row
     val = torch.randn(G * B, k, generator=g)
     nnz = torch.randint(0, k + 1, (G * B,), generator=g, dtype=torch.int32)
     nnz[torch.arange(G) * B + (B - 1)] = 0           # the last token keeps nothing anywhere
     nnz[:B] = k                                      # group 0's rows are full
+    if ascending:                                    # the live part of every row in ascending order
+        for r in range(G * B):
+            idx[r, :int(nnz[r])] = idx[r, :int(nnz[r])].sort().values
     code = pkg.ops.SparseCode(idx.flatten().to(dev), val.flatten().to(dev), (torch.arange(G * B) * k).to(dev), nnz.to(dev), G * B, F)
     got = pkg.ops.union_group_codes(code, G)
     assert got.n_tokens == B and got.d_sae == F and got.row_off.tolist() == [t * G * k for t in range(B)]
