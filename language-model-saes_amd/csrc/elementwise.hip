@@ -259,27 +259,50 @@ __global__ __launch_bounds__(256) void transpose_to_bf16_kernel(const void *__re
 
 // One workgroup per token: the token's sparse row (idx, val in slots row_off[b] .. + row_nnz[b]) written out as a
 // dense row of n_cols entries, in fp32 and / or bf16.  The row is assembled in LDS 8192 columns at a time, so every
-// global write is coalesced; indices outside [0, n_cols) are dropped.
+// global write is coalesced (16 bytes per lane where the row length and the outputs' alignment allow it); indices outside
+// [0, n_cols) are dropped.
 constexpr int C2D_CHUNK = 8192;
 __global__ __launch_bounds__(256) void code_to_dense_kernel(const int32_t *__restrict__ idx, const float *__restrict__ val,
                                                             const int64_t *__restrict__ row_off,
                                                             const int32_t *__restrict__ row_nnz, int64_t n_cols,
                                                             float *__restrict__ out_f32, uint16_t *__restrict__ out_bf16) {
-  __shared__ float row[C2D_CHUNK];
+  __shared__ __attribute__((aligned(16))) float row[C2D_CHUNK];
   const int64_t b = blockIdx.x;
   const int64_t off = row_off[b];
   const int n = row_nnz[b], tid = threadIdx.x;
+  const bool vec = (n_cols & 7) == 0 && ((((uintptr_t)out_f32) | ((uintptr_t)out_bf16)) & 15) == 0;
   for (int64_t c0 = 0; c0 < n_cols; c0 += C2D_CHUNK) {
     const int w = (int)(n_cols - c0 < C2D_CHUNK ? n_cols - c0 : C2D_CHUNK);
-    for (int i = tid; i < w; i += 256) row[i] = 0.f;
+    if (vec) {
+      const float4 z = {0.f, 0.f, 0.f, 0.f};
+      for (int i = tid * 4; i < w; i += 1024) *reinterpret_cast<float4 *>(row + i) = z;
+    } else {
+      for (int i = tid; i < w; i += 256) row[i] = 0.f;
+    }
     __syncthreads();
     for (int s = tid; s < n; s += 256) {
       const int64_t j = (int64_t)idx[off + s] - c0;
       if (j >= 0 && j < w) row[j] = val[off + s];   // a token's indices are distinct
     }
     __syncthreads();
-    if (out_f32) for (int i = tid; i < w; i += 256) out_f32[b * n_cols + c0 + i] = row[i];
-    if (out_bf16) for (int i = tid; i < w; i += 256) out_bf16[b * n_cols + c0 + i] = f32_to_bf16_bits(row[i]);
+    if (vec) {   // 16-byte stores: rows of a multiple of 8 columns from 16-byte aligned outputs
+      if (out_f32)
+        for (int i = tid * 4; i < w; i += 1024)
+          *reinterpret_cast<float4 *>(out_f32 + b * n_cols + c0 + i) = *reinterpret_cast<const float4 *>(row + i);
+      if (out_bf16)
+        for (int i = tid * 8; i < w; i += 2048) {
+          const float4 lo = *reinterpret_cast<const float4 *>(row + i), hi = *reinterpret_cast<const float4 *>(row + i + 4);
+          u32x4 o;
+          o.x = (uint32_t)f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
+          o.y = (uint32_t)f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
+          o.z = (uint32_t)f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
+          o.w = (uint32_t)f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+          *reinterpret_cast<u32x4 *>(out_bf16 + b * n_cols + c0 + i) = o;
+        }
+    } else {
+      if (out_f32) for (int i = tid; i < w; i += 256) out_f32[b * n_cols + c0 + i] = row[i];
+      if (out_bf16) for (int i = tid; i < w; i += 256) out_bf16[b * n_cols + c0 + i] = f32_to_bf16_bits(row[i]);
+    }
     __syncthreads();
   }
 }
