@@ -141,9 +141,10 @@ class _FusedCLTStep(torch.autograd.Function):
         tok_w = torch.full((B,), 1.0 / (L * B), dtype=torch.float32, device=x.device)
         w_dec_ops = m._w_dec_operands(amp)
         b_D = dec[L:]
-        grads = []
-        # the L decodes write their reconstructions and per-token losses into one buffer each and add their value gradients
-        # to one array: no stacking copy, no sum pass per layer
+        # the L decodes write their reconstructions, output gradients and per-token losses into one buffer each and add
+        # their value gradients to one array: no stacking copy, no sum pass per layer, and the backward casts / sums the
+        # output gradients of all layers in one launch each
+        grads = torch.empty(L, B, d, dtype=torch.float32, device=x.device)
         recon = torch.empty(L, B, d, dtype=torch.float32, device=x.device)
         loss_toks = torch.empty(L, B, dtype=torch.float32, device=x.device)
         dval = torch.zeros(cat.n_slots, dtype=torch.float32, device=x.device)
@@ -152,10 +153,9 @@ class _FusedCLTStep(torch.autograd.Function):
             # the merged code is sorted by layer inside a token, so a token's first prefix[b, j] slots are its entries of
             # layers <= j; the kernel visits exactly those
             code_j = dataclasses.replace(cat, row_nnz=prefix_t[j], d_sae=(j + 1) * F)
-            _, _, grad_recon, _ = ops.sparse_decode_mse_fused(
+            ops.sparse_decode_mse_fused(
                 code_j, w_dec_ops[j].view((j + 1) * F, d), b_D[j].detach(), label[j].contiguous(), tok_w,
-                recon_out=recon[j], loss_out=loss_toks[j], dval_acc=dval)
-            grads.append(grad_recon)
+                recon_out=recon[j], loss_out=loss_toks[j], dval_acc=dval, grad_out=grads[j])
         loss = loss_toks.sum()
         holder.update(code=cat, pres=pres, norms=norms, layer_cnt=layer_cnt)
         ctx.cat, ctx.grads, ctx.dval, ctx.x_op, ctx.w_enc_op = cat, grads, dval, x_op, w_enc_op
@@ -177,16 +177,16 @@ class _FusedCLTStep(torch.autograd.Function):
         dec_params = None if m is None else list(m.W_D)
         defer = (m is not None and m.W_E.grad is None and getattr(m.W_E, "_sparse_grad", None) is None
                  and all(w.grad is None and getattr(w, "_sparse_grad", None) is None for w in dec_params))
-        dW_D, db_D, dW_E, db_E = [], [], [], []
+        dW_D, dW_E, db_E = [], [], []
         enc_pieces = []
+        db_D = list((ctx.grads.sum(dim=1) * g).unbind(0))            # [L, d]: every layer's bias gradient in one reduction
+        gd_all = ops.cast_bf16(ctx.grads.view(L * B, d)).view(L, B, d) if (defer and ctx.amp) else ctx.grads
         for j in range(L):
             fi_j = ops.FeatureIndex(fi.feat_ptr[: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)      # features of layers <= j
             fi_l = ops.FeatureIndex(fi.feat_ptr[j * F: (j + 1) * F + 1], fi.feat_slot, fi.slot_tok)  # features of layer j
-            db_D.append(ops.col_sum(ctx.grads[j]) * g)
             if defer:
                 # the optimiser rebuilds the rows where it consumes them; nothing dense is written here
-                gd = ops.cast_bf16(ctx.grads[j]) if ctx.amp else ctx.grads[j]
-                dec_params[j]._sparse_grad = SparseRowGrad(fi_j, coef_dec, gd, (j + 1) * F)
+                dec_params[j]._sparse_grad = SparseRowGrad(fi_j, coef_dec, gd_all[j], (j + 1) * F)
                 enc_pieces.append((j * F, SparseRowGrad(fi_l, coef_enc, ctx.x_op[j], F)))
                 dW_D.append(None)
                 continue
@@ -211,7 +211,7 @@ class _FusedCLTStep(torch.autograd.Function):
                 parts.append(ops.sparse_decode_fwd(c, w_all, None))
             dx = torch.stack(parts, dim=1)
         if ctx.needs_input_grad[1]:
-            dlabel = -torch.stack(ctx.grads, dim=0) * g
+            dlabel = -ctx.grads * g
         return (dx, dlabel, None, None, dW_E, db_E, *dW_D, *db_D)
 
 

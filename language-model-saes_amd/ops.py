@@ -723,10 +723,11 @@ def sparse_decode_bwd_dval(code: SparseCode, grad_recon: torch.Tensor, w_dec: to
 
 def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Optional[torch.Tensor], label: torch.Tensor,
                             tok_w: Optional[torch.Tensor], want_recon: bool = True, recon_out: Optional[torch.Tensor] = None,
-                            loss_out: Optional[torch.Tensor] = None, dval_acc: Optional[torch.Tensor] = None):
-    """Returns (recon or None, loss_tok [B], grad_recon [B, d], dval [n_slots]).  `recon_out` [B, d] / `loss_out` [B]
-    (fp32, contiguous) receive those outputs in place of fresh tensors; `dval_acc` [n_slots] has the value gradients
-    added to it (and is returned as dval) instead of being overwritten: for a code several decoders share."""
+                            loss_out: Optional[torch.Tensor] = None, dval_acc: Optional[torch.Tensor] = None,
+                            grad_out: Optional[torch.Tensor] = None):
+    """Returns (recon or None, loss_tok [B], grad_recon [B, d], dval [n_slots]).  `recon_out` [B, d] / `loss_out` [B] /
+    `grad_out` [B, d] (fp32, contiguous) receive those outputs in place of fresh tensors; `dval_acc` [n_slots] has the
+    value gradients added to it (and is returned as dval) instead of being overwritten: for a code several decoders share."""
     _check_code(code, w_dec)
     _req(label, "label", torch.float32, 2)
     F, d = w_dec.shape
@@ -750,7 +751,11 @@ def sparse_decode_mse_fused(code: SparseCode, w_dec: torch.Tensor, b_dec: Option
             raise ValueError(f"dval_acc must hold {code.n_slots} values")
     recon = recon_out if recon_out is not None else (torch.empty(B, d, dtype=torch.float32, device=dev) if want_recon else None)
     loss_tok = loss_out if loss_out is not None else torch.empty(B, dtype=torch.float32, device=dev)
-    grad_recon = torch.empty(B, d, dtype=torch.float32, device=dev)
+    if grad_out is not None:
+        _req(grad_out, "grad_out", torch.float32, 2)
+        if tuple(grad_out.shape) != (B, d):
+            raise ValueError(f"grad_out must be {(B, d)}")
+    grad_recon = grad_out if grad_out is not None else torch.empty(B, d, dtype=torch.float32, device=dev)
     dval = dval_acc if dval_acc is not None else torch.empty(code.n_slots, dtype=torch.float32, device=dev)
     lib = _lib.load()
     fn = lib.sae_sparse_decode_mse_fused_acc if dval_acc is not None else lib.sae_sparse_decode_mse_fused
