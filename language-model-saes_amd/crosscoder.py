@@ -55,9 +55,17 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         norms = m._decoder_norm_nograd()                              # [H, F]
         w_dec_op = m._w_dec_operand(amp)                              # [H, F, d]
         b_sum = b_E.detach().sum(dim=0)
-        codes, recons, grads, dvals = [], [], [], []
-        loss = None
+        codes = []
         stacked = None
+        # head-major copies of the per-token operands (one launch each instead of one per head), and one buffer per output
+        # of the H decodes: reconstructions, output gradients, value gradients, per-token losses
+        label_h = label.transpose(0, 1).contiguous()                     # [H, B, d]
+        tokw_h = tok_w.t().contiguous()                                  # [H, B]
+        b_D_h = b_D.detach().contiguous()
+        recons = torch.empty(H, B, d, dtype=torch.float32, device=x.device)
+        grads = torch.empty(H, B, d, dtype=torch.float32, device=x.device)
+        loss_toks = torch.empty(H, B, dtype=torch.float32, device=x.device)
+        dvals = []
         if (amp and pre.dtype == torch.bfloat16 and getattr(m, "granule_select", True) and ops.granule_route_supported(64, F, int(k))):
             # every head selects from the same summed encoding under its own decoder norms: ONE pass for the per-granule key
             # maxima of the H * B (head, token) rows and ONE select over them, each row reading only the granules that can
@@ -73,11 +81,11 @@ class _FusedCrosscoderStep(torch.autograd.Function):
                 code = ops.SparseCode(stacked.idx[sl], stacked.val[sl], stacked.row_off[rows] - h * B * k, stacked.row_nnz[rows], B, F)
             else:
                 code = ops.select_topk_row(pre, b_sum, norms[h], k)
-            recon, loss_tok, grad_recon, dval = ops.sparse_decode_mse_fused(
-                code, w_dec_op[h], b_D.detach()[h].contiguous(), label[:, h].contiguous(), tok_w[:, h].contiguous())
-            codes.append(code); recons.append(recon); grads.append(grad_recon); dvals.append(dval)
-            loss = loss_tok.sum() if loss is None else loss + loss_tok.sum()
-        recon = torch.stack(recons, dim=1)
+            _, _, _, dval = ops.sparse_decode_mse_fused(code, w_dec_op[h], b_D_h[h], label_h[h], tokw_h[h], recon_out=recons[h],
+                                                        loss_out=loss_toks[h], grad_out=grads[h])
+            codes.append(code); dvals.append(dval)
+        loss = loss_toks.sum()
+        recon = recons.transpose(0, 1)                                   # [B, H, d]
         holder["codes"], holder["pre"], holder["norms"], holder["b_sum"] = codes, pre, norms, b_sum
         ctx.codes, ctx.grads, ctx.dvals, ctx.x_op, ctx.w_enc_op = codes, grads, dvals, x_op, w_enc_op
         ctx.stacked = stacked
@@ -93,7 +101,7 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         g = g_loss.to(torch.float32)
         m = ctx.defer_to
         defer = (m is not None and all(w.grad is None and getattr(w, "_sparse_grad", None) is None for w in (m.W_E, m.W_D)))
-        db_D = [ops.col_sum(ctx.grads[h]) * g for h in range(H)]
+        db_D = ctx.grads.sum(dim=1) * g                                  # [H, d]
         # the H codes on a virtual token axis: token h * B + b
         stacked = ctx.stacked if ctx.stacked is not None else reduce(ops.stack_codes, ctx.codes)
         coef = torch.cat(ctx.dvals) * g
@@ -110,11 +118,9 @@ class _FusedCrosscoderStep(torch.autograd.Function):
         if ctx.amp:
             # the decoder's weight gradient pairs the activations with the bf16-rounded output gradient, as the backward of
             # an autocast product does; the gathered rows then move half the bytes
-            gd = torch.empty(H * B, d, dtype=torch.bfloat16, device=stacked.val.device)
-            for h in range(H):
-                ops.cast_bf16(ctx.grads[h], gd[h * B:(h + 1) * B])
+            gd = ops.cast_bf16(ctx.grads.view(H * B, d))
         else:
-            gd = torch.cat(ctx.grads)
+            gd = ctx.grads.view(H * B, d)
         if defer:
             # The optimiser rebuilds the rows where it consumes them; nothing dense is written here.  The decoder
             # [H, F, d] is one matrix of H F rows: head h's code addresses rows h F .. (h + 1) F of it, and its dense
@@ -141,8 +147,8 @@ class _FusedCrosscoderStep(torch.autograd.Function):
                      for c, dv in zip(ctx.codes, ctx.dvals)]
             dx = reduce(torch.add, parts).view(B, H, d)
         if ctx.needs_input_grad[1]:
-            dlabel = -torch.stack(ctx.grads, dim=1) * g
-        return dx, dlabel, None, dW_E, db_E, dW_D, torch.stack(db_D), None, None, None
+            dlabel = -ctx.grads.transpose(0, 1) * g
+        return dx, dlabel, None, dW_E, db_E, dW_D, db_D, None, None, None
 
 
 @register_sae_model("crosscoder")
